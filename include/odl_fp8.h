@@ -1,0 +1,138 @@
+/*
+ * odl_fp8.h - C ABI of the MI355X (gfx950) FP8 Linear kernels.
+ *
+ * This is the native boundary under the FP8 AMP Linear path of Optimus-DL.  In
+ * the reference that boundary is the call into a third-party CUDA library:
+ *   optimus_dl/modules/model_transforms/transformer_engine.py:97-108
+ *       (TELinear builds and calls te.pytorch.Linear: amax, cast, cast+transpose,
+ *        FP8 GEMM for fwd / dgrad / wgrad)
+ *   optimus_dl/modules/amp/fp8.py:279-306,337-340,357-360
+ *       (recipe objects and the autocast contexts whose exit refreshes the scales)
+ * Each entry point below names the step of that call it stands in for.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless the comment says "host";
+ *   - matrices are dense row-major; `rows`/`cols` are in elements;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream);
+ *     nothing here synchronises with the host or allocates memory;
+ *   - return value 0 = launched; non-zero = refused, nothing was launched, and
+ *     odl_fp8_last_error() (host string, thread-local) says why;
+ *   - 8-bit codes are OCP FP8: E4M3 ("fn": no Inf, 0x7F/0xFF = NaN, max 448) and
+ *     E5M2 (max 57344).  Conversion is round-to-nearest-even after an explicit
+ *     clamp to +-max; NaN inputs give 0x7F with the input's sign bit.
+ */
+#ifndef ODL_FP8_H
+#define ODL_FP8_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *odl_stream_t;
+
+enum odl_fp8_format { ODL_FP8_E4M3 = 0, ODL_FP8_E5M2 = 1 };
+enum odl_scale_mode { ODL_SCALE_TENSOR = 0, ODL_SCALE_ROW = 1, ODL_SCALE_COL = 2 };
+enum odl_dtype { ODL_BF16 = 0, ODL_F32 = 1 };
+enum odl_amax_algo { ODL_AMAX_MAX = 0, ODL_AMAX_MOST_RECENT = 1 };
+
+enum odl_status {
+    ODL_OK = 0,
+    ODL_ERR_ARG = 1,      /* bad enum / null pointer / negative size */
+    ODL_ERR_SHAPE = 2,    /* shape or alignment the kernels do not support */
+    ODL_ERR_LAUNCH = 3    /* HIP reported an error at launch */
+};
+
+/* ABI version of this header; bumped on any signature change. */
+int odl_fp8_abi_version(void);
+
+/* Last error message of the calling host thread ("" if none). */
+const char *odl_fp8_last_error(void);
+
+/*
+ * amax = max |x| of a [rows, cols] matrix, as fp32.
+ *   mode TENSOR -> amax_out[1], ROW -> amax_out[rows], COL -> amax_out[cols]
+ *   accumulate != 0: amax_out = max(amax_out, amax(x)) (used to fold several
+ *   tensors, or microbatches, into one history slot); otherwise overwritten.
+ * NaN in x yields NaN.  Stands in for the amax reduction inside the
+ * quantisation step of te.pytorch.Linear (transformer_engine.py:106).
+ */
+int odl_fp8_amax(const void *x, int src_dtype, int64_t rows, int64_t cols, int mode,
+                 float *amax_out, int accumulate, odl_stream_t stream);
+
+/*
+ * scale[i]     = fp8_max(fmt) / amax[i] / 2^margin   (IEEE fp32 division)
+ * scale_inv[i] = 1 / scale[i]
+ * amax[i] that is 0, negative, NaN or Inf gives scale 1; an infinite quotient
+ * gives FLT_MAX.  This is the "current scaling" rule (recipe "tensorwise",
+ * fp8.py:289-294) applied to n independent amaxes.
+ */
+int odl_fp8_scale_from_amax(const float *amax, int64_t n, int fmt, int margin,
+                            float *scale, float *scale_inv, odl_stream_t stream);
+
+/*
+ * out[r,c] = fp8( clamp( fp32(x[r,c]) * s , +-max ) ), s = scale[0] | scale[r] | scale[c].
+ * amax_out (may be NULL): *amax_out = max(*amax_out, max|x|), for delayed scaling,
+ * where the cast uses an older scale while this step's amax is recorded.
+ * Stands in for the cast inside te.pytorch.Linear (transformer_engine.py:106).
+ */
+int odl_fp8_cast(const void *x, int src_dtype, int64_t rows, int64_t cols,
+                 const float *scale, int mode, int fmt,
+                 uint8_t *out, float *amax_out, odl_stream_t stream);
+
+/*
+ * Same cast, also written transposed: out_t[c,r] = out[r,c] (out may be NULL
+ * when only the transposed copy is wanted).  The transposed copies are what
+ * dgrad (W^T) and wgrad (dY^T, X^T) contract over.
+ */
+int odl_fp8_cast_transpose(const void *x, int src_dtype, int64_t rows, int64_t cols,
+                           const float *scale, int mode, int fmt,
+                           uint8_t *out, uint8_t *out_t, float *amax_out, odl_stream_t stream);
+
+/*
+ * C[M,N] = (A[M,K] . B[N,K]^T) * (sa_inv[i] * sb_inv[j]) (+ bias[j]), fp32
+ * accumulate on the MFMA units, rounded once to out_dtype (bf16 or fp32).
+ *   a, b     : FP8 codes, K contiguous ("NT"); fmt_a / fmt_b may differ
+ *   sa_inv   : 1 value (sa_n == 1) or M values; sb_inv: 1 or N values
+ *   bias     : NULL or N fp32 values (bias_dtype must be ODL_F32), added in fp32
+ *              before the single rounding to out_dtype
+ * Covers fwd (A=Xq, B=Wq), dgrad (A=dYq, B=Wq^T) and wgrad (A=dYq^T, B=Xq^T):
+ * the three GEMMs of te.pytorch.Linear forward/backward.
+ * K must be a multiple of 16; any M, N >= 1.
+ */
+int odl_fp8_gemm_nt(const uint8_t *a, const uint8_t *b, int64_t M, int64_t N, int64_t K,
+                    int fmt_a, int fmt_b,
+                    const float *sa_inv, int64_t sa_n, const float *sb_inv, int64_t sb_n,
+                    const void *bias, int bias_dtype,
+                    void *c, int out_dtype, odl_stream_t stream);
+
+/*
+ * Delayed-scaling bookkeeping for R tensor roles with H history slots each
+ * (recipe "delayed", fp8.py:279-288; runs where the reference leaves its
+ * autocast context, fp8.py:337-340,357-360).
+ *   history [H,R] fp32, row 0 = newest amax (written by the casts of the step)
+ *   a = max over the column (ODL_AMAX_MAX) or history[0] (ODL_AMAX_MOST_RECENT)
+ *   history <- roll(history, -1 along H); history[0] <- 0
+ *   scale[r] = fp8_max(fmt[r]) / a / 2^margin, kept when a is 0/NaN/Inf; Inf -> FLT_MAX
+ *   scale_inv[r] = 1 / scale[r]
+ *   fmt: R ints (odl_fp8_format) in device memory.
+ */
+int odl_fp8_delayed_update(float *history, int64_t H, int64_t R,
+                           float *scale, float *scale_inv, const int *fmt,
+                           int margin, int algo, odl_stream_t stream);
+
+/*
+ * Tuning / introspection (host only).  Selects the GEMM kernel variant:
+ * -1 = automatic choice by shape; otherwise an index < odl_fp8_gemm_num_variants().
+ * odl_fp8_gemm_variant_name returns a short description ("256x256x128 w4 s2").
+ */
+int odl_fp8_gemm_num_variants(void);
+const char *odl_fp8_gemm_variant_name(int variant);
+int odl_fp8_gemm_set_variant(int variant);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ODL_FP8_H */

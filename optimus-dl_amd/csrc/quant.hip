@@ -1,0 +1,707 @@
+// Memory-bound half of the FP8 Linear path for gfx950: amax reductions,
+// scale-and-cast, fused cast+transpose, and the scale bookkeeping kernels.
+//
+// All of these are bound by HBM bandwidth.  Design rules used throughout:
+//   * 128-bit global loads, several in flight per lane before the first use;
+//   * 64-lane wavefront reductions through DPP shuffles, one LDS slot per wave,
+//     one atomic per block (amax is a max, so any reduction tree is exact);
+//   * grids sized to a few waves of blocks per CU so all 8 XCDs stay busy and
+//     the tail is short.
+#include "common.h"
+
+#include <float.h>
+
+namespace odl {
+
+constexpr int kThreads = 256;
+
+__device__ __forceinline__ u32x4 load16(const void *p) { return *reinterpret_cast<const u32x4 *>(p); }
+
+// ---------------------------------------------------------------- fill (tiny)
+__global__ void fill_f32_kernel(float *p, int64_t n, float v) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+
+// ------------------------------------------------------------ amax, per tensor
+// x viewed as n16 chunks of 16 bytes plus a scalar tail.  Each lane keeps UNROLL
+// loads in flight; magnitudes are reduced as integer bit patterns.
+template <int SRC, int UNROLL>
+__global__ __launch_bounds__(kThreads) void amax_tensor_kernel(const void *__restrict__ x, int64_t n,
+                                                                float *__restrict__ out) {
+    __shared__ uint32_t red[kThreads / kWave];
+    constexpr int EPC = SRC == ODL_BF16 ? 8 : 4;          // elements per 16-byte chunk
+    const int64_t n16 = n / EPC;
+    const u32x4 *p = reinterpret_cast<const u32x4 *>(x);
+    const int64_t stride = (int64_t)gridDim.x * kThreads;
+    int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    uint32_t m0 = 0, m1 = 0, m2 = 0, m3 = 0;
+    for (; i + (UNROLL - 1) * stride < n16; i += UNROLL * stride) {
+        u32x4 v[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) v[u] = __builtin_nontemporal_load(p + i + u * stride);
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            if constexpr (SRC == ODL_BF16) {
+                m0 = max_u16x2(m0, abs_bf16x2(v[u].x));
+                m1 = max_u16x2(m1, abs_bf16x2(v[u].y));
+                m2 = max_u16x2(m2, abs_bf16x2(v[u].z));
+                m3 = max_u16x2(m3, abs_bf16x2(v[u].w));
+            } else {
+                m0 = max(m0, v[u].x & 0x7fffffffu);
+                m1 = max(m1, v[u].y & 0x7fffffffu);
+                m2 = max(m2, v[u].z & 0x7fffffffu);
+                m3 = max(m3, v[u].w & 0x7fffffffu);
+            }
+        }
+    }
+    for (; i < n16; i += stride) {
+        u32x4 v = p[i];
+        if constexpr (SRC == ODL_BF16) {
+            m0 = max_u16x2(m0, abs_bf16x2(v.x));
+            m1 = max_u16x2(m1, abs_bf16x2(v.y));
+            m2 = max_u16x2(m2, abs_bf16x2(v.z));
+            m3 = max_u16x2(m3, abs_bf16x2(v.w));
+        } else {
+            m0 = max(m0, v.x & 0x7fffffffu);
+            m1 = max(m1, v.y & 0x7fffffffu);
+            m2 = max(m2, v.z & 0x7fffffffu);
+            m3 = max(m3, v.w & 0x7fffffffu);
+        }
+    }
+    uint32_t m;
+    if constexpr (SRC == ODL_BF16) {
+        m = fold_u16x2_to_f32bits(max_u16x2(max_u16x2(m0, m1), max_u16x2(m2, m3)));
+    } else {
+        m = max(max(m0, m1), max(m2, m3));
+    }
+    // scalar tail (fewer than EPC elements), done by one thread
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        for (int64_t t = n16 * EPC; t < n; ++t) {
+            uint32_t b;
+            if constexpr (SRC == ODL_BF16) b = ((uint32_t) reinterpret_cast<const uint16_t *>(x)[t] & 0x7fffu) << 16;
+            else b = reinterpret_cast<const uint32_t *>(x)[t] & 0x7fffffffu;
+            m = max(m, b);
+        }
+    }
+    m = block_max_u32(m, red);
+    if (threadIdx.x == 0 && m != 0) atomicMax(reinterpret_cast<uint32_t *>(out), m);
+}
+
+// element-at-a-time variant for pointers that are not 16-byte aligned
+template <int SRC>
+__global__ __launch_bounds__(kThreads) void amax_tensor_scalar_kernel(const void *__restrict__ x, int64_t n,
+                                                                       float *__restrict__ out) {
+    __shared__ uint32_t red[kThreads / kWave];
+    uint32_t m = 0;
+    for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += (int64_t)gridDim.x * kThreads) {
+        uint32_t b;
+        if constexpr (SRC == ODL_BF16) b = ((uint32_t) reinterpret_cast<const uint16_t *>(x)[i] & 0x7fffu) << 16;
+        else b = reinterpret_cast<const uint32_t *>(x)[i] & 0x7fffffffu;
+        m = max(m, b);
+    }
+    m = block_max_u32(m, red);
+    if (threadIdx.x == 0 && m != 0) atomicMax(reinterpret_cast<uint32_t *>(out), m);
+}
+
+// ---------------------------------------------------------------- amax, per row
+// One wavefront per row, kThreads/64 rows per block.  Handles any cols; the
+// 16-byte path is used for the aligned middle of the row.
+template <int SRC, bool ACC>
+__global__ __launch_bounds__(kThreads) void amax_row_kernel(const void *__restrict__ x, int64_t rows, int64_t cols,
+                                                             float *__restrict__ out) {
+    constexpr int ESZ = SRC == ODL_BF16 ? 2 : 4;
+    constexpr int EPC = 16 / ESZ;
+    const int lane = threadIdx.x % kWave;
+    const int64_t row = (int64_t)blockIdx.x * (kThreads / kWave) + threadIdx.x / kWave;
+    if (row >= rows) return;
+    const char *base = reinterpret_cast<const char *>(x) + row * cols * ESZ;
+    // elements before the first 16-byte boundary
+    int64_t head = ((16 - (reinterpret_cast<uintptr_t>(base) & 15)) & 15) / ESZ;
+    if (head > cols) head = cols;
+    const int64_t n16 = (cols - head) / EPC;
+    auto elem_bits = [&](int64_t c) -> uint32_t {
+        if constexpr (SRC == ODL_BF16) return ((uint32_t) reinterpret_cast<const uint16_t *>(base)[c] & 0x7fffu) << 16;
+        else return reinterpret_cast<const uint32_t *>(base)[c] & 0x7fffffffu;
+    };
+    uint32_t m = 0;
+    for (int64_t c = lane; c < head; c += kWave) m = max(m, elem_bits(c));
+    for (int64_t c = head + n16 * EPC + lane; c < cols; c += kWave) m = max(m, elem_bits(c));
+    const u32x4 *p = reinterpret_cast<const u32x4 *>(base + head * ESZ);
+    uint32_t a0 = 0, a1 = 0, a2 = 0, a3 = 0;
+    int64_t i = lane;
+    for (; i + 3 * kWave < n16; i += 4 * kWave) {
+        u32x4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = __builtin_nontemporal_load(p + i + u * kWave);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            if constexpr (SRC == ODL_BF16) {
+                a0 = max_u16x2(a0, abs_bf16x2(v[u].x)); a1 = max_u16x2(a1, abs_bf16x2(v[u].y));
+                a2 = max_u16x2(a2, abs_bf16x2(v[u].z)); a3 = max_u16x2(a3, abs_bf16x2(v[u].w));
+            } else {
+                a0 = max(a0, v[u].x & 0x7fffffffu); a1 = max(a1, v[u].y & 0x7fffffffu);
+                a2 = max(a2, v[u].z & 0x7fffffffu); a3 = max(a3, v[u].w & 0x7fffffffu);
+            }
+        }
+    }
+    for (; i < n16; i += kWave) {
+        u32x4 v = p[i];
+        if constexpr (SRC == ODL_BF16) {
+            a0 = max_u16x2(a0, abs_bf16x2(v.x)); a1 = max_u16x2(a1, abs_bf16x2(v.y));
+            a2 = max_u16x2(a2, abs_bf16x2(v.z)); a3 = max_u16x2(a3, abs_bf16x2(v.w));
+        } else {
+            a0 = max(a0, v.x & 0x7fffffffu); a1 = max(a1, v.y & 0x7fffffffu);
+            a2 = max(a2, v.z & 0x7fffffffu); a3 = max(a3, v.w & 0x7fffffffu);
+        }
+    }
+    if constexpr (SRC == ODL_BF16) m = max(m, fold_u16x2_to_f32bits(max_u16x2(max_u16x2(a0, a1), max_u16x2(a2, a3))));
+    else m = max(m, max(max(a0, a1), max(a2, a3)));
+    m = wave_max_u32(m);
+    if (lane == 0) {
+        uint32_t *o = reinterpret_cast<uint32_t *>(out) + row;
+        if constexpr (ACC) { if (m > *o) *o = m; }     // one writer per row: plain read-modify-write
+        else *o = m;
+    }
+}
+
+// ------------------------------------------------------------- amax, per column
+// Block = 32 column-lanes x 8 row-lanes; each lane owns CPL consecutive columns
+// (one 16-byte load) and walks ROWS_PER_BLOCK rows in steps of 8.  Column maxima
+// are combined through LDS, then one atomicMax per column per block.
+template <int SRC>
+__global__ __launch_bounds__(kThreads) void amax_col_kernel(const void *__restrict__ x, int64_t rows, int64_t cols,
+                                                             int rows_per_block, float *__restrict__ out) {
+    constexpr int ESZ = SRC == ODL_BF16 ? 2 : 4;
+    constexpr int CPL = 16 / ESZ;                 // columns per lane
+    constexpr int CW = 32 * CPL;                  // columns per block
+    __shared__ uint32_t red[8][CW + 1];
+    const int tx = threadIdx.x % 32, ty = threadIdx.x / 32;
+    const int64_t c0 = (int64_t)blockIdx.x * CW + tx * CPL;
+    const int64_t r0 = (int64_t)blockIdx.y * rows_per_block;
+    const int64_t r1 = min(rows, r0 + rows_per_block);
+    uint32_t m[CPL];
+#pragma unroll
+    for (int j = 0; j < CPL; ++j) m[j] = 0;
+    const char *base = reinterpret_cast<const char *>(x);
+    if (c0 + CPL <= cols) {                        // host guarantees cols % CPL == 0 and 16-byte rows
+        int64_t r = r0 + ty;
+        for (; r + 24 < r1; r += 32) {
+            u32x4 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(base + ((r + 8 * u) * cols + c0) * ESZ));
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                uint32_t w[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    if constexpr (SRC == ODL_BF16) {
+                        uint32_t a = abs_bf16x2(w[q]);
+                        m[2 * q] = max(m[2 * q], (a & 0xffffu) << 16);
+                        m[2 * q + 1] = max(m[2 * q + 1], a & 0xffff0000u);
+                    } else {
+                        m[q] = max(m[q], w[q] & 0x7fffffffu);
+                    }
+                }
+            }
+        }
+        for (; r < r1; r += 8) {
+            u32x4 v = *reinterpret_cast<const u32x4 *>(base + (r * cols + c0) * ESZ);
+            uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                if constexpr (SRC == ODL_BF16) {
+                    uint32_t a = abs_bf16x2(w[q]);
+                    m[2 * q] = max(m[2 * q], (a & 0xffffu) << 16);
+                    m[2 * q + 1] = max(m[2 * q + 1], a & 0xffff0000u);
+                } else {
+                    m[q] = max(m[q], w[q] & 0x7fffffffu);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < CPL; ++j) red[ty][tx * CPL + j] = m[j];
+    __syncthreads();
+    for (int c = threadIdx.x; c < CW; c += kThreads) {
+        uint32_t v = 0;
+#pragma unroll
+        for (int y = 0; y < 8; ++y) v = max(v, red[y][c]);
+        const int64_t col = (int64_t)blockIdx.x * CW + c;
+        if (col < cols && v != 0) atomicMax(reinterpret_cast<uint32_t *>(out) + col, v);
+    }
+}
+
+// generic column amax for shapes the vector kernel refuses: one thread per column strip
+template <int SRC>
+__global__ void amax_col_scalar_kernel(const void *__restrict__ x, int64_t rows, int64_t cols, int rows_per_block,
+                                       float *__restrict__ out) {
+    const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= cols) return;
+    const int64_t r0 = (int64_t)blockIdx.y * rows_per_block, r1 = min(rows, r0 + rows_per_block);
+    uint32_t m = 0;
+    for (int64_t r = r0; r < r1; ++r) {
+        uint32_t b;
+        if constexpr (SRC == ODL_BF16) b = ((uint32_t) reinterpret_cast<const uint16_t *>(x)[r * cols + c] & 0x7fffu) << 16;
+        else b = reinterpret_cast<const uint32_t *>(x)[r * cols + c] & 0x7fffffffu;
+        m = max(m, b);
+    }
+    if (m != 0) atomicMax(reinterpret_cast<uint32_t *>(out) + c, m);
+}
+
+// ------------------------------------------------------------- scale from amax
+__device__ __forceinline__ float scale_rule(float amax, float fp8_max, int margin, float fallback) {
+    if (!(amax > 0.0f) || __builtin_isinf(amax)) return fallback;
+    float s = __fdiv_rn(fp8_max, amax);                     // IEEE division, not the fast reciprocal
+    s = ldexpf(s, -margin);
+    if (__builtin_isinf(s)) s = FLT_MAX;
+    return s;
+}
+
+__global__ void scale_from_amax_kernel(const float *__restrict__ amax, int64_t n, float fp8_max, int margin,
+                                       float *__restrict__ scale, float *__restrict__ scale_inv) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    float s = scale_rule(amax[i], fp8_max, margin, 1.0f);
+    scale[i] = s;
+    if (scale_inv) scale_inv[i] = __fdiv_rn(1.0f, s);
+}
+
+// one thread per role; H is small (<= a few thousand), latency only
+__global__ void delayed_update_kernel(float *__restrict__ history, int64_t H, int64_t R, float *__restrict__ scale,
+                                      float *__restrict__ scale_inv, const int *__restrict__ fmt, int margin, int algo) {
+    int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (r >= R) return;
+    const float first = history[r];
+    uint32_t abits = float_to_bits(first) & 0x7fffffffu;     // amaxes are >= 0 or NaN: integer max keeps NaN
+    float prev = first;
+    for (int64_t h = 1; h < H; ++h) {
+        float cur = history[h * R + r];
+        if (algo == ODL_AMAX_MAX) abits = max(abits, float_to_bits(cur) & 0x7fffffffu);
+        history[(h - 1) * R + r] = cur;                       // roll by -1
+        prev = cur;
+    }
+    (void)prev;
+    history[(H - 1) * R + r] = first;
+    history[r] = 0.0f;
+    const float fmax = fmt[r] == ODL_FP8_E5M2 ? 57344.0f : 448.0f;
+    float s = scale_rule(bits_to_float(abits), fmax, margin, scale[r]);
+    scale[r] = s;
+    scale_inv[r] = __fdiv_rn(1.0f, s);
+}
+
+// ------------------------------------------------------------------------ cast
+// 16 elements per lane per step: two (bf16) or four (fp32) 16-byte loads, one
+// 16-byte store.  cols % 16 == 0 and 16-byte aligned pointers (host-checked).
+template <int SRC, int FMT, int MODE, bool AMAX>
+__global__ __launch_bounds__(kThreads) void cast_kernel(const void *__restrict__ x, int64_t rows, int64_t cols,
+                                                         const float *__restrict__ scale, uint8_t *__restrict__ out,
+                                                         float *__restrict__ amax_out) {
+    __shared__ uint32_t red[kThreads / kWave];
+    const int64_t cpr = cols / 16;                           // chunks per row
+    const int64_t nchunk = rows * cpr;
+    const int64_t stride = (int64_t)gridDim.x * kThreads;
+    float s_t = 1.0f;
+    if constexpr (MODE == ODL_SCALE_TENSOR) s_t = scale[0];
+    uint32_t am = 0;
+    for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < nchunk; i += stride) {
+        float f[16];
+        if constexpr (SRC == ODL_BF16) {
+            const u32x4 *p = reinterpret_cast<const u32x4 *>(x) + i * 2;
+            u32x4 v0 = __builtin_nontemporal_load(p), v1 = __builtin_nontemporal_load(p + 1);
+            uint32_t w[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                f[2 * q] = bf16_lo(w[q]);
+                f[2 * q + 1] = bf16_hi(w[q]);
+                if constexpr (AMAX) am = max_u16x2(am, abs_bf16x2(w[q]));
+            }
+        } else {
+            const u32x4 *p = reinterpret_cast<const u32x4 *>(x) + i * 4;
+            u32x4 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = __builtin_nontemporal_load(p + u);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                f[4 * u] = bits_to_float(v[u].x); f[4 * u + 1] = bits_to_float(v[u].y);
+                f[4 * u + 2] = bits_to_float(v[u].z); f[4 * u + 3] = bits_to_float(v[u].w);
+                if constexpr (AMAX) am = max(am, max(max(v[u].x & 0x7fffffffu, v[u].y & 0x7fffffffu),
+                                                     max(v[u].z & 0x7fffffffu, v[u].w & 0x7fffffffu)));
+            }
+        }
+        float s[16];
+        if constexpr (MODE == ODL_SCALE_TENSOR) {
+#pragma unroll
+            for (int j = 0; j < 16; ++j) s[j] = s_t;
+        } else if constexpr (MODE == ODL_SCALE_ROW) {
+            const float sr = scale[i / cpr];
+#pragma unroll
+            for (int j = 0; j < 16; ++j) s[j] = sr;
+        } else {
+            const float4 *sp = reinterpret_cast<const float4 *>(scale + (i % cpr) * 16);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) { float4 t = sp[u]; s[4 * u] = t.x; s[4 * u + 1] = t.y; s[4 * u + 2] = t.z; s[4 * u + 3] = t.w; }
+        }
+        u32x4 o;
+        o.x = quantise4<FMT>(f[0], f[1], f[2], f[3], s[0], s[1], s[2], s[3]);
+        o.y = quantise4<FMT>(f[4], f[5], f[6], f[7], s[4], s[5], s[6], s[7]);
+        o.z = quantise4<FMT>(f[8], f[9], f[10], f[11], s[8], s[9], s[10], s[11]);
+        o.w = quantise4<FMT>(f[12], f[13], f[14], f[15], s[12], s[13], s[14], s[15]);
+        __builtin_nontemporal_store(o, reinterpret_cast<u32x4 *>(out) + i);
+    }
+    if constexpr (AMAX) {
+        if constexpr (SRC == ODL_BF16) am = fold_u16x2_to_f32bits(am);
+        am = block_max_u32(am, red);
+        if (threadIdx.x == 0 && am != 0) atomicMax(reinterpret_cast<uint32_t *>(amax_out), am);
+    }
+}
+
+// element-at-a-time cast (+ optional transposed copy) for any shape / alignment
+template <int SRC, int FMT>
+__global__ __launch_bounds__(kThreads) void cast_generic_kernel(const void *__restrict__ x, int64_t rows, int64_t cols,
+                                                                 const float *__restrict__ scale, int mode,
+                                                                 uint8_t *__restrict__ out, uint8_t *__restrict__ out_t,
+                                                                 float *__restrict__ amax_out) {
+    __shared__ uint32_t red[kThreads / kWave];
+    uint32_t am = 0;
+    const int64_t n = rows * cols;
+    for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += (int64_t)gridDim.x * kThreads) {
+        const int64_t r = i / cols, c = i % cols;
+        float f;
+        if constexpr (SRC == ODL_BF16) f = bits_to_float((uint32_t) reinterpret_cast<const uint16_t *>(x)[i] << 16);
+        else f = reinterpret_cast<const float *>(x)[i];
+        am = max(am, float_to_bits(f) & 0x7fffffffu);
+        const float s = mode == ODL_SCALE_TENSOR ? scale[0] : (mode == ODL_SCALE_ROW ? scale[r] : scale[c]);
+        const uint8_t q = (uint8_t)(quantise4<FMT>(f, 0.f, 0.f, 0.f, s, 1.f, 1.f, 1.f) & 0xffu);
+        if (out) out[i] = q;
+        if (out_t) out_t[c * rows + r] = q;
+    }
+    if (amax_out) {
+        am = block_max_u32(am, red);
+        if (threadIdx.x == 0 && am != 0) atomicMax(reinterpret_cast<uint32_t *>(amax_out), am);
+    }
+}
+
+// -------------------------------------------------------------- cast+transpose
+// Tile = 128 rows x 64 cols of x per block of 256 lanes.  A lane owns a 4 x 8
+// patch: four 16-byte (bf16) loads, one per row.  The row-major codes leave as
+// 8-byte stores (a wave covers whole 64-byte row segments); the transposed codes
+// go through a 4x4 byte transpose in registers (v_perm_b32) and an LDS tile
+// [64 cols][128 rows] so that they leave as 16-byte stores along the row axis:
+// both outputs are written in full 64/128-byte segments.
+constexpr int kTileR = 128, kTileC = 64, kLdsPitch = kTileR + 4;   // pitch in bytes; +4 keeps dword writes conflict-poor
+
+// 4x4 byte transpose: in a[j] byte k  ->  out t[k] byte j
+__device__ __forceinline__ void transpose4x4(const uint32_t a[4], uint32_t t[4]) {
+    // v_perm_b32(hi, lo, sel): result byte i = bytes{hi:lo}[sel byte i], lo = bytes 0..3, hi = 4..7
+    const uint32_t p01_lo = __builtin_amdgcn_perm(a[1], a[0], 0x05010400u);  // a0.b0 a1.b0 a0.b1 a1.b1
+    const uint32_t p01_hi = __builtin_amdgcn_perm(a[1], a[0], 0x07030602u);  // a0.b2 a1.b2 a0.b3 a1.b3
+    const uint32_t p23_lo = __builtin_amdgcn_perm(a[3], a[2], 0x05010400u);
+    const uint32_t p23_hi = __builtin_amdgcn_perm(a[3], a[2], 0x07030602u);
+    t[0] = __builtin_amdgcn_perm(p23_lo, p01_lo, 0x05040100u);               // a0.b0 a1.b0 a2.b0 a3.b0
+    t[1] = __builtin_amdgcn_perm(p23_lo, p01_lo, 0x07060302u);
+    t[2] = __builtin_amdgcn_perm(p23_hi, p01_hi, 0x05040100u);
+    t[3] = __builtin_amdgcn_perm(p23_hi, p01_hi, 0x07060302u);
+}
+
+template <int SRC, int FMT, int MODE, bool AMAX, bool WRITE_ROWMAJOR>
+__global__ __launch_bounds__(kThreads) void cast_transpose_kernel(const void *__restrict__ x, int64_t rows, int64_t cols,
+                                                                   const float *__restrict__ scale,
+                                                                   uint8_t *__restrict__ out, uint8_t *__restrict__ out_t,
+                                                                   float *__restrict__ amax_out) {
+    __shared__ __attribute__((aligned(16))) uint8_t tile[kTileC * kLdsPitch];
+    __shared__ uint32_t red[kThreads / kWave];
+    constexpr int ESZ = SRC == ODL_BF16 ? 2 : 4;
+    const int tx = threadIdx.x % 8;                 // 8 lanes across 64 columns
+    const int ty = threadIdx.x / 8;                 // 32 lane-rows, 4 rows each
+    const int64_t tiles_c = (cols + kTileC - 1) / kTileC;
+    const int64_t tr = blockIdx.x / tiles_c, tc = blockIdx.x % tiles_c;
+    const int64_t r0 = tr * kTileR + ty * 4, c0 = tc * kTileC + tx * 8;
+    const bool col_ok = c0 < cols;                  // cols % 8 == 0 (host-checked), so the whole 8-wide patch is in or out
+
+    float s_col[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) s_col[j] = 1.0f;
+    if constexpr (MODE == ODL_SCALE_TENSOR) {
+        const float st = scale[0];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) s_col[j] = st;
+    } else if constexpr (MODE == ODL_SCALE_COL) {
+        if (col_ok) {
+            float4 t0 = *reinterpret_cast<const float4 *>(scale + c0), t1 = *reinterpret_cast<const float4 *>(scale + c0 + 4);
+            s_col[0] = t0.x; s_col[1] = t0.y; s_col[2] = t0.z; s_col[3] = t0.w;
+            s_col[4] = t1.x; s_col[5] = t1.y; s_col[6] = t1.z; s_col[7] = t1.w;
+        }
+    }
+
+    // ---- load the 4 x 8 patch (rows beyond the matrix read as zero)
+    u32x4 raw[4][ESZ / 2];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const bool ok = col_ok && (r0 + i) < rows;
+        const u32x4 *p = reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(x) + ((r0 + i) * cols + c0) * ESZ);
+#pragma unroll
+        for (int h = 0; h < ESZ / 2; ++h) raw[i][h] = ok ? __builtin_nontemporal_load(p + h) : u32x4{0, 0, 0, 0};
+    }
+
+    uint32_t am = 0;
+    uint32_t lo[4], hi[4];                          // codes of columns 0..3 / 4..7 for each of the 4 rows
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        float f[8];
+        if constexpr (SRC == ODL_BF16) {
+            uint32_t w[4] = {raw[i][0].x, raw[i][0].y, raw[i][0].z, raw[i][0].w};
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                f[2 * q] = bf16_lo(w[q]);
+                f[2 * q + 1] = bf16_hi(w[q]);
+                if constexpr (AMAX) am = max_u16x2(am, abs_bf16x2(w[q]));
+            }
+        } else {
+            uint32_t w[8] = {raw[i][0].x, raw[i][0].y, raw[i][0].z, raw[i][0].w, raw[i][1].x, raw[i][1].y, raw[i][1].z, raw[i][1].w};
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                f[q] = bits_to_float(w[q]);
+                if constexpr (AMAX) am = max(am, w[q] & 0x7fffffffu);
+            }
+        }
+        float s[8];
+        if constexpr (MODE == ODL_SCALE_ROW) {
+            const float sr = (r0 + i) < rows ? scale[r0 + i] : 1.0f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) s[j] = sr;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) s[j] = s_col[j];
+        }
+        lo[i] = quantise4<FMT>(f[0], f[1], f[2], f[3], s[0], s[1], s[2], s[3]);
+        hi[i] = quantise4<FMT>(f[4], f[5], f[6], f[7], s[4], s[5], s[6], s[7]);
+        if constexpr (WRITE_ROWMAJOR) {
+            if (col_ok && (r0 + i) < rows)
+                __builtin_nontemporal_store(u32x2{lo[i], hi[i]}, reinterpret_cast<u32x2 *>(out + (r0 + i) * cols + c0));
+        }
+    }
+
+    // ---- transpose in registers, stage through LDS
+    uint32_t tl[4], th[4];
+    transpose4x4(lo, tl);                           // tl[k] = rows r0..r0+3 of column c0+k
+    transpose4x4(hi, th);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        *reinterpret_cast<uint32_t *>(&tile[(tx * 8 + k) * kLdsPitch + ty * 4]) = tl[k];
+        *reinterpret_cast<uint32_t *>(&tile[(tx * 8 + 4 + k) * kLdsPitch + ty * 4]) = th[k];
+    }
+    __syncthreads();
+    // 64 tile-columns x 8 chunks of 16 rows = 512 chunks, two per lane
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+        const int chunk = threadIdx.x + it * kThreads;
+        const int k = chunk / 8, m16 = chunk % 8;
+        const int64_t oc = tc * kTileC + k, orow = tr * kTileR + m16 * 16;
+        if (oc < cols && orow < rows) {             // rows % 16 == 0 (host-checked)
+            const uint32_t *src = reinterpret_cast<const uint32_t *>(&tile[k * kLdsPitch + m16 * 16]);
+            u32x4 v = {src[0], src[1], src[2], src[3]};
+            __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(out_t + oc * rows + orow));
+        }
+    }
+    if constexpr (AMAX) {
+        if constexpr (SRC == ODL_BF16) am = fold_u16x2_to_f32bits(am);
+        am = block_max_u32(am, red);
+        if (threadIdx.x == 0 && am != 0) atomicMax(reinterpret_cast<uint32_t *>(amax_out), am);
+    }
+}
+
+// ----------------------------------------------------------------- host helpers
+static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+static int num_cus() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) cus = prop.multiProcessorCount;
+        if (cus <= 0) cus = 256;
+    }
+    return cus;
+}
+
+static int64_t grid_for(int64_t work_items, int per_block, int blocks_per_cu) {
+    int64_t need = (work_items + per_block - 1) / per_block;
+    int64_t cap = (int64_t)num_cus() * blocks_per_cu;
+    return need < 1 ? 1 : (need < cap ? need : cap);
+}
+
+}  // namespace odl
+
+using namespace odl;
+
+extern "C" int odl_fp8_amax(const void *x, int src_dtype, int64_t rows, int64_t cols, int mode, float *amax_out,
+                            int accumulate, odl_stream_t stream_) {
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    if (!x || !amax_out) return set_error(ODL_ERR_ARG, "odl_fp8_amax: null pointer");
+    if (rows < 0 || cols < 0) return set_error(ODL_ERR_ARG, "odl_fp8_amax: negative shape %lld x %lld", (long long)rows, (long long)cols);
+    if (src_dtype != ODL_BF16 && src_dtype != ODL_F32) return set_error(ODL_ERR_ARG, "odl_fp8_amax: src_dtype %d", src_dtype);
+    if (mode < ODL_SCALE_TENSOR || mode > ODL_SCALE_COL) return set_error(ODL_ERR_ARG, "odl_fp8_amax: mode %d", mode);
+    const int64_t n_out = mode == ODL_SCALE_TENSOR ? 1 : (mode == ODL_SCALE_ROW ? rows : cols);
+    const int64_t n = rows * cols;
+    const bool atomic_path = mode != ODL_SCALE_ROW;
+    if (n_out > 0 && (!accumulate) && (atomic_path || n == 0))
+        hipLaunchKernelGGL(fill_f32_kernel, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, stream, amax_out, n_out, 0.0f);
+    if (n == 0) return check_launch("odl_fp8_amax(fill)");
+    const int esz = src_dtype == ODL_BF16 ? 2 : 4;
+    if (mode == ODL_SCALE_TENSOR) {
+        if (aligned16(x)) {
+            const int64_t g = grid_for(n * esz / 16, kThreads * 4, 8);
+            if (src_dtype == ODL_BF16) hipLaunchKernelGGL((amax_tensor_kernel<ODL_BF16, 4>), dim3((unsigned)g), dim3(kThreads), 0, stream, x, n, amax_out);
+            else hipLaunchKernelGGL((amax_tensor_kernel<ODL_F32, 4>), dim3((unsigned)g), dim3(kThreads), 0, stream, x, n, amax_out);
+        } else {
+            const int64_t g = grid_for(n, kThreads * 8, 8);
+            if (src_dtype == ODL_BF16) hipLaunchKernelGGL((amax_tensor_scalar_kernel<ODL_BF16>), dim3((unsigned)g), dim3(kThreads), 0, stream, x, n, amax_out);
+            else hipLaunchKernelGGL((amax_tensor_scalar_kernel<ODL_F32>), dim3((unsigned)g), dim3(kThreads), 0, stream, x, n, amax_out);
+        }
+    } else if (mode == ODL_SCALE_ROW) {
+        const int64_t g = (rows + (kThreads / kWave) - 1) / (kThreads / kWave);
+        if (g > 0x7fffffffLL) return set_error(ODL_ERR_SHAPE, "odl_fp8_amax: too many rows");
+#define ODL_ROW(SRC) \
+        if (accumulate) hipLaunchKernelGGL((amax_row_kernel<SRC, true>), dim3((unsigned)g), dim3(kThreads), 0, stream, x, rows, cols, amax_out); \
+        else hipLaunchKernelGGL((amax_row_kernel<SRC, false>), dim3((unsigned)g), dim3(kThreads), 0, stream, x, rows, cols, amax_out);
+        if (src_dtype == ODL_BF16) { ODL_ROW(ODL_BF16) } else { ODL_ROW(ODL_F32) }
+#undef ODL_ROW
+    } else {
+        const int cpl = 16 / esz, cw = 32 * cpl;
+        // enough row-slabs for ~8 blocks per CU, each at least 64 rows tall
+        int64_t col_blocks = (cols + cw - 1) / cw;
+        int64_t want_slabs = ((int64_t)num_cus() * 8 + col_blocks - 1) / col_blocks;
+        int64_t rpb = (rows + want_slabs - 1) / want_slabs;
+        rpb = ((rpb + 31) / 32) * 32;
+        if (rpb < 64) rpb = 64;
+        const int64_t slabs = (rows + rpb - 1) / rpb;
+        if (slabs > 65535) return set_error(ODL_ERR_SHAPE, "odl_fp8_amax: too many row slabs");
+        if (aligned16(x) && cols % cpl == 0) {
+            if (src_dtype == ODL_BF16) hipLaunchKernelGGL((amax_col_kernel<ODL_BF16>), dim3((unsigned)col_blocks, (unsigned)slabs), dim3(kThreads), 0, stream, x, rows, cols, (int)rpb, amax_out);
+            else hipLaunchKernelGGL((amax_col_kernel<ODL_F32>), dim3((unsigned)col_blocks, (unsigned)slabs), dim3(kThreads), 0, stream, x, rows, cols, (int)rpb, amax_out);
+        } else {
+            const int64_t gx = (cols + 255) / 256;
+            if (src_dtype == ODL_BF16) hipLaunchKernelGGL((amax_col_scalar_kernel<ODL_BF16>), dim3((unsigned)gx, (unsigned)slabs), dim3(256), 0, stream, x, rows, cols, (int)rpb, amax_out);
+            else hipLaunchKernelGGL((amax_col_scalar_kernel<ODL_F32>), dim3((unsigned)gx, (unsigned)slabs), dim3(256), 0, stream, x, rows, cols, (int)rpb, amax_out);
+        }
+    }
+    return check_launch("odl_fp8_amax");
+}
+
+extern "C" int odl_fp8_scale_from_amax(const float *amax, int64_t n, int fmt, int margin, float *scale, float *scale_inv,
+                                       odl_stream_t stream_) {
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    if (!amax || !scale) return set_error(ODL_ERR_ARG, "odl_fp8_scale_from_amax: null pointer");
+    if (fmt != ODL_FP8_E4M3 && fmt != ODL_FP8_E5M2) return set_error(ODL_ERR_ARG, "odl_fp8_scale_from_amax: fmt %d", fmt);
+    if (n < 0) return set_error(ODL_ERR_ARG, "odl_fp8_scale_from_amax: n < 0");
+    if (n == 0) return ODL_OK;
+    hipLaunchKernelGGL(scale_from_amax_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, amax, n,
+                       fmt == ODL_FP8_E5M2 ? 57344.0f : 448.0f, margin, scale, scale_inv);
+    return check_launch("odl_fp8_scale_from_amax");
+}
+
+extern "C" int odl_fp8_delayed_update(float *history, int64_t H, int64_t R, float *scale, float *scale_inv, const int *fmt,
+                                      int margin, int algo, odl_stream_t stream_) {
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    if (!history || !scale || !scale_inv || !fmt) return set_error(ODL_ERR_ARG, "odl_fp8_delayed_update: null pointer");
+    if (H < 1 || R < 0) return set_error(ODL_ERR_ARG, "odl_fp8_delayed_update: H=%lld R=%lld", (long long)H, (long long)R);
+    if (algo != ODL_AMAX_MAX && algo != ODL_AMAX_MOST_RECENT) return set_error(ODL_ERR_ARG, "odl_fp8_delayed_update: algo %d", algo);
+    if (R == 0) return ODL_OK;
+    hipLaunchKernelGGL(delayed_update_kernel, dim3((unsigned)((R + 63) / 64)), dim3(64), 0, stream, history, H, R, scale,
+                       scale_inv, fmt, margin, algo);
+    return check_launch("odl_fp8_delayed_update");
+}
+
+namespace odl {
+
+template <int SRC, int FMT, int MODE>
+static void launch_cast(const void *x, int64_t rows, int64_t cols, const float *scale, uint8_t *out, float *amax_out,
+                        hipStream_t stream) {
+    const int64_t g = grid_for(rows * cols / 16, kThreads, 16);
+    if (amax_out) hipLaunchKernelGGL((cast_kernel<SRC, FMT, MODE, true>), dim3((unsigned)g), dim3(kThreads), 0, stream, x, rows, cols, scale, out, amax_out);
+    else hipLaunchKernelGGL((cast_kernel<SRC, FMT, MODE, false>), dim3((unsigned)g), dim3(kThreads), 0, stream, x, rows, cols, scale, out, amax_out);
+}
+
+template <int SRC, int FMT>
+static void launch_cast_mode(int mode, const void *x, int64_t rows, int64_t cols, const float *scale, uint8_t *out,
+                             float *amax_out, hipStream_t stream) {
+    if (mode == ODL_SCALE_TENSOR) launch_cast<SRC, FMT, ODL_SCALE_TENSOR>(x, rows, cols, scale, out, amax_out, stream);
+    else if (mode == ODL_SCALE_ROW) launch_cast<SRC, FMT, ODL_SCALE_ROW>(x, rows, cols, scale, out, amax_out, stream);
+    else launch_cast<SRC, FMT, ODL_SCALE_COL>(x, rows, cols, scale, out, amax_out, stream);
+}
+
+template <int SRC, int FMT>
+static void launch_generic(const void *x, int64_t rows, int64_t cols, const float *scale, int mode, uint8_t *out,
+                           uint8_t *out_t, float *amax_out, hipStream_t stream) {
+    const int64_t g = grid_for(rows * cols, kThreads * 4, 8);
+    hipLaunchKernelGGL((cast_generic_kernel<SRC, FMT>), dim3((unsigned)g), dim3(kThreads), 0, stream, x, rows, cols, scale, mode, out, out_t, amax_out);
+}
+
+template <int SRC, int FMT, int MODE>
+static void launch_ct(const void *x, int64_t rows, int64_t cols, const float *scale, uint8_t *out, uint8_t *out_t,
+                      float *amax_out, hipStream_t stream) {
+    const int64_t g = ((rows + kTileR - 1) / kTileR) * ((cols + kTileC - 1) / kTileC);
+#define ODL_CT(AM, RM) hipLaunchKernelGGL((cast_transpose_kernel<SRC, FMT, MODE, AM, RM>), dim3((unsigned)g), dim3(kThreads), 0, stream, x, rows, cols, scale, out, out_t, amax_out)
+    if (amax_out) { if (out) ODL_CT(true, true); else ODL_CT(true, false); }
+    else { if (out) ODL_CT(false, true); else ODL_CT(false, false); }
+#undef ODL_CT
+}
+
+template <int SRC, int FMT>
+static void launch_ct_mode(int mode, const void *x, int64_t rows, int64_t cols, const float *scale, uint8_t *out,
+                           uint8_t *out_t, float *amax_out, hipStream_t stream) {
+    if (mode == ODL_SCALE_TENSOR) launch_ct<SRC, FMT, ODL_SCALE_TENSOR>(x, rows, cols, scale, out, out_t, amax_out, stream);
+    else if (mode == ODL_SCALE_ROW) launch_ct<SRC, FMT, ODL_SCALE_ROW>(x, rows, cols, scale, out, out_t, amax_out, stream);
+    else launch_ct<SRC, FMT, ODL_SCALE_COL>(x, rows, cols, scale, out, out_t, amax_out, stream);
+}
+
+static int check_cast_args(const char *who, const void *x, int src_dtype, int64_t rows, int64_t cols, const float *scale,
+                           int mode, int fmt) {
+    if (!x || !scale) return set_error(ODL_ERR_ARG, "%s: null pointer", who);
+    if (rows < 0 || cols < 0) return set_error(ODL_ERR_ARG, "%s: negative shape", who);
+    if (src_dtype != ODL_BF16 && src_dtype != ODL_F32) return set_error(ODL_ERR_ARG, "%s: src_dtype %d", who, src_dtype);
+    if (mode < ODL_SCALE_TENSOR || mode > ODL_SCALE_COL) return set_error(ODL_ERR_ARG, "%s: mode %d", who, mode);
+    if (fmt != ODL_FP8_E4M3 && fmt != ODL_FP8_E5M2) return set_error(ODL_ERR_ARG, "%s: fmt %d", who, fmt);
+    return ODL_OK;
+}
+
+}  // namespace odl
+
+#define ODL_DISPATCH_SRC_FMT(FN, ...)                                             \
+    do {                                                                          \
+        if (src_dtype == ODL_BF16) {                                              \
+            if (fmt == ODL_FP8_E4M3) FN<ODL_BF16, ODL_FP8_E4M3>(__VA_ARGS__);     \
+            else FN<ODL_BF16, ODL_FP8_E5M2>(__VA_ARGS__);                         \
+        } else {                                                                  \
+            if (fmt == ODL_FP8_E4M3) FN<ODL_F32, ODL_FP8_E4M3>(__VA_ARGS__);      \
+            else FN<ODL_F32, ODL_FP8_E5M2>(__VA_ARGS__);                          \
+        }                                                                         \
+    } while (0)
+
+extern "C" int odl_fp8_cast(const void *x, int src_dtype, int64_t rows, int64_t cols, const float *scale, int mode, int fmt,
+                            uint8_t *out, float *amax_out, odl_stream_t stream_) {
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    if (int e = check_cast_args("odl_fp8_cast", x, src_dtype, rows, cols, scale, mode, fmt)) return e;
+    if (!out) return set_error(ODL_ERR_ARG, "odl_fp8_cast: out is null");
+    if (rows * cols == 0) return ODL_OK;
+    const bool fast = cols % 16 == 0 && aligned16(x) && aligned16(out) && (mode != ODL_SCALE_COL || aligned16(scale));
+    if (fast) ODL_DISPATCH_SRC_FMT(launch_cast_mode, mode, x, rows, cols, scale, out, amax_out, stream);
+    else ODL_DISPATCH_SRC_FMT(launch_generic, x, rows, cols, scale, mode, out, (uint8_t *)nullptr, amax_out, stream);
+    return check_launch("odl_fp8_cast");
+}
+
+extern "C" int odl_fp8_cast_transpose(const void *x, int src_dtype, int64_t rows, int64_t cols, const float *scale, int mode,
+                                      int fmt, uint8_t *out, uint8_t *out_t, float *amax_out, odl_stream_t stream_) {
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    if (int e = check_cast_args("odl_fp8_cast_transpose", x, src_dtype, rows, cols, scale, mode, fmt)) return e;
+    if (!out_t) return set_error(ODL_ERR_ARG, "odl_fp8_cast_transpose: out_t is null");
+    if (rows * cols == 0) return ODL_OK;
+    const int64_t tiles = ((rows + kTileR - 1) / kTileR) * ((cols + kTileC - 1) / kTileC);
+    const bool fast = cols % 8 == 0 && rows % 16 == 0 && aligned16(x) && aligned16(out_t) &&
+                      (!out || (reinterpret_cast<uintptr_t>(out) & 7) == 0) &&
+                      (mode != ODL_SCALE_COL || aligned16(scale)) && tiles <= 0x7fffffffLL;
+    if (fast) ODL_DISPATCH_SRC_FMT(launch_ct_mode, mode, x, rows, cols, scale, out, out_t, amax_out, stream);
+    else ODL_DISPATCH_SRC_FMT(launch_generic, x, rows, cols, scale, mode, out, out_t, amax_out, stream);
+    return check_launch("odl_fp8_cast_transpose");
+}

@@ -1,0 +1,238 @@
+"""ctypes binding of ``libodl_fp8.so`` (the C ABI declared in include/odl_fp8.h).
+
+The library is the product: there is no eager / CPU fallback behind these
+functions.  If the shared object is missing or a call is refused, the caller
+gets an exception.
+
+Tensors are passed as raw device pointers together with torch's current HIP
+stream, so every kernel is ordered with the surrounding torch work and nothing
+synchronises with the host.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+
+import torch
+
+E4M3, E5M2 = 0, 1
+SCALE_TENSOR, SCALE_ROW, SCALE_COL = 0, 1, 2
+DT_BF16, DT_F32 = 0, 1
+AMAX_MAX, AMAX_MOST_RECENT = 0, 1
+FP8_MAX = {E4M3: 448.0, E5M2: 57344.0}
+TORCH_FP8 = {E4M3: torch.float8_e4m3fn, E5M2: torch.float8_e5m2}
+ABI_VERSION = 1
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libodl_fp8.so")
+
+EXPORTS = (
+    "odl_fp8_abi_version",
+    "odl_fp8_last_error",
+    "odl_fp8_amax",
+    "odl_fp8_scale_from_amax",
+    "odl_fp8_cast",
+    "odl_fp8_cast_transpose",
+    "odl_fp8_gemm_nt",
+    "odl_fp8_delayed_update",
+    "odl_fp8_gemm_num_variants",
+    "odl_fp8_gemm_variant_name",
+    "odl_fp8_gemm_set_variant",
+)
+
+_lib = None
+_lock = threading.Lock()
+
+
+class NativeError(RuntimeError):
+    """Raised when the native library is missing or refuses a call."""
+
+
+def is_built() -> bool:
+    return os.path.exists(LIB_PATH)
+
+
+def load() -> ctypes.CDLL:
+    """Load the library once (torch is imported first so that its HIP runtime,
+    which has the same SONAME, is the one the library binds to)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        if not is_built():
+            raise NativeError(
+                f"{LIB_PATH} is missing: build it with `python -m optimus_dl_amd.build` "
+                "(hipcc, gfx950). There is no fallback path."
+            )
+        L = ctypes.CDLL(LIB_PATH)
+        vp, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+        L.odl_fp8_abi_version.restype = i32
+        L.odl_fp8_last_error.restype = ctypes.c_char_p
+        L.odl_fp8_amax.argtypes = [vp, i32, i64, i64, i32, vp, i32, vp]
+        L.odl_fp8_scale_from_amax.argtypes = [vp, i64, i32, i32, vp, vp, vp]
+        L.odl_fp8_cast.argtypes = [vp, i32, i64, i64, vp, i32, i32, vp, vp, vp]
+        L.odl_fp8_cast_transpose.argtypes = [vp, i32, i64, i64, vp, i32, i32, vp, vp, vp, vp]
+        L.odl_fp8_gemm_nt.argtypes = [vp, vp, i64, i64, i64, i32, i32, vp, i64, vp, i64, vp, i32, vp, i32, vp]
+        L.odl_fp8_delayed_update.argtypes = [vp, i64, i64, vp, vp, vp, i32, i32, vp]
+        L.odl_fp8_gemm_num_variants.restype = i32
+        L.odl_fp8_gemm_variant_name.argtypes = [i32]
+        L.odl_fp8_gemm_variant_name.restype = ctypes.c_char_p
+        L.odl_fp8_gemm_set_variant.argtypes = [i32]
+        for name in EXPORTS:
+            getattr(L, name)  # AttributeError here = the library does not match the header
+        if L.odl_fp8_abi_version() != ABI_VERSION:
+            raise NativeError(f"{LIB_PATH}: ABI {L.odl_fp8_abi_version()} != expected {ABI_VERSION}; rebuild")
+        _lib = L
+    return _lib
+
+
+def _check(status: int, what: str) -> None:
+    if status != 0:
+        msg = load().odl_fp8_last_error().decode(errors="replace")
+        raise NativeError(f"{what} refused (status {status}): {msg}")
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _src_dtype(x: torch.Tensor) -> int:
+    if x.dtype == torch.bfloat16:
+        return DT_BF16
+    if x.dtype == torch.float32:
+        return DT_F32
+    raise NativeError(f"source dtype {x.dtype} is not supported (bf16 or fp32)")
+
+
+def _as_2d(x: torch.Tensor) -> torch.Tensor:
+    if not x.is_cuda:
+        raise NativeError("the FP8 kernels run on the GPU only; got a tensor on " + str(x.device))
+    if x.dim() != 2:
+        raise NativeError(f"expected a 2-D tensor, got shape {tuple(x.shape)}")
+    return x if x.is_contiguous() else x.contiguous()
+
+
+def _f32_dev(t: torch.Tensor, n: int, what: str) -> torch.Tensor:
+    if not (t.is_cuda and t.dtype == torch.float32 and t.is_contiguous() and t.numel() == n):
+        raise NativeError(f"{what}: need a contiguous fp32 CUDA tensor with {n} element(s), got "
+                          f"{t.dtype} {tuple(t.shape)} on {t.device}")
+    return t
+
+
+def _n_scales(mode: int, rows: int, cols: int) -> int:
+    return 1 if mode == SCALE_TENSOR else (rows if mode == SCALE_ROW else cols)
+
+
+# ------------------------------------------------------------------ operations
+def amax(x: torch.Tensor, mode: int = SCALE_TENSOR, out: torch.Tensor | None = None,
+         accumulate: bool = False) -> torch.Tensor:
+    x = _as_2d(x)
+    rows, cols = x.shape
+    n = _n_scales(mode, rows, cols)
+    if out is None:
+        if accumulate:
+            raise NativeError("amax(accumulate=True) needs an `out` tensor to fold into")
+        out = torch.empty(n, dtype=torch.float32, device=x.device)
+    _f32_dev(out, n, "amax out")
+    _check(load().odl_fp8_amax(x.data_ptr(), _src_dtype(x), rows, cols, mode, out.data_ptr(), int(accumulate), _stream()),
+           "odl_fp8_amax")
+    return out
+
+
+def scale_from_amax(amax_t: torch.Tensor, fmt: int, margin: int = 0):
+    n = amax_t.numel()
+    _f32_dev(amax_t, n, "scale_from_amax amax")
+    scale = torch.empty_like(amax_t)
+    scale_inv = torch.empty_like(amax_t)
+    _check(load().odl_fp8_scale_from_amax(amax_t.data_ptr(), n, fmt, margin, scale.data_ptr(), scale_inv.data_ptr(), _stream()),
+           "odl_fp8_scale_from_amax")
+    return scale, scale_inv
+
+
+def cast(x: torch.Tensor, scale: torch.Tensor, fmt: int, mode: int = SCALE_TENSOR,
+         amax_out: torch.Tensor | None = None, out: torch.Tensor | None = None) -> torch.Tensor:
+    x = _as_2d(x)
+    rows, cols = x.shape
+    _f32_dev(scale, _n_scales(mode, rows, cols), "cast scale")
+    if out is None:
+        out = torch.empty((rows, cols), dtype=torch.uint8, device=x.device)
+    if amax_out is not None:
+        _f32_dev(amax_out, 1, "cast amax_out")
+    _check(load().odl_fp8_cast(x.data_ptr(), _src_dtype(x), rows, cols, scale.data_ptr(), mode, fmt, out.data_ptr(),
+                               amax_out.data_ptr() if amax_out is not None else None, _stream()), "odl_fp8_cast")
+    return out
+
+
+def cast_transpose(x: torch.Tensor, scale: torch.Tensor, fmt: int, mode: int = SCALE_TENSOR,
+                   amax_out: torch.Tensor | None = None, want_rowmajor: bool = True):
+    """Returns (codes[rows, cols] or None, codes_t[cols, rows])."""
+    x = _as_2d(x)
+    rows, cols = x.shape
+    _f32_dev(scale, _n_scales(mode, rows, cols), "cast_transpose scale")
+    out = torch.empty((rows, cols), dtype=torch.uint8, device=x.device) if want_rowmajor else None
+    out_t = torch.empty((cols, rows), dtype=torch.uint8, device=x.device)
+    if amax_out is not None:
+        _f32_dev(amax_out, 1, "cast_transpose amax_out")
+    _check(load().odl_fp8_cast_transpose(x.data_ptr(), _src_dtype(x), rows, cols, scale.data_ptr(), mode, fmt,
+                                         out.data_ptr() if out is not None else None, out_t.data_ptr(),
+                                         amax_out.data_ptr() if amax_out is not None else None, _stream()),
+           "odl_fp8_cast_transpose")
+    return out, out_t
+
+
+def gemm_nt(a: torch.Tensor, b: torch.Tensor, fmt_a: int, fmt_b: int, sa_inv: torch.Tensor, sb_inv: torch.Tensor,
+            bias: torch.Tensor | None = None, out_dtype: torch.dtype = torch.bfloat16,
+            out: torch.Tensor | None = None) -> torch.Tensor:
+    """out[M,N] = (a[M,K] . b[N,K]^T) * (sa_inv x sb_inv) (+ bias); a, b uint8 FP8 codes."""
+    if a.dtype != torch.uint8 or b.dtype != torch.uint8:
+        raise NativeError("gemm_nt operands must be uint8 FP8 codes")
+    a, b = _as_2d(a), _as_2d(b)
+    M, K = a.shape
+    N, K2 = b.shape
+    if K != K2:
+        raise NativeError(f"gemm_nt: contraction sizes differ ({K} vs {K2})")
+    if sa_inv.numel() not in (1, M) or sb_inv.numel() not in (1, N):
+        raise NativeError(f"gemm_nt: scale vectors must have 1 or M / N entries, got {sa_inv.numel()}, {sb_inv.numel()}")
+    _f32_dev(sa_inv, sa_inv.numel(), "gemm_nt sa_inv")
+    _f32_dev(sb_inv, sb_inv.numel(), "gemm_nt sb_inv")
+    if bias is not None:
+        _f32_dev(bias, N, "gemm_nt bias")
+    odt = DT_BF16 if out_dtype == torch.bfloat16 else (DT_F32 if out_dtype == torch.float32 else None)
+    if odt is None:
+        raise NativeError(f"gemm_nt: output dtype {out_dtype} is not supported (bf16 or fp32)")
+    if out is None:
+        out = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    elif out.shape != (M, N) or out.dtype != out_dtype or not out.is_contiguous():
+        raise NativeError("gemm_nt: `out` has the wrong shape / dtype / layout")
+    _check(load().odl_fp8_gemm_nt(a.data_ptr(), b.data_ptr(), M, N, K, fmt_a, fmt_b, sa_inv.data_ptr(), sa_inv.numel(),
+                                  sb_inv.data_ptr(), sb_inv.numel(), bias.data_ptr() if bias is not None else None,
+                                  DT_F32, out.data_ptr(), odt, _stream()), "odl_fp8_gemm_nt")
+    return out
+
+
+def delayed_update(history: torch.Tensor, scale: torch.Tensor, scale_inv: torch.Tensor, fmts: torch.Tensor,
+                   margin: int = 0, algo: int = AMAX_MAX) -> None:
+    """In place: history[H,R] fp32, scale[R], scale_inv[R] fp32, fmts[R] int32 (all on the GPU)."""
+    if history.dim() != 2:
+        raise NativeError("delayed_update: history must be [H, R]")
+    H, R = history.shape
+    _f32_dev(history, H * R, "delayed_update history")
+    _f32_dev(scale, R, "delayed_update scale")
+    _f32_dev(scale_inv, R, "delayed_update scale_inv")
+    if not (fmts.is_cuda and fmts.dtype == torch.int32 and fmts.numel() == R and fmts.is_contiguous()):
+        raise NativeError("delayed_update: fmts must be a contiguous int32 CUDA tensor with R entries")
+    _check(load().odl_fp8_delayed_update(history.data_ptr(), H, R, scale.data_ptr(), scale_inv.data_ptr(), fmts.data_ptr(),
+                                         margin, algo, _stream()), "odl_fp8_delayed_update")
+
+
+def gemm_variants() -> list[str]:
+    L = load()
+    return [L.odl_fp8_gemm_variant_name(i).decode() for i in range(L.odl_fp8_gemm_num_variants())]
+
+
+def gemm_set_variant(variant: int) -> None:
+    _check(load().odl_fp8_gemm_set_variant(variant), "odl_fp8_gemm_set_variant")

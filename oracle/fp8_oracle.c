@@ -1,0 +1,260 @@
+/*
+ * CPU oracle for the FP8 Linear path.  TEST INFRASTRUCTURE ONLY: nothing in the
+ * shipped package may include, link or call this file; it exists so that the
+ * HIP kernels can be checked against an independent, plain-C restatement.
+ *
+ * What it restates.  The reference repository holds no FP8 arithmetic of its
+ * own: optimus_dl/modules/model_transforms/transformer_engine.py:97-108 and
+ * optimus_dl/modules/amp/fp8.py:254-306,337-340 forward everything to NVIDIA
+ * Transformer Engine (pyproject.toml:80-82, pinned 2.15.0 in uv.lock:5728-5757,
+ * not vendored).  The arithmetic below therefore follows the published
+ * definitions that library implements:
+ *   - OCP 8-bit floating point (E4M3 "fn" flavour, E5M2), round to nearest even
+ *   - amax = max |x|; scale = fp8_max / amax / 2^margin (IEEE fp32 division)
+ *   - cast = rne( clamp( fp32(x) * scale, +-fp8_max ) )
+ *   - emulated GEMM: upcast the 8-bit codes to fp32, accumulate in fp32,
+ *     multiply by the product of the inverse scales, round to bf16
+ *   - delayed scaling: amax history ring, scale refreshed from max / most recent
+ *
+ * How each function is pinned (see tests/test_oracle_*.py):
+ *   encode/decode : 256-entry decode tables from the format definition;
+ *                   nearest-value brute force in float64; torch CPU
+ *                   Tensor.to(float8_*) as the library routine (all bf16
+ *                   patterns and a strided sweep of all fp32 exponents)
+ *   amax / scale  : closed forms (max, IEEE division) against numpy/torch
+ *   cast          : composition of the two above, against torch CPU
+ *   cast_transpose: byte identity with cast followed by a transpose
+ *   gemm          : float64 brute force on tiny shapes, exact special cases
+ *                   (one-hot and power-of-two operands), torch._scaled_mm
+ *   delayed update: hand-worked ring-buffer sequences and window properties.
+ *                   The roll/update ORDER follows the documented behaviour of
+ *                   the third-party library and cannot be checked against it
+ *                   offline: parity unpinned for that ordering.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <string.h>
+#include <float.h>
+
+#define ORACLE_API __attribute__((visibility("default")))
+
+enum { FMT_E4M3 = 0, FMT_E5M2 = 1 };
+enum { SCALE_TENSOR = 0, SCALE_ROW = 1, SCALE_COL = 2 };
+
+static inline uint32_t f32_bits(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+static inline float bits_f32(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+static inline float bf16_to_f32(uint16_t h) { return bits_f32((uint32_t)h << 16); }
+
+/* fp32 -> bf16, round to nearest even, NaN kept quiet (what torch does). */
+static inline uint16_t f32_to_bf16(float f) {
+    uint32_t u = f32_bits(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
+    uint32_t lsb = (u >> 16) & 1u;
+    u += 0x7fffu + lsb;
+    return (uint16_t)(u >> 16);
+}
+
+/*
+ * Generic IEEE-style narrowing of an fp32 bit pattern to an 8-bit float with
+ * `mbits` mantissa bits and exponent bias `bias`, round to nearest even, done
+ * in integer arithmetic.  Returns the magnitude code WITHOUT overflow handling
+ * (the caller maps too-large codes to NaN / Inf as the format demands).
+ */
+static uint32_t narrow_magnitude(uint32_t abs_bits, int mbits, int bias) {
+    int e = (int)(abs_bits >> 23);
+    uint32_t m = abs_bits & 0x7fffffu;
+    if (e == 0) return 0;                       /* fp32 subnormal: far below any fp8 subnormal */
+    int E = e - 127 + bias;                     /* biased target exponent */
+    uint32_t full = m | 0x800000u;              /* 24-bit significand, value = full * 2^(e-150) */
+    int shift = 23 - mbits;                     /* bits dropped for a normal result */
+    uint32_t base;
+    if (E >= 1) {
+        base = ((uint32_t)E << mbits) | (m >> shift);
+        full = m;                               /* remainder comes from the fraction only */
+    } else {
+        shift += 1 - E;                         /* subnormal target: drop more bits */
+        if (shift > 25) return 0;               /* less than half of the smallest subnormal */
+        base = full >> shift;                   /* shift <= 25 keeps this well defined */
+    }
+    uint32_t rem  = full & ((1u << shift) - 1u);
+    uint32_t half = 1u << (shift - 1);
+    if (rem > half || (rem == half && (base & 1u))) base += 1;  /* carry may bump the exponent: intended */
+    return base;
+}
+
+/* OCP E4M3 (finite-only "fn"): bias 7, max 448 = 0x7E, 0x7F = NaN, no Inf.
+ * Non-saturating: anything that rounds past 448 becomes NaN (torch CPU cast). */
+ORACLE_API uint8_t oracle_f32_to_e4m3(float f) {
+    uint32_t u = f32_bits(f);
+    uint8_t sign = (uint8_t)((u >> 24) & 0x80u);
+    uint32_t a = u & 0x7fffffffu;
+    if (a >= 0x7f800000u) return sign | 0x7f;             /* Inf and NaN */
+    uint32_t c = narrow_magnitude(a, 3, 7);
+    if (c >= 0x7f) c = 0x7f;
+    return sign | (uint8_t)c;
+}
+
+/* OCP E5M2: bias 15, max 57344 = 0x7B, 0x7C = Inf, 0x7D..0x7F = NaN.
+ * Non-saturating: overflow goes to Inf.  NaN maps to 0x7F (torch CPU cast). */
+ORACLE_API uint8_t oracle_f32_to_e5m2(float f) {
+    uint32_t u = f32_bits(f);
+    uint8_t sign = (uint8_t)((u >> 24) & 0x80u);
+    uint32_t a = u & 0x7fffffffu;
+    if (a > 0x7f800000u) return sign | 0x7f;
+    if (a == 0x7f800000u) return sign | 0x7c;
+    uint32_t c = narrow_magnitude(a, 2, 15);
+    if (c >= 0x7c) c = 0x7c;
+    return sign | (uint8_t)c;
+}
+
+ORACLE_API float oracle_e4m3_to_f32(uint8_t c) {
+    int e = (c >> 3) & 0xf, m = c & 7;
+    float v;
+    if (e == 0xf && m == 7) v = NAN;
+    else if (e == 0) v = ldexpf((float)m, -9);             /* m/8 * 2^-6 */
+    else v = ldexpf(1.0f + (float)m / 8.0f, e - 7);
+    return (c & 0x80) ? -v : v;
+}
+
+ORACLE_API float oracle_e5m2_to_f32(uint8_t c) {
+    int e = (c >> 2) & 0x1f, m = c & 3;
+    float v;
+    if (e == 0x1f) v = m ? NAN : INFINITY;
+    else if (e == 0) v = ldexpf((float)m, -16);            /* m/4 * 2^-14 */
+    else v = ldexpf(1.0f + (float)m / 4.0f, e - 15);
+    return (c & 0x80) ? -v : v;
+}
+
+static inline float fp8_max_of(int fmt) { return fmt == FMT_E5M2 ? 57344.0f : 448.0f; }
+static inline uint8_t encode(float v, int fmt) {
+    return fmt == FMT_E5M2 ? oracle_f32_to_e5m2(v) : oracle_f32_to_e4m3(v);
+}
+static inline float decode(uint8_t c, int fmt) {
+    return fmt == FMT_E5M2 ? oracle_e5m2_to_f32(c) : oracle_e4m3_to_f32(c);
+}
+
+ORACLE_API void oracle_encode_f32(const float *x, int64_t n, int fmt, uint8_t *out) {
+    for (int64_t i = 0; i < n; ++i) out[i] = encode(x[i], fmt);
+}
+ORACLE_API void oracle_decode(const uint8_t *c, int64_t n, int fmt, float *out) {
+    for (int64_t i = 0; i < n; ++i) out[i] = decode(c[i], fmt);
+}
+
+/* max that propagates NaN, like torch.amax. */
+static inline float nanmax(float a, float b) {
+    if (a != a) return a;
+    if (b != b) return b;
+    return a > b ? a : b;
+}
+
+/* amax over a bf16 matrix [rows, cols] (row-major).
+ * mode SCALE_TENSOR -> out[1], SCALE_ROW -> out[rows], SCALE_COL -> out[cols]. */
+ORACLE_API void oracle_amax_bf16(const uint16_t *x, int64_t rows, int64_t cols, int mode, float *out) {
+    int64_t n_out = mode == SCALE_TENSOR ? 1 : (mode == SCALE_ROW ? rows : cols);
+    for (int64_t i = 0; i < n_out; ++i) out[i] = 0.0f;
+    for (int64_t r = 0; r < rows; ++r)
+        for (int64_t c = 0; c < cols; ++c) {
+            float a = fabsf(bf16_to_f32(x[r * cols + c]));
+            int64_t o = mode == SCALE_TENSOR ? 0 : (mode == SCALE_ROW ? r : c);
+            out[o] = nanmax(out[o], a);
+        }
+}
+
+/* scale = fp8_max / amax / 2^margin as IEEE fp32; `fallback` when amax is not a
+ * positive finite number; an infinite quotient is replaced by FLT_MAX. */
+ORACLE_API float oracle_scale(float amax, int fmt, int margin, float fallback) {
+    if (!(amax > 0.0f) || isinf(amax)) return fallback;      /* catches NaN, 0, negatives, Inf */
+    volatile float s = fp8_max_of(fmt) / amax;               /* volatile: no excess precision */
+    s = ldexpf(s, -margin);
+    if (isinf(s)) s = FLT_MAX;
+    return s;
+}
+
+ORACLE_API float oracle_scale_inv(float scale) {
+    volatile float r = 1.0f / scale;
+    return r;
+}
+
+static inline uint8_t quantise(uint16_t xb, float scale, int fmt) {
+    float x = bf16_to_f32(xb);
+    if (x != x) return (uint8_t)(((xb >> 8) & 0x80u) | 0x7fu);
+    volatile float y = x * scale;                            /* one fp32 multiply */
+    float m = fp8_max_of(fmt), v = y;
+    if (v > m) v = m;
+    if (v < -m) v = -m;
+    if (v != v) return (uint8_t)(((xb >> 8) & 0x80u) | 0x7fu);  /* 0*inf cannot occur (scale finite) */
+    return encode(v, fmt);
+}
+
+/* cast of a bf16 matrix with per-tensor / per-row / per-column scale. */
+ORACLE_API void oracle_cast_bf16(const uint16_t *x, int64_t rows, int64_t cols, const float *scale,
+                                 int mode, int fmt, uint8_t *out) {
+    for (int64_t r = 0; r < rows; ++r)
+        for (int64_t c = 0; c < cols; ++c) {
+            float s = mode == SCALE_TENSOR ? scale[0] : (mode == SCALE_ROW ? scale[r] : scale[c]);
+            out[r * cols + c] = quantise(x[r * cols + c], s, fmt);
+        }
+}
+
+/* out_t[c, r] = cast(x)[r, c]  (the copy wgrad/dgrad contract over) */
+ORACLE_API void oracle_cast_transpose_bf16(const uint16_t *x, int64_t rows, int64_t cols, const float *scale,
+                                           int mode, int fmt, uint8_t *out, uint8_t *out_t) {
+    for (int64_t r = 0; r < rows; ++r)
+        for (int64_t c = 0; c < cols; ++c) {
+            float s = mode == SCALE_TENSOR ? scale[0] : (mode == SCALE_ROW ? scale[r] : scale[c]);
+            uint8_t q = quantise(x[r * cols + c], s, fmt);
+            if (out) out[r * cols + c] = q;
+            out_t[c * rows + r] = q;
+        }
+}
+
+/*
+ * Emulated FP8 GEMM, "NT": C[M,N] = A[M,K] * B[N,K]^T, operands are 8-bit codes.
+ * fp32 accumulate over k in ascending order; epilogue multiplies by
+ * (sa_inv * sb_inv) with sa_inv scalar (sa_n == 1) or per-row of A (sa_n == M),
+ * sb_inv scalar or per-row of B (sb_n == N); then rounds to bf16.
+ * If c_f32 is not NULL the un-rounded fp32 result is stored there as well.
+ */
+ORACLE_API void oracle_gemm_nt(const uint8_t *a, const uint8_t *b, int64_t M, int64_t N, int64_t K,
+                               int fmt_a, int fmt_b, const float *sa_inv, int64_t sa_n,
+                               const float *sb_inv, int64_t sb_n, uint16_t *c_bf16, float *c_f32) {
+    float lut_a[256], lut_b[256];
+    for (int i = 0; i < 256; ++i) { lut_a[i] = decode((uint8_t)i, fmt_a); lut_b[i] = decode((uint8_t)i, fmt_b); }
+    /* built with -ffp-contract=off; the product of two 8-bit floats is exact in
+     * fp32 (at most 8 significant bits), so only the additions round */
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < M; ++i)
+        for (int64_t j = 0; j < N; ++j) {
+            float acc = 0.0f;
+            for (int64_t k = 0; k < K; ++k) acc += lut_a[a[i * K + k]] * lut_b[b[j * K + k]];
+            volatile float s = (sa_n == 1 ? sa_inv[0] : sa_inv[i]) * (sb_n == 1 ? sb_inv[0] : sb_inv[j]);
+            volatile float v = acc * s;
+            if (c_f32) c_f32[i * N + j] = v;
+            if (c_bf16) c_bf16[i * N + j] = f32_to_bf16(v);
+        }
+}
+
+/*
+ * Delayed-scaling bookkeeping for R roles with a history of H steps each,
+ * history stored [H, R] row-major with row 0 = the newest amax (written by the
+ * cast kernels of the step that just ran).
+ *   a      = max over the column (algo 0, "max") or history[0] (algo 1, "most_recent")
+ *   roll   : history <- roll(history, -1 along H); history[0] <- 0
+ *   scale  = fp8_max/a/2^margin, unchanged when a is 0 / NaN / Inf; Inf -> FLT_MAX
+ *   scale_inv = 1/scale
+ */
+ORACLE_API void oracle_delayed_update(float *history, int64_t H, int64_t R, float *scale, float *scale_inv,
+                                      const int *fmt, int margin, int algo) {
+    for (int64_t r = 0; r < R; ++r) {
+        float a = history[r];
+        if (algo == 0)
+            for (int64_t h = 1; h < H; ++h) a = nanmax(a, history[h * R + r]);
+        /* roll by -1: row h takes row h+1, last row takes old row 0, then row 0 is cleared */
+        float first = history[r];
+        for (int64_t h = 0; h + 1 < H; ++h) history[h * R + r] = history[(h + 1) * R + r];
+        history[(H - 1) * R + r] = first;
+        history[r] = 0.0f;
+        scale[r] = oracle_scale(a, fmt[r], margin, scale[r]);
+        scale_inv[r] = oracle_scale_inv(scale[r]);
+    }
+}

@@ -1,0 +1,284 @@
+"""CPU oracle for the FP8 Linear path (TEST INFRASTRUCTURE ONLY).
+
+Only ``tests/``, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of
+``bench.py`` may import this module.  It offers the same operations twice:
+
+* ``c_*``  : thin ctypes wrappers over the plain-C restatement in
+  ``fp8_oracle.c`` (scalar loops; every rounding step is spelled out).
+* ``t_*``  : the same definitions written with torch CPU library routines
+  (``Tensor.to(torch.float8_*)``, fp32 ``@``).  They are fast enough for the
+  medium-sized parity cases and serve as the CPU baseline that is timed.
+
+The reference repository contains no FP8 arithmetic (it forwards to a
+third-party CUDA library at
+optimus_dl/modules/model_transforms/transformer_engine.py:97-108 and
+optimus_dl/modules/amp/fp8.py:254-306); both families follow the definitions in
+the header of ``fp8_oracle.c`` and are cross-checked against each other, against
+the 8-bit format definitions and against brute force in ``tests/``.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+import torch
+
+E4M3, E5M2 = 0, 1
+SCALE_TENSOR, SCALE_ROW, SCALE_COL = 0, 1, 2
+FP8_MAX = {E4M3: 448.0, E5M2: 57344.0}
+TORCH_FP8 = {E4M3: torch.float8_e4m3fn, E5M2: torch.float8_e5m2}
+FLT_MAX = float(np.finfo(np.float32).max)
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "_build", "libfp8_oracle.so")
+_lib = None
+
+
+def build(force: bool = False) -> str:
+    """Compile fp8_oracle.c with the Makefile beside it (gcc only)."""
+    if force or not os.path.exists(_LIB_PATH):
+        subprocess.run(["make", "-C", _HERE] + (["-B"] if force else []), check=True, capture_output=True)
+    return _LIB_PATH
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        build()
+        L = ctypes.CDLL(_LIB_PATH)
+        vp, i64, i32, f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float
+        L.oracle_f32_to_e4m3.argtypes = [f32]
+        L.oracle_f32_to_e4m3.restype = ctypes.c_uint8
+        L.oracle_f32_to_e5m2.argtypes = [f32]
+        L.oracle_f32_to_e5m2.restype = ctypes.c_uint8
+        L.oracle_encode_f32.argtypes = [vp, i64, i32, vp]
+        L.oracle_decode.argtypes = [vp, i64, i32, vp]
+        L.oracle_amax_bf16.argtypes = [vp, i64, i64, i32, vp]
+        L.oracle_scale.argtypes = [f32, i32, i32, f32]
+        L.oracle_scale.restype = f32
+        L.oracle_scale_inv.argtypes = [f32]
+        L.oracle_scale_inv.restype = f32
+        L.oracle_cast_bf16.argtypes = [vp, i64, i64, vp, i32, i32, vp]
+        L.oracle_cast_transpose_bf16.argtypes = [vp, i64, i64, vp, i32, i32, vp, vp]
+        L.oracle_gemm_nt.argtypes = [vp, vp, i64, i64, i64, i32, i32, vp, i64, vp, i64, vp, vp]
+        L.oracle_delayed_update.argtypes = [vp, i64, i64, vp, vp, vp, i32, i32]
+        _lib = L
+    return _lib
+
+
+def _p(a: np.ndarray):
+    return a.ctypes.data_as(ctypes.c_void_p)
+
+
+def _bf16_bits(x: torch.Tensor) -> np.ndarray:
+    assert x.dtype == torch.bfloat16 and x.device.type == "cpu"
+    return np.ascontiguousarray(x.contiguous().view(torch.int16).numpy().view(np.uint16))
+
+
+def _as_f32(s) -> np.ndarray:
+    if isinstance(s, torch.Tensor):
+        s = s.detach().cpu().float().numpy()
+    return np.ascontiguousarray(np.asarray(s, dtype=np.float32).reshape(-1))
+
+
+# --------------------------------------------------------------------- C family
+def c_encode(x_f32: np.ndarray, fmt: int) -> np.ndarray:
+    x = np.ascontiguousarray(x_f32, dtype=np.float32).reshape(-1)
+    out = np.empty(x.size, dtype=np.uint8)
+    lib().oracle_encode_f32(_p(x), x.size, fmt, _p(out))
+    return out.reshape(np.shape(x_f32))
+
+
+def c_decode(codes: np.ndarray, fmt: int) -> np.ndarray:
+    c = np.ascontiguousarray(codes, dtype=np.uint8).reshape(-1)
+    out = np.empty(c.size, dtype=np.float32)
+    lib().oracle_decode(_p(c), c.size, fmt, _p(out))
+    return out.reshape(np.shape(codes))
+
+
+def c_amax(x: torch.Tensor, mode: int = SCALE_TENSOR) -> torch.Tensor:
+    rows, cols = x.shape
+    bits = _bf16_bits(x)
+    n = 1 if mode == SCALE_TENSOR else (rows if mode == SCALE_ROW else cols)
+    out = np.empty(n, dtype=np.float32)
+    lib().oracle_amax_bf16(_p(bits), rows, cols, mode, _p(out))
+    return torch.from_numpy(out)
+
+
+def c_scale(amax: float, fmt: int, margin: int = 0, fallback: float = 1.0) -> float:
+    return float(lib().oracle_scale(float(amax), fmt, margin, float(fallback)))
+
+
+def c_scale_inv(scale: float) -> float:
+    return float(lib().oracle_scale_inv(float(scale)))
+
+
+def c_cast(x: torch.Tensor, scale, fmt: int, mode: int = SCALE_TENSOR) -> torch.Tensor:
+    rows, cols = x.shape
+    bits, s = _bf16_bits(x), _as_f32(scale)
+    assert s.size == (1 if mode == SCALE_TENSOR else (rows if mode == SCALE_ROW else cols))
+    out = np.empty((rows, cols), dtype=np.uint8)
+    lib().oracle_cast_bf16(_p(bits), rows, cols, _p(s), mode, fmt, _p(out))
+    return torch.from_numpy(out)
+
+
+def c_cast_transpose(x: torch.Tensor, scale, fmt: int, mode: int = SCALE_TENSOR):
+    rows, cols = x.shape
+    bits, s = _bf16_bits(x), _as_f32(scale)
+    out = np.empty((rows, cols), dtype=np.uint8)
+    out_t = np.empty((cols, rows), dtype=np.uint8)
+    lib().oracle_cast_transpose_bf16(_p(bits), rows, cols, _p(s), mode, fmt, _p(out), _p(out_t))
+    return torch.from_numpy(out), torch.from_numpy(out_t)
+
+
+def c_gemm_nt(a: torch.Tensor, b: torch.Tensor, fmt_a: int, fmt_b: int, sa_inv, sb_inv, want_f32: bool = False):
+    """a[M,K], b[N,K] uint8 codes -> bf16 [M,N] (and the unrounded fp32 when asked)."""
+    M, K = a.shape
+    N, K2 = b.shape
+    assert K == K2
+    an = np.ascontiguousarray(a.numpy(), dtype=np.uint8)
+    bn = np.ascontiguousarray(b.numpy(), dtype=np.uint8)
+    sa, sb = _as_f32(sa_inv), _as_f32(sb_inv)
+    assert sa.size in (1, M) and sb.size in (1, N)
+    c16 = np.empty((M, N), dtype=np.uint16)
+    c32 = np.empty((M, N), dtype=np.float32) if want_f32 else None
+    lib().oracle_gemm_nt(_p(an), _p(bn), M, N, K, fmt_a, fmt_b, _p(sa), sa.size, _p(sb), sb.size,
+                         _p(c16), _p(c32) if want_f32 else None)
+    out = torch.from_numpy(c16.view(np.int16)).view(torch.bfloat16)
+    return (out, torch.from_numpy(c32)) if want_f32 else out
+
+
+def c_delayed_update(history: np.ndarray, scale: np.ndarray, scale_inv: np.ndarray, fmts, margin: int, algo: str):
+    """In-place update of history[H,R], scale[R], scale_inv[R] (fp32 numpy arrays)."""
+    H, R = history.shape
+    assert history.dtype == np.float32 and history.flags.c_contiguous
+    f = np.ascontiguousarray(np.asarray(fmts, dtype=np.int32))
+    lib().oracle_delayed_update(_p(history), H, R, _p(scale), _p(scale_inv), _p(f), margin,
+                                0 if algo == "max" else 1)
+
+
+# ----------------------------------------------------------------- torch family
+def t_amax(x: torch.Tensor, mode: int = SCALE_TENSOR) -> torch.Tensor:
+    a = x.abs()
+    if mode == SCALE_TENSOR:
+        return a.amax().float().reshape(1)
+    return a.amax(dim=1 if mode == SCALE_ROW else 0).float()
+
+
+def t_scale(amax: torch.Tensor, fmt: int, margin: int = 0, fallback=1.0) -> torch.Tensor:
+    """Vectorised fp32 scale rule; `fallback` may be a scalar or a tensor like amax."""
+    amax = amax.float()
+    s = torch.tensor(FP8_MAX[fmt], dtype=torch.float32) / amax
+    if margin:
+        s = torch.ldexp(s, torch.tensor(-margin))
+    s = torch.where(torch.isinf(s), torch.tensor(FLT_MAX), s)
+    ok = torch.isfinite(amax) & (amax > 0)
+    fb = fallback if isinstance(fallback, torch.Tensor) else torch.tensor(float(fallback))
+    return torch.where(ok, s, fb.float())
+
+
+def t_cast(x: torch.Tensor, scale, fmt: int, mode: int = SCALE_TENSOR) -> torch.Tensor:
+    s = torch.as_tensor(scale, dtype=torch.float32)
+    if mode == SCALE_ROW:
+        s = s.reshape(-1, 1)
+    elif mode == SCALE_COL:
+        s = s.reshape(1, -1)
+    m = FP8_MAX[fmt]
+    return (x.float() * s).clamp(-m, m).to(TORCH_FP8[fmt]).view(torch.uint8)
+
+
+def t_cast_transpose(x, scale, fmt, mode=SCALE_TENSOR):
+    q = t_cast(x, scale, fmt, mode)
+    return q, q.t().contiguous()
+
+
+def t_decode(codes: torch.Tensor, fmt: int) -> torch.Tensor:
+    return codes.view(TORCH_FP8[fmt]).float()
+
+
+def t_gemm_nt(a, b, fmt_a, fmt_b, sa_inv, sb_inv, want_f32: bool = False):
+    """Emulated FP8 matmul: upcast, fp32 matmul, scale product, bf16."""
+    acc = t_decode(a, fmt_a) @ t_decode(b, fmt_b).t()
+    sa = torch.as_tensor(sa_inv, dtype=torch.float32).reshape(-1, 1)
+    sb = torch.as_tensor(sb_inv, dtype=torch.float32).reshape(1, -1)
+    out = acc * (sa * sb)
+    return (out.bfloat16(), out) if want_f32 else out.bfloat16()
+
+
+# -------------------------------------------------- the Linear, end to end (torch)
+def linear_fwd_bwd(x, w, dy, fmt_fwd=E4M3, fmt_bwd=E5M2, rowwise=False, scales=None):
+    """One FP8 Linear forward + backward on CPU with dynamic scaling.
+
+    x[M,K], w[N,K], dy[M,N] bf16.  Returns dict with y, dx, dw (bf16) and the
+    quantised operands / scales used.  `scales` = (sx, sw, sg) overrides the
+    dynamic per-tensor scales (delayed scaling feeds stale ones).
+    """
+    out = {}
+    if not rowwise:
+        if scales is None:
+            sx = t_scale(t_amax(x), fmt_fwd)
+            sw = t_scale(t_amax(w), fmt_fwd)
+            sg = t_scale(t_amax(dy), fmt_bwd)
+        else:
+            sx, sw, sg = (torch.as_tensor(s, dtype=torch.float32).reshape(1) for s in scales)
+        xq, xq_t = t_cast_transpose(x, sx, fmt_fwd)
+        wq, wq_t = t_cast_transpose(w, sw, fmt_fwd)
+        gq, gq_t = t_cast_transpose(dy, sg, fmt_bwd)
+        out["y"] = t_gemm_nt(xq, wq, fmt_fwd, fmt_fwd, 1.0 / sx, 1.0 / sw)
+        out["dx"] = t_gemm_nt(gq, wq_t, fmt_bwd, fmt_fwd, 1.0 / sg, 1.0 / sw)
+        out["dw"] = t_gemm_nt(gq_t, xq_t, fmt_bwd, fmt_fwd, 1.0 / sg, 1.0 / sx)
+        out.update(xq=xq, wq=wq, gq=gq, xq_t=xq_t, wq_t=wq_t, gq_t=gq_t, sx=sx, sw=sw, sg=sg)
+        return out
+    # rowwise: every operand is scaled along its non-contracted axis, from the bf16 source
+    sx_r = t_scale(t_amax(x, SCALE_ROW), fmt_fwd)
+    sw_r = t_scale(t_amax(w, SCALE_ROW), fmt_fwd)
+    xq = t_cast(x, sx_r, fmt_fwd, SCALE_ROW)
+    wq = t_cast(w, sw_r, fmt_fwd, SCALE_ROW)
+    out["y"] = t_gemm_nt(xq, wq, fmt_fwd, fmt_fwd, 1.0 / sx_r, 1.0 / sw_r)
+    sg_r = t_scale(t_amax(dy, SCALE_ROW), fmt_bwd)
+    sw_c = t_scale(t_amax(w, SCALE_COL), fmt_fwd)
+    gq = t_cast(dy, sg_r, fmt_bwd, SCALE_ROW)
+    wq_t = t_cast(w, sw_c, fmt_fwd, SCALE_COL).t().contiguous()
+    out["dx"] = t_gemm_nt(gq, wq_t, fmt_bwd, fmt_fwd, 1.0 / sg_r, 1.0 / sw_c)
+    sg_c = t_scale(t_amax(dy, SCALE_COL), fmt_bwd)
+    sx_c = t_scale(t_amax(x, SCALE_COL), fmt_fwd)
+    gq_t = t_cast(dy, sg_c, fmt_bwd, SCALE_COL).t().contiguous()
+    xq_t = t_cast(x, sx_c, fmt_fwd, SCALE_COL).t().contiguous()
+    out["dw"] = t_gemm_nt(gq_t, xq_t, fmt_bwd, fmt_fwd, 1.0 / sg_c, 1.0 / sx_c)
+    out.update(xq=xq, wq=wq, gq=gq, xq_t=xq_t, wq_t=wq_t, gq_t=gq_t,
+               sx=sx_r, sw=sw_r, sg=sg_r, sx_c=sx_c, sw_c=sw_c, sg_c=sg_c)
+    return out
+
+
+class DelayedState:
+    """Pure-Python delayed-scaling bookkeeping (ring of H amaxes per role)."""
+
+    def __init__(self, fmts, history_len: int, margin: int = 0, algo: str = "max"):
+        self.fmts = list(fmts)
+        self.H, self.R = history_len, len(self.fmts)
+        self.margin, self.algo = margin, algo
+        self.history = np.zeros((self.H, self.R), dtype=np.float32)
+        self.scale = np.ones(self.R, dtype=np.float32)
+        self.scale_inv = np.ones(self.R, dtype=np.float32)
+
+    def record(self, role: int, amax: float):
+        self.history[0, role] = max(self.history[0, role], np.float32(amax))
+
+    def update(self):
+        for r in range(self.R):
+            col = self.history[:, r]
+            a = col.max() if self.algo == "max" else col[0]
+            if np.isnan(col).any() and self.algo == "max":
+                a = np.float32("nan")
+            self.history[:, r] = np.roll(col, -1)
+            self.history[0, r] = 0.0
+            if np.isfinite(a) and a > 0:
+                s = np.float32(FP8_MAX[self.fmts[r]]) / np.float32(a)
+                s = np.float32(np.ldexp(s, -self.margin))
+                if np.isinf(s):
+                    s = np.float32(FLT_MAX)
+                self.scale[r] = s
+            self.scale_inv[r] = np.float32(1.0) / self.scale[r]

@@ -1,0 +1,184 @@
+"""GPU parity: FP8 MFMA GEMM vs the emulated-FP8 matmul of the oracle.
+
+Tolerance (stated by the task): max|out - ref| / max|ref| <= 1e-2 on the bf16
+output, ref = upcast codes to fp32, fp32 matmul, times the scale product, bf16.
+Cases whose partial sums are all exactly representable must be bit-exact,
+whatever order the hardware accumulates in.
+"""
+import pytest
+import torch
+
+from oracle import oracle as O
+from tests.helpers import max_rel_err, seeded_bf16
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+
+
+@pytest.fixture(scope="module")
+def N():
+    from optimus_dl_amd import native
+
+    native.load()
+    yield native
+    native.gemm_set_variant(-1)
+
+
+def quantised(shape, fmt, std, seed):
+    x = seeded_bf16(shape, std=std, seed=seed)
+    s = O.t_scale(O.t_amax(x), fmt)
+    return O.t_cast(x, s, fmt), (1.0 / s).float()
+
+
+def variants(N):
+    return list(range(len(N.gemm_variants())))
+
+
+def test_variant_table(N):
+    names = N.gemm_variants()
+    assert len(names) >= 2 and "generic" in names[0]
+    print("GEMM variants:", names)
+
+
+@pytest.mark.parametrize("fmts", [(O.E4M3, O.E4M3), (O.E5M2, O.E4M3), (O.E4M3, O.E5M2), (O.E5M2, O.E5M2)])
+def test_power_of_two_operands_are_bit_exact_every_variant(N, fmts):
+    """Operands in {0, +-1, +-2, +-0.5}: every product and partial sum is exact in
+    fp32, so the result must equal the oracle bit for bit in any summation order.
+    A wrong lane->row map, a wrong output layout or a wrong format selector
+    (e4m3 vs e5m2 decode the same byte differently) all break this."""
+    fa, fb = fmts
+    M, Nn, K = 320, 288, 512
+    g = torch.Generator().manual_seed(5)
+    vals = torch.tensor([0.0, 1.0, -1.0, 2.0, -2.0, 0.5, -0.5, 4.0])
+    av = vals[torch.randint(0, 8, (M, K), generator=g)]
+    bv = vals[torch.randint(0, 8, (Nn, K), generator=g)]
+    a = av.to(O.TORCH_FP8[fa]).view(torch.uint8)
+    b = bv.to(O.TORCH_FP8[fb]).view(torch.uint8)
+    sa, sb = torch.tensor([0.25]), torch.tensor([2.0])
+    ref16, ref32 = O.t_gemm_nt(a, b, fa, fb, sa, sb, want_f32=True)
+    assert torch.equal(ref32, (av @ bv.t()) * 0.5)                                 # the oracle itself is exact here
+    for v in variants(N):
+        N.gemm_set_variant(v)
+        out32 = N.gemm_nt(a.cuda(), b.cuda(), fa, fb, sa.cuda(), sb.cuda(), out_dtype=torch.float32)
+        assert torch.equal(out32.cpu(), ref32), f"variant {v} fp32 output differs: max diff {(out32.cpu() - ref32).abs().max()}"
+        out16 = N.gemm_nt(a.cuda(), b.cuda(), fa, fb, sa.cuda(), sb.cuda())
+        assert torch.equal(out16.cpu().view(torch.int16), ref16.view(torch.int16)), f"variant {v} bf16 output differs"
+    N.gemm_set_variant(-1)
+
+
+def test_one_hot_rows_pick_single_elements(N):
+    """A = rows of an identity (as FP8 1.0) selects columns of B exactly."""
+    K, M, Nn = 256, 256, 192
+    a = torch.zeros((M, K))
+    a[torch.arange(M), (torch.arange(M) * 7) % K] = 1.0
+    bq, sb_inv = quantised((Nn, K), O.E4M3, 1.0, 3)
+    aq = a.to(torch.float8_e4m3fn).view(torch.uint8)
+    one = torch.ones(1)
+    want = O.t_decode(bq, O.E4M3)[:, (torch.arange(M) * 7) % K].t().contiguous()
+    for v in variants(N):
+        N.gemm_set_variant(v)
+        out = N.gemm_nt(aq.cuda(), bq.cuda(), O.E4M3, O.E4M3, one.cuda(), one.cuda(), out_dtype=torch.float32)
+        assert torch.equal(out.cpu(), want), f"variant {v}"
+    N.gemm_set_variant(-1)
+
+
+SHAPES = [
+    (256, 256, 128), (512, 768, 1024), (300, 200, 256), (1024, 1024, 4096), (64, 4096, 512),
+    (33, 17, 128), (257, 255, 384), (128, 130, 64), (40, 24, 48), (1, 1, 16), (520, 1032, 2048),
+]
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+def test_random_gemm_within_tolerance_auto_variant(N, shape):
+    M, Nn, K = shape
+    aq, sa_inv = quantised((M, K), O.E5M2, 1e-3, 1)
+    bq, sb_inv = quantised((Nn, K), O.E4M3, 0.02, 2)
+    ref = O.t_gemm_nt(aq, bq, O.E5M2, O.E4M3, sa_inv, sb_inv)
+    out = N.gemm_nt(aq.cuda(), bq.cuda(), O.E5M2, O.E4M3, sa_inv.cuda(), sb_inv.cuda())
+    err = max_rel_err(out, ref)
+    assert err <= TOL, f"{shape}: max rel err {err}"
+
+
+@pytest.mark.parametrize("shape", [(512, 512, 1024), (300, 520, 256), (256, 256, 128)])
+def test_random_gemm_every_variant_vs_c_oracle(N, shape):
+    """Against the plain-C oracle (sequential fp32 accumulation)."""
+    M, Nn, K = shape
+    aq, sa_inv = quantised((M, K), O.E4M3, 1.0, 4)
+    bq, sb_inv = quantised((Nn, K), O.E4M3, 0.02, 5)
+    ref = O.c_gemm_nt(aq, bq, O.E4M3, O.E4M3, sa_inv, sb_inv)
+    for v in variants(N):
+        N.gemm_set_variant(v)
+        out = N.gemm_nt(aq.cuda(), bq.cuda(), O.E4M3, O.E4M3, sa_inv.cuda(), sb_inv.cuda())
+        err = max_rel_err(out, ref)
+        assert err <= TOL, f"variant {v} {shape}: max rel err {err}"
+    N.gemm_set_variant(-1)
+
+
+def test_rowwise_scales_and_bias_epilogue(N):
+    M, Nn, K = 384, 320, 512
+    x = seeded_bf16((M, K), seed=8)
+    x[:, 5] *= 100.0                                                               # an outlier channel
+    w = seeded_bf16((Nn, K), std=0.02, seed=9)
+    sx = O.t_scale(O.t_amax(x, O.SCALE_ROW), O.E4M3)
+    sw = O.t_scale(O.t_amax(w, O.SCALE_ROW), O.E4M3)
+    xq, wq = O.t_cast(x, sx, O.E4M3, O.SCALE_ROW), O.t_cast(w, sw, O.E4M3, O.SCALE_ROW)
+    bias = torch.randn(Nn)
+    ref32 = O.t_gemm_nt(xq, wq, O.E4M3, O.E4M3, 1 / sx, 1 / sw, want_f32=True)[1]
+    ref = (ref32 + bias).bfloat16()
+    for v in variants(N):
+        N.gemm_set_variant(v)
+        out = N.gemm_nt(xq.cuda(), wq.cuda(), O.E4M3, O.E4M3, (1 / sx).cuda(), (1 / sw).cuda(), bias=bias.cuda())
+        assert max_rel_err(out, ref) <= TOL, f"variant {v}"
+    N.gemm_set_variant(-1)
+    # rank-1 epilogue identity: scaling row i of the inverse scales by 2 doubles row i of the output exactly
+    sa2 = (1 / sx).clone()
+    sa2[7] *= 2
+    o1 = N.gemm_nt(xq.cuda(), wq.cuda(), O.E4M3, O.E4M3, (1 / sx).cuda(), (1 / sw).cuda(), out_dtype=torch.float32)
+    o2 = N.gemm_nt(xq.cuda(), wq.cuda(), O.E4M3, O.E4M3, sa2.cuda(), (1 / sw).cuda(), out_dtype=torch.float32)
+    assert torch.equal(o2[7], o1[7] * 2) and torch.equal(o2[8], o1[8])
+
+
+def test_transpose_symmetry(N):
+    """gemm(a, b)^T == gemm(b, a): same products, only the roles swap."""
+    aq, sa = quantised((512, 1024), O.E4M3, 1.0, 1)
+    bq, sb = quantised((768, 1024), O.E4M3, 1.0, 2)
+    o1 = N.gemm_nt(aq.cuda(), bq.cuda(), O.E4M3, O.E4M3, sa.cuda(), sb.cuda(), out_dtype=torch.float32)
+    o2 = N.gemm_nt(bq.cuda(), aq.cuda(), O.E4M3, O.E4M3, sb.cuda(), sa.cuda(), out_dtype=torch.float32)
+    assert max_rel_err(o2.t(), o1) <= 1e-5
+
+
+def test_gemm_refuses_bad_shapes(N):
+    a = torch.zeros((32, 24), dtype=torch.uint8, device="cuda")                    # K % 16 != 0
+    one = torch.ones(1, device="cuda")
+    with pytest.raises(N.NativeError):
+        N.gemm_nt(a, a, 0, 0, one, one)
+    b = torch.zeros((32, 32), dtype=torch.uint8, device="cuda")
+    with pytest.raises(N.NativeError):
+        N.gemm_nt(b, b, 0, 0, torch.ones(5, device="cuda"), one)                   # scale vector of the wrong length
+    with pytest.raises(N.NativeError):
+        N.gemm_nt(b, torch.zeros((32, 48), dtype=torch.uint8, device="cuda"), 0, 0, one, one)
+
+
+def test_linear_fwd_bwd_three_gemms_at_llama_mlp_slice(N):
+    """One Linear (fwd, dgrad, wgrad) through the real kernels end to end at a
+    slice of the Llama-3-8B MLP shape, against the oracle's Linear."""
+    M, K, Nn = 1024, 4096, 1792
+    x, w, dy = seeded_bf16((M, K), 1.0, 0), seeded_bf16((Nn, K), 0.02, 1), seeded_bf16((M, Nn), 1e-3, 2)
+    ref = O.linear_fwd_bwd(x, w, dy)
+    xd, wd, gd = x.cuda(), w.cuda(), dy.cuda()
+    sx, sxi = N.scale_from_amax(N.amax(xd), O.E4M3)
+    sw, swi = N.scale_from_amax(N.amax(wd), O.E4M3)
+    sg, sgi = N.scale_from_amax(N.amax(gd), O.E5M2)
+    xq, xqt = N.cast_transpose(xd, sx, O.E4M3)
+    wq, wqt = N.cast_transpose(wd, sw, O.E4M3)
+    gq, gqt = N.cast_transpose(gd, sg, O.E5M2)
+    for name, got in (("xq", xq), ("wq", wq), ("gq", gq), ("xq_t", xqt), ("wq_t", wqt), ("gq_t", gqt)):
+        assert torch.equal(got.cpu(), ref[name]), name
+    for name, got in (("sx", sx), ("sw", sw), ("sg", sg)):
+        assert torch.equal(got.cpu(), ref[name]), name
+    y = N.gemm_nt(xq, wq, O.E4M3, O.E4M3, sxi, swi)
+    dx = N.gemm_nt(gq, wqt, O.E5M2, O.E4M3, sgi, swi)
+    dw = N.gemm_nt(gqt, xqt, O.E5M2, O.E4M3, sgi, sxi)
+    for name, got in (("y", y), ("dx", dx), ("dw", dw)):
+        err = max_rel_err(got, ref[name])
+        assert err <= TOL, f"{name}: {err}"

@@ -1,0 +1,194 @@
+"""GPU parity: amax / scale / cast / cast+transpose kernels vs the CPU oracle.
+
+Integer / byte results must be bit-exact.  Every call goes through the C ABI.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as O
+from tests.helpers import assert_bytes_equal, assert_f32_bits_equal, seeded_bf16
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def N():
+    from optimus_dl_amd import native
+
+    native.load()
+    return native
+
+
+SHAPES = [(128, 64), (256, 256), (1024, 768), (16, 16), (48, 80), (1000, 200), (7, 13), (1, 1), (3, 4096), (513, 1032)]
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_amax_all_modes_bit_exact(N, shape, dtype):
+    x = seeded_bf16(shape, std=3.0, seed=sum(shape))
+    x[shape[0] // 2, shape[1] // 3] = -77.5                         # a lone outlier, negative on purpose
+    xd = x.to(dtype).cuda()
+    for mode in (O.SCALE_TENSOR, O.SCALE_ROW, O.SCALE_COL):
+        got = N.amax(xd, mode)
+        assert_f32_bits_equal(got, O.t_amax(x, mode), f"amax mode {mode} {shape} {dtype}")
+        assert_f32_bits_equal(got, O.c_amax(x, mode), f"amax(C oracle) mode {mode} {shape}")
+
+
+def test_amax_accumulate_and_specials(N):
+    x = seeded_bf16((64, 128), seed=1)
+    y = seeded_bf16((64, 128), std=5.0, seed=2)
+    for mode in (O.SCALE_TENSOR, O.SCALE_ROW, O.SCALE_COL):
+        acc = N.amax(x.cuda(), mode)
+        N.amax(y.cuda(), mode, out=acc, accumulate=True)
+        assert_f32_bits_equal(acc, torch.maximum(O.t_amax(x, mode), O.t_amax(y, mode)), f"accumulate mode {mode}")
+    z = torch.zeros((32, 64), dtype=torch.bfloat16)
+    z[3, 5] = -0.0
+    assert float(N.amax(z.cuda())[0]) == 0.0
+    z[4, 7] = float("nan")
+    assert torch.isnan(N.amax(z.cuda())).all()
+    r = N.amax(z.cuda(), O.SCALE_ROW).cpu()
+    assert torch.isnan(r[4]) and float(r[3]) == 0.0
+    z[4, 7] = float("inf")
+    assert torch.isinf(N.amax(z.cuda())).all()
+    assert N.amax(torch.empty((0, 16), dtype=torch.bfloat16).cuda(), O.SCALE_COL).abs().sum().item() == 0.0
+
+
+def test_amax_unaligned_view(N):
+    flat = seeded_bf16((1, 5000), seed=6).cuda()
+    view = flat[0, 3:4003].reshape(1, 4000)
+    assert view.data_ptr() % 16 != 0
+    assert_f32_bits_equal(N.amax(view), O.t_amax(view.cpu()), "unaligned amax")
+    assert_f32_bits_equal(N.amax(view, O.SCALE_ROW), O.t_amax(view.cpu(), O.SCALE_ROW), "unaligned row amax")
+
+
+@pytest.mark.parametrize("fmt", [O.E4M3, O.E5M2])
+def test_scale_from_amax_bit_exact(N, fmt):
+    rng = np.random.default_rng(0)
+    a = np.concatenate([
+        np.abs(rng.normal(0, 1, 5000)).astype(np.float32) * 5,
+        (2.0 ** rng.uniform(-140, 127, 5000)).astype(np.float32),
+        np.array([0.0, -1.0, np.inf, np.nan, 1e-45, 3e-39, 448.0, 57344.0, 3.4e38, 1.0], dtype=np.float32),
+        torch.randn(2000).abs().bfloat16().float().numpy(),
+    ])
+    for margin in (0, 1, 3):
+        s, si = N.scale_from_amax(torch.from_numpy(a).cuda(), fmt, margin)
+        want = np.array([O.c_scale(v, fmt, margin, 1.0) for v in a], dtype=np.float32)
+        want_inv = np.array([O.c_scale_inv(v) for v in want], dtype=np.float32)
+        assert_f32_bits_equal(s, torch.from_numpy(want), f"scale fmt {fmt} margin {margin}")
+        assert_f32_bits_equal(si, torch.from_numpy(want_inv), f"scale_inv fmt {fmt} margin {margin}")
+        if margin == 0:
+            assert_f32_bits_equal(s, O.t_scale(torch.from_numpy(a), fmt), "scale vs torch rule")
+
+
+@pytest.mark.parametrize("fmt", [O.E4M3, O.E5M2])
+def test_cast_every_bf16_pattern_times_many_scales(N, fmt):
+    """All 65536 bf16 inputs x 256 scales: exercises RNE ties, subnormals, the
+    clamp, NaN/Inf and signed zeros of the hardware conversion."""
+    allbits = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    rng = np.random.default_rng(3)
+    scales = np.concatenate([
+        np.array([1.0, 0.5, 2.0, 448.0, 57344.0, 3.4028235e38, 1e-30, 2.0 ** -20, 2.0 ** 20, 0.3333333], dtype=np.float32),
+        (O.FP8_MAX[fmt] / np.abs(rng.normal(0, 2, 123)).astype(np.float32)).astype(np.float32),
+        (2.0 ** rng.uniform(-30, 30, 123)).astype(np.float32),
+    ])
+    x = allbits.reshape(1, 65536).expand(len(scales), 65536).contiguous()       # row r uses scale r
+    s = torch.from_numpy(scales)
+    got = N.cast(x.cuda(), s.cuda(), fmt, O.SCALE_ROW)
+    assert_bytes_equal(got, O.c_cast(x, s, fmt, O.SCALE_ROW), f"cast exhaustive fmt {fmt} (C oracle)")
+    assert_bytes_equal(got, O.t_cast(x, s, fmt, O.SCALE_ROW), f"cast exhaustive fmt {fmt} (torch CPU)")
+
+
+@pytest.mark.parametrize("fmt", [O.E4M3, O.E5M2])
+@pytest.mark.parametrize("mode", [O.SCALE_TENSOR, O.SCALE_ROW, O.SCALE_COL])
+@pytest.mark.parametrize("shape", [(256, 128), (128, 4096), (1000, 48), (64, 16), (33, 20), (5, 3)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_cast_and_cast_transpose_match_oracle(N, fmt, mode, shape, dtype):
+    x = seeded_bf16(shape, std=1.0, seed=shape[0] * 7 + shape[1])
+    x[0, 0] = float("nan")
+    x[-1, -1] = float("-inf")
+    x[shape[0] // 2, 0] = 300.0
+    am = O.t_amax(torch.nan_to_num(x, nan=0.0, posinf=0.0, neginf=0.0), mode)
+    s = O.t_scale(am, fmt) * (1.7 if mode == O.SCALE_TENSOR else 1.0)              # >1: makes the clamp fire
+    xd = x.to(dtype).cuda()
+    want = O.t_cast(x, s, fmt, mode)
+    got = N.cast(xd, s.cuda(), fmt, mode)
+    assert_bytes_equal(got, want, f"cast {shape} mode {mode} fmt {fmt} {dtype}")
+    q, qt = N.cast_transpose(xd, s.cuda(), fmt, mode)
+    assert_bytes_equal(q, want, f"cast_transpose row-major {shape} mode {mode}")
+    assert_bytes_equal(qt, want.t().contiguous(), f"cast_transpose transposed {shape} mode {mode}")
+    q2, qt2 = N.cast_transpose(xd, s.cuda(), fmt, mode, want_rowmajor=False)
+    assert q2 is None
+    assert_bytes_equal(qt2, want.t().contiguous(), f"cast_transpose only-T {shape} mode {mode}")
+
+
+@pytest.mark.parametrize("fmt", [O.E4M3, O.E5M2])
+def test_cast_with_fused_amax_for_delayed_scaling(N, fmt):
+    x = seeded_bf16((512, 384), std=2.0, seed=11)
+    stale = torch.tensor([O.FP8_MAX[fmt] / 3.0])                                   # smaller amax than the data: clamps
+    for fn in ("cast", "cast_transpose"):
+        slot = torch.zeros(1, device="cuda")
+        if fn == "cast":
+            q = N.cast(x.cuda(), stale.cuda(), fmt, amax_out=slot)
+        else:
+            q, qt = N.cast_transpose(x.cuda(), stale.cuda(), fmt, amax_out=slot)
+            assert_bytes_equal(qt, O.t_cast(x, stale, fmt).t().contiguous(), "fused-amax transposed codes")
+        assert_bytes_equal(q, O.t_cast(x, stale, fmt), f"{fn} with fused amax codes")
+        assert_f32_bits_equal(slot, O.t_amax(x), f"{fn} fused amax")
+        # a second tensor folds into the same slot (max), as microbatches do
+        y = seeded_bf16((512, 384), std=0.5, seed=12)
+        N.cast(y.cuda(), stale.cuda(), fmt, amax_out=slot)
+        assert_f32_bits_equal(slot, torch.maximum(O.t_amax(x), O.t_amax(y)), "amax slot folds")
+
+
+def test_cast_transpose_large_matches_cast_then_transpose(N):
+    """Size-independent property at a BASELINE shape: out_t == out^T bytewise."""
+    x = seeded_bf16((8192, 4096), seed=0).cuda()
+    am = N.amax(x)
+    s, _ = N.scale_from_amax(am, O.E4M3)
+    q, qt = N.cast_transpose(x, s, O.E4M3)
+    assert torch.equal(qt, q.t().contiguous())
+    assert torch.equal(q, N.cast(x, s, O.E4M3))
+    # against torch CPU on a slab (the whole tensor would take seconds, a slab pins the same code path)
+    want = O.t_cast(x[:512].cpu(), s.cpu(), O.E4M3)
+    assert_bytes_equal(q[:512], want, "large cast slab")
+
+
+def test_delayed_update_matches_oracle(N):
+    H, R = 16, 5
+    fmts = [O.E4M3, O.E4M3, O.E4M3, O.E5M2, O.E5M2]
+    rng = np.random.default_rng(7)
+    hist = np.zeros((H, R), dtype=np.float32)
+    scale = np.ones(R, dtype=np.float32)
+    inv = np.ones(R, dtype=np.float32)
+    dh, ds, di = torch.from_numpy(hist.copy()).cuda(), torch.from_numpy(scale.copy()).cuda(), torch.from_numpy(inv.copy()).cuda()
+    dfm = torch.tensor(fmts, dtype=torch.int32).cuda()
+    for algo_name, algo in (("max", 0), ("most_recent", 1)):
+        for step in range(40):
+            new = np.abs(rng.normal(0, 1 + step * 0.1, R)).astype(np.float32)
+            if step == 5:
+                new[1] = 0.0
+            if step == 9:
+                new[2] = np.inf
+            if step == 13:
+                new[4] = np.nan
+            hist[0] = new
+            dh[0] = torch.from_numpy(new).cuda()
+            O.c_delayed_update(hist, scale, inv, fmts, margin=1, algo=algo_name)
+            N.delayed_update(dh, ds, di, dfm, margin=1, algo=algo)
+            assert_f32_bits_equal(dh, torch.from_numpy(hist), f"history step {step} {algo_name}")
+            assert_f32_bits_equal(ds, torch.from_numpy(scale), f"scale step {step} {algo_name}")
+            assert_f32_bits_equal(di, torch.from_numpy(inv), f"scale_inv step {step} {algo_name}")
+
+
+def test_bad_arguments_are_refused(N):
+    x = seeded_bf16((16, 16)).cuda()
+    with pytest.raises(N.NativeError):
+        N.cast(x, torch.ones(3, device="cuda"), O.E4M3)                            # wrong scale count
+    with pytest.raises(N.NativeError):
+        N.cast(x.cpu(), torch.ones(1), O.E4M3)                                     # CPU tensor
+    with pytest.raises(N.NativeError):
+        N.amax(x.half())                                                           # unsupported dtype
+    with pytest.raises(N.NativeError):
+        N._check(N.load().odl_fp8_cast(x.data_ptr(), 0, 16, 16, torch.ones(1, device="cuda").data_ptr(), 0, 9,
+                                       x.data_ptr(), None, None), "bad fmt")

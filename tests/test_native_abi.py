@@ -1,0 +1,55 @@
+"""CPU-side checks of the native boundary: the library loads and exports every
+symbol that include/odl_fp8.h declares (no compute calls: there is no GPU here)."""
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "odl_fp8.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(odl_fp8_\w+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    syms = declared_symbols()
+    for must in ("odl_fp8_amax", "odl_fp8_cast", "odl_fp8_cast_transpose", "odl_fp8_gemm_nt",
+                 "odl_fp8_scale_from_amax", "odl_fp8_delayed_update"):
+        assert must in syms
+
+
+def test_library_exports_every_declared_symbol():
+    from optimus_dl_amd import native
+
+    if not native.is_built():
+        pytest.skip("libodl_fp8.so not built here (run `python -m optimus_dl_amd.build`)")
+    lib = native.load()
+    for sym in declared_symbols():
+        assert hasattr(lib, sym), f"{sym} is declared in include/odl_fp8.h but not exported"
+    assert sorted(native.EXPORTS) == declared_symbols()
+    assert lib.odl_fp8_abi_version() == native.ABI_VERSION
+    assert lib.odl_fp8_gemm_num_variants() >= 2
+    assert b"generic" in lib.odl_fp8_gemm_variant_name(0)
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    from optimus_dl_amd import native
+
+    monkeypatch.setattr(native, "_lib", None)
+    monkeypatch.setattr(native, "LIB_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(native.NativeError, match="no fallback"):
+        native.load()
+
+
+def test_cpu_tensors_are_refused_not_emulated():
+    import torch
+
+    from optimus_dl_amd import native
+
+    if not native.is_built():
+        pytest.skip("library not built")
+    with pytest.raises(native.NativeError):
+        native.amax(torch.zeros((4, 4), dtype=torch.bfloat16))
