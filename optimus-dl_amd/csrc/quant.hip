@@ -538,8 +538,8 @@ using namespace odl;
 extern "C" int odl_fp8_amax(const void *x, int src_dtype, int64_t rows, int64_t cols, int mode, float *amax_out,
                             int accumulate, odl_stream_t stream_) {
     hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
-    if (!x || !amax_out) return set_error(ODL_ERR_ARG, "odl_fp8_amax: null pointer");
     if (rows < 0 || cols < 0) return set_error(ODL_ERR_ARG, "odl_fp8_amax: negative shape %lld x %lld", (long long)rows, (long long)cols);
+    if ((!x && rows * cols > 0) || !amax_out) return set_error(ODL_ERR_ARG, "odl_fp8_amax: null pointer");
     if (src_dtype != ODL_BF16 && src_dtype != ODL_F32) return set_error(ODL_ERR_ARG, "odl_fp8_amax: src_dtype %d", src_dtype);
     if (mode < ODL_SCALE_TENSOR || mode > ODL_SCALE_COL) return set_error(ODL_ERR_ARG, "odl_fp8_amax: mode %d", mode);
     const int64_t n_out = mode == ODL_SCALE_TENSOR ? 1 : (mode == ODL_SCALE_ROW ? rows : cols);
@@ -658,8 +658,8 @@ static void launch_ct_mode(int mode, const void *x, int64_t rows, int64_t cols, 
 
 static int check_cast_args(const char *who, const void *x, int src_dtype, int64_t rows, int64_t cols, const float *scale,
                            int mode, int fmt) {
-    if (!x || !scale) return set_error(ODL_ERR_ARG, "%s: null pointer", who);
     if (rows < 0 || cols < 0) return set_error(ODL_ERR_ARG, "%s: negative shape", who);
+    if ((!x || !scale) && rows * cols > 0) return set_error(ODL_ERR_ARG, "%s: null pointer", who);
     if (src_dtype != ODL_BF16 && src_dtype != ODL_F32) return set_error(ODL_ERR_ARG, "%s: src_dtype %d", who, src_dtype);
     if (mode < ODL_SCALE_TENSOR || mode > ODL_SCALE_COL) return set_error(ODL_ERR_ARG, "%s: mode %d", who, mode);
     if (fmt != ODL_FP8_E4M3 && fmt != ODL_FP8_E5M2) return set_error(ODL_ERR_ARG, "%s: fmt %d", who, fmt);
@@ -683,8 +683,8 @@ extern "C" int odl_fp8_cast(const void *x, int src_dtype, int64_t rows, int64_t 
                             uint8_t *out, float *amax_out, odl_stream_t stream_) {
     hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
     if (int e = check_cast_args("odl_fp8_cast", x, src_dtype, rows, cols, scale, mode, fmt)) return e;
-    if (!out) return set_error(ODL_ERR_ARG, "odl_fp8_cast: out is null");
     if (rows * cols == 0) return ODL_OK;
+    if (!out) return set_error(ODL_ERR_ARG, "odl_fp8_cast: out is null");
     const bool fast = cols % 16 == 0 && aligned16(x) && aligned16(out) && (mode != ODL_SCALE_COL || aligned16(scale));
     if (fast) ODL_DISPATCH_SRC_FMT(launch_cast_mode, mode, x, rows, cols, scale, out, amax_out, stream);
     else ODL_DISPATCH_SRC_FMT(launch_generic, x, rows, cols, scale, mode, out, (uint8_t *)nullptr, amax_out, stream);
@@ -695,8 +695,8 @@ extern "C" int odl_fp8_cast_transpose(const void *x, int src_dtype, int64_t rows
                                       int fmt, uint8_t *out, uint8_t *out_t, float *amax_out, odl_stream_t stream_) {
     hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
     if (int e = check_cast_args("odl_fp8_cast_transpose", x, src_dtype, rows, cols, scale, mode, fmt)) return e;
-    if (!out_t) return set_error(ODL_ERR_ARG, "odl_fp8_cast_transpose: out_t is null");
     if (rows * cols == 0) return ODL_OK;
+    if (!out_t) return set_error(ODL_ERR_ARG, "odl_fp8_cast_transpose: out_t is null");
     const int64_t tiles = ((rows + kTileR - 1) / kTileR) * ((cols + kTileC - 1) / kTileC);
     const bool fast = cols % 8 == 0 && rows % 16 == 0 && aligned16(x) && aligned16(out_t) &&
                       (!out || (reinterpret_cast<uintptr_t>(out) & 7) == 0) &&
