@@ -112,14 +112,15 @@ int odl_fp8_gemm_nt(const uint8_t *a, const uint8_t *b, int64_t M, int64_t N, in
  * Delayed-scaling bookkeeping for R tensor roles with H history slots each
  * (recipe "delayed", fp8.py:279-288; runs where the reference leaves its
  * autocast context, fp8.py:337-340,357-360).
- *   history [H,R] fp32, row 0 = newest amax (written by the casts of the step)
+ *   history [H,R] fp32 with leading dimension ld >= R (element (h,r) at h*ld + r),
+ *   row 0 = newest amax (written by the casts of the step)
  *   a = max over the column (ODL_AMAX_MAX) or history[0] (ODL_AMAX_MOST_RECENT)
  *   history <- roll(history, -1 along H); history[0] <- 0
  *   scale[r] = fp8_max(fmt[r]) / a / 2^margin, kept when a is 0/NaN/Inf; Inf -> FLT_MAX
  *   scale_inv[r] = 1 / scale[r]
  *   fmt: R ints (odl_fp8_format) in device memory.
  */
-int odl_fp8_delayed_update(float *history, int64_t H, int64_t R,
+int odl_fp8_delayed_update(float *history, int64_t H, int64_t R, int64_t ld,
                            float *scale, float *scale_inv, const int *fmt,
                            int margin, int algo, odl_stream_t stream);
 

@@ -14,6 +14,9 @@
 namespace odl {
 
 constexpr int kThreads = 256;
+// Kernels that end in one atomicMax per block use fat blocks and a small grid:
+// same-address atomics from different XCDs retire one at a time (~8 ns each).
+constexpr int kFatThreads = 1024;
 
 __device__ __forceinline__ u32x4 load16(const void *p) { return *reinterpret_cast<const u32x4 *>(p); }
 
@@ -27,14 +30,14 @@ __global__ void fill_f32_kernel(float *p, int64_t n, float v) {
 // x viewed as n16 chunks of 16 bytes plus a scalar tail.  Each lane keeps UNROLL
 // loads in flight; magnitudes are reduced as integer bit patterns.
 template <int SRC, int UNROLL>
-__global__ __launch_bounds__(kThreads) void amax_tensor_kernel(const void *__restrict__ x, int64_t n,
-                                                                float *__restrict__ out) {
-    __shared__ uint32_t red[kThreads / kWave];
+__global__ __launch_bounds__(kFatThreads) void amax_tensor_kernel(const void *__restrict__ x, int64_t n,
+                                                                   float *__restrict__ out) {
+    __shared__ uint32_t red[kFatThreads / kWave];
     constexpr int EPC = SRC == ODL_BF16 ? 8 : 4;          // elements per 16-byte chunk
     const int64_t n16 = n / EPC;
     const u32x4 *p = reinterpret_cast<const u32x4 *>(x);
-    const int64_t stride = (int64_t)gridDim.x * kThreads;
-    int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * kFatThreads;
+    int64_t i = (int64_t)blockIdx.x * kFatThreads + threadIdx.x;
     uint32_t m0 = 0, m1 = 0, m2 = 0, m3 = 0;
     for (; i + (UNROLL - 1) * stride < n16; i += UNROLL * stride) {
         u32x4 v[UNROLL];
@@ -268,21 +271,18 @@ __global__ void scale_from_amax_kernel(const float *__restrict__ amax, int64_t n
 }
 
 // one thread per role; H is small (<= a few thousand), latency only
-__global__ void delayed_update_kernel(float *__restrict__ history, int64_t H, int64_t R, float *__restrict__ scale,
+__global__ void delayed_update_kernel(float *__restrict__ history, int64_t H, int64_t R, int64_t ld, float *__restrict__ scale,
                                       float *__restrict__ scale_inv, const int *__restrict__ fmt, int margin, int algo) {
     int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (r >= R) return;
     const float first = history[r];
     uint32_t abits = float_to_bits(first) & 0x7fffffffu;     // amaxes are >= 0 or NaN: integer max keeps NaN
-    float prev = first;
     for (int64_t h = 1; h < H; ++h) {
-        float cur = history[h * R + r];
+        float cur = history[h * ld + r];
         if (algo == ODL_AMAX_MAX) abits = max(abits, float_to_bits(cur) & 0x7fffffffu);
-        history[(h - 1) * R + r] = cur;                       // roll by -1
-        prev = cur;
+        history[(h - 1) * ld + r] = cur;                      // roll by -1
     }
-    (void)prev;
-    history[(H - 1) * R + r] = first;
+    history[(H - 1) * ld + r] = first;
     history[r] = 0.0f;
     const float fmax = fmt[r] == ODL_FP8_E5M2 ? 57344.0f : 448.0f;
     float s = scale_rule(bits_to_float(abits), fmax, margin, scale[r]);
@@ -294,17 +294,18 @@ __global__ void delayed_update_kernel(float *__restrict__ history, int64_t H, in
 // 16 elements per lane per step: two (bf16) or four (fp32) 16-byte loads, one
 // 16-byte store.  cols % 16 == 0 and 16-byte aligned pointers (host-checked).
 template <int SRC, int FMT, int MODE, bool AMAX>
-__global__ __launch_bounds__(kThreads) void cast_kernel(const void *__restrict__ x, int64_t rows, int64_t cols,
+__global__ __launch_bounds__(AMAX ? kFatThreads : kThreads) void cast_kernel(const void *__restrict__ x, int64_t rows, int64_t cols,
                                                          const float *__restrict__ scale, uint8_t *__restrict__ out,
                                                          float *__restrict__ amax_out) {
-    __shared__ uint32_t red[kThreads / kWave];
+    constexpr int kT = AMAX ? kFatThreads : kThreads;
+    __shared__ uint32_t red[kT / kWave];
     const int64_t cpr = cols / 16;                           // chunks per row
     const int64_t nchunk = rows * cpr;
-    const int64_t stride = (int64_t)gridDim.x * kThreads;
+    const int64_t stride = (int64_t)gridDim.x * kT;
     float s_t = 1.0f;
     if constexpr (MODE == ODL_SCALE_TENSOR) s_t = scale[0];
     uint32_t am = 0;
-    for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < nchunk; i += stride) {
+    for (int64_t i = (int64_t)blockIdx.x * kT + threadIdx.x; i < nchunk; i += stride) {
         float f[16];
         if constexpr (SRC == ODL_BF16) {
             const u32x4 *p = reinterpret_cast<const u32x4 *>(x) + i * 2;
@@ -415,7 +416,12 @@ __global__ __launch_bounds__(kThreads) void cast_transpose_kernel(const void *__
     const int tx = threadIdx.x % 8;                 // 8 lanes across 64 columns
     const int ty = threadIdx.x / 8;                 // 32 lane-rows, 4 rows each
     const int64_t tiles_c = (cols + kTileC - 1) / kTileC;
-    const int64_t tr = blockIdx.x / tiles_c, tc = blockIdx.x % tiles_c;
+    const int64_t ntiles = tiles_c * ((rows + kTileR - 1) / kTileR);
+    uint32_t am = 0;
+    // With a fused amax the grid is small and each block walks several tiles, so
+    // that the kernel ends in few atomics; otherwise one tile per block.
+    for (int64_t tile_id = blockIdx.x; tile_id < ntiles; tile_id += gridDim.x) {
+    const int64_t tr = tile_id / tiles_c, tc = tile_id % tiles_c;
     const int64_t r0 = tr * kTileR + ty * 4, c0 = tc * kTileC + tx * 8;
     const bool col_ok = c0 < cols;                  // cols % 8 == 0 (host-checked), so the whole 8-wide patch is in or out
 
@@ -444,7 +450,6 @@ __global__ __launch_bounds__(kThreads) void cast_transpose_kernel(const void *__
         for (int h = 0; h < ESZ / 2; ++h) raw[i][h] = ok ? __builtin_nontemporal_load(p + h) : u32x4{0, 0, 0, 0};
     }
 
-    uint32_t am = 0;
     uint32_t lo[4], hi[4];                          // codes of columns 0..3 / 4..7 for each of the 4 rows
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -504,6 +509,8 @@ __global__ __launch_bounds__(kThreads) void cast_transpose_kernel(const void *__
             __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(out_t + oc * rows + orow));
         }
     }
+    if (tile_id + gridDim.x < ntiles) __syncthreads();  // the LDS tile is reused by the next trip
+    }
     if constexpr (AMAX) {
         if constexpr (SRC == ODL_BF16) am = fold_u16x2_to_f32bits(am);
         am = block_max_u32(am, red);
@@ -551,9 +558,9 @@ extern "C" int odl_fp8_amax(const void *x, int src_dtype, int64_t rows, int64_t 
     const int esz = src_dtype == ODL_BF16 ? 2 : 4;
     if (mode == ODL_SCALE_TENSOR) {
         if (aligned16(x)) {
-            const int64_t g = grid_for(n * esz / 16, kThreads * 4, 8);
-            if (src_dtype == ODL_BF16) hipLaunchKernelGGL((amax_tensor_kernel<ODL_BF16, 4>), dim3((unsigned)g), dim3(kThreads), 0, stream, x, n, amax_out);
-            else hipLaunchKernelGGL((amax_tensor_kernel<ODL_F32, 4>), dim3((unsigned)g), dim3(kThreads), 0, stream, x, n, amax_out);
+            const int64_t g = grid_for(n * esz / 16, kFatThreads * 4, 2);
+            if (src_dtype == ODL_BF16) hipLaunchKernelGGL((amax_tensor_kernel<ODL_BF16, 4>), dim3((unsigned)g), dim3(kFatThreads), 0, stream, x, n, amax_out);
+            else hipLaunchKernelGGL((amax_tensor_kernel<ODL_F32, 4>), dim3((unsigned)g), dim3(kFatThreads), 0, stream, x, n, amax_out);
         } else {
             const int64_t g = grid_for(n, kThreads * 8, 8);
             if (src_dtype == ODL_BF16) hipLaunchKernelGGL((amax_tensor_scalar_kernel<ODL_BF16>), dim3((unsigned)g), dim3(kThreads), 0, stream, x, n, amax_out);
@@ -601,14 +608,14 @@ extern "C" int odl_fp8_scale_from_amax(const float *amax, int64_t n, int fmt, in
     return check_launch("odl_fp8_scale_from_amax");
 }
 
-extern "C" int odl_fp8_delayed_update(float *history, int64_t H, int64_t R, float *scale, float *scale_inv, const int *fmt,
-                                      int margin, int algo, odl_stream_t stream_) {
+extern "C" int odl_fp8_delayed_update(float *history, int64_t H, int64_t R, int64_t ld, float *scale, float *scale_inv,
+                                      const int *fmt, int margin, int algo, odl_stream_t stream_) {
     hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
     if (!history || !scale || !scale_inv || !fmt) return set_error(ODL_ERR_ARG, "odl_fp8_delayed_update: null pointer");
-    if (H < 1 || R < 0) return set_error(ODL_ERR_ARG, "odl_fp8_delayed_update: H=%lld R=%lld", (long long)H, (long long)R);
+    if (H < 1 || R < 0 || ld < R) return set_error(ODL_ERR_ARG, "odl_fp8_delayed_update: H=%lld R=%lld ld=%lld", (long long)H, (long long)R, (long long)ld);
     if (algo != ODL_AMAX_MAX && algo != ODL_AMAX_MOST_RECENT) return set_error(ODL_ERR_ARG, "odl_fp8_delayed_update: algo %d", algo);
     if (R == 0) return ODL_OK;
-    hipLaunchKernelGGL(delayed_update_kernel, dim3((unsigned)((R + 63) / 64)), dim3(64), 0, stream, history, H, R, scale,
+    hipLaunchKernelGGL(delayed_update_kernel, dim3((unsigned)((R + 63) / 64)), dim3(64), 0, stream, history, H, R, ld, scale,
                        scale_inv, fmt, margin, algo);
     return check_launch("odl_fp8_delayed_update");
 }
@@ -618,9 +625,13 @@ namespace odl {
 template <int SRC, int FMT, int MODE>
 static void launch_cast(const void *x, int64_t rows, int64_t cols, const float *scale, uint8_t *out, float *amax_out,
                         hipStream_t stream) {
-    const int64_t g = grid_for(rows * cols / 16, kThreads, 16);
-    if (amax_out) hipLaunchKernelGGL((cast_kernel<SRC, FMT, MODE, true>), dim3((unsigned)g), dim3(kThreads), 0, stream, x, rows, cols, scale, out, amax_out);
-    else hipLaunchKernelGGL((cast_kernel<SRC, FMT, MODE, false>), dim3((unsigned)g), dim3(kThreads), 0, stream, x, rows, cols, scale, out, amax_out);
+    if (amax_out) {
+        const int64_t g = grid_for(rows * cols / 16, kFatThreads, 2);
+        hipLaunchKernelGGL((cast_kernel<SRC, FMT, MODE, true>), dim3((unsigned)g), dim3(kFatThreads), 0, stream, x, rows, cols, scale, out, amax_out);
+    } else {
+        const int64_t g = grid_for(rows * cols / 16, kThreads, 16);
+        hipLaunchKernelGGL((cast_kernel<SRC, FMT, MODE, false>), dim3((unsigned)g), dim3(kThreads), 0, stream, x, rows, cols, scale, out, amax_out);
+    }
 }
 
 template <int SRC, int FMT>
@@ -641,7 +652,8 @@ static void launch_generic(const void *x, int64_t rows, int64_t cols, const floa
 template <int SRC, int FMT, int MODE>
 static void launch_ct(const void *x, int64_t rows, int64_t cols, const float *scale, uint8_t *out, uint8_t *out_t,
                       float *amax_out, hipStream_t stream) {
-    const int64_t g = ((rows + kTileR - 1) / kTileR) * ((cols + kTileC - 1) / kTileC);
+    int64_t g = ((rows + kTileR - 1) / kTileR) * ((cols + kTileC - 1) / kTileC);
+    if (amax_out && g > (int64_t)num_cus() * 4) g = (int64_t)num_cus() * 4;
 #define ODL_CT(AM, RM) hipLaunchKernelGGL((cast_transpose_kernel<SRC, FMT, MODE, AM, RM>), dim3((unsigned)g), dim3(kThreads), 0, stream, x, rows, cols, scale, out, out_t, amax_out)
     if (amax_out) { if (out) ODL_CT(true, true); else ODL_CT(true, false); }
     else { if (out) ODL_CT(false, true); else ODL_CT(false, false); }

@@ -1,0 +1,329 @@
+"""FP8 recipe and autocast contexts, backed by the MI355X kernels.
+
+API-compatible with optimus_dl/modules/amp/fp8.py: the enums (:40-61), the
+string parsers (:96-147) with their error texts, ``Fp8RecipeConfig`` (:151),
+``FP8Recipe`` with its constructor arguments echoed as attributes, ``.recipe``,
+``.autocast()`` and ``.backward()`` (:180-360), ``create_fp8_recipe`` (:387),
+``fp8_autocast`` (:450) and ``fp8_backward`` (:501).
+
+Where the reference hands the recipe to a third-party CUDA library, this module
+owns the scaling policy itself:
+
+  tensorwise  amax of the tensor at hand -> scale -> cast       (two passes)
+  delayed     cast with the scale from the amax history while recording this
+              step's amax; histories roll and scales refresh when the outermost
+              autocast / backward context exits                 (one pass)
+  rowwise     (extension, no reference enum) one scale per row of each operand
+              along its non-contracted axis
+  blockwise / mxfp8 are accepted by the parsers, as in the reference, but have
+  no kernels here: constructing a recipe with them raises NotImplementedError.
+"""
+
+from __future__ import annotations
+
+import logging
+from collections.abc import Iterator
+from contextlib import contextmanager
+from dataclasses import dataclass
+from enum import Enum
+from typing import Any
+
+import torch
+
+from ... import native
+from . import state as _state
+
+logger = logging.getLogger(__name__)
+_logged_once: set[str] = set()
+
+
+def _info_once(msg: str) -> None:
+    if msg not in _logged_once:
+        _logged_once.add(msg)
+        logger.info(msg)
+
+
+class Fp8Format(Enum):
+    HYBRID = "hybrid"   # E4M3 forward, E5M2 gradients
+    E4M3 = "e4m3"
+    E5M2 = "e5m2"
+
+
+class Fp8RecipeType(str, Enum):
+    DELAYED = "delayed"
+    TENSORWISE = "tensorwise"
+    BLOCKWISE = "blockwise"
+    MXFP8 = "mxfp8"
+    ROWWISE = "rowwise"   # extension: per-row / per-output-channel scales
+
+
+_FORMAT_ALIASES = {
+    Fp8Format.HYBRID: ("hybrid", "hybrid_fp8", "fp8_hybrid"),
+    Fp8Format.E4M3: ("e4m3", "fp8_e4m3", "e4m3fn", "float8_e4m3fn"),
+    Fp8Format.E5M2: ("e5m2", "fp8_e5m2", "e5m2fn", "float8_e5m2"),
+}
+_RECIPE_ALIASES = {
+    Fp8RecipeType.DELAYED: ("delayed", "delayed_scaling"),
+    Fp8RecipeType.TENSORWISE: ("tensorwise", "tensor_wise", "current", "current_scaling"),
+    Fp8RecipeType.BLOCKWISE: ("blockwise", "block_wise", "float8_block"),
+    Fp8RecipeType.MXFP8: ("mxfp8", "mxfp8_block"),
+    Fp8RecipeType.ROWWISE: ("rowwise", "row_wise", "channelwise"),
+}
+
+
+def is_native_backend_available() -> bool:
+    """True when the compiled kernel library is present and a GPU is visible."""
+    return native.is_built() and torch.cuda.is_available()
+
+
+def is_transformer_engine_available() -> bool:
+    """Name kept for drop-in use: "is an FP8 backend available?"  Here the backend
+    is the in-tree HIP library rather than the CUDA package the reference probes
+    for (fp8.py:64-77)."""
+    return is_native_backend_available()
+
+
+def get_transformer_engine_version() -> str | None:
+    if not is_native_backend_available():
+        return None
+    from ... import __version__
+
+    return f"odl-fp8-{__version__}"
+
+
+def get_fp8_format_from_string(format_str: str) -> Fp8Format:
+    key = format_str.lower()
+    for fmt, names in _FORMAT_ALIASES.items():
+        if key in names:
+            return fmt
+    raise ValueError(f"Unknown FP8 format: {format_str}. Supported formats: hybrid, e4m3, e5m2")
+
+
+def get_fp8_recipe_type_from_string(recipe_str: str) -> Fp8RecipeType:
+    key = recipe_str.lower()
+    for rt, names in _RECIPE_ALIASES.items():
+        if key in names:
+            return rt
+    raise ValueError(f"Unknown FP8 recipe type: {recipe_str}. Supported types: delayed, tensorwise, blockwise, mxfp8")
+
+
+@dataclass
+class Fp8RecipeConfig:
+    recipe_type: str = "delayed"
+    format: str = "hybrid"
+    margin: int = 0
+    amax_history_len: int = 1024
+    amax_compute_algo: str = "max"
+    reduce_amax: bool = True
+    fp8_dpa: bool = False
+    fp8_mha: bool = False
+
+
+@dataclass(frozen=True)
+class ScalingPolicy:
+    """What ``FP8Recipe.recipe`` returns: the resolved policy the kernels follow."""
+
+    kind: str                 # "delayed" | "tensorwise" | "rowwise"
+    fmt_fwd: int              # native.E4M3 / native.E5M2 for activations and weights
+    fmt_bwd: int              # ... for gradients
+    margin: int
+    amax_history_len: int
+    amax_compute_algo: str    # "max" | "most_recent"
+    reduce_amax: bool         # one GPU: the cross-rank MAX all-reduce is a no-op
+
+
+class FP8Recipe:
+    """Scaling recipe + the contexts that switch FP8 on for the Linear modules."""
+
+    def __init__(
+        self,
+        recipe_type: str | Fp8RecipeType = Fp8RecipeType.DELAYED,
+        format: str | Fp8Format = Fp8Format.HYBRID,
+        margin: int = 0,
+        amax_history_len: int = 1024,
+        amax_compute_algo: str = "max",
+        reduce_amax: bool = True,
+        fp8_dpa: bool = False,
+        fp8_mha: bool = False,
+        wgrad: bool = True,
+    ):
+        if not is_native_backend_available():
+            raise ImportError(
+                "The FP8 kernel library (libodl_fp8.so) and a visible MI355X are required for FP8 training. "
+                "Build the library with: python -m optimus_dl_amd.build"
+            )
+        self.recipe_type = get_fp8_recipe_type_from_string(recipe_type) if isinstance(recipe_type, str) else recipe_type
+        self.format = get_fp8_format_from_string(format) if isinstance(format, str) else format
+        self.margin = margin
+        self.amax_history_len = amax_history_len
+        self.amax_compute_algo = amax_compute_algo
+        self.reduce_amax = reduce_amax
+        self.fp8_dpa = fp8_dpa
+        self.fp8_mha = fp8_mha
+        self.wgrad = wgrad
+
+        if self.format == Fp8Format.HYBRID:
+            fwd, bwd = native.E4M3, native.E5M2
+        elif self.format == Fp8Format.E4M3:
+            fwd, bwd = native.E4M3, native.E4M3
+        elif self.format == Fp8Format.E5M2:
+            if self.recipe_type == Fp8RecipeType.DELAYED:
+                raise ValueError(
+                    "Pure E5M2 format is not supported by delayed recipe. Please use 'hybrid' or 'e4m3' format instead."
+                )
+            fwd, bwd = native.E5M2, native.E5M2
+        else:
+            raise ValueError(f"Unsupported FP8 format: {self.format}")
+        if amax_compute_algo not in ("max", "most_recent"):
+            raise ValueError(f"Unsupported amax_compute_algo: {amax_compute_algo} (max, most_recent)")
+        if self.recipe_type in (Fp8RecipeType.BLOCKWISE, Fp8RecipeType.MXFP8):
+            raise NotImplementedError(
+                f"FP8 recipe '{self.recipe_type.value}' has no MI355X kernels in this build; "
+                "use delayed, tensorwise or rowwise"
+            )
+        if amax_history_len < 1:
+            raise ValueError("amax_history_len must be >= 1")
+        self._recipe = ScalingPolicy(
+            kind=self.recipe_type.value, fmt_fwd=fwd, fmt_bwd=bwd, margin=margin,
+            amax_history_len=amax_history_len, amax_compute_algo=amax_compute_algo, reduce_amax=reduce_amax,
+        )
+        self._store = _state.MetaStore(amax_history_len)
+        self._depth = 0
+        _info_once(
+            f"Created FP8 recipe with format={self.format.value}, amax_history_len={amax_history_len}, "
+            f"amax_compute_algo={amax_compute_algo}"
+        )
+
+    # ------------------------------------------------------------------ policy
+    @property
+    def recipe(self) -> ScalingPolicy:
+        return self._recipe
+
+    @property
+    def is_delayed(self) -> bool:
+        return self._recipe.kind == "delayed"
+
+    def reserve_meta(self, device: torch.device, direction: str, fmts: list[int]) -> "_state.ScalingMeta":
+        return self._store.reserve(device, direction, fmts)
+
+    def update_scales(self, direction: str) -> None:
+        """Roll the histories of every role that saw a cast since the last update
+        and refresh their scales: one small kernel per arena."""
+        if not self.is_delayed:
+            return
+        algo = native.AMAX_MAX if self.amax_compute_algo == "max" else native.AMAX_MOST_RECENT
+        for arena in self._store.dirty_arenas(direction):
+            R = arena.used
+            native.delayed_update_raw(arena.history, arena.H, arena.capacity, R, arena.scale, arena.scale_inv,
+                                      arena.fmt, self.margin, algo)
+            arena.dirty = False
+
+    def state_dict(self) -> dict:
+        """Scaling state (histories and scales) of every role registered so far,
+        as CPU tensors; roles are in module-registration order."""
+        out = {}
+        for (dev, direction), chain in self._store.arenas.items():
+            out[f"{dev}/{direction}"] = [
+                {"used": a.used, "history": a.history[:, :a.used].cpu(), "scale": a.scale[:a.used].cpu(),
+                 "scale_inv": a.scale_inv[:a.used].cpu()} for a in chain]
+        return out
+
+    def load_state_dict(self, state: dict) -> None:
+        for key, blobs in state.items():
+            dev, direction = key.rsplit("/", 1)
+            chain = self._store.arenas.get((dev, direction), [])
+            for arena, blob in zip(chain, blobs):
+                n = min(arena.used, blob["used"])
+                if blob["history"].shape[0] != arena.H:
+                    raise ValueError("amax_history_len of the checkpoint differs from this recipe")
+                arena.history[:, :n].copy_(blob["history"][:, :n])
+                arena.scale[:n].copy_(blob["scale"][:n])
+                arena.scale_inv[:n].copy_(blob["scale_inv"][:n])
+
+    # ---------------------------------------------------------------- contexts
+    @contextmanager
+    def autocast(self) -> Iterator[None]:
+        """Forward context: FP8 Linears quantise while it is active.  Leaving the
+        outermost one refreshes the forward scales (delayed scaling)."""
+        _state.push_recipe(self)
+        self._depth += 1
+        try:
+            yield
+        finally:
+            self._depth -= 1
+            _state.pop_recipe()
+            if self._depth == 0:
+                self.update_scales("fwd")
+                # gradients recorded by a backward that ran outside any backward()
+                # context are folded in here, one step late but never lost
+                self.update_scales("bwd")
+
+    @contextmanager
+    def backward(self) -> Iterator[None]:
+        """Backward context: leaving it refreshes the gradient scales."""
+        _state.push_recipe(self)
+        self._depth += 1
+        try:
+            yield
+        finally:
+            self._depth -= 1
+            _state.pop_recipe()
+            if self._depth == 0:
+                self.update_scales("bwd")
+
+    def prepare_for_backward(self, *args: Any, **kwargs: Any) -> tuple[Any, ...]:
+        return args
+
+    def prepare(self, *args: Any, **kwargs: Any) -> tuple[Any, ...]:
+        return args
+
+
+def create_fp8_recipe(
+    recipe_type: str | Fp8RecipeType = Fp8RecipeType.DELAYED,
+    format: str | Fp8Format = Fp8Format.HYBRID,
+    margin: int = 0,
+    amax_history_len: int = 1024,
+    amax_compute_algo: str = "max",
+    reduce_amax: bool = True,
+    fp8_dpa: bool = False,
+    fp8_mha: bool = False,
+    wgrad: bool = True,
+) -> FP8Recipe | None:
+    """FP8Recipe when the backend is usable, else None (callers fall back to bf16 AMP)."""
+    if not is_native_backend_available():
+        logger.warning(
+            "FP8 backend not available (libodl_fp8.so missing or no GPU). FP8 training will be disabled. "
+            "Build with: python -m optimus_dl_amd.build"
+        )
+        return None
+    return FP8Recipe(recipe_type=recipe_type, format=format, margin=margin, amax_history_len=amax_history_len,
+                     amax_compute_algo=amax_compute_algo, reduce_amax=reduce_amax, fp8_dpa=fp8_dpa, fp8_mha=fp8_mha,
+                     wgrad=wgrad)
+
+
+@contextmanager
+def fp8_autocast(device: torch.device, fp8_recipe: FP8Recipe | None, enabled: bool = True,
+                 dtype: torch.dtype | None = None) -> Iterator[None]:
+    """FP8 autocast outside, ordinary AMP autocast inside (for everything that is
+    not an FP8 Linear); plain AMP when there is no recipe or no GPU."""
+    if not enabled:
+        yield
+        return
+    if dtype is None:
+        dtype = torch.bfloat16
+    if fp8_recipe is not None and device.type == "cuda":
+        with fp8_recipe.autocast():
+            with torch.autocast(device.type, dtype=dtype, enabled=True):
+                yield
+    else:
+        with torch.autocast(device.type, dtype=dtype, enabled=True):
+            yield
+
+
+@contextmanager
+def fp8_backward(fp8_recipe: FP8Recipe | None, enabled: bool = True) -> Iterator[None]:
+    if not enabled or fp8_recipe is None:
+        yield
+        return
+    with fp8_recipe.backward():
+        yield

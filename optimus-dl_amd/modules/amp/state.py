@@ -1,0 +1,128 @@
+"""Process-wide FP8 state: which recipe is active, and the scaling-factor storage.
+
+Counterpart of what the reference leaves to its third-party backend when it
+enters ``te.pytorch.autocast(enabled=True, recipe=...)``
+(optimus_dl/modules/amp/fp8.py:337-340,357-360): a global "FP8 is on, with this
+recipe" flag that FP8 modules consult in forward, and the amax-history / scale
+tensors that delayed scaling refreshes when the outermost context exits.
+
+Design for one MI355X:
+  * the active-recipe stack is a plain module global guarded by a lock, so the
+    autograd worker thread sees the same state as the thread that entered the
+    context (a thread-local would not); backward additionally carries its recipe
+    in the autograd ``ctx`` and never depends on the ambient state;
+  * all delayed-scaling roles of all modules live in ONE arena per (recipe,
+    device, direction): history [H, R], scale [R], scale_inv [R].  Casts write
+    their amax straight into row 0 of the arena and a single tiny kernel
+    refreshes every role of the model per step.
+"""
+
+from __future__ import annotations
+
+import threading
+from typing import TYPE_CHECKING
+
+import torch
+
+if TYPE_CHECKING:  # pragma: no cover
+    from .fp8 import FP8Recipe
+
+_lock = threading.RLock()
+_stack: list["FP8Recipe"] = []
+
+
+def push_recipe(recipe: "FP8Recipe") -> int:
+    with _lock:
+        _stack.append(recipe)
+        return len(_stack)
+
+
+def pop_recipe() -> int:
+    with _lock:
+        _stack.pop()
+        return len(_stack)
+
+
+def active_recipe() -> "FP8Recipe | None":
+    with _lock:
+        return _stack[-1] if _stack else None
+
+
+def is_fp8_active() -> bool:
+    return active_recipe() is not None
+
+
+class ScalingMeta:
+    """View of ``n`` consecutive roles of an arena; mirrors the attribute names
+    (``amax_history``, ``scale``, ``scale_inv``) that the reference's own FP8 test
+    inspects on its backend modules (tests/optim/test_fp8.py:609-625)."""
+
+    def __init__(self, arena: "MetaArena", first: int, n: int):
+        self.arena, self.first, self.n = arena, first, n
+
+    @property
+    def amax_history(self) -> torch.Tensor:          # [H, n] view
+        return self.arena.history[:, self.first:self.first + self.n]
+
+    @property
+    def scale(self) -> torch.Tensor:
+        return self.arena.scale[self.first:self.first + self.n]
+
+    @property
+    def scale_inv(self) -> torch.Tensor:
+        return self.arena.scale_inv[self.first:self.first + self.n]
+
+    def amax_slot(self, role: int) -> torch.Tensor:   # 1-element view: where a cast records this step's amax
+        return self.arena.history[0, self.first + role:self.first + role + 1]
+
+    def scale_of(self, role: int) -> torch.Tensor:
+        return self.arena.scale[self.first + role:self.first + role + 1]
+
+    def scale_inv_of(self, role: int) -> torch.Tensor:
+        return self.arena.scale_inv[self.first + role:self.first + role + 1]
+
+
+class MetaArena:
+    """history [H, cap], scale [cap], scale_inv [cap], fmt [cap] for one direction."""
+
+    def __init__(self, device: torch.device, history_len: int, capacity: int):
+        self.device, self.H, self.capacity = device, history_len, capacity
+        self.history = torch.zeros((history_len, capacity), dtype=torch.float32, device=device)
+        self.scale = torch.ones(capacity, dtype=torch.float32, device=device)
+        self.scale_inv = torch.ones(capacity, dtype=torch.float32, device=device)
+        self.fmt = torch.zeros(capacity, dtype=torch.int32, device=device)
+        self.used = 0
+        self.dirty = False         # some cast wrote an amax since the last update
+
+    def reserve(self, fmts: list[int]) -> ScalingMeta | None:
+        n = len(fmts)
+        if self.used + n > self.capacity:
+            return None
+        first = self.used
+        self.fmt[first:first + n] = torch.tensor(fmts, dtype=torch.int32, device=self.device)
+        self.used += n
+        return ScalingMeta(self, first, n)
+
+
+class MetaStore:
+    """All arenas of one recipe.  Arenas are never reallocated (modules hold views
+    into them), a full one is followed by a new one."""
+
+    CAPACITY = 2048
+
+    def __init__(self, history_len: int):
+        self.history_len = history_len
+        self.arenas: dict[tuple[str, str], list[MetaArena]] = {}
+
+    def reserve(self, device: torch.device, direction: str, fmts: list[int]) -> ScalingMeta:
+        key = (str(device), direction)
+        chain = self.arenas.setdefault(key, [])
+        if chain:
+            meta = chain[-1].reserve(fmts)
+            if meta is not None:
+                return meta
+        chain.append(MetaArena(device, self.history_len, self.CAPACITY))
+        return chain[-1].reserve(fmts)
+
+    def dirty_arenas(self, direction: str) -> list[MetaArena]:
+        return [a for (dev, d), chain in self.arenas.items() if d == direction for a in chain if a.dirty and a.used]

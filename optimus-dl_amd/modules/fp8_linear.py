@@ -1,0 +1,302 @@
+"""FP8Linear: an ``nn.Linear`` whose matmuls run as FP8 MFMA GEMMs on MI355X.
+
+Stands in for the reference's ``TELinear`` wrapper
+(optimus_dl/modules/model_transforms/transformer_engine.py:63-111), which nests
+a third-party ``te.pytorch.Linear``.  Differences that matter to callers:
+
+  * it IS an ``nn.Linear`` (subclass) and, when made from an existing layer,
+    keeps the very same ``Parameter`` objects.  State-dict keys stay
+    ``<name>.weight`` / ``<name>.bias`` (the reference's wrapper renames them to
+    ``<name>._te_linear.weight``), weight tying (``lm_head`` <-> ``wte``) survives,
+    and code that selects parameters with ``isinstance(m, nn.Linear)`` keeps working;
+  * outside an FP8 autocast context, on CPU, or for shapes the kernels cannot
+    take (features or tokens not multiples of 16) it behaves as a plain Linear.
+
+Per call, inside ``FP8Recipe.autocast()``:
+
+  forward   Y  = Q(X)  . Q(W)^T      X, W -> E4M3 (format "hybrid"/"e4m3")
+  backward  dX = Q(dY) . Q(W)        dY   -> E5M2 ("hybrid") or E4M3
+            dW = Q(dY)^T . Q(X)
+            db = sum_rows(dY)        (fp32 accumulate)
+
+Every GEMM is issued in the "NT" form the MFMA wants (both operands contiguous
+along the contraction axis); the cast+transpose kernel supplies the transposed
+FP8 copies, and the forward keeps only the 1-byte ``Q(X)^T`` for wgrad instead of
+the 2-byte activation.  Quantised weights (and their transposes) are cached until
+the parameter changes, so gradient-accumulation microbatches and evaluation
+re-quantise nothing.
+"""
+
+from __future__ import annotations
+
+import logging
+from typing import Any
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .. import native
+from .amp import state as _state
+from .amp.fp8 import FP8Recipe
+
+logger = logging.getLogger(__name__)
+_warned: set[str] = set()
+
+ROLE_X, ROLE_W, ROLE_Y = 0, 1, 2      # forward roles (Y is reserved: outputs stay bf16)
+ROLE_G, ROLE_DX = 0, 1                # backward roles (dX reserved likewise)
+T, R, C = native.SCALE_TENSOR, native.SCALE_ROW, native.SCALE_COL
+
+
+def _warn_once(msg: str) -> None:
+    if msg not in _warned:
+        _warned.add(msg)
+        logger.warning(msg)
+
+
+class _WeightCache:
+    """Quantised weight + transpose, valid while the Parameter is unchanged."""
+
+    __slots__ = ("key", "wq", "wq_t", "s_inv", "s_inv_t", "amax")
+
+    def __init__(self):
+        self.key = None
+        self.wq = self.wq_t = self.s_inv = self.s_inv_t = self.amax = None
+
+
+def _quantise_dynamic(x2d: torch.Tensor, fmt: int, margin: int, need_t: bool, need_rowmajor: bool = True):
+    """Per-tensor current scaling: amax pass, scale, cast (+transpose) pass."""
+    amax = native.amax(x2d, T)
+    scale, scale_inv = native.scale_from_amax(amax, fmt, margin)
+    if need_t:
+        q, q_t = native.cast_transpose(x2d, scale, fmt, T, want_rowmajor=need_rowmajor)
+    else:
+        q, q_t = native.cast(x2d, scale, fmt, T), None
+    return q, q_t, scale_inv, amax
+
+
+def _quantise_delayed(x2d: torch.Tensor, fmt: int, meta: "_state.ScalingMeta", role: int, need_t: bool,
+                      need_rowmajor: bool = True):
+    """Delayed scaling: one pass with the scale from the history, amax recorded in row 0."""
+    scale, slot = meta.scale_of(role), meta.amax_slot(role)
+    meta.arena.dirty = True
+    # the inverse scale is snapshotted: the arena entry changes at the next update
+    scale_inv = meta.scale_inv_of(role).clone()
+    if need_t:
+        q, q_t = native.cast_transpose(x2d, scale, fmt, T, amax_out=slot, want_rowmajor=need_rowmajor)
+    else:
+        q, q_t = native.cast(x2d, scale, fmt, T, amax_out=slot), None
+    return q, q_t, scale_inv
+
+
+def _quantise_axis(x2d: torch.Tensor, fmt: int, margin: int, mode: int, transposed: bool):
+    """Rowwise recipe: one scale per row (mode R) or per column (mode C) of x2d.
+    Returns the codes (transposed when asked) and the inverse scale vector."""
+    amax = native.amax(x2d, mode)
+    scale, scale_inv = native.scale_from_amax(amax, fmt, margin)
+    if transposed:
+        _, q = native.cast_transpose(x2d, scale, fmt, mode, want_rowmajor=False)
+    else:
+        q = native.cast(x2d, scale, fmt, mode)
+    return q, scale_inv
+
+
+class _Fp8LinearFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x2d: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, module: "FP8Linear",
+                recipe: FP8Recipe, out_dtype: torch.dtype):
+        pol = recipe.recipe
+        need_dgrad, need_wgrad = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        bias_f32 = None if bias is None else bias.detach().float()
+        saved: dict[str, Any] = {}
+
+        if pol.kind == "rowwise":
+            xq, sx_inv = _quantise_axis(x2d, pol.fmt_fwd, pol.margin, R, False)
+            wq, sw_inv = module._rowwise_weight(weight, pol, "row")
+            y = native.gemm_nt(xq, wq, pol.fmt_fwd, pol.fmt_fwd, sx_inv, sw_inv, bias=bias_f32, out_dtype=out_dtype)
+            if need_wgrad and recipe.wgrad:
+                saved["xq_t"], saved["sx_inv_t"] = _quantise_axis(x2d, pol.fmt_fwd, pol.margin, C, True)
+        else:
+            if pol.kind == "delayed":
+                meta = module._meta(recipe, x2d.device, "fwd")
+                xq, xq_t, sx_inv = _quantise_delayed(x2d, pol.fmt_fwd, meta, ROLE_X, need_wgrad and recipe.wgrad)
+            else:
+                xq, xq_t, sx_inv, _ = _quantise_dynamic(x2d, pol.fmt_fwd, pol.margin, need_wgrad and recipe.wgrad)
+            wq, wq_t, sw_inv = module._tensor_weight(weight, recipe, need_t=need_dgrad)
+            y = native.gemm_nt(xq, wq, pol.fmt_fwd, pol.fmt_fwd, sx_inv, sw_inv, bias=bias_f32, out_dtype=out_dtype)
+            if need_wgrad and recipe.wgrad:
+                saved["xq_t"], saved["sx_inv_t"] = xq_t, sx_inv
+            if need_dgrad:
+                saved["wq_t"], saved["sw_inv_t"] = wq_t, sw_inv
+        if need_wgrad and not recipe.wgrad:
+            saved["x_hp"] = x2d                      # wgrad=False: weight gradient in the activation dtype
+        ctx.module, ctx.recipe, ctx.saved = module, recipe, saved
+        ctx.need_wgrad, ctx.need_dgrad, ctx.has_bias = need_wgrad, need_dgrad, bias is not None
+        ctx.x_dtype, ctx.w_dtype = x2d.dtype, weight.dtype
+        ctx.bias_dtype = None if bias is None else bias.dtype
+        ctx.weight_ref = weight if pol.kind == "rowwise" and need_dgrad else None
+        return y
+
+    @staticmethod
+    def backward(ctx, dy: torch.Tensor):
+        module, recipe, saved = ctx.module, ctx.recipe, ctx.saved
+        pol = recipe.recipe
+        dy2d = dy if dy.is_contiguous() else dy.contiguous()
+        if dy2d.dtype not in (torch.bfloat16, torch.float32):
+            dy2d = dy2d.to(torch.bfloat16)
+        dx = dw = db = None
+        fp8_wgrad = ctx.need_wgrad and recipe.wgrad
+
+        if pol.kind == "rowwise":
+            if ctx.need_dgrad:
+                gq, sg_inv = _quantise_axis(dy2d, pol.fmt_bwd, pol.margin, R, False)
+                wq_t, sw_inv_t = module._rowwise_weight(ctx.weight_ref, pol, "col")
+                dx = native.gemm_nt(gq, wq_t, pol.fmt_bwd, pol.fmt_fwd, sg_inv, sw_inv_t, out_dtype=ctx.x_dtype)
+            if fp8_wgrad:
+                gq_t, sg_inv_t = _quantise_axis(dy2d, pol.fmt_bwd, pol.margin, C, True)
+                dw = native.gemm_nt(gq_t, saved["xq_t"], pol.fmt_bwd, pol.fmt_fwd, sg_inv_t, saved["sx_inv_t"],
+                                    out_dtype=ctx.w_dtype)
+        else:
+            if ctx.need_dgrad or fp8_wgrad:
+                if pol.kind == "delayed":
+                    meta = module._meta(recipe, dy2d.device, "bwd")
+                    gq, gq_t, sg_inv = _quantise_delayed(dy2d, pol.fmt_bwd, meta, ROLE_G, fp8_wgrad, ctx.need_dgrad)
+                else:
+                    gq, gq_t, sg_inv, _ = _quantise_dynamic(dy2d, pol.fmt_bwd, pol.margin, fp8_wgrad, ctx.need_dgrad)
+            if ctx.need_dgrad:
+                dx = native.gemm_nt(gq, saved["wq_t"], pol.fmt_bwd, pol.fmt_fwd, sg_inv, saved["sw_inv_t"],
+                                    out_dtype=ctx.x_dtype)
+            if fp8_wgrad:
+                dw = native.gemm_nt(gq_t, saved["xq_t"], pol.fmt_bwd, pol.fmt_fwd, sg_inv, saved["sx_inv_t"],
+                                    out_dtype=ctx.w_dtype)
+        if ctx.need_wgrad and not recipe.wgrad:
+            dw = (dy2d.t().to(saved["x_hp"].dtype) @ saved["x_hp"]).to(ctx.w_dtype)
+        if ctx.has_bias:
+            db = dy2d.sum(dim=0, dtype=torch.float32).to(ctx.bias_dtype)
+        return dx, dw, db, None, None, None
+
+
+class FP8Linear(nn.Linear):
+    """Drop-in ``nn.Linear`` with an FP8 fast path (see the module docstring)."""
+
+    def __init__(self, in_features: int, out_features: int, bias: bool = True, device=None, dtype=None, **kwargs: Any):
+        super().__init__(in_features, out_features, bias=bias, device=device, dtype=dtype)
+        self.use_bias = bias
+        self.kwargs = dict(kwargs)           # backend-specific options (e.g. sequence_parallel): accepted, unused on one GPU
+        self._init_fp8_state()
+
+    def _init_fp8_state(self) -> None:
+        self._wcache = _WeightCache()
+        self._wcache_rowwise: dict[str, tuple] = {}
+        self._metas: dict[tuple[int, str, str], "_state.ScalingMeta"] = {}
+        self.fp8_meta: dict[str, "_state.ScalingMeta"] = {}
+        self.fp8_calls = 0                   # forwards that actually took the FP8 path (for tests / logging)
+
+    @classmethod
+    def from_linear(cls, linear: nn.Linear, **kwargs: Any) -> "FP8Linear":
+        """Re-wrap an existing layer, SHARING its Parameter objects."""
+        new = cls.__new__(cls)
+        nn.Module.__init__(new)
+        new.in_features, new.out_features = linear.in_features, linear.out_features
+        new.weight = linear.weight
+        if linear.bias is not None:
+            new.bias = linear.bias
+        else:
+            new.register_parameter("bias", None)
+        new.use_bias = linear.bias is not None
+        new.kwargs = dict(kwargs)
+        new.training = linear.training
+        new._init_fp8_state()
+        return new
+
+    @property
+    def _te_linear(self) -> "FP8Linear":
+        """The reference nests the backend layer under this name; here it is the module itself."""
+        return self
+
+    # ------------------------------------------------------------ scaling state
+    def _meta(self, recipe: FP8Recipe, device: torch.device, direction: str) -> "_state.ScalingMeta":
+        key = (id(recipe), str(device), direction)
+        meta = self._metas.get(key)
+        if meta is None:
+            pol = recipe.recipe
+            fmts = [pol.fmt_fwd] * 3 if direction == "fwd" else [pol.fmt_bwd] * 2
+            meta = recipe.reserve_meta(device, direction, fmts)
+            self._metas[key] = meta
+            self.fp8_meta["scaling_fwd" if direction == "fwd" else "scaling_bwd"] = meta
+        return meta
+
+    def _tensor_weight(self, weight: torch.Tensor, recipe: FP8Recipe, need_t: bool):
+        """Per-tensor quantised weight (and transpose), cached on the parameter version."""
+        pol = recipe.recipe
+        c = self._wcache
+        key = (weight.data_ptr(), weight._version, id(recipe), pol.kind)
+        fresh = c.key != key
+        if fresh or (need_t and c.wq_t is None):
+            w2d = weight.detach()
+            if pol.kind == "delayed":
+                meta = self._meta(recipe, weight.device, "fwd")
+                c.wq, c.wq_t, c.s_inv = _quantise_delayed(w2d, pol.fmt_fwd, meta, ROLE_W, need_t)
+                c.amax = meta.amax_slot(ROLE_W).clone()      # only this weight ever writes that slot
+            else:
+                c.wq, c.wq_t, c.s_inv, c.amax = _quantise_dynamic(w2d, pol.fmt_fwd, pol.margin, need_t)
+            c.key = key
+        elif pol.kind == "delayed":
+            # cached codes are reused; this step's history still has to see the weight's amax
+            meta = self._meta(recipe, weight.device, "fwd")
+            slot = meta.amax_slot(ROLE_W)
+            torch.maximum(slot, c.amax, out=slot)
+            meta.arena.dirty = True
+        return c.wq, c.wq_t, c.s_inv
+
+    def _rowwise_weight(self, weight: torch.Tensor, pol, axis: str):
+        """Rowwise recipe: W scaled per output channel (fwd) or per input channel, transposed (dgrad)."""
+        key = (weight.data_ptr(), weight._version)
+        hit = self._wcache_rowwise.get(axis)
+        if hit is not None and hit[0] == key:
+            return hit[1], hit[2]
+        w2d = weight.detach()
+        if axis == "row":
+            q, s_inv = _quantise_axis(w2d, pol.fmt_fwd, pol.margin, R, False)
+        else:
+            q, s_inv = _quantise_axis(w2d, pol.fmt_fwd, pol.margin, C, True)
+        self._wcache_rowwise[axis] = (key, q, s_inv)
+        return q, s_inv
+
+    # ------------------------------------------------------------------ forward
+    def _fp8_eligible(self, x: torch.Tensor) -> bool:
+        if not x.is_cuda or not self.weight.is_cuda:
+            return False
+        if self.weight.dtype not in (torch.bfloat16, torch.float32):
+            _warn_once(f"FP8Linear: weight dtype {self.weight.dtype} is not bf16/fp32; running as a plain Linear")
+            return False
+        tokens = x.numel() // max(self.in_features, 1)
+        if self.in_features % 16 or self.out_features % 16 or tokens % 16 or tokens == 0:
+            _warn_once(
+                f"FP8Linear({self.in_features}->{self.out_features}) with {tokens} tokens: sizes must be multiples "
+                "of 16 for the FP8 kernels; this call runs as a plain Linear"
+            )
+            return False
+        return True
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        recipe = _state.active_recipe()
+        if recipe is None or not self._fp8_eligible(x):
+            return F.linear(x, self.weight, self.bias)
+        if torch.is_autocast_enabled("cuda"):
+            compute_dtype = torch.get_autocast_dtype("cuda")
+        else:
+            compute_dtype = x.dtype
+        if compute_dtype not in (torch.bfloat16, torch.float32):
+            compute_dtype = torch.bfloat16
+        x2d = x.reshape(-1, self.in_features)
+        if x2d.dtype != compute_dtype:
+            x2d = x2d.to(compute_dtype)
+        if not x2d.is_contiguous():
+            x2d = x2d.contiguous()
+        self.fp8_calls += 1
+        y = _Fp8LinearFn.apply(x2d, self.weight, self.bias, self, recipe, compute_dtype)
+        return y.reshape(*x.shape[:-1], self.out_features)
+
+    def extra_repr(self) -> str:
+        return f"in_features={self.in_features}, out_features={self.out_features}, bias={self.bias is not None}, fp8=True"

@@ -77,7 +77,7 @@ def load() -> ctypes.CDLL:
         L.odl_fp8_cast.argtypes = [vp, i32, i64, i64, vp, i32, i32, vp, vp, vp]
         L.odl_fp8_cast_transpose.argtypes = [vp, i32, i64, i64, vp, i32, i32, vp, vp, vp, vp]
         L.odl_fp8_gemm_nt.argtypes = [vp, vp, i64, i64, i64, i32, i32, vp, i64, vp, i64, vp, i32, vp, i32, vp]
-        L.odl_fp8_delayed_update.argtypes = [vp, i64, i64, vp, vp, vp, i32, i32, vp]
+        L.odl_fp8_delayed_update.argtypes = [vp, i64, i64, i64, vp, vp, vp, i32, i32, vp]
         L.odl_fp8_gemm_num_variants.restype = i32
         L.odl_fp8_gemm_variant_name.argtypes = [i32]
         L.odl_fp8_gemm_variant_name.restype = ctypes.c_char_p
@@ -225,8 +225,22 @@ def delayed_update(history: torch.Tensor, scale: torch.Tensor, scale_inv: torch.
     _f32_dev(scale_inv, R, "delayed_update scale_inv")
     if not (fmts.is_cuda and fmts.dtype == torch.int32 and fmts.numel() == R and fmts.is_contiguous()):
         raise NativeError("delayed_update: fmts must be a contiguous int32 CUDA tensor with R entries")
-    _check(load().odl_fp8_delayed_update(history.data_ptr(), H, R, scale.data_ptr(), scale_inv.data_ptr(), fmts.data_ptr(),
+    _check(load().odl_fp8_delayed_update(history.data_ptr(), H, R, R, scale.data_ptr(), scale_inv.data_ptr(), fmts.data_ptr(),
                                          margin, algo, _stream()), "odl_fp8_delayed_update")
+
+
+def delayed_update_raw(history: torch.Tensor, H: int, ld: int, R: int, scale: torch.Tensor, scale_inv: torch.Tensor,
+                       fmts: torch.Tensor, margin: int, algo: int) -> None:
+    """Same update on the first R roles of an arena whose rows are ld >= R wide."""
+    if not (history.is_cuda and history.dtype == torch.float32 and history.is_contiguous() and history.numel() == H * ld):
+        raise NativeError("delayed_update_raw: history must be a contiguous fp32 CUDA tensor of H*ld elements")
+    for t, name in ((scale, "scale"), (scale_inv, "scale_inv")):
+        if not (t.is_cuda and t.dtype == torch.float32 and t.is_contiguous() and t.numel() >= R):
+            raise NativeError(f"delayed_update_raw: {name} must be a contiguous fp32 CUDA tensor with >= R entries")
+    if not (fmts.is_cuda and fmts.dtype == torch.int32 and fmts.is_contiguous() and fmts.numel() >= R):
+        raise NativeError("delayed_update_raw: fmts must be a contiguous int32 CUDA tensor with >= R entries")
+    _check(load().odl_fp8_delayed_update(history.data_ptr(), H, R, ld, scale.data_ptr(), scale_inv.data_ptr(),
+                                         fmts.data_ptr(), margin, algo, _stream()), "odl_fp8_delayed_update")
 
 
 def gemm_variants() -> list[str]:

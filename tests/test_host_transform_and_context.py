@@ -1,0 +1,236 @@
+"""Host-side behaviour of the transform and the training-context decision table
+(no GPU needed).  Mirrors what the reference's tests check with mocks:
+tests/model/test_transformer_engine_transform.py:206-229 (disabled => identity),
+:231-295,:322-403 (top-level and nested swaps, in place);
+tests/optim/test_fp8_context.py:31-53 (dict keys), :152-228 (fallbacks, scaler off)."""
+from contextlib import nullcontext
+
+import pytest
+import torch
+import torch.nn as nn
+
+from optimus_dl_amd.core.registry import RegistryConfig, RegistryConfigStrict, make_registry
+from optimus_dl_amd.modules.amp import AmpConfig, Fp8Config, OptimizationConfig, fp8_autocast, fp8_backward
+from optimus_dl_amd.modules.fp8_linear import FP8Linear
+from optimus_dl_amd.modules.model import GPT2, GPT2Config, Llama, LlamaConfig, Qwen3, Qwen3Config
+from optimus_dl_amd.modules.model_transforms import build_model_transform
+from optimus_dl_amd.modules.model_transforms import fp8_linear_transform as T
+from optimus_dl_amd.recipe import TrainingContext, execute_backward_pass, execute_forward_pass
+
+
+class Nested(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.fc = nn.Linear(16, 32)
+        self.inner = nn.Sequential(nn.Linear(32, 32, bias=False), nn.LayerNorm(32), nn.ModuleList([nn.Linear(32, 16)]))
+
+    def forward(self, x):
+        return self.inner[2][0](self.inner[1](self.inner[0](self.fc(x))))
+
+
+class MyLinear(nn.Linear):
+    pass
+
+
+def test_disabled_is_identity():
+    m = Nested()
+    before = {n: id(mod) for n, mod in m.named_modules()}
+    out = build_model_transform({"_name": "transformer_engine", "enabled": False}).apply(m, device=None, collective=None)
+    assert out is m and before == {n: id(mod) for n, mod in m.named_modules()}
+
+
+def test_backend_missing_is_identity(monkeypatch):
+    monkeypatch.setattr(T, "_HAVE_TE", False)
+    m = Nested()
+    out = build_model_transform({"_name": "transformer_engine"}).apply(m)
+    assert out is m and type(m.fc) is nn.Linear
+
+
+def test_swap_nested_in_place_and_share_parameters(monkeypatch):
+    monkeypatch.setattr(T, "_HAVE_TE", True)
+    m = Nested()
+    m.sub = MyLinear(4, 4)                       # exact class match only: subclasses stay
+    w_before, b_before = m.fc.weight, m.fc.bias
+    keys_before = sorted(m.state_dict().keys())
+    x = torch.randn(3, 16)
+    y_before = m(x)
+    t = build_model_transform({"_name": "transformer_engine", "verbose": True})
+    out = t.apply(m, collective=None, device=torch.device("cpu"), is_restart=False, checkpoint_manager=None)
+    assert out is m
+    assert isinstance(m.fc, FP8Linear) and isinstance(m.inner[0], FP8Linear) and isinstance(m.inner[2][0], FP8Linear)
+    assert type(m.sub) is MyLinear and type(m.inner[1]) is nn.LayerNorm
+    assert t.last_replacements == {"Linear": 3, "RMSNorm": 0, "LayerNorm": 0, "Attention": 0}
+    assert m.fc.weight is w_before and m.fc.bias is b_before                 # same Parameter objects
+    assert sorted(m.state_dict().keys()) == keys_before                     # no key renames
+    assert m.inner[0].bias is None and m.fc.in_features == 16 and m.fc.out_features == 32 and m.fc.use_bias is True
+    assert m.fc._te_linear is m.fc
+    torch.testing.assert_close(m(x), y_before)                              # outside FP8 autocast: a plain Linear
+    assert isinstance(m.fc, nn.Linear)
+
+
+def test_replace_linear_false_and_not_inplace(monkeypatch):
+    monkeypatch.setattr(T, "_HAVE_TE", True)
+    m = Nested()
+    build_model_transform({"_name": "fp8_linear", "replace_linear": False}).apply(m)
+    assert type(m.fc) is nn.Linear
+    t = build_model_transform({"_name": "fp8_linear", "replace_inplace": False})
+    t.apply(m)
+    assert type(m.fc) is nn.Linear and t.last_replacements["Linear"] == 3    # counted, not installed
+
+
+def test_linear_kwargs_are_forwarded(monkeypatch):
+    monkeypatch.setattr(T, "_HAVE_TE", True)
+    m = Nested()
+    build_model_transform({"_name": "transformer_engine", "linear_kwargs": {"sequence_parallel": True}}).apply(m)
+    assert m.fc.kwargs == {"sequence_parallel": True}
+
+
+@pytest.mark.parametrize("family", ["llama", "qwen3", "gpt2"])
+def test_swap_on_model_families(monkeypatch, family):
+    monkeypatch.setattr(T, "_HAVE_TE", True)
+    if family == "llama":
+        m = Llama(LlamaConfig(vocab_size=256, n_layer=2, n_head=4, n_kv_head=2, n_embd=64, intermediate_size=128))
+        per_block, tied = 7, False
+    elif family == "qwen3":
+        m = Qwen3(Qwen3Config(vocab_size=256, n_layer=2, n_head=4, n_kv_head=2, n_embd=64, head_dim=32, intermediate_size=128))
+        per_block, tied = 7, True
+    else:
+        m = GPT2(GPT2Config(vocab_size=256, n_layer=2, n_head=4, n_embd=64, block_size=32))
+        per_block, tied = 6, True
+    keys = sorted(m.state_dict().keys())
+    n_params = sum(p.numel() for p in m.parameters())
+    t = build_model_transform({"_name": "transformer_engine"})
+    t.apply(m)
+    assert t.last_replacements["Linear"] == 2 * per_block + 1
+    blk = m.transformer.h[0]
+    for name in ("wq", "wk", "wv", "wo"):
+        assert isinstance(getattr(blk.attn, name), FP8Linear)
+    if family == "gpt2":
+        assert isinstance(blk.mlp.c_fc, FP8Linear) and isinstance(blk.mlp.c_proj, FP8Linear)
+    else:
+        assert isinstance(blk.mlp.w1, FP8Linear) and isinstance(blk.mlp.w2, FP8Linear) and isinstance(blk.mlp.c_proj, FP8Linear)
+    assert isinstance(m.lm_head, FP8Linear)
+    assert (m.transformer.wte.weight is m.lm_head.weight) == tied           # tying survives the swap
+    assert sorted(m.state_dict().keys()) == keys and sum(p.numel() for p in m.parameters()) == n_params
+    out = m(torch.randint(0, 256, (2, 16)))["logits"]
+    assert out.shape == (2, 16, 256)
+    out.float().mean().backward()
+    assert blk.attn.wq.weight.grad is not None
+
+
+def test_registry_basics():
+    table, register, build = make_registry("unit_test_registry")
+
+    from dataclasses import dataclass
+
+    @dataclass
+    class Cfg(RegistryConfig):
+        a: int = 1
+
+    @dataclass
+    class Strict(RegistryConfigStrict):
+        b: int = 2
+
+    @register("thing", Cfg)
+    class Thing:
+        def __init__(self, cfg, **kw):
+            self.cfg, self.kw = cfg, kw
+
+    @register("strict", Strict)
+    class StrictThing(Thing):
+        pass
+
+    t = build({"_name": "thing", "a": 5, "extra": "x"}, device="d")
+    assert t.cfg.a == 5 and t.cfg["extra"] == "x" and t.kw == {"device": "d"}
+    assert build(Cfg(_name="thing")).cfg.a == 1
+    with pytest.raises(ValueError):
+        build({"_name": "strict", "zzz": 1})
+    with pytest.raises(ValueError, match="unknown"):
+        build({"_name": "nope"})
+    with pytest.raises(ValueError):
+        build({"a": 1})
+    assert build(None) is None
+
+
+# ------------------------------------------------------------- training context
+class FakeCuda:
+    type = "cuda"
+
+
+def opt(dtype, enabled=True, fp8_enabled=True, **fp8):
+    return OptimizationConfig(amp=AmpConfig(enabled=enabled, dtype=dtype, fp8=Fp8Config(enabled=fp8_enabled, **fp8)))
+
+
+def test_context_keys_and_bf16_path():
+    ctx = TrainingContext(opt("torch.bfloat16", fp8_enabled=False)).setup_training_context(torch.device("cpu"))
+    assert set(ctx) == {"scaler", "amp_ctx", "amp_cfg", "device", "fp8_recipe", "fp8_enabled", "is_fp8_dtype", "fp8_backward_ctx"}
+    assert ctx["fp8_recipe"] is None and ctx["fp8_enabled"] is False and ctx["is_fp8_dtype"] is False
+    assert isinstance(ctx["fp8_backward_ctx"], nullcontext) and not ctx["scaler"].is_enabled()
+
+
+def test_fp8_on_cpu_raises():
+    with pytest.raises(ValueError, match="FP8 training is only supported on CUDA devices"):
+        TrainingContext(opt("torch.float8_e4m3fn")).setup_training_context(torch.device("cpu"))
+
+
+def test_fp8_dtype_but_fp8_disabled_falls_back_to_amp(monkeypatch):
+    monkeypatch.setattr(torch.cuda, "is_bf16_supported", lambda *a, **k: True)
+    ctx = TrainingContext(opt("torch.float8_e4m3fn", fp8_enabled=False)).setup_training_context(FakeCuda())
+    assert ctx["is_fp8_dtype"] is True and ctx["fp8_enabled"] is False and ctx["fp8_recipe"] is None
+    assert isinstance(ctx["amp_ctx"], torch.autocast) and ctx["amp_ctx"].fast_dtype == torch.bfloat16
+    assert not ctx["scaler"].is_enabled()                                    # FP8 dtype always switches the loss scaler off
+
+
+def test_fp8_requested_without_backend_falls_back(monkeypatch):
+    import optimus_dl_amd.recipe.training_context as tc
+
+    monkeypatch.setattr(tc, "is_transformer_engine_available", lambda: False)
+    monkeypatch.setattr(torch.cuda, "is_bf16_supported", lambda *a, **k: True)
+    ctx = TrainingContext(opt("torch.float8_e4m3fn")).setup_training_context(FakeCuda())
+    assert ctx["fp8_enabled"] is False and isinstance(ctx["amp_ctx"], torch.autocast)
+
+
+def test_scaler_for_fp16_only():
+    c16 = TrainingContext(opt("torch.float16", fp8_enabled=False)).setup_training_context(torch.device("cpu"))
+    assert c16["amp_cfg"].resolved_enable_scaler() is True
+    cbf = TrainingContext(opt("torch.bfloat16", fp8_enabled=False)).setup_training_context(torch.device("cpu"))
+    assert not cbf["scaler"].is_enabled()
+
+
+def test_create_recipe_returns_none_without_backend():
+    from optimus_dl_amd.modules.amp import FP8Recipe, create_fp8_recipe, is_transformer_engine_available
+
+    if is_transformer_engine_available():
+        pytest.skip("a GPU backend is present here")
+    assert create_fp8_recipe("delayed", "hybrid") is None
+    with pytest.raises(ImportError):
+        FP8Recipe()
+
+
+def test_autocast_helpers_without_recipe_are_plain_amp():
+    lin = nn.Linear(8, 8)
+    x = torch.randn(4, 8)
+    with fp8_autocast(torch.device("cpu"), None, dtype=torch.bfloat16):
+        assert lin(x).dtype == torch.bfloat16
+    with fp8_autocast(torch.device("cpu"), None, enabled=False):
+        assert lin(x).dtype == torch.float32
+    with fp8_backward(None):
+        lin(x).sum().backward()
+    assert lin.weight.grad is not None
+
+
+def test_forward_backward_helpers_accept_instance_or_factory():
+    lin = nn.Linear(8, 8)
+    batch = torch.randn(4, 8)
+    crit = lambda model, b: model(b).float().pow(2).mean()
+    calls = []
+
+    def factory():
+        calls.append(1)
+        return nullcontext()
+
+    loss = execute_forward_pass(lin, batch, crit, factory)
+    execute_backward_pass(loss, None, factory)
+    loss = execute_forward_pass(lin, batch, crit, nullcontext())
+    execute_backward_pass(loss, None, nullcontext())
+    assert len(calls) == 2 and lin.weight.grad is not None
