@@ -1,0 +1,241 @@
+#!/usr/bin/env python3
+"""Benchmark of the FP8 Linear path on one MI355X.
+
+Workload (BASELINE config 3): the three Linears of a Llama-3-8B SwiGLU MLP,
+forward + backward in FP8 with per-tensor dynamic scaling (E4M3 for activations
+and weights, E5M2 for gradients), M = 8192 tokens:
+    gate, up : X [8192, 4096]   W [14336, 4096]   dY [8192, 14336]
+    down     : X [8192, 14336]  W [4096, 14336]   dY [8192, 4096]
+One step = fwd + bwd of all three = 9 GEMMs (8.66 TFLOP) plus every amax, cast and
+cast+transpose they need, weights re-quantised each step as after an optimizer
+step.  Inputs are synthetic, seeded, and resident in HBM before the clock starts.
+
+Prints ONE JSON line: whole-step TFLOP/s, the GEMM kernel's MFMA roofline
+fraction, the HBM rates of the memory-bound kernels, and the same arithmetic on
+the host CPU (the oracle, on a bounded sample) as a reported baseline.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_FP8_TFLOPS = 5000.0     # MI355X dense FP8 MFMA, published
+PEAK_HBM_GBPS = 8000.0       # MI355X HBM3E, published
+M_TOKENS, D_MODEL, D_FF = 8192, 4096, 14336
+LAYERS = (("gate", D_MODEL, D_FF), ("up", D_MODEL, D_FF), ("down", D_FF, D_MODEL))   # name, K(in), N(out)
+
+
+def step_flops(m: int = M_TOKENS) -> float:
+    return sum(6.0 * m * k * n for _, k, n in LAYERS)
+
+
+class KernelTimer:
+    """Brackets each native call with HIP events on the stream it is launched on
+    (torch's current stream, which is the stream the library receives)."""
+
+    def __init__(self, native, torch):
+        self.native, self.torch = native, torch
+        self.records: dict[str, list] = {}
+        self.enabled = False
+        self._orig = {}
+
+    def install(self):
+        def wrap(name, work_fn):
+            orig = getattr(self.native, name)
+            self._orig[name] = orig
+
+            def timed(*a, **kw):
+                if not self.enabled:
+                    return orig(*a, **kw)
+                e0, e1 = self.torch.cuda.Event(enable_timing=True), self.torch.cuda.Event(enable_timing=True)
+                e0.record()
+                out = orig(*a, **kw)
+                e1.record()
+                self.records.setdefault(name, []).append((e0, e1, work_fn(*a, **kw)))
+                return out
+
+            setattr(self.native, name, timed)
+
+        def esz(x):
+            return x.element_size()
+
+        wrap("gemm_nt", lambda a, b, *r, **kw: 2.0 * a.shape[0] * b.shape[0] * a.shape[1])            # flops
+        wrap("amax", lambda x, *r, **kw: float(x.numel() * esz(x)))                                       # bytes
+        wrap("cast", lambda x, *r, **kw: float(x.numel() * (esz(x) + 1)))
+        wrap("cast_transpose",
+             lambda x, *r, **kw: float(x.numel() * (esz(x) + (2 if kw.get("want_rowmajor", True) else 1))))
+
+    def summary(self):
+        out = {}
+        for name, recs in self.records.items():
+            ms = [e0.elapsed_time(e1) for e0, e1, _ in recs]
+            work = [w for _, _, w in recs]
+            out[name] = {"launches": len(recs), "total_ms": sum(ms), "avg_us": 1e3 * sum(ms) / len(ms), "work": sum(work)}
+        return out
+
+
+def make_inputs(torch, m=M_TOKENS, device="cuda"):
+    g = torch.Generator().manual_seed(0)
+    data = {}
+    for name, k, n in LAYERS:
+        data[name] = {
+            "x": torch.randn(m, k, generator=g).bfloat16().to(device),
+            "w": (torch.randn(n, k, generator=g) * 0.02).bfloat16().to(device),
+            "dy": (torch.randn(m, n, generator=g) * 1e-3).bfloat16().to(device),
+        }
+    return data
+
+
+def cpu_baseline(torch, seconds_hint=20.0):
+    """The oracle's emulated-FP8 Linear fwd+bwd on the host cores, on a slice of the rows."""
+    from oracle import oracle as O
+
+    cores = os.cpu_count() or 1
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+    m = 4096
+    data = make_inputs(torch, m=m, device="cpu")
+    t0 = time.perf_counter()
+    for name, k, n in LAYERS:
+        d = data[name]
+        O.linear_fwd_bwd(d["x"], d["w"], d["dy"], O.E4M3, O.E5M2)
+    dt = time.perf_counter() - t0
+    return {
+        "value": step_flops(m) / dt / 1e12,
+        "unit": "TFLOP/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"rows 0..{m - 1} of {M_TOKENS} (all three Linears, fwd+bwd incl. amax/cast, 1 pass, {dt:.1f} s); "
+                  "torch CPU float8 cast + fp32 matmul",
+        "seconds": dt,
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU leg (for profiler runs)")
+    ap.add_argument("--gemm-variant", type=int, default=-1)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this build runs on ONE GPU; --gpus {args.gpus} is not supported "
+              "(no collectives are part of the FP8 Linear path).", file=sys.stderr)
+        return 2
+
+    import torch
+
+    from optimus_dl_amd import native
+    from optimus_dl_amd.modules.amp import create_fp8_recipe
+    from optimus_dl_amd.modules.fp8_linear import FP8Linear
+
+    native.load()   # raises if the HIP library is missing: there is no fallback
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 2
+    native.gemm_set_variant(args.gemm_variant)
+    dev = "cuda"
+    data = make_inputs(torch, device=dev)
+    recipe = create_fp8_recipe("tensorwise", "hybrid")
+    layers = {}
+    for name, k, n in LAYERS:
+        lin = torch.nn.Linear(k, n, bias=False, device=dev, dtype=torch.bfloat16)
+        with torch.no_grad():
+            lin.weight.copy_(data[name]["w"])
+        layers[name] = FP8Linear.from_linear(lin)
+        data[name]["x"].requires_grad_(True)
+
+    timer = KernelTimer(native, torch)
+    timer.install()
+
+    def one_step():
+        for name, _, _ in LAYERS:
+            lin, d = layers[name], data[name]
+            lin._wcache.key = None            # weights change every optimizer step: re-quantise them every step
+            lin.weight.grad = None
+            d["x"].grad = None
+            with recipe.autocast():
+                y = lin(d["x"])
+            with recipe.backward():
+                y.backward(d["dy"])
+
+    for _ in range(args.warmup):
+        one_step()
+    torch.cuda.synchronize()
+    timer.enabled = True
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        one_step()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    timer.enabled = False
+
+    ks = timer.summary()
+    ms_per_step = 1e3 * wall / args.steps
+    tflops = step_flops() / (wall / args.steps) / 1e12
+    gemm = ks["gemm_nt"]
+    gemm_tflops = gemm["work"] / (gemm["total_ms"] * 1e-3) / 1e12
+    hbm = {}
+    for name in ("amax", "cast", "cast_transpose"):
+        if name in ks:
+            gbps = ks[name]["work"] / (ks[name]["total_ms"] * 1e-3) / 1e9
+            hbm[name] = {"achieved": gbps, "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": gbps / PEAK_HBM_GBPS,
+                         "avg_us": ks[name]["avg_us"], "launches": ks[name]["launches"]}
+    quant_bytes = sum(ks[n]["work"] for n in ("amax", "cast", "cast_transpose") if n in ks)
+    quant_ms = sum(ks[n]["total_ms"] for n in ("amax", "cast", "cast_transpose") if n in ks)
+
+    line = {
+        "metric": "fp8 Linear fwd+bwd TFLOP/s (Llama-3-8B MLP, M=8192) + cast/amax HBM GB/s",
+        "value": tflops,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "fp8 (e4m3 x/w, e5m2 grads; fp32 accumulate; bf16 out)",
+        "data": "synthetic",
+        "config": {
+            "workload": "BASELINE config 3: Llama-3-8B SwiGLU MLP Linears (gate, up [14336x4096]; down [4096x14336]), "
+                        "M=8192, FP8 fwd+bwd, per-tensor dynamic scaling, fused cast+transpose for wgrad",
+            "flop_per_step": step_flops(),
+            "gemms_per_step": 9,
+            "gemm_variant": native.gemm_variants()[args.gemm_variant] if args.gemm_variant >= 0 else "auto",
+        },
+        "frac_of_fp8_peak": tflops / PEAK_FP8_TFLOPS,
+        "gemm_only_tflops": gemm_tflops,
+        "cast_amax_gbps": quant_bytes / (quant_ms * 1e-3) / 1e9 if quant_ms else None,
+        "cast_amax_frac_of_hbm_peak": (quant_bytes / (quant_ms * 1e-3) / 1e9) / PEAK_HBM_GBPS if quant_ms else None,
+        "time_split_ms_per_step": {n: ks[n]["total_ms"] / args.steps for n in ks},
+        "roofline": {
+            "kernel": "gemm_nt_tiled_kernel (FP8 MFMA GEMM; fwd, dgrad, wgrad launches)",
+            "bound": "mfma",
+            "achieved": gemm_tflops,
+            "peak": PEAK_FP8_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": gemm_tflops / PEAK_FP8_TFLOPS,
+            "traffic": None,
+            "avg_launch_us": gemm["avg_us"],
+            "launches": gemm["launches"],
+        },
+        "hbm_kernels": hbm,
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(torch)
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -261,8 +261,8 @@ struct Variant {
 
 static const Variant kVariants[] = {
     {"generic 32x32 (1 wave, no LDS)", 0, 0, 64, 0.05f},
-    {"256x256x128 4 waves (128x128 per wave)", 256, 256, 256, 1.00f},
-    {"256x256x128 8 waves (128x64 per wave)", 256, 256, 512, 0.95f},
+    {"256x256x128 4 waves (128x128 per wave)", 256, 256, 256, 0.25f},
+    {"256x256x128 8 waves (128x64 per wave)", 256, 256, 512, 1.00f},
     {"256x128x128 4 waves (128x64 per wave)", 256, 128, 256, 0.85f},
     {"128x128x128 4 waves (64x64 per wave)", 128, 128, 256, 0.70f},
 };
@@ -295,10 +295,9 @@ static int cu_count() {
 
 static int choose_variant(int64_t M, int64_t N) {
     const int cus = cu_count();
-    int best = 1;
+    int best = 2;
     double best_score = -1.0;
-    for (int v = 1; v < kNumVariants; ++v) {
-        if (v == 2) continue;                                   // same tile as 1; only by explicit request
+    for (int v = 2; v < kNumVariants; ++v) {                    // variant 1 (one wave per SIMD) only by explicit request
         const Variant &cfg = kVariants[v];
         const int64_t tiles = ((M + cfg.bm - 1) / cfg.bm) * ((N + cfg.bn - 1) / cfg.bn);
         const int per_cu = cfg.bm * cfg.bn >= 256 * 256 ? 1 : (cfg.bm * cfg.bn >= 256 * 128 ? 1 : 2);

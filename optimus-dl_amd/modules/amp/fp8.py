@@ -189,6 +189,7 @@ class FP8Recipe:
         )
         self._store = _state.MetaStore(amax_history_len)
         self._depth = 0
+        self.scale_epoch = 0      # bumped whenever the forward scales are refreshed (invalidates cached weight codes)
         _info_once(
             f"Created FP8 recipe with format={self.format.value}, amax_history_len={amax_history_len}, "
             f"amax_compute_algo={amax_compute_algo}"
@@ -212,6 +213,8 @@ class FP8Recipe:
         if not self.is_delayed:
             return
         algo = native.AMAX_MAX if self.amax_compute_algo == "max" else native.AMAX_MOST_RECENT
+        if direction == "fwd":
+            self.scale_epoch += 1
         for arena in self._store.dirty_arenas(direction):
             R = arena.used
             native.delayed_update_raw(arena.history, arena.H, arena.capacity, R, arena.scale, arena.scale_inv,

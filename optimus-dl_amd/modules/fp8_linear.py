@@ -230,7 +230,8 @@ class FP8Linear(nn.Linear):
         """Per-tensor quantised weight (and transpose), cached on the parameter version."""
         pol = recipe.recipe
         c = self._wcache
-        key = (weight.data_ptr(), weight._version, id(recipe), pol.kind)
+        # delayed scaling: the codes depend on the scale in force, which changes at every refresh
+        key = (weight.data_ptr(), weight._version, id(recipe), pol.kind, recipe.scale_epoch if pol.kind == "delayed" else 0)
         fresh = c.key != key
         if fresh or (need_t and c.wq_t is None):
             w2d = weight.detach()
