@@ -33,6 +33,13 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
     return (f != f) ? ((u >> 16) | 0x40u) : r;
 }
 
+// two fp32 -> packed bf16 (lo = a, hi = b) with the hardware's round-to-nearest-even conversion
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, bf16x2));   // v_cvt_pk_bf16_f32
+}
+
 template <int FMT> struct Fp8Lim;
 template <> struct Fp8Lim<ODL_FP8_E4M3> { static constexpr float max = 448.0f; };
 template <> struct Fp8Lim<ODL_FP8_E5M2> { static constexpr float max = 57344.0f; };
