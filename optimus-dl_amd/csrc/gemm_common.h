@@ -21,7 +21,7 @@ struct GemmArgs {
     int out_dtype;               // bias, when present, is fp32
     int tiles_m, tiles_n;
 #ifdef ODL_GEMM_TRACE
-    uint32_t *trace;             // development builds only: per-wave cycle stamps
+    unsigned long long *trace;   // development builds only: cycle stamps, [block][tile][4]
 #endif
 };
 
@@ -150,6 +150,6 @@ __device__ __forceinline__ void epilogue_staged(const GemmArgs &g, v16f (&acc)[T
 
 // launchers implemented in gemm_tiled.hip / gemm_pipe.hip (fa, fb: odl_fp8_format of A and B)
 void launch_gemm_tiled(int variant, int fa, int fb, const GemmArgs &g, hipStream_t stream);
-void launch_gemm_pipe(int fa, int fb, const GemmArgs &g, hipStream_t stream);
+void launch_gemm_pipe(int fa, int fb, const GemmArgs &g, int num_cus, hipStream_t stream);
 
 }  // namespace odl

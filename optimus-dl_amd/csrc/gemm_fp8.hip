@@ -49,9 +49,10 @@ static const Variant kVariants[] = {
     {"256x256x128 8 waves (128x64 per wave)", 256, 256, 512, 1.00f},
     {"256x128x128 4 waves (128x64 per wave)", 256, 128, 256, 0.85f},
     {"128x128x128 4 waves (64x64 per wave)", 128, 128, 256, 0.70f},
-    {"256x256x128 4 waves, software-pipelined (K % 256 == 0)", 256, 256, 256, 1.10f},
+    {"256x256x128 4 waves, software-pipelined, persistent (K % 256 == 0)", 256, 256, 256, 1.10f},
+    {"256x256x128 4 waves, software-pipelined, one tile per block", 256, 256, 256, 0.50f},
 };
-constexpr int kPipeVariant = 5;
+constexpr int kPipeVariant = 5, kPipeOneTileVariant = 6;
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 static int g_forced_variant = -1;
 
@@ -138,7 +139,7 @@ extern "C" int odl_fp8_gemm_nt(const uint8_t *a, const uint8_t *b, int64_t M, in
     // the pipelined kernel walks K in pairs of 128-byte steps and addresses rows with 32-bit byte offsets
     const bool pipe_ok = tiled_ok && K % 256 == 0 && (double)(M + 256) * (double)K < 2147483648.0 &&
                          (double)(N + 256) * (double)K < 2147483648.0;
-    if (variant == kPipeVariant && !pipe_ok) variant = 2;
+    if ((variant == kPipeVariant || variant == kPipeOneTileVariant) && !pipe_ok) variant = 2;
 
     GemmArgs g;
     g.a = a; g.b = b; g.c = c; g.sa = sa_inv; g.sb = sb_inv; g.bias = bias;
@@ -152,7 +153,8 @@ extern "C" int odl_fp8_gemm_nt(const uint8_t *a, const uint8_t *b, int64_t M, in
     g.tiles_m = (int)tm; g.tiles_n = (int)tn;
 
     if (variant == 0) launch_gemm_generic(fmt_a, fmt_b, g, stream);
-    else if (variant == kPipeVariant) launch_gemm_pipe(fmt_a, fmt_b, g, stream);
+    else if (variant == kPipeVariant) launch_gemm_pipe(fmt_a, fmt_b, g, cu_count(), stream);
+    else if (variant == kPipeOneTileVariant) launch_gemm_pipe(fmt_a, fmt_b, g, 1 << 30, stream);
     else launch_gemm_tiled(variant, fmt_a, fmt_b, g, stream);
     return check_launch("odl_fp8_gemm_nt");
 }

@@ -1,5 +1,6 @@
 // FP8 GEMM, 256x256 block tile, 4 waves (one per SIMD, 128x128 each), explicit
-// software pipeline.  C = (A[M,K] . B[N,K]^T) * scales, K % 256 == 0.
+// software pipeline, persistent over tiles.  C = (A[M,K] . B[N,K]^T) * scales,
+// K % 256 == 0.
 //
 // Why one wave per SIMD: a 128x128 wave tile needs 256 accumulator registers
 // (the whole AGPR half of the unified 512-entry file) but halves the LDS traffic
@@ -9,7 +10,7 @@
 //   per K step of 128 bytes (two halves h0, h1 of 64 bytes = one MFMA K each)
 //     phase A : 16 MFMAs on register buffer 0 (step kt, h0)
 //               interleaved with the 16 LDS reads of (kt, h1) into buffer 1
-//     wait vmcnt(0) + lgkmcnt(0), s_barrier      <- the ONLY sync per K step:
+//     wait vmcnt(2) + lgkmcnt(0), s_barrier      <- the ONLY sync per K step:
 //               step kt+1 has landed in the other LDS stage (it was requested a
 //               whole step ago) and everybody is done reading this stage
 //     phase B : 16 MFMAs on buffer 1 (kt, h1)
@@ -20,6 +21,13 @@
 //   available when the barrier is crossed, and every LDS read has ~1000 cycles
 //   of MFMA work in front of its first use.
 //
+// Persistent: one block per CU walks its share of the tiles.  When the K loop of a
+// tile ends, the first two K steps of the NEXT tile are requested before the
+// epilogue starts, so the latency of a tile's first loads (HBM: several
+// microseconds) and the drain of the output stores overlap each other instead of
+// both being paid per tile.  The epilogue therefore stages through its own small
+// LDS region (the operand stages are already being refilled).
+//
 // Global -> LDS: buffer_load_dwordx4 ... lds.  The per-lane byte offset is a
 // loop-invariant VGPR, the K position is the scalar offset, the buffer resource's
 // size makes rows past the end of the matrix read as zero: no per-load address
@@ -28,9 +36,13 @@
 // only flip bit 2 of f, each operand needs just 4 per-lane LDS address registers,
 // everything else is an immediate.
 //
-// The four LDS regions (A/B x stage 0/1) are separate __shared__ objects so that
-// the compiler can see that loads in flight into one stage never alias the reads
-// of the other, and does not fence them with vmcnt waits.
+// Every vector-memory load of the K loop is issued from inline asm, and every wait
+// on the vector-memory counter is written out by hand: the counter retires in issue
+// order, which lets the loop wait for "all but the youngest n" operations (the L2
+// prefetches, or the previous tile's output stores), something the compiler's own
+// bookkeeping cannot express across the tile loop.  Instruction order inside a phase
+// is pinned with sched_barrier so that each MFMA is followed by its share of LDS
+// reads and loads.
 #include "gemm_common.h"
 
 #include <type_traits>
@@ -43,8 +55,9 @@ constexpr int BM = 256, BN = 256, NW = 4, WM = 128, WN = 128, TM = 4, TN = 4;
 constexpr int REGION = 256 * 128;          // bytes of one operand in one stage
 constexpr int LOADS = 256 / 8 / NW;        // 1 KB direct-to-LDS loads per wave per operand per stage
 constexpr int GM = 8;
-
-constexpr unsigned MASK_MFMA = 0x008, MASK_VMEM = 0x010, MASK_DS_RD = 0x100;   // sched_group_barrier classes
+constexpr int PF = 4;                      // L2 prefetch distance in K steps
+constexpr int EPI_BYTES = 32 * (128 + 16); // one wave's epilogue slab: 32 rows x 128 bytes (+16 pad)
+static_assert(staged_epilogue_bytes<true, 2>() == EPI_BYTES && staged_epilogue_bytes<false, 1>() == EPI_BYTES, "slab size");
 
 typedef __attribute__((address_space(3))) void *lds_ptr_t;
 
@@ -54,68 +67,80 @@ __global__ __launch_bounds__(256) void gemm_nt_pipe_kernel(const GemmArgs g) {
     __shared__ __attribute__((aligned(1024))) uint8_t sB0[REGION];
     __shared__ __attribute__((aligned(1024))) uint8_t sA1[REGION];
     __shared__ __attribute__((aligned(1024))) uint8_t sB1[REGION];
-
-    // ---- tile (XCD-aware, grouped): see gemm_tiled.hip
-    const int total = g.tiles_m * g.tiles_n;
-    const int per_xcd = (total + 7) / 8;
-    const int pid = (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8);
-    if (pid >= total) return;
-    const int in_group = GM * g.tiles_n;
-    const int first_m = (pid / in_group) * GM;
-    const int group_rows = min(g.tiles_m - first_m, GM);
-    const int tile_m = first_m + (pid % in_group) % group_rows;
-    const int tile_n = (pid % in_group) / group_rows;
-    const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
+    __shared__ __attribute__((aligned(16))) uint8_t sEpi[NW * EPI_BYTES];
 
     const int lane = threadIdx.x % 64;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
     const int wm0 = (wave / 2) * WM, wn0 = (wave % 2) * WN;
+    const int lr = lane % 32, lg = lane / 32;
     const int KT = (int)(g.K / 128);
-#ifdef ODL_GEMM_TRACE
-    uint64_t t_entry; asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t_entry));
-#endif
 
-    // ---- global -> LDS
-    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc((void *)g.a, 0, (int)(g.M * g.K), 0x00020000);
-    const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc((void *)g.b, 0, (int)(g.N * g.K), 0x00020000);
-    int voff_a[LOADS], voff_b[LOADS];
+    // ---- which tiles: block ids are dealt round-robin to the 8 XCDs, so the blocks of
+    // one XCD (id % 8) walk one contiguous chunk of the grouped tile order together
+    const int total = g.tiles_m * g.tiles_n;
+    const int per_xcd = (total + 7) / 8;
+    const int xcd = (int)(blockIdx.x % 8), stride = (int)(gridDim.x / 8);
+    const int pid_end = min((xcd + 1) * per_xcd, total);
+    int pid = xcd * per_xcd + (int)(blockIdx.x / 8);
+    if (pid >= pid_end) return;
+
+    // ---- per-tile addressing.  The tile's origin lives in the buffer resources (base =
+    // first row of the tile, size = what is left of the matrix, so rows past the end read
+    // as zero); the per-lane offsets are the same for every tile and for both operands.
+    int64_t m0 = 0, n0 = 0, next_m0 = 0, next_n0 = 0;
+    v4i rsrc_a, rsrc_b, next_a, next_b;           // raw buffer descriptors (base, stride 0, bytes, format)
+    auto tile_origin = [&](int p, int64_t &tm0, int64_t &tn0) {
+        const int in_group = GM * g.tiles_n;
+        const int first_m = (p / in_group) * GM;
+        const int group_rows = min(g.tiles_m - first_m, GM);
+        tm0 = (int64_t)(first_m + (p % in_group) % group_rows) * BM;
+        tn0 = (int64_t)((p % in_group) / group_rows) * BN;
+    };
+    auto rsrc_for = [&](const uint8_t *base, int64_t row0, int64_t rows) -> v4i {
+        const uint64_t addr = reinterpret_cast<uint64_t>(base + row0 * g.K);
+        return v4i{(int)(uint32_t)addr, (int)(uint32_t)(addr >> 32), (int)((rows - row0) * g.K), 0x00020000};
+    };
+    int voff[LOADS];
 #pragma unroll
     for (int j = 0; j < LOADS; ++j) {
         const int row = (wave + j * NW) * 8 + lane / 8;
-        const int sw = ((lane % 8) ^ swz(row)) << 4;
-        voff_a[j] = (int)((m0 + row) * g.K) + sw;          // rows past M land beyond num_records -> zeros
-        voff_b[j] = (int)((n0 + row) * g.K) + sw;
+        voff[j] = row * (int)g.K + (((lane % 8) ^ swz(row)) << 4);
     }
+    // one 1 KB direct-to-LDS load: 64 lanes x 16 bytes land at lds_addr + lane * 16
+    auto dma = [&](const v4i &rsrc, uint32_t lds_addr, int vo, int so) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                     ::"s"(lds_addr), "v"(vo), "s"(rsrc), "s"(so));
+    };
+    auto lds_addr_of = [](const uint8_t *p) { return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) uint8_t *)p; };
+    // load j of a stage: j < LOADS -> operand A, else operand B
+    auto issue_one = [&](uint8_t *sa, uint8_t *sb, int kt, int j) {
+        if (j < LOADS) dma(rsrc_a, lds_addr_of(sa) + (wave + j * NW) * 1024, voff[j], kt * 128);
+        else dma(rsrc_b, lds_addr_of(sb) + (wave + (j - LOADS) * NW) * 1024, voff[j - LOADS], kt * 128);
+    };
     auto issue = [&](uint8_t *sa, uint8_t *sb, int kt) {
-        const int soff = kt * 128;
 #pragma unroll
-        for (int j = 0; j < LOADS; ++j) {
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_ptr_t)(sa + (wave + j * NW) * 1024), 16, voff_a[j], soff, 0, 0);
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_ptr_t)(sb + (wave + j * NW) * 1024), 16, voff_b[j], soff, 0, 0);
-        }
+        for (int j = 0; j < 2 * LOADS; ++j) issue_one(sa, sb, kt, j);
     };
 
     // ---- L2 prefetch.  About one line in six of a K step misses this XCD's L2 (the 32
-    // tiles running on an XCD share rows, but every row has to arrive once), and a miss
-    // costs more than the one K step the LDS stages can cover.  So each lane touches one
-    // 128-byte line of the step PF ahead with a load whose value is never used: 2 loads
-    // per wave per step pull all 512 lines of that step into L2 long before the
+    // tiles running on an XCD share rows, but every row has to arrive once).  Each lane
+    // touches one 128-byte line of the step PF ahead with a load whose value is never
+    // used: 2 loads per wave per step pull all 512 lines of that step into L2 before the
     // direct-to-LDS loads ask for them.  They are issued AFTER the DMA loads of the same
-    // phase, so "vmcnt(2)" still means "every DMA load has landed".
-    constexpr int PF = 4;
-    const uint8_t *pf_a = g.a + min(m0 + wave * 64 + lane, g.M - 1) * g.K;
-    const uint8_t *pf_b = g.b + min(n0 + wave * 64 + lane, g.N - 1) * g.K;
+    // phase, so "vmcnt(2)" still means "every DMA load has landed".  Steps past the end of
+    // this tile belong to the next tile of this block, if there is one.  The two
+    // destination registers stay allocated for the whole kernel (in-flight loads write them).
+    const int pf_off = (wave * 64 + lane) * (int)g.K;
+    bool has_next = false;
     int pfv_a = 0, pfv_b = 0;
     auto prefetch = [&](int kt) {
-        const int kp = min(kt, KT - 1) * 128;
-        // "use" the values fetched one step ago (long since returned) so that the loads stay in the program
-        asm volatile("" ::"v"(pfv_a), "v"(pfv_b));
-        pfv_a = *reinterpret_cast<const int *>(pf_a + kp);
-        pfv_b = *reinterpret_cast<const int *>(pf_b + kp);
+        const bool nx = kt >= KT && has_next;
+        const int kp = (nx ? kt - KT : min(kt, KT - 1)) * 128;
+        asm volatile("buffer_load_dword %0, %1, %2, %3 offen" : "+v"(pfv_a) : "v"(pf_off), "s"(nx ? next_a : rsrc_a), "s"(kp));
+        asm volatile("buffer_load_dword %0, %1, %2, %3 offen" : "+v"(pfv_b) : "v"(pf_off), "s"(nx ? next_b : rsrc_b), "s"(kp));
     };
 
     // ---- LDS -> registers.  chunk(t, h, e) = ((2*lg + e) ^ s0) ^ 4*(h ^ (t & 1))
-    const int lr = lane % 32, lg = lane / 32;
     int ra[2][2], rb[2][2];                     // [e][h ^ (t & 1)] byte offsets inside a region (tile 0)
     {
         const int rowa = wm0 + lr, rowb = wn0 + lr;
@@ -140,13 +165,6 @@ __global__ __launch_bounds__(256) void gemm_nt_pipe_kernel(const GemmArgs g) {
     };
 
     v16f acc[TM][TN];
-#pragma unroll
-    for (int t = 0; t < TM; ++t)
-#pragma unroll
-        for (int u = 0; u < TN; ++u)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) acc[t][u][e] = 0.0f;
-
     v8i a0[TM], b0[TN], a1[TM], b1[TN];         // register buffers 0 (h0) and 1 (h1)
 
     auto mfma_all = [&](v8i (&fa)[TM], v8i (&fb)[TN]) {
@@ -156,143 +174,172 @@ __global__ __launch_bounds__(256) void gemm_nt_pipe_kernel(const GemmArgs g) {
             for (int u = 0; u < TN; ++u) acc[t][u] = mfma_32x32x64<FB, FA>(fb[u], fa[t], acc[t][u]);
     };
 
-#ifdef ODL_GEMM_TRACE
-    // development aid: cycle stamps around the per-step wait and barrier, kept in three VGPRs (lane = K step)
-    uint32_t tr_a = 0, tr_b = 0, tr_c = 0;
-#define ODL_STAMP_ISSUE(var) uint64_t var; asm volatile("s_memtime %0" : "=s"(var))
-#define ODL_STAMP_SYNC(var) uint64_t var; asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(var))
-#endif
-
-    // One K step.  cur / nxt = LDS stage holding step kt / kt+1.
+    // One K step.  cur / nxt = LDS stage holding step kt / kt+1.  MFMA i works on tile
+    // (t, u) = (i / 4, i % 4); fragment f < 4 is A tile f, f >= 4 is B tile f - 4.
     auto step = [&](uint8_t *sa_cur, uint8_t *sb_cur, uint8_t *sa_nxt, uint8_t *sb_nxt, int kt, auto read_next, auto load_g) {
-        // phase A
+        // phase A: MFMAs on buffer 0, the 8 fragments of (kt, h1) stream into buffer 1 behind the first 8
 #pragma unroll
-        for (int t = 0; t < TM; ++t) a1[t] = read_a(sa_cur, t, 1);
-#pragma unroll
-        for (int u = 0; u < TN; ++u) b1[u] = read_b(sb_cur, u, 1);
-        mfma_all(a0, b0);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            __builtin_amdgcn_sched_group_barrier(MASK_MFMA, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(MASK_DS_RD, 2, 0);
+        for (int i = 0; i < 16; ++i) {
+            acc[i / 4][i % 4] = mfma_32x32x64<FB, FA>(b0[i % 4], a0[i / 4], acc[i / 4][i % 4]);
+            if (i < 4) a1[i] = read_a(sa_cur, i, 1);
+            else if (i < 8) b1[i - 4] = read_b(sb_cur, i - 4, 1);
+            __builtin_amdgcn_sched_barrier(0);
         }
-        __builtin_amdgcn_sched_group_barrier(MASK_MFMA, 8, 0);
-
-        __builtin_amdgcn_sched_barrier(0);      // keep all 16 MFMAs of phase A in front of the wait: they cover the LDS latency
-#ifdef ODL_GEMM_TRACE
-        ODL_STAMP_SYNC(t_a);
-#endif
         // my DMA for kt+1 has landed (the 2 younger prefetch loads may still be out), my LDS reads returned
         __builtin_amdgcn_s_waitcnt(0x0072);     // vmcnt(2) lgkmcnt(0)
-#ifdef ODL_GEMM_TRACE
-        ODL_STAMP_SYNC(t_b);
-#endif
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-#ifdef ODL_GEMM_TRACE
-        ODL_STAMP_SYNC(t_c);
-        tr_a = lane == (kt & 63) ? (uint32_t)t_a : tr_a;
-        tr_b = lane == (kt & 63) ? (uint32_t)t_b : tr_b;
-        tr_c = lane == (kt & 63) ? (uint32_t)t_c : tr_c;
-#endif
         __builtin_amdgcn_sched_barrier(0);
 
-        // phase B
-        if constexpr (decltype(read_next)::value) {
+        // phase B: MFMAs on buffer 1; (kt+1, h0) streams into buffer 0; step kt+2 is requested into this stage
 #pragma unroll
-            for (int t = 0; t < TM; ++t) a0[t] = read_a(sa_nxt, t, 0);
-#pragma unroll
-            for (int u = 0; u < TN; ++u) b0[u] = read_b(sb_nxt, u, 0);
-        }
-        if constexpr (decltype(load_g)::value) {
-            issue(sa_cur, sb_cur, kt + 2);
-            prefetch(kt + 2 + PF);
-        }
-        mfma_all(a1, b1);
-        if constexpr (decltype(read_next)::value && decltype(load_g)::value) {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                __builtin_amdgcn_sched_group_barrier(MASK_MFMA, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(MASK_DS_RD, 2, 0);
-                __builtin_amdgcn_sched_group_barrier(MASK_VMEM, 1, 0);
+        for (int i = 0; i < 16; ++i) {
+            acc[i / 4][i % 4] = mfma_32x32x64<FB, FA>(b1[i % 4], a1[i / 4], acc[i / 4][i % 4]);
+            if constexpr (decltype(read_next)::value) {
+                if (i < 4) a0[i] = read_a(sa_nxt, i, 0);
+                else if (i < 8) b0[i - 4] = read_b(sb_nxt, i - 4, 0);
             }
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                __builtin_amdgcn_sched_group_barrier(MASK_MFMA, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(MASK_VMEM, 1, 0);
+            if constexpr (decltype(load_g)::value) {
+                issue_one(sa_cur, sb_cur, kt + 2, i);
+                if (i == 15) prefetch(kt + 2 + PF);
             }
-            __builtin_amdgcn_sched_group_barrier(MASK_VMEM, 2, 0);      // the two prefetch loads go last
+            __builtin_amdgcn_sched_barrier(0);
         }
     };
     using yes = std::integral_constant<bool, true>;
     using no = std::integral_constant<bool, false>;
 
-    // ---- prologue: steps 0 and 1 requested, step 0 awaited, (0, h0) in registers
+    // ---- first tile: steps 0 and 1 requested (KT >= 2, host-checked) and awaited
+    tile_origin(pid, m0, n0);
+    rsrc_a = rsrc_for(g.a, m0, g.M);
+    rsrc_b = rsrc_for(g.b, n0, g.N);
+    next_a = rsrc_a;
+    next_b = rsrc_b;
     issue(sA0, sB0, 0);
-    issue(sA1, sB1, 1);                          // KT >= 2 (host-checked)
+    issue(sA1, sB1, 1);
     for (int k = 2; k < 2 + PF; ++k) prefetch(k);
     __builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0)
-    __syncthreads();
-#pragma unroll
-    for (int t = 0; t < TM; ++t) a0[t] = read_a(sA0, t, 0);
-#pragma unroll
-    for (int u = 0; u < TN; ++u) b0[u] = read_b(sB0, u, 0);
-
-    // ---- main loop: KT is even; the last two steps load nothing new
-    for (int kt = 0; kt < KT - 2; kt += 2) {
-        step(sA0, sB0, sA1, sB1, kt, yes{}, yes{});
-        step(sA1, sB1, sA0, sB0, kt + 1, yes{}, yes{});
-    }
-    step(sA0, sB0, sA1, sB1, KT - 2, yes{}, no{});
-    step(sA1, sB1, sA0, sB0, KT - 1, no{}, no{});
 
 #ifdef ODL_GEMM_TRACE
-    uint64_t t_loop_end; asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t_loop_end));
-    if (g.trace) {
-        uint32_t *t = g.trace + ((size_t)blockIdx.x * NW + wave) * 3 * 64;
-        t[lane] = tr_a; t[64 + lane] = tr_b; t[128 + lane] = tr_c;
-    }
+#define ODL_STAMP(var) unsigned long long var; asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(var))
+    int tile_no = 0;
+#else
+#define ODL_STAMP(var)
 #endif
-    // ---- epilogue
-    const bool interior = m0 + BM <= g.M && n0 + BN <= g.N;
-    const bool staged = interior && (g.N % 8) == 0;
-    if (staged) {
-        __syncthreads();                             // every wave is done with the operand stages: reuse them
-        uint8_t *wave_lds = wave == 0 ? sA0 : (wave == 1 ? sB0 : (wave == 2 ? sA1 : sB1));
-        if (g.out_dtype == ODL_BF16) epilogue_staged<true, TM, TN, TN>(g, acc, wave_lds, m0 + wm0, n0 + wn0, lane);
-        else epilogue_staged<false, TM, TN, TN>(g, acc, wave_lds, m0 + wm0, n0 + wn0, lane);
-    } else {
+    while (true) {
+        ODL_STAMP(t0);
+        const int64_t cm0 = m0, cn0 = n0;        // this tile's origin, kept for the epilogue
+        const int next_pid = pid + stride;
+        has_next = next_pid < pid_end;
+        if (has_next) {
+            tile_origin(next_pid, next_m0, next_n0);
+            next_a = rsrc_for(g.a, next_m0, g.M);
+            next_b = rsrc_for(g.b, next_n0, g.N);
+        }
+
+        // Steps 0 and 1 of this tile have landed.  The vector-memory counter retires in issue
+        // order, and behind those 32 loads this wave has issued at least 32 output stores of
+        // the previous tile and the L2 prefetches of the step in between ("at most 32
+        // outstanding" = the loads are in; for the first tile everything was awaited above),
+        // while the stores of the previous tile may still be draining.  (The staged epilogue
+        // issues 32 or 64 stores; the edge-tile path ends with a full wait.)
+        __builtin_amdgcn_s_waitcnt(0x8F70);      // vmcnt(32): bits 3:0 = 0, bits 15:14 = 2
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        ODL_STAMP(t1);
+#pragma unroll
+        for (int t = 0; t < TM; ++t) a0[t] = read_a(sA0, t, 0);
+#pragma unroll
+        for (int u = 0; u < TN; ++u) b0[u] = read_b(sB0, u, 0);
+#pragma unroll
+        for (int t = 0; t < TM; ++t)
+#pragma unroll
+            for (int u = 0; u < TN; ++u)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[t][u][e] = 0.0f;
+
+        // ---- K loop: KT is even; the last two steps load nothing new
+        for (int kt = 0; kt < KT - 2; kt += 2) {
+            step(sA0, sB0, sA1, sB1, kt, yes{}, yes{});
+            step(sA1, sB1, sA0, sB0, kt + 1, yes{}, yes{});
+        }
+        step(sA0, sB0, sA1, sB1, KT - 2, yes{}, no{});
+        step(sA1, sB1, sA0, sB0, KT - 1, no{}, no{});
+
+        ODL_STAMP(t2);
+        // Every wave passed the barrier of the last step after its final operand read, so
+        // the stages are free: request the next tile's first two steps before the epilogue
+        // (its first lines were pulled into L2 by the prefetches of the last steps).
+        if (has_next) {
+            pid = next_pid;
+            m0 = next_m0;
+            n0 = next_n0;
+            rsrc_a = next_a;
+            rsrc_b = next_b;
+            issue(sA0, sB0, 0);
+            issue(sA1, sB1, 1);
+        }
+        __builtin_amdgcn_sched_barrier(0);       // the loads stay in front of every store of the epilogue
+
+        // ---- epilogue of the tile just finished.  The lane / wave ids are laundered through
+        // empty asm so that the compiler computes the epilogue's addresses here, instead of
+        // once before the tile loop: kept across the K loop they would spill, and every
+        // scratch reload would wait on the vector-memory counter, i.e. on the output stores.
+        int lane_e = lane, wave_e = wave;
+        asm volatile("" : "+v"(lane_e));
+        asm volatile("" : "+s"(wave_e));
+        const bool interior = cm0 + BM <= g.M && cn0 + BN <= g.N;
+        if (interior && (g.N % 8) == 0) {
+            uint8_t *wave_lds = sEpi + wave_e * EPI_BYTES;
+            const int64_t mw = cm0 + (wave_e / 2) * WM, nw = cn0 + (wave_e % 2) * WN;
+            if (g.out_dtype == ODL_BF16) epilogue_staged<true, TM, TN, 2>(g, acc, wave_lds, mw, nw, lane_e);
+            else epilogue_staged<false, TM, TN, 1>(g, acc, wave_lds, mw, nw, lane_e);
+        } else {
 #define ODL_EPILOGUE(BF)                                                                                       \
     _Pragma("unroll") for (int t = 0; t < TM; ++t) _Pragma("unroll") for (int u = 0; u < TN; ++u)              \
-        store_tile<BF, false>(g, acc[t][u], m0 + wm0 + 32 * t + lr, n0 + wn0 + 32 * u + 4 * lg)
-        if (g.out_dtype == ODL_BF16) { ODL_EPILOGUE(true); } else { ODL_EPILOGUE(false); }
+        store_tile<BF, false>(g, acc[t][u], cm0 + wm0 + 32 * t + lr, cn0 + wn0 + 32 * u + 4 * lg)
+            if (g.out_dtype == ODL_BF16) { ODL_EPILOGUE(true); } else { ODL_EPILOGUE(false); }
 #undef ODL_EPILOGUE
-    }
+            // this path issues a data-dependent number of stores: do not count on them below
+            __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+        }
 #ifdef ODL_GEMM_TRACE
-    if (g.trace) {
-        __builtin_amdgcn_s_waitcnt(0x0070);
-        uint64_t t_exit; asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t_exit));
-        uint64_t *t64 = reinterpret_cast<uint64_t *>(g.trace + (size_t)gridDim.x * NW * 3 * 64) + ((size_t)blockIdx.x * NW + wave) * 4;
-        if (lane == 0) { t64[0] = t_entry; t64[1] = t_loop_end; t64[2] = t_exit; t64[3] = __builtin_amdgcn_s_getreg((4 << 11) | 20 /*XCC_ID*/) ; }
-    }
+        {
+            ODL_STAMP(t3);
+            if (g.trace && wave == 0 && lane == 0 && tile_no < 8) {
+                unsigned long long *t = g.trace + ((size_t)blockIdx.x * 8 + tile_no) * 4;
+                t[0] = t0; t[1] = t1; t[2] = t2; t[3] = t3;
+            }
+            ++tile_no;
+        }
 #endif
+        if (!has_next) break;
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0): nothing may still be writing the prefetch registers
+    asm volatile("" ::"v"(pfv_a), "v"(pfv_b));
 }
 
 template <int FA, int FB>
-void launch_fmt(const GemmArgs &g, hipStream_t stream) {
-    const int total = g.tiles_m * g.tiles_n;
-    const unsigned grid = (unsigned)(((total + 7) / 8) * 8);
-    hipLaunchKernelGGL((gemm_nt_pipe_kernel<FA, FB>), dim3(grid), dim3(256), 0, stream, g);
+void launch_fmt(const GemmArgs &g, int blocks_per_xcd, hipStream_t stream) {
+    hipLaunchKernelGGL((gemm_nt_pipe_kernel<FA, FB>), dim3((unsigned)(8 * blocks_per_xcd)), dim3(256), 0, stream, g);
 }
 
 }  // namespace
 
-void launch_gemm_pipe(int fa, int fb, const GemmArgs &g, hipStream_t stream) {
-    if (fa == ODL_FP8_E4M3 && fb == ODL_FP8_E4M3) launch_fmt<ODL_FP8_E4M3, ODL_FP8_E4M3>(g, stream);
-    else if (fa == ODL_FP8_E5M2 && fb == ODL_FP8_E4M3) launch_fmt<ODL_FP8_E5M2, ODL_FP8_E4M3>(g, stream);
-    else if (fa == ODL_FP8_E4M3 && fb == ODL_FP8_E5M2) launch_fmt<ODL_FP8_E4M3, ODL_FP8_E5M2>(g, stream);
-    else launch_fmt<ODL_FP8_E5M2, ODL_FP8_E5M2>(g, stream);
+// One block per CU at most (the kernel needs ~150 KB of LDS), 8 | grid so that the
+// round-robin placement gives every XCD the same number of blocks.
+void launch_gemm_pipe(int fa, int fb, const GemmArgs &g, int num_cus, hipStream_t stream) {
+    const int total = g.tiles_m * g.tiles_n;
+    const int per_xcd = (total + 7) / 8;
+    int bpx = num_cus / 8;
+    if (bpx < 1) bpx = 1;
+    if (bpx > per_xcd) bpx = per_xcd;
+    if (fa == ODL_FP8_E4M3 && fb == ODL_FP8_E4M3) launch_fmt<ODL_FP8_E4M3, ODL_FP8_E4M3>(g, bpx, stream);
+    else if (fa == ODL_FP8_E5M2 && fb == ODL_FP8_E4M3) launch_fmt<ODL_FP8_E5M2, ODL_FP8_E4M3>(g, bpx, stream);
+    else if (fa == ODL_FP8_E4M3 && fb == ODL_FP8_E5M2) launch_fmt<ODL_FP8_E4M3, ODL_FP8_E5M2>(g, bpx, stream);
+    else launch_fmt<ODL_FP8_E5M2, ODL_FP8_E5M2>(g, bpx, stream);
 }
 
 }  // namespace odl
