@@ -29,6 +29,9 @@ if ROOT not in sys.path:
 
 PEAK_FP8_TFLOPS = 5000.0     # MI355X dense FP8 MFMA, published
 PEAK_HBM_GBPS = 8000.0       # MI355X HBM3E, published
+# Memory-side bytes per GEMM launch (mean of the nine launches of a step), from two rocprofv3 --pmc runs
+# (FETCH_SIZE scaled x2.00, WRITE_SIZE x1.00 against a 256 MiB copy kernel): profiles/pmc_fetch_write__cfg3_mlp.md
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = 9.32e8
 M_TOKENS, D_MODEL, D_FF = 8192, 4096, 14336
 LAYERS = (("gate", D_MODEL, D_FF), ("up", D_MODEL, D_FF), ("down", D_FF, D_MODEL))   # name, K(in), N(out)
 
@@ -126,6 +129,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU leg (for profiler runs)")
     ap.add_argument("--gemm-variant", type=int, default=-1)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 256 MiB device copy (reference kernel for scaling FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this build runs on ONE GPU; --gpus {args.gpus} is not supported "
@@ -168,6 +173,12 @@ def main() -> int:
             with recipe.backward():
                 y.backward(d["dy"])
 
+    if args.copy_calibration:
+        src = torch.empty(256 * 1024 * 1024, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        del src, dst
     for _ in range(args.warmup):
         one_step()
     torch.cuda.synchronize()
@@ -225,7 +236,11 @@ def main() -> int:
             "peak": PEAK_FP8_TFLOPS,
             "unit": "TFLOP/s",
             "frac": gemm_tflops / PEAK_FP8_TFLOPS,
-            "traffic": None,
+            "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH,
+            "traffic_unit": "bytes per launch (FETCH_SIZE + WRITE_SIZE counters, measured separately)",
+            "algorithmic_bytes": (sum(m_ * k_ + n_ * k_ + 2 * m_ * n_ for m_, n_, k_ in
+                                      [(M_TOKENS, n, k) for _, k, n in LAYERS] + [(M_TOKENS, k, n) for _, k, n in LAYERS] +
+                                      [(n, k, M_TOKENS) for _, k, n in LAYERS]) / 9.0),
             "avg_launch_us": gemm["avg_us"],
             "launches": gemm["launches"],
         },
