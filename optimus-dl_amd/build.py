@@ -7,7 +7,9 @@ travels with the source tree to machines that have a GPU but no compiler step.
 
 from __future__ import annotations
 
+import glob
 import os
+import re
 import shutil
 import subprocess
 import sys
@@ -16,7 +18,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_NAME = "libodl_fp8.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
-SOURCES = ["api.hip", "quant.hip", "gemm_fp8.hip", "gemm_tiled.hip", "gemm_pipe.hip"]
+SOURCES = ["api.hip", "quant.hip", "gemm_fp8.hip", "gemm_tiled.hip", "gemm_pipe.hip", "gemm_stream.hip"]
 
 # -ffp-contract=off : the epilogues promise "multiply, round, add, round" (no FMA fusion)
 # packed-fp32-ops off: never let the compiler form v_pk_*_f32 from scalar float code
@@ -41,17 +43,66 @@ def hipcc_path() -> str:
     raise RuntimeError("hipcc not found (looked at $HIPCC, /opt/rocm/bin/hipcc, PATH)")
 
 
+_SGPR_OPERAND = re.compile(r"\bs(?:\[(\d+):(\d+)\]|(\d+))")
+_VALU_WRITES_SGPR = re.compile(r"^(v_readlane_b32|v_readfirstlane_b32|v_cmp\w*)\s+s(?:\[(\d+):(\d+)\]|(\d+))")
+
+
+def check_asm_hazards(asm_text: str, name: str = "") -> list[str]:
+    """Finds vector-memory instructions written as inline asm that read a scalar register less
+    than 5 wait states after a vector instruction wrote it.
+
+    The hardware needs those wait states and the compiler inserts them for its own
+    instructions, but it does not look inside asm statements.  Which registers feed an asm
+    statement depends on register allocation (spilled scalars come back through
+    ``v_readlane_b32``), so the generated code is checked after every build.
+    """
+    lines = asm_text.split("\n")
+    problems = []
+    in_asm = False
+    for i, raw in enumerate(lines):
+        text = raw.strip()
+        if text.startswith(";;#ASMSTART"):
+            in_asm = True
+            continue
+        if text.startswith(";;#ASMEND"):
+            in_asm = False
+            continue
+        if not in_asm or not text.startswith(("buffer_", "global_", "flat_", "scratch_")):
+            continue
+        used = set()
+        for lo, hi, one in _SGPR_OPERAND.findall(text):
+            used |= set(range(int(lo), int(hi) + 1)) if lo else {int(one)}
+        waited, j = 0, i - 1
+        while j >= 0 and waited < 5:
+            prev = lines[j].strip()
+            j -= 1
+            if not prev or prev.startswith((";", ".")) or prev.endswith(":"):
+                continue
+            nop = re.match(r"s_nop (\d+)", prev)
+            if nop:
+                waited += int(nop.group(1)) + 1
+                continue
+            w = _VALU_WRITES_SGPR.match(prev)
+            if w:
+                written = set(range(int(w.group(2)), int(w.group(3)) + 1)) if w.group(2) else {int(w.group(4))}
+                if written & used:
+                    problems.append(f"{name}:{i + 1}: '{text}' reads a scalar register {waited} wait states after '{prev}'")
+            waited += 1
+    return problems
+
+
 def build(verbose: bool = False, keep_asm: bool = False) -> str:
     """Compile every source and link ``libodl_fp8.so``.  Always recompiles."""
     hipcc = hipcc_path()
     objdir = os.path.join(HERE, "csrc", "_obj")
     os.makedirs(objdir, exist_ok=True)
+    for stale in glob.glob(os.path.join(objdir, "*.s")):
+        os.remove(stale)
     procs = []
     for src in SOURCES:
         obj = os.path.join(objdir, src.replace(".hip", ".o"))
         cmd = [hipcc, *HIPCC_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
-        if keep_asm:
-            cmd += ["-save-temps=obj"]
+        cmd += ["-save-temps=obj"]              # keeps the device assembly for the hazard check below
         if verbose:
             print(" ".join(cmd), flush=True)
         procs.append((src, obj, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
@@ -63,6 +114,16 @@ def build(verbose: bool = False, keep_asm: bool = False) -> str:
         if verbose and out.strip():
             print(out)
         objs.append(obj)
+    problems = []
+    for asm in sorted(glob.glob(os.path.join(objdir, "*gfx950*.s"))):
+        with open(asm) as fh:
+            problems += check_asm_hazards(fh.read(), os.path.basename(asm))
+    if problems:
+        raise RuntimeError("inline-asm hazards in the generated code:\n" + "\n".join(problems))
+    if not keep_asm:
+        for tmpf in glob.glob(os.path.join(objdir, "*")):
+            if not tmpf.endswith(".o"):
+                os.remove(tmpf)
     tmp = LIB_PATH + ".tmp"
     link = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *objs]
     r = subprocess.run(link, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)

@@ -148,8 +148,10 @@ __device__ __forceinline__ void epilogue_staged(const GemmArgs &g, v16f (&acc)[T
     }
 }
 
-// launchers implemented in gemm_tiled.hip / gemm_pipe.hip (fa, fb: odl_fp8_format of A and B)
+// launchers implemented in gemm_tiled.hip / gemm_pipe.hip / gemm_stream.hip (fa, fb: odl_fp8_format of A and B)
 void launch_gemm_tiled(int variant, int fa, int fb, const GemmArgs &g, hipStream_t stream);
 void launch_gemm_pipe(int fa, int fb, const GemmArgs &g, int num_cus, hipStream_t stream);
+bool gemm_stream_accepts(const GemmArgs &g);
+void launch_gemm_stream(int fa, int fb, const GemmArgs &g, int num_cus, hipStream_t stream);
 
 }  // namespace odl

@@ -5,6 +5,8 @@
 // Both operands are K-contiguous 8-bit codes ("NT").  Kernels:
 //   gemm_tiled.hip : BM x BN block tiles through two LDS stages
 //   gemm_pipe.hip  : 256x256 tile, one wave per SIMD, explicit software pipeline
+//   gemm_stream.hip: the same pipeline running across tile boundaries, epilogue under the
+//                    next tile's MFMAs (bf16 output, per-tensor scales, whole tiles only)
 //   here           : generic one-wave-per-32x32-tile kernel for any M, N, K % 16 == 0
 #include "gemm_common.h"
 
@@ -51,8 +53,9 @@ static const Variant kVariants[] = {
     {"128x128x128 4 waves (64x64 per wave)", 128, 128, 256, 0.70f},
     {"256x256x128 4 waves, software-pipelined, persistent (K % 256 == 0)", 256, 256, 256, 1.10f},
     {"256x256x128 4 waves, software-pipelined, one tile per block", 256, 256, 256, 0.50f},
+    {"256x256x128 4 waves, streaming across tiles, folded epilogue (whole tiles, per-tensor scales, bf16)", 256, 256, 256, 1.25f},
 };
-constexpr int kPipeVariant = 5, kPipeOneTileVariant = 6;
+constexpr int kPipeVariant = 5, kPipeOneTileVariant = 6, kStreamVariant = 7;
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 static int g_forced_variant = -1;
 
@@ -79,11 +82,12 @@ static int cu_count() {
     return cus;
 }
 
-static int choose_variant(int64_t M, int64_t N) {
+static int choose_variant(int64_t M, int64_t N, bool stream_ok) {
     const int cus = cu_count();
     int best = 2;
     double best_score = -1.0;
     for (int v = 2; v < kNumVariants; ++v) {                       // variant 1 (one wave per SIMD) only by explicit request
+        if (v == kStreamVariant && !stream_ok) continue;
         const Variant &cfg = kVariants[v];
         const int64_t tiles = ((M + cfg.bm - 1) / cfg.bm) * ((N + cfg.bn - 1) / cfg.bn);
         const int per_cu = cfg.bm * cfg.bn >= 256 * 256 ? 1 : (cfg.bm * cfg.bn >= 256 * 128 ? 1 : 2);
@@ -134,7 +138,9 @@ extern "C" int odl_fp8_gemm_nt(const uint8_t *a, const uint8_t *b, int64_t M, in
     if (M == 0 || N == 0) return ODL_OK;
 
     const bool tiled_ok = K >= 128 && K % 128 == 0 && (double)M * (double)K < 4294967296.0 && (double)N * (double)K < 4294967296.0;
-    int variant = g_forced_variant >= 0 ? g_forced_variant : (tiled_ok ? choose_variant(M, N) : 0);
+    const bool stream_ok = tiled_ok && out_dtype == ODL_BF16 && sa_n == 1 && sb_n == 1 && !bias && M % 256 == 0 && N % 256 == 0 &&
+                           K % 256 == 0 && K >= 512;
+    int variant = g_forced_variant >= 0 ? g_forced_variant : (tiled_ok ? choose_variant(M, N, stream_ok) : 0);
     if (variant != 0 && !tiled_ok) variant = 0;
     // the pipelined kernel walks K in pairs of 128-byte steps and addresses rows with 32-bit byte offsets
     const bool pipe_ok = tiled_ok && K % 256 == 0 && (double)(M + 256) * (double)K < 2147483648.0 &&
@@ -152,9 +158,14 @@ extern "C" int odl_fp8_gemm_nt(const uint8_t *a, const uint8_t *b, int64_t M, in
     if (tm * tn > 0x7ffffff0LL) return set_error(ODL_ERR_SHAPE, "odl_fp8_gemm_nt: too many tiles");
     g.tiles_m = (int)tm; g.tiles_n = (int)tn;
 
+    if (variant == kStreamVariant && !(pipe_ok && gemm_stream_accepts(g))) {
+        // the streaming kernel only takes whole tiles with per-tensor scales: next best kernel instead
+        variant = pipe_ok ? kPipeVariant : 2;
+    }
     if (variant == 0) launch_gemm_generic(fmt_a, fmt_b, g, stream);
     else if (variant == kPipeVariant) launch_gemm_pipe(fmt_a, fmt_b, g, cu_count(), stream);
     else if (variant == kPipeOneTileVariant) launch_gemm_pipe(fmt_a, fmt_b, g, 1 << 30, stream);
+    else if (variant == kStreamVariant) launch_gemm_stream(fmt_a, fmt_b, g, cu_count(), stream);
     else launch_gemm_tiled(variant, fmt_a, fmt_b, g, stream);
     return check_launch("odl_fp8_gemm_nt");
 }

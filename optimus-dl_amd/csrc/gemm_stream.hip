@@ -1,0 +1,355 @@
+// FP8 GEMM, 256x256 block tile, 4 waves (one per SIMD, 128x128 each), persistent,
+// with the epilogue of every tile folded under the first MFMAs of the next one.
+// C = (A[M,K] . B[N,K]^T) * (sa_inv * sb_inv) in bf16, for the shapes training uses:
+// M % 256 == 0, N % 256 == 0, K % 256 == 0, K >= 512, per-tensor scales, no bias.
+// Everything else goes to gemm_pipe.hip, whose K step this kernel shares:
+//
+//   per K step of 128 bytes (two halves h0, h1 of 64 bytes = one MFMA K each)
+//     phase A : 16 MFMAs on register buffer 0 (step kt, h0)
+//               interleaved with the 16 LDS reads of (kt, h1) into buffer 1
+//     wait vmcnt + lgkmcnt(0), s_barrier         <- the only sync per K step
+//     phase B : 16 MFMAs on buffer 1 (kt, h1)
+//               interleaved with the 16 LDS reads of (kt+1, h0) into buffer 0
+//               and the 16 direct-to-LDS loads of step kt+2 into this stage
+//
+// What is different here:
+//
+// * The load pipeline does not stop at a tile boundary.  The last two K steps of a
+//   tile request the first two of the block's next tile (its last tile requests from
+//   an empty buffer, which reads as zero without touching memory), so the whole
+//   kernel is one uniform stream of steps and no tile ever waits for its first loads.
+//
+// * With one wave per SIMD nobody else can use the MFMA pipe while a wave converts
+//   and stores its 128x128 results (about a sixth of a tile's time).  So phase A of a
+//   tile's step 0 starts each 32x32 sub-tile from a zero C operand, and just before
+//   MFMA i is issued the previous tile's sub-tile i is read out of the accumulators,
+//   scaled, rounded to bf16 (v_cvt_pk_bf16_f32) and written to a private LDS slab;
+//   after every second MFMA the slab (32 rows x 64 columns) is read back along the
+//   rows and leaves as full 128-byte lines.  The conversion runs on the vector ALU
+//   while the matrix pipe works on the MFMA just issued.  After a block's last tile
+//   the same phase runs once more on operands nobody uses, only to store that tile.
+//
+// * The tile loop is rotated so that the accumulators are read (by the vector ALU)
+//   in the same straight-line block in which the last MFMAs of the tile define them:
+//   the loop body is [phase B of step 0, steps 1 .. KT-1, folded phase A of the next
+//   tile].  Across the loop edge the accumulators are only ever MFMA operands.
+//
+// Vector-memory counter: all loads and stores of the loop are inline asm and every
+// wait is written by hand.  The counter retires in issue order, so "vmcnt(n)" means
+// "everything but the youngest n operations has completed":
+//   step 0 : younger than the loads of step 1 are 2 prefetch loads and the 32 output
+//            stores of the folded epilogue           -> vmcnt(34)
+//   others : younger than the loads of step kt+1 are 2 prefetch loads -> vmcnt(2)
+#include "gemm_common.h"
+
+namespace odl {
+
+namespace {
+
+constexpr int BM = 256, BN = 256, NW = 4, WM = 128, WN = 128, TM = 4, TN = 4;
+constexpr int REGION = 256 * 128;          // bytes of one operand in one stage
+constexpr int LOADS = 256 / 8 / NW;        // 1 KB direct-to-LDS loads per wave per operand per stage
+constexpr int GM = 8;
+constexpr int PF = 4;                      // L2 prefetch distance in K steps
+constexpr int PITCH = 128 + 16;            // slab row: 64 bf16 + pad
+constexpr int SLAB = 32 * PITCH;           // one wave's epilogue slab
+
+template <int FA, int FB>
+__global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
+    __shared__ __attribute__((aligned(1024))) uint8_t sA0[REGION];
+    __shared__ __attribute__((aligned(1024))) uint8_t sB0[REGION];
+    __shared__ __attribute__((aligned(1024))) uint8_t sA1[REGION];
+    __shared__ __attribute__((aligned(1024))) uint8_t sB1[REGION];
+    __shared__ __attribute__((aligned(16))) uint8_t sEpi[NW * SLAB];
+
+    const int lane = threadIdx.x % 64;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
+    const int wm0 = (wave / 2) * WM, wn0 = (wave % 2) * WN;
+    const int lr = lane % 32, lg = lane / 32;
+    const int KT = (int)(g.K / 128);
+
+    // ---- which tiles: block ids are dealt round-robin to the 8 XCDs, so the blocks of
+    // one XCD (id % 8) walk one contiguous chunk of the grouped tile order together
+    const int total = g.tiles_m * g.tiles_n;
+    const int per_xcd = (total + 7) / 8;
+    const int xcd = (int)(blockIdx.x % 8), stride = (int)(gridDim.x / 8);
+    const int pid_end = min((xcd + 1) * per_xcd, total);
+    int pid = xcd * per_xcd + (int)(blockIdx.x / 8);
+    if (pid >= pid_end) return;
+
+    // ---- per-tile addressing: the tile's origin lives in the buffer resources, the
+    // per-lane offsets are the same for every tile and for both operands
+    const v4i empty = {0, 0, 0, 0x00020000};      // zero bytes: loads read as zero, stores are dropped
+    auto tile_origin = [&](int p, int &tm0, int &tn0) {
+        const int in_group = GM * g.tiles_n;
+        const int first_m = (p / in_group) * GM;
+        const int group_rows = min(g.tiles_m - first_m, GM);
+        tm0 = (first_m + (p % in_group) % group_rows) * BM;
+        tn0 = ((p % in_group) / group_rows) * BN;
+    };
+    auto rsrc_for = [&](const uint8_t *base, int row0, int64_t rows) -> v4i {
+        const uint64_t addr = reinterpret_cast<uint64_t>(base + (int64_t)row0 * g.K);
+        return v4i{(int)(uint32_t)addr, (int)(uint32_t)(addr >> 32), (int)((rows - row0) * g.K), 0x00020000};
+    };
+    int voff[LOADS];
+#pragma unroll
+    for (int j = 0; j < LOADS; ++j) {
+        const int row = (wave + j * NW) * 8 + lane / 8;
+        voff[j] = row * (int)g.K + (((lane % 8) ^ swz(row)) << 4);
+    }
+    // one 1 KB direct-to-LDS load: 64 lanes x 16 bytes land at lds_addr + lane * 16
+    auto dma = [&](const v4i &rsrc, uint32_t lds_addr, int vo, int so) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                     ::"s"(lds_addr), "v"(vo), "s"(rsrc), "s"(so));
+    };
+    auto lds_addr_of = [](const uint8_t *p) { return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) uint8_t *)p; };
+    // load j of a stage: j < LOADS -> operand A, else operand B
+    auto issue_one = [&](uint8_t *sa, uint8_t *sb, const v4i &da, const v4i &db, int koff, int j) {
+        if (j < LOADS) dma(da, lds_addr_of(sa) + (wave + j * NW) * 1024, voff[j], koff);
+        else dma(db, lds_addr_of(sb) + (wave + (j - LOADS) * NW) * 1024, voff[j - LOADS], koff);
+    };
+
+    int m0 = 0, n0 = 0;
+    v4i rsrc_a, rsrc_b, next_a, next_b;           // raw buffer descriptors (base, stride 0, bytes, format)
+
+    // ---- L2 prefetch: each lane touches one 128-byte line of the step PF ahead with a load
+    // whose value is never used; steps past the end of this tile belong to the next one.
+    // Issued after the DMA loads of the same phase, so they are the 2 youngest operations.
+    const int pf_off = (wave * 64 + lane) * (int)g.K;
+    int pfv_a = 0, pfv_b = 0;
+    auto prefetch = [&](int kt) {
+        const bool nx = kt >= KT;
+        const int kp = (nx ? kt - KT : kt) * 128;
+        const v4i pa = nx ? next_a : rsrc_a, pb = nx ? next_b : rsrc_b;
+        asm volatile("buffer_load_dword %0, %1, %2, %3 offen" : "+v"(pfv_a) : "v"(pf_off), "s"(pa), "s"(kp));
+        asm volatile("buffer_load_dword %0, %1, %2, %3 offen" : "+v"(pfv_b) : "v"(pf_off), "s"(pb), "s"(kp));
+    };
+
+    // ---- LDS -> registers.  chunk(t, h, e) = ((2*lg + e) ^ s0) ^ 4*(h ^ (t & 1))
+    int ra[2][2], rb[2][2];                     // [e][h ^ (t & 1)] byte offsets inside a region (tile 0)
+    {
+        const int rowa = wm0 + lr, rowb = wn0 + lr;
+        const int s0a = swz(rowa), s0b = swz(rowb);
+#pragma unroll
+        for (int e = 0; e < 2; ++e)
+#pragma unroll
+            for (int p = 0; p < 2; ++p) {
+                ra[e][p] = rowa * 128 + (((((2 * lg + e) ^ s0a)) ^ (4 * p)) << 4);
+                rb[e][p] = rowb * 128 + (((((2 * lg + e) ^ s0b)) ^ (4 * p)) << 4);
+            }
+    }
+    auto read_a = [&](const uint8_t *sa, int t, int h) -> v8i {
+        const v4i lo = *reinterpret_cast<const v4i *>(sa + ra[0][h ^ (t & 1)] + t * 4096);
+        const v4i hi = *reinterpret_cast<const v4i *>(sa + ra[1][h ^ (t & 1)] + t * 4096);
+        return v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    };
+    auto read_b = [&](const uint8_t *sb, int u, int h) -> v8i {
+        const v4i lo = *reinterpret_cast<const v4i *>(sb + rb[0][h ^ (u & 1)] + u * 4096);
+        const v4i hi = *reinterpret_cast<const v4i *>(sb + rb[1][h ^ (u & 1)] + u * 4096);
+        return v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    };
+
+    v16f acc[TM][TN];
+    v8i a0[TM], b0[TN], a1[TM], b1[TN];         // register buffers 0 (h0) and 1 (h1)
+    const v16f zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+
+    // ---- output side of the folded epilogue
+    const int n2 = (int)g.N * 2;                  // bytes per output row
+    const int c_soff0 = (wm0 * (int)g.N + wn0) * 2;
+    const float s_tensor = bits_to_float((uint32_t)__builtin_amdgcn_readfirstlane((int)float_to_bits(g.sa[0] * g.sb[0])));
+    auto rsrc_out = [&](int tm0, int tn0) -> v4i {
+        const uint64_t addr = reinterpret_cast<uint64_t>(reinterpret_cast<uint8_t *>(g.c) + ((int64_t)tm0 * g.N + tn0) * 2);
+        return v4i{(int)(uint32_t)addr, (int)(uint32_t)(addr >> 32), (int)0x80000000u, 0x00020000};
+    };
+    auto store_slab = [](const u32x4 (&data)[4], int vo, const v4i &rsrc, int so_base, int row_bytes, int t, int us) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int so = so_base + (32 * t + 8 * j) * row_bytes + 64 * us;
+            // s_nop 4: a scalar register written by a vector instruction (the compiler restores
+            // spilled scalars that way) must not be read by a vector-memory instruction for 5
+            // cycles, and the compiler does not look inside asm statements for that hazard
+            asm volatile("s_nop 4\n\tbuffer_store_dwordx4 %0, %1, %2, %3 offen" ::"v"(data[j]), "v"(vo), "s"(rsrc), "s"(so));
+        }
+    };
+    auto lds_w = [](uint32_t addr) { return (__attribute__((address_space(3))) u32x2 *)addr; };
+    auto lds_r = [](uint32_t addr) { return (const __attribute__((address_space(3))) u32x4 *)addr; };
+
+    // phase A of a step: MFMA i works on sub-tile (t, u) = (i / 4, i % 4); the 8 fragments of
+    // (kt, h1) stream into buffer 1 behind the first 8 MFMAs.
+    auto phase_a = [&](const uint8_t *sa_cur, const uint8_t *sb_cur) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            acc[i / 4][i % 4] = mfma_32x32x64<FB, FA>(b0[i % 4], a0[i / 4], acc[i / 4][i % 4]);
+            if (i < 4) a1[i] = read_a(sa_cur, i, 1);
+            else if (i < 8) b1[i - 4] = read_b(sb_cur, i - 4, 1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    // phase A of step 0 of the first tile: accumulators start from zero
+    auto phase_a_first = [&](const uint8_t *sa_cur, const uint8_t *sb_cur) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            acc[i / 4][i % 4] = mfma_32x32x64<FB, FA>(b0[i % 4], a0[i / 4], zero16);
+            if (i < 4) a1[i] = read_a(sa_cur, i, 1);
+            else if (i < 8) b1[i - 4] = read_b(sb_cur, i - 4, 1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    // phase A of step 0 of a later tile (or the drain after the last one): the finished tile
+    // leaves through `rsrc_c` while its accumulators are restarted from zero
+    auto phase_a_fold = [&](const uint8_t *sa_cur, const uint8_t *sb_cur, const v4i &rsrc_c) {
+        // addresses are derived here (laundered ids), not kept in registers across the K loop
+        int lane_e = lane, wave_e = wave;
+        asm volatile("" : "+v"(lane_e));
+        asm volatile("" : "+s"(wave_e));
+        const uint32_t slab = lds_addr_of(sEpi) + wave_e * SLAB;
+        const uint32_t epi_w = slab + (lane_e % 32) * PITCH + (lane_e / 32) * 8;
+        const uint32_t epi_r = slab + (lane_e / 8) * PITCH + (lane_e % 8) * 16;
+        const int c_voff = (lane_e / 8) * n2 + (lane_e % 8) * 16;
+        u32x4 back[4];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int t = i / 4, u = i % 4;
+            uint32_t pk[8];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                pk[2 * q] = pack_bf16x2(acc[t][u][4 * q] * s_tensor, acc[t][u][4 * q + 1] * s_tensor);
+                pk[2 * q + 1] = pack_bf16x2(acc[t][u][4 * q + 2] * s_tensor, acc[t][u][4 * q + 3] * s_tensor);
+            }
+            acc[t][u] = mfma_32x32x64<FB, FA>(b0[u], a0[t], zero16);
+            // lane (lr, lg) holds columns 8q + 4lg + {0..3} of row lr of the sub-tile
+#pragma unroll
+            for (int q = 0; q < 4; ++q) *lds_w(epi_w + (u & 1) * 64 + q * 16) = u32x2{pk[2 * q], pk[2 * q + 1]};
+            if (u & 1) {
+                // slab complete: 8 lanes cover a row with 16 bytes each, 8 rows per instruction.
+                // LDS operations of a wave execute in order, so the next writes cannot overtake these reads.
+#pragma unroll
+                for (int j = 0; j < 4; ++j) back[j] = *lds_r(epi_r + j * 8 * PITCH);
+            } else if (i > 0) {
+                store_slab(back, c_voff, rsrc_c, c_soff0, n2, (i - 2) / 4, (i - 2) % 4);   // completed one MFMA ago
+            }
+            if (i < 4) a1[i] = read_a(sa_cur, i, 1);
+            else if (i < 8) b1[i - 4] = read_b(sb_cur, i - 4, 1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        store_slab(back, c_voff, rsrc_c, c_soff0, n2, 3, 2);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    auto sync = [&](int simm16) {
+        if (simm16 == 0x8072) __builtin_amdgcn_s_waitcnt(0x8072);   // vmcnt(34) lgkmcnt(0)
+        else __builtin_amdgcn_s_waitcnt(0x0072);                    // vmcnt(2) lgkmcnt(0)
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    // phase B: MFMAs on buffer 1; (kt+1, h0) streams into buffer 0; step kt+2 is requested into
+    // the stage just consumed -- from the next tile when this tile has no such step
+    auto phase_b = [&](uint8_t *sa_cur, uint8_t *sb_cur, const uint8_t *sa_nxt, const uint8_t *sb_nxt, int kt) {
+        const bool nx = kt + 2 >= KT;
+        const v4i la = nx ? next_a : rsrc_a, lb = nx ? next_b : rsrc_b;
+        const int koff = (nx ? kt + 2 - KT : kt + 2) * 128;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            acc[i / 4][i % 4] = mfma_32x32x64<FB, FA>(b1[i % 4], a1[i / 4], acc[i / 4][i % 4]);
+            if (i < 4) a0[i] = read_a(sa_nxt, i, 0);
+            else if (i < 8) b0[i - 4] = read_b(sb_nxt, i - 4, 0);
+            issue_one(sa_cur, sb_cur, la, lb, koff, i);
+            if (i == 15) prefetch(kt + 2 + PF);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    auto step = [&](uint8_t *sa_cur, uint8_t *sb_cur, uint8_t *sa_nxt, uint8_t *sb_nxt, int kt) {
+        phase_a(sa_cur, sb_cur);
+        sync(0x0072);
+        phase_b(sa_cur, sb_cur, sa_nxt, sb_nxt, kt);
+    };
+
+    // ---- first tile: steps 0 and 1 requested and awaited, then phase A of step 0
+    tile_origin(pid, m0, n0);
+    rsrc_a = rsrc_for(g.a, m0, g.M);
+    rsrc_b = rsrc_for(g.b, n0, g.N);
+    next_a = empty;
+    next_b = empty;
+#pragma unroll
+    for (int j = 0; j < 2 * LOADS; ++j) issue_one(sA0, sB0, rsrc_a, rsrc_b, 0, j);
+#pragma unroll
+    for (int j = 0; j < 2 * LOADS; ++j) issue_one(sA1, sB1, rsrc_a, rsrc_b, 128, j);
+    for (int k = 2; k < 2 + PF; ++k) prefetch(k);
+    __builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0)
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int t = 0; t < TM; ++t) a0[t] = read_a(sA0, t, 0);
+#pragma unroll
+    for (int u = 0; u < TN; ++u) b0[u] = read_b(sB0, u, 0);
+    phase_a_first(sA0, sB0);
+
+    while (true) {
+        // the block's next tile, if any (scalar work only; no branches around vector code)
+        const int next_pid = pid + stride;
+        const bool has_next = next_pid < pid_end;
+        int next_m0 = 0, next_n0 = 0;
+        tile_origin(has_next ? next_pid : pid, next_m0, next_n0);
+        const v4i na = rsrc_for(g.a, next_m0, g.M), nb = rsrc_for(g.b, next_n0, g.N);
+        next_a = has_next ? na : empty;
+        next_b = has_next ? nb : empty;
+
+        // ---- rest of step 0 (its phase A ran at the end of the previous trip), then steps 1 .. KT-1.
+        // The first trip's step 0 and every drained tile's step 0 carry 32 stores (dropped ones
+        // count too), the first tile's none: vmcnt(34) is then simply satisfied earlier.
+        sync(0x8072);
+        phase_b(sA0, sB0, sA1, sB1, 0);
+        step(sA1, sB1, sA0, sB0, 1);
+        for (int kt = 2; kt < KT - 2; kt += 2) {
+            step(sA0, sB0, sA1, sB1, kt);
+            step(sA1, sB1, sA0, sB0, kt + 1);
+        }
+        step(sA0, sB0, sA1, sB1, KT - 2);
+        step(sA1, sB1, sA0, sB0, KT - 1);
+
+        // ---- the tile is finished; buffer 0 already holds the next tile's first fragments.
+        // Phase A of the next tile's step 0 stores this tile.  Without a next tile the same
+        // phase runs on whatever the empty buffer delivered, only for its stores.
+        const v4i rsrc_c = rsrc_out(m0, n0);
+        pid = next_pid;
+        m0 = next_m0;
+        n0 = next_n0;
+        rsrc_a = next_a;
+        rsrc_b = next_b;
+        phase_a_fold(sA0, sB0, rsrc_c);
+        if (!has_next) break;
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0): nothing may still be writing the prefetch registers
+    asm volatile("" ::"v"(pfv_a), "v"(pfv_b));
+}
+
+template <int FA, int FB>
+void launch_fmt(const GemmArgs &g, int blocks_per_xcd, hipStream_t stream) {
+    hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB>), dim3((unsigned)(8 * blocks_per_xcd)), dim3(256), 0, stream, g);
+}
+
+}  // namespace
+
+// Shapes this kernel takes (the caller checks the 32-bit offset limits shared with gemm_pipe.hip).
+bool gemm_stream_accepts(const GemmArgs &g) {
+    return g.out_dtype == ODL_BF16 && !g.sa_vec && !g.sb_vec && g.bias == nullptr && g.M % BM == 0 && g.N % BN == 0 &&
+           g.K % 256 == 0 && g.K >= 512 && (double)g.N * 2.0 * (BM + 8) < 2147483648.0;
+}
+
+// One block per CU at most (the kernel needs ~150 KB of LDS), 8 | grid so that the
+// round-robin placement gives every XCD the same number of blocks.
+void launch_gemm_stream(int fa, int fb, const GemmArgs &g, int num_cus, hipStream_t stream) {
+    const int total = g.tiles_m * g.tiles_n;
+    const int per_xcd = (total + 7) / 8;
+    int bpx = num_cus / 8;
+    if (bpx < 1) bpx = 1;
+    if (bpx > per_xcd) bpx = per_xcd;
+    if (fa == ODL_FP8_E4M3 && fb == ODL_FP8_E4M3) launch_fmt<ODL_FP8_E4M3, ODL_FP8_E4M3>(g, bpx, stream);
+    else if (fa == ODL_FP8_E5M2 && fb == ODL_FP8_E4M3) launch_fmt<ODL_FP8_E5M2, ODL_FP8_E4M3>(g, bpx, stream);
+    else if (fa == ODL_FP8_E4M3 && fb == ODL_FP8_E5M2) launch_fmt<ODL_FP8_E4M3, ODL_FP8_E5M2>(g, bpx, stream);
+    else launch_fmt<ODL_FP8_E5M2, ODL_FP8_E5M2>(g, bpx, stream);
+}
+
+}  // namespace odl

@@ -53,3 +53,23 @@ def test_cpu_tensors_are_refused_not_emulated():
         pytest.skip("library not built")
     with pytest.raises(native.NativeError):
         native.amax(torch.zeros((4, 4), dtype=torch.bfloat16))
+
+
+def test_build_rejects_asm_that_reads_a_scalar_too_soon_after_a_vector_write():
+    from optimus_dl_amd.build import check_asm_hazards
+
+    bad = """
+	v_readlane_b32 s0, v180, 14
+	;;#ASMSTART
+	buffer_store_dwordx4 v[60:63], v0, s[16:19], s0 offen
+	;;#ASMEND
+"""
+    good = bad.replace("\tbuffer_store", "\ts_nop 4\n\tbuffer_store")
+    other_register = bad.replace("s_readlane", "s_readlane").replace("v_readlane_b32 s0", "v_readlane_b32 s7")
+    in_descriptor = bad.replace("v_readlane_b32 s0", "v_readlane_b32 s18")
+    assert len(check_asm_hazards(bad, "x.s")) == 1
+    assert check_asm_hazards(good, "x.s") == []
+    assert check_asm_hazards(other_register, "x.s") == []
+    assert len(check_asm_hazards(in_descriptor, "x.s")) == 1
+    # instructions the compiler emitted itself are its own business
+    assert check_asm_hazards("\tv_readlane_b32 s0, v1, 2\n\tbuffer_load_dword v1, v0, s[16:19], s0 offen\n", "x.s") == []
