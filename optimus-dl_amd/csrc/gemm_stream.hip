@@ -42,6 +42,10 @@
 //   others : younger than the loads of step kt+1 are 2 prefetch loads -> vmcnt(2)
 #include "gemm_common.h"
 
+#ifndef ODL_STREAM_PF
+#define ODL_STREAM_PF 0
+#endif
+
 namespace odl {
 
 namespace {
@@ -50,7 +54,8 @@ constexpr int BM = 256, BN = 256, NW = 4, WM = 128, WN = 128, TM = 4, TN = 4;
 constexpr int REGION = 256 * 128;          // bytes of one operand in one stage
 constexpr int LOADS = 256 / 8 / NW;        // 1 KB direct-to-LDS loads per wave per operand per stage
 constexpr int GM = 8;
-constexpr int PF = 4;                      // L2 prefetch distance in K steps
+constexpr int PF = ODL_STREAM_PF;          // L2 prefetch distance in K steps, 0 = none
+constexpr int NPF = PF > 0 ? 2 : 0;        // prefetch loads per wave per step
 constexpr int PITCH = 128 + 16;            // slab row: 64 bf16 + pad
 constexpr int SLAB = 32 * PITCH;           // one wave's epilogue slab
 
@@ -118,6 +123,7 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
     const int pf_off = (wave * 64 + lane) * (int)g.K;
     int pfv_a = 0, pfv_b = 0;
     auto prefetch = [&](int kt) {
+        if constexpr (PF == 0) return;
         const bool nx = kt >= KT;
         const int kp = (nx ? kt - KT : kt) * 128;
         const v4i pa = nx ? next_a : rsrc_a, pb = nx ? next_b : rsrc_b;
@@ -236,8 +242,9 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
         __builtin_amdgcn_sched_barrier(0);
     };
     auto sync = [&](int simm16) {
-        if (simm16 == 0x8072) __builtin_amdgcn_s_waitcnt(0x8072);   // vmcnt(34) lgkmcnt(0)
-        else __builtin_amdgcn_s_waitcnt(0x0072);                    // vmcnt(2) lgkmcnt(0)
+        // vmcnt(32 + NPF) or vmcnt(NPF), both with lgkmcnt(0)
+        if (simm16 == 0x8072) __builtin_amdgcn_s_waitcnt(0x8070 | NPF);
+        else __builtin_amdgcn_s_waitcnt(0x0070 | NPF);
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
