@@ -55,7 +55,11 @@ constexpr int BM = 256, BN = 256, NW = 4, WM = 128, WN = 128, TM = 4, TN = 4;
 constexpr int REGION = 256 * 128;          // bytes of one operand in one stage
 constexpr int LOADS = 256 / 8 / NW;        // 1 KB direct-to-LDS loads per wave per operand per stage
 constexpr int GM = 8;
-constexpr int PF = 4;                      // L2 prefetch distance in K steps
+#ifndef ODL_PIPE_PF
+#define ODL_PIPE_PF 0
+#endif
+constexpr int PF = ODL_PIPE_PF;            // L2 prefetch distance in K steps, 0 = none
+constexpr int NPF = PF > 0 ? 2 : 0;        // prefetch loads per wave per step
 constexpr int EPI_BYTES = 32 * (128 + 16); // one wave's epilogue slab: 32 rows x 128 bytes (+16 pad)
 static_assert(staged_epilogue_bytes<true, 2>() == EPI_BYTES && staged_epilogue_bytes<false, 1>() == EPI_BYTES, "slab size");
 
@@ -134,6 +138,7 @@ __global__ __launch_bounds__(256) void gemm_nt_pipe_kernel(const GemmArgs g) {
     bool has_next = false;
     int pfv_a = 0, pfv_b = 0;
     auto prefetch = [&](int kt) {
+        if constexpr (PF == 0) return;
         const bool nx = kt >= KT && has_next;
         const int kp = (nx ? kt - KT : min(kt, KT - 1)) * 128;
         asm volatile("buffer_load_dword %0, %1, %2, %3 offen" : "+v"(pfv_a) : "v"(pf_off), "s"(nx ? next_a : rsrc_a), "s"(kp));
@@ -186,7 +191,7 @@ __global__ __launch_bounds__(256) void gemm_nt_pipe_kernel(const GemmArgs g) {
             __builtin_amdgcn_sched_barrier(0);
         }
         // my DMA for kt+1 has landed (the 2 younger prefetch loads may still be out), my LDS reads returned
-        __builtin_amdgcn_s_waitcnt(0x0072);     // vmcnt(2) lgkmcnt(0)
+        __builtin_amdgcn_s_waitcnt(0x0070 | NPF);   // vmcnt(NPF) lgkmcnt(0)
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
