@@ -51,7 +51,8 @@ class KernelTimer:
         self._orig = {}
 
     def install(self):
-        def wrap(name, work_fn):
+        def wrap(name, work_fn, record_as=None):
+            record_as = record_as or name
             orig = getattr(self.native, name)
             self._orig[name] = orig
 
@@ -62,7 +63,7 @@ class KernelTimer:
                 e0.record()
                 out = orig(*a, **kw)
                 e1.record()
-                self.records.setdefault(name, []).append((e0, e1, work_fn(*a, **kw)))
+                self.records.setdefault(record_as, []).append((e0, e1, work_fn(*a, **kw)))
                 return out
 
             setattr(self.native, name, timed)
@@ -72,6 +73,7 @@ class KernelTimer:
 
         wrap("gemm_nt", lambda a, b, *r, **kw: 2.0 * a.shape[0] * b.shape[0] * a.shape[1])            # flops
         wrap("amax", lambda x, *r, **kw: float(x.numel() * esz(x)))                                       # bytes
+        wrap("amax_scale", lambda x, *r, **kw: float(x.numel() * esz(x)), record_as="amax")       # amax + scale, one launch
         wrap("cast", lambda x, *r, **kw: float(x.numel() * (esz(x) + 1)))
         wrap("cast_transpose",
              lambda x, *r, **kw: float(x.numel() * (esz(x) + (2 if kw.get("want_rowmajor", True) else 1))))
@@ -230,7 +232,7 @@ def main() -> int:
         "cast_amax_frac_of_hbm_peak": (quant_bytes / (quant_ms * 1e-3) / 1e9) / PEAK_HBM_GBPS if quant_ms else None,
         "time_split_ms_per_step": {n: ks[n]["total_ms"] / args.steps for n in ks},
         "roofline": {
-            "kernel": "gemm_nt_tiled_kernel (FP8 MFMA GEMM; fwd, dgrad, wgrad launches)",
+            "kernel": "gemm_nt_stream_kernel (FP8 MFMA GEMM; fwd, dgrad, wgrad launches)",
             "bound": "mfma",
             "achieved": gemm_tflops,
             "peak": PEAK_FP8_TFLOPS,

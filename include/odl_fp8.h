@@ -73,6 +73,19 @@ int odl_fp8_scale_from_amax(const float *amax, int64_t n, int fmt, int margin,
                             float *scale, float *scale_inv, odl_stream_t stream);
 
 /*
+ * Per-tensor amax and the scale derived from it in ONE launch: what the recipe
+ * "tensorwise" (current scaling, fp8.py:289-294) does to every tensor before its cast.
+ * Results are those of odl_fp8_amax(mode TENSOR, accumulate 0) followed by
+ * odl_fp8_scale_from_amax(n = 1).  scale_inv may be NULL.
+ * workspace: two 32-bit words of device memory that are zero before the first
+ * call; the kernel leaves them zero, so one workspace serves every call that is
+ * ordered on the same stream.  Calls that may overlap need a workspace each.
+ */
+int odl_fp8_amax_scale(const void *x, int src_dtype, int64_t rows, int64_t cols, int fmt, int margin,
+                       float *amax_out, float *scale, float *scale_inv, uint32_t *workspace,
+                       odl_stream_t stream);
+
+/*
  * out[r,c] = fp8( clamp( fp32(x[r,c]) * s , +-max ) ), s = scale[0] | scale[r] | scale[c].
  * amax_out (may be NULL): *amax_out = max(*amax_out, max|x|), for delayed scaling,
  * where the cast uses an older scale while this step's amax is recorded.

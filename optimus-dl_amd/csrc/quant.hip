@@ -26,12 +26,32 @@ __global__ void fill_f32_kernel(float *p, int64_t n, float v) {
     if (i < n) p[i] = v;
 }
 
+// scale = fp8_max / amax / 2^margin with the guards of the C ABI
+__device__ __forceinline__ float scale_rule(float amax, float fp8_max, int margin, float fallback) {
+    if (!(amax > 0.0f) || __builtin_isinf(amax)) return fallback;
+    float s = __fdiv_rn(fp8_max, amax);                     // IEEE division, not the fast reciprocal
+    s = ldexpf(s, -margin);
+    if (__builtin_isinf(s)) s = FLT_MAX;
+    return s;
+}
+
+
+// Optional tail of the per-tensor amax kernel: the block that finishes last turns the
+// amax into scale and 1/scale, so current scaling needs no second launch.  `ws` is two
+// dwords {amax bits, tickets}, zero on entry; the last block leaves them zero again.
+struct FusedScale {
+    uint32_t *ws;
+    float *scale, *scale_inv;
+    float fp8_max;
+    int margin;
+};
+
 // ------------------------------------------------------------ amax, per tensor
 // x viewed as n16 chunks of 16 bytes plus a scalar tail.  Each lane keeps UNROLL
 // loads in flight; magnitudes are reduced as integer bit patterns.
-template <int SRC, int UNROLL>
+template <int SRC, int UNROLL, bool FUSE>
 __global__ __launch_bounds__(kFatThreads) void amax_tensor_kernel(const void *__restrict__ x, int64_t n,
-                                                                   float *__restrict__ out) {
+                                                                   float *__restrict__ out, const FusedScale fs) {
     __shared__ uint32_t red[kFatThreads / kWave];
     constexpr int EPC = SRC == ODL_BF16 ? 8 : 4;          // elements per 16-byte chunk
     const int64_t n16 = n / EPC;
@@ -88,7 +108,21 @@ __global__ __launch_bounds__(kFatThreads) void amax_tensor_kernel(const void *__
         }
     }
     m = block_max_u32(m, red);
-    if (threadIdx.x == 0 && m != 0) atomicMax(reinterpret_cast<uint32_t *>(out), m);
+    if constexpr (!FUSE) {
+        if (threadIdx.x == 0 && m != 0) atomicMax(reinterpret_cast<uint32_t *>(out), m);
+    } else if (threadIdx.x == 0) {
+        if (m != 0) atomicMax(fs.ws, m);
+        __threadfence();                                     // my maximum is visible before my ticket
+        if (atomicAdd(fs.ws + 1, 1u) == gridDim.x - 1) {     // every other block has drawn its ticket
+            __threadfence();
+            const float amax = bits_to_float(atomicExch(fs.ws, 0u));
+            atomicExch(fs.ws + 1, 0u);
+            const float sc = scale_rule(amax, fs.fp8_max, fs.margin, 1.0f);
+            out[0] = amax;
+            fs.scale[0] = sc;
+            if (fs.scale_inv) fs.scale_inv[0] = __fdiv_rn(1.0f, sc);
+        }
+    }
 }
 
 // element-at-a-time variant for pointers that are not 16-byte aligned
@@ -253,14 +287,6 @@ __global__ void amax_col_scalar_kernel(const void *__restrict__ x, int64_t rows,
 }
 
 // ------------------------------------------------------------- scale from amax
-__device__ __forceinline__ float scale_rule(float amax, float fp8_max, int margin, float fallback) {
-    if (!(amax > 0.0f) || __builtin_isinf(amax)) return fallback;
-    float s = __fdiv_rn(fp8_max, amax);                     // IEEE division, not the fast reciprocal
-    s = ldexpf(s, -margin);
-    if (__builtin_isinf(s)) s = FLT_MAX;
-    return s;
-}
-
 __global__ void scale_from_amax_kernel(const float *__restrict__ amax, int64_t n, float fp8_max, int margin,
                                        float *__restrict__ scale, float *__restrict__ scale_inv) {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -559,8 +585,8 @@ extern "C" int odl_fp8_amax(const void *x, int src_dtype, int64_t rows, int64_t 
     if (mode == ODL_SCALE_TENSOR) {
         if (aligned16(x)) {
             const int64_t g = grid_for(n * esz / 16, kFatThreads * 4, 2);
-            if (src_dtype == ODL_BF16) hipLaunchKernelGGL((amax_tensor_kernel<ODL_BF16, 4>), dim3((unsigned)g), dim3(kFatThreads), 0, stream, x, n, amax_out);
-            else hipLaunchKernelGGL((amax_tensor_kernel<ODL_F32, 4>), dim3((unsigned)g), dim3(kFatThreads), 0, stream, x, n, amax_out);
+            if (src_dtype == ODL_BF16) hipLaunchKernelGGL((amax_tensor_kernel<ODL_BF16, 4, false>), dim3((unsigned)g), dim3(kFatThreads), 0, stream, x, n, amax_out, FusedScale{});
+            else hipLaunchKernelGGL((amax_tensor_kernel<ODL_F32, 4, false>), dim3((unsigned)g), dim3(kFatThreads), 0, stream, x, n, amax_out, FusedScale{});
         } else {
             const int64_t g = grid_for(n, kThreads * 8, 8);
             if (src_dtype == ODL_BF16) hipLaunchKernelGGL((amax_tensor_scalar_kernel<ODL_BF16>), dim3((unsigned)g), dim3(kThreads), 0, stream, x, n, amax_out);
@@ -594,6 +620,28 @@ extern "C" int odl_fp8_amax(const void *x, int src_dtype, int64_t rows, int64_t 
         }
     }
     return check_launch("odl_fp8_amax");
+}
+
+extern "C" int odl_fp8_amax_scale(const void *x, int src_dtype, int64_t rows, int64_t cols, int fmt, int margin, float *amax_out,
+                                  float *scale, float *scale_inv, uint32_t *workspace, odl_stream_t stream_) {
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    if (rows < 0 || cols < 0) return set_error(ODL_ERR_ARG, "odl_fp8_amax_scale: negative shape %lld x %lld", (long long)rows, (long long)cols);
+    if ((!x && rows * cols > 0) || !amax_out || !scale || !workspace) return set_error(ODL_ERR_ARG, "odl_fp8_amax_scale: null pointer");
+    if (src_dtype != ODL_BF16 && src_dtype != ODL_F32) return set_error(ODL_ERR_ARG, "odl_fp8_amax_scale: src_dtype %d", src_dtype);
+    if (fmt != ODL_FP8_E4M3 && fmt != ODL_FP8_E5M2) return set_error(ODL_ERR_ARG, "odl_fp8_amax_scale: fmt %d", fmt);
+    const int64_t n = rows * cols;
+    if (n == 0 || !aligned16(x)) {
+        // nothing to read, or a pointer the vector kernel cannot take: the two-launch route
+        int rc = odl_fp8_amax(x, src_dtype, rows, cols, ODL_SCALE_TENSOR, amax_out, 0, stream_);
+        if (rc != ODL_OK) return rc;
+        return odl_fp8_scale_from_amax(amax_out, 1, fmt, margin, scale, scale_inv, stream_);
+    }
+    const int esz = src_dtype == ODL_BF16 ? 2 : 4;
+    const int64_t g = grid_for(n * esz / 16, kFatThreads * 4, 2);
+    const FusedScale fs{workspace, scale, scale_inv, fmt == ODL_FP8_E5M2 ? 57344.0f : 448.0f, margin};
+    if (src_dtype == ODL_BF16) hipLaunchKernelGGL((amax_tensor_kernel<ODL_BF16, 4, true>), dim3((unsigned)g), dim3(kFatThreads), 0, stream, x, n, amax_out, fs);
+    else hipLaunchKernelGGL((amax_tensor_kernel<ODL_F32, 4, true>), dim3((unsigned)g), dim3(kFatThreads), 0, stream, x, n, amax_out, fs);
+    return check_launch("odl_fp8_amax_scale");
 }
 
 extern "C" int odl_fp8_scale_from_amax(const float *amax, int64_t n, int fmt, int margin, float *scale, float *scale_inv,

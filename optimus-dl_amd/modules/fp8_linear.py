@@ -66,8 +66,7 @@ class _WeightCache:
 
 def _quantise_dynamic(x2d: torch.Tensor, fmt: int, margin: int, need_t: bool, need_rowmajor: bool = True):
     """Per-tensor current scaling: amax pass, scale, cast (+transpose) pass."""
-    amax = native.amax(x2d, T)
-    scale, scale_inv = native.scale_from_amax(amax, fmt, margin)
+    amax, scale, scale_inv = native.amax_scale(x2d, fmt, margin)
     if need_t:
         q, q_t = native.cast_transpose(x2d, scale, fmt, T, want_rowmajor=need_rowmajor)
     else:

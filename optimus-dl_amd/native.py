@@ -33,6 +33,7 @@ EXPORTS = (
     "odl_fp8_last_error",
     "odl_fp8_amax",
     "odl_fp8_scale_from_amax",
+    "odl_fp8_amax_scale",
     "odl_fp8_cast",
     "odl_fp8_cast_transpose",
     "odl_fp8_gemm_nt",
@@ -74,6 +75,7 @@ def load() -> ctypes.CDLL:
         L.odl_fp8_last_error.restype = ctypes.c_char_p
         L.odl_fp8_amax.argtypes = [vp, i32, i64, i64, i32, vp, i32, vp]
         L.odl_fp8_scale_from_amax.argtypes = [vp, i64, i32, i32, vp, vp, vp]
+        L.odl_fp8_amax_scale.argtypes = [vp, i32, i64, i64, i32, i32, vp, vp, vp, vp, vp]
         L.odl_fp8_cast.argtypes = [vp, i32, i64, i64, vp, i32, i32, vp, vp, vp]
         L.odl_fp8_cast_transpose.argtypes = [vp, i32, i64, i64, vp, i32, i32, vp, vp, vp, vp]
         L.odl_fp8_gemm_nt.argtypes = [vp, vp, i64, i64, i64, i32, i32, vp, i64, vp, i64, vp, i32, vp, i32, vp]
@@ -141,6 +143,33 @@ def amax(x: torch.Tensor, mode: int = SCALE_TENSOR, out: torch.Tensor | None = N
     _check(load().odl_fp8_amax(x.data_ptr(), _src_dtype(x), rows, cols, mode, out.data_ptr(), int(accumulate), _stream()),
            "odl_fp8_amax")
     return out
+
+
+_workspaces: dict[tuple[int, int], torch.Tensor] = {}
+
+
+def _workspace(device: torch.device, stream: int) -> torch.Tensor:
+    """Two zeroed words per (device, stream): calls on one stream are ordered, and every
+    call leaves the words zero for the next one."""
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream)
+    ws = _workspaces.get(key)
+    if ws is None:
+        ws = torch.zeros(2, dtype=torch.int32, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def amax_scale(x: torch.Tensor, fmt: int, margin: int = 0):
+    """Per-tensor amax, scale and 1/scale in one launch -> (amax, scale, scale_inv), each fp32[1]."""
+    x = _as_2d(x)
+    rows, cols = x.shape
+    out = torch.empty(3, dtype=torch.float32, device=x.device)
+    stream = _stream()
+    ws = _workspace(x.device, stream)
+    base = out.data_ptr()
+    _check(load().odl_fp8_amax_scale(x.data_ptr(), _src_dtype(x), rows, cols, fmt, margin, base, base + 4, base + 8,
+                                     ws.data_ptr(), stream), "odl_fp8_amax_scale")
+    return out[0:1], out[1:2], out[2:3]
 
 
 def scale_from_amax(amax_t: torch.Tensor, fmt: int, margin: int = 0):

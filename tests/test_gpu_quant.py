@@ -63,6 +63,42 @@ def test_amax_unaligned_view(N):
 
 
 @pytest.mark.parametrize("fmt", [O.E4M3, O.E5M2])
+def test_amax_scale_in_one_launch_equals_the_two_step_route(N, fmt):
+    """One call after another on the same stream: the shared workspace must come back to zero
+    every time, whatever the grid size of the call before."""
+    cases = [((8192, 4096), 1.0, torch.bfloat16), ((16, 16), 0.02, torch.bfloat16), ((1000, 200), 3.0, torch.float32),
+             ((7, 13), 1e-3, torch.bfloat16), ((4096, 1024), 50.0, torch.bfloat16), ((1, 8), 1.0, torch.float32)]
+    for margin in (0, 2):
+        for i, (shape, std, dtype) in enumerate(cases):
+            x = seeded_bf16(shape, std=std, seed=10 + i)
+            xd = x.to(dtype).cuda()
+            amax, scale, scale_inv = N.amax_scale(xd, fmt, margin)
+            want_amax = O.t_amax(x)
+            want_scale = np.float32(O.c_scale(float(want_amax), fmt, margin, 1.0))
+            assert_f32_bits_equal(amax, want_amax, f"fused amax {shape}")
+            assert_f32_bits_equal(scale, torch.tensor([want_scale]), f"fused scale {shape}")
+            assert_f32_bits_equal(scale_inv, torch.tensor([np.float32(O.c_scale_inv(want_scale))]), f"fused 1/scale {shape}")
+            two_a = N.amax(xd)
+            two_s, two_si = N.scale_from_amax(two_a, fmt, margin)
+            assert_f32_bits_equal(torch.cat([amax, scale, scale_inv]), torch.cat([two_a, two_s, two_si]).cpu(), "fused vs two-step")
+    # specials: all zero -> scale 1; NaN propagates into amax and falls back to scale 1; unaligned and empty inputs
+    z = torch.zeros((64, 64), dtype=torch.bfloat16, device="cuda")
+    amax, scale, scale_inv = N.amax_scale(z, fmt)
+    assert amax.item() == 0.0 and scale.item() == 1.0 and scale_inv.item() == 1.0
+    z[3, 5] = float("nan")
+    amax, scale, _ = N.amax_scale(z, fmt)
+    assert torch.isnan(amax).item() and scale.item() == 1.0
+    flat = seeded_bf16((1, 5000), seed=6).cuda()
+    view = flat[0, 3:4003].reshape(1, 4000)
+    amax, scale, _ = N.amax_scale(view, fmt)
+    assert_f32_bits_equal(amax, O.t_amax(view.cpu()), "fused amax, unaligned")
+    amax, scale, _ = N.amax_scale(torch.empty((0, 16), dtype=torch.bfloat16, device="cuda"), fmt)
+    assert amax.item() == 0.0 and scale.item() == 1.0
+    # and the workspace really is zero again
+    assert all(int(w.abs().sum()) == 0 for w in N._workspaces.values())
+
+
+@pytest.mark.parametrize("fmt", [O.E4M3, O.E5M2])
 def test_scale_from_amax_bit_exact(N, fmt):
     rng = np.random.default_rng(0)
     a = np.concatenate([
