@@ -111,10 +111,14 @@ __global__ __launch_bounds__(kFatThreads) void amax_tensor_kernel(const void *__
     if constexpr (!FUSE) {
         if (threadIdx.x == 0 && m != 0) atomicMax(reinterpret_cast<uint32_t *>(out), m);
     } else if (threadIdx.x == 0) {
-        if (m != 0) atomicMax(fs.ws, m);
-        __threadfence();                                     // my maximum is visible before my ticket
-        if (atomicAdd(fs.ws + 1, 1u) == gridDim.x - 1) {     // every other block has drawn its ticket
-            __threadfence();
+        // Device-scope atomics are performed at the point of coherence, and one that returns a
+        // value has been performed when the value arrives.  The ticket is made to depend on the
+        // value returned by the max, so it is drawn after the max has landed: no fence (which would
+        // write back this XCD's whole L2) is needed to order the two.
+        uint32_t prev = atomicMax(fs.ws, m);
+        uint32_t one = 1u;
+        asm volatile("" : "+v"(one) : "v"(prev));
+        if (atomicAdd(fs.ws + 1, one) == gridDim.x - 1) {     // every other block has drawn its ticket
             const float amax = bits_to_float(atomicExch(fs.ws, 0u));
             atomicExch(fs.ws + 1, 0u);
             const float sc = scale_rule(amax, fs.fp8_max, fs.margin, 1.0f);

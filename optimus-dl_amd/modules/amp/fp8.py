@@ -189,6 +189,10 @@ class FP8Recipe:
         )
         self._store = _state.MetaStore(amax_history_len)
         self._depth = 0
+        # the last activation quantised under this recipe, so that Linears fed by the same tensor
+        # (gate/up, q/k/v) quantise it once; dropped when the outermost context is left
+        self.shared_input: dict[str, Any] | None = None
+        self.share_inputs = True
         self.scale_epoch = 0      # bumped whenever the forward scales are refreshed (invalidates cached weight codes)
         _info_once(
             f"Created FP8 recipe with format={self.format.value}, amax_history_len={amax_history_len}, "
@@ -256,6 +260,7 @@ class FP8Recipe:
             self._depth -= 1
             _state.pop_recipe()
             if self._depth == 0:
+                self.shared_input = None
                 self.update_scales("fwd")
                 # gradients recorded by a backward that ran outside any backward()
                 # context are folded in here, one step late but never lost

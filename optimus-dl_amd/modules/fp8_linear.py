@@ -74,6 +74,44 @@ def _quantise_dynamic(x2d: torch.Tensor, fmt: int, margin: int, need_t: bool, ne
     return q, q_t, scale_inv, amax
 
 
+def _input_key(x2d: torch.Tensor, kind: str, fmt: int, margin: int):
+    return (x2d.data_ptr(), x2d._version, tuple(x2d.shape), x2d.dtype, x2d.device, kind, fmt, margin)
+
+
+def _quantise_input_shared(recipe: FP8Recipe, x2d: torch.Tensor, fmt: int, margin: int, need_t: bool):
+    """Per-tensor quantisation of a Linear's input, reused by the next Linear that is fed the
+    very same tensor (gate and up of an MLP, q/k/v of an attention block).  The entry keeps
+    the tensor alive, so its address cannot be handed to another tensor while it is cached;
+    an in-place change bumps ``_version`` and misses."""
+    if not recipe.share_inputs:
+        return _quantise_dynamic(x2d, fmt, margin, need_t)[:3]
+    key = _input_key(x2d, "tensor", fmt, margin)
+    hit = recipe.shared_input
+    if hit is not None and hit["key"] == key and (hit["q_t"] is not None or not need_t):
+        return hit["q"], hit["q_t"], hit["s_inv"]
+    q, q_t, s_inv, _ = _quantise_dynamic(x2d, fmt, margin, need_t)
+    entry = {"key": key, "x": x2d, "q": q, "q_t": q_t, "s_inv": s_inv}
+    if hit is not None and hit.get("x") is x2d:          # keep the record of the conversion that produced x2d
+        entry["src_key"], entry["src"] = hit.get("src_key"), hit.get("src")
+    recipe.shared_input = entry
+    return q, q_t, s_inv
+
+
+def _converted_input(recipe: FP8Recipe, x2d: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """x2d in the compute dtype, contiguous.  Linears fed by the same tensor get the same
+    converted tensor back (one conversion, and one quantisation downstream); autograd sees an
+    ordinary tensor used twice."""
+    key = (x2d.data_ptr(), x2d._version, tuple(x2d.shape), tuple(x2d.stride()), x2d.dtype, x2d.device, dtype,
+           torch.is_grad_enabled() and x2d.requires_grad)
+    hit = recipe.shared_input
+    if recipe.share_inputs and hit is not None and hit.get("src_key") == key:
+        return hit["x"]
+    out = x2d.to(dtype).contiguous()
+    if recipe.share_inputs:
+        recipe.shared_input = {"src_key": key, "src": x2d, "x": out, "key": None, "q": None, "q_t": None, "s_inv": None}
+    return out
+
+
 def _quantise_delayed(x2d: torch.Tensor, fmt: int, meta: "_state.ScalingMeta", role: int, need_t: bool,
                       need_rowmajor: bool = True):
     """Delayed scaling: one pass with the scale from the history, amax recorded in row 0."""
@@ -120,7 +158,7 @@ class _Fp8LinearFn(torch.autograd.Function):
                 meta = module._meta(recipe, x2d.device, "fwd")
                 xq, xq_t, sx_inv = _quantise_delayed(x2d, pol.fmt_fwd, meta, ROLE_X, need_wgrad and recipe.wgrad)
             else:
-                xq, xq_t, sx_inv, _ = _quantise_dynamic(x2d, pol.fmt_fwd, pol.margin, need_wgrad and recipe.wgrad)
+                xq, xq_t, sx_inv = _quantise_input_shared(recipe, x2d, pol.fmt_fwd, pol.margin, need_wgrad and recipe.wgrad)
             wq, wq_t, sw_inv = module._tensor_weight(weight, recipe, need_t=need_dgrad)
             y = native.gemm_nt(xq, wq, pol.fmt_fwd, pol.fmt_fwd, sx_inv, sw_inv, bias=bias_f32, out_dtype=out_dtype)
             if need_wgrad and recipe.wgrad:
@@ -290,10 +328,8 @@ class FP8Linear(nn.Linear):
         if compute_dtype not in (torch.bfloat16, torch.float32):
             compute_dtype = torch.bfloat16
         x2d = x.reshape(-1, self.in_features)
-        if x2d.dtype != compute_dtype:
-            x2d = x2d.to(compute_dtype)
-        if not x2d.is_contiguous():
-            x2d = x2d.contiguous()
+        if x2d.dtype != compute_dtype or not x2d.is_contiguous():
+            x2d = _converted_input(recipe, x2d, compute_dtype)
         self.fp8_calls += 1
         y = _Fp8LinearFn.apply(x2d, self.weight, self.bias, self, recipe, compute_dtype)
         return y.reshape(*x.shape[:-1], self.out_features)

@@ -280,3 +280,75 @@ def test_training_loop_through_the_reference_shaped_glue(amp, family):
             assert n_fp8 > 0, "no Linear took the FP8 path"
     assert losses["fp8"][-1] < losses["fp8"][0] - 0.5, losses
     assert abs(losses["fp8"][-1] - losses["bf16"][-1]) < 0.25, losses
+
+
+def _count_calls(monkeypatch, native, name):
+    calls = []
+    orig = getattr(native, name)
+
+    def counted(*a, **kw):
+        calls.append(a[0].shape)
+        return orig(*a, **kw)
+
+    monkeypatch.setattr(native, name, counted)
+    return calls
+
+
+@pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float32])
+def test_linears_fed_by_the_same_tensor_quantise_it_once(amp, monkeypatch, in_dtype):
+    """gate/up of an MLP (q/k/v of an attention block): same input tensor, one amax and one cast of it.
+    Results are bit-identical to quantising it per Linear."""
+    from optimus_dl_amd import native
+
+    M, K, N = 256, 512, 384
+    x = seeded_bf16((M, K), 1.0, 40)
+    wg, wu = seeded_bf16((N, K), 0.02, 41), seeded_bf16((N, K), 0.02, 42)
+    dy = seeded_bf16((M, N), 1e-3, 43).cuda()
+
+    def run(share):
+        recipe = amp.create_fp8_recipe("tensorwise", "hybrid")
+        recipe.share_inputs = share
+        gate, up = make_linear(wg), make_linear(wu)
+        xd = x.to(in_dtype).cuda().requires_grad_(True)
+        with amp.fp8_autocast(torch.device("cuda"), recipe, dtype=torch.bfloat16):
+            h = gate(xd) * up(xd)
+        with recipe.backward():
+            h.backward(dy)
+        assert recipe.shared_input is None                      # dropped when the context was left
+        return h.detach(), xd.grad.detach(), gate.weight.grad.detach(), up.weight.grad.detach()
+
+    calls = _count_calls(monkeypatch, native, "amax_scale")
+    shared = run(True)
+    n_shared = len([s for s in calls if tuple(s) == (M, K)])
+    calls.clear()
+    separate = run(False)
+    n_separate = len([s for s in calls if tuple(s) == (M, K)])
+    assert (n_shared, n_separate) == (1, 2)
+    for i, (a, b) in enumerate(zip(shared, separate)):
+        if i == 1 and in_dtype == torch.float32:
+            # the two input gradients meet in bf16 (behind the shared conversion) instead of in fp32
+            assert max_rel_err(a, b) <= 1e-2
+        else:
+            assert torch.equal(a, b)
+
+
+def test_shared_input_is_not_reused_after_an_in_place_change_or_for_another_tensor(amp, monkeypatch):
+    from optimus_dl_amd import native
+
+    M, K, N = 128, 256, 128
+    recipe = amp.create_fp8_recipe("tensorwise", "hybrid")
+    lin = make_linear(seeded_bf16((N, K), 0.02, 50))
+    x = seeded_bf16((M, K), 1.0, 51).cuda()
+    calls = _count_calls(monkeypatch, native, "amax_scale")
+    with torch.no_grad(), recipe.autocast():
+        y1 = lin(x)
+        y1_again = lin(x)                                       # hit
+        n_after_hit = len(calls)
+        x.mul_(2.0)                                             # same address, new contents
+        y2 = lin(x)
+        other = x.clone()
+        y3 = lin(other)
+    assert n_after_hit == 2                                     # weight + x, once each
+    assert len(calls) == 4                                      # + x after the change + the clone
+    assert torch.equal(y1, y1_again) and torch.equal(y2, y3)
+    assert not torch.equal(y1, y2)
