@@ -56,7 +56,7 @@ constexpr int LOADS = 256 / 8 / NW;        // 1 KB direct-to-LDS loads per wave 
 constexpr int GM = 8;
 constexpr int PF = ODL_STREAM_PF;          // L2 prefetch distance in K steps, 0 = none
 constexpr int NPF = PF > 0 ? 2 : 0;        // prefetch loads per wave per step
-constexpr int PITCH = 128 + 16;            // slab row: 64 bf16 + pad
+constexpr int PITCH = 128 + 8;             // slab row: 64 bf16 + 8 bytes, see phase_a_fold
 constexpr int SLAB = 32 * PITCH;           // one wave's epilogue slab
 
 template <int FA, int FB>
@@ -178,7 +178,11 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
         }
     };
     auto lds_w = [](uint32_t addr) { return (__attribute__((address_space(3))) u32x2 *)addr; };
-    auto lds_r = [](uint32_t addr) { return (const __attribute__((address_space(3))) u32x4 *)addr; };
+    auto lds_r = [](uint32_t addr) -> u32x4 {   // 16 bytes as two 8-byte reads: slab rows are only 8-byte aligned
+        const u32x2 lo = *(const __attribute__((address_space(3))) u32x2 *)addr;
+        const u32x2 hi = *(const __attribute__((address_space(3))) u32x2 *)(addr + 8);
+        return u32x4{lo.x, lo.y, hi.x, hi.y};
+    };
 
     // phase A of a step: MFMA i works on sub-tile (t, u) = (i / 4, i % 4); the 8 fragments of
     // (kt, h1) stream into buffer 1 behind the first 8 MFMAs.
@@ -223,14 +227,16 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
                 pk[2 * q + 1] = pack_bf16x2(acc[t][u][4 * q + 2] * s_tensor, acc[t][u][4 * q + 3] * s_tensor);
             }
             acc[t][u] = mfma_32x32x64<FB, FA>(b0[u], a0[t], zero16);
-            // lane (lr, lg) holds columns 8q + 4lg + {0..3} of row lr of the sub-tile
+            // lane (lr, lg) holds columns 8q + 4lg + {0..3} of row lr of the sub-tile.  With a row
+            // pitch of 34 dwords the 8-byte writes of 16 consecutive rows cover all 32 banks once,
+            // and so do the 8-byte halves of the row-wise reads of two consecutive rows.
 #pragma unroll
             for (int q = 0; q < 4; ++q) *lds_w(epi_w + (u & 1) * 64 + q * 16) = u32x2{pk[2 * q], pk[2 * q + 1]};
             if (u & 1) {
                 // slab complete: 8 lanes cover a row with 16 bytes each, 8 rows per instruction.
                 // LDS operations of a wave execute in order, so the next writes cannot overtake these reads.
 #pragma unroll
-                for (int j = 0; j < 4; ++j) back[j] = *lds_r(epi_r + j * 8 * PITCH);
+                for (int j = 0; j < 4; ++j) back[j] = lds_r(epi_r + j * 8 * PITCH);
             } else if (i > 0) {
                 store_slab(back, c_voff, rsrc_c, c_soff0, n2, (i - 2) / 4, (i - 2) % 4);   // completed one MFMA ago
             }
