@@ -1,0 +1,145 @@
+"""GPU parity at the full BASELINE sizes, through properties that do not need the
+whole answer on the CPU:
+
+  * a random sample of output rows x columns against the oracle's emulated matmul
+    (the sample's operands are copied to the CPU; tolerance 1e-2 as for every GEMM);
+  * every kernel variant that takes the shape produces the same bits (the accumulation
+    order over K is the same in all of them), and C(a, b)^T == C(b, a) bit for bit;
+  * doubling a scale doubles every output exactly (power of two);
+  * casts: the transposed copy is the transpose of the row-major copy, a sample of rows
+    matches the oracle bit for bit, amax equals the maximum of block maxima.
+
+Inputs are drawn on the GPU (seeded) and are what BASELINE describes: N(0,1) activations,
+N(0,0.02) weights, N(0,1e-3) gradients.
+"""
+import pytest
+import torch
+
+from oracle import oracle as O
+from tests.helpers import assert_bytes_equal, assert_f32_bits_equal, max_rel_err
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+
+
+@pytest.fixture(scope="module")
+def N():
+    from optimus_dl_amd import native
+
+    native.load()
+    yield native
+    native.gemm_set_variant(-1)
+
+
+def draw(shape, std, seed):
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    return (torch.randn(shape, generator=g, device="cuda", dtype=torch.float32) * std).bfloat16()
+
+
+def quantise(N, x, fmt):
+    amax, scale, scale_inv = N.amax_scale(x, fmt)
+    q, q_t = N.cast_transpose(x, scale, fmt)
+    return q, q_t, scale, scale_inv, amax
+
+
+def sample_check(out, aq, bq, fa, fb, sa_inv, sb_inv, seed, what, rows=48, cols=640):
+    """out[M,N] (GPU) against the oracle on a random rows x cols sample."""
+    M, Nn = out.shape
+    g = torch.Generator().manual_seed(seed)
+    ri = torch.randperm(M, generator=g)[:rows].sort().values
+    ci = torch.randperm(Nn, generator=g)[:cols].sort().values
+    a_s, b_s = aq[ri.cuda()].cpu(), bq[ci.cuda()].cpu()
+    sa = sa_inv.cpu() if sa_inv.numel() == 1 else sa_inv[ri.cuda()].cpu()
+    sb = sb_inv.cpu() if sb_inv.numel() == 1 else sb_inv[ci.cuda()].cpu()
+    ref = O.t_gemm_nt(a_s, b_s, fa, fb, sa, sb)
+    got = out[ri.cuda()][:, ci.cuda()]
+    err = max_rel_err(got, ref)
+    assert err <= TOL, f"{what}: max rel err {err} on a {rows}x{cols} sample"
+
+
+# (M, N, K) of the GEMMs that BASELINE's configurations launch
+CFG_SHAPES = [
+    pytest.param(8192, 14336, 4096, id="cfg3-fwd-gate"),
+    pytest.param(8192, 4096, 14336, id="cfg3-fwd-down"),
+    pytest.param(14336, 4096, 8192, id="cfg3-wgrad-gate"),
+    pytest.param(8192, 1024, 4096, id="cfg2-fwd-wk"),
+    pytest.param(8192, 28672, 8192, id="cfg5-fwd-up"),
+    pytest.param(8192, 8192, 28672, id="cfg5-fwd-down"),
+]
+
+
+@pytest.mark.parametrize("M,Nn,K", CFG_SHAPES)
+def test_gemm_at_baseline_shapes(N, M, Nn, K):
+    a = draw((M, K), 1e-3, 1)            # plays dY (E5M2) against a weight-like operand (E4M3)
+    b = draw((Nn, K), 0.02, 2)
+    aq, _, _, sa_inv, _ = quantise(N, a, O.E5M2)
+    bq, _, _, sb_inv, _ = quantise(N, b, O.E4M3)
+    del a, b
+    N.gemm_set_variant(-1)
+    out = N.gemm_nt(aq, bq, O.E5M2, O.E4M3, sa_inv, sb_inv)
+    sample_check(out, aq, bq, O.E5M2, O.E4M3, sa_inv, sb_inv, seed=M + Nn, what=f"auto {M}x{Nn}x{K}")
+    # the same bits from every variant that keeps the K order (all tiled kernels do)
+    names = N.gemm_variants()
+    for v in range(2, len(names)):
+        if "one tile per block" in names[v]:
+            continue
+        N.gemm_set_variant(v)
+        other = N.gemm_nt(aq, bq, O.E5M2, O.E4M3, sa_inv, sb_inv)
+        assert torch.equal(out, other), f"variant {v} ({names[v]}) differs from the automatic choice"
+    N.gemm_set_variant(-1)
+    # operands swapped: the transpose, bit for bit
+    swapped = N.gemm_nt(bq, aq, O.E4M3, O.E5M2, sb_inv, sa_inv)
+    assert torch.equal(swapped.t(), out)
+    # a scale doubled: every output doubled (exact in bf16 away from overflow)
+    doubled = N.gemm_nt(aq, bq, O.E5M2, O.E4M3, sa_inv * 2, sb_inv)
+    assert torch.equal(doubled.float(), out.float() * 2)
+
+
+def test_rowwise_gemm_at_config_4_shape_with_outlier_channels(N):
+    M, Nn, K = 16384, 14336, 4096
+    x = draw((M, K), 1.0, 3)
+    g = torch.Generator().manual_seed(4)
+    channels = torch.randperm(K, generator=g)[:4]
+    x[:, channels.cuda()] *= 100.0
+    w = draw((Nn, K), 0.02, 5)
+    ax, aw = N.amax(x, O.SCALE_ROW), N.amax(w, O.SCALE_ROW)
+    # per-row amax: torch on the GPU as an independent check of the reduction at this size
+    assert torch.equal(ax, x.float().abs().amax(dim=1)) and torch.equal(aw, w.float().abs().amax(dim=1))
+    sx, sx_inv = N.scale_from_amax(ax, O.E4M3)
+    sw, sw_inv = N.scale_from_amax(aw, O.E4M3)
+    xq, wq = N.cast(x, sx, O.E4M3, O.SCALE_ROW), N.cast(w, sw, O.E4M3, O.SCALE_ROW)
+    rows = torch.tensor([0, 1, 4095, 8191, 16383])
+    assert_bytes_equal(xq[rows.cuda()], O.t_cast(x[rows.cuda()].cpu(), sx[rows.cuda()].cpu(), O.E4M3, O.SCALE_ROW), "rowwise codes")
+    out = N.gemm_nt(xq, wq, O.E4M3, O.E4M3, sx_inv, sw_inv)
+    sample_check(out, xq, wq, O.E4M3, O.E4M3, sx_inv, sw_inv, seed=7, what="config 4 forward")
+    # row isolation: scaling one row of X by 2^3 changes only that row's scale, no code, and only that output row
+    x2 = x.clone()
+    x2[123] *= 8.0
+    ax2 = N.amax(x2, O.SCALE_ROW)
+    sx2, sx2_inv = N.scale_from_amax(ax2, O.E4M3)
+    xq2 = N.cast(x2, sx2, O.E4M3, O.SCALE_ROW)
+    assert torch.equal(xq2, xq)
+    assert sx2[123].item() == sx[123].item() / 8 and torch.equal(sx2[:123], sx[:123]) and torch.equal(sx2[124:], sx[124:])
+
+
+@pytest.mark.parametrize("shape,std,fmt", [((8192, 4096), 1.0, O.E4M3), ((14336, 4096), 0.02, O.E4M3),
+                                           ((8192, 14336), 1e-3, O.E5M2), ((8192, 28672), 1e-3, O.E5M2)])
+def test_quantisation_at_baseline_shapes(N, shape, std, fmt):
+    x = draw(shape, std, 11)
+    q, q_t, scale, scale_inv, amax = quantise(N, x, fmt)
+    # amax: the maximum of block maxima (order does not matter for a max), and torch's own reduction
+    blocks = torch.stack([N.amax(x[i:i + 1024]) for i in range(0, shape[0], 1024)])
+    assert_f32_bits_equal(amax, blocks.max().reshape(1), "amax = max of block amaxes")
+    assert_f32_bits_equal(amax, x.float().abs().max().reshape(1), "amax vs torch")
+    want_scale = torch.tensor([O.c_scale(float(amax), fmt, 0, 1.0)])
+    assert_f32_bits_equal(scale, want_scale, "scale")
+    assert_f32_bits_equal(scale_inv, torch.tensor([O.c_scale_inv(float(want_scale))]), "1/scale")
+    # transposed copy == transpose of the row-major copy; cast alone gives the same codes
+    assert torch.equal(q_t, q.t().contiguous())
+    assert torch.equal(N.cast(x, scale, fmt), q)
+    # a sample of rows against the oracle, bit for bit
+    rows = torch.tensor([0, 7, 1023, shape[0] // 2, shape[0] - 1])
+    assert_bytes_equal(q[rows.cuda()], O.t_cast(x[rows.cuda()].cpu(), scale.cpu(), fmt), "codes of sampled rows")
+    # idempotence: decoding (fp32) and re-quantising with the same scale gives the same codes
+    again = N.cast((O.t_decode(q[rows.cuda()].cpu(), fmt) / scale.cpu()).cuda(), scale, fmt)
+    assert_bytes_equal(again, q[rows.cuda()], "requantised codes")
