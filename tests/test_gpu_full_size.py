@@ -143,3 +143,58 @@ def test_quantisation_at_baseline_shapes(N, shape, std, fmt):
     # idempotence: decoding (fp32) and re-quantising with the same scale gives the same codes
     again = N.cast((O.t_decode(q[rows.cuda()].cpu(), fmt) / scale.cpu()).cuda(), scale, fmt)
     assert_bytes_equal(again, q[rows.cuda()], "requantised codes")
+
+
+def test_delayed_scaling_config_5_twenty_steps_at_full_size(N):
+    """Llama-3-70B MLP shapes, history 16, 20 steps, input std 1.0 -> 1.5: after every step the
+    histories and scales on the GPU equal the oracle's ring-buffer simulation fed with the amaxes
+    of that step's tensors (torch reductions on the GPU supply them), bit for bit; the outputs of
+    two steps are checked on a sample against the oracle's matmul with the STALE scales."""
+    from optimus_dl_amd.modules import amp
+    from optimus_dl_amd.modules.fp8_linear import FP8Linear
+
+    M, K, F, H, STEPS = 8192, 8192, 28672, 16, 20
+    recipe = amp.create_fp8_recipe("delayed", "hybrid", amax_history_len=H)
+    up = FP8Linear(K, F, bias=False, device="cuda", dtype=torch.bfloat16)
+    down = FP8Linear(F, K, bias=False, device="cuda", dtype=torch.bfloat16)
+    with torch.no_grad():
+        up.weight.copy_(draw((F, K), 0.01, 21))
+        down.weight.copy_(draw((K, F), 0.01, 22))
+    sim = {("up", "fwd"): O.DelayedState([O.E4M3] * 3, H), ("up", "bwd"): O.DelayedState([O.E5M2] * 2, H),
+           ("down", "fwd"): O.DelayedState([O.E4M3] * 3, H), ("down", "bwd"): O.DelayedState([O.E5M2] * 2, H)}
+    amax = lambda t: t.detach().float().abs().max().item()
+    for step in range(STEPS):
+        std = 1.0 + 0.5 * step / (STEPS - 1)
+        x = draw((M, K), std, 100 + step).requires_grad_(True)
+        dy = draw((M, K), 1e-3, 200 + step)
+        stale_x, stale_w = sim[("up", "fwd")].scale[0], sim[("up", "fwd")].scale[1]
+        with recipe.autocast():
+            h = up(x)
+            y = down(h)
+        h.retain_grad()
+        with recipe.backward():
+            y.backward(dy)
+        sim[("up", "fwd")].record(0, amax(x)); sim[("up", "fwd")].record(1, amax(up.weight))
+        sim[("down", "fwd")].record(0, amax(h)); sim[("down", "fwd")].record(1, amax(down.weight))
+        sim[("down", "bwd")].record(0, amax(dy)); sim[("up", "bwd")].record(0, amax(h.grad))
+        for s in sim.values():
+            s.update()
+        for name, lin in (("up", up), ("down", down)):
+            for direction, key in (("fwd", "scaling_fwd"), ("bwd", "scaling_bwd")):
+                meta, want = lin.fp8_meta[key], sim[(name, direction)]
+                assert_f32_bits_equal(meta.amax_history, torch.from_numpy(want.history), f"{name} {direction} history, step {step}")
+                assert_f32_bits_equal(meta.scale, torch.from_numpy(want.scale), f"{name} {direction} scale, step {step}")
+                assert_f32_bits_equal(meta.scale_inv, torch.from_numpy(want.scale_inv), f"{name} {direction} 1/scale, step {step}")
+        if step in (1, STEPS - 1):
+            # h = Q(x; stale scale) . Q(W_up; stale scale)^T on a sample
+            sx, sw = torch.tensor([stale_x]), torch.tensor([stale_w])
+            g = torch.Generator().manual_seed(step)
+            ri, ci = torch.randperm(M, generator=g)[:32].sort().values, torch.randperm(F, generator=g)[:512].sort().values
+            xq = O.t_cast(x.detach()[ri.cuda()].cpu(), sx, O.E4M3)
+            wq = O.t_cast(up.weight.detach()[ci.cuda()].cpu(), sw, O.E4M3)
+            ref = O.t_gemm_nt(xq, wq, O.E4M3, O.E4M3, 1.0 / sx, 1.0 / sw)
+            err = max_rel_err(h.detach()[ri.cuda()][:, ci.cuda()], ref)
+            assert err <= TOL, f"step {step}: h vs oracle with stale scales: {err}"
+    # after 20 steps the 16-deep window has forgotten steps 0..3: the input scale is set by the last 16 amaxes only
+    hist = up.fp8_meta["scaling_fwd"].amax_history[:, 0]
+    assert int((hist > 0).sum()) == H - 1 and hist[0].item() == 0.0
