@@ -13,6 +13,10 @@
 
 namespace odl {
 
+// Row-major FP8 codes are stored with ordinary (cache-allocating) stores: the GEMM that reads them
+// is the next kernel and finds them in the memory-side cache (measured: -3 % GEMM time inside a step).
+// Transposed codes are read much later (wgrad): they are stored non-temporally.
+#define ODL_CODE_STORE(val, ptr) (*(ptr) = (val))
 constexpr int kThreads = 256;
 // Kernels that end in one atomicMax per block use fat blocks and a small grid:
 // same-address atomics from different XCDs retire one at a time (~8 ns each).
@@ -383,7 +387,7 @@ __global__ __launch_bounds__(AMAX ? kFatThreads : kThreads) void cast_kernel(con
         o.y = quantise4<FMT>(f[4], f[5], f[6], f[7], s[4], s[5], s[6], s[7]);
         o.z = quantise4<FMT>(f[8], f[9], f[10], f[11], s[8], s[9], s[10], s[11]);
         o.w = quantise4<FMT>(f[12], f[13], f[14], f[15], s[12], s[13], s[14], s[15]);
-        __builtin_nontemporal_store(o, reinterpret_cast<u32x4 *>(out) + i);
+        ODL_CODE_STORE(o, reinterpret_cast<u32x4 *>(out) + i);
     }
     if constexpr (AMAX) {
         if constexpr (SRC == ODL_BF16) am = fold_u16x2_to_f32bits(am);
@@ -518,7 +522,7 @@ __global__ __launch_bounds__(kThreads) void cast_transpose_kernel(const void *__
         hi[i] = quantise4<FMT>(f[4], f[5], f[6], f[7], s[4], s[5], s[6], s[7]);
         if constexpr (WRITE_ROWMAJOR) {
             if (col_ok && (r0 + i) < rows)
-                __builtin_nontemporal_store(u32x2{lo[i], hi[i]}, reinterpret_cast<u32x2 *>(out + (r0 + i) * cols + c0));
+                ODL_CODE_STORE((u32x2{lo[i], hi[i]}), reinterpret_cast<u32x2 *>(out + (r0 + i) * cols + c0));
         }
     }
 
