@@ -26,7 +26,8 @@ TORCH_FP8 = {E4M3: torch.float8_e4m3fn, E5M2: torch.float8_e5m2}
 ABI_VERSION = 1
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libodl_fp8.so")
+# ODL_FP8_LIB names another build of the same library (e.g. one made for an experiment)
+LIB_PATH = os.environ.get("ODL_FP8_LIB") or os.path.join(_HERE, "libodl_fp8.so")
 
 EXPORTS = (
     "odl_fp8_abi_version",
