@@ -74,6 +74,10 @@ class KernelTimer:
         wrap("gemm_nt", lambda a, b, *r, **kw: 2.0 * a.shape[0] * b.shape[0] * a.shape[1])            # flops
         wrap("amax", lambda x, *r, **kw: float(x.numel() * esz(x)))                                       # bytes
         wrap("amax_scale", lambda x, *r, **kw: float(x.numel() * esz(x)), record_as="amax")       # amax + scale, one launch
+        wrap("amax_parts", lambda x, *r, **kw: float(x.numel() * esz(x)), record_as="amax")
+        wrap("cast_dynamic", lambda x, parts, fmt, margin=0, want_rowmajor=True, want_transposed=True:
+             float(x.numel() * (esz(x) + int(want_rowmajor) + int(want_transposed))),
+             record_as="cast_transpose")
         wrap("cast", lambda x, *r, **kw: float(x.numel() * (esz(x) + 1)))
         wrap("cast_transpose",
              lambda x, *r, **kw: float(x.numel() * (esz(x) + (2 if kw.get("want_rowmajor", True) else 1))))
@@ -97,6 +101,39 @@ def make_inputs(torch, m=M_TOKENS, device="cuda"):
             "dy": (torch.randn(m, n, generator=g) * 1e-3).bfloat16().to(device),
         }
     return data
+
+
+def standalone_hbm(torch, native, iters=24):
+    """The memory-bound kernels on their own, on inputs that are not cache-resident: enough
+    buffers per shape are walked round-robin to hold three times the 256 MB memory-side cache;
+    HIP events around the whole batch, so launch gaps are included.  Algorithmic bytes as in the step."""
+    out = {}
+    for rows, cols in ((M_TOKENS, 4096), (14336, 4096), (M_TOKENS, 14336)):
+        nbuf = max(4, -(-3 * 256 * 2**20 // (2 * rows * cols)))
+        xs = [torch.randn((rows, cols), device="cuda", dtype=torch.bfloat16) for _ in range(nbuf)]
+        _, scale, _ = native.amax_scale(xs[0], native.E4M3, 0)
+        E = rows * cols
+        kernels = {
+            "amax": (lambda x: native.amax_parts(x), 2 * E),
+            "amax_rowwise": (lambda x: native.amax(x, native.SCALE_ROW), 2 * E + 4 * rows),
+            "cast": (lambda x: native.cast(x, scale, native.E4M3, native.SCALE_TENSOR), 3 * E),
+            "cast_transpose": (lambda x: native.cast_transpose(x, scale, native.E4M3, native.SCALE_TENSOR), 4 * E),
+            "amax_then_cast_transpose": (lambda x: native.quantize_dynamic(x, native.E4M3, 0), 6 * E),
+        }
+        for name, (fn, nbytes) in kernels.items():
+            for x in xs:
+                fn(x)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for i in range(iters):
+                fn(xs[i % nbuf])
+            e1.record()
+            torch.cuda.synchronize()
+            us = 1e3 * e0.elapsed_time(e1) / iters
+            gbps = nbytes / (us * 1e-6) / 1e9
+            out.setdefault(name, {})[f"{rows}x{cols}"] = {"us": round(us, 1), "GB/s": round(gbps), "frac": round(gbps / PEAK_HBM_GBPS, 3)}
+        del xs
+    return out
 
 
 def cpu_baseline(torch, seconds_hint=20.0):
@@ -247,6 +284,7 @@ def main() -> int:
             "launches": gemm["launches"],
         },
         "hbm_kernels": hbm,
+        "hbm_kernels_standalone": standalone_hbm(torch, native),
     }
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(torch)

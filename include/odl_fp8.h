@@ -86,6 +86,24 @@ int odl_fp8_amax_scale(const void *x, int src_dtype, int64_t rows, int64_t cols,
                        odl_stream_t stream);
 
 /*
+ * Current scaling ("tensorwise", fp8.py:289-294) of one tensor in two launches and no other:
+ *   odl_fp8_amax_parts  : ODL_FP8_AMAX_PARTS partial maxima of |x| (unused entries 0),
+ *                         written without atomics;
+ *   odl_fp8_cast_dynamic: every block reduces the partials, derives
+ *                         scale = fp8_max(fmt) / amax / 2^margin (rules of odl_fp8_scale_from_amax)
+ *                         and casts; out (row-major codes) and out_t (transposed codes) may
+ *                         each be NULL, not both; dyn_out[3] receives {amax, scale, 1/scale}.
+ * The codes and the three numbers equal those of odl_fp8_amax + odl_fp8_scale_from_amax +
+ * odl_fp8_cast / odl_fp8_cast_transpose, bit for bit.
+ */
+#define ODL_FP8_AMAX_PARTS 512
+int odl_fp8_amax_parts(const void *x, int src_dtype, int64_t rows, int64_t cols, float *parts,
+                       odl_stream_t stream);
+int odl_fp8_cast_dynamic(const void *x, int src_dtype, int64_t rows, int64_t cols, const float *parts,
+                         int fmt, int margin, uint8_t *out, uint8_t *out_t, float *dyn_out,
+                         odl_stream_t stream);
+
+/*
  * out[r,c] = fp8( clamp( fp32(x[r,c]) * s , +-max ) ), s = scale[0] | scale[r] | scale[c].
  * amax_out (may be NULL): *amax_out = max(*amax_out, max|x|), for delayed scaling,
  * where the cast uses an older scale while this step's amax is recorded.

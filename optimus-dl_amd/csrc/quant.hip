@@ -58,7 +58,11 @@ struct FusedScale {
 // cache if this pass left it there.  With non-temporal loads this pass is a little
 // faster but the cast runs at HBM speed (measured: 159 -> 124 us for the pair on a
 // 235 MB tensor).
-template <int SRC, int UNROLL, bool FUSE>
+// OUT: 0 = atomicMax into out[0]; 1 = fused scale (see FusedScale); 2 = out[blockIdx] = this block's
+// maximum, no atomics at all: the cast that follows reduces the kAmaxParts partials itself.
+constexpr int kAmaxParts = ODL_FP8_AMAX_PARTS;
+
+template <int SRC, int UNROLL, int OUT>
 __global__ __launch_bounds__(kFatThreads) void amax_tensor_kernel(const void *__restrict__ x, int64_t n,
                                                                    float *__restrict__ out, const FusedScale fs) {
     __shared__ uint32_t red[kFatThreads / kWave];
@@ -117,7 +121,11 @@ __global__ __launch_bounds__(kFatThreads) void amax_tensor_kernel(const void *__
         }
     }
     m = block_max_u32(m, red);
-    if constexpr (!FUSE) {
+    if constexpr (OUT == 2) {
+        if (threadIdx.x == 0) out[blockIdx.x] = bits_to_float(m);
+        if (blockIdx.x == 0)                                  // entries no block owns
+            for (int i = (int)gridDim.x + threadIdx.x; i < kAmaxParts; i += kFatThreads) out[i] = 0.0f;
+    } else if constexpr (OUT == 0) {
         if (threadIdx.x == 0 && m != 0) atomicMax(reinterpret_cast<uint32_t *>(out), m);
     } else if (threadIdx.x == 0) {
         // Device-scope atomics are performed at the point of coherence, and one that returns a
@@ -329,13 +337,47 @@ __global__ void delayed_update_kernel(float *__restrict__ history, int64_t H, in
     scale_inv[r] = __fdiv_rn(1.0f, s);
 }
 
+// ------------------------------------------------- current scaling inside the cast
+// MODE == kScaleParts: `scale` points at kAmaxParts partial maxima (amax_tensor_kernel<.., 2>).
+// Every block reduces them (2 KB from L2), derives the per-tensor scale, and block 0 records
+// {amax, scale, 1/scale} in dyn_out for the GEMM: no kernel between the amax pass and the cast.
+constexpr int kScaleParts = 3;
+
+template <int FMT>
+__device__ __forceinline__ float dynamic_scale(const float *__restrict__ parts, int margin, float *__restrict__ dyn_out,
+                                               uint32_t *red) {
+    __shared__ float s_bcast;
+    uint32_t m = 0;
+    for (int i = threadIdx.x; i < kAmaxParts; i += blockDim.x) m = max(m, float_to_bits(parts[i]));
+    m = block_max_u32(m, red);
+    if (threadIdx.x == 0) {
+        const float amax = bits_to_float(m);
+        const float sc = scale_rule(amax, Fp8Lim<FMT>::max, margin, 1.0f);
+        s_bcast = sc;
+        if (blockIdx.x == 0 && dyn_out) {
+            dyn_out[0] = amax;
+            dyn_out[1] = sc;
+            dyn_out[2] = __fdiv_rn(1.0f, sc);
+        }
+    }
+    __syncthreads();
+    return s_bcast;
+}
+
+// one block: the same reduction for the element-at-a-time route
+template <int FMT>
+__global__ __launch_bounds__(kThreads) void parts_to_scale_kernel(const float *__restrict__ parts, int margin, float *__restrict__ dyn_out) {
+    __shared__ uint32_t red[kThreads / kWave];
+    dynamic_scale<FMT>(parts, margin, dyn_out, red);
+}
+
 // ------------------------------------------------------------------------ cast
 // 16 elements per lane per step: two (bf16) or four (fp32) 16-byte loads, one
 // 16-byte store.  cols % 16 == 0 and 16-byte aligned pointers (host-checked).
 template <int SRC, int FMT, int MODE, bool AMAX>
 __global__ __launch_bounds__(AMAX ? kFatThreads : kThreads) void cast_kernel(const void *__restrict__ x, int64_t rows, int64_t cols,
                                                          const float *__restrict__ scale, uint8_t *__restrict__ out,
-                                                         float *__restrict__ amax_out) {
+                                                         float *__restrict__ amax_out, int margin, float *__restrict__ dyn_out) {
     constexpr int kT = AMAX ? kFatThreads : kThreads;
     __shared__ uint32_t red[kT / kWave];
     const int64_t cpr = cols / 16;                           // chunks per row
@@ -343,6 +385,7 @@ __global__ __launch_bounds__(AMAX ? kFatThreads : kThreads) void cast_kernel(con
     const int64_t stride = (int64_t)gridDim.x * kT;
     float s_t = 1.0f;
     if constexpr (MODE == ODL_SCALE_TENSOR) s_t = scale[0];
+    if constexpr (MODE == kScaleParts) s_t = dynamic_scale<FMT>(scale, margin, dyn_out, red);
     uint32_t am = 0;
     for (int64_t i = (int64_t)blockIdx.x * kT + threadIdx.x; i < nchunk; i += stride) {
         float f[16];
@@ -370,7 +413,7 @@ __global__ __launch_bounds__(AMAX ? kFatThreads : kThreads) void cast_kernel(con
             }
         }
         float s[16];
-        if constexpr (MODE == ODL_SCALE_TENSOR) {
+        if constexpr (MODE == ODL_SCALE_TENSOR || MODE == kScaleParts) {
 #pragma unroll
             for (int j = 0; j < 16; ++j) s[j] = s_t;
         } else if constexpr (MODE == ODL_SCALE_ROW) {
@@ -448,9 +491,11 @@ template <int SRC, int FMT, int MODE, bool AMAX, bool WRITE_ROWMAJOR>
 __global__ __launch_bounds__(kThreads) void cast_transpose_kernel(const void *__restrict__ x, int64_t rows, int64_t cols,
                                                                    const float *__restrict__ scale,
                                                                    uint8_t *__restrict__ out, uint8_t *__restrict__ out_t,
-                                                                   float *__restrict__ amax_out) {
+                                                                   float *__restrict__ amax_out, int margin, float *__restrict__ dyn_out) {
     __shared__ __attribute__((aligned(16))) uint8_t tile[kTileC * kLdsPitch];
     __shared__ uint32_t red[kThreads / kWave];
+    float s_dyn = 1.0f;
+    if constexpr (MODE == kScaleParts) s_dyn = dynamic_scale<FMT>(scale, margin, dyn_out, red);
     constexpr int ESZ = SRC == ODL_BF16 ? 2 : 4;
     const int tx = threadIdx.x % 8;                 // 8 lanes across 64 columns
     const int ty = threadIdx.x / 8;                 // 32 lane-rows, 4 rows each
@@ -467,8 +512,8 @@ __global__ __launch_bounds__(kThreads) void cast_transpose_kernel(const void *__
     float s_col[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) s_col[j] = 1.0f;
-    if constexpr (MODE == ODL_SCALE_TENSOR) {
-        const float st = scale[0];
+    if constexpr (MODE == ODL_SCALE_TENSOR || MODE == kScaleParts) {
+        const float st = MODE == kScaleParts ? s_dyn : scale[0];
 #pragma unroll
         for (int j = 0; j < 8; ++j) s_col[j] = st;
     } else if constexpr (MODE == ODL_SCALE_COL) {
@@ -598,8 +643,8 @@ extern "C" int odl_fp8_amax(const void *x, int src_dtype, int64_t rows, int64_t 
     if (mode == ODL_SCALE_TENSOR) {
         if (aligned16(x)) {
             const int64_t g = grid_for(n * esz / 16, kFatThreads * 4, 2);
-            if (src_dtype == ODL_BF16) hipLaunchKernelGGL((amax_tensor_kernel<ODL_BF16, 4, false>), dim3((unsigned)g), dim3(kFatThreads), 0, stream, x, n, amax_out, FusedScale{});
-            else hipLaunchKernelGGL((amax_tensor_kernel<ODL_F32, 4, false>), dim3((unsigned)g), dim3(kFatThreads), 0, stream, x, n, amax_out, FusedScale{});
+            if (src_dtype == ODL_BF16) hipLaunchKernelGGL((amax_tensor_kernel<ODL_BF16, 4, 0>), dim3((unsigned)g), dim3(kFatThreads), 0, stream, x, n, amax_out, FusedScale{});
+            else hipLaunchKernelGGL((amax_tensor_kernel<ODL_F32, 4, 0>), dim3((unsigned)g), dim3(kFatThreads), 0, stream, x, n, amax_out, FusedScale{});
         } else {
             const int64_t g = grid_for(n, kThreads * 8, 8);
             if (src_dtype == ODL_BF16) hipLaunchKernelGGL((amax_tensor_scalar_kernel<ODL_BF16>), dim3((unsigned)g), dim3(kThreads), 0, stream, x, n, amax_out);
@@ -652,8 +697,8 @@ extern "C" int odl_fp8_amax_scale(const void *x, int src_dtype, int64_t rows, in
     const int esz = src_dtype == ODL_BF16 ? 2 : 4;
     const int64_t g = grid_for(n * esz / 16, kFatThreads * 4, 2);
     const FusedScale fs{workspace, scale, scale_inv, fmt == ODL_FP8_E5M2 ? 57344.0f : 448.0f, margin};
-    if (src_dtype == ODL_BF16) hipLaunchKernelGGL((amax_tensor_kernel<ODL_BF16, 4, true>), dim3((unsigned)g), dim3(kFatThreads), 0, stream, x, n, amax_out, fs);
-    else hipLaunchKernelGGL((amax_tensor_kernel<ODL_F32, 4, true>), dim3((unsigned)g), dim3(kFatThreads), 0, stream, x, n, amax_out, fs);
+    if (src_dtype == ODL_BF16) hipLaunchKernelGGL((amax_tensor_kernel<ODL_BF16, 4, 1>), dim3((unsigned)g), dim3(kFatThreads), 0, stream, x, n, amax_out, fs);
+    else hipLaunchKernelGGL((amax_tensor_kernel<ODL_F32, 4, 1>), dim3((unsigned)g), dim3(kFatThreads), 0, stream, x, n, amax_out, fs);
     return check_launch("odl_fp8_amax_scale");
 }
 
@@ -685,13 +730,13 @@ namespace odl {
 
 template <int SRC, int FMT, int MODE>
 static void launch_cast(const void *x, int64_t rows, int64_t cols, const float *scale, uint8_t *out, float *amax_out,
-                        hipStream_t stream) {
+                        hipStream_t stream, int margin = 0, float *dyn_out = nullptr) {
     if (amax_out) {
         const int64_t g = grid_for(rows * cols / 16, kFatThreads, 2);
-        hipLaunchKernelGGL((cast_kernel<SRC, FMT, MODE, true>), dim3((unsigned)g), dim3(kFatThreads), 0, stream, x, rows, cols, scale, out, amax_out);
+        hipLaunchKernelGGL((cast_kernel<SRC, FMT, MODE, true>), dim3((unsigned)g), dim3(kFatThreads), 0, stream, x, rows, cols, scale, out, amax_out, margin, dyn_out);
     } else {
         const int64_t g = grid_for(rows * cols / 16, kThreads, 16);
-        hipLaunchKernelGGL((cast_kernel<SRC, FMT, MODE, false>), dim3((unsigned)g), dim3(kThreads), 0, stream, x, rows, cols, scale, out, amax_out);
+        hipLaunchKernelGGL((cast_kernel<SRC, FMT, MODE, false>), dim3((unsigned)g), dim3(kThreads), 0, stream, x, rows, cols, scale, out, amax_out, margin, dyn_out);
     }
 }
 
@@ -712,10 +757,10 @@ static void launch_generic(const void *x, int64_t rows, int64_t cols, const floa
 
 template <int SRC, int FMT, int MODE>
 static void launch_ct(const void *x, int64_t rows, int64_t cols, const float *scale, uint8_t *out, uint8_t *out_t,
-                      float *amax_out, hipStream_t stream) {
+                      float *amax_out, hipStream_t stream, int margin = 0, float *dyn_out = nullptr) {
     int64_t g = ((rows + kTileR - 1) / kTileR) * ((cols + kTileC - 1) / kTileC);
     if (amax_out && g > (int64_t)num_cus() * 4) g = (int64_t)num_cus() * 4;
-#define ODL_CT(AM, RM) hipLaunchKernelGGL((cast_transpose_kernel<SRC, FMT, MODE, AM, RM>), dim3((unsigned)g), dim3(kThreads), 0, stream, x, rows, cols, scale, out, out_t, amax_out)
+#define ODL_CT(AM, RM) hipLaunchKernelGGL((cast_transpose_kernel<SRC, FMT, MODE, AM, RM>), dim3((unsigned)g), dim3(kThreads), 0, stream, x, rows, cols, scale, out, out_t, amax_out, margin, dyn_out)
     if (amax_out) { if (out) ODL_CT(true, true); else ODL_CT(true, false); }
     else { if (out) ODL_CT(false, true); else ODL_CT(false, false); }
 #undef ODL_CT
@@ -777,4 +822,65 @@ extern "C" int odl_fp8_cast_transpose(const void *x, int src_dtype, int64_t rows
     if (fast) ODL_DISPATCH_SRC_FMT(launch_ct_mode, mode, x, rows, cols, scale, out, out_t, amax_out, stream);
     else ODL_DISPATCH_SRC_FMT(launch_generic, x, rows, cols, scale, mode, out, out_t, amax_out, stream);
     return check_launch("odl_fp8_cast_transpose");
+}
+
+namespace odl {
+
+template <int SRC, int FMT>
+static void launch_dynamic(const void *x, int64_t rows, int64_t cols, const float *parts, int margin, uint8_t *out,
+                           uint8_t *out_t, float *dyn_out, bool fast, hipStream_t stream) {
+    if (!fast) {
+        // element-at-a-time route: scale first (one block), then the generic kernel reads it from dyn_out[1]
+        hipLaunchKernelGGL((parts_to_scale_kernel<FMT>), dim3(1), dim3(kThreads), 0, stream, parts, margin, dyn_out);
+        launch_generic<SRC, FMT>(x, rows, cols, dyn_out + 1, ODL_SCALE_TENSOR, out, out_t, nullptr, stream);
+    } else if (out_t) {
+        launch_ct<SRC, FMT, kScaleParts>(x, rows, cols, parts, out, out_t, nullptr, stream, margin, dyn_out);
+    } else {
+        launch_cast<SRC, FMT, kScaleParts>(x, rows, cols, parts, out, nullptr, stream, margin, dyn_out);
+    }
+}
+
+}  // namespace odl
+
+extern "C" int odl_fp8_amax_parts(const void *x, int src_dtype, int64_t rows, int64_t cols, float *parts, odl_stream_t stream_) {
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    if (rows < 0 || cols < 0) return set_error(ODL_ERR_ARG, "odl_fp8_amax_parts: negative shape %lld x %lld", (long long)rows, (long long)cols);
+    if ((!x && rows * cols > 0) || !parts) return set_error(ODL_ERR_ARG, "odl_fp8_amax_parts: null pointer");
+    if (src_dtype != ODL_BF16 && src_dtype != ODL_F32) return set_error(ODL_ERR_ARG, "odl_fp8_amax_parts: src_dtype %d", src_dtype);
+    const int64_t n = rows * cols;
+    if (n == 0 || !aligned16(x)) {
+        // nothing to read, or a pointer the vector kernel cannot take: everything into parts[0]
+        hipLaunchKernelGGL(fill_f32_kernel, dim3((kAmaxParts + 255) / 256), dim3(256), 0, stream, parts, (int64_t)kAmaxParts, 0.0f);
+        if (n == 0) return check_launch("odl_fp8_amax_parts(fill)");
+        return odl_fp8_amax(x, src_dtype, rows, cols, ODL_SCALE_TENSOR, parts, 1, stream_);
+    }
+    const int esz = src_dtype == ODL_BF16 ? 2 : 4;
+    int64_t g = grid_for(n * esz / 16, kFatThreads * 4, 2);
+    if (g > kAmaxParts) g = kAmaxParts;
+    if (src_dtype == ODL_BF16) hipLaunchKernelGGL((amax_tensor_kernel<ODL_BF16, 4, 2>), dim3((unsigned)g), dim3(kFatThreads), 0, stream, x, n, parts, FusedScale{});
+    else hipLaunchKernelGGL((amax_tensor_kernel<ODL_F32, 4, 2>), dim3((unsigned)g), dim3(kFatThreads), 0, stream, x, n, parts, FusedScale{});
+    return check_launch("odl_fp8_amax_parts");
+}
+
+extern "C" int odl_fp8_cast_dynamic(const void *x, int src_dtype, int64_t rows, int64_t cols, const float *parts, int fmt, int margin,
+                                    uint8_t *out, uint8_t *out_t, float *dyn_out, odl_stream_t stream_) {
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    if (int e = check_cast_args("odl_fp8_cast_dynamic", x, src_dtype, rows, cols, parts, ODL_SCALE_TENSOR, fmt)) return e;
+    if (!parts || !dyn_out) return set_error(ODL_ERR_ARG, "odl_fp8_cast_dynamic: null pointer");
+    if (rows * cols == 0) {                       // nothing to cast: only the three numbers
+        if (fmt == ODL_FP8_E4M3) hipLaunchKernelGGL((parts_to_scale_kernel<ODL_FP8_E4M3>), dim3(1), dim3(kThreads), 0, stream, parts, margin, dyn_out);
+        else hipLaunchKernelGGL((parts_to_scale_kernel<ODL_FP8_E5M2>), dim3(1), dim3(kThreads), 0, stream, parts, margin, dyn_out);
+        return check_launch("odl_fp8_cast_dynamic(empty)");
+    }
+    if (!out && !out_t) return set_error(ODL_ERR_ARG, "odl_fp8_cast_dynamic: out and out_t are both null");
+    bool fast;
+    if (out_t) {
+        const int64_t tiles = ((rows + kTileR - 1) / kTileR) * ((cols + kTileC - 1) / kTileC);
+        fast = cols % 8 == 0 && rows % 16 == 0 && aligned16(x) && aligned16(out_t) && (!out || (reinterpret_cast<uintptr_t>(out) & 7) == 0) &&
+               tiles <= 0x7fffffffLL && rows * cols > 0;
+    } else {
+        fast = cols % 16 == 0 && aligned16(x) && aligned16(out) && rows * cols > 0;
+    }
+    ODL_DISPATCH_SRC_FMT(launch_dynamic, x, rows, cols, parts, margin, out, out_t, dyn_out, fast, stream);
+    return check_launch("odl_fp8_cast_dynamic");
 }

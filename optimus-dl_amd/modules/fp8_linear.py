@@ -66,11 +66,8 @@ class _WeightCache:
 
 def _quantise_dynamic(x2d: torch.Tensor, fmt: int, margin: int, need_t: bool, need_rowmajor: bool = True):
     """Per-tensor current scaling: amax pass, scale, cast (+transpose) pass."""
-    amax, scale, scale_inv = native.amax_scale(x2d, fmt, margin)
-    if need_t:
-        q, q_t = native.cast_transpose(x2d, scale, fmt, T, want_rowmajor=need_rowmajor)
-    else:
-        q, q_t = native.cast(x2d, scale, fmt, T), None
+    q, q_t, amax, _, scale_inv = native.quantize_dynamic(x2d, fmt, margin, want_rowmajor=need_rowmajor or not need_t,
+                                                        want_transposed=need_t)
     return q, q_t, scale_inv, amax
 
 

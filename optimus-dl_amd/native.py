@@ -35,6 +35,8 @@ EXPORTS = (
     "odl_fp8_amax",
     "odl_fp8_scale_from_amax",
     "odl_fp8_amax_scale",
+    "odl_fp8_amax_parts",
+    "odl_fp8_cast_dynamic",
     "odl_fp8_cast",
     "odl_fp8_cast_transpose",
     "odl_fp8_gemm_nt",
@@ -77,6 +79,8 @@ def load() -> ctypes.CDLL:
         L.odl_fp8_amax.argtypes = [vp, i32, i64, i64, i32, vp, i32, vp]
         L.odl_fp8_scale_from_amax.argtypes = [vp, i64, i32, i32, vp, vp, vp]
         L.odl_fp8_amax_scale.argtypes = [vp, i32, i64, i64, i32, i32, vp, vp, vp, vp, vp]
+        L.odl_fp8_amax_parts.argtypes = [vp, i32, i64, i64, vp, vp]
+        L.odl_fp8_cast_dynamic.argtypes = [vp, i32, i64, i64, vp, i32, i32, vp, vp, vp, vp]
         L.odl_fp8_cast.argtypes = [vp, i32, i64, i64, vp, i32, i32, vp, vp, vp]
         L.odl_fp8_cast_transpose.argtypes = [vp, i32, i64, i64, vp, i32, i32, vp, vp, vp, vp]
         L.odl_fp8_gemm_nt.argtypes = [vp, vp, i64, i64, i64, i32, i32, vp, i64, vp, i64, vp, i32, vp, i32, vp]
@@ -171,6 +175,48 @@ def amax_scale(x: torch.Tensor, fmt: int, margin: int = 0):
     _check(load().odl_fp8_amax_scale(x.data_ptr(), _src_dtype(x), rows, cols, fmt, margin, base, base + 4, base + 8,
                                      ws.data_ptr(), stream), "odl_fp8_amax_scale")
     return out[0:1], out[1:2], out[2:3]
+
+
+AMAX_PARTS = 512                       # ODL_FP8_AMAX_PARTS
+_parts: dict[tuple[int, int], torch.Tensor] = {}
+
+
+def amax_parts(x: torch.Tensor) -> torch.Tensor:
+    """AMAX_PARTS partial maxima of |x| (no atomics); input of :func:`cast_dynamic`.  The buffer is one
+    per (device, stream): it is consumed by the next launch on that stream."""
+    x = _as_2d(x)
+    rows, cols = x.shape
+    stream = _stream()
+    key = (x.device.index if x.device.index is not None else torch.cuda.current_device(), stream)
+    parts = _parts.get(key)
+    if parts is None:
+        parts = _parts[key] = torch.zeros(AMAX_PARTS, dtype=torch.float32, device=x.device)
+    _check(load().odl_fp8_amax_parts(x.data_ptr(), _src_dtype(x), rows, cols, parts.data_ptr(), stream), "odl_fp8_amax_parts")
+    return parts
+
+
+def cast_dynamic(x: torch.Tensor, parts: torch.Tensor, fmt: int, margin: int = 0, want_rowmajor: bool = True,
+                 want_transposed: bool = True):
+    """Cast with the per-tensor scale derived inside the kernel from the partial maxima.
+    -> (q or None, q_t or None, amax, scale, scale_inv); the last three are fp32[1]."""
+    if not (want_rowmajor or want_transposed):
+        raise NativeError("cast_dynamic: nothing to produce")
+    x = _as_2d(x)
+    rows, cols = x.shape
+    _f32_dev(parts, AMAX_PARTS, "cast_dynamic parts")
+    q = torch.empty((rows, cols), dtype=torch.uint8, device=x.device) if want_rowmajor else None
+    q_t = torch.empty((cols, rows), dtype=torch.uint8, device=x.device) if want_transposed else None
+    dyn = torch.empty(3, dtype=torch.float32, device=x.device)
+    _check(load().odl_fp8_cast_dynamic(x.data_ptr(), _src_dtype(x), rows, cols, parts.data_ptr(), fmt, margin,
+                                       q.data_ptr() if q is not None else None, q_t.data_ptr() if q_t is not None else None,
+                                       dyn.data_ptr(), _stream()), "odl_fp8_cast_dynamic")
+    return q, q_t, dyn[0:1], dyn[1:2], dyn[2:3]
+
+
+def quantize_dynamic(x: torch.Tensor, fmt: int, margin: int = 0, want_rowmajor: bool = True, want_transposed: bool = True):
+    """Current scaling of one tensor in two launches: partial maxima, then a cast that derives the
+    scale itself.  -> (q or None, q_t or None, amax, scale, scale_inv)."""
+    return cast_dynamic(x, amax_parts(x), fmt, margin, want_rowmajor, want_transposed)
 
 
 def scale_from_amax(amax_t: torch.Tensor, fmt: int, margin: int = 0):

@@ -317,7 +317,7 @@ def test_linears_fed_by_the_same_tensor_quantise_it_once(amp, monkeypatch, in_dt
         assert recipe.shared_input is None                      # dropped when the context was left
         return h.detach(), xd.grad.detach(), gate.weight.grad.detach(), up.weight.grad.detach()
 
-    calls = _count_calls(monkeypatch, native, "amax_scale")
+    calls = _count_calls(monkeypatch, native, "amax_parts")
     shared = run(True)
     n_shared = len([s for s in calls if tuple(s) == (M, K)])
     calls.clear()
@@ -339,7 +339,7 @@ def test_shared_input_is_not_reused_after_an_in_place_change_or_for_another_tens
     recipe = amp.create_fp8_recipe("tensorwise", "hybrid")
     lin = make_linear(seeded_bf16((N, K), 0.02, 50))
     x = seeded_bf16((M, K), 1.0, 51).cuda()
-    calls = _count_calls(monkeypatch, native, "amax_scale")
+    calls = _count_calls(monkeypatch, native, "amax_parts")
     with torch.no_grad(), recipe.autocast():
         y1 = lin(x)
         y1_again = lin(x)                                       # hit

@@ -99,6 +99,49 @@ def test_amax_scale_in_one_launch_equals_the_two_step_route(N, fmt):
 
 
 @pytest.mark.parametrize("fmt", [O.E4M3, O.E5M2])
+def test_two_launch_dynamic_quantisation_equals_the_step_by_step_route(N, fmt):
+    """amax_parts + cast_dynamic against amax -> scale_from_amax -> cast / cast_transpose (and the oracle):
+    same codes, same amax, scale and 1/scale, for shapes on the fast and on the element-at-a-time routes."""
+    cases = [((8192, 4096), 1.0, torch.bfloat16), ((256, 128), 0.02, torch.bfloat16), ((1000, 48), 3.0, torch.float32),
+             ((33, 20), 1e-3, torch.bfloat16), ((16, 16), 5.0, torch.float32), ((5, 3), 1.0, torch.bfloat16),
+             ((2048, 14336), 1e-3, torch.bfloat16)]
+    for margin in (0, 1):
+        for i, (shape, std, dtype) in enumerate(cases):
+            x = seeded_bf16(shape, std=std, seed=70 + i)
+            xd = x.to(dtype).cuda()
+            q, q_t, amax, scale, scale_inv = N.quantize_dynamic(xd, fmt, margin)
+            a2 = N.amax(xd)
+            s2, si2 = N.scale_from_amax(a2, fmt, margin)
+            q2, q2_t = N.cast_transpose(xd, s2, fmt)
+            assert_f32_bits_equal(torch.cat([amax, scale, scale_inv]), torch.cat([a2, s2, si2]).cpu(), f"dynamic numbers {shape}")
+            assert_bytes_equal(q, q2, f"dynamic codes {shape}")
+            assert_bytes_equal(q_t, q2_t, f"dynamic transposed codes {shape}")
+            assert_f32_bits_equal(amax, O.t_amax(x), f"amax vs oracle {shape}")
+            if shape[0] * shape[1] <= 1 << 20:
+                assert_bytes_equal(q, O.t_cast(x, scale.cpu(), fmt), f"codes vs oracle {shape}")
+            only_q, none_t, *_ = N.quantize_dynamic(xd, fmt, margin, want_transposed=False)
+            none_q, only_t, *_ = N.quantize_dynamic(xd, fmt, margin, want_rowmajor=False)
+            assert none_t is None and none_q is None
+            assert_bytes_equal(only_q, q2, "row-major only")
+            assert_bytes_equal(only_t, q2_t, "transposed only")
+    # specials: zeros -> scale 1; NaN -> amax NaN, scale 1, code 0x7F; empty; unaligned view
+    z = torch.zeros((64, 64), dtype=torch.bfloat16, device="cuda")
+    q, _, amax, scale, _ = N.quantize_dynamic(z, fmt)
+    assert amax.item() == 0.0 and scale.item() == 1.0 and int(q.max()) == 0
+    z[3, 5] = float("nan")
+    q, _, amax, scale, _ = N.quantize_dynamic(z, fmt)
+    assert torch.isnan(amax).item() and scale.item() == 1.0 and int(q[3, 5]) == 0x7F
+    q, q_t, amax, scale, _ = N.quantize_dynamic(torch.empty((0, 16), dtype=torch.bfloat16, device="cuda"), fmt)
+    assert q.shape == (0, 16) and q_t.shape == (16, 0)
+    flat = seeded_bf16((1, 5000), seed=6).cuda()
+    view = flat[0, 3:4003].reshape(40, 100)
+    q, q_t, amax, scale, _ = N.quantize_dynamic(view, fmt)
+    assert_f32_bits_equal(amax, O.t_amax(view.cpu()), "unaligned amax")
+    assert_bytes_equal(q, O.t_cast(view.cpu(), scale.cpu(), fmt), "unaligned codes")
+    assert torch.equal(q_t, q.t().contiguous())
+
+
+@pytest.mark.parametrize("fmt", [O.E4M3, O.E5M2])
 def test_scale_from_amax_bit_exact(N, fmt):
     rng = np.random.default_rng(0)
     a = np.concatenate([
