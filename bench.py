@@ -31,7 +31,7 @@ PEAK_FP8_TFLOPS = 5000.0     # MI355X dense FP8 MFMA, published
 PEAK_HBM_GBPS = 8000.0       # MI355X HBM3E, published
 # Memory-side bytes per GEMM launch (mean of the nine launches of a step), from two rocprofv3 --pmc runs
 # (FETCH_SIZE scaled x2.00, WRITE_SIZE x1.00 against a 256 MiB copy kernel): profiles/pmc_fetch_write__cfg3_mlp.md
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = 8.78e8
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = 8.79e8
 M_TOKENS, D_MODEL, D_FF = 8192, 4096, 14336
 LAYERS = (("gate", D_MODEL, D_FF), ("up", D_MODEL, D_FF), ("down", D_FF, D_MODEL))   # name, K(in), N(out)
 
@@ -168,6 +168,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU leg (for profiler runs)")
     ap.add_argument("--gemm-variant", type=int, default=-1)
+    ap.add_argument("--no-standalone", action="store_true",
+                    help="skip the stand-alone measurements of the memory-bound kernels (keeps profiler traces to the steps)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy (reference kernel for scaling FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -284,8 +286,9 @@ def main() -> int:
             "launches": gemm["launches"],
         },
         "hbm_kernels": hbm,
-        "hbm_kernels_standalone": standalone_hbm(torch, native),
     }
+    if not args.no_standalone:
+        line["hbm_kernels_standalone"] = standalone_hbm(torch, native)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(torch)
     print(json.dumps(line))
