@@ -505,7 +505,10 @@ __global__ __launch_bounds__(kThreads) void cast_transpose_kernel(const void *__
     // With a fused amax the grid is small and each block walks several tiles, so
     // that the kernel ends in few atomics; otherwise one tile per block.
     for (int64_t tile_id = blockIdx.x; tile_id < ntiles; tile_id += gridDim.x) {
-    const int64_t tr = tile_id / tiles_c, tc = tile_id % tiles_c;
+    // Tiles are walked from the end of the tensor: the amax pass that ran just before read it front
+    // to back, so its tail is what the memory-side cache still holds.
+    const int64_t rev = ntiles - 1 - tile_id;
+    const int64_t tr = rev / tiles_c, tc = rev % tiles_c;
     const int64_t r0 = tr * kTileR + ty * 4, c0 = tc * kTileC + tx * 8;
     const bool col_ok = c0 < cols;                  // cols % 8 == 0 (host-checked), so the whole 8-wide patch is in or out
 
