@@ -152,17 +152,20 @@ def cpu_baseline(torch, seconds_hint=20.0):
     torch.set_num_threads(cores)
     m = 4096
     data = make_inputs(torch, m=m, device="cpu")
-    t0 = time.perf_counter()
-    for name, k, n in LAYERS:
-        d = data[name]
-        O.linear_fwd_bwd(d["x"], d["w"], d["dy"], O.E4M3, O.E5M2)
-    dt = time.perf_counter() - t0
+    passes, dt = 0, 0.0
+    while dt < 10.0 and passes < 8:          # about 10-15 s of CPU work on the GPU box's host share
+        t0 = time.perf_counter()
+        for name, k, n in LAYERS:
+            d = data[name]
+            O.linear_fwd_bwd(d["x"], d["w"], d["dy"], O.E4M3, O.E5M2)
+        dt += time.perf_counter() - t0
+        passes += 1
     return {
-        "value": step_flops(m) / dt / 1e12,
+        "value": passes * step_flops(m) / dt / 1e12,
         "unit": "TFLOP/s",
         "cores": cores,
         "kind": "port",
-        "sample": f"rows 0..{m - 1} of {M_TOKENS} (all three Linears, fwd+bwd incl. amax/cast, 1 pass, {dt:.1f} s); "
+        "sample": f"rows 0..{m - 1} of {M_TOKENS} (all three Linears, fwd+bwd incl. amax/cast), {passes} passes in {dt:.1f} s; "
                   "torch CPU float8 cast + fp32 matmul",
         "seconds": dt,
     }
