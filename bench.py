@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the FP8 Linear path on one MI355X.
 
-Workload (BASELINE config 3): the three Linears of a Llama-3-8B SwiGLU MLP,
+Workload (configuration 3 of the benchmark definition, `configs[2]`): the three Linears of a Llama-3-8B SwiGLU MLP,
 forward + backward in FP8 with per-tensor dynamic scaling (E4M3 for activations
 and weights, E5M2 for gradients), M = 8192 tokens:
     gate, up : X [8192, 4096]   W [14336, 4096]   dY [8192, 14336]
@@ -276,7 +276,7 @@ def main() -> int:
         "dtype": "fp8 (e4m3 x/w, e5m2 grads; fp32 accumulate; bf16 out)",
         "data": "synthetic",
         "config": {
-            "workload": "BASELINE config 3: Llama-3-8B SwiGLU MLP Linears (gate, up [14336x4096]; down [4096x14336]), "
+            "workload": "configs[2] of BASELINE.json: Llama-3-8B SwiGLU MLP Linears (gate, up [14336x4096]; down [4096x14336]), "
                         "M=8192, FP8 fwd+bwd, per-tensor dynamic scaling, fused cast+transpose for wgrad",
             "flop_per_step": step_flops(),
             "gemms_per_step": 9,

@@ -1,4 +1,4 @@
-"""GPU parity at the full BASELINE sizes, through properties that do not need the
+"""GPU parity at the full sizes of the benchmark configurations, through properties that do not need the
 whole answer on the CPU:
 
   * a random sample of output rows x columns against the oracle's emulated matmul
@@ -9,7 +9,7 @@ whole answer on the CPU:
   * casts: the transposed copy is the transpose of the row-major copy, a sample of rows
     matches the oracle bit for bit, amax equals the maximum of block maxima.
 
-Inputs are drawn on the GPU (seeded) and are what BASELINE describes: N(0,1) activations,
+Inputs are drawn on the GPU (seeded) and are what the benchmark definition describes: N(0,1) activations,
 N(0,0.02) weights, N(0,1e-3) gradients.
 """
 import pytest
@@ -57,7 +57,7 @@ def sample_check(out, aq, bq, fa, fb, sa_inv, sb_inv, seed, what, rows=48, cols=
     assert err <= TOL, f"{what}: max rel err {err} on a {rows}x{cols} sample"
 
 
-# (M, N, K) of the GEMMs that BASELINE's configurations launch
+# (M, N, K) of the GEMMs that the benchmark configurations launch
 CFG_SHAPES = [
     pytest.param(8192, 14336, 4096, id="cfg3-fwd-gate"),
     pytest.param(8192, 4096, 14336, id="cfg3-fwd-down"),

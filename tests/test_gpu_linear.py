@@ -109,7 +109,7 @@ def test_rowwise_with_outlier_channels_matches_oracle(amp):
 
 
 def test_delayed_scaling_twenty_steps_with_drift(amp):
-    """BASELINE config 5 in miniature: history 16, 20 steps, input std 1.0 -> 1.5."""
+    """Benchmark configuration 5 in miniature: history 16, 20 steps, input std 1.0 -> 1.5."""
     M, K, N, H, STEPS = 256, 512, 384, 16, 20
     w = seeded_bf16((N, K), 0.01, 100)
     recipe = amp.create_fp8_recipe("delayed", "hybrid", amax_history_len=H)

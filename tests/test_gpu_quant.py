@@ -221,7 +221,7 @@ def test_cast_with_fused_amax_for_delayed_scaling(N, fmt):
 
 
 def test_cast_transpose_large_matches_cast_then_transpose(N):
-    """Size-independent property at a BASELINE shape: out_t == out^T bytewise."""
+    """Size-independent property at a full benchmark shape: out_t == out^T bytewise."""
     x = seeded_bf16((8192, 4096), seed=0).cuda()
     am = N.amax(x)
     s, _ = N.scale_from_amax(am, O.E4M3)
