@@ -198,3 +198,66 @@ def test_delayed_scaling_config_5_twenty_steps_at_full_size(N):
     # after 20 steps the 16-deep window has forgotten steps 0..3: the input scale is set by the last 16 amaxes only
     hist = up.fp8_meta["scaling_fwd"].amax_history[:, 0]
     assert int((hist > 0).sum()) == H - 1 and hist[0].item() == 0.0
+
+
+def test_config_1_gpt2_up_projection_forward_against_the_cpu_path(N):
+    """The one configuration the CPU emulation runs in full: X [4096, 768] ~N(0,1), W [3072, 768] ~N(0,0.02),
+    per-tensor E4M3, bf16 out [4096, 3072].  Codes and scales bit for bit, the output within 1e-2."""
+    from tests.helpers import seeded_bf16
+
+    x, w = seeded_bf16((4096, 768), 1.0, 0), seeded_bf16((3072, 768), 0.02, 1)
+    sx, sw = O.t_scale(O.t_amax(x), O.E4M3), O.t_scale(O.t_amax(w), O.E4M3)
+    xq_ref, wq_ref = O.t_cast(x, sx, O.E4M3), O.t_cast(w, sw, O.E4M3)
+    ref = O.t_gemm_nt(xq_ref, wq_ref, O.E4M3, O.E4M3, 1.0 / sx, 1.0 / sw)
+    xq, _, ax, s_x, sxi = N.quantize_dynamic(x.cuda(), O.E4M3, want_transposed=False)
+    wq, _, aw, s_w, swi = N.quantize_dynamic(w.cuda(), O.E4M3, want_transposed=False)
+    assert_bytes_equal(xq, xq_ref, "x codes")
+    assert_bytes_equal(wq, wq_ref, "w codes")
+    assert_f32_bits_equal(torch.cat([s_x, s_w]), torch.cat([sx.reshape(1), sw.reshape(1)]), "scales")
+    y = N.gemm_nt(xq, wq, O.E4M3, O.E4M3, sxi, swi)
+    assert y.shape == (4096, 3072) and y.dtype == torch.bfloat16
+    err = max_rel_err(y, ref)
+    assert err <= TOL, f"config 1 forward: {err}"
+    # and through the module, as a user would run it
+    from optimus_dl_amd.modules import amp
+    from optimus_dl_amd.modules.fp8_linear import FP8Linear
+
+    lin = FP8Linear(768, 3072, bias=False, device="cuda", dtype=torch.bfloat16)
+    with torch.no_grad():
+        lin.weight.copy_(w)
+        with amp.create_fp8_recipe("tensorwise", "e4m3").autocast():
+            y2 = lin(x.cuda().reshape(4, 1024, 768))
+    assert torch.equal(y2.reshape(4096, 3072), y)
+
+
+def test_config_2_attention_projections_forward_backward(N):
+    """Wq, Wk, Wv, Wo of Llama-3-8B at M = 8192 through FP8Linear: the three projections that share X quantise
+    it once; outputs and gradients on a sample against the oracle's matmul of the same codes."""
+    from optimus_dl_amd import native
+    from optimus_dl_amd.modules import amp
+    from optimus_dl_amd.modules.fp8_linear import FP8Linear
+
+    M, K = 8192, 4096
+    recipe = amp.create_fp8_recipe("tensorwise", "hybrid")
+    x = draw((M, K), 1.0, 51).requires_grad_(True)
+    outs = {}
+    lins = {name: FP8Linear(K, n, bias=False, device="cuda", dtype=torch.bfloat16) for name, n in
+            (("wq", 4096), ("wk", 1024), ("wv", 1024))}
+    for i, lin in enumerate(lins.values()):
+        with torch.no_grad():
+            lin.weight.copy_(draw(tuple(lin.weight.shape), 0.02, 60 + i))
+    with recipe.autocast():
+        for name, lin in lins.items():
+            outs[name] = lin(x)
+    with recipe.backward():
+        torch.autograd.backward(list(outs.values()), [draw(tuple(o.shape), 1e-3, 70 + i) for i, o in enumerate(outs.values())])
+    xq, xq_t, _, sx, sxi = native.quantize_dynamic(x.detach(), O.E4M3)
+    for name, lin in lins.items():
+        wq, _, _, sw, swi = native.quantize_dynamic(lin.weight.detach(), O.E4M3, want_transposed=False)
+        sample_check(outs[name].detach(), xq, wq, O.E4M3, O.E4M3, sxi, swi, seed=80, what=f"{name} forward", cols=256)
+        assert lin.weight.grad is not None and lin.weight.grad.shape == lin.weight.shape
+    assert x.grad is not None and torch.isfinite(x.grad.float()).all()
+    # dW of wk against the oracle on a sample: dW = Q(dY)^T . Q(X)
+    dy_k = draw((M, 1024), 1e-3, 71)
+    gq, gq_t, _, sg, sgi = native.quantize_dynamic(dy_k, O.E5M2)
+    sample_check(lins["wk"].weight.grad, gq_t, xq_t, O.E5M2, O.E4M3, sgi, sxi, seed=81, what="wk wgrad", cols=256)
