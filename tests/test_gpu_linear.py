@@ -352,3 +352,44 @@ def test_shared_input_is_not_reused_after_an_in_place_change_or_for_another_tens
     assert len(calls) == 4                                      # + x after the change + the clone
     assert torch.equal(y1, y1_again) and torch.equal(y2, y3)
     assert not torch.equal(y1, y2)
+
+
+def test_forward_backward_can_be_captured_in_a_graph_and_replayed(amp):
+    """Small Linears are launch-bound; callers capture them.  Every native call takes the capture
+    stream and allocates nothing itself, so a captured forward+backward must replay correctly:
+    three replays on new data, eager work and synchronisations in between, each against eager."""
+    M, K, N = 256, 512, 384
+    recipe = amp.create_fp8_recipe("tensorwise", "hybrid")
+    lin = make_linear(seeded_bf16((N, K), 0.02, 90))
+    x_static = torch.zeros((M, K), dtype=torch.bfloat16, device="cuda", requires_grad=True)
+    dy_static = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+
+    def fwd_bwd():
+        lin._wcache.key = None
+        with recipe.autocast():
+            y = lin(x_static)
+        with recipe.backward():
+            gx, gw = torch.autograd.grad(y, (x_static, lin.weight), dy_static)
+        return y, gx, gw
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):                       # warm-up off the default stream, as capture requires
+        for _ in range(2):
+            fwd_bwd()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y_g, gx_g, gw_g = fwd_bwd()
+    for rep in range(3):
+        x_new, dy_new = seeded_bf16((M, K), 1.0 + rep, 91 + rep).cuda(), seeded_bf16((M, N), 1e-3 * (rep + 1), 95 + rep).cuda()
+        with torch.no_grad():
+            x_static.copy_(x_new)
+            dy_static.copy_(dy_new)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in (y_g, gx_g, gw_g)]
+        want = fwd_bwd()                                # eager, same buffers
+        torch.cuda.synchronize()
+        for name, a, b in zip(("y", "dx", "dw"), got, want):
+            assert torch.equal(a, b), f"replay {rep}: {name} differs from eager"
