@@ -104,6 +104,25 @@ int odl_fp8_cast_dynamic(const void *x, int src_dtype, int64_t rows, int64_t col
                          odl_stream_t stream);
 
 /*
+ * The rowwise recipe needs every tensor twice: scaled per row for the GEMM that contracts
+ * its columns, and scaled per column, transposed, for the GEMM that contracts its rows.
+ *   odl_fp8_amax_rowcol: amax_row[rows] and amax_col[cols] in one pass over x;
+ *   odl_fp8_cast_rowcol: out[rows, cols] = codes with scale_row, out_t[cols, rows] = codes
+ *                        with scale_col, one pass; scale = fp8_max(fmt) / amax / 2^margin per
+ *                        row / column (rules of odl_fp8_scale_from_amax); the scales and their
+ *                        inverses are written to s_row, s_row_inv, s_col, s_col_inv.
+ * Results equal those of odl_fp8_amax (ROW, COL) + odl_fp8_scale_from_amax + odl_fp8_cast (ROW)
+ * + odl_fp8_cast_transpose (COL), bit for bit.  No counterpart in the reference (its recipes
+ * stop at per-tensor and block scaling, fp8.py:58-61); this is the "rowwise" extension.
+ */
+int odl_fp8_amax_rowcol(const void *x, int src_dtype, int64_t rows, int64_t cols, float *amax_row,
+                        float *amax_col, odl_stream_t stream);
+int odl_fp8_cast_rowcol(const void *x, int src_dtype, int64_t rows, int64_t cols, const float *amax_row,
+                        const float *amax_col, int fmt, int margin, uint8_t *out, uint8_t *out_t,
+                        float *s_row, float *s_row_inv, float *s_col, float *s_col_inv,
+                        odl_stream_t stream);
+
+/*
  * out[r,c] = fp8( clamp( fp32(x[r,c]) * s , +-max ) ), s = scale[0] | scale[r] | scale[c].
  * amax_out (may be NULL): *amax_out = max(*amax_out, max|x|), for delayed scaling,
  * where the cast uses an older scale while this step's amax is recorded.

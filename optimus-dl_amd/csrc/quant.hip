@@ -290,6 +290,77 @@ __global__ __launch_bounds__(kThreads) void amax_col_kernel(const void *__restri
     }
 }
 
+// ----------------------------------------------------- amax, per row AND per column
+// One pass for the rowwise recipe, which scales a tensor along its rows for one GEMM and along
+// its columns for another.  Same lane tile as amax_col_kernel; in addition every loaded 16-byte
+// piece is folded to one value and reduced over the 32 lanes that share its row (xor shuffles stay
+// inside a 32-lane half), and the first lane of the half does one atomicMax per row and block.
+// Both outputs accumulate (atomicMax): the caller zeroes them.
+template <int SRC>
+__global__ __launch_bounds__(kThreads) void amax_rowcol_kernel(const void *__restrict__ x, int64_t rows, int64_t cols,
+                                                                int rows_per_block, float *__restrict__ out_row,
+                                                                float *__restrict__ out_col) {
+    constexpr int ESZ = SRC == ODL_BF16 ? 2 : 4;
+    constexpr int CPL = 16 / ESZ;                 // columns per lane
+    constexpr int CW = 32 * CPL;                  // columns per block
+    __shared__ uint32_t red[8][CW + 1];
+    const int tx = threadIdx.x % 32, ty = threadIdx.x / 32;
+    const int64_t c0 = (int64_t)blockIdx.x * CW + tx * CPL;
+    const int64_t r0 = (int64_t)blockIdx.y * rows_per_block;
+    const int64_t r1 = min(rows, r0 + rows_per_block);
+    const bool col_ok = c0 + CPL <= cols;          // host guarantees cols % CPL == 0 and 16-byte rows
+    uint32_t m[CPL];
+#pragma unroll
+    for (int j = 0; j < CPL; ++j) m[j] = 0;
+    const char *base = reinterpret_cast<const char *>(x);
+    // every lane walks the same rows (the shuffles need all 32 lanes of a row); r1 - r0 is a multiple of 8
+    // except in the last slab, where rows past the end load nothing
+    for (int64_t rb = r0; rb < r1; rb += 32) {
+        u32x4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int64_t r = rb + ty + 8 * u;
+            v[u] = (col_ok && r < r1) ? *reinterpret_cast<const u32x4 *>(base + (r * cols + c0) * ESZ) : u32x4{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const uint32_t w[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+            uint32_t rowmax = 0;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                if constexpr (SRC == ODL_BF16) {
+                    const uint32_t a = abs_bf16x2(w[q]);
+                    const uint32_t lo = (a & 0xffffu) << 16, hi = a & 0xffff0000u;
+                    m[2 * q] = max(m[2 * q], lo);
+                    m[2 * q + 1] = max(m[2 * q + 1], hi);
+                    rowmax = max(rowmax, max(lo, hi));
+                } else {
+                    const uint32_t a = w[q] & 0x7fffffffu;
+                    m[q] = max(m[q], a);
+                    rowmax = max(rowmax, a);
+                }
+            }
+#pragma unroll
+            for (int off = 16; off > 0; off >>= 1) {
+                const uint32_t o = (uint32_t)__shfl_xor((int)rowmax, off, kWave);
+                rowmax = rowmax > o ? rowmax : o;
+            }
+            const int64_t r = rb + ty + 8 * u;
+            if (tx == 0 && r < r1 && rowmax != 0) atomicMax(reinterpret_cast<uint32_t *>(out_row) + r, rowmax);
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < CPL; ++j) red[ty][tx * CPL + j] = m[j];
+    __syncthreads();
+    for (int c = threadIdx.x; c < CW; c += kThreads) {
+        uint32_t v = 0;
+#pragma unroll
+        for (int y = 0; y < 8; ++y) v = max(v, red[y][c]);
+        const int64_t col = (int64_t)blockIdx.x * CW + c;
+        if (col < cols && v != 0) atomicMax(reinterpret_cast<uint32_t *>(out_col) + col, v);
+    }
+}
+
 // generic column amax for shapes the vector kernel refuses: one thread per column strip
 template <int SRC>
 __global__ void amax_col_scalar_kernel(const void *__restrict__ x, int64_t rows, int64_t cols, int rows_per_block,
@@ -606,6 +677,94 @@ __global__ __launch_bounds__(kThreads) void cast_transpose_kernel(const void *__
 }
 
 // ----------------------------------------------------------------- host helpers
+// ---------------------------------------- cast for the rowwise recipe, both operands at once
+// out   [rows, cols] = codes scaled per ROW    (scale derived from amax_row)
+// out_t [cols, rows] = codes scaled per COLUMN (scale derived from amax_col), transposed
+// One read of x instead of the two that a cast and a cast+transpose would make.  The 128 row
+// scales and 64 column scales of a tile are derived once per block (IEEE division) and kept in
+// LDS; the blocks of the first tile column / row also record 1/scale for the GEMM epilogues.
+template <int SRC, int FMT>
+__global__ __launch_bounds__(kThreads) void cast_rowcol_kernel(const void *__restrict__ x, int64_t rows, int64_t cols,
+                                                                const float *__restrict__ amax_row, const float *__restrict__ amax_col,
+                                                                int margin, uint8_t *__restrict__ out, uint8_t *__restrict__ out_t,
+                                                                float *__restrict__ s_row_out, float *__restrict__ s_row_inv,
+                                                                float *__restrict__ s_col_out, float *__restrict__ s_col_inv) {
+    __shared__ __attribute__((aligned(16))) uint8_t tile[kTileC * kLdsPitch];
+    __shared__ float s_row[kTileR], s_col[kTileC];
+    constexpr int ESZ = SRC == ODL_BF16 ? 2 : 4;
+    const int tx = threadIdx.x % 8;                 // 8 lanes across 64 columns
+    const int ty = threadIdx.x / 8;                 // 32 lane-rows, 4 rows each
+    const int64_t tiles_c = (cols + kTileC - 1) / kTileC;
+    const int64_t tr = blockIdx.x / tiles_c, tc = blockIdx.x % tiles_c;
+    if (threadIdx.x < kTileR) {
+        const int64_t r = tr * kTileR + threadIdx.x;
+        const float sc = r < rows ? scale_rule(amax_row[r], Fp8Lim<FMT>::max, margin, 1.0f) : 1.0f;
+        s_row[threadIdx.x] = sc;
+        if (tc == 0 && r < rows) { s_row_out[r] = sc; s_row_inv[r] = __fdiv_rn(1.0f, sc); }
+    } else if (threadIdx.x < kTileR + kTileC) {
+        const int64_t c = tc * kTileC + (threadIdx.x - kTileR);
+        const float sc = c < cols ? scale_rule(amax_col[c], Fp8Lim<FMT>::max, margin, 1.0f) : 1.0f;
+        s_col[threadIdx.x - kTileR] = sc;
+        if (tr == 0 && c < cols) { s_col_out[c] = sc; s_col_inv[c] = __fdiv_rn(1.0f, sc); }
+    }
+    __syncthreads();
+    const int64_t r0 = tr * kTileR + ty * 4, c0 = tc * kTileC + tx * 8;
+    const bool col_ok = c0 < cols;                  // cols % 8 == 0 (host-checked)
+    float sc_col[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) sc_col[j] = s_col[tx * 8 + j];
+
+    u32x4 raw[4][ESZ / 2];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const bool ok = col_ok && (r0 + i) < rows;
+        const u32x4 *p = reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(x) + ((r0 + i) * cols + c0) * ESZ);
+#pragma unroll
+        for (int h = 0; h < ESZ / 2; ++h) raw[i][h] = ok ? __builtin_nontemporal_load(p + h) : u32x4{0, 0, 0, 0};
+    }
+    uint32_t lo[4], hi[4];                          // column-scaled codes of columns 0..3 / 4..7 for each of the 4 rows
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        float f[8];
+        if constexpr (SRC == ODL_BF16) {
+            const uint32_t w[4] = {raw[i][0].x, raw[i][0].y, raw[i][0].z, raw[i][0].w};
+#pragma unroll
+            for (int q = 0; q < 4; ++q) { f[2 * q] = bf16_lo(w[q]); f[2 * q + 1] = bf16_hi(w[q]); }
+        } else {
+            const uint32_t w[8] = {raw[i][0].x, raw[i][0].y, raw[i][0].z, raw[i][0].w, raw[i][1].x, raw[i][1].y, raw[i][1].z, raw[i][1].w};
+#pragma unroll
+            for (int q = 0; q < 8; ++q) f[q] = bits_to_float(w[q]);
+        }
+        const float sr = s_row[ty * 4 + i];
+        const uint32_t rlo = quantise4<FMT>(f[0], f[1], f[2], f[3], sr, sr, sr, sr);
+        const uint32_t rhi = quantise4<FMT>(f[4], f[5], f[6], f[7], sr, sr, sr, sr);
+        if (col_ok && (r0 + i) < rows) ODL_CODE_STORE((u32x2{rlo, rhi}), reinterpret_cast<u32x2 *>(out + (r0 + i) * cols + c0));
+        lo[i] = quantise4<FMT>(f[0], f[1], f[2], f[3], sc_col[0], sc_col[1], sc_col[2], sc_col[3]);
+        hi[i] = quantise4<FMT>(f[4], f[5], f[6], f[7], sc_col[4], sc_col[5], sc_col[6], sc_col[7]);
+    }
+    // ---- transpose in registers, stage through LDS (as in cast_transpose_kernel)
+    uint32_t tl[4], th[4];
+    transpose4x4(lo, tl);
+    transpose4x4(hi, th);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        *reinterpret_cast<uint32_t *>(&tile[(tx * 8 + k) * kLdsPitch + ty * 4]) = tl[k];
+        *reinterpret_cast<uint32_t *>(&tile[(tx * 8 + 4 + k) * kLdsPitch + ty * 4]) = th[k];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+        const int chunk = threadIdx.x + it * kThreads;
+        const int k = chunk / 8, m16 = chunk % 8;
+        const int64_t oc = tc * kTileC + k, orow = tr * kTileR + m16 * 16;
+        if (oc < cols && orow < rows) {             // rows % 16 == 0 (host-checked)
+            const uint32_t *src = reinterpret_cast<const uint32_t *>(&tile[k * kLdsPitch + m16 * 16]);
+            const u32x4 v = {src[0], src[1], src[2], src[3]};
+            __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(out_t + oc * rows + orow));
+        }
+    }
+}
+
 static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 static int num_cus() {
@@ -886,4 +1045,68 @@ extern "C" int odl_fp8_cast_dynamic(const void *x, int src_dtype, int64_t rows, 
     }
     ODL_DISPATCH_SRC_FMT(launch_dynamic, x, rows, cols, parts, margin, out, out_t, dyn_out, fast, stream);
     return check_launch("odl_fp8_cast_dynamic");
+}
+
+// ------------------------------------------------------------------ rowwise recipe, fused passes
+static bool rowcol_fast(const void *x, int64_t rows, int64_t cols) {
+    return rows > 0 && cols > 0 && aligned16(x) && cols % 8 == 0 && rows % 16 == 0;
+}
+
+extern "C" int odl_fp8_amax_rowcol(const void *x, int src_dtype, int64_t rows, int64_t cols, float *amax_row, float *amax_col,
+                                   odl_stream_t stream_) {
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    if (rows < 0 || cols < 0) return set_error(ODL_ERR_ARG, "odl_fp8_amax_rowcol: negative shape");
+    if ((!x && rows * cols > 0) || (!amax_row && rows > 0) || (!amax_col && cols > 0)) return set_error(ODL_ERR_ARG, "odl_fp8_amax_rowcol: null pointer");
+    if (src_dtype != ODL_BF16 && src_dtype != ODL_F32) return set_error(ODL_ERR_ARG, "odl_fp8_amax_rowcol: src_dtype %d", src_dtype);
+    if (!rowcol_fast(x, rows, cols)) {
+        int rc = odl_fp8_amax(x, src_dtype, rows, cols, ODL_SCALE_ROW, amax_row, 0, stream_);
+        if (rc != ODL_OK) return rc;
+        return odl_fp8_amax(x, src_dtype, rows, cols, ODL_SCALE_COL, amax_col, 0, stream_);
+    }
+    hipLaunchKernelGGL(fill_f32_kernel, dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, stream, amax_row, rows, 0.0f);
+    hipLaunchKernelGGL(fill_f32_kernel, dim3((unsigned)((cols + 255) / 256)), dim3(256), 0, stream, amax_col, cols, 0.0f);
+    const int esz = src_dtype == ODL_BF16 ? 2 : 4;
+    const int cw = 32 * (16 / esz);
+    const int64_t col_blocks = (cols + cw - 1) / cw;
+    int64_t want_slabs = ((int64_t)num_cus() * 8 + col_blocks - 1) / col_blocks;
+    int64_t rpb = (rows + want_slabs - 1) / want_slabs;
+    rpb = ((rpb + 31) / 32) * 32;
+    if (rpb < 64) rpb = 64;
+    const int64_t slabs = (rows + rpb - 1) / rpb;
+    if (slabs > 65535) return set_error(ODL_ERR_SHAPE, "odl_fp8_amax_rowcol: too many row slabs");
+    if (src_dtype == ODL_BF16) hipLaunchKernelGGL((amax_rowcol_kernel<ODL_BF16>), dim3((unsigned)col_blocks, (unsigned)slabs), dim3(kThreads), 0, stream, x, rows, cols, (int)rpb, amax_row, amax_col);
+    else hipLaunchKernelGGL((amax_rowcol_kernel<ODL_F32>), dim3((unsigned)col_blocks, (unsigned)slabs), dim3(kThreads), 0, stream, x, rows, cols, (int)rpb, amax_row, amax_col);
+    return check_launch("odl_fp8_amax_rowcol");
+}
+
+template <int SRC, int FMT>
+static void launch_rowcol(const void *x, int64_t rows, int64_t cols, const float *amax_row, const float *amax_col, int margin,
+                          uint8_t *out, uint8_t *out_t, float *s_row, float *s_row_inv, float *s_col, float *s_col_inv, hipStream_t stream) {
+    const int64_t g = ((rows + kTileR - 1) / kTileR) * ((cols + kTileC - 1) / kTileC);
+    hipLaunchKernelGGL((cast_rowcol_kernel<SRC, FMT>), dim3((unsigned)g), dim3(kThreads), 0, stream, x, rows, cols, amax_row, amax_col,
+                       margin, out, out_t, s_row, s_row_inv, s_col, s_col_inv);
+}
+
+extern "C" int odl_fp8_cast_rowcol(const void *x, int src_dtype, int64_t rows, int64_t cols, const float *amax_row,
+                                   const float *amax_col, int fmt, int margin, uint8_t *out, uint8_t *out_t, float *s_row,
+                                   float *s_row_inv, float *s_col, float *s_col_inv, odl_stream_t stream_) {
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    if (rows < 0 || cols < 0) return set_error(ODL_ERR_ARG, "odl_fp8_cast_rowcol: negative shape");
+    if (src_dtype != ODL_BF16 && src_dtype != ODL_F32) return set_error(ODL_ERR_ARG, "odl_fp8_cast_rowcol: src_dtype %d", src_dtype);
+    if (fmt != ODL_FP8_E4M3 && fmt != ODL_FP8_E5M2) return set_error(ODL_ERR_ARG, "odl_fp8_cast_rowcol: fmt %d", fmt);
+    if ((rows > 0 && (!amax_row || !s_row || !s_row_inv)) || (cols > 0 && (!amax_col || !s_col || !s_col_inv)))
+        return set_error(ODL_ERR_ARG, "odl_fp8_cast_rowcol: null scale pointer");
+    if (rows * cols > 0 && (!x || !out || !out_t)) return set_error(ODL_ERR_ARG, "odl_fp8_cast_rowcol: null pointer");
+    const int64_t tiles = ((rows + kTileR - 1) / kTileR) * ((cols + kTileC - 1) / kTileC);
+    const bool fast = rowcol_fast(x, rows, cols) && aligned16(out_t) && (reinterpret_cast<uintptr_t>(out) & 7) == 0 && tiles <= 0x7fffffffLL;
+    if (!fast) {
+        // the step-by-step route: scales first, then the two casts
+        int rc = odl_fp8_scale_from_amax(amax_row, rows, fmt, margin, s_row, s_row_inv, stream_);
+        if (rc == ODL_OK) rc = odl_fp8_scale_from_amax(amax_col, cols, fmt, margin, s_col, s_col_inv, stream_);
+        if (rc == ODL_OK && rows * cols > 0) rc = odl_fp8_cast(x, src_dtype, rows, cols, s_row, ODL_SCALE_ROW, fmt, out, nullptr, stream_);
+        if (rc == ODL_OK && rows * cols > 0) rc = odl_fp8_cast_transpose(x, src_dtype, rows, cols, s_col, ODL_SCALE_COL, fmt, nullptr, out_t, nullptr, stream_);
+        return rc;
+    }
+    ODL_DISPATCH_SRC_FMT(launch_rowcol, x, rows, cols, amax_row, amax_col, margin, out, out_t, s_row, s_row_inv, s_col, s_col_inv, stream);
+    return check_launch("odl_fp8_cast_rowcol");
 }

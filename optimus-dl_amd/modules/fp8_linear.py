@@ -145,11 +145,13 @@ class _Fp8LinearFn(torch.autograd.Function):
         saved: dict[str, Any] = {}
 
         if pol.kind == "rowwise":
-            xq, sx_inv = _quantise_axis(x2d, pol.fmt_fwd, pol.margin, R, False)
-            wq, sw_inv = module._rowwise_weight(weight, pol, "row")
-            y = native.gemm_nt(xq, wq, pol.fmt_fwd, pol.fmt_fwd, sx_inv, sw_inv, bias=bias_f32, out_dtype=out_dtype)
             if need_wgrad and recipe.wgrad:
-                saved["xq_t"], saved["sx_inv_t"] = _quantise_axis(x2d, pol.fmt_fwd, pol.margin, C, True)
+                # both operands of x in two passes over it: rows for this GEMM, columns (transposed) for wgrad
+                xq, sx_inv, saved["xq_t"], saved["sx_inv_t"], _, _ = native.quantize_rowcol(x2d, pol.fmt_fwd, pol.margin)
+            else:
+                xq, sx_inv = _quantise_axis(x2d, pol.fmt_fwd, pol.margin, R, False)
+            wq, sw_inv = module._rowwise_weight(weight, pol, "row", both=need_dgrad)
+            y = native.gemm_nt(xq, wq, pol.fmt_fwd, pol.fmt_fwd, sx_inv, sw_inv, bias=bias_f32, out_dtype=out_dtype)
         else:
             if pol.kind == "delayed":
                 meta = module._meta(recipe, x2d.device, "fwd")
@@ -182,12 +184,16 @@ class _Fp8LinearFn(torch.autograd.Function):
         fp8_wgrad = ctx.need_wgrad and recipe.wgrad
 
         if pol.kind == "rowwise":
-            if ctx.need_dgrad:
+            if ctx.need_dgrad and fp8_wgrad:
+                gq, sg_inv, gq_t, sg_inv_t, _, _ = native.quantize_rowcol(dy2d, pol.fmt_bwd, pol.margin)
+            elif ctx.need_dgrad:
                 gq, sg_inv = _quantise_axis(dy2d, pol.fmt_bwd, pol.margin, R, False)
+            elif fp8_wgrad:
+                gq_t, sg_inv_t = _quantise_axis(dy2d, pol.fmt_bwd, pol.margin, C, True)
+            if ctx.need_dgrad:
                 wq_t, sw_inv_t = module._rowwise_weight(ctx.weight_ref, pol, "col")
                 dx = native.gemm_nt(gq, wq_t, pol.fmt_bwd, pol.fmt_fwd, sg_inv, sw_inv_t, out_dtype=ctx.x_dtype)
             if fp8_wgrad:
-                gq_t, sg_inv_t = _quantise_axis(dy2d, pol.fmt_bwd, pol.margin, C, True)
                 dw = native.gemm_nt(gq_t, saved["xq_t"], pol.fmt_bwd, pol.fmt_fwd, sg_inv_t, saved["sx_inv_t"],
                                     out_dtype=ctx.w_dtype)
         else:
@@ -284,13 +290,19 @@ class FP8Linear(nn.Linear):
             meta.arena.dirty = True
         return c.wq, c.wq_t, c.s_inv
 
-    def _rowwise_weight(self, weight: torch.Tensor, pol, axis: str):
-        """Rowwise recipe: W scaled per output channel (fwd) or per input channel, transposed (dgrad)."""
+    def _rowwise_weight(self, weight: torch.Tensor, pol, axis: str, both: bool = False):
+        """Rowwise recipe: W scaled per output channel (fwd) or per input channel, transposed (dgrad).
+        both: the other one will be asked for too (a backward follows): make them in one go."""
         key = (weight.data_ptr(), weight._version)
         hit = self._wcache_rowwise.get(axis)
         if hit is not None and hit[0] == key:
             return hit[1], hit[2]
         w2d = weight.detach()
+        if both:
+            q, s_inv, q_t, s_inv_t, _, _ = native.quantize_rowcol(w2d, pol.fmt_fwd, pol.margin)
+            self._wcache_rowwise["row"] = (key, q, s_inv)
+            self._wcache_rowwise["col"] = (key, q_t, s_inv_t)
+            return self._wcache_rowwise[axis][1], self._wcache_rowwise[axis][2]
         if axis == "row":
             q, s_inv = _quantise_axis(w2d, pol.fmt_fwd, pol.margin, R, False)
         else:

@@ -37,6 +37,8 @@ EXPORTS = (
     "odl_fp8_amax_scale",
     "odl_fp8_amax_parts",
     "odl_fp8_cast_dynamic",
+    "odl_fp8_amax_rowcol",
+    "odl_fp8_cast_rowcol",
     "odl_fp8_cast",
     "odl_fp8_cast_transpose",
     "odl_fp8_gemm_nt",
@@ -81,6 +83,8 @@ def load() -> ctypes.CDLL:
         L.odl_fp8_amax_scale.argtypes = [vp, i32, i64, i64, i32, i32, vp, vp, vp, vp, vp]
         L.odl_fp8_amax_parts.argtypes = [vp, i32, i64, i64, vp, vp]
         L.odl_fp8_cast_dynamic.argtypes = [vp, i32, i64, i64, vp, i32, i32, vp, vp, vp, vp]
+        L.odl_fp8_amax_rowcol.argtypes = [vp, i32, i64, i64, vp, vp, vp]
+        L.odl_fp8_cast_rowcol.argtypes = [vp, i32, i64, i64, vp, vp, i32, i32, vp, vp, vp, vp, vp, vp, vp]
         L.odl_fp8_cast.argtypes = [vp, i32, i64, i64, vp, i32, i32, vp, vp, vp]
         L.odl_fp8_cast_transpose.argtypes = [vp, i32, i64, i64, vp, i32, i32, vp, vp, vp, vp]
         L.odl_fp8_gemm_nt.argtypes = [vp, vp, i64, i64, i64, i32, i32, vp, i64, vp, i64, vp, i32, vp, i32, vp]
@@ -217,6 +221,30 @@ def quantize_dynamic(x: torch.Tensor, fmt: int, margin: int = 0, want_rowmajor: 
     """Current scaling of one tensor in two launches: partial maxima, then a cast that derives the
     scale itself.  -> (q or None, q_t or None, amax, scale, scale_inv)."""
     return cast_dynamic(x, amax_parts(x), fmt, margin, want_rowmajor, want_transposed)
+
+
+def quantize_rowcol(x: torch.Tensor, fmt: int, margin: int = 0):
+    """Rowwise recipe, both operands of one tensor in two passes over it:
+    -> (q [rows, cols] scaled per row, s_row_inv [rows], q_t [cols, rows] scaled per column, s_col_inv [cols],
+        amax_row, amax_col)."""
+    x = _as_2d(x)
+    rows, cols = x.shape
+    pr, pc = -(-rows // 4) * 4, -(-cols // 4) * 4            # every vector starts on a 16-byte boundary (the GEMM wants that)
+    buf = torch.empty(3 * (pr + pc), dtype=torch.float32, device=x.device)
+    a_row, a_col = buf[:rows], buf[pr:pr + cols]
+    o = pr + pc
+    s_row, s_col = buf[o:o + rows], buf[o + pr:o + pr + cols]
+    o = 2 * (pr + pc)
+    s_row_inv, s_col_inv = buf[o:o + rows], buf[o + pr:o + pr + cols]
+    q = torch.empty((rows, cols), dtype=torch.uint8, device=x.device)
+    q_t = torch.empty((cols, rows), dtype=torch.uint8, device=x.device)
+    L, stream = load(), _stream()
+    _check(L.odl_fp8_amax_rowcol(x.data_ptr(), _src_dtype(x), rows, cols, a_row.data_ptr(), a_col.data_ptr(), stream),
+           "odl_fp8_amax_rowcol")
+    _check(L.odl_fp8_cast_rowcol(x.data_ptr(), _src_dtype(x), rows, cols, a_row.data_ptr(), a_col.data_ptr(), fmt, margin,
+                                 q.data_ptr(), q_t.data_ptr(), s_row.data_ptr(), s_row_inv.data_ptr(), s_col.data_ptr(),
+                                 s_col_inv.data_ptr(), stream), "odl_fp8_cast_rowcol")
+    return q, s_row_inv, q_t, s_col_inv, a_row, a_col
 
 
 def scale_from_amax(amax_t: torch.Tensor, fmt: int, margin: int = 0):

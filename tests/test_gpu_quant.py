@@ -271,3 +271,32 @@ def test_bad_arguments_are_refused(N):
     with pytest.raises(N.NativeError):
         N._check(N.load().odl_fp8_cast(x.data_ptr(), 0, 16, 16, torch.ones(1, device="cuda").data_ptr(), 0, 9,
                                        x.data_ptr(), None, None), "bad fmt")
+
+
+@pytest.mark.parametrize("fmt", [O.E4M3, O.E5M2])
+def test_rowwise_pair_in_two_passes_equals_the_four_pass_route(N, fmt):
+    """amax_rowcol + cast_rowcol against amax(ROW), amax(COL), scale_from_amax, cast(ROW), cast_transpose(COL)
+    and the oracle: same amaxes, same inverse scales, same codes; outlier channels included."""
+    cases = [((1024, 512), torch.bfloat16), ((256, 128), torch.bfloat16), ((4096, 4096), torch.bfloat16),
+             ((144, 72), torch.float32), ((1000, 48), torch.bfloat16), ((33, 20), torch.bfloat16), ((16, 8), torch.float32)]
+    for i, (shape, dtype) in enumerate(cases):
+        x = seeded_bf16(shape, std=1.0, seed=120 + i)
+        x[:, 3 % shape[1]] *= 100.0                                   # an outlier channel
+        x[5 % shape[0]] *= 0.01                                       # and a quiet row
+        xd = x.to(dtype).cuda()
+        for margin in (0, 1):
+            q, s_row_inv, q_t, s_col_inv, a_row, a_col = N.quantize_rowcol(xd, fmt, margin)
+            ar, ac = N.amax(xd, O.SCALE_ROW), N.amax(xd, O.SCALE_COL)
+            assert_f32_bits_equal(a_row, ar, f"row amax {shape}")
+            assert_f32_bits_equal(a_col, ac, f"col amax {shape}")
+            assert_f32_bits_equal(a_row, O.t_amax(x, O.SCALE_ROW), f"row amax vs oracle {shape}")
+            assert_f32_bits_equal(a_col, O.t_amax(x, O.SCALE_COL), f"col amax vs oracle {shape}")
+            sr, sri = N.scale_from_amax(ar, fmt, margin)
+            sc, sci = N.scale_from_amax(ac, fmt, margin)
+            assert_f32_bits_equal(s_row_inv, sri, f"1/row scale {shape}")
+            assert_f32_bits_equal(s_col_inv, sci, f"1/col scale {shape}")
+            assert_bytes_equal(q, N.cast(xd, sr, fmt, O.SCALE_ROW), f"row-scaled codes {shape}")
+            assert_bytes_equal(q_t, N.cast_transpose(xd, sc, fmt, O.SCALE_COL, want_rowmajor=False)[1], f"col-scaled codes {shape}")
+            if margin == 0:
+                assert_bytes_equal(q, O.t_cast(x, sr.cpu(), fmt, O.SCALE_ROW), f"row-scaled codes vs oracle {shape}")
+                assert_bytes_equal(q_t, O.t_cast(x, sc.cpu(), fmt, O.SCALE_COL).t().contiguous(), f"col-scaled codes vs oracle {shape}")
