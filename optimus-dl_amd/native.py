@@ -182,20 +182,16 @@ def amax_scale(x: torch.Tensor, fmt: int, margin: int = 0):
 
 
 AMAX_PARTS = 512                       # ODL_FP8_AMAX_PARTS
-_parts: dict[tuple[int, int], torch.Tensor] = {}
 
 
 def amax_parts(x: torch.Tensor) -> torch.Tensor:
-    """AMAX_PARTS partial maxima of |x| (no atomics); input of :func:`cast_dynamic`.  The buffer is one
-    per (device, stream): it is consumed by the next launch on that stream."""
+    """AMAX_PARTS partial maxima of |x| (no atomics); input of :func:`cast_dynamic`.  The kernel
+    writes every entry, so the buffer is a fresh allocation per call: callers on several threads
+    cannot get each other's partials."""
     x = _as_2d(x)
     rows, cols = x.shape
-    stream = _stream()
-    key = (x.device.index if x.device.index is not None else torch.cuda.current_device(), stream)
-    parts = _parts.get(key)
-    if parts is None:
-        parts = _parts[key] = torch.zeros(AMAX_PARTS, dtype=torch.float32, device=x.device)
-    _check(load().odl_fp8_amax_parts(x.data_ptr(), _src_dtype(x), rows, cols, parts.data_ptr(), stream), "odl_fp8_amax_parts")
+    parts = torch.empty(AMAX_PARTS, dtype=torch.float32, device=x.device)
+    _check(load().odl_fp8_amax_parts(x.data_ptr(), _src_dtype(x), rows, cols, parts.data_ptr(), _stream()), "odl_fp8_amax_parts")
     return parts
 
 
