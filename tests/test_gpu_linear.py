@@ -393,3 +393,48 @@ def test_forward_backward_can_be_captured_in_a_graph_and_replayed(amp):
         torch.cuda.synchronize()
         for name, a, b in zip(("y", "dx", "dw"), got, want):
             assert torch.equal(a, b), f"replay {rep}: {name} differs from eager"
+
+
+@pytest.mark.parametrize("recipe_name,fmt,margin", [("tensorwise", "e5m2", 0), ("tensorwise", "hybrid", 2), ("rowwise", "e4m3", 1)])
+def test_other_formats_and_margins_match_the_oracle(amp, recipe_name, fmt, margin):
+    """Pure E5M2 (allowed for current scaling), a margin (scales divided by 2^margin) and rowwise E4M3 gradients."""
+    M, K, N = 256, 512, 384
+    x, w, dy = seeded_bf16((M, K), 1.0, 130), seeded_bf16((N, K), 0.02, 131), seeded_bf16((M, N), 1e-3, 132)
+    recipe = amp.create_fp8_recipe(recipe_name, fmt, margin=margin)
+    lin = make_linear(w)
+    y, dx, dw = run_step(lin, recipe, x, dy)
+    ff = O.E5M2 if fmt == "e5m2" else O.E4M3
+    fb = O.E4M3 if fmt == "e4m3" else O.E5M2
+    if recipe_name == "rowwise":
+        ref = O.linear_fwd_bwd(x, w, dy, ff, fb, rowwise=True) if margin == 0 else None
+    else:
+        scales = tuple(O.t_scale(O.t_amax(t), f, margin) for t, f in ((x, ff), (w, ff), (dy, fb)))
+        ref = O.linear_fwd_bwd(x, w, dy, ff, fb, scales=scales)
+    if ref is not None:
+        for name, got in (("y", y), ("dx", dx), ("dw", dw)):
+            err = max_rel_err(got, ref[name])
+            assert err <= TOL, f"{name}: {err}"
+    else:
+        # a margin only moves every scale by a power of two: codes stay far from the clamp, results match margin 0 closely
+        y0, dx0, dw0 = run_step(make_linear(w), amp.create_fp8_recipe(recipe_name, fmt), x, dy)
+        for name, a, b in (("y", y, y0), ("dx", dx, dx0), ("dw", dw, dw0)):
+            assert max_rel_err(a, b) <= 2e-2, name
+
+
+def test_nan_and_inf_inputs_do_not_poison_the_scales(amp):
+    """A NaN in the activation: its amax is NaN, the scale falls back to 1, the NaN element becomes the NaN code and
+    reaches exactly one output row; an Inf saturates.  The other rows stay finite."""
+    M, K, N = 128, 256, 128
+    recipe = amp.create_fp8_recipe("tensorwise", "hybrid")
+    lin = make_linear(seeded_bf16((N, K), 0.02, 140))
+    x = seeded_bf16((M, K), 1.0, 141)
+    x[7, 11] = float("nan")
+    with torch.no_grad(), recipe.autocast():
+        y = lin(x.cuda())
+    assert torch.isnan(y[7]).all()
+    keep = torch.ones(M, dtype=torch.bool); keep[7] = False
+    assert torch.isfinite(y[keep.cuda()].float()).all()
+    x[7, 11] = float("inf")
+    with torch.no_grad(), recipe.autocast():
+        y = lin(x.cuda())
+    assert torch.isfinite(y.float()).all()              # amax = Inf -> scale 1, the Inf element clamps to 448
