@@ -20,9 +20,6 @@ struct GemmArgs {
     int sa_vec, sb_vec;          // 0 = one value, 1 = one per row of A / B
     int out_dtype;               // bias, when present, is fp32
     int tiles_m, tiles_n;
-#ifdef ODL_GEMM_TRACE
-    unsigned long long *trace;   // development builds only: cycle stamps, [block][tile][4]
-#endif
 };
 
 __device__ __forceinline__ int swz(int row) { return (row ^ (row >> 3)) & 7; }

@@ -38,9 +38,9 @@
 //
 // Every vector-memory load of the K loop is issued from inline asm, and every wait
 // on the vector-memory counter is written out by hand: the counter retires in issue
-// order, which lets the loop wait for "all but the youngest n" operations (the L2
-// prefetches, or the previous tile's output stores), something the compiler's own
-// bookkeeping cannot express across the tile loop.  Instruction order inside a phase
+// order, which lets the loop wait for "all but the youngest n" operations (the previous
+// tile's output stores), something the compiler's own bookkeeping cannot express across
+// the tile loop.  Instruction order inside a phase
 // is pinned with sched_barrier so that each MFMA is followed by its share of LDS
 // reads and loads.
 #include "gemm_common.h"
@@ -55,11 +55,6 @@ constexpr int BM = 256, BN = 256, NW = 4, WM = 128, WN = 128, TM = 4, TN = 4;
 constexpr int REGION = 256 * 128;          // bytes of one operand in one stage
 constexpr int LOADS = 256 / 8 / NW;        // 1 KB direct-to-LDS loads per wave per operand per stage
 constexpr int GM = 8;
-#ifndef ODL_PIPE_PF
-#define ODL_PIPE_PF 0
-#endif
-constexpr int PF = ODL_PIPE_PF;            // L2 prefetch distance in K steps, 0 = none
-constexpr int NPF = PF > 0 ? 2 : 0;        // prefetch loads per wave per step
 constexpr int EPI_BYTES = 32 * (128 + 16); // one wave's epilogue slab: 32 rows x 128 bytes (+16 pad)
 static_assert(staged_epilogue_bytes<true, 2>() == EPI_BYTES && staged_epilogue_bytes<false, 1>() == EPI_BYTES, "slab size");
 
@@ -126,24 +121,7 @@ __global__ __launch_bounds__(256) void gemm_nt_pipe_kernel(const GemmArgs g) {
         for (int j = 0; j < 2 * LOADS; ++j) issue_one(sa, sb, kt, j);
     };
 
-    // ---- L2 prefetch.  About one line in six of a K step misses this XCD's L2 (the 32
-    // tiles running on an XCD share rows, but every row has to arrive once).  Each lane
-    // touches one 128-byte line of the step PF ahead with a load whose value is never
-    // used: 2 loads per wave per step pull all 512 lines of that step into L2 before the
-    // direct-to-LDS loads ask for them.  They are issued AFTER the DMA loads of the same
-    // phase, so "vmcnt(2)" still means "every DMA load has landed".  Steps past the end of
-    // this tile belong to the next tile of this block, if there is one.  The two
-    // destination registers stay allocated for the whole kernel (in-flight loads write them).
-    const int pf_off = (wave * 64 + lane) * (int)g.K;
     bool has_next = false;
-    int pfv_a = 0, pfv_b = 0;
-    auto prefetch = [&](int kt) {
-        if constexpr (PF == 0) return;
-        const bool nx = kt >= KT && has_next;
-        const int kp = (nx ? kt - KT : min(kt, KT - 1)) * 128;
-        asm volatile("buffer_load_dword %0, %1, %2, %3 offen" : "+v"(pfv_a) : "v"(pf_off), "s"(nx ? next_a : rsrc_a), "s"(kp));
-        asm volatile("buffer_load_dword %0, %1, %2, %3 offen" : "+v"(pfv_b) : "v"(pf_off), "s"(nx ? next_b : rsrc_b), "s"(kp));
-    };
 
     // ---- LDS -> registers.  chunk(t, h, e) = ((2*lg + e) ^ s0) ^ 4*(h ^ (t & 1))
     int ra[2][2], rb[2][2];                     // [e][h ^ (t & 1)] byte offsets inside a region (tile 0)
@@ -190,8 +168,8 @@ __global__ __launch_bounds__(256) void gemm_nt_pipe_kernel(const GemmArgs g) {
             else if (i < 8) b1[i - 4] = read_b(sb_cur, i - 4, 1);
             __builtin_amdgcn_sched_barrier(0);
         }
-        // my DMA for kt+1 has landed (the 2 younger prefetch loads may still be out), my LDS reads returned
-        __builtin_amdgcn_s_waitcnt(0x0070 | NPF);   // vmcnt(NPF) lgkmcnt(0)
+        // my DMA for kt+1 has landed, my LDS reads returned
+        __builtin_amdgcn_s_waitcnt(0x0070);     // vmcnt(0) lgkmcnt(0)
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
@@ -207,7 +185,6 @@ __global__ __launch_bounds__(256) void gemm_nt_pipe_kernel(const GemmArgs g) {
             }
             if constexpr (decltype(load_g)::value) {
                 issue_one(sa_cur, sb_cur, kt + 2, i);
-                if (i == 15) prefetch(kt + 2 + PF);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -223,17 +200,9 @@ __global__ __launch_bounds__(256) void gemm_nt_pipe_kernel(const GemmArgs g) {
     next_b = rsrc_b;
     issue(sA0, sB0, 0);
     issue(sA1, sB1, 1);
-    for (int k = 2; k < 2 + PF; ++k) prefetch(k);
     __builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0)
 
-#ifdef ODL_GEMM_TRACE
-#define ODL_STAMP(var) unsigned long long var; asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(var))
-    int tile_no = 0;
-#else
-#define ODL_STAMP(var)
-#endif
     while (true) {
-        ODL_STAMP(t0);
         const int64_t cm0 = m0, cn0 = n0;        // this tile's origin, kept for the epilogue
         const int next_pid = pid + stride;
         has_next = next_pid < pid_end;
@@ -245,7 +214,7 @@ __global__ __launch_bounds__(256) void gemm_nt_pipe_kernel(const GemmArgs g) {
 
         // Steps 0 and 1 of this tile have landed.  The vector-memory counter retires in issue
         // order, and behind those 32 loads this wave has issued at least 32 output stores of
-        // the previous tile and the L2 prefetches of the step in between ("at most 32
+        // the previous tile ("at most 32
         // outstanding" = the loads are in; for the first tile everything was awaited above),
         // while the stores of the previous tile may still be draining.  (The staged epilogue
         // issues 32 or 64 stores; the edge-tile path ends with a full wait.)
@@ -253,7 +222,6 @@ __global__ __launch_bounds__(256) void gemm_nt_pipe_kernel(const GemmArgs g) {
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        ODL_STAMP(t1);
 #pragma unroll
         for (int t = 0; t < TM; ++t) a0[t] = read_a(sA0, t, 0);
 #pragma unroll
@@ -273,10 +241,8 @@ __global__ __launch_bounds__(256) void gemm_nt_pipe_kernel(const GemmArgs g) {
         step(sA0, sB0, sA1, sB1, KT - 2, yes{}, no{});
         step(sA1, sB1, sA0, sB0, KT - 1, no{}, no{});
 
-        ODL_STAMP(t2);
         // Every wave passed the barrier of the last step after its final operand read, so
-        // the stages are free: request the next tile's first two steps before the epilogue
-        // (its first lines were pulled into L2 by the prefetches of the last steps).
+        // the stages are free: request the next tile's first two steps before the epilogue.
         if (has_next) {
             pid = next_pid;
             m0 = next_m0;
@@ -310,20 +276,8 @@ __global__ __launch_bounds__(256) void gemm_nt_pipe_kernel(const GemmArgs g) {
             // this path issues a data-dependent number of stores: do not count on them below
             __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
         }
-#ifdef ODL_GEMM_TRACE
-        {
-            ODL_STAMP(t3);
-            if (g.trace && wave == 0 && lane == 0 && tile_no < 8) {
-                unsigned long long *t = g.trace + ((size_t)blockIdx.x * 8 + tile_no) * 4;
-                t[0] = t0; t[1] = t1; t[2] = t2; t[3] = t3;
-            }
-            ++tile_no;
-        }
-#endif
         if (!has_next) break;
     }
-    __builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0): nothing may still be writing the prefetch registers
-    asm volatile("" ::"v"(pfv_a), "v"(pfv_b));
 }
 
 template <int FA, int FB>

@@ -37,14 +37,12 @@
 // Vector-memory counter: all loads and stores of the loop are inline asm and every
 // wait is written by hand.  The counter retires in issue order, so "vmcnt(n)" means
 // "everything but the youngest n operations has completed":
-//   step 0 : younger than the loads of step 1 are 2 prefetch loads and the 32 output
-//            stores of the folded epilogue           -> vmcnt(34)
-//   others : younger than the loads of step kt+1 are 2 prefetch loads -> vmcnt(2)
+//   step 0 : younger than the loads of step 1 are the 32 output stores of the folded
+//            epilogue                                 -> vmcnt(32)
+//   others : nothing is younger than the loads of step kt+1            -> vmcnt(0)
+// (An L2 prefetch, one lane per 128-byte line a few steps ahead, was tried and removed: the
+// scattered loads occupy the texture path that the direct-to-LDS loads need, 14 % of the K loop.)
 #include "gemm_common.h"
-
-#ifndef ODL_STREAM_PF
-#define ODL_STREAM_PF 0
-#endif
 
 namespace odl {
 
@@ -54,8 +52,6 @@ constexpr int BM = 256, BN = 256, NW = 4, WM = 128, WN = 128, TM = 4, TN = 4;
 constexpr int REGION = 256 * 128;          // bytes of one operand in one stage
 constexpr int LOADS = 256 / 8 / NW;        // 1 KB direct-to-LDS loads per wave per operand per stage
 constexpr int GM = 8;
-constexpr int PF = ODL_STREAM_PF;          // L2 prefetch distance in K steps, 0 = none
-constexpr int NPF = PF > 0 ? 2 : 0;        // prefetch loads per wave per step
 constexpr int PITCH = 128 + 8;             // slab row: 64 bf16 + 8 bytes, see phase_a_fold
 constexpr int SLAB = 32 * PITCH;           // one wave's epilogue slab
 
@@ -116,20 +112,6 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
 
     int m0 = 0, n0 = 0;
     v4i rsrc_a, rsrc_b, next_a, next_b;           // raw buffer descriptors (base, stride 0, bytes, format)
-
-    // ---- L2 prefetch: each lane touches one 128-byte line of the step PF ahead with a load
-    // whose value is never used; steps past the end of this tile belong to the next one.
-    // Issued after the DMA loads of the same phase, so they are the 2 youngest operations.
-    const int pf_off = (wave * 64 + lane) * (int)g.K;
-    int pfv_a = 0, pfv_b = 0;
-    auto prefetch = [&](int kt) {
-        if constexpr (PF == 0) return;
-        const bool nx = kt >= KT;
-        const int kp = (nx ? kt - KT : kt) * 128;
-        const v4i pa = nx ? next_a : rsrc_a, pb = nx ? next_b : rsrc_b;
-        asm volatile("buffer_load_dword %0, %1, %2, %3 offen" : "+v"(pfv_a) : "v"(pf_off), "s"(pa), "s"(kp));
-        asm volatile("buffer_load_dword %0, %1, %2, %3 offen" : "+v"(pfv_b) : "v"(pf_off), "s"(pb), "s"(kp));
-    };
 
     // ---- LDS -> registers.  chunk(t, h, e) = ((2*lg + e) ^ s0) ^ 4*(h ^ (t & 1))
     int ra[2][2], rb[2][2];                     // [e][h ^ (t & 1)] byte offsets inside a region (tile 0)
@@ -247,10 +229,9 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
         store_slab(back, c_voff, rsrc_c, c_soff0, n2, 3, 2);
         __builtin_amdgcn_sched_barrier(0);
     };
-    auto sync = [&](int simm16) {
-        // vmcnt(32 + NPF) or vmcnt(NPF), both with lgkmcnt(0)
-        if (simm16 == 0x8072) __builtin_amdgcn_s_waitcnt(0x8070 | NPF);
-        else __builtin_amdgcn_s_waitcnt(0x0070 | NPF);
+    auto sync = [&](bool after_fold) {
+        if (after_fold) __builtin_amdgcn_s_waitcnt(0x8070);          // vmcnt(32) lgkmcnt(0)
+        else __builtin_amdgcn_s_waitcnt(0x0070);                     // vmcnt(0)  lgkmcnt(0)
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
@@ -268,13 +249,12 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
             if (i < 4) a0[i] = read_a(sa_nxt, i, 0);
             else if (i < 8) b0[i - 4] = read_b(sb_nxt, i - 4, 0);
             issue_one(sa_cur, sb_cur, la, lb, koff, i);
-            if (i == 15) prefetch(kt + 2 + PF);
             __builtin_amdgcn_sched_barrier(0);
         }
     };
     auto step = [&](uint8_t *sa_cur, uint8_t *sb_cur, uint8_t *sa_nxt, uint8_t *sb_nxt, int kt) {
         phase_a(sa_cur, sb_cur);
-        sync(0x0072);
+        sync(false);
         phase_b(sa_cur, sb_cur, sa_nxt, sb_nxt, kt);
     };
 
@@ -288,7 +268,6 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
     for (int j = 0; j < 2 * LOADS; ++j) issue_one(sA0, sB0, rsrc_a, rsrc_b, 0, j);
 #pragma unroll
     for (int j = 0; j < 2 * LOADS; ++j) issue_one(sA1, sB1, rsrc_a, rsrc_b, 128, j);
-    for (int k = 2; k < 2 + PF; ++k) prefetch(k);
     __builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0)
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();
@@ -311,8 +290,8 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
 
         // ---- rest of step 0 (its phase A ran at the end of the previous trip), then steps 1 .. KT-1.
         // The first trip's step 0 and every drained tile's step 0 carry 32 stores (dropped ones
-        // count too), the first tile's none: vmcnt(34) is then simply satisfied earlier.
-        sync(0x8072);
+        // count too), the first tile's none: vmcnt(32) is then simply satisfied earlier.
+        sync(true);
         phase_b(sA0, sB0, sA1, sB1, 0);
         step(sA1, sB1, sA0, sB0, 1);
         for (int kt = 2; kt < KT - 2; kt += 2) {
@@ -334,8 +313,6 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
         phase_a_fold(sA0, sB0, rsrc_c);
         if (!has_next) break;
     }
-    __builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0): nothing may still be writing the prefetch registers
-    asm volatile("" ::"v"(pfv_a), "v"(pfv_b));
 }
 
 template <int FA, int FB>
