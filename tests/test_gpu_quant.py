@@ -300,3 +300,55 @@ def test_rowwise_pair_in_two_passes_equals_the_four_pass_route(N, fmt):
             if margin == 0:
                 assert_bytes_equal(q, O.t_cast(x, sr.cpu(), fmt, O.SCALE_ROW), f"row-scaled codes vs oracle {shape}")
                 assert_bytes_equal(q_t, O.t_cast(x, sc.cpu(), fmt, O.SCALE_COL).t().contiguous(), f"col-scaled codes vs oracle {shape}")
+
+
+def _golden(name):
+    import json
+    import os
+
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", name)) as fh:
+        return json.load(fh)
+
+
+def _f32(hexes):
+    return np.array([int(h, 16) for h in hexes], dtype=np.uint32).view(np.float32)
+
+
+@pytest.mark.parametrize("name,fmt", [("e4m3", O.E4M3), ("e5m2", O.E5M2)])
+def test_kernels_against_the_committed_golden_vectors(N, name, fmt):
+    """tests/golden/*.json: edge inputs (every tie between neighbouring codes, one ulp to either side,
+    overflow, NaN, Inf, subnormals), scale rule specials, a 20-step delayed-scaling sequence."""
+    doc = _golden("fp8_encode_edges.json")[name]
+    x = _f32(doc["x_f32_hex"])
+    want = torch.tensor(doc["code_saturating"], dtype=torch.uint8)
+    n = (len(x) // 16) * 16                                              # a multiple of 16 takes the vector kernel
+    one = torch.ones(1, device="cuda")
+    xs = torch.from_numpy(x.copy())
+    assert_bytes_equal(N.cast(xs[:n].reshape(1, n).cuda(), one, fmt).reshape(-1), want[:n], "golden edges, vector kernel")
+    assert_bytes_equal(N.cast(xs.reshape(1, -1).cuda(), one, fmt).reshape(-1), want, "golden edges, element kernel")
+    assert_bytes_equal(N.cast_transpose(xs[:n].reshape(n // 8, 8).cuda(), one, fmt)[1].t().reshape(-1), want[:n], "golden edges, cast+transpose")
+
+    doc = _golden("scale_from_amax.json")
+    amax = torch.from_numpy(_f32(doc["amax_f32_hex"]).copy()).cuda()
+    for case in doc["cases"]:
+        if case["fmt"] != name:
+            continue
+        s, si = N.scale_from_amax(amax, fmt, case["margin"])
+        assert_f32_bits_equal(s, torch.from_numpy(_f32(case["scale_f32_hex"]).copy()), f"golden scales margin {case['margin']}")
+        assert_f32_bits_equal(si, torch.from_numpy(_f32(case["scale_inv_f32_hex"]).copy()), "golden inverse scales")
+
+    doc = _golden("delayed_scaling_sequence.json")
+    H, amaxes = doc["H"], _f32(doc["amax_f32_hex"])
+    for case in doc["cases"]:
+        if case["fmt"] != name:
+            continue
+        hist = torch.zeros((H, 1), device="cuda")
+        scale, scale_inv = torch.ones(1, device="cuda"), torch.ones(1, device="cuda")
+        fmts = torch.tensor([fmt], dtype=torch.int32, device="cuda")
+        used, after = _f32(case["scale_used_f32_hex"]), _f32(case["scale_after_f32_hex"])
+        for t, a in enumerate(amaxes):
+            assert_f32_bits_equal(scale, torch.tensor([used[t]]), f"scale used at step {t}")
+            hist[0, 0] = max(hist[0, 0].item(), float(a))
+            N.delayed_update(hist, scale, scale_inv, fmts, 0, N.AMAX_MAX if case["algo"] == "max" else N.AMAX_MOST_RECENT)
+            assert_f32_bits_equal(scale, torch.tensor([after[t]]), f"scale after step {t}")
+        assert_f32_bits_equal(hist[:, 0], torch.from_numpy(_f32(case["final_history_f32_hex"]).copy()), "final history")
