@@ -180,6 +180,8 @@ def main() -> int:
     ap.add_argument("--gemm-variant", type=int, default=-1)
     ap.add_argument("--no-standalone", action="store_true",
                     help="skip the stand-alone measurements of the memory-bound kernels (keeps profiler traces to the steps)")
+    ap.add_argument("--standalone-only", action="store_true",
+                    help="run only the stand-alone measurements of the memory-bound kernels and print them (for profiling)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy (reference kernel for scaling FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -198,6 +200,9 @@ def main() -> int:
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         return 2
+    if args.standalone_only:
+        print(json.dumps({"hbm_kernels_standalone": standalone_hbm(torch, native)}))
+        return 0
     native.gemm_set_variant(args.gemm_variant)
     dev = "cuda"
     data = make_inputs(torch, device=dev)
