@@ -5,9 +5,21 @@ and ``apply(model, **kwargs) -> model``."""
 from __future__ import annotations
 
 from abc import ABC, abstractmethod
+from dataclasses import dataclass
 from typing import Any
 
 import torch.nn as nn
+
+from ...core.registry import RegistryConfig
+
+
+@dataclass
+class ModelTransformConfig(RegistryConfig):
+    """Options every model transform accepts (the role of
+    optimus_dl/modules/model_transforms/config.py:7-12).  It adds no field of its own:
+    ``_name`` selects the transform in the registry, and keys a subclass does not
+    declare are kept rather than rejected, so one YAML block can carry options for
+    transforms this build does not have."""
 
 
 class BaseModelTransform(ABC):

@@ -1,8 +1,7 @@
-from dataclasses import dataclass
+"""Import location kept for callers that take the transform options from here, as
+with optimus_dl/modules/model_transforms/config.py; the class is defined beside the
+transform base class."""
 
-from ...core.registry import RegistryConfig
+from .base import ModelTransformConfig
 
-
-@dataclass
-class ModelTransformConfig(RegistryConfig):
-    """Base config of model transforms (open: unknown keys are tolerated)."""
+__all__ = ["ModelTransformConfig"]
