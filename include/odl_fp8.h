@@ -45,7 +45,7 @@ enum odl_status {
     ODL_ERR_LAUNCH = 3    /* HIP reported an error at launch */
 };
 
-/* ABI version of this header (2); bumped when a signature changes or an entry point is added. */
+/* ABI version of this header (3); bumped when a signature changes or an entry point is added. */
 int odl_fp8_abi_version(void);
 
 /* Last error message of the calling host thread ("" if none). */
@@ -121,6 +121,45 @@ int odl_fp8_cast_rowcol(const void *x, int src_dtype, int64_t rows, int64_t cols
                         const float *amax_col, int fmt, int margin, uint8_t *out, uint8_t *out_t,
                         float *s_row, float *s_row_inv, float *s_col, float *s_col_inv,
                         odl_stream_t stream);
+
+/*
+ * Producers that hand the partial maxima of their OUTPUT to odl_fp8_cast_dynamic, so that the
+ * tensor they write is quantised without an amax pass of its own.  parts has
+ * ODL_FP8_AMAX_PARTS entries, as with odl_fp8_amax_parts.  All tensors are dense, bf16 unless
+ * said otherwise, 16-byte aligned; rows * cols (SwiGLU) or cols (RMSNorm) a multiple of 8.
+ *
+ * The arithmetic is fixed to the last bit (IEEE fp32 operations in a stated order, no hardware
+ * approximations), so a CPU restatement reproduces every output exactly:
+ *   sigmoid(g): t = clamp(-g, -80, 80); k = rint(t * 1.44269504f);
+ *               r = fma(k, -0.693359375f, t); r = fma(k, 2.12194440e-4f, r);
+ *               p = Horner by fma of {1.9875691500e-4f, 1.3981999507e-3f, 8.3334519073e-3f,
+ *                   4.1665795894e-2f, 1.6666665459e-1f, 5.0000001201e-1f} in r;
+ *               e = (fma(p, r * r, r) + 1) * 2^k; d = 1 + e;
+ *               y = bits(0x7EF311C7 - bits(d)); three times y = fma(y, fma(-d, y, 1), y);
+ *               result y, 0 where -g > 80, NaN for NaN.
+ *
+ * odl_fp8_swiglu_amax_parts: h = bf16( bf16(gate * sigmoid(gate)) * up ), the value of
+ *   silu(w1(x)) * w2(x) computed in bf16 (optimus_dl/modules/model/blocks/mlp.py:73-76);
+ *   parts = partial maxima of |h|.
+ * odl_fp8_swiglu_bwd_amax_parts: the gradients autograd derives for that expression in bf16:
+ *   d_up   = bf16( dh * bf16(gate * sigmoid(gate)) )
+ *   d_gate = bf16( bf16(dh * up) * (sig * fma(gate, 1 - sig, 1)) ),  sig = sigmoid(gate)
+ *   with the partial maxima of |d_gate| and |d_up|.
+ * odl_fp8_rmsnorm_amax_parts: y = bf16( (x * rstd) * weight ), rstd[r] = 1 / sqrt(sum_r / cols + eps)
+ *   (IEEE sqrt and division), the RMSNorm of optimus_dl/modules/model/blocks/layer_norms.py:86-119;
+ *   sum_r = sum of squares of row r in this order: lane l of 64 adds, by fma, the elements of the
+ *   8-element chunks l, l + 64, l + 128, ... in ascending order; the 64 lane sums are then combined
+ *   by the butterfly acc[l] += acc[l ^ off], off = 32, 16, 8, 4, 2, 1.  x is bf16 or fp32
+ *   (src_dtype), weight fp32[cols], 8 <= cols <= 8192.  rstd[rows] is kept for the backward.
+ */
+int odl_fp8_swiglu_amax_parts(const void *gate, const void *up, int64_t rows, int64_t cols, void *h,
+                              float *parts, odl_stream_t stream);
+int odl_fp8_swiglu_bwd_amax_parts(const void *dh, const void *gate, const void *up, int64_t rows,
+                                  int64_t cols, void *dgate, void *dup, float *parts_dgate,
+                                  float *parts_dup, odl_stream_t stream);
+int odl_fp8_rmsnorm_amax_parts(const void *x, int src_dtype, const float *weight, int64_t rows,
+                               int64_t cols, float eps, void *y, float *rstd, float *parts,
+                               odl_stream_t stream);
 
 /*
  * out[r,c] = fp8( clamp( fp32(x[r,c]) * s , +-max ) ), s = scale[0] | scale[r] | scale[c].

@@ -1,0 +1,296 @@
+// Producers of FP8 Linear inputs that also deliver the partial maxima of what they write, so
+// that the current-scaling quantisation of their output needs no amax pass of its own:
+//   SwiGLU forward   h  = silu(gate) * up                         (input of the down projection)
+//   SwiGLU backward  d_gate, d_up from d_h                         (grad_outputs of gate / up)
+//   RMSNorm forward  y  = x * rsqrt(mean(x^2) + eps) * weight      (input of q/k/v, gate/up)
+// All three are bound by HBM bandwidth; the arithmetic is written so that a plain-C restatement
+// gives the same bits: fused multiply-adds are spelled out, nothing is left to contraction, and
+// no hardware approximation (v_exp_f32, v_rcp_f32, v_rsq_f32) is used.
+#include "common.h"
+
+#pragma clang fp contract(off)
+
+namespace odl {
+
+constexpr int kFusedThreads = 1024;
+constexpr int kParts = ODL_FP8_AMAX_PARTS;
+
+// 1 / d for 1 <= d < 2^120: integer first guess, three Newton steps in fused multiply-adds.
+__device__ __forceinline__ float recip_newton(float d) {
+    float y = bits_to_float(0x7EF311C7u - float_to_bits(d));
+    y = __fmaf_rn(y, __fmaf_rn(-d, y, 1.0f), y);
+    y = __fmaf_rn(y, __fmaf_rn(-d, y, 1.0f), y);
+    y = __fmaf_rn(y, __fmaf_rn(-d, y, 1.0f), y);
+    return y;
+}
+
+// logistic function 1 / (1 + exp(-g)): range reduction by ln 2 in two pieces, degree-5 polynomial
+// for (exp(r) - 1 - r) / r^2, exact scaling by 2^k, reciprocal as above.  NaN in, NaN out.
+__device__ __forceinline__ float sigmoid_det(float g) {
+    float t = -g;
+    const bool zero = t > 80.0f;                 // exp(-g) beyond 2^115: the quotient is taken as 0
+    t = t < -80.0f ? -80.0f : t;
+    t = zero ? 80.0f : t;
+    t = (g != g) ? 0.0f : t;
+    const float kf = __builtin_rintf(__fmul_rn(t, 1.44269504f));
+    float r = __fmaf_rn(kf, -0.693359375f, t);
+    r = __fmaf_rn(kf, 2.12194440e-4f, r);
+    float p = 1.9875691500e-4f;
+    p = __fmaf_rn(p, r, 1.3981999507e-3f);
+    p = __fmaf_rn(p, r, 8.3334519073e-3f);
+    p = __fmaf_rn(p, r, 4.1665795894e-2f);
+    p = __fmaf_rn(p, r, 1.6666665459e-1f);
+    p = __fmaf_rn(p, r, 5.0000001201e-1f);
+    const float z = __fmul_rn(r, r);
+    const float y = __fadd_rn(__fmaf_rn(p, z, r), 1.0f);
+    const float e = __fmul_rn(y, bits_to_float((uint32_t)((int)kf + 127) << 23));
+    float s = recip_newton(__fadd_rn(1.0f, e));
+    s = zero ? 0.0f : s;
+    return (g != g) ? g : s;
+}
+
+// bf16 rounding of an fp32 value, returned widened again (what an eager bf16 op leaves behind)
+__device__ __forceinline__ float round_bf16(float f) { return bits_to_float(f32_to_bf16_bits(f) << 16); }
+
+// h = bf16( bf16(g * sigmoid(g)) * u ): the two roundings of silu(gate) * up evaluated in bf16
+__device__ __forceinline__ float swiglu_fwd_elem(float g, float u) {
+    const float s = round_bf16(__fmul_rn(g, sigmoid_det(g)));
+    return __fmul_rn(s, u);                      // the caller rounds to bf16
+}
+
+// d_up = bf16(dh * s), d_gate = bf16( bf16(dh * u) * sig * (1 + g * (1 - sig)) )
+__device__ __forceinline__ void swiglu_bwd_elem(float dh, float g, float u, float &dg, float &du) {
+    const float sig = sigmoid_det(g);
+    const float s = round_bf16(__fmul_rn(g, sig));
+    du = __fmul_rn(dh, s);
+    const float ds = round_bf16(__fmul_rn(dh, u));
+    const float dsilu = __fmul_rn(sig, __fmaf_rn(g, __fsub_rn(1.0f, sig), 1.0f));
+    dg = __fmul_rn(ds, dsilu);
+}
+
+__device__ __forceinline__ uint32_t pack2(float a, float b) { return f32_to_bf16_bits(a) | (f32_to_bf16_bits(b) << 16); }
+
+// ------------------------------------------------------------------ SwiGLU forward
+// n8 chunks of 8 bf16 (16 bytes) per operand; two chunks per lane in flight.  parts[blockIdx] =
+// this block's max |h|; entries no block owns are zeroed by block 0.
+__global__ __launch_bounds__(kFusedThreads) void swiglu_fwd_kernel(const u32x4 *__restrict__ gate, const u32x4 *__restrict__ up,
+                                                                    int64_t n8, u32x4 *__restrict__ h, float *__restrict__ parts) {
+    __shared__ uint32_t red[kFusedThreads / kWave];
+    const int64_t stride = (int64_t)gridDim.x * kFusedThreads;
+    uint32_t am = 0;
+    auto one = [&](const u32x4 gv, const u32x4 uv) -> u32x4 {
+        const uint32_t gw[4] = {gv.x, gv.y, gv.z, gv.w}, uw[4] = {uv.x, uv.y, uv.z, uv.w};
+        uint32_t o[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            o[q] = pack2(swiglu_fwd_elem(bf16_lo(gw[q]), bf16_lo(uw[q])), swiglu_fwd_elem(bf16_hi(gw[q]), bf16_hi(uw[q])));
+            am = max_u16x2(am, abs_bf16x2(o[q]));
+        }
+        return u32x4{o[0], o[1], o[2], o[3]};
+    };
+    int64_t i = (int64_t)blockIdx.x * kFusedThreads + threadIdx.x;
+    for (; i + stride < n8; i += 2 * stride) {
+        const u32x4 g0 = __builtin_nontemporal_load(gate + i), u0 = __builtin_nontemporal_load(up + i);
+        const u32x4 g1 = __builtin_nontemporal_load(gate + i + stride), u1 = __builtin_nontemporal_load(up + i + stride);
+        h[i] = one(g0, u0);
+        h[i + stride] = one(g1, u1);
+    }
+    for (; i < n8; i += stride) h[i] = one(__builtin_nontemporal_load(gate + i), __builtin_nontemporal_load(up + i));
+    am = block_max_u32(fold_u16x2_to_f32bits(am), red);
+    if (threadIdx.x == 0) parts[blockIdx.x] = bits_to_float(am);
+    if (blockIdx.x == 0)
+        for (int j = (int)gridDim.x + threadIdx.x; j < kParts; j += kFusedThreads) parts[j] = 0.0f;
+}
+
+// ----------------------------------------------------------------- SwiGLU backward
+__global__ __launch_bounds__(kFusedThreads) void swiglu_bwd_kernel(const u32x4 *__restrict__ dh, const u32x4 *__restrict__ gate,
+                                                                    const u32x4 *__restrict__ up, int64_t n8,
+                                                                    u32x4 *__restrict__ dgate, u32x4 *__restrict__ dup,
+                                                                    float *__restrict__ parts_dg, float *__restrict__ parts_du) {
+    __shared__ uint32_t red[kFusedThreads / kWave];
+    const int64_t stride = (int64_t)gridDim.x * kFusedThreads;
+    uint32_t am_g = 0, am_u = 0;
+    for (int64_t i = (int64_t)blockIdx.x * kFusedThreads + threadIdx.x; i < n8; i += stride) {
+        const u32x4 dv = __builtin_nontemporal_load(dh + i), gv = __builtin_nontemporal_load(gate + i),
+                    uv = __builtin_nontemporal_load(up + i);
+        const uint32_t dw[4] = {dv.x, dv.y, dv.z, dv.w}, gw[4] = {gv.x, gv.y, gv.z, gv.w}, uw[4] = {uv.x, uv.y, uv.z, uv.w};
+        uint32_t og[4], ou[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            float g0, u0, g1, u1;
+            swiglu_bwd_elem(bf16_lo(dw[q]), bf16_lo(gw[q]), bf16_lo(uw[q]), g0, u0);
+            swiglu_bwd_elem(bf16_hi(dw[q]), bf16_hi(gw[q]), bf16_hi(uw[q]), g1, u1);
+            og[q] = pack2(g0, g1);
+            ou[q] = pack2(u0, u1);
+            am_g = max_u16x2(am_g, abs_bf16x2(og[q]));
+            am_u = max_u16x2(am_u, abs_bf16x2(ou[q]));
+        }
+        dgate[i] = u32x4{og[0], og[1], og[2], og[3]};
+        dup[i] = u32x4{ou[0], ou[1], ou[2], ou[3]};
+    }
+    am_g = block_max_u32(fold_u16x2_to_f32bits(am_g), red);
+    __syncthreads();                               // red is reused
+    am_u = block_max_u32(fold_u16x2_to_f32bits(am_u), red);
+    if (threadIdx.x == 0) {
+        parts_dg[blockIdx.x] = bits_to_float(am_g);
+        parts_du[blockIdx.x] = bits_to_float(am_u);
+    }
+    if (blockIdx.x == 0)
+        for (int j = (int)gridDim.x + threadIdx.x; j < kParts; j += kFusedThreads) { parts_dg[j] = 0.0f; parts_du[j] = 0.0f; }
+}
+
+// ------------------------------------------------------------------- RMSNorm forward
+// One wavefront per row, rows handed out round-robin over all waves of the grid.  A lane holds
+// CPL chunks of 8 elements (chunk index = lane + 64 * j), so the row is read once.  Sum of
+// squares: per lane in element order by fused multiply-add, then the xor butterfly 32,16,..,1
+// (a + b is commutative, so every lane ends with the same bits).
+//   rstd = 1 / sqrt(sum / cols + eps)      (IEEE sqrt and division)
+//   y    = bf16( (x * rstd) * weight )     (two fp32 products, one rounding)
+constexpr int kRmsThreads = 256;
+
+template <int SRC>
+__device__ __forceinline__ void unpack8(const u32x4 *raw, float f[8]) {
+    if constexpr (SRC == ODL_BF16) {
+        const uint32_t w[4] = {raw[0].x, raw[0].y, raw[0].z, raw[0].w};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) { f[2 * q] = bf16_lo(w[q]); f[2 * q + 1] = bf16_hi(w[q]); }
+    } else {
+        f[0] = bits_to_float(raw[0].x); f[1] = bits_to_float(raw[0].y); f[2] = bits_to_float(raw[0].z); f[3] = bits_to_float(raw[0].w);
+        f[4] = bits_to_float(raw[1].x); f[5] = bits_to_float(raw[1].y); f[6] = bits_to_float(raw[1].z); f[7] = bits_to_float(raw[1].w);
+    }
+}
+
+template <int SRC, int CPL>
+__global__ __launch_bounds__(kRmsThreads) void rmsnorm_fwd_kernel(const void *__restrict__ x, const float *__restrict__ weight,
+                                                                   int64_t rows, int64_t cols, float eps,
+                                                                   uint16_t *__restrict__ y, float *__restrict__ rstd_out,
+                                                                   float *__restrict__ parts) {
+    __shared__ uint32_t red[kRmsThreads / kWave];
+    constexpr int VPC = SRC == ODL_BF16 ? 1 : 2;            // 16-byte vectors per chunk of 8 elements
+    const int lane = threadIdx.x % kWave;
+    const int64_t wave = (int64_t)blockIdx.x * (kRmsThreads / kWave) + threadIdx.x / kWave;
+    const int64_t nwave = (int64_t)gridDim.x * (kRmsThreads / kWave);
+    const int64_t nchunk = cols / 8;
+    uint32_t am = 0;
+    for (int64_t row = wave; row < rows; row += nwave) {
+        u32x4 raw[CPL][VPC];
+#pragma unroll
+        for (int j = 0; j < CPL; ++j) {
+            const int64_t c = lane + (int64_t)kWave * j;
+            const u32x4 *p = reinterpret_cast<const u32x4 *>(x) + (row * nchunk + c) * VPC;
+#pragma unroll
+            for (int h = 0; h < VPC; ++h) raw[j][h] = c < nchunk ? __builtin_nontemporal_load(p + h) : u32x4{0, 0, 0, 0};
+        }
+        float acc = 0.0f;
+#pragma unroll
+        for (int j = 0; j < CPL; ++j) {
+            float f[8];
+            unpack8<SRC>(raw[j], f);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc = __fmaf_rn(f[e], f[e], acc);
+        }
+#pragma unroll
+        for (int off = kWave / 2; off > 0; off >>= 1) acc = __fadd_rn(acc, __shfl_xor(acc, off, kWave));
+        const float mean = __fdiv_rn(acc, (float)cols);
+        const float rstd = __fdiv_rn(1.0f, __builtin_sqrtf(__fadd_rn(mean, eps)));
+        if (lane == 0) rstd_out[row] = rstd;
+#pragma unroll
+        for (int j = 0; j < CPL; ++j) {
+            const int64_t c = lane + (int64_t)kWave * j;
+            if (c < nchunk) {
+                float f[8];
+                unpack8<SRC>(raw[j], f);
+                const float4 w0 = *reinterpret_cast<const float4 *>(weight + c * 8), w1 = *reinterpret_cast<const float4 *>(weight + c * 8 + 4);
+                const float w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+                uint32_t o[4];
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    o[q] = pack2(__fmul_rn(__fmul_rn(f[2 * q], rstd), w[2 * q]), __fmul_rn(__fmul_rn(f[2 * q + 1], rstd), w[2 * q + 1]));
+                    am = max_u16x2(am, abs_bf16x2(o[q]));
+                }
+                reinterpret_cast<u32x4 *>(y)[row * nchunk + c] = u32x4{o[0], o[1], o[2], o[3]};
+            }
+        }
+    }
+    am = block_max_u32(fold_u16x2_to_f32bits(am), red);
+    if (threadIdx.x == 0) parts[blockIdx.x] = bits_to_float(am);
+    if (blockIdx.x == 0)
+        for (int j = (int)gridDim.x + threadIdx.x; j < kParts; j += kRmsThreads) parts[j] = 0.0f;
+}
+
+static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+// at most two fat blocks per CU, and never more blocks than there are partial maxima
+static int grid_cap() {
+    static int cap = 0;
+    if (cap == 0) {
+        int dev = 0, cus = 256;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0)
+            cus = prop.multiProcessorCount;
+        cap = cus * 2 < kParts ? cus * 2 : kParts;
+    }
+    return cap;
+}
+
+}  // namespace odl
+
+using namespace odl;
+
+extern "C" int odl_fp8_swiglu_amax_parts(const void *gate, const void *up, int64_t rows, int64_t cols, void *h, float *parts,
+                                         odl_stream_t stream_) {
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    if (rows < 0 || cols < 0) return set_error(ODL_ERR_ARG, "odl_fp8_swiglu_amax_parts: negative shape");
+    const int64_t n = rows * cols;
+    if (!parts || (n > 0 && (!gate || !up || !h))) return set_error(ODL_ERR_ARG, "odl_fp8_swiglu_amax_parts: null pointer");
+    if (n % 8 != 0 || !aligned16(gate) || !aligned16(up) || !aligned16(h))
+        return set_error(ODL_ERR_SHAPE, "odl_fp8_swiglu_amax_parts: rows*cols must be a multiple of 8 and the pointers 16-byte aligned");
+    const int64_t n8 = n / 8;
+    int64_t g = (n8 + 2 * kFusedThreads - 1) / (2 * kFusedThreads);
+    g = g < 1 ? 1 : (g < grid_cap() ? g : grid_cap());
+    hipLaunchKernelGGL(swiglu_fwd_kernel, dim3((unsigned)g), dim3(kFusedThreads), 0, stream, reinterpret_cast<const u32x4 *>(gate),
+                       reinterpret_cast<const u32x4 *>(up), n8, reinterpret_cast<u32x4 *>(h), parts);
+    return check_launch("odl_fp8_swiglu_amax_parts");
+}
+
+extern "C" int odl_fp8_swiglu_bwd_amax_parts(const void *dh, const void *gate, const void *up, int64_t rows, int64_t cols,
+                                             void *dgate, void *dup, float *parts_dgate, float *parts_dup, odl_stream_t stream_) {
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    if (rows < 0 || cols < 0) return set_error(ODL_ERR_ARG, "odl_fp8_swiglu_bwd_amax_parts: negative shape");
+    const int64_t n = rows * cols;
+    if (!parts_dgate || !parts_dup || (n > 0 && (!dh || !gate || !up || !dgate || !dup)))
+        return set_error(ODL_ERR_ARG, "odl_fp8_swiglu_bwd_amax_parts: null pointer");
+    if (n % 8 != 0 || !aligned16(dh) || !aligned16(gate) || !aligned16(up) || !aligned16(dgate) || !aligned16(dup))
+        return set_error(ODL_ERR_SHAPE, "odl_fp8_swiglu_bwd_amax_parts: rows*cols must be a multiple of 8 and the pointers 16-byte aligned");
+    const int64_t n8 = n / 8;
+    int64_t g = (n8 + kFusedThreads - 1) / kFusedThreads;
+    g = g < 1 ? 1 : (g < grid_cap() ? g : grid_cap());
+    hipLaunchKernelGGL(swiglu_bwd_kernel, dim3((unsigned)g), dim3(kFusedThreads), 0, stream, reinterpret_cast<const u32x4 *>(dh),
+                       reinterpret_cast<const u32x4 *>(gate), reinterpret_cast<const u32x4 *>(up), n8,
+                       reinterpret_cast<u32x4 *>(dgate), reinterpret_cast<u32x4 *>(dup), parts_dgate, parts_dup);
+    return check_launch("odl_fp8_swiglu_bwd_amax_parts");
+}
+
+extern "C" int odl_fp8_rmsnorm_amax_parts(const void *x, int src_dtype, const float *weight, int64_t rows, int64_t cols, float eps,
+                                          void *y, float *rstd, float *parts, odl_stream_t stream_) {
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    if (rows < 0 || cols < 0) return set_error(ODL_ERR_ARG, "odl_fp8_rmsnorm_amax_parts: negative shape");
+    if (src_dtype != ODL_BF16 && src_dtype != ODL_F32) return set_error(ODL_ERR_ARG, "odl_fp8_rmsnorm_amax_parts: src_dtype %d", src_dtype);
+    if (!parts || (rows > 0 && !rstd) || (rows * cols > 0 && (!x || !weight || !y)))
+        return set_error(ODL_ERR_ARG, "odl_fp8_rmsnorm_amax_parts: null pointer");
+    if (cols < 8 || cols % 8 != 0 || cols > 8192 || !aligned16(x) || !aligned16(y) || !aligned16(weight))
+        return set_error(ODL_ERR_SHAPE, "odl_fp8_rmsnorm_amax_parts: cols must be a multiple of 8 in [8, 8192] and the pointers 16-byte aligned");
+    const int rows_per_block = kRmsThreads / kWave;
+    int64_t g = (rows + rows_per_block - 1) / rows_per_block;
+    g = g < 1 ? 1 : (g < grid_cap() ? g : grid_cap());
+    const int64_t cpl = (cols / 8 + kWave - 1) / kWave;
+#define ODL_RMS(SRC, CPL) hipLaunchKernelGGL((rmsnorm_fwd_kernel<SRC, CPL>), dim3((unsigned)g), dim3(kRmsThreads), 0, stream, x, weight, rows, cols, eps, reinterpret_cast<uint16_t *>(y), rstd, parts)
+#define ODL_RMS_SRC(CPL) do { if (src_dtype == ODL_BF16) ODL_RMS(ODL_BF16, CPL); else ODL_RMS(ODL_F32, CPL); } while (0)
+    if (cpl <= 2) ODL_RMS_SRC(2);
+    else if (cpl <= 4) ODL_RMS_SRC(4);
+    else if (cpl <= 8) ODL_RMS_SRC(8);
+    else ODL_RMS_SRC(16);
+#undef ODL_RMS_SRC
+#undef ODL_RMS
+    return check_launch("odl_fp8_rmsnorm_amax_parts");
+}

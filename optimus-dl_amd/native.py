@@ -23,7 +23,7 @@ DT_BF16, DT_F32 = 0, 1
 AMAX_MAX, AMAX_MOST_RECENT = 0, 1
 FP8_MAX = {E4M3: 448.0, E5M2: 57344.0}
 TORCH_FP8 = {E4M3: torch.float8_e4m3fn, E5M2: torch.float8_e5m2}
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # ODL_FP8_LIB names another build of the same library (e.g. one made for an experiment)
@@ -37,6 +37,9 @@ EXPORTS = (
     "odl_fp8_amax_scale",
     "odl_fp8_amax_parts",
     "odl_fp8_cast_dynamic",
+    "odl_fp8_swiglu_amax_parts",
+    "odl_fp8_swiglu_bwd_amax_parts",
+    "odl_fp8_rmsnorm_amax_parts",
     "odl_fp8_amax_rowcol",
     "odl_fp8_cast_rowcol",
     "odl_fp8_cast",
@@ -83,6 +86,9 @@ def load() -> ctypes.CDLL:
         L.odl_fp8_amax_scale.argtypes = [vp, i32, i64, i64, i32, i32, vp, vp, vp, vp, vp]
         L.odl_fp8_amax_parts.argtypes = [vp, i32, i64, i64, vp, vp]
         L.odl_fp8_cast_dynamic.argtypes = [vp, i32, i64, i64, vp, i32, i32, vp, vp, vp, vp]
+        L.odl_fp8_swiglu_amax_parts.argtypes = [vp, vp, i64, i64, vp, vp, vp]
+        L.odl_fp8_swiglu_bwd_amax_parts.argtypes = [vp, vp, vp, i64, i64, vp, vp, vp, vp, vp]
+        L.odl_fp8_rmsnorm_amax_parts.argtypes = [vp, i32, vp, i64, i64, ctypes.c_float, vp, vp, vp, vp]
         L.odl_fp8_amax_rowcol.argtypes = [vp, i32, i64, i64, vp, vp, vp]
         L.odl_fp8_cast_rowcol.argtypes = [vp, i32, i64, i64, vp, vp, i32, i32, vp, vp, vp, vp, vp, vp, vp]
         L.odl_fp8_cast.argtypes = [vp, i32, i64, i64, vp, i32, i32, vp, vp, vp]
@@ -217,6 +223,75 @@ def quantize_dynamic(x: torch.Tensor, fmt: int, margin: int = 0, want_rowmajor: 
     """Current scaling of one tensor in two launches: partial maxima, then a cast that derives the
     scale itself.  -> (q or None, q_t or None, amax, scale, scale_inv)."""
     return cast_dynamic(x, amax_parts(x), fmt, margin, want_rowmajor, want_transposed)
+
+
+def _bf16_dense(t: torch.Tensor, what: str) -> torch.Tensor:
+    if not t.is_cuda:
+        raise NativeError(f"{what}: the kernels run on the GPU only; got a tensor on {t.device}")
+    if t.dtype != torch.bfloat16:
+        raise NativeError(f"{what}: bf16 expected, got {t.dtype}")
+    if not t.is_contiguous():
+        t = t.contiguous()
+    if t.data_ptr() % 16:
+        t = t.clone(memory_format=torch.contiguous_format)
+    return t
+
+
+def swiglu_amax_parts(gate: torch.Tensor, up: torch.Tensor):
+    """h = silu(gate) * up as eager bf16 arithmetic leaves it, and the partial maxima of |h| for
+    :func:`cast_dynamic`.  -> (h, parts)."""
+    gate, up = _bf16_dense(gate, "swiglu gate"), _bf16_dense(up, "swiglu up")
+    if gate.shape != up.shape:
+        raise NativeError(f"swiglu: gate {tuple(gate.shape)} and up {tuple(up.shape)} differ")
+    cols = gate.shape[-1] if gate.dim() else 1
+    rows = gate.numel() // max(cols, 1)
+    h = torch.empty_like(gate)
+    parts = torch.empty(AMAX_PARTS, dtype=torch.float32, device=gate.device)
+    _check(load().odl_fp8_swiglu_amax_parts(gate.data_ptr(), up.data_ptr(), rows, cols, h.data_ptr(), parts.data_ptr(), _stream()),
+           "odl_fp8_swiglu_amax_parts")
+    return h, parts
+
+
+def swiglu_bwd_amax_parts(dh: torch.Tensor, gate: torch.Tensor, up: torch.Tensor):
+    """Gradients of silu(gate) * up for grad_output dh, with their partial maxima.
+    -> (d_gate, d_up, parts_d_gate, parts_d_up)."""
+    dh, gate, up = _bf16_dense(dh, "swiglu dh"), _bf16_dense(gate, "swiglu gate"), _bf16_dense(up, "swiglu up")
+    if not (dh.shape == gate.shape == up.shape):
+        raise NativeError(f"swiglu backward: shapes {tuple(dh.shape)}, {tuple(gate.shape)}, {tuple(up.shape)} differ")
+    cols = gate.shape[-1] if gate.dim() else 1
+    rows = gate.numel() // max(cols, 1)
+    dgate, dup = torch.empty_like(gate), torch.empty_like(up)
+    parts = torch.empty(2 * AMAX_PARTS, dtype=torch.float32, device=gate.device)
+    pg, pu = parts[:AMAX_PARTS], parts[AMAX_PARTS:]
+    _check(load().odl_fp8_swiglu_bwd_amax_parts(dh.data_ptr(), gate.data_ptr(), up.data_ptr(), rows, cols, dgate.data_ptr(),
+                                                dup.data_ptr(), pg.data_ptr(), pu.data_ptr(), _stream()),
+           "odl_fp8_swiglu_bwd_amax_parts")
+    return dgate, dup, pg, pu
+
+
+def rmsnorm_amax_parts(x: torch.Tensor, weight: torch.Tensor, eps: float):
+    """y = bf16(x * rsqrt(mean(x^2, -1) + eps) * weight) over the last axis, the per-row
+    1/rms, and the partial maxima of |y|.  x: bf16 or fp32.  -> (y bf16, rstd fp32, parts)."""
+    if not x.is_cuda:
+        raise NativeError(f"rmsnorm: the kernels run on the GPU only; got a tensor on {x.device}")
+    src = _src_dtype(x)
+    if not x.is_contiguous():
+        x = x.contiguous()
+    if x.data_ptr() % 16:
+        x = x.clone(memory_format=torch.contiguous_format)
+    cols = x.shape[-1]
+    rows = x.numel() // max(cols, 1)
+    w = weight.detach()
+    if w.dtype != torch.float32 or not w.is_contiguous() or w.data_ptr() % 16:
+        w = w.float().contiguous().clone()
+    if w.numel() != cols or w.device != x.device:
+        raise NativeError(f"rmsnorm: weight has {w.numel()} elements on {w.device}, rows have {cols} on {x.device}")
+    y = torch.empty(x.shape, dtype=torch.bfloat16, device=x.device)
+    rstd = torch.empty(x.shape[:-1], dtype=torch.float32, device=x.device)
+    parts = torch.empty(AMAX_PARTS, dtype=torch.float32, device=x.device)
+    _check(load().odl_fp8_rmsnorm_amax_parts(x.data_ptr(), src, w.data_ptr(), rows, cols, float(eps), y.data_ptr(), rstd.data_ptr(),
+                                             parts.data_ptr(), _stream()), "odl_fp8_rmsnorm_amax_parts")
+    return y, rstd, parts
 
 
 def quantize_rowcol(x: torch.Tensor, fmt: int, margin: int = 0):

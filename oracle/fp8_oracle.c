@@ -258,3 +258,101 @@ ORACLE_API void oracle_delayed_update(float *history, int64_t H, int64_t R, floa
         scale_inv[r] = oracle_scale_inv(scale[r]);
     }
 }
+
+/* ------------------------------------------------------------------------------------------
+ * Producers either side of the Linear: SwiGLU (optimus_dl/modules/model/blocks/mlp.py:73-76,
+ * `silu(w1(x)) * w2(x)` evaluated in bf16 under autocast, and the gradients autograd derives
+ * for it) and RMSNorm (optimus_dl/modules/model/blocks/layer_norms.py:86-119).  The reference
+ * leaves both to PyTorch; the kernels fix the arithmetic to the last bit (documented in the C
+ * header of the library) and this is the same sequence of IEEE fp32 operations in plain C.
+ * Pinned in tests/test_oracle_fused.py: sigmoid against float64 over ALL bf16 inputs,
+ * SwiGLU forward / backward against torch's bf16 silu, multiplication and autograd on the CPU
+ * (equal up to one bf16 unit in a small fraction of elements, since torch's exp differs in the
+ * last fp32 bits), RMSNorm against the float64 closed form and against torch in fp32.
+ * Built with -ffp-contract=off: every fused multiply-add below is an explicit fmaf().
+ */
+static float recip_newton(float d) {
+    float y = bits_f32(0x7EF311C7u - f32_bits(d));
+    y = fmaf(y, fmaf(-d, y, 1.0f), y);
+    y = fmaf(y, fmaf(-d, y, 1.0f), y);
+    y = fmaf(y, fmaf(-d, y, 1.0f), y);
+    return y;
+}
+
+ORACLE_API float oracle_sigmoid(float g) {
+    if (g != g) return g;
+    float t = -g;
+    int zero = t > 80.0f;
+    if (t < -80.0f) t = -80.0f;
+    if (zero) t = 80.0f;
+    float kf = rintf(t * 1.44269504f);                 /* ties to even (default rounding mode) */
+    float r = fmaf(kf, -0.693359375f, t);
+    r = fmaf(kf, 2.12194440e-4f, r);
+    float p = 1.9875691500e-4f;
+    p = fmaf(p, r, 1.3981999507e-3f);
+    p = fmaf(p, r, 8.3334519073e-3f);
+    p = fmaf(p, r, 4.1665795894e-2f);
+    p = fmaf(p, r, 1.6666665459e-1f);
+    p = fmaf(p, r, 5.0000001201e-1f);
+    float z = r * r;
+    float y = fmaf(p, z, r) + 1.0f;
+    float e = y * bits_f32((uint32_t)((int)kf + 127) << 23);
+    float s = recip_newton(1.0f + e);
+    return zero ? 0.0f : s;
+}
+
+static inline float round_bf16(float f) { return bf16_to_f32(f32_to_bf16(f)); }
+
+ORACLE_API void oracle_swiglu_fwd(const uint16_t *gate, const uint16_t *up, int64_t n, uint16_t *h) {
+    for (int64_t i = 0; i < n; ++i) {
+        float g = bf16_to_f32(gate[i]), u = bf16_to_f32(up[i]);
+        float s = round_bf16(g * oracle_sigmoid(g));
+        h[i] = f32_to_bf16(s * u);
+    }
+}
+
+ORACLE_API void oracle_swiglu_bwd(const uint16_t *dh, const uint16_t *gate, const uint16_t *up, int64_t n,
+                                  uint16_t *dgate, uint16_t *dup) {
+    for (int64_t i = 0; i < n; ++i) {
+        float d = bf16_to_f32(dh[i]), g = bf16_to_f32(gate[i]), u = bf16_to_f32(up[i]);
+        float sig = oracle_sigmoid(g);
+        float s = round_bf16(g * sig);
+        dup[i] = f32_to_bf16(d * s);
+        float ds = round_bf16(d * u);
+        float dsilu = sig * fmaf(g, 1.0f - sig, 1.0f);
+        dgate[i] = f32_to_bf16(ds * dsilu);
+    }
+}
+
+/* x: bf16 (src 0) or fp32 (src 1), [rows, cols], cols % 8 == 0; the summation order is the one the
+ * C header of the library states (64 lanes, 8-element chunks dealt round-robin, xor butterfly). */
+ORACLE_API void oracle_rmsnorm(const void *x, int src, const float *weight, int64_t rows, int64_t cols, float eps,
+                               uint16_t *y, float *rstd_out) {
+    const int64_t nchunk = cols / 8;
+    for (int64_t r = 0; r < rows; ++r) {
+        float acc[64];
+        for (int l = 0; l < 64; ++l) {
+            float a = 0.0f;
+            for (int64_t c = l; c < nchunk; c += 64)
+                for (int e = 0; e < 8; ++e) {
+                    int64_t idx = r * cols + c * 8 + e;
+                    float v = src == 0 ? bf16_to_f32(((const uint16_t *)x)[idx]) : ((const float *)x)[idx];
+                    a = fmaf(v, v, a);
+                }
+            acc[l] = a;
+        }
+        for (int off = 32; off > 0; off >>= 1) {
+            float nxt[64];
+            for (int l = 0; l < 64; ++l) nxt[l] = acc[l] + acc[l ^ off];
+            memcpy(acc, nxt, sizeof(acc));
+        }
+        float mean = acc[0] / (float)cols;
+        float rstd = 1.0f / sqrtf(mean + eps);
+        rstd_out[r] = rstd;
+        for (int64_t c = 0; c < cols; ++c) {
+            int64_t idx = r * cols + c;
+            float v = src == 0 ? bf16_to_f32(((const uint16_t *)x)[idx]) : ((const float *)x)[idx];
+            y[idx] = f32_to_bf16((v * rstd) * weight[c]);
+        }
+    }
+}

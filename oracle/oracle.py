@@ -65,6 +65,11 @@ def lib() -> ctypes.CDLL:
         L.oracle_cast_transpose_bf16.argtypes = [vp, i64, i64, vp, i32, i32, vp, vp]
         L.oracle_gemm_nt.argtypes = [vp, vp, i64, i64, i64, i32, i32, vp, i64, vp, i64, vp, vp]
         L.oracle_delayed_update.argtypes = [vp, i64, i64, vp, vp, vp, i32, i32]
+        L.oracle_sigmoid.argtypes = [f32]
+        L.oracle_sigmoid.restype = f32
+        L.oracle_swiglu_fwd.argtypes = [vp, vp, i64, vp]
+        L.oracle_swiglu_bwd.argtypes = [vp, vp, vp, i64, vp, vp]
+        L.oracle_rmsnorm.argtypes = [vp, i32, vp, i64, i64, f32, vp, vp]
         _lib = L
     return _lib
 
@@ -161,6 +166,44 @@ def c_delayed_update(history: np.ndarray, scale: np.ndarray, scale_inv: np.ndarr
 
 
 # ----------------------------------------------------------------- torch family
+def _from_bf16_bits(bits: np.ndarray, shape) -> torch.Tensor:
+    return torch.from_numpy(np.ascontiguousarray(bits).view(np.int16).copy()).view(torch.bfloat16).reshape(shape)
+
+
+def c_sigmoid(g: float) -> float:
+    return float(lib().oracle_sigmoid(float(g)))
+
+
+def c_swiglu_fwd(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """h = silu(gate) * up with the roundings of eager bf16 arithmetic (bf16 tensors in and out)."""
+    g, u = _bf16_bits(gate), _bf16_bits(up)
+    h = np.empty_like(g)
+    lib().oracle_swiglu_fwd(_p(g), _p(u), g.size, _p(h))
+    return _from_bf16_bits(h, gate.shape)
+
+
+def c_swiglu_bwd(dh: torch.Tensor, gate: torch.Tensor, up: torch.Tensor):
+    d, g, u = _bf16_bits(dh), _bf16_bits(gate), _bf16_bits(up)
+    dg, du = np.empty_like(g), np.empty_like(g)
+    lib().oracle_swiglu_bwd(_p(d), _p(g), _p(u), g.size, _p(dg), _p(du))
+    return _from_bf16_bits(dg, gate.shape), _from_bf16_bits(du, gate.shape)
+
+
+def c_rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float):
+    """-> (y bf16, rstd fp32[rows]); x bf16 or fp32, normalised over the last axis."""
+    cols = x.shape[-1]
+    rows = x.numel() // cols
+    if x.dtype == torch.bfloat16:
+        xs, src = _bf16_bits(x), 0
+    else:
+        xs, src = np.ascontiguousarray(x.detach().float().cpu().numpy()).reshape(-1), 1
+    w = np.ascontiguousarray(weight.detach().float().cpu().numpy())
+    y = np.empty(rows * cols, dtype=np.uint16)
+    rstd = np.empty(rows, dtype=np.float32)
+    lib().oracle_rmsnorm(_p(xs), src, _p(w), rows, cols, float(eps), _p(y), _p(rstd))
+    return _from_bf16_bits(y, x.shape), torch.from_numpy(rstd).reshape(x.shape[:-1])
+
+
 def t_amax(x: torch.Tensor, mode: int = SCALE_TENSOR) -> torch.Tensor:
     a = x.abs()
     if mode == SCALE_TENSOR:

@@ -1,0 +1,168 @@
+"""GPU parity: SwiGLU forward / backward and RMSNorm producers vs the CPU oracle, bit for bit,
+through the C ABI; their partial maxima fed to the dynamic cast give the codes the plain
+two-launch quantisation gives."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as O
+from tests.helpers import assert_bytes_equal, assert_f32_bits_equal, seeded_bf16
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def N():
+    from optimus_dl_amd import native
+
+    native.load()
+    return native
+
+
+def all_bf16() -> torch.Tensor:
+    bits = np.arange(65536, dtype=np.uint16)
+    return torch.from_numpy(bits.view(np.int16).copy()).view(torch.bfloat16)
+
+
+def assert_bf16_equal(got: torch.Tensor, want: torch.Tensor, what: str):
+    """Same bits, except that any NaN matches any NaN."""
+    got, want = got.cpu().contiguous(), want.cpu().contiguous()
+    assert got.shape == want.shape and got.dtype == want.dtype == torch.bfloat16, (what, got.shape, want.shape)
+    nan_g, nan_w = torch.isnan(got), torch.isnan(want)
+    ok = (got.view(torch.int16) == want.view(torch.int16)) | (nan_g & nan_w)
+    if not bool(ok.all()):
+        bad = (~ok).nonzero()
+        first = [(tuple(i.tolist()), float(got[tuple(i)]), float(want[tuple(i)])) for i in bad[:6]]
+        raise AssertionError(f"{what}: {bad.shape[0]} of {got.numel()} values differ; first (index, got, want): {first}")
+
+
+def parts_max(parts: torch.Tensor) -> torch.Tensor:
+    p = parts.cpu()
+    return torch.tensor(float("nan")) if bool(torch.isnan(p).any()) else p.max()
+
+
+# ---------------------------------------------------------------------- SwiGLU
+def test_swiglu_forward_every_gate_pattern(N):
+    g = all_bf16().reshape(256, 256)
+    for seed, std in ((0, 1.0), (1, 30.0)):
+        u = seeded_bf16((256, 256), std, seed)
+        h, parts = N.swiglu_amax_parts(g.cuda(), u.cuda())
+        assert_bf16_equal(h, O.c_swiglu_fwd(g, u), f"swiglu fwd, all gate patterns, up std {std}")
+        assert torch.isnan(parts_max(parts))                      # NaN gates are among the inputs
+
+
+@pytest.mark.parametrize("shape", [(16, 24), (1, 8), (1000, 8), (257, 96), (3, 5, 64), (2048, 1408)])
+def test_swiglu_forward_bit_exact_and_parts(N, shape):
+    g, u = seeded_bf16(shape, 1.5, 11), seeded_bf16(shape, 1.0, 12)
+    h, parts = N.swiglu_amax_parts(g.cuda(), u.cuda())
+    want = O.c_swiglu_fwd(g, u)
+    assert_bf16_equal(h, want, f"swiglu fwd {shape}")
+    assert_f32_bits_equal(parts_max(parts).reshape(1), want.float().abs().max().reshape(1), f"swiglu fwd parts {shape}")
+    assert parts.numel() == N.AMAX_PARTS
+
+
+@pytest.mark.parametrize("shape", [(16, 24), (1, 8), (1000, 8), (257, 96), (1024, 1408)])
+def test_swiglu_backward_bit_exact_and_parts(N, shape):
+    g, u, dh = seeded_bf16(shape, 1.5, 21), seeded_bf16(shape, 1.0, 22), seeded_bf16(shape, 1e-3, 23)
+    dg, du, pg, pu = N.swiglu_bwd_amax_parts(dh.cuda(), g.cuda(), u.cuda())
+    wg, wu = O.c_swiglu_bwd(dh, g, u)
+    assert_bf16_equal(dg, wg, f"swiglu bwd d_gate {shape}")
+    assert_bf16_equal(du, wu, f"swiglu bwd d_up {shape}")
+    assert_f32_bits_equal(parts_max(pg).reshape(1), wg.float().abs().max().reshape(1), "d_gate parts")
+    assert_f32_bits_equal(parts_max(pu).reshape(1), wu.float().abs().max().reshape(1), "d_up parts")
+
+
+def test_swiglu_backward_every_gate_pattern(N):
+    g = all_bf16().reshape(256, 256)
+    u, dh = seeded_bf16((256, 256), 2.0, 3), seeded_bf16((256, 256), 0.01, 4)
+    dg, du, _, _ = N.swiglu_bwd_amax_parts(dh.cuda(), g.cuda(), u.cuda())
+    wg, wu = O.c_swiglu_bwd(dh, g, u)
+    assert_bf16_equal(dg, wg, "swiglu bwd d_gate, all gate patterns")
+    assert_bf16_equal(du, wu, "swiglu bwd d_up, all gate patterns")
+
+
+def test_swiglu_special_values(N):
+    g = torch.tensor([0.0, -0.0, 3.0, -3.0, 90.0, -90.0, float("inf"), float("-inf")], dtype=torch.bfloat16)
+    u = torch.tensor([5.0, 5.0, 0.0, -0.0, 2.0, 2.0, 1.0, 1.0], dtype=torch.bfloat16)
+    h, parts = N.swiglu_amax_parts(g.cuda(), u.cuda())
+    assert_bf16_equal(h, O.c_swiglu_fwd(g, u), "swiglu specials")
+    assert torch.isnan(parts_max(parts))                          # -inf * 0 is NaN, as in eager arithmetic
+    z = torch.zeros((4, 8), dtype=torch.bfloat16)
+    h, parts = N.swiglu_amax_parts(z.cuda(), z.cuda())
+    assert float(h.abs().max()) == 0.0 and float(parts.max()) == 0.0
+    e = torch.empty((0, 8), dtype=torch.bfloat16).cuda()
+    h, parts = N.swiglu_amax_parts(e, e)
+    assert h.numel() == 0 and float(parts.abs().max()) == 0.0
+
+
+def test_swiglu_refusals(N):
+    a = torch.zeros((3, 5), dtype=torch.bfloat16).cuda()
+    with pytest.raises(N.NativeError, match="multiple of 8"):
+        N.swiglu_amax_parts(a, a)
+    with pytest.raises(N.NativeError, match="bf16"):
+        N.swiglu_amax_parts(a.float(), a.float())
+    with pytest.raises(N.NativeError, match="differ"):
+        N.swiglu_amax_parts(torch.zeros((2, 8), dtype=torch.bfloat16).cuda(), torch.zeros((4, 8), dtype=torch.bfloat16).cuda())
+    with pytest.raises(N.NativeError, match="GPU only"):
+        N.swiglu_amax_parts(torch.zeros((2, 8), dtype=torch.bfloat16), torch.zeros((2, 8), dtype=torch.bfloat16))
+
+
+@pytest.mark.parametrize("fmt", [O.E4M3, O.E5M2])
+def test_swiglu_parts_feed_the_dynamic_cast(N, fmt):
+    shape = (512, 384)
+    g, u = seeded_bf16(shape, 2.0, 31), seeded_bf16(shape, 1.0, 32)
+    h, parts = N.swiglu_amax_parts(g.cuda(), u.cuda())
+    q, q_t, amax, scale, scale_inv = N.cast_dynamic(h, parts, fmt, 0)
+    q2, q2_t, amax2, scale2, scale_inv2 = N.quantize_dynamic(h, fmt, 0)
+    assert_bytes_equal(q, q2, "codes with producer parts")
+    assert_bytes_equal(q_t, q2_t, "transposed codes with producer parts")
+    assert_f32_bits_equal(torch.cat([amax, scale, scale_inv]), torch.cat([amax2, scale2, scale_inv2]), "amax/scale")
+    want_h = O.c_swiglu_fwd(g, u)
+    s = O.c_scale(float(want_h.float().abs().max()), fmt)
+    assert_bytes_equal(q, O.c_cast(want_h, s, fmt), "codes vs oracle")
+
+
+# --------------------------------------------------------------------- RMSNorm
+@pytest.mark.parametrize("cols", [8, 64, 520, 1024, 4096, 8192])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("rows", [1, 37])
+def test_rmsnorm_bit_exact(N, rows, cols, dtype):
+    gen = torch.Generator().manual_seed(rows * 100003 + cols)
+    x = (torch.randn((rows, cols), generator=gen) * 2.5).to(dtype)
+    w = (torch.randn(cols, generator=gen) * 0.3 + 1.0)
+    eps = 1e-5
+    y, rstd, parts = N.rmsnorm_amax_parts(x.cuda(), w.cuda(), eps)
+    wy, wr = O.c_rmsnorm(x, w, eps)
+    assert_f32_bits_equal(rstd, wr, f"rmsnorm rstd {rows}x{cols} {dtype}")
+    assert_bf16_equal(y, wy, f"rmsnorm y {rows}x{cols} {dtype}")
+    assert_f32_bits_equal(parts_max(parts).reshape(1), wy.float().abs().max().reshape(1), "rmsnorm parts")
+
+
+def test_rmsnorm_many_rows_and_leading_dims(N):
+    x = seeded_bf16((4, 700, 256), 1.0, 9)                        # 2800 rows: more than one trip per wave
+    w = torch.linspace(0.5, 1.5, 256)
+    y, rstd, parts = N.rmsnorm_amax_parts(x.cuda(), w.cuda(), 1e-6)
+    wy, wr = O.c_rmsnorm(x, w, 1e-6)
+    assert y.shape == x.shape and rstd.shape == x.shape[:-1]
+    assert_bf16_equal(y, wy, "rmsnorm 3-D")
+    assert_f32_bits_equal(rstd, wr, "rmsnorm 3-D rstd")
+    q, _, amax, _, _ = N.cast_dynamic(y.reshape(-1, 256), parts, O.E4M3, 0, want_transposed=False)
+    q2, _, amax2, _, _ = N.quantize_dynamic(y.reshape(-1, 256), O.E4M3, 0, want_transposed=False)
+    assert_bytes_equal(q, q2, "rmsnorm parts feed the cast")
+    assert_f32_bits_equal(amax, amax2, "rmsnorm amax")
+
+
+def test_rmsnorm_exact_case_and_refusals(N):
+    rows, cols = 6, 136
+    sign = torch.where(torch.arange(cols) % 3 == 0, -1.0, 1.0)
+    x = torch.stack([sign * 2.0 ** r for r in range(rows)]).bfloat16()
+    w = torch.arange(1, cols + 1, dtype=torch.float32) / 8.0
+    y, rstd, _ = N.rmsnorm_amax_parts(x.cuda(), w.cuda(), 0.0)
+    assert torch.equal(rstd.cpu(), torch.tensor([2.0 ** -r for r in range(rows)]))
+    assert torch.equal(y.cpu(), (sign * w).bfloat16().expand(rows, cols))
+    with pytest.raises(N.NativeError, match="multiple of 8"):
+        N.rmsnorm_amax_parts(torch.zeros((4, 12), dtype=torch.bfloat16).cuda(), torch.ones(12).cuda(), 1e-5)
+    with pytest.raises(N.NativeError, match="8192"):
+        N.rmsnorm_amax_parts(torch.zeros((1, 32768), dtype=torch.bfloat16).cuda(), torch.ones(32768).cuda(), 1e-5)
+    with pytest.raises(N.NativeError, match="weight"):
+        N.rmsnorm_amax_parts(torch.zeros((4, 16), dtype=torch.bfloat16).cuda(), torch.ones(8).cuda(), 1e-5)
