@@ -25,13 +25,12 @@ __device__ __forceinline__ float recip_newton(float d) {
 }
 
 // logistic function 1 / (1 + exp(-g)): range reduction by ln 2 in two pieces, degree-5 polynomial
-// for (exp(r) - 1 - r) / r^2, exact scaling by 2^k, reciprocal as above.  NaN in, NaN out.
+// for (exp(r) - 1 - r) / r^2, exact scaling by 2^k, reciprocal as above.  A NaN argument is
+// evaluated as 0 here (every use below multiplies by the argument again, which restores the NaN).
 __device__ __forceinline__ float sigmoid_det(float g) {
-    float t = -g;
+    float t = (g != g) ? 0.0f : -g;
     const bool zero = t > 80.0f;                 // exp(-g) beyond 2^115: the quotient is taken as 0
-    t = t < -80.0f ? -80.0f : t;
-    t = zero ? 80.0f : t;
-    t = (g != g) ? 0.0f : t;
+    t = __builtin_amdgcn_fmed3f(t, -80.0f, 80.0f);
     const float kf = __builtin_rintf(__fmul_rn(t, 1.44269504f));
     float r = __fmaf_rn(kf, -0.693359375f, t);
     r = __fmaf_rn(kf, 2.12194440e-4f, r);
@@ -44,31 +43,34 @@ __device__ __forceinline__ float sigmoid_det(float g) {
     const float z = __fmul_rn(r, r);
     const float y = __fadd_rn(__fmaf_rn(p, z, r), 1.0f);
     const float e = __fmul_rn(y, bits_to_float((uint32_t)((int)kf + 127) << 23));
-    float s = recip_newton(__fadd_rn(1.0f, e));
-    s = zero ? 0.0f : s;
-    return (g != g) ? g : s;
+    const float s = recip_newton(__fadd_rn(1.0f, e));
+    return zero ? 0.0f : s;
 }
 
-// bf16 rounding of an fp32 value, returned widened again (what an eager bf16 op leaves behind)
-__device__ __forceinline__ float round_bf16(float f) { return bits_to_float(f32_to_bf16_bits(f) << 16); }
+// Roundings to bf16 use the hardware's round-to-nearest-even conversion of a pair (subnormal
+// results are kept: the kernels run with fp32 denormals enabled).
 
-// h = bf16( bf16(g * sigmoid(g)) * u ): the two roundings of silu(gate) * up evaluated in bf16
-__device__ __forceinline__ float swiglu_fwd_elem(float g, float u) {
-    const float s = round_bf16(__fmul_rn(g, sigmoid_det(g)));
-    return __fmul_rn(s, u);                      // the caller rounds to bf16
+// h = bf16( bf16(g * sigmoid(g)) * u ), the two roundings of silu(gate) * up evaluated in bf16, for
+// the two elements of a packed pair
+__device__ __forceinline__ uint32_t swiglu_fwd_pair(uint32_t gw, uint32_t uw) {
+    const float g0 = bf16_lo(gw), g1 = bf16_hi(gw);
+    const uint32_t s = pack_bf16x2(__fmul_rn(g0, sigmoid_det(g0)), __fmul_rn(g1, sigmoid_det(g1)));
+    return pack_bf16x2(__fmul_rn(bf16_lo(s), bf16_lo(uw)), __fmul_rn(bf16_hi(s), bf16_hi(uw)));
 }
 
-// d_up = bf16(dh * s), d_gate = bf16( bf16(dh * u) * sig * (1 + g * (1 - sig)) )
-__device__ __forceinline__ void swiglu_bwd_elem(float dh, float g, float u, float &dg, float &du) {
-    const float sig = sigmoid_det(g);
-    const float s = round_bf16(__fmul_rn(g, sig));
-    du = __fmul_rn(dh, s);
-    const float ds = round_bf16(__fmul_rn(dh, u));
-    const float dsilu = __fmul_rn(sig, __fmaf_rn(g, __fsub_rn(1.0f, sig), 1.0f));
-    dg = __fmul_rn(ds, dsilu);
+// d_up = bf16(dh * s), d_gate = bf16( bf16(dh * u) * (sig * (1 + g * (1 - sig))) ), s = bf16(g * sig)
+__device__ __forceinline__ void swiglu_bwd_pair(uint32_t dw, uint32_t gw, uint32_t uw, uint32_t &dg, uint32_t &du) {
+    const float g0 = bf16_lo(gw), g1 = bf16_hi(gw), d0 = bf16_lo(dw), d1 = bf16_hi(dw);
+    const float sig0 = sigmoid_det(g0), sig1 = sigmoid_det(g1);
+    const uint32_t s = pack_bf16x2(__fmul_rn(g0, sig0), __fmul_rn(g1, sig1));
+    du = pack_bf16x2(__fmul_rn(d0, bf16_lo(s)), __fmul_rn(d1, bf16_hi(s)));
+    const uint32_t ds = pack_bf16x2(__fmul_rn(d0, bf16_lo(uw)), __fmul_rn(d1, bf16_hi(uw)));
+    const float ds0 = __fmul_rn(sig0, __fmaf_rn(g0, __fsub_rn(1.0f, sig0), 1.0f));
+    const float ds1 = __fmul_rn(sig1, __fmaf_rn(g1, __fsub_rn(1.0f, sig1), 1.0f));
+    dg = pack_bf16x2(__fmul_rn(bf16_lo(ds), ds0), __fmul_rn(bf16_hi(ds), ds1));
 }
 
-__device__ __forceinline__ uint32_t pack2(float a, float b) { return f32_to_bf16_bits(a) | (f32_to_bf16_bits(b) << 16); }
+__device__ __forceinline__ uint32_t pack2(float a, float b) { return pack_bf16x2(a, b); }
 
 // ------------------------------------------------------------------ SwiGLU forward
 // n8 chunks of 8 bf16 (16 bytes) per operand; two chunks per lane in flight.  parts[blockIdx] =
@@ -83,7 +85,7 @@ __global__ __launch_bounds__(kFusedThreads) void swiglu_fwd_kernel(const u32x4 *
         uint32_t o[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            o[q] = pack2(swiglu_fwd_elem(bf16_lo(gw[q]), bf16_lo(uw[q])), swiglu_fwd_elem(bf16_hi(gw[q]), bf16_hi(uw[q])));
+            o[q] = swiglu_fwd_pair(gw[q], uw[q]);
             am = max_u16x2(am, abs_bf16x2(o[q]));
         }
         return u32x4{o[0], o[1], o[2], o[3]};
@@ -117,11 +119,7 @@ __global__ __launch_bounds__(kFusedThreads) void swiglu_bwd_kernel(const u32x4 *
         uint32_t og[4], ou[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            float g0, u0, g1, u1;
-            swiglu_bwd_elem(bf16_lo(dw[q]), bf16_lo(gw[q]), bf16_lo(uw[q]), g0, u0);
-            swiglu_bwd_elem(bf16_hi(dw[q]), bf16_hi(gw[q]), bf16_hi(uw[q]), g1, u1);
-            og[q] = pack2(g0, g1);
-            ou[q] = pack2(u0, u1);
+            swiglu_bwd_pair(dw[q], gw[q], uw[q], og[q], ou[q]);
             am_g = max_u16x2(am_g, abs_bf16x2(og[q]));
             am_u = max_u16x2(am_u, abs_bf16x2(ou[q]));
         }
@@ -146,7 +144,8 @@ __global__ __launch_bounds__(kFusedThreads) void swiglu_bwd_kernel(const u32x4 *
 // (a + b is commutative, so every lane ends with the same bits).
 //   rstd = 1 / sqrt(sum / cols + eps)      (IEEE sqrt and division)
 //   y    = bf16( (x * rstd) * weight )     (two fp32 products, one rounding)
-constexpr int kRmsThreads = 256;
+// Rows up to 64 * 8 * 8 elements keep a lane's share in few registers and run in fat blocks (one
+// row per wave and trip, many rows in flight per CU); wider rows use 256-lane blocks.
 
 template <int SRC>
 __device__ __forceinline__ void unpack8(const u32x4 *raw, float f[8]) {
@@ -160,7 +159,7 @@ __device__ __forceinline__ void unpack8(const u32x4 *raw, float f[8]) {
     }
 }
 
-template <int SRC, int CPL>
+template <int SRC, int CPL, int kRmsThreads>
 __global__ __launch_bounds__(kRmsThreads) void rmsnorm_fwd_kernel(const void *__restrict__ x, const float *__restrict__ weight,
                                                                    int64_t rows, int64_t cols, float eps,
                                                                    uint16_t *__restrict__ y, float *__restrict__ rstd_out,
@@ -280,16 +279,17 @@ extern "C" int odl_fp8_rmsnorm_amax_parts(const void *x, int src_dtype, const fl
         return set_error(ODL_ERR_ARG, "odl_fp8_rmsnorm_amax_parts: null pointer");
     if (cols < 8 || cols % 8 != 0 || cols > 8192 || !aligned16(x) || !aligned16(y) || !aligned16(weight))
         return set_error(ODL_ERR_SHAPE, "odl_fp8_rmsnorm_amax_parts: cols must be a multiple of 8 in [8, 8192] and the pointers 16-byte aligned");
-    const int rows_per_block = kRmsThreads / kWave;
+    const int64_t cpl = (cols / 8 + kWave - 1) / kWave;
+    const int threads = cpl <= 8 ? kFusedThreads : 256;
+    const int rows_per_block = threads / kWave;
     int64_t g = (rows + rows_per_block - 1) / rows_per_block;
     g = g < 1 ? 1 : (g < grid_cap() ? g : grid_cap());
-    const int64_t cpl = (cols / 8 + kWave - 1) / kWave;
-#define ODL_RMS(SRC, CPL) hipLaunchKernelGGL((rmsnorm_fwd_kernel<SRC, CPL>), dim3((unsigned)g), dim3(kRmsThreads), 0, stream, x, weight, rows, cols, eps, reinterpret_cast<uint16_t *>(y), rstd, parts)
-#define ODL_RMS_SRC(CPL) do { if (src_dtype == ODL_BF16) ODL_RMS(ODL_BF16, CPL); else ODL_RMS(ODL_F32, CPL); } while (0)
-    if (cpl <= 2) ODL_RMS_SRC(2);
-    else if (cpl <= 4) ODL_RMS_SRC(4);
-    else if (cpl <= 8) ODL_RMS_SRC(8);
-    else ODL_RMS_SRC(16);
+#define ODL_RMS(SRC, CPL, THR) hipLaunchKernelGGL((rmsnorm_fwd_kernel<SRC, CPL, THR>), dim3((unsigned)g), dim3(THR), 0, stream, x, weight, rows, cols, eps, reinterpret_cast<uint16_t *>(y), rstd, parts)
+#define ODL_RMS_SRC(CPL, THR) do { if (src_dtype == ODL_BF16) ODL_RMS(ODL_BF16, CPL, THR); else ODL_RMS(ODL_F32, CPL, THR); } while (0)
+    if (cpl <= 2) ODL_RMS_SRC(2, kFusedThreads);
+    else if (cpl <= 4) ODL_RMS_SRC(4, kFusedThreads);
+    else if (cpl <= 8) ODL_RMS_SRC(8, kFusedThreads);
+    else ODL_RMS_SRC(16, 256);
 #undef ODL_RMS_SRC
 #undef ODL_RMS
     return check_launch("odl_fp8_rmsnorm_amax_parts");

@@ -193,6 +193,9 @@ class FP8Recipe:
         # (gate/up, q/k/v) quantise it once; dropped when the outermost context is left
         self.shared_input: dict[str, Any] | None = None
         self.share_inputs = True
+        # partial maxima handed over by the kernel that produced a tensor (SwiGLU, RMSNorm), so that
+        # the Linear that quantises this very tensor skips its amax pass; a handful of entries
+        self.producer_parts: list[tuple[tuple, torch.Tensor, torch.Tensor]] = []
         self.scale_epoch = 0      # bumped whenever the forward scales are refreshed (invalidates cached weight codes)
         _info_once(
             f"Created FP8 recipe with format={self.format.value}, amax_history_len={amax_history_len}, "
@@ -247,6 +250,32 @@ class FP8Recipe:
                 arena.scale[:n].copy_(blob["scale"][:n])
                 arena.scale_inv[:n].copy_(blob["scale_inv"][:n])
 
+    # ------------------------------------------------------- producer hand-over
+    @staticmethod
+    def _tensor_key(t: torch.Tensor) -> tuple:
+        return (t.data_ptr(), t._version, t.numel(), t.dtype, t.device)
+
+    def offer_parts(self, tensor: torch.Tensor, parts: torch.Tensor) -> None:
+        """Record the partial maxima of |tensor| that its producer computed.  The entry keeps the
+        tensor alive (its address cannot be reused meanwhile); an in-place change bumps the
+        version and the entry no longer matches."""
+        if self._recipe.kind != "tensorwise":
+            return
+        self.producer_parts.append((self._tensor_key(tensor), tensor, parts))
+        if len(self.producer_parts) > 8:
+            del self.producer_parts[0]
+
+    def take_parts(self, tensor: torch.Tensor) -> torch.Tensor | None:
+        """Partial maxima for exactly this tensor (or a view of all of it), if a producer left them."""
+        if not self.producer_parts:
+            return None
+        key = self._tensor_key(tensor)
+        for i, (k, _, parts) in enumerate(self.producer_parts):
+            if k == key:
+                del self.producer_parts[i]
+                return parts
+        return None
+
     # ---------------------------------------------------------------- contexts
     @contextmanager
     def autocast(self) -> Iterator[None]:
@@ -261,6 +290,7 @@ class FP8Recipe:
             _state.pop_recipe()
             if self._depth == 0:
                 self.shared_input = None
+                self.producer_parts.clear()
                 self.update_scales("fwd")
                 # gradients recorded by a backward that ran outside any backward()
                 # context are folded in here, one step late but never lost
@@ -277,6 +307,7 @@ class FP8Recipe:
             self._depth -= 1
             _state.pop_recipe()
             if self._depth == 0:
+                self.producer_parts.clear()
                 self.update_scales("bwd")
 
     def prepare_for_backward(self, *args: Any, **kwargs: Any) -> tuple[Any, ...]:

@@ -64,10 +64,13 @@ class _WeightCache:
         self.wq = self.wq_t = self.s_inv = self.s_inv_t = self.amax = None
 
 
-def _quantise_dynamic(x2d: torch.Tensor, fmt: int, margin: int, need_t: bool, need_rowmajor: bool = True):
-    """Per-tensor current scaling: amax pass, scale, cast (+transpose) pass."""
+def _quantise_dynamic(x2d: torch.Tensor, fmt: int, margin: int, need_t: bool, need_rowmajor: bool = True,
+                      recipe: FP8Recipe | None = None):
+    """Per-tensor current scaling: amax pass, scale, cast (+transpose) pass.  The amax pass is
+    skipped when the kernel that produced x2d left its partial maxima with the recipe."""
+    parts = recipe.take_parts(x2d) if recipe is not None else None
     q, q_t, amax, _, scale_inv = native.quantize_dynamic(x2d, fmt, margin, want_rowmajor=need_rowmajor or not need_t,
-                                                        want_transposed=need_t)
+                                                        want_transposed=need_t, parts=parts)
     return q, q_t, scale_inv, amax
 
 
@@ -81,12 +84,12 @@ def _quantise_input_shared(recipe: FP8Recipe, x2d: torch.Tensor, fmt: int, margi
     the tensor alive, so its address cannot be handed to another tensor while it is cached;
     an in-place change bumps ``_version`` and misses."""
     if not recipe.share_inputs:
-        return _quantise_dynamic(x2d, fmt, margin, need_t)[:3]
+        return _quantise_dynamic(x2d, fmt, margin, need_t, recipe=recipe)[:3]
     key = _input_key(x2d, "tensor", fmt, margin)
     hit = recipe.shared_input
     if hit is not None and hit["key"] == key and (hit["q_t"] is not None or not need_t):
         return hit["q"], hit["q_t"], hit["s_inv"]
-    q, q_t, s_inv, _ = _quantise_dynamic(x2d, fmt, margin, need_t)
+    q, q_t, s_inv, _ = _quantise_dynamic(x2d, fmt, margin, need_t, recipe=recipe)
     entry = {"key": key, "x": x2d, "q": q, "q_t": q_t, "s_inv": s_inv}
     if hit is not None and hit.get("x") is x2d:          # keep the record of the conversion that produced x2d
         entry["src_key"], entry["src"] = hit.get("src_key"), hit.get("src")
@@ -202,7 +205,8 @@ class _Fp8LinearFn(torch.autograd.Function):
                     meta = module._meta(recipe, dy2d.device, "bwd")
                     gq, gq_t, sg_inv = _quantise_delayed(dy2d, pol.fmt_bwd, meta, ROLE_G, fp8_wgrad, ctx.need_dgrad)
                 else:
-                    gq, gq_t, sg_inv, _ = _quantise_dynamic(dy2d, pol.fmt_bwd, pol.margin, fp8_wgrad, ctx.need_dgrad)
+                    gq, gq_t, sg_inv, _ = _quantise_dynamic(dy2d, pol.fmt_bwd, pol.margin, fp8_wgrad, ctx.need_dgrad,
+                                                            recipe=recipe)
             if ctx.need_dgrad:
                 dx = native.gemm_nt(gq, saved["wq_t"], pol.fmt_bwd, pol.fmt_fwd, sg_inv, saved["sw_inv_t"],
                                     out_dtype=ctx.x_dtype)

@@ -1,0 +1,148 @@
+"""Producers either side of the FP8 Linear that hand their output's partial maxima to it.
+
+The reference leaves these to PyTorch: ``silu(w1(x)) * w2(x)`` in
+optimus_dl/modules/model/blocks/mlp.py:73-76 and RMSNorm in
+optimus_dl/modules/model/blocks/layer_norms.py:86-119.  Here one kernel writes the bf16
+result and, on the way, the partial maxima of its magnitude; the FP8 Linear that consumes
+that very tensor finds them (``FP8Recipe.take_parts``) and casts without an amax pass.
+Modules are not replaced but re-classed in place (``module.__class__`` becomes a subclass of
+its own class with the forward below), so attributes, parameter names, state-dict keys and
+``isinstance`` checks stay what they were.
+
+Without an active FP8 recipe, on the CPU, or for dtypes the kernels do not take, every
+forward below is the module's own.
+"""
+
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .. import native
+from .amp import state as _state
+from .amp.fp8 import FP8Recipe
+from .fp8_linear import FP8Linear
+
+
+def _bf16_cuda(*tensors: torch.Tensor) -> bool:
+    return all(t.is_cuda and t.dtype == torch.bfloat16 for t in tensors)
+
+
+# ------------------------------------------------------------------------- SwiGLU
+class _SwiGLUFn(torch.autograd.Function):
+    """h = silu(gate) * up with the roundings of eager bf16 arithmetic; gate and up are kept for
+    the backward, h is not (the down projection keeps its FP8 codes only)."""
+
+    @staticmethod
+    def forward(ctx, gate: torch.Tensor, up: torch.Tensor, recipe: FP8Recipe):
+        h, parts = native.swiglu_amax_parts(gate, up)
+        recipe.offer_parts(h, parts)
+        ctx.save_for_backward(gate, up)
+        ctx.recipe = recipe
+        return h
+
+    @staticmethod
+    def backward(ctx, dh: torch.Tensor):
+        gate, up = ctx.saved_tensors
+        if dh.dtype != torch.bfloat16:
+            dh = dh.to(torch.bfloat16)
+        dgate, dup, parts_g, parts_u = native.swiglu_bwd_amax_parts(dh, gate, up)
+        ctx.recipe.offer_parts(dgate, parts_g)
+        ctx.recipe.offer_parts(dup, parts_u)
+        return dgate, dup, None
+
+
+def swiglu(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """silu(gate) * up; fused (and feeding the next FP8 Linear) when an FP8 recipe is active."""
+    recipe = _state.active_recipe()
+    if recipe is None or not _bf16_cuda(gate, up) or gate.shape != up.shape or gate.numel() % 8:
+        return F.silu(gate) * up
+    return _SwiGLUFn.apply(gate, up, recipe)
+
+
+class _FusedSwiGLUForward:
+    """Mixed into the class of an MLP with ``w1`` (gate), ``w2`` (up) and ``c_proj`` (down)."""
+
+    _odl_fused_swiglu = True
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if _state.active_recipe() is None or not x.is_cuda:
+            return super().forward(x)
+        return self.c_proj(swiglu(self.w1(x), self.w2(x)))
+
+
+def fuse_swiglu_mlp(mlp: nn.Module) -> bool:
+    """Re-class ``mlp`` in place so that its forward is the fused one.  Only modules whose three
+    projections are FP8 Linears named as in the reference's SwiGLUMLP (mlp.py:47-49) qualify."""
+    if getattr(mlp, "_odl_fused_swiglu", False):
+        return False
+    if not all(isinstance(getattr(mlp, n, None), FP8Linear) for n in ("w1", "w2", "c_proj")):
+        return False
+    cls = mlp.__class__
+    mlp.__class__ = type(cls.__name__, (_FusedSwiGLUForward, cls), {"__module__": cls.__module__})
+    return True
+
+
+# ------------------------------------------------------------------------ RMSNorm
+class _RMSNormFn(torch.autograd.Function):
+    """y = (x * rsqrt(mean(x^2) + eps)) * weight rounded once to bf16."""
+
+    @staticmethod
+    def forward(ctx, x: torch.Tensor, weight: torch.Tensor, eps: float, recipe: FP8Recipe):
+        y, rstd, parts = native.rmsnorm_amax_parts(x, weight, eps)
+        recipe.offer_parts(y, parts)
+        ctx.save_for_backward(x, weight, rstd)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy: torch.Tensor):
+        x, weight, rstd = ctx.saved_tensors
+        dyf = dy.float()
+        xhat = x.float() * rstd.unsqueeze(-1)
+        dw = None
+        if ctx.needs_input_grad[1]:
+            dw = (dyf * xhat).reshape(-1, x.shape[-1]).sum(0).to(weight.dtype)
+        dx = None
+        if ctx.needs_input_grad[0]:
+            dyw = dyf * weight.float()
+            dx = (rstd.unsqueeze(-1) * (dyw - xhat * (dyw * xhat).mean(-1, keepdim=True))).to(x.dtype)
+        return dx, dw, None, None
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor | None:
+    """Fused RMSNorm when an FP8 recipe is active and the kernel takes the input; else None."""
+    recipe = _state.active_recipe()
+    if recipe is None or not x.is_cuda or x.dtype not in (torch.bfloat16, torch.float32):
+        return None
+    if x.dtype != torch.bfloat16 and not (torch.is_autocast_enabled("cuda") and torch.get_autocast_dtype("cuda") == torch.bfloat16):
+        return None                    # an fp32 result is expected downstream: the module's own forward
+    cols = x.shape[-1]
+    if cols % 8 or cols < 8 or cols > 8192 or weight.numel() != cols or x.numel() == 0:
+        return None
+    return _RMSNormFn.apply(x, weight, float(eps), recipe)
+
+
+class _FusedRMSNormForward:
+    """Mixed into the class of an RMSNorm with ``weight`` and ``eps`` (layer_norms.py:64-67).
+
+    Under an FP8 recipe the output is bf16 whatever the input dtype: the recipe's context nests
+    a bf16 autocast (fp8.py:488-493), so the Linear that follows would round an fp32 output to
+    bf16 anyway; the values are the same, the fp32 copy is never written."""
+
+    _odl_fused_rmsnorm = True
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        y = rmsnorm(x, self.weight, self.eps)
+        return super().forward(x) if y is None else y
+
+
+def fuse_rmsnorm(norm: nn.Module) -> bool:
+    if getattr(norm, "_odl_fused_rmsnorm", False):
+        return False
+    w = getattr(norm, "weight", None)
+    if not isinstance(w, torch.Tensor) or w.dim() != 1 or not hasattr(norm, "eps"):
+        return False
+    cls = norm.__class__
+    norm.__class__ = type(cls.__name__, (_FusedRMSNormForward, cls), {"__module__": cls.__module__})
+    return True

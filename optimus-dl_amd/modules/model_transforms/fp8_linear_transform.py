@@ -16,8 +16,11 @@ optimus_dl/modules/model_transforms/transformer_engine.py:
 Deviations, on purpose:
   * the replacement shares the original ``Parameter`` objects instead of copying
     them (:278-290 copies, which unties ``lm_head`` from ``wte``);
-  * ``replace_norm`` / ``replace_attention`` are accepted and ignored: this path
-    is Linear-only;
+  * ``replace_norm`` re-classes RMSNorm modules in place (same object, same keys) so that
+    their forward is the fused kernel that also feeds the next Linear's quantisation;
+    LayerNorm is left alone; ``replace_attention`` is accepted and ignored;
+  * ``fuse_swiglu`` (an extra key, default on) does the same for SwiGLU MLPs whose three
+    projections were converted: ``silu(w1 x) * w2 x`` becomes one kernel;
   * a conversion that throws is logged at WARNING (the reference logs at DEBUG).
 """
 
@@ -31,6 +34,7 @@ import torch.nn as nn
 
 from ... import native
 from ..fp8_linear import FP8Linear
+from ..fused import fuse_rmsnorm, fuse_swiglu_mlp
 from . import register_model_transform
 from .base import BaseModelTransform
 from .config import ModelTransformConfig
@@ -67,17 +71,30 @@ def _convert_linear(original: nn.Linear, **kwargs: Any) -> FP8Linear:
 _register_replacement("torch.nn.modules.linear.Linear", FP8Linear, _convert_linear, "linear")
 
 
+def _convert_rmsnorm(original: nn.Module, **kwargs: Any) -> nn.Module | None:
+    """In place: the module keeps its identity, parameters and keys; None if nothing changed."""
+    return original if fuse_rmsnorm(original) else None
+
+
+# the reference's RMSNorm (layer_norms.py:50) and the one of this package's own blocks
+for _path in ("optimus_dl.modules.model.blocks.layer_norms.RMSNorm", "optimus_dl_amd.modules.model.blocks.RMSNorm",
+              "optimus-dl_amd.modules.model.blocks.RMSNorm"):
+    _register_replacement(_path, nn.Module, _convert_rmsnorm, "norm")
+
+
 @dataclass
 class TransformerEngineTransformConfig(ModelTransformConfig):
     enabled: bool = True
     replace_linear: bool = True
-    replace_norm: bool = True          # accepted, no effect here
+    replace_norm: bool = True          # RMSNorm -> fused forward (in place); LayerNorm untouched
     replace_attention: bool = False    # accepted, no effect here
     linear_kwargs: dict = None
     norm_kwargs: dict = None
     attention_kwargs: dict = None
     replace_inplace: bool = True
     verbose: bool = False
+    fuse_swiglu: bool = True           # not in the reference: SwiGLU MLPs get the fused activation
+    swiglu_classes: tuple = ("SwiGLUMLP",)
 
     def __post_init__(self):
         self.linear_kwargs = dict(self.linear_kwargs or {})
@@ -133,6 +150,8 @@ class TransformerEngineTransform(BaseModelTransform):
             replacement_class, converter, module_type = entry
             enabled, mod_kwargs, key = self._pick(module_type, module.__class__.__name__, replace_linear, replace_norm,
                                                   replace_attention)
+            if enabled and module_type == "norm" and not self.cfg.replace_inplace:
+                enabled = False            # the norm conversion only exists in place
             if enabled:
                 try:
                     new_module = converter(module, **mod_kwargs) if converter else replacement_class(**module.__dict__)
@@ -148,6 +167,10 @@ class TransformerEngineTransform(BaseModelTransform):
         for child_name, child in list(module.named_children()):
             self._replace_modules_recursive(child, replacements, replace_linear, replace_norm, replace_attention,
                                             parent=module, name=child_name)
+        # after the children: the three projections of an MLP are FP8 Linears by now
+        if (self.cfg.fuse_swiglu and self.cfg.replace_inplace and module.__class__.__name__ in tuple(self.cfg.swiglu_classes)
+                and fuse_swiglu_mlp(module)):
+            replacements["SwiGLU"] = replacements.get("SwiGLU", 0) + 1
 
 
 Fp8LinearTransform = TransformerEngineTransform

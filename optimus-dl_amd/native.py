@@ -219,10 +219,12 @@ def cast_dynamic(x: torch.Tensor, parts: torch.Tensor, fmt: int, margin: int = 0
     return q, q_t, dyn[0:1], dyn[1:2], dyn[2:3]
 
 
-def quantize_dynamic(x: torch.Tensor, fmt: int, margin: int = 0, want_rowmajor: bool = True, want_transposed: bool = True):
+def quantize_dynamic(x: torch.Tensor, fmt: int, margin: int = 0, want_rowmajor: bool = True, want_transposed: bool = True,
+                     parts: torch.Tensor | None = None):
     """Current scaling of one tensor in two launches: partial maxima, then a cast that derives the
-    scale itself.  -> (q or None, q_t or None, amax, scale, scale_inv)."""
-    return cast_dynamic(x, amax_parts(x), fmt, margin, want_rowmajor, want_transposed)
+    scale itself.  parts: the partial maxima, when the kernel that produced x already delivered
+    them (one launch then).  -> (q or None, q_t or None, amax, scale, scale_inv)."""
+    return cast_dynamic(x, amax_parts(x) if parts is None else parts, fmt, margin, want_rowmajor, want_transposed)
 
 
 def _bf16_dense(t: torch.Tensor, what: str) -> torch.Tensor:

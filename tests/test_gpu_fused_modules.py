@@ -1,0 +1,224 @@
+"""GPU: the fused SwiGLU / RMSNorm forwards inside real module trees.  What must hold:
+the hand-over of partial maxima changes no bit (same codes, same outputs as the amax pass it
+replaces), the amax passes it replaces are really gone, and the fused modules agree with the
+modules' own PyTorch forwards to within a bf16 unit here and there (GEMM tolerance downstream)."""
+import pytest
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from oracle import oracle as O
+from tests.helpers import max_rel_err, seeded_bf16
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def amp():
+    from optimus_dl_amd.modules import amp as A
+
+    return A
+
+
+def make_mlp(n_embd=256, hidden=512, fuse=True, seed=0):
+    from optimus_dl_amd.modules.model.blocks import SwiGLUMLP
+    from optimus_dl_amd.modules.model_transforms import build_model_transform
+
+    torch.manual_seed(seed)
+    mlp = SwiGLUMLP(n_embd, hidden).to("cuda", torch.bfloat16)
+    t = build_model_transform({"_name": "fp8_linear", "fuse_swiglu": fuse})
+    t.apply(mlp)
+    return mlp, t
+
+
+def step(module, recipe, x, dy):
+    xd = x.clone().requires_grad_(True)
+    for p in module.parameters():
+        p.grad = None
+    with recipe.autocast():
+        y = module(xd)
+    with recipe.backward():
+        y.backward(dy)
+    return [y.detach(), xd.grad.detach()] + [p.grad.detach().clone() for p in module.parameters()]
+
+
+def count_calls(monkeypatch, native, name):
+    calls = []
+    orig = getattr(native, name)
+
+    def counted(*a, **kw):
+        calls.append(tuple(a[0].shape))
+        return orig(*a, **kw)
+
+    monkeypatch.setattr(native, name, counted)
+    return calls
+
+
+def test_fused_mlp_skips_three_amax_passes_and_changes_no_bit(amp, monkeypatch):
+    from optimus_dl_amd import native
+
+    M, C, H = 384, 256, 512
+    x = seeded_bf16((M, C), 1.0, 1).cuda()
+    dy = seeded_bf16((M, C), 1e-3, 2).cuda()
+    mlp, t = make_mlp(C, H, fuse=True)
+    assert t.last_replacements.get("SwiGLU") == 1
+    recipe = amp.FP8Recipe(recipe_type="tensorwise")
+    amax_calls = count_calls(monkeypatch, native, "amax_parts")
+    fused = step(mlp, recipe, x, dy)
+    # x (shared by w1/w2), three weights, dy of c_proj: h, d_gate and d_up come with their maxima
+    assert sorted(amax_calls) == sorted([(M, C), (H, C), (H, C), (C, H), (M, C)])
+    assert recipe.producer_parts == []                                   # all three were taken
+    # same modules, hand-over switched off: every tensor gets its own amax pass, results identical
+    monkeypatch.setattr(type(recipe), "offer_parts", lambda self, t_, p_: None)
+    amax_calls.clear()
+    plain = step(mlp, recipe, x, dy)
+    # the weights' codes are cached (unchanged Parameters): x, h, dy and the two gradients remain
+    assert sorted(amax_calls) == sorted([(M, C), (M, H), (M, C), (M, H), (M, H)])
+    for a, b in zip(fused, plain):
+        assert torch.equal(a, b)
+
+
+def test_fused_mlp_agrees_with_the_eager_activation(amp):
+    M, C, H = 512, 256, 768
+    x = seeded_bf16((M, C), 1.0, 3).cuda()
+    dy = seeded_bf16((M, C), 1e-3, 4).cuda()
+    fused_mlp, _ = make_mlp(C, H, fuse=True, seed=5)
+    eager_mlp, t = make_mlp(C, H, fuse=False, seed=5)
+    assert "SwiGLU" not in t.last_replacements
+    recipe = amp.FP8Recipe(recipe_type="tensorwise")
+    got = step(fused_mlp, recipe, x, dy)
+    want = step(eager_mlp, recipe, x, dy)
+    for name, a, b in zip(["y", "dx", "dw1", "dw2", "dwc"], got, want):
+        assert max_rel_err(a, b) <= 1e-2, name
+
+
+def test_swiglu_function_matches_torch_autograd(amp):
+    from optimus_dl_amd.modules.fused import swiglu
+
+    g = seeded_bf16((64, 256), 1.5, 6).cuda().requires_grad_(True)
+    u = seeded_bf16((64, 256), 1.0, 7).cuda().requires_grad_(True)
+    dh = seeded_bf16((64, 256), 1e-2, 8).cuda()
+    recipe = amp.FP8Recipe(recipe_type="tensorwise")
+    with recipe.autocast():
+        h = swiglu(g, u)
+    h.backward(dh)
+    gc, uc, dhc = g.detach().cpu(), u.detach().cpu(), dh.cpu()
+    assert torch.equal(h.detach().cpu().view(torch.int16), O.c_swiglu_fwd(gc, uc).view(torch.int16))
+    wg, wu = O.c_swiglu_bwd(dhc, gc, uc)
+    assert torch.equal(g.grad.cpu().view(torch.int16), wg.view(torch.int16))
+    assert torch.equal(u.grad.cpu().view(torch.int16), wu.view(torch.int16))
+    # outside a recipe: plain PyTorch
+    h2 = swiglu(g.detach(), u.detach())
+    assert torch.equal(h2, F.silu(g.detach()) * u.detach())
+
+
+@pytest.mark.parametrize("in_dtype", [torch.float32, torch.bfloat16])
+def test_fused_rmsnorm_feeds_the_linear_and_backpropagates(amp, monkeypatch, in_dtype):
+    from optimus_dl_amd import native
+    from optimus_dl_amd.modules.model.blocks import RMSNorm
+    from optimus_dl_amd.modules.model_transforms import build_model_transform
+
+    class Pre(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.ln = RMSNorm(256, 1e-5)
+            self.wq = nn.Linear(256, 320, bias=False)
+            self.wk = nn.Linear(256, 128, bias=False)
+
+        def forward(self, x):
+            n = self.ln(x)
+            return self.wq(n).float().sum(-1) + self.wk(n).float().sum(-1)
+
+    torch.manual_seed(0)
+    net = Pre().cuda()
+    with torch.no_grad():
+        net.ln.weight.copy_(torch.linspace(0.5, 1.5, 256))
+    ref = Pre().cuda()
+    ref.load_state_dict(net.state_dict())
+    t = build_model_transform({"_name": "transformer_engine"})
+    t.apply(net)
+    assert t.last_replacements["RMSNorm"] == 1 and t.last_replacements["Linear"] == 2
+    build_model_transform({"_name": "transformer_engine", "replace_norm": False}).apply(ref)
+    x = (torch.randn(4, 96, 256, generator=torch.Generator().manual_seed(1)) * 2).to(in_dtype).cuda()
+    recipe = amp.FP8Recipe(recipe_type="tensorwise")
+    amax_calls = count_calls(monkeypatch, native, "amax_parts")
+    outs = {}
+    for name, m in (("fused", net), ("plain", ref)):
+        xd = x.clone().requires_grad_(True)
+        amax_calls.clear()
+        with amp.fp8_autocast(torch.device("cuda"), recipe):
+            y = m(xd)
+        with amp.fp8_backward(recipe):
+            y.sum().backward()
+        outs[name] = (y.detach(), xd.grad.detach(), m.ln.weight.grad.detach(), m.wq.weight.grad.detach())
+        if name == "fused":
+            # the normalised activation arrives with its maxima: only the two weights and the two dy
+            assert sorted(amax_calls) == sorted([(320, 256), (128, 256), (384, 320), (384, 128)])
+        else:
+            assert (4 * 96, 256) in amax_calls
+    f, p = outs["fused"], outs["plain"]
+    assert f[1].dtype == in_dtype
+    assert max_rel_err(f[0], p[0]) <= 1e-2
+    assert max_rel_err(f[1], p[1]) <= 2e-2
+    assert max_rel_err(f[2], p[2]) <= 2e-2
+    assert max_rel_err(f[3], p[3]) <= 1e-2
+
+
+def test_fused_rmsnorm_equals_oracle_and_leaves_other_cases_alone(amp):
+    from optimus_dl_amd.modules.fused import fuse_rmsnorm
+    from optimus_dl_amd.modules.model.blocks import RMSNorm
+
+    norm = RMSNorm(512, 1e-6).cuda()
+    with torch.no_grad():
+        norm.weight.copy_(torch.linspace(0.25, 2.0, 512))
+    assert fuse_rmsnorm(norm) and not fuse_rmsnorm(norm)
+    x = seeded_bf16((3, 40, 512), 3.0, 9)
+    recipe = amp.FP8Recipe(recipe_type="tensorwise")
+    with amp.fp8_autocast(torch.device("cuda"), recipe):
+        y = norm(x.cuda())
+        y32 = norm(x.float().cuda())                     # fp32 in, bf16 out under the bf16 autocast
+    want, _ = O.c_rmsnorm(x, norm.weight.detach().cpu(), 1e-6)
+    assert y.dtype == torch.bfloat16 and torch.equal(y.cpu().view(torch.int16), want.view(torch.int16))
+    assert y32.dtype == torch.bfloat16 and torch.equal(y32.cpu().view(torch.int16), want.view(torch.int16))
+    # no recipe: the module's own forward, dtype of the input
+    y_plain = norm(x.float().cuda())
+    assert y_plain.dtype == torch.float32
+    # a recipe without the bf16 autocast around it and an fp32 input: own forward as well
+    with recipe.autocast():
+        assert norm(x.float().cuda()).dtype == torch.float32
+        assert norm(x.cuda()).dtype == torch.bfloat16
+
+
+@pytest.mark.parametrize("recipe_name", ["tensorwise", "delayed", "rowwise"])
+def test_llama_block_with_fusions_trains_like_the_unfused_one(amp, recipe_name):
+    from optimus_dl_amd.modules.model import Llama, LlamaConfig
+    from optimus_dl_amd.modules.model_transforms import build_model_transform
+
+    def build(fuse):
+        torch.manual_seed(0)
+        m = Llama(LlamaConfig(vocab_size=256, n_layer=2, n_head=4, n_kv_head=2, n_embd=128, intermediate_size=256)).cuda()
+        t = build_model_transform({"_name": "transformer_engine", "replace_norm": fuse, "fuse_swiglu": fuse})
+        t.apply(m)
+        return m, t
+
+    ids = torch.randint(0, 256, (4, 33), generator=torch.Generator().manual_seed(2)).cuda()
+    traces = {}
+    for fuse in (True, False):
+        m, t = build(fuse)
+        assert (t.last_replacements.get("SwiGLU", 0) == 2) == fuse and (t.last_replacements["RMSNorm"] == 5) == fuse
+        recipe = amp.FP8Recipe(recipe_type=recipe_name, amax_history_len=4)
+        opt = torch.optim.AdamW(m.parameters(), lr=3e-3)
+        trace = []
+        for _ in range(6):
+            opt.zero_grad(set_to_none=True)
+            with amp.fp8_autocast(torch.device("cuda"), recipe):
+                logits = m(ids[:, :-1])["logits"].float()
+                loss = F.cross_entropy(logits.reshape(-1, 256), ids[:, 1:].reshape(-1))
+            with amp.fp8_backward(recipe):
+                loss.backward()
+            opt.step()
+            trace.append(loss.item())
+        assert all(p.grad is not None for p in m.parameters())
+        traces[fuse] = trace
+    assert traces[True][-1] < traces[True][0] - 0.3, traces
+    assert abs(traces[True][-1] - traces[False][-1]) < 0.15, traces

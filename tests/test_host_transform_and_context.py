@@ -234,3 +234,78 @@ def test_forward_backward_helpers_accept_instance_or_factory():
     loss = execute_forward_pass(lin, batch, crit, nullcontext())
     execute_backward_pass(loss, None, nullcontext())
     assert len(calls) == 2 and lin.weight.grad is not None
+
+
+# ------------------------------------------------- fused producers: transform and hand-over (host side)
+def _llama_tree():
+    from optimus_dl_amd.modules.model import Llama, LlamaConfig
+
+    torch.manual_seed(0)
+    return Llama(LlamaConfig(vocab_size=64, n_layer=2, n_head=2, n_kv_head=1, n_embd=32, intermediate_size=64))
+
+
+def test_transform_fuses_swiglu_and_rmsnorm_in_place(monkeypatch):
+    from optimus_dl_amd.modules.model.blocks import RMSNorm, SwiGLUMLP
+
+    monkeypatch.setattr(T, "_HAVE_TE", True)
+    m = _llama_tree()
+    keys = sorted(m.state_dict().keys())
+    mlp, norm = m.transformer.h[0].mlp, m.transformer.h[0].ln_1
+    ids = torch.randint(0, 64, (2, 8))
+    before = m(ids)["logits"]
+    t = build_model_transform({"_name": "transformer_engine"})
+    assert t.apply(m) is m
+    n_lin = sum(isinstance(x, FP8Linear) for x in m.modules())
+    assert t.last_replacements == {"Linear": n_lin, "RMSNorm": 5, "LayerNorm": 0, "Attention": 0, "SwiGLU": 2}
+    assert m.transformer.h[0].mlp is mlp and m.transformer.h[0].ln_1 is norm          # same objects
+    assert isinstance(mlp, SwiGLUMLP) and isinstance(norm, RMSNorm)
+    assert type(mlp).__name__ == "SwiGLUMLP" and type(norm).__module__ == RMSNorm.__module__
+    assert getattr(mlp, "_odl_fused_swiglu", False) and getattr(norm, "_odl_fused_rmsnorm", False)
+    assert sorted(m.state_dict().keys()) == keys
+    torch.testing.assert_close(m(ids)["logits"], before)                              # no recipe active: own forwards
+    again = build_model_transform({"_name": "transformer_engine"})
+    again.apply(m)
+    assert again.last_replacements == {"Linear": 0, "RMSNorm": 0, "LayerNorm": 0, "Attention": 0}
+
+
+def test_transform_fusion_switches(monkeypatch):
+    monkeypatch.setattr(T, "_HAVE_TE", True)
+    m = _llama_tree()
+    t = build_model_transform({"_name": "fp8_linear", "replace_norm": False, "fuse_swiglu": False})
+    t.apply(m)
+    assert t.last_replacements["RMSNorm"] == 0 and "SwiGLU" not in t.last_replacements
+    assert not hasattr(m.transformer.h[0].mlp, "_odl_fused_swiglu") and not hasattr(m.transformer.ln_f, "_odl_fused_rmsnorm")
+    m = _llama_tree()
+    t = build_model_transform({"_name": "fp8_linear", "replace_linear": False})
+    t.apply(m)
+    assert "SwiGLU" not in t.last_replacements and t.last_replacements["RMSNorm"] == 5   # MLP projections are plain Linears
+    m = _llama_tree()
+    t = build_model_transform({"_name": "fp8_linear", "replace_inplace": False})
+    t.apply(m)
+    assert not hasattr(m.transformer.ln_f, "_odl_fused_rmsnorm") and not hasattr(m.transformer.h[0].mlp, "_odl_fused_swiglu")
+
+
+def test_producer_parts_hand_over(monkeypatch):
+    from optimus_dl_amd.modules import amp as A
+    from optimus_dl_amd.modules.amp import fp8 as fp8_mod
+
+    monkeypatch.setattr(fp8_mod, "is_native_backend_available", lambda: True)   # bookkeeping only, no kernel runs
+    r = A.FP8Recipe(recipe_type="tensorwise")
+    x = torch.zeros(4, 6)
+    parts = torch.ones(3)
+    r.offer_parts(x, parts)
+    assert r.take_parts(torch.zeros(4, 6)) is None                    # another tensor
+    assert r.take_parts(x.reshape(2, 12)) is parts                    # a view of all of it
+    assert r.take_parts(x) is None                                    # handed over once
+    r.offer_parts(x, parts)
+    x.add_(1)                                                         # changed in place since
+    assert r.take_parts(x) is None
+    for i in range(12):
+        r.offer_parts(torch.zeros(1), parts)
+    assert len(r.producer_parts) == 8
+    with r.autocast():
+        pass
+    assert r.producer_parts == []
+    d = A.FP8Recipe(recipe_type="delayed")
+    d.offer_parts(x, parts)
+    assert d.producer_parts == []                                     # only current scaling reads an amax per tensor
