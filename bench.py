@@ -127,6 +127,19 @@ def standalone_hbm(torch, native, iters=24):
             "cast_transpose": (lambda x: native.cast_transpose(x, scale, native.E4M3, native.SCALE_TENSOR), 4 * E),
             "amax_then_cast_transpose": (lambda x: native.quantize_dynamic(x, native.E4M3, 0), 6 * E),
         }
+        if cols == D_FF:                   # the SwiGLU producers run on the [tokens, d_ff] activations
+            nxt = {id(x): (xs[(i + 1) % nbuf], xs[(i + 2) % nbuf]) for i, x in enumerate(xs)}
+            kernels["swiglu_fwd_amax"] = (lambda x: native.swiglu_amax_parts(x, nxt[id(x)][0]), 6 * E)
+            kernels["swiglu_bwd_amax"] = (lambda x: native.swiglu_bwd_amax_parts(x, nxt[id(x)][0], nxt[id(x)][1]), 10 * E)
+        if cols == D_MODEL and rows == M_TOKENS:   # RMSNorm in front of q/k/v and gate/up: bf16 and fp32 residual streams
+            w_norm = torch.ones(cols, device="cuda")
+            kernels["rmsnorm_amax_bf16_in"] = (lambda x: native.rmsnorm_amax_parts(x, w_norm, 1e-5), 4 * E)
+            xs32 = [x.float() for x in xs]
+            to32 = {id(x): y for x, y in zip(xs, xs32)}
+            kernels["rmsnorm_amax_fp32_in"] = (lambda x: native.rmsnorm_amax_parts(to32[id(x)], w_norm, 1e-5), 6 * E)
+            _, rstd_b, _ = native.rmsnorm_amax_parts(xs[0], w_norm, 1e-5)
+            dy_of = {id(x): xs[(i + 1) % nbuf] for i, x in enumerate(xs)}
+            kernels["rmsnorm_bwd_bf16"] = (lambda x: native.rmsnorm_bwd(dy_of[id(x)], x, w_norm, rstd_b), 6 * E)
         for name, (fn, nbytes) in kernels.items():
             for x in xs:
                 fn(x)
@@ -140,6 +153,45 @@ def standalone_hbm(torch, native, iters=24):
             gbps = nbytes / (us * 1e-6) / 1e9
             out.setdefault(name, {})[f"{rows}x{cols}"] = {"us": round(us, 1), "GB/s": round(gbps), "frac": round(gbps / PEAK_HBM_GBPS, 3)}
         del xs
+    return out
+
+
+def mlp_block(torch, native, recipe, steps=10, warmup=3):
+    """The same three Linears wired as the MLP they come from (optimus_dl/modules/model/blocks/mlp.py:73-78):
+    c_proj(silu(w1 x) * w2 x), forward + backward, weights re-quantised every step; once with the fused
+    activation (which also spares the amax passes over h, d_gate, d_up) and once with PyTorch's."""
+    from optimus_dl_amd.modules.model.blocks import SwiGLUMLP
+    from optimus_dl_amd.modules.model_transforms import build_model_transform
+
+    out = {}
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(M_TOKENS, D_MODEL, generator=g).bfloat16().cuda().requires_grad_(True)
+    dy = (torch.randn(M_TOKENS, D_MODEL, generator=g) * 1e-3).bfloat16().cuda()
+    for label, fuse in (("fused_activation", True), ("pytorch_activation", False)):
+        torch.manual_seed(0)
+        mlp = SwiGLUMLP(D_MODEL, D_FF).to("cuda", torch.bfloat16)
+        build_model_transform({"_name": "fp8_linear", "fuse_swiglu": fuse}).apply(mlp)
+
+        def one():
+            for lin in (mlp.w1, mlp.w2, mlp.c_proj):
+                lin._wcache.key = None
+                lin.weight.grad = None
+            x.grad = None
+            with recipe.autocast():
+                y = mlp(x)
+            with recipe.backward():
+                y.backward(dy)
+
+        for _ in range(warmup):
+            one()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            one()
+        torch.cuda.synchronize()
+        ms = 1e3 * (time.perf_counter() - t0) / steps
+        out[label] = {"ms_per_step": ms, "TFLOP/s": step_flops() / (ms * 1e-3) / 1e12}
+        del mlp
     return out
 
 
@@ -312,6 +364,9 @@ def main() -> int:
     }
     if not args.no_standalone:
         line["hbm_kernels_standalone"] = standalone_hbm(torch, native)
+    if not args.no_standalone:
+        del layers, data
+        line["mlp_block_fwd_bwd"] = mlp_block(torch, native, recipe)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(torch)
     print(json.dumps(line))

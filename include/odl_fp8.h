@@ -162,6 +162,19 @@ int odl_fp8_rmsnorm_amax_parts(const void *x, int src_dtype, const float *weight
                                odl_stream_t stream);
 
 /*
+ * Backward of that RMSNorm (what autograd derives for layer_norms.py:86-119), dy in bf16:
+ *   xh = x * rstd, t = dy * weight, c = sum_row(t * xh) / cols  (summed in the order of the forward)
+ *   dx = rstd * fma(-xh, c, t), rounded once to the dtype of x (src_dtype)
+ *   dweight[col] = sum over rows of dy * xh, fp32 (per-wave, per-block and per-slab partial sums
+ *   in a fixed order: reproducible from run to run on one device)
+ * workspace: ODL_FP8_RMSNORM_BWD_SLABS * cols floats of device memory, contents irrelevant.
+ */
+#define ODL_FP8_RMSNORM_BWD_SLABS 512
+int odl_fp8_rmsnorm_bwd(const void *dy, const void *x, int src_dtype, const float *weight,
+                        const float *rstd, int64_t rows, int64_t cols, void *dx, float *dweight,
+                        float *workspace, odl_stream_t stream);
+
+/*
  * out[r,c] = fp8( clamp( fp32(x[r,c]) * s , +-max ) ), s = scale[0] | scale[r] | scale[c].
  * amax_out (may be NULL): *amax_out = max(*amax_out, max|x|), for delayed scaling,
  * where the cast uses an older scale while this step's amax is recorded.

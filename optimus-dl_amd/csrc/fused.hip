@@ -217,6 +217,139 @@ __global__ __launch_bounds__(kRmsThreads) void rmsnorm_fwd_kernel(const void *__
         for (int j = (int)gridDim.x + threadIdx.x; j < kParts; j += kRmsThreads) parts[j] = 0.0f;
 }
 
+// ------------------------------------------------------------------ RMSNorm backward
+// Same work split as the forward (one wavefront per row, lane l holds chunks l, l + 64, ...).
+//   xh = x * rstd, t = dy * weight, c = sum(t * xh) / cols  (per lane by fma in element order,
+//   then the xor butterfly), dx = rstd * fma(-xh, c, t): every dx is a fixed sequence of IEEE
+//   operations, rounded once to the dtype of x.
+// d_weight[col] = sum over rows of dy * xh: a lane adds up its columns over the rows its wave
+// visits, the waves of a block are combined through LDS in wave order, each block writes one
+// slab of `cols` sums to the workspace, and a second kernel adds the slabs in block order.
+constexpr int kRmsBwdThreads = 256;
+
+template <int SRC, int CPL>
+__global__ __launch_bounds__(kRmsBwdThreads) void rmsnorm_bwd_kernel(const u32x4 *__restrict__ dy, const void *__restrict__ x,
+                                                                      const float *__restrict__ weight, const float *__restrict__ rstd_in,
+                                                                      int64_t rows, int64_t cols, void *__restrict__ dx,
+                                                                      float *__restrict__ slabs) {
+    extern __shared__ float lds_dw[];                        // cols floats
+    constexpr int VPC = SRC == ODL_BF16 ? 1 : 2;
+    const int lane = threadIdx.x % kWave, wave_in_block = threadIdx.x / kWave;
+    const int64_t wave = (int64_t)blockIdx.x * (kRmsBwdThreads / kWave) + wave_in_block;
+    const int64_t nwave = (int64_t)gridDim.x * (kRmsBwdThreads / kWave);
+    const int64_t nchunk = cols / 8;
+    float dw[CPL][8];
+#pragma unroll
+    for (int j = 0; j < CPL; ++j)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) dw[j][e] = 0.0f;
+    for (int64_t row = wave; row < rows; row += nwave) {
+        u32x4 xr[CPL][VPC], dr[CPL];
+#pragma unroll
+        for (int j = 0; j < CPL; ++j) {
+            const int64_t c = lane + (int64_t)kWave * j;
+            const bool ok = c < nchunk;
+            const u32x4 *p = reinterpret_cast<const u32x4 *>(x) + (row * nchunk + c) * VPC;
+#pragma unroll
+            for (int h = 0; h < VPC; ++h) xr[j][h] = ok ? __builtin_nontemporal_load(p + h) : u32x4{0, 0, 0, 0};
+            dr[j] = ok ? __builtin_nontemporal_load(dy + row * nchunk + c) : u32x4{0, 0, 0, 0};
+        }
+        const float rstd = rstd_in[row];
+        float acc = 0.0f;
+#pragma unroll
+        for (int j = 0; j < CPL; ++j) {
+            const int64_t c = lane + (int64_t)kWave * j;
+            if (c < nchunk) {
+                float xf[8], df[8];
+                unpack8<SRC>(xr[j], xf);
+                unpack8<ODL_BF16>(&dr[j], df);
+                const float4 w0 = *reinterpret_cast<const float4 *>(weight + c * 8), w1 = *reinterpret_cast<const float4 *>(weight + c * 8 + 4);
+                const float w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float xh = __fmul_rn(xf[e], rstd);
+                    acc = __fmaf_rn(__fmul_rn(df[e], w[e]), xh, acc);
+                    dw[j][e] = __fmaf_rn(df[e], xh, dw[j][e]);
+                }
+            }
+        }
+#pragma unroll
+        for (int off = kWave / 2; off > 0; off >>= 1) acc = __fadd_rn(acc, __shfl_xor(acc, off, kWave));
+        const float cmean = __fdiv_rn(acc, (float)cols);
+#pragma unroll
+        for (int j = 0; j < CPL; ++j) {
+            const int64_t c = lane + (int64_t)kWave * j;
+            if (c < nchunk) {
+                float xf[8], df[8], o[8];
+                unpack8<SRC>(xr[j], xf);
+                unpack8<ODL_BF16>(&dr[j], df);
+                const float4 w0 = *reinterpret_cast<const float4 *>(weight + c * 8), w1 = *reinterpret_cast<const float4 *>(weight + c * 8 + 4);
+                const float w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float xh = __fmul_rn(xf[e], rstd);
+                    o[e] = __fmul_rn(rstd, __fmaf_rn(-xh, cmean, __fmul_rn(df[e], w[e])));
+                }
+                if constexpr (SRC == ODL_BF16) {
+                    reinterpret_cast<u32x4 *>(dx)[row * nchunk + c] =
+                        u32x4{pack2(o[0], o[1]), pack2(o[2], o[3]), pack2(o[4], o[5]), pack2(o[6], o[7])};
+                } else {
+                    float4 *q = reinterpret_cast<float4 *>(dx) + (row * nchunk + c) * 2;
+                    q[0] = float4{o[0], o[1], o[2], o[3]};
+                    q[1] = float4{o[4], o[5], o[6], o[7]};
+                }
+            }
+        }
+    }
+    // waves of the block, in order, into the LDS row; then the block's slab
+    for (int wv = 0; wv < kRmsBwdThreads / kWave; ++wv) {
+        if (wave_in_block == wv) {
+#pragma unroll
+            for (int j = 0; j < CPL; ++j) {
+                const int64_t c = lane + (int64_t)kWave * j;
+                if (c < nchunk) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        float *slot = &lds_dw[c * 8 + e];
+                        *slot = wv == 0 ? dw[j][e] : __fadd_rn(*slot, dw[j][e]);
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+    for (int64_t c = threadIdx.x; c < cols; c += kRmsBwdThreads) slabs[(int64_t)blockIdx.x * cols + c] = lds_dw[c];
+}
+
+// slabs -> d_weight: a block owns 64 columns; 16 groups of lanes each add every 16th slab (8 loads in
+// flight), the groups are combined through LDS in group order.  The order is fixed by the code.
+__global__ __launch_bounds__(1024) void rmsnorm_bwd_reduce_kernel(const float *__restrict__ slabs, int nslab, int64_t cols,
+                                                                   float *__restrict__ dw) {
+    __shared__ float part[16][64];
+    const int cx = threadIdx.x % 64, grp = threadIdx.x / 64;
+    const int64_t c = (int64_t)blockIdx.x * 64 + cx;
+    float a = 0.0f;
+    if (c < cols) {
+        int b = grp;
+        for (; b + 7 * 16 < nslab; b += 8 * 16) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = slabs[(int64_t)(b + u * 16) * cols + c];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) a = __fadd_rn(a, v[u]);
+        }
+        for (; b < nslab; b += 16) a = __fadd_rn(a, slabs[(int64_t)b * cols + c]);
+    }
+    part[grp][cx] = a;
+    __syncthreads();
+    if (grp == 0 && c < cols) {
+        float t = part[0][cx];
+#pragma unroll
+        for (int g = 1; g < 16; ++g) t = __fadd_rn(t, part[g][cx]);
+        dw[c] = t;
+    }
+}
+
 static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 // at most two fat blocks per CU, and never more blocks than there are partial maxima
@@ -293,4 +426,30 @@ extern "C" int odl_fp8_rmsnorm_amax_parts(const void *x, int src_dtype, const fl
 #undef ODL_RMS_SRC
 #undef ODL_RMS
     return check_launch("odl_fp8_rmsnorm_amax_parts");
+}
+
+extern "C" int odl_fp8_rmsnorm_bwd(const void *dy, const void *x, int src_dtype, const float *weight, const float *rstd, int64_t rows,
+                                   int64_t cols, void *dx, float *dweight, float *workspace, odl_stream_t stream_) {
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    if (rows < 0 || cols < 0) return set_error(ODL_ERR_ARG, "odl_fp8_rmsnorm_bwd: negative shape");
+    if (src_dtype != ODL_BF16 && src_dtype != ODL_F32) return set_error(ODL_ERR_ARG, "odl_fp8_rmsnorm_bwd: src_dtype %d", src_dtype);
+    if (!dweight || !workspace || !weight || (rows > 0 && !rstd) || (rows * cols > 0 && (!dy || !x || !dx)))
+        return set_error(ODL_ERR_ARG, "odl_fp8_rmsnorm_bwd: null pointer");
+    if (cols < 8 || cols % 8 != 0 || cols > 8192 || !aligned16(x) || !aligned16(dy) || !aligned16(dx) || !aligned16(weight))
+        return set_error(ODL_ERR_SHAPE, "odl_fp8_rmsnorm_bwd: cols must be a multiple of 8 in [8, 8192] and the pointers 16-byte aligned");
+    const int rows_per_block = kRmsBwdThreads / kWave;
+    int64_t g = (rows + rows_per_block - 1) / rows_per_block;
+    g = g < 1 ? 1 : (g < ODL_FP8_RMSNORM_BWD_SLABS ? g : ODL_FP8_RMSNORM_BWD_SLABS);
+    const int64_t cpl = (cols / 8 + kWave - 1) / kWave;
+    const size_t lds = (size_t)cols * sizeof(float);
+#define ODL_RMSB(SRC, CPL) hipLaunchKernelGGL((rmsnorm_bwd_kernel<SRC, CPL>), dim3((unsigned)g), dim3(kRmsBwdThreads), lds, stream, reinterpret_cast<const u32x4 *>(dy), x, weight, rstd, rows, cols, dx, workspace)
+#define ODL_RMSB_SRC(CPL) do { if (src_dtype == ODL_BF16) ODL_RMSB(ODL_BF16, CPL); else ODL_RMSB(ODL_F32, CPL); } while (0)
+    if (cpl <= 2) ODL_RMSB_SRC(2);
+    else if (cpl <= 4) ODL_RMSB_SRC(4);
+    else if (cpl <= 8) ODL_RMSB_SRC(8);
+    else ODL_RMSB_SRC(16);
+#undef ODL_RMSB_SRC
+#undef ODL_RMSB
+    hipLaunchKernelGGL(rmsnorm_bwd_reduce_kernel, dim3((unsigned)((cols + 63) / 64)), dim3(1024), 0, stream, workspace, (int)g, cols, dweight);
+    return check_launch("odl_fp8_rmsnorm_bwd");
 }

@@ -98,16 +98,10 @@ class _RMSNormFn(torch.autograd.Function):
     @staticmethod
     def backward(ctx, dy: torch.Tensor):
         x, weight, rstd = ctx.saved_tensors
-        dyf = dy.float()
-        xhat = x.float() * rstd.unsqueeze(-1)
-        dw = None
-        if ctx.needs_input_grad[1]:
-            dw = (dyf * xhat).reshape(-1, x.shape[-1]).sum(0).to(weight.dtype)
-        dx = None
-        if ctx.needs_input_grad[0]:
-            dyw = dyf * weight.float()
-            dx = (rstd.unsqueeze(-1) * (dyw - xhat * (dyw * xhat).mean(-1, keepdim=True))).to(x.dtype)
-        return dx, dw, None, None
+        if dy.dtype != torch.bfloat16:
+            dy = dy.to(torch.bfloat16)
+        dx, dw = native.rmsnorm_bwd(dy, x, weight, rstd)
+        return (dx if ctx.needs_input_grad[0] else None), (dw.to(weight.dtype) if ctx.needs_input_grad[1] else None), None, None
 
 
 def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor | None:

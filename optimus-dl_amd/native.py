@@ -40,6 +40,7 @@ EXPORTS = (
     "odl_fp8_swiglu_amax_parts",
     "odl_fp8_swiglu_bwd_amax_parts",
     "odl_fp8_rmsnorm_amax_parts",
+    "odl_fp8_rmsnorm_bwd",
     "odl_fp8_amax_rowcol",
     "odl_fp8_cast_rowcol",
     "odl_fp8_cast",
@@ -89,6 +90,7 @@ def load() -> ctypes.CDLL:
         L.odl_fp8_swiglu_amax_parts.argtypes = [vp, vp, i64, i64, vp, vp, vp]
         L.odl_fp8_swiglu_bwd_amax_parts.argtypes = [vp, vp, vp, i64, i64, vp, vp, vp, vp, vp]
         L.odl_fp8_rmsnorm_amax_parts.argtypes = [vp, i32, vp, i64, i64, ctypes.c_float, vp, vp, vp, vp]
+        L.odl_fp8_rmsnorm_bwd.argtypes = [vp, vp, i32, vp, vp, i64, i64, vp, vp, vp, vp]
         L.odl_fp8_amax_rowcol.argtypes = [vp, i32, i64, i64, vp, vp, vp]
         L.odl_fp8_cast_rowcol.argtypes = [vp, i32, i64, i64, vp, vp, i32, i32, vp, vp, vp, vp, vp, vp, vp]
         L.odl_fp8_cast.argtypes = [vp, i32, i64, i64, vp, i32, i32, vp, vp, vp]
@@ -294,6 +296,35 @@ def rmsnorm_amax_parts(x: torch.Tensor, weight: torch.Tensor, eps: float):
     _check(load().odl_fp8_rmsnorm_amax_parts(x.data_ptr(), src, w.data_ptr(), rows, cols, float(eps), y.data_ptr(), rstd.data_ptr(),
                                              parts.data_ptr(), _stream()), "odl_fp8_rmsnorm_amax_parts")
     return y, rstd, parts
+
+
+RMSNORM_BWD_SLABS = 512
+
+
+def rmsnorm_bwd(dy: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, rstd: torch.Tensor):
+    """Gradients of :func:`rmsnorm_amax_parts`'s y for grad_output dy (bf16).
+    -> (dx in the dtype of x, d_weight fp32[cols])."""
+    dy = _bf16_dense(dy, "rmsnorm dy")
+    src = _src_dtype(x)
+    if not x.is_contiguous():
+        x = x.contiguous()
+    if x.data_ptr() % 16:
+        x = x.clone(memory_format=torch.contiguous_format)
+    if dy.shape != x.shape:
+        raise NativeError(f"rmsnorm backward: dy {tuple(dy.shape)} and x {tuple(x.shape)} differ")
+    cols = x.shape[-1]
+    rows = x.numel() // max(cols, 1)
+    w = weight.detach()
+    if w.dtype != torch.float32 or not w.is_contiguous() or w.data_ptr() % 16:
+        w = w.float().contiguous().clone()
+    _f32_dev(rstd.reshape(-1) if rstd.is_contiguous() else rstd.contiguous().reshape(-1), rows, "rmsnorm backward rstd")
+    rstd = rstd.contiguous()
+    dx = torch.empty_like(x)
+    dw = torch.empty(cols, dtype=torch.float32, device=x.device)
+    ws = torch.empty(RMSNORM_BWD_SLABS * cols, dtype=torch.float32, device=x.device)
+    _check(load().odl_fp8_rmsnorm_bwd(dy.data_ptr(), x.data_ptr(), src, w.data_ptr(), rstd.data_ptr(), rows, cols, dx.data_ptr(),
+                                      dw.data_ptr(), ws.data_ptr(), _stream()), "odl_fp8_rmsnorm_bwd")
+    return dx, dw
 
 
 def quantize_rowcol(x: torch.Tensor, fmt: int, margin: int = 0):

@@ -35,6 +35,7 @@
 #include <stdint.h>
 #include <string.h>
 #include <float.h>
+#include <stdlib.h>
 
 #define ORACLE_API __attribute__((visibility("default")))
 
@@ -355,4 +356,47 @@ ORACLE_API void oracle_rmsnorm(const void *x, int src, const float *weight, int6
             y[idx] = f32_to_bf16((v * rstd) * weight[c]);
         }
     }
+}
+
+/* Backward of the RMSNorm above for bf16 dy.  dx follows the library's stated sequence of IEEE
+ * operations (bit-exact target); d_weight is accumulated in double here, because the library only
+ * promises a fixed but device-dependent order of fp32 partial sums (tolerance target).  Pinned in
+ * tests/test_oracle_fused.py against torch autograd of the reference module's expression. */
+ORACLE_API void oracle_rmsnorm_bwd(const uint16_t *dy, const void *x, int src, const float *weight, const float *rstd_in,
+                                   int64_t rows, int64_t cols, void *dx, float *dweight) {
+    const int64_t nchunk = cols / 8;
+    double *dw = (double *)calloc((size_t)cols, sizeof(double));
+    for (int64_t r = 0; r < rows; ++r) {
+        const float rstd = rstd_in[r];
+        float acc[64];
+        for (int l = 0; l < 64; ++l) {
+            float a = 0.0f;
+            for (int64_t c = l; c < nchunk; c += 64)
+                for (int e = 0; e < 8; ++e) {
+                    int64_t idx = r * cols + c * 8 + e;
+                    float xv = src == 0 ? bf16_to_f32(((const uint16_t *)x)[idx]) : ((const float *)x)[idx];
+                    float xh = xv * rstd;
+                    float t = bf16_to_f32(dy[idx]) * weight[c * 8 + e];
+                    a = fmaf(t, xh, a);
+                }
+            acc[l] = a;
+        }
+        for (int off = 32; off > 0; off >>= 1) {
+            float nxt[64];
+            for (int l = 0; l < 64; ++l) nxt[l] = acc[l] + acc[l ^ off];
+            memcpy(acc, nxt, sizeof(acc));
+        }
+        const float cmean = acc[0] / (float)cols;
+        for (int64_t c = 0; c < cols; ++c) {
+            int64_t idx = r * cols + c;
+            float xv = src == 0 ? bf16_to_f32(((const uint16_t *)x)[idx]) : ((const float *)x)[idx];
+            float xh = xv * rstd;
+            float d = bf16_to_f32(dy[idx]);
+            float o = rstd * fmaf(-xh, cmean, d * weight[c]);
+            if (src == 0) ((uint16_t *)dx)[idx] = f32_to_bf16(o); else ((float *)dx)[idx] = o;
+            dw[c] += (double)d * (double)xh;
+        }
+    }
+    for (int64_t c = 0; c < cols; ++c) dweight[c] = (float)dw[c];
+    free(dw);
 }

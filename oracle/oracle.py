@@ -70,6 +70,7 @@ def lib() -> ctypes.CDLL:
         L.oracle_swiglu_fwd.argtypes = [vp, vp, i64, vp]
         L.oracle_swiglu_bwd.argtypes = [vp, vp, vp, i64, vp, vp]
         L.oracle_rmsnorm.argtypes = [vp, i32, vp, i64, i64, f32, vp, vp]
+        L.oracle_rmsnorm_bwd.argtypes = [vp, vp, i32, vp, vp, i64, i64, vp, vp]
         _lib = L
     return _lib
 
@@ -202,6 +203,23 @@ def c_rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float):
     rstd = np.empty(rows, dtype=np.float32)
     lib().oracle_rmsnorm(_p(xs), src, _p(w), rows, cols, float(eps), _p(y), _p(rstd))
     return _from_bf16_bits(y, x.shape), torch.from_numpy(rstd).reshape(x.shape[:-1])
+
+
+def c_rmsnorm_bwd(dy: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, rstd: torch.Tensor):
+    """-> (dx in the dtype of x, d_weight fp32); dy bf16."""
+    cols = x.shape[-1]
+    rows = x.numel() // cols
+    d = _bf16_bits(dy)
+    if x.dtype == torch.bfloat16:
+        xs, src, dx = _bf16_bits(x), 0, np.empty(rows * cols, dtype=np.uint16)
+    else:
+        xs, src, dx = np.ascontiguousarray(x.detach().float().cpu().numpy()).reshape(-1), 1, np.empty(rows * cols, dtype=np.float32)
+    w = np.ascontiguousarray(weight.detach().float().cpu().numpy())
+    rs = np.ascontiguousarray(rstd.detach().float().cpu().numpy().reshape(-1))
+    dw = np.empty(cols, dtype=np.float32)
+    lib().oracle_rmsnorm_bwd(_p(d), _p(xs), src, _p(w), _p(rs), rows, cols, _p(dx), _p(dw))
+    dx_t = _from_bf16_bits(dx, x.shape) if src == 0 else torch.from_numpy(dx).reshape(x.shape)
+    return dx_t, torch.from_numpy(dw)
 
 
 def t_amax(x: torch.Tensor, mode: int = SCALE_TENSOR) -> torch.Tensor:

@@ -166,3 +166,28 @@ def test_rmsnorm_exact_case_and_refusals(N):
         N.rmsnorm_amax_parts(torch.zeros((1, 32768), dtype=torch.bfloat16).cuda(), torch.ones(32768).cuda(), 1e-5)
     with pytest.raises(N.NativeError, match="weight"):
         N.rmsnorm_amax_parts(torch.zeros((4, 16), dtype=torch.bfloat16).cuda(), torch.ones(8).cuda(), 1e-5)
+
+
+@pytest.mark.parametrize("cols", [8, 64, 520, 4096, 8192])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("rows", [1, 37, 2100])
+def test_rmsnorm_backward(N, rows, cols, dtype):
+    if rows == 2100 and cols > 520:
+        pytest.skip("covered by the narrower cases; keeps the oracle's run short")
+    gen = torch.Generator().manual_seed(rows * 7 + cols)
+    x = (torch.randn((rows, cols), generator=gen) * 2.0).to(dtype)
+    w = torch.randn(cols, generator=gen) * 0.3 + 1.0
+    dy = (torch.randn((rows, cols), generator=gen) * 1e-2).bfloat16()
+    _, rstd = O.c_rmsnorm(x, w, 1e-5)
+    dx, dw = N.rmsnorm_bwd(dy.cuda(), x.cuda(), w.cuda(), rstd.cuda())
+    wdx, wdw = O.c_rmsnorm_bwd(dy, x, w, rstd)
+    if dtype == torch.bfloat16:
+        assert_bf16_equal(dx, wdx, f"rmsnorm dx {rows}x{cols}")                  # bit for bit
+    else:
+        assert_f32_bits_equal(dx, wdx, f"rmsnorm dx fp32 {rows}x{cols}")
+    # d_weight: fp32 partial sums in a fixed order on the device, double in the oracle: 1e-5 of the largest entry
+    err = (dw.cpu().double() - wdw.double()).abs().max().item()
+    assert err <= 1e-5 * max(wdw.abs().max().item(), 1e-30), (err, wdw.abs().max().item())
+    dx2, dw2 = N.rmsnorm_bwd(dy.cuda(), x.cuda(), w.cuda(), rstd.cuda())
+    assert torch.equal(dw, dw2) and torch.equal(dx.view(torch.int16 if dtype == torch.bfloat16 else torch.int32),
+                                                dx2.view(torch.int16 if dtype == torch.bfloat16 else torch.int32))

@@ -179,3 +179,47 @@ def test_rmsnorm_summation_order_is_the_documented_one():
         mean = np.float32(acc[0] / np.float32(cols))
         want = np.float32(1.0) / np.sqrt(np.float32(mean + np.float32(eps)), dtype=np.float32)
         assert rstd[r].item() == want
+
+
+@pytest.mark.parametrize("cols", [8, 520, 2048])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_rmsnorm_backward_against_torch_autograd(cols, dtype):
+    rows, eps = 21, 1e-5
+    g = torch.Generator().manual_seed(cols + 7)
+    x = (torch.randn((rows, cols), generator=g) * 2.0).to(dtype)
+    w = torch.randn(cols, generator=g) * 0.5 + 1.0
+    dy = (torch.randn((rows, cols), generator=g) * 1e-2).bfloat16()
+    _, rstd = O.c_rmsnorm(x, w, eps)
+    dx, dw = O.c_rmsnorm_bwd(dy, x, w, rstd)
+    # autograd through the reference module's expression (layer_norms.py:86-119), in float64
+    xa = x.double().requires_grad_(True)
+    wa = w.double().requires_grad_(True)
+    y = (xa * torch.rsqrt(xa.pow(2).mean(-1, keepdim=True) + eps)) * wa
+    y.backward(dy.double())
+    assert dx.dtype == dtype
+    scale = xa.grad.abs().max().item()
+    tol = 2.0 ** -8 if dtype == torch.bfloat16 else 1e-5             # half a bf16 unit at the top of the range / fp32 noise
+    assert (dx.double() - xa.grad).abs().max().item() <= tol * scale
+    assert ((dw.double() - wa.grad).abs() / wa.grad.abs().max()).max().item() < 1e-5
+
+
+def test_rmsnorm_backward_exact_case():
+    # x[r, :] = +-2^r, weight = 1, eps = 0: xh = +-1, rstd = 2^-r.  With dy = xh * 2^-3 the projection
+    # removes everything: t = dy, c = mean(dy * xh) = 2^-3, dx = rstd * (dy - xh * 2^-3) = 0 exactly;
+    # d_weight[col] = sum_r dy * xh = rows * 2^-3
+    rows, cols = 5, 64
+    sign = torch.where(torch.arange(cols) % 2 == 0, -1.0, 1.0)
+    x = torch.stack([sign * 2.0 ** r for r in range(rows)]).bfloat16()
+    w = torch.ones(cols)
+    _, rstd = O.c_rmsnorm(x, w, 0.0)
+    dy = (sign * 0.125).bfloat16().expand(rows, cols).contiguous()
+    dx, dw = O.c_rmsnorm_bwd(dy, x, w, rstd)
+    assert torch.all(dx.float() == 0)
+    assert torch.equal(dw, torch.full((cols,), rows * 0.125))
+    # a gradient along one column only: dx[r, k] = rstd * (w_k dy - xh_k * xh_k w_k dy / cols) for that column
+    dy = torch.zeros((rows, cols), dtype=torch.bfloat16)
+    dy[:, 3] = 1.0
+    dx, dw = O.c_rmsnorm_bwd(dy, x, w, rstd)
+    want3 = torch.tensor([2.0 ** -r * (1 - 1 / cols) for r in range(rows)]).bfloat16()
+    assert torch.equal(dx[:, 3], want3)
+    assert torch.equal(dw, torch.nn.functional.one_hot(torch.tensor(3), cols).float() * rows * sign[3])
