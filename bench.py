@@ -123,6 +123,7 @@ def standalone_hbm(torch, native, iters=24):
         kernels = {
             "amax": (lambda x: native.amax_parts(x), 2 * E),
             "amax_rowwise": (lambda x: native.amax(x, native.SCALE_ROW), 2 * E + 4 * rows),
+            "amax_and_column_sums": (lambda x: native.amax_parts_colsum(x), 2 * E + 4 * cols),
             "cast": (lambda x: native.cast(x, scale, native.E4M3, native.SCALE_TENSOR), 3 * E),
             "cast_transpose": (lambda x: native.cast_transpose(x, scale, native.E4M3, native.SCALE_TENSOR), 4 * E),
             "amax_then_cast_transpose": (lambda x: native.quantize_dynamic(x, native.E4M3, 0), 6 * E),

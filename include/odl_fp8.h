@@ -104,6 +104,19 @@ int odl_fp8_cast_dynamic(const void *x, int src_dtype, int64_t rows, int64_t col
                          odl_stream_t stream);
 
 /*
+ * odl_fp8_amax_parts that also adds up the columns: colsum[c] = sum over rows of x[r, c] in fp32.
+ * For the grad_output of a Linear with a bias, whose bias gradient is that sum (the `db` of
+ * te.pytorch.Linear's backward, transformer_engine.py:97-108): dY is read by this pass and by the
+ * cast, not a third time.  The sum is formed from per-lane, per-block and per-slab partial sums in
+ * a fixed order (reproducible on one device).  rows, cols > 0; cols a multiple of 8 (bf16) / 4
+ * (fp32) and at most 512 * 256 (bf16) / 512 * 128 (fp32).
+ * workspace: ODL_FP8_COLSUM_WORKSPACE floats of device memory, contents irrelevant.
+ */
+#define ODL_FP8_COLSUM_WORKSPACE (512 * 256)
+int odl_fp8_amax_parts_colsum(const void *x, int src_dtype, int64_t rows, int64_t cols, float *parts,
+                              float *colsum, float *workspace, odl_stream_t stream);
+
+/*
  * The rowwise recipe needs every tensor twice: scaled per row for the GEMM that contracts
  * its columns, and scaled per column, transposed, for the GEMM that contracts its rows.
  *   odl_fp8_amax_rowcol: amax_row[rows] and amax_col[cols] in one pass over x;

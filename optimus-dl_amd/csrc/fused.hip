@@ -350,6 +350,74 @@ __global__ __launch_bounds__(1024) void rmsnorm_bwd_reduce_kernel(const float *_
     }
 }
 
+// ------------------------------------------------ partial maxima + column sums in one pass
+// For the grad_output of a Linear with a bias: the amax pass of its quantisation also adds up the
+// columns (the bias gradient), so dY is not read a third time.  Block = 32 column-lanes (8 bf16 /
+// 4 fp32 columns each) x 32 row-lanes; a lane adds its columns over rows ty, ty + 32, ... of the
+// block's row slab in fp32, the 32 row-lanes are combined through LDS in order, and the block
+// writes one slab row of column sums; rmsnorm_bwd_reduce_kernel adds the slabs in order.
+template <int SRC>
+__global__ __launch_bounds__(kFusedThreads) void amax_colsum_kernel(const void *__restrict__ x, int64_t rows, int64_t cols,
+                                                                     int rows_per_block, float *__restrict__ parts,
+                                                                     float *__restrict__ slabs) {
+    constexpr int ESZ = SRC == ODL_BF16 ? 2 : 4;
+    constexpr int CPL = 16 / ESZ;                 // columns per lane
+    constexpr int CW = 32 * CPL;                  // columns per block
+    __shared__ float sums[32][CW + 1];
+    __shared__ uint32_t red[kFusedThreads / kWave];
+    const int tx = threadIdx.x % 32, ty = threadIdx.x / 32;
+    const int64_t c0 = (int64_t)blockIdx.x * CW + tx * CPL;
+    const int64_t r0 = (int64_t)blockIdx.y * rows_per_block;
+    const int64_t r1 = r0 + rows_per_block < rows ? r0 + rows_per_block : rows;
+    const bool col_ok = c0 + CPL <= cols;          // host guarantees cols % CPL == 0
+    float acc[CPL];
+#pragma unroll
+    for (int j = 0; j < CPL; ++j) acc[j] = 0.0f;
+    uint32_t am = 0;
+    const char *base = reinterpret_cast<const char *>(x);
+    auto take = [&](const u32x4 v) {
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            if constexpr (SRC == ODL_BF16) {
+                acc[2 * q] = __fadd_rn(acc[2 * q], bf16_lo(w[q]));
+                acc[2 * q + 1] = __fadd_rn(acc[2 * q + 1], bf16_hi(w[q]));
+                am = max_u16x2(am, abs_bf16x2(w[q]));
+            } else {
+                acc[q] = __fadd_rn(acc[q], bits_to_float(w[q]));
+                am = max(am, w[q] & 0x7fffffffu);
+            }
+        }
+    };
+    if (col_ok) {
+        int64_t r = r0 + ty;
+        for (; r + 96 < r1; r += 128) {
+            u32x4 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = *reinterpret_cast<const u32x4 *>(base + ((r + 32 * u) * cols + c0) * ESZ);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) take(v[u]);
+        }
+        for (; r < r1; r += 32) take(*reinterpret_cast<const u32x4 *>(base + (r * cols + c0) * ESZ));
+    }
+#pragma unroll
+    for (int j = 0; j < CPL; ++j) sums[ty][tx * CPL + j] = acc[j];
+    if constexpr (SRC == ODL_BF16) am = fold_u16x2_to_f32bits(am);
+    am = block_max_u32(am, red);                   // has the barrier that also publishes sums[][]
+    const int64_t slab = blockIdx.y;
+    for (int c = threadIdx.x; c < CW; c += kFusedThreads) {
+        float t = sums[0][c];
+#pragma unroll
+        for (int y = 1; y < 32; ++y) t = __fadd_rn(t, sums[y][c]);
+        const int64_t col = (int64_t)blockIdx.x * CW + c;
+        if (col < cols) slabs[slab * cols + col] = t;
+    }
+    const int bid = blockIdx.y * gridDim.x + blockIdx.x, nblk = gridDim.x * gridDim.y;
+    if (threadIdx.x == 0) parts[bid] = bits_to_float(am);
+    if (bid == 0)
+        for (int j = nblk + threadIdx.x; j < kParts; j += kFusedThreads) parts[j] = 0.0f;
+}
+
 static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 // at most two fat blocks per CU, and never more blocks than there are partial maxima
@@ -452,4 +520,24 @@ extern "C" int odl_fp8_rmsnorm_bwd(const void *dy, const void *x, int src_dtype,
 #undef ODL_RMSB
     hipLaunchKernelGGL(rmsnorm_bwd_reduce_kernel, dim3((unsigned)((cols + 63) / 64)), dim3(1024), 0, stream, workspace, (int)g, cols, dweight);
     return check_launch("odl_fp8_rmsnorm_bwd");
+}
+
+extern "C" int odl_fp8_amax_parts_colsum(const void *x, int src_dtype, int64_t rows, int64_t cols, float *parts, float *colsum,
+                                         float *workspace, odl_stream_t stream_) {
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    if (rows <= 0 || cols <= 0) return set_error(ODL_ERR_ARG, "odl_fp8_amax_parts_colsum: empty or negative shape");
+    if (!x || !parts || !colsum || !workspace) return set_error(ODL_ERR_ARG, "odl_fp8_amax_parts_colsum: null pointer");
+    if (src_dtype != ODL_BF16 && src_dtype != ODL_F32) return set_error(ODL_ERR_ARG, "odl_fp8_amax_parts_colsum: src_dtype %d", src_dtype);
+    const int cpl = src_dtype == ODL_BF16 ? 8 : 4, cw = 32 * cpl;
+    const int64_t col_blocks = (cols + cw - 1) / cw;
+    if (cols % cpl != 0 || !aligned16(x) || col_blocks > kParts)
+        return set_error(ODL_ERR_SHAPE, "odl_fp8_amax_parts_colsum: cols must be a multiple of %d and at most %d, x 16-byte aligned", cpl, kParts * cw);
+    int64_t slabs = kParts / col_blocks;                      // one partial maximum per block
+    int64_t rpb = (rows + slabs - 1) / slabs;
+    rpb = ((rpb + 31) / 32) * 32;
+    slabs = (rows + rpb - 1) / rpb;
+    if (src_dtype == ODL_BF16) hipLaunchKernelGGL((amax_colsum_kernel<ODL_BF16>), dim3((unsigned)col_blocks, (unsigned)slabs), dim3(kFusedThreads), 0, stream, x, rows, cols, (int)rpb, parts, workspace);
+    else hipLaunchKernelGGL((amax_colsum_kernel<ODL_F32>), dim3((unsigned)col_blocks, (unsigned)slabs), dim3(kFusedThreads), 0, stream, x, rows, cols, (int)rpb, parts, workspace);
+    hipLaunchKernelGGL(rmsnorm_bwd_reduce_kernel, dim3((unsigned)((cols + 63) / 64)), dim3(1024), 0, stream, workspace, (int)slabs, cols, colsum);
+    return check_launch("odl_fp8_amax_parts_colsum");
 }

@@ -65,10 +65,12 @@ class _WeightCache:
 
 
 def _quantise_dynamic(x2d: torch.Tensor, fmt: int, margin: int, need_t: bool, need_rowmajor: bool = True,
-                      recipe: FP8Recipe | None = None):
+                      recipe: FP8Recipe | None = None, parts: torch.Tensor | None = None):
     """Per-tensor current scaling: amax pass, scale, cast (+transpose) pass.  The amax pass is
-    skipped when the kernel that produced x2d left its partial maxima with the recipe."""
-    parts = recipe.take_parts(x2d) if recipe is not None else None
+    skipped when the caller has the partial maxima, or when the kernel that produced x2d left them
+    with the recipe."""
+    if parts is None and recipe is not None:
+        parts = recipe.take_parts(x2d)
     q, q_t, amax, _, scale_inv = native.quantize_dynamic(x2d, fmt, margin, want_rowmajor=need_rowmajor or not need_t,
                                                         want_transposed=need_t, parts=parts)
     return q, q_t, scale_inv, amax
@@ -205,8 +207,13 @@ class _Fp8LinearFn(torch.autograd.Function):
                     meta = module._meta(recipe, dy2d.device, "bwd")
                     gq, gq_t, sg_inv = _quantise_delayed(dy2d, pol.fmt_bwd, meta, ROLE_G, fp8_wgrad, ctx.need_dgrad)
                 else:
+                    parts = recipe.take_parts(dy2d)
+                    if parts is None and ctx.has_bias and native.colsum_supported(dy2d):
+                        # the amax pass also adds up the columns: the bias gradient costs no extra read of dy
+                        parts, colsum = native.amax_parts_colsum(dy2d)
+                        db = colsum.to(ctx.bias_dtype)
                     gq, gq_t, sg_inv, _ = _quantise_dynamic(dy2d, pol.fmt_bwd, pol.margin, fp8_wgrad, ctx.need_dgrad,
-                                                            recipe=recipe)
+                                                            parts=parts)
             if ctx.need_dgrad:
                 dx = native.gemm_nt(gq, saved["wq_t"], pol.fmt_bwd, pol.fmt_fwd, sg_inv, saved["sw_inv_t"],
                                     out_dtype=ctx.x_dtype)
@@ -215,7 +222,7 @@ class _Fp8LinearFn(torch.autograd.Function):
                                     out_dtype=ctx.w_dtype)
         if ctx.need_wgrad and not recipe.wgrad:
             dw = (dy2d.t().to(saved["x_hp"].dtype) @ saved["x_hp"]).to(ctx.w_dtype)
-        if ctx.has_bias:
+        if ctx.has_bias and db is None:
             db = dy2d.sum(dim=0, dtype=torch.float32).to(ctx.bias_dtype)
         return dx, dw, db, None, None, None
 

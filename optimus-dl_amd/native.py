@@ -37,6 +37,7 @@ EXPORTS = (
     "odl_fp8_amax_scale",
     "odl_fp8_amax_parts",
     "odl_fp8_cast_dynamic",
+    "odl_fp8_amax_parts_colsum",
     "odl_fp8_swiglu_amax_parts",
     "odl_fp8_swiglu_bwd_amax_parts",
     "odl_fp8_rmsnorm_amax_parts",
@@ -87,6 +88,7 @@ def load() -> ctypes.CDLL:
         L.odl_fp8_amax_scale.argtypes = [vp, i32, i64, i64, i32, i32, vp, vp, vp, vp, vp]
         L.odl_fp8_amax_parts.argtypes = [vp, i32, i64, i64, vp, vp]
         L.odl_fp8_cast_dynamic.argtypes = [vp, i32, i64, i64, vp, i32, i32, vp, vp, vp, vp]
+        L.odl_fp8_amax_parts_colsum.argtypes = [vp, i32, i64, i64, vp, vp, vp, vp]
         L.odl_fp8_swiglu_amax_parts.argtypes = [vp, vp, i64, i64, vp, vp, vp]
         L.odl_fp8_swiglu_bwd_amax_parts.argtypes = [vp, vp, vp, i64, i64, vp, vp, vp, vp, vp]
         L.odl_fp8_rmsnorm_amax_parts.argtypes = [vp, i32, vp, i64, i64, ctypes.c_float, vp, vp, vp, vp]
@@ -201,6 +203,29 @@ def amax_parts(x: torch.Tensor) -> torch.Tensor:
     parts = torch.empty(AMAX_PARTS, dtype=torch.float32, device=x.device)
     _check(load().odl_fp8_amax_parts(x.data_ptr(), _src_dtype(x), rows, cols, parts.data_ptr(), _stream()), "odl_fp8_amax_parts")
     return parts
+
+
+COLSUM_WORKSPACE = 512 * 256
+
+
+def colsum_supported(x: torch.Tensor) -> bool:
+    """Shapes :func:`amax_parts_colsum` takes (others: amax_parts and a separate sum)."""
+    if x.dim() != 2 or x.numel() == 0 or x.dtype not in (torch.bfloat16, torch.float32):
+        return False
+    cpl = 8 if x.dtype == torch.bfloat16 else 4
+    return x.shape[1] % cpl == 0 and x.shape[1] <= AMAX_PARTS * 32 * cpl and x.is_contiguous() and x.data_ptr() % 16 == 0
+
+
+def amax_parts_colsum(x: torch.Tensor):
+    """Partial maxima of |x| and the fp32 column sums of x in one pass.  -> (parts, colsum[cols])."""
+    x = _as_2d(x)
+    rows, cols = x.shape
+    parts = torch.empty(AMAX_PARTS, dtype=torch.float32, device=x.device)
+    colsum = torch.empty(cols, dtype=torch.float32, device=x.device)
+    ws = torch.empty(COLSUM_WORKSPACE, dtype=torch.float32, device=x.device)
+    _check(load().odl_fp8_amax_parts_colsum(x.data_ptr(), _src_dtype(x), rows, cols, parts.data_ptr(), colsum.data_ptr(),
+                                            ws.data_ptr(), _stream()), "odl_fp8_amax_parts_colsum")
+    return parts, colsum
 
 
 def cast_dynamic(x: torch.Tensor, parts: torch.Tensor, fmt: int, margin: int = 0, want_rowmajor: bool = True,

@@ -189,3 +189,37 @@ def test_rmsnorm_backward(N, rows, cols, dtype):
     dx2, dw2 = N.rmsnorm_bwd(dy.cuda(), x.cuda(), w.cuda(), rstd.cuda())
     assert torch.equal(dw, dw2) and torch.equal(dx.view(torch.int16 if dtype == torch.bfloat16 else torch.int32),
                                                 dx2.view(torch.int16 if dtype == torch.bfloat16 else torch.int32))
+
+
+# ------------------------------------------------- partial maxima + column sums (bias gradient)
+@pytest.mark.parametrize("shape", [(1, 8), (33, 256), (1000, 264), (4096, 768), (777, 3072), (64, 14336)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_amax_parts_colsum(N, shape, dtype):
+    x = seeded_bf16(shape, 1e-2, sum(shape)).to(dtype)
+    x[shape[0] // 2, shape[1] // 3] = -3.5
+    parts, colsum = N.amax_parts_colsum(x.cuda())
+    assert_f32_bits_equal(parts_max(parts).reshape(1), x.float().abs().max().reshape(1), f"colsum parts {shape}")
+    assert_f32_bits_equal(parts_max(parts).reshape(1), parts_max(N.amax_parts(x.cuda())).reshape(1), "same maximum as amax_parts")
+    want = x.double().sum(0)
+    # fp32 partial sums in a fixed order against a double-precision sum: 1e-5 of sum |x| per column
+    bound = 1e-5 * x.double().abs().sum(0) + 1e-30
+    assert bool(((colsum.cpu().double() - want).abs() <= bound).all())
+    _, again = N.amax_parts_colsum(x.cuda())
+    assert torch.equal(colsum, again)                               # reproducible
+
+
+def test_amax_parts_colsum_exact_and_refusals(N):
+    # integers: every partial sum is exact, so the result is too, whatever the order
+    rows, cols = 515, 264
+    x = (torch.arange(rows * cols).reshape(rows, cols) % 7 - 3).bfloat16()
+    _, colsum = N.amax_parts_colsum(x.cuda())
+    assert torch.equal(colsum.cpu(), x.float().sum(0))
+    z = torch.zeros((16, 16), dtype=torch.bfloat16)
+    z[3, 4] = float("nan")
+    parts, colsum = N.amax_parts_colsum(z.cuda())
+    assert torch.isnan(parts_max(parts)) and torch.isnan(colsum[4]) and colsum[5].item() == 0.0
+    with pytest.raises(N.NativeError, match="multiple of"):
+        N.amax_parts_colsum(torch.zeros((4, 12), dtype=torch.bfloat16).cuda())
+    assert not N.colsum_supported(torch.zeros((4, 12), dtype=torch.bfloat16).cuda())
+    assert not N.colsum_supported(torch.zeros((0, 16), dtype=torch.bfloat16).cuda())
+    assert N.colsum_supported(torch.zeros((4, 16), dtype=torch.bfloat16).cuda())

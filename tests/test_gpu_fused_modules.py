@@ -222,3 +222,36 @@ def test_llama_block_with_fusions_trains_like_the_unfused_one(amp, recipe_name):
         traces[fuse] = trace
     assert traces[True][-1] < traces[True][0] - 0.3, traces
     assert abs(traces[True][-1] - traces[False][-1]) < 0.15, traces
+
+
+def test_bias_gradient_comes_out_of_the_amax_pass(amp, monkeypatch):
+    from optimus_dl_amd import native
+    from optimus_dl_amd.modules.fp8_linear import FP8Linear
+
+    M, K, Nn = 320, 256, 768
+    torch.manual_seed(0)
+    lin = FP8Linear.from_linear(nn.Linear(K, Nn, bias=True).to("cuda", torch.bfloat16))
+    x = seeded_bf16((M, K), 1.0, 1).cuda().requires_grad_(True)
+    dy = seeded_bf16((M, Nn), 1e-2, 2)
+    recipe = amp.FP8Recipe(recipe_type="tensorwise")
+    amax_calls = count_calls(monkeypatch, native, "amax_parts")
+    colsum_calls = count_calls(monkeypatch, native, "amax_parts_colsum")
+    with recipe.autocast():
+        y = lin(x)
+    with recipe.backward():
+        y.backward(dy.cuda())
+    assert colsum_calls == [(M, Nn)] and (M, Nn) not in amax_calls
+    want = dy.double().sum(0)
+    got = lin.bias.grad.float().cpu().double()
+    assert lin.bias.grad.dtype == torch.bfloat16
+    assert ((got - want).abs() <= 2.0 ** -8 * want.abs() + 1e-6).all()           # one bf16 rounding of an fp32 sum
+    # the codes are those of the plain route: same dx, dw as a bias-free twin fed the same tensors
+    twin = FP8Linear.from_linear(nn.Linear(K, Nn, bias=False).to("cuda", torch.bfloat16))
+    with torch.no_grad():
+        twin.weight.copy_(lin.weight)
+    x2 = x.detach().clone().requires_grad_(True)
+    with recipe.autocast():
+        y2 = twin(x2)
+    with recipe.backward():
+        y2.backward(dy.cuda())
+    assert torch.equal(x.grad, x2.grad) and torch.equal(lin.weight.grad, twin.weight.grad)
