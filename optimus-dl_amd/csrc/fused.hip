@@ -1,11 +1,13 @@
 // Producers of FP8 Linear inputs that also deliver the partial maxima of what they write, so
 // that the current-scaling quantisation of their output needs no amax pass of its own:
-//   SwiGLU forward   h  = silu(gate) * up                         (input of the down projection)
-//   SwiGLU backward  d_gate, d_up from d_h                         (grad_outputs of gate / up)
-//   RMSNorm forward  y  = x * rsqrt(mean(x^2) + eps) * weight      (input of q/k/v, gate/up)
-// All three are bound by HBM bandwidth; the arithmetic is written so that a plain-C restatement
-// gives the same bits: fused multiply-adds are spelled out, nothing is left to contraction, and
-// no hardware approximation (v_exp_f32, v_rcp_f32, v_rsq_f32) is used.
+//   SwiGLU forward    h  = silu(gate) * up                        (input of the down projection)
+//   SwiGLU backward   d_gate, d_up from d_h                        (grad_outputs of gate / up)
+//   RMSNorm forward   y  = x * rsqrt(mean(x^2) + eps) * weight     (input of q/k/v, gate/up)
+// plus the RMSNorm backward and the amax pass that also yields the bias gradient (column sums).
+// All are bound by HBM bandwidth.  Elementwise results and per-row reductions are written so that
+// a plain-C restatement gives the same bits: fused multiply-adds are spelled out, nothing is left
+// to contraction, no hardware approximation (v_exp_f32, v_rcp_f32, v_rsq_f32) is used.  Sums over
+// rows (d_weight, column sums) are fp32 partial sums in a fixed order.
 #include "common.h"
 
 #pragma clang fp contract(off)

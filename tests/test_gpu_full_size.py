@@ -261,3 +261,71 @@ def test_config_2_attention_projections_forward_backward(N):
     dy_k = draw((M, 1024), 1e-3, 71)
     gq, gq_t, _, sg, sgi = native.quantize_dynamic(dy_k, O.E5M2)
     sample_check(lins["wk"].weight.grad, gq_t, xq_t, O.E5M2, O.E4M3, sgi, sxi, seed=81, what="wk wgrad", cols=256)
+
+
+# The transform swaps EVERY nn.Linear, the output head included (transformer_engine.py:501-513):
+# vocabulary-sized N that is not a multiple of the big tiles (GPT-2 50304, Qwen3-0.6B 151936).
+@pytest.mark.parametrize("M,K,V", [pytest.param(2048, 768, 50304, id="gpt2-lm_head"),
+                                   pytest.param(1024, 1024, 151936, id="qwen3-0.6b-lm_head")])
+def test_lm_head_shapes_forward_backward(N, M, K, V):
+    from optimus_dl_amd.modules import amp as A
+    from optimus_dl_amd.modules.fp8_linear import FP8Linear
+
+    x, w, dy = draw((M, K), 1.0, 11), draw((V, K), 0.02, 12), draw((M, V), 1e-3, 13)
+    lin = torch.nn.Linear(K, V, bias=False, device="cuda", dtype=torch.bfloat16)
+    with torch.no_grad():
+        lin.weight.copy_(w)
+    lin = FP8Linear.from_linear(lin)
+    recipe = A.FP8Recipe(recipe_type="tensorwise")
+    xd = x.clone().requires_grad_(True)
+    with recipe.autocast():
+        y = lin(xd)
+    with recipe.backward():
+        y.backward(dy)
+    assert lin.fp8_calls == 1
+    xq, xq_t, _, sx_inv, _ = quantise(N, x, O.E4M3)
+    wq, wq_t, _, sw_inv, _ = quantise(N, w, O.E4M3)
+    gq, gq_t, _, sg_inv, _ = quantise(N, dy, O.E5M2)
+    sample_check(y.detach(), xq, wq, O.E4M3, O.E4M3, sx_inv, sw_inv, seed=V, what="lm_head fwd")
+    sample_check(xd.grad, gq, wq_t, O.E5M2, O.E4M3, sg_inv, sw_inv, seed=V + 1, what="lm_head dgrad", cols=min(640, K))
+    sample_check(lin.weight.grad, gq_t, xq_t, O.E5M2, O.E4M3, sg_inv, sx_inv, seed=V + 2, what="lm_head wgrad", cols=min(640, K))
+
+
+def test_fused_producers_at_config_3_size(N):
+    """SwiGLU forward / backward on the [8192, 14336] activations and RMSNorm on [8192, 4096]: a sample of
+    rows against the oracle bit for bit (both are row-local), the partial maxima against the whole output."""
+    M, H, C = 8192, 14336, 4096
+    g, u, dh = draw((M, H), 1.5, 21), draw((M, H), 1.0, 22), draw((M, H), 1e-3, 23)
+    h, parts = N.swiglu_amax_parts(g, u)
+    dg, du, pg, pu = N.swiglu_bwd_amax_parts(dh, g, u)
+    ri = torch.randperm(M, generator=torch.Generator().manual_seed(5))[:24].sort().values.cuda()
+    gs, us, ds = g[ri].cpu(), u[ri].cpu(), dh[ri].cpu()
+    assert torch.equal(h[ri].cpu().view(torch.int16), O.c_swiglu_fwd(gs, us).view(torch.int16))
+    wg, wu = O.c_swiglu_bwd(ds, gs, us)
+    assert torch.equal(dg[ri].cpu().view(torch.int16), wg.view(torch.int16))
+    assert torch.equal(du[ri].cpu().view(torch.int16), wu.view(torch.int16))
+    for t, p, what in ((h, parts, "h"), (dg, pg, "d_gate"), (du, pu, "d_up")):
+        assert_f32_bits_equal(p.max().reshape(1), t.float().abs().max().reshape(1), f"partial maxima of {what}")
+    # the cast fed by the producer's maxima equals the two-launch quantisation of the same tensor
+    q, q_t, amax, scale, _ = N.cast_dynamic(h, parts, O.E4M3, 0)
+    q2, q2_t, amax2, scale2, _ = N.quantize_dynamic(h, O.E4M3, 0)
+    assert torch.equal(q, q2) and torch.equal(q_t, q2_t) and torch.equal(scale, scale2)
+    del g, u, dh, h, dg, du, q, q_t, q2, q2_t
+    for dtype in (torch.bfloat16, torch.float32):
+        x = draw((M, C), 2.0, 31).to(dtype)
+        w = torch.linspace(0.5, 1.5, C, device="cuda")
+        y, rstd, parts = N.rmsnorm_amax_parts(x, w, 1e-5)
+        dy = draw((M, C), 1e-2, 32)
+        dx, dw = N.rmsnorm_bwd(dy, x, w, rstd)
+        xs = x[ri].cpu()
+        wy, wr = O.c_rmsnorm(xs, w.cpu(), 1e-5)
+        assert torch.equal(y[ri].cpu().view(torch.int16), wy.view(torch.int16))
+        assert_f32_bits_equal(rstd[ri], wr, "rstd")
+        assert_f32_bits_equal(parts.max().reshape(1), y.float().abs().max().reshape(1), "partial maxima of y")
+        wdx, _ = O.c_rmsnorm_bwd(dy[ri].cpu(), xs, w.cpu(), wr)
+        if dtype == torch.bfloat16:
+            assert torch.equal(dx[ri].cpu().view(torch.int16), wdx.view(torch.int16))
+        else:
+            assert_f32_bits_equal(dx[ri], wdx, "dx")
+        want_dw = (dy.double() * (x.double() * rstd.double()[:, None])).sum(0)
+        assert ((dw.double() - want_dw).abs().max() / want_dw.abs().max()).item() < 1e-5
