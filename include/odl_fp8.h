@@ -188,6 +188,25 @@ int odl_fp8_rmsnorm_bwd(const void *dy, const void *x, int src_dtype, const floa
                         float *workspace, odl_stream_t stream);
 
 /*
+ * LayerNorm (F.layer_norm over the last axis, optimus_dl/modules/model/blocks/layer_norms.py:21-47
+ * and torch.nn.LayerNorm, both of which the reference's transform replaces,
+ * transformer_engine.py:338-352) with the partial maxima of its output, and its backward.
+ * Same row split and summation order as the RMSNorm entry points; 8 <= cols <= 4096.
+ *   mean = sum(x) / cols; d = x - mean; rstd = 1 / sqrt(sum(d * d) / cols + eps)  (d * d added by fma)
+ *   y    = bf16( ((d * rstd) * weight) + bias ), bias may be NULL
+ *   backward (dy bf16): xh = d * rstd, t = dy * weight, c1 = sum(t) / cols, c2 = sum(t * xh) / cols,
+ *   dx = rstd * fma(-xh, c2, t - c1) in the dtype of x; dweight = sum_rows dy * xh and
+ *   dbias = sum_rows dy, fp32, fixed-order partial sums.  dbias must be dweight + cols (one
+ *   buffer of 2 * cols floats); workspace: 2 * ODL_FP8_RMSNORM_BWD_SLABS * cols floats.
+ */
+int odl_fp8_layernorm_amax_parts(const void *x, int src_dtype, const float *weight, const float *bias,
+                                 int64_t rows, int64_t cols, float eps, void *y, float *mean,
+                                 float *rstd, float *parts, odl_stream_t stream);
+int odl_fp8_layernorm_bwd(const void *dy, const void *x, int src_dtype, const float *weight,
+                          const float *mean, const float *rstd, int64_t rows, int64_t cols, void *dx,
+                          float *dweight, float *dbias, float *workspace, odl_stream_t stream);
+
+/*
  * out[r,c] = fp8( clamp( fp32(x[r,c]) * s , +-max ) ), s = scale[0] | scale[r] | scale[c].
  * amax_out (may be NULL): *amax_out = max(*amax_out, max|x|), for delayed scaling,
  * where the cast uses an older scale while this step's amax is recorded.

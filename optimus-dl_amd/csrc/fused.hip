@@ -323,6 +323,193 @@ __global__ __launch_bounds__(kRmsBwdThreads) void rmsnorm_bwd_kernel(const u32x4
     for (int64_t c = threadIdx.x; c < cols; c += kRmsBwdThreads) slabs[(int64_t)blockIdx.x * cols + c] = lds_dw[c];
 }
 
+// ------------------------------------------------------------------------ LayerNorm
+// Same work split and summation order as the RMSNorm kernels.  Forward, per row:
+//   mean = sum(x) / cols;  d = x - mean;  rstd = 1 / sqrt(sum(d * d) / cols + eps)   (d * d by fma)
+//   y = bf16( ((d * rstd) * weight) + bias )          (bias may be absent)
+// Backward, dy in bf16:  xh = d * rstd, t = dy * weight, c1 = sum(t) / cols, c2 = sum(t * xh) / cols
+//   dx = rstd * fma(-xh, c2, t - c1);  d_weight = sum_rows dy * xh;  d_bias = sum_rows dy
+// (slabs hold d_weight in [0, cols) and d_bias in [cols, 2 cols) of each block's row).
+__device__ __forceinline__ float wave_sum_butterfly(float acc) {
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) acc = __fadd_rn(acc, __shfl_xor(acc, off, kWave));
+    return acc;
+}
+
+template <int SRC, int CPL, int THREADS>
+__global__ __launch_bounds__(THREADS) void layernorm_fwd_kernel(const void *__restrict__ x, const float *__restrict__ weight,
+                                                                 const float *__restrict__ bias, int64_t rows, int64_t cols, float eps,
+                                                                 uint16_t *__restrict__ y, float *__restrict__ mean_out,
+                                                                 float *__restrict__ rstd_out, float *__restrict__ parts) {
+    __shared__ uint32_t red[THREADS / kWave];
+    constexpr int VPC = SRC == ODL_BF16 ? 1 : 2;
+    const int lane = threadIdx.x % kWave;
+    const int64_t wave = (int64_t)blockIdx.x * (THREADS / kWave) + threadIdx.x / kWave;
+    const int64_t nwave = (int64_t)gridDim.x * (THREADS / kWave);
+    const int64_t nchunk = cols / 8;
+    uint32_t am = 0;
+    for (int64_t row = wave; row < rows; row += nwave) {
+        u32x4 raw[CPL][VPC];
+#pragma unroll
+        for (int j = 0; j < CPL; ++j) {
+            const int64_t c = lane + (int64_t)kWave * j;
+            const u32x4 *p = reinterpret_cast<const u32x4 *>(x) + (row * nchunk + c) * VPC;
+#pragma unroll
+            for (int h = 0; h < VPC; ++h) raw[j][h] = c < nchunk ? __builtin_nontemporal_load(p + h) : u32x4{0, 0, 0, 0};
+        }
+        float acc = 0.0f;
+#pragma unroll
+        for (int j = 0; j < CPL; ++j) {
+            float f[8];
+            unpack8<SRC>(raw[j], f);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc = __fadd_rn(acc, f[e]);
+        }
+        const float mean = __fdiv_rn(wave_sum_butterfly(acc), (float)cols);
+        acc = 0.0f;
+#pragma unroll
+        for (int j = 0; j < CPL; ++j) {
+            if (lane + (int64_t)kWave * j < nchunk) {      // padding chunks must not contribute (0 - mean)^2
+                float f[8];
+                unpack8<SRC>(raw[j], f);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float d = __fsub_rn(f[e], mean);
+                    acc = __fmaf_rn(d, d, acc);
+                }
+            }
+        }
+        const float var = __fdiv_rn(wave_sum_butterfly(acc), (float)cols);
+        const float rstd = __fdiv_rn(1.0f, __builtin_sqrtf(__fadd_rn(var, eps)));
+        if (lane == 0) { mean_out[row] = mean; rstd_out[row] = rstd; }
+#pragma unroll
+        for (int j = 0; j < CPL; ++j) {
+            const int64_t c = lane + (int64_t)kWave * j;
+            if (c < nchunk) {
+                float f[8], o[8];
+                unpack8<SRC>(raw[j], f);
+                const float4 w0 = *reinterpret_cast<const float4 *>(weight + c * 8), w1 = *reinterpret_cast<const float4 *>(weight + c * 8 + 4);
+                const float w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+#pragma unroll
+                for (int e = 0; e < 8; ++e) o[e] = __fmul_rn(__fmul_rn(__fsub_rn(f[e], mean), rstd), w[e]);
+                if (bias) {
+                    const float4 b0 = *reinterpret_cast<const float4 *>(bias + c * 8), b1 = *reinterpret_cast<const float4 *>(bias + c * 8 + 4);
+                    const float b[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) o[e] = __fadd_rn(o[e], b[e]);
+                }
+                uint32_t pk[4];
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    pk[q] = pack2(o[2 * q], o[2 * q + 1]);
+                    am = max_u16x2(am, abs_bf16x2(pk[q]));
+                }
+                reinterpret_cast<u32x4 *>(y)[row * nchunk + c] = u32x4{pk[0], pk[1], pk[2], pk[3]};
+            }
+        }
+    }
+    am = block_max_u32(fold_u16x2_to_f32bits(am), red);
+    if (threadIdx.x == 0) parts[blockIdx.x] = bits_to_float(am);
+    if (blockIdx.x == 0)
+        for (int j = (int)gridDim.x + threadIdx.x; j < kParts; j += THREADS) parts[j] = 0.0f;
+}
+
+template <int SRC, int CPL>
+__global__ __launch_bounds__(kRmsBwdThreads) void layernorm_bwd_kernel(const u32x4 *__restrict__ dy, const void *__restrict__ x,
+                                                                        const float *__restrict__ weight, const float *__restrict__ mean_in,
+                                                                        const float *__restrict__ rstd_in, int64_t rows, int64_t cols,
+                                                                        void *__restrict__ dx, float *__restrict__ slabs) {
+    extern __shared__ float lds_dw[];                        // 2 * cols floats: d_weight, d_bias
+    constexpr int VPC = SRC == ODL_BF16 ? 1 : 2;
+    const int lane = threadIdx.x % kWave, wave_in_block = threadIdx.x / kWave;
+    const int64_t wave = (int64_t)blockIdx.x * (kRmsBwdThreads / kWave) + wave_in_block;
+    const int64_t nwave = (int64_t)gridDim.x * (kRmsBwdThreads / kWave);
+    const int64_t nchunk = cols / 8;
+    float dw[CPL][8], db[CPL][8];
+#pragma unroll
+    for (int j = 0; j < CPL; ++j)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { dw[j][e] = 0.0f; db[j][e] = 0.0f; }
+    for (int64_t row = wave; row < rows; row += nwave) {
+        u32x4 xr[CPL][VPC], dr[CPL];
+#pragma unroll
+        for (int j = 0; j < CPL; ++j) {
+            const int64_t c = lane + (int64_t)kWave * j;
+            const bool ok = c < nchunk;
+            const u32x4 *p = reinterpret_cast<const u32x4 *>(x) + (row * nchunk + c) * VPC;
+#pragma unroll
+            for (int h = 0; h < VPC; ++h) xr[j][h] = ok ? __builtin_nontemporal_load(p + h) : u32x4{0, 0, 0, 0};
+            dr[j] = ok ? __builtin_nontemporal_load(dy + row * nchunk + c) : u32x4{0, 0, 0, 0};
+        }
+        const float mean = mean_in[row], rstd = rstd_in[row];
+        float a1 = 0.0f, a2 = 0.0f;
+#pragma unroll
+        for (int j = 0; j < CPL; ++j) {
+            const int64_t c = lane + (int64_t)kWave * j;
+            if (c < nchunk) {
+                float xf[8], df[8];
+                unpack8<SRC>(xr[j], xf);
+                unpack8<ODL_BF16>(&dr[j], df);
+                const float4 w0 = *reinterpret_cast<const float4 *>(weight + c * 8), w1 = *reinterpret_cast<const float4 *>(weight + c * 8 + 4);
+                const float w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float xh = __fmul_rn(__fsub_rn(xf[e], mean), rstd);
+                    const float t = __fmul_rn(df[e], w[e]);
+                    a1 = __fadd_rn(a1, t);
+                    a2 = __fmaf_rn(t, xh, a2);
+                    dw[j][e] = __fmaf_rn(df[e], xh, dw[j][e]);
+                    db[j][e] = __fadd_rn(db[j][e], df[e]);
+                }
+            }
+        }
+        const float c1 = __fdiv_rn(wave_sum_butterfly(a1), (float)cols);
+        const float c2 = __fdiv_rn(wave_sum_butterfly(a2), (float)cols);
+#pragma unroll
+        for (int j = 0; j < CPL; ++j) {
+            const int64_t c = lane + (int64_t)kWave * j;
+            if (c < nchunk) {
+                float xf[8], df[8], o[8];
+                unpack8<SRC>(xr[j], xf);
+                unpack8<ODL_BF16>(&dr[j], df);
+                const float4 w0 = *reinterpret_cast<const float4 *>(weight + c * 8), w1 = *reinterpret_cast<const float4 *>(weight + c * 8 + 4);
+                const float w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float xh = __fmul_rn(__fsub_rn(xf[e], mean), rstd);
+                    o[e] = __fmul_rn(rstd, __fmaf_rn(-xh, c2, __fsub_rn(__fmul_rn(df[e], w[e]), c1)));
+                }
+                if constexpr (SRC == ODL_BF16) {
+                    reinterpret_cast<u32x4 *>(dx)[row * nchunk + c] =
+                        u32x4{pack2(o[0], o[1]), pack2(o[2], o[3]), pack2(o[4], o[5]), pack2(o[6], o[7])};
+                } else {
+                    float4 *q = reinterpret_cast<float4 *>(dx) + (row * nchunk + c) * 2;
+                    q[0] = float4{o[0], o[1], o[2], o[3]};
+                    q[1] = float4{o[4], o[5], o[6], o[7]};
+                }
+            }
+        }
+    }
+    for (int wv = 0; wv < kRmsBwdThreads / kWave; ++wv) {
+        if (wave_in_block == wv) {
+#pragma unroll
+            for (int j = 0; j < CPL; ++j) {
+                const int64_t c = lane + (int64_t)kWave * j;
+                if (c < nchunk) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        float *sw = &lds_dw[c * 8 + e], *sb = &lds_dw[cols + c * 8 + e];
+                        *sw = wv == 0 ? dw[j][e] : __fadd_rn(*sw, dw[j][e]);
+                        *sb = wv == 0 ? db[j][e] : __fadd_rn(*sb, db[j][e]);
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+    for (int64_t c = threadIdx.x; c < 2 * cols; c += kRmsBwdThreads) slabs[(int64_t)blockIdx.x * 2 * cols + c] = lds_dw[c];
+}
+
 // slabs -> d_weight: a block owns 64 columns; 16 groups of lanes each add every 16th slab (8 loads in
 // flight), the groups are combined through LDS in group order.  The order is fixed by the code.
 __global__ __launch_bounds__(1024) void rmsnorm_bwd_reduce_kernel(const float *__restrict__ slabs, int nslab, int64_t cols,
@@ -542,4 +729,57 @@ extern "C" int odl_fp8_amax_parts_colsum(const void *x, int src_dtype, int64_t r
     else hipLaunchKernelGGL((amax_colsum_kernel<ODL_F32>), dim3((unsigned)col_blocks, (unsigned)slabs), dim3(kFusedThreads), 0, stream, x, rows, cols, (int)rpb, parts, workspace);
     hipLaunchKernelGGL(rmsnorm_bwd_reduce_kernel, dim3((unsigned)((cols + 63) / 64)), dim3(1024), 0, stream, workspace, (int)slabs, cols, colsum);
     return check_launch("odl_fp8_amax_parts_colsum");
+}
+
+extern "C" int odl_fp8_layernorm_amax_parts(const void *x, int src_dtype, const float *weight, const float *bias, int64_t rows,
+                                            int64_t cols, float eps, void *y, float *mean, float *rstd, float *parts,
+                                            odl_stream_t stream_) {
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    if (rows < 0 || cols < 0) return set_error(ODL_ERR_ARG, "odl_fp8_layernorm_amax_parts: negative shape");
+    if (src_dtype != ODL_BF16 && src_dtype != ODL_F32) return set_error(ODL_ERR_ARG, "odl_fp8_layernorm_amax_parts: src_dtype %d", src_dtype);
+    if (!parts || (rows > 0 && (!rstd || !mean)) || (rows * cols > 0 && (!x || !weight || !y)))
+        return set_error(ODL_ERR_ARG, "odl_fp8_layernorm_amax_parts: null pointer");
+    if (cols < 8 || cols % 8 != 0 || cols > 4096 || !aligned16(x) || !aligned16(y) || !aligned16(weight) || !aligned16(bias))
+        return set_error(ODL_ERR_SHAPE, "odl_fp8_layernorm_amax_parts: cols must be a multiple of 8 in [8, 4096] and the pointers 16-byte aligned");
+    const int64_t cpl = (cols / 8 + kWave - 1) / kWave;
+    const int threads = cpl <= 4 ? kFusedThreads : 512;
+    const int rows_per_block = threads / kWave;
+    int64_t g = (rows + rows_per_block - 1) / rows_per_block;
+    g = g < 1 ? 1 : (g < grid_cap() ? g : grid_cap());
+#define ODL_LN(SRC, CPL, THR) hipLaunchKernelGGL((layernorm_fwd_kernel<SRC, CPL, THR>), dim3((unsigned)g), dim3(THR), 0, stream, x, weight, bias, rows, cols, eps, reinterpret_cast<uint16_t *>(y), mean, rstd, parts)
+#define ODL_LN_SRC(CPL, THR) do { if (src_dtype == ODL_BF16) ODL_LN(ODL_BF16, CPL, THR); else ODL_LN(ODL_F32, CPL, THR); } while (0)
+    if (cpl <= 2) ODL_LN_SRC(2, kFusedThreads);
+    else if (cpl <= 4) ODL_LN_SRC(4, kFusedThreads);
+    else ODL_LN_SRC(8, 512);
+#undef ODL_LN_SRC
+#undef ODL_LN
+    return check_launch("odl_fp8_layernorm_amax_parts");
+}
+
+extern "C" int odl_fp8_layernorm_bwd(const void *dy, const void *x, int src_dtype, const float *weight, const float *mean,
+                                     const float *rstd, int64_t rows, int64_t cols, void *dx, float *dweight, float *dbias,
+                                     float *workspace, odl_stream_t stream_) {
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    if (rows < 0 || cols < 0) return set_error(ODL_ERR_ARG, "odl_fp8_layernorm_bwd: negative shape");
+    if (src_dtype != ODL_BF16 && src_dtype != ODL_F32) return set_error(ODL_ERR_ARG, "odl_fp8_layernorm_bwd: src_dtype %d", src_dtype);
+    if (!dweight || !dbias || !workspace || !weight || (rows > 0 && (!rstd || !mean)) || (rows * cols > 0 && (!dy || !x || !dx)))
+        return set_error(ODL_ERR_ARG, "odl_fp8_layernorm_bwd: null pointer");
+    if (dbias != dweight + cols) return set_error(ODL_ERR_ARG, "odl_fp8_layernorm_bwd: dbias must follow dweight (dweight + cols)");
+    if (cols < 8 || cols % 8 != 0 || cols > 4096 || !aligned16(x) || !aligned16(dy) || !aligned16(dx) || !aligned16(weight))
+        return set_error(ODL_ERR_SHAPE, "odl_fp8_layernorm_bwd: cols must be a multiple of 8 in [8, 4096] and the pointers 16-byte aligned");
+    const int rows_per_block = kRmsBwdThreads / kWave;
+    int64_t g = (rows + rows_per_block - 1) / rows_per_block;
+    g = g < 1 ? 1 : (g < ODL_FP8_RMSNORM_BWD_SLABS ? g : ODL_FP8_RMSNORM_BWD_SLABS);
+    const int64_t cpl = (cols / 8 + kWave - 1) / kWave;
+    const size_t lds = (size_t)cols * 2 * sizeof(float);
+#define ODL_LNB(SRC, CPL) hipLaunchKernelGGL((layernorm_bwd_kernel<SRC, CPL>), dim3((unsigned)g), dim3(kRmsBwdThreads), lds, stream, reinterpret_cast<const u32x4 *>(dy), x, weight, mean, rstd, rows, cols, dx, workspace)
+#define ODL_LNB_SRC(CPL) do { if (src_dtype == ODL_BF16) ODL_LNB(ODL_BF16, CPL); else ODL_LNB(ODL_F32, CPL); } while (0)
+    if (cpl <= 2) ODL_LNB_SRC(2);
+    else if (cpl <= 4) ODL_LNB_SRC(4);
+    else ODL_LNB_SRC(8);
+#undef ODL_LNB_SRC
+#undef ODL_LNB
+    // slabs are rows of 2 * cols sums (d_weight, d_bias); dweight and dbias are adjacent, so one reduction writes both
+    hipLaunchKernelGGL(rmsnorm_bwd_reduce_kernel, dim3((unsigned)((2 * cols + 63) / 64)), dim3(1024), 0, stream, workspace, (int)g, 2 * cols, dweight);
+    return check_launch("odl_fp8_layernorm_bwd");
 }

@@ -140,3 +140,64 @@ def fuse_rmsnorm(norm: nn.Module) -> bool:
     cls = norm.__class__
     norm.__class__ = type(cls.__name__, (_FusedRMSNormForward, cls), {"__module__": cls.__module__})
     return True
+
+
+# ---------------------------------------------------------------------- LayerNorm
+class _LayerNormFn(torch.autograd.Function):
+    """y = layer_norm(x) * weight + bias rounded once to bf16."""
+
+    @staticmethod
+    def forward(ctx, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, eps: float, recipe: FP8Recipe):
+        y, mean, rstd, parts = native.layernorm_amax_parts(x, weight, bias, eps)
+        recipe.offer_parts(y, parts)
+        ctx.save_for_backward(x, weight, mean, rstd)
+        ctx.bias_dtype = None if bias is None else bias.dtype
+        return y
+
+    @staticmethod
+    def backward(ctx, dy: torch.Tensor):
+        x, weight, mean, rstd = ctx.saved_tensors
+        if dy.dtype != torch.bfloat16:
+            dy = dy.to(torch.bfloat16)
+        dx, dw, db = native.layernorm_bwd(dy, x, weight, mean, rstd)
+        return (dx if ctx.needs_input_grad[0] else None, dw.to(weight.dtype) if ctx.needs_input_grad[1] else None,
+                db.to(ctx.bias_dtype) if ctx.bias_dtype is not None and ctx.needs_input_grad[2] else None, None, None)
+
+
+def layernorm(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, eps: float) -> torch.Tensor | None:
+    """Fused LayerNorm when an FP8 recipe is active and the kernel takes the input; else None."""
+    recipe = _state.active_recipe()
+    if recipe is None or not x.is_cuda or x.dtype not in (torch.bfloat16, torch.float32):
+        return None
+    if x.dtype != torch.bfloat16 and not (torch.is_autocast_enabled("cuda") and torch.get_autocast_dtype("cuda") == torch.bfloat16):
+        return None
+    cols = x.shape[-1]
+    if cols % 8 or cols < 8 or cols > 4096 or weight is None or weight.numel() != cols or x.numel() == 0:
+        return None
+    return _LayerNormFn.apply(x, weight, bias, float(eps), recipe)
+
+
+class _FusedLayerNormForward:
+    """Mixed into the class of a LayerNorm over the last axis: ``torch.nn.LayerNorm`` (``normalized_shape``
+    of one dimension, affine) or the reference's bias-optional one (layer_norms.py:21-47, eps 1e-5).
+    Output dtype under an FP8 recipe: as for the fused RMSNorm."""
+
+    _odl_fused_layernorm = True
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        y = layernorm(x, self.weight, getattr(self, "bias", None), getattr(self, "eps", 1e-5))
+        return super().forward(x) if y is None else y
+
+
+def fuse_layernorm(norm: nn.Module) -> bool:
+    if getattr(norm, "_odl_fused_layernorm", False):
+        return False
+    w = getattr(norm, "weight", None)
+    if not isinstance(w, torch.Tensor) or w.dim() != 1:
+        return False                       # no affine weight, or normalisation over several axes
+    shape = getattr(norm, "normalized_shape", None)
+    if shape is not None and tuple(shape) != (w.numel(),):
+        return False
+    cls = norm.__class__
+    norm.__class__ = type(cls.__name__, (_FusedLayerNormForward, cls), {"__module__": cls.__module__})
+    return True

@@ -16,9 +16,9 @@ optimus_dl/modules/model_transforms/transformer_engine.py:
 Deviations, on purpose:
   * the replacement shares the original ``Parameter`` objects instead of copying
     them (:278-290 copies, which unties ``lm_head`` from ``wte``);
-  * ``replace_norm`` re-classes RMSNorm modules in place (same object, same keys) so that
-    their forward is the fused kernel that also feeds the next Linear's quantisation;
-    LayerNorm is left alone; ``replace_attention`` is accepted and ignored;
+  * ``replace_norm`` re-classes RMSNorm and LayerNorm modules in place (same object, same
+    keys) so that their forward is the fused kernel that also feeds the next Linear's
+    quantisation; ``replace_attention`` is accepted and ignored;
   * ``fuse_swiglu`` (an extra key, default on) does the same for SwiGLU MLPs whose three
     projections were converted: ``silu(w1 x) * w2 x`` becomes one kernel;
   * a conversion that throws is logged at WARNING (the reference logs at DEBUG).
@@ -34,7 +34,7 @@ import torch.nn as nn
 
 from ... import native
 from ..fp8_linear import FP8Linear
-from ..fused import fuse_rmsnorm, fuse_swiglu_mlp
+from ..fused import fuse_layernorm, fuse_rmsnorm, fuse_swiglu_mlp
 from . import register_model_transform
 from .base import BaseModelTransform
 from .config import ModelTransformConfig
@@ -76,6 +76,14 @@ def _convert_rmsnorm(original: nn.Module, **kwargs: Any) -> nn.Module | None:
     return original if fuse_rmsnorm(original) else None
 
 
+def _convert_layernorm(original: nn.Module, **kwargs: Any) -> nn.Module | None:
+    return original if fuse_layernorm(original) else None
+
+
+# the LayerNorm classes the reference's table names (transformer_engine.py:344-352)
+for _path in ("optimus_dl.modules.model.blocks.layer_norms.LayerNorm", "torch.nn.modules.normalization.LayerNorm"):
+    _register_replacement(_path, nn.Module, _convert_layernorm, "norm")
+
 # the reference's RMSNorm (layer_norms.py:50) and the one of this package's own blocks
 for _path in ("optimus_dl.modules.model.blocks.layer_norms.RMSNorm", "optimus_dl_amd.modules.model.blocks.RMSNorm",
               "optimus-dl_amd.modules.model.blocks.RMSNorm"):
@@ -86,7 +94,7 @@ for _path in ("optimus_dl.modules.model.blocks.layer_norms.RMSNorm", "optimus_dl
 class TransformerEngineTransformConfig(ModelTransformConfig):
     enabled: bool = True
     replace_linear: bool = True
-    replace_norm: bool = True          # RMSNorm -> fused forward (in place); LayerNorm untouched
+    replace_norm: bool = True          # RMSNorm / LayerNorm -> fused forward (in place)
     replace_attention: bool = False    # accepted, no effect here
     linear_kwargs: dict = None
     norm_kwargs: dict = None

@@ -42,6 +42,8 @@ EXPORTS = (
     "odl_fp8_swiglu_bwd_amax_parts",
     "odl_fp8_rmsnorm_amax_parts",
     "odl_fp8_rmsnorm_bwd",
+    "odl_fp8_layernorm_amax_parts",
+    "odl_fp8_layernorm_bwd",
     "odl_fp8_amax_rowcol",
     "odl_fp8_cast_rowcol",
     "odl_fp8_cast",
@@ -93,6 +95,8 @@ def load() -> ctypes.CDLL:
         L.odl_fp8_swiglu_bwd_amax_parts.argtypes = [vp, vp, vp, i64, i64, vp, vp, vp, vp, vp]
         L.odl_fp8_rmsnorm_amax_parts.argtypes = [vp, i32, vp, i64, i64, ctypes.c_float, vp, vp, vp, vp]
         L.odl_fp8_rmsnorm_bwd.argtypes = [vp, vp, i32, vp, vp, i64, i64, vp, vp, vp, vp]
+        L.odl_fp8_layernorm_amax_parts.argtypes = [vp, i32, vp, vp, i64, i64, ctypes.c_float, vp, vp, vp, vp, vp]
+        L.odl_fp8_layernorm_bwd.argtypes = [vp, vp, i32, vp, vp, vp, i64, i64, vp, vp, vp, vp, vp]
         L.odl_fp8_amax_rowcol.argtypes = [vp, i32, i64, i64, vp, vp, vp]
         L.odl_fp8_cast_rowcol.argtypes = [vp, i32, i64, i64, vp, vp, i32, i32, vp, vp, vp, vp, vp, vp, vp]
         L.odl_fp8_cast.argtypes = [vp, i32, i64, i64, vp, i32, i32, vp, vp, vp]
@@ -350,6 +354,68 @@ def rmsnorm_bwd(dy: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, rstd: t
     _check(load().odl_fp8_rmsnorm_bwd(dy.data_ptr(), x.data_ptr(), src, w.data_ptr(), rstd.data_ptr(), rows, cols, dx.data_ptr(),
                                       dw.data_ptr(), ws.data_ptr(), _stream()), "odl_fp8_rmsnorm_bwd")
     return dx, dw
+
+
+def _f32_vector(t: torch.Tensor | None, n: int, device, what: str) -> torch.Tensor | None:
+    if t is None:
+        return None
+    v = t.detach()
+    if v.dtype != torch.float32 or not v.is_contiguous() or v.data_ptr() % 16:
+        v = v.float().contiguous().clone()
+    if v.numel() != n or v.device != device:
+        raise NativeError(f"{what}: {v.numel()} elements on {v.device}, expected {n} on {device}")
+    return v
+
+
+def _dense_16(x: torch.Tensor) -> torch.Tensor:
+    if not x.is_contiguous():
+        x = x.contiguous()
+    if x.data_ptr() % 16:
+        x = x.clone(memory_format=torch.contiguous_format)
+    return x
+
+
+def layernorm_amax_parts(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, eps: float):
+    """y = bf16(layer_norm(x) * weight + bias) over the last axis, per-row mean and 1/std, and the
+    partial maxima of |y|.  x: bf16 or fp32.  -> (y bf16, mean fp32, rstd fp32, parts)."""
+    if not x.is_cuda:
+        raise NativeError(f"layernorm: the kernels run on the GPU only; got a tensor on {x.device}")
+    src = _src_dtype(x)
+    x = _dense_16(x)
+    cols = x.shape[-1]
+    rows = x.numel() // max(cols, 1)
+    w = _f32_vector(weight, cols, x.device, "layernorm weight")
+    b = _f32_vector(bias, cols, x.device, "layernorm bias")
+    y = torch.empty(x.shape, dtype=torch.bfloat16, device=x.device)
+    stats = torch.empty((2,) + tuple(x.shape[:-1]), dtype=torch.float32, device=x.device)
+    parts = torch.empty(AMAX_PARTS, dtype=torch.float32, device=x.device)
+    _check(load().odl_fp8_layernorm_amax_parts(x.data_ptr(), src, w.data_ptr(), b.data_ptr() if b is not None else None, rows, cols,
+                                               float(eps), y.data_ptr(), stats[0].data_ptr(), stats[1].data_ptr(), parts.data_ptr(),
+                                               _stream()), "odl_fp8_layernorm_amax_parts")
+    return y, stats[0], stats[1], parts
+
+
+def layernorm_bwd(dy: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, mean: torch.Tensor, rstd: torch.Tensor):
+    """Gradients of :func:`layernorm_amax_parts`'s y for grad_output dy (bf16).
+    -> (dx in the dtype of x, d_weight fp32[cols], d_bias fp32[cols])."""
+    dy = _bf16_dense(dy, "layernorm dy")
+    src = _src_dtype(x)
+    x = _dense_16(x)
+    if dy.shape != x.shape:
+        raise NativeError(f"layernorm backward: dy {tuple(dy.shape)} and x {tuple(x.shape)} differ")
+    cols = x.shape[-1]
+    rows = x.numel() // max(cols, 1)
+    w = _f32_vector(weight, cols, x.device, "layernorm weight")
+    mean, rstd = mean.contiguous(), rstd.contiguous()
+    _f32_dev(mean.reshape(-1), rows, "layernorm backward mean")
+    _f32_dev(rstd.reshape(-1), rows, "layernorm backward rstd")
+    dx = torch.empty_like(x)
+    dwb = torch.empty(2 * cols, dtype=torch.float32, device=x.device)
+    ws = torch.empty(2 * RMSNORM_BWD_SLABS * cols, dtype=torch.float32, device=x.device)
+    _check(load().odl_fp8_layernorm_bwd(dy.data_ptr(), x.data_ptr(), src, w.data_ptr(), mean.data_ptr(), rstd.data_ptr(), rows, cols,
+                                        dx.data_ptr(), dwb.data_ptr(), dwb[cols:].data_ptr(), ws.data_ptr(), _stream()),
+           "odl_fp8_layernorm_bwd")
+    return dx, dwb[:cols], dwb[cols:]
 
 
 def quantize_rowcol(x: torch.Tensor, fmt: int, margin: int = 0):

@@ -400,3 +400,89 @@ ORACLE_API void oracle_rmsnorm_bwd(const uint16_t *dy, const void *x, int src, c
     for (int64_t c = 0; c < cols; ++c) dweight[c] = (float)dw[c];
     free(dw);
 }
+
+/* LayerNorm (F.layer_norm, optimus_dl/modules/model/blocks/layer_norms.py:21-47) in the library's
+ * stated order of IEEE operations, and its backward (dx bit-exact target; d_weight / d_bias summed
+ * in double: tolerance targets).  Pinned in tests/test_oracle_fused.py against float64 closed
+ * forms, torch's F.layer_norm and autograd, and exact special cases. */
+static float lane_butterfly(float *acc) {
+    for (int off = 32; off > 0; off >>= 1) {
+        float nxt[64];
+        for (int l = 0; l < 64; ++l) nxt[l] = acc[l] + acc[l ^ off];
+        memcpy(acc, nxt, 64 * sizeof(float));
+    }
+    return acc[0];
+}
+
+static inline float load_src(const void *x, int src, int64_t idx) {
+    return src == 0 ? bf16_to_f32(((const uint16_t *)x)[idx]) : ((const float *)x)[idx];
+}
+
+ORACLE_API void oracle_layernorm(const void *x, int src, const float *weight, const float *bias, int64_t rows, int64_t cols,
+                                 float eps, uint16_t *y, float *mean_out, float *rstd_out) {
+    const int64_t nchunk = cols / 8;
+    for (int64_t r = 0; r < rows; ++r) {
+        float acc[64];
+        for (int l = 0; l < 64; ++l) {
+            float a = 0.0f;
+            for (int64_t c = l; c < nchunk; c += 64)
+                for (int e = 0; e < 8; ++e) a = a + load_src(x, src, r * cols + c * 8 + e);
+            acc[l] = a;
+        }
+        const float mean = lane_butterfly(acc) / (float)cols;
+        for (int l = 0; l < 64; ++l) {
+            float a = 0.0f;
+            for (int64_t c = l; c < nchunk; c += 64)
+                for (int e = 0; e < 8; ++e) {
+                    float d = load_src(x, src, r * cols + c * 8 + e) - mean;
+                    a = fmaf(d, d, a);
+                }
+            acc[l] = a;
+        }
+        const float var = lane_butterfly(acc) / (float)cols;
+        const float rstd = 1.0f / sqrtf(var + eps);
+        mean_out[r] = mean;
+        rstd_out[r] = rstd;
+        for (int64_t c = 0; c < cols; ++c) {
+            float o = ((load_src(x, src, r * cols + c) - mean) * rstd) * weight[c];
+            if (bias) o = o + bias[c];
+            y[r * cols + c] = f32_to_bf16(o);
+        }
+    }
+}
+
+ORACLE_API void oracle_layernorm_bwd(const uint16_t *dy, const void *x, int src, const float *weight, const float *mean_in,
+                                     const float *rstd_in, int64_t rows, int64_t cols, void *dx, float *dweight, float *dbias) {
+    const int64_t nchunk = cols / 8;
+    double *dw = (double *)calloc((size_t)cols * 2, sizeof(double));
+    for (int64_t r = 0; r < rows; ++r) {
+        const float mean = mean_in[r], rstd = rstd_in[r];
+        float a1[64], a2[64];
+        for (int l = 0; l < 64; ++l) {
+            float s1 = 0.0f, s2 = 0.0f;
+            for (int64_t c = l; c < nchunk; c += 64)
+                for (int e = 0; e < 8; ++e) {
+                    int64_t idx = r * cols + c * 8 + e;
+                    float xh = (load_src(x, src, idx) - mean) * rstd;
+                    float t = bf16_to_f32(dy[idx]) * weight[c * 8 + e];
+                    s1 = s1 + t;
+                    s2 = fmaf(t, xh, s2);
+                }
+            a1[l] = s1;
+            a2[l] = s2;
+        }
+        const float c1 = lane_butterfly(a1) / (float)cols;
+        const float c2 = lane_butterfly(a2) / (float)cols;
+        for (int64_t c = 0; c < cols; ++c) {
+            int64_t idx = r * cols + c;
+            float xh = (load_src(x, src, idx) - mean) * rstd;
+            float d = bf16_to_f32(dy[idx]);
+            float o = rstd * fmaf(-xh, c2, d * weight[c] - c1);
+            if (src == 0) ((uint16_t *)dx)[idx] = f32_to_bf16(o); else ((float *)dx)[idx] = o;
+            dw[c] += (double)d * (double)xh;
+            dw[cols + c] += (double)d;
+        }
+    }
+    for (int64_t c = 0; c < cols; ++c) { dweight[c] = (float)dw[c]; dbias[c] = (float)dw[cols + c]; }
+    free(dw);
+}

@@ -71,6 +71,8 @@ def lib() -> ctypes.CDLL:
         L.oracle_swiglu_bwd.argtypes = [vp, vp, vp, i64, vp, vp]
         L.oracle_rmsnorm.argtypes = [vp, i32, vp, i64, i64, f32, vp, vp]
         L.oracle_rmsnorm_bwd.argtypes = [vp, vp, i32, vp, vp, i64, i64, vp, vp]
+        L.oracle_layernorm.argtypes = [vp, i32, vp, vp, i64, i64, f32, vp, vp, vp]
+        L.oracle_layernorm_bwd.argtypes = [vp, vp, i32, vp, vp, vp, i64, i64, vp, vp, vp]
         _lib = L
     return _lib
 
@@ -220,6 +222,42 @@ def c_rmsnorm_bwd(dy: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, rstd:
     lib().oracle_rmsnorm_bwd(_p(d), _p(xs), src, _p(w), _p(rs), rows, cols, _p(dx), _p(dw))
     dx_t = _from_bf16_bits(dx, x.shape) if src == 0 else torch.from_numpy(dx).reshape(x.shape)
     return dx_t, torch.from_numpy(dw)
+
+
+def _src_array(x: torch.Tensor):
+    if x.dtype == torch.bfloat16:
+        return _bf16_bits(x), 0
+    return np.ascontiguousarray(x.detach().float().cpu().numpy()).reshape(-1), 1
+
+
+def c_layernorm(x: torch.Tensor, weight: torch.Tensor, bias, eps: float):
+    """-> (y bf16, mean fp32, rstd fp32); x bf16 or fp32, normalised over the last axis; bias may be None."""
+    cols = x.shape[-1]
+    rows = x.numel() // cols
+    xs, src = _src_array(x)
+    w = np.ascontiguousarray(weight.detach().float().cpu().numpy())
+    b = None if bias is None else np.ascontiguousarray(bias.detach().float().cpu().numpy())
+    y = np.empty(rows * cols, dtype=np.uint16)
+    mean, rstd = np.empty(rows, dtype=np.float32), np.empty(rows, dtype=np.float32)
+    lib().oracle_layernorm(_p(xs), src, _p(w), None if b is None else _p(b), rows, cols, float(eps), _p(y), _p(mean), _p(rstd))
+    lead = x.shape[:-1]
+    return _from_bf16_bits(y, x.shape), torch.from_numpy(mean).reshape(lead), torch.from_numpy(rstd).reshape(lead)
+
+
+def c_layernorm_bwd(dy: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, mean: torch.Tensor, rstd: torch.Tensor):
+    """-> (dx in the dtype of x, d_weight fp32, d_bias fp32); dy bf16."""
+    cols = x.shape[-1]
+    rows = x.numel() // cols
+    d = _bf16_bits(dy)
+    xs, src = _src_array(x)
+    dx = np.empty(rows * cols, dtype=np.uint16 if src == 0 else np.float32)
+    w = np.ascontiguousarray(weight.detach().float().cpu().numpy())
+    mu = np.ascontiguousarray(mean.detach().float().cpu().numpy().reshape(-1))
+    rs = np.ascontiguousarray(rstd.detach().float().cpu().numpy().reshape(-1))
+    dw, db = np.empty(cols, dtype=np.float32), np.empty(cols, dtype=np.float32)
+    lib().oracle_layernorm_bwd(_p(d), _p(xs), src, _p(w), _p(mu), _p(rs), rows, cols, _p(dx), _p(dw), _p(db))
+    dx_t = _from_bf16_bits(dx, x.shape) if src == 0 else torch.from_numpy(dx).reshape(x.shape)
+    return dx_t, torch.from_numpy(dw), torch.from_numpy(db)
 
 
 def t_amax(x: torch.Tensor, mode: int = SCALE_TENSOR) -> torch.Tensor:

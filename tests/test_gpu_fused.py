@@ -223,3 +223,37 @@ def test_amax_parts_colsum_exact_and_refusals(N):
     assert not N.colsum_supported(torch.zeros((4, 12), dtype=torch.bfloat16).cuda())
     assert not N.colsum_supported(torch.zeros((0, 16), dtype=torch.bfloat16).cuda())
     assert N.colsum_supported(torch.zeros((4, 16), dtype=torch.bfloat16).cuda())
+
+
+# ------------------------------------------------------------------- LayerNorm
+@pytest.mark.parametrize("rows,cols", [(1, 8), (37, 64), (2100, 64), (37, 520), (300, 768), (37, 1600), (37, 4096)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("with_bias", [True, False])
+def test_layernorm_forward_and_backward(N, rows, cols, dtype, with_bias):
+    gen = torch.Generator().manual_seed(rows * 13 + cols)
+    x = (torch.randn((rows, cols), generator=gen) * 2.0 + 0.5).to(dtype)
+    w = torch.randn(cols, generator=gen) * 0.3 + 1.0
+    b = torch.randn(cols, generator=gen) * 0.2 if with_bias else None
+    dy = (torch.randn((rows, cols), generator=gen) * 1e-2).bfloat16()
+    y, mean, rstd, parts = N.layernorm_amax_parts(x.cuda(), w.cuda(), None if b is None else b.cuda(), 1e-5)
+    wy, wm, wr = O.c_layernorm(x, w, b, 1e-5)
+    assert_f32_bits_equal(mean, wm, f"layernorm mean {rows}x{cols}")
+    assert_f32_bits_equal(rstd, wr, f"layernorm rstd {rows}x{cols}")
+    assert_bf16_equal(y, wy, f"layernorm y {rows}x{cols} {dtype}")
+    assert_f32_bits_equal(parts_max(parts).reshape(1), wy.float().abs().max().reshape(1), "layernorm parts")
+    dx, dw, db = N.layernorm_bwd(dy.cuda(), x.cuda(), w.cuda(), mean, rstd)
+    wdx, wdw, wdb = O.c_layernorm_bwd(dy, x, w, wm, wr)
+    if dtype == torch.bfloat16:
+        assert_bf16_equal(dx, wdx, f"layernorm dx {rows}x{cols}")
+    else:
+        assert_f32_bits_equal(dx, wdx, f"layernorm dx fp32 {rows}x{cols}")
+    for got, want, what in ((dw, wdw, "d_weight"), (db, wdb, "d_bias")):
+        err = (got.cpu().double() - want.double()).abs().max().item()
+        assert err <= 1e-5 * max(want.abs().max().item(), 1e-30), (what, err)
+
+
+def test_layernorm_refusals(N):
+    with pytest.raises(N.NativeError, match="multiple of 8"):
+        N.layernorm_amax_parts(torch.zeros((4, 12), dtype=torch.bfloat16).cuda(), torch.ones(12).cuda(), None, 1e-5)
+    with pytest.raises(N.NativeError, match="4096"):
+        N.layernorm_amax_parts(torch.zeros((1, 8192), dtype=torch.bfloat16).cuda(), torch.ones(8192).cuda(), None, 1e-5)

@@ -255,3 +255,49 @@ def test_bias_gradient_comes_out_of_the_amax_pass(amp, monkeypatch):
     with recipe.backward():
         y2.backward(dy.cuda())
     assert torch.equal(x.grad, x2.grad) and torch.equal(lin.weight.grad, twin.weight.grad)
+
+
+@pytest.mark.parametrize("in_dtype", [torch.float32, torch.bfloat16])
+def test_fused_layernorm_in_a_gpt2_block(amp, monkeypatch, in_dtype):
+    """nn.LayerNorm -> Linear as in a GPT-2 block: the transform re-classes the norm, the Linear takes its maxima,
+    outputs and gradients agree with the untouched norm."""
+    from optimus_dl_amd import native
+    from optimus_dl_amd.modules.model_transforms import build_model_transform
+
+    class Pre(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.ln = nn.LayerNorm(256)
+            self.c_fc = nn.Linear(256, 512)
+
+        def forward(self, x):
+            return self.c_fc(self.ln(x))
+
+    torch.manual_seed(0)
+    net = Pre().cuda()
+    with torch.no_grad():
+        net.ln.weight.copy_(torch.linspace(0.5, 1.5, 256))
+        net.ln.bias.copy_(torch.linspace(-0.2, 0.2, 256))
+    ref = Pre().cuda()
+    ref.load_state_dict(net.state_dict())
+    t = build_model_transform({"_name": "transformer_engine"})
+    t.apply(net)
+    assert t.last_replacements["LayerNorm"] == 1 and isinstance(net.ln, nn.LayerNorm)
+    build_model_transform({"_name": "transformer_engine", "replace_norm": False}).apply(ref)
+    x = (torch.randn(3, 128, 256, generator=torch.Generator().manual_seed(1)) * 2 + 0.3).to(in_dtype).cuda()
+    dy = seeded_bf16((3, 128, 512), 1e-2, 2).cuda()
+    recipe = amp.FP8Recipe(recipe_type="tensorwise")
+    amax_calls = count_calls(monkeypatch, native, "amax_parts")
+    outs = {}
+    for name, m in (("fused", net), ("plain", ref)):
+        xd = x.clone().requires_grad_(True)
+        amax_calls.clear()
+        with amp.fp8_autocast(torch.device("cuda"), recipe):
+            y = m(xd)
+        with amp.fp8_backward(recipe):
+            y.backward(dy)
+        outs[name] = (y.detach(), xd.grad.detach(), m.ln.weight.grad.detach(), m.ln.bias.grad.detach(), m.c_fc.weight.grad.detach())
+        assert ((384, 256) in amax_calls) == (name == "plain")          # the normalised activation's own amax pass
+    for a, b, tol in zip(outs["fused"], outs["plain"], (1e-2, 2e-2, 2e-2, 2e-2, 1e-2)):
+        assert max_rel_err(a, b) <= tol
+    assert outs["fused"][1].dtype == in_dtype

@@ -58,8 +58,10 @@ def test_swap_nested_in_place_and_share_parameters(monkeypatch):
     out = t.apply(m, collective=None, device=torch.device("cpu"), is_restart=False, checkpoint_manager=None)
     assert out is m
     assert isinstance(m.fc, FP8Linear) and isinstance(m.inner[0], FP8Linear) and isinstance(m.inner[2][0], FP8Linear)
-    assert type(m.sub) is MyLinear and type(m.inner[1]) is nn.LayerNorm
-    assert t.last_replacements == {"Linear": 3, "RMSNorm": 0, "LayerNorm": 0, "Attention": 0}
+    assert type(m.sub) is MyLinear
+    # the LayerNorm is the same object, still an nn.LayerNorm, with the fused forward mixed in
+    assert isinstance(m.inner[1], nn.LayerNorm) and type(m.inner[1]).__name__ == "LayerNorm" and m.inner[1]._odl_fused_layernorm
+    assert t.last_replacements == {"Linear": 3, "RMSNorm": 0, "LayerNorm": 1, "Attention": 0}
     assert m.fc.weight is w_before and m.fc.bias is b_before                 # same Parameter objects
     assert sorted(m.state_dict().keys()) == keys_before                     # no key renames
     assert m.inner[0].bias is None and m.fc.in_features == 16 and m.fc.out_features == 32 and m.fc.use_bias is True

@@ -223,3 +223,61 @@ def test_rmsnorm_backward_exact_case():
     want3 = torch.tensor([2.0 ** -r * (1 - 1 / cols) for r in range(rows)]).bfloat16()
     assert torch.equal(dx[:, 3], want3)
     assert torch.equal(dw, torch.nn.functional.one_hot(torch.tensor(3), cols).float() * rows * sign[3])
+
+
+# ------------------------------------------------------------------- LayerNorm
+@pytest.mark.parametrize("cols", [8, 520, 768, 4096])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("with_bias", [True, False])
+def test_layernorm_against_float64_and_torch(cols, dtype, with_bias):
+    rows, eps = 11, 1e-5
+    g = torch.Generator().manual_seed(cols + 3)
+    x = (torch.randn((rows, cols), generator=g) * 2.0 + 0.7).to(dtype)
+    w = torch.randn(cols, generator=g) * 0.5 + 1.0
+    b = torch.randn(cols, generator=g) * 0.2 if with_bias else None
+    y, mean, rstd = O.c_layernorm(x, w, b, eps)
+    x64 = x.double()
+    mean64 = x64.mean(-1)
+    rstd64 = 1.0 / torch.sqrt(x64.var(-1, unbiased=False) + eps)
+    assert (mean.double() - mean64).abs().max() < 1e-6 and ((rstd.double() - rstd64).abs() / rstd64).max() < 1e-6
+    want = (x64 - mean64[:, None]) * rstd64[:, None] * w.double() + (0 if b is None else b.double())
+    d = ulp_distance(y, want.float().bfloat16())
+    assert d.max() <= 1 and (d > 0).mean() < 0.01
+    ref = F.layer_norm(x.float(), (cols,), w, b, eps).bfloat16()            # the routine the reference module calls
+    d = ulp_distance(y, ref)
+    assert d.max() <= 1 and (d > 0).mean() < 0.01
+
+
+def test_layernorm_exact_case_reveals_indexing():
+    # row r holds +-2^r in equal numbers: mean 0, variance 4^r, rstd 2^-r (eps = 0): y = +-weight + bias exactly
+    rows, cols = 5, 144
+    sign = torch.where(torch.arange(cols) % 2 == 0, -1.0, 1.0)
+    x = torch.stack([sign * 2.0 ** r for r in range(rows)]).bfloat16()
+    w = torch.arange(1, cols + 1, dtype=torch.float32) / 16.0
+    b = torch.arange(cols, dtype=torch.float32) / 4.0
+    y, mean, rstd = O.c_layernorm(x, w, b, 0.0)
+    assert torch.equal(mean, torch.zeros(rows)) and torch.equal(rstd, torch.tensor([2.0 ** -r for r in range(rows)]))
+    assert torch.equal(y, (sign * w + b).bfloat16().expand(rows, cols))
+    # a constant shift changes nothing but the mean
+    y2, mean2, _ = O.c_layernorm((x.float() + 8.0).bfloat16()[:3], w, b, 0.0)
+    assert torch.equal(mean2, torch.full((3,), 8.0)) and torch.equal(y2, y[:3])
+
+
+@pytest.mark.parametrize("cols", [8, 520, 768])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_layernorm_backward_against_torch_autograd(cols, dtype):
+    rows, eps = 19, 1e-5
+    g = torch.Generator().manual_seed(cols + 11)
+    x = (torch.randn((rows, cols), generator=g) * 2.0 - 0.3).to(dtype)
+    w = torch.randn(cols, generator=g) * 0.5 + 1.0
+    b = torch.randn(cols, generator=g) * 0.1
+    dy = (torch.randn((rows, cols), generator=g) * 1e-2).bfloat16()
+    _, mean, rstd = O.c_layernorm(x, w, b, eps)
+    dx, dw, db = O.c_layernorm_bwd(dy, x, w, mean, rstd)
+    xa, wa, ba = x.double().requires_grad_(True), w.double().requires_grad_(True), b.double().requires_grad_(True)
+    F.layer_norm(xa, (cols,), wa, ba, eps).backward(dy.double())
+    scale = xa.grad.abs().max().item()
+    tol = 2.0 ** -8 if dtype == torch.bfloat16 else 1e-5
+    assert dx.dtype == dtype and (dx.double() - xa.grad).abs().max().item() <= tol * scale
+    assert ((dw.double() - wa.grad).abs() / wa.grad.abs().max()).max().item() < 1e-5
+    assert ((db.double() - ba.grad).abs() / ba.grad.abs().max()).max().item() < 1e-5
