@@ -70,7 +70,8 @@ class KernelTimer:
                 e0.record()
                 out = orig(*a, **kw)
                 e1.record()
-                self.records.setdefault(record_as, []).append((e0, e1, work_fn(*a, **kw)))
+                key = record_as(*a, **kw) if callable(record_as) else record_as
+                self.records.setdefault(key, []).append((e0, e1, work_fn(*a, **kw)))
                 return out
 
             setattr(self.native, name, timed)
@@ -79,12 +80,16 @@ class KernelTimer:
             return x.element_size()
 
         wrap("gemm_nt", lambda a, b, *r, **kw: 2.0 * a.shape[0] * b.shape[0] * a.shape[1])            # flops
+        # operands stored K-slow are [K, rows]: the product of both shapes is M * K * N * K either way
+        wrap("gemm_layouts", lambda a, b, *r, **kw: 2.0 * a.numel() * b.numel() / (a.shape[0] if r[2] else a.shape[1]),
+             record_as="gemm_nt")
         wrap("amax", lambda x, *r, **kw: float(x.numel() * esz(x)))                                       # bytes
         wrap("amax_scale", lambda x, *r, **kw: float(x.numel() * esz(x)), record_as="amax")       # amax + scale, one launch
         wrap("amax_parts", lambda x, *r, **kw: float(x.numel() * esz(x)), record_as="amax")
         wrap("cast_dynamic", lambda x, parts, fmt, margin=0, want_rowmajor=True, want_transposed=True:
              float(x.numel() * (esz(x) + int(want_rowmajor) + int(want_transposed))),
-             record_as="cast_transpose")
+             record_as=lambda x, parts, fmt, margin=0, want_rowmajor=True, want_transposed=True:
+             "cast_transpose" if want_transposed else "cast")
         wrap("cast", lambda x, *r, **kw: float(x.numel() * (esz(x) + 1)))
         wrap("cast_transpose",
              lambda x, *r, **kw: float(x.numel() * (esz(x) + (2 if kw.get("want_rowmajor", True) else 1))))

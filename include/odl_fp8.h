@@ -243,6 +243,23 @@ int odl_fp8_gemm_nt(const uint8_t *a, const uint8_t *b, int64_t M, int64_t N, in
                     void *c, int out_dtype, odl_stream_t stream);
 
 /*
+ * The same product for operands that need no transposed copy.  layout_a / layout_b say how an
+ * operand is stored: ODL_K_FAST = [rows, K] row-major (what odl_fp8_gemm_nt takes), ODL_K_SLOW =
+ * [K, rows] row-major.  With per-tensor scaling the three GEMMs of te.pytorch.Linear then read the
+ * row-major codes of X [M,K], W [N,K] and dY [M,N] directly:
+ *   fwd   Y  = X . W^T      a = X  (K_FAST), b = W  (K_FAST)
+ *   dgrad dX = dY . W       a = dY (K_FAST), b = W  (K_SLOW: contraction over N, W is [N, K])
+ *   wgrad dW = dY^T . X     a = dY (K_SLOW), b = X  (K_SLOW: contraction over M)
+ * Results equal those of odl_fp8_gemm_nt on the transposed copies bit for bit (same order of
+ * accumulation).  One scale per operand, bf16 output, no bias; M, N, K multiples of 256, K >= 512:
+ * anything else is refused with ODL_ERR_SHAPE (make the transposed copy and use odl_fp8_gemm_nt).
+ */
+enum odl_operand_layout { ODL_K_FAST = 0, ODL_K_SLOW = 1 };
+int odl_fp8_gemm_layouts(const uint8_t *a, const uint8_t *b, int64_t M, int64_t N, int64_t K,
+                         int fmt_a, int fmt_b, int layout_a, int layout_b, const float *sa_inv,
+                         const float *sb_inv, void *c, odl_stream_t stream);
+
+/*
  * Delayed-scaling bookkeeping for R tensor roles with H history slots each
  * (recipe "delayed", fp8.py:279-288; runs where the reference leaves its
  * autocast context, fp8.py:337-340,357-360).

@@ -20,6 +20,7 @@ struct GemmArgs {
     int sa_vec, sb_vec;          // 0 = one value, 1 = one per row of A / B
     int out_dtype;               // bias, when present, is fp32
     int tiles_m, tiles_n;
+    int ta = 0, tb = 0;          // operand stored [K, M] / [K, N] (contraction index slow); streaming kernel only
 };
 
 __device__ __forceinline__ int swz(int row) { return (row ^ (row >> 3)) & 7; }

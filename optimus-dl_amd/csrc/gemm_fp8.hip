@@ -169,3 +169,30 @@ extern "C" int odl_fp8_gemm_nt(const uint8_t *a, const uint8_t *b, int64_t M, in
     else launch_gemm_tiled(variant, fmt_a, fmt_b, g, stream);
     return check_launch("odl_fp8_gemm_nt");
 }
+
+extern "C" int odl_fp8_gemm_layouts(const uint8_t *a, const uint8_t *b, int64_t M, int64_t N, int64_t K, int fmt_a, int fmt_b,
+                                    int layout_a, int layout_b, const float *sa_inv, const float *sb_inv, void *c,
+                                    odl_stream_t stream_) {
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    if (!a || !b || !c || !sa_inv || !sb_inv) return set_error(ODL_ERR_ARG, "odl_fp8_gemm_layouts: null pointer");
+    if ((fmt_a != ODL_FP8_E4M3 && fmt_a != ODL_FP8_E5M2) || (fmt_b != ODL_FP8_E4M3 && fmt_b != ODL_FP8_E5M2))
+        return set_error(ODL_ERR_ARG, "odl_fp8_gemm_layouts: formats %d, %d", fmt_a, fmt_b);
+    if ((layout_a != ODL_K_FAST && layout_a != ODL_K_SLOW) || (layout_b != ODL_K_FAST && layout_b != ODL_K_SLOW))
+        return set_error(ODL_ERR_ARG, "odl_fp8_gemm_layouts: layouts %d, %d", layout_a, layout_b);
+    if ((reinterpret_cast<uintptr_t>(a) & 15) || (reinterpret_cast<uintptr_t>(b) & 15) || (reinterpret_cast<uintptr_t>(c) & 15))
+        return set_error(ODL_ERR_SHAPE, "odl_fp8_gemm_layouts: operands and output must be 16-byte aligned");
+    GemmArgs g;
+    g.a = a; g.b = b; g.c = c; g.sa = sa_inv; g.sb = sb_inv; g.bias = nullptr;
+    g.M = M; g.N = N; g.K = K;
+    g.sa_vec = 0; g.sb_vec = 0;
+    g.out_dtype = ODL_BF16;
+    g.ta = layout_a == ODL_K_SLOW;
+    g.tb = layout_b == ODL_K_SLOW;
+    const bool sizes_ok = M > 0 && N > 0 && K >= 512 && M % 256 == 0 && N % 256 == 0 && K % 256 == 0 &&
+                          (double)(M + 256) * (double)K < 2147483648.0 && (double)(N + 256) * (double)K < 2147483648.0;
+    if (!sizes_ok) return set_error(ODL_ERR_SHAPE, "odl_fp8_gemm_layouts: M, N, K must be multiples of 256 (K >= 512) and each operand under 2 GiB; got %lld x %lld x %lld", (long long)M, (long long)N, (long long)K);
+    g.tiles_m = (int)(M / 256); g.tiles_n = (int)(N / 256);
+    if (!gemm_stream_accepts(g)) return set_error(ODL_ERR_SHAPE, "odl_fp8_gemm_layouts: shape not taken by the streaming kernel");
+    launch_gemm_stream(fmt_a, fmt_b, g, cu_count(), stream);
+    return check_launch("odl_fp8_gemm_layouts");
+}

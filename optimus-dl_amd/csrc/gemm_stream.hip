@@ -55,7 +55,14 @@ constexpr int GM = 8;
 constexpr int PITCH = 128 + 8;             // slab row: 64 bf16 + 8 bytes, see phase_a_fold
 constexpr int SLAB = 32 * PITCH;           // one wave's epilogue slab
 
-template <int FA, int FB>
+// TA / TB: the operand is stored with the contraction index as the SLOW axis ([K, M] resp. [K, N]
+// row-major) instead of the fast one.  A stage then holds 128 K-rows of 256 bytes; the 1 KB loads
+// bring 4 such rows each, and fragments are read with ds_read_b64_tr_b8, which hands every lane
+// of a 16-lane group one byte column of an 8 x 16 byte block (8 consecutive K for its own row).
+// The 16-byte chunks of a K-row are placed at chunk ^ (k & 7): the 8 rows a group reads in one
+// instruction then sit in 8 different bank quads.  Same K order, same accumulation, same bits
+// as the other layout: wgrad and dgrad no longer need transposed copies of their operands.
+template <int FA, int FB, bool TA, bool TB>
 __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
     __shared__ __attribute__((aligned(1024))) uint8_t sA0[REGION];
     __shared__ __attribute__((aligned(1024))) uint8_t sB0[REGION];
@@ -88,16 +95,26 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
         tm0 = (first_m + (p % in_group) % group_rows) * BM;
         tn0 = ((p % in_group) / group_rows) * BN;
     };
-    auto rsrc_for = [&](const uint8_t *base, int row0, int64_t rows) -> v4i {
+    auto rsrc_for = [&](const uint8_t *base, int row0, int64_t rows, bool transposed) -> v4i {
+        if (transposed) {                          // [K, rows] storage: the tile starts at column row0
+            const uint64_t addr = reinterpret_cast<uint64_t>(base + row0);
+            return v4i{(int)(uint32_t)addr, (int)(uint32_t)(addr >> 32), (int)(g.K * rows - row0), 0x00020000};
+        }
         const uint64_t addr = reinterpret_cast<uint64_t>(base + (int64_t)row0 * g.K);
         return v4i{(int)(uint32_t)addr, (int)(uint32_t)(addr >> 32), (int)((rows - row0) * g.K), 0x00020000};
     };
-    int voff[LOADS];
+    // per-lane source offsets of the LOADS 1 KB loads of a stage
+    int voff_a[LOADS], voff_b[LOADS];
 #pragma unroll
     for (int j = 0; j < LOADS; ++j) {
-        const int row = (wave + j * NW) * 8 + lane / 8;
-        voff[j] = row * (int)g.K + (((lane % 8) ^ swz(row)) << 4);
+        const int row = (wave + j * NW) * 8 + lane / 8;                   // K fast: 8 rows of 128 bytes per load
+        const int nt = row * (int)g.K + (((lane % 8) ^ swz(row)) << 4);
+        const int kb = (wave + j * NW) * 4 + lane / 16;                   // K slow: 4 K-rows of 256 bytes per load
+        const int chunk = ((lane % 16) ^ (kb & 7)) << 4;
+        voff_a[j] = TA ? kb * (int)g.M + chunk : nt;
+        voff_b[j] = TB ? kb * (int)g.N + chunk : nt;
     }
+    const int kstep_a = TA ? 128 * (int)g.M : 128, kstep_b = TB ? 128 * (int)g.N : 128;   // bytes between K steps
     // one 1 KB direct-to-LDS load: 64 lanes x 16 bytes land at lds_addr + lane * 16
     auto dma = [&](const v4i &rsrc, uint32_t lds_addr, int vo, int so) {
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
@@ -105,9 +122,9 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
     };
     auto lds_addr_of = [](const uint8_t *p) { return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) uint8_t *)p; };
     // load j of a stage: j < LOADS -> operand A, else operand B
-    auto issue_one = [&](uint8_t *sa, uint8_t *sb, const v4i &da, const v4i &db, int koff, int j) {
-        if (j < LOADS) dma(da, lds_addr_of(sa) + (wave + j * NW) * 1024, voff[j], koff);
-        else dma(db, lds_addr_of(sb) + (wave + (j - LOADS) * NW) * 1024, voff[j - LOADS], koff);
+    auto issue_one = [&](uint8_t *sa, uint8_t *sb, const v4i &da, const v4i &db, int kstep, int j) {
+        if (j < LOADS) dma(da, lds_addr_of(sa) + (wave + j * NW) * 1024, voff_a[j], kstep * kstep_a);
+        else dma(db, lds_addr_of(sb) + (wave + (j - LOADS) * NW) * 1024, voff_b[j - LOADS], kstep * kstep_b);
     };
 
     int m0 = 0, n0 = 0;
@@ -126,12 +143,30 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
                 rb[e][p] = rowb * 128 + (((((2 * lg + e) ^ s0b)) ^ (4 * p)) << 4);
             }
     }
+    // K-slow layout: fragment t covers tile rows row0 + 32 t .. + 31 = the 16-byte chunks c0 + 2t, c0 + 2t + 1
+    // of a K-row; a lane of a 16-lane group addresses K-row 32 lg + (lane % 16) / 2 (+ 8p, + 64h) and the
+    // 8-byte half lane % 2 of chunk (c0 + 2t) ^ (k & 7).  c0 has bits 0 and 3 only, so the t-dependence
+    // is an XOR on the address.
+    const int tj = (lane % 16) / 2;
+    const int tra = (lg * 32 + tj) * 256 + ((((wm0 / 16) + (lr / 16)) ^ tj) << 4) + (lane % 2) * 8;
+    const int trb = (lg * 32 + tj) * 256 + ((((wn0 / 16) + (lr / 16)) ^ tj) << 4) + (lane % 2) * 8;
+    auto read_tr = [&](const uint8_t *sx, int lane_off, int t, int h) -> v8i {
+        typedef int v2i_t __attribute__((ext_vector_type(2)));
+        const uint32_t base = lds_addr_of(sx) + (uint32_t)(lane_off ^ (t << 5)) + h * 64 * 256;
+        v2i_t p[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            p[q] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i_t *)(base + q * 8 * 256));
+        return v8i{p[0].x, p[0].y, p[1].x, p[1].y, p[2].x, p[2].y, p[3].x, p[3].y};
+    };
     auto read_a = [&](const uint8_t *sa, int t, int h) -> v8i {
+        if constexpr (TA) return read_tr(sa, tra, t, h);
         const v4i lo = *reinterpret_cast<const v4i *>(sa + ra[0][h ^ (t & 1)] + t * 4096);
         const v4i hi = *reinterpret_cast<const v4i *>(sa + ra[1][h ^ (t & 1)] + t * 4096);
         return v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
     };
     auto read_b = [&](const uint8_t *sb, int u, int h) -> v8i {
+        if constexpr (TB) return read_tr(sb, trb, u, h);
         const v4i lo = *reinterpret_cast<const v4i *>(sb + rb[0][h ^ (u & 1)] + u * 4096);
         const v4i hi = *reinterpret_cast<const v4i *>(sb + rb[1][h ^ (u & 1)] + u * 4096);
         return v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
@@ -242,7 +277,7 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
     auto phase_b = [&](uint8_t *sa_cur, uint8_t *sb_cur, const uint8_t *sa_nxt, const uint8_t *sb_nxt, int kt) {
         const bool nx = kt + 2 >= KT;
         const v4i la = nx ? next_a : rsrc_a, lb = nx ? next_b : rsrc_b;
-        const int koff = (nx ? kt + 2 - KT : kt + 2) * 128;
+        const int koff = nx ? kt + 2 - KT : kt + 2;               // K step to request
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             acc[i / 4][i % 4] = mfma_32x32x64<FB, FA>(b1[i % 4], a1[i / 4], acc[i / 4][i % 4]);
@@ -260,14 +295,14 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
 
     // ---- first tile: steps 0 and 1 requested and awaited, then phase A of step 0
     tile_origin(pid, m0, n0);
-    rsrc_a = rsrc_for(g.a, m0, g.M);
-    rsrc_b = rsrc_for(g.b, n0, g.N);
+    rsrc_a = rsrc_for(g.a, m0, g.M, TA);
+    rsrc_b = rsrc_for(g.b, n0, g.N, TB);
     next_a = empty;
     next_b = empty;
 #pragma unroll
     for (int j = 0; j < 2 * LOADS; ++j) issue_one(sA0, sB0, rsrc_a, rsrc_b, 0, j);
 #pragma unroll
-    for (int j = 0; j < 2 * LOADS; ++j) issue_one(sA1, sB1, rsrc_a, rsrc_b, 128, j);
+    for (int j = 0; j < 2 * LOADS; ++j) issue_one(sA1, sB1, rsrc_a, rsrc_b, 1, j);
     __builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0)
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();
@@ -284,7 +319,7 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
         const bool has_next = next_pid < pid_end;
         int next_m0 = 0, next_n0 = 0;
         tile_origin(has_next ? next_pid : pid, next_m0, next_n0);
-        const v4i na = rsrc_for(g.a, next_m0, g.M), nb = rsrc_for(g.b, next_n0, g.N);
+        const v4i na = rsrc_for(g.a, next_m0, g.M, TA), nb = rsrc_for(g.b, next_n0, g.N, TB);
         next_a = has_next ? na : empty;
         next_b = has_next ? nb : empty;
 
@@ -317,7 +352,11 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
 
 template <int FA, int FB>
 void launch_fmt(const GemmArgs &g, int blocks_per_xcd, hipStream_t stream) {
-    hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB>), dim3((unsigned)(8 * blocks_per_xcd)), dim3(256), 0, stream, g);
+    const dim3 grid((unsigned)(8 * blocks_per_xcd)), block(256);
+    if (g.ta && g.tb) hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB, true, true>), grid, block, 0, stream, g);
+    else if (g.tb) hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB, false, true>), grid, block, 0, stream, g);
+    else if (g.ta) hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB, true, false>), grid, block, 0, stream, g);
+    else hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB, false, false>), grid, block, 0, stream, g);
 }
 
 }  // namespace

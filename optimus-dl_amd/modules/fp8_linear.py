@@ -148,6 +148,7 @@ class _Fp8LinearFn(torch.autograd.Function):
         need_dgrad, need_wgrad = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         bias_f32 = None if bias is None else bias.detach().float()
         saved: dict[str, Any] = {}
+        ctx.wgrad_direct = ctx.dgrad_direct = False
 
         if pol.kind == "rowwise":
             if need_wgrad and recipe.wgrad:
@@ -158,17 +159,27 @@ class _Fp8LinearFn(torch.autograd.Function):
             wq, sw_inv = module._rowwise_weight(weight, pol, "row", both=need_dgrad)
             y = native.gemm_nt(xq, wq, pol.fmt_fwd, pol.fmt_fwd, sx_inv, sw_inv, bias=bias_f32, out_dtype=out_dtype)
         else:
+            # With whole 256 x 256 tiles the backward GEMMs read the row-major codes with the contraction
+            # index as the slow axis (native.gemm_layouts): no transposed copy of x, w or dy is made.
+            tokens, n_in, n_out = x2d.shape[0], x2d.shape[1], weight.shape[0]
+            direct = recipe.direct_layouts and out_dtype == torch.bfloat16
+            wgrad_direct = direct and x2d.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and \
+                native.gemm_layouts_supported(n_out, n_in, tokens)
+            dgrad_direct = direct and x2d.dtype == torch.bfloat16 and native.gemm_layouts_supported(tokens, n_in, n_out)
+            fp8_wgrad = need_wgrad and recipe.wgrad
+            x_t_needed = fp8_wgrad and not wgrad_direct
             if pol.kind == "delayed":
                 meta = module._meta(recipe, x2d.device, "fwd")
-                xq, xq_t, sx_inv = _quantise_delayed(x2d, pol.fmt_fwd, meta, ROLE_X, need_wgrad and recipe.wgrad)
+                xq, xq_t, sx_inv = _quantise_delayed(x2d, pol.fmt_fwd, meta, ROLE_X, x_t_needed)
             else:
-                xq, xq_t, sx_inv = _quantise_input_shared(recipe, x2d, pol.fmt_fwd, pol.margin, need_wgrad and recipe.wgrad)
-            wq, wq_t, sw_inv = module._tensor_weight(weight, recipe, need_t=need_dgrad)
+                xq, xq_t, sx_inv = _quantise_input_shared(recipe, x2d, pol.fmt_fwd, pol.margin, x_t_needed)
+            wq, wq_t, sw_inv = module._tensor_weight(weight, recipe, need_t=need_dgrad and not dgrad_direct)
             y = native.gemm_nt(xq, wq, pol.fmt_fwd, pol.fmt_fwd, sx_inv, sw_inv, bias=bias_f32, out_dtype=out_dtype)
-            if need_wgrad and recipe.wgrad:
-                saved["xq_t"], saved["sx_inv_t"] = xq_t, sx_inv
+            if fp8_wgrad:
+                saved["xq_t" if not wgrad_direct else "xq"], saved["sx_inv_t"] = (xq_t if not wgrad_direct else xq), sx_inv
             if need_dgrad:
-                saved["wq_t"], saved["sw_inv_t"] = wq_t, sw_inv
+                saved["wq_t" if not dgrad_direct else "wq"], saved["sw_inv_t"] = (wq_t if not dgrad_direct else wq), sw_inv
+            ctx.wgrad_direct, ctx.dgrad_direct = wgrad_direct, dgrad_direct
         if need_wgrad and not recipe.wgrad:
             saved["x_hp"] = x2d                      # wgrad=False: weight gradient in the activation dtype
         ctx.module, ctx.recipe, ctx.saved = module, recipe, saved
@@ -202,24 +213,36 @@ class _Fp8LinearFn(torch.autograd.Function):
                 dw = native.gemm_nt(gq_t, saved["xq_t"], pol.fmt_bwd, pol.fmt_fwd, sg_inv_t, saved["sx_inv_t"],
                                     out_dtype=ctx.w_dtype)
         else:
+            # the transposed codes of dy are only needed by a wgrad that cannot read them K-slow;
+            # the row-major ones by dgrad and by the K-slow wgrad
+            g_t_needed = fp8_wgrad and not ctx.wgrad_direct
+            g_rm_needed = ctx.need_dgrad or (fp8_wgrad and ctx.wgrad_direct)
             if ctx.need_dgrad or fp8_wgrad:
                 if pol.kind == "delayed":
                     meta = module._meta(recipe, dy2d.device, "bwd")
-                    gq, gq_t, sg_inv = _quantise_delayed(dy2d, pol.fmt_bwd, meta, ROLE_G, fp8_wgrad, ctx.need_dgrad)
+                    gq, gq_t, sg_inv = _quantise_delayed(dy2d, pol.fmt_bwd, meta, ROLE_G, g_t_needed, g_rm_needed)
                 else:
                     parts = recipe.take_parts(dy2d)
                     if parts is None and ctx.has_bias and native.colsum_supported(dy2d):
                         # the amax pass also adds up the columns: the bias gradient costs no extra read of dy
                         parts, colsum = native.amax_parts_colsum(dy2d)
                         db = colsum.to(ctx.bias_dtype)
-                    gq, gq_t, sg_inv, _ = _quantise_dynamic(dy2d, pol.fmt_bwd, pol.margin, fp8_wgrad, ctx.need_dgrad,
+                    gq, gq_t, sg_inv, _ = _quantise_dynamic(dy2d, pol.fmt_bwd, pol.margin, g_t_needed, g_rm_needed,
                                                             parts=parts)
             if ctx.need_dgrad:
-                dx = native.gemm_nt(gq, saved["wq_t"], pol.fmt_bwd, pol.fmt_fwd, sg_inv, saved["sw_inv_t"],
-                                    out_dtype=ctx.x_dtype)
+                if ctx.dgrad_direct:        # dX = dY . W: W [N, K] read with N (the contraction) as the slow axis
+                    dx = native.gemm_layouts(gq, saved["wq"], pol.fmt_bwd, pol.fmt_fwd, native.K_FAST, native.K_SLOW,
+                                             sg_inv, saved["sw_inv_t"])
+                else:
+                    dx = native.gemm_nt(gq, saved["wq_t"], pol.fmt_bwd, pol.fmt_fwd, sg_inv, saved["sw_inv_t"],
+                                        out_dtype=ctx.x_dtype)
             if fp8_wgrad:
-                dw = native.gemm_nt(gq_t, saved["xq_t"], pol.fmt_bwd, pol.fmt_fwd, sg_inv, saved["sx_inv_t"],
-                                    out_dtype=ctx.w_dtype)
+                if ctx.wgrad_direct:        # dW = dY^T . X: both read with the tokens as the slow axis
+                    dw = native.gemm_layouts(gq, saved["xq"], pol.fmt_bwd, pol.fmt_fwd, native.K_SLOW, native.K_SLOW,
+                                             sg_inv, saved["sx_inv_t"])
+                else:
+                    dw = native.gemm_nt(gq_t, saved["xq_t"], pol.fmt_bwd, pol.fmt_fwd, sg_inv, saved["sx_inv_t"],
+                                        out_dtype=ctx.w_dtype)
         if ctx.need_wgrad and not recipe.wgrad:
             dw = (dy2d.t().to(saved["x_hp"].dtype) @ saved["x_hp"]).to(ctx.w_dtype)
         if ctx.has_bias and db is None:

@@ -49,6 +49,7 @@ EXPORTS = (
     "odl_fp8_cast",
     "odl_fp8_cast_transpose",
     "odl_fp8_gemm_nt",
+    "odl_fp8_gemm_layouts",
     "odl_fp8_delayed_update",
     "odl_fp8_gemm_num_variants",
     "odl_fp8_gemm_variant_name",
@@ -102,6 +103,7 @@ def load() -> ctypes.CDLL:
         L.odl_fp8_cast.argtypes = [vp, i32, i64, i64, vp, i32, i32, vp, vp, vp]
         L.odl_fp8_cast_transpose.argtypes = [vp, i32, i64, i64, vp, i32, i32, vp, vp, vp, vp]
         L.odl_fp8_gemm_nt.argtypes = [vp, vp, i64, i64, i64, i32, i32, vp, i64, vp, i64, vp, i32, vp, i32, vp]
+        L.odl_fp8_gemm_layouts.argtypes = [vp, vp, i64, i64, i64, i32, i32, i32, i32, vp, vp, vp, vp]
         L.odl_fp8_delayed_update.argtypes = [vp, i64, i64, i64, vp, vp, vp, i32, i32, vp]
         L.odl_fp8_gemm_num_variants.restype = i32
         L.odl_fp8_gemm_variant_name.argtypes = [i32]
@@ -510,6 +512,37 @@ def gemm_nt(a: torch.Tensor, b: torch.Tensor, fmt_a: int, fmt_b: int, sa_inv: to
     _check(load().odl_fp8_gemm_nt(a.data_ptr(), b.data_ptr(), M, N, K, fmt_a, fmt_b, sa_inv.data_ptr(), sa_inv.numel(),
                                   sb_inv.data_ptr(), sb_inv.numel(), bias.data_ptr() if bias is not None else None,
                                   DT_F32, out.data_ptr(), odt, _stream()), "odl_fp8_gemm_nt")
+    return out
+
+
+K_FAST, K_SLOW = 0, 1
+
+
+def gemm_layouts_supported(M: int, N: int, K: int) -> bool:
+    """Shapes :func:`gemm_layouts` takes (whole 256 x 256 tiles, operands under 2 GiB)."""
+    return (M > 0 and N > 0 and K >= 512 and M % 256 == 0 and N % 256 == 0 and K % 256 == 0
+            and (M + 256) * K < 2**31 and (N + 256) * K < 2**31 and N * 2 * 264 < 2**31)
+
+
+def gemm_layouts(a: torch.Tensor, b: torch.Tensor, fmt_a: int, fmt_b: int, layout_a: int, layout_b: int,
+                 sa_inv: torch.Tensor, sb_inv: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """out[M,N] (bf16) = (A . B^T) * sa_inv * sb_inv where an operand is given either as [rows, K]
+    (K_FAST) or as [K, rows] (K_SLOW): no transposed copies for dgrad / wgrad."""
+    if a.dtype != torch.uint8 or b.dtype != torch.uint8:
+        raise NativeError("gemm_layouts operands must be uint8 FP8 codes")
+    a, b = _as_2d(a), _as_2d(b)
+    M, K = (a.shape[1], a.shape[0]) if layout_a == K_SLOW else a.shape
+    N, K2 = (b.shape[1], b.shape[0]) if layout_b == K_SLOW else b.shape
+    if K != K2:
+        raise NativeError(f"gemm_layouts: contraction sizes differ ({K} vs {K2})")
+    _f32_dev(sa_inv, 1, "gemm_layouts sa_inv")
+    _f32_dev(sb_inv, 1, "gemm_layouts sb_inv")
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=a.device)
+    elif out.shape != (M, N) or out.dtype != torch.bfloat16 or not out.is_contiguous():
+        raise NativeError("gemm_layouts: `out` has the wrong shape / dtype / layout")
+    _check(load().odl_fp8_gemm_layouts(a.data_ptr(), b.data_ptr(), M, N, K, fmt_a, fmt_b, layout_a, layout_b, sa_inv.data_ptr(),
+                                       sb_inv.data_ptr(), out.data_ptr(), _stream()), "odl_fp8_gemm_layouts")
     return out
 
 

@@ -329,3 +329,20 @@ def test_fused_producers_at_config_3_size(N):
             assert_f32_bits_equal(dx[ri], wdx, "dx")
         want_dw = (dy.double() * (x.double() * rstd.double()[:, None])).sum(0)
         assert ((dw.double() - want_dw).abs().max() / want_dw.abs().max()).item() < 1e-5
+
+
+@pytest.mark.parametrize("M,Nn,K,la,lb", [pytest.param(14336, 4096, 8192, 1, 1, id="cfg3-wgrad-gate"),
+                                          pytest.param(8192, 4096, 14336, 0, 1, id="cfg3-dgrad-gate"),
+                                          pytest.param(4096, 14336, 8192, 1, 1, id="cfg3-wgrad-down"),
+                                          pytest.param(8192, 8192, 28672, 0, 1, id="cfg5-dgrad-up")])
+def test_k_slow_layouts_at_baseline_shapes(N, M, Nn, K, la, lb):
+    """dgrad / wgrad reading row-major codes (contraction index slow) against the same kernel on transposed copies."""
+    a = draw((M, K), 1e-3, 41)
+    b = draw((Nn, K), 1.0, 42)
+    aq, aq_t, _, sa_inv, _ = quantise(N, a, O.E5M2)
+    bq, bq_t, _, sb_inv, _ = quantise(N, b, O.E4M3)
+    del a, b
+    ref = N.gemm_nt(aq, bq, O.E5M2, O.E4M3, sa_inv, sb_inv)
+    out = N.gemm_layouts(aq_t if la else aq, bq_t if lb else bq, O.E5M2, O.E4M3, la, lb, sa_inv, sb_inv)
+    assert torch.equal(out, ref)
+    sample_check(out, aq, bq, O.E5M2, O.E4M3, sa_inv, sb_inv, seed=M + K, what=f"k-slow {M}x{Nn}x{K}")

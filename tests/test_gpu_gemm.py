@@ -182,3 +182,49 @@ def test_linear_fwd_bwd_three_gemms_at_llama_mlp_slice(N):
     for name, got in (("y", y), ("dx", dx), ("dw", dw)):
         err = max_rel_err(got, ref[name])
         assert err <= TOL, f"{name}: {err}"
+
+
+# ------------------------------------------------ operands stored with the contraction index slow
+@pytest.mark.parametrize("fmts", [(O.E4M3, O.E4M3), (O.E5M2, O.E4M3), (O.E4M3, O.E5M2), (O.E5M2, O.E5M2)])
+@pytest.mark.parametrize("shape", [(256, 256, 512), (512, 768, 1024), (1024, 256, 2560)])
+def test_k_slow_layouts_equal_the_transposed_copies_bit_for_bit(N, fmts, shape):
+    M, Nn, K = shape
+    fa, fb = fmts
+    a, sa = quantised((M, K), fa, 1.0, 1)
+    b, sb = quantised((Nn, K), fb, 0.05, 2)
+    a, b, sa, sb = a.cuda(), b.cuda(), sa.cuda(), sb.cuda()
+    a_t, b_t = a.t().contiguous(), b.t().contiguous()                 # [K, M], [K, N]
+    ref = N.gemm_nt(a, b, fa, fb, sa, sb)
+    assert max_rel_err(ref, O.t_gemm_nt(a.cpu(), b.cpu(), fa, fb, sa.cpu(), sb.cpu())) <= TOL
+    for la, lb in ((N.K_FAST, N.K_FAST), (N.K_FAST, N.K_SLOW), (N.K_SLOW, N.K_FAST), (N.K_SLOW, N.K_SLOW)):
+        out = N.gemm_layouts(a_t if la else a, b_t if lb else b, fa, fb, la, lb, sa, sb)
+        assert torch.equal(out, ref), f"layouts {la}{lb} of {shape}"
+
+
+def test_k_slow_layouts_index_check_with_one_hot_operands(N):
+    # A[m, k] = 1 at k = (7 m + 3) % K, B[n, k] = 2^(n % 5) at k = (5 n + 1) % K, stored K-slow:
+    # C[m, n] is that power of two where the two columns coincide and 0 elsewhere, exactly
+    M, Nn, K = 256, 512, 768
+    a = torch.zeros((M, K)); b = torch.zeros((Nn, K))
+    ka = (7 * torch.arange(M) + 3) % K
+    kb = (5 * torch.arange(Nn) + 1) % K
+    a[torch.arange(M), ka] = 1.0
+    b[torch.arange(Nn), kb] = 2.0 ** (torch.arange(Nn) % 5).float()
+    one = torch.ones(1)
+    aq, bq = O.t_cast(a.bfloat16(), one, O.E4M3).cuda(), O.t_cast(b.bfloat16(), one, O.E4M3).cuda()
+    want = ((ka[:, None] == kb[None, :]).float() * b.sum(1)[None, :]).bfloat16()
+    out = N.gemm_layouts(aq.t().contiguous(), bq.t().contiguous(), O.E4M3, O.E4M3, N.K_SLOW, N.K_SLOW, one.cuda(), one.cuda())
+    assert torch.equal(out.cpu(), want)
+
+
+def test_k_slow_layouts_refusals(N):
+    one = torch.ones(1, device="cuda")
+    a = torch.zeros((256, 512), dtype=torch.uint8, device="cuda")
+    with pytest.raises(N.NativeError, match="multiples of 256"):
+        N.gemm_layouts(a[:128], a, O.E4M3, O.E4M3, N.K_FAST, N.K_FAST, one, one)
+    with pytest.raises(N.NativeError, match="multiples of 256"):
+        N.gemm_layouts(a[:, :256], a[:, :256], O.E4M3, O.E4M3, N.K_FAST, N.K_FAST, one, one)       # K = 256 < 512
+    with pytest.raises(N.NativeError, match="contraction sizes differ"):
+        N.gemm_layouts(a, a.t().contiguous(), O.E4M3, O.E4M3, N.K_FAST, N.K_FAST, one, one)
+    assert not N.gemm_layouts_supported(256, 256, 256) and not N.gemm_layouts_supported(384, 256, 512)
+    assert N.gemm_layouts_supported(256, 256, 512)
