@@ -193,8 +193,8 @@ class FP8Recipe:
         # (gate/up, q/k/v) quantise it once; dropped when the outermost context is left
         self.shared_input: dict[str, Any] | None = None
         self.share_inputs = True
-        # backward GEMMs read row-major codes with the contraction index slow where the shapes allow
-        # (no transposed copies); False keeps the cast+transpose route everywhere
+        # wgrad reads the row-major codes of dy with the tokens as the slow axis where the shapes allow
+        # (no transposed copy of dy); False keeps the cast+transpose route everywhere
         self.direct_layouts = True
         # partial maxima handed over by the kernel that produced a tensor (SwiGLU, RMSNorm), so that
         # the Linear that quantises this very tensor skips its amax pass; a handful of entries

@@ -148,7 +148,7 @@ class _Fp8LinearFn(torch.autograd.Function):
         need_dgrad, need_wgrad = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         bias_f32 = None if bias is None else bias.detach().float()
         saved: dict[str, Any] = {}
-        ctx.wgrad_direct = ctx.dgrad_direct = False
+        ctx.wgrad_direct = False
 
         if pol.kind == "rowwise":
             if need_wgrad and recipe.wgrad:
@@ -159,27 +159,25 @@ class _Fp8LinearFn(torch.autograd.Function):
             wq, sw_inv = module._rowwise_weight(weight, pol, "row", both=need_dgrad)
             y = native.gemm_nt(xq, wq, pol.fmt_fwd, pol.fmt_fwd, sx_inv, sw_inv, bias=bias_f32, out_dtype=out_dtype)
         else:
-            # With whole 256 x 256 tiles the backward GEMMs read the row-major codes with the contraction
-            # index as the slow axis (native.gemm_layouts): no transposed copy of x, w or dy is made.
+            # With whole 256 x 256 tiles wgrad reads the ROW-MAJOR codes of dy with the tokens as the slow
+            # axis (native.gemm_layouts): dy, the largest tensor of the backward, gets no transposed copy.
+            # x and w keep theirs: they are cold by the time the backward runs, and reading a cold operand
+            # K-slow costs the GEMM more than the copy (measured), while dy has just been written.
             tokens, n_in, n_out = x2d.shape[0], x2d.shape[1], weight.shape[0]
-            direct = recipe.direct_layouts and out_dtype == torch.bfloat16
-            wgrad_direct = direct and x2d.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and \
-                native.gemm_layouts_supported(n_out, n_in, tokens)
-            dgrad_direct = direct and x2d.dtype == torch.bfloat16 and native.gemm_layouts_supported(tokens, n_in, n_out)
             fp8_wgrad = need_wgrad and recipe.wgrad
-            x_t_needed = fp8_wgrad and not wgrad_direct
+            ctx.wgrad_direct = (fp8_wgrad and recipe.direct_layouts and weight.dtype == torch.bfloat16
+                                and native.gemm_layouts_supported(n_out, n_in, tokens))
             if pol.kind == "delayed":
                 meta = module._meta(recipe, x2d.device, "fwd")
-                xq, xq_t, sx_inv = _quantise_delayed(x2d, pol.fmt_fwd, meta, ROLE_X, x_t_needed)
+                xq, xq_t, sx_inv = _quantise_delayed(x2d, pol.fmt_fwd, meta, ROLE_X, fp8_wgrad)
             else:
-                xq, xq_t, sx_inv = _quantise_input_shared(recipe, x2d, pol.fmt_fwd, pol.margin, x_t_needed)
-            wq, wq_t, sw_inv = module._tensor_weight(weight, recipe, need_t=need_dgrad and not dgrad_direct)
+                xq, xq_t, sx_inv = _quantise_input_shared(recipe, x2d, pol.fmt_fwd, pol.margin, fp8_wgrad)
+            wq, wq_t, sw_inv = module._tensor_weight(weight, recipe, need_t=need_dgrad)
             y = native.gemm_nt(xq, wq, pol.fmt_fwd, pol.fmt_fwd, sx_inv, sw_inv, bias=bias_f32, out_dtype=out_dtype)
             if fp8_wgrad:
-                saved["xq_t" if not wgrad_direct else "xq"], saved["sx_inv_t"] = (xq_t if not wgrad_direct else xq), sx_inv
+                saved["xq_t"], saved["sx_inv_t"] = xq_t, sx_inv
             if need_dgrad:
-                saved["wq_t" if not dgrad_direct else "wq"], saved["sw_inv_t"] = (wq_t if not dgrad_direct else wq), sw_inv
-            ctx.wgrad_direct, ctx.dgrad_direct = wgrad_direct, dgrad_direct
+                saved["wq_t"], saved["sw_inv_t"] = wq_t, sw_inv
         if need_wgrad and not recipe.wgrad:
             saved["x_hp"] = x2d                      # wgrad=False: weight gradient in the activation dtype
         ctx.module, ctx.recipe, ctx.saved = module, recipe, saved
@@ -213,8 +211,7 @@ class _Fp8LinearFn(torch.autograd.Function):
                 dw = native.gemm_nt(gq_t, saved["xq_t"], pol.fmt_bwd, pol.fmt_fwd, sg_inv_t, saved["sx_inv_t"],
                                     out_dtype=ctx.w_dtype)
         else:
-            # the transposed codes of dy are only needed by a wgrad that cannot read them K-slow;
-            # the row-major ones by dgrad and by the K-slow wgrad
+            # the transposed codes of dy are only needed by a wgrad that cannot read the row-major ones
             g_t_needed = fp8_wgrad and not ctx.wgrad_direct
             g_rm_needed = ctx.need_dgrad or (fp8_wgrad and ctx.wgrad_direct)
             if ctx.need_dgrad or fp8_wgrad:
@@ -230,15 +227,11 @@ class _Fp8LinearFn(torch.autograd.Function):
                     gq, gq_t, sg_inv, _ = _quantise_dynamic(dy2d, pol.fmt_bwd, pol.margin, g_t_needed, g_rm_needed,
                                                             parts=parts)
             if ctx.need_dgrad:
-                if ctx.dgrad_direct:        # dX = dY . W: W [N, K] read with N (the contraction) as the slow axis
-                    dx = native.gemm_layouts(gq, saved["wq"], pol.fmt_bwd, pol.fmt_fwd, native.K_FAST, native.K_SLOW,
-                                             sg_inv, saved["sw_inv_t"])
-                else:
-                    dx = native.gemm_nt(gq, saved["wq_t"], pol.fmt_bwd, pol.fmt_fwd, sg_inv, saved["sw_inv_t"],
-                                        out_dtype=ctx.x_dtype)
+                dx = native.gemm_nt(gq, saved["wq_t"], pol.fmt_bwd, pol.fmt_fwd, sg_inv, saved["sw_inv_t"],
+                                    out_dtype=ctx.x_dtype)
             if fp8_wgrad:
-                if ctx.wgrad_direct:        # dW = dY^T . X: both read with the tokens as the slow axis
-                    dw = native.gemm_layouts(gq, saved["xq"], pol.fmt_bwd, pol.fmt_fwd, native.K_SLOW, native.K_SLOW,
+                if ctx.wgrad_direct:        # dW = dY^T . X with dY [tokens, N] as stored, X^T from the forward
+                    dw = native.gemm_layouts(gq, saved["xq_t"], pol.fmt_bwd, pol.fmt_fwd, native.K_SLOW, native.K_FAST,
                                              sg_inv, saved["sx_inv_t"])
                 else:
                     dw = native.gemm_nt(gq_t, saved["xq_t"], pol.fmt_bwd, pol.fmt_fwd, sg_inv, saved["sx_inv_t"],
