@@ -7,7 +7,8 @@ and weights, E5M2 for gradients), M = 8192 tokens:
     gate, up : X [8192, 4096]   W [14336, 4096]   dY [8192, 14336]
     down     : X [8192, 14336]  W [4096, 14336]   dY [8192, 4096]
 One step = fwd + bwd of all three = 9 GEMMs (8.66 TFLOP) plus every amax, cast and
-cast+transpose they need, weights re-quantised each step as after an optimizer
+cast+transpose they need (x and w get a transposed FP8 copy for dgrad / wgrad; dY is cast
+once and read by wgrad as stored), weights re-quantised each step as after an optimizer
 step.  Inputs are synthetic, seeded, and resident in HBM before the clock starts.
 
 Two passes over the same steps: the timed one (`value`, `ms_per_step`) has nothing
@@ -340,7 +341,7 @@ def main() -> int:
         "data": "synthetic",
         "config": {
             "workload": "configs[2] of BASELINE.json: Llama-3-8B SwiGLU MLP Linears (gate, up [14336x4096]; down [4096x14336]), "
-                        "M=8192, FP8 fwd+bwd, per-tensor dynamic scaling, fused cast+transpose for wgrad",
+                        "M=8192, FP8 fwd+bwd, per-tensor dynamic scaling, fused cast+transpose of x and w, dY read by wgrad as stored",
             "flop_per_step": step_flops(),
             "gemms_per_step": 9,
             "gemm_variant": native.gemm_variants()[args.gemm_variant] if args.gemm_variant >= 0 else "auto",
