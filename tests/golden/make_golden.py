@@ -3,8 +3,8 @@
 ``python tests/golden/make_golden.py``).
 
 Nothing here uses the oracle or the GPU kernels: the vectors come from the OCP FP8 format
-definitions, from torch's CPU conversion ``Tensor.to(torch.float8_*)`` and from numpy float32
-arithmetic, so that they pin the oracle (tests/test_golden_vectors.py) and, through it and
+definitions, from torch's CPU routines (``Tensor.to(torch.float8_*)``, ``F.silu``, bf16 multiply and
+autograd), from float64 closed forms and from numpy float32 arithmetic, so that they pin the oracle (tests/test_golden_vectors.py) and, through it and
 directly, the kernels.  The files are small JSON documents; floats are stored as the hex of
 their IEEE bit patterns so that nothing depends on decimal printing.
 """
@@ -131,9 +131,64 @@ def delayed_sequence():
     return out
 
 
+def bf16_hex(t):
+    return [f"{int(v) & 0xffff:04x}" for v in t.contiguous().view(torch.int16).flatten().tolist()]
+
+
+def swiglu_vectors():
+    """silu(gate) * up and its gradients as torch computes them in bf16 on the CPU (F.silu, tensor multiply, autograd).
+    Gates: every 37th bf16 pattern above -80 (finite), the exact points 0 / +-1 / saturation, and Gaussian draws."""
+    import torch.nn.functional as F
+
+    bits = torch.arange(0, 65536, 37, dtype=torch.int32)
+    gates = bits.to(torch.int16).view(torch.bfloat16)
+    gates = gates[torch.isfinite(gates.float()) & (gates.float() >= -80.0)]
+    gen = torch.Generator().manual_seed(5)
+    extra = torch.cat([torch.tensor([0.0, -0.0, 1.0, -1.0, 30.0, -30.0, 79.5, -79.5, 100.0]),
+                       torch.randn(600, generator=gen) * 2.0]).bfloat16()
+    g = torch.cat([gates, extra])
+    u = (torch.randn(g.numel(), generator=gen) * 1.5).bfloat16()
+    dh = (torch.randn(g.numel(), generator=gen) * 1e-2).bfloat16()
+    ga, ua = g.clone().requires_grad_(True), u.clone().requires_grad_(True)
+    h = F.silu(ga) * ua
+    h.backward(dh)
+    return {"gate_bf16_hex": bf16_hex(g), "up_bf16_hex": bf16_hex(u), "dh_bf16_hex": bf16_hex(dh),
+            "silu_bf16_hex": bf16_hex(F.silu(g)), "h_bf16_hex": bf16_hex(h.detach()),
+            "d_up_bf16_hex": bf16_hex(ua.grad), "d_gate_bf16_hex": bf16_hex(ga.grad),
+            "note": "d_gate is torch's association (grad * sig) * (1 + g (1 - sig)); the library's differs: within one bf16 unit"}
+
+
+def norm_vectors():
+    """RMSNorm and LayerNorm rows with outputs from float64 closed forms, rounded once to bf16 (y) / float32 (statistics)."""
+    gen = torch.Generator().manual_seed(9)
+    out = {"cases": []}
+    for cols, dtype in ((8, "bf16"), (264, "bf16"), (768, "f32")):
+        rows = 3
+        x = torch.randn((rows, cols), generator=gen) * 2.5 + 0.4
+        x = x.bfloat16() if dtype == "bf16" else x
+        w = torch.randn(cols, generator=gen) * 0.4 + 1.0
+        b = torch.randn(cols, generator=gen) * 0.2
+        eps = 1e-5
+        x64 = x.double()
+        rstd_rms = 1.0 / torch.sqrt((x64 * x64).mean(-1) + eps)
+        y_rms = (x64 * rstd_rms[:, None] * w.double()).float().bfloat16()
+        mean = x64.mean(-1)
+        rstd_ln = 1.0 / torch.sqrt(x64.var(-1, unbiased=False) + eps)
+        y_ln = ((x64 - mean[:, None]) * rstd_ln[:, None] * w.double() + b.double()).float().bfloat16()
+        out["cases"].append({
+            "rows": rows, "cols": cols, "dtype": dtype, "eps": eps,
+            "x_hex": bf16_hex(x) if dtype == "bf16" else f32_hex(x.numpy()),
+            "weight_f32_hex": f32_hex(w.numpy()), "bias_f32_hex": f32_hex(b.numpy()),
+            "rms_rstd_f32_hex": f32_hex(rstd_rms.float().numpy()), "rms_y_bf16_hex": bf16_hex(y_rms),
+            "ln_mean_f32_hex": f32_hex(mean.float().numpy()), "ln_rstd_f32_hex": f32_hex(rstd_ln.float().numpy()),
+            "ln_y_bf16_hex": bf16_hex(y_ln)})
+    return out
+
+
 def main():
     docs = {"fp8_decode_tables.json": decode_tables(), "fp8_encode_edges.json": encode_vectors(),
-            "scale_from_amax.json": scale_vectors(), "delayed_scaling_sequence.json": delayed_sequence()}
+            "scale_from_amax.json": scale_vectors(), "delayed_scaling_sequence.json": delayed_sequence(),
+            "swiglu_bf16.json": swiglu_vectors(), "norm_rows.json": norm_vectors()}
     for name, doc in docs.items():
         with open(os.path.join(HERE, name), "w") as fh:
             json.dump(doc, fh, separators=(",", ":"))

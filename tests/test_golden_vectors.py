@@ -93,3 +93,52 @@ def test_delayed_scaling_sequence():
             assert same_bits(py.scale, after[t:t + 1]) and same_bits(scale, after[t:t + 1]), (case, t)
         assert same_bits(hist[:, 0], f32(case["final_history_f32_hex"]))
         assert same_bits(py.history[:, 0], f32(case["final_history_f32_hex"]))
+
+
+# ----------------------------------------------------------------- producers: SwiGLU, RMSNorm, LayerNorm
+def bf16(hexes, shape=None):
+    a = np.array([int(h, 16) for h in hexes], dtype=np.uint16)
+    t = torch.from_numpy(a.view(np.int16).copy()).view(torch.bfloat16)
+    return t if shape is None else t.reshape(shape)
+
+
+def bf16_units_apart(a: torch.Tensor, b: torch.Tensor) -> np.ndarray:
+    ai = a.contiguous().view(torch.int16).numpy().astype(np.int32)
+    bi = b.contiguous().view(torch.int16).numpy().astype(np.int32)
+    return np.abs(ai - bi)
+
+
+def test_swiglu_vectors_from_torch_bf16():
+    doc = load("swiglu_bf16.json")
+    g, u, dh = bf16(doc["gate_bf16_hex"]), bf16(doc["up_bf16_hex"]), bf16(doc["dh_bf16_hex"])
+    assert g.numel() > 1500
+    ones = torch.ones_like(g)
+    assert torch.equal(O.c_swiglu_fwd(g, ones).view(torch.int16), bf16(doc["silu_bf16_hex"]).view(torch.int16))
+    assert torch.equal(O.c_swiglu_fwd(g, u).view(torch.int16), bf16(doc["h_bf16_hex"]).view(torch.int16))
+    dg, du = O.c_swiglu_bwd(dh, g, u)
+    assert torch.equal(du.view(torch.int16), bf16(doc["d_up_bf16_hex"]).view(torch.int16))
+    d = bf16_units_apart(dg, bf16(doc["d_gate_bf16_hex"]))
+    assert d.max() <= 1 and (d > 0).mean() < 0.02                  # torch associates the product differently
+
+
+def norm_case_tensors(case):
+    shape = (case["rows"], case["cols"])
+    x = bf16(case["x_hex"], shape) if case["dtype"] == "bf16" else torch.from_numpy(f32(case["x_hex"]).copy()).reshape(shape)
+    w = torch.from_numpy(f32(case["weight_f32_hex"]).copy())
+    b = torch.from_numpy(f32(case["bias_f32_hex"]).copy())
+    return x, w, b
+
+
+def test_norm_vectors_from_float64_closed_forms():
+    for case in load("norm_rows.json")["cases"]:
+        x, w, b = norm_case_tensors(case)
+        shape = tuple(x.shape)
+        y, rstd = O.c_rmsnorm(x, w, case["eps"])
+        assert np.allclose(rstd.numpy(), f32(case["rms_rstd_f32_hex"]), rtol=1e-6, atol=0)
+        d = bf16_units_apart(y, bf16(case["rms_y_bf16_hex"], shape))
+        assert d.max() <= 1 and (d > 0).mean() < 0.01
+        y, mean, rstd = O.c_layernorm(x, w, b, case["eps"])
+        assert np.allclose(mean.numpy(), f32(case["ln_mean_f32_hex"]), rtol=1e-5, atol=1e-6)
+        assert np.allclose(rstd.numpy(), f32(case["ln_rstd_f32_hex"]), rtol=1e-6, atol=0)
+        d = bf16_units_apart(y, bf16(case["ln_y_bf16_hex"], shape))
+        assert d.max() <= 1 and (d > 0).mean() < 0.01

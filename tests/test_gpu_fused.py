@@ -257,3 +257,56 @@ def test_layernorm_refusals(N):
         N.layernorm_amax_parts(torch.zeros((4, 12), dtype=torch.bfloat16).cuda(), torch.ones(12).cuda(), None, 1e-5)
     with pytest.raises(N.NativeError, match="4096"):
         N.layernorm_amax_parts(torch.zeros((1, 8192), dtype=torch.bfloat16).cuda(), torch.ones(8192).cuda(), None, 1e-5)
+
+
+# ------------------------------------------------------------------ committed golden vectors
+def _golden(name):
+    import json
+    import os
+
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", name)) as fh:
+        return json.load(fh)
+
+
+def _bf16_from_hex(hexes, shape=None):
+    a = np.array([int(h, 16) for h in hexes], dtype=np.uint16)
+    t = torch.from_numpy(a.view(np.int16).copy()).view(torch.bfloat16)
+    return t if shape is None else t.reshape(shape)
+
+
+def _f32_from_hex(hexes):
+    return torch.from_numpy(np.array([int(h, 16) for h in hexes], dtype=np.uint32).view(np.float32).copy())
+
+
+def test_kernels_against_golden_swiglu_vectors(N):
+    """tests/golden/swiglu_bf16.json holds what torch's CPU bf16 silu / multiply / autograd give."""
+    doc = _golden("swiglu_bf16.json")
+    g, u, dh = (_bf16_from_hex(doc[k]) for k in ("gate_bf16_hex", "up_bf16_hex", "dh_bf16_hex"))
+    n8 = g.numel() // 8 * 8
+    g, u, dh = g[:n8].reshape(-1, 8), u[:n8].reshape(-1, 8), dh[:n8].reshape(-1, 8)
+    h, _ = N.swiglu_amax_parts(g.cuda(), u.cuda())
+    assert_bf16_equal(h, _bf16_from_hex(doc["h_bf16_hex"])[:n8].reshape(-1, 8), "h vs golden")
+    s, _ = N.swiglu_amax_parts(g.cuda(), torch.ones_like(g).cuda())
+    assert_bf16_equal(s, _bf16_from_hex(doc["silu_bf16_hex"])[:n8].reshape(-1, 8), "silu vs golden")
+    dg, du, _, _ = N.swiglu_bwd_amax_parts(dh.cuda(), g.cuda(), u.cuda())
+    assert_bf16_equal(du, _bf16_from_hex(doc["d_up_bf16_hex"])[:n8].reshape(-1, 8), "d_up vs golden")
+    want = _bf16_from_hex(doc["d_gate_bf16_hex"])[:n8].reshape(-1, 8)
+    d = (dg.cpu().view(torch.int16).int() - want.view(torch.int16).int()).abs()
+    assert int(d.max()) <= 1 and float((d > 0).float().mean()) < 0.02
+
+
+def test_kernels_against_golden_norm_vectors(N):
+    """tests/golden/norm_rows.json holds float64 closed forms rounded once: within one bf16 unit."""
+    for case in _golden("norm_rows.json")["cases"]:
+        shape = (case["rows"], case["cols"])
+        x = _bf16_from_hex(case["x_hex"], shape) if case["dtype"] == "bf16" else _f32_from_hex(case["x_hex"]).reshape(shape)
+        w, b = _f32_from_hex(case["weight_f32_hex"]), _f32_from_hex(case["bias_f32_hex"])
+        y, rstd, _ = N.rmsnorm_amax_parts(x.cuda(), w.cuda(), case["eps"])
+        assert torch.allclose(rstd.cpu(), _f32_from_hex(case["rms_rstd_f32_hex"]), rtol=1e-6, atol=0)
+        d = (y.cpu().view(torch.int16).int() - _bf16_from_hex(case["rms_y_bf16_hex"], shape).view(torch.int16).int()).abs()
+        assert int(d.max()) <= 1 and float((d > 0).float().mean()) < 0.01
+        y, mean, rstd, _ = N.layernorm_amax_parts(x.cuda(), w.cuda(), b.cuda(), case["eps"])
+        assert torch.allclose(mean.cpu(), _f32_from_hex(case["ln_mean_f32_hex"]), rtol=1e-5, atol=1e-6)
+        assert torch.allclose(rstd.cpu(), _f32_from_hex(case["ln_rstd_f32_hex"]), rtol=1e-6, atol=0)
+        d = (y.cpu().view(torch.int16).int() - _bf16_from_hex(case["ln_y_bf16_hex"], shape).view(torch.int16).int()).abs()
+        assert int(d.max()) <= 1 and float((d > 0).float().mean()) < 0.01
