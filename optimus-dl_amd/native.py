@@ -310,17 +310,10 @@ def rmsnorm_amax_parts(x: torch.Tensor, weight: torch.Tensor, eps: float):
     if not x.is_cuda:
         raise NativeError(f"rmsnorm: the kernels run on the GPU only; got a tensor on {x.device}")
     src = _src_dtype(x)
-    if not x.is_contiguous():
-        x = x.contiguous()
-    if x.data_ptr() % 16:
-        x = x.clone(memory_format=torch.contiguous_format)
+    x = _dense_16(x)
     cols = x.shape[-1]
     rows = x.numel() // max(cols, 1)
-    w = weight.detach()
-    if w.dtype != torch.float32 or not w.is_contiguous() or w.data_ptr() % 16:
-        w = w.float().contiguous().clone()
-    if w.numel() != cols or w.device != x.device:
-        raise NativeError(f"rmsnorm: weight has {w.numel()} elements on {w.device}, rows have {cols} on {x.device}")
+    w = _f32_vector(weight, cols, x.device, "rmsnorm weight")
     y = torch.empty(x.shape, dtype=torch.bfloat16, device=x.device)
     rstd = torch.empty(x.shape[:-1], dtype=torch.float32, device=x.device)
     parts = torch.empty(AMAX_PARTS, dtype=torch.float32, device=x.device)
@@ -337,19 +330,14 @@ def rmsnorm_bwd(dy: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, rstd: t
     -> (dx in the dtype of x, d_weight fp32[cols])."""
     dy = _bf16_dense(dy, "rmsnorm dy")
     src = _src_dtype(x)
-    if not x.is_contiguous():
-        x = x.contiguous()
-    if x.data_ptr() % 16:
-        x = x.clone(memory_format=torch.contiguous_format)
+    x = _dense_16(x)
     if dy.shape != x.shape:
         raise NativeError(f"rmsnorm backward: dy {tuple(dy.shape)} and x {tuple(x.shape)} differ")
     cols = x.shape[-1]
     rows = x.numel() // max(cols, 1)
-    w = weight.detach()
-    if w.dtype != torch.float32 or not w.is_contiguous() or w.data_ptr() % 16:
-        w = w.float().contiguous().clone()
-    _f32_dev(rstd.reshape(-1) if rstd.is_contiguous() else rstd.contiguous().reshape(-1), rows, "rmsnorm backward rstd")
+    w = _f32_vector(weight, cols, x.device, "rmsnorm weight")
     rstd = rstd.contiguous()
+    _f32_dev(rstd.reshape(-1), rows, "rmsnorm backward rstd")
     dx = torch.empty_like(x)
     dw = torch.empty(cols, dtype=torch.float32, device=x.device)
     ws = torch.empty(RMSNORM_BWD_SLABS * cols, dtype=torch.float32, device=x.device)
