@@ -207,6 +207,24 @@ int odl_fp8_layernorm_bwd(const void *dy, const void *x, int src_dtype, const fl
                           float *dweight, float *dbias, float *workspace, odl_stream_t stream);
 
 /*
+ * Exact (erf) GELU between c_fc and c_proj of a GPT-2 MLP (optimus_dl/modules/model/blocks/mlp.py:141-157,
+ * nn.GELU()), bf16 in and out, with the partial maxima of the output, and its backward.  GELU of a
+ * bf16 value is a function of 16 bits, so both run from a table that odl_fp8_gelu_table fills once
+ * (ODL_FP8_GELU_TABLE_BYTES of device memory owned by the caller; double-precision evaluation):
+ *   fwd[x] = bf16( float( x * Phi(x) ) ),  Phi(x) = erfc(-x / sqrt 2) / 2
+ *   bwd[x] = float( Phi(x) + x * exp(-x^2 / 2) / sqrt(2 pi) )
+ *   odl_fp8_gelu_amax_parts     : y  = fwd[x];                  parts = partial maxima of |y|
+ *   odl_fp8_gelu_bwd_amax_parts : dx = bf16( dy * bwd[x] );     parts = partial maxima of |dx|
+ * rows * cols a multiple of 8, 16-byte aligned pointers.
+ */
+#define ODL_FP8_GELU_TABLE_BYTES (65536 * 2 + 65536 * 4)
+int odl_fp8_gelu_table(void *table, odl_stream_t stream);
+int odl_fp8_gelu_amax_parts(const void *x, int64_t rows, int64_t cols, const void *table, void *y,
+                            float *parts, odl_stream_t stream);
+int odl_fp8_gelu_bwd_amax_parts(const void *dy, const void *x, int64_t rows, int64_t cols,
+                                const void *table, void *dx, float *parts, odl_stream_t stream);
+
+/*
  * out[r,c] = fp8( clamp( fp32(x[r,c]) * s , +-max ) ), s = scale[0] | scale[r] | scale[c].
  * amax_out (may be NULL): *amax_out = max(*amax_out, max|x|), for delayed scaling,
  * where the cast uses an older scale while this step's amax is recorded.

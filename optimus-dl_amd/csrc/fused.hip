@@ -607,6 +607,70 @@ __global__ __launch_bounds__(kFusedThreads) void amax_colsum_kernel(const void *
         for (int j = nblk + threadIdx.x; j < kParts; j += kFusedThreads) parts[j] = 0.0f;
 }
 
+// ------------------------------------------------------------------------------ GELU
+// The exact (erf) GELU of a bf16 input is a function of 16 bits: a table, made once per device by
+// gelu_table_kernel in double precision, holds for every bf16 pattern x
+//   fwd[x] = bf16( float( x * Phi(x) ) )            Phi(x) = erfc(-x / sqrt 2) / 2
+//   bwd[x] = float( Phi(x) + x * phi(x) )           phi(x) = exp(-x^2 / 2) / sqrt(2 pi)
+// (65536 bf16 values, then 65536 floats: 384 KB, resident in L2 while in use).  The kernels gather:
+//   y = fwd[x],   dx = bf16( dy * bwd[x] ),   each with the partial maxima of what it writes.
+constexpr int kGeluFwdBytes = 65536 * 2;
+
+__global__ void gelu_table_kernel(uint16_t *__restrict__ fwd, float *__restrict__ bwd) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= 65536u) return;
+    const double x = (double)bits_to_float(i << 16);
+    const double cdf = 0.5 * erfc(-x * 0.70710678118654752440);
+    const double pdf = exp(-0.5 * x * x) * 0.39894228040143267794;
+    fwd[i] = (uint16_t)f32_to_bf16_bits((float)(x * cdf));
+    bwd[i] = (float)(cdf + x * pdf);
+}
+
+__global__ __launch_bounds__(kFusedThreads) void gelu_fwd_kernel(const u32x4 *__restrict__ x, int64_t n8, const uint16_t *__restrict__ fwd,
+                                                                  u32x4 *__restrict__ y, float *__restrict__ parts) {
+    __shared__ uint32_t red[kFusedThreads / kWave];
+    const int64_t stride = (int64_t)gridDim.x * kFusedThreads;
+    uint32_t am = 0;
+    for (int64_t i = (int64_t)blockIdx.x * kFusedThreads + threadIdx.x; i < n8; i += stride) {
+        const u32x4 v = __builtin_nontemporal_load(x + i);
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+        uint32_t o[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            o[q] = (uint32_t)fwd[w[q] & 0xffffu] | ((uint32_t)fwd[w[q] >> 16] << 16);
+            am = max_u16x2(am, abs_bf16x2(o[q]));
+        }
+        y[i] = u32x4{o[0], o[1], o[2], o[3]};
+    }
+    am = block_max_u32(fold_u16x2_to_f32bits(am), red);
+    if (threadIdx.x == 0) parts[blockIdx.x] = bits_to_float(am);
+    if (blockIdx.x == 0)
+        for (int j = (int)gridDim.x + threadIdx.x; j < kParts; j += kFusedThreads) parts[j] = 0.0f;
+}
+
+__global__ __launch_bounds__(kFusedThreads) void gelu_bwd_kernel(const u32x4 *__restrict__ dy, const u32x4 *__restrict__ x, int64_t n8,
+                                                                  const float *__restrict__ bwd, u32x4 *__restrict__ dx,
+                                                                  float *__restrict__ parts) {
+    __shared__ uint32_t red[kFusedThreads / kWave];
+    const int64_t stride = (int64_t)gridDim.x * kFusedThreads;
+    uint32_t am = 0;
+    for (int64_t i = (int64_t)blockIdx.x * kFusedThreads + threadIdx.x; i < n8; i += stride) {
+        const u32x4 v = __builtin_nontemporal_load(x + i), d = __builtin_nontemporal_load(dy + i);
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w}, dw[4] = {d.x, d.y, d.z, d.w};
+        uint32_t o[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            o[q] = pack2(__fmul_rn(bf16_lo(dw[q]), bwd[w[q] & 0xffffu]), __fmul_rn(bf16_hi(dw[q]), bwd[w[q] >> 16]));
+            am = max_u16x2(am, abs_bf16x2(o[q]));
+        }
+        dx[i] = u32x4{o[0], o[1], o[2], o[3]};
+    }
+    am = block_max_u32(fold_u16x2_to_f32bits(am), red);
+    if (threadIdx.x == 0) parts[blockIdx.x] = bits_to_float(am);
+    if (blockIdx.x == 0)
+        for (int j = (int)gridDim.x + threadIdx.x; j < kParts; j += kFusedThreads) parts[j] = 0.0f;
+}
+
 static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 // at most two fat blocks per CU, and never more blocks than there are partial maxima
@@ -782,4 +846,46 @@ extern "C" int odl_fp8_layernorm_bwd(const void *dy, const void *x, int src_dtyp
     // slabs are rows of 2 * cols sums (d_weight, d_bias); dweight and dbias are adjacent, so one reduction writes both
     hipLaunchKernelGGL(rmsnorm_bwd_reduce_kernel, dim3((unsigned)((2 * cols + 63) / 64)), dim3(1024), 0, stream, workspace, (int)g, 2 * cols, dweight);
     return check_launch("odl_fp8_layernorm_bwd");
+}
+
+extern "C" int odl_fp8_gelu_table(void *table, odl_stream_t stream_) {
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    if (!table || !aligned16(table)) return set_error(ODL_ERR_ARG, "odl_fp8_gelu_table: null or misaligned table");
+    hipLaunchKernelGGL(gelu_table_kernel, dim3(65536 / 256), dim3(256), 0, stream, reinterpret_cast<uint16_t *>(table),
+                       reinterpret_cast<float *>(reinterpret_cast<uint8_t *>(table) + kGeluFwdBytes));
+    return check_launch("odl_fp8_gelu_table");
+}
+
+extern "C" int odl_fp8_gelu_amax_parts(const void *x, int64_t rows, int64_t cols, const void *table, void *y, float *parts,
+                                       odl_stream_t stream_) {
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    if (rows < 0 || cols < 0) return set_error(ODL_ERR_ARG, "odl_fp8_gelu_amax_parts: negative shape");
+    const int64_t n = rows * cols;
+    if (!parts || !table || (n > 0 && (!x || !y))) return set_error(ODL_ERR_ARG, "odl_fp8_gelu_amax_parts: null pointer");
+    if (n % 8 != 0 || !aligned16(x) || !aligned16(y) || !aligned16(table))
+        return set_error(ODL_ERR_SHAPE, "odl_fp8_gelu_amax_parts: rows*cols must be a multiple of 8 and the pointers 16-byte aligned");
+    const int64_t n8 = n / 8;
+    int64_t g = (n8 + kFusedThreads - 1) / kFusedThreads;
+    g = g < 1 ? 1 : (g < grid_cap() ? g : grid_cap());
+    hipLaunchKernelGGL(gelu_fwd_kernel, dim3((unsigned)g), dim3(kFusedThreads), 0, stream, reinterpret_cast<const u32x4 *>(x), n8,
+                       reinterpret_cast<const uint16_t *>(table), reinterpret_cast<u32x4 *>(y), parts);
+    return check_launch("odl_fp8_gelu_amax_parts");
+}
+
+extern "C" int odl_fp8_gelu_bwd_amax_parts(const void *dy, const void *x, int64_t rows, int64_t cols, const void *table, void *dx,
+                                           float *parts, odl_stream_t stream_) {
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    if (rows < 0 || cols < 0) return set_error(ODL_ERR_ARG, "odl_fp8_gelu_bwd_amax_parts: negative shape");
+    const int64_t n = rows * cols;
+    if (!parts || !table || (n > 0 && (!x || !dy || !dx))) return set_error(ODL_ERR_ARG, "odl_fp8_gelu_bwd_amax_parts: null pointer");
+    if (n % 8 != 0 || !aligned16(x) || !aligned16(dy) || !aligned16(dx) || !aligned16(table))
+        return set_error(ODL_ERR_SHAPE, "odl_fp8_gelu_bwd_amax_parts: rows*cols must be a multiple of 8 and the pointers 16-byte aligned");
+    const int64_t n8 = n / 8;
+    int64_t g = (n8 + kFusedThreads - 1) / kFusedThreads;
+    g = g < 1 ? 1 : (g < grid_cap() ? g : grid_cap());
+    hipLaunchKernelGGL(gelu_bwd_kernel, dim3((unsigned)g), dim3(kFusedThreads), 0, stream, reinterpret_cast<const u32x4 *>(dy),
+                       reinterpret_cast<const u32x4 *>(x), n8,
+                       reinterpret_cast<const float *>(reinterpret_cast<const uint8_t *>(table) + kGeluFwdBytes),
+                       reinterpret_cast<u32x4 *>(dx), parts);
+    return check_launch("odl_fp8_gelu_bwd_amax_parts");
 }

@@ -201,3 +201,52 @@ def fuse_layernorm(norm: nn.Module) -> bool:
     cls = norm.__class__
     norm.__class__ = type(cls.__name__, (_FusedLayerNormForward, cls), {"__module__": cls.__module__})
     return True
+
+
+# --------------------------------------------------------------------------- GELU
+class _GeluFn(torch.autograd.Function):
+    """Exact (erf) GELU of a bf16 tensor, its input kept for the backward."""
+
+    @staticmethod
+    def forward(ctx, x: torch.Tensor, recipe: FP8Recipe):
+        y, parts = native.gelu_amax_parts(x)
+        recipe.offer_parts(y, parts)
+        ctx.save_for_backward(x)
+        ctx.recipe = recipe
+        return y
+
+    @staticmethod
+    def backward(ctx, dy: torch.Tensor):
+        (x,) = ctx.saved_tensors
+        if dy.dtype != torch.bfloat16:
+            dy = dy.to(torch.bfloat16)
+        dx, parts = native.gelu_bwd_amax_parts(dy, x)
+        ctx.recipe.offer_parts(dx, parts)
+        return dx, None
+
+
+def gelu(x: torch.Tensor) -> torch.Tensor | None:
+    """Fused GELU when an FP8 recipe is active and the input is a bf16 GPU tensor; else None."""
+    recipe = _state.active_recipe()
+    if recipe is None or not _bf16_cuda(x) or x.numel() % 8 or x.numel() == 0:
+        return None
+    return _GeluFn.apply(x, recipe)
+
+
+class _FusedGeluForward:
+    """Mixed into the class of an ``nn.GELU`` with the exact (erf) form, the activation of the
+    reference's GELUMLP (mlp.py:141-157)."""
+
+    _odl_fused_gelu = True
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        y = gelu(x)
+        return super().forward(x) if y is None else y
+
+
+def fuse_gelu(act: nn.Module) -> bool:
+    if getattr(act, "_odl_fused_gelu", False) or not isinstance(act, nn.GELU) or getattr(act, "approximate", "none") != "none":
+        return False
+    cls = act.__class__
+    act.__class__ = type(cls.__name__, (_FusedGeluForward, cls), {"__module__": cls.__module__})
+    return True

@@ -20,7 +20,8 @@ Deviations, on purpose:
     keys) so that their forward is the fused kernel that also feeds the next Linear's
     quantisation; ``replace_attention`` is accepted and ignored;
   * ``fuse_swiglu`` (an extra key, default on) does the same for SwiGLU MLPs whose three
-    projections were converted: ``silu(w1 x) * w2 x`` becomes one kernel;
+    projections were converted: ``silu(w1 x) * w2 x`` becomes one kernel; ``fuse_gelu`` (likewise)
+    for exact ``nn.GELU`` modules (the activation of the GPT-2 MLP);
   * a conversion that throws is logged at WARNING (the reference logs at DEBUG).
 """
 
@@ -34,7 +35,7 @@ import torch.nn as nn
 
 from ... import native
 from ..fp8_linear import FP8Linear
-from ..fused import fuse_layernorm, fuse_rmsnorm, fuse_swiglu_mlp
+from ..fused import fuse_gelu, fuse_layernorm, fuse_rmsnorm, fuse_swiglu_mlp
 from . import register_model_transform
 from .base import BaseModelTransform
 from .config import ModelTransformConfig
@@ -103,6 +104,7 @@ class TransformerEngineTransformConfig(ModelTransformConfig):
     verbose: bool = False
     fuse_swiglu: bool = True           # not in the reference: SwiGLU MLPs get the fused activation
     swiglu_classes: tuple = ("SwiGLUMLP",)
+    fuse_gelu: bool = True             # not in the reference: exact nn.GELU modules get the fused activation
 
     def __post_init__(self):
         self.linear_kwargs = dict(self.linear_kwargs or {})
@@ -175,6 +177,9 @@ class TransformerEngineTransform(BaseModelTransform):
         for child_name, child in list(module.named_children()):
             self._replace_modules_recursive(child, replacements, replace_linear, replace_norm, replace_attention,
                                             parent=module, name=child_name)
+        if self.cfg.fuse_gelu and self.cfg.replace_inplace and _get_module_class_name(module) == "torch.nn.modules.activation.GELU" \
+                and fuse_gelu(module):
+            replacements["GELU"] = replacements.get("GELU", 0) + 1
         # after the children: the three projections of an MLP are FP8 Linears by now
         if (self.cfg.fuse_swiglu and self.cfg.replace_inplace and module.__class__.__name__ in tuple(self.cfg.swiglu_classes)
                 and fuse_swiglu_mlp(module)):

@@ -44,6 +44,9 @@ EXPORTS = (
     "odl_fp8_rmsnorm_bwd",
     "odl_fp8_layernorm_amax_parts",
     "odl_fp8_layernorm_bwd",
+    "odl_fp8_gelu_table",
+    "odl_fp8_gelu_amax_parts",
+    "odl_fp8_gelu_bwd_amax_parts",
     "odl_fp8_amax_rowcol",
     "odl_fp8_cast_rowcol",
     "odl_fp8_cast",
@@ -97,6 +100,9 @@ def load() -> ctypes.CDLL:
         L.odl_fp8_rmsnorm_amax_parts.argtypes = [vp, i32, vp, i64, i64, ctypes.c_float, vp, vp, vp, vp]
         L.odl_fp8_rmsnorm_bwd.argtypes = [vp, vp, i32, vp, vp, i64, i64, vp, vp, vp, vp]
         L.odl_fp8_layernorm_amax_parts.argtypes = [vp, i32, vp, vp, i64, i64, ctypes.c_float, vp, vp, vp, vp, vp]
+        L.odl_fp8_gelu_table.argtypes = [vp, vp]
+        L.odl_fp8_gelu_amax_parts.argtypes = [vp, i64, i64, vp, vp, vp, vp]
+        L.odl_fp8_gelu_bwd_amax_parts.argtypes = [vp, vp, i64, i64, vp, vp, vp, vp]
         L.odl_fp8_layernorm_bwd.argtypes = [vp, vp, i32, vp, vp, vp, i64, i64, vp, vp, vp, vp, vp]
         L.odl_fp8_amax_rowcol.argtypes = [vp, i32, i64, i64, vp, vp, vp]
         L.odl_fp8_cast_rowcol.argtypes = [vp, i32, i64, i64, vp, vp, i32, i32, vp, vp, vp, vp, vp, vp, vp]
@@ -406,6 +412,52 @@ def layernorm_bwd(dy: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, mean:
                                         dx.data_ptr(), dwb.data_ptr(), dwb[cols:].data_ptr(), ws.data_ptr(), _stream()),
            "odl_fp8_layernorm_bwd")
     return dx, dwb[:cols], dwb[cols:]
+
+
+GELU_TABLE_BYTES = 65536 * 2 + 65536 * 4
+_gelu_tables: dict[int, torch.Tensor] = {}
+
+
+def gelu_table(device: torch.device) -> torch.Tensor:
+    """The GELU lookup table of ``device`` (384 KB, filled on first use and kept for the process)."""
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    t = _gelu_tables.get(idx)
+    if t is None:
+        with _lock:
+            t = _gelu_tables.get(idx)
+            if t is None:
+                t = torch.empty(GELU_TABLE_BYTES, dtype=torch.uint8, device=torch.device("cuda", idx))
+                with torch.cuda.device(idx):
+                    _check(load().odl_fp8_gelu_table(t.data_ptr(), _stream()), "odl_fp8_gelu_table")
+                    torch.cuda.current_stream().synchronize()     # other streams may use it right away
+                _gelu_tables[idx] = t
+    return t
+
+
+def gelu_amax_parts(x: torch.Tensor):
+    """Exact GELU of a bf16 tensor and the partial maxima of the result.  -> (y, parts)."""
+    x = _bf16_dense(x, "gelu x")
+    cols = x.shape[-1] if x.dim() else 1
+    rows = x.numel() // max(cols, 1)
+    y = torch.empty_like(x)
+    parts = torch.empty(AMAX_PARTS, dtype=torch.float32, device=x.device)
+    _check(load().odl_fp8_gelu_amax_parts(x.data_ptr(), rows, cols, gelu_table(x.device).data_ptr(), y.data_ptr(), parts.data_ptr(),
+                                          _stream()), "odl_fp8_gelu_amax_parts")
+    return y, parts
+
+
+def gelu_bwd_amax_parts(dy: torch.Tensor, x: torch.Tensor):
+    """dx = dy * gelu'(x) in bf16 and its partial maxima.  -> (dx, parts)."""
+    dy, x = _bf16_dense(dy, "gelu dy"), _bf16_dense(x, "gelu x")
+    if dy.shape != x.shape:
+        raise NativeError(f"gelu backward: dy {tuple(dy.shape)} and x {tuple(x.shape)} differ")
+    cols = x.shape[-1] if x.dim() else 1
+    rows = x.numel() // max(cols, 1)
+    dx = torch.empty_like(x)
+    parts = torch.empty(AMAX_PARTS, dtype=torch.float32, device=x.device)
+    _check(load().odl_fp8_gelu_bwd_amax_parts(dy.data_ptr(), x.data_ptr(), rows, cols, gelu_table(x.device).data_ptr(), dx.data_ptr(),
+                                              parts.data_ptr(), _stream()), "odl_fp8_gelu_bwd_amax_parts")
+    return dx, parts
 
 
 def quantize_rowcol(x: torch.Tensor, fmt: int, margin: int = 0):

@@ -486,3 +486,26 @@ ORACLE_API void oracle_layernorm_bwd(const uint16_t *dy, const void *x, int src,
     for (int64_t c = 0; c < cols; ++c) { dweight[c] = (float)dw[c]; dbias[c] = (float)dw[cols + c]; }
     free(dw);
 }
+
+/* Exact (erf) GELU of a bf16 input, nn.GELU() in optimus_dl/modules/model/blocks/mlp.py:141-157, and
+ * its derivative, evaluated in double precision with libm and rounded once to float (then bf16 for
+ * the forward): the definition of the library's lookup table.  Pinned in tests/test_oracle_fused.py
+ * against torch's F.gelu and autograd over every bf16 input (torch evaluates 1 + erf(x / sqrt 2) in
+ * float, which loses the far negative tail: there the comparison is absolute). */
+ORACLE_API void oracle_gelu_fwd(const uint16_t *x, int64_t n, uint16_t *y) {
+    for (int64_t i = 0; i < n; ++i) {
+        double v = (double)bf16_to_f32(x[i]);
+        double cdf = 0.5 * erfc(-v * 0.70710678118654752440);
+        y[i] = f32_to_bf16((float)(v * cdf));
+    }
+}
+
+ORACLE_API void oracle_gelu_bwd(const uint16_t *dy, const uint16_t *x, int64_t n, uint16_t *dx) {
+    for (int64_t i = 0; i < n; ++i) {
+        double v = (double)bf16_to_f32(x[i]);
+        double cdf = 0.5 * erfc(-v * 0.70710678118654752440);
+        double pdf = exp(-0.5 * v * v) * 0.39894228040143267794;
+        float d = (float)(cdf + v * pdf);
+        dx[i] = f32_to_bf16(bf16_to_f32(dy[i]) * d);
+    }
+}

@@ -71,6 +71,8 @@ def lib() -> ctypes.CDLL:
         L.oracle_swiglu_bwd.argtypes = [vp, vp, vp, i64, vp, vp]
         L.oracle_rmsnorm.argtypes = [vp, i32, vp, i64, i64, f32, vp, vp]
         L.oracle_rmsnorm_bwd.argtypes = [vp, vp, i32, vp, vp, i64, i64, vp, vp]
+        L.oracle_gelu_fwd.argtypes = [vp, i64, vp]
+        L.oracle_gelu_bwd.argtypes = [vp, vp, i64, vp]
         L.oracle_layernorm.argtypes = [vp, i32, vp, vp, i64, i64, f32, vp, vp, vp]
         L.oracle_layernorm_bwd.argtypes = [vp, vp, i32, vp, vp, vp, i64, i64, vp, vp, vp]
         _lib = L
@@ -258,6 +260,20 @@ def c_layernorm_bwd(dy: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, mea
     lib().oracle_layernorm_bwd(_p(d), _p(xs), src, _p(w), _p(mu), _p(rs), rows, cols, _p(dx), _p(dw), _p(db))
     dx_t = _from_bf16_bits(dx, x.shape) if src == 0 else torch.from_numpy(dx).reshape(x.shape)
     return dx_t, torch.from_numpy(dw), torch.from_numpy(db)
+
+
+def c_gelu_fwd(x: torch.Tensor) -> torch.Tensor:
+    xs = _bf16_bits(x)
+    y = np.empty_like(xs)
+    lib().oracle_gelu_fwd(_p(xs), xs.size, _p(y))
+    return _from_bf16_bits(y, x.shape)
+
+
+def c_gelu_bwd(dy: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
+    d, xs = _bf16_bits(dy), _bf16_bits(x)
+    dx = np.empty_like(xs)
+    lib().oracle_gelu_bwd(_p(d), _p(xs), xs.size, _p(dx))
+    return _from_bf16_bits(dx, x.shape)
 
 
 def t_amax(x: torch.Tensor, mode: int = SCALE_TENSOR) -> torch.Tensor:

@@ -310,3 +310,37 @@ def test_kernels_against_golden_norm_vectors(N):
         assert torch.allclose(rstd.cpu(), _f32_from_hex(case["ln_rstd_f32_hex"]), rtol=1e-6, atol=0)
         d = (y.cpu().view(torch.int16).int() - _bf16_from_hex(case["ln_y_bf16_hex"], shape).view(torch.int16).int()).abs()
         assert int(d.max()) <= 1 and float((d > 0).float().mean()) < 0.01
+
+
+# ------------------------------------------------------------------------ GELU
+def test_gelu_forward_every_bf16_input(N):
+    x = all_bf16().reshape(256, 256)
+    y, parts = N.gelu_amax_parts(x.cuda())
+    assert_bf16_equal(y, O.c_gelu_fwd(x), "gelu, every bf16 input")
+    assert torch.isnan(parts_max(parts))
+    fin = torch.where(torch.isfinite(x.float()), x, torch.zeros_like(x))
+    y, parts = N.gelu_amax_parts(fin.cuda())
+    assert_f32_bits_equal(parts_max(parts).reshape(1), O.c_gelu_fwd(fin).float().abs().max().reshape(1), "gelu parts")
+
+
+@pytest.mark.parametrize("dy_std", [1.0, 1e-3])
+def test_gelu_backward_every_bf16_input(N, dy_std):
+    x = all_bf16().reshape(256, 256)
+    dy = seeded_bf16((256, 256), dy_std, 17)
+    dx, parts = N.gelu_bwd_amax_parts(dy.cuda(), x.cuda())
+    assert_bf16_equal(dx, O.c_gelu_bwd(dy, x), "gelu backward, every bf16 input")
+
+
+@pytest.mark.parametrize("shape", [(16, 24), (1, 8), (1000, 8), (4, 96, 768), (2048, 3072)])
+def test_gelu_shapes_and_parts(N, shape):
+    x, dy = seeded_bf16(shape, 1.5, 41), seeded_bf16(shape, 1e-2, 42)
+    y, parts = N.gelu_amax_parts(x.cuda())
+    want = O.c_gelu_fwd(x)
+    assert_bf16_equal(y, want, f"gelu {shape}")
+    assert_f32_bits_equal(parts_max(parts).reshape(1), want.float().abs().max().reshape(1), "gelu parts")
+    dx, parts = N.gelu_bwd_amax_parts(dy.cuda(), x.cuda())
+    wdx = O.c_gelu_bwd(dy, x)
+    assert_bf16_equal(dx, wdx, f"gelu bwd {shape}")
+    assert_f32_bits_equal(parts_max(parts).reshape(1), wdx.float().abs().max().reshape(1), "gelu bwd parts")
+    with pytest.raises(N.NativeError, match="multiple of 8"):
+        N.gelu_amax_parts(torch.zeros((3, 5), dtype=torch.bfloat16).cuda())

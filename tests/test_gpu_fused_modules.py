@@ -301,3 +301,34 @@ def test_fused_layernorm_in_a_gpt2_block(amp, monkeypatch, in_dtype):
     for a, b, tol in zip(outs["fused"], outs["plain"], (1e-2, 2e-2, 2e-2, 2e-2, 1e-2)):
         assert max_rel_err(a, b) <= tol
     assert outs["fused"][1].dtype == in_dtype
+
+
+def test_gpt2_mlp_with_fused_gelu(amp, monkeypatch):
+    """c_proj(gelu(c_fc(x))) with biases: the transform re-classes nn.GELU, c_proj takes the activation's maxima,
+    c_fc's backward takes the gradient's, and the results agree with PyTorch's GELU."""
+    from optimus_dl_amd import native
+    from optimus_dl_amd.modules.model.blocks import GELUMLP
+    from optimus_dl_amd.modules.model_transforms import build_model_transform
+
+    def build(fuse):
+        torch.manual_seed(0)
+        m = GELUMLP(256, 1024, bias=True).to("cuda", torch.bfloat16)
+        t = build_model_transform({"_name": "transformer_engine", "fuse_gelu": fuse})
+        t.apply(m)
+        assert t.last_replacements.get("GELU", 0) == (1 if fuse else 0) and isinstance(m.gelu, nn.GELU)
+        return m
+
+    M = 384
+    x = seeded_bf16((M, 256), 1.0, 1).cuda()
+    dy = seeded_bf16((M, 256), 1e-2, 2).cuda()
+    recipe = amp.FP8Recipe(recipe_type="tensorwise")
+    amax_calls = count_calls(monkeypatch, native, "amax_parts")
+    colsum_calls = count_calls(monkeypatch, native, "amax_parts_colsum")
+    fused = step(build(True), recipe, x, dy)
+    # x and the two weights by amax_parts; dy of c_proj by the amax + column-sum pass (bias); h and dh's product arrive with maxima
+    assert sorted(amax_calls) == sorted([(M, 256), (1024, 256), (256, 1024)]) and colsum_calls == [(M, 256)]
+    amax_calls.clear(); colsum_calls.clear()
+    plain = step(build(False), recipe, x, dy)
+    assert (M, 1024) in amax_calls and (M, 1024) in colsum_calls
+    for a, b in zip(fused, plain):
+        assert max_rel_err(a, b) <= 1e-2

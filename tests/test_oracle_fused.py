@@ -281,3 +281,48 @@ def test_layernorm_backward_against_torch_autograd(cols, dtype):
     assert dx.dtype == dtype and (dx.double() - xa.grad).abs().max().item() <= tol * scale
     assert ((dw.double() - wa.grad).abs() / wa.grad.abs().max()).max().item() < 1e-5
     assert ((db.double() - ba.grad).abs() / ba.grad.abs().max()).max().item() < 1e-5
+
+
+# ------------------------------------------------------------------------ GELU
+def test_gelu_every_bf16_input_against_torch_and_float64():
+    x = all_bf16()
+    with np.errstate(invalid="ignore"):
+        xs = x.float().numpy().astype(np.float64)
+    y = O.c_gelu_fwd(x)
+    finite = np.isfinite(xs)
+    # float64 closed form with scipy's erfc: the oracle is its value rounded to float, then to bf16
+    from scipy.special import erfc
+
+    with np.errstate(over="ignore", invalid="ignore"):
+        exact = xs[finite] * 0.5 * erfc(-xs[finite] / np.sqrt(2.0))
+    want = torch.from_numpy(exact.astype(np.float32)).bfloat16()
+    assert torch.equal(y[torch.from_numpy(finite)].view(torch.int16), want.view(torch.int16))
+    # torch's own F.gelu (1 + erf evaluated in float): identical wherever that formula is accurate and neither
+    # side is in the denormal / overflow range; below -3 torch loses the tail: absolute comparison there
+    t = F.gelu(x)
+    ys, ts = y.float().numpy(), t.float().numpy()
+    core = finite & (xs >= -3.0) & (np.abs(xs) < 1e38) & (np.abs(ys) >= 1.2e-38)
+    assert core.sum() > 48000
+    assert np.array_equal(y.view(torch.int16).numpy()[core], t.view(torch.int16).numpy()[core])
+    tail = finite & (xs < -3.0)
+    assert np.abs(ys[tail] - ts[tail]).max() < 2e-5
+    assert np.isnan(ys[np.isnan(xs)]).all() and ys[xs == np.inf][0] == np.inf
+
+
+def test_gelu_backward_against_torch_autograd():
+    x = all_bf16()
+    keep = torch.isfinite(x.float())
+    xk = x[keep]
+    for scale in (1.0, -0.0078125, 3.0):
+        dy = torch.full_like(xk, scale)
+        xa = xk.clone().requires_grad_(True)
+        F.gelu(xa).backward(dy)
+        dx = O.c_gelu_bwd(dy, xk)
+        xs = xk.float().numpy()
+        core = (xs >= -3.0) & (np.abs(xs) < 1e38)
+        d = ulp_distance(dx, xa.grad)
+        assert d[core].max() <= 1 and (d[core] > 0).mean() < 0.01
+        assert np.abs(dx.float().numpy() - xa.grad.float().numpy())[~core & np.isfinite(xa.grad.float().numpy())].max() < 4e-5 * abs(scale) + 1e-30
+    # closed-form spot values: gelu'(0) = 1/2, gelu'(large) = 1, gelu'(-large) = 0
+    pts = torch.tensor([0.0, 20.0, -20.0], dtype=torch.bfloat16)
+    assert O.c_gelu_bwd(torch.ones_like(pts), pts).tolist() == [0.5, 1.0, 0.0]
