@@ -202,6 +202,57 @@ def mlp_block(torch, native, recipe, steps=10, warmup=3):
     return out
 
 
+def llama_block(torch, steps=6, warmup=2):
+    """One Llama-3-8B decoder block (RMSNorm, GQA attention with 32 / 8 heads, SwiGLU MLP; fp32 residual stream,
+    batch 4 x 2048 tokens), forward + backward, weights re-quantised every step: bf16 autocast, FP8 Linears alone, and FP8
+    Linears with the fused RMSNorm / SwiGLU producers.  Attention itself is PyTorch's scaled_dot_product_attention in all three."""
+    from optimus_dl_amd.modules import amp as A
+    from optimus_dl_amd.modules.model.blocks import LlamaBlock
+    from optimus_dl_amd.modules.model_transforms import build_model_transform
+
+    B, T = 4, 2048
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    x = torch.randn(B, T, D_MODEL, device="cuda", generator=gen).requires_grad_(True)
+    dy = torch.randn(B, T, D_MODEL, device="cuda", generator=gen) * 1e-3
+    out = {}
+    for label, cfg in (("bf16_autocast", None),
+                       ("fp8_linears", {"_name": "fp8_linear", "replace_norm": False, "fuse_swiglu": False}),
+                       ("fp8_linears_fused_norm_swiglu", {"_name": "fp8_linear"})):
+        torch.manual_seed(0)
+        blk = LlamaBlock(D_MODEL, 32, 8, D_FF).cuda()
+        if cfg:
+            build_model_transform(cfg).apply(blk)
+        recipe = A.FP8Recipe(recipe_type="tensorwise")
+
+        def one():
+            for p_ in blk.parameters():
+                p_.grad = None
+            x.grad = None
+            for m in blk.modules():
+                if hasattr(m, "_wcache"):
+                    m._wcache.key = None
+            if cfg:
+                with A.fp8_autocast(torch.device("cuda"), recipe):
+                    y = blk(x)
+                with A.fp8_backward(recipe):
+                    y.backward(dy)
+            else:
+                with torch.autocast("cuda", dtype=torch.bfloat16):
+                    y = blk(x)
+                y.backward(dy)
+
+        for _ in range(warmup):
+            one()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            one()
+        torch.cuda.synchronize()
+        out[label] = {"ms_per_step": 1e3 * (time.perf_counter() - t0) / steps}
+        del blk
+    return out
+
+
 def cpu_baseline(torch, seconds_hint=20.0):
     """The oracle's emulated-FP8 Linear fwd+bwd on the host cores, on a slice of the rows."""
     from oracle import oracle as O
@@ -374,6 +425,7 @@ def main() -> int:
     if not args.no_standalone:
         del layers, data
         line["mlp_block_fwd_bwd"] = mlp_block(torch, native, recipe)
+        line["llama3_8b_block_fwd_bwd"] = llama_block(torch)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(torch)
     print(json.dumps(line))
