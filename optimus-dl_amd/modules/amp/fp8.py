@@ -193,6 +193,10 @@ class FP8Recipe:
         # (gate/up, q/k/v) quantise it once; dropped when the outermost context is left
         self.shared_input: dict[str, Any] | None = None
         self.share_inputs = True
+        # quantised weights are kept while the Parameter's version counter stands still (microbatches of one
+        # optimizer step).  Code that rewrites weights through ``param.data`` does not move that counter:
+        # set this to False there, and every forward quantises its weight again (what the reference does).
+        self.cache_weights = True
         # wgrad reads the row-major codes of dy with the tokens as the slow axis where the shapes allow
         # (no transposed copy of dy); False keeps the cast+transpose route everywhere
         self.direct_layouts = True

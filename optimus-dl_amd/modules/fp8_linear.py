@@ -156,6 +156,8 @@ class _Fp8LinearFn(torch.autograd.Function):
                 xq, sx_inv, saved["xq_t"], saved["sx_inv_t"], _, _ = native.quantize_rowcol(x2d, pol.fmt_fwd, pol.margin)
             else:
                 xq, sx_inv = _quantise_axis(x2d, pol.fmt_fwd, pol.margin, R, False)
+            if not recipe.cache_weights:
+                module._wcache_rowwise.clear()          # the backward of this call still finds what is made now
             wq, sw_inv = module._rowwise_weight(weight, pol, "row", both=need_dgrad)
             y = native.gemm_nt(xq, wq, pol.fmt_fwd, pol.fmt_fwd, sx_inv, sw_inv, bias=bias_f32, out_dtype=out_dtype)
         else:
@@ -299,7 +301,7 @@ class FP8Linear(nn.Linear):
         c = self._wcache
         # delayed scaling: the codes depend on the scale in force, which changes at every refresh
         key = (weight.data_ptr(), weight._version, id(recipe), pol.kind, recipe.scale_epoch if pol.kind == "delayed" else 0)
-        fresh = c.key != key
+        fresh = c.key != key or not recipe.cache_weights
         if fresh or (need_t and c.wq_t is None):
             w2d = weight.detach()
             if pol.kind == "delayed":

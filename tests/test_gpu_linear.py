@@ -438,3 +438,25 @@ def test_nan_and_inf_inputs_do_not_poison_the_scales(amp):
     with torch.no_grad(), recipe.autocast():
         y = lin(x.cuda())
     assert torch.isfinite(y.float()).all()              # amax = Inf -> scale 1, the Inf element clamps to 448
+
+
+def test_cache_weights_switch_requantises_after_a_data_write(amp, monkeypatch):
+    from optimus_dl_amd import native
+
+    w = seeded_bf16((256, 512), 0.02, 1)
+    lin = make_linear(w)
+    x = seeded_bf16((256, 512), 1.0, 2).cuda()
+    recipe = amp.create_fp8_recipe("tensorwise", "hybrid")
+    with recipe.autocast():
+        y0 = lin(x)
+    lin.weight.data.mul_(2.0)                      # does not move weight._version
+    with recipe.autocast():
+        stale = lin(x)
+    assert torch.equal(stale, y0)                  # the cached codes were used: the documented caveat
+    recipe.cache_weights = False
+    calls = _count_calls(monkeypatch, native, "amax_parts")
+    with recipe.autocast():
+        fresh = lin(x)
+        again = lin(x)
+    assert calls.count((256, 512)) >= 2            # the weight (and x, same shape here) quantised on every forward
+    assert torch.equal(fresh, again) and max_rel_err(fresh, 2 * y0.float()) <= TOL
