@@ -356,8 +356,12 @@ def _f32_vector(t: torch.Tensor | None, n: int, device, what: str) -> torch.Tens
     if t is None:
         return None
     v = t.detach()
-    if v.dtype != torch.float32 or not v.is_contiguous() or v.data_ptr() % 16:
-        v = v.float().contiguous().clone()
+    if v.dtype != torch.float32:
+        v = v.float()
+    if not v.is_contiguous():
+        v = v.contiguous()
+    if v.data_ptr() % 16:
+        v = v.clone()
     if v.numel() != n or v.device != device:
         raise NativeError(f"{what}: {v.numel()} elements on {v.device}, expected {n} on {device}")
     return v
