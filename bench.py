@@ -144,9 +144,14 @@ def standalone_hbm(torch, native, iters=24):
             xs32 = [x.float() for x in xs]
             to32 = {id(x): y for x, y in zip(xs, xs32)}
             kernels["rmsnorm_amax_fp32_in"] = (lambda x: native.rmsnorm_amax_parts(to32[id(x)], w_norm, 1e-5), 6 * E)
+            kernels["layernorm_amax_bf16_in"] = (lambda x: native.layernorm_amax_parts(x, w_norm, w_norm, 1e-5), 4 * E)
+            kernels["gelu_fwd_amax"] = (lambda x: native.gelu_amax_parts(x), 4 * E)
             _, rstd_b, _ = native.rmsnorm_amax_parts(xs[0], w_norm, 1e-5)
             dy_of = {id(x): xs[(i + 1) % nbuf] for i, x in enumerate(xs)}
             kernels["rmsnorm_bwd_bf16"] = (lambda x: native.rmsnorm_bwd(dy_of[id(x)], x, w_norm, rstd_b), 6 * E)
+            _, mean_l, rstd_l, _ = native.layernorm_amax_parts(xs[0], w_norm, w_norm, 1e-5)
+            kernels["layernorm_bwd_bf16"] = (lambda x: native.layernorm_bwd(dy_of[id(x)], x, w_norm, mean_l, rstd_l), 6 * E)
+            kernels["gelu_bwd_amax"] = (lambda x: native.gelu_bwd_amax_parts(dy_of[id(x)], x), 6 * E)
         for name, (fn, nbytes) in kernels.items():
             for x in xs:
                 fn(x)
