@@ -176,10 +176,14 @@ int odl_fp8_rmsnorm_amax_parts(const void *x, int src_dtype, const float *weight
 
 /*
  * Backward of that RMSNorm (what autograd derives for layer_norms.py:86-119), dy in bf16:
- *   xh = x * rstd, t = dy * weight, c = sum_row(t * xh) / cols  (summed in the order of the forward)
+ *   xh = x * rstd, t = dy * weight, c = sum_row(t * xh) / cols
  *   dx = rstd * fma(-xh, c, t), rounded once to the dtype of x (src_dtype)
- *   dweight[col] = sum over rows of dy * xh, fp32 (per-wave, per-block and per-slab partial sums
- *   in a fixed order: reproducible from run to run on one device)
+ *   Row sums of the backward kernels (this one and the LayerNorm one): the 8-element chunk k of a row
+ *   belongs to wave (k / 64) % 4 and lane k % 64 of a 4-wave block; a lane adds its chunks in ascending
+ *   order (t * xh by fma, elements in order), the 64 lanes of a wave are combined by the butterfly
+ *   acc[l] += acc[l ^ off], off = 32 .. 1, and the four waves as ((s0 + s1) + s2) + s3.
+ *   dweight[col] = sum over rows of dy * xh, fp32 (per-lane sums over the rows of a block, then the
+ *   blocks' slabs in a fixed order: reproducible from run to run on one device)
  * workspace: ODL_FP8_RMSNORM_BWD_SLABS * cols floats of device memory, contents irrelevant.
  */
 #define ODL_FP8_RMSNORM_BWD_SLABS 512
@@ -191,7 +195,8 @@ int odl_fp8_rmsnorm_bwd(const void *dy, const void *x, int src_dtype, const floa
  * LayerNorm (F.layer_norm over the last axis, optimus_dl/modules/model/blocks/layer_norms.py:21-47
  * and torch.nn.LayerNorm, both of which the reference's transform replaces,
  * transformer_engine.py:338-352) with the partial maxima of its output, and its backward.
- * Same row split and summation order as the RMSNorm entry points; 8 <= cols <= 4096.
+ * Forward: row split and summation order of the RMSNorm forward; backward: those of the RMSNorm
+ * backward; 8 <= cols <= 4096.
  *   mean = sum(x) / cols; d = x - mean; rstd = 1 / sqrt(sum(d * d) / cols + eps)  (d * d added by fma)
  *   y    = bf16( ((d * rstd) * weight) + bias ), bias may be NULL
  *   backward (dy bf16): xh = d * rstd, t = dy * weight, c1 = sum(t) / cols, c2 = sum(t * xh) / cols,

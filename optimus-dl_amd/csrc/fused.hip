@@ -219,123 +219,144 @@ __global__ __launch_bounds__(kRmsThreads) void rmsnorm_fwd_kernel(const void *__
         for (int j = (int)gridDim.x + threadIdx.x; j < kParts; j += kRmsThreads) parts[j] = 0.0f;
 }
 
-// ------------------------------------------------------------------ RMSNorm backward
-// Same work split as the forward (one wavefront per row, lane l holds chunks l, l + 64, ...).
-//   xh = x * rstd, t = dy * weight, c = sum(t * xh) / cols  (per lane by fma in element order,
-//   then the xor butterfly), dx = rstd * fma(-xh, c, t): every dx is a fixed sequence of IEEE
-//   operations, rounded once to the dtype of x.
-// d_weight[col] = sum over rows of dy * xh: a lane adds up its columns over the rows its wave
-// visits, the waves of a block are combined through LDS in wave order, each block writes one
-// slab of `cols` sums to the workspace, and a second kernel adds the slabs in block order.
-constexpr int kRmsBwdThreads = 256;
-
-template <int SRC, int CPL>
-__global__ __launch_bounds__(kRmsBwdThreads) void rmsnorm_bwd_kernel(const u32x4 *__restrict__ dy, const void *__restrict__ x,
-                                                                      const float *__restrict__ weight, const float *__restrict__ rstd_in,
-                                                                      int64_t rows, int64_t cols, void *__restrict__ dx,
-                                                                      float *__restrict__ slabs) {
-    extern __shared__ float lds_dw[];                        // cols floats
-    constexpr int VPC = SRC == ODL_BF16 ? 1 : 2;
-    const int lane = threadIdx.x % kWave, wave_in_block = threadIdx.x / kWave;
-    const int64_t wave = (int64_t)blockIdx.x * (kRmsBwdThreads / kWave) + wave_in_block;
-    const int64_t nwave = (int64_t)gridDim.x * (kRmsBwdThreads / kWave);
-    const int64_t nchunk = cols / 8;
-    float dw[CPL][8];
-#pragma unroll
-    for (int j = 0; j < CPL; ++j)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) dw[j][e] = 0.0f;
-    for (int64_t row = wave; row < rows; row += nwave) {
-        u32x4 xr[CPL][VPC], dr[CPL];
-#pragma unroll
-        for (int j = 0; j < CPL; ++j) {
-            const int64_t c = lane + (int64_t)kWave * j;
-            const bool ok = c < nchunk;
-            const u32x4 *p = reinterpret_cast<const u32x4 *>(x) + (row * nchunk + c) * VPC;
-#pragma unroll
-            for (int h = 0; h < VPC; ++h) xr[j][h] = ok ? __builtin_nontemporal_load(p + h) : u32x4{0, 0, 0, 0};
-            dr[j] = ok ? __builtin_nontemporal_load(dy + row * nchunk + c) : u32x4{0, 0, 0, 0};
-        }
-        const float rstd = rstd_in[row];
-        float acc = 0.0f;
-#pragma unroll
-        for (int j = 0; j < CPL; ++j) {
-            const int64_t c = lane + (int64_t)kWave * j;
-            if (c < nchunk) {
-                float xf[8], df[8];
-                unpack8<SRC>(xr[j], xf);
-                unpack8<ODL_BF16>(&dr[j], df);
-                const float4 w0 = *reinterpret_cast<const float4 *>(weight + c * 8), w1 = *reinterpret_cast<const float4 *>(weight + c * 8 + 4);
-                const float w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const float xh = __fmul_rn(xf[e], rstd);
-                    acc = __fmaf_rn(__fmul_rn(df[e], w[e]), xh, acc);
-                    dw[j][e] = __fmaf_rn(df[e], xh, dw[j][e]);
-                }
-            }
-        }
-#pragma unroll
-        for (int off = kWave / 2; off > 0; off >>= 1) acc = __fadd_rn(acc, __shfl_xor(acc, off, kWave));
-        const float cmean = __fdiv_rn(acc, (float)cols);
-#pragma unroll
-        for (int j = 0; j < CPL; ++j) {
-            const int64_t c = lane + (int64_t)kWave * j;
-            if (c < nchunk) {
-                float xf[8], df[8], o[8];
-                unpack8<SRC>(xr[j], xf);
-                unpack8<ODL_BF16>(&dr[j], df);
-                const float4 w0 = *reinterpret_cast<const float4 *>(weight + c * 8), w1 = *reinterpret_cast<const float4 *>(weight + c * 8 + 4);
-                const float w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const float xh = __fmul_rn(xf[e], rstd);
-                    o[e] = __fmul_rn(rstd, __fmaf_rn(-xh, cmean, __fmul_rn(df[e], w[e])));
-                }
-                if constexpr (SRC == ODL_BF16) {
-                    reinterpret_cast<u32x4 *>(dx)[row * nchunk + c] =
-                        u32x4{pack2(o[0], o[1]), pack2(o[2], o[3]), pack2(o[4], o[5]), pack2(o[6], o[7])};
-                } else {
-                    float4 *q = reinterpret_cast<float4 *>(dx) + (row * nchunk + c) * 2;
-                    q[0] = float4{o[0], o[1], o[2], o[3]};
-                    q[1] = float4{o[4], o[5], o[6], o[7]};
-                }
-            }
-        }
-    }
-    // waves of the block, in order, into the LDS row; then the block's slab
-    for (int wv = 0; wv < kRmsBwdThreads / kWave; ++wv) {
-        if (wave_in_block == wv) {
-#pragma unroll
-            for (int j = 0; j < CPL; ++j) {
-                const int64_t c = lane + (int64_t)kWave * j;
-                if (c < nchunk) {
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        float *slot = &lds_dw[c * 8 + e];
-                        *slot = wv == 0 ? dw[j][e] : __fadd_rn(*slot, dw[j][e]);
-                    }
-                }
-            }
-        }
-        __syncthreads();
-    }
-    for (int64_t c = threadIdx.x; c < cols; c += kRmsBwdThreads) slabs[(int64_t)blockIdx.x * cols + c] = lds_dw[c];
-}
-
-// ------------------------------------------------------------------------ LayerNorm
-// Same work split and summation order as the RMSNorm kernels.  Forward, per row:
-//   mean = sum(x) / cols;  d = x - mean;  rstd = 1 / sqrt(sum(d * d) / cols + eps)   (d * d by fma)
-//   y = bf16( ((d * rstd) * weight) + bias )          (bias may be absent)
-// Backward, dy in bf16:  xh = d * rstd, t = dy * weight, c1 = sum(t) / cols, c2 = sum(t * xh) / cols
-//   dx = rstd * fma(-xh, c2, t - c1);  d_weight = sum_rows dy * xh;  d_bias = sum_rows dy
-// (slabs hold d_weight in [0, cols) and d_bias in [cols, 2 cols) of each block's row).
 __device__ __forceinline__ float wave_sum_butterfly(float acc) {
 #pragma unroll
     for (int off = kWave / 2; off > 0; off >>= 1) acc = __fadd_rn(acc, __shfl_xor(acc, off, kWave));
     return acc;
 }
 
+// ------------------------------------------------------- RMSNorm / LayerNorm backward
+// One BLOCK of four waves per row, rows dealt round-robin to the blocks; the next row's loads are in
+// flight while the current one is worked on.  The 8-element chunk c of a row belongs to wave
+// (c / 64) % 4, lane c % 64, slot c / 256, so a lane owns the same columns in every row: the weights
+// of those columns stay in registers and d_weight / d_bias are plain per-lane sums over the rows of
+// the block (no reduction inside the block), written as one slab per block and added up over the
+// blocks by rmsnorm_bwd_reduce_kernel.
+//   xh = (x - mean) * rstd   (RMSNorm: x * rstd),   t = dy * weight
+//   row sums  S1 = sum t (LayerNorm only), S2 = sum t * xh: per lane over its slots in ascending order and
+//   the elements of a chunk in order (t * xh by fma), xor butterfly 32..1 inside the wave, then the four
+//   wave sums as ((s0 + s1) + s2) + s3;  c1 = S1 / cols, c2 = S2 / cols
+//   dx = rstd * fma(-xh, c2, t - c1)   (RMSNorm: rstd * fma(-xh, c2, t)), rounded once to the dtype of x.
+constexpr int kRmsBwdThreads = 256;
+
+template <int SRC, bool LN, int CPLW>
+__global__ __launch_bounds__(kRmsBwdThreads) void norm_bwd_kernel(const u32x4 *__restrict__ dy, const void *__restrict__ x,
+                                                                   const float *__restrict__ weight, const float *__restrict__ mean_in,
+                                                                   const float *__restrict__ rstd_in, int64_t rows, int64_t cols,
+                                                                   void *__restrict__ dx, float *__restrict__ slabs) {
+    __shared__ float rsum[2][2][kRmsBwdThreads / kWave];
+    constexpr int VPC = SRC == ODL_BF16 ? 1 : 2;
+    constexpr int NS = LN ? 2 : 1;                            // accumulator sets per lane (d_weight, d_bias)
+    const int lane = threadIdx.x % kWave, wv = threadIdx.x / kWave;
+    const int64_t nchunk = cols / 8;
+    int64_t chunk[CPLW];
+    float wreg[CPLW][8], dw[CPLW][8], db[LN ? CPLW : 1][8];
+#pragma unroll
+    for (int j = 0; j < CPLW; ++j) {
+        chunk[j] = (int64_t)(j * 4 + wv) * kWave + lane;
+        const bool ok = chunk[j] < nchunk;
+        const float4 w0 = ok ? *reinterpret_cast<const float4 *>(weight + chunk[j] * 8) : float4{0, 0, 0, 0};
+        const float4 w1 = ok ? *reinterpret_cast<const float4 *>(weight + chunk[j] * 8 + 4) : float4{0, 0, 0, 0};
+        wreg[j][0] = w0.x; wreg[j][1] = w0.y; wreg[j][2] = w0.z; wreg[j][3] = w0.w;
+        wreg[j][4] = w1.x; wreg[j][5] = w1.y; wreg[j][6] = w1.z; wreg[j][7] = w1.w;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { dw[j][e] = 0.0f; if constexpr (LN) db[j][e] = 0.0f; }
+    }
+    u32x4 nx[CPLW][VPC], nd[CPLW];
+    auto fetch = [&](int64_t row) {
+#pragma unroll
+        for (int j = 0; j < CPLW; ++j) {
+            const bool ok = chunk[j] < nchunk && row < rows;
+            const u32x4 *p = reinterpret_cast<const u32x4 *>(x) + (row * nchunk + chunk[j]) * VPC;
+#pragma unroll
+            for (int h = 0; h < VPC; ++h) nx[j][h] = ok ? __builtin_nontemporal_load(p + h) : u32x4{0, 0, 0, 0};
+            nd[j] = ok ? __builtin_nontemporal_load(dy + row * nchunk + chunk[j]) : u32x4{0, 0, 0, 0};
+        }
+    };
+    fetch(blockIdx.x);
+    int par = 0;
+    for (int64_t row = blockIdx.x; row < rows; row += gridDim.x, par ^= 1) {
+        u32x4 xr[CPLW][VPC], dr[CPLW];
+#pragma unroll
+        for (int j = 0; j < CPLW; ++j) {
+#pragma unroll
+            for (int h = 0; h < VPC; ++h) xr[j][h] = nx[j][h];
+            dr[j] = nd[j];
+        }
+        fetch(row + gridDim.x);                               // rows past the end load nothing
+        const float rstd = rstd_in[row];
+        const float mean = LN ? mean_in[row] : 0.0f;
+        float a1 = 0.0f, a2 = 0.0f;
+#pragma unroll
+        for (int j = 0; j < CPLW; ++j) {
+            if (chunk[j] < nchunk) {
+                float xf[8], df[8];
+                unpack8<SRC>(xr[j], xf);
+                unpack8<ODL_BF16>(&dr[j], df);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float xh = LN ? __fmul_rn(__fsub_rn(xf[e], mean), rstd) : __fmul_rn(xf[e], rstd);
+                    const float t = __fmul_rn(df[e], wreg[j][e]);
+                    if constexpr (LN) a1 = __fadd_rn(a1, t);
+                    a2 = __fmaf_rn(t, xh, a2);
+                    dw[j][e] = __fmaf_rn(df[e], xh, dw[j][e]);
+                    if constexpr (LN) db[j][e] = __fadd_rn(db[j][e], df[e]);
+                }
+            }
+        }
+        a2 = wave_sum_butterfly(a2);
+        if constexpr (LN) a1 = wave_sum_butterfly(a1);
+        if (lane == 0) { rsum[par][1][wv] = a2; if constexpr (LN) rsum[par][0][wv] = a1; }
+        __syncthreads();
+        const float c2 = __fdiv_rn(__fadd_rn(__fadd_rn(__fadd_rn(rsum[par][1][0], rsum[par][1][1]), rsum[par][1][2]), rsum[par][1][3]), (float)cols);
+        float c1 = 0.0f;
+        if constexpr (LN) c1 = __fdiv_rn(__fadd_rn(__fadd_rn(__fadd_rn(rsum[par][0][0], rsum[par][0][1]), rsum[par][0][2]), rsum[par][0][3]), (float)cols);
+#pragma unroll
+        for (int j = 0; j < CPLW; ++j) {
+            if (chunk[j] < nchunk) {
+                float xf[8], df[8], o[8];
+                unpack8<SRC>(xr[j], xf);
+                unpack8<ODL_BF16>(&dr[j], df);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float xh = LN ? __fmul_rn(__fsub_rn(xf[e], mean), rstd) : __fmul_rn(xf[e], rstd);
+                    const float t = __fmul_rn(df[e], wreg[j][e]);
+                    o[e] = __fmul_rn(rstd, __fmaf_rn(-xh, c2, LN ? __fsub_rn(t, c1) : t));
+                }
+                if constexpr (SRC == ODL_BF16) {
+                    reinterpret_cast<u32x4 *>(dx)[row * nchunk + chunk[j]] =
+                        u32x4{pack2(o[0], o[1]), pack2(o[2], o[3]), pack2(o[4], o[5]), pack2(o[6], o[7])};
+                } else {
+                    float4 *q = reinterpret_cast<float4 *>(dx) + (row * nchunk + chunk[j]) * 2;
+                    q[0] = float4{o[0], o[1], o[2], o[3]};
+                    q[1] = float4{o[4], o[5], o[6], o[7]};
+                }
+            }
+        }
+    }
+    // every lane owns its columns: the block's slab needs no reduction
+    float *slab = slabs + (int64_t)blockIdx.x * NS * cols;
+#pragma unroll
+    for (int j = 0; j < CPLW; ++j) {
+        if (chunk[j] < nchunk) {
+            float4 *q = reinterpret_cast<float4 *>(slab + chunk[j] * 8);
+            q[0] = float4{dw[j][0], dw[j][1], dw[j][2], dw[j][3]};
+            q[1] = float4{dw[j][4], dw[j][5], dw[j][6], dw[j][7]};
+            if constexpr (LN) {
+                float4 *qb = reinterpret_cast<float4 *>(slab + cols + chunk[j] * 8);
+                qb[0] = float4{db[j][0], db[j][1], db[j][2], db[j][3]};
+                qb[1] = float4{db[j][4], db[j][5], db[j][6], db[j][7]};
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------ LayerNorm
+// Same work split and summation order as the RMSNorm kernels.  Forward, per row:
+//   mean = sum(x) / cols;  d = x - mean;  rstd = 1 / sqrt(sum(d * d) / cols + eps)   (d * d by fma)
+//   y = bf16( ((d * rstd) * weight) + bias )          (bias may be absent)
+// The backward is norm_bwd_kernel<.., LN = true, ..> above (slabs hold d_weight in [0, cols) and d_bias in
+// [cols, 2 cols) of each block's row).
 template <int SRC, int CPL, int THREADS>
 __global__ __launch_bounds__(THREADS) void layernorm_fwd_kernel(const void *__restrict__ x, const float *__restrict__ weight,
                                                                  const float *__restrict__ bias, int64_t rows, int64_t cols, float eps,
@@ -412,102 +433,6 @@ __global__ __launch_bounds__(THREADS) void layernorm_fwd_kernel(const void *__re
     if (threadIdx.x == 0) parts[blockIdx.x] = bits_to_float(am);
     if (blockIdx.x == 0)
         for (int j = (int)gridDim.x + threadIdx.x; j < kParts; j += THREADS) parts[j] = 0.0f;
-}
-
-template <int SRC, int CPL>
-__global__ __launch_bounds__(kRmsBwdThreads) void layernorm_bwd_kernel(const u32x4 *__restrict__ dy, const void *__restrict__ x,
-                                                                        const float *__restrict__ weight, const float *__restrict__ mean_in,
-                                                                        const float *__restrict__ rstd_in, int64_t rows, int64_t cols,
-                                                                        void *__restrict__ dx, float *__restrict__ slabs) {
-    extern __shared__ float lds_dw[];                        // 2 * cols floats: d_weight, d_bias
-    constexpr int VPC = SRC == ODL_BF16 ? 1 : 2;
-    const int lane = threadIdx.x % kWave, wave_in_block = threadIdx.x / kWave;
-    const int64_t wave = (int64_t)blockIdx.x * (kRmsBwdThreads / kWave) + wave_in_block;
-    const int64_t nwave = (int64_t)gridDim.x * (kRmsBwdThreads / kWave);
-    const int64_t nchunk = cols / 8;
-    float dw[CPL][8], db[CPL][8];
-#pragma unroll
-    for (int j = 0; j < CPL; ++j)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) { dw[j][e] = 0.0f; db[j][e] = 0.0f; }
-    for (int64_t row = wave; row < rows; row += nwave) {
-        u32x4 xr[CPL][VPC], dr[CPL];
-#pragma unroll
-        for (int j = 0; j < CPL; ++j) {
-            const int64_t c = lane + (int64_t)kWave * j;
-            const bool ok = c < nchunk;
-            const u32x4 *p = reinterpret_cast<const u32x4 *>(x) + (row * nchunk + c) * VPC;
-#pragma unroll
-            for (int h = 0; h < VPC; ++h) xr[j][h] = ok ? __builtin_nontemporal_load(p + h) : u32x4{0, 0, 0, 0};
-            dr[j] = ok ? __builtin_nontemporal_load(dy + row * nchunk + c) : u32x4{0, 0, 0, 0};
-        }
-        const float mean = mean_in[row], rstd = rstd_in[row];
-        float a1 = 0.0f, a2 = 0.0f;
-#pragma unroll
-        for (int j = 0; j < CPL; ++j) {
-            const int64_t c = lane + (int64_t)kWave * j;
-            if (c < nchunk) {
-                float xf[8], df[8];
-                unpack8<SRC>(xr[j], xf);
-                unpack8<ODL_BF16>(&dr[j], df);
-                const float4 w0 = *reinterpret_cast<const float4 *>(weight + c * 8), w1 = *reinterpret_cast<const float4 *>(weight + c * 8 + 4);
-                const float w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const float xh = __fmul_rn(__fsub_rn(xf[e], mean), rstd);
-                    const float t = __fmul_rn(df[e], w[e]);
-                    a1 = __fadd_rn(a1, t);
-                    a2 = __fmaf_rn(t, xh, a2);
-                    dw[j][e] = __fmaf_rn(df[e], xh, dw[j][e]);
-                    db[j][e] = __fadd_rn(db[j][e], df[e]);
-                }
-            }
-        }
-        const float c1 = __fdiv_rn(wave_sum_butterfly(a1), (float)cols);
-        const float c2 = __fdiv_rn(wave_sum_butterfly(a2), (float)cols);
-#pragma unroll
-        for (int j = 0; j < CPL; ++j) {
-            const int64_t c = lane + (int64_t)kWave * j;
-            if (c < nchunk) {
-                float xf[8], df[8], o[8];
-                unpack8<SRC>(xr[j], xf);
-                unpack8<ODL_BF16>(&dr[j], df);
-                const float4 w0 = *reinterpret_cast<const float4 *>(weight + c * 8), w1 = *reinterpret_cast<const float4 *>(weight + c * 8 + 4);
-                const float w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const float xh = __fmul_rn(__fsub_rn(xf[e], mean), rstd);
-                    o[e] = __fmul_rn(rstd, __fmaf_rn(-xh, c2, __fsub_rn(__fmul_rn(df[e], w[e]), c1)));
-                }
-                if constexpr (SRC == ODL_BF16) {
-                    reinterpret_cast<u32x4 *>(dx)[row * nchunk + c] =
-                        u32x4{pack2(o[0], o[1]), pack2(o[2], o[3]), pack2(o[4], o[5]), pack2(o[6], o[7])};
-                } else {
-                    float4 *q = reinterpret_cast<float4 *>(dx) + (row * nchunk + c) * 2;
-                    q[0] = float4{o[0], o[1], o[2], o[3]};
-                    q[1] = float4{o[4], o[5], o[6], o[7]};
-                }
-            }
-        }
-    }
-    for (int wv = 0; wv < kRmsBwdThreads / kWave; ++wv) {
-        if (wave_in_block == wv) {
-#pragma unroll
-            for (int j = 0; j < CPL; ++j) {
-                const int64_t c = lane + (int64_t)kWave * j;
-                if (c < nchunk) {
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        float *sw = &lds_dw[c * 8 + e], *sb = &lds_dw[cols + c * 8 + e];
-                        *sw = wv == 0 ? dw[j][e] : __fadd_rn(*sw, dw[j][e]);
-                        *sb = wv == 0 ? db[j][e] : __fadd_rn(*sb, db[j][e]);
-                    }
-                }
-            }
-        }
-        __syncthreads();
-    }
-    for (int64_t c = threadIdx.x; c < 2 * cols; c += kRmsBwdThreads) slabs[(int64_t)blockIdx.x * 2 * cols + c] = lds_dw[c];
 }
 
 // slabs -> d_weight: a block owns 64 columns; 16 groups of lanes each add every 16th slab (8 loads in
@@ -758,17 +683,13 @@ extern "C" int odl_fp8_rmsnorm_bwd(const void *dy, const void *x, int src_dtype,
         return set_error(ODL_ERR_ARG, "odl_fp8_rmsnorm_bwd: null pointer");
     if (cols < 8 || cols % 8 != 0 || cols > 8192 || !aligned16(x) || !aligned16(dy) || !aligned16(dx) || !aligned16(weight))
         return set_error(ODL_ERR_SHAPE, "odl_fp8_rmsnorm_bwd: cols must be a multiple of 8 in [8, 8192] and the pointers 16-byte aligned");
-    const int rows_per_block = kRmsBwdThreads / kWave;
-    int64_t g = (rows + rows_per_block - 1) / rows_per_block;
-    g = g < 1 ? 1 : (g < ODL_FP8_RMSNORM_BWD_SLABS ? g : ODL_FP8_RMSNORM_BWD_SLABS);
-    const int64_t cpl = (cols / 8 + kWave - 1) / kWave;
-    const size_t lds = (size_t)cols * sizeof(float);
-#define ODL_RMSB(SRC, CPL) hipLaunchKernelGGL((rmsnorm_bwd_kernel<SRC, CPL>), dim3((unsigned)g), dim3(kRmsBwdThreads), lds, stream, reinterpret_cast<const u32x4 *>(dy), x, weight, rstd, rows, cols, dx, workspace)
-#define ODL_RMSB_SRC(CPL) do { if (src_dtype == ODL_BF16) ODL_RMSB(ODL_BF16, CPL); else ODL_RMSB(ODL_F32, CPL); } while (0)
-    if (cpl <= 2) ODL_RMSB_SRC(2);
-    else if (cpl <= 4) ODL_RMSB_SRC(4);
-    else if (cpl <= 8) ODL_RMSB_SRC(8);
-    else ODL_RMSB_SRC(16);
+    int64_t g = rows < 1 ? 1 : (rows < ODL_FP8_RMSNORM_BWD_SLABS ? rows : ODL_FP8_RMSNORM_BWD_SLABS);
+    const int64_t cplw = (cols / 8 + kRmsBwdThreads - 1) / kRmsBwdThreads;
+#define ODL_RMSB(SRC, CPLW) hipLaunchKernelGGL((norm_bwd_kernel<SRC, false, CPLW>), dim3((unsigned)g), dim3(kRmsBwdThreads), 0, stream, reinterpret_cast<const u32x4 *>(dy), x, weight, (const float *)nullptr, rstd, rows, cols, dx, workspace)
+#define ODL_RMSB_SRC(CPLW) do { if (src_dtype == ODL_BF16) ODL_RMSB(ODL_BF16, CPLW); else ODL_RMSB(ODL_F32, CPLW); } while (0)
+    if (cplw <= 1) ODL_RMSB_SRC(1);
+    else if (cplw <= 2) ODL_RMSB_SRC(2);
+    else ODL_RMSB_SRC(4);
 #undef ODL_RMSB_SRC
 #undef ODL_RMSB
     hipLaunchKernelGGL(rmsnorm_bwd_reduce_kernel, dim3((unsigned)((cols + 63) / 64)), dim3(1024), 0, stream, workspace, (int)g, cols, dweight);
@@ -831,16 +752,12 @@ extern "C" int odl_fp8_layernorm_bwd(const void *dy, const void *x, int src_dtyp
     if (dbias != dweight + cols) return set_error(ODL_ERR_ARG, "odl_fp8_layernorm_bwd: dbias must follow dweight (dweight + cols)");
     if (cols < 8 || cols % 8 != 0 || cols > 4096 || !aligned16(x) || !aligned16(dy) || !aligned16(dx) || !aligned16(weight))
         return set_error(ODL_ERR_SHAPE, "odl_fp8_layernorm_bwd: cols must be a multiple of 8 in [8, 4096] and the pointers 16-byte aligned");
-    const int rows_per_block = kRmsBwdThreads / kWave;
-    int64_t g = (rows + rows_per_block - 1) / rows_per_block;
-    g = g < 1 ? 1 : (g < ODL_FP8_RMSNORM_BWD_SLABS ? g : ODL_FP8_RMSNORM_BWD_SLABS);
-    const int64_t cpl = (cols / 8 + kWave - 1) / kWave;
-    const size_t lds = (size_t)cols * 2 * sizeof(float);
-#define ODL_LNB(SRC, CPL) hipLaunchKernelGGL((layernorm_bwd_kernel<SRC, CPL>), dim3((unsigned)g), dim3(kRmsBwdThreads), lds, stream, reinterpret_cast<const u32x4 *>(dy), x, weight, mean, rstd, rows, cols, dx, workspace)
-#define ODL_LNB_SRC(CPL) do { if (src_dtype == ODL_BF16) ODL_LNB(ODL_BF16, CPL); else ODL_LNB(ODL_F32, CPL); } while (0)
-    if (cpl <= 2) ODL_LNB_SRC(2);
-    else if (cpl <= 4) ODL_LNB_SRC(4);
-    else ODL_LNB_SRC(8);
+    int64_t g = rows < 1 ? 1 : (rows < ODL_FP8_RMSNORM_BWD_SLABS ? rows : ODL_FP8_RMSNORM_BWD_SLABS);
+    const int64_t cplw = (cols / 8 + kRmsBwdThreads - 1) / kRmsBwdThreads;
+#define ODL_LNB(SRC, CPLW) hipLaunchKernelGGL((norm_bwd_kernel<SRC, true, CPLW>), dim3((unsigned)g), dim3(kRmsBwdThreads), 0, stream, reinterpret_cast<const u32x4 *>(dy), x, weight, mean, rstd, rows, cols, dx, workspace)
+#define ODL_LNB_SRC(CPLW) do { if (src_dtype == ODL_BF16) ODL_LNB(ODL_BF16, CPLW); else ODL_LNB(ODL_F32, CPLW); } while (0)
+    if (cplw <= 1) ODL_LNB_SRC(1);
+    else ODL_LNB_SRC(2);
 #undef ODL_LNB_SRC
 #undef ODL_LNB
     // slabs are rows of 2 * cols sums (d_weight, d_bias); dweight and dbias are adjacent, so one reduction writes both

@@ -362,35 +362,66 @@ ORACLE_API void oracle_rmsnorm(const void *x, int src, const float *weight, int6
  * operations (bit-exact target); d_weight is accumulated in double here, because the library only
  * promises a fixed but device-dependent order of fp32 partial sums (tolerance target).  Pinned in
  * tests/test_oracle_fused.py against torch autograd of the reference module's expression. */
-ORACLE_API void oracle_rmsnorm_bwd(const uint16_t *dy, const void *x, int src, const float *weight, const float *rstd_in,
-                                   int64_t rows, int64_t cols, void *dx, float *dweight) {
+static float lane_butterfly(float *acc) {
+    for (int off = 32; off > 0; off >>= 1) {
+        float nxt[64];
+        for (int l = 0; l < 64; ++l) nxt[l] = acc[l] + acc[l ^ off];
+        memcpy(acc, nxt, 64 * sizeof(float));
+    }
+    return acc[0];
+}
+
+static inline float load_src(const void *x, int src, int64_t idx) {
+    return src == 0 ? bf16_to_f32(((const uint16_t *)x)[idx]) : ((const float *)x)[idx];
+}
+
+/* Row sums of the backward kernels: the 8-element chunk c of a row belongs to wave (c / 64) % 4, lane c % 64;
+ * a lane adds its chunks in ascending order (elements in order), the 64 lanes of a wave are combined by the
+ * xor butterfly, the four waves as ((s0 + s1) + s2) + s3.  term(idx, which) is the summand of element idx. */
+typedef float (*row_term_fn)(const void *ctx, int64_t idx, int which);
+static float row_sum_4waves(const void *ctx, row_term_fn term, int which, int64_t r, int64_t cols) {
     const int64_t nchunk = cols / 8;
-    double *dw = (double *)calloc((size_t)cols, sizeof(double));
-    for (int64_t r = 0; r < rows; ++r) {
-        const float rstd = rstd_in[r];
+    float wave_sum[4];
+    for (int w = 0; w < 4; ++w) {
         float acc[64];
         for (int l = 0; l < 64; ++l) {
             float a = 0.0f;
-            for (int64_t c = l; c < nchunk; c += 64)
+            for (int64_t c = (int64_t)w * 64 + l; c < nchunk; c += 256)
                 for (int e = 0; e < 8; ++e) {
                     int64_t idx = r * cols + c * 8 + e;
-                    float xv = src == 0 ? bf16_to_f32(((const uint16_t *)x)[idx]) : ((const float *)x)[idx];
-                    float xh = xv * rstd;
-                    float t = bf16_to_f32(dy[idx]) * weight[c * 8 + e];
-                    a = fmaf(t, xh, a);
+                    float t = term(ctx, idx, 0);
+                    if (which == 0) a = a + t;                       /* plain sum of t */
+                    else a = fmaf(t, term(ctx, idx, 1), a);          /* sum of t * xh by fma */
                 }
             acc[l] = a;
         }
-        for (int off = 32; off > 0; off >>= 1) {
-            float nxt[64];
-            for (int l = 0; l < 64; ++l) nxt[l] = acc[l] + acc[l ^ off];
-            memcpy(acc, nxt, sizeof(acc));
-        }
-        const float cmean = acc[0] / (float)cols;
+        wave_sum[w] = lane_butterfly(acc);
+    }
+    return ((wave_sum[0] + wave_sum[1]) + wave_sum[2]) + wave_sum[3];
+}
+
+struct norm_ctx { const uint16_t *dy; const void *x; int src; const float *weight; float mean, rstd; int64_t cols; };
+static float norm_term(const void *vctx, int64_t idx, int which) {
+    const struct norm_ctx *c = (const struct norm_ctx *)vctx;
+    if (which == 0) return bf16_to_f32(c->dy[idx]) * c->weight[idx % c->cols];
+    return (load_src(c->x, c->src, idx) - c->mean) * c->rstd;
+}
+static float rms_term(const void *vctx, int64_t idx, int which) {
+    const struct norm_ctx *c = (const struct norm_ctx *)vctx;
+    if (which == 0) return bf16_to_f32(c->dy[idx]) * c->weight[idx % c->cols];
+    return load_src(c->x, c->src, idx) * c->rstd;
+}
+
+ORACLE_API void oracle_rmsnorm_bwd(const uint16_t *dy, const void *x, int src, const float *weight, const float *rstd_in,
+                                   int64_t rows, int64_t cols, void *dx, float *dweight) {
+    double *dw = (double *)calloc((size_t)cols, sizeof(double));
+    for (int64_t r = 0; r < rows; ++r) {
+        const float rstd = rstd_in[r];
+        struct norm_ctx ctx = {dy, x, src, weight, 0.0f, rstd, cols};
+        const float cmean = row_sum_4waves(&ctx, rms_term, 1, r, cols) / (float)cols;
         for (int64_t c = 0; c < cols; ++c) {
             int64_t idx = r * cols + c;
-            float xv = src == 0 ? bf16_to_f32(((const uint16_t *)x)[idx]) : ((const float *)x)[idx];
-            float xh = xv * rstd;
+            float xh = load_src(x, src, idx) * rstd;
             float d = bf16_to_f32(dy[idx]);
             float o = rstd * fmaf(-xh, cmean, d * weight[c]);
             if (src == 0) ((uint16_t *)dx)[idx] = f32_to_bf16(o); else ((float *)dx)[idx] = o;
@@ -405,19 +436,6 @@ ORACLE_API void oracle_rmsnorm_bwd(const uint16_t *dy, const void *x, int src, c
  * stated order of IEEE operations, and its backward (dx bit-exact target; d_weight / d_bias summed
  * in double: tolerance targets).  Pinned in tests/test_oracle_fused.py against float64 closed
  * forms, torch's F.layer_norm and autograd, and exact special cases. */
-static float lane_butterfly(float *acc) {
-    for (int off = 32; off > 0; off >>= 1) {
-        float nxt[64];
-        for (int l = 0; l < 64; ++l) nxt[l] = acc[l] + acc[l ^ off];
-        memcpy(acc, nxt, 64 * sizeof(float));
-    }
-    return acc[0];
-}
-
-static inline float load_src(const void *x, int src, int64_t idx) {
-    return src == 0 ? bf16_to_f32(((const uint16_t *)x)[idx]) : ((const float *)x)[idx];
-}
-
 ORACLE_API void oracle_layernorm(const void *x, int src, const float *weight, const float *bias, int64_t rows, int64_t cols,
                                  float eps, uint16_t *y, float *mean_out, float *rstd_out) {
     const int64_t nchunk = cols / 8;
@@ -453,26 +471,12 @@ ORACLE_API void oracle_layernorm(const void *x, int src, const float *weight, co
 
 ORACLE_API void oracle_layernorm_bwd(const uint16_t *dy, const void *x, int src, const float *weight, const float *mean_in,
                                      const float *rstd_in, int64_t rows, int64_t cols, void *dx, float *dweight, float *dbias) {
-    const int64_t nchunk = cols / 8;
     double *dw = (double *)calloc((size_t)cols * 2, sizeof(double));
     for (int64_t r = 0; r < rows; ++r) {
         const float mean = mean_in[r], rstd = rstd_in[r];
-        float a1[64], a2[64];
-        for (int l = 0; l < 64; ++l) {
-            float s1 = 0.0f, s2 = 0.0f;
-            for (int64_t c = l; c < nchunk; c += 64)
-                for (int e = 0; e < 8; ++e) {
-                    int64_t idx = r * cols + c * 8 + e;
-                    float xh = (load_src(x, src, idx) - mean) * rstd;
-                    float t = bf16_to_f32(dy[idx]) * weight[c * 8 + e];
-                    s1 = s1 + t;
-                    s2 = fmaf(t, xh, s2);
-                }
-            a1[l] = s1;
-            a2[l] = s2;
-        }
-        const float c1 = lane_butterfly(a1) / (float)cols;
-        const float c2 = lane_butterfly(a2) / (float)cols;
+        struct norm_ctx ctx = {dy, x, src, weight, mean, rstd, cols};
+        const float c1 = row_sum_4waves(&ctx, norm_term, 0, r, cols) / (float)cols;
+        const float c2 = row_sum_4waves(&ctx, norm_term, 1, r, cols) / (float)cols;
         for (int64_t c = 0; c < cols; ++c) {
             int64_t idx = r * cols + c;
             float xh = (load_src(x, src, idx) - mean) * rstd;
