@@ -59,8 +59,9 @@ constexpr int SLAB = 32 * PITCH;           // one wave's epilogue slab
 // row-major) instead of the fast one.  A stage then holds 128 K-rows of 256 bytes; the 1 KB loads
 // bring 4 such rows each, and fragments are read with ds_read_b64_tr_b8, which hands every lane
 // of a 16-lane group one byte column of an 8 x 16 byte block (8 consecutive K for its own row).
-// The 16-byte chunks of a K-row are placed at chunk ^ (k & 7): the 8 rows a group reads in one
-// instruction then sit in 8 different bank quads.  Same K order, same accumulation, same bits
+// The 16-byte chunks of a K-row are placed at chunk ^ 2 (k & 7): the 8 rows x 32 bytes that the two
+// 16-lane groups of a half-wave read together then cover all 16 chunk positions = all 64 banks once
+// (with chunk ^ (k & 7) the two groups met in the same 8 positions: 2 extra cycles per read, measured).  Same K order, same accumulation, same bits
 // as the other layout: wgrad and dgrad no longer need transposed copies of their operands.
 template <int FA, int FB, bool TA, bool TB>
 __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
@@ -110,7 +111,7 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
         const int row = (wave + j * NW) * 8 + lane / 8;                   // K fast: 8 rows of 128 bytes per load
         const int nt = row * (int)g.K + (((lane % 8) ^ swz(row)) << 4);
         const int kb = (wave + j * NW) * 4 + lane / 16;                   // K slow: 4 K-rows of 256 bytes per load
-        const int chunk = ((lane % 16) ^ (kb & 7)) << 4;
+        const int chunk = ((lane % 16) ^ ((kb & 7) << 1)) << 4;
         voff_a[j] = TA ? kb * (int)g.M + chunk : nt;
         voff_b[j] = TB ? kb * (int)g.N + chunk : nt;
     }
@@ -145,11 +146,11 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
     }
     // K-slow layout: fragment t covers tile rows row0 + 32 t .. + 31 = the 16-byte chunks c0 + 2t, c0 + 2t + 1
     // of a K-row; a lane of a 16-lane group addresses K-row 32 lg + (lane % 16) / 2 (+ 8p, + 64h) and the
-    // 8-byte half lane % 2 of chunk (c0 + 2t) ^ (k & 7).  c0 has bits 0 and 3 only, so the t-dependence
+    // 8-byte half lane % 2 of chunk (c0 + 2t) ^ 2 (k & 7).  c0 has bits 0 and 3 only, so the t-dependence
     // is an XOR on the address.
     const int tj = (lane % 16) / 2;
-    const int tra = (lg * 32 + tj) * 256 + ((((wm0 / 16) + (lr / 16)) ^ tj) << 4) + (lane % 2) * 8;
-    const int trb = (lg * 32 + tj) * 256 + ((((wn0 / 16) + (lr / 16)) ^ tj) << 4) + (lane % 2) * 8;
+    const int tra = (lg * 32 + tj) * 256 + ((((wm0 / 16) + (lr / 16)) ^ (tj << 1)) << 4) + (lane % 2) * 8;
+    const int trb = (lg * 32 + tj) * 256 + ((((wn0 / 16) + (lr / 16)) ^ (tj << 1)) << 4) + (lane % 2) * 8;
     auto read_tr = [&](const uint8_t *sx, int lane_off, int t, int h) -> v8i {
         typedef int v2i_t __attribute__((ext_vector_type(2)));
         const uint32_t base = lds_addr_of(sx) + (uint32_t)(lane_off ^ (t << 5)) + h * 64 * 256;
