@@ -140,7 +140,9 @@ __device__ __forceinline__ void epilogue_staged(const GemmArgs &g, v16f (&acc)[T
                 const int r = i * RPI + lane / LPR, chunk = lane % LPR;
                 const u32x4 val = *reinterpret_cast<const u32x4 *>(wave_lds + r * PITCH + chunk * 16);
                 uint8_t *dst = out + ((m_wave + 32 * t + r) * g.N + n_wave + 32 * us) * ESZ + chunk * 16;
-                *reinterpret_cast<u32x4 *>(dst) = val;
+                // non-temporal: the output is not read by the next kernel, and written through the memory-side
+                // cache it would still be draining to HBM while the next (memory-bound) kernel runs
+                __builtin_nontemporal_store(val, reinterpret_cast<u32x4 *>(dst));
             }
         }
     }

@@ -191,8 +191,10 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
             const int so = so_base + (32 * t + 8 * j) * row_bytes + 64 * us;
             // s_nop 4: a scalar register written by a vector instruction (the compiler restores
             // spilled scalars that way) must not be read by a vector-memory instruction for 5
-            // cycles, and the compiler does not look inside asm statements for that hazard
-            asm volatile("s_nop 4\n\tbuffer_store_dwordx4 %0, %1, %2, %3 offen" ::"v"(data[j]), "v"(vo), "s"(rsrc), "s"(so));
+            // cycles, and the compiler does not look inside asm statements for that hazard.
+            // nt: the output is not an operand of the next kernel; stored normally it sits dirty in the
+            // memory-side cache and its write-back competes with the amax / cast pass that follows
+            asm volatile("s_nop 4\n\tbuffer_store_dwordx4 %0, %1, %2, %3 offen nt" ::"v"(data[j]), "v"(vo), "s"(rsrc), "s"(so));
         }
     };
     auto lds_w = [](uint32_t addr) { return (__attribute__((address_space(3))) u32x2 *)addr; };
