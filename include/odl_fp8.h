@@ -274,13 +274,14 @@ int odl_fp8_gemm_nt(const uint8_t *a, const uint8_t *b, int64_t M, int64_t N, in
  *   dgrad dX = dY . W       a = dY (K_FAST), b = W  (K_SLOW: contraction over N, W is [N, K])
  *   wgrad dW = dY^T . X     a = dY (K_SLOW), b = X  (K_SLOW: contraction over M)
  * Results equal those of odl_fp8_gemm_nt on the transposed copies bit for bit (same order of
- * accumulation).  One scale per operand, bf16 output, no bias; M, N, K multiples of 256, K >= 512:
- * anything else is refused with ODL_ERR_SHAPE (make the transposed copy and use odl_fp8_gemm_nt).
+ * accumulation).  One scale per operand, no bias, out_dtype ODL_BF16 or ODL_F32 (weight gradients
+ * of fp32 master weights); M, N, K multiples of 256, K >= 512: anything else is refused with
+ * ODL_ERR_SHAPE (make the transposed copy and use odl_fp8_gemm_nt).
  */
 enum odl_operand_layout { ODL_K_FAST = 0, ODL_K_SLOW = 1 };
 int odl_fp8_gemm_layouts(const uint8_t *a, const uint8_t *b, int64_t M, int64_t N, int64_t K,
                          int fmt_a, int fmt_b, int layout_a, int layout_b, const float *sa_inv,
-                         const float *sb_inv, void *c, odl_stream_t stream);
+                         const float *sb_inv, void *c, int out_dtype, odl_stream_t stream);
 
 /*
  * Delayed-scaling bookkeeping for R tensor roles with H history slots each

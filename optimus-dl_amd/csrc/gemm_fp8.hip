@@ -53,7 +53,7 @@ static const Variant kVariants[] = {
     {"128x128x128 4 waves (64x64 per wave)", 128, 128, 256, 0.70f},
     {"256x256x128 4 waves, software-pipelined, persistent (K % 256 == 0)", 256, 256, 256, 1.10f},
     {"256x256x128 4 waves, software-pipelined, one tile per block", 256, 256, 256, 0.50f},
-    {"256x256x128 4 waves, streaming across tiles, folded epilogue (whole tiles, per-tensor scales, bf16)", 256, 256, 256, 1.25f},
+    {"256x256x128 4 waves, streaming across tiles, folded epilogue (whole tiles, per-tensor scales)", 256, 256, 256, 1.25f},
 };
 constexpr int kPipeVariant = 5, kPipeOneTileVariant = 6, kStreamVariant = 7;
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
@@ -138,7 +138,7 @@ extern "C" int odl_fp8_gemm_nt(const uint8_t *a, const uint8_t *b, int64_t M, in
     if (M == 0 || N == 0) return ODL_OK;
 
     const bool tiled_ok = K >= 128 && K % 128 == 0 && (double)M * (double)K < 4294967296.0 && (double)N * (double)K < 4294967296.0;
-    const bool stream_ok = tiled_ok && out_dtype == ODL_BF16 && sa_n == 1 && sb_n == 1 && !bias && M % 256 == 0 && N % 256 == 0 &&
+    const bool stream_ok = tiled_ok && sa_n == 1 && sb_n == 1 && !bias && M % 256 == 0 && N % 256 == 0 &&
                            K % 256 == 0 && K >= 512;
     int variant = g_forced_variant >= 0 ? g_forced_variant : (tiled_ok ? choose_variant(M, N, stream_ok) : 0);
     if (variant != 0 && !tiled_ok) variant = 0;
@@ -172,20 +172,21 @@ extern "C" int odl_fp8_gemm_nt(const uint8_t *a, const uint8_t *b, int64_t M, in
 
 extern "C" int odl_fp8_gemm_layouts(const uint8_t *a, const uint8_t *b, int64_t M, int64_t N, int64_t K, int fmt_a, int fmt_b,
                                     int layout_a, int layout_b, const float *sa_inv, const float *sb_inv, void *c,
-                                    odl_stream_t stream_) {
+                                    int out_dtype, odl_stream_t stream_) {
     hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
     if (!a || !b || !c || !sa_inv || !sb_inv) return set_error(ODL_ERR_ARG, "odl_fp8_gemm_layouts: null pointer");
     if ((fmt_a != ODL_FP8_E4M3 && fmt_a != ODL_FP8_E5M2) || (fmt_b != ODL_FP8_E4M3 && fmt_b != ODL_FP8_E5M2))
         return set_error(ODL_ERR_ARG, "odl_fp8_gemm_layouts: formats %d, %d", fmt_a, fmt_b);
     if ((layout_a != ODL_K_FAST && layout_a != ODL_K_SLOW) || (layout_b != ODL_K_FAST && layout_b != ODL_K_SLOW))
         return set_error(ODL_ERR_ARG, "odl_fp8_gemm_layouts: layouts %d, %d", layout_a, layout_b);
+    if (out_dtype != ODL_BF16 && out_dtype != ODL_F32) return set_error(ODL_ERR_ARG, "odl_fp8_gemm_layouts: out_dtype %d", out_dtype);
     if ((reinterpret_cast<uintptr_t>(a) & 15) || (reinterpret_cast<uintptr_t>(b) & 15) || (reinterpret_cast<uintptr_t>(c) & 15))
         return set_error(ODL_ERR_SHAPE, "odl_fp8_gemm_layouts: operands and output must be 16-byte aligned");
     GemmArgs g;
     g.a = a; g.b = b; g.c = c; g.sa = sa_inv; g.sb = sb_inv; g.bias = nullptr;
     g.M = M; g.N = N; g.K = K;
     g.sa_vec = 0; g.sb_vec = 0;
-    g.out_dtype = ODL_BF16;
+    g.out_dtype = out_dtype;
     g.ta = layout_a == ODL_K_SLOW;
     g.tb = layout_b == ODL_K_SLOW;
     const bool sizes_ok = M > 0 && N > 0 && K >= 512 && M % 256 == 0 && N % 256 == 0 && K % 256 == 0 &&

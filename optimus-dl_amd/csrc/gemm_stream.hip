@@ -1,6 +1,6 @@
 // FP8 GEMM, 256x256 block tile, 4 waves (one per SIMD, 128x128 each), persistent,
 // with the epilogue of every tile folded under the first MFMAs of the next one.
-// C = (A[M,K] . B[N,K]^T) * (sa_inv * sb_inv) in bf16, for the shapes training uses:
+// C = (A[M,K] . B[N,K]^T) * (sa_inv * sb_inv) in bf16 or fp32, for the shapes training uses:
 // M % 256 == 0, N % 256 == 0, K % 256 == 0, K >= 512, per-tensor scales, no bias.
 // Everything else goes to gemm_pipe.hip, whose K step this kernel shares:
 //
@@ -39,6 +39,8 @@
 // "everything but the youngest n operations has completed":
 //   step 0 : younger than the loads of step 1 are the 32 output stores of the folded
 //            epilogue                                 -> vmcnt(32)
+//            (fp32 output: 64 stores, and the counter field ends at 63 -> vmcnt(63), which also
+//            waits for the first of those stores, issued a thousand cycles earlier)
 //   others : nothing is younger than the loads of step kt+1            -> vmcnt(0)
 // (An L2 prefetch, one lane per 128-byte line a few steps ahead, was tried and removed: the
 // scattered loads occupy the texture path that the direct-to-LDS loads need, 14 % of the K loop.)
@@ -63,8 +65,11 @@ constexpr int SLAB = 32 * PITCH;           // one wave's epilogue slab
 // 16-lane groups of a half-wave read together then cover all 16 chunk positions = all 64 banks once
 // (with chunk ^ (k & 7) the two groups met in the same 8 positions: 2 extra cycles per read, measured).  Same K order, same accumulation, same bits
 // as the other layout: wgrad and dgrad no longer need transposed copies of their operands.
-template <int FA, int FB, bool TA, bool TB>
+// F32: fp32 output (weight gradients of fp32 master weights).  A 32 x 32 sub-tile is then a whole slab
+// (32 rows of 128 bytes) and leaves right after its own MFMA: 64 stores per wave and tile instead of 32.
+template <int FA, int FB, bool TA, bool TB, bool F32>
 __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
+    constexpr int ESZ = F32 ? 4 : 2;
     __shared__ __attribute__((aligned(1024))) uint8_t sA0[REGION];
     __shared__ __attribute__((aligned(1024))) uint8_t sB0[REGION];
     __shared__ __attribute__((aligned(1024))) uint8_t sA1[REGION];
@@ -178,17 +183,18 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
     const v16f zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 
     // ---- output side of the folded epilogue
-    const int n2 = (int)g.N * 2;                  // bytes per output row
-    const int c_soff0 = (wm0 * (int)g.N + wn0) * 2;
+    const int n2 = (int)g.N * ESZ;                // bytes per output row
+    const int c_soff0 = (wm0 * (int)g.N + wn0) * ESZ;
     const float s_tensor = bits_to_float((uint32_t)__builtin_amdgcn_readfirstlane((int)float_to_bits(g.sa[0] * g.sb[0])));
     auto rsrc_out = [&](int tm0, int tn0) -> v4i {
-        const uint64_t addr = reinterpret_cast<uint64_t>(reinterpret_cast<uint8_t *>(g.c) + ((int64_t)tm0 * g.N + tn0) * 2);
+        const uint64_t addr = reinterpret_cast<uint64_t>(reinterpret_cast<uint8_t *>(g.c) + ((int64_t)tm0 * g.N + tn0) * ESZ);
         return v4i{(int)(uint32_t)addr, (int)(uint32_t)(addr >> 32), (int)0x80000000u, 0x00020000};
     };
+    // `us`: the slab's position in the wave tile's row, in slabs of 128 bytes
     auto store_slab = [](const u32x4 (&data)[4], int vo, const v4i &rsrc, int so_base, int row_bytes, int t, int us) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const int so = so_base + (32 * t + 8 * j) * row_bytes + 64 * us;
+            const int so = so_base + (32 * t + 8 * j) * row_bytes + 128 * us;
             // s_nop 4: a scalar register written by a vector instruction (the compiler restores
             // spilled scalars that way) must not be read by a vector-memory instruction for 5
             // cycles, and the compiler does not look inside asm statements for that hazard.
@@ -258,17 +264,52 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) back[j] = lds_r(epi_r + j * 8 * PITCH);
             } else if (i > 0) {
-                store_slab(back, c_voff, rsrc_c, c_soff0, n2, (i - 2) / 4, (i - 2) % 4);   // completed one MFMA ago
+                store_slab(back, c_voff, rsrc_c, c_soff0, n2, (i - 2) / 4, ((i - 2) % 4) / 2);   // completed one MFMA ago
             }
             if (i < 4) a1[i] = read_a(sa_cur, i, 1);
             else if (i < 8) b1[i - 4] = read_b(sb_cur, i - 4, 1);
             __builtin_amdgcn_sched_barrier(0);
         }
-        store_slab(back, c_voff, rsrc_c, c_soff0, n2, 3, 2);
+        store_slab(back, c_voff, rsrc_c, c_soff0, n2, 3, 1);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    // the same for fp32 output: sub-tile i is scaled, written to the slab as 32 rows x 32 floats, read
+    // back along the rows and stored while MFMA i + 1 runs
+    auto phase_a_fold_f32 = [&](const uint8_t *sa_cur, const uint8_t *sb_cur, const v4i &rsrc_c) {
+        int lane_e = lane, wave_e = wave;
+        asm volatile("" : "+v"(lane_e));
+        asm volatile("" : "+s"(wave_e));
+        const uint32_t slab = lds_addr_of(sEpi) + wave_e * SLAB;
+        const uint32_t epi_w = slab + (lane_e % 32) * PITCH + (lane_e / 32) * 16;
+        const uint32_t epi_r = slab + (lane_e / 8) * PITCH + (lane_e % 8) * 16;
+        const int c_voff = (lane_e / 8) * n2 + (lane_e % 8) * 16;
+        u32x4 back[4];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int t = i / 4, u = i % 4;
+            float v[16];
+#pragma unroll
+            for (int e = 0; e < 16; ++e) v[e] = acc[t][u][e] * s_tensor;
+            acc[t][u] = mfma_32x32x64<FB, FA>(b0[u], a0[t], zero16);
+            if (i > 0) store_slab(back, c_voff, rsrc_c, c_soff0, n2, (i - 1) / 4, (i - 1) % 4);
+            // lane (lr, lg) holds columns 8q + 4lg + {0..3} of row lr: 16 bytes at 32q + 16lg, as two 8-byte
+            // writes (the row pitch of 34 dwords spreads the 32 rows of a half-wave over all 64 banks)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                *lds_w(epi_w + q * 32) = u32x2{float_to_bits(v[4 * q]), float_to_bits(v[4 * q + 1])};
+                *lds_w(epi_w + q * 32 + 8) = u32x2{float_to_bits(v[4 * q + 2]), float_to_bits(v[4 * q + 3])};
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) back[j] = lds_r(epi_r + j * 8 * PITCH);
+            if (i < 4) a1[i] = read_a(sa_cur, i, 1);
+            else if (i < 8) b1[i - 4] = read_b(sb_cur, i - 4, 1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        store_slab(back, c_voff, rsrc_c, c_soff0, n2, 3, 3);
         __builtin_amdgcn_sched_barrier(0);
     };
     auto sync = [&](bool after_fold) {
-        if (after_fold) __builtin_amdgcn_s_waitcnt(0x8070);          // vmcnt(32) lgkmcnt(0)
+        if (after_fold) __builtin_amdgcn_s_waitcnt(F32 ? 0xC07F : 0x8070);   // vmcnt(63 | 32) lgkmcnt(0)
         else __builtin_amdgcn_s_waitcnt(0x0070);                     // vmcnt(0)  lgkmcnt(0)
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
@@ -348,26 +389,34 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
         n0 = next_n0;
         rsrc_a = next_a;
         rsrc_b = next_b;
-        phase_a_fold(sA0, sB0, rsrc_c);
+        if constexpr (F32) phase_a_fold_f32(sA0, sB0, rsrc_c);
+        else phase_a_fold(sA0, sB0, rsrc_c);
         if (!has_next) break;
     }
 }
 
+template <int FA, int FB, bool F32>
+void launch_out(const GemmArgs &g, int blocks_per_xcd, hipStream_t stream) {
+    const dim3 grid((unsigned)(8 * blocks_per_xcd)), block(256);
+    if (g.ta && g.tb) hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB, true, true, F32>), grid, block, 0, stream, g);
+    else if (g.tb) hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB, false, true, F32>), grid, block, 0, stream, g);
+    else if (g.ta) hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB, true, false, F32>), grid, block, 0, stream, g);
+    else hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB, false, false, F32>), grid, block, 0, stream, g);
+}
+
 template <int FA, int FB>
 void launch_fmt(const GemmArgs &g, int blocks_per_xcd, hipStream_t stream) {
-    const dim3 grid((unsigned)(8 * blocks_per_xcd)), block(256);
-    if (g.ta && g.tb) hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB, true, true>), grid, block, 0, stream, g);
-    else if (g.tb) hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB, false, true>), grid, block, 0, stream, g);
-    else if (g.ta) hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB, true, false>), grid, block, 0, stream, g);
-    else hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB, false, false>), grid, block, 0, stream, g);
+    if (g.out_dtype == ODL_F32) launch_out<FA, FB, true>(g, blocks_per_xcd, stream);
+    else launch_out<FA, FB, false>(g, blocks_per_xcd, stream);
 }
 
 }  // namespace
 
 // Shapes this kernel takes (the caller checks the 32-bit offset limits shared with gemm_pipe.hip).
 bool gemm_stream_accepts(const GemmArgs &g) {
-    return g.out_dtype == ODL_BF16 && !g.sa_vec && !g.sb_vec && g.bias == nullptr && g.M % BM == 0 && g.N % BN == 0 &&
-           g.K % 256 == 0 && g.K >= 512 && (double)g.N * 2.0 * (BM + 8) < 2147483648.0;
+    const double esz = g.out_dtype == ODL_F32 ? 4.0 : 2.0;
+    return (g.out_dtype == ODL_BF16 || g.out_dtype == ODL_F32) && !g.sa_vec && !g.sb_vec && g.bias == nullptr &&
+           g.M % BM == 0 && g.N % BN == 0 && g.K % 256 == 0 && g.K >= 512 && (double)g.N * esz * (BM + 8) < 2147483648.0;
 }
 
 // One block per CU at most (the kernel needs ~150 KB of LDS), 8 | grid so that the

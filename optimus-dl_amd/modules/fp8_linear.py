@@ -167,8 +167,8 @@ class _Fp8LinearFn(torch.autograd.Function):
             # K-slow costs the GEMM more than the copy (measured), while dy has just been written.
             tokens, n_in, n_out = x2d.shape[0], x2d.shape[1], weight.shape[0]
             fp8_wgrad = need_wgrad and recipe.wgrad
-            ctx.wgrad_direct = (fp8_wgrad and recipe.direct_layouts and weight.dtype == torch.bfloat16
-                                and native.gemm_layouts_supported(n_out, n_in, tokens))
+            ctx.wgrad_direct = (fp8_wgrad and recipe.direct_layouts
+                                and native.gemm_layouts_supported(n_out, n_in, tokens, weight.dtype))
             if pol.kind == "delayed":
                 meta = module._meta(recipe, x2d.device, "fwd")
                 xq, xq_t, sx_inv = _quantise_delayed(x2d, pol.fmt_fwd, meta, ROLE_X, fp8_wgrad)
@@ -234,7 +234,7 @@ class _Fp8LinearFn(torch.autograd.Function):
             if fp8_wgrad:
                 if ctx.wgrad_direct:        # dW = dY^T . X with dY [tokens, N] as stored, X^T from the forward
                     dw = native.gemm_layouts(gq, saved["xq_t"], pol.fmt_bwd, pol.fmt_fwd, native.K_SLOW, native.K_FAST,
-                                             sg_inv, saved["sx_inv_t"])
+                                             sg_inv, saved["sx_inv_t"], out_dtype=ctx.w_dtype)
                 else:
                     dw = native.gemm_nt(gq_t, saved["xq_t"], pol.fmt_bwd, pol.fmt_fwd, sg_inv, saved["sx_inv_t"],
                                         out_dtype=ctx.w_dtype)

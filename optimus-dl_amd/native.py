@@ -23,7 +23,7 @@ DT_BF16, DT_F32 = 0, 1
 AMAX_MAX, AMAX_MOST_RECENT = 0, 1
 FP8_MAX = {E4M3: 448.0, E5M2: 57344.0}
 TORCH_FP8 = {E4M3: torch.float8_e4m3fn, E5M2: torch.float8_e5m2}
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # ODL_FP8_LIB names another build of the same library (e.g. one made for an experiment)
@@ -109,7 +109,7 @@ def load() -> ctypes.CDLL:
         L.odl_fp8_cast.argtypes = [vp, i32, i64, i64, vp, i32, i32, vp, vp, vp]
         L.odl_fp8_cast_transpose.argtypes = [vp, i32, i64, i64, vp, i32, i32, vp, vp, vp, vp]
         L.odl_fp8_gemm_nt.argtypes = [vp, vp, i64, i64, i64, i32, i32, vp, i64, vp, i64, vp, i32, vp, i32, vp]
-        L.odl_fp8_gemm_layouts.argtypes = [vp, vp, i64, i64, i64, i32, i32, i32, i32, vp, vp, vp, vp]
+        L.odl_fp8_gemm_layouts.argtypes = [vp, vp, i64, i64, i64, i32, i32, i32, i32, vp, vp, vp, i32, vp]
         L.odl_fp8_delayed_update.argtypes = [vp, i64, i64, i64, vp, vp, vp, i32, i32, vp]
         L.odl_fp8_gemm_num_variants.restype = i32
         L.odl_fp8_gemm_variant_name.argtypes = [i32]
@@ -562,16 +562,20 @@ def gemm_nt(a: torch.Tensor, b: torch.Tensor, fmt_a: int, fmt_b: int, sa_inv: to
 K_FAST, K_SLOW = 0, 1
 
 
-def gemm_layouts_supported(M: int, N: int, K: int) -> bool:
+def gemm_layouts_supported(M: int, N: int, K: int, out_dtype: torch.dtype = torch.bfloat16) -> bool:
     """Shapes :func:`gemm_layouts` takes (whole 256 x 256 tiles, operands under 2 GiB)."""
+    if out_dtype not in (torch.bfloat16, torch.float32):
+        return False
     return (M > 0 and N > 0 and K >= 512 and M % 256 == 0 and N % 256 == 0 and K % 256 == 0
-            and (M + 256) * K < 2**31 and (N + 256) * K < 2**31 and N * 2 * 264 < 2**31)
+            and (M + 256) * K < 2**31 and (N + 256) * K < 2**31 and N * out_dtype.itemsize * 264 < 2**31)
 
 
 def gemm_layouts(a: torch.Tensor, b: torch.Tensor, fmt_a: int, fmt_b: int, layout_a: int, layout_b: int,
-                 sa_inv: torch.Tensor, sb_inv: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
-    """out[M,N] (bf16) = (A . B^T) * sa_inv * sb_inv where an operand is given either as [rows, K]
-    (K_FAST) or as [K, rows] (K_SLOW): no transposed copies for dgrad / wgrad."""
+                 sa_inv: torch.Tensor, sb_inv: torch.Tensor, out: torch.Tensor | None = None,
+                 out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """out[M,N] (bf16 or fp32) = (A . B^T) * sa_inv * sb_inv where an operand is given either as
+    [rows, K] (K_FAST) or as [K, rows] (K_SLOW): no transposed copies for dgrad / wgrad.  A given
+    ``out`` decides the output type, else ``out_dtype`` does."""
     if a.dtype != torch.uint8 or b.dtype != torch.uint8:
         raise NativeError("gemm_layouts operands must be uint8 FP8 codes")
     a, b = _as_2d(a), _as_2d(b)
@@ -582,11 +586,12 @@ def gemm_layouts(a: torch.Tensor, b: torch.Tensor, fmt_a: int, fmt_b: int, layou
     _f32_dev(sa_inv, 1, "gemm_layouts sa_inv")
     _f32_dev(sb_inv, 1, "gemm_layouts sb_inv")
     if out is None:
-        out = torch.empty((M, N), dtype=torch.bfloat16, device=a.device)
-    elif out.shape != (M, N) or out.dtype != torch.bfloat16 or not out.is_contiguous():
+        out = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    elif out.shape != (M, N) or out.dtype not in (torch.bfloat16, torch.float32) or not out.is_contiguous():
         raise NativeError("gemm_layouts: `out` has the wrong shape / dtype / layout")
     _check(load().odl_fp8_gemm_layouts(a.data_ptr(), b.data_ptr(), M, N, K, fmt_a, fmt_b, layout_a, layout_b, sa_inv.data_ptr(),
-                                       sb_inv.data_ptr(), out.data_ptr(), _stream()), "odl_fp8_gemm_layouts")
+                                       sb_inv.data_ptr(), out.data_ptr(), _src_dtype(out), _stream()),
+           "odl_fp8_gemm_layouts")
     return out
 
 

@@ -346,3 +346,15 @@ def test_k_slow_layouts_at_baseline_shapes(N, M, Nn, K, la, lb):
     out = N.gemm_layouts(aq_t if la else aq, bq_t if lb else bq, O.E5M2, O.E4M3, la, lb, sa_inv, sb_inv)
     assert torch.equal(out, ref)
     sample_check(out, aq, bq, O.E5M2, O.E4M3, sa_inv, sb_inv, seed=M + K, what=f"k-slow {M}x{Nn}x{K}")
+
+
+def test_fp32_weight_gradient_at_the_baseline_shape(N):
+    """wgrad of the gate projection (config 3) with fp32 output, dY read as stored: rounding it to bf16 gives the
+    bf16 output of the same launch bit for bit, and a sample agrees with the oracle."""
+    M, Nn, K = 14336, 4096, 8192
+    aq, aq_t, _, sa_inv, _ = quantise(N, draw((M, K), 1e-3, 51), O.E5M2)
+    bq, _, _, sb_inv, _ = quantise(N, draw((Nn, K), 1.0, 52), O.E4M3)
+    out32 = N.gemm_layouts(aq_t, bq, O.E5M2, O.E4M3, N.K_SLOW, N.K_FAST, sa_inv, sb_inv, out_dtype=torch.float32)
+    out16 = N.gemm_layouts(aq_t, bq, O.E5M2, O.E4M3, N.K_SLOW, N.K_FAST, sa_inv, sb_inv)
+    assert out32.dtype == torch.float32 and torch.equal(out32.bfloat16(), out16)
+    sample_check(out32, aq, bq, O.E5M2, O.E4M3, sa_inv, sb_inv, seed=7, what="fp32 wgrad 14336x4096x8192")

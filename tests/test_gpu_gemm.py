@@ -201,6 +201,42 @@ def test_k_slow_layouts_equal_the_transposed_copies_bit_for_bit(N, fmts, shape):
         assert torch.equal(out, ref), f"layouts {la}{lb} of {shape}"
 
 
+@pytest.mark.parametrize("shape", [(256, 256, 512), (512, 768, 1024), (768, 512, 1536)])
+def test_streaming_kernel_fp32_output(N, shape):
+    """fp32 output of the streaming kernel (weight gradients of fp32 master weights), every layout:
+    exact on power-of-two operands; on random ones bit-identical to the pipelined kernel (same order of
+    accumulation), and rounding it to bf16 gives the kernel's own bf16 output (one rounding either way)."""
+    M, Nn, K = shape
+    g = torch.Generator().manual_seed(11)
+    vals = torch.tensor([0.0, 1.0, -1.0, 2.0, -2.0, 0.5, -0.5, 4.0])
+    av, bv = vals[torch.randint(0, 8, (M, K), generator=g)], vals[torch.randint(0, 8, (Nn, K), generator=g)]
+    a2 = av.to(O.TORCH_FP8[O.E5M2]).view(torch.uint8).cuda()
+    b2 = bv.to(O.TORCH_FP8[O.E4M3]).view(torch.uint8).cuda()
+    s1, s2 = torch.tensor([0.25]).cuda(), torch.tensor([2.0]).cuda()
+    exact = (av @ bv.t()) * 0.5
+    a, sa = quantised((M, K), O.E5M2, 1e-3, 3)
+    b, sb = quantised((Nn, K), O.E4M3, 1.0, 4)
+    a, b, sa, sb = a.cuda(), b.cuda(), sa.cuda(), sb.cuda()
+    N.gemm_set_variant(5)                                              # software-pipelined kernel, staged epilogue
+    ref32 = N.gemm_nt(a, b, O.E5M2, O.E4M3, sa, sb, out_dtype=torch.float32)
+    N.gemm_set_variant(-1)
+    ref32_cpu = O.t_gemm_nt(a.cpu(), b.cpu(), O.E5M2, O.E4M3, sa.cpu(), sb.cpu(), want_f32=True)[1]
+    assert max_rel_err(ref32, ref32_cpu) <= 1e-4                       # fp32 sums in a different order (and the MFMA's own inside 64 products)
+    for la, lb in ((N.K_FAST, N.K_FAST), (N.K_FAST, N.K_SLOW), (N.K_SLOW, N.K_FAST), (N.K_SLOW, N.K_SLOW)):
+        lay = lambda t, l: t.t().contiguous() if l else t
+        out = N.gemm_layouts(lay(a2, la), lay(b2, lb), O.E5M2, O.E4M3, la, lb, s1, s2, out_dtype=torch.float32)
+        assert out.dtype == torch.float32 and torch.equal(out.cpu(), exact), f"layouts {la}{lb}: power-of-two case"
+        out = N.gemm_layouts(lay(a, la), lay(b, lb), O.E5M2, O.E4M3, la, lb, sa, sb, out_dtype=torch.float32)
+        assert torch.equal(out, ref32), f"layouts {la}{lb}: differs from the pipelined kernel"
+        out16 = N.gemm_layouts(lay(a, la), lay(b, lb), O.E5M2, O.E4M3, la, lb, sa, sb)
+        assert torch.equal(out.bfloat16(), out16), f"layouts {la}{lb}: bf16(fp32 output) != bf16 output"
+    given = torch.full((M, Nn), 7.0, device="cuda")
+    assert N.gemm_layouts(a, b, O.E5M2, O.E4M3, N.K_FAST, N.K_FAST, sa, sb, out=given) is given
+    assert torch.equal(given, ref32)
+    # the automatic choice of odl_fp8_gemm_nt takes the same kernel for fp32 output
+    assert torch.equal(N.gemm_nt(a, b, O.E5M2, O.E4M3, sa, sb, out_dtype=torch.float32), ref32)
+
+
 def test_k_slow_layouts_index_check_with_one_hot_operands(N):
     # A[m, k] = 1 at k = (7 m + 3) % K, B[n, k] = 2^(n % 5) at k = (5 n + 1) % K, stored K-slow:
     # C[m, n] is that power of two where the two columns coincide and 0 elsewhere, exactly
@@ -227,4 +263,7 @@ def test_k_slow_layouts_refusals(N):
     with pytest.raises(N.NativeError, match="contraction sizes differ"):
         N.gemm_layouts(a, a.t().contiguous(), O.E4M3, O.E4M3, N.K_FAST, N.K_FAST, one, one)
     assert not N.gemm_layouts_supported(256, 256, 256) and not N.gemm_layouts_supported(384, 256, 512)
-    assert N.gemm_layouts_supported(256, 256, 512)
+    assert N.gemm_layouts_supported(256, 256, 512) and N.gemm_layouts_supported(256, 256, 512, torch.float32)
+    assert not N.gemm_layouts_supported(256, 256, 512, torch.float16)
+    with pytest.raises(N.NativeError, match="wrong shape / dtype"):
+        N.gemm_layouts(a, a, O.E4M3, O.E4M3, N.K_FAST, N.K_FAST, one, one, out=torch.empty((256, 256), dtype=torch.float16, device="cuda"))

@@ -460,3 +460,34 @@ def test_cache_weights_switch_requantises_after_a_data_write(amp, monkeypatch):
         again = lin(x)
     assert calls.count((256, 512)) >= 2            # the weight (and x, same shape here) quantised on every forward
     assert torch.equal(fresh, again) and max_rel_err(fresh, 2 * y0.float()) <= TOL
+
+
+@pytest.mark.parametrize("wdtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("recipe_name", ["tensorwise", "delayed"])
+def test_wgrad_reads_dy_as_stored_and_matches_the_transposed_copy_route(amp, monkeypatch, wdtype, recipe_name):
+    """With whole 256 x 256 tiles the weight gradient is computed from the row-major codes of dy
+    (no transposed copy), in the weight's own type (fp32 master weights get an fp32 gradient): the
+    result equals the route over the transposed copy bit for bit."""
+    from optimus_dl_amd import native
+
+    M, K, N = 1024, 512, 768
+    x, w, dy = seeded_bf16((M, K), 1.0, 50), seeded_bf16((N, K), 0.02, 51), seeded_bf16((M, N), 1e-3, 52)
+    results = {}
+    for direct in (True, False):
+        recipe = amp.create_fp8_recipe(recipe_name, "hybrid", amax_history_len=4)
+        recipe.direct_layouts = direct
+        lin = make_linear(w, dtype=wdtype)
+        run_step(lin, recipe, x, dy)               # delayed scaling: the second step runs on measured scales
+        seen = []
+        real = native.gemm_layouts
+        monkeypatch.setattr(native, "gemm_layouts", lambda *a, **k: (seen.append(k.get("out_dtype")), real(*a, **k))[1])
+        y, dx, dw = run_step(lin, recipe, x, dy)
+        monkeypatch.setattr(native, "gemm_layouts", real)
+        assert dw.dtype == wdtype and y.dtype == torch.bfloat16
+        assert seen == ([wdtype] if direct else [])
+        results[direct] = (y, dx, dw)
+    for got, want in zip(results[True], results[False]):
+        assert torch.equal(got, want)
+    ref = O.linear_fwd_bwd(x, w, dy) if recipe_name == "tensorwise" else None
+    if ref is not None:
+        assert max_rel_err(results[True][2], ref["dw"]) <= TOL
