@@ -53,7 +53,7 @@ static const Variant kVariants[] = {
     {"128x128x128 4 waves (64x64 per wave)", 128, 128, 256, 0.70f},
     {"256x256x128 4 waves, software-pipelined, persistent (K % 256 == 0)", 256, 256, 256, 1.10f},
     {"256x256x128 4 waves, software-pipelined, one tile per block", 256, 256, 256, 0.50f},
-    {"256x256x128 4 waves, streaming across tiles, folded epilogue (whole tiles, per-tensor scales)", 256, 256, 256, 1.25f},
+    {"256x256x128 4 waves, streaming across tiles, folded epilogue (whole tiles)", 256, 256, 256, 1.25f},
 };
 constexpr int kPipeVariant = 5, kPipeOneTileVariant = 6, kStreamVariant = 7;
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
@@ -138,7 +138,7 @@ extern "C" int odl_fp8_gemm_nt(const uint8_t *a, const uint8_t *b, int64_t M, in
     if (M == 0 || N == 0) return ODL_OK;
 
     const bool tiled_ok = K >= 128 && K % 128 == 0 && (double)M * (double)K < 4294967296.0 && (double)N * (double)K < 4294967296.0;
-    const bool stream_ok = tiled_ok && sa_n == 1 && sb_n == 1 && !bias && M % 256 == 0 && N % 256 == 0 &&
+    const bool stream_ok = tiled_ok && M % 256 == 0 && N % 256 == 0 &&
                            K % 256 == 0 && K >= 512;
     int variant = g_forced_variant >= 0 ? g_forced_variant : (tiled_ok ? choose_variant(M, N, stream_ok) : 0);
     if (variant != 0 && !tiled_ok) variant = 0;
@@ -159,7 +159,7 @@ extern "C" int odl_fp8_gemm_nt(const uint8_t *a, const uint8_t *b, int64_t M, in
     g.tiles_m = (int)tm; g.tiles_n = (int)tn;
 
     if (variant == kStreamVariant && !(pipe_ok && gemm_stream_accepts(g))) {
-        // the streaming kernel only takes whole tiles with per-tensor scales: next best kernel instead
+        // the streaming kernel only takes whole tiles: next best kernel instead
         variant = pipe_ok ? kPipeVariant : 2;
     }
     if (variant == 0) launch_gemm_generic(fmt_a, fmt_b, g, stream);

@@ -1,7 +1,7 @@
 // FP8 GEMM, 256x256 block tile, 4 waves (one per SIMD, 128x128 each), persistent,
 // with the epilogue of every tile folded under the first MFMAs of the next one.
-// C = (A[M,K] . B[N,K]^T) * (sa_inv * sb_inv) in bf16 or fp32, for the shapes training uses:
-// M % 256 == 0, N % 256 == 0, K % 256 == 0, K >= 512, per-tensor scales, no bias.
+// C = (A[M,K] . B[N,K]^T) * (sa_inv * sb_inv) (+ bias) in bf16 or fp32, for the shapes training uses:
+// M % 256 == 0, N % 256 == 0, K % 256 == 0, K >= 512; scales per tensor or per row of A / B.
 // Everything else goes to gemm_pipe.hip, whose K step this kernel shares:
 //
 //   per K step of 128 bytes (two halves h0, h1 of 64 bytes = one MFMA K each)
@@ -56,6 +56,7 @@ constexpr int LOADS = 256 / 8 / NW;        // 1 KB direct-to-LDS loads per wave 
 constexpr int GM = 8;
 constexpr int PITCH = 128 + 8;             // slab row: 64 bf16 + 8 bytes, see phase_a_fold
 constexpr int SLAB = 32 * PITCH;           // one wave's epilogue slab
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 // TA / TB: the operand is stored with the contraction index as the SLOW axis ([K, M] resp. [K, N]
 // row-major) instead of the fast one.  A stage then holds 128 K-rows of 256 bytes; the 1 KB loads
@@ -67,14 +68,18 @@ constexpr int SLAB = 32 * PITCH;           // one wave's epilogue slab
 // as the other layout: wgrad and dgrad no longer need transposed copies of their operands.
 // F32: fp32 output (weight gradients of fp32 master weights).  A 32 x 32 sub-tile is then a whole slab
 // (32 rows of 128 bytes) and leaves right after its own MFMA: 64 stores per wave and tile instead of 32.
-template <int FA, int FB, bool TA, bool TB, bool F32>
+// EPI: 0 = one scale per operand; 1 = a scale per row of A and / or per row of B (rowwise recipe);
+// 2 = the same plus an fp32 bias per output column.
+template <int FA, int FB, bool TA, bool TB, bool F32, int EPI>
 __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
     constexpr int ESZ = F32 ? 4 : 2;
+    constexpr int VEC_BYTES = 3 * 128 * 4;     // per wave: 128 row scales, 128 column scales, 128 bias values
     __shared__ __attribute__((aligned(1024))) uint8_t sA0[REGION];
     __shared__ __attribute__((aligned(1024))) uint8_t sB0[REGION];
     __shared__ __attribute__((aligned(1024))) uint8_t sA1[REGION];
     __shared__ __attribute__((aligned(1024))) uint8_t sB1[REGION];
     __shared__ __attribute__((aligned(16))) uint8_t sEpi[NW * SLAB];
+    __shared__ __attribute__((aligned(16))) uint8_t sVec[EPI > 0 ? NW * VEC_BYTES : 16];
 
     const int lane = threadIdx.x % 64;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
@@ -232,81 +237,122 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
         }
     };
     // phase A of step 0 of a later tile (or the drain after the last one): the finished tile
-    // leaves through `rsrc_c` while its accumulators are restarted from zero
+    // leaves through `rsrc_c` while its accumulators are restarted from zero.
+    //   bf16: sub-tiles (t, u), (t, u + 1) make one slab of 32 rows x 64 columns; it is read back after
+    //         the odd one and stored one MFMA later
+    //   fp32: every sub-tile is a slab of 32 rows x 32 floats, read back at once and stored one MFMA later
+    // EPI > 0: the wave's slices of the scale vectors (and of the bias) were brought to LDS by
+    // `request_vectors`; those of sub-tile i + 1 are read while MFMA i runs.
     auto phase_a_fold = [&](const uint8_t *sa_cur, const uint8_t *sb_cur, const v4i &rsrc_c) {
         // addresses are derived here (laundered ids), not kept in registers across the K loop
         int lane_e = lane, wave_e = wave;
         asm volatile("" : "+v"(lane_e));
         asm volatile("" : "+s"(wave_e));
         const uint32_t slab = lds_addr_of(sEpi) + wave_e * SLAB;
-        const uint32_t epi_w = slab + (lane_e % 32) * PITCH + (lane_e / 32) * 8;
+        const uint32_t epi_w = slab + (lane_e % 32) * PITCH + (lane_e / 32) * (F32 ? 16 : 8);
         const uint32_t epi_r = slab + (lane_e / 8) * PITCH + (lane_e % 8) * 16;
         const int c_voff = (lane_e / 8) * n2 + (lane_e % 8) * 16;
-        u32x4 back[4];
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const int t = i / 4, u = i % 4;
-            uint32_t pk[8];
+        const uint32_t vec_row = lds_addr_of(sVec) + wave_e * VEC_BYTES + (lane_e % 32) * 4;          // sa of row lr
+        const uint32_t vec_col = lds_addr_of(sVec) + wave_e * VEC_BYTES + 512 + (lane_e / 32) * 16;   // sb of columns 4 lg ..
+        float sa_next = 0.0f;
+        f32x4 sb_next[4], bias_next[4];
+        auto read_vectors = [&](int t, int u) {
+            sa_next = *(const __attribute__((address_space(3))) float *)(vec_row + t * 128);
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                pk[2 * q] = pack_bf16x2(acc[t][u][4 * q] * s_tensor, acc[t][u][4 * q + 1] * s_tensor);
-                pk[2 * q + 1] = pack_bf16x2(acc[t][u][4 * q + 2] * s_tensor, acc[t][u][4 * q + 3] * s_tensor);
+                sb_next[q] = *(const __attribute__((address_space(3))) f32x4 *)(vec_col + u * 128 + q * 32);
+                if constexpr (EPI == 2) bias_next[q] = *(const __attribute__((address_space(3))) f32x4 *)(vec_col + 512 + u * 128 + q * 32);
             }
-            acc[t][u] = mfma_32x32x64<FB, FA>(b0[u], a0[t], zero16);
-            // lane (lr, lg) holds columns 8q + 4lg + {0..3} of row lr of the sub-tile.  With a row
-            // pitch of 34 dwords the 8-byte writes of 16 consecutive rows cover all 32 banks once,
-            // and so do the 8-byte halves of the row-wise reads of two consecutive rows.
-#pragma unroll
-            for (int q = 0; q < 4; ++q) *lds_w(epi_w + (u & 1) * 64 + q * 16) = u32x2{pk[2 * q], pk[2 * q + 1]};
-            if (u & 1) {
-                // slab complete: 8 lanes cover a row with 16 bytes each, 8 rows per instruction.
-                // LDS operations of a wave execute in order, so the next writes cannot overtake these reads.
-#pragma unroll
-                for (int j = 0; j < 4; ++j) back[j] = lds_r(epi_r + j * 8 * PITCH);
-            } else if (i > 0) {
-                store_slab(back, c_voff, rsrc_c, c_soff0, n2, (i - 2) / 4, ((i - 2) % 4) / 2);   // completed one MFMA ago
-            }
-            if (i < 4) a1[i] = read_a(sa_cur, i, 1);
-            else if (i < 8) b1[i - 4] = read_b(sb_cur, i - 4, 1);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        store_slab(back, c_voff, rsrc_c, c_soff0, n2, 3, 1);
-        __builtin_amdgcn_sched_barrier(0);
-    };
-    // the same for fp32 output: sub-tile i is scaled, written to the slab as 32 rows x 32 floats, read
-    // back along the rows and stored while MFMA i + 1 runs
-    auto phase_a_fold_f32 = [&](const uint8_t *sa_cur, const uint8_t *sb_cur, const v4i &rsrc_c) {
-        int lane_e = lane, wave_e = wave;
-        asm volatile("" : "+v"(lane_e));
-        asm volatile("" : "+s"(wave_e));
-        const uint32_t slab = lds_addr_of(sEpi) + wave_e * SLAB;
-        const uint32_t epi_w = slab + (lane_e % 32) * PITCH + (lane_e / 32) * 16;
-        const uint32_t epi_r = slab + (lane_e / 8) * PITCH + (lane_e % 8) * 16;
-        const int c_voff = (lane_e / 8) * n2 + (lane_e % 8) * 16;
+        };
+        if constexpr (EPI > 0) read_vectors(0, 0);
         u32x4 back[4];
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             const int t = i / 4, u = i % 4;
             float v[16];
+            if constexpr (EPI > 0) {
 #pragma unroll
-            for (int e = 0; e < 16; ++e) v[e] = acc[t][u][e] * s_tensor;
-            acc[t][u] = mfma_32x32x64<FB, FA>(b0[u], a0[t], zero16);
-            if (i > 0) store_slab(back, c_voff, rsrc_c, c_soff0, n2, (i - 1) / 4, (i - 1) % 4);
-            // lane (lr, lg) holds columns 8q + 4lg + {0..3} of row lr: 16 bytes at 32q + 16lg, as two 8-byte
-            // writes (the row pitch of 34 dwords spreads the 32 rows of a half-wave over all 64 banks)
+                for (int q = 0; q < 4; ++q)
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                *lds_w(epi_w + q * 32) = u32x2{float_to_bits(v[4 * q]), float_to_bits(v[4 * q + 1])};
-                *lds_w(epi_w + q * 32 + 8) = u32x2{float_to_bits(v[4 * q + 2]), float_to_bits(v[4 * q + 3])};
+                    for (int e = 0; e < 4; ++e) {
+                        v[4 * q + e] = acc[t][u][4 * q + e] * (sa_next * sb_next[q][e]);
+                        if constexpr (EPI == 2) v[4 * q + e] = v[4 * q + e] + bias_next[q][e];
+                    }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) v[e] = acc[t][u][e] * s_tensor;
             }
+            uint32_t pk[8];
+            if constexpr (!F32) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) back[j] = lds_r(epi_r + j * 8 * PITCH);
+                for (int q = 0; q < 4; ++q) {
+                    pk[2 * q] = pack_bf16x2(v[4 * q], v[4 * q + 1]);
+                    pk[2 * q + 1] = pack_bf16x2(v[4 * q + 2], v[4 * q + 3]);
+                }
+            }
+            acc[t][u] = mfma_32x32x64<FB, FA>(b0[u], a0[t], zero16);
+            if constexpr (EPI > 0) {
+                if (i < 15) read_vectors((i + 1) / 4, (i + 1) % 4);
+            }
+            if constexpr (F32) {
+                if (i > 0) store_slab(back, c_voff, rsrc_c, c_soff0, n2, (i - 1) / 4, (i - 1) % 4);
+                // lane (lr, lg) holds columns 8q + 4lg + {0..3} of row lr: 16 bytes at 32q + 16lg, as two 8-byte
+                // writes (the row pitch of 34 dwords spreads the 32 rows of a half-wave over all 64 banks)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    *lds_w(epi_w + q * 32) = u32x2{float_to_bits(v[4 * q]), float_to_bits(v[4 * q + 1])};
+                    *lds_w(epi_w + q * 32 + 8) = u32x2{float_to_bits(v[4 * q + 2]), float_to_bits(v[4 * q + 3])};
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) back[j] = lds_r(epi_r + j * 8 * PITCH);
+            } else {
+                // lane (lr, lg) holds columns 8q + 4lg + {0..3} of row lr of the sub-tile.  With a row
+                // pitch of 34 dwords the 8-byte writes of 16 consecutive rows cover all 32 banks once,
+                // and so do the 8-byte halves of the row-wise reads of two consecutive rows.
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    *lds_w(epi_w + (u & 1) * 64 + q * 16) = u32x2{pk[2 * q], pk[2 * q + 1]};
+                if (u & 1) {
+                    // slab complete: 8 lanes cover a row with 16 bytes each, 8 rows per instruction.
+                    // LDS operations of a wave execute in order, so the next writes cannot overtake these reads.
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) back[j] = lds_r(epi_r + j * 8 * PITCH);
+                } else if (i > 0) {
+                    store_slab(back, c_voff, rsrc_c, c_soff0, n2, (i - 2) / 4, ((i - 2) % 4) / 2);   // completed one MFMA ago
+                }
+            }
             if (i < 4) a1[i] = read_a(sa_cur, i, 1);
             else if (i < 8) b1[i - 4] = read_b(sb_cur, i - 4, 1);
             __builtin_amdgcn_sched_barrier(0);
         }
-        store_slab(back, c_voff, rsrc_c, c_soff0, n2, 3, 3);
+        store_slab(back, c_voff, rsrc_c, c_soff0, n2, 3, F32 ? 3 : 1);
         __builtin_amdgcn_sched_barrier(0);
+    };
+    // EPI > 0: this wave's 128 row scales, 128 column scales (and 128 bias values) of the tile at (tm0, tn0)
+    // go straight to LDS, 64 floats per load.  A vector that is a single value is read with stride 0; the
+    // loads are issued one K step before the tile ends and are covered by that step's vmcnt(0).
+    auto request_vectors = [&](int tm0, int tn0) {
+        const uint32_t dst = lds_addr_of(sVec) + wave * VEC_BYTES;
+        auto rsrc_vec = [](const void *p, int64_t count) -> v4i {
+            const uint64_t addr = reinterpret_cast<uint64_t>(p);
+            return v4i{(int)(uint32_t)addr, (int)(uint32_t)(addr >> 32), (int)(count * 4), 0x00020000};
+        };
+        auto dma4 = [](const v4i &rsrc, uint32_t lds_addr, int vo, int so) {
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tbuffer_load_dword %1, %2, %3 offen lds"
+                         ::"s"(lds_addr), "v"(vo), "s"(rsrc), "s"(so));
+        };
+        const v4i ra_ = rsrc_vec(g.sa, g.sa_vec ? g.M : 1), rb_ = rsrc_vec(g.sb, g.sb_vec ? g.N : 1);
+        const int va = lane * 4 * g.sa_vec, vb = lane * 4 * g.sb_vec;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            dma4(ra_, dst + j * 256, va, (tm0 + wm0 + 64 * j) * 4 * g.sa_vec);
+            dma4(rb_, dst + 512 + j * 256, vb, (tn0 + wn0 + 64 * j) * 4 * g.sb_vec);
+        }
+        if constexpr (EPI == 2) {
+            const v4i rc_ = rsrc_vec(g.bias, g.N);
+#pragma unroll
+            for (int j = 0; j < 2; ++j) dma4(rc_, dst + 1024 + j * 256, lane * 4, (tn0 + wn0 + 64 * j) * 4);
+        }
     };
     auto sync = [&](bool after_fold) {
         if (after_fold) __builtin_amdgcn_s_waitcnt(F32 ? 0xC07F : 0x8070);   // vmcnt(63 | 32) lgkmcnt(0)
@@ -378,6 +424,7 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
             step(sA1, sB1, sA0, sB0, kt + 1);
         }
         step(sA0, sB0, sA1, sB1, KT - 2);
+        if constexpr (EPI > 0) request_vectors(m0, n0);
         step(sA1, sB1, sA0, sB0, KT - 1);
 
         // ---- the tile is finished; buffer 0 already holds the next tile's first fragments.
@@ -389,8 +436,7 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
         n0 = next_n0;
         rsrc_a = next_a;
         rsrc_b = next_b;
-        if constexpr (F32) phase_a_fold_f32(sA0, sB0, rsrc_c);
-        else phase_a_fold(sA0, sB0, rsrc_c);
+        phase_a_fold(sA0, sB0, rsrc_c);
         if (!has_next) break;
     }
 }
@@ -398,10 +444,12 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
 template <int FA, int FB, bool F32>
 void launch_out(const GemmArgs &g, int blocks_per_xcd, hipStream_t stream) {
     const dim3 grid((unsigned)(8 * blocks_per_xcd)), block(256);
-    if (g.ta && g.tb) hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB, true, true, F32>), grid, block, 0, stream, g);
-    else if (g.tb) hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB, false, true, F32>), grid, block, 0, stream, g);
-    else if (g.ta) hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB, true, false, F32>), grid, block, 0, stream, g);
-    else hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB, false, false, F32>), grid, block, 0, stream, g);
+    if (g.bias) hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB, false, false, F32, 2>), grid, block, 0, stream, g);
+    else if (g.sa_vec || g.sb_vec) hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB, false, false, F32, 1>), grid, block, 0, stream, g);
+    else if (g.ta && g.tb) hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB, true, true, F32, 0>), grid, block, 0, stream, g);
+    else if (g.tb) hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB, false, true, F32, 0>), grid, block, 0, stream, g);
+    else if (g.ta) hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB, true, false, F32, 0>), grid, block, 0, stream, g);
+    else hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB, false, false, F32, 0>), grid, block, 0, stream, g);
 }
 
 template <int FA, int FB>
@@ -415,7 +463,8 @@ void launch_fmt(const GemmArgs &g, int blocks_per_xcd, hipStream_t stream) {
 // Shapes this kernel takes (the caller checks the 32-bit offset limits shared with gemm_pipe.hip).
 bool gemm_stream_accepts(const GemmArgs &g) {
     const double esz = g.out_dtype == ODL_F32 ? 4.0 : 2.0;
-    return (g.out_dtype == ODL_BF16 || g.out_dtype == ODL_F32) && !g.sa_vec && !g.sb_vec && g.bias == nullptr &&
+    const bool vectors = g.sa_vec || g.sb_vec || g.bias != nullptr;      // only with both operands stored [rows, K]
+    return (g.out_dtype == ODL_BF16 || g.out_dtype == ODL_F32) && !(vectors && (g.ta || g.tb)) &&
            g.M % BM == 0 && g.N % BN == 0 && g.K % 256 == 0 && g.K >= 512 && (double)g.N * esz * (BM + 8) < 2147483648.0;
 }
 

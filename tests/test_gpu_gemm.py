@@ -138,6 +138,40 @@ def test_rowwise_scales_and_bias_epilogue(N):
     assert torch.equal(o2[7], o1[7] * 2) and torch.equal(o2[8], o1[8])
 
 
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("which", ["rows+cols", "rows", "cols", "rows+cols+bias", "bias"])
+def test_streaming_kernel_scale_vectors_and_bias(N, which, out_dtype):
+    """Whole-tile shapes with scale vectors and / or a bias go through the streaming kernel's folded
+    epilogue (vectors staged in LDS): bit-identical to the pipelined kernel's staged epilogue, which
+    evaluates the same expression acc * (sa * sb) + bias, and within tolerance of the oracle."""
+    M, Nn, K = 768, 512, 1024
+    x = seeded_bf16((M, K), seed=18)
+    x[:, 5] *= 100.0
+    w = seeded_bf16((Nn, K), std=0.02, seed=19)
+    rows, cols, with_bias = "rows" in which, "cols" in which, "bias" in which
+    sx = O.t_scale(O.t_amax(x, O.SCALE_ROW if rows else O.SCALE_TENSOR), O.E4M3)
+    sw = O.t_scale(O.t_amax(w, O.SCALE_ROW if cols else O.SCALE_TENSOR), O.E4M3)
+    xq = O.t_cast(x, sx, O.E4M3, O.SCALE_ROW if rows else O.SCALE_TENSOR)
+    wq = O.t_cast(w, sw, O.E4M3, O.SCALE_ROW if cols else O.SCALE_TENSOR)
+    sa_inv, sb_inv = (1 / sx).float().reshape(-1), (1 / sw).float().reshape(-1)
+    bias = torch.randn(Nn, generator=torch.Generator().manual_seed(3)) if with_bias else None
+    ref32 = O.t_gemm_nt(xq, wq, O.E4M3, O.E4M3, sa_inv, sb_inv, want_f32=True)[1]
+    if with_bias:
+        ref32 = ref32 + bias
+    args = (xq.cuda(), wq.cuda(), O.E4M3, O.E4M3, sa_inv.cuda(), sb_inv.cuda())
+    kw = dict(bias=bias.cuda() if with_bias else None, out_dtype=out_dtype)
+    N.gemm_set_variant(5)
+    pipe = N.gemm_nt(*args, **kw)
+    N.gemm_set_variant(7)
+    stream = N.gemm_nt(*args, **kw)
+    N.gemm_set_variant(-1)
+    auto = N.gemm_nt(*args, **kw)
+    assert "streaming" in N.gemm_variants()[7]
+    assert torch.equal(stream, pipe) and torch.equal(auto, pipe)
+    # fp32 output: the outlier channel makes the sums cancel, and the MFMA adds its 64 products in its own order
+    assert max_rel_err(stream, ref32.to(out_dtype)) <= (TOL if out_dtype == torch.bfloat16 else 1e-3)
+
+
 def test_transpose_symmetry(N):
     """gemm(a, b)^T == gemm(b, a): same products, only the roles swap."""
     aq, sa = quantised((512, 1024), O.E4M3, 1.0, 1)
