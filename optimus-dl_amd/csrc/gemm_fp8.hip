@@ -138,13 +138,13 @@ extern "C" int odl_fp8_gemm_nt(const uint8_t *a, const uint8_t *b, int64_t M, in
     if (M == 0 || N == 0) return ODL_OK;
 
     const bool tiled_ok = K >= 128 && K % 128 == 0 && (double)M * (double)K < 4294967296.0 && (double)N * (double)K < 4294967296.0;
-    const bool stream_ok = tiled_ok && M % 256 == 0 && N % 256 == 0 &&
-                           K % 256 == 0 && K >= 512;
+    // the pipelined and the streaming kernel address rows with 32-bit byte offsets
+    const bool lim32 = (double)(M + 256) * (double)K < 2147483648.0 && (double)(N + 256) * (double)K < 2147483648.0;
+    const bool stream_ok = tiled_ok && lim32 && M % 128 == 0 && N % 128 == 0 && K >= 512;
     int variant = g_forced_variant >= 0 ? g_forced_variant : (tiled_ok ? choose_variant(M, N, stream_ok) : 0);
     if (variant != 0 && !tiled_ok) variant = 0;
-    // the pipelined kernel walks K in pairs of 128-byte steps and addresses rows with 32-bit byte offsets
-    const bool pipe_ok = tiled_ok && K % 256 == 0 && (double)(M + 256) * (double)K < 2147483648.0 &&
-                         (double)(N + 256) * (double)K < 2147483648.0;
+    // the pipelined kernel walks K in pairs of 128-byte steps
+    const bool pipe_ok = tiled_ok && K % 256 == 0 && lim32;
     if ((variant == kPipeVariant || variant == kPipeOneTileVariant) && !pipe_ok) variant = 2;
 
     GemmArgs g;
@@ -158,8 +158,8 @@ extern "C" int odl_fp8_gemm_nt(const uint8_t *a, const uint8_t *b, int64_t M, in
     if (tm * tn > 0x7ffffff0LL) return set_error(ODL_ERR_SHAPE, "odl_fp8_gemm_nt: too many tiles");
     g.tiles_m = (int)tm; g.tiles_n = (int)tn;
 
-    if (variant == kStreamVariant && !(pipe_ok && gemm_stream_accepts(g))) {
-        // the streaming kernel only takes whole tiles: next best kernel instead
+    if (variant == kStreamVariant && !(stream_ok && gemm_stream_accepts(g))) {
+        // the streaming kernel wants M, N in multiples of 128: next best kernel instead
         variant = pipe_ok ? kPipeVariant : 2;
     }
     if (variant == 0) launch_gemm_generic(fmt_a, fmt_b, g, stream);

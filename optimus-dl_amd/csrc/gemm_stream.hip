@@ -1,7 +1,7 @@
 // FP8 GEMM, 256x256 block tile, 4 waves (one per SIMD, 128x128 each), persistent,
 // with the epilogue of every tile folded under the first MFMAs of the next one.
 // C = (A[M,K] . B[N,K]^T) * (sa_inv * sb_inv) (+ bias) in bf16 or fp32, for the shapes training uses:
-// M % 256 == 0, N % 256 == 0, K % 256 == 0, K >= 512; scales per tensor or per row of A / B.
+// M % 128 == 0, N % 128 == 0, K % 128 == 0, K >= 512; scales per tensor or per row of A / B.
 // Everything else goes to gemm_pipe.hip, whose K step this kernel shares:
 //
 //   per K step of 128 bytes (two halves h0, h1 of 64 bytes = one MFMA K each)
@@ -85,7 +85,10 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
     const int wm0 = (wave / 2) * WM, wn0 = (wave % 2) * WN;
     const int lr = lane % 32, lg = lane / 32;
-    const int KT = (int)(g.K / 128);
+    // K steps of 128 bytes come in pairs (two LDS stages): an odd count is rounded up, and the padding
+    // step is requested through the empty descriptor, so it multiplies zeros
+    const int KT = ((int)(g.K / 128) + 1) & ~1;
+    const bool padded = KT != (int)(g.K / 128);
 
     // ---- which tiles: block ids are dealt round-robin to the 8 XCDs, so the blocks of
     // one XCD (id % 8) walk one contiguous chunk of the grouped tile order together
@@ -191,9 +194,14 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
     const int n2 = (int)g.N * ESZ;                // bytes per output row
     const int c_soff0 = (wm0 * (int)g.N + wn0) * ESZ;
     const float s_tensor = bits_to_float((uint32_t)__builtin_amdgcn_readfirstlane((int)float_to_bits(g.sa[0] * g.sb[0])));
+    // M and N are multiples of 128 = the wave tile: in the last tile row / column of a matrix that is not a
+    // multiple of 256 a wave is either wholly inside or wholly outside.  One that is outside computes on the
+    // zeros that the bounded operand loads deliver and stores through the empty descriptor (nothing is written).
+    auto wave_inside = [&](int tm0, int tn0) { return tm0 + wm0 < (int)g.M && tn0 + wn0 < (int)g.N; };
     auto rsrc_out = [&](int tm0, int tn0) -> v4i {
         const uint64_t addr = reinterpret_cast<uint64_t>(reinterpret_cast<uint8_t *>(g.c) + ((int64_t)tm0 * g.N + tn0) * ESZ);
-        return v4i{(int)(uint32_t)addr, (int)(uint32_t)(addr >> 32), (int)0x80000000u, 0x00020000};
+        const v4i whole = {(int)(uint32_t)addr, (int)(uint32_t)(addr >> 32), (int)0x80000000u, 0x00020000};
+        return wave_inside(tm0, tn0) ? whole : empty;
     };
     // `us`: the slab's position in the wave tile's row, in slabs of 128 bytes
     auto store_slab = [](const u32x4 (&data)[4], int vo, const v4i &rsrc, int so_base, int row_bytes, int t, int us) {
@@ -341,7 +349,10 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
             asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tbuffer_load_dword %1, %2, %3 offen lds"
                          ::"s"(lds_addr), "v"(vo), "s"(rsrc), "s"(so));
         };
-        const v4i ra_ = rsrc_vec(g.sa, g.sa_vec ? g.M : 1), rb_ = rsrc_vec(g.sb, g.sb_vec ? g.N : 1);
+        // the bounds of a descriptor cover the per-lane offset only, not the scalar one: a wave outside the matrix
+        // must not request its (non-existent) slices at all
+        const bool inside = wave_inside(tm0, tn0);
+        const v4i ra_ = inside ? rsrc_vec(g.sa, g.sa_vec ? g.M : 1) : empty, rb_ = inside ? rsrc_vec(g.sb, g.sb_vec ? g.N : 1) : empty;
         const int va = lane * 4 * g.sa_vec, vb = lane * 4 * g.sb_vec;
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
@@ -349,7 +360,7 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
             dma4(rb_, dst + 512 + j * 256, vb, (tn0 + wn0 + 64 * j) * 4 * g.sb_vec);
         }
         if constexpr (EPI == 2) {
-            const v4i rc_ = rsrc_vec(g.bias, g.N);
+            const v4i rc_ = inside ? rsrc_vec(g.bias, g.N) : empty;
 #pragma unroll
             for (int j = 0; j < 2; ++j) dma4(rc_, dst + 1024 + j * 256, lane * 4, (tn0 + wn0 + 64 * j) * 4);
         }
@@ -366,7 +377,8 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
     // the stage just consumed -- from the next tile when this tile has no such step
     auto phase_b = [&](uint8_t *sa_cur, uint8_t *sb_cur, const uint8_t *sa_nxt, const uint8_t *sb_nxt, int kt) {
         const bool nx = kt + 2 >= KT;
-        const v4i la = nx ? next_a : rsrc_a, lb = nx ? next_b : rsrc_b;
+        const bool pad = padded && kt + 3 == KT;                  // the step requested is the padding step
+        const v4i la = nx ? next_a : (pad ? empty : rsrc_a), lb = nx ? next_b : (pad ? empty : rsrc_b);
         const int koff = nx ? kt + 2 - KT : kt + 2;               // K step to request
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
@@ -461,11 +473,13 @@ void launch_fmt(const GemmArgs &g, int blocks_per_xcd, hipStream_t stream) {
 }  // namespace
 
 // Shapes this kernel takes (the caller checks the 32-bit offset limits shared with gemm_pipe.hip).
+// An operand stored [K, rows] must fill whole tiles: the loads of a partial tile would run past the
+// end of its last K-row.  One stored [rows, K] may end after half a tile (see wave_inside).
 bool gemm_stream_accepts(const GemmArgs &g) {
     const double esz = g.out_dtype == ODL_F32 ? 4.0 : 2.0;
     const bool vectors = g.sa_vec || g.sb_vec || g.bias != nullptr;      // only with both operands stored [rows, K]
     return (g.out_dtype == ODL_BF16 || g.out_dtype == ODL_F32) && !(vectors && (g.ta || g.tb)) &&
-           g.M % BM == 0 && g.N % BN == 0 && g.K % 256 == 0 && g.K >= 512 && (double)g.N * esz * (BM + 8) < 2147483648.0;
+           g.M % (g.ta ? BM : WM) == 0 && g.N % (g.tb ? BN : WN) == 0 && g.K % 128 == 0 && g.K >= 512 && (double)g.N * esz * (BM + 8) < 2147483648.0;
 }
 
 // One block per CU at most (the kernel needs ~150 KB of LDS), 8 | grid so that the

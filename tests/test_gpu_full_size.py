@@ -289,6 +289,12 @@ def test_lm_head_shapes_forward_backward(N, M, K, V):
     sample_check(y.detach(), xq, wq, O.E4M3, O.E4M3, sx_inv, sw_inv, seed=V, what="lm_head fwd")
     sample_check(xd.grad, gq, wq_t, O.E5M2, O.E4M3, sg_inv, sw_inv, seed=V + 1, what="lm_head dgrad", cols=min(640, K))
     sample_check(lin.weight.grad, gq_t, xq_t, O.E5M2, O.E4M3, sg_inv, sx_inv, seed=V + 2, what="lm_head wgrad", cols=min(640, K))
+    # the vocabulary ends half way through a 256-wide tile: the last 384 entries on their own
+    tail = slice(V - 384, V)
+    sample_check(y.detach()[:, tail].contiguous(), xq, wq[tail], O.E4M3, O.E4M3, sx_inv, sw_inv, seed=V + 3,
+                 what="lm_head fwd, last columns", cols=384)
+    sample_check(lin.weight.grad[tail], gq_t[tail], xq_t, O.E5M2, O.E4M3, sg_inv, sx_inv, seed=V + 4,
+                 what="lm_head wgrad, last rows", cols=min(640, K))
 
 
 def test_fused_producers_at_config_3_size(N):

@@ -139,12 +139,17 @@ def test_rowwise_scales_and_bias_epilogue(N):
 
 
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("which", ["rows+cols", "rows", "cols", "rows+cols+bias", "bias"])
-def test_streaming_kernel_scale_vectors_and_bias(N, which, out_dtype):
+@pytest.mark.parametrize("which", ["tensor", "rows+cols", "rows", "cols", "rows+cols+bias", "bias"])
+@pytest.mark.parametrize("shape", [(768, 512, 1024), (384, 640, 512), (128, 128, 512), (384, 256, 640), (256, 512, 1152)])
+def test_streaming_kernel_scale_vectors_and_bias(N, which, out_dtype, shape):
     """Whole-tile shapes with scale vectors and / or a bias go through the streaming kernel's folded
     epilogue (vectors staged in LDS): bit-identical to the pipelined kernel's staged epilogue, which
-    evaluates the same expression acc * (sa * sb) + bias, and within tolerance of the oracle."""
-    M, Nn, K = 768, 512, 1024
+    evaluates the same expression acc * (sa * sb) + bias, and within tolerance of the oracle.
+    M and N need only be multiples of 128: in the last tile row / column the waves that lie outside
+    the matrix store nothing (the canary rows behind the output stay untouched).  K need only be a
+    multiple of 128: an odd number of 128-byte steps is padded with a step of zeros (the reference
+    kernel for those shapes is the tiled one, the pipelined kernel wants K % 256 == 0)."""
+    M, Nn, K = shape
     x = seeded_bf16((M, K), seed=18)
     x[:, 5] *= 100.0
     w = seeded_bf16((Nn, K), std=0.02, seed=19)
@@ -160,10 +165,12 @@ def test_streaming_kernel_scale_vectors_and_bias(N, which, out_dtype):
         ref32 = ref32 + bias
     args = (xq.cuda(), wq.cuda(), O.E4M3, O.E4M3, sa_inv.cuda(), sb_inv.cuda())
     kw = dict(bias=bias.cuda() if with_bias else None, out_dtype=out_dtype)
-    N.gemm_set_variant(5)
+    N.gemm_set_variant(5 if K % 256 == 0 else 2)
     pipe = N.gemm_nt(*args, **kw)
     N.gemm_set_variant(7)
-    stream = N.gemm_nt(*args, **kw)
+    guarded = torch.full((M + 256, Nn), 7.0, dtype=out_dtype, device="cuda")      # 256 canary rows behind the output
+    stream = N.gemm_nt(*args, out=guarded[:M], **kw)
+    assert (guarded[M:] == 7.0).all(), "rows beyond M were written"
     N.gemm_set_variant(-1)
     auto = N.gemm_nt(*args, **kw)
     assert "streaming" in N.gemm_variants()[7]
