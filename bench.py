@@ -168,6 +168,58 @@ def standalone_hbm(torch, native, iters=24):
     return out
 
 
+def other_configs(torch, steps=8, warmup=3):
+    """Whole steps (forward + backward of every Linear, weights re-quantised every step) of the other
+    configurations of BASELINE.json and of configuration 3 with fp32 master weights (the reference's
+    usual AMP set-up: the weight gradient is then fp32).  Same harness as the headline, fewer steps."""
+    from optimus_dl_amd.modules.amp import create_fp8_recipe
+    from optimus_dl_amd.modules.fp8_linear import FP8Linear
+
+    cases = [
+        ("configs[1] attention projections, tensorwise", "tensorwise", {}, [(4096, 4096), (4096, 1024), (4096, 1024), (4096, 4096)], 8192, torch.bfloat16),
+        ("configs[2] with fp32 master weights", "tensorwise", {}, [(k, n) for _, k, n in LAYERS], M_TOKENS, torch.float32),
+        ("configs[3] rowwise, M=16384", "rowwise", {}, [(4096, 14336)], 16384, torch.bfloat16),
+        ("configs[4] delayed H=16, Llama-3-70B MLP up/down", "delayed", {"amax_history_len": 16}, [(8192, 28672), (28672, 8192)], 8192, torch.bfloat16),
+    ]
+    out = {}
+    for label, kind, kw, shapes, m, wdtype in cases:
+        recipe = create_fp8_recipe(kind, "hybrid", **kw)
+        g = torch.Generator().manual_seed(0)
+        mods, xs, dys = [], [], []
+        for k, n in shapes:
+            lin = FP8Linear(k, n, bias=False, device="cuda", dtype=wdtype)
+            with torch.no_grad():
+                lin.weight.copy_((torch.randn(n, k, generator=g) * 0.02).to(wdtype))
+            mods.append(lin)
+            xs.append(torch.randn(m, k, generator=g).bfloat16().cuda().requires_grad_(True))
+            dys.append((torch.randn(m, n, generator=g) * 1e-3).bfloat16().cuda())
+
+        def one():
+            for lin, x, dy in zip(mods, xs, dys):
+                lin._wcache.key = None
+                lin._wcache_rowwise.clear()
+                lin.weight.grad = None
+                x.grad = None
+                with recipe.autocast():
+                    y = lin(x)
+                with recipe.backward():
+                    y.backward(dy)
+
+        for _ in range(warmup):
+            one()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            one()
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / steps
+        flop = sum(6.0 * m * k * n for k, n in shapes)
+        out[label] = {"ms_per_step": 1e3 * dt, "TFLOP/s": flop / dt / 1e12, "flop_per_step": flop}
+        del mods, xs, dys
+        torch.cuda.empty_cache()
+    return out
+
+
 def mlp_block(torch, native, recipe, steps=10, warmup=3):
     """The same three Linears wired as the MLP they come from (optimus_dl/modules/model/blocks/mlp.py:73-78):
     c_proj(silu(w1 x) * w2 x), forward + backward, weights re-quantised every step; once with the fused
@@ -431,6 +483,7 @@ def main() -> int:
         del layers, data
         line["mlp_block_fwd_bwd"] = mlp_block(torch, native, recipe)
         line["llama3_8b_block_fwd_bwd"] = llama_block(torch)
+        line["other_configs_fwd_bwd"] = other_configs(torch)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(torch)
     print(json.dumps(line))
