@@ -284,6 +284,25 @@ int odl_fp8_gemm_layouts(const uint8_t *a, const uint8_t *b, int64_t M, int64_t 
                          const float *sb_inv, void *c, int out_dtype, odl_stream_t stream);
 
 /*
+ * The same product for an output of few 256 x 256 tiles and a long contraction (weight gradients of
+ * small layers, the input gradient of a vocabulary-sized head): K is cut into `splits` runs that are
+ * computed side by side as unscaled fp32 partial results in `workspace` ([splits, M, N] floats,
+ * caller-owned, no other use while the call is in flight on its stream), then added in run order,
+ * scaled (sa_n / sb_n as for odl_fp8_gemm_nt), biased (fp32, may be NULL) and rounded once.  The sum
+ * is therefore taken in a different order than by odl_fp8_gemm_nt: equal within fp32 rounding,
+ * bit-identical where every partial sum is exact.  odl_fp8_gemm_split_count proposes `splits`
+ * for a shape (1 = not worth splitting); any 2 <= splits <= 64 that leaves every run at least 512
+ * long is accepted.  M, N, K multiples of 128 (256 for an operand stored K-slow), K-run >= 512.
+ * No counterpart in the reference, whose GEMMs are cuBLASLt's choice inside te.pytorch.Linear.
+ */
+int odl_fp8_gemm_split_count(int64_t M, int64_t N, int64_t K);
+int odl_fp8_gemm_splitk(const uint8_t *a, const uint8_t *b, int64_t M, int64_t N, int64_t K,
+                        int fmt_a, int fmt_b, int layout_a, int layout_b,
+                        const float *sa_inv, int64_t sa_n, const float *sb_inv, int64_t sb_n,
+                        const float *bias, void *c, int out_dtype, int splits,
+                        void *workspace, int64_t workspace_bytes, odl_stream_t stream);
+
+/*
  * Delayed-scaling bookkeeping for R tensor roles with H history slots each
  * (recipe "delayed", fp8.py:279-288; runs where the reference leaves its
  * autocast context, fp8.py:337-340,357-360).

@@ -21,6 +21,9 @@ struct GemmArgs {
     int out_dtype;               // bias, when present, is fp32
     int tiles_m, tiles_n;
     int ta = 0, tb = 0;          // operand stored [K, M] / [K, N] (contraction index slow); streaming kernel only
+    // streaming kernel only: splits > 1 cuts K into `splits` runs of `split_steps` 128-byte steps (an even number;
+    // the last run may be shorter) and `c` is an fp32 workspace [splits, M, N] of unscaled partial results
+    int splits = 1, split_steps = 0;
 };
 
 __device__ __forceinline__ int swz(int row) { return (row ^ (row >> 3)) & 7; }

@@ -6,7 +6,8 @@
 //   gemm_tiled.hip : BM x BN block tiles through two LDS stages
 //   gemm_pipe.hip  : 256x256 tile, one wave per SIMD, explicit software pipeline
 //   gemm_stream.hip: the same pipeline running across tile boundaries, epilogue under the
-//                    next tile's MFMAs (bf16 output, per-tensor scales, whole tiles only)
+//                    next tile's MFMAs (M, N, K multiples of 128); with a split over K for
+//                    outputs of few tiles, summed by splitk_reduce_kernel below
 //   here           : generic one-wave-per-32x32-tile kernel for any M, N, K % 16 == 0
 #include "gemm_common.h"
 
@@ -36,6 +37,38 @@ __global__ __launch_bounds__(64) void gemm_nt_generic_kernel(const GemmArgs g) {
     }
     if (g.out_dtype == ODL_BF16) store_tile<true, false>(g, acc, m0 + lr, n0 + 4 * lg);
     else store_tile<false, false>(g, acc, m0 + lr, n0 + 4 * lg);
+}
+
+// ---------------------------------------------------------------- sum of K splits
+// out[m, n] = ((p_0 + p_1) + ... + p_{S-1})[m, n] * (sa[m] * sb[n]) (+ bias[n]), fp32 throughout, one
+// rounding to the output type; the partial results are added in split order, so the result does not
+// depend on how the splits were scheduled.  Four consecutive columns per lane (N % 4 == 0).
+template <bool OUT_BF16>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restrict__ parts, int splits, int64_t M, int64_t N,
+                                                            const float *__restrict__ sa, int sa_vec, const float *__restrict__ sb,
+                                                            int sb_vec, const float *__restrict__ bias, void *__restrict__ out) {
+    const int64_t quads = M * N / 4, slice = M * N;
+    for (int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; q < quads; q += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t e = q * 4, m = e / N, n = e % N;
+        typedef float f32x4 __attribute__((ext_vector_type(4)));
+        f32x4 acc = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(parts + e));
+        for (int s = 1; s < splits; ++s) {
+            const f32x4 p = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(parts + s * slice + e));
+            acc.x = acc.x + p.x; acc.y = acc.y + p.y; acc.z = acc.z + p.z; acc.w = acc.w + p.w;
+        }
+        const float a = sa[m * sa_vec];
+        float v[4] = {acc.x * (a * sb[n * sb_vec]), acc.y * (a * sb[(n + 1) * sb_vec]), acc.z * (a * sb[(n + 2) * sb_vec]),
+                      acc.w * (a * sb[(n + 3) * sb_vec])};
+        if (bias) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) v[j] = v[j] + bias[n + j];
+        }
+        if constexpr (OUT_BF16) {
+            *reinterpret_cast<u32x2 *>(reinterpret_cast<uint16_t *>(out) + e) = u32x2{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+        } else {
+            *reinterpret_cast<float4 *>(reinterpret_cast<float *>(out) + e) = float4{v[0], v[1], v[2], v[3]};
+        }
+    }
 }
 
 // ------------------------------------------------------------------- host side
@@ -196,4 +229,80 @@ extern "C" int odl_fp8_gemm_layouts(const uint8_t *a, const uint8_t *b, int64_t 
     if (!gemm_stream_accepts(g)) return set_error(ODL_ERR_SHAPE, "odl_fp8_gemm_layouts: shape not taken by the streaming kernel");
     launch_gemm_stream(fmt_a, fmt_b, g, cu_count(), stream);
     return check_launch("odl_fp8_gemm_layouts");
+}
+
+// How many runs to cut K into for an output of few tiles (1 = do not split).  Cost model in units of one
+// K step of a tile (128 bytes of K, about 1.1 us): a tile costs its steps plus about 3 for prologue and
+// epilogue; the runs of a split execute side by side as long as tiles x runs fit the compute units; the
+// reduction reads runs x M x N floats at about 5 TB/s and costs a launch.  A split must win by 20 %.
+extern "C" int odl_fp8_gemm_split_count(int64_t M, int64_t N, int64_t K) {
+    if (M <= 0 || N <= 0 || M % 128 || N % 128 || K % 128 || K < 2048) return 1;
+    const int64_t tiles = ((M + 255) / 256) * ((N + 255) / 256);
+    const int cus = cu_count();
+    const int64_t steps = K / 128;
+    int64_t most = cus / tiles;
+    if (most > 16) most = 16;
+    const double whole = (double)steps + 3.0;
+    double best = whole;
+    int best_splits = 1;
+    for (int64_t splits = 2; splits <= most; ++splits) {
+        const int64_t per = ((steps + splits - 1) / splits + 1) & ~(int64_t)1;
+        const int64_t last = steps - (splits - 1) * per;
+        if (per < 8 || last < 4) continue;
+        const double reduce_us = (double)splits * (double)M * (double)N * 4.0 / 5.0e6 + 3.0;
+        const double cost = (double)per + 3.0 + reduce_us / 1.1;
+        if (cost < 0.8 * whole && cost < best) { best = cost; best_splits = (int)splits; }
+    }
+    return best_splits;
+}
+
+extern "C" int odl_fp8_gemm_splitk(const uint8_t *a, const uint8_t *b, int64_t M, int64_t N, int64_t K, int fmt_a, int fmt_b,
+                                   int layout_a, int layout_b, const float *sa_inv, int64_t sa_n, const float *sb_inv,
+                                   int64_t sb_n, const float *bias, void *c, int out_dtype, int splits, void *workspace,
+                                   int64_t workspace_bytes, odl_stream_t stream_) {
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    if (!a || !b || !c || !sa_inv || !sb_inv || !workspace) return set_error(ODL_ERR_ARG, "odl_fp8_gemm_splitk: null pointer");
+    if ((fmt_a != ODL_FP8_E4M3 && fmt_a != ODL_FP8_E5M2) || (fmt_b != ODL_FP8_E4M3 && fmt_b != ODL_FP8_E5M2))
+        return set_error(ODL_ERR_ARG, "odl_fp8_gemm_splitk: formats %d, %d", fmt_a, fmt_b);
+    if ((layout_a != ODL_K_FAST && layout_a != ODL_K_SLOW) || (layout_b != ODL_K_FAST && layout_b != ODL_K_SLOW))
+        return set_error(ODL_ERR_ARG, "odl_fp8_gemm_splitk: layouts %d, %d", layout_a, layout_b);
+    if (out_dtype != ODL_BF16 && out_dtype != ODL_F32) return set_error(ODL_ERR_ARG, "odl_fp8_gemm_splitk: out_dtype %d", out_dtype);
+    if (sa_n != 1 && sa_n != M) return set_error(ODL_ERR_ARG, "odl_fp8_gemm_splitk: sa_n=%lld is neither 1 nor M", (long long)sa_n);
+    if (sb_n != 1 && sb_n != N) return set_error(ODL_ERR_ARG, "odl_fp8_gemm_splitk: sb_n=%lld is neither 1 nor N", (long long)sb_n);
+    if ((reinterpret_cast<uintptr_t>(a) & 15) || (reinterpret_cast<uintptr_t>(b) & 15) || (reinterpret_cast<uintptr_t>(c) & 15) ||
+        (reinterpret_cast<uintptr_t>(workspace) & 15))
+        return set_error(ODL_ERR_SHAPE, "odl_fp8_gemm_splitk: operands, output and workspace must be 16-byte aligned");
+    const int ta = layout_a == ODL_K_SLOW, tb = layout_b == ODL_K_SLOW;
+    const bool sizes_ok = M > 0 && N > 0 && M % (ta ? 256 : 128) == 0 && N % (tb ? 256 : 128) == 0 && K % 128 == 0 &&
+                          (double)(M + 256) * (double)K < 2147483648.0 && (double)(N + 256) * (double)K < 2147483648.0;
+    if (!sizes_ok)
+        return set_error(ODL_ERR_SHAPE, "odl_fp8_gemm_splitk: M, N, K must be multiples of 128 (256 for an operand stored K-slow) and each operand under 2 GiB; got %lld x %lld x %lld", (long long)M, (long long)N, (long long)K);
+    const int64_t steps = K / 128;
+    const int64_t per = ((steps + splits - 1) / (splits > 0 ? splits : 1) + 1) & ~(int64_t)1;
+    if (splits < 2 || splits > 64 || per < 4 || steps - (splits - 1) * per < 4)
+        return set_error(ODL_ERR_ARG, "odl_fp8_gemm_splitk: %d splits of K=%lld leave a run shorter than 512", splits, (long long)K);
+    if (workspace_bytes < (int64_t)splits * M * N * 4)
+        return set_error(ODL_ERR_ARG, "odl_fp8_gemm_splitk: workspace of %lld bytes, %lld needed", (long long)workspace_bytes,
+                         (long long)splits * M * N * 4);
+    GemmArgs g;
+    g.a = a; g.b = b; g.c = workspace; g.sa = sa_inv; g.sb = sb_inv; g.bias = nullptr;
+    g.M = M; g.N = N; g.K = K;
+    g.sa_vec = 0; g.sb_vec = 0;
+    g.out_dtype = ODL_F32;
+    g.ta = ta; g.tb = tb;
+    g.splits = splits; g.split_steps = (int)per;
+    g.tiles_m = (int)((M + 255) / 256); g.tiles_n = (int)((N + 255) / 256);
+    if (!gemm_stream_accepts(g)) return set_error(ODL_ERR_SHAPE, "odl_fp8_gemm_splitk: shape not taken by the streaming kernel");
+    launch_gemm_stream(fmt_a, fmt_b, g, cu_count(), stream);
+    const int64_t quads = M * N / 4;
+    int64_t blocks = (quads + 255) / 256;
+    if (blocks > 4 * (int64_t)cu_count()) blocks = 4 * (int64_t)cu_count();
+    const int sa_vec = sa_n == M && M != 1, sb_vec = sb_n == N && N != 1;
+    if (out_dtype == ODL_BF16)
+        hipLaunchKernelGGL((splitk_reduce_kernel<true>), dim3((unsigned)blocks), dim3(256), 0, stream, (const float *)workspace, splits, M, N,
+                           sa_inv, sa_vec, sb_inv, sb_vec, bias, c);
+    else
+        hipLaunchKernelGGL((splitk_reduce_kernel<false>), dim3((unsigned)blocks), dim3(256), 0, stream, (const float *)workspace, splits, M, N,
+                           sa_inv, sa_vec, sb_inv, sb_vec, bias, c);
+    return check_launch("odl_fp8_gemm_splitk");
 }

@@ -86,13 +86,22 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
     const int wm0 = (wave / 2) * WM, wn0 = (wave % 2) * WN;
     const int lr = lane % 32, lg = lane / 32;
     // K steps of 128 bytes come in pairs (two LDS stages): an odd count is rounded up, and the padding
-    // step is requested through the empty descriptor, so it multiplies zeros
-    const int KT = ((int)(g.K / 128) + 1) & ~1;
-    const bool padded = KT != (int)(g.K / 128);
+    // step is requested through the empty descriptor, so it multiplies zeros.  With g.splits > 1 a work item
+    // is (tile, split): the steps [split * split_steps, + split_steps) of that tile, written as an fp32
+    // partial result to slice `split` of the workspace that g.c then points to.
+    int KT = 0;
+    bool padded = false;
+    const int tiles = g.tiles_m * g.tiles_n;
+    auto item_steps = [&](int p, int &first_step, int &kt, bool &pad) {
+        first_step = __builtin_amdgcn_readfirstlane((p / tiles) * g.split_steps);
+        const int real = min(g.split_steps, (int)(g.K / 128) - first_step);
+        kt = (real + 1) & ~1;
+        pad = kt != real;
+    };
 
-    // ---- which tiles: block ids are dealt round-robin to the 8 XCDs, so the blocks of
+    // ---- which items: block ids are dealt round-robin to the 8 XCDs, so the blocks of
     // one XCD (id % 8) walk one contiguous chunk of the grouped tile order together
-    const int total = g.tiles_m * g.tiles_n;
+    const int total = tiles * g.splits;
     const int per_xcd = (total + 7) / 8;
     const int xcd = (int)(blockIdx.x % 8), stride = (int)(gridDim.x / 8);
     const int pid_end = min((xcd + 1) * per_xcd, total);
@@ -102,20 +111,25 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
     // ---- per-tile addressing: the tile's origin lives in the buffer resources, the
     // per-lane offsets are the same for every tile and for both operands
     const v4i empty = {0, 0, 0, 0x00020000};      // zero bytes: loads read as zero, stores are dropped
-    auto tile_origin = [&](int p, int &tm0, int &tn0) {
+    auto tile_origin = [&](int item, int &tm0, int &tn0) {
+        const int p = item % tiles;
         const int in_group = GM * g.tiles_n;
         const int first_m = (p / in_group) * GM;
         const int group_rows = min(g.tiles_m - first_m, GM);
-        tm0 = (first_m + (p % in_group) % group_rows) * BM;
-        tn0 = ((p % in_group) / group_rows) * BN;
+        // (integer division runs on the vector unit: readfirstlane states that the results are uniform)
+        tm0 = __builtin_amdgcn_readfirstlane((first_m + (p % in_group) % group_rows) * BM);
+        tn0 = __builtin_amdgcn_readfirstlane(((p % in_group) / group_rows) * BN);
     };
-    auto rsrc_for = [&](const uint8_t *base, int row0, int64_t rows, bool transposed) -> v4i {
-        if (transposed) {                          // [K, rows] storage: the tile starts at column row0
-            const uint64_t addr = reinterpret_cast<uint64_t>(base + row0);
-            return v4i{(int)(uint32_t)addr, (int)(uint32_t)(addr >> 32), (int)(g.K * rows - row0), 0x00020000};
+    // descriptor of an operand for the tile rows from row0 on and the K steps from first_step on
+    auto rsrc_for = [&](const uint8_t *base, int row0, int64_t rows, bool transposed, int first_step) -> v4i {
+        // an operand is smaller than 2 GiB (checked by the caller): 32-bit products, which stay scalar
+        const int k0 = first_step * 128, nrows = (int)rows, nk = (int)g.K;
+        if (transposed) {                          // [K, rows] storage: the tile starts at column row0 of K-row k0
+            const uint64_t addr = reinterpret_cast<uint64_t>(base) + (uint32_t)(k0 * nrows + row0);
+            return v4i{(int)(uint32_t)addr, (int)(uint32_t)(addr >> 32), (nk - k0) * nrows - row0, 0x00020000};
         }
-        const uint64_t addr = reinterpret_cast<uint64_t>(base + (int64_t)row0 * g.K);
-        return v4i{(int)(uint32_t)addr, (int)(uint32_t)(addr >> 32), (int)((rows - row0) * g.K), 0x00020000};
+        const uint64_t addr = reinterpret_cast<uint64_t>(base) + (uint32_t)(row0 * nk + k0);
+        return v4i{(int)(uint32_t)addr, (int)(uint32_t)(addr >> 32), (nrows - row0) * nk - k0, 0x00020000};
     };
     // per-lane source offsets of the LOADS 1 KB loads of a stage
     int voff_a[LOADS], voff_b[LOADS];
@@ -193,13 +207,16 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
     // ---- output side of the folded epilogue
     const int n2 = (int)g.N * ESZ;                // bytes per output row
     const int c_soff0 = (wm0 * (int)g.N + wn0) * ESZ;
-    const float s_tensor = bits_to_float((uint32_t)__builtin_amdgcn_readfirstlane((int)float_to_bits(g.sa[0] * g.sb[0])));
+    const float s_tensor = g.splits > 1 ? 1.0f :       // partial results leave unscaled
+        bits_to_float((uint32_t)__builtin_amdgcn_readfirstlane((int)float_to_bits(g.sa[0] * g.sb[0])));
     // M and N are multiples of 128 = the wave tile: in the last tile row / column of a matrix that is not a
     // multiple of 256 a wave is either wholly inside or wholly outside.  One that is outside computes on the
     // zeros that the bounded operand loads deliver and stores through the empty descriptor (nothing is written).
     auto wave_inside = [&](int tm0, int tn0) { return tm0 + wm0 < (int)g.M && tn0 + wn0 < (int)g.N; };
-    auto rsrc_out = [&](int tm0, int tn0) -> v4i {
-        const uint64_t addr = reinterpret_cast<uint64_t>(reinterpret_cast<uint8_t *>(g.c) + ((int64_t)tm0 * g.N + tn0) * ESZ);
+    auto rsrc_out = [&](int item, int tm0, int tn0) -> v4i {
+        const int split = __builtin_amdgcn_readfirstlane(item / tiles);
+        const uint64_t addr = reinterpret_cast<uint64_t>(reinterpret_cast<uint8_t *>(g.c) +
+                                                         ((int64_t)split * g.M * g.N + (int64_t)tm0 * g.N + tn0) * ESZ);
         const v4i whole = {(int)(uint32_t)addr, (int)(uint32_t)(addr >> 32), (int)0x80000000u, 0x00020000};
         return wave_inside(tm0, tn0) ? whole : empty;
     };
@@ -378,7 +395,11 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
     auto phase_b = [&](uint8_t *sa_cur, uint8_t *sb_cur, const uint8_t *sa_nxt, const uint8_t *sb_nxt, int kt) {
         const bool nx = kt + 2 >= KT;
         const bool pad = padded && kt + 3 == KT;                  // the step requested is the padding step
-        const v4i la = nx ? next_a : (pad ? empty : rsrc_a), lb = nx ? next_b : (pad ? empty : rsrc_b);
+        // (a nested select between three descriptors is not compiled as scalar code; the padding step
+        // instead clears the size field, which makes every load of the step read zeros)
+        v4i la = nx ? next_a : rsrc_a, lb = nx ? next_b : rsrc_b;
+        la.z = pad && !nx ? 0 : la.z;
+        lb.z = pad && !nx ? 0 : lb.z;
         const int koff = nx ? kt + 2 - KT : kt + 2;               // K step to request
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
@@ -397,8 +418,12 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
 
     // ---- first tile: steps 0 and 1 requested and awaited, then phase A of step 0
     tile_origin(pid, m0, n0);
-    rsrc_a = rsrc_for(g.a, m0, g.M, TA);
-    rsrc_b = rsrc_for(g.b, n0, g.N, TB);
+    {
+        int first_step = 0;
+        item_steps(pid, first_step, KT, padded);
+        rsrc_a = rsrc_for(g.a, m0, g.M, TA, first_step);
+        rsrc_b = rsrc_for(g.b, n0, g.N, TB, first_step);
+    }
     next_a = empty;
     next_b = empty;
 #pragma unroll
@@ -419,9 +444,11 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
         // the block's next tile, if any (scalar work only; no branches around vector code)
         const int next_pid = pid + stride;
         const bool has_next = next_pid < pid_end;
-        int next_m0 = 0, next_n0 = 0;
+        int next_m0 = 0, next_n0 = 0, next_first = 0, next_kt = 0;
+        bool next_padded = false;
         tile_origin(has_next ? next_pid : pid, next_m0, next_n0);
-        const v4i na = rsrc_for(g.a, next_m0, g.M, TA), nb = rsrc_for(g.b, next_n0, g.N, TB);
+        item_steps(has_next ? next_pid : pid, next_first, next_kt, next_padded);
+        const v4i na = rsrc_for(g.a, next_m0, g.M, TA, next_first), nb = rsrc_for(g.b, next_n0, g.N, TB, next_first);
         next_a = has_next ? na : empty;
         next_b = has_next ? nb : empty;
 
@@ -442,8 +469,10 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
         // ---- the tile is finished; buffer 0 already holds the next tile's first fragments.
         // Phase A of the next tile's step 0 stores this tile.  Without a next tile the same
         // phase runs on whatever the empty buffer delivered, only for its stores.
-        const v4i rsrc_c = rsrc_out(m0, n0);
+        const v4i rsrc_c = rsrc_out(pid, m0, n0);
         pid = next_pid;
+        KT = next_kt;
+        padded = next_padded;
         m0 = next_m0;
         n0 = next_n0;
         rsrc_a = next_a;
@@ -456,8 +485,9 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
 template <int FA, int FB, bool F32>
 void launch_out(const GemmArgs &g, int blocks_per_xcd, hipStream_t stream) {
     const dim3 grid((unsigned)(8 * blocks_per_xcd)), block(256);
-    if (g.bias) hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB, false, false, F32, 2>), grid, block, 0, stream, g);
-    else if (g.sa_vec || g.sb_vec) hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB, false, false, F32, 1>), grid, block, 0, stream, g);
+    const bool vectors = g.splits == 1 && (g.bias || g.sa_vec || g.sb_vec);     // partial results carry no scales
+    if (vectors && g.bias) hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB, false, false, F32, 2>), grid, block, 0, stream, g);
+    else if (vectors) hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB, false, false, F32, 1>), grid, block, 0, stream, g);
     else if (g.ta && g.tb) hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB, true, true, F32, 0>), grid, block, 0, stream, g);
     else if (g.tb) hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB, false, true, F32, 0>), grid, block, 0, stream, g);
     else if (g.ta) hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB, true, false, F32, 0>), grid, block, 0, stream, g);
@@ -466,7 +496,7 @@ void launch_out(const GemmArgs &g, int blocks_per_xcd, hipStream_t stream) {
 
 template <int FA, int FB>
 void launch_fmt(const GemmArgs &g, int blocks_per_xcd, hipStream_t stream) {
-    if (g.out_dtype == ODL_F32) launch_out<FA, FB, true>(g, blocks_per_xcd, stream);
+    if (g.out_dtype == ODL_F32 || g.splits > 1) launch_out<FA, FB, true>(g, blocks_per_xcd, stream);
     else launch_out<FA, FB, false>(g, blocks_per_xcd, stream);
 }
 
@@ -476,16 +506,21 @@ void launch_fmt(const GemmArgs &g, int blocks_per_xcd, hipStream_t stream) {
 // An operand stored [K, rows] must fill whole tiles: the loads of a partial tile would run past the
 // end of its last K-row.  One stored [rows, K] may end after half a tile (see wave_inside).
 bool gemm_stream_accepts(const GemmArgs &g) {
-    const double esz = g.out_dtype == ODL_F32 ? 4.0 : 2.0;
-    const bool vectors = g.sa_vec || g.sb_vec || g.bias != nullptr;      // only with both operands stored [rows, K]
+    const double esz = (g.out_dtype == ODL_F32 || g.splits > 1) ? 4.0 : 2.0;
+    const bool vectors = g.splits == 1 && (g.sa_vec || g.sb_vec || g.bias != nullptr);   // only with both operands stored [rows, K]
     return (g.out_dtype == ODL_BF16 || g.out_dtype == ODL_F32) && !(vectors && (g.ta || g.tb)) &&
            g.M % (g.ta ? BM : WM) == 0 && g.N % (g.tb ? BN : WN) == 0 && g.K % 128 == 0 && g.K >= 512 && (double)g.N * esz * (BM + 8) < 2147483648.0;
 }
 
 // One block per CU at most (the kernel needs ~150 KB of LDS), 8 | grid so that the
 // round-robin placement gives every XCD the same number of blocks.
-void launch_gemm_stream(int fa, int fb, const GemmArgs &g, int num_cus, hipStream_t stream) {
-    const int total = g.tiles_m * g.tiles_n;
+void launch_gemm_stream(int fa, int fb, const GemmArgs &args, int num_cus, hipStream_t stream) {
+    GemmArgs g = args;
+    if (g.splits <= 1) {
+        g.splits = 1;
+        g.split_steps = ((int)(g.K / 128) + 1) & ~1;
+    }
+    const int total = g.tiles_m * g.tiles_n * g.splits;
     const int per_xcd = (total + 7) / 8;
     int bpx = num_cus / 8;
     if (bpx < 1) bpx = 1;

@@ -23,7 +23,7 @@ DT_BF16, DT_F32 = 0, 1
 AMAX_MAX, AMAX_MOST_RECENT = 0, 1
 FP8_MAX = {E4M3: 448.0, E5M2: 57344.0}
 TORCH_FP8 = {E4M3: torch.float8_e4m3fn, E5M2: torch.float8_e5m2}
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # ODL_FP8_LIB names another build of the same library (e.g. one made for an experiment)
@@ -53,6 +53,8 @@ EXPORTS = (
     "odl_fp8_cast_transpose",
     "odl_fp8_gemm_nt",
     "odl_fp8_gemm_layouts",
+    "odl_fp8_gemm_split_count",
+    "odl_fp8_gemm_splitk",
     "odl_fp8_delayed_update",
     "odl_fp8_gemm_num_variants",
     "odl_fp8_gemm_variant_name",
@@ -110,6 +112,9 @@ def load() -> ctypes.CDLL:
         L.odl_fp8_cast_transpose.argtypes = [vp, i32, i64, i64, vp, i32, i32, vp, vp, vp, vp]
         L.odl_fp8_gemm_nt.argtypes = [vp, vp, i64, i64, i64, i32, i32, vp, i64, vp, i64, vp, i32, vp, i32, vp]
         L.odl_fp8_gemm_layouts.argtypes = [vp, vp, i64, i64, i64, i32, i32, i32, i32, vp, vp, vp, i32, vp]
+        L.odl_fp8_gemm_split_count.argtypes = [i64, i64, i64]
+        L.odl_fp8_gemm_split_count.restype = i32
+        L.odl_fp8_gemm_splitk.argtypes = [vp, vp, i64, i64, i64, i32, i32, i32, i32, vp, i64, vp, i64, vp, vp, i32, i32, vp, i64, vp]
         L.odl_fp8_delayed_update.argtypes = [vp, i64, i64, i64, vp, vp, vp, i32, i32, vp]
         L.odl_fp8_gemm_num_variants.restype = i32
         L.odl_fp8_gemm_variant_name.argtypes = [i32]
@@ -553,6 +558,9 @@ def gemm_nt(a: torch.Tensor, b: torch.Tensor, fmt_a: int, fmt_b: int, sa_inv: to
         out = torch.empty((M, N), dtype=out_dtype, device=a.device)
     elif out.shape != (M, N) or out.dtype != out_dtype or not out.is_contiguous():
         raise NativeError("gemm_nt: `out` has the wrong shape / dtype / layout")
+    splits = gemm_split_count(M, N, K)
+    if splits > 1:
+        return _gemm_splitk(a, b, M, N, K, fmt_a, fmt_b, K_FAST, K_FAST, sa_inv, sb_inv, bias, out, splits)
     _check(load().odl_fp8_gemm_nt(a.data_ptr(), b.data_ptr(), M, N, K, fmt_a, fmt_b, sa_inv.data_ptr(), sa_inv.numel(),
                                   sb_inv.data_ptr(), sb_inv.numel(), bias.data_ptr() if bias is not None else None,
                                   DT_F32, out.data_ptr(), odt, _stream()), "odl_fp8_gemm_nt")
@@ -560,6 +568,50 @@ def gemm_nt(a: torch.Tensor, b: torch.Tensor, fmt_a: int, fmt_b: int, sa_inv: to
 
 
 K_FAST, K_SLOW = 0, 1
+split_k = True            # outputs of few tiles with a long contraction are computed as K runs side by side
+_forced_variant = -1
+
+
+def gemm_split_count(M: int, N: int, K: int) -> int:
+    """Number of K runs the library proposes for this shape (1: one launch of the ordinary kernel).
+    Always 1 while a kernel variant is forced or ``split_k`` is off."""
+    if not split_k or _forced_variant >= 0 or (M + 256) * K >= 2**31 or (N + 256) * K >= 2**31:
+        return 1
+    return int(load().odl_fp8_gemm_split_count(M, N, K))
+
+
+def _gemm_splitk(a, b, M, N, K, fmt_a, fmt_b, layout_a, layout_b, sa_inv, sb_inv, bias, out, splits):
+    workspace = torch.empty((splits, M, N), dtype=torch.float32, device=a.device)
+    _check(load().odl_fp8_gemm_splitk(a.data_ptr(), b.data_ptr(), M, N, K, fmt_a, fmt_b, layout_a, layout_b, sa_inv.data_ptr(),
+                                      sa_inv.numel(), sb_inv.data_ptr(), sb_inv.numel(),
+                                      bias.data_ptr() if bias is not None else None, out.data_ptr(), _src_dtype(out), splits,
+                                      workspace.data_ptr(), workspace.numel() * 4, _stream()), "odl_fp8_gemm_splitk")
+    return out
+
+
+def gemm_splitk(a: torch.Tensor, b: torch.Tensor, fmt_a: int, fmt_b: int, sa_inv: torch.Tensor, sb_inv: torch.Tensor,
+                splits: int, bias: torch.Tensor | None = None, out_dtype: torch.dtype = torch.bfloat16,
+                layout_a: int = K_FAST, layout_b: int = K_FAST) -> torch.Tensor:
+    """The product of :func:`gemm_nt` / :func:`gemm_layouts` with K cut into ``splits`` runs that are computed
+    side by side and added in run order (fp32).  :func:`gemm_nt` and :func:`gemm_layouts` take this route by
+    themselves where :func:`gemm_split_count` says so; this entry is for choosing ``splits`` by hand."""
+    if a.dtype != torch.uint8 or b.dtype != torch.uint8:
+        raise NativeError("gemm_splitk operands must be uint8 FP8 codes")
+    a, b = _as_2d(a), _as_2d(b)
+    M, K = (a.shape[1], a.shape[0]) if layout_a == K_SLOW else a.shape
+    N, K2 = (b.shape[1], b.shape[0]) if layout_b == K_SLOW else b.shape
+    if K != K2:
+        raise NativeError(f"gemm_splitk: contraction sizes differ ({K} vs {K2})")
+    if sa_inv.numel() not in (1, M) or sb_inv.numel() not in (1, N):
+        raise NativeError(f"gemm_splitk: scale vectors must have 1 or M / N entries, got {sa_inv.numel()}, {sb_inv.numel()}")
+    _f32_dev(sa_inv, sa_inv.numel(), "gemm_splitk sa_inv")
+    _f32_dev(sb_inv, sb_inv.numel(), "gemm_splitk sb_inv")
+    if bias is not None:
+        _f32_dev(bias, N, "gemm_splitk bias")
+    if out_dtype not in (torch.bfloat16, torch.float32):
+        raise NativeError(f"gemm_splitk: output dtype {out_dtype} is not supported (bf16 or fp32)")
+    out = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    return _gemm_splitk(a, b, M, N, K, fmt_a, fmt_b, layout_a, layout_b, sa_inv, sb_inv, bias, out, int(splits))
 
 
 def gemm_layouts_supported(M: int, N: int, K: int, out_dtype: torch.dtype = torch.bfloat16) -> bool:
@@ -589,6 +641,9 @@ def gemm_layouts(a: torch.Tensor, b: torch.Tensor, fmt_a: int, fmt_b: int, layou
         out = torch.empty((M, N), dtype=out_dtype, device=a.device)
     elif out.shape != (M, N) or out.dtype not in (torch.bfloat16, torch.float32) or not out.is_contiguous():
         raise NativeError("gemm_layouts: `out` has the wrong shape / dtype / layout")
+    splits = gemm_split_count(M, N, K) if gemm_layouts_supported(M, N, K, out.dtype) else 1
+    if splits > 1:
+        return _gemm_splitk(a, b, M, N, K, fmt_a, fmt_b, layout_a, layout_b, sa_inv, sb_inv, None, out, splits)
     _check(load().odl_fp8_gemm_layouts(a.data_ptr(), b.data_ptr(), M, N, K, fmt_a, fmt_b, layout_a, layout_b, sa_inv.data_ptr(),
                                        sb_inv.data_ptr(), out.data_ptr(), _src_dtype(out), _stream()),
            "odl_fp8_gemm_layouts")
@@ -630,4 +685,6 @@ def gemm_variants() -> list[str]:
 
 
 def gemm_set_variant(variant: int) -> None:
+    global _forced_variant
     _check(load().odl_fp8_gemm_set_variant(variant), "odl_fp8_gemm_set_variant")
+    _forced_variant = variant

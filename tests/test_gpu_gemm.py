@@ -308,3 +308,77 @@ def test_k_slow_layouts_refusals(N):
     assert not N.gemm_layouts_supported(256, 256, 512, torch.float16)
     with pytest.raises(N.NativeError, match="wrong shape / dtype"):
         N.gemm_layouts(a, a, O.E4M3, O.E4M3, N.K_FAST, N.K_FAST, one, one, out=torch.empty((256, 256), dtype=torch.float16, device="cuda"))
+
+
+# ------------------------------------------------------------------ K cut into runs (few tiles, long contraction)
+def _runs_ok(K, splits):
+    steps = K // 128
+    per = (-(-steps // splits) + 1) & ~1
+    return per >= 4 and steps - (splits - 1) * per >= 4
+
+
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("splits", [2, 3, 4, 7])
+@pytest.mark.parametrize("shape", [(256, 384, 4096), (128, 128, 2688), (384, 256, 5248)])
+def test_split_k_equals_the_single_launch(N, shape, splits, out_dtype):
+    """Power-of-two operands: every partial sum is exact, so the runs added up must equal the single
+    launch (and the oracle) bit for bit, for every layout -- a run that starts at the wrong K offset, reads a
+    neighbour's steps or misses the padding step of an odd run breaks this.  Random operands with scale
+    vectors and a bias: within the GEMM tolerance of the oracle and close to the single launch."""
+    M, Nn, K = shape
+    if not _runs_ok(K, splits):
+        one = torch.ones(1, device="cuda")
+        z = torch.zeros((M, K), dtype=torch.uint8, device="cuda")
+        with pytest.raises(N.NativeError, match="shorter than 512"):
+            N.gemm_splitk(z, torch.zeros((Nn, K), dtype=torch.uint8, device="cuda"), O.E4M3, O.E4M3, one, one, splits)
+        return
+    g = torch.Generator().manual_seed(21)
+    vals = torch.tensor([0.0, 1.0, -1.0, 2.0, -2.0, 0.5, -0.5, 4.0])
+    av, bv = vals[torch.randint(0, 8, (M, K), generator=g)], vals[torch.randint(0, 8, (Nn, K), generator=g)]
+    a2 = av.to(O.TORCH_FP8[O.E5M2]).view(torch.uint8).cuda()
+    b2 = bv.to(O.TORCH_FP8[O.E4M3]).view(torch.uint8).cuda()
+    s1, s2 = torch.tensor([0.25]).cuda(), torch.tensor([2.0]).cuda()
+    exact = ((av @ bv.t()) * 0.5).to(out_dtype)
+    layouts = [(N.K_FAST, N.K_FAST)]
+    if M % 256 == 0 and Nn % 256 == 0:
+        layouts += [(N.K_SLOW, N.K_FAST), (N.K_FAST, N.K_SLOW), (N.K_SLOW, N.K_SLOW)]
+    for la, lb in layouts:
+        lay = lambda t, l: t.t().contiguous() if l else t
+        out = N.gemm_splitk(lay(a2, la), lay(b2, lb), O.E5M2, O.E4M3, s1, s2, splits, out_dtype=out_dtype, layout_a=la, layout_b=lb)
+        assert torch.equal(out.cpu(), exact), f"layouts {la}{lb}"
+    x = seeded_bf16((M, K), seed=28)
+    w = seeded_bf16((Nn, K), std=0.02, seed=29)
+    sx, sw = O.t_scale(O.t_amax(x, O.SCALE_ROW), O.E4M3), O.t_scale(O.t_amax(w, O.SCALE_ROW), O.E4M3)
+    xq, wq = O.t_cast(x, sx, O.E4M3, O.SCALE_ROW), O.t_cast(w, sw, O.E4M3, O.SCALE_ROW)
+    sa_inv, sb_inv = (1 / sx).float().reshape(-1), (1 / sw).float().reshape(-1)
+    bias = torch.randn(Nn, generator=g)
+    ref32 = O.t_gemm_nt(xq, wq, O.E4M3, O.E4M3, sa_inv, sb_inv, want_f32=True)[1] + bias
+    args = (xq.cuda(), wq.cuda(), O.E4M3, O.E4M3, sa_inv.cuda(), sb_inv.cuda())
+    out = N.gemm_splitk(*args, splits, bias=bias.cuda(), out_dtype=out_dtype)
+    N.gemm_set_variant(7)                           # a forced variant is never split
+    single = N.gemm_nt(*args, bias=bias.cuda(), out_dtype=out_dtype)
+    N.gemm_set_variant(-1)
+    assert max_rel_err(out, ref32.to(out_dtype)) <= (TOL if out_dtype == torch.bfloat16 else 1e-3)
+    assert max_rel_err(out, single) <= (8e-3 if out_dtype == torch.bfloat16 else 1e-5)     # one bf16 ulp / fp32 sum order
+
+
+def test_split_k_is_chosen_for_few_tiles_and_a_long_contraction(N, monkeypatch):
+    assert N.gemm_split_count(8192, 14336, 4096) == 1          # 1792 tiles: nothing to gain
+    assert N.gemm_split_count(8192, 1024, 4096) == 1           # 128 tiles, 32 steps: the reduction would cost the gain
+    assert N.gemm_split_count(1024, 4096, 8192) >= 2           # wgrad of a key / value projection
+    assert N.gemm_split_count(768, 768, 16384) >= 8            # wgrad of a small model's projection: 9 tiles
+    assert N.gemm_split_count(8192, 1024, 151936) == 2         # dgrad of a vocabulary-sized head
+    assert N.gemm_split_count(300, 512, 8192) == 1 and N.gemm_split_count(256, 256, 1024) == 1
+    a, sa = quantised((768, 8192), O.E5M2, 1e-3, 31)
+    b, sb = quantised((768, 8192), O.E4M3, 1.0, 32)
+    a, b, sa, sb = a.cuda(), b.cuda(), sa.cuda(), sb.cuda()
+    seen = []
+    real = N._gemm_splitk
+    monkeypatch.setattr(N, "_gemm_splitk", lambda *args: (seen.append(args[-1]), real(*args))[1])
+    out = N.gemm_nt(a, b, O.E5M2, O.E4M3, sa, sb)
+    assert seen == [N.gemm_split_count(768, 768, 8192)] and seen[0] > 1
+    assert max_rel_err(out, O.t_gemm_nt(a.cpu(), b.cpu(), O.E5M2, O.E4M3, sa.cpu(), sb.cpu())) <= TOL
+    monkeypatch.setattr(N, "split_k", False)
+    unsplit = N.gemm_nt(a, b, O.E5M2, O.E4M3, sa, sb)
+    assert len(seen) == 1 and max_rel_err(out, unsplit) <= 8e-3
+
