@@ -39,7 +39,7 @@ PEAK_FP8_TFLOPS = 5000.0     # MI355X dense FP8 MFMA, published
 PEAK_HBM_GBPS = 8000.0       # MI355X HBM3E, published
 # Memory-side bytes per GEMM launch (mean of the nine launches of a step), from two rocprofv3 --pmc runs
 # (FETCH_SIZE scaled x2.00, WRITE_SIZE x1.00 against a 256 MiB copy kernel): profiles/pmc_fetch_write__cfg3_mlp.md
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = 8.79e8
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = 8.78e8
 M_TOKENS, D_MODEL, D_FF = 8192, 4096, 14336
 LAYERS = (("gate", D_MODEL, D_FF), ("up", D_MODEL, D_FF), ("down", D_FF, D_MODEL))   # name, K(in), N(out)
 
