@@ -45,7 +45,7 @@ enum odl_status {
     ODL_ERR_LAUNCH = 3    /* HIP reported an error at launch */
 };
 
-/* ABI version of this header (3); bumped when a signature changes or an entry point is added. */
+/* ABI version of this header (5); bumped when a signature changes or an entry point is added. */
 int odl_fp8_abi_version(void);
 
 /* Last error message of the calling host thread ("" if none). */
