@@ -351,6 +351,102 @@ __global__ __launch_bounds__(kRmsBwdThreads) void norm_bwd_kernel(const u32x4 *_
     }
 }
 
+// Rows of at most 512 elements (the per-head q / k norms of Qwen3: 128): a row fits LPR <= 64 lanes, so a wave
+// works on 64 / LPR rows at a time and never meets the other waves (no barrier per row).  Row sums: the same
+// per-lane order, then the xor butterfly over the row's LPR lanes only; the steps 32 .. LPR of the wide kernel's
+// butterfly and its three other wave sums would add exact zeros, so dx is the same bits.  d_weight / d_bias: per-lane
+// sums over the rows a lane sees, combined over the block's row groups through LDS in group order.
+template <int SRC, bool LN, int LPR>
+__global__ __launch_bounds__(kRmsBwdThreads) void norm_bwd_narrow_kernel(const u32x4 *__restrict__ dy, const void *__restrict__ x,
+                                                                          const float *__restrict__ weight, const float *__restrict__ mean_in,
+                                                                          const float *__restrict__ rstd_in, int64_t rows, int64_t cols,
+                                                                          void *__restrict__ dx, float *__restrict__ slabs) {
+    constexpr int VPC = SRC == ODL_BF16 ? 1 : 2;
+    constexpr int NS = LN ? 2 : 1;
+    constexpr int RPW = kWave / LPR, RPB = (kRmsBwdThreads / kWave) * RPW;      // rows per wave / per block and pass
+    __shared__ float part[NS][RPB][LPR * 8];
+    const int lane = threadIdx.x % kWave, wv = threadIdx.x / kWave;
+    const int grp = wv * RPW + lane / LPR, c = lane % LPR;
+    const int64_t nchunk = cols / 8;
+    const bool ok = c < nchunk;
+    float wreg[8], dw[8], db[8];
+    {
+        const float4 w0 = ok ? *reinterpret_cast<const float4 *>(weight + c * 8) : float4{0, 0, 0, 0};
+        const float4 w1 = ok ? *reinterpret_cast<const float4 *>(weight + c * 8 + 4) : float4{0, 0, 0, 0};
+        wreg[0] = w0.x; wreg[1] = w0.y; wreg[2] = w0.z; wreg[3] = w0.w;
+        wreg[4] = w1.x; wreg[5] = w1.y; wreg[6] = w1.z; wreg[7] = w1.w;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { dw[e] = 0.0f; db[e] = 0.0f; }
+    }
+    u32x4 nx[VPC], nd;
+    auto fetch = [&](int64_t row) {
+        const bool in = ok && row < rows;
+        const u32x4 *p = reinterpret_cast<const u32x4 *>(x) + (row * nchunk + c) * VPC;
+#pragma unroll
+        for (int h = 0; h < VPC; ++h) nx[h] = in ? __builtin_nontemporal_load(p + h) : u32x4{0, 0, 0, 0};
+        nd = in ? __builtin_nontemporal_load(dy + row * nchunk + c) : u32x4{0, 0, 0, 0};
+    };
+    const int64_t stride = (int64_t)gridDim.x * RPB;
+    int64_t row = (int64_t)blockIdx.x * RPB + grp;
+    fetch(row);
+    // every lane of a wave runs the same number of passes (the shuffles need all of them): rows past the end are zeros
+    for (int64_t base = (int64_t)blockIdx.x * RPB; base < rows; base += stride, row += stride) {
+        u32x4 xr[VPC];
+#pragma unroll
+        for (int h = 0; h < VPC; ++h) xr[h] = nx[h];
+        const u32x4 dr = nd;
+        fetch(row + stride);
+        const bool live = row < rows;
+        const float rstd = live ? rstd_in[row] : 0.0f;
+        const float mean = (LN && live) ? mean_in[row] : 0.0f;
+        float xf[8], df[8], xh[8], t[8];
+        unpack8<SRC>(xr, xf);
+        unpack8<ODL_BF16>(&dr, df);
+        float a1 = 0.0f, a2 = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            xh[e] = LN ? __fmul_rn(__fsub_rn(xf[e], mean), rstd) : __fmul_rn(xf[e], rstd);
+            t[e] = __fmul_rn(df[e], wreg[e]);
+            if constexpr (LN) a1 = __fadd_rn(a1, t[e]);
+            a2 = __fmaf_rn(t[e], xh[e], a2);
+            dw[e] = __fmaf_rn(df[e], xh[e], dw[e]);
+            if constexpr (LN) db[e] = __fadd_rn(db[e], df[e]);
+        }
+#pragma unroll
+        for (int off = LPR / 2; off > 0; off >>= 1) {
+            a2 = __fadd_rn(a2, __shfl_xor(a2, off, kWave));
+            if constexpr (LN) a1 = __fadd_rn(a1, __shfl_xor(a1, off, kWave));
+        }
+        const float c2 = __fdiv_rn(a2, (float)cols), c1 = LN ? __fdiv_rn(a1, (float)cols) : 0.0f;
+        if (ok && live) {
+            float o[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = __fmul_rn(rstd, __fmaf_rn(-xh[e], c2, LN ? __fsub_rn(t[e], c1) : t[e]));
+            if constexpr (SRC == ODL_BF16) {
+                reinterpret_cast<u32x4 *>(dx)[row * nchunk + c] = u32x4{pack2(o[0], o[1]), pack2(o[2], o[3]), pack2(o[4], o[5]), pack2(o[6], o[7])};
+            } else {
+                float4 *q = reinterpret_cast<float4 *>(dx) + (row * nchunk + c) * 2;
+                q[0] = float4{o[0], o[1], o[2], o[3]};
+                q[1] = float4{o[4], o[5], o[6], o[7]};
+            }
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        part[0][grp][c * 8 + e] = dw[e];
+        if constexpr (LN) part[1][grp][c * 8 + e] = db[e];
+    }
+    __syncthreads();
+    float *slab = slabs + (int64_t)blockIdx.x * NS * cols;
+    for (int col = threadIdx.x; col < NS * cols; col += kRmsBwdThreads) {
+        const int set = col >= cols ? 1 : 0, cc = col - set * (int)cols;
+        float acc = part[set][0][cc];
+#pragma unroll
+        for (int r = 1; r < RPB; ++r) acc = __fadd_rn(acc, part[set][r][cc]);
+        slab[col] = acc;
+    }
+}
+
 // ------------------------------------------------------------------------ LayerNorm
 // Same work split and summation order as the RMSNorm kernels.  Forward, per row:
 //   mean = sum(x) / cols;  d = x - mean;  rstd = 1 / sqrt(sum(d * d) / cols + eps)   (d * d by fma)
@@ -684,6 +780,21 @@ extern "C" int odl_fp8_rmsnorm_bwd(const void *dy, const void *x, int src_dtype,
     if (cols < 8 || cols % 8 != 0 || cols > 8192 || !aligned16(x) || !aligned16(dy) || !aligned16(dx) || !aligned16(weight))
         return set_error(ODL_ERR_SHAPE, "odl_fp8_rmsnorm_bwd: cols must be a multiple of 8 in [8, 8192] and the pointers 16-byte aligned");
     int64_t g = rows < 1 ? 1 : (rows < ODL_FP8_RMSNORM_BWD_SLABS ? rows : ODL_FP8_RMSNORM_BWD_SLABS);
+    if (cols <= 512) {                                        // a row fits one wave: several rows per wave
+        const int lpr = cols <= 64 ? 8 : (cols <= 128 ? 16 : (cols <= 256 ? 32 : 64)), rpb = (kRmsBwdThreads / kWave) * (kWave / lpr);
+        g = (rows + rpb - 1) / rpb;
+        g = g < 1 ? 1 : (g < ODL_FP8_RMSNORM_BWD_SLABS ? g : ODL_FP8_RMSNORM_BWD_SLABS);
+#define ODL_RMSN(SRC, LPR) hipLaunchKernelGGL((norm_bwd_narrow_kernel<SRC, false, LPR>), dim3((unsigned)g), dim3(kRmsBwdThreads), 0, stream, reinterpret_cast<const u32x4 *>(dy), x, weight, (const float *)nullptr, rstd, rows, cols, dx, workspace)
+#define ODL_RMSN_SRC(LPR) do { if (src_dtype == ODL_BF16) ODL_RMSN(ODL_BF16, LPR); else ODL_RMSN(ODL_F32, LPR); } while (0)
+        if (lpr == 8) ODL_RMSN_SRC(8);
+        else if (lpr == 16) ODL_RMSN_SRC(16);
+        else if (lpr == 32) ODL_RMSN_SRC(32);
+        else ODL_RMSN_SRC(64);
+#undef ODL_RMSN_SRC
+#undef ODL_RMSN
+        hipLaunchKernelGGL(rmsnorm_bwd_reduce_kernel, dim3((unsigned)((cols + 63) / 64)), dim3(1024), 0, stream, workspace, (int)g, cols, dweight);
+        return check_launch("odl_fp8_rmsnorm_bwd");
+    }
     const int64_t cplw = (cols / 8 + kRmsBwdThreads - 1) / kRmsBwdThreads;
 #define ODL_RMSB(SRC, CPLW) hipLaunchKernelGGL((norm_bwd_kernel<SRC, false, CPLW>), dim3((unsigned)g), dim3(kRmsBwdThreads), 0, stream, reinterpret_cast<const u32x4 *>(dy), x, weight, (const float *)nullptr, rstd, rows, cols, dx, workspace)
 #define ODL_RMSB_SRC(CPLW) do { if (src_dtype == ODL_BF16) ODL_RMSB(ODL_BF16, CPLW); else ODL_RMSB(ODL_F32, CPLW); } while (0)
@@ -753,6 +864,21 @@ extern "C" int odl_fp8_layernorm_bwd(const void *dy, const void *x, int src_dtyp
     if (cols < 8 || cols % 8 != 0 || cols > 4096 || !aligned16(x) || !aligned16(dy) || !aligned16(dx) || !aligned16(weight))
         return set_error(ODL_ERR_SHAPE, "odl_fp8_layernorm_bwd: cols must be a multiple of 8 in [8, 4096] and the pointers 16-byte aligned");
     int64_t g = rows < 1 ? 1 : (rows < ODL_FP8_RMSNORM_BWD_SLABS ? rows : ODL_FP8_RMSNORM_BWD_SLABS);
+    if (cols <= 512) {                                        // a row fits one wave: several rows per wave
+        const int lpr = cols <= 64 ? 8 : (cols <= 128 ? 16 : (cols <= 256 ? 32 : 64)), rpb = (kRmsBwdThreads / kWave) * (kWave / lpr);
+        g = (rows + rpb - 1) / rpb;
+        g = g < 1 ? 1 : (g < ODL_FP8_RMSNORM_BWD_SLABS ? g : ODL_FP8_RMSNORM_BWD_SLABS);
+#define ODL_LNN(SRC, LPR) hipLaunchKernelGGL((norm_bwd_narrow_kernel<SRC, true, LPR>), dim3((unsigned)g), dim3(kRmsBwdThreads), 0, stream, reinterpret_cast<const u32x4 *>(dy), x, weight, mean, rstd, rows, cols, dx, workspace)
+#define ODL_LNN_SRC(LPR) do { if (src_dtype == ODL_BF16) ODL_LNN(ODL_BF16, LPR); else ODL_LNN(ODL_F32, LPR); } while (0)
+        if (lpr == 8) ODL_LNN_SRC(8);
+        else if (lpr == 16) ODL_LNN_SRC(16);
+        else if (lpr == 32) ODL_LNN_SRC(32);
+        else ODL_LNN_SRC(64);
+#undef ODL_LNN_SRC
+#undef ODL_LNN
+        hipLaunchKernelGGL(rmsnorm_bwd_reduce_kernel, dim3((unsigned)((2 * cols + 63) / 64)), dim3(1024), 0, stream, workspace, (int)g, 2 * cols, dweight);
+        return check_launch("odl_fp8_layernorm_bwd");
+    }
     const int64_t cplw = (cols / 8 + kRmsBwdThreads - 1) / kRmsBwdThreads;
 #define ODL_LNB(SRC, CPLW) hipLaunchKernelGGL((norm_bwd_kernel<SRC, true, CPLW>), dim3((unsigned)g), dim3(kRmsBwdThreads), 0, stream, reinterpret_cast<const u32x4 *>(dy), x, weight, mean, rstd, rows, cols, dx, workspace)
 #define ODL_LNB_SRC(CPLW) do { if (src_dtype == ODL_BF16) ODL_LNB(ODL_BF16, CPLW); else ODL_LNB(ODL_F32, CPLW); } while (0)

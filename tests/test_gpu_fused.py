@@ -169,7 +169,8 @@ def test_rmsnorm_exact_case_and_refusals(N):
 
 
 @pytest.mark.parametrize("rows,cols", [(1, 8), (37, 8), (2100, 8), (1, 64), (37, 64), (2100, 64), (1, 520), (37, 520), (2100, 520),
-                                       (1, 4096), (37, 4096), (1, 8192), (37, 8192)])
+                                       (1, 4096), (37, 4096), (1, 8192), (37, 8192),
+                                       (37, 96), (2100, 128), (9000, 128), (5000, 256), (2100, 512)])   # several rows per wave
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_rmsnorm_backward(N, rows, cols, dtype):
     gen = torch.Generator().manual_seed(rows * 7 + cols)
@@ -226,7 +227,8 @@ def test_amax_parts_colsum_exact_and_refusals(N):
 
 
 # ------------------------------------------------------------------- LayerNorm
-@pytest.mark.parametrize("rows,cols", [(1, 8), (37, 64), (2100, 64), (37, 520), (300, 768), (37, 1600), (37, 4096)])
+@pytest.mark.parametrize("rows,cols", [(1, 8), (37, 64), (2100, 64), (37, 520), (300, 768), (37, 1600), (37, 4096),
+                                       (37, 96), (9000, 128), (2100, 512)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("with_bias", [True, False])
 def test_layernorm_forward_and_backward(N, rows, cols, dtype, with_bias):
