@@ -117,6 +117,10 @@ static int cu_count() {
 
 static int choose_variant(int64_t M, int64_t N, bool stream_ok) {
     const int cus = cu_count();
+    // an output of at most cus / 2 tiles of 256 x 256 leaves half the chip idle with the big tiles: the 128 x 128
+    // kernel (two blocks per compute unit) spreads it four times wider (measured 15-20 % faster than either
+    // 256-wide kernel at 8192 x 1024, 8192 x 768 and 2048 x 4096 outputs, K = 768 .. 4096)
+    if (((M + 255) / 256) * ((N + 255) / 256) * 2 <= cus) return 4;
     int best = 2;
     double best_score = -1.0;
     for (int v = 2; v < kNumVariants; ++v) {                       // variant 1 (one wave per SIMD) only by explicit request
@@ -231,10 +235,15 @@ extern "C" int odl_fp8_gemm_layouts(const uint8_t *a, const uint8_t *b, int64_t 
     return check_launch("odl_fp8_gemm_layouts");
 }
 
-// How many runs to cut K into for an output of few tiles (1 = do not split).  Cost model in units of one
-// K step of a tile (128 bytes of K, about 1.1 us): a tile costs its steps plus about 3 for prologue and
-// epilogue; the runs of a split execute side by side as long as tiles x runs fit the compute units; the
-// reduction reads runs x M x N floats at about 5 TB/s and costs a launch.  A split must win by 20 %.
+// How many runs to cut K into for an output of few tiles (1 = do not split).  A model in microseconds, fitted to
+// measurements on this GPU (outputs 768 x 768 .. 8192 x 1024, K = 8192 .. 151936):
+//   one launch, 256 x 256 tiles : 0.92 us per K step of 128 (few compute units busy: high clock) + 3 steps of overhead
+//   one launch, 128 x 128 tiles : 0.60 us per step (what odl_fp8_gemm_nt takes for outputs of <= cus / 2 big tiles),
+//                                 but it reads every operand panel twice as often
+//   split                       : 1.45 us per step of a run (the whole chip busy: lower clock) + the reduction, which
+//                                 reads splits x M x N floats at about 5 TB/s, + 3 us for its launch
+//   each bounded below by its operand traffic (tiles x panel bytes) at about 12 TB/s out of the caches.
+// The runs of a split must fit the compute units at once, and a split must win by 15 %.
 extern "C" int odl_fp8_gemm_split_count(int64_t M, int64_t N, int64_t K) {
     if (M <= 0 || N <= 0 || M % 128 || N % 128 || K % 128 || K < 2048) return 1;
     const int64_t tiles = ((M + 255) / 256) * ((N + 255) / 256);
@@ -242,16 +251,25 @@ extern "C" int odl_fp8_gemm_split_count(int64_t M, int64_t N, int64_t K) {
     const int64_t steps = K / 128;
     int64_t most = cus / tiles;
     if (most > 16) most = 16;
-    const double whole = (double)steps + 3.0;
+    const double traffic_us = (double)tiles * 512.0 * (double)K / 12.0e6;
+    double whole = 0.92 * ((double)steps + 3.0);
+    if (whole < traffic_us) whole = traffic_us;
+    if (tiles * 2 <= cus) {
+        double small = 0.60 * ((double)steps + 3.0);
+        const double small_traffic_us = (double)((M + 127) / 128) * (double)((N + 127) / 128) * 256.0 * (double)K / 12.0e6;
+        if (small < small_traffic_us) small = small_traffic_us;
+        if (small < whole) whole = small;
+    }
     double best = whole;
     int best_splits = 1;
     for (int64_t splits = 2; splits <= most; ++splits) {
         const int64_t per = ((steps + splits - 1) / splits + 1) & ~(int64_t)1;
         const int64_t last = steps - (splits - 1) * per;
         if (per < 8 || last < 4) continue;
-        const double reduce_us = (double)splits * (double)M * (double)N * 4.0 / 5.0e6 + 3.0;
-        const double cost = (double)per + 3.0 + reduce_us / 1.1;
-        if (cost < 0.8 * whole && cost < best) { best = cost; best_splits = (int)splits; }
+        double run = 1.45 * ((double)per + 3.0);
+        if (run < traffic_us) run = traffic_us;
+        const double cost = run + (double)splits * (double)M * (double)N * 4.0 / 5.0e6 + 3.0;
+        if (cost < 0.85 * whole && cost < best) { best = cost; best_splits = (int)splits; }
     }
     return best_splits;
 }

@@ -365,7 +365,8 @@ def test_split_k_equals_the_single_launch(N, shape, splits, out_dtype):
 def test_split_k_is_chosen_for_few_tiles_and_a_long_contraction(N, monkeypatch):
     assert N.gemm_split_count(8192, 14336, 4096) == 1          # 1792 tiles: nothing to gain
     assert N.gemm_split_count(8192, 1024, 4096) == 1           # 128 tiles, 32 steps: the reduction would cost the gain
-    assert N.gemm_split_count(1024, 4096, 8192) >= 2           # wgrad of a key / value projection
+    assert N.gemm_split_count(1024, 4096, 8192) == 1           # wgrad of a key / value projection: 128 x 128 tiles in one launch win
+    assert N.gemm_split_count(1024, 1024, 16384) >= 8
     assert N.gemm_split_count(768, 768, 16384) >= 8            # wgrad of a small model's projection: 9 tiles
     assert N.gemm_split_count(8192, 1024, 151936) == 2         # dgrad of a vocabulary-sized head
     assert N.gemm_split_count(300, 512, 8192) == 1 and N.gemm_split_count(256, 256, 1024) == 1
