@@ -73,3 +73,22 @@ def test_build_rejects_asm_that_reads_a_scalar_too_soon_after_a_vector_write():
     assert len(check_asm_hazards(in_descriptor, "x.s")) == 1
     # instructions the compiler emitted itself are its own business
     assert check_asm_hazards("\tv_readlane_b32 s0, v1, 2\n\tbuffer_load_dword v1, v0, s[16:19], s0 offen\n", "x.s") == []
+
+
+def test_split_count_is_a_host_side_decision_with_the_documented_shape_rules():
+    """odl_fp8_gemm_split_count launches nothing; without a GPU it plans for 256 compute units."""
+    from optimus_dl_amd import native
+
+    if not native.is_built():
+        pytest.skip("library not built")
+    count = native.load().odl_fp8_gemm_split_count
+    assert count(8192, 14336, 4096) == 1                    # enough tiles: one launch
+    assert count(8192, 1024, 4096) == 1                     # 128 tiles, short contraction
+    for M, N, K in ((768, 768, 16384), (2304, 768, 16384), (1024, 1024, 16384), (8192, 1024, 151936), (8192, 768, 50304)):
+        s = count(M, N, K)
+        assert 2 <= s <= 16
+        assert ((M + 255) // 256) * ((N + 255) // 256) * s <= 256             # the runs fit the chip at once
+        steps, per = K // 128, ((-(-(K // 128) // s)) + 1) & ~1
+        assert per >= 8 and steps - (s - 1) * per >= 4                        # no run shorter than 512
+    for M, N, K in ((300, 512, 8192), (768, 768, 1024), (768, 776, 16384), (768, 768, 16400), (0, 768, 16384)):
+        assert count(M, N, K) == 1                          # not multiples of 128, or too short to split
