@@ -314,6 +314,7 @@ class FP8Recipe:
             self._depth -= 1
             _state.pop_recipe()
             if self._depth == 0:
+                self.shared_input = None          # a forward recomputed by activation checkpointing may have left one
                 self.producer_parts.clear()
                 self.update_scales("bwd")
 

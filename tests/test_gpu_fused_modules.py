@@ -332,3 +332,48 @@ def test_gpt2_mlp_with_fused_gelu(amp, monkeypatch):
     assert (M, 1024) in amax_calls and (M, 1024) in colsum_calls
     for a, b in zip(fused, plain):
         assert max_rel_err(a, b) <= 1e-2
+
+
+# ------------------------------------------------ activation checkpointing around the converted blocks
+@pytest.mark.parametrize("fuse", [True, False])
+def test_checkpointed_blocks_recompute_the_same_fp8_forward(amp, fuse):
+    """The reference wraps blocks in torch.utils.checkpoint (its `activation_checkpoint` transform,
+    model_transforms/checkpoint.py:45-81, non-reentrant by default) and runs backward inside the FP8
+    backward context: the recomputation then finds the recipe, takes the FP8 path again, saves the same
+    tensors, and with per-tensor current scaling reproduces the first forward bit for bit, so every gradient
+    equals the one of the run without checkpointing."""
+    from torch.utils.checkpoint import checkpoint
+
+    from optimus_dl_amd.modules.model import Llama, LlamaConfig
+    from optimus_dl_amd.modules.model_transforms import build_model_transform
+
+    torch.manual_seed(0)
+    m = Llama(LlamaConfig(vocab_size=256, n_layer=2, n_head=4, n_kv_head=2, n_embd=128, intermediate_size=256)).cuda()
+    build_model_transform({"_name": "fp8_linear", "replace_norm": fuse, "fuse_swiglu": fuse}).apply(m)
+    ids = torch.randint(0, 256, (4, 64), generator=torch.Generator().manual_seed(2)).cuda()
+    recipe = amp.FP8Recipe(recipe_type="tensorwise")
+
+    def run(ckpt):
+        for p in m.parameters():
+            p.grad = None
+        with amp.fp8_autocast(torch.device("cuda"), recipe):
+            x = m.embed(ids)
+            for block in m.transformer.h:
+                x = checkpoint(block, x, use_reentrant=False) if ckpt else block(x)
+            logits = m.lm_head(m.transformer.ln_f(x)).float()
+            loss = F.cross_entropy(logits.reshape(-1, 256), ids.reshape(-1))
+        with amp.fp8_backward(recipe):
+            loss.backward()
+        assert recipe.shared_input is None and not recipe.producer_parts        # nothing is kept alive after the step
+        return loss.detach(), [p.grad.detach().clone() for p in m.parameters()]
+
+    calls_before = sum(mod.fp8_calls for mod in m.modules() if hasattr(mod, "fp8_calls"))
+    loss0, grads0 = run(False)
+    calls_plain = sum(mod.fp8_calls for mod in m.modules() if hasattr(mod, "fp8_calls")) - calls_before
+    loss1, grads1 = run(True)
+    calls_ckpt = sum(mod.fp8_calls for mod in m.modules() if hasattr(mod, "fp8_calls")) - calls_before - calls_plain
+    # the Linears inside the blocks ran again on the FP8 path (the recomputation stops at a block's last saved tensor)
+    assert calls_plain + 10 <= calls_ckpt <= 2 * calls_plain - 1
+    assert torch.equal(loss0, loss1)
+    for g0, g1 in zip(grads0, grads1):
+        assert torch.equal(g0, g1)
