@@ -356,6 +356,15 @@ class FP8Linear(nn.Linear):
         return True
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if _state.active_recipe() is None:
+            return F.linear(x, self.weight, self.bias)
+        return self._forward_fp8(x)
+
+    # The FP8 path calls the native library through ctypes and keeps per-step state on the recipe: a graph
+    # compiler (the reference has a torch.compile transform, model_transforms/compile.py) must not trace into
+    # it.  Marked like this it runs as written, between the compiled parts of the model.
+    @torch.compiler.disable
+    def _forward_fp8(self, x: torch.Tensor) -> torch.Tensor:
         recipe = _state.active_recipe()
         if recipe is None or not self._fp8_eligible(x):
             return F.linear(x, self.weight, self.bias)

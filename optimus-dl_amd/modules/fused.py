@@ -53,6 +53,7 @@ class _SwiGLUFn(torch.autograd.Function):
         return dgate, dup, None
 
 
+@torch.compiler.disable
 def swiglu(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     """silu(gate) * up; fused (and feeding the next FP8 Linear) when an FP8 recipe is active."""
     recipe = _state.active_recipe()
@@ -104,6 +105,7 @@ class _RMSNormFn(torch.autograd.Function):
         return (dx if ctx.needs_input_grad[0] else None), (dw.to(weight.dtype) if ctx.needs_input_grad[1] else None), None, None
 
 
+@torch.compiler.disable
 def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor | None:
     """Fused RMSNorm when an FP8 recipe is active and the kernel takes the input; else None."""
     recipe = _state.active_recipe()
@@ -164,6 +166,7 @@ class _LayerNormFn(torch.autograd.Function):
                 db.to(ctx.bias_dtype) if ctx.bias_dtype is not None and ctx.needs_input_grad[2] else None, None, None)
 
 
+@torch.compiler.disable
 def layernorm(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, eps: float) -> torch.Tensor | None:
     """Fused LayerNorm when an FP8 recipe is active and the kernel takes the input; else None."""
     recipe = _state.active_recipe()
@@ -225,6 +228,7 @@ class _GeluFn(torch.autograd.Function):
         return dx, None
 
 
+@torch.compiler.disable
 def gelu(x: torch.Tensor) -> torch.Tensor | None:
     """Fused GELU when an FP8 recipe is active and the input is a bf16 GPU tensor; else None."""
     recipe = _state.active_recipe()

@@ -377,3 +377,42 @@ def test_checkpointed_blocks_recompute_the_same_fp8_forward(amp, fuse):
     assert torch.equal(loss0, loss1)
     for g0, g1 in zip(grads0, grads1):
         assert torch.equal(g0, g1)
+
+
+@pytest.mark.parametrize("fuse", [True, False])
+def test_a_graph_compiler_steps_around_the_fp8_modules(amp, fuse):
+    """The reference can wrap the model in torch.compile (model_transforms/compile.py).  The FP8 modules call the
+    native library and are marked so that the tracer leaves them alone: traced with the plain "eager" backend
+    (no code generation) the model gives the same bits as without the tracer, forward and backward."""
+    import torch._dynamo
+
+    from optimus_dl_amd.modules.model import Llama, LlamaConfig
+    from optimus_dl_amd.modules.model_transforms import build_model_transform
+
+    torch.manual_seed(0)
+    m = Llama(LlamaConfig(vocab_size=256, n_layer=2, n_head=4, n_kv_head=2, n_embd=128, intermediate_size=256)).cuda()
+    build_model_transform({"_name": "fp8_linear", "replace_norm": fuse, "fuse_swiglu": fuse}).apply(m)
+    ids = torch.randint(0, 256, (4, 64), generator=torch.Generator().manual_seed(2)).cuda()
+    recipe = amp.FP8Recipe(recipe_type="tensorwise")
+
+    def run(model):
+        for p in m.parameters():
+            p.grad = None
+        with amp.fp8_autocast(torch.device("cuda"), recipe):
+            logits = model(ids)["logits"].float()
+            loss = F.cross_entropy(logits.reshape(-1, 256), ids.reshape(-1))
+        with amp.fp8_backward(recipe):
+            loss.backward()
+        return loss.detach(), [p.grad.detach().clone() for p in m.parameters()]
+
+    before = sum(mod.fp8_calls for mod in m.modules() if hasattr(mod, "fp8_calls"))
+    loss0, grads0 = run(m)
+    plain_calls = sum(mod.fp8_calls for mod in m.modules() if hasattr(mod, "fp8_calls")) - before
+    torch._dynamo.reset()
+    compiled = torch.compile(m, backend="eager")
+    loss1, grads1 = run(compiled)
+    assert sum(mod.fp8_calls for mod in m.modules() if hasattr(mod, "fp8_calls")) - before == 2 * plain_calls
+    assert torch.equal(loss0, loss1)
+    for g0, g1 in zip(grads0, grads1):
+        assert torch.equal(g0, g1)
+    torch._dynamo.reset()
