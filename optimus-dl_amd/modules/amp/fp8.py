@@ -260,7 +260,7 @@ class FP8Recipe:
     # ------------------------------------------------------- producer hand-over
     @staticmethod
     def _tensor_key(t: torch.Tensor) -> tuple:
-        return (t.data_ptr(), t._version, t.numel(), t.dtype, t.device)
+        return (t.data_ptr(), _state.tensor_version(t), t.numel(), t.dtype, t.device)
 
     def offer_parts(self, tensor: torch.Tensor, parts: torch.Tensor) -> None:
         """Record the partial maxima of |tensor| that its producer computed.  The entry keeps the

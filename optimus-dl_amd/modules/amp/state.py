@@ -126,3 +126,17 @@ class MetaStore:
 
     def dirty_arenas(self, direction: str) -> list[MetaArena]:
         return [a for (dev, d), chain in self.arenas.items() if d == direction for a in chain if a.dirty and a.used]
+
+
+def tensor_version(t) -> int:
+    """The tensor's in-place modification counter, or a fresh negative number for a tensor made under
+    ``torch.inference_mode`` (those keep no counter): such a tensor then never matches a cached entry."""
+    try:
+        return t._version
+    except RuntimeError:
+        global _no_version
+        _no_version -= 1
+        return _no_version
+
+
+_no_version = 0

@@ -77,7 +77,7 @@ def _quantise_dynamic(x2d: torch.Tensor, fmt: int, margin: int, need_t: bool, ne
 
 
 def _input_key(x2d: torch.Tensor, kind: str, fmt: int, margin: int):
-    return (x2d.data_ptr(), x2d._version, tuple(x2d.shape), x2d.dtype, x2d.device, kind, fmt, margin)
+    return (x2d.data_ptr(), _state.tensor_version(x2d), tuple(x2d.shape), x2d.dtype, x2d.device, kind, fmt, margin)
 
 
 def _quantise_input_shared(recipe: FP8Recipe, x2d: torch.Tensor, fmt: int, margin: int, need_t: bool):
@@ -103,7 +103,7 @@ def _converted_input(recipe: FP8Recipe, x2d: torch.Tensor, dtype: torch.dtype) -
     """x2d in the compute dtype, contiguous.  Linears fed by the same tensor get the same
     converted tensor back (one conversion, and one quantisation downstream); autograd sees an
     ordinary tensor used twice."""
-    key = (x2d.data_ptr(), x2d._version, tuple(x2d.shape), tuple(x2d.stride()), x2d.dtype, x2d.device, dtype,
+    key = (x2d.data_ptr(), _state.tensor_version(x2d), tuple(x2d.shape), tuple(x2d.stride()), x2d.dtype, x2d.device, dtype,
            torch.is_grad_enabled() and x2d.requires_grad)
     hit = recipe.shared_input
     if recipe.share_inputs and hit is not None and hit.get("src_key") == key:
@@ -300,7 +300,7 @@ class FP8Linear(nn.Linear):
         pol = recipe.recipe
         c = self._wcache
         # delayed scaling: the codes depend on the scale in force, which changes at every refresh
-        key = (weight.data_ptr(), weight._version, id(recipe), pol.kind, recipe.scale_epoch if pol.kind == "delayed" else 0)
+        key = (weight.data_ptr(), _state.tensor_version(weight), id(recipe), pol.kind, recipe.scale_epoch if pol.kind == "delayed" else 0)
         fresh = c.key != key or not recipe.cache_weights
         if fresh or (need_t and c.wq_t is None):
             w2d = weight.detach()
@@ -322,7 +322,7 @@ class FP8Linear(nn.Linear):
     def _rowwise_weight(self, weight: torch.Tensor, pol, axis: str, both: bool = False):
         """Rowwise recipe: W scaled per output channel (fwd) or per input channel, transposed (dgrad).
         both: the other one will be asked for too (a backward follows): make them in one go."""
-        key = (weight.data_ptr(), weight._version)
+        key = (weight.data_ptr(), _state.tensor_version(weight))
         hit = self._wcache_rowwise.get(axis)
         if hit is not None and hit[0] == key:
             return hit[1], hit[2]

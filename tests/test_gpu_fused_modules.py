@@ -416,3 +416,24 @@ def test_a_graph_compiler_steps_around_the_fp8_modules(amp, fuse):
     for g0, g1 in zip(grads0, grads1):
         assert torch.equal(g0, g1)
     torch._dynamo.reset()
+
+
+@pytest.mark.parametrize("fuse", [True, False])
+def test_inference_mode_forward_equals_the_no_grad_forward(amp, fuse):
+    """Tensors made under torch.inference_mode keep no version counter, which the hand-over caches key on:
+    they must simply miss (every Linear quantises its own input) and the outputs stay the same bits."""
+    from optimus_dl_amd.modules.model import Llama, LlamaConfig
+    from optimus_dl_amd.modules.model_transforms import build_model_transform
+
+    torch.manual_seed(0)
+    m = Llama(LlamaConfig(vocab_size=256, n_layer=2, n_head=4, n_kv_head=2, n_embd=128, intermediate_size=256)).cuda().eval()
+    build_model_transform({"_name": "fp8_linear", "replace_norm": fuse, "fuse_swiglu": fuse}).apply(m)
+    ids = torch.randint(0, 256, (4, 64), generator=torch.Generator().manual_seed(2)).cuda()
+    recipe = amp.FP8Recipe(recipe_type="tensorwise")
+    before = sum(mod.fp8_calls for mod in m.modules() if hasattr(mod, "fp8_calls"))
+    with torch.no_grad(), amp.fp8_autocast(torch.device("cuda"), recipe):
+        want = m(ids)["logits"]
+    with torch.inference_mode(), amp.fp8_autocast(torch.device("cuda"), recipe):
+        got = m(ids)["logits"]
+    assert sum(mod.fp8_calls for mod in m.modules() if hasattr(mod, "fp8_calls")) - before == 2 * 15
+    assert torch.equal(got, want)
