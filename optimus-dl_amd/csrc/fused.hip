@@ -219,6 +219,61 @@ __global__ __launch_bounds__(kRmsThreads) void rmsnorm_fwd_kernel(const void *__
         for (int j = (int)gridDim.x + threadIdx.x; j < kParts; j += kRmsThreads) parts[j] = 0.0f;
 }
 
+// Rows of at most 256 elements (per-head q / k norms): LPR <= 32 lanes hold a row, a wave works on 64 / LPR rows
+// per trip.  The row sum is the same per-lane fma chain and the xor butterfly over the row's lanes; the steps
+// 32 .. LPR of the full butterfly would add exact zeros, so rstd and y are the same bits as from the kernel above.
+template <int SRC, int LPR>
+__global__ __launch_bounds__(kFusedThreads) void rmsnorm_fwd_narrow_kernel(const void *__restrict__ x, const float *__restrict__ weight,
+                                                                            int64_t rows, int64_t cols, float eps,
+                                                                            uint16_t *__restrict__ y, float *__restrict__ rstd_out,
+                                                                            float *__restrict__ parts) {
+    __shared__ uint32_t red[kFusedThreads / kWave];
+    constexpr int VPC = SRC == ODL_BF16 ? 1 : 2, RPW = kWave / LPR;
+    const int lane = threadIdx.x % kWave, c = lane % LPR;
+    const int64_t wave = (int64_t)blockIdx.x * (kFusedThreads / kWave) + threadIdx.x / kWave;
+    const int64_t nwave = (int64_t)gridDim.x * (kFusedThreads / kWave);
+    const int64_t nchunk = cols / 8;
+    const bool ok = c < nchunk;
+    float w[8];
+    {
+        const float4 w0 = ok ? *reinterpret_cast<const float4 *>(weight + c * 8) : float4{0, 0, 0, 0};
+        const float4 w1 = ok ? *reinterpret_cast<const float4 *>(weight + c * 8 + 4) : float4{0, 0, 0, 0};
+        w[0] = w0.x; w[1] = w0.y; w[2] = w0.z; w[3] = w0.w; w[4] = w1.x; w[5] = w1.y; w[6] = w1.z; w[7] = w1.w;
+    }
+    uint32_t am = 0;
+    for (int64_t row0 = wave * RPW; row0 < rows; row0 += nwave * RPW) {      // uniform per wave: every lane shuffles
+        const int64_t row = row0 + lane / LPR;
+        const bool live = ok && row < rows;
+        u32x4 raw[VPC];
+        const u32x4 *p = reinterpret_cast<const u32x4 *>(x) + (row * nchunk + c) * VPC;
+#pragma unroll
+        for (int h = 0; h < VPC; ++h) raw[h] = live ? __builtin_nontemporal_load(p + h) : u32x4{0, 0, 0, 0};
+        float f[8];
+        unpack8<SRC>(raw, f);
+        float acc = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc = __fmaf_rn(f[e], f[e], acc);
+#pragma unroll
+        for (int off = LPR / 2; off > 0; off >>= 1) acc = __fadd_rn(acc, __shfl_xor(acc, off, kWave));
+        const float mean = __fdiv_rn(acc, (float)cols);
+        const float rstd = __fdiv_rn(1.0f, __builtin_sqrtf(__fadd_rn(mean, eps)));
+        if (c == 0 && row < rows) rstd_out[row] = rstd;
+        if (live) {
+            uint32_t o[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                o[q] = pack2(__fmul_rn(__fmul_rn(f[2 * q], rstd), w[2 * q]), __fmul_rn(__fmul_rn(f[2 * q + 1], rstd), w[2 * q + 1]));
+                am = max_u16x2(am, abs_bf16x2(o[q]));
+            }
+            reinterpret_cast<u32x4 *>(y)[row * nchunk + c] = u32x4{o[0], o[1], o[2], o[3]};
+        }
+    }
+    am = block_max_u32(fold_u16x2_to_f32bits(am), red);
+    if (threadIdx.x == 0) parts[blockIdx.x] = bits_to_float(am);
+    if (blockIdx.x == 0)
+        for (int j = (int)gridDim.x + threadIdx.x; j < kParts; j += kFusedThreads) parts[j] = 0.0f;
+}
+
 __device__ __forceinline__ float wave_sum_butterfly(float acc) {
 #pragma unroll
     for (int off = kWave / 2; off > 0; off >>= 1) acc = __fadd_rn(acc, __shfl_xor(acc, off, kWave));
@@ -754,6 +809,19 @@ extern "C" int odl_fp8_rmsnorm_amax_parts(const void *x, int src_dtype, const fl
         return set_error(ODL_ERR_ARG, "odl_fp8_rmsnorm_amax_parts: null pointer");
     if (cols < 8 || cols % 8 != 0 || cols > 8192 || !aligned16(x) || !aligned16(y) || !aligned16(weight))
         return set_error(ODL_ERR_SHAPE, "odl_fp8_rmsnorm_amax_parts: cols must be a multiple of 8 in [8, 8192] and the pointers 16-byte aligned");
+    if (cols <= 256) {                                        // several rows per wave
+        const int lpr = cols <= 64 ? 8 : (cols <= 128 ? 16 : 32), rpb = (kFusedThreads / kWave) * (kWave / lpr);
+        int64_t gn = (rows + rpb - 1) / rpb;
+        gn = gn < 1 ? 1 : (gn < grid_cap() ? gn : grid_cap());
+#define ODL_RMSF(SRC, LPR) hipLaunchKernelGGL((rmsnorm_fwd_narrow_kernel<SRC, LPR>), dim3((unsigned)gn), dim3(kFusedThreads), 0, stream, x, weight, rows, cols, eps, reinterpret_cast<uint16_t *>(y), rstd, parts)
+#define ODL_RMSF_SRC(LPR) do { if (src_dtype == ODL_BF16) ODL_RMSF(ODL_BF16, LPR); else ODL_RMSF(ODL_F32, LPR); } while (0)
+        if (lpr == 8) ODL_RMSF_SRC(8);
+        else if (lpr == 16) ODL_RMSF_SRC(16);
+        else ODL_RMSF_SRC(32);
+#undef ODL_RMSF_SRC
+#undef ODL_RMSF
+        return check_launch("odl_fp8_rmsnorm_amax_parts");
+    }
     const int64_t cpl = (cols / 8 + kWave - 1) / kWave;
     const int threads = cpl <= 8 ? kFusedThreads : 256;
     const int rows_per_block = threads / kWave;
