@@ -383,3 +383,32 @@ def test_split_k_is_chosen_for_few_tiles_and_a_long_contraction(N, monkeypatch):
     unsplit = N.gemm_nt(a, b, O.E5M2, O.E4M3, sa, sb)
     assert len(seen) == 1 and max_rel_err(out, unsplit) <= 8e-3
 
+
+def test_split_k_entry_refuses_what_it_cannot_run(N):
+    """Straight at the C entry point: a workspace that is too small, a null pointer, shapes off the 128 grid,
+    an operand stored K-slow that does not fill whole tiles.  Nothing is launched in any of these cases."""
+    L = N.load()
+    M, Nn, K = 256, 384, 4096
+    a = torch.zeros((M, K), dtype=torch.uint8, device="cuda")
+    b = torch.zeros((Nn, K), dtype=torch.uint8, device="cuda")
+    one = torch.ones(1, device="cuda")
+    out = torch.full((M, Nn), 3.0, dtype=torch.bfloat16, device="cuda")
+    ws = torch.empty((2, M, Nn), dtype=torch.float32, device="cuda")
+    s = torch.cuda.current_stream().cuda_stream
+
+    def call(M_=M, N_=Nn, K_=K, la=0, lb=0, splits=2, ws_bytes=ws.numel() * 4, ws_ptr=ws.data_ptr(), out_dtype=0):
+        return L.odl_fp8_gemm_splitk(a.data_ptr(), b.data_ptr(), M_, N_, K_, 0, 0, la, lb, one.data_ptr(), 1, one.data_ptr(), 1,
+                                     None, out.data_ptr(), out_dtype, splits, ws_ptr, ws_bytes, s)
+
+    assert call() == 0
+    torch.cuda.synchronize()
+    assert (out == 0).all()                                        # zero codes: the product is zero
+    out.fill_(3.0)
+    for kwargs, text in ((dict(ws_bytes=ws.numel() * 4 - 4), "workspace"), (dict(ws_ptr=None), "null pointer"),
+                         (dict(M_=200), "multiples of 128"), (dict(K_=4100), "multiples of 128"),
+                         (dict(M_=128, la=1), "256 for an operand stored K-slow"), (dict(splits=1), "splits"),
+                         (dict(splits=65), "splits"), (dict(splits=9), "shorter than 512"), (dict(out_dtype=7), "out_dtype")):
+        assert call(**kwargs) != 0, kwargs
+        assert text in L.odl_fp8_last_error().decode(), (kwargs, L.odl_fp8_last_error().decode())
+    torch.cuda.synchronize()
+    assert (out == 3.0).all()                                      # nothing ran
