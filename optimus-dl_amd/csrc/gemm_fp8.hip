@@ -86,7 +86,7 @@ static const Variant kVariants[] = {
     {"128x128x128 4 waves (64x64 per wave)", 128, 128, 256, 0.70f},
     {"256x256x128 4 waves, software-pipelined, persistent (K % 256 == 0)", 256, 256, 256, 1.10f},
     {"256x256x128 4 waves, software-pipelined, one tile per block", 256, 256, 256, 0.50f},
-    {"256x256x128 4 waves, streaming across tiles, folded epilogue (whole tiles)", 256, 256, 256, 1.25f},
+    {"256x256x128 4 waves, streaming across tiles, folded epilogue (M, N, K multiples of 128)", 256, 256, 256, 1.25f},
 };
 constexpr int kPipeVariant = 5, kPipeOneTileVariant = 6, kStreamVariant = 7;
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
