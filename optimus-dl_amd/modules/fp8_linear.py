@@ -222,8 +222,10 @@ class _Fp8LinearFn(torch.autograd.Function):
                     gq, gq_t, sg_inv = _quantise_delayed(dy2d, pol.fmt_bwd, meta, ROLE_G, g_t_needed, g_rm_needed)
                 else:
                     parts = recipe.take_parts(dy2d)
-                    if parts is None and ctx.has_bias and native.colsum_supported(dy2d):
-                        # the amax pass also adds up the columns: the bias gradient costs no extra read of dy
+                    if ctx.has_bias and native.colsum_supported(dy2d):
+                        # the amax pass also adds up the columns: the bias gradient costs no extra read of dy.  It
+                        # runs for the column sums even when the producer of dy left its partial maxima (which are
+                        # the same numbers): one pass of this kernel is cheaper than a separate sum over the rows
                         parts, colsum = native.amax_parts_colsum(dy2d)
                         db = colsum.to(ctx.bias_dtype)
                     gq, gq_t, sg_inv, _ = _quantise_dynamic(dy2d, pol.fmt_bwd, pol.margin, g_t_needed, g_rm_needed,
