@@ -310,6 +310,70 @@ def llama_block(torch, steps=6, warmup=2):
     return out
 
 
+def whole_models(torch, which=("gpt2_124m", "qwen3_0.6b"), steps=5, warmup=3, labels=None):
+    """The reference's own small presets as whole models (GPT-2 124M at 16 x 1024 tokens, Qwen3-0.6B at 4 x 2048;
+    fp32 master weights, random init, random tokens): forward + cross-entropy + backward, weights re-quantised every
+    step.  bf16 autocast, the FP8 Linears alone, and the default transform (fused norms / activations as well);
+    attention and the loss are PyTorch's in all three."""
+    import torch.nn.functional as F
+
+    from optimus_dl_amd.modules import amp as A
+    from optimus_dl_amd.modules.model.families import GPT2, GPT2Config, Qwen3, Qwen3Config
+    from optimus_dl_amd.modules.model_transforms import build_model_transform
+
+    def make(name):
+        torch.manual_seed(0)
+        if name == "gpt2_124m":
+            return GPT2(GPT2Config(n_layer=12)), 16, 1024, 50304
+        return Qwen3(Qwen3Config(vocab_size=151936, n_layer=28, n_head=16, n_kv_head=8, n_embd=1024, head_dim=128,
+                                 intermediate_size=3072)), 4, 2048, 151936
+
+    out = {}
+    for name in which:
+        out[name] = {}
+        for label, cfg in (("bf16_autocast", None),
+                           ("fp8_linears", {"_name": "fp8_linear", "replace_norm": False, "fuse_swiglu": False, "fuse_gelu": False}),
+                           ("fp8_linears_fused_producers", {"_name": "fp8_linear"})):
+            if labels is not None and label not in labels:
+                continue
+            model, B, T, V = make(name)
+            model = model.cuda()
+            if cfg:
+                build_model_transform(cfg).apply(model)
+            recipe = A.FP8Recipe(recipe_type="tensorwise")
+            ids = torch.randint(0, V, (B, T), device="cuda")
+            tgt = torch.randint(0, V, (B * T,), device="cuda")
+
+            def one():
+                for p_ in model.parameters():
+                    p_.grad = None
+                for m in model.modules():
+                    if hasattr(m, "_wcache"):
+                        m._wcache.key = None
+                if cfg:
+                    with A.fp8_autocast(torch.device("cuda"), recipe):
+                        loss = F.cross_entropy(model(ids)["logits"].view(-1, V).float(), tgt)
+                    with A.fp8_backward(recipe):
+                        loss.backward()
+                else:
+                    with torch.autocast("cuda", dtype=torch.bfloat16):
+                        loss = F.cross_entropy(model(ids)["logits"].view(-1, V).float(), tgt)
+                    loss.backward()
+
+            for _ in range(warmup):
+                one()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                one()
+            torch.cuda.synchronize()
+            dt = (time.perf_counter() - t0) / steps
+            out[name][label] = {"ms_per_step": 1e3 * dt, "tokens_per_s": B * T / dt}
+            del model
+            torch.cuda.empty_cache()
+    return out
+
+
 def cpu_baseline(torch, seconds_hint=20.0):
     """The oracle's emulated-FP8 Linear fwd+bwd on the host cores, on a slice of the rows."""
     from oracle import oracle as O
@@ -349,6 +413,8 @@ def main() -> int:
                     help="skip the stand-alone measurements of the memory-bound kernels (keeps profiler traces to the steps)")
     ap.add_argument("--standalone-only", action="store_true",
                     help="run only the stand-alone measurements of the memory-bound kernels and print them (for profiling)")
+    ap.add_argument("--whole-models-only", default="",
+                    help="run only the whole-model step of gpt2_124m or qwen3_0.6b with the default transform and print it (for profiling)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy (reference kernel for scaling FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -369,6 +435,10 @@ def main() -> int:
         return 2
     if args.standalone_only:
         print(json.dumps({"hbm_kernels_standalone": standalone_hbm(torch, native)}))
+        return 0
+    if args.whole_models_only:
+        print(json.dumps({"whole_models_fwd_bwd": whole_models(torch, which=(args.whole_models_only,), steps=args.steps,
+                                                                   labels=("fp8_linears_fused_producers",))}))
         return 0
     native.gemm_set_variant(args.gemm_variant)
     dev = "cuda"
@@ -484,6 +554,7 @@ def main() -> int:
         line["mlp_block_fwd_bwd"] = mlp_block(torch, native, recipe)
         line["llama3_8b_block_fwd_bwd"] = llama_block(torch)
         line["other_configs_fwd_bwd"] = other_configs(torch)
+        line["whole_models_fwd_bwd"] = whole_models(torch)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(torch)
     print(json.dumps(line))

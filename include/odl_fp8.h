@@ -45,7 +45,7 @@ enum odl_status {
     ODL_ERR_LAUNCH = 3    /* HIP reported an error at launch */
 };
 
-/* ABI version of this header (5); bumped when a signature changes or an entry point is added. */
+/* ABI version of this header (6); bumped when a signature changes or an entry point is added. */
 int odl_fp8_abi_version(void);
 
 /* Last error message of the calling host thread ("" if none). */
@@ -291,11 +291,11 @@ int odl_fp8_gemm_layouts(const uint8_t *a, const uint8_t *b, int64_t M, int64_t 
  * scaled (sa_n / sb_n as for odl_fp8_gemm_nt), biased (fp32, may be NULL) and rounded once.  The sum
  * is therefore taken in a different order than by odl_fp8_gemm_nt: equal within fp32 rounding,
  * bit-identical where every partial sum is exact.  odl_fp8_gemm_split_count proposes `splits`
- * for a shape (1 = not worth splitting); any 2 <= splits <= 64 that leaves every run at least 512
+ * for a shape (1 = not worth splitting; k_slow != 0: an operand will be passed K-slow); any 2 <= splits <= 64 that leaves every run at least 512
  * long is accepted.  M, N, K multiples of 128 (256 for an operand stored K-slow), K-run >= 512.
  * No counterpart in the reference, whose GEMMs are cuBLASLt's choice inside te.pytorch.Linear.
  */
-int odl_fp8_gemm_split_count(int64_t M, int64_t N, int64_t K);
+int odl_fp8_gemm_split_count(int64_t M, int64_t N, int64_t K, int k_slow);
 int odl_fp8_gemm_splitk(const uint8_t *a, const uint8_t *b, int64_t M, int64_t N, int64_t K,
                         int fmt_a, int fmt_b, int layout_a, int layout_b,
                         const float *sa_inv, int64_t sa_n, const float *sb_inv, int64_t sb_n,

@@ -24,6 +24,6 @@ int check_launch(const char *what) {
 
 }  // namespace odl
 
-extern "C" int odl_fp8_abi_version(void) { return 5; }
+extern "C" int odl_fp8_abi_version(void) { return 6; }
 
 extern "C" const char *odl_fp8_last_error(void) { return odl::g_err; }

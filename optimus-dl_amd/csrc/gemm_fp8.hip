@@ -244,7 +244,9 @@ extern "C" int odl_fp8_gemm_layouts(const uint8_t *a, const uint8_t *b, int64_t 
 //                                 reads splits x M x N floats at about 5 TB/s, + 3 us for its launch
 //   each bounded below by its operand traffic (tiles x panel bytes) at about 12 TB/s out of the caches.
 // The runs of a split must fit the compute units at once, and a split must win by 15 %.
-extern "C" int odl_fp8_gemm_split_count(int64_t M, int64_t N, int64_t K) {
+// k_slow: an operand is stored with the contraction index slow (odl_fp8_gemm_layouts), which only the streaming
+// kernel reads: the 128 x 128 kernel is then not an alternative.
+extern "C" int odl_fp8_gemm_split_count(int64_t M, int64_t N, int64_t K, int k_slow) {
     if (M <= 0 || N <= 0 || M % 128 || N % 128 || K % 128 || K < 2048) return 1;
     const int64_t tiles = ((M + 255) / 256) * ((N + 255) / 256);
     const int cus = cu_count();
@@ -254,7 +256,7 @@ extern "C" int odl_fp8_gemm_split_count(int64_t M, int64_t N, int64_t K) {
     const double traffic_us = (double)tiles * 512.0 * (double)K / 12.0e6;
     double whole = 0.92 * ((double)steps + 3.0);
     if (whole < traffic_us) whole = traffic_us;
-    if (tiles * 2 <= cus) {
+    if (tiles * 2 <= cus && !k_slow) {
         double small = 0.60 * ((double)steps + 3.0);
         const double small_traffic_us = (double)((M + 127) / 128) * (double)((N + 127) / 128) * 256.0 * (double)K / 12.0e6;
         if (small < small_traffic_us) small = small_traffic_us;

@@ -23,7 +23,7 @@ DT_BF16, DT_F32 = 0, 1
 AMAX_MAX, AMAX_MOST_RECENT = 0, 1
 FP8_MAX = {E4M3: 448.0, E5M2: 57344.0}
 TORCH_FP8 = {E4M3: torch.float8_e4m3fn, E5M2: torch.float8_e5m2}
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # ODL_FP8_LIB names another build of the same library (e.g. one made for an experiment)
@@ -112,7 +112,7 @@ def load() -> ctypes.CDLL:
         L.odl_fp8_cast_transpose.argtypes = [vp, i32, i64, i64, vp, i32, i32, vp, vp, vp, vp]
         L.odl_fp8_gemm_nt.argtypes = [vp, vp, i64, i64, i64, i32, i32, vp, i64, vp, i64, vp, i32, vp, i32, vp]
         L.odl_fp8_gemm_layouts.argtypes = [vp, vp, i64, i64, i64, i32, i32, i32, i32, vp, vp, vp, i32, vp]
-        L.odl_fp8_gemm_split_count.argtypes = [i64, i64, i64]
+        L.odl_fp8_gemm_split_count.argtypes = [i64, i64, i64, i32]
         L.odl_fp8_gemm_split_count.restype = i32
         L.odl_fp8_gemm_splitk.argtypes = [vp, vp, i64, i64, i64, i32, i32, i32, i32, vp, i64, vp, i64, vp, vp, i32, i32, vp, i64, vp]
         L.odl_fp8_delayed_update.argtypes = [vp, i64, i64, i64, vp, vp, vp, i32, i32, vp]
@@ -572,12 +572,13 @@ split_k = True            # outputs of few tiles with a long contraction are com
 _forced_variant = -1
 
 
-def gemm_split_count(M: int, N: int, K: int) -> int:
+def gemm_split_count(M: int, N: int, K: int, k_slow: bool = False) -> int:
     """Number of K runs the library proposes for this shape (1: one launch of the ordinary kernel).
+    k_slow: an operand is passed with the contraction index slow (only the streaming kernel reads that).
     Always 1 while a kernel variant is forced or ``split_k`` is off."""
     if not split_k or _forced_variant >= 0 or (M + 256) * K >= 2**31 or (N + 256) * K >= 2**31:
         return 1
-    return int(load().odl_fp8_gemm_split_count(M, N, K))
+    return int(load().odl_fp8_gemm_split_count(M, N, K, 1 if k_slow else 0))
 
 
 def _gemm_splitk(a, b, M, N, K, fmt_a, fmt_b, layout_a, layout_b, sa_inv, sb_inv, bias, out, splits):
@@ -641,7 +642,7 @@ def gemm_layouts(a: torch.Tensor, b: torch.Tensor, fmt_a: int, fmt_b: int, layou
         out = torch.empty((M, N), dtype=out_dtype, device=a.device)
     elif out.shape != (M, N) or out.dtype not in (torch.bfloat16, torch.float32) or not out.is_contiguous():
         raise NativeError("gemm_layouts: `out` has the wrong shape / dtype / layout")
-    splits = gemm_split_count(M, N, K) if gemm_layouts_supported(M, N, K, out.dtype) else 1
+    splits = gemm_split_count(M, N, K, layout_a == K_SLOW or layout_b == K_SLOW) if gemm_layouts_supported(M, N, K, out.dtype) else 1
     if splits > 1:
         return _gemm_splitk(a, b, M, N, K, fmt_a, fmt_b, layout_a, layout_b, sa_inv, sb_inv, None, out, splits)
     _check(load().odl_fp8_gemm_layouts(a.data_ptr(), b.data_ptr(), M, N, K, fmt_a, fmt_b, layout_a, layout_b, sa_inv.data_ptr(),

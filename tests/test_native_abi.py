@@ -81,9 +81,11 @@ def test_split_count_is_a_host_side_decision_with_the_documented_shape_rules():
 
     if not native.is_built():
         pytest.skip("library not built")
-    count = native.load().odl_fp8_gemm_split_count
+    raw = native.load().odl_fp8_gemm_split_count
+    count = lambda M, N, K, k_slow=0: raw(M, N, K, k_slow)
     assert count(8192, 14336, 4096) == 1                    # enough tiles: one launch
     assert count(8192, 1024, 4096) == 1                     # 128 tiles, short contraction
+    assert count(1024, 4096, 8192) == 1 and count(1024, 4096, 8192, 1) >= 2      # no 128 x 128 alternative for K-slow operands
     for M, N, K in ((768, 768, 16384), (2304, 768, 16384), (1024, 1024, 16384), (8192, 1024, 151936), (8192, 768, 50304)):
         s = count(M, N, K)
         assert 2 <= s <= 16
