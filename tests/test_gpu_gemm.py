@@ -412,3 +412,32 @@ def test_split_k_entry_refuses_what_it_cannot_run(N):
         assert text in L.odl_fp8_last_error().decode(), (kwargs, L.odl_fp8_last_error().decode())
     torch.cuda.synchronize()
     assert (out == 3.0).all()                                      # nothing ran
+
+@pytest.mark.parametrize("seed", range(48))
+def test_seeded_random_shapes_through_the_automatic_choice(N, seed):
+    """Shapes drawn on the grids the kernels distinguish (16, 128, 256), with and without scale vectors, bias and fp32
+    output: whichever kernel the library picks (generic, tiled, pipelined, streaming, K runs), the result is the oracle's."""
+    g = torch.Generator().manual_seed(1000 + seed)
+    def draw(grids, hi):
+        step = grids[int(torch.randint(0, len(grids), (1,), generator=g))]
+        return step * int(torch.randint(1, hi // step + 1, (1,), generator=g))
+    M, Nn = draw((16, 128, 256), 1024), draw((16, 128, 256), 1024)
+    K = draw((16, 128, 256), 2048) if seed % 4 else 128 * int(torch.randint(16, 80, (1,), generator=g))   # every 4th: long contraction
+    rows, cols, with_bias, f32 = (bool(int(torch.randint(0, 2, (1,), generator=g))) for _ in range(4))
+    fa = O.E5M2 if seed % 3 == 0 else O.E4M3
+    x = seeded_bf16((M, K), seed=2000 + seed)
+    w = seeded_bf16((Nn, K), std=0.02, seed=3000 + seed)
+    sx = O.t_scale(O.t_amax(x, O.SCALE_ROW if rows else O.SCALE_TENSOR), fa)
+    sw = O.t_scale(O.t_amax(w, O.SCALE_ROW if cols else O.SCALE_TENSOR), O.E4M3)
+    xq = O.t_cast(x, sx, fa, O.SCALE_ROW if rows else O.SCALE_TENSOR)
+    wq = O.t_cast(w, sw, O.E4M3, O.SCALE_ROW if cols else O.SCALE_TENSOR)
+    sa_inv, sb_inv = (1 / sx).float().reshape(-1), (1 / sw).float().reshape(-1)
+    bias = torch.randn(Nn, generator=g) * 0.1 if with_bias else None
+    ref32 = O.t_gemm_nt(xq, wq, fa, O.E4M3, sa_inv, sb_inv, want_f32=True)[1]
+    if with_bias:
+        ref32 = ref32 + bias
+    out_dtype = torch.float32 if f32 else torch.bfloat16
+    out = N.gemm_nt(xq.cuda(), wq.cuda(), fa, O.E4M3, sa_inv.cuda(), sb_inv.cuda(), bias=bias.cuda() if with_bias else None,
+                    out_dtype=out_dtype)
+    err = max_rel_err(out, ref32.to(out_dtype))
+    assert err <= (1e-3 if f32 else TOL), f"{M}x{Nn}x{K} rows={rows} cols={cols} bias={with_bias} f32={f32}: {err}"
