@@ -491,3 +491,33 @@ def test_wgrad_reads_dy_as_stored_and_matches_the_transposed_copy_route(amp, mon
     ref = O.linear_fwd_bwd(x, w, dy) if recipe_name == "tensorwise" else None
     if ref is not None:
         assert max_rel_err(results[True][2], ref["dw"]) <= TOL
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_seeded_random_linears_match_the_oracle(amp, seed):
+    """Layer sizes on the grids the kernels distinguish, tokens likewise, bf16 or fp32 master weights, with and
+    without bias, per-tensor or rowwise scaling: forward, dgrad, wgrad and the bias gradient against the oracle."""
+    g = torch.Generator().manual_seed(500 + seed)
+    def draw(grids, hi):
+        step = grids[int(torch.randint(0, len(grids), (1,), generator=g))]
+        return step * int(torch.randint(1, hi // step + 1, (1,), generator=g))
+    M, K, N = draw((16, 128, 256), 1024), draw((16, 128, 256), 1024), draw((16, 128, 256), 1024)
+    if seed % 6 == 5:
+        M = 128 * int(torch.randint(16, 40, (1,), generator=g))          # long token axis: wgrad is cut into K runs
+    rowwise, with_bias, w_f32 = seed % 3 == 2, seed % 2 == 1, seed % 4 >= 2
+    x, w, dy = seeded_bf16((M, K), 1.0, 600 + seed), seeded_bf16((N, K), 0.02, 700 + seed), seeded_bf16((M, N), 1e-3, 800 + seed)
+    bias = seeded_bf16((N,), 0.1, 900 + seed) if with_bias else None
+    recipe = amp.create_fp8_recipe("rowwise" if rowwise else "tensorwise", "hybrid")
+    lin = make_linear(w, bias, dtype=torch.float32 if w_f32 else torch.bfloat16)
+    y, dx, dw = run_step(lin, recipe, x, dy)
+    assert lin.fp8_calls == 1 and y.dtype == torch.bfloat16 and dw.dtype == lin.weight.dtype
+    ref = O.linear_fwd_bwd(x, w, dy, rowwise=rowwise)
+    want_y = ref["y"] if bias is None else (ref["y"].float() + bias.float()).bfloat16()
+    what = f"{M}x{K}->{N} rowwise={rowwise} bias={with_bias} fp32 weights={w_f32}"
+    for name, got, want in (("y", y, want_y), ("dx", dx, ref["dx"]), ("dw", dw, ref["dw"])):
+        err = max_rel_err(got, want)
+        assert err <= TOL, f"{what}: {name} {err}"
+    if with_bias:
+        want_db = dy.float().sum(0)
+        err = (lin.bias.grad.float().cpu() - want_db).abs().max().item() / max(want_db.abs().max().item(), 1e-30)
+        assert err <= (1e-2 if lin.bias.dtype == torch.bfloat16 else 1e-5), f"{what}: db {err}"
