@@ -502,6 +502,133 @@ __global__ __launch_bounds__(kRmsBwdThreads) void norm_bwd_narrow_kernel(const u
     }
 }
 
+// Rows of 513 .. 1024 elements (the model widths 768 and 1024): one WAVE per row and trip, four rows per block in
+// flight, no barrier per row.  Lane l holds the chunks l and 64 + l, i.e. what lane l of waves 0 and 1 of the
+// block-per-row kernel holds (with SETS = 4, rows up to 2048, the kernel needs 300 registers and was measured
+// slower than the block-per-row kernel: not used); the row sums are formed the same way (one butterfly per set of 64 chunks,
+// then ((s0 + s1) + s2) + s3), so dx is the same bits.  d_weight / d_bias: per-lane sums over the rows a wave sees,
+// the block's four waves combined through LDS in wave order, one slab per block.
+template <int SRC, bool LN, int SETS>
+__global__ __launch_bounds__(kRmsBwdThreads) void norm_bwd_wave_kernel(const u32x4 *__restrict__ dy, const void *__restrict__ x,
+                                                                        const float *__restrict__ weight, const float *__restrict__ mean_in,
+                                                                        const float *__restrict__ rstd_in, int64_t rows, int64_t cols,
+                                                                        void *__restrict__ dx, float *__restrict__ slabs) {
+    constexpr int VPC = SRC == ODL_BF16 ? 1 : 2;
+    constexpr int NS = LN ? 2 : 1, NW = kRmsBwdThreads / kWave;
+    __shared__ float part[NS][NW][kWave * 8];
+    const int lane = threadIdx.x % kWave, wv = threadIdx.x / kWave;
+    const int64_t nchunk = cols / 8;
+    float wreg[SETS][8], dw[SETS][8], db[LN ? SETS : 1][8];
+#pragma unroll
+    for (int j = 0; j < SETS; ++j) {
+        const int64_t c = j * kWave + lane;
+        const bool ok = c < nchunk;
+        const float4 w0 = ok ? *reinterpret_cast<const float4 *>(weight + c * 8) : float4{0, 0, 0, 0};
+        const float4 w1 = ok ? *reinterpret_cast<const float4 *>(weight + c * 8 + 4) : float4{0, 0, 0, 0};
+        wreg[j][0] = w0.x; wreg[j][1] = w0.y; wreg[j][2] = w0.z; wreg[j][3] = w0.w;
+        wreg[j][4] = w1.x; wreg[j][5] = w1.y; wreg[j][6] = w1.z; wreg[j][7] = w1.w;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { dw[j][e] = 0.0f; if constexpr (LN) db[j][e] = 0.0f; }
+    }
+    u32x4 nx[SETS][VPC], nd[SETS];
+    auto fetch = [&](int64_t row) {
+#pragma unroll
+        for (int j = 0; j < SETS; ++j) {
+            const int64_t c = j * kWave + lane;
+            const bool in = c < nchunk && row < rows;
+            const u32x4 *p = reinterpret_cast<const u32x4 *>(x) + (row * nchunk + c) * VPC;
+#pragma unroll
+            for (int h = 0; h < VPC; ++h) nx[j][h] = in ? __builtin_nontemporal_load(p + h) : u32x4{0, 0, 0, 0};
+            nd[j] = in ? __builtin_nontemporal_load(dy + row * nchunk + c) : u32x4{0, 0, 0, 0};
+        }
+    };
+    const int64_t stride = (int64_t)gridDim.x * NW;
+    int64_t row = (int64_t)blockIdx.x * NW + wv;
+    fetch(row);
+    for (; row < rows; row += stride) {                       // uniform per wave
+        u32x4 xr[SETS][VPC], dr[SETS];
+#pragma unroll
+        for (int j = 0; j < SETS; ++j) {
+#pragma unroll
+            for (int h = 0; h < VPC; ++h) xr[j][h] = nx[j][h];
+            dr[j] = nd[j];
+        }
+        fetch(row + stride);
+        const float rstd = rstd_in[row];
+        const float mean = LN ? mean_in[row] : 0.0f;
+        float s1[SETS], s2[SETS];
+#pragma unroll
+        for (int j = 0; j < SETS; ++j) {
+            float xf[8], df[8];
+            unpack8<SRC>(xr[j], xf);
+            unpack8<ODL_BF16>(&dr[j], df);
+            float a1 = 0.0f, a2 = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float xh = LN ? __fmul_rn(__fsub_rn(xf[e], mean), rstd) : __fmul_rn(xf[e], rstd);
+                const float t = __fmul_rn(df[e], wreg[j][e]);
+                if constexpr (LN) a1 = __fadd_rn(a1, t);
+                a2 = __fmaf_rn(t, xh, a2);
+                dw[j][e] = __fmaf_rn(df[e], xh, dw[j][e]);
+                if constexpr (LN) db[j][e] = __fadd_rn(db[j][e], df[e]);
+            }
+            s2[j] = wave_sum_butterfly(a2);
+            s1[j] = LN ? wave_sum_butterfly(a1) : 0.0f;
+        }
+        float t2 = s2[0], t1 = s1[0];
+#pragma unroll
+        for (int j = 1; j < 4; ++j) {                         // the block-per-row kernel always adds four wave sums
+            t2 = __fadd_rn(t2, j < SETS ? s2[j] : 0.0f);
+            if constexpr (LN) t1 = __fadd_rn(t1, j < SETS ? s1[j] : 0.0f);
+        }
+        const float c2 = __fdiv_rn(t2, (float)cols), c1 = LN ? __fdiv_rn(t1, (float)cols) : 0.0f;
+#pragma unroll
+        for (int j = 0; j < SETS; ++j) {
+            const int64_t c = j * kWave + lane;
+            if (c < nchunk) {
+                float xf[8], df[8], o[8];
+                unpack8<SRC>(xr[j], xf);
+                unpack8<ODL_BF16>(&dr[j], df);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float xh = LN ? __fmul_rn(__fsub_rn(xf[e], mean), rstd) : __fmul_rn(xf[e], rstd);
+                    const float t = __fmul_rn(df[e], wreg[j][e]);
+                    o[e] = __fmul_rn(rstd, __fmaf_rn(-xh, c2, LN ? __fsub_rn(t, c1) : t));
+                }
+                if constexpr (SRC == ODL_BF16) {
+                    reinterpret_cast<u32x4 *>(dx)[row * nchunk + c] = u32x4{pack2(o[0], o[1]), pack2(o[2], o[3]), pack2(o[4], o[5]), pack2(o[6], o[7])};
+                } else {
+                    float4 *q = reinterpret_cast<float4 *>(dx) + (row * nchunk + c) * 2;
+                    q[0] = float4{o[0], o[1], o[2], o[3]};
+                    q[1] = float4{o[4], o[5], o[6], o[7]};
+                }
+            }
+        }
+    }
+    // one set of 64 chunks at a time through LDS: the four waves' sums of a column are added in wave order
+    float *slab = slabs + (int64_t)blockIdx.x * NS * cols;
+#pragma unroll
+    for (int j = 0; j < SETS; ++j) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            part[0][wv][lane * 8 + e] = dw[j][e];
+            if constexpr (LN) part[1][wv][lane * 8 + e] = db[j][e];
+        }
+        __syncthreads();
+        for (int i = threadIdx.x; i < NS * kWave * 8; i += kRmsBwdThreads) {
+            const int set = i / (kWave * 8), cc = i % (kWave * 8);
+            const int64_t col = (int64_t)j * kWave * 8 + cc;
+            if (col < cols) {
+                float acc = part[set][0][cc];
+#pragma unroll
+                for (int w = 1; w < NW; ++w) acc = __fadd_rn(acc, part[set][w][cc]);
+                slab[set * cols + col] = acc;
+            }
+        }
+        __syncthreads();
+    }
+}
+
 // ------------------------------------------------------------------------ LayerNorm
 // Same work split and summation order as the RMSNorm kernels.  Forward, per row:
 //   mean = sum(x) / cols;  d = x - mean;  rstd = 1 / sqrt(sum(d * d) / cols + eps)   (d * d by fma)
@@ -863,6 +990,18 @@ extern "C" int odl_fp8_rmsnorm_bwd(const void *dy, const void *x, int src_dtype,
         hipLaunchKernelGGL(rmsnorm_bwd_reduce_kernel, dim3((unsigned)((cols + 63) / 64)), dim3(1024), 0, stream, workspace, (int)g, cols, dweight);
         return check_launch("odl_fp8_rmsnorm_bwd");
     }
+    if (cols <= 1024) {                                       // a wave per row, four rows per block in flight
+        const int64_t rpb = kRmsBwdThreads / kWave;
+        g = (rows + rpb - 1) / rpb;
+        g = g < 1 ? 1 : (g < ODL_FP8_RMSNORM_BWD_SLABS ? g : ODL_FP8_RMSNORM_BWD_SLABS);
+#define ODL_RMSW(SRC, SETS) hipLaunchKernelGGL((norm_bwd_wave_kernel<SRC, false, SETS>), dim3((unsigned)g), dim3(kRmsBwdThreads), 0, stream, reinterpret_cast<const u32x4 *>(dy), x, weight, (const float *)nullptr, rstd, rows, cols, dx, workspace)
+#define ODL_RMSW_SRC(SETS) do { if (src_dtype == ODL_BF16) ODL_RMSW(ODL_BF16, SETS); else ODL_RMSW(ODL_F32, SETS); } while (0)
+        ODL_RMSW_SRC(2);
+#undef ODL_RMSW_SRC
+#undef ODL_RMSW
+        hipLaunchKernelGGL(rmsnorm_bwd_reduce_kernel, dim3((unsigned)((cols + 63) / 64)), dim3(1024), 0, stream, workspace, (int)g, cols, dweight);
+        return check_launch("odl_fp8_rmsnorm_bwd");
+    }
     const int64_t cplw = (cols / 8 + kRmsBwdThreads - 1) / kRmsBwdThreads;
 #define ODL_RMSB(SRC, CPLW) hipLaunchKernelGGL((norm_bwd_kernel<SRC, false, CPLW>), dim3((unsigned)g), dim3(kRmsBwdThreads), 0, stream, reinterpret_cast<const u32x4 *>(dy), x, weight, (const float *)nullptr, rstd, rows, cols, dx, workspace)
 #define ODL_RMSB_SRC(CPLW) do { if (src_dtype == ODL_BF16) ODL_RMSB(ODL_BF16, CPLW); else ODL_RMSB(ODL_F32, CPLW); } while (0)
@@ -944,6 +1083,18 @@ extern "C" int odl_fp8_layernorm_bwd(const void *dy, const void *x, int src_dtyp
         else ODL_LNN_SRC(64);
 #undef ODL_LNN_SRC
 #undef ODL_LNN
+        hipLaunchKernelGGL(rmsnorm_bwd_reduce_kernel, dim3((unsigned)((2 * cols + 63) / 64)), dim3(1024), 0, stream, workspace, (int)g, 2 * cols, dweight);
+        return check_launch("odl_fp8_layernorm_bwd");
+    }
+    if (cols <= 1024) {                                       // a wave per row, four rows per block in flight
+        const int64_t rpb = kRmsBwdThreads / kWave;
+        g = (rows + rpb - 1) / rpb;
+        g = g < 1 ? 1 : (g < ODL_FP8_RMSNORM_BWD_SLABS ? g : ODL_FP8_RMSNORM_BWD_SLABS);
+#define ODL_LNW(SRC, SETS) hipLaunchKernelGGL((norm_bwd_wave_kernel<SRC, true, SETS>), dim3((unsigned)g), dim3(kRmsBwdThreads), 0, stream, reinterpret_cast<const u32x4 *>(dy), x, weight, mean, rstd, rows, cols, dx, workspace)
+#define ODL_LNW_SRC(SETS) do { if (src_dtype == ODL_BF16) ODL_LNW(ODL_BF16, SETS); else ODL_LNW(ODL_F32, SETS); } while (0)
+        ODL_LNW_SRC(2);
+#undef ODL_LNW_SRC
+#undef ODL_LNW
         hipLaunchKernelGGL(rmsnorm_bwd_reduce_kernel, dim3((unsigned)((2 * cols + 63) / 64)), dim3(1024), 0, stream, workspace, (int)g, 2 * cols, dweight);
         return check_launch("odl_fp8_layernorm_bwd");
     }
