@@ -234,6 +234,7 @@ class FP8Recipe:
             native.delayed_update_raw(arena.history, arena.H, arena.capacity, R, arena.scale, arena.scale_inv,
                                       arena.fmt, self.margin, algo)
             arena.dirty = False
+            arena.epoch += 1
 
     def state_dict(self) -> dict:
         """Scaling state (histories and scales) of every role registered so far,
@@ -256,6 +257,7 @@ class FP8Recipe:
                 arena.history[:, :n].copy_(blob["history"][:, :n])
                 arena.scale[:n].copy_(blob["scale"][:n])
                 arena.scale_inv[:n].copy_(blob["scale_inv"][:n])
+                arena.invalidate_snapshot()
 
     # ------------------------------------------------------- producer hand-over
     @staticmethod

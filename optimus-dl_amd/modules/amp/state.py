@@ -81,6 +81,12 @@ class ScalingMeta:
     def scale_inv_of(self, role: int) -> torch.Tensor:
         return self.arena.scale_inv[self.first + role:self.first + role + 1]
 
+    def scale_inv_snapshot_of(self, role: int) -> torch.Tensor:
+        """The inverse scale in force now, in storage that the next refresh does not touch (what a
+        GEMM of this step, or its backward after the refresh, has to multiply by)."""
+        snap = self.arena.snapshot_inv()
+        return snap[self.first + role:self.first + role + 1]
+
 
 class MetaArena:
     """history [H, cap], scale [cap], scale_inv [cap], fmt [cap] for one direction."""
@@ -93,6 +99,20 @@ class MetaArena:
         self.fmt = torch.zeros(capacity, dtype=torch.int32, device=device)
         self.used = 0
         self.dirty = False         # some cast wrote an amax since the last update
+        self.epoch = 0             # bumped by every refresh of scale / scale_inv (they are updated in place)
+        self._snap: torch.Tensor | None = None
+        self._snap_epoch = -1
+
+    def snapshot_inv(self) -> torch.Tensor:
+        """A copy of ``scale_inv`` made once per epoch: one small copy per arena and step instead of one per
+        cast.  A copy of an earlier epoch lives on for as long as a saved tensor of that step refers to it."""
+        if self._snap is None or self._snap_epoch != self.epoch:
+            self._snap = self.scale_inv.clone()
+            self._snap_epoch = self.epoch
+        return self._snap
+
+    def invalidate_snapshot(self) -> None:
+        self._snap = None
 
     def reserve(self, fmts: list[int]) -> ScalingMeta | None:
         n = len(fmts)

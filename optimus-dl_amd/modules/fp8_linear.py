@@ -119,8 +119,8 @@ def _quantise_delayed(x2d: torch.Tensor, fmt: int, meta: "_state.ScalingMeta", r
     """Delayed scaling: one pass with the scale from the history, amax recorded in row 0."""
     scale, slot = meta.scale_of(role), meta.amax_slot(role)
     meta.arena.dirty = True
-    # the inverse scale is snapshotted: the arena entry changes at the next update
-    scale_inv = meta.scale_inv_of(role).clone()
+    # the inverse scale comes from the arena's per-step snapshot: the arena entry itself changes at the next update
+    scale_inv = meta.scale_inv_snapshot_of(role)
     if need_t:
         q, q_t = native.cast_transpose(x2d, scale, fmt, T, amax_out=slot, want_rowmajor=need_rowmajor)
     else:
@@ -243,7 +243,11 @@ class _Fp8LinearFn(torch.autograd.Function):
         if ctx.need_wgrad and not recipe.wgrad:
             dw = (dy2d.t().to(saved["x_hp"].dtype) @ saved["x_hp"]).to(ctx.w_dtype)
         if ctx.has_bias and db is None:
-            db = dy2d.sum(dim=0, dtype=torch.float32).to(ctx.bias_dtype)
+            if dy2d.is_cuda and native.colsum_supported(dy2d):
+                # delayed and rowwise scaling have no amax pass to ride on: the same kernel, for its column sums only
+                db = native.amax_parts_colsum(dy2d)[1].to(ctx.bias_dtype)
+            else:
+                db = dy2d.sum(dim=0, dtype=torch.float32).to(ctx.bias_dtype)
         return dx, dw, db, None, None, None
 
 
