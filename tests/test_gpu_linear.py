@@ -395,6 +395,61 @@ def test_forward_backward_can_be_captured_in_a_graph_and_replayed(amp):
             assert torch.equal(a, b), f"replay {rep}: {name} differs from eager"
 
 
+def test_delayed_scaling_step_replays_from_a_graph_like_the_eager_twin(amp):
+    """Delayed scaling keeps state between steps (histories, scales): they are refreshed in place, so a captured step
+    carries them forward from replay to replay.  A twin layer runs the same steps eagerly; every replay must give the
+    twin's bits, and the scaling state must be the same afterwards."""
+    M, K, N = 256, 512, 384
+    w = seeded_bf16((N, K), 0.02, 190)
+    setups = []
+    for _ in range(2):
+        recipe = amp.create_fp8_recipe("delayed", "hybrid", amax_history_len=4)
+        lin = make_linear(w)
+        x_s = torch.zeros((M, K), dtype=torch.bfloat16, device="cuda", requires_grad=True)
+        dy_s = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+        setups.append((recipe, lin, x_s, dy_s))
+
+    def fwd_bwd(recipe, lin, x_s, dy_s):
+        lin._wcache.key = None
+        with recipe.autocast():
+            y = lin(x_s)
+        with recipe.backward():
+            gx, gw = torch.autograd.grad(y, (x_s, lin.weight), dy_s)
+        return y, gx, gw
+
+    def feed(step):
+        x_new, dy_new = seeded_bf16((M, K), 1.0 + step, 191 + step).cuda(), seeded_bf16((M, N), 1e-3 * (step + 1), 195 + step).cuda()
+        with torch.no_grad():
+            for _, _, x_s, dy_s in setups:
+                x_s.copy_(x_new)
+                dy_s.copy_(dy_new)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):                       # two real steps each, off the default stream
+        for step in range(2):
+            feed(step)
+            for s_ in setups:
+                fwd_bwd(*s_)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs_g = fwd_bwd(*setups[0])
+    for step in range(2, 6):                            # more replays than the history is long
+        feed(step)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in outs_g]
+        want = fwd_bwd(*setups[1])
+        torch.cuda.synchronize()
+        for name, a, b in zip(("y", "dx", "dw"), got, want):
+            assert torch.equal(a, b), f"step {step}: {name} from the replay differs from the eager twin"
+    for direction in ("scaling_fwd", "scaling_bwd"):
+        ma, mb = setups[0][1].fp8_meta[direction], setups[1][1].fp8_meta[direction]
+        assert torch.equal(ma.scale, mb.scale) and torch.equal(ma.amax_history, mb.amax_history)
+        assert ma.scale[0] != 1.0                       # the scales did move (the reserved output roles keep 1.0)
+
+
 @pytest.mark.parametrize("recipe_name,fmt,margin", [("tensorwise", "e5m2", 0), ("tensorwise", "hybrid", 2), ("rowwise", "e4m3", 1)])
 def test_other_formats_and_margins_match_the_oracle(amp, recipe_name, fmt, margin):
     """Pure E5M2 (allowed for current scaling), a margin (scales divided by 2^margin) and rowwise E4M3 gradients."""
