@@ -1,8 +1,5 @@
 """Shared helpers for the GPU parity tests."""
-import numpy as np
 import torch
-
-from oracle import oracle as O
 
 
 def seeded_bf16(shape, std=1.0, seed=0):

@@ -4,7 +4,6 @@ GEMM outputs: max|out-ref|/max|ref| <= 1e-2 (bf16 out).  Scales and histories:
 bit-exact.  The module is driven exactly as a training loop drives it: through
 the FP8Recipe contexts.
 """
-import numpy as np
 import pytest
 import torch
 import torch.nn as nn
