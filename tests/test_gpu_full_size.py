@@ -364,3 +364,23 @@ def test_fp32_weight_gradient_at_the_baseline_shape(N):
     out16 = N.gemm_layouts(aq_t, bq, O.E5M2, O.E4M3, N.K_SLOW, N.K_FAST, sa_inv, sb_inv)
     assert out32.dtype == torch.float32 and torch.equal(out32.bfloat16(), out16)
     sample_check(out32, aq, bq, O.E5M2, O.E4M3, sa_inv, sb_inv, seed=7, what="fp32 wgrad 14336x4096x8192")
+
+
+@pytest.mark.parametrize("M,Nn,K,kernel", [pytest.param(16384, 1024, 151936, "tiled", id="2.5GB-operand"),
+                                           pytest.param(32768, 256, 151936, "generic", id="5GB-operand")])
+def test_operands_beyond_the_32_bit_offset_limits(N, M, Nn, K, kernel):
+    """The input gradient of a vocabulary-sized head at many tokens: dY codes of 2.5 GB (beyond the 2 GiB that the
+    streaming and the pipelined kernel address: the tiled kernels take it) and of 5 GB (beyond 4 GiB: only the generic
+    kernel, with 64-bit addressing, does).  The automatic choice must pick a kernel that can address the operand; a
+    sample of the output against the oracle, the last rows included (highest addresses)."""
+    g = torch.Generator(device="cuda").manual_seed(M + K)
+    aq = torch.randint(0, 256, (M, K), generator=g, device="cuda", dtype=torch.uint8)
+    aq[(aq & 0x7F) > 0x7B] = 0                          # no E5M2 Inf / NaN codes
+    bq = torch.randint(0, 256, (Nn, K), generator=g, device="cuda", dtype=torch.uint8)
+    bq[(bq & 0x7F) == 0x7F] = 0                         # no E4M3 NaN codes
+    sa_inv, sb_inv = torch.tensor([2.0 ** -12], device="cuda"), torch.tensor([2.0 ** -6], device="cuda")
+    assert N.gemm_split_count(M, Nn, K) == 1            # the K split rides on the streaming kernel: not for these
+    out = N.gemm_nt(aq, bq, O.E5M2, O.E4M3, sa_inv, sb_inv)
+    sample_check(out, aq, bq, O.E5M2, O.E4M3, sa_inv, sb_inv, seed=K, what=f"{kernel} kernel, {M}x{Nn}x{K}", rows=24, cols=128)
+    tail = out[M - 64:].contiguous()
+    sample_check(tail, aq[M - 64:], bq, O.E5M2, O.E4M3, sa_inv, sb_inv, seed=K + 1, what=f"{kernel} kernel, last rows", rows=16, cols=128)
