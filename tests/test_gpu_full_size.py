@@ -384,3 +384,21 @@ def test_operands_beyond_the_32_bit_offset_limits(N, M, Nn, K, kernel):
     sample_check(out, aq, bq, O.E5M2, O.E4M3, sa_inv, sb_inv, seed=K, what=f"{kernel} kernel, {M}x{Nn}x{K}", rows=24, cols=128)
     tail = out[M - 64:].contiguous()
     sample_check(tail, aq[M - 64:], bq, O.E5M2, O.E4M3, sa_inv, sb_inv, seed=K + 1, what=f"{kernel} kernel, last rows", rows=16, cols=128)
+
+
+def test_quantisation_of_a_tensor_with_more_than_2_31_elements(N):
+    """The logits gradient of a vocabulary-sized head at 16384 tokens: 2.49e9 elements (5 GB of bf16).  amax, cast and
+    cast+transpose index with 64 bits: the maximum planted in the last row is found, rows from both ends of the tensor
+    have the oracle's codes, and the transposed copy is the transpose."""
+    M, V = 16384, 151936
+    x = draw((M, V), 1e-3, 77)
+    x[M - 1, V - 3] = -0.75                             # the maximum sits behind element 2^31
+    parts = N.amax_parts(x)
+    q, q_t, amax, scale, _ = N.cast_dynamic(x, parts, O.E5M2, 0, want_rowmajor=True, want_transposed=True)
+    assert amax.item() == 0.75 and scale.item() == O.t_scale(torch.tensor([0.75]), O.E5M2).item()
+    rows = torch.tensor([0, 1, 8191, 8192, M - 2, M - 1])
+    want = O.t_cast(x[rows.cuda()].cpu(), scale.cpu(), O.E5M2)
+    assert_bytes_equal(q[rows.cuda()], want, "codes of rows from both ends")
+    assert_bytes_equal(q_t[:, rows.cuda()], want.t(), "the same rows in the transposed copy")
+    cols = torch.tensor([0, 77, V - 1]).cuda()
+    assert torch.equal(q_t[cols], q[:, cols].t())
