@@ -347,3 +347,16 @@ def test_gelu_shapes_and_parts(N, shape):
     assert_f32_bits_equal(parts_max(parts).reshape(1), wdx.float().abs().max().reshape(1), "gelu bwd parts")
     with pytest.raises(N.NativeError, match="multiple of 8"):
         N.gelu_amax_parts(torch.zeros((3, 5), dtype=torch.bfloat16).cuda())
+
+
+def test_producers_take_empty_inputs(N):
+    """Zero rows: empty outputs, all-zero partial maxima, zero weight / bias gradients, no launch fault."""
+    e = torch.empty((0, 64), dtype=torch.bfloat16, device="cuda")
+    w = torch.ones(64, device="cuda")
+    none = torch.empty(0, device="cuda")
+    for out in (N.swiglu_amax_parts(e, e), N.swiglu_bwd_amax_parts(e, e, e), N.rmsnorm_amax_parts(e, w, 1e-5),
+                N.rmsnorm_bwd(e, e, w, none), N.layernorm_amax_parts(e, w, None, 1e-5), N.layernorm_bwd(e, e, w, none, none),
+                N.gelu_amax_parts(e), N.gelu_bwd_amax_parts(e, e)):
+        torch.cuda.synchronize()
+        for t in out if isinstance(out, tuple) else (out,):
+            assert t.numel() == 0 or float(t.abs().max()) == 0.0
