@@ -62,7 +62,35 @@ def swiglu(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     return _SwiGLUFn.apply(gate, up, recipe)
 
 
-class _FusedSwiGLUForward:
+# ---------------------------------------------------------------- in-place re-classing
+# A module is fused by giving it a subclass of its own class with the fused forward mixed in: same object, same
+# parameters, same state-dict keys, isinstance() checks keep working.  The subclass is made on the fly, so pickling
+# it by name would find the original class instead: the mixins carry a __reduce_ex__ that rebuilds the subclass
+# from (original class, mixin) -- copy.deepcopy (EMA copies of a model) and torch.save of a whole module both work.
+_RECLASSED: dict[tuple[type, type], type] = {}
+
+
+def _fused_class(base: type, mixin: type) -> type:
+    key = (base, mixin)
+    cls = _RECLASSED.get(key)
+    if cls is None:
+        cls = type(base.__name__, (mixin, base), {"__module__": base.__module__})
+        _RECLASSED[key] = cls
+    return cls
+
+
+def _rebuild_fused(base: type, mixin: type):
+    cls = _fused_class(base, mixin)
+    return cls.__new__(cls)
+
+
+class _Reclassed:
+    def __reduce_ex__(self, protocol):
+        mro = type(self).__mro__                      # (made-up subclass, mixin, _Reclassed, original class, ...)
+        return _rebuild_fused, (mro[mro.index(_Reclassed) + 1], mro[1]), self.__dict__
+
+
+class _FusedSwiGLUForward(_Reclassed):
     """Mixed into the class of an MLP with ``w1`` (gate), ``w2`` (up) and ``c_proj`` (down)."""
 
     _odl_fused_swiglu = True
@@ -81,7 +109,7 @@ def fuse_swiglu_mlp(mlp: nn.Module) -> bool:
     if not all(isinstance(getattr(mlp, n, None), FP8Linear) for n in ("w1", "w2", "c_proj")):
         return False
     cls = mlp.__class__
-    mlp.__class__ = type(cls.__name__, (_FusedSwiGLUForward, cls), {"__module__": cls.__module__})
+    mlp.__class__ = _fused_class(cls, _FusedSwiGLUForward)
     return True
 
 
@@ -119,7 +147,7 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor |
     return _RMSNormFn.apply(x, weight, float(eps), recipe)
 
 
-class _FusedRMSNormForward:
+class _FusedRMSNormForward(_Reclassed):
     """Mixed into the class of an RMSNorm with ``weight`` and ``eps`` (layer_norms.py:64-67).
 
     Under an FP8 recipe the output is bf16 whatever the input dtype: the recipe's context nests
@@ -140,7 +168,7 @@ def fuse_rmsnorm(norm: nn.Module) -> bool:
     if not isinstance(w, torch.Tensor) or w.dim() != 1 or not hasattr(norm, "eps"):
         return False
     cls = norm.__class__
-    norm.__class__ = type(cls.__name__, (_FusedRMSNormForward, cls), {"__module__": cls.__module__})
+    norm.__class__ = _fused_class(cls, _FusedRMSNormForward)
     return True
 
 
@@ -180,7 +208,7 @@ def layernorm(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, 
     return _LayerNormFn.apply(x, weight, bias, float(eps), recipe)
 
 
-class _FusedLayerNormForward:
+class _FusedLayerNormForward(_Reclassed):
     """Mixed into the class of a LayerNorm over the last axis: ``torch.nn.LayerNorm`` (``normalized_shape``
     of one dimension, affine) or the reference's bias-optional one (layer_norms.py:21-47, eps 1e-5).
     Output dtype under an FP8 recipe: as for the fused RMSNorm."""
@@ -202,7 +230,7 @@ def fuse_layernorm(norm: nn.Module) -> bool:
     if shape is not None and tuple(shape) != (w.numel(),):
         return False
     cls = norm.__class__
-    norm.__class__ = type(cls.__name__, (_FusedLayerNormForward, cls), {"__module__": cls.__module__})
+    norm.__class__ = _fused_class(cls, _FusedLayerNormForward)
     return True
 
 
@@ -237,7 +265,7 @@ def gelu(x: torch.Tensor) -> torch.Tensor | None:
     return _GeluFn.apply(x, recipe)
 
 
-class _FusedGeluForward:
+class _FusedGeluForward(_Reclassed):
     """Mixed into the class of an ``nn.GELU`` with the exact (erf) form, the activation of the
     reference's GELUMLP (mlp.py:141-157)."""
 
@@ -252,5 +280,5 @@ def fuse_gelu(act: nn.Module) -> bool:
     if getattr(act, "_odl_fused_gelu", False) or not isinstance(act, nn.GELU) or getattr(act, "approximate", "none") != "none":
         return False
     cls = act.__class__
-    act.__class__ = type(cls.__name__, (_FusedGeluForward, cls), {"__module__": cls.__module__})
+    act.__class__ = _fused_class(cls, _FusedGeluForward)
     return True

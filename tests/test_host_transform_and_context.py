@@ -311,3 +311,30 @@ def test_producer_parts_hand_over(monkeypatch):
     d = A.FP8Recipe(recipe_type="delayed")
     d.offer_parts(x, parts)
     assert d.producer_parts == []                                     # only current scaling reads an amax per tensor
+
+
+def test_converted_and_fused_modules_survive_deepcopy_and_pickling():
+    """An EMA copy (copy.deepcopy) and torch.save of a whole module: the FP8 Linears and the modules re-classed in
+    place for the fused forwards come back as the same types with the same state-dict keys and the same outputs."""
+    import copy
+    import io
+
+    from optimus_dl_amd.modules.fp8_linear import FP8Linear
+    from optimus_dl_amd.modules.model.blocks import GPT2Block, LlamaBlock
+    from optimus_dl_amd.modules.model_transforms import build_model_transform
+
+    for blk in (LlamaBlock(64, 4, 2, 128), GPT2Block(64, 4)):
+        build_model_transform({"_name": "transformer_engine"}).apply(blk)
+        x = torch.randn(2, 8, 64)
+        want = blk(x)
+        buf = io.BytesIO()
+        torch.save(blk, buf)
+        buf.seek(0)
+        for other in (copy.deepcopy(blk), torch.load(buf, weights_only=False)):
+            assert type(other.ln_1) is type(blk.ln_1) and type(other.mlp) is type(blk.mlp)
+            assert all(isinstance(m, FP8Linear) for m in other.modules() if isinstance(m, torch.nn.Linear))
+            assert list(other.state_dict().keys()) == list(blk.state_dict().keys())
+            assert torch.equal(other(x), want)
+            again = build_model_transform({"_name": "transformer_engine"})
+            again.apply(other)                                  # already converted: nothing left to do
+            assert not any(again.last_replacements.values())
