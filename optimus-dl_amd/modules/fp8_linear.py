@@ -267,6 +267,20 @@ class FP8Linear(nn.Linear):
         self.fp8_meta: dict[str, "_state.ScalingMeta"] = {}
         self.fp8_calls = 0                   # forwards that actually took the FP8 path (for tests / logging)
 
+    # Quantised weights and scaling-state views are per-process run-time state: a copy or a pickle of the module
+    # starts without them (they are rebuilt on first use) instead of dragging device buffers and arenas along.
+    _RUNTIME_STATE = ("_wcache", "_wcache_rowwise", "_metas", "fp8_meta", "fp8_calls")
+
+    def __getstate__(self) -> dict:
+        state = self.__dict__.copy()
+        for name in self._RUNTIME_STATE:
+            state.pop(name, None)
+        return state
+
+    def __setstate__(self, state: dict) -> None:
+        super().__setstate__(state)
+        self._init_fp8_state()
+
     @classmethod
     def from_linear(cls, linear: nn.Linear, **kwargs: Any) -> "FP8Linear":
         """Re-wrap an existing layer, SHARING its Parameter objects."""
