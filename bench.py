@@ -121,19 +121,32 @@ def standalone_hbm(torch, native, iters=24):
     buffers per shape are walked round-robin to hold three times the 256 MB memory-side cache;
     HIP events around the whole batch, so launch gaps are included.  Algorithmic bytes as in the step."""
     out = {}
-    for rows, cols in ((M_TOKENS, 4096), (14336, 4096), (M_TOKENS, 14336)):
+    # the last three shapes: norm rows of the small presets (per-head q / k norm of Qwen3, GPT-2 and Qwen3 model widths)
+    for rows, cols in ((M_TOKENS, 4096), (14336, 4096), (M_TOKENS, 14336), (131072, 128), (16384, 768), (8192, 1024)):
         nbuf = max(4, -(-3 * 256 * 2**20 // (2 * rows * cols)))
         xs = [torch.randn((rows, cols), device="cuda", dtype=torch.bfloat16) for _ in range(nbuf)]
         _, scale, _ = native.amax_scale(xs[0], native.E4M3, 0)
         E = rows * cols
-        kernels = {
-            "amax": (lambda x: native.amax_parts(x), 2 * E),
-            "amax_rowwise": (lambda x: native.amax(x, native.SCALE_ROW), 2 * E + 4 * rows),
-            "amax_and_column_sums": (lambda x: native.amax_parts_colsum(x), 2 * E + 4 * cols),
-            "cast": (lambda x: native.cast(x, scale, native.E4M3, native.SCALE_TENSOR), 3 * E),
-            "cast_transpose": (lambda x: native.cast_transpose(x, scale, native.E4M3, native.SCALE_TENSOR), 4 * E),
-            "amax_then_cast_transpose": (lambda x: native.quantize_dynamic(x, native.E4M3, 0), 6 * E),
-        }
+        if cols < 4096:
+            w_norm = torch.ones(cols, device="cuda")
+            _, rstd_b, _ = native.rmsnorm_amax_parts(xs[0], w_norm, 1e-5)
+            _, mean_l, rstd_l, _ = native.layernorm_amax_parts(xs[0], w_norm, w_norm, 1e-5)
+            dy_of = {id(x): xs[(i + 1) % nbuf] for i, x in enumerate(xs)}
+            kernels = {
+                "rmsnorm_amax_bf16_in": (lambda x: native.rmsnorm_amax_parts(x, w_norm, 1e-5), 4 * E),
+                "rmsnorm_bwd_bf16": (lambda x: native.rmsnorm_bwd(dy_of[id(x)], x, w_norm, rstd_b), 6 * E),
+                "layernorm_amax_bf16_in": (lambda x: native.layernorm_amax_parts(x, w_norm, w_norm, 1e-5), 4 * E),
+                "layernorm_bwd_bf16": (lambda x: native.layernorm_bwd(dy_of[id(x)], x, w_norm, mean_l, rstd_l), 6 * E),
+            }
+        else:
+            kernels = {
+                "amax": (lambda x: native.amax_parts(x), 2 * E),
+                "amax_rowwise": (lambda x: native.amax(x, native.SCALE_ROW), 2 * E + 4 * rows),
+                "amax_and_column_sums": (lambda x: native.amax_parts_colsum(x), 2 * E + 4 * cols),
+                "cast": (lambda x: native.cast(x, scale, native.E4M3, native.SCALE_TENSOR), 3 * E),
+                "cast_transpose": (lambda x: native.cast_transpose(x, scale, native.E4M3, native.SCALE_TENSOR), 4 * E),
+                "amax_then_cast_transpose": (lambda x: native.quantize_dynamic(x, native.E4M3, 0), 6 * E),
+            }
         if cols == D_FF:                   # the SwiGLU producers run on the [tokens, d_ff] activations
             nxt = {id(x): (xs[(i + 1) % nbuf], xs[(i + 2) % nbuf]) for i, x in enumerate(xs)}
             kernels["swiglu_fwd_amax"] = (lambda x: native.swiglu_amax_parts(x, nxt[id(x)][0]), 6 * E)
