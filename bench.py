@@ -421,7 +421,6 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU leg (for profiler runs)")
-    ap.add_argument("--gemm-variant", type=int, default=-1)
     ap.add_argument("--no-standalone", action="store_true",
                     help="skip the stand-alone measurements of the memory-bound kernels (keeps profiler traces to the steps)")
     ap.add_argument("--standalone-only", action="store_true",
@@ -453,7 +452,6 @@ def main() -> int:
         print(json.dumps({"whole_models_fwd_bwd": whole_models(torch, which=(args.whole_models_only,), steps=args.steps,
                                                                    labels=("fp8_linears_fused_producers",))}))
         return 0
-    native.gemm_set_variant(args.gemm_variant)
     dev = "cuda"
     data = make_inputs(torch, device=dev)
     recipe = create_fp8_recipe("tensorwise", "hybrid")
@@ -535,7 +533,7 @@ def main() -> int:
                         "M=8192, FP8 fwd+bwd, per-tensor dynamic scaling, fused cast+transpose of x and w, dY read by wgrad as stored",
             "flop_per_step": step_flops(),
             "gemms_per_step": 9,
-            "gemm_variant": native.gemm_variants()[args.gemm_variant] if args.gemm_variant >= 0 else "auto",
+            "gemm_variant": "auto",
         },
         "frac_of_fp8_peak": tflops / PEAK_FP8_TFLOPS,
         "gemm_only_tflops": gemm_tflops,

@@ -45,7 +45,7 @@ enum odl_status {
     ODL_ERR_LAUNCH = 3    /* HIP reported an error at launch */
 };
 
-/* ABI version of this header (6); bumped when a signature changes or an entry point is added. */
+/* ABI version of this header (7); bumped when a signature changes or an entry point is added. */
 int odl_fp8_abi_version(void);
 
 /* Last error message of the calling host thread ("" if none). */
@@ -319,9 +319,12 @@ int odl_fp8_delayed_update(float *history, int64_t H, int64_t R, int64_t ld,
                            int margin, int algo, odl_stream_t stream);
 
 /*
- * Tuning / introspection (host only).  Selects the GEMM kernel variant:
- * -1 = automatic choice by shape; otherwise an index < odl_fp8_gemm_num_variants().
- * odl_fp8_gemm_variant_name returns a short description ("256x256x128 w4 s2").
+ * Testing / tuning / introspection (host only).  odl_fp8_gemm_set_variant pins the GEMM kernel variant
+ * for calls made from the CALLING HOST THREAD only (thread-local, like odl_fp8_last_error): -1 =
+ * automatic choice by shape (the state every thread starts in); otherwise an index <
+ * odl_fp8_gemm_num_variants().  It exists for tests that cross-check the kernels against each other
+ * and for tuning sweeps; production callers never call it, and nothing else in the library is
+ * mutable process state.  odl_fp8_gemm_variant_name returns a short description ("256x256x128 w4 s2").
  */
 int odl_fp8_gemm_num_variants(void);
 const char *odl_fp8_gemm_variant_name(int variant);

@@ -22,8 +22,25 @@ int check_launch(const char *what) {
     return set_error(ODL_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
 }
 
+// Compute units of the device that is current on the calling thread.  One slot per device ordinal: a
+// process that drives several GPUs sizes every grid for the GPU it launches on.  The slots are plain
+// ints: two threads that fill one at the same time write the same value.
+int device_cu_count() {
+    constexpr int kMaxDevices = 64;
+    static int cached[kMaxDevices] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) dev = 0;
+    int cus = cached[dev];
+    if (cus == 0) {
+        hipDeviceProp_t prop;
+        cus = hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+        cached[dev] = cus;
+    }
+    return cus;
+}
+
 }  // namespace odl
 
-extern "C" int odl_fp8_abi_version(void) { return 6; }
+extern "C" int odl_fp8_abi_version(void) { return 7; }
 
 extern "C" const char *odl_fp8_last_error(void) { return odl::g_err; }

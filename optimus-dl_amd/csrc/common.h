@@ -18,6 +18,7 @@ typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
 
 int set_error(int code, const char *fmt, ...);   // defined in api.hip
 int check_launch(const char *what);              // hipGetLastError -> status
+int device_cu_count();                           // compute units of the CURRENT device (cached per device, api.hip)
 
 __device__ __forceinline__ float bits_to_float(uint32_t u) { return __builtin_bit_cast(float, u); }
 __device__ __forceinline__ uint32_t float_to_bits(float f) { return __builtin_bit_cast(uint32_t, f); }

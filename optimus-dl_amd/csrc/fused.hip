@@ -878,15 +878,8 @@ static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t
 
 // at most two fat blocks per CU, and never more blocks than there are partial maxima
 static int grid_cap() {
-    static int cap = 0;
-    if (cap == 0) {
-        int dev = 0, cus = 256;
-        hipDeviceProp_t prop;
-        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0)
-            cus = prop.multiProcessorCount;
-        cap = cus * 2 < kParts ? cus * 2 : kParts;
-    }
-    return cap;
+    const int cus = device_cu_count();
+    return cus * 2 < kParts ? cus * 2 : kParts;
 }
 
 }  // namespace odl

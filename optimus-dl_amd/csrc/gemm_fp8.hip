@@ -90,7 +90,9 @@ static const Variant kVariants[] = {
 };
 constexpr int kPipeVariant = 5, kPipeOneTileVariant = 6, kStreamVariant = 7;
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
-static int g_forced_variant = -1;
+// Forced kernel variant of the calling host thread (-1: choose by shape).  Thread-local: a test or a tuning
+// sweep that pins a variant cannot change the kernels another thread (e.g. the autograd worker) launches.
+static thread_local int t_forced_variant = -1;
 
 template <int FA, int FB>
 static void launch_generic_fmt(const GemmArgs &g, hipStream_t stream) {
@@ -104,16 +106,7 @@ static void launch_gemm_generic(int fa, int fb, const GemmArgs &g, hipStream_t s
     else launch_generic_fmt<ODL_FP8_E5M2, ODL_FP8_E5M2>(g, stream);
 }
 
-static int cu_count() {
-    static int cus = 0;
-    if (cus == 0) {
-        int dev = 0;
-        hipDeviceProp_t prop;
-        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) cus = prop.multiProcessorCount;
-        if (cus <= 0) cus = 256;
-    }
-    return cus;
-}
+static int cu_count() { return device_cu_count(); }
 
 static int choose_variant(int64_t M, int64_t N, bool stream_ok) {
     const int cus = cu_count();
@@ -149,7 +142,7 @@ extern "C" const char *odl_fp8_gemm_variant_name(int variant) {
 
 extern "C" int odl_fp8_gemm_set_variant(int variant) {
     if (variant < -1 || variant >= kNumVariants) return set_error(ODL_ERR_ARG, "odl_fp8_gemm_set_variant: %d out of range", variant);
-    g_forced_variant = variant;
+    t_forced_variant = variant;
     return ODL_OK;
 }
 
@@ -178,7 +171,7 @@ extern "C" int odl_fp8_gemm_nt(const uint8_t *a, const uint8_t *b, int64_t M, in
     // the pipelined and the streaming kernel address rows with 32-bit byte offsets
     const bool lim32 = (double)(M + 256) * (double)K < 2147483648.0 && (double)(N + 256) * (double)K < 2147483648.0;
     const bool stream_ok = tiled_ok && lim32 && M % 128 == 0 && N % 128 == 0 && K >= 512;
-    int variant = g_forced_variant >= 0 ? g_forced_variant : (tiled_ok ? choose_variant(M, N, stream_ok) : 0);
+    int variant = t_forced_variant >= 0 ? t_forced_variant : (tiled_ok ? choose_variant(M, N, stream_ok) : 0);
     if (variant != 0 && !tiled_ok) variant = 0;
     // the pipelined kernel walks K in pairs of 128-byte steps
     const bool pipe_ok = tiled_ok && K % 256 == 0 && lim32;

@@ -767,16 +767,7 @@ __global__ __launch_bounds__(kThreads) void cast_rowcol_kernel(const void *__res
 
 static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-static int num_cus() {
-    static int cus = 0;
-    if (cus == 0) {
-        int dev = 0;
-        hipDeviceProp_t prop;
-        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) cus = prop.multiProcessorCount;
-        if (cus <= 0) cus = 256;
-    }
-    return cus;
-}
+static int num_cus() { return device_cu_count(); }
 
 static int64_t grid_for(int64_t work_items, int per_block, int blocks_per_cu) {
     int64_t need = (work_items + per_block - 1) / per_block;

@@ -96,7 +96,7 @@ def get_fp8_format_from_string(format_str: str) -> Fp8Format:
     for fmt, names in _FORMAT_ALIASES.items():
         if key in names:
             return fmt
-    raise ValueError(f"Unknown FP8 format: {format_str}. Supported formats: hybrid, e4m3, e5m2")
+    raise ValueError(f"Unknown FP8 format: {key}. Supported formats: hybrid, e4m3, e5m2")
 
 
 def get_fp8_recipe_type_from_string(recipe_str: str) -> Fp8RecipeType:
@@ -104,7 +104,7 @@ def get_fp8_recipe_type_from_string(recipe_str: str) -> Fp8RecipeType:
     for rt, names in _RECIPE_ALIASES.items():
         if key in names:
             return rt
-    raise ValueError(f"Unknown FP8 recipe type: {recipe_str}. Supported types: delayed, tensorwise, blockwise, mxfp8")
+    raise ValueError(f"Unknown FP8 recipe type: {key}. Supported types: delayed, tensorwise, blockwise, mxfp8")
 
 
 @dataclass
@@ -187,6 +187,9 @@ class FP8Recipe:
             kind=self.recipe_type.value, fmt_fwd=fwd, fmt_bwd=bwd, margin=margin,
             amax_history_len=amax_history_len, amax_compute_algo=amax_compute_algo, reduce_amax=reduce_amax,
         )
+        # the arenas that modules reserve their delayed-scaling roles in when they first run under this recipe.
+        # The modules keep the views (the state is theirs): another recipe of the same shape -- the one an
+        # evaluation forward builds -- finds the roles on the module and reserves nothing here
         self._store = _state.MetaStore(amax_history_len)
         self._depth = 0
         # the last activation quantised under this recipe, so that Linears fed by the same tensor
@@ -203,7 +206,6 @@ class FP8Recipe:
         # partial maxima handed over by the kernel that produced a tensor (SwiGLU, RMSNorm), so that
         # the Linear that quantises this very tensor skips its amax pass; a handful of entries
         self.producer_parts: list[tuple[tuple, torch.Tensor, torch.Tensor]] = []
-        self.scale_epoch = 0      # bumped whenever the forward scales are refreshed (invalidates cached weight codes)
         _info_once(
             f"Created FP8 recipe with format={self.format.value}, amax_history_len={amax_history_len}, "
             f"amax_compute_algo={amax_compute_algo}"
@@ -227,8 +229,6 @@ class FP8Recipe:
         if not self.is_delayed:
             return
         algo = native.AMAX_MAX if self.amax_compute_algo == "max" else native.AMAX_MOST_RECENT
-        if direction == "fwd":
-            self.scale_epoch += 1
         for arena in self._store.dirty_arenas(direction):
             R = arena.used
             native.delayed_update_raw(arena.history, arena.H, arena.capacity, R, arena.scale, arena.scale_inv,
@@ -236,28 +236,69 @@ class FP8Recipe:
             arena.dirty = False
             arena.epoch += 1
 
-    def state_dict(self) -> dict:
-        """Scaling state (histories and scales) of every role registered so far,
-        as CPU tensors; roles are in module-registration order."""
-        out = {}
-        for (dev, direction), chain in self._store.arenas.items():
-            out[f"{dev}/{direction}"] = [
-                {"used": a.used, "history": a.history[:, :a.used].cpu(), "scale": a.scale[:a.used].cpu(),
-                 "scale_inv": a.scale_inv[:a.used].cpu()} for a in chain]
+    # ---------------------------------------------------------- checkpointing
+    _DIRECTIONS = (("fwd", "scaling_fwd"), ("bwd", "scaling_bwd"))
+
+    @staticmethod
+    def _fp8_modules(model: torch.nn.Module):
+        return [(name, mod) for name, mod in model.named_modules() if hasattr(mod, "_meta") and hasattr(mod, "fp8_meta")]
+
+    def state_dict(self, model: torch.nn.Module) -> dict:
+        """Delayed-scaling state (amax histories, scales) of every FP8 module of ``model``, as CPU
+        tensors keyed by the module's qualified name.  The state lives with the modules, but it is not
+        part of ``model.state_dict()`` (whose keys stay those of the plain model): a trainer that
+        checkpoints a delayed-scaling run saves this dict next to the model's and hands it to
+        :meth:`load_state_dict` after building model and recipe, before the first step.  Empty for
+        the recipes that keep no state between steps (tensorwise, rowwise)."""
+        out: dict[str, Any] = {"format_version": 1, "amax_history_len": self.amax_history_len, "modules": {}}
+        if not self.is_delayed:
+            return out
+        for name, mod in self._fp8_modules(model):
+            entry = {}
+            for direction, _ in self._DIRECTIONS:
+                meta = mod._meta(self, mod.weight.device, direction)
+                entry[direction] = {"amax_history": meta.amax_history.detach().cpu().clone(),
+                                    "scale": meta.scale.detach().cpu().clone(),
+                                    "scale_inv": meta.scale_inv.detach().cpu().clone(),
+                                    "trained": meta.trained}
+            out["modules"][name] = entry
         return out
 
-    def load_state_dict(self, state: dict) -> None:
-        for key, blobs in state.items():
-            dev, direction = key.rsplit("/", 1)
-            chain = self._store.arenas.get((dev, direction), [])
-            for arena, blob in zip(chain, blobs):
-                n = min(arena.used, blob["used"])
-                if blob["history"].shape[0] != arena.H:
-                    raise ValueError("amax_history_len of the checkpoint differs from this recipe")
-                arena.history[:, :n].copy_(blob["history"][:, :n])
-                arena.scale[:n].copy_(blob["scale"][:n])
-                arena.scale_inv[:n].copy_(blob["scale_inv"][:n])
-                arena.invalidate_snapshot()
+    def load_state_dict(self, model: torch.nn.Module, state: dict, strict: bool = True) -> None:
+        """Restore what :meth:`state_dict` saved.  The roles of every module are reserved here, so the
+        call works on a freshly built model that has not run a forward yet.  Quantised weights cached
+        under other scales are invalidated.  strict: module names that are in ``state`` and not in the
+        model, or the reverse, raise ``KeyError``."""
+        if not self.is_delayed:
+            return
+        if state.get("amax_history_len", self.amax_history_len) != self.amax_history_len:
+            raise ValueError(f"amax_history_len of the checkpoint ({state.get('amax_history_len')}) differs from this "
+                             f"recipe's ({self.amax_history_len})")
+        saved = state.get("modules", {})
+        mods = dict(self._fp8_modules(model))
+        if strict:
+            missing, unexpected = sorted(set(mods) - set(saved)), sorted(set(saved) - set(mods))
+            if missing or unexpected:
+                raise KeyError(f"FP8 scaling state does not match the model: no state for {missing}, no module for {unexpected}")
+        touched: set = set()
+        for name, entry in saved.items():
+            mod = mods.get(name)
+            if mod is None:
+                continue
+            for direction, _ in self._DIRECTIONS:
+                blob = entry[direction]
+                meta = mod._meta(self, mod.weight.device, direction)
+                touched.add(meta.arena)
+                if tuple(blob["amax_history"].shape) != tuple(meta.amax_history.shape):
+                    raise ValueError(f"{name}/{direction}: saved history {tuple(blob['amax_history'].shape)} does not fit "
+                                     f"{tuple(meta.amax_history.shape)}")
+                meta.amax_history.copy_(blob["amax_history"])
+                meta.scale.copy_(blob["scale"])
+                meta.scale_inv.copy_(blob["scale_inv"])
+                if blob.get("trained", True):
+                    meta.first_record_epoch = -1
+        for arena in touched:          # codes and inverse-scale snapshots made under the old scales are stale
+            arena.epoch += 1
 
     # ------------------------------------------------------- producer hand-over
     @staticmethod

@@ -11,10 +11,18 @@ Design for one MI355X:
     autograd worker thread sees the same state as the thread that entered the
     context (a thread-local would not); backward additionally carries its recipe
     in the autograd ``ctx`` and never depends on the ambient state;
-  * all delayed-scaling roles of all modules live in ONE arena per (recipe,
-    device, direction): history [H, R], scale [R], scale_inv [R].  Casts write
-    their amax straight into row 0 of the arena and a single tiny kernel
-    refreshes every role of the model per step.
+  * all delayed-scaling roles of the modules that first ran under a recipe live in
+    ONE arena per (recipe, device, direction): history [H, R], scale [R],
+    scale_inv [R].  Casts write their amax straight into row 0 of the arena and a
+    single tiny kernel refreshes every role of the model per step;
+  * the scaling state belongs to the MODULES, as in the reference's backend (which
+    keeps ``fp8_meta`` on each layer): a module finds its roles again by history
+    length, formats and device, whatever recipe object is active.  The fresh recipe
+    that an evaluation forward builds
+    (optimus_dl/recipe/train/mixins/managers/evaluation_manager.py:98-144) therefore
+    works with the scales that training arrived at and reserves nothing; a recipe
+    that records into roles it did not reserve adopts their arena and refreshes it
+    when its own context exits.
 """
 
 from __future__ import annotations
@@ -59,6 +67,22 @@ class ScalingMeta:
 
     def __init__(self, arena: "MetaArena", first: int, n: int):
         self.arena, self.first, self.n = arena, first, n
+        self.first_record_epoch: int | None = None   # arena epoch at the first cast that recorded an amax here
+
+    def note_record(self, store: "MetaStore") -> None:
+        """A cast running under the recipe that owns ``store`` is about to record this step's amax in
+        row 0 of the history: that recipe's context exit has to refresh this arena."""
+        if self.first_record_epoch is None:
+            self.first_record_epoch = self.arena.epoch
+        self.arena.dirty = True
+        if self.arena.owner is not store:
+            store.adopted.add(self.arena)
+
+    @property
+    def trained(self) -> bool:
+        """True once the scales have been refreshed from at least one recorded amax; until then
+        these roles carry the initial scale 1."""
+        return self.first_record_epoch is not None and self.arena.epoch > self.first_record_epoch
 
     @property
     def amax_history(self) -> torch.Tensor:          # [H, n] view
@@ -91,8 +115,9 @@ class ScalingMeta:
 class MetaArena:
     """history [H, cap], scale [cap], scale_inv [cap], fmt [cap] for one direction."""
 
-    def __init__(self, device: torch.device, history_len: int, capacity: int):
+    def __init__(self, device: torch.device, history_len: int, capacity: int, direction: str = "fwd", owner=None):
         self.device, self.H, self.capacity = device, history_len, capacity
+        self.direction, self.owner = direction, owner
         self.history = torch.zeros((history_len, capacity), dtype=torch.float32, device=device)
         self.scale = torch.ones(capacity, dtype=torch.float32, device=device)
         self.scale_inv = torch.ones(capacity, dtype=torch.float32, device=device)
@@ -126,13 +151,15 @@ class MetaArena:
 
 class MetaStore:
     """All arenas of one recipe.  Arenas are never reallocated (modules hold views
-    into them), a full one is followed by a new one."""
+    into them), a full one is followed by a new one.  ``adopted``: arenas reserved under
+    another recipe into which a cast under this one has recorded an amax."""
 
     CAPACITY = 2048
 
     def __init__(self, history_len: int):
         self.history_len = history_len
         self.arenas: dict[tuple[str, str], list[MetaArena]] = {}
+        self.adopted: set[MetaArena] = set()
 
     def reserve(self, device: torch.device, direction: str, fmts: list[int]) -> ScalingMeta:
         key = (str(device), direction)
@@ -141,11 +168,12 @@ class MetaStore:
             meta = chain[-1].reserve(fmts)
             if meta is not None:
                 return meta
-        chain.append(MetaArena(device, self.history_len, self.CAPACITY))
+        chain.append(MetaArena(device, self.history_len, self.CAPACITY, direction, self))
         return chain[-1].reserve(fmts)
 
     def dirty_arenas(self, direction: str) -> list[MetaArena]:
-        return [a for (dev, d), chain in self.arenas.items() if d == direction for a in chain if a.dirty and a.used]
+        own = [a for (dev, d), chain in self.arenas.items() if d == direction for a in chain if a.dirty and a.used]
+        return own + [a for a in self.adopted if a.direction == direction and a.dirty and a.used]
 
 
 def tensor_version(t) -> int:

@@ -114,11 +114,20 @@ def _converted_input(recipe: FP8Recipe, x2d: torch.Tensor, dtype: torch.dtype) -
     return out
 
 
-def _quantise_delayed(x2d: torch.Tensor, fmt: int, meta: "_state.ScalingMeta", role: int, need_t: bool,
-                      need_rowmajor: bool = True):
-    """Delayed scaling: one pass with the scale from the history, amax recorded in row 0."""
-    scale, slot = meta.scale_of(role), meta.amax_slot(role)
-    meta.arena.dirty = True
+def _quantise_delayed(x2d: torch.Tensor, fmt: int, meta: "_state.ScalingMeta | None", role: int, need_t: bool,
+                      need_rowmajor: bool = True, recipe: FP8Recipe | None = None, record: bool = True, margin: int = 0):
+    """Delayed scaling: one pass with the scale from the history, amax recorded in row 0.
+    record=False (a module in eval mode): the scales that training arrived at are used as they are and
+    the histories are left alone; roles that do not exist yet (meta None) or have never been through a
+    refresh still stand at the initial scale 1 (a weight of std 0.02 would land in the subnormals), so
+    such a tensor is scaled from its own amax instead."""
+    if not record and (meta is None or not meta.trained):
+        q, q_t, scale_inv, _ = _quantise_dynamic(x2d, fmt, margin, need_t, need_rowmajor)
+        return q, q_t, scale_inv
+    scale = meta.scale_of(role)
+    slot = meta.amax_slot(role) if record else None
+    if record:
+        meta.note_record(recipe._store)
     # the inverse scale comes from the arena's per-step snapshot: the arena entry itself changes at the next update
     scale_inv = meta.scale_inv_snapshot_of(role)
     if need_t:
@@ -170,8 +179,9 @@ class _Fp8LinearFn(torch.autograd.Function):
             ctx.wgrad_direct = (fp8_wgrad and recipe.direct_layouts
                                 and native.gemm_layouts_supported(n_out, n_in, tokens, weight.dtype))
             if pol.kind == "delayed":
-                meta = module._meta(recipe, x2d.device, "fwd")
-                xq, xq_t, sx_inv = _quantise_delayed(x2d, pol.fmt_fwd, meta, ROLE_X, fp8_wgrad)
+                meta = module._meta(recipe, x2d.device, "fwd", create=module.training)
+                xq, xq_t, sx_inv = _quantise_delayed(x2d, pol.fmt_fwd, meta, ROLE_X, fp8_wgrad, recipe=recipe,
+                                                     record=module.training, margin=pol.margin)
             else:
                 xq, xq_t, sx_inv = _quantise_input_shared(recipe, x2d, pol.fmt_fwd, pol.margin, fp8_wgrad)
             wq, wq_t, sw_inv = module._tensor_weight(weight, recipe, need_t=need_dgrad)
@@ -182,16 +192,24 @@ class _Fp8LinearFn(torch.autograd.Function):
                 saved["wq_t"], saved["sw_inv_t"] = wq_t, sw_inv
         if need_wgrad and not recipe.wgrad:
             saved["x_hp"] = x2d                      # wgrad=False: weight gradient in the activation dtype
-        ctx.module, ctx.recipe, ctx.saved = module, recipe, saved
+        if pol.kind == "rowwise" and need_dgrad:
+            saved["weight"] = weight                 # dgrad scales W per input channel, from the weight itself
+        # Everything the backward reads goes through autograd's saved-tensor machinery: activation
+        # checkpointing drops it after the forward and recomputes it, saved-tensor hooks (offloading) see it,
+        # an in-place change of an input between forward and backward is detected, and the tensors are
+        # released as soon as this node has run.
+        ctx.saved_names = tuple(saved)
+        ctx.save_for_backward(*saved.values())
+        ctx.module, ctx.recipe = module, recipe
         ctx.need_wgrad, ctx.need_dgrad, ctx.has_bias = need_wgrad, need_dgrad, bias is not None
         ctx.x_dtype, ctx.w_dtype = x2d.dtype, weight.dtype
         ctx.bias_dtype = None if bias is None else bias.dtype
-        ctx.weight_ref = weight if pol.kind == "rowwise" and need_dgrad else None
         return y
 
     @staticmethod
     def backward(ctx, dy: torch.Tensor):
-        module, recipe, saved = ctx.module, ctx.recipe, ctx.saved
+        module, recipe = ctx.module, ctx.recipe
+        saved = dict(zip(ctx.saved_names, ctx.saved_tensors))
         pol = recipe.recipe
         dy2d = dy if dy.is_contiguous() else dy.contiguous()
         if dy2d.dtype not in (torch.bfloat16, torch.float32):
@@ -207,7 +225,7 @@ class _Fp8LinearFn(torch.autograd.Function):
             elif fp8_wgrad:
                 gq_t, sg_inv_t = _quantise_axis(dy2d, pol.fmt_bwd, pol.margin, C, True)
             if ctx.need_dgrad:
-                wq_t, sw_inv_t = module._rowwise_weight(ctx.weight_ref, pol, "col")
+                wq_t, sw_inv_t = module._rowwise_weight(saved["weight"], pol, "col")
                 dx = native.gemm_nt(gq, wq_t, pol.fmt_bwd, pol.fmt_fwd, sg_inv, sw_inv_t, out_dtype=ctx.x_dtype)
             if fp8_wgrad:
                 dw = native.gemm_nt(gq_t, saved["xq_t"], pol.fmt_bwd, pol.fmt_fwd, sg_inv_t, saved["sx_inv_t"],
@@ -218,8 +236,9 @@ class _Fp8LinearFn(torch.autograd.Function):
             g_rm_needed = ctx.need_dgrad or (fp8_wgrad and ctx.wgrad_direct)
             if ctx.need_dgrad or fp8_wgrad:
                 if pol.kind == "delayed":
-                    meta = module._meta(recipe, dy2d.device, "bwd")
-                    gq, gq_t, sg_inv = _quantise_delayed(dy2d, pol.fmt_bwd, meta, ROLE_G, g_t_needed, g_rm_needed)
+                    meta = module._meta(recipe, dy2d.device, "bwd", create=module.training)
+                    gq, gq_t, sg_inv = _quantise_delayed(dy2d, pol.fmt_bwd, meta, ROLE_G, g_t_needed, g_rm_needed,
+                                                         recipe=recipe, record=module.training, margin=pol.margin)
                 else:
                     parts = recipe.take_parts(dy2d)
                     if ctx.has_bias and native.colsum_supported(dy2d):
@@ -263,7 +282,7 @@ class FP8Linear(nn.Linear):
     def _init_fp8_state(self) -> None:
         self._wcache = _WeightCache()
         self._wcache_rowwise: dict[str, tuple] = {}
-        self._metas: dict[tuple[int, str, str], "_state.ScalingMeta"] = {}
+        self._metas: dict[tuple, "_state.ScalingMeta"] = {}
         self.fp8_meta: dict[str, "_state.ScalingMeta"] = {}
         self.fp8_calls = 0                   # forwards that actually took the FP8 path (for tests / logging)
 
@@ -304,39 +323,53 @@ class FP8Linear(nn.Linear):
         return self
 
     # ------------------------------------------------------------ scaling state
-    def _meta(self, recipe: FP8Recipe, device: torch.device, direction: str) -> "_state.ScalingMeta":
-        key = (id(recipe), str(device), direction)
+    def _meta(self, recipe: FP8Recipe, device: torch.device, direction: str, create: bool = True) -> "_state.ScalingMeta | None":
+        """This module's delayed-scaling roles for one direction.  Keyed by what the state depends on
+        (history length, formats, device), not by the recipe object: the reference's backend keeps
+        ``fp8_meta`` on the layer, and a second recipe of the same shape -- the one an evaluation forward
+        builds per call -- continues with the scales the first one measured.  create=False: None when
+        the roles do not exist yet (nothing is reserved)."""
+        pol = recipe.recipe
+        key = (pol.amax_history_len, pol.fmt_fwd, pol.fmt_bwd, str(device), direction)
         meta = self._metas.get(key)
         if meta is None:
-            pol = recipe.recipe
+            if not create:
+                return None
             fmts = [pol.fmt_fwd] * 3 if direction == "fwd" else [pol.fmt_bwd] * 2
             meta = recipe.reserve_meta(device, direction, fmts)
             self._metas[key] = meta
-            self.fp8_meta["scaling_fwd" if direction == "fwd" else "scaling_bwd"] = meta
+        self.fp8_meta["scaling_fwd" if direction == "fwd" else "scaling_bwd"] = meta
         return meta
 
     def _tensor_weight(self, weight: torch.Tensor, recipe: FP8Recipe, need_t: bool):
         """Per-tensor quantised weight (and transpose), cached on the parameter version."""
         pol = recipe.recipe
         c = self._wcache
-        # delayed scaling: the codes depend on the scale in force, which changes at every refresh
-        key = (weight.data_ptr(), _state.tensor_version(weight), id(recipe), pol.kind, recipe.scale_epoch if pol.kind == "delayed" else 0)
+        record = self.training
+        meta = None
+        # the codes depend on the parameter's contents, the format and how the scale is found; under delayed
+        # scaling also on the scale in force, which changes with every refresh of the arena
+        if pol.kind == "delayed":
+            meta = self._meta(recipe, weight.device, "fwd", create=record)
+            how = ("delayed", pol.amax_history_len, id(meta.arena), meta.arena.epoch, record) if meta is not None else ("own amax", pol.margin)
+        else:
+            how = (pol.kind, pol.margin)
+        key = (weight.data_ptr(), _state.tensor_version(weight), pol.fmt_fwd, how)
         fresh = c.key != key or not recipe.cache_weights
         if fresh or (need_t and c.wq_t is None):
             w2d = weight.detach()
             if pol.kind == "delayed":
-                meta = self._meta(recipe, weight.device, "fwd")
-                c.wq, c.wq_t, c.s_inv = _quantise_delayed(w2d, pol.fmt_fwd, meta, ROLE_W, need_t)
-                c.amax = meta.amax_slot(ROLE_W).clone()      # only this weight ever writes that slot
+                c.wq, c.wq_t, c.s_inv = _quantise_delayed(w2d, pol.fmt_fwd, meta, ROLE_W, need_t, recipe=recipe, record=record,
+                                                          margin=pol.margin)
+                c.amax = meta.amax_slot(ROLE_W).clone() if record else None     # only this weight ever writes that slot
             else:
                 c.wq, c.wq_t, c.s_inv, c.amax = _quantise_dynamic(w2d, pol.fmt_fwd, pol.margin, need_t)
             c.key = key
-        elif pol.kind == "delayed":
+        elif pol.kind == "delayed" and record:
             # cached codes are reused; this step's history still has to see the weight's amax
-            meta = self._meta(recipe, weight.device, "fwd")
             slot = meta.amax_slot(ROLE_W)
             torch.maximum(slot, c.amax, out=slot)
-            meta.arena.dirty = True
+            meta.note_record(recipe._store)
         return c.wq, c.wq_t, c.s_inv
 
     def _rowwise_weight(self, weight: torch.Tensor, pol, axis: str, both: bool = False):

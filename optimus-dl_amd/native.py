@@ -23,7 +23,7 @@ DT_BF16, DT_F32 = 0, 1
 AMAX_MAX, AMAX_MOST_RECENT = 0, 1
 FP8_MAX = {E4M3: 448.0, E5M2: 57344.0}
 TORCH_FP8 = {E4M3: torch.float8_e4m3fn, E5M2: torch.float8_e5m2}
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # ODL_FP8_LIB names another build of the same library (e.g. one made for an experiment)
@@ -568,15 +568,15 @@ def gemm_nt(a: torch.Tensor, b: torch.Tensor, fmt_a: int, fmt_b: int, sa_inv: to
 
 
 K_FAST, K_SLOW = 0, 1
-split_k = True            # outputs of few tiles with a long contraction are computed as K runs side by side
-_forced_variant = -1
+split_k = True            # tuning knob: outputs of few tiles with a long contraction are computed as K runs side by side
+_tls = threading.local()  # .forced_variant mirrors the library's per-thread switch (see gemm_set_variant)
 
 
 def gemm_split_count(M: int, N: int, K: int, k_slow: bool = False) -> int:
     """Number of K runs the library proposes for this shape (1: one launch of the ordinary kernel).
     k_slow: an operand is passed with the contraction index slow (only the streaming kernel reads that).
     Always 1 while a kernel variant is forced or ``split_k`` is off."""
-    if not split_k or _forced_variant >= 0 or (M + 256) * K >= 2**31 or (N + 256) * K >= 2**31:
+    if not split_k or getattr(_tls, "forced_variant", -1) >= 0 or (M + 256) * K >= 2**31 or (N + 256) * K >= 2**31:
         return 1
     return int(load().odl_fp8_gemm_split_count(M, N, K, 1 if k_slow else 0))
 
@@ -686,6 +686,8 @@ def gemm_variants() -> list[str]:
 
 
 def gemm_set_variant(variant: int) -> None:
-    global _forced_variant
+    """Pin the GEMM kernel variant (-1: choose by shape) for calls made from THIS host thread.  A
+    testing / tuning switch: it does not reach other threads, so the GEMMs that autograd's worker
+    thread launches in a backward pass keep the automatic choice."""
     _check(load().odl_fp8_gemm_set_variant(variant), "odl_fp8_gemm_set_variant")
-    _forced_variant = variant
+    _tls.forced_variant = variant

@@ -8,8 +8,8 @@ dtype an FP8 dtype? is the device "cuda"? is the backend there? is
 .../iteration_mixin.py:101-185: ``amp_ctx`` and ``fp8_backward_ctx`` may be a
 context-manager instance or a zero-argument factory, re-entered every microbatch.
 ``forward_context`` is the evaluation-side wrapper
-(.../managers/evaluation_manager.py:98-144): a fresh recipe per call, FP8 autocast
-with bf16 inside.
+(.../managers/evaluation_manager.py:98-144): FP8 autocast with bf16 inside, on the
+scales the training steps measured.
 """
 
 from __future__ import annotations
@@ -127,21 +127,38 @@ def execute_backward_pass(loss: torch.Tensor, scaler=None, fp8_backward_ctx=None
             loss.backward()
 
 
-@contextmanager
-def forward_context(amp_cfg: AmpConfig, device: torch.device):
-    """Evaluation forward: FP8 autocast when the config asks for it and the
-    backend is there, else ordinary AMP."""
-    dtype = str_to_dtype(amp_cfg.dtype)
-    if amp_cfg.enabled and is_fp8_dtype(dtype) and amp_cfg.fp8.enabled and device.type == "cuda" \
-            and is_transformer_engine_available():
-        f = amp_cfg.fp8
+_eval_recipes: dict[tuple, FP8Recipe] = {}
+
+
+def _eval_recipe(f) -> FP8Recipe | None:
+    """The recipe of an evaluation forward.  The reference builds a new recipe object on every call
+    (evaluation_manager.py:126-135); a recipe here carries no scaling state of its own (that lives with
+    the modules), so one object per distinct configuration is kept and handed out again."""
+    key = (str(f.recipe).lower(), str(f.format).lower(), f.margin, f.amax_history_len, f.amax_compute_algo, f.reduce_amax,
+           f.fp8_dpa, f.fp8_mha)
+    recipe = _eval_recipes.get(key)
+    if recipe is None:
         recipe = create_fp8_recipe(recipe_type=f.recipe, format=f.format, margin=f.margin,
                                    amax_history_len=f.amax_history_len, amax_compute_algo=f.amax_compute_algo,
                                    reduce_amax=f.reduce_amax, fp8_dpa=f.fp8_dpa, fp8_mha=f.fp8_mha)
-        with fp8_autocast(device, recipe, dtype=torch.bfloat16):
-            yield
-    else:
-        if is_fp8_dtype(dtype):
-            dtype = torch.bfloat16
-        with torch.autocast(device.type, dtype=dtype, enabled=amp_cfg.enabled):
-            yield
+        if recipe is not None:
+            _eval_recipes[key] = recipe
+    return recipe
+
+
+@contextmanager
+def forward_context(amp_cfg: AmpConfig, device: torch.device):
+    """Evaluation forward (evaluation_manager.py:98-144): nothing when AMP is off; FP8 autocast with bf16
+    inside when the AMP dtype is an FP8 dtype, ``fp8.enabled`` is set and the backend is there; ordinary
+    autocast otherwise (bf16 standing in for an FP8 dtype).  Modules in eval mode use the delayed-scaling
+    scales that training measured and leave the amax histories alone."""
+    if not amp_cfg.enabled:
+        yield
+        return
+    dtype = str_to_dtype(amp_cfg.dtype)
+    is_fp8 = is_fp8_dtype(dtype)
+    recipe = None
+    if is_fp8 and getattr(amp_cfg, "fp8", None) and amp_cfg.fp8.enabled and is_transformer_engine_available():
+        recipe = _eval_recipe(amp_cfg.fp8)
+    with fp8_autocast(device=device, fp8_recipe=recipe, enabled=True, dtype=torch.bfloat16 if is_fp8 else dtype):
+        yield

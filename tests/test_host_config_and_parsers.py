@@ -88,6 +88,9 @@ def test_format_parser():
         assert get_fp8_format_from_string(s) == Fp8Format.E5M2
     with pytest.raises(ValueError, match="Unknown FP8 format"):
         get_fp8_format_from_string("invalid_format")
+    # the message names the lower-cased string, as optimus_dl/modules/amp/fp8.py:109,116 prints it
+    with pytest.raises(ValueError, match=r"Unknown FP8 format: bogus_fmt\. Supported formats: hybrid, e4m3, e5m2"):
+        get_fp8_format_from_string("Bogus_FMT")
 
 
 def test_recipe_parser():
@@ -104,6 +107,8 @@ def test_recipe_parser():
             assert get_fp8_recipe_type_from_string(n) == want
     with pytest.raises(ValueError, match="Unknown FP8 recipe type"):
         get_fp8_recipe_type_from_string("nope")
+    with pytest.raises(ValueError, match=r"Unknown FP8 recipe type: nope_x\. Supported types: delayed, tensorwise, blockwise, mxfp8"):
+        get_fp8_recipe_type_from_string("NOPE_x")
 
 
 def test_recipe_config_defaults():

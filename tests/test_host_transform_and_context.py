@@ -338,3 +338,53 @@ def test_converted_and_fused_modules_survive_deepcopy_and_pickling():
             again = build_model_transform({"_name": "transformer_engine"})
             again.apply(other)                                  # already converted: nothing left to do
             assert not any(again.last_replacements.values())
+
+
+# ---------------------------------------------------------------- evaluation forward context
+def test_forward_context_fallbacks_follow_the_reference_evaluator(monkeypatch):
+    """optimus_dl/recipe/train/mixins/managers/evaluation_manager.py:98-144: nothing when AMP is off; plain
+    autocast in the AMP dtype; bf16 autocast standing in for an FP8 dtype when ``fp8.enabled`` is off or the
+    backend is missing; an FP8 recipe only with dtype + flag + backend together."""
+    import optimus_dl_amd.recipe.training_context as tc
+
+    cpu = torch.device("cpu")
+    lin, x = nn.Linear(8, 8), torch.randn(4, 8)
+    with tc.forward_context(opt("torch.bfloat16", enabled=False).amp, cpu):
+        assert not torch.is_autocast_enabled("cpu") and lin(x).dtype == torch.float32
+    with tc.forward_context(opt("torch.bfloat16", fp8_enabled=False).amp, cpu):
+        assert torch.is_autocast_enabled("cpu") and lin(x).dtype == torch.bfloat16
+    with tc.forward_context(opt("torch.float16", fp8_enabled=False).amp, cpu):
+        assert torch.get_autocast_dtype("cpu") == torch.float16
+    with tc.forward_context(opt("torch.float8_e4m3fn", fp8_enabled=False).amp, cpu):          # FP8 dtype, flag off
+        assert torch.get_autocast_dtype("cpu") == torch.bfloat16 and lin(x).dtype == torch.bfloat16
+    monkeypatch.setattr(tc, "is_transformer_engine_available", lambda: False)                    # FP8 asked for, no backend
+    made = []
+    monkeypatch.setattr(tc, "create_fp8_recipe", lambda **kw: made.append(kw))
+    with tc.forward_context(opt("torch.float8_e4m3fn").amp, cpu):
+        assert torch.get_autocast_dtype("cpu") == torch.bfloat16
+    assert made == []
+    # dtype + flag + backend: a recipe is built from the config's keys, once per distinct configuration
+    monkeypatch.setattr(tc, "is_transformer_engine_available", lambda: True)
+    monkeypatch.setattr(tc, "_eval_recipes", {})
+
+    class Rec:
+        def __init__(self, **kw):
+            self.kw, self.entered = kw, 0
+
+        def autocast(self):
+            self.entered += 1
+            return nullcontext()
+
+    monkeypatch.setattr(tc, "create_fp8_recipe", lambda **kw: made.append(Rec(**kw)) or made[-1])
+    cfg = opt("torch.float8_e4m3fn", recipe="tensorwise", format="e4m3", margin=1, amax_history_len=8).amp
+    for _ in range(3):
+        with tc.forward_context(cfg, FakeCuda()):
+            pass
+    assert len(made) == 1 and made[0].entered == 3
+    assert made[0].kw == dict(recipe_type="tensorwise", format="e4m3", margin=1, amax_history_len=8, amax_compute_algo="max",
+                              reduce_amax=True, fp8_dpa=False, fp8_mha=False)
+    with tc.forward_context(opt("torch.float8_e4m3fn", recipe="delayed").amp, FakeCuda()):
+        pass
+    assert len(made) == 2                                          # another configuration, another recipe
+    with tc.forward_context(cfg, cpu):                             # a recipe off the GPU: ordinary bf16 autocast (fp8.py:488)
+        assert torch.get_autocast_dtype("cpu") == torch.bfloat16
