@@ -104,6 +104,23 @@ int odl_fp8_cast_dynamic(const void *x, int src_dtype, int64_t rows, int64_t col
                          odl_stream_t stream);
 
 /*
+ * odl_fp8_amax_parts + odl_fp8_cast_dynamic in one call that ALLOCATES NOTHING and takes no workspace:
+ * the partial maxima go through a 2 KB array that is part of the library's device image (one copy per
+ * GPU, held until the process ends).  It has no counterpart in the reference; it is for callers that
+ * cannot allocate device memory or carry a workspace around: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  out, out_t, dyn_out and the results are those of
+ * odl_fp8_cast_dynamic, bit for bit.  rows * cols above ODL_FP8_NOALLOC_MAX_ELEMS is refused with
+ * ODL_ERR_SHAPE (use the two calls above with a buffer of your own).
+ * Every call on a GPU uses that GPU's one array: calls that may overlap on the same GPU (different
+ * streams, or different host threads without ordering between their streams) race on it and must be
+ * ordered by the caller; calls on one stream are safe.  The first call on a device looks up the array's
+ * address (hipGetSymbolAddress): make it once outside of graph capture.
+ */
+#define ODL_FP8_NOALLOC_MAX_ELEMS ((int64_t)1 << 31)
+int odl_fp8_cast_dynamic_noalloc(const void *x, int src_dtype, int64_t rows, int64_t cols, int fmt, int margin,
+                                 uint8_t *out, uint8_t *out_t, float *dyn_out, odl_stream_t stream);
+
+/*
  * odl_fp8_amax_parts that also adds up the columns: colsum[c] = sum over rows of x[r, c] in fp32.
  * For the grad_output of a Linear with a bias, whose bias gradient is that sum (the `db` of
  * te.pytorch.Linear's backward, transformer_engine.py:97-108): dY is read by this pass and by the

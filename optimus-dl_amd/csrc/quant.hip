@@ -1038,6 +1038,59 @@ extern "C" int odl_fp8_cast_dynamic(const void *x, int src_dtype, int64_t rows, 
     return check_launch("odl_fp8_cast_dynamic");
 }
 
+// ------------------------------------------------ current scaling without a caller-side workspace
+// The partial maxima that odl_fp8_amax_parts hands to odl_fp8_cast_dynamic normally live in a buffer the
+// caller allocates.  Callers that cannot allocate (code under HIP graph capture, serving loops) use this
+// array instead: one copy per GPU, held until the process ends.  In host code the array's NAME is only a
+// handle for hipGetSymbolAddress; the address that kernels, copies and fills take is the pointer that
+// call returns, looked up once per device with that device current and kept in `g_scratch_ptr`.
+static __device__ __align__(256) float scratch[ODL_FP8_AMAX_PARTS];
+
+namespace odl {
+
+constexpr int kMaxScratchDevices = 64;
+static float *g_scratch_ptr[kMaxScratchDevices] = {};
+
+// Device address of `scratch` on the device that is current on this thread (nullptr + error text on failure).
+// Two threads that resolve the same device at once store the same pointer.
+static float *scratch_for_current_device(const char *who) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) { set_error(ODL_ERR_LAUNCH, "%s: hipGetDevice: %s", who, hipGetErrorString(e)); return nullptr; }
+    if (dev < 0 || dev >= kMaxScratchDevices) { set_error(ODL_ERR_ARG, "%s: device ordinal %d is not below %d", who, dev, kMaxScratchDevices); return nullptr; }
+    float *ptr = __atomic_load_n(&g_scratch_ptr[dev], __ATOMIC_ACQUIRE);
+    if (!ptr) {
+        void *addr = nullptr;
+        e = hipGetSymbolAddress(&addr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !addr) {
+            set_error(ODL_ERR_LAUNCH, "%s: hipGetSymbolAddress(scratch) on device %d: %s", who, dev, hipGetErrorString(e));
+            return nullptr;
+        }
+        ptr = static_cast<float *>(addr);
+        __atomic_store_n(&g_scratch_ptr[dev], ptr, __ATOMIC_RELEASE);
+    }
+    return ptr;
+}
+
+}  // namespace odl
+
+extern "C" int odl_fp8_cast_dynamic_noalloc(const void *x, int src_dtype, int64_t rows, int64_t cols, int fmt, int margin,
+                                            uint8_t *out, uint8_t *out_t, float *dyn_out, odl_stream_t stream_) {
+    if (int e = check_cast_args("odl_fp8_cast_dynamic_noalloc", x, src_dtype, rows, cols, reinterpret_cast<const float *>(x), ODL_SCALE_TENSOR, fmt)) return e;
+    if (!dyn_out) return set_error(ODL_ERR_ARG, "odl_fp8_cast_dynamic_noalloc: dyn_out is null");
+    if (rows * cols > 0 && !out && !out_t) return set_error(ODL_ERR_ARG, "odl_fp8_cast_dynamic_noalloc: out and out_t are both null");
+    // rows, cols >= 0 here; the product is formed in floating point so that it cannot wrap
+    if ((double)rows * (double)cols > (double)ODL_FP8_NOALLOC_MAX_ELEMS)
+        return set_error(ODL_ERR_SHAPE, "odl_fp8_cast_dynamic_noalloc: %lld x %lld elements exceed the limit of %lld of the entry point that "
+                         "allocates nothing; use odl_fp8_amax_parts + odl_fp8_cast_dynamic with a workspace of your own",
+                         (long long)rows, (long long)cols, (long long)ODL_FP8_NOALLOC_MAX_ELEMS);
+    float *parts = scratch_for_current_device("odl_fp8_cast_dynamic_noalloc");
+    if (!parts) return ODL_ERR_LAUNCH;
+    // the amax pass writes all ODL_FP8_AMAX_PARTS entries (unused ones as 0), so what the last call left is overwritten
+    if (int e = odl_fp8_amax_parts(x, src_dtype, rows, cols, parts, stream_)) return e;
+    return odl_fp8_cast_dynamic(x, src_dtype, rows, cols, parts, fmt, margin, out, out_t, dyn_out, stream_);
+}
+
 // ------------------------------------------------------------------ rowwise recipe, fused passes
 static bool rowcol_fast(const void *x, int64_t rows, int64_t cols) {
     return rows > 0 && cols > 0 && aligned16(x) && cols % 8 == 0 && rows % 16 == 0;

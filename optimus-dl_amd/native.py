@@ -37,6 +37,7 @@ EXPORTS = (
     "odl_fp8_amax_scale",
     "odl_fp8_amax_parts",
     "odl_fp8_cast_dynamic",
+    "odl_fp8_cast_dynamic_noalloc",
     "odl_fp8_amax_parts_colsum",
     "odl_fp8_swiglu_amax_parts",
     "odl_fp8_swiglu_bwd_amax_parts",
@@ -96,6 +97,7 @@ def load() -> ctypes.CDLL:
         L.odl_fp8_amax_scale.argtypes = [vp, i32, i64, i64, i32, i32, vp, vp, vp, vp, vp]
         L.odl_fp8_amax_parts.argtypes = [vp, i32, i64, i64, vp, vp]
         L.odl_fp8_cast_dynamic.argtypes = [vp, i32, i64, i64, vp, i32, i32, vp, vp, vp, vp]
+        L.odl_fp8_cast_dynamic_noalloc.argtypes = [vp, i32, i64, i64, i32, i32, vp, vp, vp, vp]
         L.odl_fp8_amax_parts_colsum.argtypes = [vp, i32, i64, i64, vp, vp, vp, vp]
         L.odl_fp8_swiglu_amax_parts.argtypes = [vp, vp, i64, i64, vp, vp, vp]
         L.odl_fp8_swiglu_bwd_amax_parts.argtypes = [vp, vp, vp, i64, i64, vp, vp, vp, vp, vp]
@@ -261,6 +263,28 @@ def cast_dynamic(x: torch.Tensor, parts: torch.Tensor, fmt: int, margin: int = 0
                                        q.data_ptr() if q is not None else None, q_t.data_ptr() if q_t is not None else None,
                                        dyn.data_ptr(), _stream()), "odl_fp8_cast_dynamic")
     return q, q_t, dyn[0:1], dyn[1:2], dyn[2:3]
+
+
+NOALLOC_MAX_ELEMS = 1 << 31            # ODL_FP8_NOALLOC_MAX_ELEMS
+
+
+def cast_dynamic_noalloc(x: torch.Tensor, fmt: int, margin: int, out: torch.Tensor | None, out_t: torch.Tensor | None,
+                         dyn_out: torch.Tensor) -> None:
+    """Current scaling of ``x`` into buffers the CALLER owns, through the entry point that allocates
+    nothing: the partial maxima pass through the library's per-GPU static array instead of a workspace.
+    Neither this wrapper nor the library allocates; calls that may overlap on one GPU race on that array.
+    out [rows, cols] / out_t [cols, rows] uint8 (either may be None), dyn_out fp32[3] = {amax, scale, 1/scale}."""
+    if not (x.is_cuda and x.dim() == 2 and x.is_contiguous()):
+        raise NativeError("cast_dynamic_noalloc: x must be a contiguous 2-D CUDA tensor (no copy is made here)")
+    rows, cols = x.shape
+    for t, shape, what in ((out, (rows, cols), "out"), (out_t, (cols, rows), "out_t")):
+        if t is not None and not (t.is_cuda and t.dtype == torch.uint8 and t.is_contiguous() and tuple(t.shape) == shape):
+            raise NativeError(f"cast_dynamic_noalloc: {what} must be a contiguous uint8 CUDA tensor of shape {shape}")
+    _f32_dev(dyn_out, 3, "cast_dynamic_noalloc dyn_out")
+    _check(load().odl_fp8_cast_dynamic_noalloc(x.data_ptr(), _src_dtype(x), rows, cols, fmt, margin,
+                                               out.data_ptr() if out is not None else None,
+                                               out_t.data_ptr() if out_t is not None else None, dyn_out.data_ptr(), _stream()),
+           "odl_fp8_cast_dynamic_noalloc")
 
 
 def quantize_dynamic(x: torch.Tensor, fmt: int, margin: int = 0, want_rowmajor: bool = True, want_transposed: bool = True,
