@@ -543,7 +543,33 @@ __global__ __launch_bounds__(kThreads) void cast_generic_kernel(const void *__re
 // go through a 4x4 byte transpose in registers (v_perm_b32) and an LDS tile
 // [64 cols][128 rows] so that they leave as 16-byte stores along the row axis:
 // both outputs are written in full 64/128-byte segments.
-constexpr int kTileR = 128, kTileC = 64, kLdsPitch = kTileR + 4;   // pitch in bytes; +4 keeps dword writes conflict-poor
+constexpr int kTileR = 128, kTileC = 64;
+
+// LDS placement of the transposed tile.  The LDS of gfx950 serves 64 four-byte banks per cycle, so the
+// tile is kept as 32 lines of 256 bytes, one per PAIR of tile columns (even column in the first 128
+// bytes), and each line is rotated by a multiple of 16 bytes that depends on the column:
+//   * a wave's dword writes (8 column groups x 8 consecutive row groups) land in 64 different banks,
+//   * the 16-byte reads stay aligned (ds_read_b128), and 16 consecutive lanes read one whole line.
+// Offsets in bytes; `ty` is the lane's group of 4 rows (0..31), `m16` a chunk of 16 rows (0..7).
+// Order in which consecutive blocks take tiles: panels of kCtPanel tile rows, down the rows of a panel first.
+// Blocks that run at the same time then write neighbouring 128-byte pieces of the same rows of the
+// transposed output instead of pieces that lie a whole output row (a power of two for the usual token
+// counts) apart; measured alone at 8192 x 4096 / 8192 x 14336: 28.6 -> 25.8 us, 90.3 -> 85.1 us.
+constexpr int kCtPanel = 16;
+__device__ __forceinline__ void ct_tile_of(int64_t id, int64_t tiles_r, int64_t tiles_c, int64_t &tr, int64_t &tc) {
+    const int64_t pn = id / (kCtPanel * tiles_c), local = id % (kCtPanel * tiles_c);
+    const int64_t gl = min((int64_t)kCtPanel, tiles_r - pn * kCtPanel);
+    tr = pn * kCtPanel + local % gl;
+    tc = local / gl;
+}
+
+__device__ __forceinline__ int ct_lds_rot(int col) { return 8 * (col >> 3) + 4 * ((col >> 1) & 3); }
+__device__ __forceinline__ int ct_lds_write_off(int col, int ty) {
+    return (col >> 1) * 256 + ((((col & 1) * 32) + ty + ct_lds_rot(col)) & 63) * 4;
+}
+__device__ __forceinline__ int ct_lds_read_off(int col, int m16) {
+    return (col >> 1) * 256 + ((((col & 1) * 32) + m16 * 4 + ct_lds_rot(col)) & 63) * 4;
+}
 
 // 4x4 byte transpose: in a[j] byte k  ->  out t[k] byte j
 __device__ __forceinline__ void transpose4x4(const uint32_t a[4], uint32_t t[4]) {
@@ -563,7 +589,7 @@ __global__ __launch_bounds__(kThreads) void cast_transpose_kernel(const void *__
                                                                    const float *__restrict__ scale,
                                                                    uint8_t *__restrict__ out, uint8_t *__restrict__ out_t,
                                                                    float *__restrict__ amax_out, int margin, float *__restrict__ dyn_out) {
-    __shared__ __attribute__((aligned(16))) uint8_t tile[kTileC * kLdsPitch];
+    __shared__ __attribute__((aligned(16))) uint8_t tile[kTileC * kTileR];
     __shared__ uint32_t red[kThreads / kWave];
     float s_dyn = 1.0f;
     if constexpr (MODE == kScaleParts) s_dyn = dynamic_scale<FMT>(scale, margin, dyn_out, red);
@@ -579,7 +605,8 @@ __global__ __launch_bounds__(kThreads) void cast_transpose_kernel(const void *__
     // Tiles are walked from the end of the tensor: the amax pass that ran just before read it front
     // to back, so its tail is what the memory-side cache still holds.
     const int64_t rev = ntiles - 1 - tile_id;
-    const int64_t tr = rev / tiles_c, tc = rev % tiles_c;
+    int64_t tr, tc;
+    ct_tile_of(rev, (rows + kTileR - 1) / kTileR, tiles_c, tr, tc);
     const int64_t r0 = tr * kTileR + ty * 4, c0 = tc * kTileC + tx * 8;
     const bool col_ok = c0 < cols;                  // cols % 8 == 0 (host-checked), so the whole 8-wide patch is in or out
 
@@ -651,8 +678,8 @@ __global__ __launch_bounds__(kThreads) void cast_transpose_kernel(const void *__
     transpose4x4(hi, th);
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
-        *reinterpret_cast<uint32_t *>(&tile[(tx * 8 + k) * kLdsPitch + ty * 4]) = tl[k];
-        *reinterpret_cast<uint32_t *>(&tile[(tx * 8 + 4 + k) * kLdsPitch + ty * 4]) = th[k];
+        *reinterpret_cast<uint32_t *>(&tile[ct_lds_write_off(tx * 8 + k, ty)]) = tl[k];
+        *reinterpret_cast<uint32_t *>(&tile[ct_lds_write_off(tx * 8 + 4 + k, ty)]) = th[k];
     }
     __syncthreads();
     // 64 tile-columns x 8 chunks of 16 rows = 512 chunks, two per lane
@@ -662,8 +689,7 @@ __global__ __launch_bounds__(kThreads) void cast_transpose_kernel(const void *__
         const int k = chunk / 8, m16 = chunk % 8;
         const int64_t oc = tc * kTileC + k, orow = tr * kTileR + m16 * 16;
         if (oc < cols && orow < rows) {             // rows % 16 == 0 (host-checked)
-            const uint32_t *src = reinterpret_cast<const uint32_t *>(&tile[k * kLdsPitch + m16 * 16]);
-            u32x4 v = {src[0], src[1], src[2], src[3]};
+            const u32x4 v = *reinterpret_cast<const u32x4 *>(&tile[ct_lds_read_off(k, m16)]);
             __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(out_t + oc * rows + orow));
         }
     }
@@ -689,13 +715,14 @@ __global__ __launch_bounds__(kThreads) void cast_rowcol_kernel(const void *__res
                                                                 int margin, uint8_t *__restrict__ out, uint8_t *__restrict__ out_t,
                                                                 float *__restrict__ s_row_out, float *__restrict__ s_row_inv,
                                                                 float *__restrict__ s_col_out, float *__restrict__ s_col_inv) {
-    __shared__ __attribute__((aligned(16))) uint8_t tile[kTileC * kLdsPitch];
+    __shared__ __attribute__((aligned(16))) uint8_t tile[kTileC * kTileR];
     __shared__ float s_row[kTileR], s_col[kTileC];
     constexpr int ESZ = SRC == ODL_BF16 ? 2 : 4;
     const int tx = threadIdx.x % 8;                 // 8 lanes across 64 columns
     const int ty = threadIdx.x / 8;                 // 32 lane-rows, 4 rows each
     const int64_t tiles_c = (cols + kTileC - 1) / kTileC;
-    const int64_t tr = blockIdx.x / tiles_c, tc = blockIdx.x % tiles_c;
+    int64_t tr, tc;
+    ct_tile_of(blockIdx.x, (rows + kTileR - 1) / kTileR, tiles_c, tr, tc);
     if (threadIdx.x < kTileR) {
         const int64_t r = tr * kTileR + threadIdx.x;
         const float sc = r < rows ? scale_rule(amax_row[r], Fp8Lim<FMT>::max, margin, 1.0f) : 1.0f;
@@ -748,8 +775,8 @@ __global__ __launch_bounds__(kThreads) void cast_rowcol_kernel(const void *__res
     transpose4x4(hi, th);
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
-        *reinterpret_cast<uint32_t *>(&tile[(tx * 8 + k) * kLdsPitch + ty * 4]) = tl[k];
-        *reinterpret_cast<uint32_t *>(&tile[(tx * 8 + 4 + k) * kLdsPitch + ty * 4]) = th[k];
+        *reinterpret_cast<uint32_t *>(&tile[ct_lds_write_off(tx * 8 + k, ty)]) = tl[k];
+        *reinterpret_cast<uint32_t *>(&tile[ct_lds_write_off(tx * 8 + 4 + k, ty)]) = th[k];
     }
     __syncthreads();
 #pragma unroll
@@ -758,8 +785,7 @@ __global__ __launch_bounds__(kThreads) void cast_rowcol_kernel(const void *__res
         const int k = chunk / 8, m16 = chunk % 8;
         const int64_t oc = tc * kTileC + k, orow = tr * kTileR + m16 * 16;
         if (oc < cols && orow < rows) {             // rows % 16 == 0 (host-checked)
-            const uint32_t *src = reinterpret_cast<const uint32_t *>(&tile[k * kLdsPitch + m16 * 16]);
-            const u32x4 v = {src[0], src[1], src[2], src[3]};
+            const u32x4 v = *reinterpret_cast<const u32x4 *>(&tile[ct_lds_read_off(k, m16)]);
             __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(out_t + oc * rows + orow));
         }
     }

@@ -122,6 +122,64 @@ def test_rowwise_gemm_at_config_4_shape_with_outlier_channels(N):
     assert sx2[123].item() == sx[123].item() / 8 and torch.equal(sx2[:123], sx[:123]) and torch.equal(sx2[124:], sx[124:])
 
 
+def test_rowwise_backward_at_config_4_shape(N):
+    """dgrad and wgrad of configuration 4 at its full size.  Each operand is scaled along its non-contracted axis
+    from the bf16 source: dY per row (dgrad) and per column, transposed (wgrad), W per input channel, X per channel.
+    Vectors of maxima against torch's reductions, sampled rows / columns of the codes bit for bit against the oracle's
+    cast, sampled outputs against the oracle's emulated matmul, and the module's backward equal to the direct calls."""
+    M, Nn, K = 16384, 14336, 4096
+    x = draw((M, K), 1.0, 3)
+    g = torch.Generator().manual_seed(4)
+    channels = torch.randperm(K, generator=g)[:4]
+    x[:, channels.cuda()] *= 100.0
+    w = draw((Nn, K), 0.02, 5)
+    dy = draw((M, Nn), 1e-3, 6)
+    fb, ff = O.E5M2, O.E4M3
+
+    def check_rowcol(t, fmt, what, seed):
+        q, s_row_inv, q_t, s_col_inv, a_row, a_col = N.quantize_rowcol(t, fmt)
+        assert torch.equal(a_row, t.float().abs().amax(dim=1)) and torch.equal(a_col, t.float().abs().amax(dim=0)), what
+        s_row, s_col = O.t_scale(a_row.cpu(), fmt), O.t_scale(a_col.cpu(), fmt)
+        assert_f32_bits_equal(s_row_inv, 1.0 / s_row, f"{what}: 1/scale per row")
+        assert_f32_bits_equal(s_col_inv, 1.0 / s_col, f"{what}: 1/scale per column")
+        gen = torch.Generator().manual_seed(seed)
+        ri = torch.cat([torch.tensor([0, t.shape[0] - 1]), torch.randperm(t.shape[0], generator=gen)[:6]])
+        ci = torch.cat([torch.tensor([0, t.shape[1] - 1]), torch.randperm(t.shape[1], generator=gen)[:6]])
+        assert_bytes_equal(q[ri.cuda()], O.t_cast(t[ri.cuda()].cpu(), s_row[ri], fmt, O.SCALE_ROW), f"{what}: codes scaled per row")
+        want_t = O.t_cast(t[:, ci.cuda()].cpu(), s_col[ci], fmt, O.SCALE_COL).t().contiguous()
+        assert_bytes_equal(q_t[ci.cuda()], want_t, f"{what}: transposed codes scaled per column")
+        return q, s_row_inv, q_t, s_col_inv
+
+    gq, sg_inv, gq_t, sg_inv_t = check_rowcol(dy, fb, "dY", 21)
+    _, _, wq_t, sw_inv_t = check_rowcol(w, ff, "W", 22)
+    _, _, xq_t, sx_inv_t = check_rowcol(x, ff, "X", 23)
+    # the outlier channels are isolated by the per-channel scales of X: every other channel keeps its own range
+    plain = torch.ones(K, dtype=torch.bool)
+    plain[channels] = False
+    assert (1.0 / sx_inv_t.cpu()[plain]).min() > 20 * (1.0 / sx_inv_t.cpu()[channels]).max()
+    N.gemm_set_variant(-1)
+    dx = N.gemm_nt(gq, wq_t, fb, ff, sg_inv, sw_inv_t)                       # [M, K] = dY . W
+    sample_check(dx, gq, wq_t, fb, ff, sg_inv, sw_inv_t, seed=31, what="config 4 dgrad")
+    dw = N.gemm_nt(gq_t, xq_t, fb, ff, sg_inv_t, sx_inv_t)                   # [N, K] = dY^T . X
+    sample_check(dw, gq_t, xq_t, fb, ff, sg_inv_t, sx_inv_t, seed=32, what="config 4 wgrad")
+    del gq, gq_t, wq_t, xq_t
+    # the module's backward under the rowwise recipe gives these very bits
+    from optimus_dl_amd.modules.amp import create_fp8_recipe
+    from optimus_dl_amd.modules.fp8_linear import FP8Linear
+
+    lin = FP8Linear(K, Nn, bias=False, device="cuda", dtype=torch.bfloat16)
+    with torch.no_grad():
+        lin.weight.copy_(w)
+    recipe = create_fp8_recipe("rowwise", "hybrid")
+    xr = x.requires_grad_(True)
+    with recipe.autocast():
+        y = lin(xr)
+    with recipe.backward():
+        y.backward(dy)
+    assert torch.equal(xr.grad, dx), "module dgrad differs from the direct calls"
+    assert torch.equal(lin.weight.grad, dw), "module wgrad differs from the direct calls"
+
+
 @pytest.mark.parametrize("shape,std,fmt", [((8192, 4096), 1.0, O.E4M3), ((14336, 4096), 0.02, O.E4M3),
                                            ((8192, 14336), 1e-3, O.E5M2), ((8192, 28672), 1e-3, O.E5M2)])
 def test_quantisation_at_baseline_shapes(N, shape, std, fmt):
