@@ -45,7 +45,7 @@ enum odl_status {
     ODL_ERR_LAUNCH = 3    /* HIP reported an error at launch */
 };
 
-/* ABI version of this header (7); bumped when a signature changes or an entry point is added. */
+/* ABI version of this header (8); bumped when a signature changes or an entry point is added. */
 int odl_fp8_abi_version(void);
 
 /* Last error message of the calling host thread ("" if none). */
@@ -266,6 +266,20 @@ int odl_fp8_cast_transpose(const void *x, int src_dtype, int64_t rows, int64_t c
                            uint8_t *out, uint8_t *out_t, float *amax_out, odl_stream_t stream);
 
 /*
+ * The cast of the delayed-scaling recipe in one launch (recipe "delayed", fp8.py:279-288; the cast inside
+ * te.pytorch.Linear, transformer_engine.py:106, under that recipe): codes with the per-tensor scale in force
+ * (scale[0], device memory), row-major (out), transposed (out_t) or both (either may be NULL, not both);
+ *   amax_parts    : ODL_FP8_AMAX_PARTS floats (or NULL: nothing is recorded).  Block b folds its maximum of |x|
+ *                   into amax_parts[b % ODL_FP8_AMAX_PARTS] (integer atomicMax of the magnitude bits, spread
+ *                   over many words instead of one); the entries are NOT cleared first, so several casts of
+ *                   one step accumulate.  odl_fp8_delayed_update folds and clears them.
+ *   scale_inv_out : 1 float (or NULL) <- 1 / scale[0] (IEEE division), the factor for the GEMM, in storage
+ *                   that the refresh after the step does not touch.
+ */
+int odl_fp8_cast_delayed(const void *x, int src_dtype, int64_t rows, int64_t cols, const float *scale, int fmt,
+                         uint8_t *out, uint8_t *out_t, float *amax_parts, float *scale_inv_out, odl_stream_t stream);
+
+/*
  * C[M,N] = (A[M,K] . B[N,K]^T) * (sa_inv[i] * sb_inv[j]) (+ bias[j]), fp32
  * accumulate on the MFMA units, rounded once to out_dtype (bf16 or fp32).
  *   a, b     : FP8 codes, K contiguous ("NT"); fmt_a / fmt_b may differ
@@ -330,10 +344,15 @@ int odl_fp8_gemm_splitk(const uint8_t *a, const uint8_t *b, int64_t M, int64_t N
  *   scale[r] = fp8_max(fmt[r]) / a / 2^margin, kept when a is 0/NaN/Inf; Inf -> FLT_MAX
  *   scale_inv[r] = 1 / scale[r]
  *   fmt: R ints (odl_fp8_format) in device memory.
+ *   amax_parts (or NULL): [R, ODL_FP8_AMAX_PARTS] partial maxima recorded by odl_fp8_cast_delayed, role r at
+ *   amax_parts + r * ODL_FP8_AMAX_PARTS, 16-byte aligned; history[0, r] <- max(history[0, r], max of the
+ *   role's entries) before anything else, and the entries are cleared for the next step.
+ * One launch for all R roles; the cost grows with H * R (the roll moves the whole history), not with a chain
+ * of H dependent reads per role.
  */
 int odl_fp8_delayed_update(float *history, int64_t H, int64_t R, int64_t ld,
                            float *scale, float *scale_inv, const int *fmt,
-                           int margin, int algo, odl_stream_t stream);
+                           int margin, int algo, float *amax_parts, odl_stream_t stream);
 
 /*
  * Testing / tuning / introspection (host only).  odl_fp8_gemm_set_variant pins the GEMM kernel variant

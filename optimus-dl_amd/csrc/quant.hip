@@ -388,24 +388,95 @@ __global__ void scale_from_amax_kernel(const float *__restrict__ amax, int64_t n
     if (scale_inv) scale_inv[i] = __fdiv_rn(1.0f, s);
 }
 
-// one thread per role; H is small (<= a few thousand), latency only
-__global__ void delayed_update_kernel(float *__restrict__ history, int64_t H, int64_t R, int64_t ld, float *__restrict__ scale,
-                                      float *__restrict__ scale_inv, const int *__restrict__ fmt, int margin, int algo) {
-    int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (r >= R) return;
-    const float first = history[r];
-    uint32_t abits = float_to_bits(first) & 0x7fffffffu;     // amaxes are >= 0 or NaN: integer max keeps NaN
-    for (int64_t h = 1; h < H; ++h) {
-        float cur = history[h * ld + r];
-        if (algo == ODL_AMAX_MAX) abits = max(abits, float_to_bits(cur) & 0x7fffffffu);
-        history[(h - 1) * ld + r] = cur;                      // roll by -1
+// Delayed-scaling refresh of R roles: amax = max over the window (or the newest entry), history rolled by -1
+// with row 0 cleared, scale and 1/scale by the scale rule.  `parts` (optional) holds kAmaxParts partial maxima
+// per role that the casts of this step recorded: they are folded into row 0 first and cleared.
+// A block owns 16 roles; its 256 lanes are 16 lanes per role.  The roll runs in place: lane `seg` of a role
+// moves rows [seg*S, (seg+1)*S) down by one, reading ahead of its own writes; the one row that a neighbouring
+// lane overwrites (the last of the segment) is read before a block-wide barrier.  History lengths of 1024
+// (the reference's default) cost 64 rows per lane instead of a chain of 1024 dependent loads.
+constexpr int kUpdRoles = 16, kUpdSegs = kThreads / kUpdRoles;
+
+__global__ __launch_bounds__(kThreads) void delayed_update_kernel(float *__restrict__ history, int64_t H, int64_t R, int64_t ld,
+                                                                  float *__restrict__ scale, float *__restrict__ scale_inv,
+                                                                  const int *__restrict__ fmt, int margin, int algo,
+                                                                  float *__restrict__ parts) {
+    __shared__ uint32_t s_part[kUpdRoles];
+    __shared__ uint32_t s_max[kUpdSegs][kUpdRoles];
+    const int64_t r_base = (int64_t)blockIdx.x * kUpdRoles;
+    // ---- partial maxima of this step: 16 lanes per role, 8 x 16 bytes per lane
+    {
+        const int role = threadIdx.x / kUpdSegs, lane = threadIdx.x % kUpdSegs;
+        const int64_t r = r_base + role;
+        uint32_t m = 0;
+        if (parts && r < R) {
+            u32x4 *p = reinterpret_cast<u32x4 *>(parts + r * kAmaxParts);
+            u32x4 v[kAmaxParts / 4 / kUpdSegs];
+#pragma unroll
+            for (int j = 0; j < kAmaxParts / 4 / kUpdSegs; ++j) v[j] = p[lane + kUpdSegs * j];
+#pragma unroll
+            for (int j = 0; j < kAmaxParts / 4 / kUpdSegs; ++j) {
+                m = max(m, max(max(v[j].x & 0x7fffffffu, v[j].y & 0x7fffffffu), max(v[j].z & 0x7fffffffu, v[j].w & 0x7fffffffu)));
+                p[lane + kUpdSegs * j] = u32x4{0, 0, 0, 0};
+            }
+        }
+#pragma unroll
+        for (int off = kUpdSegs / 2; off > 0; off >>= 1) m = max(m, (uint32_t)__shfl_xor((int)m, off, kUpdSegs));
+        if (lane == 0) s_part[role] = m;
     }
-    history[(H - 1) * ld + r] = first;
-    history[r] = 0.0f;
-    const float fmax = fmt[r] == ODL_FP8_E5M2 ? 57344.0f : 448.0f;
-    float s = scale_rule(bits_to_float(abits), fmax, margin, scale[r]);
-    scale[r] = s;
-    scale_inv[r] = __fdiv_rn(1.0f, s);
+    __syncthreads();
+    // ---- the roll: lane (c, seg) owns rows [lo, hi) of role r
+    const int c = threadIdx.x % kUpdRoles, seg = threadIdx.x / kUpdRoles;
+    const int64_t r = r_base + c;
+    const bool valid = r < R;
+    const int64_t S = (H + kUpdSegs - 1) / kUpdSegs;
+    const int64_t lo = seg * S, hi = min(H, lo + S);
+    const bool has_rows = valid && lo < hi;
+    // amaxes are >= 0 or NaN: the integer maximum of the magnitude bits keeps a NaN
+    // (what is stored back are the entries as they were, sign and NaN payload included)
+    uint32_t first = 0, first_mag = 0, tail = 0, abits = 0;
+    if (has_rows) tail = float_to_bits(history[(hi - 1) * ld + r]);
+    if (valid && seg == 0) {
+        first = float_to_bits(history[r]);
+        first_mag = first & 0x7fffffffu;
+        if (s_part[c] > first_mag) first = first_mag = s_part[c];
+    }
+    __syncthreads();                                          // every segment's last row is in a register
+    if (has_rows) {
+        abits = tail & 0x7fffffffu;
+        constexpr int kAhead = 8;
+        int64_t h = max(lo, (int64_t)1);                      // row 0 moves to row H - 1 (below), not down
+        for (; h + kAhead <= hi - 1; h += kAhead) {
+            uint32_t v[kAhead];
+#pragma unroll
+            for (int u = 0; u < kAhead; ++u) v[u] = float_to_bits(history[(h + u) * ld + r]);
+#pragma unroll
+            for (int u = 0; u < kAhead; ++u) {
+                abits = max(abits, v[u] & 0x7fffffffu);
+                history[(h + u - 1) * ld + r] = (h + u == 1) ? 0.0f : bits_to_float(v[u]);
+            }
+        }
+        for (; h < hi - 1; ++h) {
+            const uint32_t v = float_to_bits(history[h * ld + r]);
+            abits = max(abits, v & 0x7fffffffu);
+            history[(h - 1) * ld + r] = h == 1 ? 0.0f : bits_to_float(v);
+        }
+        if (hi - 1 >= 1) history[(hi - 2) * ld + r] = hi - 1 == 1 ? 0.0f : bits_to_float(tail);   // the row read before the barrier
+    }
+    s_max[seg][c] = abits;
+    __syncthreads();
+    if (valid && seg == 0) {
+        // row 0 held this step's amax (seg 0 read it as its tail when S == 1, as `first` always)
+        uint32_t window = first_mag;
+        if (algo == ODL_AMAX_MAX)
+            for (int g = 0; g < kUpdSegs; ++g) window = max(window, s_max[g][c]);
+        history[(H - 1) * ld + r] = bits_to_float(first);
+        history[r] = 0.0f;                                    // also when H == 1: the only row starts the next step empty
+        const float fmax = fmt[r] == ODL_FP8_E5M2 ? 57344.0f : 448.0f;
+        const float sc = scale_rule(bits_to_float(window), fmax, margin, scale[r]);
+        scale[r] = sc;
+        scale_inv[r] = __fdiv_rn(1.0f, sc);
+    }
 }
 
 // ------------------------------------------------- current scaling inside the cast
@@ -442,20 +513,31 @@ __global__ __launch_bounds__(kThreads) void parts_to_scale_kernel(const float *_
     dynamic_scale<FMT>(parts, margin, dyn_out, red);
 }
 
+// Per-tensor scale given (delayed scaling): the first block also hands back 1/scale, the factor the GEMM
+// multiplies by, in storage of the caller's.  The scale itself is refreshed in place after the step; a GEMM
+// of this step, or its backward, must not read the refreshed value.
+__device__ __forceinline__ void record_scale_inv(float s, float *__restrict__ scale_inv_out) {
+    if (scale_inv_out && blockIdx.x == 0 && threadIdx.x == 0) scale_inv_out[0] = __fdiv_rn(1.0f, s);
+}
+
 // ------------------------------------------------------------------------ cast
 // 16 elements per lane per step: two (bf16) or four (fp32) 16-byte loads, one
 // 16-byte store.  cols % 16 == 0 and 16-byte aligned pointers (host-checked).
 template <int SRC, int FMT, int MODE, bool AMAX>
 __global__ __launch_bounds__(AMAX ? kFatThreads : kThreads) void cast_kernel(const void *__restrict__ x, int64_t rows, int64_t cols,
                                                          const float *__restrict__ scale, uint8_t *__restrict__ out,
-                                                         float *__restrict__ amax_out, int margin, float *__restrict__ dyn_out) {
+                                                         float *__restrict__ amax_out, int margin, float *__restrict__ dyn_out,
+                                                         int amax_mask) {
     constexpr int kT = AMAX ? kFatThreads : kThreads;
     __shared__ uint32_t red[kT / kWave];
     const int64_t cpr = cols / 16;                           // chunks per row
     const int64_t nchunk = rows * cpr;
     const int64_t stride = (int64_t)gridDim.x * kT;
     float s_t = 1.0f;
-    if constexpr (MODE == ODL_SCALE_TENSOR) s_t = scale[0];
+    if constexpr (MODE == ODL_SCALE_TENSOR) {
+        s_t = scale[0];
+        record_scale_inv(s_t, dyn_out);
+    }
     if constexpr (MODE == kScaleParts) s_t = dynamic_scale<FMT>(scale, margin, dyn_out, red);
     uint32_t am = 0;
     for (int64_t i = (int64_t)blockIdx.x * kT + threadIdx.x; i < nchunk; i += stride) {
@@ -506,7 +588,7 @@ __global__ __launch_bounds__(AMAX ? kFatThreads : kThreads) void cast_kernel(con
     if constexpr (AMAX) {
         if constexpr (SRC == ODL_BF16) am = fold_u16x2_to_f32bits(am);
         am = block_max_u32(am, red);
-        if (threadIdx.x == 0 && am != 0) atomicMax(reinterpret_cast<uint32_t *>(amax_out), am);
+        if (threadIdx.x == 0 && am != 0) atomicMax(reinterpret_cast<uint32_t *>(amax_out) + (blockIdx.x & amax_mask), am);
     }
 }
 
@@ -588,11 +670,13 @@ template <int SRC, int FMT, int MODE, bool AMAX, bool WRITE_ROWMAJOR>
 __global__ __launch_bounds__(kThreads) void cast_transpose_kernel(const void *__restrict__ x, int64_t rows, int64_t cols,
                                                                    const float *__restrict__ scale,
                                                                    uint8_t *__restrict__ out, uint8_t *__restrict__ out_t,
-                                                                   float *__restrict__ amax_out, int margin, float *__restrict__ dyn_out) {
+                                                                   float *__restrict__ amax_out, int margin, float *__restrict__ dyn_out,
+                                                                   int amax_mask) {
     __shared__ __attribute__((aligned(16))) uint8_t tile[kTileC * kTileR];
     __shared__ uint32_t red[kThreads / kWave];
     float s_dyn = 1.0f;
     if constexpr (MODE == kScaleParts) s_dyn = dynamic_scale<FMT>(scale, margin, dyn_out, red);
+    if constexpr (MODE == ODL_SCALE_TENSOR) record_scale_inv(scale[0], dyn_out);
     constexpr int ESZ = SRC == ODL_BF16 ? 2 : 4;
     const int tx = threadIdx.x % 8;                 // 8 lanes across 64 columns
     const int ty = threadIdx.x / 8;                 // 32 lane-rows, 4 rows each
@@ -698,7 +782,7 @@ __global__ __launch_bounds__(kThreads) void cast_transpose_kernel(const void *__
     if constexpr (AMAX) {
         if constexpr (SRC == ODL_BF16) am = fold_u16x2_to_f32bits(am);
         am = block_max_u32(am, red);
-        if (threadIdx.x == 0 && am != 0) atomicMax(reinterpret_cast<uint32_t *>(amax_out), am);
+        if (threadIdx.x == 0 && am != 0) atomicMax(reinterpret_cast<uint32_t *>(amax_out) + (blockIdx.x & amax_mask), am);
     }
 }
 
@@ -894,14 +978,15 @@ extern "C" int odl_fp8_scale_from_amax(const float *amax, int64_t n, int fmt, in
 }
 
 extern "C" int odl_fp8_delayed_update(float *history, int64_t H, int64_t R, int64_t ld, float *scale, float *scale_inv,
-                                      const int *fmt, int margin, int algo, odl_stream_t stream_) {
+                                      const int *fmt, int margin, int algo, float *amax_parts, odl_stream_t stream_) {
     hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
     if (!history || !scale || !scale_inv || !fmt) return set_error(ODL_ERR_ARG, "odl_fp8_delayed_update: null pointer");
     if (H < 1 || R < 0 || ld < R) return set_error(ODL_ERR_ARG, "odl_fp8_delayed_update: H=%lld R=%lld ld=%lld", (long long)H, (long long)R, (long long)ld);
     if (algo != ODL_AMAX_MAX && algo != ODL_AMAX_MOST_RECENT) return set_error(ODL_ERR_ARG, "odl_fp8_delayed_update: algo %d", algo);
+    if (amax_parts && !aligned16(amax_parts)) return set_error(ODL_ERR_ARG, "odl_fp8_delayed_update: amax_parts must be 16-byte aligned");
     if (R == 0) return ODL_OK;
-    hipLaunchKernelGGL(delayed_update_kernel, dim3((unsigned)((R + 63) / 64)), dim3(64), 0, stream, history, H, R, ld, scale,
-                       scale_inv, fmt, margin, algo);
+    hipLaunchKernelGGL(delayed_update_kernel, dim3((unsigned)((R + kUpdRoles - 1) / kUpdRoles)), dim3(kThreads), 0, stream, history, H, R,
+                       ld, scale, scale_inv, fmt, margin, algo, amax_parts);
     return check_launch("odl_fp8_delayed_update");
 }
 
@@ -909,13 +994,13 @@ namespace odl {
 
 template <int SRC, int FMT, int MODE>
 static void launch_cast(const void *x, int64_t rows, int64_t cols, const float *scale, uint8_t *out, float *amax_out,
-                        hipStream_t stream, int margin = 0, float *dyn_out = nullptr) {
+                        hipStream_t stream, int margin = 0, float *dyn_out = nullptr, int amax_mask = 0) {
     if (amax_out) {
         const int64_t g = grid_for(rows * cols / 16, kFatThreads, 2);
-        hipLaunchKernelGGL((cast_kernel<SRC, FMT, MODE, true>), dim3((unsigned)g), dim3(kFatThreads), 0, stream, x, rows, cols, scale, out, amax_out, margin, dyn_out);
+        hipLaunchKernelGGL((cast_kernel<SRC, FMT, MODE, true>), dim3((unsigned)g), dim3(kFatThreads), 0, stream, x, rows, cols, scale, out, amax_out, margin, dyn_out, amax_mask);
     } else {
         const int64_t g = grid_for(rows * cols / 16, kThreads, 16);
-        hipLaunchKernelGGL((cast_kernel<SRC, FMT, MODE, false>), dim3((unsigned)g), dim3(kThreads), 0, stream, x, rows, cols, scale, out, amax_out, margin, dyn_out);
+        hipLaunchKernelGGL((cast_kernel<SRC, FMT, MODE, false>), dim3((unsigned)g), dim3(kThreads), 0, stream, x, rows, cols, scale, out, amax_out, margin, dyn_out, amax_mask);
     }
 }
 
@@ -936,10 +1021,12 @@ static void launch_generic(const void *x, int64_t rows, int64_t cols, const floa
 
 template <int SRC, int FMT, int MODE>
 static void launch_ct(const void *x, int64_t rows, int64_t cols, const float *scale, uint8_t *out, uint8_t *out_t,
-                      float *amax_out, hipStream_t stream, int margin = 0, float *dyn_out = nullptr) {
+                      float *amax_out, hipStream_t stream, int margin = 0, float *dyn_out = nullptr, int amax_mask = 0) {
     int64_t g = ((rows + kTileR - 1) / kTileR) * ((cols + kTileC - 1) / kTileC);
-    if (amax_out && g > (int64_t)num_cus() * 4) g = (int64_t)num_cus() * 4;
-#define ODL_CT(AM, RM) hipLaunchKernelGGL((cast_transpose_kernel<SRC, FMT, MODE, AM, RM>), dim3((unsigned)g), dim3(kThreads), 0, stream, x, rows, cols, scale, out, out_t, amax_out, margin, dyn_out)
+    // maxima folded into ONE word: few blocks that walk several tiles each, so that the kernel ends in few
+    // atomics on that word; spread over many words (amax_mask != 0), one tile per block as without a maximum
+    if (amax_out && amax_mask == 0 && g > (int64_t)num_cus() * 4) g = (int64_t)num_cus() * 4;
+#define ODL_CT(AM, RM) hipLaunchKernelGGL((cast_transpose_kernel<SRC, FMT, MODE, AM, RM>), dim3((unsigned)g), dim3(kThreads), 0, stream, x, rows, cols, scale, out, out_t, amax_out, margin, dyn_out, amax_mask)
     if (amax_out) { if (out) ODL_CT(true, true); else ODL_CT(true, false); }
     else { if (out) ODL_CT(false, true); else ODL_CT(false, false); }
 #undef ODL_CT
@@ -1001,6 +1088,44 @@ extern "C" int odl_fp8_cast_transpose(const void *x, int src_dtype, int64_t rows
     if (fast) ODL_DISPATCH_SRC_FMT(launch_ct_mode, mode, x, rows, cols, scale, out, out_t, amax_out, stream);
     else ODL_DISPATCH_SRC_FMT(launch_generic, x, rows, cols, scale, mode, out, out_t, amax_out, stream);
     return check_launch("odl_fp8_cast_transpose");
+}
+
+namespace odl {
+__global__ void scale_inv_kernel(const float *__restrict__ scale, float *__restrict__ scale_inv_out) {
+    scale_inv_out[0] = __fdiv_rn(1.0f, scale[0]);
+}
+
+template <int SRC, int FMT>
+static void launch_delayed(const void *x, int64_t rows, int64_t cols, const float *scale, uint8_t *out, uint8_t *out_t,
+                           float *amax_parts, float *scale_inv_out, bool fast, hipStream_t stream) {
+    if (!fast) {
+        // element-at-a-time route: the whole maximum goes into amax_parts[0]
+        launch_generic<SRC, FMT>(x, rows, cols, scale, ODL_SCALE_TENSOR, out, out_t, amax_parts, stream);
+        if (scale_inv_out) hipLaunchKernelGGL(scale_inv_kernel, dim3(1), dim3(1), 0, stream, scale, scale_inv_out);
+    } else if (out_t) {
+        launch_ct<SRC, FMT, ODL_SCALE_TENSOR>(x, rows, cols, scale, out, out_t, amax_parts, stream, 0, scale_inv_out, kAmaxParts - 1);
+    } else {
+        launch_cast<SRC, FMT, ODL_SCALE_TENSOR>(x, rows, cols, scale, out, amax_parts, stream, 0, scale_inv_out, kAmaxParts - 1);
+    }
+}
+}  // namespace odl
+
+extern "C" int odl_fp8_cast_delayed(const void *x, int src_dtype, int64_t rows, int64_t cols, const float *scale, int fmt,
+                                    uint8_t *out, uint8_t *out_t, float *amax_parts, float *scale_inv_out, odl_stream_t stream_) {
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    if (int e = check_cast_args("odl_fp8_cast_delayed", x, src_dtype, rows, cols, scale, ODL_SCALE_TENSOR, fmt)) return e;
+    if (!scale) return set_error(ODL_ERR_ARG, "odl_fp8_cast_delayed: scale is null");
+    if (rows * cols == 0) {                       // nothing to cast and nothing to record: only the inverse scale
+        if (scale_inv_out) hipLaunchKernelGGL(scale_inv_kernel, dim3(1), dim3(1), 0, stream, scale, scale_inv_out);
+        return check_launch("odl_fp8_cast_delayed");
+    }
+    if (!out && !out_t) return set_error(ODL_ERR_ARG, "odl_fp8_cast_delayed: out and out_t are both null");
+    const int64_t tiles = ((rows + kTileR - 1) / kTileR) * ((cols + kTileC - 1) / kTileC);
+    const bool fast = out_t ? (cols % 8 == 0 && rows % 16 == 0 && aligned16(x) && aligned16(out_t) &&
+                               (!out || (reinterpret_cast<uintptr_t>(out) & 7) == 0) && tiles <= 0x7fffffffLL)
+                            : (cols % 16 == 0 && aligned16(x) && aligned16(out));
+    ODL_DISPATCH_SRC_FMT(launch_delayed, x, rows, cols, scale, out, out_t, amax_parts, scale_inv_out, fast, stream);
+    return check_launch("odl_fp8_cast_delayed");
 }
 
 namespace odl {

@@ -232,7 +232,7 @@ class FP8Recipe:
         for arena in self._store.dirty_arenas(direction):
             R = arena.used
             native.delayed_update_raw(arena.history, arena.H, arena.capacity, R, arena.scale, arena.scale_inv,
-                                      arena.fmt, self.margin, algo)
+                                      arena.fmt, self.margin, algo, amax_parts=arena.parts)
             arena.dirty = False
             arena.epoch += 1
 
@@ -297,7 +297,7 @@ class FP8Recipe:
                 meta.scale_inv.copy_(blob["scale_inv"])
                 if blob.get("trained", True):
                     meta.first_record_epoch = -1
-        for arena in touched:          # codes and inverse-scale snapshots made under the old scales are stale
+        for arena in touched:          # codes made under the old scales are stale
             arena.epoch += 1
 
     # ------------------------------------------------------- producer hand-over

@@ -13,8 +13,10 @@ Design for one MI355X:
     in the autograd ``ctx`` and never depends on the ambient state;
   * all delayed-scaling roles of the modules that first ran under a recipe live in
     ONE arena per (recipe, device, direction): history [H, R], scale [R],
-    scale_inv [R].  Casts write their amax straight into row 0 of the arena and a
-    single tiny kernel refreshes every role of the model per step;
+    scale_inv [R], parts [R, 512].  Casts fold their block maxima into the role's
+    strip of partial maxima and hand back the inverse scale they used; a single small
+    kernel per arena folds the strips into row 0 and refreshes every role of the
+    model per step;
   * the scaling state belongs to the MODULES, as in the reference's backend (which
     keeps ``fp8_meta`` on each layer): a module finds its roles again by history
     length, formats and device, whatever recipe object is active.  The fresh recipe
@@ -31,6 +33,8 @@ import threading
 from typing import TYPE_CHECKING
 
 import torch
+
+from ... import native
 
 if TYPE_CHECKING:  # pragma: no cover
     from .fp8 import FP8Recipe
@@ -85,8 +89,12 @@ class ScalingMeta:
         return self.first_record_epoch is not None and self.arena.epoch > self.first_record_epoch
 
     @property
-    def amax_history(self) -> torch.Tensor:          # [H, n] view
+    def amax_history(self) -> torch.Tensor:          # [H, n] view; row 0 is filled by the refresh at the end of a step
         return self.arena.history[:, self.first:self.first + self.n]
+
+    @property
+    def pending_amax(self) -> torch.Tensor:          # [n]: amax per role of the step in progress (0 after a refresh)
+        return self.arena.parts[self.first:self.first + self.n].amax(dim=1)
 
     @property
     def scale(self) -> torch.Tensor:
@@ -96,8 +104,10 @@ class ScalingMeta:
     def scale_inv(self) -> torch.Tensor:
         return self.arena.scale_inv[self.first:self.first + self.n]
 
-    def amax_slot(self, role: int) -> torch.Tensor:   # 1-element view: where a cast records this step's amax
-        return self.arena.history[0, self.first + role:self.first + role + 1]
+    def amax_slot(self, role: int) -> torch.Tensor:
+        """Where the casts of the step in progress record the role's partial maxima (``native.AMAX_PARTS``
+        floats); the refresh folds them into row 0 of the history and clears them."""
+        return self.arena.parts[self.first + role]
 
     def scale_of(self, role: int) -> torch.Tensor:
         return self.arena.scale[self.first + role:self.first + role + 1]
@@ -105,15 +115,9 @@ class ScalingMeta:
     def scale_inv_of(self, role: int) -> torch.Tensor:
         return self.arena.scale_inv[self.first + role:self.first + role + 1]
 
-    def scale_inv_snapshot_of(self, role: int) -> torch.Tensor:
-        """The inverse scale in force now, in storage that the next refresh does not touch (what a
-        GEMM of this step, or its backward after the refresh, has to multiply by)."""
-        snap = self.arena.snapshot_inv()
-        return snap[self.first + role:self.first + role + 1]
-
 
 class MetaArena:
-    """history [H, cap], scale [cap], scale_inv [cap], fmt [cap] for one direction."""
+    """history [H, cap], scale [cap], scale_inv [cap], fmt [cap], parts [cap, AMAX_PARTS] for one direction."""
 
     def __init__(self, device: torch.device, history_len: int, capacity: int, direction: str = "fwd", owner=None):
         self.device, self.H, self.capacity = device, history_len, capacity
@@ -122,22 +126,12 @@ class MetaArena:
         self.scale = torch.ones(capacity, dtype=torch.float32, device=device)
         self.scale_inv = torch.ones(capacity, dtype=torch.float32, device=device)
         self.fmt = torch.zeros(capacity, dtype=torch.int32, device=device)
+        # partial maxima of the step in progress, AMAX_PARTS per role: the casts fold their block maxima into
+        # many words instead of one (same-address atomics retire one at a time), the refresh reduces them
+        self.parts = torch.zeros((capacity, native.AMAX_PARTS), dtype=torch.float32, device=device)
         self.used = 0
         self.dirty = False         # some cast wrote an amax since the last update
         self.epoch = 0             # bumped by every refresh of scale / scale_inv (they are updated in place)
-        self._snap: torch.Tensor | None = None
-        self._snap_epoch = -1
-
-    def snapshot_inv(self) -> torch.Tensor:
-        """A copy of ``scale_inv`` made once per epoch: one small copy per arena and step instead of one per
-        cast.  A copy of an earlier epoch lives on for as long as a saved tensor of that step refers to it."""
-        if self._snap is None or self._snap_epoch != self.epoch:
-            self._snap = self.scale_inv.clone()
-            self._snap_epoch = self.epoch
-        return self._snap
-
-    def invalidate_snapshot(self) -> None:
-        self._snap = None
 
     def reserve(self, fmts: list[int]) -> ScalingMeta | None:
         n = len(fmts)

@@ -116,7 +116,7 @@ def _converted_input(recipe: FP8Recipe, x2d: torch.Tensor, dtype: torch.dtype) -
 
 def _quantise_delayed(x2d: torch.Tensor, fmt: int, meta: "_state.ScalingMeta | None", role: int, need_t: bool,
                       need_rowmajor: bool = True, recipe: FP8Recipe | None = None, record: bool = True, margin: int = 0):
-    """Delayed scaling: one pass with the scale from the history, amax recorded in row 0.
+    """Delayed scaling: one pass with the scale from the history, this step's partial maxima recorded with the role.
     record=False (a module in eval mode): the scales that training arrived at are used as they are and
     the histories are left alone; roles that do not exist yet (meta None) or have never been through a
     refresh still stand at the initial scale 1 (a weight of std 0.02 would land in the subnormals), so
@@ -124,17 +124,12 @@ def _quantise_delayed(x2d: torch.Tensor, fmt: int, meta: "_state.ScalingMeta | N
     if not record and (meta is None or not meta.trained):
         q, q_t, scale_inv, _ = _quantise_dynamic(x2d, fmt, margin, need_t, need_rowmajor)
         return q, q_t, scale_inv
-    scale = meta.scale_of(role)
     slot = meta.amax_slot(role) if record else None
     if record:
         meta.note_record(recipe._store)
-    # the inverse scale comes from the arena's per-step snapshot: the arena entry itself changes at the next update
-    scale_inv = meta.scale_inv_snapshot_of(role)
-    if need_t:
-        q, q_t = native.cast_transpose(x2d, scale, fmt, T, amax_out=slot, want_rowmajor=need_rowmajor)
-    else:
-        q, q_t = native.cast(x2d, scale, fmt, T, amax_out=slot), None
-    return q, q_t, scale_inv
+    # the scale is refreshed in place after the step; the cast hands back the inverse of the one it used
+    return native.cast_delayed(x2d, meta.scale_of(role), fmt, amax_parts=slot, want_rowmajor=need_rowmajor or not need_t,
+                               want_transposed=need_t)
 
 
 def _quantise_axis(x2d: torch.Tensor, fmt: int, margin: int, mode: int, transposed: bool):

@@ -23,7 +23,7 @@ DT_BF16, DT_F32 = 0, 1
 AMAX_MAX, AMAX_MOST_RECENT = 0, 1
 FP8_MAX = {E4M3: 448.0, E5M2: 57344.0}
 TORCH_FP8 = {E4M3: torch.float8_e4m3fn, E5M2: torch.float8_e5m2}
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # ODL_FP8_LIB names another build of the same library (e.g. one made for an experiment)
@@ -52,6 +52,7 @@ EXPORTS = (
     "odl_fp8_cast_rowcol",
     "odl_fp8_cast",
     "odl_fp8_cast_transpose",
+    "odl_fp8_cast_delayed",
     "odl_fp8_gemm_nt",
     "odl_fp8_gemm_layouts",
     "odl_fp8_gemm_split_count",
@@ -112,12 +113,13 @@ def load() -> ctypes.CDLL:
         L.odl_fp8_cast_rowcol.argtypes = [vp, i32, i64, i64, vp, vp, i32, i32, vp, vp, vp, vp, vp, vp, vp]
         L.odl_fp8_cast.argtypes = [vp, i32, i64, i64, vp, i32, i32, vp, vp, vp]
         L.odl_fp8_cast_transpose.argtypes = [vp, i32, i64, i64, vp, i32, i32, vp, vp, vp, vp]
+        L.odl_fp8_cast_delayed.argtypes = [vp, i32, i64, i64, vp, i32, vp, vp, vp, vp, vp]
         L.odl_fp8_gemm_nt.argtypes = [vp, vp, i64, i64, i64, i32, i32, vp, i64, vp, i64, vp, i32, vp, i32, vp]
         L.odl_fp8_gemm_layouts.argtypes = [vp, vp, i64, i64, i64, i32, i32, i32, i32, vp, vp, vp, i32, vp]
         L.odl_fp8_gemm_split_count.argtypes = [i64, i64, i64, i32]
         L.odl_fp8_gemm_split_count.restype = i32
         L.odl_fp8_gemm_splitk.argtypes = [vp, vp, i64, i64, i64, i32, i32, i32, i32, vp, i64, vp, i64, vp, vp, i32, i32, vp, i64, vp]
-        L.odl_fp8_delayed_update.argtypes = [vp, i64, i64, i64, vp, vp, vp, i32, i32, vp]
+        L.odl_fp8_delayed_update.argtypes = [vp, i64, i64, i64, vp, vp, vp, i32, i32, vp, vp]
         L.odl_fp8_gemm_num_variants.restype = i32
         L.odl_fp8_gemm_variant_name.argtypes = [i32]
         L.odl_fp8_gemm_variant_name.restype = ctypes.c_char_p
@@ -558,6 +560,34 @@ def cast_transpose(x: torch.Tensor, scale: torch.Tensor, fmt: int, mode: int = S
     return out, out_t
 
 
+AMAX_PARTS = 512                       # ODL_FP8_AMAX_PARTS
+
+
+def cast_delayed(x: torch.Tensor, scale: torch.Tensor, fmt: int, amax_parts: torch.Tensor | None = None,
+                 want_rowmajor: bool = True, want_transposed: bool = False):
+    """The cast of the delayed-scaling recipe, one launch: codes with the per-tensor ``scale`` in force
+    (row-major, transposed, or both), this step's partial maxima folded into ``amax_parts``
+    (AMAX_PARTS floats of a role, accumulated, cleared by the next ``delayed_update``; None: nothing is
+    recorded), and 1/scale in a fresh 1-element tensor that later refreshes of ``scale`` do not touch.
+    -> (codes or None, codes_t or None, scale_inv[1])."""
+    x = _as_2d(x)
+    rows, cols = x.shape
+    _f32_dev(scale, 1, "cast_delayed scale")
+    if amax_parts is not None:
+        _f32_dev(amax_parts, AMAX_PARTS, "cast_delayed amax_parts")
+    if not (want_rowmajor or want_transposed):
+        raise NativeError("cast_delayed: neither layout asked for")
+    out = torch.empty((rows, cols), dtype=torch.uint8, device=x.device) if want_rowmajor else None
+    out_t = torch.empty((cols, rows), dtype=torch.uint8, device=x.device) if want_transposed else None
+    scale_inv = torch.empty(1, dtype=torch.float32, device=x.device)
+    _check(load().odl_fp8_cast_delayed(x.data_ptr(), _src_dtype(x), rows, cols, scale.data_ptr(), fmt,
+                                       out.data_ptr() if out is not None else None,
+                                       out_t.data_ptr() if out_t is not None else None,
+                                       amax_parts.data_ptr() if amax_parts is not None else None, scale_inv.data_ptr(), _stream()),
+           "odl_fp8_cast_delayed")
+    return out, out_t, scale_inv
+
+
 def gemm_nt(a: torch.Tensor, b: torch.Tensor, fmt_a: int, fmt_b: int, sa_inv: torch.Tensor, sb_inv: torch.Tensor,
             bias: torch.Tensor | None = None, out_dtype: torch.dtype = torch.bfloat16,
             out: torch.Tensor | None = None) -> torch.Tensor:
@@ -676,22 +706,17 @@ def gemm_layouts(a: torch.Tensor, b: torch.Tensor, fmt_a: int, fmt_b: int, layou
 
 
 def delayed_update(history: torch.Tensor, scale: torch.Tensor, scale_inv: torch.Tensor, fmts: torch.Tensor,
-                   margin: int = 0, algo: int = AMAX_MAX) -> None:
-    """In place: history[H,R] fp32, scale[R], scale_inv[R] fp32, fmts[R] int32 (all on the GPU)."""
+                   margin: int = 0, algo: int = AMAX_MAX, amax_parts: torch.Tensor | None = None) -> None:
+    """In place: history[H,R] fp32, scale[R], scale_inv[R] fp32, fmts[R] int32 (all on the GPU);
+    amax_parts [R, AMAX_PARTS] (optional): partial maxima of this step, folded into history[0] and cleared."""
     if history.dim() != 2:
         raise NativeError("delayed_update: history must be [H, R]")
     H, R = history.shape
-    _f32_dev(history, H * R, "delayed_update history")
-    _f32_dev(scale, R, "delayed_update scale")
-    _f32_dev(scale_inv, R, "delayed_update scale_inv")
-    if not (fmts.is_cuda and fmts.dtype == torch.int32 and fmts.numel() == R and fmts.is_contiguous()):
-        raise NativeError("delayed_update: fmts must be a contiguous int32 CUDA tensor with R entries")
-    _check(load().odl_fp8_delayed_update(history.data_ptr(), H, R, R, scale.data_ptr(), scale_inv.data_ptr(), fmts.data_ptr(),
-                                         margin, algo, _stream()), "odl_fp8_delayed_update")
+    delayed_update_raw(history, H, R, R, scale, scale_inv, fmts, margin, algo, amax_parts)
 
 
 def delayed_update_raw(history: torch.Tensor, H: int, ld: int, R: int, scale: torch.Tensor, scale_inv: torch.Tensor,
-                       fmts: torch.Tensor, margin: int, algo: int) -> None:
+                       fmts: torch.Tensor, margin: int, algo: int, amax_parts: torch.Tensor | None = None) -> None:
     """Same update on the first R roles of an arena whose rows are ld >= R wide."""
     if not (history.is_cuda and history.dtype == torch.float32 and history.is_contiguous() and history.numel() == H * ld):
         raise NativeError("delayed_update_raw: history must be a contiguous fp32 CUDA tensor of H*ld elements")
@@ -700,8 +725,12 @@ def delayed_update_raw(history: torch.Tensor, H: int, ld: int, R: int, scale: to
             raise NativeError(f"delayed_update_raw: {name} must be a contiguous fp32 CUDA tensor with >= R entries")
     if not (fmts.is_cuda and fmts.dtype == torch.int32 and fmts.is_contiguous() and fmts.numel() >= R):
         raise NativeError("delayed_update_raw: fmts must be a contiguous int32 CUDA tensor with >= R entries")
+    if amax_parts is not None and not (amax_parts.is_cuda and amax_parts.dtype == torch.float32 and amax_parts.is_contiguous()
+                                       and amax_parts.numel() >= R * AMAX_PARTS):
+        raise NativeError("delayed_update_raw: amax_parts must be a contiguous fp32 CUDA tensor with >= R * AMAX_PARTS entries")
     _check(load().odl_fp8_delayed_update(history.data_ptr(), H, R, ld, scale.data_ptr(), scale_inv.data_ptr(),
-                                         fmts.data_ptr(), margin, algo, _stream()), "odl_fp8_delayed_update")
+                                         fmts.data_ptr(), margin, algo,
+                                         amax_parts.data_ptr() if amax_parts is not None else None, _stream()), "odl_fp8_delayed_update")
 
 
 def gemm_variants() -> list[str]:

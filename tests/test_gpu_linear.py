@@ -146,15 +146,18 @@ def test_history_has_a_value_after_one_step_like_the_reference_test(amp):
     recipe = amp.create_fp8_recipe("delayed", "hybrid", amax_history_len=16)
     lin = TELinear(32, 64).to("cuda", torch.bfloat16)
     x = torch.randn(16, 32, device="cuda", dtype=torch.bfloat16, requires_grad=True)
-    # amaxes are recorded during the step and rolled on context exit; look before the exit
+    # during the step the casts' maxima wait with the roles; leaving the context folds them into the history and rolls it
     with recipe.autocast():
         y = lin(x)
-        hist = lin._te_linear.fp8_meta["scaling_fwd"].amax_history
-        assert hist.dim() == 2 and hist.shape == (16, 3) and (hist > 0).any()
+        meta = lin._te_linear.fp8_meta["scaling_fwd"]
+        assert meta.pending_amax.shape == (3,) and (meta.pending_amax > 0).sum() == 2      # input and weight; the output role is unused
+        assert not (meta.amax_history > 0).any()
+    hist = lin._te_linear.fp8_meta["scaling_fwd"].amax_history
+    assert hist.dim() == 2 and hist.shape == (16, 3) and (hist > 0).any() and not meta.pending_amax.any()
     with recipe.backward():
         y.sum().backward()
-        hb = lin.fp8_meta["scaling_bwd"].amax_history
-        assert hb.shape == (16, 2) and (hb > 0).any()
+    hb = lin.fp8_meta["scaling_bwd"].amax_history
+    assert hb.shape == (16, 2) and (hb > 0).any()
     assert (lin.fp8_meta["scaling_fwd"].amax_history > 0).any() and x.grad is not None and lin.weight.grad is not None
 
 

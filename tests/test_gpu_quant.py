@@ -220,6 +220,54 @@ def test_cast_with_fused_amax_for_delayed_scaling(N, fmt):
         assert_f32_bits_equal(slot, torch.maximum(O.t_amax(x), O.t_amax(y)), "amax slot folds")
 
 
+@pytest.mark.parametrize("fmt", [O.E4M3, O.E5M2])
+@pytest.mark.parametrize("shape", [(512, 384), (2048, 1536), (48, 40), (17, 16)])
+def test_cast_delayed_codes_partial_maxima_and_inverse_scale(N, fmt, shape):
+    """The one-launch cast of the delayed recipe: codes as odl_fp8_cast / _cast_transpose with the same scale (the oracle's
+    cast), the maximum of the recorded partial maxima equal to the tensor's amax, 1/scale by IEEE division; a second cast
+    into the same strip accumulates; nothing is recorded without a strip.  (48, 40) and (17, 16) take the
+    element-at-a-time route (rows not a multiple of 16 / columns not of 16)."""
+    x = seeded_bf16(shape, std=2.0, seed=11)
+    stale = torch.tensor([O.FP8_MAX[fmt] / 3.0])                                   # smaller amax than the data: clamps
+    want = O.t_cast(x, stale, fmt)
+    inv = torch.tensor([np.float32(1.0) / np.float32(stale.item())])
+    for rm, t in ((True, False), (True, True), (False, True)):
+        parts = torch.zeros(N.AMAX_PARTS, device="cuda")
+        q, qt, s_inv = N.cast_delayed(x.cuda(), stale.cuda(), fmt, amax_parts=parts, want_rowmajor=rm, want_transposed=t)
+        assert (q is None) == (not rm) and (qt is None) == (not t)
+        if rm:
+            assert_bytes_equal(q, want, f"row-major codes {shape}")
+        if t:
+            assert_bytes_equal(qt, want.t().contiguous(), f"transposed codes {shape}")
+        assert_f32_bits_equal(s_inv, inv, "inverse scale")
+        assert_f32_bits_equal(parts.max().reshape(1), O.t_amax(x), "maximum of the partial maxima")
+        y = seeded_bf16(shape, std=0.5, seed=12)
+        y[0, 0] = 300.0
+        N.cast_delayed(y.cuda(), stale.cuda(), fmt, amax_parts=parts, want_rowmajor=rm, want_transposed=t)
+        assert_f32_bits_equal(parts.max().reshape(1), torch.tensor([300.0]), "a second cast accumulates")
+    q, _, s_inv = N.cast_delayed(x.cuda(), stale.cuda(), fmt)                        # eval mode: nothing recorded
+    assert_bytes_equal(q, want, "codes without a strip")
+    assert_f32_bits_equal(s_inv, inv, "inverse scale without a strip")
+    # fp32 source
+    q, qt, _ = N.cast_delayed(x.float().cuda(), stale.cuda(), fmt, want_transposed=True)
+    assert_bytes_equal(q, want, "fp32 source")
+    assert_bytes_equal(qt, want.t().contiguous(), "fp32 source, transposed")
+
+
+def test_cast_delayed_spreads_the_maxima_of_a_large_tensor(N):
+    """8192 x 4096: 4096 tiles of the cast+transpose kernel fold into 512 words; the amax sits in the very last tile."""
+    x = seeded_bf16((8192, 4096), seed=3).cuda()
+    x[8191, 4095] = 123.0
+    s = torch.tensor([2.0], device="cuda")
+    for t in (False, True):
+        parts = torch.zeros(N.AMAX_PARTS, device="cuda")
+        q, qt, _ = N.cast_delayed(x, s, O.E4M3, amax_parts=parts, want_transposed=t)
+        assert parts.max().item() == 123.0 and (parts > 0).sum().item() > 64
+        assert torch.equal(q, N.cast(x, s, O.E4M3))
+        if t:
+            assert torch.equal(qt, q.t().contiguous())
+
+
 def test_cast_transpose_large_matches_cast_then_transpose(N):
     """Size-independent property at a full benchmark shape: out_t == out^T bytewise."""
     x = seeded_bf16((8192, 4096), seed=0).cuda()
@@ -258,6 +306,38 @@ def test_delayed_update_matches_oracle(N):
             assert_f32_bits_equal(dh, torch.from_numpy(hist), f"history step {step} {algo_name}")
             assert_f32_bits_equal(ds, torch.from_numpy(scale), f"scale step {step} {algo_name}")
             assert_f32_bits_equal(di, torch.from_numpy(inv), f"scale_inv step {step} {algo_name}")
+
+@pytest.mark.parametrize("H,R", [(1, 3), (2, 17), (15, 16), (16, 40), (17, 5), (33, 1), (64, 33), (1024, 21)])
+@pytest.mark.parametrize("algo_name,algo", [("max", 0), ("most_recent", 1)])
+def test_delayed_update_every_history_length_with_partial_maxima(N, H, R, algo_name, algo):
+    """History lengths around the 16 lanes that share a role (one row per lane, several, a ragged last segment, the
+    reference's default of 1024), role counts around the 16 roles of a block, the step's amax arriving as partial maxima
+    (folded into row 0 and cleared) or directly in row 0, against the oracle value for value."""
+    rng = np.random.default_rng(H * 131 + R)
+    fmts = [int(f) for f in rng.integers(0, 2, R)]
+    hist = np.abs(rng.normal(0, 1, (H, R))).astype(np.float32)                      # a full window to start with
+    hist[0] = 0
+    scale, inv = np.ones(R, dtype=np.float32), np.ones(R, dtype=np.float32)
+    dh, ds, di = torch.from_numpy(hist.copy()).cuda(), torch.from_numpy(scale.copy()).cuda(), torch.from_numpy(inv.copy()).cuda()
+    dfm = torch.tensor(fmts, dtype=torch.int32).cuda()
+    parts = torch.zeros((R, N.AMAX_PARTS), device="cuda")
+    for step in range(H + 3 if H <= 64 else 6):
+        new = np.abs(rng.normal(0, 1 + step * 0.1, R)).astype(np.float32)
+        if step == 2:
+            new[0] = 0.0
+        direct = np.where(rng.random(R) < 0.5, new, 0).astype(np.float32)            # some roles in row 0, some as partials
+        dh[0] = torch.from_numpy(direct).cuda()
+        where = torch.from_numpy(rng.integers(0, N.AMAX_PARTS, R)).cuda()
+        parts[torch.arange(R, device="cuda"), where] = torch.from_numpy(new).cuda()
+        parts[:, 7] = torch.maximum(parts[:, 7], torch.from_numpy(new * 0.5).cuda())  # a smaller entry elsewhere in the strip
+        hist[0] = new
+        O.c_delayed_update(hist, scale, inv, fmts, margin=0, algo=algo_name)
+        N.delayed_update(dh, ds, di, dfm, margin=0, algo=algo, amax_parts=parts)
+        assert_f32_bits_equal(dh, torch.from_numpy(hist), f"history step {step}")
+        assert_f32_bits_equal(ds, torch.from_numpy(scale), f"scale step {step}")
+        assert_f32_bits_equal(di, torch.from_numpy(inv), f"scale_inv step {step}")
+        assert not parts.any(), "the partial maxima are cleared"
+
 
 
 def test_bad_arguments_are_refused(N):
