@@ -326,8 +326,9 @@ def llama_block(torch, steps=6, warmup=2):
 def whole_models(torch, which=("gpt2_124m", "qwen3_0.6b"), steps=5, warmup=3, labels=None):
     """The reference's own small presets as whole models (GPT-2 124M at 16 x 1024 tokens, Qwen3-0.6B at 4 x 2048;
     fp32 master weights, random init, random tokens): forward + cross-entropy + backward, weights re-quantised every
-    step.  bf16 autocast, the FP8 Linears alone, and the default transform (fused norms / activations as well);
-    attention and the loss are PyTorch's in all three."""
+    step.  bf16 autocast, the FP8 Linears alone, the default transform (fused norms / activations as well), and the same
+    with the weights quantised by the `fp8.param` set (two launches per step for all of them); attention and the loss are
+    PyTorch's in all four."""
     import torch.nn.functional as F
 
     from optimus_dl_amd.modules import amp as A
@@ -346,7 +347,8 @@ def whole_models(torch, which=("gpt2_124m", "qwen3_0.6b"), steps=5, warmup=3, la
         out[name] = {}
         for label, cfg in (("bf16_autocast", None),
                            ("fp8_linears", {"_name": "fp8_linear", "replace_norm": False, "fuse_swiglu": False, "fuse_gelu": False}),
-                           ("fp8_linears_fused_producers", {"_name": "fp8_linear"})):
+                           ("fp8_linears_fused_producers", {"_name": "fp8_linear"}),
+                           ("fp8_linears_fused_producers_param_set", {"_name": "fp8_linear"})):
             if labels is not None and label not in labels:
                 continue
             model, B, T, V = make(name)
@@ -354,15 +356,20 @@ def whole_models(torch, which=("gpt2_124m", "qwen3_0.6b"), steps=5, warmup=3, la
             if cfg:
                 build_model_transform(cfg).apply(model)
             recipe = A.FP8Recipe(recipe_type="tensorwise")
+            # `fp8.param`: all weights re-quantised in two launches per step instead of two per weight
+            param_set = recipe.attach_params(model) if label.endswith("param_set") else None
             ids = torch.randint(0, V, (B, T), device="cuda")
             tgt = torch.randint(0, V, (B * T,), device="cuda")
 
             def one():
                 for p_ in model.parameters():
                     p_.grad = None
-                for m in model.modules():
-                    if hasattr(m, "_wcache"):
-                        m._wcache.key = None
+                if param_set is not None:
+                    param_set.sync()                 # where the optimizer step's hook would run it
+                else:
+                    for m in model.modules():
+                        if hasattr(m, "_wcache"):
+                            m._wcache.key = None
                 if cfg:
                     with A.fp8_autocast(torch.device("cuda"), recipe):
                         loss = F.cross_entropy(model(ids)["logits"].view(-1, V).float(), tgt)

@@ -45,7 +45,7 @@ enum odl_status {
     ODL_ERR_LAUNCH = 3    /* HIP reported an error at launch */
 };
 
-/* ABI version of this header (8); bumped when a signature changes or an entry point is added. */
+/* ABI version of this header (9); bumped when a signature changes or an entry point is added. */
 int odl_fp8_abi_version(void);
 
 /* Last error message of the calling host thread ("" if none). */
@@ -102,6 +102,38 @@ int odl_fp8_amax_parts(const void *x, int src_dtype, int64_t rows, int64_t cols,
 int odl_fp8_cast_dynamic(const void *x, int src_dtype, int64_t rows, int64_t cols, const float *parts,
                          int fmt, int margin, uint8_t *out, uint8_t *out_t, float *dyn_out,
                          odl_stream_t stream);
+
+/*
+ * Current scaling of MANY tensors in two launches: every weight of a model after an optimizer step (what
+ * te.pytorch.Linear does per weight and forward, transformer_engine.py:106; `fp8.param`, optim/config.py:36-37,
+ * asks for weights that are kept quantised between steps).  Results per tensor are those of odl_fp8_amax_parts +
+ * odl_fp8_cast_dynamic with both outputs, bit for bit.
+ *   odl_fp8_mt_tensor : one tensor; the table of n of them is read by the kernels from DEVICE memory.
+ *   odl_fp8_multi_plan: host only.  Checks a HOST copy of the table (rows a positive multiple of 16, cols of 8;
+ *                       x, out_t, parts 16-byte aligned, out 8-byte, no NULL) and writes the work list of a phase,
+ *                       pairs {tensor, local index} of int32, into `work` (host memory, room for `capacity` pairs;
+ *                       NULL or too small: only counts).  Returns the number of pairs, -1 on error.  Tables and work
+ *                       lists depend on addresses and shapes only: build them once, copy them to the device.
+ *   odl_fp8_multi_amax_parts  (phase ODL_MT_AMAX): parts of every tensor <- its partial maxima.
+ *   odl_fp8_multi_cast_dynamic (phase ODL_MT_CAST): codes, transposed codes and dyn_out = {amax, scale, 1/scale}
+ *                       of every tensor, one format and margin for all.
+ * Nothing is allocated; the device tables are not validated again at launch.
+ */
+typedef struct odl_fp8_mt_tensor {
+    const void *x;      /* source [rows, cols], src_dtype */
+    uint8_t *out;       /* codes [rows, cols] */
+    uint8_t *out_t;     /* codes [cols, rows] */
+    float *parts;       /* ODL_FP8_AMAX_PARTS floats */
+    float *dyn_out;     /* 3 floats */
+    int64_t rows, cols;
+    int32_t src_dtype;  /* odl_dtype */
+    int32_t reserved;   /* 0 */
+} odl_fp8_mt_tensor;    /* 64 bytes */
+enum odl_mt_phase { ODL_MT_AMAX = 0, ODL_MT_CAST = 1 };
+int64_t odl_fp8_multi_plan(const odl_fp8_mt_tensor *tensors_host, int64_t n, int phase, int32_t *work_host, int64_t capacity);
+int odl_fp8_multi_amax_parts(const odl_fp8_mt_tensor *tensors_dev, const int32_t *work_dev, int64_t n_work, odl_stream_t stream);
+int odl_fp8_multi_cast_dynamic(const odl_fp8_mt_tensor *tensors_dev, const int32_t *work_dev, int64_t n_work, int fmt, int margin,
+                               odl_stream_t stream);
 
 /*
  * odl_fp8_amax_parts + odl_fp8_cast_dynamic in one call that ALLOCATES NOTHING and takes no workspace:

@@ -62,15 +62,12 @@ struct FusedScale {
 // maximum, no atomics at all: the cast that follows reduces the kAmaxParts partials itself.
 constexpr int kAmaxParts = ODL_FP8_AMAX_PARTS;
 
-template <int SRC, int UNROLL, int OUT>
-__global__ __launch_bounds__(kFatThreads) void amax_tensor_kernel(const void *__restrict__ x, int64_t n,
-                                                                   float *__restrict__ out, const FusedScale fs) {
-    __shared__ uint32_t red[kFatThreads / kWave];
-    constexpr int EPC = SRC == ODL_BF16 ? 8 : 4;          // elements per 16-byte chunk
-    const int64_t n16 = n / EPC;
+// Maximum of |x| over the 16-byte chunks i0, i0 + stride, ... < n16 of x, as fp32 magnitude bits; UNROLL loads
+// in flight per lane.
+template <int SRC, int UNROLL>
+__device__ __forceinline__ uint32_t amax_chunks(const void *__restrict__ x, int64_t n16, int64_t i0, int64_t stride) {
     const u32x4 *p = reinterpret_cast<const u32x4 *>(x);
-    const int64_t stride = (int64_t)gridDim.x * kFatThreads;
-    int64_t i = (int64_t)blockIdx.x * kFatThreads + threadIdx.x;
+    int64_t i = i0;
     uint32_t m0 = 0, m1 = 0, m2 = 0, m3 = 0;
     for (; i + (UNROLL - 1) * stride < n16; i += UNROLL * stride) {
         u32x4 v[UNROLL];
@@ -105,12 +102,17 @@ __global__ __launch_bounds__(kFatThreads) void amax_tensor_kernel(const void *__
             m3 = max(m3, v.w & 0x7fffffffu);
         }
     }
-    uint32_t m;
-    if constexpr (SRC == ODL_BF16) {
-        m = fold_u16x2_to_f32bits(max_u16x2(max_u16x2(m0, m1), max_u16x2(m2, m3)));
-    } else {
-        m = max(max(m0, m1), max(m2, m3));
-    }
+    if constexpr (SRC == ODL_BF16) return fold_u16x2_to_f32bits(max_u16x2(max_u16x2(m0, m1), max_u16x2(m2, m3)));
+    else return max(max(m0, m1), max(m2, m3));
+}
+
+template <int SRC, int UNROLL, int OUT>
+__global__ __launch_bounds__(kFatThreads) void amax_tensor_kernel(const void *__restrict__ x, int64_t n,
+                                                                   float *__restrict__ out, const FusedScale fs) {
+    __shared__ uint32_t red[kFatThreads / kWave];
+    constexpr int EPC = SRC == ODL_BF16 ? 8 : 4;          // elements per 16-byte chunk
+    const int64_t n16 = n / EPC;
+    uint32_t m = amax_chunks<SRC, UNROLL>(x, n16, (int64_t)blockIdx.x * kFatThreads + threadIdx.x, (int64_t)gridDim.x * kFatThreads);
     // scalar tail (fewer than EPC elements), done by one thread
     if (blockIdx.x == 0 && threadIdx.x == 0) {
         for (int64_t t = n16 * EPC; t < n; ++t) {
@@ -487,7 +489,7 @@ constexpr int kScaleParts = 3;
 
 template <int FMT>
 __device__ __forceinline__ float dynamic_scale(const float *__restrict__ parts, int margin, float *__restrict__ dyn_out,
-                                               uint32_t *red) {
+                                               uint32_t *red, bool record) {
     __shared__ float s_bcast;
     uint32_t m = 0;
     for (int i = threadIdx.x; i < kAmaxParts; i += blockDim.x) m = max(m, float_to_bits(parts[i]));
@@ -496,7 +498,7 @@ __device__ __forceinline__ float dynamic_scale(const float *__restrict__ parts, 
         const float amax = bits_to_float(m);
         const float sc = scale_rule(amax, Fp8Lim<FMT>::max, margin, 1.0f);
         s_bcast = sc;
-        if (blockIdx.x == 0 && dyn_out) {
+        if (record && dyn_out) {
             dyn_out[0] = amax;
             dyn_out[1] = sc;
             dyn_out[2] = __fdiv_rn(1.0f, sc);
@@ -510,7 +512,7 @@ __device__ __forceinline__ float dynamic_scale(const float *__restrict__ parts, 
 template <int FMT>
 __global__ __launch_bounds__(kThreads) void parts_to_scale_kernel(const float *__restrict__ parts, int margin, float *__restrict__ dyn_out) {
     __shared__ uint32_t red[kThreads / kWave];
-    dynamic_scale<FMT>(parts, margin, dyn_out, red);
+    dynamic_scale<FMT>(parts, margin, dyn_out, red, true);
 }
 
 // Per-tensor scale given (delayed scaling): the first block also hands back 1/scale, the factor the GEMM
@@ -538,7 +540,7 @@ __global__ __launch_bounds__(AMAX ? kFatThreads : kThreads) void cast_kernel(con
         s_t = scale[0];
         record_scale_inv(s_t, dyn_out);
     }
-    if constexpr (MODE == kScaleParts) s_t = dynamic_scale<FMT>(scale, margin, dyn_out, red);
+    if constexpr (MODE == kScaleParts) s_t = dynamic_scale<FMT>(scale, margin, dyn_out, red, blockIdx.x == 0);
     uint32_t am = 0;
     for (int64_t i = (int64_t)blockIdx.x * kT + threadIdx.x; i < nchunk; i += stride) {
         float f[16];
@@ -666,31 +668,16 @@ __device__ __forceinline__ void transpose4x4(const uint32_t a[4], uint32_t t[4])
     t[3] = __builtin_amdgcn_perm(p23_hi, p01_hi, 0x07060302u);
 }
 
+// One 128 x 64 tile (tr, tc) of x: convert, write the row-major codes, transpose through `tile` (LDS), write the
+// transposed codes.  `st` is the per-tensor scale (modes TENSOR and parts), `scale` the vector of the ROW / COL modes.
+// Ends after the transposed stores: a caller that reuses `tile` puts a barrier in between.
 template <int SRC, int FMT, int MODE, bool AMAX, bool WRITE_ROWMAJOR>
-__global__ __launch_bounds__(kThreads) void cast_transpose_kernel(const void *__restrict__ x, int64_t rows, int64_t cols,
-                                                                   const float *__restrict__ scale,
-                                                                   uint8_t *__restrict__ out, uint8_t *__restrict__ out_t,
-                                                                   float *__restrict__ amax_out, int margin, float *__restrict__ dyn_out,
-                                                                   int amax_mask) {
-    __shared__ __attribute__((aligned(16))) uint8_t tile[kTileC * kTileR];
-    __shared__ uint32_t red[kThreads / kWave];
-    float s_dyn = 1.0f;
-    if constexpr (MODE == kScaleParts) s_dyn = dynamic_scale<FMT>(scale, margin, dyn_out, red);
-    if constexpr (MODE == ODL_SCALE_TENSOR) record_scale_inv(scale[0], dyn_out);
+__device__ __forceinline__ void ct_one_tile(const void *__restrict__ x, int64_t rows, int64_t cols, const float *__restrict__ scale,
+                                            float st, uint8_t *__restrict__ out, uint8_t *__restrict__ out_t, int64_t tr,
+                                            int64_t tc, uint8_t *tile, uint32_t &am) {
     constexpr int ESZ = SRC == ODL_BF16 ? 2 : 4;
     const int tx = threadIdx.x % 8;                 // 8 lanes across 64 columns
     const int ty = threadIdx.x / 8;                 // 32 lane-rows, 4 rows each
-    const int64_t tiles_c = (cols + kTileC - 1) / kTileC;
-    const int64_t ntiles = tiles_c * ((rows + kTileR - 1) / kTileR);
-    uint32_t am = 0;
-    // With a fused amax the grid is small and each block walks several tiles, so
-    // that the kernel ends in few atomics; otherwise one tile per block.
-    for (int64_t tile_id = blockIdx.x; tile_id < ntiles; tile_id += gridDim.x) {
-    // Tiles are walked from the end of the tensor: the amax pass that ran just before read it front
-    // to back, so its tail is what the memory-side cache still holds.
-    const int64_t rev = ntiles - 1 - tile_id;
-    int64_t tr, tc;
-    ct_tile_of(rev, (rows + kTileR - 1) / kTileR, tiles_c, tr, tc);
     const int64_t r0 = tr * kTileR + ty * 4, c0 = tc * kTileC + tx * 8;
     const bool col_ok = c0 < cols;                  // cols % 8 == 0 (host-checked), so the whole 8-wide patch is in or out
 
@@ -698,7 +685,6 @@ __global__ __launch_bounds__(kThreads) void cast_transpose_kernel(const void *__
 #pragma unroll
     for (int j = 0; j < 8; ++j) s_col[j] = 1.0f;
     if constexpr (MODE == ODL_SCALE_TENSOR || MODE == kScaleParts) {
-        const float st = MODE == kScaleParts ? s_dyn : scale[0];
 #pragma unroll
         for (int j = 0; j < 8; ++j) s_col[j] = st;
     } else if constexpr (MODE == ODL_SCALE_COL) {
@@ -777,7 +763,34 @@ __global__ __launch_bounds__(kThreads) void cast_transpose_kernel(const void *__
             __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(out_t + oc * rows + orow));
         }
     }
-    if (tile_id + gridDim.x < ntiles) __syncthreads();  // the LDS tile is reused by the next trip
+}
+
+template <int SRC, int FMT, int MODE, bool AMAX, bool WRITE_ROWMAJOR>
+__global__ __launch_bounds__(kThreads) void cast_transpose_kernel(const void *__restrict__ x, int64_t rows, int64_t cols,
+                                                                   const float *__restrict__ scale,
+                                                                   uint8_t *__restrict__ out, uint8_t *__restrict__ out_t,
+                                                                   float *__restrict__ amax_out, int margin, float *__restrict__ dyn_out,
+                                                                   int amax_mask) {
+    __shared__ __attribute__((aligned(16))) uint8_t tile[kTileC * kTileR];
+    __shared__ uint32_t red[kThreads / kWave];
+    float st = 1.0f;
+    if constexpr (MODE == kScaleParts) st = dynamic_scale<FMT>(scale, margin, dyn_out, red, blockIdx.x == 0);
+    if constexpr (MODE == ODL_SCALE_TENSOR) {
+        st = scale[0];
+        record_scale_inv(st, dyn_out);
+    }
+    const int64_t tiles_c = (cols + kTileC - 1) / kTileC;
+    const int64_t ntiles = tiles_c * ((rows + kTileR - 1) / kTileR);
+    uint32_t am = 0;
+    // With a maximum folded into one word the grid is small and each block walks several tiles, so
+    // that the kernel ends in few atomics; otherwise one tile per block.
+    for (int64_t tile_id = blockIdx.x; tile_id < ntiles; tile_id += gridDim.x) {
+        // Tiles are walked from the end of the tensor: the amax pass that ran just before read it front
+        // to back, so its tail is what the memory-side cache still holds.
+        int64_t tr, tc;
+        ct_tile_of(ntiles - 1 - tile_id, (rows + kTileR - 1) / kTileR, tiles_c, tr, tc);
+        ct_one_tile<SRC, FMT, MODE, AMAX, WRITE_ROWMAJOR>(x, rows, cols, scale, st, out, out_t, tr, tc, tile, am);
+        if (tile_id + gridDim.x < ntiles) __syncthreads();  // the LDS tile is reused by the next trip
     }
     if constexpr (AMAX) {
         if constexpr (SRC == ODL_BF16) am = fold_u16x2_to_f32bits(am);
@@ -1187,6 +1200,99 @@ extern "C" int odl_fp8_cast_dynamic(const void *x, int src_dtype, int64_t rows, 
     }
     ODL_DISPATCH_SRC_FMT(launch_dynamic, x, rows, cols, parts, margin, out, out_t, dyn_out, fast, stream);
     return check_launch("odl_fp8_cast_dynamic");
+}
+
+// ------------------------------------------------ current scaling of many tensors in two launches
+// All weights of a model per optimizer step: one amax launch and one cast+transpose launch instead of a pair per
+// weight.  The tensors are described by a table in device memory (odl_fp8_mt_tensor); a second table lists the work
+// items, (tensor, local index) pairs, one per block: the blocks of the amax pass, the 128 x 64 tiles of the cast.
+// Both tables depend only on addresses and shapes, so a caller builds them once (odl_fp8_multi_plan).
+namespace odl {
+
+// blocks of the amax pass for a tensor of n16 16-byte chunks: one per 64 KB, at most one per partial maximum
+__host__ __device__ inline int mt_amax_blocks(int64_t n16) {
+    const int64_t nb = (n16 + 4095) / 4096;
+    return nb < 1 ? 1 : (nb > kAmaxParts ? kAmaxParts : (int)nb);
+}
+
+__global__ __launch_bounds__(kFatThreads) void multi_amax_kernel(const odl_fp8_mt_tensor *__restrict__ tensors,
+                                                                  const int32_t *__restrict__ work) {
+    __shared__ uint32_t red[kFatThreads / kWave];
+    const int32_t t = work[2 * (int64_t)blockIdx.x], b = work[2 * (int64_t)blockIdx.x + 1];
+    const odl_fp8_mt_tensor e = tensors[t];
+    const int64_t n16 = e.rows * e.cols / (e.src_dtype == ODL_BF16 ? 8 : 4);
+    const int nb = mt_amax_blocks(n16);
+    const int64_t i0 = (int64_t)b * kFatThreads + threadIdx.x, stride = (int64_t)nb * kFatThreads;
+    uint32_t m = e.src_dtype == ODL_BF16 ? amax_chunks<ODL_BF16, 4>(e.x, n16, i0, stride) : amax_chunks<ODL_F32, 4>(e.x, n16, i0, stride);
+    m = block_max_u32(m, red);
+    if (threadIdx.x == 0) e.parts[b] = bits_to_float(m);
+    if (b == 0)                                                   // entries no block owns
+        for (int i = nb + threadIdx.x; i < kAmaxParts; i += kFatThreads) e.parts[i] = 0.0f;
+}
+
+template <int FMT>
+__global__ __launch_bounds__(kThreads) void multi_cast_dynamic_kernel(const odl_fp8_mt_tensor *__restrict__ tensors,
+                                                                       const int32_t *__restrict__ work, int margin) {
+    __shared__ __attribute__((aligned(16))) uint8_t tile[kTileC * kTileR];
+    __shared__ uint32_t red[kThreads / kWave];
+    const int32_t t = work[2 * (int64_t)blockIdx.x], local = work[2 * (int64_t)blockIdx.x + 1];
+    const odl_fp8_mt_tensor e = tensors[t];
+    const float st = dynamic_scale<FMT>(e.parts, margin, e.dyn_out, red, local == 0);
+    const int64_t tiles_r = (e.rows + kTileR - 1) / kTileR, tiles_c = (e.cols + kTileC - 1) / kTileC;
+    int64_t tr, tc;
+    ct_tile_of(tiles_r * tiles_c - 1 - local, tiles_r, tiles_c, tr, tc);
+    uint32_t am = 0;
+    if (e.src_dtype == ODL_BF16) ct_one_tile<ODL_BF16, FMT, kScaleParts, false, true>(e.x, e.rows, e.cols, nullptr, st, e.out, e.out_t, tr, tc, tile, am);
+    else ct_one_tile<ODL_F32, FMT, kScaleParts, false, true>(e.x, e.rows, e.cols, nullptr, st, e.out, e.out_t, tr, tc, tile, am);
+}
+
+}  // namespace odl
+
+extern "C" int64_t odl_fp8_multi_plan(const odl_fp8_mt_tensor *tensors, int64_t n, int phase, int32_t *work, int64_t capacity) {
+    if (n < 0 || (!tensors && n > 0)) { set_error(ODL_ERR_ARG, "odl_fp8_multi_plan: bad table (n = %lld)", (long long)n); return -1; }
+    if (phase != ODL_MT_AMAX && phase != ODL_MT_CAST) { set_error(ODL_ERR_ARG, "odl_fp8_multi_plan: phase %d", phase); return -1; }
+    int64_t count = 0;
+    for (int64_t t = 0; t < n; ++t) {
+        const odl_fp8_mt_tensor &e = tensors[t];
+        if (e.src_dtype != ODL_BF16 && e.src_dtype != ODL_F32) { set_error(ODL_ERR_ARG, "odl_fp8_multi_plan: tensor %lld: src_dtype %d", (long long)t, e.src_dtype); return -1; }
+        if (e.rows <= 0 || e.cols <= 0 || e.rows % 16 || e.cols % 8) {
+            set_error(ODL_ERR_SHAPE, "odl_fp8_multi_plan: tensor %lld is %lld x %lld; rows must be a positive multiple of 16, cols of 8", (long long)t, (long long)e.rows, (long long)e.cols);
+            return -1;
+        }
+        if (!e.x || !e.out || !e.out_t || !e.parts || !e.dyn_out || !aligned16(e.x) || !aligned16(e.out_t) || !aligned16(e.parts) ||
+            (reinterpret_cast<uintptr_t>(e.out) & 7)) {
+            set_error(ODL_ERR_ARG, "odl_fp8_multi_plan: tensor %lld: null or misaligned pointer (x, out_t, parts: 16 bytes; out: 8)", (long long)t);
+            return -1;
+        }
+        const int64_t items = phase == ODL_MT_AMAX ? mt_amax_blocks(e.rows * e.cols / (e.src_dtype == ODL_BF16 ? 8 : 4))
+                                                   : ((e.rows + kTileR - 1) / kTileR) * ((e.cols + kTileC - 1) / kTileC);
+        if (t > 0x7fffffffLL || items > 0x7fffffffLL) { set_error(ODL_ERR_SHAPE, "odl_fp8_multi_plan: tensor %lld is too large", (long long)t); return -1; }
+        if (work && count + items <= capacity)
+            for (int64_t i = 0; i < items; ++i) { work[2 * (count + i)] = (int32_t)t; work[2 * (count + i) + 1] = (int32_t)i; }
+        count += items;
+    }
+    if (count > 0x7fffffffLL) { set_error(ODL_ERR_SHAPE, "odl_fp8_multi_plan: %lld work items exceed one launch", (long long)count); return -1; }
+    return count;
+}
+
+extern "C" int odl_fp8_multi_amax_parts(const odl_fp8_mt_tensor *tensors_dev, const int32_t *work_dev, int64_t n_work, odl_stream_t stream_) {
+    if (n_work < 0 || n_work > 0x7fffffffLL) return set_error(ODL_ERR_ARG, "odl_fp8_multi_amax_parts: n_work %lld", (long long)n_work);
+    if (n_work == 0) return ODL_OK;
+    if (!tensors_dev || !work_dev) return set_error(ODL_ERR_ARG, "odl_fp8_multi_amax_parts: null table");
+    hipLaunchKernelGGL(multi_amax_kernel, dim3((unsigned)n_work), dim3(kFatThreads), 0, reinterpret_cast<hipStream_t>(stream_), tensors_dev, work_dev);
+    return check_launch("odl_fp8_multi_amax_parts");
+}
+
+extern "C" int odl_fp8_multi_cast_dynamic(const odl_fp8_mt_tensor *tensors_dev, const int32_t *work_dev, int64_t n_work, int fmt, int margin,
+                                          odl_stream_t stream_) {
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    if (n_work < 0 || n_work > 0x7fffffffLL) return set_error(ODL_ERR_ARG, "odl_fp8_multi_cast_dynamic: n_work %lld", (long long)n_work);
+    if (fmt != ODL_FP8_E4M3 && fmt != ODL_FP8_E5M2) return set_error(ODL_ERR_ARG, "odl_fp8_multi_cast_dynamic: fmt %d", fmt);
+    if (n_work == 0) return ODL_OK;
+    if (!tensors_dev || !work_dev) return set_error(ODL_ERR_ARG, "odl_fp8_multi_cast_dynamic: null table");
+    if (fmt == ODL_FP8_E4M3) hipLaunchKernelGGL((multi_cast_dynamic_kernel<ODL_FP8_E4M3>), dim3((unsigned)n_work), dim3(kThreads), 0, stream, tensors_dev, work_dev, margin);
+    else hipLaunchKernelGGL((multi_cast_dynamic_kernel<ODL_FP8_E5M2>), dim3((unsigned)n_work), dim3(kThreads), 0, stream, tensors_dev, work_dev, margin);
+    return check_launch("odl_fp8_multi_cast_dynamic");
 }
 
 // ------------------------------------------------ current scaling without a caller-side workspace

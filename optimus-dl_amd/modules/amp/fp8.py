@@ -236,6 +236,21 @@ class FP8Recipe:
             arena.dirty = False
             arena.epoch += 1
 
+    # ------------------------------------------------------- fp8.param
+    def attach_params(self, model: torch.nn.Module, optimizer: "torch.optim.Optimizer | None" = None):
+        """``fp8.param: true`` (optimus_dl/modules/optim/config.py:36-37): keep the weights of the model's FP8
+        Linears quantised between optimizer steps.  All of them are quantised in two launches now and, when the
+        optimizer is given, after each of its steps (a step post-hook); the forwards in between launch nothing
+        for the weights.  Returns the ``Fp8ParamSet`` (call its ``sync()`` yourself after a step when no optimizer
+        was given), or None for the recipes that keep the per-module route (delayed, rowwise)."""
+        from ..fp8_linear import Fp8ParamSet
+
+        if self._recipe.kind != "tensorwise":
+            _info_once(f"fp8.param: the '{self._recipe.kind}' recipe quantises each weight in its own module (cached per parameter "
+                       "version); nothing to attach")
+            return None
+        return Fp8ParamSet.attach(model, self, optimizer)
+
     # ---------------------------------------------------------- checkpointing
     _DIRECTIONS = (("fwd", "scaling_fwd"), ("bwd", "scaling_bwd"))
 

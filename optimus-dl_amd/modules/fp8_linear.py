@@ -64,6 +64,12 @@ class _WeightCache:
         self.wq = self.wq_t = self.s_inv = self.s_inv_t = self.amax = None
 
 
+def _weight_key(weight: torch.Tensor, fmt: int, how: tuple) -> tuple:
+    """What cached codes of a weight depend on: its storage, its contents (version counter), the format and
+    how the scale is found."""
+    return (weight.data_ptr(), _state.tensor_version(weight), fmt, how)
+
+
 def _quantise_dynamic(x2d: torch.Tensor, fmt: int, margin: int, need_t: bool, need_rowmajor: bool = True,
                       recipe: FP8Recipe | None = None, parts: torch.Tensor | None = None):
     """Per-tensor current scaling: amax pass, scale, cast (+transpose) pass.  The amax pass is
@@ -349,7 +355,7 @@ class FP8Linear(nn.Linear):
             how = ("delayed", pol.amax_history_len, id(meta.arena), meta.arena.epoch, record) if meta is not None else ("own amax", pol.margin)
         else:
             how = (pol.kind, pol.margin)
-        key = (weight.data_ptr(), _state.tensor_version(weight), pol.fmt_fwd, how)
+        key = _weight_key(weight, pol.fmt_fwd, how)
         fresh = c.key != key or not recipe.cache_weights
         if fresh or (need_t and c.wq_t is None):
             w2d = weight.detach()
@@ -431,3 +437,74 @@ class FP8Linear(nn.Linear):
 
     def extra_repr(self) -> str:
         return f"in_features={self.in_features}, out_features={self.out_features}, bias={self.bias is not None}, fp8=True"
+
+
+class Fp8ParamSet:
+    """The weights of a model's FP8 Linears kept quantised between optimizer steps (``fp8.param: true``,
+    optimus_dl/modules/optim/config.py:36-37,56: declared there and never read).
+
+    Without it every ``FP8Linear`` quantises its own weight on the first forward after the weight changed: an
+    amax launch and a cast+transpose launch per weight and optimizer step (a model of 196 Linears: 392 launches
+    and as many allocations).  With it, :meth:`sync` quantises all of them in TWO launches into buffers that live
+    as long as the set, and stamps every module's weight cache with the parameter version it quantised, so the
+    forwards that follow launch nothing for the weights.  The codes and scales are the same bits either way.
+
+    ``sync`` belongs right after ``optimizer.step()`` (``attach`` registers it as a step post-hook when handed the
+    optimizer); it rewrites the buffers in place, so no backward that still needs the previous codes may be pending,
+    the same rule as for the optimizer's own in-place update.  A weight that changes without a ``sync`` (a
+    checkpoint load, a manual edit) is simply quantised by its module on the next forward, as without the set.
+    Current scaling ("tensorwise") only: the other recipes keep their per-module route."""
+
+    def __init__(self, modules: list["FP8Linear"], recipe: FP8Recipe):
+        pol = recipe.recipe
+        if pol.kind != "tensorwise":
+            raise ValueError(f"Fp8ParamSet serves the tensorwise recipe, not '{pol.kind}'")
+        self.recipe = recipe
+        self.modules: list[FP8Linear] = []
+        self.skipped: list[FP8Linear] = []          # shapes / dtypes the two-launch route does not take: per-module route
+        for m in modules:
+            (self.modules if native.MultiTensorPlan.eligible(m.weight.detach()) else self.skipped).append(m)
+        self._plan: native.MultiTensorPlan | None = None
+        self._index: list[int] = []
+        self.syncs = 0
+
+    def _build(self) -> None:
+        sources, index, seen = [], [], {}
+        for m in self.modules:
+            w = m.weight.detach()
+            at = seen.get(w.data_ptr())
+            if at is None:                           # Linears that share one Parameter share its codes
+                at = seen[w.data_ptr()] = len(sources)
+                sources.append(w)
+            index.append(at)
+        pol = self.recipe.recipe
+        self._plan = native.MultiTensorPlan(sources, pol.fmt_fwd, pol.margin) if sources else None
+        self._index = index
+
+    @torch.no_grad()
+    def sync(self) -> None:
+        """Quantise every weight of the set now (two launches on the current stream)."""
+        if not self.modules:
+            return
+        if self._plan is None or len(self._index) != len(self.modules) or self._plan.stale() or \
+                any(m.weight.data_ptr() != self._plan.sources[i].data_ptr() for m, i in zip(self.modules, self._index)):
+            self._build()                            # first use, or a parameter's storage moved (.to(), a new optimizer state)
+        plan, pol = self._plan, self.recipe.recipe
+        plan.run()
+        how = (pol.kind, pol.margin)
+        for m, i in zip(self.modules, self._index):
+            c = m._wcache
+            c.wq, c.wq_t = plan.codes[i], plan.codes_t[i]
+            c.amax, c.s_inv = plan.dyn[i, 0:1], plan.dyn[i, 2:3]
+            c.key = _weight_key(m.weight, pol.fmt_fwd, how)
+        self.syncs += 1
+
+    @classmethod
+    def attach(cls, model: nn.Module, recipe: FP8Recipe, optimizer: "torch.optim.Optimizer | None" = None) -> "Fp8ParamSet":
+        """The set of every ``FP8Linear`` under ``model``, quantised once now; with an optimizer, again after each
+        of its steps."""
+        ps = cls([m for m in model.modules() if isinstance(m, FP8Linear)], recipe)
+        ps.sync()
+        if optimizer is not None:
+            ps.hook = optimizer.register_step_post_hook(lambda *_a, **_k: ps.sync())
+        return ps

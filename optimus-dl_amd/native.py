@@ -15,6 +15,7 @@ import ctypes
 import os
 import threading
 
+import numpy as np
 import torch
 
 E4M3, E5M2 = 0, 1
@@ -23,7 +24,8 @@ DT_BF16, DT_F32 = 0, 1
 AMAX_MAX, AMAX_MOST_RECENT = 0, 1
 FP8_MAX = {E4M3: 448.0, E5M2: 57344.0}
 TORCH_FP8 = {E4M3: torch.float8_e4m3fn, E5M2: torch.float8_e5m2}
-ABI_VERSION = 8
+ABI_VERSION = 9
+AMAX_PARTS = 512                       # ODL_FP8_AMAX_PARTS
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # ODL_FP8_LIB names another build of the same library (e.g. one made for an experiment)
@@ -38,6 +40,9 @@ EXPORTS = (
     "odl_fp8_amax_parts",
     "odl_fp8_cast_dynamic",
     "odl_fp8_cast_dynamic_noalloc",
+    "odl_fp8_multi_plan",
+    "odl_fp8_multi_amax_parts",
+    "odl_fp8_multi_cast_dynamic",
     "odl_fp8_amax_parts_colsum",
     "odl_fp8_swiglu_amax_parts",
     "odl_fp8_swiglu_bwd_amax_parts",
@@ -99,6 +104,10 @@ def load() -> ctypes.CDLL:
         L.odl_fp8_amax_parts.argtypes = [vp, i32, i64, i64, vp, vp]
         L.odl_fp8_cast_dynamic.argtypes = [vp, i32, i64, i64, vp, i32, i32, vp, vp, vp, vp]
         L.odl_fp8_cast_dynamic_noalloc.argtypes = [vp, i32, i64, i64, i32, i32, vp, vp, vp, vp]
+        L.odl_fp8_multi_plan.argtypes = [vp, i64, i32, vp, i64]
+        L.odl_fp8_multi_plan.restype = ctypes.c_int64
+        L.odl_fp8_multi_amax_parts.argtypes = [vp, vp, i64, vp]
+        L.odl_fp8_multi_cast_dynamic.argtypes = [vp, vp, i64, i32, i32, vp]
         L.odl_fp8_amax_parts_colsum.argtypes = [vp, i32, i64, i64, vp, vp, vp, vp]
         L.odl_fp8_swiglu_amax_parts.argtypes = [vp, vp, i64, i64, vp, vp, vp]
         L.odl_fp8_swiglu_bwd_amax_parts.argtypes = [vp, vp, vp, i64, i64, vp, vp, vp, vp, vp]
@@ -212,9 +221,6 @@ def amax_scale(x: torch.Tensor, fmt: int, margin: int = 0):
     return out[0:1], out[1:2], out[2:3]
 
 
-AMAX_PARTS = 512                       # ODL_FP8_AMAX_PARTS
-
-
 def amax_parts(x: torch.Tensor) -> torch.Tensor:
     """AMAX_PARTS partial maxima of |x| (no atomics); input of :func:`cast_dynamic`.  The kernel
     writes every entry, so the buffer is a fresh allocation per call: callers on several threads
@@ -287,6 +293,71 @@ def cast_dynamic_noalloc(x: torch.Tensor, fmt: int, margin: int, out: torch.Tens
                                                out.data_ptr() if out is not None else None,
                                                out_t.data_ptr() if out_t is not None else None, dyn_out.data_ptr(), _stream()),
            "odl_fp8_cast_dynamic_noalloc")
+
+
+class MultiTensorPlan:
+    """Current scaling of many tensors in two launches (``odl_fp8_multi_amax_parts`` + ``odl_fp8_multi_cast_dynamic``).
+
+    Built once from the source tensors: allocates every output (codes, transposed codes, partial maxima,
+    {amax, scale, 1/scale} per tensor), the table that describes them and the two work lists, all on the
+    tensors' device.  :meth:`run` allocates nothing and launches two kernels on the current stream; it writes
+    the same buffers every time.  Sources must be 2-D, contiguous, bf16 or fp32, rows a multiple of 16 and
+    columns of 8 (``eligible``).  The plan holds the sources' ADDRESSES: ``stale()`` tells whether one moved."""
+
+    MT_AMAX, MT_CAST = 0, 1
+
+    @staticmethod
+    def eligible(x: torch.Tensor) -> bool:
+        return (x.is_cuda and x.dim() == 2 and x.is_contiguous() and x.dtype in (torch.bfloat16, torch.float32)
+                and x.shape[0] > 0 and x.shape[0] % 16 == 0 and x.shape[1] > 0 and x.shape[1] % 8 == 0 and x.data_ptr() % 16 == 0)
+
+    def __init__(self, sources: list[torch.Tensor], fmt: int, margin: int = 0):
+        if not sources:
+            raise NativeError("MultiTensorPlan: no tensors")
+        for x in sources:
+            if not self.eligible(x):
+                raise NativeError(f"MultiTensorPlan: a {x.dtype} tensor of shape {tuple(x.shape)} on {x.device} cannot take the "
+                                  "multi-tensor route (2-D contiguous bf16 / fp32 on the GPU, rows % 16 == 0, cols % 8 == 0)")
+        dev = sources[0].device
+        if any(x.device != dev for x in sources):
+            raise NativeError("MultiTensorPlan: tensors on different devices")
+        self.sources, self.fmt, self.margin, self.device = list(sources), fmt, margin, dev
+        n = len(sources)
+        self.codes = [torch.empty(tuple(x.shape), dtype=torch.uint8, device=dev) for x in sources]
+        self.codes_t = [torch.empty((x.shape[1], x.shape[0]), dtype=torch.uint8, device=dev) for x in sources]
+        self.parts = torch.zeros((n, AMAX_PARTS), dtype=torch.float32, device=dev)
+        self.dyn = torch.zeros((n, 3), dtype=torch.float32, device=dev)          # rows {amax, scale, 1/scale}
+        self._ptrs = [x.data_ptr() for x in sources]
+        # odl_fp8_mt_tensor: five pointers, rows, cols, {src_dtype, reserved} = 8 x 8 bytes
+        table = np.zeros((n, 8), dtype=np.int64)
+        for i, x in enumerate(sources):
+            table[i] = (x.data_ptr(), self.codes[i].data_ptr(), self.codes_t[i].data_ptr(), self.parts[i].data_ptr(),
+                        self.dyn[i].data_ptr(), x.shape[0], x.shape[1], _src_dtype(x))
+        self._work = [self.plan_work(table, phase).to(dev) for phase in (self.MT_AMAX, self.MT_CAST)]
+        self._table = torch.from_numpy(table).to(dev)
+
+    @staticmethod
+    def plan_work(table: "np.ndarray", phase: int) -> torch.Tensor:
+        """The work list of one phase for a host copy of the table ([n, 8] int64), as a [count, 2] int32 CPU tensor."""
+        L = load()
+        n = table.shape[0]
+        count = L.odl_fp8_multi_plan(table.ctypes.data, n, phase, None, 0)
+        if count < 0:
+            raise NativeError(f"odl_fp8_multi_plan: {L.odl_fp8_last_error().decode()}")
+        work = torch.empty((count, 2), dtype=torch.int32)
+        if L.odl_fp8_multi_plan(table.ctypes.data, n, phase, work.data_ptr(), count) != count:
+            raise NativeError(f"odl_fp8_multi_plan: {L.odl_fp8_last_error().decode()}")
+        return work
+
+    def stale(self) -> bool:
+        return any(x.data_ptr() != p for x, p in zip(self.sources, self._ptrs))
+
+    def run(self) -> None:
+        L, stream = load(), _stream()
+        w_amax, w_cast = self._work
+        _check(L.odl_fp8_multi_amax_parts(self._table.data_ptr(), w_amax.data_ptr(), w_amax.shape[0], stream), "odl_fp8_multi_amax_parts")
+        _check(L.odl_fp8_multi_cast_dynamic(self._table.data_ptr(), w_cast.data_ptr(), w_cast.shape[0], self.fmt, self.margin, stream),
+               "odl_fp8_multi_cast_dynamic")
 
 
 def quantize_dynamic(x: torch.Tensor, fmt: int, margin: int = 0, want_rowmajor: bool = True, want_transposed: bool = True,
@@ -558,9 +629,6 @@ def cast_transpose(x: torch.Tensor, scale: torch.Tensor, fmt: int, mode: int = S
                                          amax_out.data_ptr() if amax_out is not None else None, _stream()),
            "odl_fp8_cast_transpose")
     return out, out_t
-
-
-AMAX_PARTS = 512                       # ODL_FP8_AMAX_PARTS
 
 
 def cast_delayed(x: torch.Tensor, scale: torch.Tensor, fmt: int, amax_parts: torch.Tensor | None = None,

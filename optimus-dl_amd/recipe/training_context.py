@@ -92,6 +92,16 @@ class TrainingContext:
             "fp8_backward_ctx": self.get_fp8_backward_ctx(),
         }
 
+    def attach_fp8_params(self, model: torch.nn.Module, optimizer: "torch.optim.Optimizer | None" = None):
+        """``amp.fp8.param: true``: the weights of the model's FP8 Linears stay quantised between optimizer steps
+        (all of them re-quantised in two launches after each step).  Call once, after ``setup_training_context``
+        and after model and optimizer exist.  Returns the parameter set, or None when the key is off, FP8 is not
+        in use, or the recipe keeps the per-module route.  The reference declares the key and never reads it
+        (optimus_dl/modules/optim/config.py:36-37,56)."""
+        if self._fp8_recipe is None or not self.optimization_config.amp.fp8.param:
+            return None
+        return self._fp8_recipe.attach_params(model, optimizer)
+
     def _create_fp8_autocast(self, device: torch.device, fp8_recipe: FP8Recipe | None) -> Any:
         if fp8_recipe is not None:
             return lambda: fp8_autocast(device=device, fp8_recipe=fp8_recipe)   # a fresh context per microbatch

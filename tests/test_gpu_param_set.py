@@ -1,0 +1,171 @@
+"""Many weights quantised in two launches (odl_fp8_multi_amax_parts + odl_fp8_multi_cast_dynamic) and the
+``fp8.param`` parameter set built on them: the same bits as the per-tensor route, and no weight quantisation
+launches in the forwards between optimizer steps."""
+import pytest
+import torch
+import torch.nn as nn
+
+from oracle import oracle as O
+from tests.helpers import assert_bytes_equal, assert_f32_bits_equal, seeded_bf16
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def N():
+    from optimus_dl_amd import native
+
+    native.load()
+    return native
+
+
+@pytest.fixture(scope="module")
+def amp():
+    from optimus_dl_amd.modules import amp as A
+
+    return A
+
+
+SHAPES = [(1024, 768, torch.bfloat16, 0.02), (16, 8, torch.float32, 1.0), (3072, 1024, torch.float32, 0.02),
+          (4096, 4096, torch.bfloat16, 0.5), (144, 200, torch.bfloat16, 3.0), (2048, 64, torch.float32, 1e-3)]
+
+
+@pytest.mark.parametrize("fmt,margin", [(O.E4M3, 0), (O.E5M2, 2)])
+def test_multi_tensor_route_equals_the_per_tensor_route_and_the_oracle(N, fmt, margin):
+    xs = [seeded_bf16((r, c), std, 40 + i).to(dt).cuda() for i, (r, c, dt, std) in enumerate(SHAPES)]
+    xs[3][4095, 4095] = 77.0                                       # the amax of the big one sits in its last block
+    plan = N.MultiTensorPlan(xs, fmt, margin)
+    for trip in range(2):
+        plan.run()
+        torch.cuda.synchronize()
+        for i, x in enumerate(xs):
+            q, q_t, amax, scale, s_inv = N.quantize_dynamic(x, fmt, margin)
+            assert_bytes_equal(plan.codes[i], q, f"tensor {i}: codes")
+            assert_bytes_equal(plan.codes_t[i], q_t, f"tensor {i}: transposed codes")
+            assert_f32_bits_equal(plan.dyn[i], torch.cat([amax, scale, s_inv]), f"tensor {i}: amax / scale / 1/scale")
+            if x.numel() <= 1 << 20:                               # and the oracle, where it takes no time
+                a = O.t_amax(x.cpu())
+                assert float(plan.dyn[i, 0]) == float(a)
+                assert_bytes_equal(plan.codes[i], O.t_cast(x.cpu(), O.t_scale(a, fmt, margin), fmt), f"tensor {i}: codes vs oracle")
+            assert plan.parts[i].max().item() == plan.dyn[i, 0].item()
+        for x in xs:                                               # second trip: new contents, same buffers
+            x.mul_(-1.7)
+    assert not plan.stale()
+    xs[0].data = xs[0].data.clone()
+    assert plan.stale()
+
+
+def test_multi_tensor_plan_refuses_what_the_kernels_cannot_take(N):
+    ok = torch.zeros((32, 16), dtype=torch.bfloat16, device="cuda")
+    for bad in (torch.zeros((30, 16), dtype=torch.bfloat16, device="cuda"), torch.zeros((32, 12), dtype=torch.bfloat16, device="cuda"),
+                torch.zeros((32, 16), dtype=torch.float16, device="cuda"), torch.zeros((64, 16), dtype=torch.bfloat16, device="cuda")[::2],
+                torch.zeros((32, 16), dtype=torch.bfloat16)):
+        assert not N.MultiTensorPlan.eligible(bad)
+        with pytest.raises(N.NativeError):
+            N.MultiTensorPlan([ok, bad], O.E4M3)
+    with pytest.raises(N.NativeError):
+        N.MultiTensorPlan([], O.E4M3)
+
+
+class Net(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.a, self.b = nn.Linear(256, 512, bias=False), nn.Linear(512, 256, bias=True)
+        self.odd = nn.Linear(256, 24, bias=False)                  # 24 output channels: no FP8 for this one, and the set skips it
+        self.tied = nn.Linear(256, 512, bias=False)
+        self.tied.weight = self.a.weight
+
+    def forward(self, x):
+        return self.b(torch.relu(self.a(x)) + self.tied(x)), self.odd(x)
+
+
+def build(seed=0):
+    from optimus_dl_amd.modules.model_transforms import build_model_transform
+
+    torch.manual_seed(seed)
+    net = Net().cuda()                                             # fp32 master weights, the usual AMP set-up
+    build_model_transform({"_name": "fp8_linear"}).apply(net)
+    return net
+
+
+def count_weight_quantisations(N, monkeypatch):
+    calls = {"n": 0}
+    real = N.quantize_dynamic
+
+    def counted(x, *a, **kw):
+        if x.dim() == 2 and x.dtype == torch.float32:              # weights here are fp32, activations bf16
+            calls["n"] += 1
+        return real(x, *a, **kw)
+
+    monkeypatch.setattr(N, "quantize_dynamic", counted)
+    return calls
+
+
+def test_param_set_trains_like_the_per_module_route_without_weight_launches(N, amp, monkeypatch):
+    from optimus_dl_amd.modules.fp8_linear import Fp8ParamSet
+
+    plain, kept = build(), build()
+    recipe_a, recipe_b = amp.create_fp8_recipe("tensorwise", "hybrid"), amp.create_fp8_recipe("tensorwise", "hybrid")
+    opt_a, opt_b = torch.optim.SGD(plain.parameters(), lr=0.05), torch.optim.SGD(kept.parameters(), lr=0.05)
+    ps = recipe_b.attach_params(kept, opt_b)
+    assert isinstance(ps, Fp8ParamSet) and len(ps.modules) == 3 and len(ps.skipped) == 1 and ps.syncs == 1
+    assert len(ps._plan.sources) == 2                              # a and tied share one Parameter: quantised once
+    calls = count_weight_quantisations(N, monkeypatch)
+    for step in range(4):
+        x = seeded_bf16((64, 256), 1.0, 300 + step).cuda()
+        outs = []
+        for net, recipe, opt in ((plain, recipe_a, opt_a), (kept, recipe_b, opt_b)):
+            before = calls["n"]
+            for micro in range(2):                                 # two microbatches per optimizer step
+                with amp.fp8_autocast(torch.device("cuda"), recipe):
+                    y, z = net(x)
+                    loss = y.float().square().mean() + z.float().square().mean()
+                with amp.fp8_backward(recipe):
+                    loss.backward()
+            outs.append((y.detach().clone(), z.detach().clone(), calls["n"] - before))
+            opt.step()
+            opt.zero_grad(set_to_none=True)
+        assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1]), f"step {step}: outputs differ"
+        assert outs[0][2] == 3 and outs[1][2] == 0, outs           # per module: a, tied and b once per optimizer step; kept: none
+    assert ps.syncs == 5                                           # once at attach, once after each optimizer step
+    for pa, pb in zip(plain.parameters(), kept.parameters()):
+        assert torch.equal(pa, pb)
+    # a weight changed behind the set's back is quantised by its module on the next forward (and matches again after a sync)
+    with torch.no_grad():
+        kept.b.weight.mul_(0.5)
+        plain.b.weight.mul_(0.5)
+    x = seeded_bf16((64, 256), 1.0, 999).cuda()
+    with amp.fp8_autocast(torch.device("cuda"), recipe_a), torch.no_grad():
+        want = plain(x)[0]
+    before = calls["n"]
+    with amp.fp8_autocast(torch.device("cuda"), recipe_b), torch.no_grad():
+        got = kept(x)[0]
+    assert torch.equal(got, want) and calls["n"] - before == 1
+    # parameters that move (here: to bf16 and back is a new storage) are picked up by the next sync
+    kept.b.weight.data = kept.b.weight.data.clone()
+    ps.sync()
+    assert ps._plan.sources[ps._index[ps.modules.index(kept.b)]].data_ptr() == kept.b.weight.data_ptr()
+    with amp.fp8_autocast(torch.device("cuda"), recipe_b), torch.no_grad():
+        assert torch.equal(kept(x)[0], want)
+
+
+def test_training_context_attaches_the_set_when_the_config_says_param(amp):
+    from optimus_dl_amd.modules.optim.config import AmpConfig, Fp8Config, OptimizationConfig
+    from optimus_dl_amd.recipe.training_context import TrainingContext
+
+    def ctx_for(**kw):
+        tc = TrainingContext(OptimizationConfig(amp=AmpConfig(enabled=True, dtype="torch.float8_e4m3fn", fp8=Fp8Config(enabled=True, **kw))))
+        tc.setup_training_context(torch.device("cuda"))
+        return tc
+
+    net = build()
+    opt = torch.optim.SGD(net.parameters(), lr=0.1)
+    assert ctx_for(recipe="tensorwise", param=False).attach_fp8_params(net, opt) is None
+    assert ctx_for(recipe="delayed", param=True).attach_fp8_params(net, opt) is None        # per-module route for that recipe
+    ps = ctx_for(recipe="tensorwise", param=True).attach_fp8_params(net, opt)
+    assert ps is not None and ps.syncs == 1
+    opt.step()
+    assert ps.syncs == 2
+    bf16 = TrainingContext(OptimizationConfig(amp=AmpConfig(enabled=True, dtype="torch.bfloat16", fp8=Fp8Config(enabled=True, param=True))))
+    bf16.setup_training_context(torch.device("cuda"))
+    assert bf16.attach_fp8_params(net, opt) is None
