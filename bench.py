@@ -37,9 +37,24 @@ if ROOT not in sys.path:
 
 PEAK_FP8_TFLOPS = 5000.0     # MI355X dense FP8 MFMA, published
 PEAK_HBM_GBPS = 8000.0       # MI355X HBM3E, published
-# Memory-side bytes per GEMM launch (mean of the nine launches of a step), from two rocprofv3 --pmc runs
-# (FETCH_SIZE scaled x2.00, WRITE_SIZE x1.00 against a 256 MiB copy kernel): profiles/pmc_fetch_write__cfg3_mlp.md
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = 8.78e8
+# Memory-side bytes per GEMM launch come from a tracked data file that names the profiler runs behind it
+GEMM_TRAFFIC_FILE = os.path.join(ROOT, "profiles", "gemm_traffic__cfg3_mlp.json")
+
+
+def gemm_traffic_bytes_per_launch():
+    """Mean over the launches of a step of (FETCH_SIZE x its scale + WRITE_SIZE x its scale), from the counter
+    values recorded in profiles/gemm_traffic__cfg3_mlp.json; None when the file is not there."""
+    try:
+        with open(GEMM_TRAFFIC_FILE) as fh:
+            t = json.load(fh)
+    except OSError:
+        return None, None
+    n = sum(t["launches_per_step"].values())
+    kib = sum(t["launches_per_step"][k] * (t["fetch_size_kib_per_dispatch"][k] * t["fetch_scale"] +
+                                           t["write_size_kib_per_dispatch"][k] * t["write_scale"]) for k in t["launches_per_step"])
+    return kib * 1024.0 / n, t["source"]
+
+
 M_TOKENS, D_MODEL, D_FF = 8192, 4096, 14336
 LAYERS = (("gate", D_MODEL, D_FF), ("up", D_MODEL, D_FF), ("down", D_FF, D_MODEL))   # name, K(in), N(out)
 
@@ -394,6 +409,82 @@ def whole_models(torch, which=("gpt2_124m", "qwen3_0.6b"), steps=5, warmup=3, la
     return out
 
 
+def clock_probe(torch, native, launches=20, settle=40):
+    """What clock the board grants while the matrix pipe is busy, and what the pipe delivers at that clock.
+
+    (1) The forward GEMM of the gate projection (8192 x 14336 x 4096) back to back, once on operands quantised from
+    Gaussian data and once on all-zero codes, with a clock stamp (shader-clock counter and constant 100 MHz counter,
+    read by a one-wave kernel) before and after the run: time per launch, TFLOP/s, and the average shader clock over
+    the run.  (2) The same MFMA instruction in a register-only loop (one wave per SIMD on every compute unit, no
+    memory traffic), zero and Gaussian-like operands: rate and clock.  `of_peak_at_clock` prices a rate against
+    CUs x 8192 flop per clock x the measured clock instead of the nominal 2.4 GHz.
+    Every measurement follows `settle` launches of the same work: from idle the board runs a handful of launches
+    at a high clock, then drops well below its sustained clock and takes some 30 launches (10 ms) to come back."""
+    import ctypes
+
+    from optimus_dl_amd.build import PROBE_LIB_PATH
+
+    lib = ctypes.CDLL(PROBE_LIB_PATH)                      # built in-tree by optimus_dl_amd.build.build_probe()
+    vp = ctypes.c_void_p
+    lib.odl_probe_clock_stamp.argtypes = [vp, vp]
+    lib.odl_probe_mfma_loop.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, vp, vp]
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    flop_per_clock = cus * 8192.0                          # dense FP8 MFMA: 4 SIMDs x (2 x 32 x 32 x 64 flop / 64 clocks) per CU
+
+    def stream():
+        return torch.cuda.current_stream().cuda_stream
+
+    def priced(tflops, mhz):
+        return {"TFLOP/s": round(tflops, 1), "shader_clock_mhz": round(mhz), "of_nominal_peak": round(tflops / PEAK_FP8_TFLOPS, 3),
+                "of_peak_at_clock": round(tflops * 1e12 / (flop_per_clock * mhz * 1e6), 3)}
+
+    out = {"compute_units": cus, "flop_per_clock": flop_per_clock, "gemm_8192x14336x4096": {}, "mfma_register_loop": {}}
+    M, N, K = M_TOKENS, D_FF, D_MODEL
+    g = torch.Generator(device="cuda").manual_seed(0)
+    x = torch.randn((M, K), generator=g, device="cuda").bfloat16()
+    w = (torch.randn((N, K), generator=g, device="cuda") * 0.02).bfloat16()
+    xq, _, _, _, sx = native.quantize_dynamic(x, native.E4M3, 0, want_transposed=False)
+    wq, _, _, _, sw = native.quantize_dynamic(w, native.E4M3, 0, want_transposed=False)
+    c = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+    stamps = torch.zeros((2, 2), dtype=torch.int64, device="cuda")
+    for label, a, b in (("gaussian_operands", xq, wq), ("zero_operands", torch.zeros_like(xq), torch.zeros_like(wq))):
+        for _ in range(settle):
+            native.gemm_nt(a, b, native.E4M3, native.E4M3, sx, sw, out=c)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        lib.odl_probe_clock_stamp(stamps[0].data_ptr(), stream())
+        e0.record()
+        for _ in range(launches):
+            native.gemm_nt(a, b, native.E4M3, native.E4M3, sx, sw, out=c)
+        e1.record()
+        lib.odl_probe_clock_stamp(stamps[1].data_ptr(), stream())
+        torch.cuda.synchronize()
+        d = (stamps[1] - stamps[0]).tolist()
+        us = 1e3 * e0.elapsed_time(e1) / launches
+        entry = priced(2.0 * M * N * K / (us * 1e-6) / 1e12, 100.0 * d[0] / d[1])
+        entry["us_per_launch"] = round(us, 1)
+        out["gemm_8192x14336x4096"][label] = entry
+    sink = torch.zeros(1, device="cuda")
+    cycles = torch.zeros((cus, 2), dtype=torch.int64, device="cuda")
+    iters = 4000                                           # x 16 MFMAs x 64 clocks: about 2 ms per launch
+    for label, rnd in (("gaussian_like_operands", 1), ("zero_operands", 0)):
+        for _ in range(settle // 4):
+            lib.odl_probe_mfma_loop(rnd, iters, cus, sink.data_ptr(), cycles.data_ptr(), stream())
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(4):
+            lib.odl_probe_mfma_loop(rnd, iters, cus, sink.data_ptr(), cycles.data_ptr(), stream())
+        e1.record()
+        torch.cuda.synchronize()
+        us = 1e3 * e0.elapsed_time(e1) / 4
+        cyc = cycles.double()
+        mhz = float((100.0 * cyc[:, 0] / cyc[:, 1]).median())
+        entry = priced(cus * 4 * iters * 16 * 2.0 * 32 * 32 * 64 / (us * 1e-6) / 1e12, mhz)
+        entry["us_per_launch"] = round(us, 1)
+        entry["clocks_per_mfma"] = round(float(cyc[:, 0].median()) / (iters * 16), 2)
+        out["mfma_register_loop"][label] = entry
+    return out
+
+
 def cpu_baseline(torch, seconds_hint=20.0):
     """The oracle's emulated-FP8 Linear fwd+bwd on the host cores, on a slice of the rows."""
     from oracle import oracle as O
@@ -434,6 +525,8 @@ def main() -> int:
                     help="run only the stand-alone measurements of the memory-bound kernels and print them (for profiling)")
     ap.add_argument("--whole-models-only", default="",
                     help="run only the whole-model step of gpt2_124m or qwen3_0.6b with the default transform and print it (for profiling)")
+    ap.add_argument("--clock-probe-only", action="store_true",
+                    help="run only the clock probe (GEMM back to back on Gaussian / zero operands, register-only MFMA loop) and print it")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy (reference kernel for scaling FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -454,6 +547,9 @@ def main() -> int:
         return 2
     if args.standalone_only:
         print(json.dumps({"hbm_kernels_standalone": standalone_hbm(torch, native)}))
+        return 0
+    if args.clock_probe_only:
+        print(json.dumps({"clock_probe": clock_probe(torch, native)}))
         return 0
     if args.whole_models_only:
         print(json.dumps({"whole_models_fwd_bwd": whole_models(torch, which=(args.whole_models_only,), steps=args.steps,
@@ -555,8 +651,9 @@ def main() -> int:
             "peak": PEAK_FP8_TFLOPS,
             "unit": "TFLOP/s",
             "frac": gemm_tflops / PEAK_FP8_TFLOPS,
-            "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH,
+            "traffic": gemm_traffic_bytes_per_launch()[0],
             "traffic_unit": "bytes per launch (FETCH_SIZE + WRITE_SIZE counters, measured separately)",
+            "traffic_source": gemm_traffic_bytes_per_launch()[1],
             "algorithmic_bytes": (sum(m_ * k_ + n_ * k_ + 2 * m_ * n_ for m_, n_, k_ in
                                       [(M_TOKENS, n, k) for _, k, n in LAYERS] + [(M_TOKENS, k, n) for _, k, n in LAYERS] +
                                       [(n, k, M_TOKENS) for _, k, n in LAYERS]) / 9.0),
@@ -566,6 +663,9 @@ def main() -> int:
         "hbm_kernels": hbm,
     }
     if not args.no_standalone:
+        line["clock_probe"] = clock_probe(torch, native)
+        # the same GEMM back to back with the clock measured: what the roofline fraction is at the clock the board grants
+        line["roofline"]["granted_clock"] = line["clock_probe"]["gemm_8192x14336x4096"]["gaussian_operands"]
         line["hbm_kernels_standalone"] = standalone_hbm(torch, native)
     if not args.no_standalone:
         del layers, data
