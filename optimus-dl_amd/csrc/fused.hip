@@ -168,48 +168,67 @@ __global__ __launch_bounds__(kRmsThreads) void rmsnorm_fwd_kernel(const void *__
                                                                    float *__restrict__ parts) {
     __shared__ uint32_t red[kRmsThreads / kWave];
     constexpr int VPC = SRC == ODL_BF16 ? 1 : 2;            // 16-byte vectors per chunk of 8 elements
+    // Short rows: a wave takes RB consecutive rows per trip, so that as many loads are in flight per lane as for a long
+    // row and the RB reductions (a chain of dependent cross-lane steps and two divisions each) overlap one another.
+    constexpr int RB = CPL <= 2 ? 4 : (CPL <= 4 ? 2 : 1);
     const int lane = threadIdx.x % kWave;
     const int64_t wave = (int64_t)blockIdx.x * (kRmsThreads / kWave) + threadIdx.x / kWave;
     const int64_t nwave = (int64_t)gridDim.x * (kRmsThreads / kWave);
     const int64_t nchunk = cols / 8;
     uint32_t am = 0;
-    for (int64_t row = wave; row < rows; row += nwave) {
-        u32x4 raw[CPL][VPC];
+    for (int64_t row0 = wave * RB; row0 < rows; row0 += nwave * RB) {
+        u32x4 raw[RB][CPL][VPC];
 #pragma unroll
-        for (int j = 0; j < CPL; ++j) {
-            const int64_t c = lane + (int64_t)kWave * j;
-            const u32x4 *p = reinterpret_cast<const u32x4 *>(x) + (row * nchunk + c) * VPC;
+        for (int b = 0; b < RB; ++b)
 #pragma unroll
-            for (int h = 0; h < VPC; ++h) raw[j][h] = c < nchunk ? __builtin_nontemporal_load(p + h) : u32x4{0, 0, 0, 0};
+            for (int j = 0; j < CPL; ++j) {
+                const int64_t c = lane + (int64_t)kWave * j;
+                const u32x4 *p = reinterpret_cast<const u32x4 *>(x) + ((row0 + b) * nchunk + c) * VPC;
+#pragma unroll
+                for (int h = 0; h < VPC; ++h) raw[b][j][h] = (c < nchunk && row0 + b < rows) ? __builtin_nontemporal_load(p + h) : u32x4{0, 0, 0, 0};
+            }
+        float acc[RB], rstd[RB];
+#pragma unroll
+        for (int b = 0; b < RB; ++b) {
+            acc[b] = 0.0f;
+#pragma unroll
+            for (int j = 0; j < CPL; ++j) {
+                float f[8];
+                unpack8<SRC>(raw[b][j], f);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) acc[b] = __fmaf_rn(f[e], f[e], acc[b]);
+            }
         }
-        float acc = 0.0f;
 #pragma unroll
-        for (int j = 0; j < CPL; ++j) {
-            float f[8];
-            unpack8<SRC>(raw[j], f);
+        for (int off = kWave / 2; off > 0; off >>= 1)
 #pragma unroll
-            for (int e = 0; e < 8; ++e) acc = __fmaf_rn(f[e], f[e], acc);
+            for (int b = 0; b < RB; ++b) acc[b] = __fadd_rn(acc[b], __shfl_xor(acc[b], off, kWave));
+#pragma unroll
+        for (int b = 0; b < RB; ++b) {
+            const float mean = __fdiv_rn(acc[b], (float)cols);
+            rstd[b] = __fdiv_rn(1.0f, __builtin_sqrtf(__fadd_rn(mean, eps)));
+            if (lane == 0 && row0 + b < rows) rstd_out[row0 + b] = rstd[b];
         }
-#pragma unroll
-        for (int off = kWave / 2; off > 0; off >>= 1) acc = __fadd_rn(acc, __shfl_xor(acc, off, kWave));
-        const float mean = __fdiv_rn(acc, (float)cols);
-        const float rstd = __fdiv_rn(1.0f, __builtin_sqrtf(__fadd_rn(mean, eps)));
-        if (lane == 0) rstd_out[row] = rstd;
 #pragma unroll
         for (int j = 0; j < CPL; ++j) {
             const int64_t c = lane + (int64_t)kWave * j;
             if (c < nchunk) {
-                float f[8];
-                unpack8<SRC>(raw[j], f);
                 const float4 w0 = *reinterpret_cast<const float4 *>(weight + c * 8), w1 = *reinterpret_cast<const float4 *>(weight + c * 8 + 4);
                 const float w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
-                uint32_t o[4];
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    o[q] = pack2(__fmul_rn(__fmul_rn(f[2 * q], rstd), w[2 * q]), __fmul_rn(__fmul_rn(f[2 * q + 1], rstd), w[2 * q + 1]));
-                    am = max_u16x2(am, abs_bf16x2(o[q]));
+                for (int b = 0; b < RB; ++b) {
+                    if (row0 + b < rows) {
+                        float f[8];
+                        unpack8<SRC>(raw[b][j], f);
+                        uint32_t o[4];
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            o[q] = pack2(__fmul_rn(__fmul_rn(f[2 * q], rstd[b]), w[2 * q]), __fmul_rn(__fmul_rn(f[2 * q + 1], rstd[b]), w[2 * q + 1]));
+                            am = max_u16x2(am, abs_bf16x2(o[q]));
+                        }
+                        reinterpret_cast<u32x4 *>(y)[(row0 + b) * nchunk + c] = u32x4{o[0], o[1], o[2], o[3]};
+                    }
                 }
-                reinterpret_cast<u32x4 *>(y)[row * nchunk + c] = u32x4{o[0], o[1], o[2], o[3]};
             }
         }
     }
@@ -278,6 +297,15 @@ __device__ __forceinline__ float wave_sum_butterfly(float acc) {
 #pragma unroll
     for (int off = kWave / 2; off > 0; off >>= 1) acc = __fadd_rn(acc, __shfl_xor(acc, off, kWave));
     return acc;
+}
+
+// the same butterfly on N independent values, step by step across all of them (the N chains overlap)
+template <int N>
+__device__ __forceinline__ void wave_sum_butterfly_n(float (&acc)[N]) {
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1)
+#pragma unroll
+        for (int b = 0; b < N; ++b) acc[b] = __fadd_rn(acc[b], __shfl_xor(acc[b], off, kWave));
 }
 
 // ------------------------------------------------------- RMSNorm / LayerNorm backward
@@ -635,75 +663,112 @@ __global__ __launch_bounds__(kRmsBwdThreads) void norm_bwd_wave_kernel(const u32
 //   y = bf16( ((d * rstd) * weight) + bias )          (bias may be absent)
 // The backward is norm_bwd_kernel<.., LN = true, ..> above (slabs hold d_weight in [0, cols) and d_bias in
 // [cols, 2 cols) of each block's row).
+// Wide rows (CPL == 8): weight and bias are staged in LDS once per block.  Read from global memory in the output pass, the
+// compiler hoists the loads of all eight chunks above the reductions, which takes 144 registers and leaves room for one
+// 512-lane block per compute unit; from LDS a bf16 row needs 128 and two blocks fit (an fp32 row, twice the registers
+// of input, keeps one block).
 template <int SRC, int CPL, int THREADS>
-__global__ __launch_bounds__(THREADS) void layernorm_fwd_kernel(const void *__restrict__ x, const float *__restrict__ weight,
+__global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu((CPL == 8 && SRC == ODL_BF16) ? 4 : 1, 8))) void layernorm_fwd_kernel(const void *__restrict__ x, const float *__restrict__ weight,
                                                                  const float *__restrict__ bias, int64_t rows, int64_t cols, float eps,
                                                                  uint16_t *__restrict__ y, float *__restrict__ mean_out,
                                                                  float *__restrict__ rstd_out, float *__restrict__ parts) {
     __shared__ uint32_t red[THREADS / kWave];
+    constexpr bool kStage = CPL == 8;
+    __shared__ __attribute__((aligned(16))) float s_w[kStage ? CPL * kWave * 8 : 4], s_b[kStage ? CPL * kWave * 8 : 4];
+    if constexpr (kStage) {
+        for (int64_t c = threadIdx.x; c < cols; c += THREADS) {
+            s_w[c] = weight[c];
+            s_b[c] = bias ? bias[c] : 0.0f;
+        }
+        __syncthreads();
+    }
     constexpr int VPC = SRC == ODL_BF16 ? 1 : 2;
+    constexpr int RB = CPL <= 2 ? 2 : 1;                    // rows per wave and trip, as in rmsnorm_fwd_kernel (more would spill here)
     const int lane = threadIdx.x % kWave;
     const int64_t wave = (int64_t)blockIdx.x * (THREADS / kWave) + threadIdx.x / kWave;
     const int64_t nwave = (int64_t)gridDim.x * (THREADS / kWave);
     const int64_t nchunk = cols / 8;
     uint32_t am = 0;
-    for (int64_t row = wave; row < rows; row += nwave) {
-        u32x4 raw[CPL][VPC];
+    for (int64_t row0 = wave * RB; row0 < rows; row0 += nwave * RB) {
+        u32x4 raw[RB][CPL][VPC];
 #pragma unroll
-        for (int j = 0; j < CPL; ++j) {
-            const int64_t c = lane + (int64_t)kWave * j;
-            const u32x4 *p = reinterpret_cast<const u32x4 *>(x) + (row * nchunk + c) * VPC;
+        for (int b = 0; b < RB; ++b)
 #pragma unroll
-            for (int h = 0; h < VPC; ++h) raw[j][h] = c < nchunk ? __builtin_nontemporal_load(p + h) : u32x4{0, 0, 0, 0};
-        }
-        float acc = 0.0f;
+            for (int j = 0; j < CPL; ++j) {
+                const int64_t c = lane + (int64_t)kWave * j;
+                const u32x4 *p = reinterpret_cast<const u32x4 *>(x) + ((row0 + b) * nchunk + c) * VPC;
 #pragma unroll
-        for (int j = 0; j < CPL; ++j) {
-            float f[8];
-            unpack8<SRC>(raw[j], f);
+                for (int h = 0; h < VPC; ++h) raw[b][j][h] = (c < nchunk && row0 + b < rows) ? __builtin_nontemporal_load(p + h) : u32x4{0, 0, 0, 0};
+            }
+        float acc[RB], mean[RB], rstd[RB];
 #pragma unroll
-            for (int e = 0; e < 8; ++e) acc = __fadd_rn(acc, f[e]);
-        }
-        const float mean = __fdiv_rn(wave_sum_butterfly(acc), (float)cols);
-        acc = 0.0f;
+        for (int b = 0; b < RB; ++b) {
+            acc[b] = 0.0f;
 #pragma unroll
-        for (int j = 0; j < CPL; ++j) {
-            if (lane + (int64_t)kWave * j < nchunk) {      // padding chunks must not contribute (0 - mean)^2
+            for (int j = 0; j < CPL; ++j) {
                 float f[8];
-                unpack8<SRC>(raw[j], f);
+                unpack8<SRC>(raw[b][j], f);
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const float d = __fsub_rn(f[e], mean);
-                    acc = __fmaf_rn(d, d, acc);
+                for (int e = 0; e < 8; ++e) acc[b] = __fadd_rn(acc[b], f[e]);
+            }
+        }
+        wave_sum_butterfly_n<RB>(acc);
+#pragma unroll
+        for (int b = 0; b < RB; ++b) {
+            mean[b] = __fdiv_rn(acc[b], (float)cols);
+            acc[b] = 0.0f;
+#pragma unroll
+            for (int j = 0; j < CPL; ++j) {
+                if (lane + (int64_t)kWave * j < nchunk) {      // padding chunks must not contribute (0 - mean)^2
+                    float f[8];
+                    unpack8<SRC>(raw[b][j], f);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const float d = __fsub_rn(f[e], mean[b]);
+                        acc[b] = __fmaf_rn(d, d, acc[b]);
+                    }
                 }
             }
         }
-        const float var = __fdiv_rn(wave_sum_butterfly(acc), (float)cols);
-        const float rstd = __fdiv_rn(1.0f, __builtin_sqrtf(__fadd_rn(var, eps)));
-        if (lane == 0) { mean_out[row] = mean; rstd_out[row] = rstd; }
+        wave_sum_butterfly_n<RB>(acc);
+#pragma unroll
+        for (int b = 0; b < RB; ++b) {
+            const float var = __fdiv_rn(acc[b], (float)cols);
+            rstd[b] = __fdiv_rn(1.0f, __builtin_sqrtf(__fadd_rn(var, eps)));
+            if (lane == 0 && row0 + b < rows) { mean_out[row0 + b] = mean[b]; rstd_out[row0 + b] = rstd[b]; }
+        }
 #pragma unroll
         for (int j = 0; j < CPL; ++j) {
             const int64_t c = lane + (int64_t)kWave * j;
             if (c < nchunk) {
-                float f[8], o[8];
-                unpack8<SRC>(raw[j], f);
-                const float4 w0 = *reinterpret_cast<const float4 *>(weight + c * 8), w1 = *reinterpret_cast<const float4 *>(weight + c * 8 + 4);
+                const float *wp = kStage ? s_w : weight, *bp = kStage ? s_b : bias;
+                const float4 w0 = *reinterpret_cast<const float4 *>(wp + c * 8), w1 = *reinterpret_cast<const float4 *>(wp + c * 8 + 4);
                 const float w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
-#pragma unroll
-                for (int e = 0; e < 8; ++e) o[e] = __fmul_rn(__fmul_rn(__fsub_rn(f[e], mean), rstd), w[e]);
+                float bv[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
                 if (bias) {
-                    const float4 b0 = *reinterpret_cast<const float4 *>(bias + c * 8), b1 = *reinterpret_cast<const float4 *>(bias + c * 8 + 4);
-                    const float b[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) o[e] = __fadd_rn(o[e], b[e]);
+                    const float4 b0 = *reinterpret_cast<const float4 *>(bp + c * 8), b1 = *reinterpret_cast<const float4 *>(bp + c * 8 + 4);
+                    bv[0] = b0.x; bv[1] = b0.y; bv[2] = b0.z; bv[3] = b0.w; bv[4] = b1.x; bv[5] = b1.y; bv[6] = b1.z; bv[7] = b1.w;
                 }
-                uint32_t pk[4];
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    pk[q] = pack2(o[2 * q], o[2 * q + 1]);
-                    am = max_u16x2(am, abs_bf16x2(pk[q]));
+                for (int b = 0; b < RB; ++b) {
+                    if (row0 + b < rows) {
+                        float f[8], o[8];
+                        unpack8<SRC>(raw[b][j], f);
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) o[e] = __fmul_rn(__fmul_rn(__fsub_rn(f[e], mean[b]), rstd[b]), w[e]);
+                        if (bias) {
+#pragma unroll
+                            for (int e = 0; e < 8; ++e) o[e] = __fadd_rn(o[e], bv[e]);
+                        }
+                        uint32_t pk[4];
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            pk[q] = pack2(o[2 * q], o[2 * q + 1]);
+                            am = max_u16x2(am, abs_bf16x2(pk[q]));
+                        }
+                        reinterpret_cast<u32x4 *>(y)[(row0 + b) * nchunk + c] = u32x4{pk[0], pk[1], pk[2], pk[3]};
+                    }
                 }
-                reinterpret_cast<u32x4 *>(y)[row * nchunk + c] = u32x4{pk[0], pk[1], pk[2], pk[3]};
             }
         }
     }
@@ -815,7 +880,7 @@ __global__ __launch_bounds__(kFusedThreads) void amax_colsum_kernel(const void *
 // gelu_table_kernel in double precision, holds for every bf16 pattern x
 //   fwd[x] = bf16( float( x * Phi(x) ) )            Phi(x) = erfc(-x / sqrt 2) / 2
 //   bwd[x] = float( Phi(x) + x * phi(x) )           phi(x) = exp(-x^2 / 2) / sqrt(2 pi)
-// (65536 bf16 values, then 65536 floats: 384 KB, resident in L2 while in use).  The kernels gather:
+// (65536 bf16 values, then 65536 floats: 384 KB).  The kernels gather:
 //   y = fwd[x],   dx = bf16( dy * bwd[x] ),   each with the partial maxima of what it writes.
 constexpr int kGeluFwdBytes = 65536 * 2;
 
@@ -829,22 +894,56 @@ __global__ void gelu_table_kernel(uint16_t *__restrict__ fwd, float *__restrict_
     bwd[i] = (float)(cdf + x * pdf);
 }
 
+// The gathers are served from LDS for the inputs that occur: a window of the table, the bf16 patterns with
+// exponent fields kGeluExpLo .. kGeluExpHi - 1 (2^-31 <= |x| < 2^8) of both signs, is copied into LDS by every block
+// (20 KB of the forward table, 39 KB of the backward one); zeros, denormals, tiny and huge inputs go to the full
+// table in global memory.  One L2 access per element held the kernels to 40 % / 50 % of the HBM rate.
+constexpr int kGeluExpLo = 96, kGeluExpHi = 135;
+constexpr uint32_t kGeluWinLo = kGeluExpLo << 7, kGeluWin = (kGeluExpHi - kGeluExpLo) << 7;   // 4992 magnitudes per sign
+
+template <typename T>
+__device__ __forceinline__ void gelu_window_to_lds(const T *__restrict__ table, T *win) {
+    for (uint32_t i = threadIdx.x; i < 2 * kGeluWin; i += kFusedThreads) {
+        const uint32_t sign = i >= kGeluWin ? 1u : 0u;
+        win[i] = table[(sign << 15) | (kGeluWinLo + i - sign * kGeluWin)];
+    }
+    __syncthreads();
+}
+
+template <typename T>
+__device__ __forceinline__ T gelu_lookup(uint32_t bits16, const T *win, const T *__restrict__ table) {
+    const uint32_t t = (bits16 & 0x7fffu) - kGeluWinLo;
+    if (t < kGeluWin) return win[t + (bits16 >> 15) * kGeluWin];
+    return table[bits16];
+}
+
 __global__ __launch_bounds__(kFusedThreads) void gelu_fwd_kernel(const u32x4 *__restrict__ x, int64_t n8, const uint16_t *__restrict__ fwd,
                                                                   u32x4 *__restrict__ y, float *__restrict__ parts) {
     __shared__ uint32_t red[kFusedThreads / kWave];
+    __shared__ uint16_t win[2 * kGeluWin];
+    gelu_window_to_lds(fwd, win);
     const int64_t stride = (int64_t)gridDim.x * kFusedThreads;
     uint32_t am = 0;
-    for (int64_t i = (int64_t)blockIdx.x * kFusedThreads + threadIdx.x; i < n8; i += stride) {
-        const u32x4 v = __builtin_nontemporal_load(x + i);
+    constexpr int U = 2;                                   // 16-byte chunks in flight per lane
+    int64_t i = (int64_t)blockIdx.x * kFusedThreads + threadIdx.x;
+    auto one = [&](const u32x4 v, int64_t at) {
         const uint32_t w[4] = {v.x, v.y, v.z, v.w};
         uint32_t o[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            o[q] = (uint32_t)fwd[w[q] & 0xffffu] | ((uint32_t)fwd[w[q] >> 16] << 16);
+            o[q] = (uint32_t)gelu_lookup(w[q] & 0xffffu, win, fwd) | ((uint32_t)gelu_lookup(w[q] >> 16, win, fwd) << 16);
             am = max_u16x2(am, abs_bf16x2(o[q]));
         }
-        y[i] = u32x4{o[0], o[1], o[2], o[3]};
+        y[at] = u32x4{o[0], o[1], o[2], o[3]};
+    };
+    for (; i + (U - 1) * stride < n8; i += U * stride) {
+        u32x4 v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[u] = __builtin_nontemporal_load(x + i + u * stride);
+#pragma unroll
+        for (int u = 0; u < U; ++u) one(v[u], i + u * stride);
     }
+    for (; i < n8; i += stride) one(__builtin_nontemporal_load(x + i), i);
     am = block_max_u32(fold_u16x2_to_f32bits(am), red);
     if (threadIdx.x == 0) parts[blockIdx.x] = bits_to_float(am);
     if (blockIdx.x == 0)
@@ -855,19 +954,31 @@ __global__ __launch_bounds__(kFusedThreads) void gelu_bwd_kernel(const u32x4 *__
                                                                   const float *__restrict__ bwd, u32x4 *__restrict__ dx,
                                                                   float *__restrict__ parts) {
     __shared__ uint32_t red[kFusedThreads / kWave];
+    __shared__ float win[2 * kGeluWin];
+    gelu_window_to_lds(bwd, win);
     const int64_t stride = (int64_t)gridDim.x * kFusedThreads;
     uint32_t am = 0;
-    for (int64_t i = (int64_t)blockIdx.x * kFusedThreads + threadIdx.x; i < n8; i += stride) {
-        const u32x4 v = __builtin_nontemporal_load(x + i), d = __builtin_nontemporal_load(dy + i);
+    constexpr int U = 2;
+    int64_t i = (int64_t)blockIdx.x * kFusedThreads + threadIdx.x;
+    auto one = [&](const u32x4 v, const u32x4 d, int64_t at) {
         const uint32_t w[4] = {v.x, v.y, v.z, v.w}, dw[4] = {d.x, d.y, d.z, d.w};
         uint32_t o[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            o[q] = pack2(__fmul_rn(bf16_lo(dw[q]), bwd[w[q] & 0xffffu]), __fmul_rn(bf16_hi(dw[q]), bwd[w[q] >> 16]));
+            o[q] = pack2(__fmul_rn(bf16_lo(dw[q]), gelu_lookup(w[q] & 0xffffu, win, bwd)),
+                         __fmul_rn(bf16_hi(dw[q]), gelu_lookup(w[q] >> 16, win, bwd)));
             am = max_u16x2(am, abs_bf16x2(o[q]));
         }
-        dx[i] = u32x4{o[0], o[1], o[2], o[3]};
+        dx[at] = u32x4{o[0], o[1], o[2], o[3]};
+    };
+    for (; i + (U - 1) * stride < n8; i += U * stride) {
+        u32x4 v[U], d[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) { v[u] = __builtin_nontemporal_load(x + i + u * stride); d[u] = __builtin_nontemporal_load(dy + i + u * stride); }
+#pragma unroll
+        for (int u = 0; u < U; ++u) one(v[u], d[u], i + u * stride);
     }
+    for (; i < n8; i += stride) one(__builtin_nontemporal_load(x + i), __builtin_nontemporal_load(dy + i), i);
     am = block_max_u32(fold_u16x2_to_f32bits(am), red);
     if (threadIdx.x == 0) parts[blockIdx.x] = bits_to_float(am);
     if (blockIdx.x == 0)
@@ -944,7 +1055,7 @@ extern "C" int odl_fp8_rmsnorm_amax_parts(const void *x, int src_dtype, const fl
     }
     const int64_t cpl = (cols / 8 + kWave - 1) / kWave;
     const int threads = cpl <= 8 ? kFusedThreads : 256;
-    const int rows_per_block = threads / kWave;
+    const int rows_per_block = (threads / kWave) * (cpl <= 2 ? 4 : (cpl <= 4 ? 2 : 1));   // RB rows per wave and trip
     int64_t g = (rows + rows_per_block - 1) / rows_per_block;
     g = g < 1 ? 1 : (g < grid_cap() ? g : grid_cap());
 #define ODL_RMS(SRC, CPL, THR) hipLaunchKernelGGL((rmsnorm_fwd_kernel<SRC, CPL, THR>), dim3((unsigned)g), dim3(THR), 0, stream, x, weight, rows, cols, eps, reinterpret_cast<uint16_t *>(y), rstd, parts)
@@ -1038,8 +1149,8 @@ extern "C" int odl_fp8_layernorm_amax_parts(const void *x, int src_dtype, const 
     if (cols < 8 || cols % 8 != 0 || cols > 4096 || !aligned16(x) || !aligned16(y) || !aligned16(weight) || !aligned16(bias))
         return set_error(ODL_ERR_SHAPE, "odl_fp8_layernorm_amax_parts: cols must be a multiple of 8 in [8, 4096] and the pointers 16-byte aligned");
     const int64_t cpl = (cols / 8 + kWave - 1) / kWave;
-    const int threads = cpl <= 4 ? kFusedThreads : 512;
-    const int rows_per_block = threads / kWave;
+    const int threads = cpl <= 4 ? kFusedThreads : 512;     // wider rows need more than the 128 registers of a 1024-lane block
+    const int rows_per_block = (threads / kWave) * (cpl <= 2 ? 2 : 1);   // RB rows per wave and trip
     int64_t g = (rows + rows_per_block - 1) / rows_per_block;
     g = g < 1 ? 1 : (g < grid_cap() ? g : grid_cap());
 #define ODL_LN(SRC, CPL, THR) hipLaunchKernelGGL((layernorm_fwd_kernel<SRC, CPL, THR>), dim3((unsigned)g), dim3(THR), 0, stream, x, weight, bias, rows, cols, eps, reinterpret_cast<uint16_t *>(y), mean, rstd, parts)
