@@ -292,6 +292,8 @@ extern "C" int odl_fp8_gemm_splitk(const uint8_t *a, const uint8_t *b, int64_t M
         return set_error(ODL_ERR_SHAPE, "odl_fp8_gemm_splitk: M, N, K must be multiples of 128 (256 for an operand stored K-slow) and each operand under 2 GiB; got %lld x %lld x %lld", (long long)M, (long long)N, (long long)K);
     const int64_t steps = K / 128;
     const int64_t per = ((steps + splits - 1) / (splits > 0 ? splits : 1) + 1) & ~(int64_t)1;
+    // what the kernel needs to be correct: every run at least four K steps (its load pipeline is two steps deep and runs
+    // in pairs).  odl_fp8_gemm_split_count proposes only runs of eight steps and more, which is where a split pays.
     if (splits < 2 || splits > 64 || per < 4 || steps - (splits - 1) * per < 4)
         return set_error(ODL_ERR_ARG, "odl_fp8_gemm_splitk: %d splits of K=%lld leave a run shorter than 512", splits, (long long)K);
     if (workspace_bytes < (int64_t)splits * M * N * 4)

@@ -542,12 +542,12 @@ __global__ __launch_bounds__(AMAX ? kFatThreads : kThreads) void cast_kernel(con
     }
     if constexpr (MODE == kScaleParts) s_t = dynamic_scale<FMT>(scale, margin, dyn_out, red, blockIdx.x == 0);
     uint32_t am = 0;
-    for (int64_t i = (int64_t)blockIdx.x * kT + threadIdx.x; i < nchunk; i += stride) {
+    constexpr int VP = SRC == ODL_BF16 ? 2 : 4;              // 16-byte loads per chunk of 16 elements
+    constexpr int U = SRC == ODL_BF16 ? 2 : 1;               // chunks in flight per lane
+    auto one = [&](const int64_t i, const u32x4 (&v)[VP]) {
         float f[16];
         if constexpr (SRC == ODL_BF16) {
-            const u32x4 *p = reinterpret_cast<const u32x4 *>(x) + i * 2;
-            u32x4 v0 = __builtin_nontemporal_load(p), v1 = __builtin_nontemporal_load(p + 1);
-            uint32_t w[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+            const uint32_t w[8] = {v[0].x, v[0].y, v[0].z, v[0].w, v[1].x, v[1].y, v[1].z, v[1].w};
 #pragma unroll
             for (int q = 0; q < 8; ++q) {
                 f[2 * q] = bf16_lo(w[q]);
@@ -555,10 +555,6 @@ __global__ __launch_bounds__(AMAX ? kFatThreads : kThreads) void cast_kernel(con
                 if constexpr (AMAX) am = max_u16x2(am, abs_bf16x2(w[q]));
             }
         } else {
-            const u32x4 *p = reinterpret_cast<const u32x4 *>(x) + i * 4;
-            u32x4 v[4];
-#pragma unroll
-            for (int u = 0; u < 4; ++u) v[u] = __builtin_nontemporal_load(p + u);
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
                 f[4 * u] = bits_to_float(v[u].x); f[4 * u + 1] = bits_to_float(v[u].y);
@@ -586,6 +582,23 @@ __global__ __launch_bounds__(AMAX ? kFatThreads : kThreads) void cast_kernel(con
         o.z = quantise4<FMT>(f[8], f[9], f[10], f[11], s[8], s[9], s[10], s[11]);
         o.w = quantise4<FMT>(f[12], f[13], f[14], f[15], s[12], s[13], s[14], s[15]);
         ODL_CODE_STORE(o, reinterpret_cast<u32x4 *>(out) + i);
+    };
+    const u32x4 *px = reinterpret_cast<const u32x4 *>(x);
+    int64_t i = (int64_t)blockIdx.x * kT + threadIdx.x;
+    for (; i + (U - 1) * stride < nchunk; i += U * stride) {
+        u32x4 v[U][VP];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int h = 0; h < VP; ++h) v[u][h] = __builtin_nontemporal_load(px + (i + u * stride) * VP + h);
+#pragma unroll
+        for (int u = 0; u < U; ++u) one(i + u * stride, v[u]);
+    }
+    for (; i < nchunk; i += stride) {
+        u32x4 v[VP];
+#pragma unroll
+        for (int h = 0; h < VP; ++h) v[h] = __builtin_nontemporal_load(px + i * VP + h);
+        one(i, v);
     }
     if constexpr (AMAX) {
         if constexpr (SRC == ODL_BF16) am = fold_u16x2_to_f32bits(am);
