@@ -642,12 +642,6 @@ __global__ __launch_bounds__(kThreads) void cast_generic_kernel(const void *__re
 // both outputs are written in full 64/128-byte segments.
 constexpr int kTileR = 128, kTileC = 64;
 
-// LDS placement of the transposed tile.  The LDS of gfx950 serves 64 four-byte banks per cycle, so the
-// tile is kept as 32 lines of 256 bytes, one per PAIR of tile columns (even column in the first 128
-// bytes), and each line is rotated by a multiple of 16 bytes that depends on the column:
-//   * a wave's dword writes (8 column groups x 8 consecutive row groups) land in 64 different banks,
-//   * the 16-byte reads stay aligned (ds_read_b128), and 16 consecutive lanes read one whole line.
-// Offsets in bytes; `ty` is the lane's group of 4 rows (0..31), `m16` a chunk of 16 rows (0..7).
 // Order in which consecutive blocks take tiles: panels of kCtPanel tile rows, down the rows of a panel first.
 // Blocks that run at the same time then write neighbouring 128-byte pieces of the same rows of the
 // transposed output instead of pieces that lie a whole output row (a power of two for the usual token
@@ -660,12 +654,24 @@ __device__ __forceinline__ void ct_tile_of(int64_t id, int64_t tiles_r, int64_t 
     tc = local / gl;
 }
 
-__device__ __forceinline__ int ct_lds_rot(int col) { return 8 * (col >> 3) + 4 * ((col >> 1) & 3); }
+// LDS placement of the transposed tile.  Measured on gfx950 (counting conflict cycles of single instructions):
+// a 4-byte access is served 32 lanes per cycle and its lanes must differ in (dword address mod 32); 8- and 16-byte
+// accesses are served 32 / 16 lanes per cycle over 64 four-byte banks.  The tile is kept as 32 lines of 256 bytes,
+// one per PAIR of tile columns (even column in the first 128 bytes), each line rotated by 16 bytes per group of 8
+// columns:
+//   * the dword writes of a half-wave (8 column groups x 4 consecutive row groups) differ mod 32,
+//   * the 16-byte reads stay aligned (ds_read_b128), and 16 consecutive lanes read one whole line.
+// Offsets in bytes; `ty` is the lane's group of 4 rows (0..31), `m16` a chunk of 16 rows (0..7).
+__device__ __forceinline__ int ct_lds_rot(int col) { return 4 * (col >> 3); }
 __device__ __forceinline__ int ct_lds_write_off(int col, int ty) {
     return (col >> 1) * 256 + ((((col & 1) * 32) + ty + ct_lds_rot(col)) & 63) * 4;
 }
 __device__ __forceinline__ int ct_lds_read_off(int col, int m16) {
     return (col >> 1) * 256 + ((((col & 1) * 32) + m16 * 4 + ct_lds_rot(col)) & 63) * 4;
+}
+// 16 bytes of rows m16*16.. of tile column col
+__device__ __forceinline__ u32x4 ct_lds_read(const uint8_t *tile, int col, int m16) {
+    return *reinterpret_cast<const u32x4 *>(&tile[ct_lds_read_off(col, m16)]);
 }
 
 // 4x4 byte transpose: in a[j] byte k  ->  out t[k] byte j
@@ -772,7 +778,7 @@ __device__ __forceinline__ void ct_one_tile(const void *__restrict__ x, int64_t 
         const int k = chunk / 8, m16 = chunk % 8;
         const int64_t oc = tc * kTileC + k, orow = tr * kTileR + m16 * 16;
         if (oc < cols && orow < rows) {             // rows % 16 == 0 (host-checked)
-            const u32x4 v = *reinterpret_cast<const u32x4 *>(&tile[ct_lds_read_off(k, m16)]);
+            const u32x4 v = ct_lds_read(tile, k, m16);
             __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(out_t + oc * rows + orow));
         }
     }
@@ -895,7 +901,7 @@ __global__ __launch_bounds__(kThreads) void cast_rowcol_kernel(const void *__res
         const int k = chunk / 8, m16 = chunk % 8;
         const int64_t oc = tc * kTileC + k, orow = tr * kTileR + m16 * 16;
         if (oc < cols && orow < rows) {             // rows % 16 == 0 (host-checked)
-            const u32x4 v = *reinterpret_cast<const u32x4 *>(&tile[ct_lds_read_off(k, m16)]);
+            const u32x4 v = ct_lds_read(tile, k, m16);
             __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(out_t + oc * rows + orow));
         }
     }
