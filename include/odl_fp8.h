@@ -45,7 +45,7 @@ enum odl_status {
     ODL_ERR_LAUNCH = 3    /* HIP reported an error at launch */
 };
 
-/* ABI version of this header (9); bumped when a signature changes or an entry point is added. */
+/* ABI version of this header (10); bumped when a signature changes or an entry point is added. */
 int odl_fp8_abi_version(void);
 
 /* Last error message of the calling host thread ("" if none). */
@@ -104,19 +104,25 @@ int odl_fp8_cast_dynamic(const void *x, int src_dtype, int64_t rows, int64_t col
                          odl_stream_t stream);
 
 /*
- * Current scaling of MANY tensors in two launches: every weight of a model after an optimizer step (what
- * te.pytorch.Linear does per weight and forward, transformer_engine.py:106; `fp8.param`, optim/config.py:36-37,
- * asks for weights that are kept quantised between steps).  Results per tensor are those of odl_fp8_amax_parts +
- * odl_fp8_cast_dynamic with both outputs, bit for bit.
+ * MANY tensors per launch: every weight of a model after an optimizer step (what te.pytorch.Linear does per
+ * weight and forward, transformer_engine.py:106; `fp8.param`, optim/config.py:36-37, asks for weights that are kept
+ * quantised between steps).  Results per tensor are those of the single-tensor calls, bit for bit.
  *   odl_fp8_mt_tensor : one tensor; the table of n of them is read by the kernels from DEVICE memory.
  *   odl_fp8_multi_plan: host only.  Checks a HOST copy of the table (rows a positive multiple of 16, cols of 8;
- *                       x, out_t, parts 16-byte aligned, out 8-byte, no NULL) and writes the work list of a phase,
- *                       pairs {tensor, local index} of int32, into `work` (host memory, room for `capacity` pairs;
- *                       NULL or too small: only counts).  Returns the number of pairs, -1 on error.  Tables and work
- *                       lists depend on addresses and shapes only: build them once, copy them to the device.
- *   odl_fp8_multi_amax_parts  (phase ODL_MT_AMAX): parts of every tensor <- its partial maxima.
- *   odl_fp8_multi_cast_dynamic (phase ODL_MT_CAST): codes, transposed codes and dyn_out = {amax, scale, 1/scale}
- *                       of every tensor, one format and margin for all.
+ *                       x, out_t, parts 16-byte aligned, out 8-byte, no NULL; `scale` non-NULL for the delayed phase)
+ *                       and writes the work list of a phase, pairs {tensor, local index} of int32, into `work` (host
+ *                       memory, room for `capacity` pairs; NULL or too small: only counts).  Returns the number of
+ *                       pairs, -1 on error.  Tables and work lists depend on addresses and shapes only: build them
+ *                       once, copy them to the device.
+ *   current scaling (recipe "tensorwise"), two launches:
+ *     odl_fp8_multi_amax_parts  (phase ODL_MT_AMAX): parts of every tensor <- its partial maxima;
+ *     odl_fp8_multi_cast_dynamic (phase ODL_MT_CAST): codes, transposed codes and dyn_out = {amax, scale, 1/scale}
+ *                       of every tensor as odl_fp8_amax_parts + odl_fp8_cast_dynamic give them; one format and
+ *                       margin for all.
+ *   delayed scaling (recipe "delayed"), one launch:
+ *     odl_fp8_multi_cast_delayed (phase ODL_MT_CAST_DELAYED): codes and transposed codes with the scale in force
+ *                       (*scale), block maxima folded into parts (accumulated, as odl_fp8_cast_delayed does),
+ *                       dyn_out[1] = scale, dyn_out[2] = 1/scale.
  * Nothing is allocated; the device tables are not validated again at launch.
  */
 typedef struct odl_fp8_mt_tensor {
@@ -125,14 +131,17 @@ typedef struct odl_fp8_mt_tensor {
     uint8_t *out_t;     /* codes [cols, rows] */
     float *parts;       /* ODL_FP8_AMAX_PARTS floats */
     float *dyn_out;     /* 3 floats */
+    const float *scale; /* delayed scaling: 1 float, the scale in force; NULL for current scaling */
     int64_t rows, cols;
     int32_t src_dtype;  /* odl_dtype */
     int32_t reserved;   /* 0 */
-} odl_fp8_mt_tensor;    /* 64 bytes */
-enum odl_mt_phase { ODL_MT_AMAX = 0, ODL_MT_CAST = 1 };
+} odl_fp8_mt_tensor;    /* 72 bytes */
+enum odl_mt_phase { ODL_MT_AMAX = 0, ODL_MT_CAST = 1, ODL_MT_CAST_DELAYED = 2 };
 int64_t odl_fp8_multi_plan(const odl_fp8_mt_tensor *tensors_host, int64_t n, int phase, int32_t *work_host, int64_t capacity);
 int odl_fp8_multi_amax_parts(const odl_fp8_mt_tensor *tensors_dev, const int32_t *work_dev, int64_t n_work, odl_stream_t stream);
 int odl_fp8_multi_cast_dynamic(const odl_fp8_mt_tensor *tensors_dev, const int32_t *work_dev, int64_t n_work, int fmt, int margin,
+                               odl_stream_t stream);
+int odl_fp8_multi_cast_delayed(const odl_fp8_mt_tensor *tensors_dev, const int32_t *work_dev, int64_t n_work, int fmt,
                                odl_stream_t stream);
 
 /*

@@ -1265,11 +1265,37 @@ __global__ __launch_bounds__(kThreads) void multi_cast_dynamic_kernel(const odl_
     else ct_one_tile<ODL_F32, FMT, kScaleParts, false, true>(e.x, e.rows, e.cols, nullptr, st, e.out, e.out_t, tr, tc, tile, am);
 }
 
+template <int FMT>
+__global__ __launch_bounds__(kThreads) void multi_cast_delayed_kernel(const odl_fp8_mt_tensor *__restrict__ tensors,
+                                                                       const int32_t *__restrict__ work) {
+    __shared__ __attribute__((aligned(16))) uint8_t tile[kTileC * kTileR];
+    __shared__ uint32_t red[kThreads / kWave];
+    const int32_t t = work[2 * (int64_t)blockIdx.x], local = work[2 * (int64_t)blockIdx.x + 1];
+    const odl_fp8_mt_tensor e = tensors[t];
+    const float st = e.scale[0];
+    if (local == 0 && threadIdx.x == 0) {
+        e.dyn_out[1] = st;
+        e.dyn_out[2] = __fdiv_rn(1.0f, st);
+    }
+    const int64_t tiles_r = (e.rows + kTileR - 1) / kTileR, tiles_c = (e.cols + kTileC - 1) / kTileC;
+    int64_t tr, tc;
+    ct_tile_of(tiles_r * tiles_c - 1 - local, tiles_r, tiles_c, tr, tc);
+    uint32_t am = 0;
+    if (e.src_dtype == ODL_BF16) {
+        ct_one_tile<ODL_BF16, FMT, ODL_SCALE_TENSOR, true, true>(e.x, e.rows, e.cols, nullptr, st, e.out, e.out_t, tr, tc, tile, am);
+        am = fold_u16x2_to_f32bits(am);
+    } else {
+        ct_one_tile<ODL_F32, FMT, ODL_SCALE_TENSOR, true, true>(e.x, e.rows, e.cols, nullptr, st, e.out, e.out_t, tr, tc, tile, am);
+    }
+    am = block_max_u32(am, red);
+    if (threadIdx.x == 0 && am != 0) atomicMax(reinterpret_cast<uint32_t *>(e.parts) + (local & (kAmaxParts - 1)), am);
+}
+
 }  // namespace odl
 
 extern "C" int64_t odl_fp8_multi_plan(const odl_fp8_mt_tensor *tensors, int64_t n, int phase, int32_t *work, int64_t capacity) {
     if (n < 0 || (!tensors && n > 0)) { set_error(ODL_ERR_ARG, "odl_fp8_multi_plan: bad table (n = %lld)", (long long)n); return -1; }
-    if (phase != ODL_MT_AMAX && phase != ODL_MT_CAST) { set_error(ODL_ERR_ARG, "odl_fp8_multi_plan: phase %d", phase); return -1; }
+    if (phase != ODL_MT_AMAX && phase != ODL_MT_CAST && phase != ODL_MT_CAST_DELAYED) { set_error(ODL_ERR_ARG, "odl_fp8_multi_plan: phase %d", phase); return -1; }
     int64_t count = 0;
     for (int64_t t = 0; t < n; ++t) {
         const odl_fp8_mt_tensor &e = tensors[t];
@@ -1283,6 +1309,7 @@ extern "C" int64_t odl_fp8_multi_plan(const odl_fp8_mt_tensor *tensors, int64_t 
             set_error(ODL_ERR_ARG, "odl_fp8_multi_plan: tensor %lld: null or misaligned pointer (x, out_t, parts: 16 bytes; out: 8)", (long long)t);
             return -1;
         }
+        if (phase == ODL_MT_CAST_DELAYED && !e.scale) { set_error(ODL_ERR_ARG, "odl_fp8_multi_plan: tensor %lld: the delayed phase needs `scale`", (long long)t); return -1; }
         const int64_t items = phase == ODL_MT_AMAX ? mt_amax_blocks(e.rows * e.cols / (e.src_dtype == ODL_BF16 ? 8 : 4))
                                                    : ((e.rows + kTileR - 1) / kTileR) * ((e.cols + kTileC - 1) / kTileC);
         if (t > 0x7fffffffLL || items > 0x7fffffffLL) { set_error(ODL_ERR_SHAPE, "odl_fp8_multi_plan: tensor %lld is too large", (long long)t); return -1; }
@@ -1300,6 +1327,18 @@ extern "C" int odl_fp8_multi_amax_parts(const odl_fp8_mt_tensor *tensors_dev, co
     if (!tensors_dev || !work_dev) return set_error(ODL_ERR_ARG, "odl_fp8_multi_amax_parts: null table");
     hipLaunchKernelGGL(multi_amax_kernel, dim3((unsigned)n_work), dim3(kFatThreads), 0, reinterpret_cast<hipStream_t>(stream_), tensors_dev, work_dev);
     return check_launch("odl_fp8_multi_amax_parts");
+}
+
+extern "C" int odl_fp8_multi_cast_delayed(const odl_fp8_mt_tensor *tensors_dev, const int32_t *work_dev, int64_t n_work, int fmt,
+                                          odl_stream_t stream_) {
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    if (n_work < 0 || n_work > 0x7fffffffLL) return set_error(ODL_ERR_ARG, "odl_fp8_multi_cast_delayed: n_work %lld", (long long)n_work);
+    if (fmt != ODL_FP8_E4M3 && fmt != ODL_FP8_E5M2) return set_error(ODL_ERR_ARG, "odl_fp8_multi_cast_delayed: fmt %d", fmt);
+    if (n_work == 0) return ODL_OK;
+    if (!tensors_dev || !work_dev) return set_error(ODL_ERR_ARG, "odl_fp8_multi_cast_delayed: null table");
+    if (fmt == ODL_FP8_E4M3) hipLaunchKernelGGL((multi_cast_delayed_kernel<ODL_FP8_E4M3>), dim3((unsigned)n_work), dim3(kThreads), 0, stream, tensors_dev, work_dev);
+    else hipLaunchKernelGGL((multi_cast_delayed_kernel<ODL_FP8_E5M2>), dim3((unsigned)n_work), dim3(kThreads), 0, stream, tensors_dev, work_dev);
+    return check_launch("odl_fp8_multi_cast_delayed");
 }
 
 extern "C" int odl_fp8_multi_cast_dynamic(const odl_fp8_mt_tensor *tensors_dev, const int32_t *work_dev, int64_t n_work, int fmt, int margin,

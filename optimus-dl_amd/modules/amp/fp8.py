@@ -239,13 +239,13 @@ class FP8Recipe:
     # ------------------------------------------------------- fp8.param
     def attach_params(self, model: torch.nn.Module, optimizer: "torch.optim.Optimizer | None" = None):
         """``fp8.param: true`` (optimus_dl/modules/optim/config.py:36-37): keep the weights of the model's FP8
-        Linears quantised between optimizer steps.  All of them are quantised in two launches now and, when the
-        optimizer is given, after each of its steps (a step post-hook); the forwards in between launch nothing
+        Linears quantised between optimizer steps.  All of them are quantised in one or two launches now and, when
+        the optimizer is given, after each of its steps (a step post-hook); the forwards in between launch nothing
         for the weights.  Returns the ``Fp8ParamSet`` (call its ``sync()`` yourself after a step when no optimizer
-        was given), or None for the recipes that keep the per-module route (delayed, rowwise)."""
+        was given), or None for the rowwise recipe, which keeps the per-module route."""
         from ..fp8_linear import Fp8ParamSet
 
-        if self._recipe.kind != "tensorwise":
+        if self._recipe.kind not in ("tensorwise", "delayed"):
             _info_once(f"fp8.param: the '{self._recipe.kind}' recipe quantises each weight in its own module (cached per parameter "
                        "version); nothing to attach")
             return None

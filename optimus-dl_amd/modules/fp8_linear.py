@@ -57,17 +57,25 @@ def _warn_once(msg: str) -> None:
 class _WeightCache:
     """Quantised weight + transpose, valid while the Parameter is unchanged."""
 
-    __slots__ = ("key", "wq", "wq_t", "s_inv", "s_inv_t", "amax")
+    __slots__ = ("key", "wq", "wq_t", "s_inv", "s_inv_t", "amax", "kept")
 
     def __init__(self):
         self.key = None
         self.wq = self.wq_t = self.s_inv = self.s_inv_t = self.amax = None
+        # set by an Fp8ParamSet: what its codes were made from (address, version, format, recipe kind, margin); while
+        # that still describes the weight and the recipe, the codes are used as they are, whatever the scale has done
+        # since (under delayed scaling the set quantises once per optimizer step, not once per microbatch)
+        self.kept = None
 
 
 def _weight_key(weight: torch.Tensor, fmt: int, how: tuple) -> tuple:
     """What cached codes of a weight depend on: its storage, its contents (version counter), the format and
     how the scale is found."""
     return (weight.data_ptr(), _state.tensor_version(weight), fmt, how)
+
+
+def _kept_stamp(weight: torch.Tensor, pol) -> tuple:
+    return (weight.data_ptr(), _state.tensor_version(weight), pol.fmt_fwd, pol.kind, pol.margin)
 
 
 def _quantise_dynamic(x2d: torch.Tensor, fmt: int, margin: int, need_t: bool, need_rowmajor: bool = True,
@@ -346,6 +354,8 @@ class FP8Linear(nn.Linear):
         """Per-tensor quantised weight (and transpose), cached on the parameter version."""
         pol = recipe.recipe
         c = self._wcache
+        if c.kept is not None and recipe.cache_weights and c.kept == _kept_stamp(weight, pol):
+            return c.wq, c.wq_t, c.s_inv
         record = self.training
         meta = None
         # the codes depend on the parameter's contents, the format and how the scale is found; under delayed
@@ -443,47 +453,64 @@ class Fp8ParamSet:
     """The weights of a model's FP8 Linears kept quantised between optimizer steps (``fp8.param: true``,
     optimus_dl/modules/optim/config.py:36-37,56: declared there and never read).
 
-    Without it every ``FP8Linear`` quantises its own weight on the first forward after the weight changed: an
-    amax launch and a cast+transpose launch per weight and optimizer step (a model of 196 Linears: 392 launches
-    and as many allocations).  With it, :meth:`sync` quantises all of them in TWO launches into buffers that live
-    as long as the set, and stamps every module's weight cache with the parameter version it quantised, so the
-    forwards that follow launch nothing for the weights.  The codes and scales are the same bits either way.
+    Without it every ``FP8Linear`` quantises its own weight on the first forward after the weight changed (under
+    delayed scaling: in every forward, with the scale refreshed since): one or two launches per weight (a model of 196
+    Linears: up to 392 launches and as many allocations per step).  With it, :meth:`sync` quantises all of them in TWO
+    launches (current scaling) or ONE (delayed scaling) into buffers that live as long as the set, and stamps every
+    module's weight cache, so the forwards that follow launch nothing for the weights.
+
+    * tensorwise: codes and scales are the same bits as on the per-module route.
+    * delayed: the weights are cast with the scales in force at the ``sync`` and their maxima recorded for the next
+      refresh; the microbatches of one optimizer step all use these codes (what the reference's backend does when it is
+      told that the weights are cached), where the per-module route casts again in every forward.  With one forward per
+      optimizer step both routes give the same bits.
 
     ``sync`` belongs right after ``optimizer.step()`` (``attach`` registers it as a step post-hook when handed the
     optimizer); it rewrites the buffers in place, so no backward that still needs the previous codes may be pending,
-    the same rule as for the optimizer's own in-place update.  A weight that changes without a ``sync`` (a
-    checkpoint load, a manual edit) is simply quantised by its module on the next forward, as without the set.
-    Current scaling ("tensorwise") only: the other recipes keep their per-module route."""
+    the same rule as for the optimizer's own in-place update.  A weight that changes without a ``sync`` (a checkpoint
+    load, a manual edit) is simply quantised by its module on the next forward, as without the set.  The rowwise
+    recipe keeps its per-module route."""
 
     def __init__(self, modules: list["FP8Linear"], recipe: FP8Recipe):
         pol = recipe.recipe
-        if pol.kind != "tensorwise":
-            raise ValueError(f"Fp8ParamSet serves the tensorwise recipe, not '{pol.kind}'")
+        if pol.kind not in ("tensorwise", "delayed"):
+            raise ValueError(f"Fp8ParamSet serves the tensorwise and delayed recipes, not '{pol.kind}'")
         self.recipe = recipe
         self.modules: list[FP8Linear] = []
-        self.skipped: list[FP8Linear] = []          # shapes / dtypes the two-launch route does not take: per-module route
+        self.skipped: list[FP8Linear] = []          # shapes / dtypes the multi-tensor route does not take: per-module route
         for m in modules:
             (self.modules if native.MultiTensorPlan.eligible(m.weight.detach()) else self.skipped).append(m)
         self._plan: native.MultiTensorPlan | None = None
         self._index: list[int] = []
+        self._metas: list = []
         self.syncs = 0
 
     def _build(self) -> None:
-        sources, index, seen = [], [], {}
+        pol = self.recipe.recipe
+        sources, index, seen, scales, parts, metas = [], [], {}, [], [], []
         for m in self.modules:
             w = m.weight.detach()
             at = seen.get(w.data_ptr())
             if at is None:                           # Linears that share one Parameter share its codes
                 at = seen[w.data_ptr()] = len(sources)
                 sources.append(w)
+                if pol.kind == "delayed":            # the first module of a shared Parameter lends its weight role
+                    meta = m._meta(self.recipe, w.device, "fwd")
+                    scales.append(meta.scale_of(ROLE_W))
+                    parts.append(meta.amax_slot(ROLE_W))
+                    metas.append(meta)
             index.append(at)
-        pol = self.recipe.recipe
-        self._plan = native.MultiTensorPlan(sources, pol.fmt_fwd, pol.margin) if sources else None
-        self._index = index
+        if not sources:
+            self._plan = None
+        elif pol.kind == "delayed":
+            self._plan = native.MultiTensorPlan(sources, pol.fmt_fwd, pol.margin, scales=scales, parts=parts)
+        else:
+            self._plan = native.MultiTensorPlan(sources, pol.fmt_fwd, pol.margin)
+        self._index, self._metas = index, metas
 
     @torch.no_grad()
     def sync(self) -> None:
-        """Quantise every weight of the set now (two launches on the current stream)."""
+        """Quantise every weight of the set now (on the current stream)."""
         if not self.modules:
             return
         if self._plan is None or len(self._index) != len(self.modules) or self._plan.stale() or \
@@ -491,12 +518,18 @@ class Fp8ParamSet:
             self._build()                            # first use, or a parameter's storage moved (.to(), a new optimizer state)
         plan, pol = self._plan, self.recipe.recipe
         plan.run()
+        for meta in self._metas:                     # delayed: the next refresh has to fold what was just recorded
+            meta.note_record(self.recipe._store)
         how = (pol.kind, pol.margin)
         for m, i in zip(self.modules, self._index):
             c = m._wcache
-            c.wq, c.wq_t = plan.codes[i], plan.codes_t[i]
-            c.amax, c.s_inv = plan.dyn[i, 0:1], plan.dyn[i, 2:3]
-            c.key = _weight_key(m.weight, pol.fmt_fwd, how)
+            c.wq, c.wq_t, c.s_inv = plan.codes[i], plan.codes_t[i], plan.dyn[i, 2:3]
+            c.kept = _kept_stamp(m.weight, pol)
+            if pol.kind == "tensorwise":
+                c.amax = plan.dyn[i, 0:1]
+                c.key = _weight_key(m.weight, pol.fmt_fwd, how)
+            else:
+                c.amax, c.key = None, None
         self.syncs += 1
 
     @classmethod

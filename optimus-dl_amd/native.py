@@ -24,7 +24,7 @@ DT_BF16, DT_F32 = 0, 1
 AMAX_MAX, AMAX_MOST_RECENT = 0, 1
 FP8_MAX = {E4M3: 448.0, E5M2: 57344.0}
 TORCH_FP8 = {E4M3: torch.float8_e4m3fn, E5M2: torch.float8_e5m2}
-ABI_VERSION = 9
+ABI_VERSION = 10
 AMAX_PARTS = 512                       # ODL_FP8_AMAX_PARTS
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
@@ -43,6 +43,7 @@ EXPORTS = (
     "odl_fp8_multi_plan",
     "odl_fp8_multi_amax_parts",
     "odl_fp8_multi_cast_dynamic",
+    "odl_fp8_multi_cast_delayed",
     "odl_fp8_amax_parts_colsum",
     "odl_fp8_swiglu_amax_parts",
     "odl_fp8_swiglu_bwd_amax_parts",
@@ -108,6 +109,7 @@ def load() -> ctypes.CDLL:
         L.odl_fp8_multi_plan.restype = ctypes.c_int64
         L.odl_fp8_multi_amax_parts.argtypes = [vp, vp, i64, vp]
         L.odl_fp8_multi_cast_dynamic.argtypes = [vp, vp, i64, i32, i32, vp]
+        L.odl_fp8_multi_cast_delayed.argtypes = [vp, vp, i64, i32, vp]
         L.odl_fp8_amax_parts_colsum.argtypes = [vp, i32, i64, i64, vp, vp, vp, vp]
         L.odl_fp8_swiglu_amax_parts.argtypes = [vp, vp, i64, i64, vp, vp, vp]
         L.odl_fp8_swiglu_bwd_amax_parts.argtypes = [vp, vp, vp, i64, i64, vp, vp, vp, vp, vp]
@@ -296,22 +298,26 @@ def cast_dynamic_noalloc(x: torch.Tensor, fmt: int, margin: int, out: torch.Tens
 
 
 class MultiTensorPlan:
-    """Current scaling of many tensors in two launches (``odl_fp8_multi_amax_parts`` + ``odl_fp8_multi_cast_dynamic``).
+    """Many tensors quantised per launch.  Current scaling (``scales`` None): ``odl_fp8_multi_amax_parts`` +
+    ``odl_fp8_multi_cast_dynamic``, two launches.  Delayed scaling (``scales`` and ``parts`` given, one 1-element scale
+    and one AMAX_PARTS strip per tensor, e.g. views into a scaling arena): ``odl_fp8_multi_cast_delayed``, one launch
+    that casts with the scales in force and folds the maxima into the strips.
 
-    Built once from the source tensors: allocates every output (codes, transposed codes, partial maxima,
-    {amax, scale, 1/scale} per tensor), the table that describes them and the two work lists, all on the
-    tensors' device.  :meth:`run` allocates nothing and launches two kernels on the current stream; it writes
-    the same buffers every time.  Sources must be 2-D, contiguous, bf16 or fp32, rows a multiple of 16 and
-    columns of 8 (``eligible``).  The plan holds the sources' ADDRESSES: ``stale()`` tells whether one moved."""
+    Built once from the source tensors: allocates every output (codes, transposed codes, {amax, scale, 1/scale} per
+    tensor, and the partial maxima for current scaling), the table that describes them and the work lists, all on the
+    tensors' device.  :meth:`run` allocates nothing and writes the same buffers every time.  Sources must be 2-D,
+    contiguous, bf16 or fp32, rows a multiple of 16 and columns of 8 (``eligible``).  The plan holds ADDRESSES:
+    ``stale()`` tells whether a source (or a scale / strip) moved."""
 
-    MT_AMAX, MT_CAST = 0, 1
+    MT_AMAX, MT_CAST, MT_CAST_DELAYED = 0, 1, 2
 
     @staticmethod
     def eligible(x: torch.Tensor) -> bool:
         return (x.is_cuda and x.dim() == 2 and x.is_contiguous() and x.dtype in (torch.bfloat16, torch.float32)
                 and x.shape[0] > 0 and x.shape[0] % 16 == 0 and x.shape[1] > 0 and x.shape[1] % 8 == 0 and x.data_ptr() % 16 == 0)
 
-    def __init__(self, sources: list[torch.Tensor], fmt: int, margin: int = 0):
+    def __init__(self, sources: list[torch.Tensor], fmt: int, margin: int = 0, scales: list[torch.Tensor] | None = None,
+                 parts: list[torch.Tensor] | None = None):
         if not sources:
             raise NativeError("MultiTensorPlan: no tensors")
         for x in sources:
@@ -321,24 +327,40 @@ class MultiTensorPlan:
         dev = sources[0].device
         if any(x.device != dev for x in sources):
             raise NativeError("MultiTensorPlan: tensors on different devices")
-        self.sources, self.fmt, self.margin, self.device = list(sources), fmt, margin, dev
+        self.delayed = scales is not None
         n = len(sources)
+        if self.delayed:
+            if parts is None or len(scales) != n or len(parts) != n:
+                raise NativeError("MultiTensorPlan: delayed scaling needs one scale and one strip of partial maxima per tensor")
+            for sc, pt in zip(scales, parts):
+                _f32_dev(sc, 1, "MultiTensorPlan scale")
+                _f32_dev(pt, AMAX_PARTS, "MultiTensorPlan partial maxima")
+            self.scales, self.parts = list(scales), list(parts)
+        else:
+            self.scales = None
+            strips = torch.zeros((n, AMAX_PARTS), dtype=torch.float32, device=dev)
+            self.parts = [strips[i] for i in range(n)]
+        self.sources, self.fmt, self.margin, self.device = list(sources), fmt, margin, dev
         self.codes = [torch.empty(tuple(x.shape), dtype=torch.uint8, device=dev) for x in sources]
         self.codes_t = [torch.empty((x.shape[1], x.shape[0]), dtype=torch.uint8, device=dev) for x in sources]
-        self.parts = torch.zeros((n, AMAX_PARTS), dtype=torch.float32, device=dev)
         self.dyn = torch.zeros((n, 3), dtype=torch.float32, device=dev)          # rows {amax, scale, 1/scale}
-        self._ptrs = [x.data_ptr() for x in sources]
-        # odl_fp8_mt_tensor: five pointers, rows, cols, {src_dtype, reserved} = 8 x 8 bytes
-        table = np.zeros((n, 8), dtype=np.int64)
+        self._ptrs = self._addresses()
+        # odl_fp8_mt_tensor: six pointers, rows, cols, {src_dtype, reserved} = 9 x 8 bytes
+        table = np.zeros((n, 9), dtype=np.int64)
         for i, x in enumerate(sources):
             table[i] = (x.data_ptr(), self.codes[i].data_ptr(), self.codes_t[i].data_ptr(), self.parts[i].data_ptr(),
-                        self.dyn[i].data_ptr(), x.shape[0], x.shape[1], _src_dtype(x))
-        self._work = [self.plan_work(table, phase).to(dev) for phase in (self.MT_AMAX, self.MT_CAST)]
+                        self.dyn[i].data_ptr(), self.scales[i].data_ptr() if self.delayed else 0, x.shape[0], x.shape[1], _src_dtype(x))
+        phases = (self.MT_CAST_DELAYED,) if self.delayed else (self.MT_AMAX, self.MT_CAST)
+        self._work = [self.plan_work(table, phase).to(dev) for phase in phases]
         self._table = torch.from_numpy(table).to(dev)
+
+    def _addresses(self) -> list[int]:
+        extra = (self.scales + self.parts) if self.delayed else []
+        return [t.data_ptr() for t in self.sources + extra]
 
     @staticmethod
     def plan_work(table: "np.ndarray", phase: int) -> torch.Tensor:
-        """The work list of one phase for a host copy of the table ([n, 8] int64), as a [count, 2] int32 CPU tensor."""
+        """The work list of one phase for a host copy of the table ([n, 9] int64), as a [count, 2] int32 CPU tensor."""
         L = load()
         n = table.shape[0]
         count = L.odl_fp8_multi_plan(table.ctypes.data, n, phase, None, 0)
@@ -350,10 +372,15 @@ class MultiTensorPlan:
         return work
 
     def stale(self) -> bool:
-        return any(x.data_ptr() != p for x, p in zip(self.sources, self._ptrs))
+        return self._addresses() != self._ptrs
 
     def run(self) -> None:
         L, stream = load(), _stream()
+        if self.delayed:
+            (w_cast,) = self._work
+            _check(L.odl_fp8_multi_cast_delayed(self._table.data_ptr(), w_cast.data_ptr(), w_cast.shape[0], self.fmt, stream),
+                   "odl_fp8_multi_cast_delayed")
+            return
         w_amax, w_cast = self._work
         _check(L.odl_fp8_multi_amax_parts(self._table.data_ptr(), w_amax.data_ptr(), w_amax.shape[0], stream), "odl_fp8_multi_amax_parts")
         _check(L.odl_fp8_multi_cast_dynamic(self._table.data_ptr(), w_cast.data_ptr(), w_cast.shape[0], self.fmt, self.margin, stream),

@@ -94,9 +94,9 @@ class TrainingContext:
 
     def attach_fp8_params(self, model: torch.nn.Module, optimizer: "torch.optim.Optimizer | None" = None):
         """``amp.fp8.param: true``: the weights of the model's FP8 Linears stay quantised between optimizer steps
-        (all of them re-quantised in two launches after each step).  Call once, after ``setup_training_context``
+        (all of them re-quantised in one or two launches after each step).  Call once, after ``setup_training_context``
         and after model and optimizer exist.  Returns the parameter set, or None when the key is off, FP8 is not
-        in use, or the recipe keeps the per-module route.  The reference declares the key and never reads it
+        in use, or the recipe (rowwise) keeps the per-module route.  The reference declares the key and never reads it
         (optimus_dl/modules/optim/config.py:36-37,56)."""
         if self._fp8_recipe is None or not self.optimization_config.amp.fp8.param:
             return None

@@ -55,6 +55,34 @@ def test_multi_tensor_route_equals_the_per_tensor_route_and_the_oracle(N, fmt, m
     assert plan.stale()
 
 
+@pytest.mark.parametrize("fmt", [O.E4M3, O.E5M2])
+def test_multi_tensor_delayed_cast_equals_the_single_tensor_call(N, fmt):
+    """One launch for all tensors under delayed scaling: codes, transposed codes, recorded maxima and 1/scale as
+    odl_fp8_cast_delayed gives them per tensor; the strips accumulate over two runs."""
+    xs = [seeded_bf16((r, c), std, 60 + i).to(dt).cuda() for i, (r, c, dt, std) in enumerate(SHAPES)]
+    n = len(xs)
+    scales = torch.tensor([2.0, 0.5, 448.0 / 3, 1.0, 64.0, 3000.0], device="cuda")
+    strips = torch.zeros((n, N.AMAX_PARTS), device="cuda")
+    plan = N.MultiTensorPlan(xs, fmt, scales=[scales[i:i + 1] for i in range(n)], parts=[strips[i] for i in range(n)])
+    plan.run()
+    torch.cuda.synchronize()
+    for i, x in enumerate(xs):
+        own = torch.zeros(N.AMAX_PARTS, device="cuda")
+        q, q_t, s_inv = N.cast_delayed(x, scales[i:i + 1], fmt, amax_parts=own, want_transposed=True)
+        assert_bytes_equal(plan.codes[i], q, f"tensor {i}: codes")
+        assert_bytes_equal(plan.codes_t[i], q_t, f"tensor {i}: transposed codes")
+        assert_f32_bits_equal(plan.dyn[i, 2:3], s_inv, f"tensor {i}: 1/scale")
+        assert plan.dyn[i, 1].item() == scales[i].item()
+        assert strips[i].max().item() == own.max().item() == x.float().abs().max().item()
+        if x.numel() <= 1 << 20:
+            assert_bytes_equal(plan.codes[i], O.t_cast(x.cpu(), scales[i:i + 1].cpu(), fmt), f"tensor {i}: codes vs oracle")
+    before = strips.amax(dim=1).clone()
+    for x in xs:
+        x.mul_(0.25)
+    plan.run()                                                     # smaller values: the strips keep the earlier maxima
+    assert torch.equal(strips.amax(dim=1), before)
+
+
 def test_multi_tensor_plan_refuses_what_the_kernels_cannot_take(N):
     ok = torch.zeros((32, 16), dtype=torch.bfloat16, device="cuda")
     for bad in (torch.zeros((30, 16), dtype=torch.bfloat16, device="cuda"), torch.zeros((32, 12), dtype=torch.bfloat16, device="cuda"),
@@ -161,7 +189,9 @@ def test_training_context_attaches_the_set_when_the_config_says_param(amp):
     net = build()
     opt = torch.optim.SGD(net.parameters(), lr=0.1)
     assert ctx_for(recipe="tensorwise", param=False).attach_fp8_params(net, opt) is None
-    assert ctx_for(recipe="delayed", param=True).attach_fp8_params(net, opt) is None        # per-module route for that recipe
+    assert ctx_for(recipe="rowwise", param=True).attach_fp8_params(net, opt) is None        # per-module route for that recipe
+    delayed = ctx_for(recipe="delayed", param=True, amax_history_len=8).attach_fp8_params(build(), None)
+    assert delayed is not None and delayed._plan.delayed
     ps = ctx_for(recipe="tensorwise", param=True).attach_fp8_params(net, opt)
     assert ps is not None and ps.syncs == 1
     opt.step()
@@ -169,3 +199,57 @@ def test_training_context_attaches_the_set_when_the_config_says_param(amp):
     bf16 = TrainingContext(OptimizationConfig(amp=AmpConfig(enabled=True, dtype="torch.bfloat16", fp8=Fp8Config(enabled=True, param=True))))
     bf16.setup_training_context(torch.device("cuda"))
     assert bf16.attach_fp8_params(net, opt) is None
+
+
+def test_param_set_under_delayed_scaling_matches_the_per_module_route(N, amp):
+    """One forward per optimizer step: the set casts every weight right after the step with the scale the next forward
+    would use and records its amax for the same refresh, so outputs, histories and scales are the bits of the
+    per-module route.  With two microbatches the set's codes are reused (no weight launches), where the per-module
+    route casts again with the refreshed scale."""
+    plain, kept = build(), build()
+    recipe_a = amp.create_fp8_recipe("delayed", "hybrid", amax_history_len=4)
+    recipe_b = amp.create_fp8_recipe("delayed", "hybrid", amax_history_len=4)
+    opt_a, opt_b = torch.optim.SGD(plain.parameters(), lr=0.05), torch.optim.SGD(kept.parameters(), lr=0.05)
+    ps = recipe_b.attach_params(kept, opt_b)
+    assert ps is not None and len(ps.modules) == 3 and ps._plan.delayed and len(ps._plan.sources) == 2
+    calls = {"n": 0}
+    real = N.cast_delayed
+
+    def counted(x, *a, **kw):
+        if x.dtype == torch.float32:                               # weights here are fp32, activations bf16
+            calls["n"] += 1
+        return real(x, *a, **kw)
+
+    try:
+        N.cast_delayed = counted
+        for step in range(6):
+            x = seeded_bf16((64, 256), 1.0 + 0.2 * step, 400 + step).cuda()
+            outs = []
+            for net, recipe, opt in ((plain, recipe_a, opt_a), (kept, recipe_b, opt_b)):
+                before = calls["n"]
+                with amp.fp8_autocast(torch.device("cuda"), recipe):
+                    y, z = net(x)
+                    loss = y.float().square().mean() + z.float().square().mean()
+                with amp.fp8_backward(recipe):
+                    loss.backward()
+                outs.append((y.detach().clone(), calls["n"] - before))
+                opt.step()
+                opt.zero_grad(set_to_none=True)
+            assert torch.equal(outs[0][0], outs[1][0]), f"step {step}: outputs differ"
+            assert outs[0][1] == 3 and outs[1][1] == 0, outs
+            for name in ("a", "b"):
+                for direction in ("scaling_fwd", "scaling_bwd"):
+                    ma, mb = getattr(plain, name).fp8_meta[direction], getattr(kept, name).fp8_meta[direction]
+                    assert torch.equal(ma.amax_history, mb.amax_history) and torch.equal(ma.scale, mb.scale), (step, name, direction)
+        assert (kept.a.fp8_meta["scaling_fwd"].scale != 1.0).any()
+        # two microbatches per optimizer step: nothing is launched for the weights in either forward
+        before = calls["n"]
+        for micro in range(2):
+            with amp.fp8_autocast(torch.device("cuda"), recipe_b):
+                y, z = kept(x)
+            with amp.fp8_backward(recipe_b):
+                (y.float().square().mean() + z.float().square().mean()).backward()
+        assert calls["n"] == before
+        opt_b.step()
+    finally:
+        N.cast_delayed = real

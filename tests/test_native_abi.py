@@ -35,6 +35,12 @@ def test_library_exports_every_declared_symbol():
     assert b"generic" in lib.odl_fp8_gemm_variant_name(0)
 
 
+def torch_equal(a, b):
+    import torch
+
+    return torch.equal(a, b)
+
+
 def test_multi_tensor_planner_counts_work_and_refuses_bad_tables():
     """odl_fp8_multi_plan is host code: blocks of the amax pass (one per 64 KB, at most 512 per tensor), tiles of the
     cast (128 x 64), and the checks on shapes and pointers."""
@@ -44,19 +50,23 @@ def test_multi_tensor_planner_counts_work_and_refuses_bad_tables():
 
     if not native.is_built():
         pytest.skip("library not built")
-    table = np.zeros((3, 8), dtype=np.int64)
-    table[0] = (4096, 8192, 16384, 32768, 64, 1024, 1024, native.DT_BF16)           # 2 MB: 32 blocks, 8 x 16 tiles
-    table[1] = (4096, 8192, 16384, 32768, 64, 3072, 1024, native.DT_F32)            # 12 MB: 192 blocks, 24 x 16 tiles
-    table[2] = (4096, 8192, 16384, 32768, 64, 16384, 16384, native.DT_BF16)         # 512 MB: capped at 512 blocks
+    table = np.zeros((3, 9), dtype=np.int64)       # x, out, out_t, parts, dyn_out, scale, rows, cols, {src_dtype, reserved}
+    table[0] = (4096, 8192, 16384, 32768, 64, 0, 1024, 1024, native.DT_BF16)           # 2 MB: 32 blocks, 8 x 16 tiles
+    table[1] = (4096, 8192, 16384, 32768, 64, 0, 3072, 1024, native.DT_F32)            # 12 MB: 192 blocks, 24 x 16 tiles
+    table[2] = (4096, 8192, 16384, 32768, 64, 0, 16384, 16384, native.DT_BF16)         # 512 MB: capped at 512 blocks
     amax, cast = native.MultiTensorPlan.plan_work(table, 0), native.MultiTensorPlan.plan_work(table, 1)
     assert amax.shape == (32 + 192 + 512, 2) and cast.shape == (128 + 384 + 128 * 256, 2)
     assert amax[:32, 0].eq(0).all() and amax[:32, 1].tolist() == list(range(32)) and amax[32, :].tolist() == [1, 0]
     assert cast[-1].tolist() == [2, 128 * 256 - 1]
-    for col, bad in ((5, 1000), (6, 1020), (7, 5), (0, 0), (2, 16392), (1, 8196), (3, 0)):
+    for col, bad in ((6, 1000), (7, 1020), (8, 5), (0, 0), (2, 16392), (1, 8196), (3, 0)):
         t = table.copy()
         t[1, col] = bad
         with pytest.raises(native.NativeError, match="odl_fp8_multi_plan"):
             native.MultiTensorPlan.plan_work(t, 0)
+    with pytest.raises(native.NativeError, match="needs `scale`"):                      # the delayed phase reads *scale
+        native.MultiTensorPlan.plan_work(table, 2)
+    table[:, 5] = 128
+    assert torch_equal(native.MultiTensorPlan.plan_work(table, 2), cast)
     assert native.load().odl_fp8_multi_plan(None, 0, 0, None, 0) == 0
     assert native.load().odl_fp8_multi_plan(table.ctypes.data, 3, 7, None, 0) == -1
 
