@@ -292,7 +292,7 @@ def mlp_block(torch, native, recipe, steps=10, warmup=3):
     return out
 
 
-def llama_block(torch, steps=6, warmup=2):
+def llama_block(torch, steps=6, warmup=3):
     """One Llama-3-8B decoder block (RMSNorm, GQA attention with 32 / 8 heads, SwiGLU MLP; fp32 residual stream,
     batch 4 x 2048 tokens), forward + backward, weights re-quantised every step: bf16 autocast, FP8 Linears alone, and FP8
     Linears with the fused RMSNorm / SwiGLU producers.  Attention itself is PyTorch's scaled_dot_product_attention in all three."""
@@ -418,9 +418,9 @@ def clock_probe(torch, native, launches=20, settle=40):
     """What clock the board grants while the matrix pipe is busy, and what the pipe delivers at that clock.
 
     (1) The forward GEMM of the gate projection (8192 x 14336 x 4096) back to back, once on operands quantised from
-    Gaussian data and once on all-zero codes, with a clock stamp (shader-clock counter and constant 100 MHz counter,
-    read by a one-wave kernel) before and after the run: time per launch, TFLOP/s, and the average shader clock over
-    the run.  (2) The same MFMA instruction in a register-only loop (one wave per SIMD on every compute unit, no
+    Gaussian data and once on all-zero codes: time per launch, TFLOP/s, and the shader clock during the launches (the
+    kernel's first wave reads the shader-clock counter and the constant 100 MHz counter on entry and on exit:
+    `odl_fp8_gemm_set_clock_probe`).  (2) The same MFMA instruction in a register-only loop (one wave per SIMD on every compute unit, no
     memory traffic), zero and Gaussian-like operands: rate and clock.  `of_peak_at_clock` prices a rate against
     CUs x 8192 flop per clock x the measured clock instead of the nominal 2.4 GHz.
     Every measurement follows `settle` launches of the same work: from idle the board runs a handful of launches
@@ -431,7 +431,6 @@ def clock_probe(torch, native, launches=20, settle=40):
 
     lib = ctypes.CDLL(PROBE_LIB_PATH)                      # built in-tree by optimus_dl_amd.build.build_probe()
     vp = ctypes.c_void_p
-    lib.odl_probe_clock_stamp.argtypes = [vp, vp]
     lib.odl_probe_mfma_loop.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, vp, vp]
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     flop_per_clock = cus * 8192.0                          # dense FP8 MFMA: 4 SIMDs x (2 x 32 x 32 x 64 flop / 64 clocks) per CU
@@ -451,21 +450,22 @@ def clock_probe(torch, native, launches=20, settle=40):
     xq, _, _, _, sx = native.quantize_dynamic(x, native.E4M3, 0, want_transposed=False)
     wq, _, _, _, sw = native.quantize_dynamic(w, native.E4M3, 0, want_transposed=False)
     c = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
-    stamps = torch.zeros((2, 2), dtype=torch.int64, device="cuda")
+    records = torch.zeros((launches, 4), dtype=torch.int64, device="cuda")     # per launch: clocks and 100 MHz ticks, entry and exit
     for label, a, b in (("gaussian_operands", xq, wq), ("zero_operands", torch.zeros_like(xq), torch.zeros_like(wq))):
         for _ in range(settle):
             native.gemm_nt(a, b, native.E4M3, native.E4M3, sx, sw, out=c)
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        lib.odl_probe_clock_stamp(stamps[0].data_ptr(), stream())
+        native.gemm_set_clock_probe(records)
         e0.record()
         for _ in range(launches):
             native.gemm_nt(a, b, native.E4M3, native.E4M3, sx, sw, out=c)
         e1.record()
-        lib.odl_probe_clock_stamp(stamps[1].data_ptr(), stream())
+        native.gemm_set_clock_probe(None)
         torch.cuda.synchronize()
-        d = (stamps[1] - stamps[0]).tolist()
+        r = records.double()
+        mhz = float((100.0 * (r[:, 2] - r[:, 0]) / (r[:, 3] - r[:, 1])).mean())     # counters read by one wave inside each launch
         us = 1e3 * e0.elapsed_time(e1) / launches
-        entry = priced(2.0 * M * N * K / (us * 1e-6) / 1e12, 100.0 * d[0] / d[1])
+        entry = priced(2.0 * M * N * K / (us * 1e-6) / 1e12, mhz)
         entry["us_per_launch"] = round(us, 1)
         out["gemm_8192x14336x4096"][label] = entry
     sink = torch.zeros(1, device="cuda")

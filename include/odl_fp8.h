@@ -45,7 +45,7 @@ enum odl_status {
     ODL_ERR_LAUNCH = 3    /* HIP reported an error at launch */
 };
 
-/* ABI version of this header (10); bumped when a signature changes or an entry point is added. */
+/* ABI version of this header (11); bumped when a signature changes or an entry point is added. */
 int odl_fp8_abi_version(void);
 
 /* Last error message of the calling host thread ("" if none). */
@@ -404,6 +404,13 @@ int odl_fp8_delayed_update(float *history, int64_t H, int64_t R, int64_t ld,
  * mutable process state.  odl_fp8_gemm_variant_name returns a short description ("256x256x128 w4 s2").
  */
 int odl_fp8_gemm_num_variants(void);
+/*
+ * Measurement aid (host thread-local, like odl_fp8_gemm_set_variant; NULL switches it off): launch i of the streaming
+ * GEMM kernel made from this thread afterwards writes record i % capacity of records_dev, 4 x uint64 =
+ * {shader-clock counter, 100 MHz counter} on entry and on exit of the kernel's first wave.  (exit - entry) of the
+ * first over (exit - entry) of the second, times 100 MHz, is the average shader clock the board granted that launch.
+ */
+int odl_fp8_gemm_set_clock_probe(uint64_t *records_dev, int capacity);
 const char *odl_fp8_gemm_variant_name(int variant);
 int odl_fp8_gemm_set_variant(int variant);
 

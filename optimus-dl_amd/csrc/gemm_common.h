@@ -24,6 +24,9 @@ struct GemmArgs {
     // streaming kernel only: splits > 1 cuts K into `splits` runs of `split_steps` 128-byte steps (an even number;
     // the last run may be shorter) and `c` is an fp32 workspace [splits, M, N] of unscaled partial results
     int splits = 1, split_steps = 0;
+    // streaming kernel only, measurement aid: when set, the first wave of block 0 writes {shader-clock counter,
+    // 100 MHz counter} on entry and on exit (4 x uint64): the average clock the board granted this launch
+    unsigned long long *clock_out = nullptr;
 };
 
 __device__ __forceinline__ int swz(int row) { return (row ^ (row >> 3)) & 7; }

@@ -93,6 +93,10 @@ constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 // Forced kernel variant of the calling host thread (-1: choose by shape).  Thread-local: a test or a tuning
 // sweep that pins a variant cannot change the kernels another thread (e.g. the autograd worker) launches.
 static thread_local int t_forced_variant = -1;
+// Clock probe of the calling host thread (see odl_fp8_gemm_set_clock_probe): launch i of the streaming kernel writes
+// record i % capacity.
+static thread_local unsigned long long *t_clock_probe = nullptr;
+static thread_local int t_clock_capacity = 0, t_clock_next = 0;
 
 template <int FA, int FB>
 static void launch_generic_fmt(const GemmArgs &g, hipStream_t stream) {
@@ -138,6 +142,20 @@ extern "C" int odl_fp8_gemm_num_variants(void) { return kNumVariants; }
 
 extern "C" const char *odl_fp8_gemm_variant_name(int variant) {
     return (variant >= 0 && variant < kNumVariants) ? kVariants[variant].name : "";
+}
+
+static void attach_clock_probe(GemmArgs &g) {
+    if (!t_clock_probe) return;
+    g.clock_out = t_clock_probe + 4 * (size_t)(t_clock_next % t_clock_capacity);
+    ++t_clock_next;
+}
+
+extern "C" int odl_fp8_gemm_set_clock_probe(uint64_t *records_dev, int capacity) {
+    if (records_dev && capacity < 1) return set_error(ODL_ERR_ARG, "odl_fp8_gemm_set_clock_probe: capacity %d", capacity);
+    t_clock_probe = reinterpret_cast<unsigned long long *>(records_dev);
+    t_clock_capacity = records_dev ? capacity : 0;
+    t_clock_next = 0;
+    return ODL_OK;
 }
 
 extern "C" int odl_fp8_gemm_set_variant(int variant) {
@@ -195,7 +213,7 @@ extern "C" int odl_fp8_gemm_nt(const uint8_t *a, const uint8_t *b, int64_t M, in
     if (variant == 0) launch_gemm_generic(fmt_a, fmt_b, g, stream);
     else if (variant == kPipeVariant) launch_gemm_pipe(fmt_a, fmt_b, g, cu_count(), stream);
     else if (variant == kPipeOneTileVariant) launch_gemm_pipe(fmt_a, fmt_b, g, 1 << 30, stream);
-    else if (variant == kStreamVariant) launch_gemm_stream(fmt_a, fmt_b, g, cu_count(), stream);
+    else if (variant == kStreamVariant) { attach_clock_probe(g); launch_gemm_stream(fmt_a, fmt_b, g, cu_count(), stream); }
     else launch_gemm_tiled(variant, fmt_a, fmt_b, g, stream);
     return check_launch("odl_fp8_gemm_nt");
 }
@@ -224,6 +242,7 @@ extern "C" int odl_fp8_gemm_layouts(const uint8_t *a, const uint8_t *b, int64_t 
     if (!sizes_ok) return set_error(ODL_ERR_SHAPE, "odl_fp8_gemm_layouts: M, N, K must be multiples of 256 (K >= 512) and each operand under 2 GiB; got %lld x %lld x %lld", (long long)M, (long long)N, (long long)K);
     g.tiles_m = (int)(M / 256); g.tiles_n = (int)(N / 256);
     if (!gemm_stream_accepts(g)) return set_error(ODL_ERR_SHAPE, "odl_fp8_gemm_layouts: shape not taken by the streaming kernel");
+    attach_clock_probe(g);
     launch_gemm_stream(fmt_a, fmt_b, g, cu_count(), stream);
     return check_launch("odl_fp8_gemm_layouts");
 }
@@ -308,6 +327,7 @@ extern "C" int odl_fp8_gemm_splitk(const uint8_t *a, const uint8_t *b, int64_t M
     g.splits = splits; g.split_steps = (int)per;
     g.tiles_m = (int)((M + 255) / 256); g.tiles_n = (int)((N + 255) / 256);
     if (!gemm_stream_accepts(g)) return set_error(ODL_ERR_SHAPE, "odl_fp8_gemm_splitk: shape not taken by the streaming kernel");
+    attach_clock_probe(g);
     launch_gemm_stream(fmt_a, fmt_b, g, cu_count(), stream);
     const int64_t quads = M * N / 4;
     int64_t blocks = (quads + 255) / 256;

@@ -107,6 +107,11 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
     const int pid_end = min((xcd + 1) * per_xcd, total);
     int pid = xcd * per_xcd + (int)(blockIdx.x / 8);
     if (pid >= pid_end) return;
+    const bool stamps = g.clock_out != nullptr && blockIdx.x == 0 && threadIdx.x == 0;
+    if (stamps) {
+        g.clock_out[0] = clock64();
+        g.clock_out[1] = wall_clock64();
+    }
 
     // ---- per-tile addressing: the tile's origin lives in the buffer resources, the
     // per-lane offsets are the same for every tile and for both operands
@@ -479,6 +484,10 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
         rsrc_b = next_b;
         phase_a_fold(sA0, sB0, rsrc_c);
         if (!has_next) break;
+    }
+    if (stamps) {
+        g.clock_out[2] = clock64();
+        g.clock_out[3] = wall_clock64();
     }
 }
 

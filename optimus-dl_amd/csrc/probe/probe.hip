@@ -1,8 +1,5 @@
 // Measurement aids for bench.py: not part of the FP8 library's ABI (a library of their own, libodl_probe.so).
 //
-//   odl_probe_clock_stamp : one wave records {shader-clock counter, constant 100 MHz counter}.  Two stamps around a
-//                           stretch of work on the same stream give the average shader clock over that stretch:
-//                           (cycles1 - cycles0) / (ticks1 - ticks0) * 100 MHz.
 //   odl_probe_mfma_loop   : the FP8 MFMA of the GEMM kernels (32x32x64, 16 accumulator tiles per wave, one wave per
 //                           SIMD, nothing but registers) issued back to back, with operands that are all zero or
 //                           spread like quantised Gaussian data: the matrix pipe's rate with no memory system behind
@@ -13,13 +10,6 @@
 #include "../gemm_common.h"
 
 namespace {
-
-__global__ void clock_stamp_kernel(uint64_t *out) {
-    if (threadIdx.x == 0) {
-        out[0] = clock64();          // s_memtime: counts shader clocks
-        out[1] = wall_clock64();     // s_memrealtime: constant 100 MHz
-    }
-}
 
 __device__ __forceinline__ uint32_t mix(uint32_t x) {
     x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16;
@@ -78,11 +68,6 @@ __global__ __launch_bounds__(256) void mfma_loop_kernel(int random_operands, int
 }
 
 }  // namespace
-
-extern "C" int odl_probe_clock_stamp(uint64_t *out_dev, void *stream) {
-    hipLaunchKernelGGL(clock_stamp_kernel, dim3(1), dim3(64), 0, reinterpret_cast<hipStream_t>(stream), out_dev);
-    return (int)hipGetLastError();
-}
 
 // blocks x 4 waves x iters x 16 MFMAs of 2 * 32 * 32 * 64 flop.  cycles_dev: [blocks][2] = {shader clocks, 100 MHz ticks}
 // spent in the loop by each block's first wave.

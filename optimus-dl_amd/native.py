@@ -24,7 +24,7 @@ DT_BF16, DT_F32 = 0, 1
 AMAX_MAX, AMAX_MOST_RECENT = 0, 1
 FP8_MAX = {E4M3: 448.0, E5M2: 57344.0}
 TORCH_FP8 = {E4M3: torch.float8_e4m3fn, E5M2: torch.float8_e5m2}
-ABI_VERSION = 10
+ABI_VERSION = 11
 AMAX_PARTS = 512                       # ODL_FP8_AMAX_PARTS
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
@@ -67,6 +67,7 @@ EXPORTS = (
     "odl_fp8_gemm_num_variants",
     "odl_fp8_gemm_variant_name",
     "odl_fp8_gemm_set_variant",
+    "odl_fp8_gemm_set_clock_probe",
 )
 
 _lib = None
@@ -135,6 +136,7 @@ def load() -> ctypes.CDLL:
         L.odl_fp8_gemm_variant_name.argtypes = [i32]
         L.odl_fp8_gemm_variant_name.restype = ctypes.c_char_p
         L.odl_fp8_gemm_set_variant.argtypes = [i32]
+        L.odl_fp8_gemm_set_clock_probe.argtypes = [vp, i32]
         for name in EXPORTS:
             getattr(L, name)  # AttributeError here = the library does not match the header
         if L.odl_fp8_abi_version() != ABI_VERSION:
@@ -839,3 +841,15 @@ def gemm_set_variant(variant: int) -> None:
     thread launches in a backward pass keep the automatic choice."""
     _check(load().odl_fp8_gemm_set_variant(variant), "odl_fp8_gemm_set_variant")
     _tls.forced_variant = variant
+
+
+def gemm_set_clock_probe(records: torch.Tensor | None) -> None:
+    """Measurement aid: the streaming GEMM launches that THIS host thread makes from now on record, in turn, into the
+    rows of ``records`` (int64 [capacity, 4] on the GPU: shader-clock counter and 100 MHz counter on entry and exit of
+    the kernel's first wave).  None switches it off."""
+    if records is None:
+        _check(load().odl_fp8_gemm_set_clock_probe(None, 0), "odl_fp8_gemm_set_clock_probe")
+        return
+    if not (records.is_cuda and records.dtype == torch.int64 and records.dim() == 2 and records.shape[1] == 4 and records.is_contiguous()):
+        raise NativeError("gemm_set_clock_probe: records must be a contiguous int64 CUDA tensor of shape [capacity, 4]")
+    _check(load().odl_fp8_gemm_set_clock_probe(records.data_ptr(), records.shape[0]), "odl_fp8_gemm_set_clock_probe")
