@@ -236,6 +236,68 @@ ORACLE_API void oracle_gemm_nt(const uint8_t *a, const uint8_t *b, int64_t M, in
 }
 
 /*
+ * MXFP8 (recipe "mxfp8", optimus_dl/modules/amp/fp8.py:301-306 -> the third-party library's MXFP8BlockScaling): blocks of 32
+ * consecutive elements along the contraction axis share a power-of-two scale, stored as one E8M0 byte (value 2^(byte - 127)).
+ * The conversion follows the OCP Microscaling Formats (MX) specification v1.0, section 6.3:
+ *   shared_exp = floor(log2(max |v|)) - emax_elem      (emax_elem: 8 for E4M3, 15 for E5M2), clamped to [-127, 127]
+ *   scale byte = shared_exp + 127; a block of zeros gets byte 0; a block holding a NaN or an infinity gets 0xFF
+ *   element    = rne( clamp( v * 2^-shared_exp, +-fp8_max ) )    (saturating, as every cast of this library)
+ * The third-party library rounds the shared exponent its own way (towards larger scales, so that nothing saturates);
+ * that choice cannot be checked offline: parity unpinned against it, pinned against the specification's formula.
+ */
+static inline int emax_elem(int fmt) { return fmt == FMT_E5M2 ? 15 : 8; }
+
+ORACLE_API void oracle_mx_quantise_bf16(const uint16_t *x, int64_t rows, int64_t cols, int fmt, uint8_t *codes, uint8_t *scales) {
+    const int64_t nb = cols / 32;
+    for (int64_t r = 0; r < rows; ++r)
+        for (int64_t b = 0; b < nb; ++b) {
+            const uint16_t *v = x + r * cols + b * 32;
+            uint32_t mag = 0;
+            for (int i = 0; i < 32; ++i) { uint32_t m = (uint32_t)(v[i] & 0x7fffu) << 16; if (m > mag) mag = m; }
+            uint8_t sb;
+            float mul;
+            if (mag >= 0x7f800000u) { sb = 0xff; mul = 1.0f; }                 /* Inf / NaN in the block */
+            else if (mag == 0) { sb = 0; mul = 1.0f; }
+            else {
+                int e;                                                            /* floor(log2(amax)), subnormals included */
+                (void)frexpf(bits_f32(mag), &e);
+                int se = (e - 1) - emax_elem(fmt);
+                if (se < -127) se = -127;
+                if (se > 127) se = 127;
+                sb = (uint8_t)(se + 127);
+                mul = ldexpf(1.0f, -se);                                          /* 2^-se: exact, at most 2^127 */
+            }
+            scales[r * nb + b] = sb;
+            for (int i = 0; i < 32; ++i) codes[r * cols + b * 32 + i] = quantise(v[i], mul, fmt);
+        }
+}
+
+/* C[M,N] = sum over 32-blocks kb of 2^(sa[m,kb] - 127 + sb[n,kb] - 127) * dot(A[m, kb], B[n, kb]); fp32 accumulation, block dots
+ * added in ascending kb; a scale byte 0xFF makes the result NaN.  bias (fp32, may be NULL) is added before the rounding. */
+ORACLE_API void oracle_mx_gemm_nt(const uint8_t *a, const uint8_t *sa, const uint8_t *b, const uint8_t *sb, int64_t M, int64_t N,
+                                  int64_t K, int fmt_a, int fmt_b, const float *bias, uint16_t *c_bf16, float *c_f32) {
+    float lut_a[256], lut_b[256];
+    for (int i = 0; i < 256; ++i) { lut_a[i] = decode((uint8_t)i, fmt_a); lut_b[i] = decode((uint8_t)i, fmt_b); }
+    const int64_t nb = K / 32;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < M; ++i)
+        for (int64_t j = 0; j < N; ++j) {
+            float acc = 0.0f;
+            for (int64_t kb = 0; kb < nb; ++kb) {
+                float dot = 0.0f;
+                for (int k = 0; k < 32; ++k) dot += lut_a[a[i * K + kb * 32 + k]] * lut_b[b[j * K + kb * 32 + k]];
+                const uint8_t ea = sa[i * nb + kb], eb = sb[j * nb + kb];
+                if (ea == 0xff || eb == 0xff) { acc = NAN; continue; }
+                volatile float term = ldexpf(dot, (int)ea + (int)eb - 254);
+                acc += term;
+            }
+            volatile float v = bias ? acc + bias[j] : acc;
+            if (c_f32) c_f32[i * N + j] = v;
+            if (c_bf16) c_bf16[i * N + j] = f32_to_bf16(v);
+        }
+}
+
+/*
  * Delayed-scaling bookkeeping for R roles with a history of H steps each,
  * history stored [H, R] row-major with row 0 = the newest amax (written by the
  * cast kernels of the step that just ran).

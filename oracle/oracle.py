@@ -65,6 +65,8 @@ def lib() -> ctypes.CDLL:
         L.oracle_cast_transpose_bf16.argtypes = [vp, i64, i64, vp, i32, i32, vp, vp]
         L.oracle_gemm_nt.argtypes = [vp, vp, i64, i64, i64, i32, i32, vp, i64, vp, i64, vp, vp]
         L.oracle_delayed_update.argtypes = [vp, i64, i64, vp, vp, vp, i32, i32]
+        L.oracle_mx_quantise_bf16.argtypes = [vp, i64, i64, i32, vp, vp]
+        L.oracle_mx_gemm_nt.argtypes = [vp, vp, vp, vp, i64, i64, i64, i32, i32, vp, vp, vp]
         L.oracle_sigmoid.argtypes = [f32]
         L.oracle_sigmoid.restype = f32
         L.oracle_swiglu_fwd.argtypes = [vp, vp, i64, vp]
@@ -397,3 +399,62 @@ class DelayedState:
                     s = np.float32(FLT_MAX)
                 self.scale[r] = s
             self.scale_inv[r] = np.float32(1.0) / self.scale[r]
+
+
+# ------------------------------------------------------------------------ MXFP8
+MX_BLOCK = 32
+MX_EMAX = {E4M3: 8, E5M2: 15}
+
+
+def c_mx_quantise(x: torch.Tensor, fmt: int):
+    """MXFP8 of a bf16 matrix, blocks of 32 along the last axis -> (codes uint8 [R, C], scale bytes uint8 [R, C/32])."""
+    rows, cols = x.shape
+    assert cols % MX_BLOCK == 0
+    xb = _bf16_bits(x)
+    codes, scales = np.empty((rows, cols), dtype=np.uint8), np.empty((rows, cols // MX_BLOCK), dtype=np.uint8)
+    lib().oracle_mx_quantise_bf16(_p(xb), rows, cols, fmt, _p(codes), _p(scales))
+    return torch.from_numpy(codes), torch.from_numpy(scales)
+
+
+def t_mx_quantise(x: torch.Tensor, fmt: int):
+    """The same conversion with torch routines (frexp for floor(log2), exact power-of-two scaling, the CPU float8 cast)."""
+    rows, cols = x.shape
+    v = x.float().reshape(rows, cols // MX_BLOCK, MX_BLOCK)
+    amax = v.abs().amax(dim=2)
+    _, e = torch.frexp(amax)                                   # amax = m * 2^e with 0.5 <= m < 1: floor(log2) = e - 1
+    se = (e - 1 - MX_EMAX[fmt]).clamp(-127, 127)
+    bad = ~torch.isfinite(amax)
+    se = torch.where((amax == 0) | bad, torch.full_like(se, -127), se)
+    scaled = torch.ldexp(v, (-se).unsqueeze(2).expand_as(v).to(torch.int32))
+    scaled = torch.where(bad.unsqueeze(2), v, scaled)          # such a block keeps its values (scale byte 0xFF)
+    m = FP8_MAX[fmt]
+    codes = scaled.clamp(-m, m).to(TORCH_FP8[fmt]).view(torch.uint8).reshape(rows, cols)
+    scales = torch.where(bad, torch.full_like(se, 255), se + 127).to(torch.uint8)
+    return codes, scales
+
+
+def t_mx_dequantise(codes: torch.Tensor, scales: torch.Tensor, fmt: int) -> torch.Tensor:
+    rows, cols = codes.shape
+    v = t_decode(codes, fmt).reshape(rows, cols // MX_BLOCK, MX_BLOCK)
+    out = torch.ldexp(v, (scales.to(torch.int32) - 127).unsqueeze(2).expand_as(v))
+    out = torch.where((scales == 255).unsqueeze(2), torch.full_like(out, float("nan")), out)
+    return out.reshape(rows, cols)
+
+
+def t_mx_gemm_nt(a, sa, b, sb, fmt_a, fmt_b, bias=None, want_f32: bool = False):
+    """Emulated MXFP8 matmul: dequantise both operands (exact in fp32), fp32 matmul, optional bias, bf16."""
+    out = t_mx_dequantise(a, sa, fmt_a) @ t_mx_dequantise(b, sb, fmt_b).t()
+    if bias is not None:
+        out = out + bias.float()
+    return (out.bfloat16(), out) if want_f32 else out.bfloat16()
+
+
+def c_mx_gemm_nt(a, sa, b, sb, fmt_a, fmt_b, bias=None):
+    M, K = a.shape
+    N = b.shape[0]
+    arrs = [np.ascontiguousarray(t.numpy()) for t in (a, sa, b, sb)]
+    out_bf16, out_f32 = np.empty((M, N), dtype=np.uint16), np.empty((M, N), dtype=np.float32)
+    bias_np = None if bias is None else np.ascontiguousarray(bias.float().numpy())
+    lib().oracle_mx_gemm_nt(_p(arrs[0]), _p(arrs[1]), _p(arrs[2]), _p(arrs[3]), M, N, K, fmt_a, fmt_b,
+                            _p(bias_np) if bias_np is not None else None, _p(out_bf16), _p(out_f32))
+    return torch.from_numpy(out_bf16.view(np.int16)).view(torch.bfloat16), torch.from_numpy(out_f32)
