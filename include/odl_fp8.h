@@ -45,7 +45,7 @@ enum odl_status {
     ODL_ERR_LAUNCH = 3    /* HIP reported an error at launch */
 };
 
-/* ABI version of this header (11); bumped when a signature changes or an entry point is added. */
+/* ABI version of this header (12); bumped when a signature changes or an entry point is added. */
 int odl_fp8_abi_version(void);
 
 /* Last error message of the calling host thread ("" if none). */
@@ -413,6 +413,32 @@ int odl_fp8_gemm_num_variants(void);
 int odl_fp8_gemm_set_clock_probe(uint64_t *records_dev, int capacity);
 const char *odl_fp8_gemm_variant_name(int variant);
 int odl_fp8_gemm_set_variant(int variant);
+
+/* ---------------------------------------------------------------------------------------------------------------
+ * MXFP8: blocks of 32 consecutive elements along the contraction axis share one power-of-two scale, stored as an
+ * E8M0 byte (value 2^(byte - 127); 0xFF = NaN).  Replaces, for the recipe string "mxfp8", what the reference hands to
+ * its backend as MXFP8BlockScaling (optimus_dl/modules/amp/fp8.py:301-306) around the same Linear
+ * (optimus_dl/modules/model/blocks/layers/linear.py:55-86).  The conversion rule is the one of the OCP Microscaling
+ * Formats specification v1.0, section 6.3: shared exponent = floor(log2(block amax)) - emax_elem (8 for E4M3, 15 for
+ * E5M2), clamped to [-127, 127]; elements = rne(clamp(v / 2^shared, +-fp8_max)); a block of zeros gets byte 0, a block
+ * that holds Inf or NaN gets 0xFF.  There is no amax pass and no scale state: one kernel reads x once.
+ *
+ *   out    [rows, cols]      codes, blocks along the columns;  scales   [rows, cols / 32]   (cols % 32 == 0)
+ *   out_t  [cols, rows]      codes of x^T, blocks along the rows of x;  scales_t [cols, rows / 32]   (rows % 32 == 0)
+ * Either pair may be NULL (both members together).  cols % 8 == 0, x and out_t 16-byte aligned, out 8-byte aligned.
+ */
+int odl_fp8_mx_cast(const void *x, int src_dtype, int64_t rows, int64_t cols, int fmt, uint8_t *out, uint8_t *scales,
+                    uint8_t *out_t, uint8_t *scales_t, odl_stream_t stream);
+
+/*
+ * C[M, N] = sum over blocks kb of 2^(sa[m, kb] - 127) * 2^(sb[n, kb] - 127) * dot(A[m, 32 kb .. +32], B[n, 32 kb .. +32])
+ * (+ bias[n]), accumulated in fp32 by the scaled MFMA (V_MFMA_SCALE_F32_32X32X64_F8F6F4 applies the two block scales to
+ * the products), one rounding to out_dtype.  a [M, K], b [N, K] codes; sa [M, K / 32], sb [N, K / 32] scale bytes;
+ * K % 32 == 0; a, b, c and bias 16-byte aligned.  K % 128 == 0 with 4-byte aligned scale arrays runs the LDS-tiled
+ * kernel; other shapes a plain one-wave-per-tile kernel.
+ */
+int odl_fp8_mx_gemm_nt(const uint8_t *a, const uint8_t *sa, const uint8_t *b, const uint8_t *sb, int64_t M, int64_t N, int64_t K,
+                       int fmt_a, int fmt_b, const float *bias, void *c, int out_dtype, odl_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -18,7 +18,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_NAME = "libodl_fp8.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
-SOURCES = ["api.hip", "quant.hip", "gemm_fp8.hip", "gemm_tiled.hip", "gemm_pipe.hip", "gemm_stream.hip", "fused.hip"]
+SOURCES = ["api.hip", "quant.hip", "gemm_fp8.hip", "gemm_tiled.hip", "gemm_pipe.hip", "gemm_stream.hip", "fused.hip", "mx.hip"]
 
 # -ffp-contract=off : the epilogues promise "multiply, round, add, round" (no FMA fusion)
 # packed-fp32-ops off: never let the compiler form v_pk_*_f32 from scalar float code

@@ -31,8 +31,10 @@ struct GemmArgs {
 
 __device__ __forceinline__ int swz(int row) { return (row ^ (row >> 3)) & 7; }
 
-// D[i][j] += sum_k first[i][k] * second[j][k]; lane l supplies row l%32 and the
-// K-bytes [32*(l/32), +32) of both operands.  F1 / F2: 0 = E4M3, 1 = E5M2.
+// D[i][j] += sum_k first[i][k] * second[j][k]; lane l supplies row l%32 and 32 K-bytes
+// of both operands (which 32 does not matter as long as both operands use the same ones;
+// the instruction itself takes registers 0..3 as K [16 g, +16) and 4..7 as K [32 + 16 g, +16),
+// g = l/32, which only the block-scaled kernels in mx.hip depend on).  F1 / F2: 0 = E4M3, 1 = E5M2.
 template <int F1, int F2>
 __device__ __forceinline__ v16f mfma_32x32x64(v8i first, v8i second, v16f acc) {
     return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(first, second, acc, F1, F2, 0, 0, 0, 0);

@@ -1,0 +1,443 @@
+// MXFP8 on gfx950: blocks of 32 consecutive elements along the contraction axis share a power-of-two scale (one
+// E8M0 byte, value 2^(byte - 127)), and the MFMA applies the scales itself (V_MFMA_SCALE_F32_32X32X64_F8F6F4: a lane
+// feeds 32 K-bytes of one row, which is exactly one block, together with that block's scale byte).
+//
+//   odl_fp8_mx_cast    : x [rows, cols] -> codes + scale bytes with the blocks along the columns (`out`, `scales`)
+//                        and / or, transposed, with the blocks along the rows (`out_t`, `scales_t`); one pass over x,
+//                        no amax pass before it: the scale of a block is found inside the tile.
+//   odl_fp8_mx_gemm_nt : C[M, N] = sum over blocks kb of 2^(sa[m, kb] + sb[n, kb] - 254) * dot(A[m, kb], B[n, kb])
+//
+// Operand layout of the instruction, measured (one nonzero byte at a time against two different block scales): of the
+// 8 registers a lane supplies for row (lane % 32), registers 0..3 are the 16 K-bytes [16 g, 16 g + 16) and registers
+// 4..7 the 16 K-bytes [32 + 16 g, 32 + 16 g + 16), g = lane / 32; the products of registers 0..3 of ALL lanes (K 0..31)
+// take the scale byte supplied by lanes 0..31, those of registers 4..7 (K 32..63) the byte supplied by lanes 32..63.
+//
+// Conversion rule (OCP Microscaling Formats v1.0, 6.3): shared exponent = floor(log2(block amax)) - emax of the element
+// format (8 for E4M3, 15 for E5M2), clamped to [-127, 127]; elements = rne(clamp(v * 2^-shared, +-fp8_max)).  A block of
+// zeros gets byte 0, a block holding Inf / NaN gets 0xFF (a NaN scale: the products it enters are NaN).
+#include <hip/hip_runtime.h>
+
+#include "common.h"
+#include "ct_tile.h"
+#include "gemm_common.h"
+
+namespace odl {
+
+constexpr int kMxBlock = 32;
+constexpr int kMxThreads = 256;
+
+template <int FMT> struct MxEmax { static constexpr int value = FMT == ODL_FP8_E5M2 ? 15 : 8; };
+
+// magnitude bits (fp32 layout) of a block's amax -> scale byte and the multiplier 2^-shared
+template <int FMT>
+__device__ __forceinline__ void mx_scale_of(uint32_t amax_bits, uint32_t &byte, float &mul) {
+    if (amax_bits >= 0x7f800000u) { byte = 0xffu; mul = 1.0f; return; }     // Inf / NaN in the block
+    if (amax_bits == 0) { byte = 0u; mul = 1.0f; return; }
+    // floor(log2): the exponent field, or for a subnormal (only bf16 / fp32 subnormal inputs) the position of its top bit
+    int e = (int)(amax_bits >> 23) - 127;
+    if ((amax_bits >> 23) == 0) e = -127 - (__builtin_clz(amax_bits) - 9);   // mantissa bit 22 is 2^-127
+    int se = e - MxEmax<FMT>::value;
+    se = se < -127 ? -127 : se;                                            // (the upper clamp cannot be reached: e <= 127)
+    byte = (uint32_t)(se + 127);
+    mul = bits_to_float((uint32_t)(127 - se) << 23);                       // 2^-se, 127 - se in [8, 254]
+}
+
+// 128 x 64 tile per block of 256 lanes, lane (tx, ty) owns rows 4 ty .. 4 ty + 3 and columns 8 tx .. 8 tx + 7 as in
+// cast_transpose_kernel.  A block along the columns (32 of them) is held by 4 neighbouring lanes; a block along the rows
+// (32 of them) by the 8 lanes of a wave that share tx: both maxima are xor-shuffles inside the wave.
+template <int SRC, int FMT, bool WANT_ROW, bool WANT_COL>
+__global__ __launch_bounds__(kMxThreads) void mx_cast_kernel(const void *__restrict__ x, int64_t rows, int64_t cols,
+                                                              uint8_t *__restrict__ out, uint8_t *__restrict__ scales,
+                                                              uint8_t *__restrict__ out_t, uint8_t *__restrict__ scales_t) {
+    __shared__ __attribute__((aligned(16))) uint8_t tile[kTileC * kTileR];
+    constexpr int ESZ = SRC == ODL_BF16 ? 2 : 4;
+    const int tx = threadIdx.x % 8, ty = threadIdx.x / 8;
+    const int64_t tiles_r = (rows + kTileR - 1) / kTileR, tiles_c = (cols + kTileC - 1) / kTileC;
+    int64_t tr, tc;
+    ct_tile_of(blockIdx.x, tiles_r, tiles_c, tr, tc);
+    const int64_t r0 = tr * kTileR + ty * 4, c0 = tc * kTileC + tx * 8;
+    const bool col_ok = c0 < cols;                 // cols % 8 == 0 (host-checked)
+
+    float f[4][8];
+    uint32_t mag[4][8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const bool ok = col_ok && (r0 + i) < rows;
+        const u32x4 *p = reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(x) + ((r0 + i) * cols + c0) * ESZ);
+        u32x4 raw[ESZ / 2];
+#pragma unroll
+        for (int h = 0; h < ESZ / 2; ++h) raw[h] = ok ? __builtin_nontemporal_load(p + h) : u32x4{0, 0, 0, 0};
+        if constexpr (SRC == ODL_BF16) {
+            const uint32_t w[4] = {raw[0].x, raw[0].y, raw[0].z, raw[0].w};
+#pragma unroll
+            for (int q = 0; q < 4; ++q) { f[i][2 * q] = bf16_lo(w[q]); f[i][2 * q + 1] = bf16_hi(w[q]); }
+        } else {
+            const uint32_t w[8] = {raw[0].x, raw[0].y, raw[0].z, raw[0].w, raw[1].x, raw[1].y, raw[1].z, raw[1].w};
+#pragma unroll
+            for (int q = 0; q < 8; ++q) f[i][q] = bits_to_float(w[q]);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) mag[i][j] = float_to_bits(f[i][j]) & 0x7fffffffu;
+    }
+
+    if constexpr (WANT_ROW) {
+        const int64_t nb = cols / kMxBlock;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            uint32_t m = 0;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) m = max(m, mag[i][j]);
+            m = max(m, (uint32_t)__shfl_xor((int)m, 1, kWave));
+            m = max(m, (uint32_t)__shfl_xor((int)m, 2, kWave));          // the 4 lanes tx = 4 b .. 4 b + 3 hold the block
+            uint32_t byte;
+            float mul;
+            mx_scale_of<FMT>(m, byte, mul);
+            if (col_ok && (r0 + i) < rows) {
+                const uint32_t lo = quantise4<FMT>(f[i][0], f[i][1], f[i][2], f[i][3], mul, mul, mul, mul);
+                const uint32_t hi = quantise4<FMT>(f[i][4], f[i][5], f[i][6], f[i][7], mul, mul, mul, mul);
+                *reinterpret_cast<u32x2 *>(out + (r0 + i) * cols + c0) = u32x2{lo, hi};
+                if ((tx & 3) == 0) scales[(r0 + i) * nb + c0 / kMxBlock] = (uint8_t)byte;
+            }
+        }
+    }
+
+    if constexpr (WANT_COL) {
+        const int64_t nbt = rows / kMxBlock;
+        uint32_t lo[4] = {0, 0, 0, 0}, hi[4] = {0, 0, 0, 0};
+        float mul_c[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            uint32_t m = max(max(mag[0][j], mag[1][j]), max(mag[2][j], mag[3][j]));
+            m = max(m, (uint32_t)__shfl_xor((int)m, 8, kWave));
+            m = max(m, (uint32_t)__shfl_xor((int)m, 16, kWave));
+            m = max(m, (uint32_t)__shfl_xor((int)m, 32, kWave));         // the 8 lanes of the wave with this tx: 32 rows
+            uint32_t byte;
+            mx_scale_of<FMT>(m, byte, mul_c[j]);
+            // rows % 32 == 0 (host-checked): a row block is inside the matrix as a whole or not at all
+            if ((ty & 7) == 0 && col_ok && r0 < rows) scales_t[(c0 + j) * nbt + r0 / kMxBlock] = (uint8_t)byte;
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            lo[i] = quantise4<FMT>(f[i][0], f[i][1], f[i][2], f[i][3], mul_c[0], mul_c[1], mul_c[2], mul_c[3]);
+            hi[i] = quantise4<FMT>(f[i][4], f[i][5], f[i][6], f[i][7], mul_c[4], mul_c[5], mul_c[6], mul_c[7]);
+        }
+        uint32_t tl[4], th[4];
+        transpose4x4(lo, tl);
+        transpose4x4(hi, th);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            *reinterpret_cast<uint32_t *>(&tile[ct_lds_write_off(tx * 8 + k, ty)]) = tl[k];
+            *reinterpret_cast<uint32_t *>(&tile[ct_lds_write_off(tx * 8 + 4 + k, ty)]) = th[k];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+            const int chunk = threadIdx.x + it * kMxThreads;
+            const int k = chunk / 8, m16 = chunk % 8;
+            const int64_t oc = tc * kTileC + k, orow = tr * kTileR + m16 * 16;
+            if (oc < cols && orow < rows)
+                __builtin_nontemporal_store(ct_lds_read(tile, k, m16), reinterpret_cast<u32x4 *>(out_t + oc * rows + orow));
+        }
+    }
+}
+
+// ------------------------------------------------------------------ GEMM, tiled
+// The structure of gemm_nt_tiled_kernel (two LDS stages of BM + BN rows x 128 bytes, direct-to-LDS loads, swizzled
+// 16-byte chunks, MFMA operands swapped so that a lane ends up with 4 consecutive output columns) plus the scale
+// bytes: per K step of 128 bytes a row has 4 of them (one dword); thread i of the block fetches the dword of
+// A row i and of B row i for the NEXT step together with that step's operand loads and parks it in LDS after the
+// barrier; a lane reads the dword of each of its rows and shifts it right by 8 bits when it sits in the upper half of the
+// wave, so that byte 0 / byte 2 are the scales it supplies in the first / second MFMA of the step (lanes 0..31: blocks 0
+// and 2 of the step, lanes 32..63: blocks 1 and 3).
+template <int BM, int BN, int WAVES_M, int WAVES_N, int FA, int FB>
+__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mx_gemm_tiled_kernel(const GemmArgs g, const uint8_t *__restrict__ sa,
+                                                                              const uint8_t *__restrict__ sb) {
+    constexpr int NW = WAVES_M * WAVES_N, NT = NW * 64;
+    constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, TM = WM / 32, TN = WN / 32;
+    constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128, STAGE = A_BYTES + B_BYTES;
+    constexpr int LA = BM / 8 / NW, LB = BN / 8 / NW;
+    constexpr int GM = 8;
+    static_assert(BM <= NT && BN <= NT, "one scale dword per thread and operand");
+
+    __shared__ __attribute__((aligned(1024))) uint8_t lds0[STAGE];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds1[STAGE];
+    __shared__ uint32_t sc0[BM + BN], sc1[BM + BN];
+
+    const int total = g.tiles_m * g.tiles_n;
+    const int per_xcd = (total + 7) / 8;
+    const int pid = (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8);
+    if (pid >= total) return;
+    const int in_group = GM * g.tiles_n;
+    const int first_m = (pid / in_group) * GM;
+    const int group_rows = min(g.tiles_m - first_m, GM);
+    const int tile_m = first_m + (pid % in_group) % group_rows;
+    const int tile_n = (pid % in_group) / group_rows;
+    const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
+
+    const int lane = threadIdx.x % 64;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
+    const int wm0 = (wave / WAVES_N) * WM, wn0 = (wave % WAVES_N) * WN;
+    const int KT = (int)(g.K / 128);
+    const int64_t nb = g.K / kMxBlock;
+
+    uint32_t off_a[LA], off_b[LB];
+#pragma unroll
+    for (int j = 0; j < LA; ++j) {
+        const int row = (wave + j * NW) * 8 + lane / 8;
+        const int64_t gr = min(m0 + row, g.M - 1);
+        off_a[j] = (uint32_t)(gr * g.K + (((lane % 8) ^ swz(row)) << 4));
+    }
+#pragma unroll
+    for (int j = 0; j < LB; ++j) {
+        const int row = (wave + j * NW) * 8 + lane / 8;
+        const int64_t gr = min(n0 + row, g.N - 1);
+        off_b[j] = (uint32_t)(gr * g.K + (((lane % 8) ^ swz(row)) << 4));
+    }
+    // the scale dwords this thread fetches: A row threadIdx.x, B row threadIdx.x (rows past the edge re-read the last row)
+    const uint32_t *sa_row = reinterpret_cast<const uint32_t *>(sa + min(m0 + (int64_t)threadIdx.x, g.M - 1) * nb);
+    const uint32_t *sb_row = reinterpret_cast<const uint32_t *>(sb + min(n0 + (int64_t)threadIdx.x, g.N - 1) * nb);
+    uint32_t ra = 0, rb = 0;
+    auto issue = [&](uint8_t *lds, int kt) {
+        const uint8_t *ga = g.a + (int64_t)kt * 128, *gb = g.b + (int64_t)kt * 128;
+#pragma unroll
+        for (int j = 0; j < LA; ++j)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(ga + off_a[j]),
+                                             (__attribute__((address_space(3))) void *)(lds + (wave + j * NW) * 1024), 16, 0, 0);
+#pragma unroll
+        for (int j = 0; j < LB; ++j)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(gb + off_b[j]),
+                                             (__attribute__((address_space(3))) void *)(lds + A_BYTES + (wave + j * NW) * 1024), 16, 0, 0);
+        if ((int)threadIdx.x < BM) ra = sa_row[kt];
+        if ((int)threadIdx.x < BN) rb = sb_row[kt];
+    };
+    auto park = [&](uint32_t *sc) {                // after vmcnt(0): this thread's two dwords into the stage's scale slots
+        if ((int)threadIdx.x < BM) sc[threadIdx.x] = ra;
+        if ((int)threadIdx.x < BN) sc[BM + threadIdx.x] = rb;
+    };
+
+    const int lr = lane % 32, lg = lane / 32;
+    int a_off[TM], a_sw[TM], b_off[TN], b_sw[TN];
+#pragma unroll
+    for (int t = 0; t < TM; ++t) { const int row = wm0 + 32 * t + lr; a_off[t] = row * 128; a_sw[t] = swz(row); }
+#pragma unroll
+    for (int u = 0; u < TN; ++u) { const int row = wn0 + 32 * u + lr; b_off[u] = A_BYTES + row * 128; b_sw[u] = swz(row); }
+
+    v16f acc[TM][TN];
+#pragma unroll
+    for (int t = 0; t < TM; ++t)
+#pragma unroll
+        for (int u = 0; u < TN; ++u)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[t][u][e] = 0.0f;
+
+    auto compute = [&](const uint8_t *lds, const uint32_t *sc) {
+        int esa[TM], esb[TN];                       // this lane's scale bytes: byte 0 for the first K half, byte 2 for the second
+#pragma unroll
+        for (int t = 0; t < TM; ++t) esa[t] = (int)(sc[wm0 + 32 * t + lr] >> (8 * lg));
+#pragma unroll
+        for (int u = 0; u < TN; ++u) esb[u] = (int)(sc[BM + wn0 + 32 * u + lr] >> (8 * lg));
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int c = 4 * h + lg;               // 16-byte chunks c (first block) and c + 2 (second block) of the row
+            v8i af[TM], bf[TN];
+#pragma unroll
+            for (int t = 0; t < TM; ++t) {
+                const uint8_t *p = lds + a_off[t];
+                const v4i lo = *reinterpret_cast<const v4i *>(p + ((c ^ a_sw[t]) << 4));
+                const v4i hi = *reinterpret_cast<const v4i *>(p + (((c + 2) ^ a_sw[t]) << 4));
+                af[t] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+            }
+#pragma unroll
+            for (int u = 0; u < TN; ++u) {
+                const uint8_t *p = lds + b_off[u];
+                const v4i lo = *reinterpret_cast<const v4i *>(p + ((c ^ b_sw[u]) << 4));
+                const v4i hi = *reinterpret_cast<const v4i *>(p + (((c + 2) ^ b_sw[u]) << 4));
+                bf[u] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+            }
+#pragma unroll
+            for (int t = 0; t < TM; ++t)
+#pragma unroll
+                for (int u = 0; u < TN; ++u) {
+                    if (h == 0) acc[t][u] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[u], af[t], acc[t][u], FB, FA, 0, esb[u], 0, esa[t]);
+                    else acc[t][u] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[u], af[t], acc[t][u], FB, FA, 2, esb[u], 2, esa[t]);
+                }
+        }
+    };
+
+    issue(lds0, 0);
+    for (int kt = 0; kt < KT; kt += 2) {
+        __builtin_amdgcn_s_waitcnt(0x0F70);                     // vmcnt(0): my loads into lds0 and my scale dwords have landed
+        park(sc0);
+        __syncthreads();
+        if (kt + 1 < KT) issue(lds1, kt + 1);
+        compute(lds0, sc0);
+        if (kt + 1 < KT) {
+            __builtin_amdgcn_s_waitcnt(0x0F70);
+            park(sc1);
+            __syncthreads();
+            if (kt + 2 < KT) issue(lds0, kt + 2);
+            compute(lds1, sc1);
+        }
+    }
+
+    const bool interior = m0 + BM <= g.M && n0 + BN <= g.N;
+    constexpr int EPI_BYTES = 32 * (TN * 32 * 4 + 16);
+    static_assert(NW * EPI_BYTES <= 2 * STAGE, "epilogue staging must fit in the operand stages");
+    if (interior && (g.N % 8) == 0) {
+        __syncthreads();
+        uint8_t *wave_lds = (wave * EPI_BYTES + EPI_BYTES <= STAGE) ? lds0 + wave * EPI_BYTES
+                                                                    : lds1 + (wave - STAGE / EPI_BYTES) * EPI_BYTES;
+        if (g.out_dtype == ODL_BF16) epilogue_staged<true, TM, TN, TN>(g, acc, wave_lds, m0 + wm0, n0 + wn0, lane);
+        else epilogue_staged<false, TM, TN, TN>(g, acc, wave_lds, m0 + wm0, n0 + wn0, lane);
+    } else {
+#define ODL_EPILOGUE(BF)                                                                                       \
+    _Pragma("unroll") for (int t = 0; t < TM; ++t) _Pragma("unroll") for (int u = 0; u < TN; ++u)              \
+        store_tile<BF, false>(g, acc[t][u], m0 + wm0 + 32 * t + lr, n0 + wn0 + 32 * u + 4 * lg)
+        if (g.out_dtype == ODL_BF16) { ODL_EPILOGUE(true); } else { ODL_EPILOGUE(false); }
+#undef ODL_EPILOGUE
+    }
+}
+
+// ------------------------------------------------------------------ GEMM, any shape with K % 32 == 0
+// One wave per 32 x 32 output tile, operands and scale bytes straight from global memory, 64 K-bytes per trip; a last
+// half trip (K % 64 == 32) feeds zeros as the second block.
+template <int FA, int FB>
+__global__ __launch_bounds__(64) void mx_gemm_generic_kernel(const GemmArgs g, const uint8_t *__restrict__ sa, const uint8_t *__restrict__ sb) {
+    const int lane = threadIdx.x, lr = lane % 32, lg = lane / 32;
+    const int64_t m0 = (int64_t)blockIdx.y * 32, n0 = (int64_t)blockIdx.x * 32;
+    const int64_t ra = min(m0 + lr, g.M - 1), rb = min(n0 + lr, g.N - 1), nb = g.K / kMxBlock;
+    v16f acc;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[e] = 0.0f;
+    for (int64_t k = 0; k < g.K; k += 64) {
+        const bool second = k + 32 < g.K;                           // false in the half trip at the end
+        const v4i zero = {0, 0, 0, 0};
+        const v4i *pa = reinterpret_cast<const v4i *>(g.a + ra * g.K + k + 16 * lg), *pb = reinterpret_cast<const v4i *>(g.b + rb * g.K + k + 16 * lg);
+        const v4i a0 = pa[0], b0 = pb[0], a1 = second ? pa[2] : zero, b1 = second ? pb[2] : zero;
+        const v8i af = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w}, bf = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+        int ea = 127, eb = 127;                                     // lanes 0..31: scale of block k / 32, lanes 32..63: of the next
+        if (lg == 0 || second) { ea = sa[ra * nb + k / kMxBlock + lg]; eb = sb[rb * nb + k / kMxBlock + lg]; }
+        acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf, af, acc, FB, FA, 0, eb, 0, ea);
+    }
+    if (g.out_dtype == ODL_BF16) store_tile<true, false>(g, acc, m0 + lr, n0 + 4 * lg);
+    else store_tile<false, false>(g, acc, m0 + lr, n0 + 4 * lg);
+}
+
+}  // namespace odl
+
+// The epilogues multiply by *g.sa * *g.sb: a 1.0f that is part of the library's device image (one copy per GPU; the name is
+// only a handle for hipGetSymbolAddress, the address the kernels take is looked up once per device).
+static __device__ float mx_unit_scale = 1.0f;
+
+namespace odl {
+
+static const float *unit_scale_for_current_device(const char *who) {
+    constexpr int kMaxDevices = 64;
+    static const float *cached[kMaxDevices] = {};
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) { set_error(ODL_ERR_LAUNCH, "%s: hipGetDevice: %s", who, hipGetErrorString(e)); return nullptr; }
+    const float *ptr = __atomic_load_n(&cached[dev], __ATOMIC_ACQUIRE);
+    if (!ptr) {
+        void *addr = nullptr;
+        e = hipGetSymbolAddress(&addr, HIP_SYMBOL(mx_unit_scale));
+        if (e != hipSuccess || !addr) { set_error(ODL_ERR_LAUNCH, "%s: hipGetSymbolAddress on device %d: %s", who, dev, hipGetErrorString(e)); return nullptr; }
+        ptr = static_cast<const float *>(addr);
+        __atomic_store_n(&cached[dev], ptr, __ATOMIC_RELEASE);
+    }
+    return ptr;
+}
+
+template <int SRC, int FMT>
+static void launch_mx_cast(const void *x, int64_t rows, int64_t cols, uint8_t *out, uint8_t *scales, uint8_t *out_t, uint8_t *scales_t,
+                           hipStream_t stream) {
+    const int64_t g = ((rows + kTileR - 1) / kTileR) * ((cols + kTileC - 1) / kTileC);
+#define ODL_MX(R, C) hipLaunchKernelGGL((mx_cast_kernel<SRC, FMT, R, C>), dim3((unsigned)g), dim3(kMxThreads), 0, stream, x, rows, cols, out, scales, out_t, scales_t)
+    if (out && out_t) ODL_MX(true, true);
+    else if (out) ODL_MX(true, false);
+    else ODL_MX(false, true);
+#undef ODL_MX
+}
+
+template <int FA, int FB>
+static void launch_mx_gemm(const GemmArgs &g, const uint8_t *sa, const uint8_t *sb, bool tiled, int cus, hipStream_t stream) {
+    if (!tiled) {
+        hipLaunchKernelGGL((mx_gemm_generic_kernel<FA, FB>), dim3((unsigned)((g.N + 31) / 32), (unsigned)((g.M + 31) / 32)), dim3(64), 0, stream, g, sa, sb);
+        return;
+    }
+    GemmArgs t = g;
+    // 256 x 256 tiles (8 waves of 128 x 64) when they fill the chip, else 128 x 128 (two blocks per compute unit)
+    const int64_t big = ((g.M + 255) / 256) * ((g.N + 255) / 256);
+    if (big >= cus) {
+        t.tiles_m = (int)((g.M + 255) / 256); t.tiles_n = (int)((g.N + 255) / 256);
+        const unsigned grid = (unsigned)(((t.tiles_m * t.tiles_n + 7) / 8) * 8);
+        hipLaunchKernelGGL((mx_gemm_tiled_kernel<256, 256, 2, 4, FA, FB>), dim3(grid), dim3(512), 0, stream, t, sa, sb);
+    } else {
+        t.tiles_m = (int)((g.M + 127) / 128); t.tiles_n = (int)((g.N + 127) / 128);
+        const unsigned grid = (unsigned)(((t.tiles_m * t.tiles_n + 7) / 8) * 8);
+        hipLaunchKernelGGL((mx_gemm_tiled_kernel<128, 128, 2, 2, FA, FB>), dim3(grid), dim3(256), 0, stream, t, sa, sb);
+    }
+}
+
+}  // namespace odl
+
+using namespace odl;
+
+extern "C" int odl_fp8_mx_cast(const void *x, int src_dtype, int64_t rows, int64_t cols, int fmt, uint8_t *out, uint8_t *scales,
+                               uint8_t *out_t, uint8_t *scales_t, odl_stream_t stream_) {
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    if (rows < 0 || cols < 0) return set_error(ODL_ERR_ARG, "odl_fp8_mx_cast: negative shape");
+    if (src_dtype != ODL_BF16 && src_dtype != ODL_F32) return set_error(ODL_ERR_ARG, "odl_fp8_mx_cast: src_dtype %d", src_dtype);
+    if (fmt != ODL_FP8_E4M3 && fmt != ODL_FP8_E5M2) return set_error(ODL_ERR_ARG, "odl_fp8_mx_cast: fmt %d", fmt);
+    if (rows * cols == 0) return ODL_OK;
+    if ((out == nullptr) != (scales == nullptr) || (out_t == nullptr) != (scales_t == nullptr))
+        return set_error(ODL_ERR_ARG, "odl_fp8_mx_cast: codes and scale bytes of a layout go together");
+    if (!out && !out_t) return set_error(ODL_ERR_ARG, "odl_fp8_mx_cast: neither layout asked for");
+    if (!x) return set_error(ODL_ERR_ARG, "odl_fp8_mx_cast: x is null");
+    if (cols % 8 != 0 || (out && cols % kMxBlock != 0) || (out_t && rows % kMxBlock != 0))
+        return set_error(ODL_ERR_SHAPE, "odl_fp8_mx_cast: %lld x %lld: the blocked axis must be a multiple of 32 (cols for out, rows for out_t) and cols of 8",
+                         (long long)rows, (long long)cols);
+    auto mis = [](const void *p, uintptr_t a) { return p && (reinterpret_cast<uintptr_t>(p) & (a - 1)); };
+    if (mis(x, 16) || mis(out, 8) || mis(out_t, 16)) return set_error(ODL_ERR_SHAPE, "odl_fp8_mx_cast: x and out_t must be 16-byte aligned, out 8-byte");
+    const int64_t tiles = ((rows + kTileR - 1) / kTileR) * ((cols + kTileC - 1) / kTileC);
+    if (tiles > 0x7fffffffLL) return set_error(ODL_ERR_SHAPE, "odl_fp8_mx_cast: too many tiles for one launch");
+    if (src_dtype == ODL_BF16) {
+        if (fmt == ODL_FP8_E4M3) launch_mx_cast<ODL_BF16, ODL_FP8_E4M3>(x, rows, cols, out, scales, out_t, scales_t, stream);
+        else launch_mx_cast<ODL_BF16, ODL_FP8_E5M2>(x, rows, cols, out, scales, out_t, scales_t, stream);
+    } else {
+        if (fmt == ODL_FP8_E4M3) launch_mx_cast<ODL_F32, ODL_FP8_E4M3>(x, rows, cols, out, scales, out_t, scales_t, stream);
+        else launch_mx_cast<ODL_F32, ODL_FP8_E5M2>(x, rows, cols, out, scales, out_t, scales_t, stream);
+    }
+    return check_launch("odl_fp8_mx_cast");
+}
+
+extern "C" int odl_fp8_mx_gemm_nt(const uint8_t *a, const uint8_t *sa, const uint8_t *b, const uint8_t *sb, int64_t M, int64_t N, int64_t K,
+                                  int fmt_a, int fmt_b, const float *bias, void *c, int out_dtype, odl_stream_t stream_) {
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    if (M < 0 || N < 0 || K < 0) return set_error(ODL_ERR_ARG, "odl_fp8_mx_gemm_nt: negative shape");
+    if ((fmt_a != ODL_FP8_E4M3 && fmt_a != ODL_FP8_E5M2) || (fmt_b != ODL_FP8_E4M3 && fmt_b != ODL_FP8_E5M2))
+        return set_error(ODL_ERR_ARG, "odl_fp8_mx_gemm_nt: formats %d, %d", fmt_a, fmt_b);
+    if (out_dtype != ODL_BF16 && out_dtype != ODL_F32) return set_error(ODL_ERR_ARG, "odl_fp8_mx_gemm_nt: out_dtype %d", out_dtype);
+    if (M == 0 || N == 0) return ODL_OK;
+    if (!a || !sa || !b || !sb || !c) return set_error(ODL_ERR_ARG, "odl_fp8_mx_gemm_nt: null pointer");
+    if (K == 0 || K % kMxBlock != 0) return set_error(ODL_ERR_SHAPE, "odl_fp8_mx_gemm_nt: K = %lld must be a positive multiple of 32", (long long)K);
+    auto mis = [](const void *p, uintptr_t al) { return (reinterpret_cast<uintptr_t>(p) & (al - 1)) != 0; };
+    if (mis(a, 16) || mis(b, 16) || mis(c, 16) || (bias && mis(bias, 16)))
+        return set_error(ODL_ERR_SHAPE, "odl_fp8_mx_gemm_nt: operands, output and bias must be 16-byte aligned");
+    const float *one = unit_scale_for_current_device("odl_fp8_mx_gemm_nt");
+    if (!one) return ODL_ERR_LAUNCH;
+    GemmArgs g{};
+    g.a = a; g.b = b; g.c = c; g.sa = one; g.sb = one; g.bias = bias;
+    g.M = M; g.N = N; g.K = K; g.sa_vec = 0; g.sb_vec = 0; g.out_dtype = out_dtype;
+    // the tiled kernel addresses rows with 32-bit offsets and reads whole scale dwords (4 blocks = one 128-byte K step)
+    const bool tiled = K % 128 == 0 && !mis(sa, 4) && !mis(sb, 4) && (double)(M + 256) * (double)K < 2147483648.0 &&
+                       (double)(N + 256) * (double)K < 2147483648.0 && M >= 32 && N >= 32;
+    const int cus = device_cu_count();
+#define ODL_MXG(FA_, FB_) launch_mx_gemm<FA_, FB_>(g, sa, sb, tiled, cus, stream)
+    if (fmt_a == ODL_FP8_E4M3 && fmt_b == ODL_FP8_E4M3) ODL_MXG(ODL_FP8_E4M3, ODL_FP8_E4M3);
+    else if (fmt_a == ODL_FP8_E5M2 && fmt_b == ODL_FP8_E4M3) ODL_MXG(ODL_FP8_E5M2, ODL_FP8_E4M3);
+    else if (fmt_a == ODL_FP8_E4M3 && fmt_b == ODL_FP8_E5M2) ODL_MXG(ODL_FP8_E4M3, ODL_FP8_E5M2);
+    else ODL_MXG(ODL_FP8_E5M2, ODL_FP8_E5M2);
+#undef ODL_MXG
+    return check_launch("odl_fp8_mx_gemm_nt");
+}

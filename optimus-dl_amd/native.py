@@ -24,7 +24,7 @@ DT_BF16, DT_F32 = 0, 1
 AMAX_MAX, AMAX_MOST_RECENT = 0, 1
 FP8_MAX = {E4M3: 448.0, E5M2: 57344.0}
 TORCH_FP8 = {E4M3: torch.float8_e4m3fn, E5M2: torch.float8_e5m2}
-ABI_VERSION = 11
+ABI_VERSION = 12
 AMAX_PARTS = 512                       # ODL_FP8_AMAX_PARTS
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
@@ -68,6 +68,8 @@ EXPORTS = (
     "odl_fp8_gemm_variant_name",
     "odl_fp8_gemm_set_variant",
     "odl_fp8_gemm_set_clock_probe",
+    "odl_fp8_mx_cast",
+    "odl_fp8_mx_gemm_nt",
 )
 
 _lib = None
@@ -137,6 +139,8 @@ def load() -> ctypes.CDLL:
         L.odl_fp8_gemm_variant_name.restype = ctypes.c_char_p
         L.odl_fp8_gemm_set_variant.argtypes = [i32]
         L.odl_fp8_gemm_set_clock_probe.argtypes = [vp, i32]
+        L.odl_fp8_mx_cast.argtypes = [vp, i32, i64, i64, i32, vp, vp, vp, vp, vp]
+        L.odl_fp8_mx_gemm_nt.argtypes = [vp, vp, vp, vp, i64, i64, i64, i32, i32, vp, vp, i32, vp]
         for name in EXPORTS:
             getattr(L, name)  # AttributeError here = the library does not match the header
         if L.odl_fp8_abi_version() != ABI_VERSION:
@@ -715,6 +719,56 @@ def gemm_nt(a: torch.Tensor, b: torch.Tensor, fmt_a: int, fmt_b: int, sa_inv: to
     _check(load().odl_fp8_gemm_nt(a.data_ptr(), b.data_ptr(), M, N, K, fmt_a, fmt_b, sa_inv.data_ptr(), sa_inv.numel(),
                                   sb_inv.data_ptr(), sb_inv.numel(), bias.data_ptr() if bias is not None else None,
                                   DT_F32, out.data_ptr(), odt, _stream()), "odl_fp8_gemm_nt")
+    return out
+
+
+MX_BLOCK = 32
+
+
+def mx_cast(x: torch.Tensor, fmt: int, want_rowmajor: bool = True, want_transposed: bool = False):
+    """MXFP8 conversion of ``x`` [rows, cols] in one launch -> (codes [rows, cols], scales [rows, cols/32],
+    codes_t [cols, rows], scales_t [cols, rows/32]); the pair that was not asked for is (None, None).  Scales are E8M0
+    bytes, one per 32 elements along the last axis of the codes they belong to."""
+    x = _as_2d(x)
+    rows, cols = x.shape
+    if not (want_rowmajor or want_transposed):
+        raise NativeError("mx_cast: neither layout asked for")
+    dev = x.device
+    out = sc = out_t = sc_t = None
+    if want_rowmajor:
+        out = torch.empty((rows, cols), dtype=torch.uint8, device=dev)
+        sc = torch.empty((rows, cols // MX_BLOCK), dtype=torch.uint8, device=dev)
+    if want_transposed:
+        out_t = torch.empty((cols, rows), dtype=torch.uint8, device=dev)
+        sc_t = torch.empty((cols, rows // MX_BLOCK), dtype=torch.uint8, device=dev)
+    ptr = lambda t: t.data_ptr() if t is not None else None
+    _check(load().odl_fp8_mx_cast(x.data_ptr(), _src_dtype(x), rows, cols, fmt, ptr(out), ptr(sc), ptr(out_t), ptr(sc_t), _stream()),
+           "odl_fp8_mx_cast")
+    return out, sc, out_t, sc_t
+
+
+def mx_gemm_nt(a: torch.Tensor, sa: torch.Tensor, b: torch.Tensor, sb: torch.Tensor, fmt_a: int, fmt_b: int,
+               bias: torch.Tensor | None = None, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """out[M,N] = sum over 32-blocks of 2^(sa-127) 2^(sb-127) (a_block . b_block) (+ bias); a [M,K], b [N,K] codes,
+    sa [M,K/32], sb [N,K/32] E8M0 bytes."""
+    for t, what in ((a, "a"), (b, "b"), (sa, "sa"), (sb, "sb")):
+        if t.dtype != torch.uint8 or not t.is_cuda or not t.is_contiguous() or t.dim() != 2:
+            raise NativeError(f"mx_gemm_nt: {what} must be a dense 2-D uint8 device tensor")
+    M, K = a.shape
+    N, K2 = b.shape
+    if K != K2:
+        raise NativeError(f"mx_gemm_nt: contraction sizes differ ({K} vs {K2})")
+    if K % MX_BLOCK or tuple(sa.shape) != (M, K // MX_BLOCK) or tuple(sb.shape) != (N, K // MX_BLOCK):
+        raise NativeError(f"mx_gemm_nt: scales must be [M, K/32] and [N, K/32] with K % 32 == 0, got {tuple(sa.shape)}, {tuple(sb.shape)} for K = {K}")
+    if bias is not None:
+        _f32_dev(bias, N, "mx_gemm_nt bias")
+    odt = DT_BF16 if out_dtype == torch.bfloat16 else (DT_F32 if out_dtype == torch.float32 else None)
+    if odt is None:
+        raise NativeError(f"mx_gemm_nt: output dtype {out_dtype} is not supported (bf16 or fp32)")
+    out = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    _check(load().odl_fp8_mx_gemm_nt(a.data_ptr(), sa.data_ptr(), b.data_ptr(), sb.data_ptr(), M, N, K, fmt_a, fmt_b,
+                                     bias.data_ptr() if bias is not None else None, out.data_ptr(), odt, _stream()),
+           "odl_fp8_mx_gemm_nt")
     return out
 
 

@@ -1,0 +1,216 @@
+"""GPU parity of the MXFP8 kernels (32-element blocks, E8M0 scale bytes) against the CPU oracle.
+
+Codes and scale bytes must be bit-exact (C restatement and the independent torch restatement).  The block-scaled
+matmul is compared with the emulated one (exact dequantisation, fp32 matmul): max|err| / max|ref| <= 1e-2 on the bf16
+output, the bar of the FP8 GEMMs, and element by element on the fp32 output against what the matrix instruction's
+internal adder can lose.
+Every call goes through the C ABI.
+"""
+import pytest
+import torch
+
+from oracle import oracle as O
+from tests.helpers import assert_bytes_equal, max_rel_err, seeded_bf16
+
+pytestmark = pytest.mark.gpu
+
+E4M3, E5M2 = O.E4M3, O.E5M2
+
+
+@pytest.fixture(scope="module")
+def N():
+    from optimus_dl_amd import native
+
+    native.load()
+    return native
+
+
+def _mixed(shape, seed):
+    """Gaussian values whose magnitude changes by powers of two from block to block and row to row, so that the scale
+    bytes cover a wide range, plus zeros, an all-zero block and a few large outliers."""
+    g = torch.Generator().manual_seed(seed)
+    rows, cols = shape
+    x = torch.randn(shape, generator=g)
+    x = x * torch.exp2(torch.randint(-20, 20, (rows, 1), generator=g).float())
+    x = x * torch.exp2(torch.randint(-6, 6, (1, cols), generator=g).float())
+    x[torch.rand(shape, generator=g) < 0.05] = 0.0
+    if rows >= 32 and cols >= 32:
+        x[:32, :32] = 0.0                                   # a zero block in both directions
+        x[rows - 1, cols - 1] = 3.0e38
+        x[rows // 2, cols // 2] = -1.0e-38
+    return x.bfloat16()
+
+
+CAST_SHAPES = [(32, 32), (128, 64), (64, 96), (160, 224), (256, 1024), (1024, 768), (96, 4096), (2016, 160)]
+
+
+@pytest.mark.parametrize("shape", CAST_SHAPES)
+@pytest.mark.parametrize("fmt", [E4M3, E5M2])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_mx_cast_both_layouts_bit_exact(N, shape, fmt, dtype):
+    x = _mixed(shape, seed=shape[0] * 7 + shape[1] + fmt)
+    out, sc, out_t, sc_t = N.mx_cast(x.to(dtype).cuda(), fmt, want_rowmajor=True, want_transposed=True)
+    wc, ws = O.c_mx_quantise(x, fmt)
+    assert_bytes_equal(sc, ws, f"scale bytes {shape} fmt {fmt}")
+    assert_bytes_equal(out, wc, f"codes {shape} fmt {fmt}")
+    tc, ts = O.t_mx_quantise(x, fmt)
+    assert_bytes_equal(sc, ts, f"scale bytes (torch restatement) {shape}")
+    assert_bytes_equal(out, tc, f"codes (torch restatement) {shape}")
+    wct, wst = O.c_mx_quantise(x.t().contiguous(), fmt)
+    assert_bytes_equal(sc_t, wst, f"transposed scale bytes {shape} fmt {fmt}")
+    assert_bytes_equal(out_t, wct, f"transposed codes {shape} fmt {fmt}")
+
+
+@pytest.mark.parametrize("fmt", [E4M3, E5M2])
+def test_mx_cast_single_layouts_match_the_pair(N, fmt):
+    x = _mixed((384, 320), seed=5).cuda()
+    out, sc, out_t, sc_t = N.mx_cast(x, fmt, True, True)
+    o1, s1, n1, n2 = N.mx_cast(x, fmt, True, False)
+    assert n1 is None and n2 is None
+    assert_bytes_equal(o1, out, "row-major only: codes")
+    assert_bytes_equal(s1, sc, "row-major only: scales")
+    n1, n2, o2, s2 = N.mx_cast(x, fmt, False, True)
+    assert n1 is None and n2 is None
+    assert_bytes_equal(o2, out_t, "transposed only: codes")
+    assert_bytes_equal(s2, sc_t, "transposed only: scales")
+
+
+def test_mx_cast_row_major_accepts_any_row_count(N):
+    x = _mixed((45, 64), seed=9)
+    out, sc, _, _ = N.mx_cast(x.cuda(), E4M3, True, False)
+    wc, ws = O.c_mx_quantise(x, E4M3)
+    assert_bytes_equal(out, wc, "codes, 45 rows")
+    assert_bytes_equal(sc, ws, "scales, 45 rows")
+
+
+def test_mx_cast_specials(N):
+    x = torch.zeros((64, 64), dtype=torch.bfloat16)
+    x[0, 0] = float("inf")
+    x[1, 40] = float("nan")
+    x[2, :32] = torch.tensor(2.0 ** -130).bfloat16()         # bf16 subnormals: scale byte at the lower clamp
+    x[3, 0] = 448.0
+    x[3, 1] = 260.0
+    x[40, 5] = -float("inf")
+    for fmt in (E4M3, E5M2):
+        out, sc, out_t, sc_t = N.mx_cast(x.cuda(), fmt, True, True)
+        wc, ws = O.c_mx_quantise(x, fmt)
+        assert_bytes_equal(sc, ws, f"special scale bytes fmt {fmt}")
+        assert_bytes_equal(out, wc, f"special codes fmt {fmt}")
+        wct, wst = O.c_mx_quantise(x.t().contiguous(), fmt)
+        assert_bytes_equal(sc_t, wst, f"special transposed scale bytes fmt {fmt}")
+        assert_bytes_equal(out_t, wct, f"special transposed codes fmt {fmt}")
+        assert int(sc[0, 0]) == 255 and int(sc[1, 1]) == 255 and int(sc[5, 0]) == 0
+
+
+def test_mx_cast_rejects_bad_shapes(N):
+    with pytest.raises(N.NativeError, match="multiple of 32"):
+        N.mx_cast(torch.zeros((32, 48), dtype=torch.bfloat16, device="cuda"), E4M3, True, False)
+    with pytest.raises(N.NativeError, match="multiple of 32"):
+        N.mx_cast(torch.zeros((48, 64), dtype=torch.bfloat16, device="cuda"), E4M3, False, True)
+    out = N.mx_cast(torch.zeros((0, 64), dtype=torch.bfloat16, device="cuda"), E4M3, True, True)
+    assert out[0].shape == (0, 64) and out[2].shape == (64, 0)
+
+
+# ------------------------------------------------------------------------------------------------ GEMM
+def _operands(M, N_, K, fa, fb, seed):
+    a = _mixed((M, K), seed)
+    b = _mixed((N_, K), seed + 1)
+    # keep the products inside fp32 / bf16 range: the outliers of _mixed are for the cast tests
+    a = a.float().clamp(-1e4, 1e4).bfloat16()
+    b = b.float().clamp(-1e4, 1e4).bfloat16()
+    ac, asc = O.c_mx_quantise(a, fa)
+    bc, bsc = O.c_mx_quantise(b, fb)
+    return ac, asc, bc, bsc
+
+
+def _assert_within_hardware_sum(got32, ac, asc, bc, bsc, fa, fb, bias=None):
+    """Element by element against the exact (float64) block-scaled dot product.  The FP8 MFMA adds the 8 products of two
+    consecutive operand dwords in an adder aligned to the largest of them that keeps 13 bits below it (measured: a
+    product 2^-14 of the largest in its group of 8 is dropped, 2^-13 is kept; between groups the sum is fp32), so
+    |error| <= 7 * 2^-14 * sum|a||b| plus fp32 rounding; 2^-10 * sum|a||b| is the bar here."""
+    A, B = O.t_mx_dequantise(ac, asc, fa).double(), O.t_mx_dequantise(bc, bsc, fb).double()
+    exact, absdot = A @ B.t(), A.abs() @ B.abs().t()
+    if bias is not None:
+        exact, absdot = exact + bias.double(), absdot + bias.double().abs()
+    err = (got32.double() - exact).abs()
+    worst = float((err / absdot.clamp_min(1e-30)).max())
+    assert bool((err <= absdot * 2.0 ** -10 + 1e-30).all()), worst      # 1e-30: results below the fp32 range become 0
+
+
+GEMM_SHAPES = [
+    (32, 32, 32), (32, 32, 96), (64, 96, 160), (100, 72, 224), (7, 13, 64),            # plain kernel (K % 128 != 0 or tiny)
+    (128, 128, 128), (256, 256, 512), (384, 640, 1024), (200, 136, 256), (130, 70, 384),  # 128 x 128 tiles, edges
+    (4096, 4096, 256), (4100, 4232, 128),                                                # 256 x 256 tiles, interior and edges
+]
+
+
+@pytest.mark.parametrize("shape", GEMM_SHAPES)
+@pytest.mark.parametrize("fmts", [(E4M3, E4M3), (E5M2, E4M3), (E4M3, E5M2)])
+def test_mx_gemm_matches_emulation(N, shape, fmts):
+    M, N_, K = shape
+    if M * N_ > 4096 * 1024 and fmts != (E4M3, E4M3):
+        pytest.skip("large shapes once")
+    fa, fb = fmts
+    ac, asc, bc, bsc = _operands(M, N_, K, fa, fb, seed=M + N_ + K)
+    ref_bf16, ref_f32 = O.t_mx_gemm_nt(ac, asc, bc, bsc, fa, fb, want_f32=True)
+    got32 = N.mx_gemm_nt(ac.cuda(), asc.cuda(), bc.cuda(), bsc.cuda(), fa, fb, out_dtype=torch.float32).cpu()
+    assert got32.shape == (M, N_)
+    _assert_within_hardware_sum(got32, ac, asc, bc, bsc, fa, fb)
+    got = N.mx_gemm_nt(ac.cuda(), asc.cuda(), bc.cuda(), bsc.cuda(), fa, fb).cpu()
+    assert max_rel_err(got.float(), ref_bf16.float()) <= 1e-2
+    # one rounding of the fp32 result: the bf16 output is the fp32 output rounded
+    assert torch.equal(got, got32.bfloat16())
+
+
+def test_mx_gemm_small_case_against_the_c_oracle_and_bias(N):
+    M, N_, K = 48, 40, 96
+    ac, asc, bc, bsc = _operands(M, N_, K, E4M3, E4M3, seed=3)
+    bias = torch.randn(N_)
+    c_bf16, c_f32 = O.c_mx_gemm_nt(ac, asc, bc, bsc, E4M3, E4M3, bias)
+    got = N.mx_gemm_nt(ac.cuda(), asc.cuda(), bc.cuda(), bsc.cuda(), E4M3, E4M3, bias=bias.cuda(), out_dtype=torch.float32).cpu()
+    assert max_rel_err(got, c_f32) <= 2e-3
+    _assert_within_hardware_sum(got, ac, asc, bc, bsc, E4M3, E4M3, bias)
+    M, N_, K = 256, 384, 256
+    ac, asc, bc, bsc = _operands(M, N_, K, E4M3, E4M3, seed=4)
+    bias = torch.randn(N_)
+    got = N.mx_gemm_nt(ac.cuda(), asc.cuda(), bc.cuda(), bsc.cuda(), E4M3, E4M3, bias=bias.cuda(), out_dtype=torch.float32).cpu()
+    _assert_within_hardware_sum(got, ac, asc, bc, bsc, E4M3, E4M3, bias)
+    gotb = N.mx_gemm_nt(ac.cuda(), asc.cuda(), bc.cuda(), bsc.cuda(), E4M3, E4M3, bias=bias.cuda()).cpu()
+    assert torch.equal(gotb, got.bfloat16())
+
+
+def test_mx_gemm_block_scales_act_per_block(N):
+    """Raising one scale byte of A by 1 doubles exactly that block's contribution: with every other block zeroed the
+    output doubles bit for bit; and a NaN scale byte poisons its row only."""
+    M, N_, K = 128, 128, 256
+    ac, asc, bc, bsc = _operands(M, N_, K, E4M3, E4M3, seed=11)
+    keep = torch.zeros_like(ac)
+    keep[:, 64:96] = ac[:, 64:96]
+    base = N.mx_gemm_nt(keep.cuda(), asc.cuda(), bc.cuda(), bsc.cuda(), E4M3, E4M3, out_dtype=torch.float32).cpu()
+    asc2 = asc.clone()
+    asc2[:, 2] = (asc2[:, 2].int() + 1).clamp(max=254).to(torch.uint8)
+    grown = asc2[:, 2] != asc[:, 2]
+    twice = N.mx_gemm_nt(keep.cuda(), asc2.cuda(), bc.cuda(), bsc.cuda(), E4M3, E4M3, out_dtype=torch.float32).cpu()
+    assert torch.equal(twice[grown], 2 * base[grown])
+    asc3 = asc.clone()
+    asc3[5, 7] = 255
+    out = N.mx_gemm_nt(ac.cuda(), asc3.cuda(), bc.cuda(), bsc.cuda(), E4M3, E4M3, out_dtype=torch.float32).cpu()
+    assert bool(torch.isnan(out[5]).all()) and not bool(torch.isnan(out[:5]).any()) and not bool(torch.isnan(out[6:]).any())
+
+
+def test_mx_round_trip_error_bound_at_full_size(N):
+    """Size-independent property at a model-sized shape: |x - dequant(quant(x))| <= 2^-3 * block amax for E4M3 (the
+    scaled amax lies in [256, 512): up to 448 the spacing is 32, above it the value saturates, at most 64 away), in
+    both layouts."""
+    rows, cols = 4096, 4096
+    x = seeded_bf16((rows, cols), std=1.0, seed=21)
+    out, sc, out_t, sc_t = N.mx_cast(x.cuda(), E4M3, True, True)
+    deq = O.t_mx_dequantise(out.cpu(), sc.cpu(), E4M3)
+    v = x.float().reshape(rows, cols // 32, 32)
+    amax = v.abs().amax(dim=2, keepdim=True)
+    err = (deq.reshape(rows, cols // 32, 32) - v).abs()
+    assert bool((err <= amax * 2.0 ** -3).all())
+    deq_t = O.t_mx_dequantise(out_t.cpu(), sc_t.cpu(), E4M3)
+    vt = x.t().float().reshape(cols, rows // 32, 32)
+    amax_t = vt.abs().amax(dim=2, keepdim=True)
+    assert bool(((deq_t.reshape(cols, rows // 32, 32) - vt).abs() <= amax_t * 2.0 ** -3).all())
