@@ -19,6 +19,10 @@ Per call, inside ``FP8Recipe.autocast()``:
             dW = Q(dY)^T . Q(X)
             db = sum_rows(dY)        (fp32 accumulate)
 
+Under the "mxfp8" recipe every operand is quantised in blocks of 32 along the axis its GEMM contracts (X and W along
+the input features for the forward, dY and W along the output features for dgrad, dY and X along the tokens for wgrad),
+each block with its own power-of-two scale byte; there is no amax pass and no scaling state.
+
 Every GEMM is issued in the "NT" form the MFMA wants (both operands contiguous
 along the contraction axis); the cast+transpose kernel supplies the transposed
 FP8 copies, and the forward keeps only the 1-byte ``Q(X)^T`` for wgrad instead of
@@ -113,6 +117,23 @@ def _quantise_input_shared(recipe: FP8Recipe, x2d: torch.Tensor, fmt: int, margi
     return q, q_t, s_inv
 
 
+def _mx_input_shared(recipe: FP8Recipe, x2d: torch.Tensor, fmt: int, need_t: bool):
+    """MXFP8 codes and scale bytes of a Linear's input (blocks along the features; with need_t also of its transpose,
+    blocks along the tokens), made once for the Linears fed by the very same tensor."""
+    key = _input_key(x2d, "mx", fmt, 0)
+    hit = recipe.shared_input if recipe.share_inputs else None
+    if hit is not None and hit["key"] == key and (hit["q_t"] is not None or not need_t):
+        return hit["q"], hit["s_inv"], hit["q_t"], hit["s_t"]
+    q, sc, q_t, sc_t = native.mx_cast(x2d, fmt, want_rowmajor=True, want_transposed=need_t)
+    if recipe.share_inputs:
+        entry = {"key": key, "x": x2d, "q": q, "q_t": q_t, "s_inv": sc, "s_t": sc_t}
+        prev = recipe.shared_input
+        if prev is not None and prev.get("x") is x2d:
+            entry["src_key"], entry["src"] = prev.get("src_key"), prev.get("src")
+        recipe.shared_input = entry
+    return q, sc, q_t, sc_t
+
+
 def _converted_input(recipe: FP8Recipe, x2d: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
     """x2d in the compute dtype, contiguous.  Linears fed by the same tensor get the same
     converted tensor back (one conversion, and one quantisation downstream); autograd sees an
@@ -168,7 +189,16 @@ class _Fp8LinearFn(torch.autograd.Function):
         saved: dict[str, Any] = {}
         ctx.wgrad_direct = False
 
-        if pol.kind == "rowwise":
+        if pol.kind == "mxfp8":
+            fp8_wgrad = need_wgrad and recipe.wgrad
+            xq, xs, xq_t, xs_t = _mx_input_shared(recipe, x2d, pol.fmt_fwd, fp8_wgrad)
+            wq, ws, wq_t, ws_t = module._mx_weight(weight, recipe, need_t=need_dgrad)
+            y = native.mx_gemm_nt(xq, xs, wq, ws, pol.fmt_fwd, pol.fmt_fwd, bias=bias_f32, out_dtype=out_dtype)
+            if fp8_wgrad:
+                saved["xq_t"], saved["xs_t"] = xq_t, xs_t
+            if need_dgrad:
+                saved["wq_t"], saved["ws_t"] = wq_t, ws_t
+        elif pol.kind == "rowwise":
             if need_wgrad and recipe.wgrad:
                 # both operands of x in two passes over it: rows for this GEMM, columns (transposed) for wgrad
                 xq, sx_inv, saved["xq_t"], saved["sx_inv_t"], _, _ = native.quantize_rowcol(x2d, pol.fmt_fwd, pol.margin)
@@ -226,7 +256,15 @@ class _Fp8LinearFn(torch.autograd.Function):
         dx = dw = db = None
         fp8_wgrad = ctx.need_wgrad and recipe.wgrad
 
-        if pol.kind == "rowwise":
+        if pol.kind == "mxfp8":
+            if ctx.need_dgrad or fp8_wgrad:
+                # one pass over dy: blocks along the output features for dgrad, along the tokens (transposed) for wgrad
+                gq, gs, gq_t, gs_t = native.mx_cast(dy2d, pol.fmt_bwd, want_rowmajor=ctx.need_dgrad, want_transposed=fp8_wgrad)
+            if ctx.need_dgrad:
+                dx = native.mx_gemm_nt(gq, gs, saved["wq_t"], saved["ws_t"], pol.fmt_bwd, pol.fmt_fwd, out_dtype=ctx.x_dtype)
+            if fp8_wgrad:
+                dw = native.mx_gemm_nt(gq_t, gs_t, saved["xq_t"], saved["xs_t"], pol.fmt_bwd, pol.fmt_fwd, out_dtype=ctx.w_dtype)
+        elif pol.kind == "rowwise":
             if ctx.need_dgrad and fp8_wgrad:
                 gq, sg_inv, gq_t, sg_inv_t, _, _ = native.quantize_rowcol(dy2d, pol.fmt_bwd, pol.margin)
             elif ctx.need_dgrad:
@@ -403,6 +441,18 @@ class FP8Linear(nn.Linear):
         self._wcache_rowwise[axis] = (key, q, s_inv)
         return q, s_inv
 
+    def _mx_weight(self, weight: torch.Tensor, recipe: FP8Recipe, need_t: bool):
+        """MXFP8 codes and scale bytes of W (blocks along the input features) and, with need_t, of W^T (blocks along
+        the output features, for dgrad); kept while the Parameter is unchanged."""
+        fmt = recipe.recipe.fmt_fwd
+        key = _weight_key(weight, fmt, ("mx",))
+        hit = self._wcache_rowwise.get("mx")
+        if hit is not None and hit[0] == key and recipe.cache_weights and (hit[3] is not None or not need_t):
+            return hit[1:]
+        q, sc, q_t, sc_t = native.mx_cast(weight.detach(), fmt, want_rowmajor=True, want_transposed=need_t)
+        self._wcache_rowwise["mx"] = (key, q, sc, q_t, sc_t)
+        return q, sc, q_t, sc_t
+
     # ------------------------------------------------------------------ forward
     def _fp8_eligible(self, x: torch.Tensor) -> bool:
         if not x.is_cuda or not self.weight.is_cuda:
@@ -411,10 +461,13 @@ class FP8Linear(nn.Linear):
             _warn_once(f"FP8Linear: weight dtype {self.weight.dtype} is not bf16/fp32; running as a plain Linear")
             return False
         tokens = x.numel() // max(self.in_features, 1)
-        if self.in_features % 16 or self.out_features % 16 or tokens % 16 or tokens == 0:
+        recipe = _state.active_recipe()
+        # MXFP8 blocks are 32 long along every axis a GEMM of this layer contracts (features in and out, tokens)
+        mult = 32 if recipe is not None and recipe.recipe.kind == "mxfp8" else 16
+        if self.in_features % mult or self.out_features % mult or tokens % mult or tokens == 0:
             _warn_once(
                 f"FP8Linear({self.in_features}->{self.out_features}) with {tokens} tokens: sizes must be multiples "
-                "of 16 for the FP8 kernels; this call runs as a plain Linear"
+                f"of {mult} for the FP8 kernels; this call runs as a plain Linear"
             )
             return False
         return True

@@ -218,7 +218,8 @@ def test_e5m2_delayed_is_refused_and_block_recipes_have_no_kernels(amp):
     r = amp.FP8Recipe("tensorwise", "e5m2")
     assert r.format == amp.Fp8Format.E5M2 and r.recipe.fmt_fwd == O.E5M2
     with pytest.raises(NotImplementedError):
-        amp.FP8Recipe("mxfp8", "hybrid")
+        amp.FP8Recipe("blockwise", "hybrid")
+    assert amp.FP8Recipe("mxfp8", "hybrid").recipe.kind == "mxfp8"
     rec = amp.create_fp8_recipe("delayed", "hybrid", margin=2, amax_history_len=32, amax_compute_algo="most_recent", reduce_amax=False)
     assert (rec.margin, rec.amax_history_len, rec.amax_compute_algo, rec.reduce_amax, rec.fp8_dpa, rec.fp8_mha) == (2, 32, "most_recent", False, False, False)
     assert rec.recipe_type == amp.Fp8RecipeType.DELAYED and rec.format == amp.Fp8Format.HYBRID and rec.recipe is not None

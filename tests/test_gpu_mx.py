@@ -214,3 +214,120 @@ def test_mx_round_trip_error_bound_at_full_size(N):
     vt = x.t().float().reshape(cols, rows // 32, 32)
     amax_t = vt.abs().amax(dim=2, keepdim=True)
     assert bool(((deq_t.reshape(cols, rows // 32, 32) - vt).abs() <= amax_t * 2.0 ** -3).all())
+
+
+# ------------------------------------------------------------------------------------------------ the Linear
+def _mx_linear_reference(x, w, dy, fmt_fwd, fmt_bwd, bias=None):
+    """The three GEMMs of a Linear under MXFP8, emulated: every operand quantised along the axis its GEMM contracts."""
+    q = O.c_mx_quantise
+    y = O.t_mx_gemm_nt(*q(x, fmt_fwd), *q(w, fmt_fwd), fmt_fwd, fmt_fwd, bias=bias)
+    gq, gs = q(dy, fmt_bwd)
+    wtq, wts = q(w.t().contiguous(), fmt_fwd)
+    dx = O.t_mx_gemm_nt(gq, gs, wtq, wts, fmt_bwd, fmt_fwd)
+    gtq, gts = q(dy.t().contiguous(), fmt_bwd)
+    xtq, xts = q(x.t().contiguous(), fmt_fwd)
+    dw = O.t_mx_gemm_nt(gtq, gts, xtq, xts, fmt_bwd, fmt_fwd)
+    return {"y": y, "dx": dx, "dw": dw}
+
+
+@pytest.mark.parametrize("fmt", ["hybrid", "e4m3"])
+@pytest.mark.parametrize("shape", [(512, 1024, 768), (96, 160, 224)])
+def test_mxfp8_linear_matches_emulation(fmt, shape):
+    from optimus_dl_amd.modules import amp
+    from tests.test_gpu_linear import make_linear, run_step
+
+    M, K, N_ = shape
+    x, w, dy = seeded_bf16((M, K), 1.0, 0), seeded_bf16((N_, K), 0.02, 1), seeded_bf16((M, N_), 1e-3, 2)
+    x[:, 7] *= 64.0                                           # an outlier channel: block scales isolate it
+    recipe = amp.create_fp8_recipe("mxfp8", fmt)
+    assert recipe.recipe.kind == "mxfp8" and recipe.recipe_type == amp.Fp8RecipeType.MXFP8
+    lin = make_linear(w)
+    y, dx, dw = run_step(lin, recipe, x, dy)
+    assert lin.fp8_calls == 1
+    fb = O.E5M2 if fmt == "hybrid" else O.E4M3
+    ref = _mx_linear_reference(x, w, dy, O.E4M3, fb)
+    for name, got in (("y", y), ("dx", dx), ("dw", dw)):
+        assert got.dtype == torch.bfloat16
+        err = max_rel_err(got, ref[name])
+        assert err <= 1e-2, f"{name}: {err}"
+    # and it is a Linear: near the bf16 product.  (The floor rule of the shared exponent lets a block amax in the top
+    # eighth of its binade saturate, up to 12.5 % off on that element, which the outlier channel makes visible.)
+    want = x.float() @ w.float().t()
+    assert max_rel_err(y, want) <= 0.2
+
+
+def test_mxfp8_linear_bias_fp32_weights_and_weight_cache():
+    from optimus_dl_amd.modules import amp
+    from tests.test_gpu_linear import make_linear
+
+    B, S, K, N_ = 2, 64, 256, 512
+    x = seeded_bf16((B * S, K), 1.0, 3)
+    # fp32 master weights whose values bf16 holds exactly, so that the oracle (bf16 input) quantises the same numbers
+    w32 = (torch.randn(N_, K, generator=torch.Generator().manual_seed(4)) * 0.02).bfloat16().float()
+    bias = torch.randn(N_, generator=torch.Generator().manual_seed(5)) * 0.1
+    dy = seeded_bf16((B * S, N_), 1e-2, 6)
+    recipe = amp.create_fp8_recipe("mxfp8", "hybrid")
+    lin = make_linear(w32, bias, dtype=torch.float32)
+    xd = x.cuda().reshape(B, S, K).requires_grad_(True)
+    with amp.fp8_autocast(torch.device("cuda"), recipe, dtype=torch.bfloat16):
+        y = lin(xd)
+    assert y.shape == (B, S, N_) and y.dtype == torch.bfloat16
+    with amp.fp8_backward(recipe):
+        y.backward(dy.cuda().reshape(B, S, N_))
+    ref = _mx_linear_reference(x, w32.bfloat16(), dy, O.E4M3, O.E5M2, bias=bias)
+    assert max_rel_err(y.reshape(B * S, N_), ref["y"]) <= 1e-2
+    assert max_rel_err(xd.grad.reshape(B * S, K), ref["dx"]) <= 1e-2
+    assert lin.weight.grad.dtype == torch.float32 and max_rel_err(lin.weight.grad, ref["dw"]) <= 1e-2
+    want_db = dy.float().sum(dim=0)
+    assert max_rel_err(lin.bias.grad, want_db) <= 1e-3
+    # the weight's codes are kept while the Parameter is unchanged, and made again after an update
+    first = lin._wcache_rowwise["mx"][1]
+    with recipe.autocast():
+        lin(xd.detach())
+    assert lin._wcache_rowwise["mx"][1] is first
+    with torch.no_grad():
+        lin.weight.mul_(2.0)
+    with recipe.autocast():
+        y2 = lin(xd.detach())
+    assert lin._wcache_rowwise["mx"][1] is not first
+    assert max_rel_err(y2.reshape(B * S, N_) - bias.cuda().bfloat16(), 2 * (ref["y"].cuda() - bias.cuda().bfloat16())) <= 3e-2
+
+
+def test_mxfp8_linear_falls_back_for_sizes_that_are_not_multiples_of_32():
+    from optimus_dl_amd.modules import amp
+    from tests.test_gpu_linear import make_linear
+
+    recipe = amp.create_fp8_recipe("mxfp8", "hybrid")
+    lin = make_linear(seeded_bf16((48, 64), 0.02, 1))             # 48 outputs
+    with recipe.autocast():
+        y = lin(seeded_bf16((32, 64), 1.0, 2).cuda())
+    assert lin.fp8_calls == 0 and y.shape == (32, 48)
+    lin2 = make_linear(seeded_bf16((64, 64), 0.02, 1))
+    with recipe.autocast():
+        lin2(seeded_bf16((48, 64), 1.0, 3).cuda())                # 48 tokens
+    assert lin2.fp8_calls == 0
+    with recipe.autocast():
+        lin2(seeded_bf16((64, 64), 1.0, 3).cuda())
+    assert lin2.fp8_calls == 1
+
+
+def test_mxfp8_shared_input_is_quantised_once():
+    from optimus_dl_amd.modules import amp
+    from optimus_dl_amd import native
+    from tests.test_gpu_linear import make_linear
+
+    recipe = amp.create_fp8_recipe("mxfp8", "hybrid")
+    a, b = make_linear(seeded_bf16((64, 128), 0.02, 1)), make_linear(seeded_bf16((96, 128), 0.02, 2))
+    x = seeded_bf16((32, 128), 1.0, 3).cuda().requires_grad_(True)
+    calls = []
+    real = native.mx_cast
+    native.mx_cast = lambda t, *a_, **k_: (calls.append(tuple(t.shape)), real(t, *a_, **k_))[1]
+    try:
+        with recipe.autocast():
+            ya, yb = a(x), b(x)
+    finally:
+        native.mx_cast = real
+    assert calls.count((32, 128)) == 1 and len(calls) == 3, calls   # x once, each weight once
+    with recipe.backward():
+        (ya.sum() + yb.sum()).backward()
+    assert x.grad is not None and a.weight.grad is not None and b.weight.grad is not None
