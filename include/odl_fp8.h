@@ -423,22 +423,33 @@ int odl_fp8_gemm_set_variant(int variant);
  * E5M2), clamped to [-127, 127]; elements = rne(clamp(v / 2^shared, +-fp8_max)); a block of zeros gets byte 0, a block
  * that holds Inf or NaN gets 0xFF.  There is no amax pass and no scale state: one kernel reads x once.
  *
- *   out    [rows, cols]      codes, blocks along the columns;  scales   [rows, cols / 32]   (cols % 32 == 0)
- *   out_t  [cols, rows]      codes of x^T, blocks along the rows of x;  scales_t [cols, rows / 32]   (rows % 32 == 0)
+ *   out    [rows, cols]      codes, blocks along the columns;  scales   for [rows, cols / 32] blocks   (cols % 32 == 0)
+ *   out_t  [cols, rows]      codes of x^T, blocks along the rows of x;  scales_t for [cols, rows / 32] blocks   (rows % 32 == 0)
  * Either pair may be NULL (both members together).  cols % 8 == 0, x and out_t 16-byte aligned, out 8-byte aligned.
+ *
+ * Scale bytes of R rows x B blocks are stored in one of two layouts (chosen per output):
+ *   ODL_MX_SCALES_ROWMAJOR  [R][B]: byte (r, b) at r * B + b
+ *   ODL_MX_SCALES_KSTEP     [B / 4][R][4]: byte (r, b) at ((b / 4) * R + r) * 4 + b % 4; needs B % 4 == 0 (the blocked axis a
+ *                           multiple of 128).  The 4 scales a row needs for one 128-byte K step of a GEMM are one dword, and
+ *                           the dwords of consecutive rows are consecutive: a GEMM tile fetches its scales for a step as
+ *                           one contiguous run.  The streaming GEMM kernel takes only this layout.
  */
+#define ODL_MX_SCALES_ROWMAJOR 0
+#define ODL_MX_SCALES_KSTEP 1
 int odl_fp8_mx_cast(const void *x, int src_dtype, int64_t rows, int64_t cols, int fmt, uint8_t *out, uint8_t *scales,
-                    uint8_t *out_t, uint8_t *scales_t, odl_stream_t stream);
+                    int scales_layout, uint8_t *out_t, uint8_t *scales_t, int scales_t_layout, odl_stream_t stream);
 
 /*
  * C[M, N] = sum over blocks kb of 2^(sa[m, kb] - 127) * 2^(sb[n, kb] - 127) * dot(A[m, 32 kb .. +32], B[n, 32 kb .. +32])
  * (+ bias[n]), accumulated in fp32 by the scaled MFMA (V_MFMA_SCALE_F32_32X32X64_F8F6F4 applies the two block scales to
- * the products), one rounding to out_dtype.  a [M, K], b [N, K] codes; sa [M, K / 32], sb [N, K / 32] scale bytes;
- * K % 32 == 0; a, b, c and bias 16-byte aligned.  K % 128 == 0 with 4-byte aligned scale arrays runs the LDS-tiled
- * kernel; other shapes a plain one-wave-per-tile kernel.
+ * the products), one rounding to out_dtype.  a [M, K], b [N, K] codes; sa, sb the scale bytes of the M x K / 32 and
+ * N x K / 32 blocks, both in `scales_layout`; K % 32 == 0; a, b, c and bias 16-byte aligned.  With K-step-major scales,
+ * M % 128 == 0, N % 128 == 0, K >= 512 and enough tiles to fill the chip the persistent streaming kernel runs (the one of
+ * odl_fp8_gemm_nt, with the scale dwords riding beside the operand loads); K % 128 == 0 with 4-byte aligned scale arrays
+ * otherwise runs an LDS-tiled kernel; other shapes a plain one-wave-per-tile kernel.
  */
-int odl_fp8_mx_gemm_nt(const uint8_t *a, const uint8_t *sa, const uint8_t *b, const uint8_t *sb, int64_t M, int64_t N, int64_t K,
-                       int fmt_a, int fmt_b, const float *bias, void *c, int out_dtype, odl_stream_t stream);
+int odl_fp8_mx_gemm_nt(const uint8_t *a, const uint8_t *sa, const uint8_t *b, const uint8_t *sb, int scales_layout, int64_t M,
+                       int64_t N, int64_t K, int fmt_a, int fmt_b, const float *bias, void *c, int out_dtype, odl_stream_t stream);
 
 #ifdef __cplusplus
 }

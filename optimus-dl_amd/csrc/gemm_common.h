@@ -27,6 +27,9 @@ struct GemmArgs {
     // streaming kernel only, measurement aid: when set, the first wave of block 0 writes {shader-clock counter,
     // 100 MHz counter} on entry and on exit (4 x uint64): the average clock the board granted this launch
     unsigned long long *clock_out = nullptr;
+    // streaming kernel only: block scales of A and B (E8M0 bytes, one per 32 K-bytes), stored K-step-major:
+    // dword [K / 128][rows] = the 4 scale bytes of a row in one 128-byte K step.  Set: the MFMAs apply them.
+    const uint8_t *mx_sa = nullptr, *mx_sb = nullptr;
 };
 
 __device__ __forceinline__ int swz(int row) { return (row ^ (row >> 3)) & 7; }

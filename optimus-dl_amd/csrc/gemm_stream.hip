@@ -70,8 +70,22 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 // (32 rows of 128 bytes) and leaves right after its own MFMA: 64 stores per wave and tile instead of 32.
 // EPI: 0 = one scale per operand; 1 = a scale per row of A and / or per row of B (rowwise recipe);
 // 2 = the same plus an fp32 bias per output column.
-template <int FA, int FB, bool TA, bool TB, bool F32, int EPI>
+// MX: block-scaled operands (32 K-bytes share an E8M0 scale byte, applied by the MFMA itself).  g.mx_sa / g.mx_sb hold
+// the scale bytes K-step-major: dword [kstep][row] = the 4 scale bytes of row `row` in the 128-byte K step `kstep`.
+// Per K step a wave brings 64 such dwords of A and 64 of B to LDS with two 256-byte loads issued beside the operand
+// loads of the same step, placed so that a lane finds the dwords of its 4 fragment rows (32 apart) side by side: one
+// 16-byte LDS read per operand and step, made in phase B of the step before.  Lanes 32..63 shift the dword right by 8:
+// byte 0 / byte 2 are then the scales a lane supplies in phase A / phase B (the MFMA takes the scale of K 0..31 from
+// lanes 0..31 and of K 32..63 from lanes 32..63, and a lane's registers 0..3 / 4..7 as K 16 g.. / 32 + 16 g..).
+template <int FB, int FA, bool MX, int H>
+__device__ __forceinline__ v16f mma_step(const v8i &b, const v8i &a, const v16f &c, int eb, int ea) {
+    if constexpr (MX) return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(b, a, c, FB, FA, 2 * H, eb, 2 * H, ea);
+    else return mfma_32x32x64<FB, FA>(b, a, c);
+}
+
+template <int FA, int FB, bool TA, bool TB, bool F32, int EPI, bool MX = false>
 __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
+    static_assert(!MX || (!TA && !TB && EPI != 1), "block scales: both operands stored [rows, K], no scale vectors");
     constexpr int ESZ = F32 ? 4 : 2;
     constexpr int VEC_BYTES = 3 * 128 * 4;     // per wave: 128 row scales, 128 column scales, 128 bias values
     __shared__ __attribute__((aligned(1024))) uint8_t sA0[REGION];
@@ -80,6 +94,7 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
     __shared__ __attribute__((aligned(1024))) uint8_t sB1[REGION];
     __shared__ __attribute__((aligned(16))) uint8_t sEpi[NW * SLAB];
     __shared__ __attribute__((aligned(16))) uint8_t sVec[EPI > 0 ? NW * VEC_BYTES : 16];
+    __shared__ __attribute__((aligned(16))) uint32_t sScale[MX ? 2 * 512 : 4];     // [stage][A rows 0..255 | B rows 0..255], permuted
 
     const int lane = threadIdx.x % 64;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
@@ -163,7 +178,56 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
     int m0 = 0, n0 = 0;
     v4i rsrc_a, rsrc_b, next_a, next_b;           // raw buffer descriptors (base, stride 0, bytes, format)
 
-    // ---- LDS -> registers.  chunk(t, h, e) = ((2*lg + e) ^ s0) ^ 4*(h ^ (t & 1))
+    // one 256-byte direct-to-LDS load: 64 lanes x 4 bytes land at lds_addr + lane * 4
+    auto dma4 = [](const v4i &rsrc, uint32_t lds_addr, int vo, int so) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tbuffer_load_dword %1, %2, %3 offen lds"
+                     ::"s"(lds_addr), "v"(vo), "s"(rsrc), "s"(so));
+    };
+    // ---- block scales (MX).  One descriptor per operand covers the whole array; a tile and a K step are reached through
+    // the scalar offset, and a load that must deliver nothing (rows outside the matrix, the padding step, no next tile)
+    // gets the size field cleared.  Of each operand this wave fetches 64 dwords per step: LDS dword d = 64 wave + lane
+    // holds tile row 128 (d / 128) + 32 (d % 4) + (d % 128) / 4, so that rows r, r + 32, r + 64, r + 96 of a wave tile
+    // lie side by side.
+    auto whole_scales = [&](const uint8_t *p, int64_t rows) -> v4i {
+        const uint64_t addr = reinterpret_cast<uint64_t>(p);
+        return v4i{(int)(uint32_t)addr, (int)(uint32_t)(addr >> 32), (int)((uint32_t)(g.K / 128) * (uint32_t)rows * 4u), 0x00020000};
+    };
+    const v4i whole_sa = MX ? whole_scales(g.mx_sa, g.M) : empty, whole_sb = MX ? whole_scales(g.mx_sb, g.N) : empty;
+    const int sc_d = 64 * wave + lane;
+    const int sc_voff = (128 * (sc_d / 128) + 32 * (sc_d % 4) + (sc_d % 128) / 4) * 4;
+    const int sc_region = 128 * (wave / 2);       // first tile row of the 128 rows this wave fetches from (both operands)
+    int sc_off_a = 0, sc_off_b = 0, sc_next_a = 0, sc_next_b = 0;                    // bytes to (tile row 0, the item's first K step)
+    int sc_in_a = 0, sc_in_b = 0, sc_nin_a = 0, sc_nin_b = 0;                        // 1: those 128 rows exist (kept as
+    // integers and applied by multiplication: selects on loop-carried flags do not stay scalar code)
+    auto scale_origin = [&](int tm0, int tn0, int first_step, int &oa, int &ob, int &ia, int &ib) {
+        oa = (first_step * (int)g.M + tm0) * 4;
+        ob = (first_step * (int)g.N + tn0) * 4;
+        ia = tm0 + sc_region < (int)g.M ? 1 : 0;
+        ib = tn0 + sc_region < (int)g.N ? 1 : 0;
+    };
+    auto issue_scales = [&](int stage, int ok_a, int ok_b, int off_a, int off_b, int kstep) {
+        v4i da = whole_sa, db = whole_sb;
+        da.z = __builtin_amdgcn_readfirstlane(whole_sa.z * ok_a);
+        db.z = __builtin_amdgcn_readfirstlane(whole_sb.z * ok_b);
+        off_a = __builtin_amdgcn_readfirstlane(off_a);
+        off_b = __builtin_amdgcn_readfirstlane(off_b);
+        const uint32_t dst = lds_addr_of(reinterpret_cast<const uint8_t *>(sScale)) + (stage * 512 + 64 * wave) * 4;
+        dma4(da, dst, sc_voff, off_a + kstep * (int)g.M * 4);
+        dma4(db, dst + 1024, sc_voff, off_b + kstep * (int)g.N * 4);
+    };
+    int sca[2][4] = {}, scb[2][4] = {};           // [K step parity][fragment]: this lane's scale dwords, already shifted
+    auto read_scales = [&](int stage, int (&ea)[4], int (&eb)[4]) {
+        const uint32_t *base = sScale + stage * 512;
+        const v4i va = *reinterpret_cast<const v4i *>(base + 128 * (wave / 2) + 4 * lr);
+        const v4i vb = *reinterpret_cast<const v4i *>(base + 256 + 128 * (wave % 2) + 4 * lr);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            ea[t] = (int)((uint32_t)va[t] >> (8 * lg));
+            eb[t] = (int)((uint32_t)vb[t] >> (8 * lg));
+        }
+    };
+
+    // ---- LDS -> registers.  chunk(t, h, e) = ((2*lg + e) ^ s0) ^ 4*(h ^ (t & 1))   (block scales: lg + 2*e)
     int ra[2][2], rb[2][2];                     // [e][h ^ (t & 1)] byte offsets inside a region (tile 0)
     {
         const int rowa = wm0 + lr, rowb = wn0 + lr;
@@ -172,8 +236,11 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
         for (int e = 0; e < 2; ++e)
 #pragma unroll
             for (int p = 0; p < 2; ++p) {
-                ra[e][p] = rowa * 128 + (((((2 * lg + e) ^ s0a)) ^ (4 * p)) << 4);
-                rb[e][p] = rowb * 128 + (((((2 * lg + e) ^ s0b)) ^ (4 * p)) << 4);
+                // which 32 of the 64 K-bytes of a half a lane takes is free without block scales (both operands agree);
+                // with them the instruction's own order decides: registers 0..3 = chunk lg, registers 4..7 = chunk 2 + lg
+                const int chunk = MX ? lg + 2 * e : 2 * lg + e;
+                ra[e][p] = rowa * 128 + ((((chunk ^ s0a)) ^ (4 * p)) << 4);
+                rb[e][p] = rowb * 128 + ((((chunk ^ s0b)) ^ (4 * p)) << 4);
             }
     }
     // K-slow layout: fragment t covers tile rows row0 + 32 t .. + 31 = the 16-byte chunks c0 + 2t, c0 + 2t + 1
@@ -247,10 +314,10 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
 
     // phase A of a step: MFMA i works on sub-tile (t, u) = (i / 4, i % 4); the 8 fragments of
     // (kt, h1) stream into buffer 1 behind the first 8 MFMAs.
-    auto phase_a = [&](const uint8_t *sa_cur, const uint8_t *sb_cur) {
+    auto phase_a = [&](const uint8_t *sa_cur, const uint8_t *sb_cur, const int par) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            acc[i / 4][i % 4] = mfma_32x32x64<FB, FA>(b0[i % 4], a0[i / 4], acc[i / 4][i % 4]);
+            acc[i / 4][i % 4] = mma_step<FB, FA, MX, 0>(b0[i % 4], a0[i / 4], acc[i / 4][i % 4], scb[par][i % 4], sca[par][i / 4]);
             if (i < 4) a1[i] = read_a(sa_cur, i, 1);
             else if (i < 8) b1[i - 4] = read_b(sb_cur, i - 4, 1);
             __builtin_amdgcn_sched_barrier(0);
@@ -260,7 +327,7 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
     auto phase_a_first = [&](const uint8_t *sa_cur, const uint8_t *sb_cur) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            acc[i / 4][i % 4] = mfma_32x32x64<FB, FA>(b0[i % 4], a0[i / 4], zero16);
+            acc[i / 4][i % 4] = mma_step<FB, FA, MX, 0>(b0[i % 4], a0[i / 4], zero16, scb[0][i % 4], sca[0][i / 4]);
             if (i < 4) a1[i] = read_a(sa_cur, i, 1);
             else if (i < 8) b1[i - 4] = read_b(sb_cur, i - 4, 1);
             __builtin_amdgcn_sched_barrier(0);
@@ -320,7 +387,7 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
                     pk[2 * q + 1] = pack_bf16x2(v[4 * q + 2], v[4 * q + 3]);
                 }
             }
-            acc[t][u] = mfma_32x32x64<FB, FA>(b0[u], a0[t], zero16);
+            acc[t][u] = mma_step<FB, FA, MX, 0>(b0[u], a0[t], zero16, scb[0][u], sca[0][t]);
             if constexpr (EPI > 0) {
                 if (i < 15) read_vectors((i + 1) / 4, (i + 1) % 4);
             }
@@ -367,10 +434,6 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
             const uint64_t addr = reinterpret_cast<uint64_t>(p);
             return v4i{(int)(uint32_t)addr, (int)(uint32_t)(addr >> 32), (int)(count * 4), 0x00020000};
         };
-        auto dma4 = [](const v4i &rsrc, uint32_t lds_addr, int vo, int so) {
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tbuffer_load_dword %1, %2, %3 offen lds"
-                         ::"s"(lds_addr), "v"(vo), "s"(rsrc), "s"(so));
-        };
         // the bounds of a descriptor cover the per-lane offset only, not the scalar one: a wave outside the matrix
         // must not request its (non-existent) slices at all
         const bool inside = wave_inside(tm0, tn0);
@@ -397,7 +460,7 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
     };
     // phase B: MFMAs on buffer 1; (kt+1, h0) streams into buffer 0; step kt+2 is requested into
     // the stage just consumed -- from the next tile when this tile has no such step
-    auto phase_b = [&](uint8_t *sa_cur, uint8_t *sb_cur, const uint8_t *sa_nxt, const uint8_t *sb_nxt, int kt) {
+    auto phase_b = [&](uint8_t *sa_cur, uint8_t *sb_cur, const uint8_t *sa_nxt, const uint8_t *sb_nxt, int kt, const int par) {
         const bool nx = kt + 2 >= KT;
         const bool pad = padded && kt + 3 == KT;                  // the step requested is the padding step
         // (a nested select between three descriptors is not compiled as scalar code; the padding step
@@ -408,17 +471,27 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
         const int koff = nx ? kt + 2 - KT : kt + 2;               // K step to request
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            acc[i / 4][i % 4] = mfma_32x32x64<FB, FA>(b1[i % 4], a1[i / 4], acc[i / 4][i % 4]);
+            acc[i / 4][i % 4] = mma_step<FB, FA, MX, 1>(b1[i % 4], a1[i / 4], acc[i / 4][i % 4], scb[par][i % 4], sca[par][i / 4]);
             if (i < 4) a0[i] = read_a(sa_nxt, i, 0);
             else if (i < 8) b0[i - 4] = read_b(sb_nxt, i - 4, 0);
             issue_one(sa_cur, sb_cur, la, lb, koff, i);
+            if constexpr (MX) {
+                // the scales of step kt + 1 arrived with its operands; those of the step requested above go to the stage
+                // whose dwords every wave read one phase B ago
+                if (i == 8) read_scales(par ^ 1, sca[par ^ 1], scb[par ^ 1]);
+                if (i == 15) {
+                    const int live = pad && !nx ? 0 : 1;
+                    issue_scales(par, (nx ? sc_nin_a : sc_in_a) * live, (nx ? sc_nin_b : sc_in_b) * live,
+                                 nx ? sc_next_a : sc_off_a, nx ? sc_next_b : sc_off_b, koff);
+                }
+            }
             __builtin_amdgcn_sched_barrier(0);
         }
     };
-    auto step = [&](uint8_t *sa_cur, uint8_t *sb_cur, uint8_t *sa_nxt, uint8_t *sb_nxt, int kt) {
-        phase_a(sa_cur, sb_cur);
+    auto step = [&](uint8_t *sa_cur, uint8_t *sb_cur, uint8_t *sa_nxt, uint8_t *sb_nxt, int kt, const int par) {
+        phase_a(sa_cur, sb_cur, par);
         sync(false);
-        phase_b(sa_cur, sb_cur, sa_nxt, sb_nxt, kt);
+        phase_b(sa_cur, sb_cur, sa_nxt, sb_nxt, kt, par);
     };
 
     // ---- first tile: steps 0 and 1 requested and awaited, then phase A of step 0
@@ -428,6 +501,7 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
         item_steps(pid, first_step, KT, padded);
         rsrc_a = rsrc_for(g.a, m0, g.M, TA, first_step);
         rsrc_b = rsrc_for(g.b, n0, g.N, TB, first_step);
+        if constexpr (MX) scale_origin(m0, n0, first_step, sc_off_a, sc_off_b, sc_in_a, sc_in_b);
     }
     next_a = empty;
     next_b = empty;
@@ -435,10 +509,15 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
     for (int j = 0; j < 2 * LOADS; ++j) issue_one(sA0, sB0, rsrc_a, rsrc_b, 0, j);
 #pragma unroll
     for (int j = 0; j < 2 * LOADS; ++j) issue_one(sA1, sB1, rsrc_a, rsrc_b, 1, j);
+    if constexpr (MX) {
+        issue_scales(0, sc_in_a, sc_in_b, sc_off_a, sc_off_b, 0);
+        issue_scales(1, sc_in_a, sc_in_b, sc_off_a, sc_off_b, 1);
+    }
     __builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0)
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
+    if constexpr (MX) read_scales(0, sca[0], scb[0]);
 #pragma unroll
     for (int t = 0; t < TM; ++t) a0[t] = read_a(sA0, t, 0);
 #pragma unroll
@@ -456,20 +535,25 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
         const v4i na = rsrc_for(g.a, next_m0, g.M, TA, next_first), nb = rsrc_for(g.b, next_n0, g.N, TB, next_first);
         next_a = has_next ? na : empty;
         next_b = has_next ? nb : empty;
+        if constexpr (MX) {
+            scale_origin(next_m0, next_n0, next_first, sc_next_a, sc_next_b, sc_nin_a, sc_nin_b);
+            sc_nin_a *= has_next ? 1 : 0;
+            sc_nin_b *= has_next ? 1 : 0;
+        }
 
         // ---- rest of step 0 (its phase A ran at the end of the previous trip), then steps 1 .. KT-1.
         // The first trip's step 0 and every drained tile's step 0 carry 32 stores (dropped ones
         // count too), the first tile's none: vmcnt(32) is then simply satisfied earlier.
         sync(true);
-        phase_b(sA0, sB0, sA1, sB1, 0);
-        step(sA1, sB1, sA0, sB0, 1);
+        phase_b(sA0, sB0, sA1, sB1, 0, 0);
+        step(sA1, sB1, sA0, sB0, 1, 1);
         for (int kt = 2; kt < KT - 2; kt += 2) {
-            step(sA0, sB0, sA1, sB1, kt);
-            step(sA1, sB1, sA0, sB0, kt + 1);
+            step(sA0, sB0, sA1, sB1, kt, 0);
+            step(sA1, sB1, sA0, sB0, kt + 1, 1);
         }
-        step(sA0, sB0, sA1, sB1, KT - 2);
+        step(sA0, sB0, sA1, sB1, KT - 2, 0);
         if constexpr (EPI > 0) request_vectors(m0, n0);
-        step(sA1, sB1, sA0, sB0, KT - 1);
+        step(sA1, sB1, sA0, sB0, KT - 1, 1);
 
         // ---- the tile is finished; buffer 0 already holds the next tile's first fragments.
         // Phase A of the next tile's step 0 stores this tile.  Without a next tile the same
@@ -482,6 +566,10 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
         n0 = next_n0;
         rsrc_a = next_a;
         rsrc_b = next_b;
+        sc_off_a = sc_next_a;
+        sc_off_b = sc_next_b;
+        sc_in_a = sc_nin_a;
+        sc_in_b = sc_nin_b;
         phase_a_fold(sA0, sB0, rsrc_c);
         if (!has_next) break;
     }
@@ -495,7 +583,10 @@ template <int FA, int FB, bool F32>
 void launch_out(const GemmArgs &g, int blocks_per_xcd, hipStream_t stream) {
     const dim3 grid((unsigned)(8 * blocks_per_xcd)), block(256);
     const bool vectors = g.splits == 1 && (g.bias || g.sa_vec || g.sb_vec);     // partial results carry no scales
-    if (vectors && g.bias) hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB, false, false, F32, 2>), grid, block, 0, stream, g);
+    if (g.mx_sa) {
+        if (vectors) hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB, false, false, F32, 2, true>), grid, block, 0, stream, g);
+        else hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB, false, false, F32, 0, true>), grid, block, 0, stream, g);
+    } else if (vectors && g.bias) hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB, false, false, F32, 2>), grid, block, 0, stream, g);
     else if (vectors) hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB, false, false, F32, 1>), grid, block, 0, stream, g);
     else if (g.ta && g.tb) hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB, true, true, F32, 0>), grid, block, 0, stream, g);
     else if (g.tb) hipLaunchKernelGGL((gemm_nt_stream_kernel<FA, FB, false, true, F32, 0>), grid, block, 0, stream, g);
@@ -517,6 +608,7 @@ void launch_fmt(const GemmArgs &g, int blocks_per_xcd, hipStream_t stream) {
 bool gemm_stream_accepts(const GemmArgs &g) {
     const double esz = (g.out_dtype == ODL_F32 || g.splits > 1) ? 4.0 : 2.0;
     const bool vectors = g.splits == 1 && (g.sa_vec || g.sb_vec || g.bias != nullptr);   // only with both operands stored [rows, K]
+    if (g.mx_sa && (g.ta || g.tb || g.sa_vec || g.sb_vec || !g.mx_sb)) return false;
     return (g.out_dtype == ODL_BF16 || g.out_dtype == ODL_F32) && !(vectors && (g.ta || g.tb)) &&
            g.M % (g.ta ? BM : WM) == 0 && g.N % (g.tb ? BN : WN) == 0 && g.K % 128 == 0 && g.K >= 512 && (double)g.N * esz * (BM + 8) < 2147483648.0;
 }

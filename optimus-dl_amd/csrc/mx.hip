@@ -26,6 +26,13 @@ namespace odl {
 constexpr int kMxBlock = 32;
 constexpr int kMxThreads = 256;
 
+// Where the scale byte of (row, block) lives.  Row-major: [rows][blocks].  K-step-major: [blocks / 4][rows][4], i.e.
+// the 4 bytes a row needs for one 128-byte K step of a GEMM are one dword and the dwords of consecutive rows are
+// consecutive: what the GEMM kernels fetch per step is contiguous (blocks % 4 == 0).
+__device__ __forceinline__ int64_t mx_scale_at(int kstep_major, int64_t row, int64_t block, int64_t rows, int64_t blocks) {
+    return kstep_major ? ((block >> 2) * rows + row) * 4 + (block & 3) : row * blocks + block;
+}
+
 template <int FMT> struct MxEmax { static constexpr int value = FMT == ODL_FP8_E5M2 ? 15 : 8; };
 
 // magnitude bits (fp32 layout) of a block's amax -> scale byte and the multiplier 2^-shared
@@ -48,7 +55,8 @@ __device__ __forceinline__ void mx_scale_of(uint32_t amax_bits, uint32_t &byte, 
 template <int SRC, int FMT, bool WANT_ROW, bool WANT_COL>
 __global__ __launch_bounds__(kMxThreads) void mx_cast_kernel(const void *__restrict__ x, int64_t rows, int64_t cols,
                                                               uint8_t *__restrict__ out, uint8_t *__restrict__ scales,
-                                                              uint8_t *__restrict__ out_t, uint8_t *__restrict__ scales_t) {
+                                                              uint8_t *__restrict__ out_t, uint8_t *__restrict__ scales_t,
+                                                              int layout, int layout_t) {
     __shared__ __attribute__((aligned(16))) uint8_t tile[kTileC * kTileR];
     constexpr int ESZ = SRC == ODL_BF16 ? 2 : 4;
     const int tx = threadIdx.x % 8, ty = threadIdx.x / 8;
@@ -96,7 +104,7 @@ __global__ __launch_bounds__(kMxThreads) void mx_cast_kernel(const void *__restr
                 const uint32_t lo = quantise4<FMT>(f[i][0], f[i][1], f[i][2], f[i][3], mul, mul, mul, mul);
                 const uint32_t hi = quantise4<FMT>(f[i][4], f[i][5], f[i][6], f[i][7], mul, mul, mul, mul);
                 *reinterpret_cast<u32x2 *>(out + (r0 + i) * cols + c0) = u32x2{lo, hi};
-                if ((tx & 3) == 0) scales[(r0 + i) * nb + c0 / kMxBlock] = (uint8_t)byte;
+                if ((tx & 3) == 0) scales[mx_scale_at(layout, r0 + i, c0 / kMxBlock, rows, nb)] = (uint8_t)byte;
             }
         }
     }
@@ -114,7 +122,7 @@ __global__ __launch_bounds__(kMxThreads) void mx_cast_kernel(const void *__restr
             uint32_t byte;
             mx_scale_of<FMT>(m, byte, mul_c[j]);
             // rows % 32 == 0 (host-checked): a row block is inside the matrix as a whole or not at all
-            if ((ty & 7) == 0 && col_ok && r0 < rows) scales_t[(c0 + j) * nbt + r0 / kMxBlock] = (uint8_t)byte;
+            if ((ty & 7) == 0 && col_ok && r0 < rows) scales_t[mx_scale_at(layout_t, c0 + j, r0 / kMxBlock, cols, nbt)] = (uint8_t)byte;
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -149,7 +157,7 @@ __global__ __launch_bounds__(kMxThreads) void mx_cast_kernel(const void *__restr
 // barrier; a lane reads the dword of each of its rows and shifts it right by 8 bits when it sits in the upper half of the
 // wave, so that byte 0 / byte 2 are the scales it supplies in the first / second MFMA of the step (lanes 0..31: blocks 0
 // and 2 of the step, lanes 32..63: blocks 1 and 3).
-template <int BM, int BN, int WAVES_M, int WAVES_N, int FA, int FB>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int FA, int FB, bool KS>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mx_gemm_tiled_kernel(const GemmArgs g, const uint8_t *__restrict__ sa,
                                                                               const uint8_t *__restrict__ sb) {
     constexpr int NW = WAVES_M * WAVES_N, NT = NW * 64;
@@ -194,8 +202,11 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mx_gemm_tiled_kernel(co
         off_b[j] = (uint32_t)(gr * g.K + (((lane % 8) ^ swz(row)) << 4));
     }
     // the scale dwords this thread fetches: A row threadIdx.x, B row threadIdx.x (rows past the edge re-read the last row)
-    const uint32_t *sa_row = reinterpret_cast<const uint32_t *>(sa + min(m0 + (int64_t)threadIdx.x, g.M - 1) * nb);
-    const uint32_t *sb_row = reinterpret_cast<const uint32_t *>(sb + min(n0 + (int64_t)threadIdx.x, g.N - 1) * nb);
+    // (K-step-major: the dword of step kt is [kt][row]; row-major: dword kt of the row's nb bytes)
+    const int64_t row_a = min(m0 + (int64_t)threadIdx.x, g.M - 1), row_b = min(n0 + (int64_t)threadIdx.x, g.N - 1);
+    const uint32_t *sa_row = reinterpret_cast<const uint32_t *>(sa) + (KS ? row_a : row_a * (nb / 4));
+    const uint32_t *sb_row = reinterpret_cast<const uint32_t *>(sb) + (KS ? row_b : row_b * (nb / 4));
+    const int64_t step_a = KS ? g.M : 1, step_b = KS ? g.N : 1;
     uint32_t ra = 0, rb = 0;
     auto issue = [&](uint8_t *lds, int kt) {
         const uint8_t *ga = g.a + (int64_t)kt * 128, *gb = g.b + (int64_t)kt * 128;
@@ -207,8 +218,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mx_gemm_tiled_kernel(co
         for (int j = 0; j < LB; ++j)
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(gb + off_b[j]),
                                              (__attribute__((address_space(3))) void *)(lds + A_BYTES + (wave + j * NW) * 1024), 16, 0, 0);
-        if ((int)threadIdx.x < BM) ra = sa_row[kt];
-        if ((int)threadIdx.x < BN) rb = sb_row[kt];
+        if ((int)threadIdx.x < BM) ra = sa_row[kt * step_a];
+        if ((int)threadIdx.x < BN) rb = sb_row[kt * step_b];
     };
     auto park = [&](uint32_t *sc) {                // after vmcnt(0): this thread's two dwords into the stage's scale slots
         if ((int)threadIdx.x < BM) sc[threadIdx.x] = ra;
@@ -302,7 +313,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mx_gemm_tiled_kernel(co
 // One wave per 32 x 32 output tile, operands and scale bytes straight from global memory, 64 K-bytes per trip; a last
 // half trip (K % 64 == 32) feeds zeros as the second block.
 template <int FA, int FB>
-__global__ __launch_bounds__(64) void mx_gemm_generic_kernel(const GemmArgs g, const uint8_t *__restrict__ sa, const uint8_t *__restrict__ sb) {
+__global__ __launch_bounds__(64) void mx_gemm_generic_kernel(const GemmArgs g, const uint8_t *__restrict__ sa, const uint8_t *__restrict__ sb,
+                                                             int kstep_major) {
     const int lane = threadIdx.x, lr = lane % 32, lg = lane / 32;
     const int64_t m0 = (int64_t)blockIdx.y * 32, n0 = (int64_t)blockIdx.x * 32;
     const int64_t ra = min(m0 + lr, g.M - 1), rb = min(n0 + lr, g.N - 1), nb = g.K / kMxBlock;
@@ -316,7 +328,10 @@ __global__ __launch_bounds__(64) void mx_gemm_generic_kernel(const GemmArgs g, c
         const v4i a0 = pa[0], b0 = pb[0], a1 = second ? pa[2] : zero, b1 = second ? pb[2] : zero;
         const v8i af = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w}, bf = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
         int ea = 127, eb = 127;                                     // lanes 0..31: scale of block k / 32, lanes 32..63: of the next
-        if (lg == 0 || second) { ea = sa[ra * nb + k / kMxBlock + lg]; eb = sb[rb * nb + k / kMxBlock + lg]; }
+        if (lg == 0 || second) {
+            ea = sa[mx_scale_at(kstep_major, ra, k / kMxBlock + lg, g.M, nb)];
+            eb = sb[mx_scale_at(kstep_major, rb, k / kMxBlock + lg, g.N, nb)];
+        }
         acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf, af, acc, FB, FA, 0, eb, 0, ea);
     }
     if (g.out_dtype == ODL_BF16) store_tile<true, false>(g, acc, m0 + lr, n0 + 4 * lg);
@@ -350,32 +365,45 @@ static const float *unit_scale_for_current_device(const char *who) {
 
 template <int SRC, int FMT>
 static void launch_mx_cast(const void *x, int64_t rows, int64_t cols, uint8_t *out, uint8_t *scales, uint8_t *out_t, uint8_t *scales_t,
-                           hipStream_t stream) {
+                           int layout, int layout_t, hipStream_t stream) {
     const int64_t g = ((rows + kTileR - 1) / kTileR) * ((cols + kTileC - 1) / kTileC);
-#define ODL_MX(R, C) hipLaunchKernelGGL((mx_cast_kernel<SRC, FMT, R, C>), dim3((unsigned)g), dim3(kMxThreads), 0, stream, x, rows, cols, out, scales, out_t, scales_t)
+#define ODL_MX(R, C) hipLaunchKernelGGL((mx_cast_kernel<SRC, FMT, R, C>), dim3((unsigned)g), dim3(kMxThreads), 0, stream, x, rows, cols, out, scales, out_t, scales_t, layout, layout_t)
     if (out && out_t) ODL_MX(true, true);
     else if (out) ODL_MX(true, false);
     else ODL_MX(false, true);
 #undef ODL_MX
 }
 
-template <int FA, int FB>
-static void launch_mx_gemm(const GemmArgs &g, const uint8_t *sa, const uint8_t *sb, bool tiled, int cus, hipStream_t stream) {
-    if (!tiled) {
-        hipLaunchKernelGGL((mx_gemm_generic_kernel<FA, FB>), dim3((unsigned)((g.N + 31) / 32), (unsigned)((g.M + 31) / 32)), dim3(64), 0, stream, g, sa, sb);
-        return;
-    }
+template <int FA, int FB, bool KS>
+static void launch_mx_tiled(const GemmArgs &g, const uint8_t *sa, const uint8_t *sb, int cus, hipStream_t stream) {
     GemmArgs t = g;
     // 256 x 256 tiles (8 waves of 128 x 64) when they fill the chip, else 128 x 128 (two blocks per compute unit)
     const int64_t big = ((g.M + 255) / 256) * ((g.N + 255) / 256);
     if (big >= cus) {
         t.tiles_m = (int)((g.M + 255) / 256); t.tiles_n = (int)((g.N + 255) / 256);
         const unsigned grid = (unsigned)(((t.tiles_m * t.tiles_n + 7) / 8) * 8);
-        hipLaunchKernelGGL((mx_gemm_tiled_kernel<256, 256, 2, 4, FA, FB>), dim3(grid), dim3(512), 0, stream, t, sa, sb);
+        hipLaunchKernelGGL((mx_gemm_tiled_kernel<256, 256, 2, 4, FA, FB, KS>), dim3(grid), dim3(512), 0, stream, t, sa, sb);
     } else {
         t.tiles_m = (int)((g.M + 127) / 128); t.tiles_n = (int)((g.N + 127) / 128);
         const unsigned grid = (unsigned)(((t.tiles_m * t.tiles_n + 7) / 8) * 8);
-        hipLaunchKernelGGL((mx_gemm_tiled_kernel<128, 128, 2, 2, FA, FB>), dim3(grid), dim3(256), 0, stream, t, sa, sb);
+        hipLaunchKernelGGL((mx_gemm_tiled_kernel<128, 128, 2, 2, FA, FB, KS>), dim3(grid), dim3(256), 0, stream, t, sa, sb);
+    }
+}
+
+// kernel: 0 = one wave per 32 x 32 tile, 1 = LDS-tiled, 2 = the streaming kernel of gemm_stream.hip with block scales
+template <int FA, int FB>
+static void launch_mx_gemm(const GemmArgs &g, const uint8_t *sa, const uint8_t *sb, int kernel, int kstep_major, int cus, hipStream_t stream) {
+    if (kernel == 2) {
+        GemmArgs t = g;
+        t.mx_sa = sa; t.mx_sb = sb;
+        t.tiles_m = (int)((g.M + 255) / 256); t.tiles_n = (int)((g.N + 255) / 256);
+        launch_gemm_stream(FA, FB, t, cus, stream);
+    } else if (kernel == 1) {
+        if (kstep_major) launch_mx_tiled<FA, FB, true>(g, sa, sb, cus, stream);
+        else launch_mx_tiled<FA, FB, false>(g, sa, sb, cus, stream);
+    } else {
+        hipLaunchKernelGGL((mx_gemm_generic_kernel<FA, FB>), dim3((unsigned)((g.N + 31) / 32), (unsigned)((g.M + 31) / 32)), dim3(64), 0, stream, g, sa, sb,
+                           kstep_major);
     }
 }
 
@@ -384,7 +412,7 @@ static void launch_mx_gemm(const GemmArgs &g, const uint8_t *sa, const uint8_t *
 using namespace odl;
 
 extern "C" int odl_fp8_mx_cast(const void *x, int src_dtype, int64_t rows, int64_t cols, int fmt, uint8_t *out, uint8_t *scales,
-                               uint8_t *out_t, uint8_t *scales_t, odl_stream_t stream_) {
+                               int scales_layout, uint8_t *out_t, uint8_t *scales_t, int scales_t_layout, odl_stream_t stream_) {
     hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
     if (rows < 0 || cols < 0) return set_error(ODL_ERR_ARG, "odl_fp8_mx_cast: negative shape");
     if (src_dtype != ODL_BF16 && src_dtype != ODL_F32) return set_error(ODL_ERR_ARG, "odl_fp8_mx_cast: src_dtype %d", src_dtype);
@@ -393,6 +421,12 @@ extern "C" int odl_fp8_mx_cast(const void *x, int src_dtype, int64_t rows, int64
     if ((out == nullptr) != (scales == nullptr) || (out_t == nullptr) != (scales_t == nullptr))
         return set_error(ODL_ERR_ARG, "odl_fp8_mx_cast: codes and scale bytes of a layout go together");
     if (!out && !out_t) return set_error(ODL_ERR_ARG, "odl_fp8_mx_cast: neither layout asked for");
+    auto bad_layout = [](int l) { return l != ODL_MX_SCALES_ROWMAJOR && l != ODL_MX_SCALES_KSTEP; };
+    if ((out && bad_layout(scales_layout)) || (out_t && bad_layout(scales_t_layout)))
+        return set_error(ODL_ERR_ARG, "odl_fp8_mx_cast: scale layouts %d, %d", scales_layout, scales_t_layout);
+    if ((out && scales_layout == ODL_MX_SCALES_KSTEP && cols % 128 != 0) || (out_t && scales_t_layout == ODL_MX_SCALES_KSTEP && rows % 128 != 0))
+        return set_error(ODL_ERR_SHAPE, "odl_fp8_mx_cast: K-step-major scales need the blocked axis to be a multiple of 128 (%lld x %lld)",
+                         (long long)rows, (long long)cols);
     if (!x) return set_error(ODL_ERR_ARG, "odl_fp8_mx_cast: x is null");
     if (cols % 8 != 0 || (out && cols % kMxBlock != 0) || (out_t && rows % kMxBlock != 0))
         return set_error(ODL_ERR_SHAPE, "odl_fp8_mx_cast: %lld x %lld: the blocked axis must be a multiple of 32 (cols for out, rows for out_t) and cols of 8",
@@ -402,17 +436,17 @@ extern "C" int odl_fp8_mx_cast(const void *x, int src_dtype, int64_t rows, int64
     const int64_t tiles = ((rows + kTileR - 1) / kTileR) * ((cols + kTileC - 1) / kTileC);
     if (tiles > 0x7fffffffLL) return set_error(ODL_ERR_SHAPE, "odl_fp8_mx_cast: too many tiles for one launch");
     if (src_dtype == ODL_BF16) {
-        if (fmt == ODL_FP8_E4M3) launch_mx_cast<ODL_BF16, ODL_FP8_E4M3>(x, rows, cols, out, scales, out_t, scales_t, stream);
-        else launch_mx_cast<ODL_BF16, ODL_FP8_E5M2>(x, rows, cols, out, scales, out_t, scales_t, stream);
+        if (fmt == ODL_FP8_E4M3) launch_mx_cast<ODL_BF16, ODL_FP8_E4M3>(x, rows, cols, out, scales, out_t, scales_t, scales_layout, scales_t_layout, stream);
+        else launch_mx_cast<ODL_BF16, ODL_FP8_E5M2>(x, rows, cols, out, scales, out_t, scales_t, scales_layout, scales_t_layout, stream);
     } else {
-        if (fmt == ODL_FP8_E4M3) launch_mx_cast<ODL_F32, ODL_FP8_E4M3>(x, rows, cols, out, scales, out_t, scales_t, stream);
-        else launch_mx_cast<ODL_F32, ODL_FP8_E5M2>(x, rows, cols, out, scales, out_t, scales_t, stream);
+        if (fmt == ODL_FP8_E4M3) launch_mx_cast<ODL_F32, ODL_FP8_E4M3>(x, rows, cols, out, scales, out_t, scales_t, scales_layout, scales_t_layout, stream);
+        else launch_mx_cast<ODL_F32, ODL_FP8_E5M2>(x, rows, cols, out, scales, out_t, scales_t, scales_layout, scales_t_layout, stream);
     }
     return check_launch("odl_fp8_mx_cast");
 }
 
-extern "C" int odl_fp8_mx_gemm_nt(const uint8_t *a, const uint8_t *sa, const uint8_t *b, const uint8_t *sb, int64_t M, int64_t N, int64_t K,
-                                  int fmt_a, int fmt_b, const float *bias, void *c, int out_dtype, odl_stream_t stream_) {
+extern "C" int odl_fp8_mx_gemm_nt(const uint8_t *a, const uint8_t *sa, const uint8_t *b, const uint8_t *sb, int scales_layout, int64_t M,
+                                  int64_t N, int64_t K, int fmt_a, int fmt_b, const float *bias, void *c, int out_dtype, odl_stream_t stream_) {
     hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
     if (M < 0 || N < 0 || K < 0) return set_error(ODL_ERR_ARG, "odl_fp8_mx_gemm_nt: negative shape");
     if ((fmt_a != ODL_FP8_E4M3 && fmt_a != ODL_FP8_E5M2) || (fmt_b != ODL_FP8_E4M3 && fmt_b != ODL_FP8_E5M2))
@@ -421,6 +455,10 @@ extern "C" int odl_fp8_mx_gemm_nt(const uint8_t *a, const uint8_t *sa, const uin
     if (M == 0 || N == 0) return ODL_OK;
     if (!a || !sa || !b || !sb || !c) return set_error(ODL_ERR_ARG, "odl_fp8_mx_gemm_nt: null pointer");
     if (K == 0 || K % kMxBlock != 0) return set_error(ODL_ERR_SHAPE, "odl_fp8_mx_gemm_nt: K = %lld must be a positive multiple of 32", (long long)K);
+    if (scales_layout != ODL_MX_SCALES_ROWMAJOR && scales_layout != ODL_MX_SCALES_KSTEP)
+        return set_error(ODL_ERR_ARG, "odl_fp8_mx_gemm_nt: scales_layout %d", scales_layout);
+    const int ks = scales_layout == ODL_MX_SCALES_KSTEP;
+    if (ks && K % 128 != 0) return set_error(ODL_ERR_SHAPE, "odl_fp8_mx_gemm_nt: K-step-major scales need K %% 128 == 0 (K = %lld)", (long long)K);
     auto mis = [](const void *p, uintptr_t al) { return (reinterpret_cast<uintptr_t>(p) & (al - 1)) != 0; };
     if (mis(a, 16) || mis(b, 16) || mis(c, 16) || (bias && mis(bias, 16)))
         return set_error(ODL_ERR_SHAPE, "odl_fp8_mx_gemm_nt: operands, output and bias must be 16-byte aligned");
@@ -429,11 +467,16 @@ extern "C" int odl_fp8_mx_gemm_nt(const uint8_t *a, const uint8_t *sa, const uin
     GemmArgs g{};
     g.a = a; g.b = b; g.c = c; g.sa = one; g.sb = one; g.bias = bias;
     g.M = M; g.N = N; g.K = K; g.sa_vec = 0; g.sb_vec = 0; g.out_dtype = out_dtype;
-    // the tiled kernel addresses rows with 32-bit offsets and reads whole scale dwords (4 blocks = one 128-byte K step)
-    const bool tiled = K % 128 == 0 && !mis(sa, 4) && !mis(sb, 4) && (double)(M + 256) * (double)K < 2147483648.0 &&
-                       (double)(N + 256) * (double)K < 2147483648.0 && M >= 32 && N >= 32;
+    // the tiled and the streaming kernel address rows with 32-bit offsets and read whole scale dwords (4 blocks = one
+    // 128-byte K step); the streaming kernel wants the scales K-step-major and the shapes of gemm_stream_accepts
+    const bool lim32 = (double)(M + 256) * (double)K < 2147483648.0 && (double)(N + 256) * (double)K < 2147483648.0;
+    const bool tiled = K % 128 == 0 && !mis(sa, 4) && !mis(sb, 4) && lim32 && M >= 32 && N >= 32;
+    GemmArgs probe = g;
+    probe.mx_sa = sa; probe.mx_sb = sb;
     const int cus = device_cu_count();
-#define ODL_MXG(FA_, FB_) launch_mx_gemm<FA_, FB_>(g, sa, sb, tiled, cus, stream)
+    const bool stream_ok = ks && tiled && ((M + 255) / 256) * ((N + 255) / 256) >= cus / 2 && gemm_stream_accepts(probe);
+    const int kernel = stream_ok ? 2 : (tiled ? 1 : 0);
+#define ODL_MXG(FA_, FB_) launch_mx_gemm<FA_, FB_>(g, sa, sb, kernel, ks, cus, stream)
     if (fmt_a == ODL_FP8_E4M3 && fmt_b == ODL_FP8_E4M3) ODL_MXG(ODL_FP8_E4M3, ODL_FP8_E4M3);
     else if (fmt_a == ODL_FP8_E5M2 && fmt_b == ODL_FP8_E4M3) ODL_MXG(ODL_FP8_E5M2, ODL_FP8_E4M3);
     else if (fmt_a == ODL_FP8_E4M3 && fmt_b == ODL_FP8_E5M2) ODL_MXG(ODL_FP8_E4M3, ODL_FP8_E5M2);

@@ -139,8 +139,8 @@ def load() -> ctypes.CDLL:
         L.odl_fp8_gemm_variant_name.restype = ctypes.c_char_p
         L.odl_fp8_gemm_set_variant.argtypes = [i32]
         L.odl_fp8_gemm_set_clock_probe.argtypes = [vp, i32]
-        L.odl_fp8_mx_cast.argtypes = [vp, i32, i64, i64, i32, vp, vp, vp, vp, vp]
-        L.odl_fp8_mx_gemm_nt.argtypes = [vp, vp, vp, vp, i64, i64, i64, i32, i32, vp, vp, i32, vp]
+        L.odl_fp8_mx_cast.argtypes = [vp, i32, i64, i64, i32, vp, vp, i32, vp, vp, i32, vp]
+        L.odl_fp8_mx_gemm_nt.argtypes = [vp, vp, vp, vp, i32, i64, i64, i64, i32, i32, vp, vp, i32, vp]
         for name in EXPORTS:
             getattr(L, name)  # AttributeError here = the library does not match the header
         if L.odl_fp8_abi_version() != ABI_VERSION:
@@ -723,50 +723,80 @@ def gemm_nt(a: torch.Tensor, b: torch.Tensor, fmt_a: int, fmt_b: int, sa_inv: to
 
 
 MX_BLOCK = 32
+MX_ROWMAJOR, MX_KSTEP = 0, 1           # ODL_MX_SCALES_*
 
 
-def mx_cast(x: torch.Tensor, fmt: int, want_rowmajor: bool = True, want_transposed: bool = False):
-    """MXFP8 conversion of ``x`` [rows, cols] in one launch -> (codes [rows, cols], scales [rows, cols/32],
-    codes_t [cols, rows], scales_t [cols, rows/32]); the pair that was not asked for is (None, None).  Scales are E8M0
-    bytes, one per 32 elements along the last axis of the codes they belong to."""
+def _mx_scales(rows: int, length: int, layout: int | None, device) -> tuple[torch.Tensor, int]:
+    """An empty scale tensor for `rows` rows blocked along an axis of `length` elements.  Row-major: [rows, length/32].
+    K-step-major: [length/128, rows, 4] (what the streaming GEMM reads; the default whenever length % 128 == 0).  The
+    number of dimensions tells the GEMM wrapper which one it got."""
+    if layout is None:
+        layout = MX_KSTEP if length % 128 == 0 and length > 0 else MX_ROWMAJOR
+    if layout == MX_KSTEP:
+        if length % 128:
+            raise NativeError(f"mx_cast: K-step-major scales need the blocked axis ({length}) to be a multiple of 128")
+        return torch.empty((length // 128, rows, 4), dtype=torch.uint8, device=device), layout
+    return torch.empty((rows, length // MX_BLOCK), dtype=torch.uint8, device=device), layout
+
+
+def mx_scales_rowmajor(scales: torch.Tensor) -> torch.Tensor:
+    """Scale bytes as [rows, blocks], whichever layout they are stored in."""
+    if scales.dim() == 3:
+        return scales.permute(1, 0, 2).reshape(scales.shape[1], -1)
+    return scales
+
+
+def mx_cast(x: torch.Tensor, fmt: int, want_rowmajor: bool = True, want_transposed: bool = False, layout: int | None = None):
+    """MXFP8 conversion of ``x`` [rows, cols] in one launch -> (codes [rows, cols], their scales, codes_t [cols, rows],
+    their scales); the pair that was not asked for is (None, None).  Scales are E8M0 bytes, one per 32 elements along
+    the last axis of the codes they belong to, stored as ``_mx_scales`` describes (layout None: K-step-major where the
+    blocked axis allows it)."""
     x = _as_2d(x)
     rows, cols = x.shape
     if not (want_rowmajor or want_transposed):
         raise NativeError("mx_cast: neither layout asked for")
     dev = x.device
     out = sc = out_t = sc_t = None
+    lay = lay_t = MX_ROWMAJOR
     if want_rowmajor:
         out = torch.empty((rows, cols), dtype=torch.uint8, device=dev)
-        sc = torch.empty((rows, cols // MX_BLOCK), dtype=torch.uint8, device=dev)
+        sc, lay = _mx_scales(rows, cols, layout, dev)
     if want_transposed:
         out_t = torch.empty((cols, rows), dtype=torch.uint8, device=dev)
-        sc_t = torch.empty((cols, rows // MX_BLOCK), dtype=torch.uint8, device=dev)
+        sc_t, lay_t = _mx_scales(cols, rows, layout, dev)
     ptr = lambda t: t.data_ptr() if t is not None else None
-    _check(load().odl_fp8_mx_cast(x.data_ptr(), _src_dtype(x), rows, cols, fmt, ptr(out), ptr(sc), ptr(out_t), ptr(sc_t), _stream()),
-           "odl_fp8_mx_cast")
+    _check(load().odl_fp8_mx_cast(x.data_ptr(), _src_dtype(x), rows, cols, fmt, ptr(out), ptr(sc), lay, ptr(out_t), ptr(sc_t), lay_t,
+                                  _stream()), "odl_fp8_mx_cast")
     return out, sc, out_t, sc_t
 
 
 def mx_gemm_nt(a: torch.Tensor, sa: torch.Tensor, b: torch.Tensor, sb: torch.Tensor, fmt_a: int, fmt_b: int,
                bias: torch.Tensor | None = None, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
     """out[M,N] = sum over 32-blocks of 2^(sa-127) 2^(sb-127) (a_block . b_block) (+ bias); a [M,K], b [N,K] codes,
-    sa [M,K/32], sb [N,K/32] E8M0 bytes."""
+    sa, sb their E8M0 scale bytes as ``mx_cast`` returns them (both row-major [rows, K/32] or both K-step-major
+    [K/128, rows, 4])."""
     for t, what in ((a, "a"), (b, "b"), (sa, "sa"), (sb, "sb")):
-        if t.dtype != torch.uint8 or not t.is_cuda or not t.is_contiguous() or t.dim() != 2:
-            raise NativeError(f"mx_gemm_nt: {what} must be a dense 2-D uint8 device tensor")
+        if t.dtype != torch.uint8 or not t.is_cuda or not t.is_contiguous():
+            raise NativeError(f"mx_gemm_nt: {what} must be a dense uint8 device tensor")
+    if a.dim() != 2 or b.dim() != 2:
+        raise NativeError("mx_gemm_nt: operands must be 2-D")
     M, K = a.shape
     N, K2 = b.shape
     if K != K2:
         raise NativeError(f"mx_gemm_nt: contraction sizes differ ({K} vs {K2})")
-    if K % MX_BLOCK or tuple(sa.shape) != (M, K // MX_BLOCK) or tuple(sb.shape) != (N, K // MX_BLOCK):
-        raise NativeError(f"mx_gemm_nt: scales must be [M, K/32] and [N, K/32] with K % 32 == 0, got {tuple(sa.shape)}, {tuple(sb.shape)} for K = {K}")
+    if sa.dim() != sb.dim():
+        raise NativeError("mx_gemm_nt: the two scale tensors are stored in different layouts")
+    layout = MX_KSTEP if sa.dim() == 3 else MX_ROWMAJOR
+    want = (lambda rows: (K // 128, rows, 4)) if layout == MX_KSTEP else (lambda rows: (rows, K // MX_BLOCK))
+    if K % MX_BLOCK or (layout == MX_KSTEP and K % 128) or tuple(sa.shape) != want(M) or tuple(sb.shape) != want(N):
+        raise NativeError(f"mx_gemm_nt: scale shapes {tuple(sa.shape)}, {tuple(sb.shape)} do not fit M, N, K = {M}, {N}, {K}")
     if bias is not None:
         _f32_dev(bias, N, "mx_gemm_nt bias")
     odt = DT_BF16 if out_dtype == torch.bfloat16 else (DT_F32 if out_dtype == torch.float32 else None)
     if odt is None:
         raise NativeError(f"mx_gemm_nt: output dtype {out_dtype} is not supported (bf16 or fp32)")
     out = torch.empty((M, N), dtype=out_dtype, device=a.device)
-    _check(load().odl_fp8_mx_gemm_nt(a.data_ptr(), sa.data_ptr(), b.data_ptr(), sb.data_ptr(), M, N, K, fmt_a, fmt_b,
+    _check(load().odl_fp8_mx_gemm_nt(a.data_ptr(), sa.data_ptr(), b.data_ptr(), sb.data_ptr(), layout, M, N, K, fmt_a, fmt_b,
                                      bias.data_ptr() if bias is not None else None, out.data_ptr(), odt, _stream()),
            "odl_fp8_mx_gemm_nt")
     return out

@@ -44,12 +44,23 @@ def _mixed(shape, seed):
 CAST_SHAPES = [(32, 32), (128, 64), (64, 96), (160, 224), (256, 1024), (1024, 768), (96, 4096), (2016, 160)]
 
 
+def _kstep(scales: torch.Tensor) -> torch.Tensor:
+    """Row-major scale bytes [rows, blocks] -> the K-step-major layout [blocks / 4, rows, 4]."""
+    rows, blocks = scales.shape
+    return scales.reshape(rows, blocks // 4, 4).permute(1, 0, 2).contiguous()
+
+
 @pytest.mark.parametrize("shape", CAST_SHAPES)
 @pytest.mark.parametrize("fmt", [E4M3, E5M2])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_mx_cast_both_layouts_bit_exact(N, shape, fmt, dtype):
     x = _mixed(shape, seed=shape[0] * 7 + shape[1] + fmt)
     out, sc, out_t, sc_t = N.mx_cast(x.to(dtype).cuda(), fmt, want_rowmajor=True, want_transposed=True)
+    # by default the scales are K-step-major wherever the blocked axis is a multiple of 128
+    assert sc.dim() == (3 if shape[1] % 128 == 0 else 2) and sc_t.dim() == (3 if shape[0] % 128 == 0 else 2)
+    if sc.dim() == 3:
+        assert_bytes_equal(sc, _kstep(O.c_mx_quantise(x, fmt)[1]), f"K-step-major scale bytes {shape}")
+    sc, sc_t = N.mx_scales_rowmajor(sc), N.mx_scales_rowmajor(sc_t)
     wc, ws = O.c_mx_quantise(x, fmt)
     assert_bytes_equal(sc, ws, f"scale bytes {shape} fmt {fmt}")
     assert_bytes_equal(out, wc, f"codes {shape} fmt {fmt}")
@@ -65,6 +76,12 @@ def test_mx_cast_both_layouts_bit_exact(N, shape, fmt, dtype):
 def test_mx_cast_single_layouts_match_the_pair(N, fmt):
     x = _mixed((384, 320), seed=5).cuda()
     out, sc, out_t, sc_t = N.mx_cast(x, fmt, True, True)
+    # the same bytes in the other storage order when the row-major layout is asked for explicitly
+    r = N.mx_cast(x, fmt, True, True, layout=N.MX_ROWMAJOR)
+    assert r[1].dim() == 2 and r[3].dim() == 2
+    assert_bytes_equal(r[1], N.mx_scales_rowmajor(sc), "explicit row-major scales")
+    assert_bytes_equal(r[3], N.mx_scales_rowmajor(sc_t), "explicit row-major transposed scales")
+    assert_bytes_equal(r[0], out, "codes do not depend on the scale layout")
     o1, s1, n1, n2 = N.mx_cast(x, fmt, True, False)
     assert n1 is None and n2 is None
     assert_bytes_equal(o1, out, "row-major only: codes")
@@ -93,6 +110,7 @@ def test_mx_cast_specials(N):
     x[40, 5] = -float("inf")
     for fmt in (E4M3, E5M2):
         out, sc, out_t, sc_t = N.mx_cast(x.cuda(), fmt, True, True)
+        sc, sc_t = N.mx_scales_rowmajor(sc), N.mx_scales_rowmajor(sc_t)
         wc, ws = O.c_mx_quantise(x, fmt)
         assert_bytes_equal(sc, ws, f"special scale bytes fmt {fmt}")
         assert_bytes_equal(out, wc, f"special codes fmt {fmt}")
@@ -107,6 +125,8 @@ def test_mx_cast_rejects_bad_shapes(N):
         N.mx_cast(torch.zeros((32, 48), dtype=torch.bfloat16, device="cuda"), E4M3, True, False)
     with pytest.raises(N.NativeError, match="multiple of 32"):
         N.mx_cast(torch.zeros((48, 64), dtype=torch.bfloat16, device="cuda"), E4M3, False, True)
+    with pytest.raises(N.NativeError, match="multiple of 128"):
+        N.mx_cast(torch.zeros((64, 64), dtype=torch.bfloat16, device="cuda"), E4M3, True, False, layout=N.MX_KSTEP)
     out = N.mx_cast(torch.zeros((0, 64), dtype=torch.bfloat16, device="cuda"), E4M3, True, True)
     assert out[0].shape == (0, 64) and out[2].shape == (64, 0)
 
@@ -141,6 +161,7 @@ GEMM_SHAPES = [
     (32, 32, 32), (32, 32, 96), (64, 96, 160), (100, 72, 224), (7, 13, 64),            # plain kernel (K % 128 != 0 or tiny)
     (128, 128, 128), (256, 256, 512), (384, 640, 1024), (200, 136, 256), (130, 70, 384),  # 128 x 128 tiles, edges
     (4096, 4096, 256), (4100, 4232, 128),                                                # 256 x 256 tiles, interior and edges
+    (4096, 4096, 512), (4224, 4480, 640), (3968, 4352, 1152),      # K-step-major: the streaming kernel, also with half tiles at the edges and an odd number of K steps
 ]
 
 
@@ -148,18 +169,20 @@ GEMM_SHAPES = [
 @pytest.mark.parametrize("fmts", [(E4M3, E4M3), (E5M2, E4M3), (E4M3, E5M2)])
 def test_mx_gemm_matches_emulation(N, shape, fmts):
     M, N_, K = shape
-    if M * N_ > 4096 * 1024 and fmts != (E4M3, E4M3):
-        pytest.skip("large shapes once")
+    if M * N_ > 4096 * 1024 and fmts != (E4M3, E4M3) and (shape != (4224, 4480, 640) or fmts != (E5M2, E4M3)):
+        pytest.skip("large shapes once (one of them also with E5M2 gradients)")
     fa, fb = fmts
     ac, asc, bc, bsc = _operands(M, N_, K, fa, fb, seed=M + N_ + K)
     ref_bf16, ref_f32 = O.t_mx_gemm_nt(ac, asc, bc, bsc, fa, fb, want_f32=True)
-    got32 = N.mx_gemm_nt(ac.cuda(), asc.cuda(), bc.cuda(), bsc.cuda(), fa, fb, out_dtype=torch.float32).cpu()
-    assert got32.shape == (M, N_)
-    _assert_within_hardware_sum(got32, ac, asc, bc, bsc, fa, fb)
-    got = N.mx_gemm_nt(ac.cuda(), asc.cuda(), bc.cuda(), bsc.cuda(), fa, fb).cpu()
-    assert max_rel_err(got.float(), ref_bf16.float()) <= 1e-2
-    # one rounding of the fp32 result: the bf16 output is the fp32 output rounded
-    assert torch.equal(got, got32.bfloat16())
+    # every scale layout the shape allows: row-major always, K-step-major when K is a multiple of 128
+    for kstep in ((False, True) if K % 128 == 0 else (False,)):
+        sa_d, sb_d = (_kstep(asc).cuda(), _kstep(bsc).cuda()) if kstep else (asc.cuda(), bsc.cuda())
+        got32 = N.mx_gemm_nt(ac.cuda(), sa_d, bc.cuda(), sb_d, fa, fb, out_dtype=torch.float32).cpu()
+        assert got32.shape == (M, N_)
+        _assert_within_hardware_sum(got32, ac, asc, bc, bsc, fa, fb)
+        got = N.mx_gemm_nt(ac.cuda(), sa_d, bc.cuda(), sb_d, fa, fb).cpu()
+        assert max_rel_err(got.float(), ref_bf16.float()) <= 1e-2
+        assert torch.equal(got, got32.bfloat16())
 
 
 def test_mx_gemm_small_case_against_the_c_oracle_and_bias(N):
@@ -177,6 +200,26 @@ def test_mx_gemm_small_case_against_the_c_oracle_and_bias(N):
     _assert_within_hardware_sum(got, ac, asc, bc, bsc, E4M3, E4M3, bias)
     gotb = N.mx_gemm_nt(ac.cuda(), asc.cuda(), bc.cuda(), bsc.cuda(), E4M3, E4M3, bias=bias.cuda()).cpu()
     assert torch.equal(gotb, got.bfloat16())
+
+
+def test_mx_gemm_streaming_kernel_with_bias_and_repeated_launches(N):
+    """K-step-major scales at a shape the streaming kernel takes: bias, fp32 and bf16 outputs, and the same launch three
+    times (a persistent kernel that leaves LDS or descriptors in a bad state shows on the second one)."""
+    M, N_, K = 4096, 4096, 768
+    ac, asc, bc, bsc = _operands(M, N_, K, E5M2, E4M3, seed=17)
+    bias = torch.randn(N_)
+    dev = [t.cuda() for t in (ac, _kstep(asc), bc, _kstep(bsc))]
+    first = None
+    for _ in range(3):
+        got = N.mx_gemm_nt(dev[0], dev[1], dev[2], dev[3], E5M2, E4M3, bias=bias.cuda(), out_dtype=torch.float32)
+        first = got if first is None else first
+        assert torch.equal(got, first)
+    _assert_within_hardware_sum(first.cpu(), ac, asc, bc, bsc, E5M2, E4M3, bias)
+    gotb = N.mx_gemm_nt(dev[0], dev[1], dev[2], dev[3], E5M2, E4M3, bias=bias.cuda())
+    assert torch.equal(gotb, first.bfloat16())
+    # and the row-major route (LDS-tiled kernel) sums the same blocks in another order: close, not equal
+    rm = N.mx_gemm_nt(dev[0], asc.cuda(), dev[2], bsc.cuda(), E5M2, E4M3, bias=bias.cuda(), out_dtype=torch.float32)
+    assert max_rel_err(rm.cpu(), first.cpu()) <= 1e-3
 
 
 def test_mx_gemm_block_scales_act_per_block(N):
@@ -205,6 +248,7 @@ def test_mx_round_trip_error_bound_at_full_size(N):
     rows, cols = 4096, 4096
     x = seeded_bf16((rows, cols), std=1.0, seed=21)
     out, sc, out_t, sc_t = N.mx_cast(x.cuda(), E4M3, True, True)
+    sc, sc_t = N.mx_scales_rowmajor(sc), N.mx_scales_rowmajor(sc_t)
     deq = O.t_mx_dequantise(out.cpu(), sc.cpu(), E4M3)
     v = x.float().reshape(rows, cols // 32, 32)
     amax = v.abs().amax(dim=2, keepdim=True)
