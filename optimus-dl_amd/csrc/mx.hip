@@ -49,6 +49,36 @@ __device__ __forceinline__ void mx_scale_of(uint32_t amax_bits, uint32_t &byte, 
     mul = bits_to_float((uint32_t)(127 - se) << 23);                       // 2^-se, 127 - se in [8, 254]
 }
 
+// Maxima across lanes without the LDS crossbar: DPP inside a row of 16 lanes, and the two swap instructions of gfx950
+// (v_permlane16_swap exchanges the odd rows of one register with the even rows of another, v_permlane32_swap the wave's
+// halves: applied to two copies of a value they leave "mine" in one and "my partner's" in the other).
+template <int CTRL>
+__device__ __forceinline__ uint32_t max_with_dpp(uint32_t m) {
+    return max(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, CTRL, 0xf, 0xf, false));
+}
+// over the 4 lanes l ^ {0, 1, 2, 3}
+__device__ __forceinline__ uint32_t max_quad(uint32_t m) {
+    m = max_with_dpp<0xB1>(m);            // quad_perm [1, 0, 3, 2]
+    return max_with_dpp<0x4E>(m);         // quad_perm [2, 3, 0, 1]
+}
+// over the 8 lanes l ^ {0, 8, 16, 24, 32, 40, 48, 56}
+__device__ __forceinline__ uint32_t max_stride8(uint32_t m) {
+    m = max_with_dpp<0x128>(m);           // row_ror:8 = lane ^ 8 inside a row of 16
+    const auto r = __builtin_amdgcn_permlane16_swap(m, m, false, false);
+    m = max(r[0], r[1]);
+    const auto q = __builtin_amdgcn_permlane32_swap(m, m, false, false);
+    return max(q[0], q[1]);
+}
+
+// the same for a pair of 16-bit magnitudes per lane
+__device__ __forceinline__ uint32_t max_stride8_u16x2(uint32_t m) {
+    m = max_u16x2(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x128, 0xf, 0xf, false));
+    const auto r = __builtin_amdgcn_permlane16_swap(m, m, false, false);
+    m = max_u16x2(r[0], r[1]);
+    const auto q = __builtin_amdgcn_permlane32_swap(m, m, false, false);
+    return max_u16x2(q[0], q[1]);
+}
+
 // 128 x 64 tile per block of 256 lanes, lane (tx, ty) owns rows 4 ty .. 4 ty + 3 and columns 8 tx .. 8 tx + 7 as in
 // cast_transpose_kernel.  A block along the columns (32 of them) is held by 4 neighbouring lanes; a block along the rows
 // (32 of them) by the 8 lanes of a wave that share tx: both maxima are xor-shuffles inside the wave.
@@ -66,43 +96,49 @@ __global__ __launch_bounds__(kMxThreads) void mx_cast_kernel(const void *__restr
     const int64_t r0 = tr * kTileR + ty * 4, c0 = tc * kTileC + tx * 8;
     const bool col_ok = c0 < cols;                 // cols % 8 == 0 (host-checked)
 
-    float f[4][8];
-    uint32_t mag[4][8];
+    // The patch stays in registers as loaded (bf16: 4 dwords a row) and is widened row by row where it is used; magnitudes
+    // of bf16 pairs are compared as packed 16-bit integers, two columns at a time.
+    constexpr int DW = SRC == ODL_BF16 ? 4 : 8;
+    uint32_t raw[4][DW];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const bool ok = col_ok && (r0 + i) < rows;
         const u32x4 *p = reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(x) + ((r0 + i) * cols + c0) * ESZ);
-        u32x4 raw[ESZ / 2];
 #pragma unroll
-        for (int h = 0; h < ESZ / 2; ++h) raw[h] = ok ? __builtin_nontemporal_load(p + h) : u32x4{0, 0, 0, 0};
-        if constexpr (SRC == ODL_BF16) {
-            const uint32_t w[4] = {raw[0].x, raw[0].y, raw[0].z, raw[0].w};
-#pragma unroll
-            for (int q = 0; q < 4; ++q) { f[i][2 * q] = bf16_lo(w[q]); f[i][2 * q + 1] = bf16_hi(w[q]); }
-        } else {
-            const uint32_t w[8] = {raw[0].x, raw[0].y, raw[0].z, raw[0].w, raw[1].x, raw[1].y, raw[1].z, raw[1].w};
-#pragma unroll
-            for (int q = 0; q < 8; ++q) f[i][q] = bits_to_float(w[q]);
+        for (int h = 0; h < DW / 4; ++h) {
+            const u32x4 v = ok ? __builtin_nontemporal_load(p + h) : u32x4{0, 0, 0, 0};
+            raw[i][4 * h] = v.x; raw[i][4 * h + 1] = v.y; raw[i][4 * h + 2] = v.z; raw[i][4 * h + 3] = v.w;
         }
-#pragma unroll
-        for (int j = 0; j < 8; ++j) mag[i][j] = float_to_bits(f[i][j]) & 0x7fffffffu;
     }
+    auto widen = [&](int i, float (&f)[8]) {
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+            if constexpr (SRC == ODL_BF16) f[q] = (q & 1) ? bf16_hi(raw[i][q / 2]) : bf16_lo(raw[i][q / 2]);
+            else f[q] = bits_to_float(raw[i][q]);
+        }
+    };
 
     if constexpr (WANT_ROW) {
         const int64_t nb = cols / kMxBlock;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             uint32_t m = 0;
+            if constexpr (SRC == ODL_BF16) {
+                uint32_t m2 = max_u16x2(max_u16x2(abs_bf16x2(raw[i][0]), abs_bf16x2(raw[i][1])), max_u16x2(abs_bf16x2(raw[i][2]), abs_bf16x2(raw[i][3])));
+                m = fold_u16x2_to_f32bits(m2);
+            } else {
 #pragma unroll
-            for (int j = 0; j < 8; ++j) m = max(m, mag[i][j]);
-            m = max(m, (uint32_t)__shfl_xor((int)m, 1, kWave));
-            m = max(m, (uint32_t)__shfl_xor((int)m, 2, kWave));          // the 4 lanes tx = 4 b .. 4 b + 3 hold the block
+                for (int j = 0; j < 8; ++j) m = max(m, raw[i][j] & 0x7fffffffu);
+            }
+            m = max_quad(m);                                             // the 4 lanes tx = 4 b .. 4 b + 3 hold the block
             uint32_t byte;
             float mul;
             mx_scale_of<FMT>(m, byte, mul);
             if (col_ok && (r0 + i) < rows) {
-                const uint32_t lo = quantise4<FMT>(f[i][0], f[i][1], f[i][2], f[i][3], mul, mul, mul, mul);
-                const uint32_t hi = quantise4<FMT>(f[i][4], f[i][5], f[i][6], f[i][7], mul, mul, mul, mul);
+                float f[8];
+                widen(i, f);
+                const uint32_t lo = quantise4<FMT>(f[0], f[1], f[2], f[3], mul, mul, mul, mul);
+                const uint32_t hi = quantise4<FMT>(f[4], f[5], f[6], f[7], mul, mul, mul, mul);
                 *reinterpret_cast<u32x2 *>(out + (r0 + i) * cols + c0) = u32x2{lo, hi};
                 if ((tx & 3) == 0) scales[mx_scale_at(layout, r0 + i, c0 / kMxBlock, rows, nb)] = (uint8_t)byte;
             }
@@ -113,21 +149,33 @@ __global__ __launch_bounds__(kMxThreads) void mx_cast_kernel(const void *__restr
         const int64_t nbt = rows / kMxBlock;
         uint32_t lo[4] = {0, 0, 0, 0}, hi[4] = {0, 0, 0, 0};
         float mul_c[8];
+        uint32_t cmax[8];                                                // fp32 magnitude bits per column, over the 32 rows
+        if constexpr (SRC == ODL_BF16) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                uint32_t m2 = max_u16x2(max_u16x2(abs_bf16x2(raw[0][q]), abs_bf16x2(raw[1][q])), max_u16x2(abs_bf16x2(raw[2][q]), abs_bf16x2(raw[3][q])));
+                m2 = max_stride8_u16x2(m2);                              // the 8 lanes of the wave with this tx: 32 rows
+                cmax[2 * q] = m2 << 16;
+                cmax[2 * q + 1] = m2 & 0xffff0000u;
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                cmax[j] = max_stride8(max(max(raw[0][j] & 0x7fffffffu, raw[1][j] & 0x7fffffffu), max(raw[2][j] & 0x7fffffffu, raw[3][j] & 0x7fffffffu)));
+        }
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            uint32_t m = max(max(mag[0][j], mag[1][j]), max(mag[2][j], mag[3][j]));
-            m = max(m, (uint32_t)__shfl_xor((int)m, 8, kWave));
-            m = max(m, (uint32_t)__shfl_xor((int)m, 16, kWave));
-            m = max(m, (uint32_t)__shfl_xor((int)m, 32, kWave));         // the 8 lanes of the wave with this tx: 32 rows
             uint32_t byte;
-            mx_scale_of<FMT>(m, byte, mul_c[j]);
+            mx_scale_of<FMT>(cmax[j], byte, mul_c[j]);
             // rows % 32 == 0 (host-checked): a row block is inside the matrix as a whole or not at all
             if ((ty & 7) == 0 && col_ok && r0 < rows) scales_t[mx_scale_at(layout_t, c0 + j, r0 / kMxBlock, cols, nbt)] = (uint8_t)byte;
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            lo[i] = quantise4<FMT>(f[i][0], f[i][1], f[i][2], f[i][3], mul_c[0], mul_c[1], mul_c[2], mul_c[3]);
-            hi[i] = quantise4<FMT>(f[i][4], f[i][5], f[i][6], f[i][7], mul_c[4], mul_c[5], mul_c[6], mul_c[7]);
+            float f[8];
+            widen(i, f);
+            lo[i] = quantise4<FMT>(f[0], f[1], f[2], f[3], mul_c[0], mul_c[1], mul_c[2], mul_c[3]);
+            hi[i] = quantise4<FMT>(f[4], f[5], f[6], f[7], mul_c[4], mul_c[5], mul_c[6], mul_c[7]);
         }
         uint32_t tl[4], th[4];
         transpose4x4(lo, tl);
