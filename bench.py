@@ -433,6 +433,7 @@ def clock_probe(torch, native, launches=20, settle=40):
     lib = ctypes.CDLL(PROBE_LIB_PATH)                      # built in-tree by optimus_dl_amd.build.build_probe()
     vp = ctypes.c_void_p
     lib.odl_probe_mfma_loop.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, vp, vp]
+    lib.odl_probe_mfma_loop_scaled.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, vp, vp]
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     flop_per_clock = cus * 8192.0                          # dense FP8 MFMA: 4 SIMDs x (2 x 32 x 32 x 64 flop / 64 clocks) per CU
 
@@ -469,16 +470,37 @@ def clock_probe(torch, native, launches=20, settle=40):
         entry = priced(2.0 * M * N * K / (us * 1e-6) / 1e12, mhz)
         entry["us_per_launch"] = round(us, 1)
         out["gemm_8192x14336x4096"][label] = entry
+    # the same product under MXFP8 (block scales applied by the MFMA, scale dwords fetched beside the operands)
+    xm, xs, _, _ = native.mx_cast(x, native.E4M3)
+    wm, ws, _, _ = native.mx_cast(w, native.E4M3)
+    for _ in range(settle):
+        native.mx_gemm_nt(xm, xs, wm, ws, native.E4M3, native.E4M3)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    native.gemm_set_clock_probe(records)
+    e0.record()
+    for _ in range(launches):
+        native.mx_gemm_nt(xm, xs, wm, ws, native.E4M3, native.E4M3)
+    e1.record()
+    native.gemm_set_clock_probe(None)
+    torch.cuda.synchronize()
+    r = records.double()
+    mhz = float((100.0 * (r[:, 2] - r[:, 0]) / (r[:, 3] - r[:, 1])).mean())
+    us = 1e3 * e0.elapsed_time(e1) / launches
+    entry = priced(2.0 * M * N * K / (us * 1e-6) / 1e12, mhz)
+    entry["us_per_launch"] = round(us, 1)
+    out["gemm_8192x14336x4096"]["mxfp8_gaussian_operands"] = entry
+    del xm, xs, wm, ws
     sink = torch.zeros(1, device="cuda")
     cycles = torch.zeros((cus, 2), dtype=torch.int64, device="cuda")
     iters = 4000                                           # x 16 MFMAs x 64 clocks: about 2 ms per launch
-    for label, rnd in (("gaussian_like_operands", 1), ("zero_operands", 0)):
+    for label, rnd, loop in (("gaussian_like_operands", 1, lib.odl_probe_mfma_loop), ("zero_operands", 0, lib.odl_probe_mfma_loop),
+                             ("block_scaled_gaussian_like_operands", 1, lib.odl_probe_mfma_loop_scaled)):
         for _ in range(settle // 4):
-            lib.odl_probe_mfma_loop(rnd, iters, cus, sink.data_ptr(), cycles.data_ptr(), stream())
+            loop(rnd, iters, cus, sink.data_ptr(), cycles.data_ptr(), stream())
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         for _ in range(4):
-            lib.odl_probe_mfma_loop(rnd, iters, cus, sink.data_ptr(), cycles.data_ptr(), stream())
+            loop(rnd, iters, cus, sink.data_ptr(), cycles.data_ptr(), stream())
         e1.record()
         torch.cuda.synchronize()
         us = 1e3 * e0.elapsed_time(e1) / 4

@@ -164,5 +164,7 @@ void launch_gemm_tiled(int variant, int fa, int fb, const GemmArgs &g, hipStream
 void launch_gemm_pipe(int fa, int fb, const GemmArgs &g, int num_cus, hipStream_t stream);
 bool gemm_stream_accepts(const GemmArgs &g);
 void launch_gemm_stream(int fa, int fb, const GemmArgs &g, int num_cus, hipStream_t stream);
+// gemm_fp8.hip: hands the calling thread's clock-probe record (odl_fp8_gemm_set_clock_probe), if any, to a streaming launch
+void attach_clock_probe(GemmArgs &g);
 
 }  // namespace odl

@@ -144,7 +144,7 @@ extern "C" const char *odl_fp8_gemm_variant_name(int variant) {
     return (variant >= 0 && variant < kNumVariants) ? kVariants[variant].name : "";
 }
 
-static void attach_clock_probe(GemmArgs &g) {
+void odl::attach_clock_probe(GemmArgs &g) {
     if (!t_clock_probe) return;
     g.clock_out = t_clock_probe + 4 * (size_t)(t_clock_next % t_clock_capacity);
     ++t_clock_next;

@@ -216,15 +216,23 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
         dma4(db, dst + 1024, sc_voff, off_b + kstep * (int)g.N * 4);
     };
     int sca[2][4] = {}, scb[2][4] = {};           // [K step parity][fragment]: this lane's scale dwords, already shifted
-    auto read_scales = [&](int stage, int (&ea)[4], int (&eb)[4]) {
+    // in two parts, so that the shift (which waits for the data) can sit a few MFMAs after the read
+    v4i sc_raw_a = {0, 0, 0, 0}, sc_raw_b = {0, 0, 0, 0};
+    auto fetch_scales = [&](int stage) {
         const uint32_t *base = sScale + stage * 512;
-        const v4i va = *reinterpret_cast<const v4i *>(base + 128 * (wave / 2) + 4 * lr);
-        const v4i vb = *reinterpret_cast<const v4i *>(base + 256 + 128 * (wave % 2) + 4 * lr);
+        sc_raw_a = *reinterpret_cast<const v4i *>(base + 128 * (wave / 2) + 4 * lr);
+        sc_raw_b = *reinterpret_cast<const v4i *>(base + 256 + 128 * (wave % 2) + 4 * lr);
+    };
+    auto place_scales = [&](int (&ea)[4], int (&eb)[4]) {
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-            ea[t] = (int)((uint32_t)va[t] >> (8 * lg));
-            eb[t] = (int)((uint32_t)vb[t] >> (8 * lg));
+            ea[t] = (int)((uint32_t)sc_raw_a[t] >> (8 * lg));
+            eb[t] = (int)((uint32_t)sc_raw_b[t] >> (8 * lg));
         }
+    };
+    auto read_scales = [&](int stage, int (&ea)[4], int (&eb)[4]) {
+        fetch_scales(stage);
+        place_scales(ea, eb);
     };
 
     // ---- LDS -> registers.  chunk(t, h, e) = ((2*lg + e) ^ s0) ^ 4*(h ^ (t & 1))   (block scales: lg + 2*e)
@@ -478,7 +486,8 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
             if constexpr (MX) {
                 // the scales of step kt + 1 arrived with its operands; those of the step requested above go to the stage
                 // whose dwords every wave read one phase B ago
-                if (i == 8) read_scales(par ^ 1, sca[par ^ 1], scb[par ^ 1]);
+                if (i == 8) fetch_scales(par ^ 1);
+                if (i == 13) place_scales(sca[par ^ 1], scb[par ^ 1]);
                 if (i == 15) {
                     const int live = pad && !nx ? 0 : 1;
                     issue_scales(par, (nx ? sc_nin_a : sc_in_a) * live, (nx ? sc_nin_b : sc_in_b) * live,

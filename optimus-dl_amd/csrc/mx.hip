@@ -445,6 +445,7 @@ static void launch_mx_gemm(const GemmArgs &g, const uint8_t *sa, const uint8_t *
         GemmArgs t = g;
         t.mx_sa = sa; t.mx_sb = sb;
         t.tiles_m = (int)((g.M + 255) / 256); t.tiles_n = (int)((g.N + 255) / 256);
+        attach_clock_probe(t);
         launch_gemm_stream(FA, FB, t, cus, stream);
     } else if (kernel == 1) {
         if (kstep_major) launch_mx_tiled<FA, FB, true>(g, sa, sb, cus, stream);

@@ -4,6 +4,7 @@
 //                           SIMD, nothing but registers) issued back to back, with operands that are all zero or
 //                           spread like quantised Gaussian data: the matrix pipe's rate with no memory system behind
 //                           it, and how it depends on what the operands hold.
+//   odl_probe_mfma_loop_scaled : the same with the block-scaled form of the instruction (MXFP8).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -29,8 +30,12 @@ __device__ __forceinline__ uint32_t gaussian_like_codes(uint32_t seed) {
     return w;
 }
 
+// SCALED: the block-scaled form of the instruction (an E8M0 scale byte per lane and operand, as the MXFP8 GEMM issues it)
+template <bool SCALED>
 __global__ __launch_bounds__(256) void mfma_loop_kernel(int random_operands, int iters, float *sink, uint64_t *cycles) {
     using namespace odl;
+    // scale bytes 119 .. 134 (2^-8 .. 2^7) when the operands are random, 127 (1.0) otherwise
+    const int sc = random_operands ? (int)(119u + (mix(blockIdx.x * 256 + threadIdx.x) & 15u)) : 127;
     v8i a[4], b[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
@@ -50,7 +55,12 @@ __global__ __launch_bounds__(256) void mfma_loop_kernel(int random_operands, int
     const uint64_t c0 = clock64(), t0 = wall_clock64();
     for (int it = 0; it < iters; ++it) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) acc[i / 4][i % 4] = mfma_32x32x64<0, 0>(b[i % 4], a[i / 4], acc[i / 4][i % 4]);
+        for (int i = 0; i < 16; ++i) {
+            if constexpr (SCALED)
+                acc[i / 4][i % 4] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(b[i % 4], a[i / 4], acc[i / 4][i % 4], 0, 0, 0, sc, 0, sc ^ 3);
+            else
+                acc[i / 4][i % 4] = mfma_32x32x64<0, 0>(b[i % 4], a[i / 4], acc[i / 4][i % 4]);
+        }
     }
     const uint64_t c1 = clock64(), t1 = wall_clock64();
     float s = 0.0f;
@@ -73,7 +83,15 @@ __global__ __launch_bounds__(256) void mfma_loop_kernel(int random_operands, int
 // spent in the loop by each block's first wave.
 extern "C" int odl_probe_mfma_loop(int random_operands, int iters, int blocks, float *sink_dev, uint64_t *cycles_dev, void *stream) {
     if (iters < 1 || blocks < 1 || !sink_dev || !cycles_dev) return -1;
-    hipLaunchKernelGGL(mfma_loop_kernel, dim3(blocks), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), random_operands, iters,
+    hipLaunchKernelGGL(mfma_loop_kernel<false>, dim3(blocks), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), random_operands, iters,
+                       sink_dev, cycles_dev);
+    return (int)hipGetLastError();
+}
+
+// The same loop with the block-scaled form of the instruction.
+extern "C" int odl_probe_mfma_loop_scaled(int random_operands, int iters, int blocks, float *sink_dev, uint64_t *cycles_dev, void *stream) {
+    if (iters < 1 || blocks < 1 || !sink_dev || !cycles_dev) return -1;
+    hipLaunchKernelGGL(mfma_loop_kernel<true>, dim3(blocks), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), random_operands, iters,
                        sink_dev, cycles_dev);
     return (int)hipGetLastError();
 }
