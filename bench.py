@@ -201,7 +201,7 @@ def standalone_hbm(torch, native, iters=24):
     return out
 
 
-def other_configs(torch, steps=8, warmup=3):
+def other_configs(torch, steps=8, warmup=3, only=""):
     """Whole steps (forward + backward of every Linear, weights re-quantised every step) of the other
     configurations of BASELINE.json and of configuration 3 with fp32 master weights (the reference's
     usual AMP set-up: the weight gradient is then fp32).  Same harness as the headline, fewer steps."""
@@ -217,6 +217,8 @@ def other_configs(torch, steps=8, warmup=3):
     ]
     out = {}
     for label, kind, kw, shapes, m, wdtype in cases:
+        if only and only not in label:
+            continue
         recipe = create_fp8_recipe(kind, "hybrid", **kw)
         g = torch.Generator().manual_seed(0)
         mods, xs, dys = [], [], []
@@ -553,6 +555,9 @@ def main() -> int:
                     help="run only the stand-alone measurements of the memory-bound kernels and print them (for profiling)")
     ap.add_argument("--whole-models-only", default="",
                     help="run only the whole-model step of gpt2_124m or qwen3_0.6b with the default transform and print it (for profiling)")
+    ap.add_argument("--other-configs-only", default="",
+                    help="run only the whole steps of the other configurations whose label contains this text (e.g. mxfp8, rowwise, "
+                         "delayed) and print them (for profiling)")
     ap.add_argument("--clock-probe-only", action="store_true",
                     help="run only the clock probe (GEMM back to back on Gaussian / zero operands, register-only MFMA loop) and print it")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -578,6 +583,9 @@ def main() -> int:
         return 0
     if args.clock_probe_only:
         print(json.dumps({"clock_probe": clock_probe(torch, native)}))
+        return 0
+    if args.other_configs_only:
+        print(json.dumps({"other_configs_fwd_bwd": other_configs(torch, steps=args.steps, only=args.other_configs_only)}))
         return 0
     if args.whole_models_only:
         print(json.dumps({"whole_models_fwd_bwd": whole_models(torch, which=(args.whole_models_only,), steps=args.steps,

@@ -488,7 +488,7 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
                 // whose dwords every wave read one phase B ago
                 if (i == 8) fetch_scales(par ^ 1);
                 if (i == 13) place_scales(sca[par ^ 1], scb[par ^ 1]);
-                if (i == 15) {
+                if (i == 0) {          // first: the youngest load of a step is the one the next barrier waits for longest
                     const int live = pad && !nx ? 0 : 1;
                     issue_scales(par, (nx ? sc_nin_a : sc_in_a) * live, (nx ? sc_nin_b : sc_in_b) * live,
                                  nx ? sc_next_a : sc_off_a, nx ? sc_next_b : sc_off_b, koff);
