@@ -235,8 +235,9 @@ def test_wgrad_false_keeps_weight_gradient_in_bf16(amp):
     assert max_rel_err(dw, want) <= 1e-2
 
 
-@pytest.mark.parametrize("family", ["llama", "qwen3", "gpt2"])
-def test_training_loop_through_the_reference_shaped_glue(amp, family):
+@pytest.mark.parametrize("family,recipe_name", [("llama", "delayed"), ("qwen3", "delayed"), ("gpt2", "delayed"),
+                                                ("llama", "mxfp8"), ("gpt2", "mxfp8"), ("qwen3", "tensorwise")])
+def test_training_loop_through_the_reference_shaped_glue(amp, family, recipe_name):
     """Transform -> training context -> a few optimizer steps, FP8 vs bf16 on the same init."""
     from optimus_dl_amd.modules.model import GPT2, GPT2Config, Llama, LlamaConfig, Qwen3, Qwen3Config
     from optimus_dl_amd.modules.model_transforms import build_model_transform
@@ -264,7 +265,7 @@ def test_training_loop_through_the_reference_shaped_glue(amp, family):
         if mode == "fp8":
             t = build_model_transform({"_name": "transformer_engine"})
             model = t.apply(model, device=torch.device("cuda"), collective=None, is_restart=False, checkpoint_manager=None)
-            cfg = OptimizationConfig(amp=AmpConfig(enabled=True, dtype="torch.float8_e4m3fn", fp8=Fp8Config(enabled=True, recipe="delayed", amax_history_len=4)))
+            cfg = OptimizationConfig(amp=AmpConfig(enabled=True, dtype="torch.float8_e4m3fn", fp8=Fp8Config(enabled=True, recipe=recipe_name, amax_history_len=4)))
         else:
             cfg = OptimizationConfig(amp=AmpConfig(enabled=True, dtype="torch.bfloat16"))
         ctx = TrainingContext(cfg).setup_training_context(torch.device("cuda"))
@@ -357,18 +358,20 @@ def test_shared_input_is_not_reused_after_an_in_place_change_or_for_another_tens
     assert not torch.equal(y1, y2)
 
 
-def test_forward_backward_can_be_captured_in_a_graph_and_replayed(amp):
+@pytest.mark.parametrize("recipe_name", ["tensorwise", "mxfp8"])
+def test_forward_backward_can_be_captured_in_a_graph_and_replayed(amp, recipe_name):
     """Small Linears are launch-bound; callers capture them.  Every native call takes the capture
     stream and allocates nothing itself, so a captured forward+backward must replay correctly:
     three replays on new data, eager work and synchronisations in between, each against eager."""
     M, K, N = 256, 512, 384
-    recipe = amp.create_fp8_recipe("tensorwise", "hybrid")
+    recipe = amp.create_fp8_recipe(recipe_name, "hybrid")
     lin = make_linear(seeded_bf16((N, K), 0.02, 90))
     x_static = torch.zeros((M, K), dtype=torch.bfloat16, device="cuda", requires_grad=True)
     dy_static = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
 
     def fwd_bwd():
         lin._wcache.key = None
+        lin._wcache_rowwise.clear()
         with recipe.autocast():
             y = lin(x_static)
         with recipe.backward():
