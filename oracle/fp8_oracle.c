@@ -30,6 +30,16 @@
  *                   The roll/update ORDER follows the documented behaviour of
  *                   the third-party library and cannot be checked against it
  *                   offline: parity unpinned for that ordering.
+ *   mxfp8         : the OCP Microscaling v1.0 conversion formula restated in
+ *                   float64 and with torch routines, hand-worked blocks,
+ *                   power-of-two invariance (tests/test_oracle_mx.py).  The
+ *                   third-party library's own rounding of the shared exponent
+ *                   cannot be checked offline: parity unpinned for that choice.
+ *   blockwise     : "the per-tensor rule on every block, scale rounded down to
+ *                   a power of two" against the cast / scale functions above
+ *                   block by block, a torch restatement, hand-worked blocks
+ *                   (tests/test_oracle_block.py).  Parity unpinned likewise for
+ *                   the third-party library's rounding of the block scale.
  */
 #include <math.h>
 #include <stdint.h>
@@ -294,6 +304,41 @@ ORACLE_API void oracle_mx_gemm_nt(const uint8_t *a, const uint8_t *sa, const uin
             volatile float v = bias ? acc + bias[j] : acc;
             if (c_f32) c_f32[i * N + j] = v;
             if (c_bf16) c_bf16[i * N + j] = f32_to_bf16(v);
+        }
+}
+
+/*
+ * Blockwise recipe (the reference's "blockwise", optimus_dl/modules/amp/fp8.py:295-300, which hands its backend a
+ * Float8BlockScaling recipe: 1 x 128 blocks along the contraction axis for activations and gradients, 128 x 128 blocks
+ * for weights, power-of-two scales).  Restated as: the per-tensor rule of oracle_scale applied to the amax of each block
+ * of block_r x block_c elements, the result rounded DOWN to a power of two (mantissa cleared; a subnormal result becomes
+ * 2^-126), elements = rne(clamp(v * scale)).  Rounding down keeps amax * scale <= fp8_max: nothing saturates.  The inverse
+ * of such a scale is an E8M0 byte, 254 - (exponent field of the scale); a block whose amax is 0, NaN or Inf keeps scale 1
+ * (byte 127).  The backend's own rounding of the scale cannot be checked here: parity unpinned for that choice; everything
+ * else is pinned by tests/test_oracle_block.py.
+ *   codes [rows, cols]; scale_bytes [rows / block_r, cols / block_c]
+ */
+ORACLE_API void oracle_block_quantise_bf16(const uint16_t *x, int64_t rows, int64_t cols, int64_t block_r, int64_t block_c,
+                                           int fmt, int margin, uint8_t *codes, uint8_t *scale_bytes) {
+    const int64_t nbr = rows / block_r, nbc = cols / block_c;
+    for (int64_t br = 0; br < nbr; ++br)
+        for (int64_t bc = 0; bc < nbc; ++bc) {
+            uint32_t mag = 0;
+            for (int64_t r = 0; r < block_r; ++r)
+                for (int64_t c = 0; c < block_c; ++c) {
+                    uint32_t m = (uint32_t)(x[(br * block_r + r) * cols + bc * block_c + c] & 0x7fffu) << 16;
+                    if (m > mag) mag = m;                                  /* NaN patterns sort above Inf */
+                }
+            float s = oracle_scale(bits_f32(mag), fmt, margin, 1.0f);
+            uint32_t sb = f32_bits(s) & 0xff800000u;
+            if ((sb >> 23) == 0) sb = 0x00800000u;
+            s = bits_f32(sb);
+            scale_bytes[br * nbc + bc] = (uint8_t)(254u - (sb >> 23));
+            for (int64_t r = 0; r < block_r; ++r)
+                for (int64_t c = 0; c < block_c; ++c) {
+                    const int64_t i = (br * block_r + r) * cols + bc * block_c + c;
+                    codes[i] = quantise(x[i], s, fmt);
+                }
         }
 }
 

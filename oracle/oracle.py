@@ -67,6 +67,7 @@ def lib() -> ctypes.CDLL:
         L.oracle_delayed_update.argtypes = [vp, i64, i64, vp, vp, vp, i32, i32]
         L.oracle_mx_quantise_bf16.argtypes = [vp, i64, i64, i32, vp, vp]
         L.oracle_mx_gemm_nt.argtypes = [vp, vp, vp, vp, i64, i64, i64, i32, i32, vp, vp, vp]
+        L.oracle_block_quantise_bf16.argtypes = [vp, i64, i64, i64, i64, i32, i32, vp, vp]
         L.oracle_sigmoid.argtypes = [f32]
         L.oracle_sigmoid.restype = f32
         L.oracle_swiglu_fwd.argtypes = [vp, vp, i64, vp]
@@ -458,3 +459,37 @@ def c_mx_gemm_nt(a, sa, b, sb, fmt_a, fmt_b, bias=None):
     lib().oracle_mx_gemm_nt(_p(arrs[0]), _p(arrs[1]), _p(arrs[2]), _p(arrs[3]), M, N, K, fmt_a, fmt_b,
                             _p(bias_np) if bias_np is not None else None, _p(out_bf16), _p(out_f32))
     return torch.from_numpy(out_bf16.view(np.int16)).view(torch.bfloat16), torch.from_numpy(out_f32)
+
+
+# ------------------------------------------------------------------------------------------------ blockwise recipe
+def c_block_quantise(x: torch.Tensor, block_r: int, block_c: int, fmt: int, margin: int = 0):
+    """Blockwise quantisation of a bf16 matrix (power-of-two scale per block of block_r x block_c elements) ->
+    (codes uint8 [R, C], E8M0 bytes of the inverse scales uint8 [R / block_r, C / block_c])."""
+    rows, cols = x.shape
+    assert rows % block_r == 0 and cols % block_c == 0
+    xb = _bf16_bits(x)
+    codes = np.empty((rows, cols), dtype=np.uint8)
+    sb = np.empty((rows // block_r, cols // block_c), dtype=np.uint8)
+    lib().oracle_block_quantise_bf16(_p(xb), rows, cols, block_r, block_c, fmt, margin, _p(codes), _p(sb))
+    return torch.from_numpy(codes), torch.from_numpy(sb)
+
+
+def t_block_quantise(x: torch.Tensor, block_r: int, block_c: int, fmt: int, margin: int = 0):
+    """The same with torch routines: the per-tensor scale rule on every block's amax, frexp for the power of two below
+    it, exact power-of-two scaling, the CPU float8 cast."""
+    rows, cols = x.shape
+    v = x.float().reshape(rows // block_r, block_r, cols // block_c, block_c)
+    amax = v.abs().amax(dim=(1, 3))
+    s = t_scale(amax, fmt, margin, 1.0)
+    _, e = torch.frexp(s)                                       # s = m * 2^e, 0.5 <= m < 1: the power of two below is 2^(e-1)
+    e = (e - 1).clamp(min=-126)
+    scaled = torch.ldexp(v, e[:, None, :, None].expand_as(v).to(torch.int32))
+    m = FP8_MAX[fmt]
+    codes = scaled.clamp(-m, m).to(TORCH_FP8[fmt]).view(torch.uint8).reshape(rows, cols)
+    return codes, (127 - e).to(torch.uint8)
+
+
+def block_scales_as_mx(scale_bytes: torch.Tensor, block_r: int, block_c: int) -> torch.Tensor:
+    """Block scale bytes [R / block_r, C / block_c] spread out to one byte per row and 32 columns ([R, C / 32]): the
+    layout of the MXFP8 functions above, which then dequantise and multiply blockwise tensors as well."""
+    return scale_bytes.repeat_interleave(block_r, dim=0).repeat_interleave(block_c // MX_BLOCK, dim=1).contiguous()
