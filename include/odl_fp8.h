@@ -45,7 +45,7 @@ enum odl_status {
     ODL_ERR_LAUNCH = 3    /* HIP reported an error at launch */
 };
 
-/* ABI version of this header (12); bumped when a signature changes or an entry point is added. */
+/* ABI version of this header (13); bumped when a signature changes or an entry point is added. */
 int odl_fp8_abi_version(void);
 
 /* Last error message of the calling host thread ("" if none). */
@@ -450,6 +450,21 @@ int odl_fp8_mx_cast(const void *x, int src_dtype, int64_t rows, int64_t cols, in
  */
 int odl_fp8_mx_gemm_nt(const uint8_t *a, const uint8_t *sa, const uint8_t *b, const uint8_t *sb, int scales_layout, int64_t M,
                        int64_t N, int64_t K, int fmt_a, int fmt_b, const float *bias, void *c, int out_dtype, odl_stream_t stream);
+
+/*
+ * The cast of the "blockwise" recipe (what the reference hands to its backend as Float8BlockScaling,
+ * optimus_dl/modules/amp/fp8.py:295-300): blocks of 128 elements along the contraction axis for activations and gradients
+ * (two_d = 0: one scale per row and 128 columns for `out`, one per column and 128 rows for `out_t`), blocks of 128 x 128
+ * for weights (two_d = 1: both outputs share the block's scale).  Scale of a block = fp8_max / amax / 2^margin (the rule of
+ * odl_fp8_scale_from_amax; 1 when the amax is 0, NaN or Inf) rounded DOWN to a power of two, so nothing saturates;
+ * elements = rne(clamp(v * scale)).  The inverse of such a scale is an E8M0 byte (254 - exponent field), and a 128-block is
+ * four MX blocks with the same byte: `scales` / `scales_t` are written in the ODL_MX_SCALES_KSTEP layout ([cols / 128][rows]
+ * and [rows / 128][cols] dwords of four equal bytes), and odl_fp8_mx_gemm_nt multiplies the results as they are.
+ * rows and cols multiples of 128; x and the codes 16-byte aligned.  Either pair may be NULL.
+ */
+int odl_fp8_block_cast(const void *x, int src_dtype, int64_t rows, int64_t cols, int fmt, int margin, int two_d, uint8_t *out,
+                       uint8_t *scales, uint8_t *out_t, uint8_t *scales_t, odl_stream_t stream);
+
 
 #ifdef __cplusplus
 }

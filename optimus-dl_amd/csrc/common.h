@@ -4,6 +4,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <float.h>
 #include <stdint.h>
 
 #include "../../include/odl_fp8.h"
@@ -73,6 +74,15 @@ __device__ __forceinline__ uint32_t quantise4(float x0, float x1, float x2, floa
         if (x3 != x3) r = (r & 0x00ffffffu) | ((0x7fu | ((float_to_bits(x3) >> 24) & 0x80u)) << 24);
     }
     return r;
+}
+
+// scale = fp8_max / amax / 2^margin with the guards of the C ABI
+__device__ __forceinline__ float scale_rule(float amax, float fp8_max, int margin, float fallback) {
+    if (!(amax > 0.0f) || __builtin_isinf(amax)) return fallback;
+    float s = __fdiv_rn(fp8_max, amax);                     // IEEE division, not the fast reciprocal
+    s = ldexpf(s, -margin);
+    if (__builtin_isinf(s)) s = FLT_MAX;
+    return s;
 }
 
 // |x| bit pattern of a packed pair of bf16, per 16-bit half.  For bf16 (and

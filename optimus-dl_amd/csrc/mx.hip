@@ -197,6 +197,171 @@ __global__ __launch_bounds__(kMxThreads) void mx_cast_kernel(const void *__restr
     }
 }
 
+// ------------------------------------------------------------------ blockwise recipe
+// Blocks of 128 along the contraction axis (activations, gradients) or of 128 x 128 (weights), each with the per-tensor
+// scale rule applied to its amax and rounded down to a power of two.  The inverse of such a scale is an E8M0 byte, and a
+// 128-block is four MX blocks with the same byte: the kernel writes that byte four times as the dword [K step][row] of
+// the K-step-major layout, and the MXFP8 GEMMs serve this recipe unchanged.
+template <int FMT>
+__device__ __forceinline__ void block_scale_of(uint32_t amax_bits, int margin, uint32_t &dword, float &mul) {
+    const float s = scale_rule(bits_to_float(amax_bits), Fp8Lim<FMT>::max, margin, 1.0f);
+    uint32_t b = float_to_bits(s) & 0xff800000u;                     // the power of two below (s > 0 always)
+    if ((b >> 23) == 0) b = 0x00800000u;
+    mul = bits_to_float(b);
+    dword = (254u - (b >> 23)) * 0x01010101u;
+}
+
+// Byte offset of (column, dword of 4 rows) in the transposed 128 x 128 tile: two halves of 64 columns, each laid out as the
+// 64-column tile of ct_tile.h (a 256-byte line per pair of columns, rotated by 16 bytes per 8 columns), the second half
+// rotated by 16 bytes more.  The dword writes of a half-wave (8 column groups of 16 x 4 row groups) then differ mod 32,
+// and the 16-byte reads stay aligned with 16 consecutive lanes reading one whole line.
+__device__ __forceinline__ int block_lds_off(int col, int dw) {
+    const int half = col >> 6, c = col & 63;
+    return half * 8192 + (c >> 1) * 256 + ((((c & 1) * 32) + dw + 4 * (c >> 3) + 4 * half) & 63) * 4;
+}
+
+// 128 x 128 tile per block of 256 lanes; lane (tx = lane % 8, ty = lane / 8) owns rows 4 ty .. 4 ty + 3 and columns
+// 16 tx .. 16 tx + 15.  TWO_D: one scale for the whole tile (weights); else one per row of the tile for the row-major
+// codes and one per column for the transposed codes.  rows, cols multiples of 128.
+template <int SRC, int FMT, bool TWO_D, bool WANT_ROW, bool WANT_COL>
+__global__ __launch_bounds__(256) void block_cast_kernel(const void *__restrict__ x, int64_t rows, int64_t cols, int margin,
+                                                         uint8_t *__restrict__ out, uint32_t *__restrict__ scales,
+                                                         uint8_t *__restrict__ out_t, uint32_t *__restrict__ scales_t) {
+    __shared__ __attribute__((aligned(16))) uint8_t tile[WANT_COL ? 128 * 128 : 16];
+    __shared__ uint32_t red[4][128];                 // per wave: column maxima (1-D), or slot 0: the wave's maximum (2-D)
+    __shared__ __attribute__((aligned(16))) float col_mul[128];
+    constexpr int ESZ = SRC == ODL_BF16 ? 2 : 4, DW = 16 * ESZ / 4;
+    const int tx = threadIdx.x % 8, ty = threadIdx.x / 8, wave = threadIdx.x / 64;
+    const int64_t tiles_r = rows / 128, tiles_c = cols / 128;
+    int64_t tr, tc;
+    ct_tile_of(blockIdx.x, tiles_r, tiles_c, tr, tc);
+    const int64_t r0 = tr * 128 + ty * 4, c0 = tc * 128 + tx * 16;
+
+    uint32_t raw[4][DW];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const u32x4 *p = reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(x) + ((r0 + i) * cols + c0) * ESZ);
+#pragma unroll
+        for (int h = 0; h < DW / 4; ++h) {
+            const u32x4 v = __builtin_nontemporal_load(p + h);
+            raw[i][4 * h] = v.x; raw[i][4 * h + 1] = v.y; raw[i][4 * h + 2] = v.z; raw[i][4 * h + 3] = v.w;
+        }
+    }
+    auto widen4 = [&](int i, int g, float (&f)[4]) {            // columns 4 g .. 4 g + 3 of row i
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            if constexpr (SRC == ODL_BF16) f[q] = (q & 1) ? bf16_hi(raw[i][2 * g + q / 2]) : bf16_lo(raw[i][2 * g + q / 2]);
+            else f[q] = bits_to_float(raw[i][4 * g + q]);
+        }
+    };
+    // magnitude bits (fp32 layout) of row i over the lane's 16 columns
+    auto row_mag = [&](int i) -> uint32_t {
+        if constexpr (SRC == ODL_BF16) {
+            uint32_t m2 = 0;
+#pragma unroll
+            for (int d = 0; d < DW; ++d) m2 = max_u16x2(m2, abs_bf16x2(raw[i][d]));
+            return fold_u16x2_to_f32bits(m2);
+        } else {
+            uint32_t m = 0;
+#pragma unroll
+            for (int d = 0; d < DW; ++d) m = max(m, raw[i][d] & 0x7fffffffu);
+            return m;
+        }
+    };
+
+    float mul_all = 1.0f;
+    if constexpr (TWO_D) {
+        uint32_t m = max(max(row_mag(0), row_mag(1)), max(row_mag(2), row_mag(3)));
+        m = wave_max_u32(m);
+        if (threadIdx.x % 64 == 0) red[wave][0] = m;
+        __syncthreads();
+        m = max(max(red[0][0], red[1][0]), max(red[2][0], red[3][0]));
+        uint32_t dword;
+        block_scale_of<FMT>(m, margin, dword, mul_all);
+        if (threadIdx.x < 128) {
+            if (WANT_ROW) scales[tc * rows + tr * 128 + threadIdx.x] = dword;
+            if (WANT_COL) scales_t[tr * cols + tc * 128 + threadIdx.x] = dword;
+        }
+    }
+
+    if constexpr (WANT_ROW) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float mul = mul_all;
+            if constexpr (!TWO_D) {
+                uint32_t m = max_quad(row_mag(i));
+                m = max_with_dpp<0x141>(m);                              // row_half_mirror: lane l <-> 7 - l of its 8: the other quad
+                uint32_t dword;
+                block_scale_of<FMT>(m, margin, dword, mul);
+                if (tx == 0) scales[tc * rows + r0 + i] = dword;
+            }
+            uint32_t q[4];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                float f[4];
+                widen4(i, g, f);
+                q[g] = quantise4<FMT>(f[0], f[1], f[2], f[3], mul, mul, mul, mul);
+            }
+            *reinterpret_cast<u32x4 *>(out + (r0 + i) * cols + c0) = u32x4{q[0], q[1], q[2], q[3]};
+        }
+    }
+
+    if constexpr (WANT_COL) {
+        if constexpr (!TWO_D) {
+            // column maxima: over the lane's 4 rows, over the 8 lanes of the wave with this tx (32 rows), over the 4 waves
+#pragma unroll
+            for (int d = 0; d < DW; ++d) {
+                uint32_t m;
+                if constexpr (SRC == ODL_BF16) {
+                    m = max_u16x2(max_u16x2(abs_bf16x2(raw[0][d]), abs_bf16x2(raw[1][d])), max_u16x2(abs_bf16x2(raw[2][d]), abs_bf16x2(raw[3][d])));
+                    m = max_stride8_u16x2(m);
+                    if ((ty & 7) == 0) { red[wave][16 * tx + 2 * d] = m << 16; red[wave][16 * tx + 2 * d + 1] = m & 0xffff0000u; }
+                } else {
+                    m = max(max(raw[0][d] & 0x7fffffffu, raw[1][d] & 0x7fffffffu), max(raw[2][d] & 0x7fffffffu, raw[3][d] & 0x7fffffffu));
+                    m = max_stride8(m);
+                    if ((ty & 7) == 0) red[wave][16 * tx + d] = m;
+                }
+            }
+            __syncthreads();
+            if (threadIdx.x < 128) {
+                const uint32_t m = max(max(red[0][threadIdx.x], red[1][threadIdx.x]), max(red[2][threadIdx.x], red[3][threadIdx.x]));
+                uint32_t dword;
+                float mul;
+                block_scale_of<FMT>(m, margin, dword, mul);
+                col_mul[threadIdx.x] = mul;
+                scales_t[tr * cols + tc * 128 + threadIdx.x] = dword;
+            }
+            __syncthreads();
+        }
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            float mc[4] = {mul_all, mul_all, mul_all, mul_all};
+            if constexpr (!TWO_D) {
+                const float4 v = *reinterpret_cast<const float4 *>(&col_mul[16 * tx + 4 * g]);
+                mc[0] = v.x; mc[1] = v.y; mc[2] = v.z; mc[3] = v.w;
+            }
+            uint32_t q[4], t[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float f[4];
+                widen4(i, g, f);
+                q[i] = quantise4<FMT>(f[0], f[1], f[2], f[3], mc[0], mc[1], mc[2], mc[3]);
+            }
+            transpose4x4(q, t);                                          // t[k] = rows 4 ty .. + 3 of column 16 tx + 4 g + k
+#pragma unroll
+            for (int k = 0; k < 4; ++k) *reinterpret_cast<uint32_t *>(&tile[block_lds_off(16 * tx + 4 * g + k, ty)]) = t[k];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+            const int chunk = threadIdx.x + it * 256;
+            const int col = chunk / 8, m16 = chunk % 8;
+            const u32x4 v = *reinterpret_cast<const u32x4 *>(&tile[block_lds_off(col, 4 * m16)]);
+            __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(out_t + (tc * 128 + col) * rows + tr * 128 + m16 * 16));
+        }
+    }
+}
+
 // ------------------------------------------------------------------ GEMM, tiled
 // The structure of gemm_nt_tiled_kernel (two LDS stages of BM + BN rows x 128 bytes, direct-to-LDS loads, swizzled
 // 16-byte chunks, MFMA operands swapped so that a lane ends up with 4 consecutive output columns) plus the scale
@@ -456,6 +621,18 @@ static void launch_mx_gemm(const GemmArgs &g, const uint8_t *sa, const uint8_t *
     }
 }
 
+template <int SRC, int FMT, bool TWO_D>
+static void launch_block_cast(const void *x, int64_t rows, int64_t cols, int margin, uint8_t *out, uint8_t *scales, uint8_t *out_t,
+                              uint8_t *scales_t, hipStream_t stream) {
+    const dim3 grid((unsigned)((rows / 128) * (cols / 128))), block(256);
+    uint32_t *s = reinterpret_cast<uint32_t *>(scales), *st = reinterpret_cast<uint32_t *>(scales_t);
+#define ODL_BLK(R, C) hipLaunchKernelGGL((block_cast_kernel<SRC, FMT, TWO_D, R, C>), grid, block, 0, stream, x, rows, cols, margin, out, s, out_t, st)
+    if (out && out_t) ODL_BLK(true, true);
+    else if (out) ODL_BLK(true, false);
+    else ODL_BLK(false, true);
+#undef ODL_BLK
+}
+
 }  // namespace odl
 
 using namespace odl;
@@ -532,4 +709,31 @@ extern "C" int odl_fp8_mx_gemm_nt(const uint8_t *a, const uint8_t *sa, const uin
     else ODL_MXG(ODL_FP8_E5M2, ODL_FP8_E5M2);
 #undef ODL_MXG
     return check_launch("odl_fp8_mx_gemm_nt");
+}
+
+extern "C" int odl_fp8_block_cast(const void *x, int src_dtype, int64_t rows, int64_t cols, int fmt, int margin, int two_d, uint8_t *out,
+                                  uint8_t *scales, uint8_t *out_t, uint8_t *scales_t, odl_stream_t stream_) {
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    if (rows < 0 || cols < 0) return set_error(ODL_ERR_ARG, "odl_fp8_block_cast: negative shape");
+    if (src_dtype != ODL_BF16 && src_dtype != ODL_F32) return set_error(ODL_ERR_ARG, "odl_fp8_block_cast: src_dtype %d", src_dtype);
+    if (fmt != ODL_FP8_E4M3 && fmt != ODL_FP8_E5M2) return set_error(ODL_ERR_ARG, "odl_fp8_block_cast: fmt %d", fmt);
+    if (margin < -64 || margin > 64) return set_error(ODL_ERR_ARG, "odl_fp8_block_cast: margin %d", margin);
+    if (rows * cols == 0) return ODL_OK;
+    if ((out == nullptr) != (scales == nullptr) || (out_t == nullptr) != (scales_t == nullptr))
+        return set_error(ODL_ERR_ARG, "odl_fp8_block_cast: codes and scale bytes of a layout go together");
+    if (!out && !out_t) return set_error(ODL_ERR_ARG, "odl_fp8_block_cast: neither layout asked for");
+    if (!x) return set_error(ODL_ERR_ARG, "odl_fp8_block_cast: x is null");
+    if (rows % 128 != 0 || cols % 128 != 0)
+        return set_error(ODL_ERR_SHAPE, "odl_fp8_block_cast: %lld x %lld: both sizes must be multiples of 128", (long long)rows, (long long)cols);
+    auto mis = [](const void *p, uintptr_t a) { return p && (reinterpret_cast<uintptr_t>(p) & (a - 1)); };
+    if (mis(x, 16) || mis(out, 16) || mis(out_t, 16) || mis(scales, 4) || mis(scales_t, 4))
+        return set_error(ODL_ERR_SHAPE, "odl_fp8_block_cast: x and the codes must be 16-byte aligned, the scale arrays 4-byte");
+    if ((rows / 128) * (cols / 128) > 0x7fffffffLL) return set_error(ODL_ERR_SHAPE, "odl_fp8_block_cast: too many tiles for one launch");
+#define ODL_BLK(S, F) \
+    do { if (two_d) launch_block_cast<S, F, true>(x, rows, cols, margin, out, scales, out_t, scales_t, stream); \
+         else launch_block_cast<S, F, false>(x, rows, cols, margin, out, scales, out_t, scales_t, stream); } while (0)
+    if (src_dtype == ODL_BF16) { if (fmt == ODL_FP8_E4M3) ODL_BLK(ODL_BF16, ODL_FP8_E4M3); else ODL_BLK(ODL_BF16, ODL_FP8_E5M2); }
+    else { if (fmt == ODL_FP8_E4M3) ODL_BLK(ODL_F32, ODL_FP8_E4M3); else ODL_BLK(ODL_F32, ODL_FP8_E5M2); }
+#undef ODL_BLK
+    return check_launch("odl_fp8_block_cast");
 }

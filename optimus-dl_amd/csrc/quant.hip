@@ -31,14 +31,6 @@ __global__ void fill_f32_kernel(float *p, int64_t n, float v) {
     if (i < n) p[i] = v;
 }
 
-// scale = fp8_max / amax / 2^margin with the guards of the C ABI
-__device__ __forceinline__ float scale_rule(float amax, float fp8_max, int margin, float fallback) {
-    if (!(amax > 0.0f) || __builtin_isinf(amax)) return fallback;
-    float s = __fdiv_rn(fp8_max, amax);                     // IEEE division, not the fast reciprocal
-    s = ldexpf(s, -margin);
-    if (__builtin_isinf(s)) s = FLT_MAX;
-    return s;
-}
 
 
 // Optional tail of the per-tensor amax kernel: the block that finishes last turns the

@@ -123,7 +123,7 @@ class Fp8RecipeConfig:
 class ScalingPolicy:
     """What ``FP8Recipe.recipe`` returns: the resolved policy the kernels follow."""
 
-    kind: str                 # "delayed" | "tensorwise" | "rowwise" | "mxfp8"
+    kind: str                 # "delayed" | "tensorwise" | "rowwise" | "mxfp8" | "blockwise"
     fmt_fwd: int              # native.E4M3 / native.E5M2 for activations and weights
     fmt_bwd: int              # ... for gradients
     margin: int
@@ -176,11 +176,6 @@ class FP8Recipe:
             raise ValueError(f"Unsupported FP8 format: {self.format}")
         if amax_compute_algo not in ("max", "most_recent"):
             raise ValueError(f"Unsupported amax_compute_algo: {amax_compute_algo} (max, most_recent)")
-        if self.recipe_type == Fp8RecipeType.BLOCKWISE:
-            raise NotImplementedError(
-                f"FP8 recipe '{self.recipe_type.value}' has no MI355X kernels in this build; "
-                "use delayed, tensorwise, rowwise or mxfp8"
-            )
         if amax_history_len < 1:
             raise ValueError("amax_history_len must be >= 1")
         self._recipe = ScalingPolicy(

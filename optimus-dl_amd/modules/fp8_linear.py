@@ -21,7 +21,9 @@ Per call, inside ``FP8Recipe.autocast()``:
 
 Under the "mxfp8" recipe every operand is quantised in blocks of 32 along the axis its GEMM contracts (X and W along
 the input features for the forward, dY and W along the output features for dgrad, dY and X along the tokens for wgrad),
-each block with its own power-of-two scale byte; there is no amax pass and no scaling state.
+each block with its own power-of-two scale byte; there is no amax pass and no scaling state.  "blockwise" is the same
+with blocks of 128 for activations and gradients and of 128 x 128 for the weight (one scale serves W and W^T), the
+scale being the per-tensor rule on the block's amax rounded down to a power of two; the same GEMM multiplies both.
 
 Every GEMM is issued in the "NT" form the MFMA wants (both operands contiguous
 along the contraction axis); the cast+transpose kernel supplies the transposed
@@ -117,14 +119,23 @@ def _quantise_input_shared(recipe: FP8Recipe, x2d: torch.Tensor, fmt: int, margi
     return q, q_t, s_inv
 
 
+def _block_cast(pol, x2d: torch.Tensor, fmt: int, want_rowmajor: bool, want_transposed: bool, weight: bool = False):
+    """Codes and E8M0 scale bytes of the two block-scaled recipes: 32-element blocks (mxfp8) or 128-element blocks with
+    128 x 128 ones for a weight (blockwise)."""
+    if pol.kind == "mxfp8":
+        return native.mx_cast(x2d, fmt, want_rowmajor=want_rowmajor, want_transposed=want_transposed)
+    return native.block_cast(x2d, fmt, pol.margin, two_d=weight, want_rowmajor=want_rowmajor, want_transposed=want_transposed)
+
+
 def _mx_input_shared(recipe: FP8Recipe, x2d: torch.Tensor, fmt: int, need_t: bool):
-    """MXFP8 codes and scale bytes of a Linear's input (blocks along the features; with need_t also of its transpose,
-    blocks along the tokens), made once for the Linears fed by the very same tensor."""
-    key = _input_key(x2d, "mx", fmt, 0)
+    """Block-scaled codes and scale bytes of a Linear's input (blocks along the features; with need_t also of its
+    transpose, blocks along the tokens), made once for the Linears fed by the very same tensor."""
+    pol = recipe.recipe
+    key = _input_key(x2d, pol.kind, fmt, pol.margin)
     hit = recipe.shared_input if recipe.share_inputs else None
     if hit is not None and hit["key"] == key and (hit["q_t"] is not None or not need_t):
         return hit["q"], hit["s_inv"], hit["q_t"], hit["s_t"]
-    q, sc, q_t, sc_t = native.mx_cast(x2d, fmt, want_rowmajor=True, want_transposed=need_t)
+    q, sc, q_t, sc_t = _block_cast(pol, x2d, fmt, True, need_t)
     if recipe.share_inputs:
         entry = {"key": key, "x": x2d, "q": q, "q_t": q_t, "s_inv": sc, "s_t": sc_t}
         prev = recipe.shared_input
@@ -189,7 +200,7 @@ class _Fp8LinearFn(torch.autograd.Function):
         saved: dict[str, Any] = {}
         ctx.wgrad_direct = False
 
-        if pol.kind == "mxfp8":
+        if pol.kind in ("mxfp8", "blockwise"):
             fp8_wgrad = need_wgrad and recipe.wgrad
             xq, xs, xq_t, xs_t = _mx_input_shared(recipe, x2d, pol.fmt_fwd, fp8_wgrad)
             wq, ws, wq_t, ws_t = module._mx_weight(weight, recipe, need_t=need_dgrad)
@@ -256,10 +267,10 @@ class _Fp8LinearFn(torch.autograd.Function):
         dx = dw = db = None
         fp8_wgrad = ctx.need_wgrad and recipe.wgrad
 
-        if pol.kind == "mxfp8":
+        if pol.kind in ("mxfp8", "blockwise"):
             if ctx.need_dgrad or fp8_wgrad:
                 # one pass over dy: blocks along the output features for dgrad, along the tokens (transposed) for wgrad
-                gq, gs, gq_t, gs_t = native.mx_cast(dy2d, pol.fmt_bwd, want_rowmajor=ctx.need_dgrad, want_transposed=fp8_wgrad)
+                gq, gs, gq_t, gs_t = _block_cast(pol, dy2d, pol.fmt_bwd, ctx.need_dgrad, fp8_wgrad)
             if ctx.need_dgrad:
                 dx = native.mx_gemm_nt(gq, gs, saved["wq_t"], saved["ws_t"], pol.fmt_bwd, pol.fmt_fwd, out_dtype=ctx.x_dtype)
             if fp8_wgrad:
@@ -442,14 +453,16 @@ class FP8Linear(nn.Linear):
         return q, s_inv
 
     def _mx_weight(self, weight: torch.Tensor, recipe: FP8Recipe, need_t: bool):
-        """MXFP8 codes and scale bytes of W (blocks along the input features) and, with need_t, of W^T (blocks along
-        the output features, for dgrad); kept while the Parameter is unchanged."""
-        fmt = recipe.recipe.fmt_fwd
-        key = _weight_key(weight, fmt, ("mx",))
+        """Block-scaled codes and scale bytes of W (blocks along the input features) and, with need_t, of W^T (blocks along
+        the output features, for dgrad; under the blockwise recipe both share the scales of the 128 x 128 blocks); kept
+        while the Parameter is unchanged."""
+        pol = recipe.recipe
+        fmt = pol.fmt_fwd
+        key = _weight_key(weight, fmt, (pol.kind, pol.margin))
         hit = self._wcache_rowwise.get("mx")
         if hit is not None and hit[0] == key and recipe.cache_weights and (hit[3] is not None or not need_t):
             return hit[1:]
-        q, sc, q_t, sc_t = native.mx_cast(weight.detach(), fmt, want_rowmajor=True, want_transposed=need_t)
+        q, sc, q_t, sc_t = _block_cast(pol, weight.detach(), fmt, True, need_t, weight=True)
         self._wcache_rowwise["mx"] = (key, q, sc, q_t, sc_t)
         return q, sc, q_t, sc_t
 
@@ -462,8 +475,10 @@ class FP8Linear(nn.Linear):
             return False
         tokens = x.numel() // max(self.in_features, 1)
         recipe = _state.active_recipe()
-        # MXFP8 blocks are 32 long along every axis a GEMM of this layer contracts (features in and out, tokens)
-        mult = 32 if recipe is not None and recipe.recipe.kind == "mxfp8" else 16
+        # MXFP8 blocks are 32 long along every axis a GEMM of this layer contracts (features in and out, tokens), the
+        # blocks of the blockwise recipe 128
+        kind = recipe.recipe.kind if recipe is not None else ""
+        mult = 32 if kind == "mxfp8" else (128 if kind == "blockwise" else 16)
         if self.in_features % mult or self.out_features % mult or tokens % mult or tokens == 0:
             _warn_once(
                 f"FP8Linear({self.in_features}->{self.out_features}) with {tokens} tokens: sizes must be multiples "

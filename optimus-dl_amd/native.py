@@ -24,7 +24,7 @@ DT_BF16, DT_F32 = 0, 1
 AMAX_MAX, AMAX_MOST_RECENT = 0, 1
 FP8_MAX = {E4M3: 448.0, E5M2: 57344.0}
 TORCH_FP8 = {E4M3: torch.float8_e4m3fn, E5M2: torch.float8_e5m2}
-ABI_VERSION = 12
+ABI_VERSION = 13
 AMAX_PARTS = 512                       # ODL_FP8_AMAX_PARTS
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
@@ -70,6 +70,7 @@ EXPORTS = (
     "odl_fp8_gemm_set_clock_probe",
     "odl_fp8_mx_cast",
     "odl_fp8_mx_gemm_nt",
+    "odl_fp8_block_cast",
 )
 
 _lib = None
@@ -141,6 +142,7 @@ def load() -> ctypes.CDLL:
         L.odl_fp8_gemm_set_clock_probe.argtypes = [vp, i32]
         L.odl_fp8_mx_cast.argtypes = [vp, i32, i64, i64, i32, vp, vp, i32, vp, vp, i32, vp]
         L.odl_fp8_mx_gemm_nt.argtypes = [vp, vp, vp, vp, i32, i64, i64, i64, i32, i32, vp, vp, i32, vp]
+        L.odl_fp8_block_cast.argtypes = [vp, i32, i64, i64, i32, i32, i32, vp, vp, vp, vp, vp]
         for name in EXPORTS:
             getattr(L, name)  # AttributeError here = the library does not match the header
         if L.odl_fp8_abi_version() != ABI_VERSION:
@@ -767,6 +769,36 @@ def mx_cast(x: torch.Tensor, fmt: int, want_rowmajor: bool = True, want_transpos
     ptr = lambda t: t.data_ptr() if t is not None else None
     _check(load().odl_fp8_mx_cast(x.data_ptr(), _src_dtype(x), rows, cols, fmt, ptr(out), ptr(sc), lay, ptr(out_t), ptr(sc_t), lay_t,
                                   _stream()), "odl_fp8_mx_cast")
+    return out, sc, out_t, sc_t
+
+
+BLOCK = 128
+
+
+def block_cast(x: torch.Tensor, fmt: int, margin: int = 0, two_d: bool = False, want_rowmajor: bool = True,
+               want_transposed: bool = False):
+    """The cast of the blockwise recipe in one launch: power-of-two scales per 128 elements of the contraction axis
+    (two_d False: per row and 128 columns for the row-major codes, per column and 128 rows for the transposed ones) or
+    per 128 x 128 block (two_d True, weights).  -> (codes [rows, cols], scales [cols/128, rows, 4], codes_t [cols, rows],
+    scales_t [rows/128, cols, 4]); the scale tensors hold E8M0 bytes in the K-step-major layout, each block's byte four
+    times, and go to ``mx_gemm_nt`` as they are.  The pair that was not asked for is (None, None)."""
+    x = _as_2d(x)
+    rows, cols = x.shape
+    if not (want_rowmajor or want_transposed):
+        raise NativeError("block_cast: neither layout asked for")
+    if rows % BLOCK or cols % BLOCK:
+        raise NativeError(f"block_cast: {rows} x {cols}: both sizes must be multiples of 128")
+    dev = x.device
+    out = sc = out_t = sc_t = None
+    if want_rowmajor:
+        out = torch.empty((rows, cols), dtype=torch.uint8, device=dev)
+        sc = torch.empty((cols // BLOCK, rows, 4), dtype=torch.uint8, device=dev)
+    if want_transposed:
+        out_t = torch.empty((cols, rows), dtype=torch.uint8, device=dev)
+        sc_t = torch.empty((rows // BLOCK, cols, 4), dtype=torch.uint8, device=dev)
+    ptr = lambda t: t.data_ptr() if t is not None else None
+    _check(load().odl_fp8_block_cast(x.data_ptr(), _src_dtype(x), rows, cols, fmt, margin, 1 if two_d else 0, ptr(out), ptr(sc),
+                                     ptr(out_t), ptr(sc_t), _stream()), "odl_fp8_block_cast")
     return out, sc, out_t, sc_t
 
 

@@ -212,14 +212,13 @@ def test_unsupported_shapes_run_as_plain_linear(amp):
     assert lin2.fp8_calls == 0
 
 
-def test_e5m2_delayed_is_refused_and_block_recipes_have_no_kernels(amp):
+def test_e5m2_delayed_is_refused_and_every_recipe_type_constructs(amp):
     with pytest.raises(ValueError, match="Pure E5M2 format is not supported"):
         amp.FP8Recipe("delayed", "e5m2")
     r = amp.FP8Recipe("tensorwise", "e5m2")
     assert r.format == amp.Fp8Format.E5M2 and r.recipe.fmt_fwd == O.E5M2
-    with pytest.raises(NotImplementedError):
-        amp.FP8Recipe("blockwise", "hybrid")
     assert amp.FP8Recipe("mxfp8", "hybrid").recipe.kind == "mxfp8"
+    assert amp.FP8Recipe("blockwise", "hybrid").recipe.kind == "blockwise"
     rec = amp.create_fp8_recipe("delayed", "hybrid", margin=2, amax_history_len=32, amax_compute_algo="most_recent", reduce_amax=False)
     assert (rec.margin, rec.amax_history_len, rec.amax_compute_algo, rec.reduce_amax, rec.fp8_dpa, rec.fp8_mha) == (2, 32, "most_recent", False, False, False)
     assert rec.recipe_type == amp.Fp8RecipeType.DELAYED and rec.format == amp.Fp8Format.HYBRID and rec.recipe is not None
@@ -236,7 +235,7 @@ def test_wgrad_false_keeps_weight_gradient_in_bf16(amp):
 
 
 @pytest.mark.parametrize("family,recipe_name", [("llama", "delayed"), ("qwen3", "delayed"), ("gpt2", "delayed"),
-                                                ("llama", "mxfp8"), ("gpt2", "mxfp8"), ("qwen3", "tensorwise")])
+                                                ("llama", "mxfp8"), ("gpt2", "mxfp8"), ("qwen3", "tensorwise"), ("llama", "blockwise")])
 def test_training_loop_through_the_reference_shaped_glue(amp, family, recipe_name):
     """Transform -> training context -> a few optimizer steps, FP8 vs bf16 on the same init."""
     from optimus_dl_amd.modules.model import GPT2, GPT2Config, Llama, LlamaConfig, Qwen3, Qwen3Config
