@@ -446,7 +446,8 @@ int odl_fp8_mx_cast(const void *x, int src_dtype, int64_t rows, int64_t cols, in
  * N x K / 32 blocks, both in `scales_layout`; K % 32 == 0; a, b, c and bias 16-byte aligned.  With K-step-major scales,
  * M % 128 == 0, N % 128 == 0, K >= 512 and enough tiles to fill the chip the persistent streaming kernel runs (the one of
  * odl_fp8_gemm_nt, with the scale dwords riding beside the operand loads); K % 128 == 0 with 4-byte aligned scale arrays
- * otherwise runs an LDS-tiled kernel; other shapes a plain one-wave-per-tile kernel.
+ * otherwise runs an LDS-tiled kernel; other shapes a plain one-wave-per-tile kernel.  The first call on a device looks up a
+ * constant in the library's device image (hipGetSymbolAddress): make it outside of stream capture.
  */
 int odl_fp8_mx_gemm_nt(const uint8_t *a, const uint8_t *sa, const uint8_t *b, const uint8_t *sb, int scales_layout, int64_t M,
                        int64_t N, int64_t K, int fmt_a, int fmt_b, const float *bias, void *c, int out_dtype, odl_stream_t stream);
