@@ -158,7 +158,7 @@ def _assert_within_hardware_sum(got32, ac, asc, bc, bsc, fa, fb, bias=None):
 
 
 GEMM_SHAPES = [
-    (32, 32, 32), (32, 32, 96), (64, 96, 160), (100, 72, 224), (7, 13, 64),            # plain kernel (K % 128 != 0 or tiny)
+    (32, 32, 32), (32, 32, 96), (64, 96, 160), (100, 72, 224), (7, 13, 64), (16, 24, 256),   # plain kernel (K % 128 != 0 or tiny)
     (128, 128, 128), (256, 256, 512), (384, 640, 1024), (200, 136, 256), (130, 70, 384),  # 128 x 128 tiles, edges
     (4096, 4096, 256), (4100, 4232, 128),                                                # 256 x 256 tiles, interior and edges
     (4096, 4096, 512), (4224, 4480, 640), (3968, 4352, 1152),      # K-step-major: the streaming kernel, also with half tiles at the edges and an odd number of K steps
