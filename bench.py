@@ -12,10 +12,11 @@ once and read by wgrad as stored), weights re-quantised each step as after an op
 step.  Inputs are synthetic, seeded, and resident in HBM before the clock starts.
 
 Two passes over the same steps: the timed one (`value`, `ms_per_step`) has nothing
-on the stream but the work itself; the second brackets every native call with a pair
-of HIP events on the launch stream for the per-kernel figures (`roofline`,
-`hbm_kernels`, `time_split_ms_per_step`); the events themselves cost about 4 % of a
-step, reported as `ms_per_step_with_kernel_events`.
+on the stream but the work itself; the second records a HIP event on the launch stream
+after every native call, and a call's time runs from the previous call's event to its
+own (`roofline`, `hbm_kernels`, `time_split_ms_per_step`: kernel + launch gap + one
+event each, adding up to the step); the events cost about 2 % of a step, reported as
+`ms_per_step_with_kernel_events`.
 
 Prints ONE JSON line: whole-step TFLOP/s, the GEMM kernel's MFMA roofline
 fraction, the HBM rates of the memory-bound kernels inside the step and on their own,
@@ -64,14 +65,21 @@ def step_flops(m: int = M_TOKENS) -> float:
 
 
 class KernelTimer:
-    """Brackets each native call with HIP events on the stream it is launched on
-    (torch's current stream, which is the stream the library receives)."""
+    """One HIP event after every native call, on the stream it is launched on (torch's current stream, which is the
+    stream the library receives): a call's time runs from the event after the previous call to its own, so the figures
+    of a step add up to the step and every launch carries one event, not two."""
 
     def __init__(self, native, torch):
         self.native, self.torch = native, torch
         self.records: dict[str, list] = {}
         self.enabled = False
         self._orig = {}
+        self._last = None
+
+    def start(self):
+        self._last = self.torch.cuda.Event(enable_timing=True)
+        self._last.record()
+        self.enabled = True
 
     def install(self):
         def wrap(name, work_fn, record_as=None):
@@ -82,10 +90,10 @@ class KernelTimer:
             def timed(*a, **kw):
                 if not self.enabled:
                     return orig(*a, **kw)
-                e0, e1 = self.torch.cuda.Event(enable_timing=True), self.torch.cuda.Event(enable_timing=True)
-                e0.record()
                 out = orig(*a, **kw)
+                e0, e1 = self._last, self.torch.cuda.Event(enable_timing=True)
                 e1.record()
+                self._last = e1
                 key = record_as(*a, **kw) if callable(record_as) else record_as
                 self.records.setdefault(key, []).append((e0, e1, work_fn(*a, **kw)))
                 return out
@@ -632,8 +640,8 @@ def main() -> int:
         one_step()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    # the same steps again with a pair of HIP events around every native call (per-kernel figures)
-    timer.enabled = True
+    # the same steps again with a HIP event after every native call (per-kernel figures)
+    timer.start()
     t0 = time.perf_counter()
     for _ in range(args.steps):
         one_step()
