@@ -460,3 +460,56 @@ def test_quantisation_of_a_tensor_with_more_than_2_31_elements(N):
     assert_bytes_equal(q_t[:, rows.cuda()], want.t(), "the same rows in the transposed copy")
     cols = torch.tensor([0, 77, V - 1]).cuda()
     assert torch.equal(q_t[cols], q[:, cols].t())
+
+
+# ------------------------------------------------------------------------------------------- block-scaled recipes
+def _sampled_block_product(out, aq, asb, bq, bsb, fa, fb, seed, what, rows=48, cols=640):
+    """out[M, N] against the emulated block-scaled product on a random rows x cols sample; asb / bsb are the scale bytes
+    as [rows, K / 32]."""
+    M, Nn = out.shape
+    g = torch.Generator().manual_seed(seed)
+    ri = torch.randperm(M, generator=g)[:rows].sort().values.cuda()
+    ci = torch.randperm(Nn, generator=g)[:cols].sort().values.cuda()
+    ref = O.t_mx_gemm_nt(aq[ri].cpu(), asb[ri].cpu(), bq[ci].cpu(), bsb[ci].cpu(), fa, fb)
+    err = max_rel_err(out[ri][:, ci], ref)
+    assert err <= TOL, f"{what}: max rel err {err} on a {rows}x{cols} sample"
+
+
+@pytest.mark.parametrize("M,Nn,K", [pytest.param(8192, 14336, 4096, id="cfg3-fwd-gate"), pytest.param(8192, 4096, 14336, id="cfg3-dgrad-gate"),
+                                    pytest.param(14336, 4096, 8192, id="cfg3-wgrad-gate")])
+@pytest.mark.parametrize("recipe", ["mxfp8", "blockwise"])
+def test_block_scaled_gemm_at_baseline_shapes(N, M, Nn, K, recipe):
+    a = draw((M, K), 1e-3, 11)           # plays dY (E5M2) against a weight-like operand (E4M3)
+    b = draw((Nn, K), 0.02, 12)
+    if recipe == "mxfp8":
+        aq, asc, _, _ = N.mx_cast(a, O.E5M2, True, False)
+        bq, bsc, _, _ = N.mx_cast(b, O.E4M3, True, False)
+    else:
+        aq, asc, _, _ = N.block_cast(a, O.E5M2, 0, False, True, False)
+        bq, bsc, _, _ = N.block_cast(b, O.E4M3, 0, True, True, False)
+    # the casts themselves on sampled rows: bit-exact against the oracle (a row's blocks depend on that row only,
+    # except for the 128 x 128 weight blocks, which are checked on whole row blocks)
+    g = torch.Generator().manual_seed(M + K)
+    ri = torch.randperm(M, generator=g)[:64].sort().values
+    a_rows = a[ri.cuda()].cpu()
+    asb = N.mx_scales_rowmajor(asc)
+    if recipe == "mxfp8":
+        wc, ws = O.c_mx_quantise(a_rows, O.E5M2)
+        assert torch.equal(asb[ri.cuda()].cpu(), ws), "scale bytes of sampled rows"
+    else:
+        wc, ws = O.c_block_quantise(a_rows, 1, 128, O.E5M2, 0)
+        assert torch.equal(asb[ri.cuda()].cpu(), O.block_scales_as_mx(ws, 1, 128)), "scale bytes of sampled rows"
+        blk = int(torch.randint(0, Nn // 128, (1,), generator=g))
+        wcb, wsb = O.c_block_quantise(b[128 * blk:128 * (blk + 1)].cpu(), 128, 128, O.E4M3, 0)
+        assert torch.equal(bq[128 * blk:128 * (blk + 1)].cpu(), wcb), "codes of a sampled row of 128 x 128 weight blocks"
+        assert torch.equal(N.mx_scales_rowmajor(bsc)[128 * blk:128 * (blk + 1)].cpu(), O.block_scales_as_mx(wsb, 128, 128))
+    assert torch.equal(aq[ri.cuda()].cpu(), wc), "codes of sampled rows"
+    del a, b
+    out = N.mx_gemm_nt(aq, asc, bq, bsc, O.E5M2, O.E4M3)
+    _sampled_block_product(out, aq, asb, bq, N.mx_scales_rowmajor(bsc), O.E5M2, O.E4M3, seed=M + Nn, what=f"{recipe} {M}x{Nn}x{K}")
+    # operands swapped: the transpose, bit for bit (same kernel, same K order)
+    swapped = N.mx_gemm_nt(bq, bsc, aq, asc, O.E4M3, O.E5M2)
+    assert torch.equal(swapped.t(), out)
+    # one more on every scale byte of A: every output doubled (exact in bf16 away from overflow)
+    doubled = N.mx_gemm_nt(aq, asc + 1, bq, bsc, O.E5M2, O.E4M3)
+    assert torch.equal(doubled.float(), out.float() * 2)
