@@ -355,7 +355,7 @@ def llama_block(torch, steps=6, warmup=3):
     return out
 
 
-def whole_models(torch, which=("gpt2_124m", "qwen3_0.6b"), steps=5, warmup=3, labels=None):
+def whole_models(torch, which=("gpt2_124m", "qwen3_0.6b"), steps=5, warmup=3, labels=None, recipe_type="tensorwise"):
     """The reference's own small presets as whole models (GPT-2 124M at 16 x 1024 tokens, Qwen3-0.6B at 4 x 2048;
     fp32 master weights, random init, random tokens): forward + cross-entropy + backward, weights re-quantised every
     step.  bf16 autocast, the FP8 Linears alone, the default transform (fused norms / activations as well), and the same
@@ -387,7 +387,7 @@ def whole_models(torch, which=("gpt2_124m", "qwen3_0.6b"), steps=5, warmup=3, la
             model = model.cuda()
             if cfg:
                 build_model_transform(cfg).apply(model)
-            recipe = A.FP8Recipe(recipe_type="tensorwise")
+            recipe = A.FP8Recipe(recipe_type=recipe_type)
             # `fp8.param`: all weights re-quantised in two launches per step instead of two per weight
             param_set = recipe.attach_params(model) if label.endswith("param_set") else None
             ids = torch.randint(0, V, (B, T), device="cuda")
@@ -402,6 +402,7 @@ def whole_models(torch, which=("gpt2_124m", "qwen3_0.6b"), steps=5, warmup=3, la
                     for m in model.modules():
                         if hasattr(m, "_wcache"):
                             m._wcache.key = None
+                            m._wcache_rowwise.clear()
                 if cfg:
                     with A.fp8_autocast(torch.device("cuda"), recipe):
                         loss = F.cross_entropy(model(ids)["logits"].view(-1, V).float(), tgt)
@@ -564,6 +565,8 @@ def main() -> int:
                     help="run only the stand-alone measurements of the memory-bound kernels and print them (for profiling)")
     ap.add_argument("--whole-models-only", default="",
                     help="run only the whole-model step of gpt2_124m or qwen3_0.6b with the default transform and print it (for profiling)")
+    ap.add_argument("--recipe", default="tensorwise",
+                    help="with --whole-models-only: the scaling recipe (tensorwise, delayed, rowwise, mxfp8, blockwise)")
     ap.add_argument("--other-configs-only", default="",
                     help="run only the whole steps of the other configurations whose label contains this text (e.g. mxfp8, rowwise, "
                          "delayed) and print them (for profiling)")
@@ -598,7 +601,8 @@ def main() -> int:
         return 0
     if args.whole_models_only:
         print(json.dumps({"whole_models_fwd_bwd": whole_models(torch, which=(args.whole_models_only,), steps=args.steps,
-                                                                   labels=("fp8_linears_fused_producers",))}))
+                                                                   labels=("fp8_linears_fused_producers",), recipe_type=args.recipe),
+                          "recipe": args.recipe}))
         return 0
     dev = "cuda"
     data = make_inputs(torch, device=dev)

@@ -45,7 +45,7 @@ enum odl_status {
     ODL_ERR_LAUNCH = 3    /* HIP reported an error at launch */
 };
 
-/* ABI version of this header (13); bumped when a signature changes or an entry point is added. */
+/* ABI version of this header (14); bumped when a signature changes or an entry point is added. */
 int odl_fp8_abi_version(void);
 
 /* Last error message of the calling host thread ("" if none). */
@@ -451,6 +451,17 @@ int odl_fp8_mx_cast(const void *x, int src_dtype, int64_t rows, int64_t cols, in
  */
 int odl_fp8_mx_gemm_nt(const uint8_t *a, const uint8_t *sa, const uint8_t *b, const uint8_t *sb, int scales_layout, int64_t M,
                        int64_t N, int64_t K, int fmt_a, int fmt_b, const float *bias, void *c, int out_dtype, odl_stream_t stream);
+
+/*
+ * odl_fp8_mx_gemm_nt with K cut into `splits` runs that are computed side by side, for outputs of few tiles and a long
+ * contraction (weight gradients of small layers), exactly as odl_fp8_gemm_splitk does for per-tensor scales
+ * (odl_fp8_gemm_split_count says when and how many): fp32 partial results in `workspace` (splits * M * N floats, 16-byte
+ * aligned, caller-owned), added in run order, bias added, one rounding.  K-step-major scales only; M, N, K multiples of
+ * 128; every run at least 512 long.
+ */
+int odl_fp8_mx_gemm_splitk(const uint8_t *a, const uint8_t *sa, const uint8_t *b, const uint8_t *sb, int64_t M, int64_t N, int64_t K,
+                           int fmt_a, int fmt_b, const float *bias, void *c, int out_dtype, int splits, void *workspace,
+                           int64_t workspace_bytes, odl_stream_t stream);
 
 /*
  * The cast of the "blockwise" recipe (what the reference hands to its backend as Float8BlockScaling,

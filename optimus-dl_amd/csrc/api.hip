@@ -41,6 +41,6 @@ int device_cu_count() {
 
 }  // namespace odl
 
-extern "C" int odl_fp8_abi_version(void) { return 13; }
+extern "C" int odl_fp8_abi_version(void) { return 14; }
 
 extern "C" const char *odl_fp8_last_error(void) { return odl::g_err; }

@@ -166,5 +166,8 @@ bool gemm_stream_accepts(const GemmArgs &g);
 void launch_gemm_stream(int fa, int fb, const GemmArgs &g, int num_cus, hipStream_t stream);
 // gemm_fp8.hip: hands the calling thread's clock-probe record (odl_fp8_gemm_set_clock_probe), if any, to a streaming launch
 void attach_clock_probe(GemmArgs &g);
+// gemm_fp8.hip: out = (sum of the `splits` fp32 partial results in `workspace`, in split order) * (sa x sb) (+ bias), one rounding
+void launch_splitk_reduce(const float *workspace, int splits, int64_t M, int64_t N, const float *sa, int sa_vec, const float *sb, int sb_vec,
+                          const float *bias, void *c, int out_dtype, hipStream_t stream);
 
 }  // namespace odl

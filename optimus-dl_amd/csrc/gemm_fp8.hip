@@ -144,6 +144,19 @@ extern "C" const char *odl_fp8_gemm_variant_name(int variant) {
     return (variant >= 0 && variant < kNumVariants) ? kVariants[variant].name : "";
 }
 
+void odl::launch_splitk_reduce(const float *workspace, int splits, int64_t M, int64_t N, const float *sa, int sa_vec, const float *sb,
+                               int sb_vec, const float *bias, void *c, int out_dtype, hipStream_t stream) {
+    const int64_t quads = M * N / 4;
+    int64_t blocks = (quads + 255) / 256;
+    if (blocks > 4 * (int64_t)cu_count()) blocks = 4 * (int64_t)cu_count();
+    if (out_dtype == ODL_BF16)
+        hipLaunchKernelGGL((splitk_reduce_kernel<true>), dim3((unsigned)blocks), dim3(256), 0, stream, workspace, splits, M, N, sa, sa_vec, sb,
+                           sb_vec, bias, c);
+    else
+        hipLaunchKernelGGL((splitk_reduce_kernel<false>), dim3((unsigned)blocks), dim3(256), 0, stream, workspace, splits, M, N, sa, sa_vec, sb,
+                           sb_vec, bias, c);
+}
+
 void odl::attach_clock_probe(GemmArgs &g) {
     if (!t_clock_probe) return;
     g.clock_out = t_clock_probe + 4 * (size_t)(t_clock_next % t_clock_capacity);
@@ -329,15 +342,7 @@ extern "C" int odl_fp8_gemm_splitk(const uint8_t *a, const uint8_t *b, int64_t M
     if (!gemm_stream_accepts(g)) return set_error(ODL_ERR_SHAPE, "odl_fp8_gemm_splitk: shape not taken by the streaming kernel");
     attach_clock_probe(g);
     launch_gemm_stream(fmt_a, fmt_b, g, cu_count(), stream);
-    const int64_t quads = M * N / 4;
-    int64_t blocks = (quads + 255) / 256;
-    if (blocks > 4 * (int64_t)cu_count()) blocks = 4 * (int64_t)cu_count();
     const int sa_vec = sa_n == M && M != 1, sb_vec = sb_n == N && N != 1;
-    if (out_dtype == ODL_BF16)
-        hipLaunchKernelGGL((splitk_reduce_kernel<true>), dim3((unsigned)blocks), dim3(256), 0, stream, (const float *)workspace, splits, M, N,
-                           sa_inv, sa_vec, sb_inv, sb_vec, bias, c);
-    else
-        hipLaunchKernelGGL((splitk_reduce_kernel<false>), dim3((unsigned)blocks), dim3(256), 0, stream, (const float *)workspace, splits, M, N,
-                           sa_inv, sa_vec, sb_inv, sb_vec, bias, c);
+    launch_splitk_reduce((const float *)workspace, splits, M, N, sa_inv, sa_vec, sb_inv, sb_vec, bias, c, out_dtype, stream);
     return check_launch("odl_fp8_gemm_splitk");
 }

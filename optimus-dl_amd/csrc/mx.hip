@@ -737,3 +737,44 @@ extern "C" int odl_fp8_block_cast(const void *x, int src_dtype, int64_t rows, in
 #undef ODL_BLK
     return check_launch("odl_fp8_block_cast");
 }
+
+// The block-scaled GEMM with K cut into `splits` runs computed side by side (outputs of few tiles and a long contraction:
+// weight gradients of small layers), as odl_fp8_gemm_splitk does for per-tensor scales: every run leaves an fp32 partial
+// result in the caller's workspace, a second kernel adds them in run order, adds the bias and rounds once.
+extern "C" int odl_fp8_mx_gemm_splitk(const uint8_t *a, const uint8_t *sa, const uint8_t *b, const uint8_t *sb, int64_t M, int64_t N, int64_t K,
+                                      int fmt_a, int fmt_b, const float *bias, void *c, int out_dtype, int splits, void *workspace,
+                                      int64_t workspace_bytes, odl_stream_t stream_) {
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    if (!a || !sa || !b || !sb || !c || !workspace) return set_error(ODL_ERR_ARG, "odl_fp8_mx_gemm_splitk: null pointer");
+    if ((fmt_a != ODL_FP8_E4M3 && fmt_a != ODL_FP8_E5M2) || (fmt_b != ODL_FP8_E4M3 && fmt_b != ODL_FP8_E5M2))
+        return set_error(ODL_ERR_ARG, "odl_fp8_mx_gemm_splitk: formats %d, %d", fmt_a, fmt_b);
+    if (out_dtype != ODL_BF16 && out_dtype != ODL_F32) return set_error(ODL_ERR_ARG, "odl_fp8_mx_gemm_splitk: out_dtype %d", out_dtype);
+    auto mis = [](const void *p, uintptr_t al) { return (reinterpret_cast<uintptr_t>(p) & (al - 1)) != 0; };
+    if (mis(a, 16) || mis(b, 16) || mis(c, 16) || mis(workspace, 16) || mis(sa, 4) || mis(sb, 4) || (bias && mis(bias, 16)))
+        return set_error(ODL_ERR_SHAPE, "odl_fp8_mx_gemm_splitk: operands, output, workspace and bias must be 16-byte aligned, scales 4-byte");
+    const bool sizes_ok = M > 0 && N > 0 && M % 128 == 0 && N % 128 == 0 && K % 128 == 0 &&
+                          (double)(M + 256) * (double)K < 2147483648.0 && (double)(N + 256) * (double)K < 2147483648.0;
+    if (!sizes_ok)
+        return set_error(ODL_ERR_SHAPE, "odl_fp8_mx_gemm_splitk: M, N, K must be multiples of 128 and each operand under 2 GiB; got %lld x %lld x %lld",
+                         (long long)M, (long long)N, (long long)K);
+    const int64_t steps = K / 128;
+    const int64_t per = ((steps + splits - 1) / (splits > 0 ? splits : 1) + 1) & ~(int64_t)1;
+    if (splits < 2 || splits > 64 || per < 4 || steps - (splits - 1) * per < 4)
+        return set_error(ODL_ERR_ARG, "odl_fp8_mx_gemm_splitk: %d splits of K=%lld leave a run shorter than 512", splits, (long long)K);
+    if (workspace_bytes < (int64_t)splits * M * N * 4)
+        return set_error(ODL_ERR_ARG, "odl_fp8_mx_gemm_splitk: workspace of %lld bytes, %lld needed", (long long)workspace_bytes,
+                         (long long)splits * M * N * 4);
+    const float *one = unit_scale_for_current_device("odl_fp8_mx_gemm_splitk");
+    if (!one) return ODL_ERR_LAUNCH;
+    GemmArgs g{};
+    g.a = a; g.b = b; g.c = workspace; g.sa = one; g.sb = one; g.bias = nullptr;
+    g.M = M; g.N = N; g.K = K; g.sa_vec = 0; g.sb_vec = 0; g.out_dtype = ODL_F32;
+    g.splits = splits; g.split_steps = (int)per;
+    g.mx_sa = sa; g.mx_sb = sb;
+    g.tiles_m = (int)((M + 255) / 256); g.tiles_n = (int)((N + 255) / 256);
+    if (!gemm_stream_accepts(g)) return set_error(ODL_ERR_SHAPE, "odl_fp8_mx_gemm_splitk: shape not taken by the streaming kernel");
+    attach_clock_probe(g);
+    launch_gemm_stream(fmt_a, fmt_b, g, device_cu_count(), stream);
+    launch_splitk_reduce((const float *)workspace, splits, M, N, one, 0, one, 0, bias, c, out_dtype, stream);
+    return check_launch("odl_fp8_mx_gemm_splitk");
+}

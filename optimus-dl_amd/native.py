@@ -24,7 +24,7 @@ DT_BF16, DT_F32 = 0, 1
 AMAX_MAX, AMAX_MOST_RECENT = 0, 1
 FP8_MAX = {E4M3: 448.0, E5M2: 57344.0}
 TORCH_FP8 = {E4M3: torch.float8_e4m3fn, E5M2: torch.float8_e5m2}
-ABI_VERSION = 13
+ABI_VERSION = 14
 AMAX_PARTS = 512                       # ODL_FP8_AMAX_PARTS
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
@@ -71,6 +71,7 @@ EXPORTS = (
     "odl_fp8_mx_cast",
     "odl_fp8_mx_gemm_nt",
     "odl_fp8_block_cast",
+    "odl_fp8_mx_gemm_splitk",
 )
 
 _lib = None
@@ -143,6 +144,7 @@ def load() -> ctypes.CDLL:
         L.odl_fp8_mx_cast.argtypes = [vp, i32, i64, i64, i32, vp, vp, i32, vp, vp, i32, vp]
         L.odl_fp8_mx_gemm_nt.argtypes = [vp, vp, vp, vp, i32, i64, i64, i64, i32, i32, vp, vp, i32, vp]
         L.odl_fp8_block_cast.argtypes = [vp, i32, i64, i64, i32, i32, i32, vp, vp, vp, vp, vp]
+        L.odl_fp8_mx_gemm_splitk.argtypes = [vp, vp, vp, vp, i64, i64, i64, i32, i32, vp, vp, i32, i32, vp, i64, vp]
         for name in EXPORTS:
             getattr(L, name)  # AttributeError here = the library does not match the header
         if L.odl_fp8_abi_version() != ABI_VERSION:
@@ -828,6 +830,14 @@ def mx_gemm_nt(a: torch.Tensor, sa: torch.Tensor, b: torch.Tensor, sb: torch.Ten
     if odt is None:
         raise NativeError(f"mx_gemm_nt: output dtype {out_dtype} is not supported (bf16 or fp32)")
     out = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    # outputs of few tiles with a long contraction: K in runs side by side, like gemm_nt
+    splits = gemm_split_count(M, N, K) if layout == MX_KSTEP else 1
+    if splits > 1:
+        workspace = torch.empty((splits, M, N), dtype=torch.float32, device=a.device)
+        _check(load().odl_fp8_mx_gemm_splitk(a.data_ptr(), sa.data_ptr(), b.data_ptr(), sb.data_ptr(), M, N, K, fmt_a, fmt_b,
+                                             bias.data_ptr() if bias is not None else None, out.data_ptr(), odt, splits,
+                                             workspace.data_ptr(), workspace.numel() * 4, _stream()), "odl_fp8_mx_gemm_splitk")
+        return out
     _check(load().odl_fp8_mx_gemm_nt(a.data_ptr(), sa.data_ptr(), b.data_ptr(), sb.data_ptr(), layout, M, N, K, fmt_a, fmt_b,
                                      bias.data_ptr() if bias is not None else None, out.data_ptr(), odt, _stream()),
            "odl_fp8_mx_gemm_nt")

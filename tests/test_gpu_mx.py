@@ -375,3 +375,36 @@ def test_mxfp8_shared_input_is_quantised_once():
     with recipe.backward():
         (ya.sum() + yb.sum()).backward()
     assert x.grad is not None and a.weight.grad is not None and b.weight.grad is not None
+
+
+@pytest.mark.parametrize("shape", [(768, 768, 16384), (2304, 768, 16384), (1024, 1024, 16384)])
+def test_mx_gemm_split_over_k_matches_the_single_launch(N, shape):
+    """Weight-gradient shapes of small models: few output tiles, a long contraction.  The wrapper cuts K into runs
+    (odl_fp8_mx_gemm_splitk); the result is the emulated product, and equal to a single launch up to fp32 rounding of
+    the partial sums."""
+    M, N_, K = shape
+    a = seeded_bf16((M, K), 1e-3, 31)
+    b = seeded_bf16((N_, K), 1.0, 32)
+    aq, asc, _, _ = N.mx_cast(a.cuda(), E5M2, True, False)
+    bq, bsc, _, _ = N.mx_cast(b.cuda(), E4M3, True, False)
+    assert N.gemm_split_count(M, N_, K) > 1, "the shape is meant to be split"
+    bias = torch.randn(N_).cuda()
+    real = N.load().odl_fp8_mx_gemm_splitk
+    got = N.mx_gemm_nt(aq, asc, bq, bsc, E5M2, E4M3, bias=bias, out_dtype=torch.float32)
+    N.split_k = False
+    try:
+        single = N.mx_gemm_nt(aq, asc, bq, bsc, E5M2, E4M3, bias=bias, out_dtype=torch.float32)
+    finally:
+        N.split_k = True
+    assert max_rel_err(got.cpu(), single.cpu()) <= 1e-5
+    ref = O.t_mx_gemm_nt(aq.cpu(), N.mx_scales_rowmajor(asc).cpu(), bq.cpu(), N.mx_scales_rowmajor(bsc).cpu(), E5M2, E4M3,
+                         bias=bias.cpu(), want_f32=True)[1]
+    assert max_rel_err(got.cpu(), ref) <= 1e-3
+    gotb = N.mx_gemm_nt(aq, asc, bq, bsc, E5M2, E4M3, bias=bias)
+    assert torch.equal(gotb, got.bfloat16())
+    # called directly with a workspace that is too small: refused
+    ws = torch.empty(16, dtype=torch.float32, device="cuda")
+    out = torch.empty((M, N_), dtype=torch.float32, device="cuda")
+    rc = real(aq.data_ptr(), asc.data_ptr(), bq.data_ptr(), bsc.data_ptr(), M, N_, K, E5M2, E4M3, None, out.data_ptr(), 1, 4,
+              ws.data_ptr(), 64, None)
+    assert rc != 0
