@@ -130,3 +130,34 @@ def test_split_count_is_a_host_side_decision_with_the_documented_shape_rules():
         assert per >= 8 and steps - (s - 1) * per >= 4                        # no run shorter than 512
     for M, N, K in ((300, 512, 8192), (768, 768, 1024), (768, 776, 16384), (768, 768, 16400), (0, 768, 16384)):
         assert count(M, N, K) == 1                          # not multiples of 128, or too short to split
+
+
+def test_block_scaled_entry_points_refuse_bad_arguments_before_touching_a_device():
+    """Argument and shape checks of the MXFP8 / blockwise entry points are host code that runs before any HIP call: they
+    answer with an error code and a message here, where no GPU exists."""
+    from optimus_dl_amd import native
+
+    if not native.is_built():
+        pytest.skip("library not built")
+    L = native.load()
+    err = lambda: L.odl_fp8_last_error().decode()
+    p = 4096                                                     # any aligned non-null address: it is never dereferenced
+    # cast: negative shape, unknown format, scale bytes without codes, blocked axis not a multiple of 32 / of 128
+    assert L.odl_fp8_mx_cast(p, 0, -1, 64, 0, p, p, 0, None, None, 0, None) != 0 and "negative" in err()
+    assert L.odl_fp8_mx_cast(p, 0, 64, 64, 7, p, p, 0, None, None, 0, None) != 0 and "fmt" in err()
+    assert L.odl_fp8_mx_cast(p, 0, 64, 64, 0, p, None, 0, None, None, 0, None) != 0 and "go together" in err()
+    assert L.odl_fp8_mx_cast(p, 0, 64, 48, 0, p, p, 0, None, None, 0, None) != 0 and "multiple of 32" in err()
+    assert L.odl_fp8_mx_cast(p, 0, 64, 64, 0, p, p, 1, None, None, 0, None) != 0 and "multiple of 128" in err()
+    assert L.odl_fp8_mx_cast(p, 0, 0, 64, 0, None, None, 0, None, None, 0, None) == 0           # nothing to do
+    # GEMM: K not a multiple of 32, unknown layout, K-step-major scales with K % 128 != 0, misaligned operand
+    assert L.odl_fp8_mx_gemm_nt(p, p, p, p, 0, 64, 64, 48, 0, 0, None, p, 0, None) != 0 and "multiple of 32" in err()
+    assert L.odl_fp8_mx_gemm_nt(p, p, p, p, 5, 64, 64, 64, 0, 0, None, p, 0, None) != 0 and "scales_layout" in err()
+    assert L.odl_fp8_mx_gemm_nt(p, p, p, p, 1, 64, 64, 64, 0, 0, None, p, 0, None) != 0 and "128" in err()
+    assert L.odl_fp8_mx_gemm_nt(p + 8, p, p, p, 0, 64, 64, 64, 0, 0, None, p, 0, None) != 0 and "aligned" in err()
+    assert L.odl_fp8_mx_gemm_nt(p, p, p, p, 0, 0, 64, 64, 0, 0, None, p, 0, None) == 0           # empty output
+    # split over K: too few steps per run, workspace too small
+    assert L.odl_fp8_mx_gemm_splitk(p, p, p, p, 256, 256, 1024, 0, 0, None, p, 0, 4, p, 1 << 30, None) != 0 and "shorter than 512" in err()
+    assert L.odl_fp8_mx_gemm_splitk(p, p, p, p, 256, 256, 8192, 0, 0, None, p, 0, 4, p, 64, None) != 0 and "workspace" in err()
+    # blockwise cast: sizes must be multiples of 128, margin in range
+    assert L.odl_fp8_block_cast(p, 0, 128, 192, 0, 0, 0, p, p, None, None, None) != 0 and "multiples of 128" in err()
+    assert L.odl_fp8_block_cast(p, 0, 128, 128, 0, 1000, 0, p, p, None, None, None) != 0 and "margin" in err()
