@@ -219,6 +219,7 @@ def other_configs(torch, steps=8, warmup=3, only=""):
     cases = [
         ("configs[1] attention projections, tensorwise", "tensorwise", {}, [(4096, 4096), (4096, 1024), (4096, 1024), (4096, 4096)], 8192, torch.bfloat16),
         ("configs[2] with fp32 master weights", "tensorwise", {}, [(k, n) for _, k, n in LAYERS], M_TOKENS, torch.float32),
+        ("configs[2] under delayed scaling (history 16; the reference's default recipe)", "delayed", {"amax_history_len": 16}, [(k, n) for _, k, n in LAYERS], M_TOKENS, torch.bfloat16),
         ("configs[2] under mxfp8 (32-element blocks, E8M0 scales, scaled MFMA)", "mxfp8", {}, [(k, n) for _, k, n in LAYERS], M_TOKENS, torch.bfloat16),
         ("configs[2] under blockwise (1x128 / 128x128 blocks, power-of-two scales, scaled MFMA)", "blockwise", {}, [(k, n) for _, k, n in LAYERS], M_TOKENS, torch.bfloat16),
         ("configs[3] rowwise, M=16384", "rowwise", {}, [(4096, 14336)], 16384, torch.bfloat16),
