@@ -85,6 +85,14 @@ __device__ __forceinline__ float scale_rule(float amax, float fp8_max, int margi
     return s;
 }
 
+// The same for values known to hold no NaN (the caller has their amax): no patching.
+template <int FMT>
+__device__ __forceinline__ uint32_t quantise4_finite(float x0, float x1, float x2, float x3, float s0, float s1, float s2, float s3) {
+    uint32_t r = 0;
+    r = cvt_pk<FMT, false>(x0 * s0, x1 * s1, r);
+    return cvt_pk<FMT, true>(x2 * s2, x3 * s3, r);
+}
+
 // |x| bit pattern of a packed pair of bf16, per 16-bit half.  For bf16 (and
 // fp32) the magnitude ordering equals the unsigned ordering of these bits, and
 // every NaN pattern sorts above Inf, so an unsigned max propagates NaN.

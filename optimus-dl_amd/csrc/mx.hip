@@ -137,8 +137,14 @@ __global__ __launch_bounds__(kMxThreads) void mx_cast_kernel(const void *__restr
             if (col_ok && (r0 + i) < rows) {
                 float f[8];
                 widen(i, f);
-                const uint32_t lo = quantise4<FMT>(f[0], f[1], f[2], f[3], mul, mul, mul, mul);
-                const uint32_t hi = quantise4<FMT>(f[4], f[5], f[6], f[7], mul, mul, mul, mul);
+                uint32_t lo, hi;
+                if (__builtin_expect(m >= 0x7f800000u, 0)) {            // only a block whose amax is Inf / NaN can hold a NaN
+                    lo = quantise4<FMT>(f[0], f[1], f[2], f[3], mul, mul, mul, mul);
+                    hi = quantise4<FMT>(f[4], f[5], f[6], f[7], mul, mul, mul, mul);
+                } else {
+                    lo = quantise4_finite<FMT>(f[0], f[1], f[2], f[3], mul, mul, mul, mul);
+                    hi = quantise4_finite<FMT>(f[4], f[5], f[6], f[7], mul, mul, mul, mul);
+                }
                 *reinterpret_cast<u32x2 *>(out + (r0 + i) * cols + c0) = u32x2{lo, hi};
                 if ((tx & 3) == 0) scales[mx_scale_at(layout, r0 + i, c0 / kMxBlock, rows, nb)] = (uint8_t)byte;
             }
@@ -170,12 +176,25 @@ __global__ __launch_bounds__(kMxThreads) void mx_cast_kernel(const void *__restr
             // rows % 32 == 0 (host-checked): a row block is inside the matrix as a whole or not at all
             if ((ty & 7) == 0 && col_ok && r0 < rows) scales_t[mx_scale_at(layout_t, c0 + j, r0 / kMxBlock, cols, nbt)] = (uint8_t)byte;
         }
+        uint32_t worst = 0;                                              // Inf / NaN in any of the lane's 8 column blocks?
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            float f[8];
-            widen(i, f);
-            lo[i] = quantise4<FMT>(f[0], f[1], f[2], f[3], mul_c[0], mul_c[1], mul_c[2], mul_c[3]);
-            hi[i] = quantise4<FMT>(f[4], f[5], f[6], f[7], mul_c[4], mul_c[5], mul_c[6], mul_c[7]);
+        for (int j = 0; j < 8; ++j) worst = max(worst, cmax[j]);
+        if (__builtin_expect(worst >= 0x7f800000u, 0)) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float f[8];
+                widen(i, f);
+                lo[i] = quantise4<FMT>(f[0], f[1], f[2], f[3], mul_c[0], mul_c[1], mul_c[2], mul_c[3]);
+                hi[i] = quantise4<FMT>(f[4], f[5], f[6], f[7], mul_c[4], mul_c[5], mul_c[6], mul_c[7]);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float f[8];
+                widen(i, f);
+                lo[i] = quantise4_finite<FMT>(f[0], f[1], f[2], f[3], mul_c[0], mul_c[1], mul_c[2], mul_c[3]);
+                hi[i] = quantise4_finite<FMT>(f[4], f[5], f[6], f[7], mul_c[4], mul_c[5], mul_c[6], mul_c[7]);
+            }
         }
         uint32_t tl[4], th[4];
         transpose4x4(lo, tl);
