@@ -247,7 +247,7 @@ __global__ __launch_bounds__(256) void block_cast_kernel(const void *__restrict_
                                                          uint8_t *__restrict__ out, uint32_t *__restrict__ scales,
                                                          uint8_t *__restrict__ out_t, uint32_t *__restrict__ scales_t) {
     __shared__ __attribute__((aligned(16))) uint8_t tile[WANT_COL ? 128 * 128 : 16];
-    __shared__ uint32_t red[4][128];                 // per wave: column maxima (1-D), or slot 0: the wave's maximum (2-D)
+    __shared__ __attribute__((aligned(8))) uint32_t red[4][128];   // per wave: column maxima (1-D), or slot 0: the wave's maximum (2-D)
     __shared__ __attribute__((aligned(16))) float col_mul[128];
     constexpr int ESZ = SRC == ODL_BF16 ? 2 : 4, DW = 16 * ESZ / 4;
     const int tx = threadIdx.x % 8, ty = threadIdx.x / 8, wave = threadIdx.x / 64;
@@ -331,14 +331,16 @@ __global__ __launch_bounds__(256) void block_cast_kernel(const void *__restrict_
 #pragma unroll
             for (int d = 0; d < DW; ++d) {
                 uint32_t m;
+                // after the exchange all 8 lanes with this tx hold the maximum: each of them stores one eighth of the 16
+                // columns (an 8-byte store), instead of one lane storing all of them through the same few banks
                 if constexpr (SRC == ODL_BF16) {
                     m = max_u16x2(max_u16x2(abs_bf16x2(raw[0][d]), abs_bf16x2(raw[1][d])), max_u16x2(abs_bf16x2(raw[2][d]), abs_bf16x2(raw[3][d])));
                     m = max_stride8_u16x2(m);
-                    if ((ty & 7) == 0) { red[wave][16 * tx + 2 * d] = m << 16; red[wave][16 * tx + 2 * d + 1] = m & 0xffff0000u; }
+                    if ((ty & 7) == d) *reinterpret_cast<u32x2 *>(&red[wave][16 * tx + 2 * d]) = u32x2{m << 16, m & 0xffff0000u};
                 } else {
                     m = max(max(raw[0][d] & 0x7fffffffu, raw[1][d] & 0x7fffffffu), max(raw[2][d] & 0x7fffffffu, raw[3][d] & 0x7fffffffu));
                     m = max_stride8(m);
-                    if ((ty & 7) == 0) red[wave][16 * tx + d] = m;
+                    if ((ty & 7) == d / 2) red[wave][16 * tx + d] = m;
                 }
             }
             __syncthreads();
