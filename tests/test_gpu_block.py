@@ -161,3 +161,30 @@ def test_blockwise_round_trip_at_full_size(N):
     deq_t = O.t_mx_dequantise(out_t.cpu(), O.block_scales_as_mx(_bytes(sc_t), 1, 128), E4M3)
     vt = x.t().float().reshape(cols, rows // 128, 128)
     assert bool(((deq_t.reshape(cols, rows // 128, 128) - vt).abs() <= vt.abs().amax(dim=2, keepdim=True) * 2.0 ** -4).all())
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_seeded_random_block_scaled_linears_match_the_emulation(seed):
+    """Random shapes (multiples of 128, so that both block-scaled recipes take them), recipe, format and data scale:
+    forward, dgrad and wgrad of the module against the emulated block-scaled Linear."""
+    import random
+
+    from optimus_dl_amd.modules import amp
+    from tests.test_gpu_linear import make_linear, run_step
+    from tests.test_gpu_mx import _mx_linear_reference
+
+    rng = random.Random(seed)
+    M, K, N_ = (128 * rng.randint(1, 6) for _ in range(3))
+    recipe_name, fmt = rng.choice(["mxfp8", "blockwise"]), rng.choice(["hybrid", "e4m3"])
+    x = seeded_bf16((M, K), 10.0 ** rng.uniform(-2, 2), 3 * seed)
+    w = seeded_bf16((N_, K), 10.0 ** rng.uniform(-3, 0), 3 * seed + 1)
+    dy = seeded_bf16((M, N_), 10.0 ** rng.uniform(-5, 0), 3 * seed + 2)
+    x[:, rng.randrange(K)] *= 30.0
+    lin = make_linear(w)
+    y, dx, dw = run_step(lin, amp.create_fp8_recipe(recipe_name, fmt), x, dy)
+    assert lin.fp8_calls == 1
+    fb = O.E5M2 if fmt == "hybrid" else O.E4M3
+    ref = _mx_linear_reference(x, w, dy, O.E4M3, fb) if recipe_name == "mxfp8" else _block_linear_reference(x, w, dy, O.E4M3, fb)
+    for name, got in (("y", y), ("dx", dx), ("dw", dw)):
+        err = max_rel_err(got, ref[name])
+        assert err <= 1e-2, f"seed {seed} {recipe_name} {fmt} {M}x{K}x{N_} {name}: {err}"
