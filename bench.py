@@ -56,6 +56,17 @@ def gemm_traffic_bytes_per_launch():
     return kib * 1024.0 / n, t["source"]
 
 
+def profiled_kernel_durations():
+    """Average kernel durations inside the step from the tracked rocprofv3 summary (kernel time only: no launch gap, no
+    event), as recorded in profiles/step_kernel_durations__cfg3_mlp.json; ({}, None) when the file is not there."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "step_kernel_durations__cfg3_mlp.json")) as fh:
+            t = json.load(fh)
+    except OSError:
+        return {}, None
+    return {k: v["avg_us"] for k, v in t["kernels"].items()}, t["source"]
+
+
 M_TOKENS, D_MODEL, D_FF = 8192, 4096, 14336
 LAYERS = (("gate", D_MODEL, D_FF), ("up", D_MODEL, D_FF), ("down", D_FF, D_MODEL))   # name, K(in), N(out)
 
@@ -665,6 +676,16 @@ def main() -> int:
             gbps = ks[name]["work"] / (ks[name]["total_ms"] * 1e-3) / 1e9
             hbm[name] = {"achieved": gbps, "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": gbps / PEAK_HBM_GBPS,
                          "avg_us": ks[name]["avg_us"], "launches": ks[name]["launches"]}
+    # the same kernels by the tracked profile's kernel durations (what rocprofv3 saw inside the step on the box it ran on)
+    prof_us, prof_src = profiled_kernel_durations()
+    prof_bytes = prof_time = 0.0
+    for name in hbm:
+        if name in prof_us:
+            per_launch = ks[name]["work"] / ks[name]["launches"]
+            hbm[name]["by_profiled_kernel_time"] = {"avg_us": prof_us[name], "GB/s": per_launch / (prof_us[name] * 1e-6) / 1e9,
+                                                    "frac": per_launch / (prof_us[name] * 1e-6) / 1e9 / PEAK_HBM_GBPS}
+            prof_bytes += ks[name]["work"]
+            prof_time += prof_us[name] * 1e-6 * ks[name]["launches"]
     quant_bytes = sum(ks[n]["work"] for n in ("amax", "cast", "cast_transpose") if n in ks)
     quant_ms = sum(ks[n]["total_ms"] for n in ("amax", "cast", "cast_transpose") if n in ks)
 
@@ -692,6 +713,8 @@ def main() -> int:
         "gemm_only_tflops": gemm_tflops,
         "cast_amax_gbps": quant_bytes / (quant_ms * 1e-3) / 1e9 if quant_ms else None,
         "cast_amax_frac_of_hbm_peak": (quant_bytes / (quant_ms * 1e-3) / 1e9) / PEAK_HBM_GBPS if quant_ms else None,
+        "cast_amax_frac_of_hbm_peak_by_profiled_kernel_time": (prof_bytes / prof_time / 1e9 / PEAK_HBM_GBPS) if prof_time else None,
+        "profiled_kernel_time_source": prof_src,
         "time_split_ms_per_step": {n: ks[n]["total_ms"] / args.steps for n in ks},
         "ms_per_step_with_kernel_events": 1e3 * wall_instrumented / args.steps,
         "roofline": {
