@@ -205,15 +205,17 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
         ia = tm0 + sc_region < (int)g.M ? 1 : 0;
         ib = tn0 + sc_region < (int)g.N ? 1 : 0;
     };
+    // one operand's 64 scale dwords of a K step (which: 0 = A, 1 = B)
+    auto issue_scale = [&](int which, int stage, int ok, int off, int kstep) {
+        v4i d = which ? whole_sb : whole_sa;
+        d.z = __builtin_amdgcn_readfirstlane(d.z * ok);
+        off = __builtin_amdgcn_readfirstlane(off);
+        const uint32_t dst = lds_addr_of(reinterpret_cast<const uint8_t *>(sScale)) + (stage * 512 + which * 256 + 64 * wave) * 4;
+        dma4(d, dst, sc_voff, off + kstep * (int)(which ? g.N : g.M) * 4);
+    };
     auto issue_scales = [&](int stage, int ok_a, int ok_b, int off_a, int off_b, int kstep) {
-        v4i da = whole_sa, db = whole_sb;
-        da.z = __builtin_amdgcn_readfirstlane(whole_sa.z * ok_a);
-        db.z = __builtin_amdgcn_readfirstlane(whole_sb.z * ok_b);
-        off_a = __builtin_amdgcn_readfirstlane(off_a);
-        off_b = __builtin_amdgcn_readfirstlane(off_b);
-        const uint32_t dst = lds_addr_of(reinterpret_cast<const uint8_t *>(sScale)) + (stage * 512 + 64 * wave) * 4;
-        dma4(da, dst, sc_voff, off_a + kstep * (int)g.M * 4);
-        dma4(db, dst + 1024, sc_voff, off_b + kstep * (int)g.N * 4);
+        issue_scale(0, stage, ok_a, off_a, kstep);
+        issue_scale(1, stage, ok_b, off_b, kstep);
     };
     int sca[2][4] = {}, scb[2][4] = {};           // [K step parity][fragment]: this lane's scale dwords, already shifted
     // in two parts, so that the shift (which waits for the data) can sit a few MFMAs after the read
@@ -223,12 +225,17 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
         sc_raw_a = *reinterpret_cast<const v4i *>(base + 128 * (wave / 2) + 4 * lr);
         sc_raw_b = *reinterpret_cast<const v4i *>(base + 256 + 128 * (wave % 2) + 4 * lr);
     };
-    auto place_scales = [&](int (&ea)[4], int (&eb)[4]) {
+    auto place_a = [&](int (&ea)[4]) {
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            ea[t] = (int)((uint32_t)sc_raw_a[t] >> (8 * lg));
-            eb[t] = (int)((uint32_t)sc_raw_b[t] >> (8 * lg));
-        }
+        for (int t = 0; t < 4; ++t) ea[t] = (int)((uint32_t)sc_raw_a[t] >> (8 * lg));
+    };
+    auto place_b = [&](int (&eb)[4]) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) eb[t] = (int)((uint32_t)sc_raw_b[t] >> (8 * lg));
+    };
+    auto place_scales = [&](int (&ea)[4], int (&eb)[4]) {
+        place_a(ea);
+        place_b(eb);
     };
     auto read_scales = [&](int stage, int (&ea)[4], int (&eb)[4]) {
         fetch_scales(stage);
@@ -486,13 +493,14 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
             if constexpr (MX) {
                 // the scales of step kt + 1 arrived with its operands; those of the step requested above go to the stage
                 // whose dwords every wave read one phase B ago
+                // spread over the MFMA slots that carry no fragment reads (i >= 8), one small piece each: a slot has room
+                // for about a dozen instructions beside its MFMA
+                const int live = pad && !nx ? 0 : 1;
                 if (i == 8) fetch_scales(par ^ 1);
-                if (i == 13) place_scales(sca[par ^ 1], scb[par ^ 1]);
-                if (i == 0) {          // first: the youngest load of a step is the one the next barrier waits for longest
-                    const int live = pad && !nx ? 0 : 1;
-                    issue_scales(par, (nx ? sc_nin_a : sc_in_a) * live, (nx ? sc_nin_b : sc_in_b) * live,
-                                 nx ? sc_next_a : sc_off_a, nx ? sc_next_b : sc_off_b, koff);
-                }
+                if (i == 9) issue_scale(0, par, (nx ? sc_nin_a : sc_in_a) * live, nx ? sc_next_a : sc_off_a, koff);
+                if (i == 10) issue_scale(1, par, (nx ? sc_nin_b : sc_in_b) * live, nx ? sc_next_b : sc_off_b, koff);
+                if (i == 12) place_a(sca[par ^ 1]);
+                if (i == 14) place_b(scb[par ^ 1]);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
