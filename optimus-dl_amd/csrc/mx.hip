@@ -1,11 +1,17 @@
-// MXFP8 on gfx950: blocks of 32 consecutive elements along the contraction axis share a power-of-two scale (one
-// E8M0 byte, value 2^(byte - 127)), and the MFMA applies the scales itself (V_MFMA_SCALE_F32_32X32X64_F8F6F4: a lane
-// feeds 32 K-bytes of one row, which is exactly one block, together with that block's scale byte).
+// Block-scaled FP8 on gfx950.  MXFP8: blocks of 32 consecutive elements along the contraction axis share a power-of-two
+// scale (one E8M0 byte, value 2^(byte - 127)), and the MFMA applies the scales itself (V_MFMA_SCALE_F32_32X32X64_F8F6F4:
+// the 64 K-bytes of a row that one instruction consumes are two blocks, each with its scale byte).  The blockwise recipe
+// (128-element and 128 x 128 blocks with power-of-two scales) rides on the same GEMMs: its cast writes every block's byte
+// four times.
 //
-//   odl_fp8_mx_cast    : x [rows, cols] -> codes + scale bytes with the blocks along the columns (`out`, `scales`)
-//                        and / or, transposed, with the blocks along the rows (`out_t`, `scales_t`); one pass over x,
-//                        no amax pass before it: the scale of a block is found inside the tile.
-//   odl_fp8_mx_gemm_nt : C[M, N] = sum over blocks kb of 2^(sa[m, kb] + sb[n, kb] - 254) * dot(A[m, kb], B[n, kb])
+//   odl_fp8_mx_cast       : x [rows, cols] -> codes + scale bytes with the blocks along the columns (`out`, `scales`)
+//                           and / or, transposed, with the blocks along the rows (`out_t`, `scales_t`); one pass over x,
+//                           no amax pass before it: the scale of a block is found inside the tile.
+//   odl_fp8_block_cast    : the same for the blockwise recipe.
+//   odl_fp8_mx_gemm_nt    : C[M, N] = sum over blocks kb of 2^(sa[m, kb] + sb[n, kb] - 254) * dot(A[m, kb], B[n, kb]); the
+//                           streaming kernel of gemm_stream.hip with block scales where the shape allows, else the
+//                           tiled or the plain kernel of this file.
+//   odl_fp8_mx_gemm_splitk: the same with K cut into runs (outputs of few tiles).
 //
 // Operand layout of the instruction, measured (one nonzero byte at a time against two different block scales): of the
 // 8 registers a lane supplies for row (lane % 32), registers 0..3 are the 16 K-bytes [16 g, 16 g + 16) and registers
