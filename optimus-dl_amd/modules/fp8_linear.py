@@ -435,7 +435,7 @@ class FP8Linear(nn.Linear):
     def _rowwise_weight(self, weight: torch.Tensor, pol, axis: str, both: bool = False):
         """Rowwise recipe: W scaled per output channel (fwd) or per input channel, transposed (dgrad).
         both: the other one will be asked for too (a backward follows): make them in one go."""
-        key = (weight.data_ptr(), _state.tensor_version(weight))
+        key = _weight_key(weight, pol.fmt_fwd, ("rowwise", pol.margin))
         hit = self._wcache_rowwise.get(axis)
         if hit is not None and hit[0] == key:
             return hit[1], hit[2]
