@@ -20,6 +20,7 @@ event each, adding up to the step); the events cost about 2 % of a step, reporte
 
 Prints ONE JSON line: whole-step TFLOP/s, the GEMM kernel's MFMA roofline
 fraction, the HBM rates of the memory-bound kernels inside the step and on their own,
+the clock and the board power under the GEMM (`clock_probe`, `power_probe`: the board's own sensor against its limit),
 and the same arithmetic on the host CPU (the oracle, on a bounded sample) as a
 reported baseline.
 """
@@ -148,6 +149,109 @@ def make_inputs(torch, m=M_TOKENS, device="cuda"):
             "dy": (torch.randn(m, n, generator=g) * 1e-3).bfloat16().to(device),
         }
     return data
+
+
+def power_probe(torch, native, step=None, seconds=1.5):
+    """The board's own power reading (amdgpu hwmon `power1_input`, microwatts, a value the driver filters over a few
+    tenths of a second; `power1_cap` is the limit it regulates to) while one kind of work runs back to back for
+    `seconds`: the GEMM on Gaussian and on zero operands, the MXFP8 GEMM, the register-only MFMA loop, the three
+    memory-bound kernels and (step given) whole steps of the benchmark.  Per workload: the mean of the readings of the last
+    third of the run, the time per launch, and the energy per launch = watts x time (for the GEMM and the loop also
+    per flop).  Read-only; {"sensor": None} where the file is not there."""
+    import ctypes
+    import glob
+    import threading
+
+    from optimus_dl_amd.build import PROBE_LIB_PATH
+
+    sensors = sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input"))
+    if not sensors:
+        return {"sensor": None}
+    sensor = sensors[0]
+
+    def watts(path=sensor):
+        try:
+            with open(path) as fh:
+                return int(fh.read()) / 1e6
+        except (OSError, ValueError):
+            return None
+
+    if watts() is None:
+        return {"sensor": None}
+    out = {"sensor": sensor, "cap_w": watts(os.path.join(os.path.dirname(sensor), "power1_cap")), "seconds_per_workload": seconds,
+           "workloads": {}}
+    torch.cuda.synchronize()
+    time.sleep(0.8)
+    out["idle_w"] = round(watts(), 1)
+
+    def run(label, fn, flop=None, burst=32):
+        # the sensor is read by a second thread (a read takes the driver some 0.1 ms and must not sit between launches)
+        reads, done = [], threading.Event()
+
+        def sample():
+            while not done.is_set():
+                reads.append((time.perf_counter(), watts()))
+                time.sleep(0.005)
+
+        torch.cuda.synchronize()
+        th = threading.Thread(target=sample, daemon=True)
+        t0 = time.perf_counter()
+        th.start()
+        n = 0
+        while time.perf_counter() - t0 < seconds:
+            for _ in range(burst):
+                fn()
+            torch.cuda.synchronize()
+            n += burst
+        dt = time.perf_counter() - t0
+        done.set()
+        th.join()
+        tail = [w for t, w in reads if t0 + 2.0 * seconds / 3.0 <= t <= t0 + dt and w is not None]
+        w = sum(tail) / len(tail) if tail else None
+        us = 1e6 * dt / n
+        entry = {"watts": round(w, 1) if w is not None else None, "us_per_launch": round(us, 1), "launches": n,
+                 "joules_per_launch": round(w * us * 1e-6, 4) if w is not None else None}
+        if flop and w is not None:
+            entry["pj_per_flop"] = round(w * us * 1e-6 / flop * 1e12, 4)
+        out["workloads"][label] = entry
+        time.sleep(0.5)          # the reading falls back towards idle before the next workload starts
+
+    M, N, K = M_TOKENS, D_FF, D_MODEL
+    g = torch.Generator(device="cuda").manual_seed(0)
+    x = torch.randn((M, K), generator=g, device="cuda").bfloat16()
+    w = (torch.randn((N, K), generator=g, device="cuda") * 0.02).bfloat16()
+    xq, _, _, _, sx = native.quantize_dynamic(x, native.E4M3, 0, want_transposed=False)
+    wq, _, _, _, sw = native.quantize_dynamic(w, native.E4M3, 0, want_transposed=False)
+    c = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+    flop = 2.0 * M * N * K
+    run("gemm_8192x14336x4096 gaussian_operands", lambda: native.gemm_nt(xq, wq, native.E4M3, native.E4M3, sx, sw, out=c), flop)
+    zx, zw = torch.zeros_like(xq), torch.zeros_like(wq)
+    run("gemm_8192x14336x4096 zero_operands", lambda: native.gemm_nt(zx, zw, native.E4M3, native.E4M3, sx, sw, out=c), flop)
+    del zx, zw
+    xm, xs, _, _ = native.mx_cast(x, native.E4M3)
+    wm, ws, _, _ = native.mx_cast(w, native.E4M3)
+    run("gemm_8192x14336x4096 mxfp8_gaussian_operands", lambda: native.mx_gemm_nt(xm, xs, wm, ws, native.E4M3, native.E4M3), flop)
+    del xm, xs, wm, ws, xq, wq, c
+    lib = ctypes.CDLL(PROBE_LIB_PATH)
+    vp = ctypes.c_void_p
+    lib.odl_probe_mfma_loop.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, vp, vp]
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    sink = torch.zeros(1, device="cuda")
+    cycles = torch.zeros((cus, 2), dtype=torch.int64, device="cuda")
+    iters = 4000
+    loop_flop = cus * 4 * iters * 16 * 2.0 * 32 * 32 * 64
+    stream = torch.cuda.current_stream().cuda_stream
+    for label, rnd in (("mfma_register_loop gaussian_like_operands", 1), ("mfma_register_loop zero_operands", 0)):
+        run(label, lambda: lib.odl_probe_mfma_loop(rnd, iters, cus, sink.data_ptr(), cycles.data_ptr(), stream), loop_flop, burst=4)
+    big = torch.randn((M_TOKENS, D_FF), generator=g, device="cuda").bfloat16()
+    one = torch.ones(1, device="cuda")
+    run("amax 8192x14336", lambda: native.amax_parts(big), burst=128)
+    run("cast 8192x14336", lambda: native.cast(big, one, native.E5M2), burst=64)
+    run("cast_transpose 8192x14336", lambda: native.cast_transpose(big, one, native.E4M3, want_rowmajor=True), burst=64)
+    del big
+    if step is not None:
+        run("whole step (configs[2], tensorwise)", step, step_flops(), burst=4)
+    return out
 
 
 def standalone_hbm(torch, native, iters=24):
@@ -584,6 +688,8 @@ def main() -> int:
                          "delayed) and print them (for profiling)")
     ap.add_argument("--clock-probe-only", action="store_true",
                     help="run only the clock probe (GEMM back to back on Gaussian / zero operands, register-only MFMA loop) and print it")
+    ap.add_argument("--power-probe-only", action="store_true",
+                    help="run only the board-power probe (GEMM, MFMA loop, memory-bound kernels, whole steps back to back) and print it")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy (reference kernel for scaling FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -650,6 +756,9 @@ def main() -> int:
     for _ in range(args.warmup):
         one_step()
     torch.cuda.synchronize()
+    if args.power_probe_only:
+        print(json.dumps({"power_probe": power_probe(torch, native, step=one_step)}))
+        return 0
     # the timed region: exactly `steps` steps, nothing else on the stream
     t0 = time.perf_counter()
     for _ in range(args.steps):
@@ -740,6 +849,8 @@ def main() -> int:
         # the same GEMM back to back with the clock measured: what the roofline fraction is at the clock the board grants
         line["roofline"]["granted_clock"] = line["clock_probe"]["gemm_8192x14336x4096"]["gaussian_operands"]
         line["hbm_kernels_standalone"] = standalone_hbm(torch, native)
+        # what the board draws under each kind of work, against the limit it regulates to
+        line["power_probe"] = power_probe(torch, native, step=one_step)
     if not args.no_standalone:
         del layers, data
         line["mlp_block_fwd_bwd"] = mlp_block(torch, native, recipe)
