@@ -167,7 +167,18 @@ def power_probe(torch, native, step=None, seconds=1.5):
     sensors = sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input"))
     if not sensors:
         return {"sensor": None}
-    sensor = sensors[0]
+    # the card whose PCI address is that of the device the work runs on (a host may hold several boards)
+    sensor, matched = sensors[0], len(sensors) == 1
+    try:
+        pr = torch.cuda.get_device_properties(torch.cuda.current_device())
+        want = f"{pr.pci_domain_id:04x}:{pr.pci_bus_id:02x}:{pr.pci_device_id:02x}."
+        for cand in sensors:
+            pci = os.path.basename(os.path.realpath(os.path.join(os.path.dirname(cand), "..", "..")))
+            if pci.startswith(want):
+                sensor, matched = cand, True
+                break
+    except (AttributeError, OSError):
+        pass
 
     def watts(path=sensor):
         try:
@@ -178,7 +189,7 @@ def power_probe(torch, native, step=None, seconds=1.5):
 
     if watts() is None:
         return {"sensor": None}
-    out = {"sensor": sensor, "cap_w": watts(os.path.join(os.path.dirname(sensor), "power1_cap")), "seconds_per_workload": seconds,
+    out = {"sensor": sensor, "sensor_is_this_device": matched, "cap_w": watts(os.path.join(os.path.dirname(sensor), "power1_cap")), "seconds_per_workload": seconds,
            "workloads": {}}
     torch.cuda.synchronize()
     time.sleep(0.8)
