@@ -91,6 +91,27 @@ def check_asm_hazards(asm_text: str, name: str = "") -> list[str]:
     return problems
 
 
+def check_saturating_conversions(asm_text: str, name: str = "") -> list[str]:
+    """The block-scaled casts rely on the scaled FP8 conversions of gfx950 saturating, which they do only while the
+    wave's MODE.FP16_OVFL bit is set; the kernels set it first thing.  Nothing ties the conversions to that
+    ``s_setreg`` in the compiler's eyes, so the order is checked in the generated code: inside every function, no
+    ``v_cvt_scalef32_pk_*`` before the mode has been set."""
+    problems = []
+    func, mode_set = "", False
+    for i, raw in enumerate(asm_text.split("\n")):
+        text = raw.strip()
+        m = re.match(r"^(_Z\w+):", raw)
+        if m:
+            func, mode_set = m.group(1), False
+            continue
+        if text.startswith("s_setreg_imm32_b32 hwreg(HW_REG_MODE, 23, 1), 1"):
+            mode_set = True
+        elif text.startswith("v_cvt_scalef32_pk_") and not mode_set:
+            problems.append(f"{name}:{i + 1}: '{text}' in {func} before MODE.FP16_OVFL is set")
+            mode_set = True          # one report per function
+    return problems
+
+
 def build(verbose: bool = False, keep_asm: bool = False) -> str:
     """Compile every source and link ``libodl_fp8.so``.  Always recompiles."""
     hipcc = hipcc_path()
@@ -117,9 +138,11 @@ def build(verbose: bool = False, keep_asm: bool = False) -> str:
     problems = []
     for asm in sorted(glob.glob(os.path.join(objdir, "*gfx950*.s"))):
         with open(asm) as fh:
-            problems += check_asm_hazards(fh.read(), os.path.basename(asm))
+            text = fh.read()
+        problems += check_asm_hazards(text, os.path.basename(asm))
+        problems += check_saturating_conversions(text, os.path.basename(asm))
     if problems:
-        raise RuntimeError("inline-asm hazards in the generated code:\n" + "\n".join(problems))
+        raise RuntimeError("hazards in the generated code:\n" + "\n".join(problems))
     if not keep_asm:
         for tmpf in glob.glob(os.path.join(objdir, "*")):
             if not tmpf.endswith(".o"):

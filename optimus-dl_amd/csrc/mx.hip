@@ -85,6 +85,46 @@ __device__ __forceinline__ uint32_t max_stride8_u16x2(uint32_t m) {
     return max_u16x2(q[0], q[1]);
 }
 
+// gfx950's scaled conversions: two bf16 (or two floats) divided by 2^(E - 127), E = the exponent field of `scale` (an
+// E8M0 byte sitting where a float keeps its exponent; mantissa and sign are ignored and E = 0 acts as 2^-127), rounded
+// to nearest even into the two FP8 bytes of the low (HIGH = false) or the high half of `old`.  With MODE.FP16_OVFL set
+// (saturate_fp8_conversions) a result beyond the format's largest value becomes that value.  Measured on all 65536
+// bf16 inputs, both sources and both formats, at 16 exponents from 0 to 254: bit for bit round(clamp(v * 2^(127 - E))),
+// the rule of the block-scaled casts, for every input except NaN (0xFF / 0xFE whatever the sign), which the kernels
+// therefore keep away from these instructions.
+typedef short v2i16_t __attribute__((ext_vector_type(2)));
+typedef __bf16 v2bf16_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ void saturate_fp8_conversions() {
+    __builtin_amdgcn_s_setreg(1 | (23 << 6) | (0 << 11), 1);          // hwreg(HW_REG_MODE, 23, 1) = FP16_OVFL, this wave only
+}
+
+template <int FMT, bool HIGH>
+__device__ __forceinline__ uint32_t cvt_scaled_bf16x2(uint32_t old, uint32_t pair, float scale) {
+    const v2i16_t o = __builtin_bit_cast(v2i16_t, old);
+    const v2bf16_t v = __builtin_bit_cast(v2bf16_t, pair);
+    if constexpr (FMT == ODL_FP8_E4M3) return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(o, v, scale, HIGH));
+    else return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf8_bf16(o, v, scale, HIGH));
+}
+
+template <int FMT, bool HIGH>
+__device__ __forceinline__ uint32_t cvt_scaled_f32x2(uint32_t old, float a, float b, float scale) {
+    const v2i16_t o = __builtin_bit_cast(v2i16_t, old);
+    if constexpr (FMT == ODL_FP8_E4M3) return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(o, a, b, scale, HIGH));
+    else return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf8_f32(o, a, b, scale, HIGH));
+}
+
+// four codes from two dwords of bf16 pairs (SRC bf16: p0, p1) or four floats (SRC fp32: p0 .. p3 as bits), one scale
+template <int SRC, int FMT>
+__device__ __forceinline__ uint32_t cvt_scaled4(uint32_t p0, uint32_t p1, uint32_t p2, uint32_t p3, float scale) {
+    if constexpr (SRC == ODL_BF16) {
+        return cvt_scaled_bf16x2<FMT, true>(cvt_scaled_bf16x2<FMT, false>(0u, p0, scale), p1, scale);
+    } else {
+        return cvt_scaled_f32x2<FMT, true>(cvt_scaled_f32x2<FMT, false>(0u, bits_to_float(p0), bits_to_float(p1), scale),
+                                           bits_to_float(p2), bits_to_float(p3), scale);
+    }
+}
+
 // 128 x 64 tile per block of 256 lanes, lane (tx, ty) owns rows 4 ty .. 4 ty + 3 and columns 8 tx .. 8 tx + 7 as in
 // cast_transpose_kernel.  A block along the columns (32 of them) is held by 4 neighbouring lanes; a block along the rows
 // (32 of them) by the 8 lanes of a wave that share tx: both maxima are xor-shuffles inside the wave.
@@ -94,9 +134,18 @@ __global__ __launch_bounds__(kMxThreads) void mx_cast_kernel(const void *__restr
                                                               uint8_t *__restrict__ out_t, uint8_t *__restrict__ scales_t,
                                                               int layout, int layout_t) {
     __shared__ __attribute__((aligned(16))) uint8_t tile[kTileC * kTileR];
+    // K-step-major scale bytes leave the block as whole runs: the tile's 4 row blocks are one dword per column (256
+    // contiguous bytes per tile), its 2 column blocks one 16-bit half of a dword per row.  Stored a byte at a time from
+    // the lanes that hold them they were hundreds of masked one-byte writes per tile and cost a tenth of the kernel.
+    __shared__ __attribute__((aligned(16))) uint8_t stage_t[kTileC * 4];
+    __shared__ __attribute__((aligned(16))) uint8_t stage_r[kTileR * 2];
+    saturate_fp8_conversions();
     constexpr int ESZ = SRC == ODL_BF16 ? 2 : 4;
     const int tx = threadIdx.x % 8, ty = threadIdx.x / 8;
     const int64_t tiles_r = (rows + kTileR - 1) / kTileR, tiles_c = (cols + kTileC - 1) / kTileC;
+    // (K-step-major implies whole dwords: cols % 128 == 0 for `scales`, rows % 128 == 0 for `scales_t`; host-checked)
+    const bool staged_r = WANT_ROW && WANT_COL && layout == ODL_MX_SCALES_KSTEP;
+    const bool staged_t = WANT_COL && layout_t == ODL_MX_SCALES_KSTEP;
     int64_t tr, tc;
     ct_tile_of(blockIdx.x, tiles_r, tiles_c, tr, tc);
     const int64_t r0 = tr * kTileR + ty * 4, c0 = tc * kTileC + tx * 8;
@@ -141,26 +190,34 @@ __global__ __launch_bounds__(kMxThreads) void mx_cast_kernel(const void *__restr
             float mul;
             mx_scale_of<FMT>(m, byte, mul);
             if (col_ok && (r0 + i) < rows) {
-                float f[8];
-                widen(i, f);
                 uint32_t lo, hi;
                 if (__builtin_expect(m >= 0x7f800000u, 0)) {            // only a block whose amax is Inf / NaN can hold a NaN
+                    float f[8];
+                    widen(i, f);
                     lo = quantise4<FMT>(f[0], f[1], f[2], f[3], mul, mul, mul, mul);
                     hi = quantise4<FMT>(f[4], f[5], f[6], f[7], mul, mul, mul, mul);
-                } else {
-                    lo = quantise4_finite<FMT>(f[0], f[1], f[2], f[3], mul, mul, mul, mul);
-                    hi = quantise4_finite<FMT>(f[4], f[5], f[6], f[7], mul, mul, mul, mul);
+                } else {                                                // the hardware divides by 2^(byte - 127) and saturates
+                    const float e8 = bits_to_float(byte << 23);
+                    if constexpr (SRC == ODL_BF16) {
+                        lo = cvt_scaled4<SRC, FMT>(raw[i][0], raw[i][1], 0u, 0u, e8);
+                        hi = cvt_scaled4<SRC, FMT>(raw[i][2], raw[i][3], 0u, 0u, e8);
+                    } else {
+                        lo = cvt_scaled4<SRC, FMT>(raw[i][0], raw[i][1], raw[i][2], raw[i][3], e8);
+                        hi = cvt_scaled4<SRC, FMT>(raw[i][4], raw[i][5], raw[i][6], raw[i][7], e8);
+                    }
                 }
                 *reinterpret_cast<u32x2 *>(out + (r0 + i) * cols + c0) = u32x2{lo, hi};
-                if ((tx & 3) == 0) scales[mx_scale_at(layout, r0 + i, c0 / kMxBlock, rows, nb)] = (uint8_t)byte;
+                if ((tx & 3) == 0) {
+                    if (staged_r) stage_r[(ty * 4 + i) * 2 + tx / 4] = (uint8_t)byte;
+                    else scales[mx_scale_at(layout, r0 + i, c0 / kMxBlock, rows, nb)] = (uint8_t)byte;
+                }
             }
         }
     }
 
     if constexpr (WANT_COL) {
         const int64_t nbt = rows / kMxBlock;
-        uint32_t lo[4] = {0, 0, 0, 0}, hi[4] = {0, 0, 0, 0};
-        float mul_c[8];
+        float mul_c[8], e8_c[8];
         uint32_t cmax[8];                                                // fp32 magnitude bits per column, over the 32 rows
         if constexpr (SRC == ODL_BF16) {
 #pragma unroll
@@ -179,13 +236,19 @@ __global__ __launch_bounds__(kMxThreads) void mx_cast_kernel(const void *__restr
         for (int j = 0; j < 8; ++j) {
             uint32_t byte;
             mx_scale_of<FMT>(cmax[j], byte, mul_c[j]);
+            e8_c[j] = bits_to_float(byte << 23);
             // rows % 32 == 0 (host-checked): a row block is inside the matrix as a whole or not at all
-            if ((ty & 7) == 0 && col_ok && r0 < rows) scales_t[mx_scale_at(layout_t, c0 + j, r0 / kMxBlock, cols, nbt)] = (uint8_t)byte;
+            if ((ty & 7) == 0 && col_ok && r0 < rows) {
+                if (staged_t) stage_t[(tx * 8 + j) * 4 + ty / 8] = (uint8_t)byte;
+                else scales_t[mx_scale_at(layout_t, c0 + j, r0 / kMxBlock, cols, nbt)] = (uint8_t)byte;
+            }
         }
         uint32_t worst = 0;                                              // Inf / NaN in any of the lane's 8 column blocks?
 #pragma unroll
         for (int j = 0; j < 8; ++j) worst = max(worst, cmax[j]);
+        uint32_t tl[4], th[4];                                           // tl[k] / th[k]: rows 4 ty .. + 3 of column k / 4 + k
         if (__builtin_expect(worst >= 0x7f800000u, 0)) {
+            uint32_t lo[4], hi[4];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 float f[8];
@@ -193,18 +256,25 @@ __global__ __launch_bounds__(kMxThreads) void mx_cast_kernel(const void *__restr
                 lo[i] = quantise4<FMT>(f[0], f[1], f[2], f[3], mul_c[0], mul_c[1], mul_c[2], mul_c[3]);
                 hi[i] = quantise4<FMT>(f[4], f[5], f[6], f[7], mul_c[4], mul_c[5], mul_c[6], mul_c[7]);
             }
+            transpose4x4(lo, tl);
+            transpose4x4(hi, th);
         } else {
+            // the four rows of one column side by side are the operands of one pair of conversions: the codes come out
+            // transposed (bf16: the two halves of the rows' dwords are regrouped per column first)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                float f[8];
-                widen(i, f);
-                lo[i] = quantise4_finite<FMT>(f[0], f[1], f[2], f[3], mul_c[0], mul_c[1], mul_c[2], mul_c[3]);
-                hi[i] = quantise4_finite<FMT>(f[4], f[5], f[6], f[7], mul_c[4], mul_c[5], mul_c[6], mul_c[7]);
+            for (int j = 0; j < 8; ++j) {
+                uint32_t t;
+                if constexpr (SRC == ODL_BF16) {
+                    const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
+                    const uint32_t r01 = __builtin_amdgcn_perm(raw[1][j / 2], raw[0][j / 2], sel);
+                    const uint32_t r23 = __builtin_amdgcn_perm(raw[3][j / 2], raw[2][j / 2], sel);
+                    t = cvt_scaled4<SRC, FMT>(r01, r23, 0u, 0u, e8_c[j]);
+                } else {
+                    t = cvt_scaled4<SRC, FMT>(raw[0][j], raw[1][j], raw[2][j], raw[3][j], e8_c[j]);
+                }
+                if (j < 4) tl[j] = t; else th[j - 4] = t;
             }
         }
-        uint32_t tl[4], th[4];
-        transpose4x4(lo, tl);
-        transpose4x4(hi, th);
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
             *reinterpret_cast<uint32_t *>(&tile[ct_lds_write_off(tx * 8 + k, ty)]) = tl[k];
@@ -218,6 +288,19 @@ __global__ __launch_bounds__(kMxThreads) void mx_cast_kernel(const void *__restr
             const int64_t oc = tc * kTileC + k, orow = tr * kTileR + m16 * 16;
             if (oc < cols && orow < rows)
                 __builtin_nontemporal_store(ct_lds_read(tile, k, m16), reinterpret_cast<u32x4 *>(out_t + oc * rows + orow));
+        }
+        // the staged scale bytes: dword [tile row][column] of scales_t from the first wave, the 16-bit half
+        // [tile column / 2][row] of scales from the next two
+        if (staged_t && threadIdx.x < kTileC) {
+            const int64_t oc = tc * kTileC + threadIdx.x;
+            if (oc < cols && tr * kTileR < rows)
+                reinterpret_cast<uint32_t *>(scales_t)[tr * cols + oc] = reinterpret_cast<const uint32_t *>(stage_t)[threadIdx.x];
+        }
+        if (staged_r && threadIdx.x >= 64 && threadIdx.x < 64 + kTileR) {
+            const int r = threadIdx.x - 64;
+            const int64_t orow = tr * kTileR + r;
+            if (orow < rows && tc * kTileC < cols)
+                reinterpret_cast<uint16_t *>(scales)[((tc >> 1) * rows + orow) * 2 + (tc & 1)] = reinterpret_cast<const uint16_t *>(stage_r)[r];
         }
     }
 }
@@ -254,7 +337,10 @@ __global__ __launch_bounds__(256) void block_cast_kernel(const void *__restrict_
                                                          uint8_t *__restrict__ out_t, uint32_t *__restrict__ scales_t) {
     __shared__ __attribute__((aligned(16))) uint8_t tile[WANT_COL ? 128 * 128 : 16];
     __shared__ __attribute__((aligned(8))) uint32_t red[4][128];   // per wave: column maxima (1-D), or slot 0: the wave's maximum (2-D)
-    __shared__ __attribute__((aligned(16))) float col_mul[128];
+    __shared__ __attribute__((aligned(16))) float col_e8[128];     // per column: its E8M0 byte where a float keeps its exponent
+    __shared__ int odd_tile;                                       // 1-D blocks: some column of the tile holds Inf / NaN
+    __shared__ uint32_t row_dw[128];                               // 1-D blocks, both outputs: the scale dwords of the tile's rows
+    saturate_fp8_conversions();
     constexpr int ESZ = SRC == ODL_BF16 ? 2 : 4, DW = 16 * ESZ / 4;
     const int tx = threadIdx.x % 8, ty = threadIdx.x / 8, wave = threadIdx.x / 64;
     const int64_t tiles_r = rows / 128, tiles_c = cols / 128;
@@ -294,15 +380,22 @@ __global__ __launch_bounds__(256) void block_cast_kernel(const void *__restrict_
         }
     };
 
-    float mul_all = 1.0f;
+    // A block whose amax is Inf / NaN (the only kind that can hold a NaN) goes through quantise4, which gives NaN its code;
+    // every other block through the hardware's scaled conversions, which divide by 2^(byte - 127) and saturate.
+    auto e8_of = [](uint32_t dword) { return bits_to_float((dword & 0xffu) << 23); };
+    auto mul_of = [](float e8) { return bits_to_float((254u - (float_to_bits(e8) >> 23)) << 23); };     // byte <= 253
+    float e8_all = 1.0f;
+    uint32_t m_all = 0;
     if constexpr (TWO_D) {
         uint32_t m = max(max(row_mag(0), row_mag(1)), max(row_mag(2), row_mag(3)));
         m = wave_max_u32(m);
         if (threadIdx.x % 64 == 0) red[wave][0] = m;
         __syncthreads();
-        m = max(max(red[0][0], red[1][0]), max(red[2][0], red[3][0]));
+        m_all = max(max(red[0][0], red[1][0]), max(red[2][0], red[3][0]));
         uint32_t dword;
-        block_scale_of<FMT>(m, margin, dword, mul_all);
+        float mul;
+        block_scale_of<FMT>(m_all, margin, dword, mul);
+        e8_all = e8_of(dword);
         if (threadIdx.x < 128) {
             if (WANT_ROW) scales[tc * rows + tr * 128 + threadIdx.x] = dword;
             if (WANT_COL) scales_t[tr * cols + tc * 128 + threadIdx.x] = dword;
@@ -312,26 +405,43 @@ __global__ __launch_bounds__(256) void block_cast_kernel(const void *__restrict_
     if constexpr (WANT_ROW) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            float mul = mul_all;
+            float e8 = e8_all;
+            uint32_t m = m_all;
             if constexpr (!TWO_D) {
-                uint32_t m = max_quad(row_mag(i));
+                m = max_quad(row_mag(i));
                 m = max_with_dpp<0x141>(m);                              // row_half_mirror: lane l <-> 7 - l of its 8: the other quad
                 uint32_t dword;
+                float mul;
                 block_scale_of<FMT>(m, margin, dword, mul);
-                if (tx == 0) scales[tc * rows + r0 + i] = dword;
+                e8 = e8_of(dword);
+                // with the transposed output to follow, the tile's 128 row dwords leave as one 512-byte run after the next barrier
+                if (tx == 0) {
+                    if constexpr (WANT_COL) row_dw[ty * 4 + i] = dword;
+                    else scales[tc * rows + r0 + i] = dword;
+                }
             }
             uint32_t q[4];
+            if (__builtin_expect(m >= 0x7f800000u, 0)) {
+                const float mul = mul_of(e8);
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                float f[4];
-                widen4(i, g, f);
-                q[g] = quantise4<FMT>(f[0], f[1], f[2], f[3], mul, mul, mul, mul);
+                for (int g = 0; g < 4; ++g) {
+                    float f[4];
+                    widen4(i, g, f);
+                    q[g] = quantise4<FMT>(f[0], f[1], f[2], f[3], mul, mul, mul, mul);
+                }
+            } else {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    if constexpr (SRC == ODL_BF16) q[g] = cvt_scaled4<SRC, FMT>(raw[i][2 * g], raw[i][2 * g + 1], 0u, 0u, e8);
+                    else q[g] = cvt_scaled4<SRC, FMT>(raw[i][4 * g], raw[i][4 * g + 1], raw[i][4 * g + 2], raw[i][4 * g + 3], e8);
+                }
             }
             *reinterpret_cast<u32x4 *>(out + (r0 + i) * cols + c0) = u32x4{q[0], q[1], q[2], q[3]};
         }
     }
 
     if constexpr (WANT_COL) {
+        bool plain = m_all < 0x7f800000u;                                // no Inf / NaN anywhere in the tile
         if constexpr (!TWO_D) {
             // column maxima: over the lane's 4 rows, over the 8 lanes of the wave with this tx (32 rows), over the 4 waves
 #pragma unroll
@@ -349,32 +459,53 @@ __global__ __launch_bounds__(256) void block_cast_kernel(const void *__restrict_
                     if ((ty & 7) == d / 2) red[wave][16 * tx + d] = m;
                 }
             }
+            if (threadIdx.x == 0) odd_tile = 0;
             __syncthreads();
             if (threadIdx.x < 128) {
                 const uint32_t m = max(max(red[0][threadIdx.x], red[1][threadIdx.x]), max(red[2][threadIdx.x], red[3][threadIdx.x]));
                 uint32_t dword;
                 float mul;
                 block_scale_of<FMT>(m, margin, dword, mul);
-                col_mul[threadIdx.x] = mul;
+                col_e8[threadIdx.x] = e8_of(dword);
                 scales_t[tr * cols + tc * 128 + threadIdx.x] = dword;
+                if constexpr (WANT_ROW) scales[tc * rows + tr * 128 + threadIdx.x] = row_dw[threadIdx.x];
+                if (m >= 0x7f800000u) odd_tile = 1;                      // (every writer writes the same value)
             }
             __syncthreads();
+            plain = odd_tile == 0;
         }
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-            float mc[4] = {mul_all, mul_all, mul_all, mul_all};
+            float ec[4] = {e8_all, e8_all, e8_all, e8_all};
             if constexpr (!TWO_D) {
-                const float4 v = *reinterpret_cast<const float4 *>(&col_mul[16 * tx + 4 * g]);
-                mc[0] = v.x; mc[1] = v.y; mc[2] = v.z; mc[3] = v.w;
+                const float4 v = *reinterpret_cast<const float4 *>(&col_e8[16 * tx + 4 * g]);
+                ec[0] = v.x; ec[1] = v.y; ec[2] = v.z; ec[3] = v.w;
             }
-            uint32_t q[4], t[4];
+            uint32_t t[4];
+            if (__builtin_expect(!plain, 0)) {
+                uint32_t q[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                float f[4];
-                widen4(i, g, f);
-                q[i] = quantise4<FMT>(f[0], f[1], f[2], f[3], mc[0], mc[1], mc[2], mc[3]);
+                for (int i = 0; i < 4; ++i) {
+                    float f[4];
+                    widen4(i, g, f);
+                    q[i] = quantise4<FMT>(f[0], f[1], f[2], f[3], mul_of(ec[0]), mul_of(ec[1]), mul_of(ec[2]), mul_of(ec[3]));
+                }
+                transpose4x4(q, t);                                      // t[k] = rows 4 ty .. + 3 of column 16 tx + 4 g + k
+            } else {
+                // the four rows of a column side by side feed one pair of conversions: the codes come out transposed
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const int c = 4 * g + k;
+                    if constexpr (SRC == ODL_BF16) {
+                        const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
+                        const uint32_t r01 = __builtin_amdgcn_perm(raw[1][c / 2], raw[0][c / 2], sel);
+                        const uint32_t r23 = __builtin_amdgcn_perm(raw[3][c / 2], raw[2][c / 2], sel);
+                        t[k] = cvt_scaled4<SRC, FMT>(r01, r23, 0u, 0u, ec[k]);
+                    } else {
+                        t[k] = cvt_scaled4<SRC, FMT>(raw[0][c], raw[1][c], raw[2][c], raw[3][c], ec[k]);
+                    }
+                }
             }
-            transpose4x4(q, t);                                          // t[k] = rows 4 ty .. + 3 of column 16 tx + 4 g + k
 #pragma unroll
             for (int k = 0; k < 4; ++k) *reinterpret_cast<uint32_t *>(&tile[block_lds_off(16 * tx + 4 * g + k, ty)]) = t[k];
         }

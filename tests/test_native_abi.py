@@ -111,6 +111,18 @@ def test_build_rejects_asm_that_reads_a_scalar_too_soon_after_a_vector_write():
     assert check_asm_hazards("\tv_readlane_b32 s0, v1, 2\n\tbuffer_load_dword v1, v0, s[16:19], s0 offen\n", "x.s") == []
 
 
+def test_build_rejects_scaled_conversions_that_run_before_the_saturation_mode_is_set():
+    from optimus_dl_amd.build import check_saturating_conversions
+
+    mode = "\ts_setreg_imm32_b32 hwreg(HW_REG_MODE, 23, 1), 1\n"
+    cvt = "\tv_cvt_scalef32_pk_fp8_bf16 v3, v1, s2\n"
+    assert check_saturating_conversions("_Z1kv:\n" + mode + "\tv_mov_b32 v0, 0\n" + cvt, "x.s") == []
+    assert len(check_saturating_conversions("_Z1kv:\n" + cvt + mode, "x.s")) == 1
+    # the mode belongs to the wave that set it: the next function starts without it
+    assert len(check_saturating_conversions("_Z1kv:\n" + mode + cvt + "_Z1lv:\n" + cvt + cvt, "x.s")) == 1
+    assert check_saturating_conversions("_Z1kv:\n\tv_cvt_pk_fp8_f32 v3, v1, v2\n", "x.s") == []
+
+
 def test_split_count_is_a_host_side_decision_with_the_documented_shape_rules():
     """odl_fp8_gemm_split_count launches nothing; without a GPU it plans for 256 compute units."""
     from optimus_dl_amd import native
