@@ -77,6 +77,29 @@ def test_block_cast_two_dimensional_blocks_bit_exact(N, shape, fmt, dtype):
     assert_bytes_equal(_bytes(sc_t), ws.t().repeat_interleave(128, dim=0), f"transposed scale bytes {shape}")
 
 
+@pytest.mark.parametrize("order", ["sorted", "shuffled"])
+@pytest.mark.parametrize("fmt", [E4M3, E5M2])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_block_cast_every_bf16_pattern(N, fmt, order, dtype):
+    """All 65536 bf16 bit patterns, sorted by magnitude (elements close to their block's amax) and shuffled (far below
+    it; Inf and NaN scattered over the blocks), 1 x 128 blocks in both directions and 128 x 128 blocks."""
+    from tests.test_gpu_mx import _every_bf16_pattern
+
+    x = _every_bf16_pattern(order)                                        # [128, 512]
+    out, sc, out_t, sc_t = N.block_cast(x.to(dtype).cuda(), fmt, 0, False, True, True)
+    wc, ws = O.c_block_quantise(x, 1, 128, fmt, 0)
+    assert_bytes_equal(_bytes(sc), ws, f"scale bytes, {order}")
+    assert_bytes_equal(out, wc, f"codes, {order}")
+    wct, wst = O.c_block_quantise(x.t().contiguous(), 1, 128, fmt, 0)
+    assert_bytes_equal(_bytes(sc_t), wst, f"transposed scale bytes, {order}")
+    assert_bytes_equal(out_t, wct, f"transposed codes, {order}")
+    out, sc, out_t, sc_t = N.block_cast(x.to(dtype).cuda(), fmt, 0, True, True, True)
+    wc, ws = O.c_block_quantise(x, 128, 128, fmt, 0)
+    assert_bytes_equal(out, wc, f"codes, 128 x 128 blocks, {order}")
+    assert_bytes_equal(out_t, wc.t().contiguous(), f"transposed codes, 128 x 128 blocks, {order}")
+    assert_bytes_equal(_bytes(sc), ws.repeat_interleave(128, dim=0), f"scale bytes, 128 x 128 blocks, {order}")
+
+
 def test_block_cast_single_layouts_and_specials(N):
     x = _mixed((256, 384), seed=7)
     x[5, 200] = float("inf")

@@ -120,6 +120,74 @@ def test_mx_cast_specials(N):
         assert int(sc[0, 0]) == 255 and int(sc[1, 1]) == 255 and int(sc[5, 0]) == 0
 
 
+def _every_bf16_pattern(order: str) -> torch.Tensor:
+    """All 65536 bf16 bit patterns as a [128, 512] matrix: sorted by magnitude (the neighbours that share a block are
+    close to its amax, where the conversion saturates) or shuffled (most elements far below the block amax: subnormal
+    codes, underflow to zero; about one block in eight holds an Inf or a NaN)."""
+    import numpy as np
+
+    pats = np.arange(65536, dtype=np.uint32)
+    if order == "sorted":
+        pats = pats[np.argsort(pats & 0x7fff, kind="stable")]
+    else:
+        pats = pats[np.random.default_rng(1).permutation(65536)]
+    return torch.from_numpy(pats.astype(np.uint16).view(np.int16).copy()).view(torch.bfloat16).reshape(128, 512)
+
+
+@pytest.mark.parametrize("order", ["sorted", "shuffled"])
+@pytest.mark.parametrize("fmt", [E4M3, E5M2])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_mx_cast_every_bf16_pattern(N, fmt, order, dtype):
+    x = _every_bf16_pattern(order)
+    out, sc, out_t, sc_t = N.mx_cast(x.to(dtype).cuda(), fmt, want_rowmajor=True, want_transposed=True)
+    sc, sc_t = N.mx_scales_rowmajor(sc), N.mx_scales_rowmajor(sc_t)
+    wc, ws = O.c_mx_quantise(x, fmt)
+    assert_bytes_equal(sc, ws, f"scale bytes, {order}")
+    assert_bytes_equal(out, wc, f"codes, {order}")
+    wct, wst = O.c_mx_quantise(x.t().contiguous(), fmt)
+    assert_bytes_equal(sc_t, wst, f"transposed scale bytes, {order}")
+    assert_bytes_equal(out_t, wct, f"transposed codes, {order}")
+
+
+@pytest.mark.parametrize("fmt", [E4M3, E5M2])
+def test_mx_cast_fp32_inputs_around_every_rounding_midpoint(N, fmt):
+    """fp32 inputs on, one ulp below and one ulp above every midpoint between neighbouring FP8 values (a tie goes to
+    the even code, one fp32 ulp decides the others) and around the largest value (saturation), at several shared
+    exponents.  Every block holds 31 of them and an anchor just below the next binade that fixes the block's scale."""
+    top = 0x7E if fmt == E4M3 else 0x7B                                  # code of the largest finite value
+    vals = O.t_decode(torch.arange(0, top + 1, dtype=torch.uint8), fmt).double()
+    step_up = vals[-1] - vals[-2]
+    mids = torch.cat([(vals[:-1] + vals[1:]) / 2, (vals[-1] + step_up / 2).reshape(1)]).float()
+    assert bool((mids.double() == torch.cat([(vals[:-1] + vals[1:]) / 2, (vals[-1] + step_up / 2).reshape(1)])).all())
+    inf = torch.tensor(float("inf"))
+    cands = torch.cat([torch.nextafter(mids, -inf), mids, torch.nextafter(mids, inf)])
+    cands = torch.cat([cands, -cands])
+    pad = (-cands.numel()) % 31
+    cands = torch.cat([cands, cands[:pad]]).reshape(-1, 31)
+    emax = O.MX_EMAX[fmt]
+    blocks = []
+    for se in (-30, -3, 0, 11, 40):
+        anchor = torch.full((cands.shape[0], 1), 1.984375 * 2.0 ** emax)
+        blk = torch.cat([cands[:, :7], anchor, cands[:, 7:]], dim=1)
+        blocks.append(torch.ldexp(blk, torch.tensor(se)))
+    x = torch.cat(blocks)                                                # [blocks, 32] fp32
+    x = torch.cat([x, x[: (-x.shape[0]) % 64]])                          # a row count the transposed call accepts
+    want_codes, want_scales = O.t_mx_quantise(x, fmt)
+    assert sorted(set(int(b) for b in want_scales.flatten())) == [127 + se for se in (-30, -3, 0, 11, 40)]
+    out, sc, _, _ = N.mx_cast(x.cuda(), fmt, want_rowmajor=True, want_transposed=False)
+    assert_bytes_equal(N.mx_scales_rowmajor(sc), want_scales, "scale bytes")
+    assert_bytes_equal(out, want_codes, "codes of fp32 inputs around the midpoints")
+    # the other direction: the same blocks run down the columns of the transposed matrix
+    _, _, out_t, sc_t = N.mx_cast(x.t().contiguous().cuda(), fmt, want_rowmajor=False, want_transposed=True)
+    assert_bytes_equal(N.mx_scales_rowmajor(sc_t), want_scales, "scale bytes, blocks down the columns")
+    assert_bytes_equal(out_t, want_codes, "codes, blocks down the columns")
+    # ties really are among the inputs and go to the even code
+    tie = torch.ldexp(mids[5], torch.tensor(0)).item()
+    row = torch.tensor([tie] + [1.984375 * 2.0 ** emax] + [0.0] * 30).reshape(1, 32)
+    code = int(O.t_mx_quantise(row, fmt)[0][0, 0])
+    assert code % 2 == 0 and code in (5, 6)
+
+
 def test_mx_cast_rejects_bad_shapes(N):
     with pytest.raises(N.NativeError, match="multiple of 32"):
         N.mx_cast(torch.zeros((32, 48), dtype=torch.bfloat16, device="cuda"), E4M3, True, False)
