@@ -175,6 +175,7 @@ __global__ __launch_bounds__(kMxThreads) void mx_cast_kernel(const void *__restr
 
     if constexpr (WANT_ROW) {
         const int64_t nb = cols / kMxBlock;
+        uint32_t row_pairs[2] = {0u, 0u};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             uint32_t m = 0;
@@ -207,17 +208,23 @@ __global__ __launch_bounds__(kMxThreads) void mx_cast_kernel(const void *__restr
                     }
                 }
                 *reinterpret_cast<u32x2 *>(out + (r0 + i) * cols + c0) = u32x2{lo, hi};
-                if ((tx & 3) == 0) {
-                    if (staged_r) stage_r[(ty * 4 + i) * 2 + tx / 4] = (uint8_t)byte;
-                    else scales[mx_scale_at(layout, r0 + i, c0 / kMxBlock, rows, nb)] = (uint8_t)byte;
+                if (staged_r) {
+                    // both bytes of the row in one lane: row_shl:4 hands lane l the value of lane l + 4, which holds the
+                    // row's second block; the lane's four rows then go to LDS as one 8-byte write
+                    const uint32_t second = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)byte, 0x104, 0xf, 0xf, false);
+                    row_pairs[i / 2] |= (byte | (second << 8)) << (16 * (i & 1));
+                } else if ((tx & 3) == 0) {
+                    scales[mx_scale_at(layout, r0 + i, c0 / kMxBlock, rows, nb)] = (uint8_t)byte;
                 }
             }
         }
+        if (staged_r && tx == 0) *reinterpret_cast<u32x2 *>(&stage_r[ty * 8]) = u32x2{row_pairs[0], row_pairs[1]};
     }
 
     if constexpr (WANT_COL) {
         const int64_t nbt = rows / kMxBlock;
         float mul_c[8], e8_c[8];
+        uint32_t col_bytes[2] = {0u, 0u};                                // the scale bytes of the lane's 8 columns, packed
         uint32_t cmax[8];                                                // fp32 magnitude bits per column, over the 32 rows
         if constexpr (SRC == ODL_BF16) {
 #pragma unroll
@@ -238,11 +245,12 @@ __global__ __launch_bounds__(kMxThreads) void mx_cast_kernel(const void *__restr
             mx_scale_of<FMT>(cmax[j], byte, mul_c[j]);
             e8_c[j] = bits_to_float(byte << 23);
             // rows % 32 == 0 (host-checked): a row block is inside the matrix as a whole or not at all
-            if ((ty & 7) == 0 && col_ok && r0 < rows) {
-                if (staged_t) stage_t[(tx * 8 + j) * 4 + ty / 8] = (uint8_t)byte;
-                else scales_t[mx_scale_at(layout_t, c0 + j, r0 / kMxBlock, cols, nbt)] = (uint8_t)byte;
-            }
+            col_bytes[j / 4] |= byte << (8 * (j % 4));
+            if (!staged_t && (ty & 7) == 0 && col_ok && r0 < rows)
+                scales_t[mx_scale_at(layout_t, c0 + j, r0 / kMxBlock, cols, nbt)] = (uint8_t)byte;
         }
+        // staged: the wave's row block is one plane of 64 bytes, a lane's 8 columns one 8-byte write
+        if (staged_t && (ty & 7) == 0) *reinterpret_cast<u32x2 *>(&stage_t[(ty / 8) * kTileC + tx * 8]) = u32x2{col_bytes[0], col_bytes[1]};
         uint32_t worst = 0;                                              // Inf / NaN in any of the lane's 8 column blocks?
 #pragma unroll
         for (int j = 0; j < 8; ++j) worst = max(worst, cmax[j]);
@@ -293,8 +301,10 @@ __global__ __launch_bounds__(kMxThreads) void mx_cast_kernel(const void *__restr
         // [tile column / 2][row] of scales from the next two
         if (staged_t && threadIdx.x < kTileC) {
             const int64_t oc = tc * kTileC + threadIdx.x;
+            const int c = threadIdx.x;
             if (oc < cols && tr * kTileR < rows)
-                reinterpret_cast<uint32_t *>(scales_t)[tr * cols + oc] = reinterpret_cast<const uint32_t *>(stage_t)[threadIdx.x];
+                reinterpret_cast<uint32_t *>(scales_t)[tr * cols + oc] = (uint32_t)stage_t[c] | ((uint32_t)stage_t[kTileC + c] << 8) |
+                                                                         ((uint32_t)stage_t[2 * kTileC + c] << 16) | ((uint32_t)stage_t[3 * kTileC + c] << 24);
         }
         if (staged_r && threadIdx.x >= 64 && threadIdx.x < 64 + kTileR) {
             const int r = threadIdx.x - 64;
