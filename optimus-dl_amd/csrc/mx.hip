@@ -533,9 +533,9 @@ __global__ __launch_bounds__(256) void block_cast_kernel(const void *__restrict_
 // ------------------------------------------------------------------ GEMM, tiled
 // The structure of gemm_nt_tiled_kernel (two LDS stages of BM + BN rows x 128 bytes, direct-to-LDS loads, swizzled
 // 16-byte chunks, MFMA operands swapped so that a lane ends up with 4 consecutive output columns) plus the scale
-// bytes: per K step of 128 bytes a row has 4 of them (one dword); thread i of the block fetches the dword of
-// A row i and of B row i for the NEXT step together with that step's operand loads and parks it in LDS after the
-// barrier; a lane reads the dword of each of its rows and shifts it right by 8 bits when it sits in the upper half of the
+// bytes: per K step of 128 bytes a row has 4 of them (one dword); every thread of the block fetches the dword of one
+// row of A or B for the NEXT step with that step's operand loads, like them straight into LDS;
+// a lane reads the dword of each of its rows and shifts it right by 8 bits when it sits in the upper half of the
 // wave, so that byte 0 / byte 2 are the scales it supplies in the first / second MFMA of the step (lanes 0..31: blocks 0
 // and 2 of the step, lanes 32..63: blocks 1 and 3).
 template <int BM, int BN, int WAVES_M, int WAVES_N, int FA, int FB, bool KS>
@@ -546,11 +546,12 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mx_gemm_tiled_kernel(co
     constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128, STAGE = A_BYTES + B_BYTES;
     constexpr int LA = BM / 8 / NW, LB = BN / 8 / NW;
     constexpr int GM = 8;
-    static_assert(BM <= NT && BN <= NT, "one scale dword per thread and operand");
+    static_assert(BM + BN == NT, "one scale dword per thread: the first BM threads serve A, the others B");
 
     __shared__ __attribute__((aligned(1024))) uint8_t lds0[STAGE];
     __shared__ __attribute__((aligned(1024))) uint8_t lds1[STAGE];
-    __shared__ uint32_t sc0[BM + BN], sc1[BM + BN];
+    __shared__ __attribute__((aligned(256))) uint32_t sc0[BM + BN];
+    __shared__ __attribute__((aligned(256))) uint32_t sc1[BM + BN];
 
     const int total = g.tiles_m * g.tiles_n;
     const int per_xcd = (total + 7) / 8;
@@ -582,14 +583,15 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mx_gemm_tiled_kernel(co
         const int64_t gr = min(n0 + row, g.N - 1);
         off_b[j] = (uint32_t)(gr * g.K + (((lane % 8) ^ swz(row)) << 4));
     }
-    // the scale dwords this thread fetches: A row threadIdx.x, B row threadIdx.x (rows past the edge re-read the last row)
-    // (K-step-major: the dword of step kt is [kt][row]; row-major: dword kt of the row's nb bytes)
-    const int64_t row_a = min(m0 + (int64_t)threadIdx.x, g.M - 1), row_b = min(n0 + (int64_t)threadIdx.x, g.N - 1);
-    const uint32_t *sa_row = reinterpret_cast<const uint32_t *>(sa) + (KS ? row_a : row_a * (nb / 4));
-    const uint32_t *sb_row = reinterpret_cast<const uint32_t *>(sb) + (KS ? row_b : row_b * (nb / 4));
-    const int64_t step_a = KS ? g.M : 1, step_b = KS ? g.N : 1;
-    uint32_t ra = 0, rb = 0;
-    auto issue = [&](uint8_t *lds, int kt) {
+    // the scale dword this thread fetches per step: thread i < BM that of A row i, the others that of B row i - BM (rows
+    // past the edge re-read the last row); K-step-major: the dword of step kt is [kt][row], row-major: dword kt of the
+    // row's nb bytes.  It travels like the operands, straight into the stage's scale slots (64 lanes x 4 bytes land at
+    // the wave's 256 bytes), and is complete when the operand loads of the stage are.
+    const bool mine_a = (int)threadIdx.x < BM;
+    const int64_t my_row = mine_a ? min(m0 + (int64_t)threadIdx.x, g.M - 1) : min(n0 + (int64_t)threadIdx.x - BM, g.N - 1);
+    const uint32_t *my_scales = reinterpret_cast<const uint32_t *>(mine_a ? sa : sb) + (KS ? my_row : my_row * (nb / 4));
+    const int64_t my_step = KS ? (mine_a ? g.M : g.N) : 1;
+    auto issue = [&](uint8_t *lds, uint32_t *sc, int kt) {
         const uint8_t *ga = g.a + (int64_t)kt * 128, *gb = g.b + (int64_t)kt * 128;
 #pragma unroll
         for (int j = 0; j < LA; ++j)
@@ -599,12 +601,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mx_gemm_tiled_kernel(co
         for (int j = 0; j < LB; ++j)
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(gb + off_b[j]),
                                              (__attribute__((address_space(3))) void *)(lds + A_BYTES + (wave + j * NW) * 1024), 16, 0, 0);
-        if ((int)threadIdx.x < BM) ra = sa_row[kt * step_a];
-        if ((int)threadIdx.x < BN) rb = sb_row[kt * step_b];
-    };
-    auto park = [&](uint32_t *sc) {                // after vmcnt(0): this thread's two dwords into the stage's scale slots
-        if ((int)threadIdx.x < BM) sc[threadIdx.x] = ra;
-        if ((int)threadIdx.x < BN) sc[BM + threadIdx.x] = rb;
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(my_scales + kt * my_step),
+                                         (__attribute__((address_space(3))) void *)(sc + wave * 64), 4, 0, 0);
     };
 
     const int lr = lane % 32, lg = lane / 32;
@@ -656,18 +654,16 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mx_gemm_tiled_kernel(co
         }
     };
 
-    issue(lds0, 0);
+    issue(lds0, sc0, 0);
     for (int kt = 0; kt < KT; kt += 2) {
-        __builtin_amdgcn_s_waitcnt(0x0F70);                     // vmcnt(0): my loads into lds0 and my scale dwords have landed
-        park(sc0);
+        __builtin_amdgcn_s_waitcnt(0x0F70);                     // vmcnt(0): my loads into lds0 and sc0 have landed
         __syncthreads();
-        if (kt + 1 < KT) issue(lds1, kt + 1);
+        if (kt + 1 < KT) issue(lds1, sc1, kt + 1);
         compute(lds0, sc0);
         if (kt + 1 < KT) {
             __builtin_amdgcn_s_waitcnt(0x0F70);
-            park(sc1);
             __syncthreads();
-            if (kt + 2 < KT) issue(lds0, kt + 2);
+            if (kt + 2 < KT) issue(lds0, sc0, kt + 2);
             compute(lds1, sc1);
         }
     }
@@ -862,13 +858,15 @@ extern "C" int odl_fp8_mx_gemm_nt(const uint8_t *a, const uint8_t *sa, const uin
     g.a = a; g.b = b; g.c = c; g.sa = one; g.sb = one; g.bias = bias;
     g.M = M; g.N = N; g.K = K; g.sa_vec = 0; g.sb_vec = 0; g.out_dtype = out_dtype;
     // the tiled and the streaming kernel address rows with 32-bit offsets and read whole scale dwords (4 blocks = one
-    // 128-byte K step); the streaming kernel wants the scales K-step-major and the shapes of gemm_stream_accepts
+    // 128-byte K step); the streaming kernel wants the scales K-step-major and the shapes of gemm_stream_accepts, and
+    // pays only when more than half the compute units get one of its 256 x 256 tiles (at exactly half, outputs of
+    // 8192 x 1024, the 128 x 128 kernel is 3 us faster at K = 1024 .. 3072, as for the per-tensor GEMMs)
     const bool lim32 = (double)(M + 256) * (double)K < 2147483648.0 && (double)(N + 256) * (double)K < 2147483648.0;
     const bool tiled = K % 128 == 0 && !mis(sa, 4) && !mis(sb, 4) && lim32 && M >= 32 && N >= 32;
     GemmArgs probe = g;
     probe.mx_sa = sa; probe.mx_sb = sb;
     const int cus = device_cu_count();
-    const bool stream_ok = ks && tiled && ((M + 255) / 256) * ((N + 255) / 256) >= cus / 2 && gemm_stream_accepts(probe);
+    const bool stream_ok = ks && tiled && ((M + 255) / 256) * ((N + 255) / 256) * 2 > cus && gemm_stream_accepts(probe);
     const int kernel = stream_ok ? 2 : (tiled ? 1 : 0);
 #define ODL_MXG(FA_, FB_) launch_mx_gemm<FA_, FB_>(g, sa, sb, kernel, ks, cus, stream)
     if (fmt_a == ODL_FP8_E4M3 && fmt_b == ODL_FP8_E4M3) ODL_MXG(ODL_FP8_E4M3, ODL_FP8_E4M3);
