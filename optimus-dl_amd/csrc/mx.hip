@@ -20,7 +20,9 @@
 //
 // Conversion rule (OCP Microscaling Formats v1.0, 6.3): shared exponent = floor(log2(block amax)) - emax of the element
 // format (8 for E4M3, 15 for E5M2), clamped to [-127, 127]; elements = rne(clamp(v * 2^-shared, +-fp8_max)).  A block of
-// zeros gets byte 0, a block holding Inf / NaN gets 0xFF (a NaN scale: the products it enters are NaN).
+// zeros gets byte 0, a block holding Inf / NaN gets 0xFF (a NaN scale: the products it enters are NaN).  The element
+// conversion is one instruction per two elements (the scaled conversions of gfx950, see cvt_scaled_bf16x2); only blocks
+// that hold Inf / NaN are converted step by step.
 #include <hip/hip_runtime.h>
 
 #include "common.h"
