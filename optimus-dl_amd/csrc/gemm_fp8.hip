@@ -263,12 +263,13 @@ extern "C" int odl_fp8_gemm_layouts(const uint8_t *a, const uint8_t *b, int64_t 
 // How many runs to cut K into for an output of few tiles (1 = do not split).  A model in microseconds, fitted to
 // measurements on this GPU (outputs 768 x 768 .. 8192 x 1024, K = 8192 .. 151936):
 //   one launch, 256 x 256 tiles : 0.92 us per K step of 128 (few compute units busy: high clock) + 3 steps of overhead
-//   one launch, 128 x 128 tiles : 0.60 us per step (what odl_fp8_gemm_nt takes for outputs of <= cus / 2 big tiles),
-//                                 but it reads every operand panel twice as often
-//   split                       : 1.45 us per step of a run (the whole chip busy: lower clock) + the reduction, which
-//                                 reads splits x M x N floats at about 5 TB/s, + 3 us for its launch
+//   one launch, 128 x 128 tiles : 0.55 us per step where every block has a compute unit to itself (the four-stage form
+//                                 of the kernel), 0.62 with two blocks per unit (what odl_fp8_gemm_nt takes for outputs
+//                                 of <= cus / 2 big tiles); it reads every operand panel twice as often
+//   split                       : 0.96 us per step of a run + 9 us (pipeline fill, the fp32 epilogue, the second launch)
+//                                 + the partial results, splits x M x N floats written and read back, at 2.7 TB/s in all
 //   each bounded below by its operand traffic (tiles x panel bytes) at about 12 TB/s out of the caches.
-// The runs of a split must fit the compute units at once, and a split must win by 15 %.
+// The runs of a split must fit the compute units at once, and a split must win by 10 %.
 // k_slow: an operand is stored with the contraction index slow (odl_fp8_gemm_layouts), which only the streaming
 // kernel reads: the 128 x 128 kernel is then not an alternative.
 extern "C" int odl_fp8_gemm_split_count(int64_t M, int64_t N, int64_t K, int k_slow) {
@@ -282,8 +283,9 @@ extern "C" int odl_fp8_gemm_split_count(int64_t M, int64_t N, int64_t K, int k_s
     double whole = 0.92 * ((double)steps + 3.0);
     if (whole < traffic_us) whole = traffic_us;
     if (tiles * 2 <= cus && !k_slow) {
-        double small = 0.60 * ((double)steps + 3.0);
-        const double small_traffic_us = (double)((M + 127) / 128) * (double)((N + 127) / 128) * 256.0 * (double)K / 12.0e6;
+        const int64_t small_tiles = ((M + 127) / 128) * ((N + 127) / 128);
+        double small = (small_tiles <= cus ? 0.55 : 0.62) * ((double)steps + 3.0);
+        const double small_traffic_us = (double)small_tiles * 256.0 * (double)K / 12.0e6;
         if (small < small_traffic_us) small = small_traffic_us;
         if (small < whole) whole = small;
     }
@@ -293,10 +295,10 @@ extern "C" int odl_fp8_gemm_split_count(int64_t M, int64_t N, int64_t K, int k_s
         const int64_t per = ((steps + splits - 1) / splits + 1) & ~(int64_t)1;
         const int64_t last = steps - (splits - 1) * per;
         if (per < 8 || last < 4) continue;
-        double run = 1.45 * ((double)per + 3.0);
+        double run = 0.96 * (double)per + 9.0;
         if (run < traffic_us) run = traffic_us;
-        const double cost = run + (double)splits * (double)M * (double)N * 4.0 / 5.0e6 + 3.0;
-        if (cost < 0.85 * whole && cost < best) { best = cost; best_splits = (int)splits; }
+        const double cost = run + (double)splits * (double)M * (double)N * 4.0 / 2.7e6;
+        if (cost < 0.90 * whole && cost < best) { best = cost; best_splits = (int)splits; }
     }
     return best_splits;
 }

@@ -28,8 +28,9 @@
 namespace odl {
 
 // ------------------------------------------------------------------ tiled kernel
-template <int BM, int BN, int WAVES_M, int WAVES_N, int FA, int FB>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int FA, int FB, int STAGES = 2>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_nt_tiled_kernel(const GemmArgs g) {
+    static_assert(STAGES == 2 || STAGES == 4, "two LDS stages, or four for launches of at most one block per compute unit");
     constexpr int NW = WAVES_M * WAVES_N;
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, TM = WM / 32, TN = WN / 32;
     constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128, STAGE = A_BYTES + B_BYTES;
@@ -40,6 +41,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_nt_tiled_kernel(co
 
     __shared__ __attribute__((aligned(1024))) uint8_t lds0[STAGE];
     __shared__ __attribute__((aligned(1024))) uint8_t lds1[STAGE];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds2[STAGES == 4 ? STAGE : 1024];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds3[STAGES == 4 ? STAGE : 1024];
 
     // ---- which tile (XCD-aware, grouped)
     const int total = g.tiles_m * g.tiles_n;
@@ -126,6 +129,47 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_nt_tiled_kernel(co
         }
     };
 
+    if constexpr (STAGES == 4) {
+        // A block that has a compute unit to itself cannot hide the latency of its loads behind another block's MFMAs:
+        // with two stages a load has one step's compute (0.25 us) to arrive from the L2 or beyond, and the block waits
+        // out the rest every step.  Four stages keep three steps of loads in flight.  A wave's loads complete in order,
+        // so "stage kt has landed" is "at most the loads of the later stages are outstanding": vmcnt(2, 1 or 0 stages).
+        // Loads, waits and barriers are written as instructions here: the compiler, shown direct-to-LDS loads into four
+        // buffers, puts a wait for ALL of them in front of every LDS read (it tracks only a few such loads apart), and
+        // __syncthreads() carries a fence that does the same; either is the two-stage kernel again.  The "memory"
+        // clobber of the barrier keeps the LDS reads of a stage behind it.
+        constexpr int PER = LA + LB;                            // direct-to-LDS instructions of a wave per stage
+        static_assert(2 * PER <= 63, "the counter holds 63 loads");
+        auto lds_addr_of = [](const uint8_t *p) { return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) uint8_t *)p; };
+        auto dma = [](const uint8_t *src, uint32_t lds_addr) {  // 64 lanes x 16 bytes land at lds_addr + lane * 16
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(src));
+        };
+        auto fetch = [&](uint8_t *lds, int kt) {
+            const uint8_t *ga = g.a + (int64_t)kt * 128, *gb = g.b + (int64_t)kt * 128;
+            const uint32_t base = lds_addr_of(lds);
+#pragma unroll
+            for (int j = 0; j < LA; ++j) dma(ga + off_a[j], base + (wave + j * NW) * 1024);
+#pragma unroll
+            for (int j = 0; j < LB; ++j) dma(gb + off_b[j], base + A_BYTES + (wave + j * NW) * 1024);
+        };
+        auto phase = [&](const uint8_t *cur, uint8_t *refill, int kt) {
+            // everyone's loads of stage kt are in, and everyone has read stage kt - 1
+            if (kt + 2 < KT) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * PER) : "memory");
+            else if (kt + 1 < KT) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(PER) : "memory");
+            else asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+            if (kt + 3 < KT) fetch(refill, kt + 3);             // into the stage that step kt - 1 used
+            compute(cur);
+        };
+        fetch(lds0, 0);
+        if (KT > 1) fetch(lds1, 1);
+        if (KT > 2) fetch(lds2, 2);
+        for (int kt = 0; kt < KT; kt += 4) {
+            phase(lds0, lds3, kt);
+            if (kt + 1 < KT) phase(lds1, lds0, kt + 1);
+            if (kt + 2 < KT) phase(lds2, lds1, kt + 2);
+            if (kt + 3 < KT) phase(lds3, lds2, kt + 3);
+        }
+    } else {
     // ---- main loop, two K-steps per trip so each stage is a fixed LDS object
     issue(lds0, 0);
     for (int kt = 0; kt < KT; kt += 2) {
@@ -139,6 +183,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_nt_tiled_kernel(co
             if (kt + 2 < KT) issue(lds0, kt + 2);
             compute(lds1);
         }
+    }
     }
 
     // ---- epilogue (uniform choice per block: staged through LDS for interior tiles, direct stores at the edges)
@@ -169,7 +214,13 @@ static void launch_tiled_fmt(int variant, const GemmArgs &g, hipStream_t stream)
     case 1: hipLaunchKernelGGL((gemm_nt_tiled_kernel<256, 256, 2, 2, FA, FB>), dim3(grid), dim3(256), 0, stream, g); break;
     case 2: hipLaunchKernelGGL((gemm_nt_tiled_kernel<256, 256, 2, 4, FA, FB>), dim3(grid), dim3(512), 0, stream, g); break;
     case 3: hipLaunchKernelGGL((gemm_nt_tiled_kernel<256, 128, 2, 2, FA, FB>), dim3(grid), dim3(256), 0, stream, g); break;
-    default: hipLaunchKernelGGL((gemm_nt_tiled_kernel<128, 128, 2, 2, FA, FB>), dim3(grid), dim3(256), 0, stream, g); break;
+    default:
+        // at most one block per compute unit: the four-stage form (128 KB of LDS, which leaves room for one block only)
+        if (total <= device_cu_count())
+            hipLaunchKernelGGL((gemm_nt_tiled_kernel<128, 128, 2, 4, FA, FB, 4>), dim3(grid), dim3(512), 0, stream, g);
+        else
+            hipLaunchKernelGGL((gemm_nt_tiled_kernel<128, 128, 2, 2, FA, FB>), dim3(grid), dim3(256), 0, stream, g);
+        break;
     }
 }
 

@@ -540,20 +540,26 @@ __global__ __launch_bounds__(256) void block_cast_kernel(const void *__restrict_
 // a lane reads the dword of each of its rows and shifts it right by 8 bits when it sits in the upper half of the
 // wave, so that byte 0 / byte 2 are the scales it supplies in the first / second MFMA of the step (lanes 0..31: blocks 0
 // and 2 of the step, lanes 32..63: blocks 1 and 3).
-template <int BM, int BN, int WAVES_M, int WAVES_N, int FA, int FB, bool KS>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int FA, int FB, bool KS, int STAGES = 2>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mx_gemm_tiled_kernel(const GemmArgs g, const uint8_t *__restrict__ sa,
                                                                               const uint8_t *__restrict__ sb) {
+    static_assert(STAGES == 2 || STAGES == 4, "two LDS stages, or four for launches of at most one block per compute unit");
     constexpr int NW = WAVES_M * WAVES_N, NT = NW * 64;
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, TM = WM / 32, TN = WN / 32;
     constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128, STAGE = A_BYTES + B_BYTES;
     constexpr int LA = BM / 8 / NW, LB = BN / 8 / NW;
     constexpr int GM = 8;
-    static_assert(BM + BN == NT, "one scale dword per thread: the first BM threads serve A, the others B");
+    static_assert(BM + BN <= NT && (BM + BN) % 64 == 0, "one scale dword per thread of the first (BM + BN) / 64 waves: BM threads serve A, the next BN serve B");
+    constexpr int SCALE_WAVES = (BM + BN) / 64;
 
     __shared__ __attribute__((aligned(1024))) uint8_t lds0[STAGE];
     __shared__ __attribute__((aligned(1024))) uint8_t lds1[STAGE];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds2[STAGES == 4 ? STAGE : 1024];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds3[STAGES == 4 ? STAGE : 1024];
     __shared__ __attribute__((aligned(256))) uint32_t sc0[BM + BN];
     __shared__ __attribute__((aligned(256))) uint32_t sc1[BM + BN];
+    __shared__ __attribute__((aligned(256))) uint32_t sc2[STAGES == 4 ? BM + BN : 64];
+    __shared__ __attribute__((aligned(256))) uint32_t sc3[STAGES == 4 ? BM + BN : 64];
 
     const int total = g.tiles_m * g.tiles_n;
     const int per_xcd = (total + 7) / 8;
@@ -590,7 +596,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mx_gemm_tiled_kernel(co
     // row's nb bytes.  It travels like the operands, straight into the stage's scale slots (64 lanes x 4 bytes land at
     // the wave's 256 bytes), and is complete when the operand loads of the stage are.
     const bool mine_a = (int)threadIdx.x < BM;
-    const int64_t my_row = mine_a ? min(m0 + (int64_t)threadIdx.x, g.M - 1) : min(n0 + (int64_t)threadIdx.x - BM, g.N - 1);
+    const int64_t my_row = mine_a ? min(m0 + (int64_t)threadIdx.x, g.M - 1) : min(n0 + min((int64_t)threadIdx.x - BM, (int64_t)BN - 1), g.N - 1);
     const uint32_t *my_scales = reinterpret_cast<const uint32_t *>(mine_a ? sa : sb) + (KS ? my_row : my_row * (nb / 4));
     const int64_t my_step = KS ? (mine_a ? g.M : g.N) : 1;
     auto issue = [&](uint8_t *lds, uint32_t *sc, int kt) {
@@ -603,8 +609,9 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mx_gemm_tiled_kernel(co
         for (int j = 0; j < LB; ++j)
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(gb + off_b[j]),
                                              (__attribute__((address_space(3))) void *)(lds + A_BYTES + (wave + j * NW) * 1024), 16, 0, 0);
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(my_scales + kt * my_step),
-                                         (__attribute__((address_space(3))) void *)(sc + wave * 64), 4, 0, 0);
+        if (wave < SCALE_WAVES)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(my_scales + kt * my_step),
+                                             (__attribute__((address_space(3))) void *)(sc + wave * 64), 4, 0, 0);
     };
 
     const int lr = lane % 32, lg = lane / 32;
@@ -656,6 +663,51 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mx_gemm_tiled_kernel(co
         }
     };
 
+    if constexpr (STAGES == 4) {
+        // The four-stage form of gemm_nt_tiled_kernel (a block alone on its compute unit keeps three K steps of loads in
+        // flight); loads, waits and barriers written as instructions for the reasons given there.  The waves that also
+        // fetch scale dwords have one more load per stage to count.
+        constexpr int PER = LA + LB;
+        static_assert(2 * (PER + 1) <= 63, "the counter holds 63 loads");
+        auto lds_addr_of = [](const void *p) { return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) uint8_t *)p; };
+        auto dma16 = [](const uint8_t *src, uint32_t lds_addr) {
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(src));
+        };
+        auto dma4 = [](const uint32_t *src, uint32_t lds_addr) {
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(lds_addr), "v"(src));
+        };
+        auto fetch = [&](uint8_t *lds, uint32_t *sc, int kt) {
+            const uint8_t *ga = g.a + (int64_t)kt * 128, *gb = g.b + (int64_t)kt * 128;
+            const uint32_t base = lds_addr_of(lds);
+#pragma unroll
+            for (int j = 0; j < LA; ++j) dma16(ga + off_a[j], base + (wave + j * NW) * 1024);
+#pragma unroll
+            for (int j = 0; j < LB; ++j) dma16(gb + off_b[j], base + A_BYTES + (wave + j * NW) * 1024);
+            if (wave < SCALE_WAVES) dma4(my_scales + kt * my_step, lds_addr_of(sc) + wave * 256);
+        };
+        auto phase = [&](const uint8_t *cur, const uint32_t *cur_sc, uint8_t *refill, uint32_t *refill_sc, int kt) {
+            if (wave < SCALE_WAVES) {
+                if (kt + 2 < KT) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * (PER + 1)) : "memory");
+                else if (kt + 1 < KT) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(PER + 1) : "memory");
+                else asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+            } else {
+                if (kt + 2 < KT) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * PER) : "memory");
+                else if (kt + 1 < KT) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(PER) : "memory");
+                else asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+            }
+            if (kt + 3 < KT) fetch(refill, refill_sc, kt + 3);
+            compute(cur, cur_sc);
+        };
+        fetch(lds0, sc0, 0);
+        if (KT > 1) fetch(lds1, sc1, 1);
+        if (KT > 2) fetch(lds2, sc2, 2);
+        for (int kt = 0; kt < KT; kt += 4) {
+            phase(lds0, sc0, lds3, sc3, kt);
+            if (kt + 1 < KT) phase(lds1, sc1, lds0, sc0, kt + 1);
+            if (kt + 2 < KT) phase(lds2, sc2, lds1, sc1, kt + 2);
+            if (kt + 3 < KT) phase(lds3, sc3, lds2, sc2, kt + 3);
+        }
+    } else {
     issue(lds0, sc0, 0);
     for (int kt = 0; kt < KT; kt += 2) {
         __builtin_amdgcn_s_waitcnt(0x0F70);                     // vmcnt(0): my loads into lds0 and sc0 have landed
@@ -668,6 +720,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mx_gemm_tiled_kernel(co
             if (kt + 2 < KT) issue(lds0, sc0, kt + 2);
             compute(lds1, sc1);
         }
+    }
     }
 
     const bool interior = m0 + BM <= g.M && n0 + BN <= g.N;
@@ -765,7 +818,11 @@ static void launch_mx_tiled(const GemmArgs &g, const uint8_t *sa, const uint8_t 
     } else {
         t.tiles_m = (int)((g.M + 127) / 128); t.tiles_n = (int)((g.N + 127) / 128);
         const unsigned grid = (unsigned)(((t.tiles_m * t.tiles_n + 7) / 8) * 8);
-        hipLaunchKernelGGL((mx_gemm_tiled_kernel<128, 128, 2, 2, FA, FB, KS>), dim3(grid), dim3(256), 0, stream, t, sa, sb);
+        // at most one block per compute unit: eight waves and four stages (see gemm_nt_tiled_kernel)
+        if (t.tiles_m * t.tiles_n <= cus)
+            hipLaunchKernelGGL((mx_gemm_tiled_kernel<128, 128, 2, 4, FA, FB, KS, 4>), dim3(grid), dim3(512), 0, stream, t, sa, sb);
+        else
+            hipLaunchKernelGGL((mx_gemm_tiled_kernel<128, 128, 2, 2, FA, FB, KS>), dim3(grid), dim3(256), 0, stream, t, sa, sb);
     }
 }
 
