@@ -99,6 +99,27 @@ def test_random_gemm_within_tolerance_auto_variant(N, shape):
     assert err <= TOL, f"{shape}: max rel err {err}"
 
 
+@pytest.mark.parametrize("k_steps", [1, 2, 3, 4, 5, 6, 7, 9, 13])
+def test_few_tile_outputs_at_every_pipeline_depth(N, k_steps):
+    """Outputs of at most one 128 x 128 tile per compute unit take the four-stage form of the tiled kernel: every length
+    of its prologue and tail (1 .. 3 K steps in flight, a trip count that is not a multiple of four), interior and
+    ragged tiles, one-hot rows so that a misplaced stage shows as a wrong element rather than as noise."""
+    M, Nn, K = 384, 200, 128 * k_steps
+    aq, sa_inv = quantised((M, K), O.E5M2, 1e-3, 40 + k_steps)
+    bq, sb_inv = quantised((Nn, K), O.E4M3, 0.02, 60 + k_steps)
+    out = N.gemm_nt(aq.cuda(), bq.cuda(), O.E5M2, O.E4M3, sa_inv.cuda(), sb_inv.cuda())
+    assert max_rel_err(out, O.t_gemm_nt(aq, bq, O.E5M2, O.E4M3, sa_inv, sb_inv)) <= TOL
+    # A = rows that are zero except for the code of 1.0 at column (7 i) mod K: out[i, j] = B[j, (7 i) mod K] exactly
+    one = torch.ones(1)
+    a1 = torch.zeros((M, K), dtype=torch.uint8)
+    cols = (7 * torch.arange(M)) % K
+    a1[torch.arange(M), cols] = 0x38                                   # 1.0 in E4M3
+    b1 = O.t_cast(seeded_bf16((Nn, K), 1.0, 80 + k_steps).float(), one, O.E4M3)
+    got = N.gemm_nt(a1.cuda(), b1.cuda(), O.E4M3, O.E4M3, one.cuda(), one.cuda(), out_dtype=torch.float32).cpu()
+    want = O.t_decode(b1, O.E4M3)[:, cols].t()
+    assert torch.equal(got, want)
+
+
 @pytest.mark.parametrize("shape", [(512, 512, 1024), (300, 520, 256), (256, 256, 128)])
 def test_random_gemm_every_variant_vs_c_oracle(N, shape):
     """Against the plain-C oracle (sequential fp32 accumulation)."""

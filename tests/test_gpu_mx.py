@@ -255,6 +255,22 @@ def test_mx_gemm_matches_emulation(N, shape, fmts):
         assert torch.equal(got, got32.bfloat16())
 
 
+@pytest.mark.parametrize("k_steps", [1, 2, 3, 4, 5, 6, 7, 9, 13])
+def test_mx_gemm_few_tile_outputs_at_every_pipeline_depth(N, k_steps):
+    """The four-stage form of the tiled kernel (outputs of at most one 128 x 128 tile per compute unit): every length of
+    its prologue and tail, with scale bytes that differ from K step to K step so that a scale dword that arrives with
+    the wrong stage shows."""
+    M, N_, K = 384, 200, 128 * k_steps
+    ac, asc, bc, bsc = _operands(M, N_, K, E5M2, E4M3, seed=500 + k_steps)
+    ref_bf16, _ = O.t_mx_gemm_nt(ac, asc, bc, bsc, E5M2, E4M3, want_f32=True)
+    assert len(set(int(b) for b in asc[0])) > 1 or k_steps == 1
+    for sa_d, sb_d in ((asc.cuda(), bsc.cuda()), (_kstep(asc).cuda(), _kstep(bsc).cuda())):
+        got32 = N.mx_gemm_nt(ac.cuda(), sa_d, bc.cuda(), sb_d, E5M2, E4M3, out_dtype=torch.float32).cpu()
+        _assert_within_hardware_sum(got32, ac, asc, bc, bsc, E5M2, E4M3)
+        got = N.mx_gemm_nt(ac.cuda(), sa_d, bc.cuda(), sb_d, E5M2, E4M3).cpu()
+        assert max_rel_err(got.float(), ref_bf16.float()) <= 1e-2
+
+
 def test_mx_gemm_small_case_against_the_c_oracle_and_bias(N):
     M, N_, K = 48, 40, 96
     ac, asc, bc, bsc = _operands(M, N_, K, E4M3, E4M3, seed=3)
