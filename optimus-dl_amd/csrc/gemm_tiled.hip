@@ -18,6 +18,8 @@
 //   * the two stages are separate __shared__ objects and the K loop is unrolled
 //     by two, so the compiler can prove that the loads in flight into one stage
 //     do not alias the LDS reads of the other (no vmcnt stall in front of them);
+//   * launches of at most one 128 x 128 tile per compute unit use four stages and eight waves instead (three K steps of
+//     loads in flight; see the STAGES == 4 branch);
 //   * block id -> tile mapping is XCD-aware: ids are dealt round-robin to the 8
 //     XCDs by the hardware, so tile = (id % 8) * chunk + id / 8 keeps each XCD on
 //     a contiguous run of tiles, walked in groups of GM rows for L2 reuse.
