@@ -139,6 +139,33 @@ class KernelTimer:
         return out
 
 
+def timed_steps(torch, one, steps, warmup):
+    """`warmup` untimed calls of `one`, then `steps` timed ones.  ms_per_step is wall time over all of them (host clock,
+    synchronised on both sides); min / median / max are per step, from one HIP event between consecutive steps, so a
+    single slow step (an allocator that has to grow, a first-use set-up) shows up as max >> median instead of hiding in
+    the mean.  `allocator` tells whether torch's caching allocator had to go back to the driver during the timed steps."""
+    for _ in range(warmup):
+        one()
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_stats()
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    t0 = time.perf_counter()
+    marks[0].record()
+    for i in range(steps):
+        one()
+        marks[i + 1].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    after = torch.cuda.memory_stats()
+    per = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(steps))
+    return {"ms_per_step": 1e3 * wall / steps, "min_ms": per[0], "median_ms": per[len(per) // 2], "max_ms": per[-1],
+            "max_over_median": per[-1] / per[len(per) // 2],
+            "allocator": {"segments_allocated_during_timed_steps": after.get("num_device_alloc", 0) - before.get("num_device_alloc", 0),
+                          "alloc_retries_during_timed_steps": after.get("num_alloc_retries", 0) - before.get("num_alloc_retries", 0),
+                          "reserved_mib_before": before.get("reserved_bytes.all.current", 0) >> 20,
+                          "reserved_mib_after": after.get("reserved_bytes.all.current", 0) >> 20}}
+
+
 def make_inputs(torch, m=M_TOKENS, device="cuda"):
     g = torch.Generator().manual_seed(0)
     data = {}
@@ -162,7 +189,7 @@ def power_probe(torch, native, step=None, seconds=1.5):
     import glob
     import threading
 
-    from optimus_dl_amd.build import PROBE_LIB_PATH
+    from bench_probe.build import PROBE_LIB_PATH
 
     sensors = sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input"))
     if not sensors:
@@ -377,17 +404,10 @@ def other_configs(torch, steps=8, warmup=3, only=""):
                 with recipe.backward():
                     y.backward(dy)
 
-        for _ in range(warmup):
-            one()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(steps):
-            one()
-        torch.cuda.synchronize()
-        dt = (time.perf_counter() - t0) / steps
+        t = timed_steps(torch, one, steps, warmup)
         flop = sum(6.0 * m * k * n for k, n in shapes)
-        out[label] = {"ms_per_step": 1e3 * dt, "TFLOP/s": flop / dt / 1e12, "flop_per_step": flop}
-        del mods, xs, dys
+        out[label] = {**t, "TFLOP/s": flop / (t["ms_per_step"] * 1e-3) / 1e12, "flop_per_step": flop}
+        del mods, xs, dys, one
         torch.cuda.empty_cache()
     return out
 
@@ -418,20 +438,14 @@ def mlp_block(torch, native, recipe, steps=10, warmup=3):
             with recipe.backward():
                 y.backward(dy)
 
-        for _ in range(warmup):
-            one()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(steps):
-            one()
-        torch.cuda.synchronize()
-        ms = 1e3 * (time.perf_counter() - t0) / steps
-        out[label] = {"ms_per_step": ms, "TFLOP/s": step_flops() / (ms * 1e-3) / 1e12}
-        del mlp
+        t = timed_steps(torch, one, steps, warmup)
+        out[label] = {**t, "TFLOP/s": step_flops() / (t["ms_per_step"] * 1e-3) / 1e12}
+        del mlp, one
+        torch.cuda.empty_cache()
     return out
 
 
-def llama_block(torch, steps=6, warmup=3):
+def llama_block(torch, steps=12, warmup=4):
     """One Llama-3-8B decoder block (RMSNorm, GQA attention with 32 / 8 heads, SwiGLU MLP; fp32 residual stream,
     batch 4 x 2048 tokens), forward + backward, weights re-quantised every step: bf16 autocast, FP8 Linears alone, and FP8
     Linears with the fused RMSNorm / SwiGLU producers.  Attention itself is PyTorch's scaled_dot_product_attention in all three."""
@@ -470,15 +484,9 @@ def llama_block(torch, steps=6, warmup=3):
                     y = blk(x)
                 y.backward(dy)
 
-        for _ in range(warmup):
-            one()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(steps):
-            one()
-        torch.cuda.synchronize()
-        out[label] = {"ms_per_step": 1e3 * (time.perf_counter() - t0) / steps}
-        del blk
+        out[label] = timed_steps(torch, one, steps, warmup)
+        del blk, one, recipe
+        torch.cuda.empty_cache()
     return out
 
 
@@ -540,16 +548,9 @@ def whole_models(torch, which=("gpt2_124m", "qwen3_0.6b"), steps=5, warmup=3, la
                         loss = F.cross_entropy(model(ids)["logits"].view(-1, V).float(), tgt)
                     loss.backward()
 
-            for _ in range(warmup):
-                one()
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            for _ in range(steps):
-                one()
-            torch.cuda.synchronize()
-            dt = (time.perf_counter() - t0) / steps
-            out[name][label] = {"ms_per_step": 1e3 * dt, "tokens_per_s": B * T / dt}
-            del model
+            t = timed_steps(torch, one, steps, warmup)
+            out[name][label] = {**t, "tokens_per_s": B * T / (t["ms_per_step"] * 1e-3)}
+            del model, one, param_set, recipe
             torch.cuda.empty_cache()
     return out
 
@@ -567,9 +568,9 @@ def clock_probe(torch, native, launches=20, settle=40):
     at a high clock, then drops well below its sustained clock and takes some 30 launches (10 ms) to come back."""
     import ctypes
 
-    from optimus_dl_amd.build import PROBE_LIB_PATH
+    from bench_probe.build import PROBE_LIB_PATH
 
-    lib = ctypes.CDLL(PROBE_LIB_PATH)                      # built in-tree by optimus_dl_amd.build.build_probe()
+    lib = ctypes.CDLL(PROBE_LIB_PATH)                      # built in-tree by bench_probe/build.py
     vp = ctypes.c_void_p
     lib.odl_probe_mfma_loop.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, vp, vp]
     lib.odl_probe_mfma_loop_scaled.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, vp, vp]
@@ -870,6 +871,13 @@ def main() -> int:
         line["whole_models_fwd_bwd"] = whole_models(torch)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(torch)
+    # processes this run started that are still alive (none are expected: nothing here forks or spawns)
+    try:
+        import psutil
+
+        line["child_processes_at_exit"] = [" ".join(c.cmdline()[:4]) or c.name() for c in psutil.Process().children(recursive=True)]
+    except Exception as exc:  # psutil missing or /proc unreadable: say so, the figures above do not depend on it
+        line["child_processes_at_exit"] = f"unknown ({type(exc).__name__})"
     print(json.dumps(line))
     return 0
 

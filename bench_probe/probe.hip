@@ -8,7 +8,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
-#include "../gemm_common.h"
+#include "../optimus-dl_amd/csrc/gemm_common.h"
 
 namespace {
 

@@ -45,8 +45,18 @@ enum odl_status {
     ODL_ERR_LAUNCH = 3    /* HIP reported an error at launch */
 };
 
-/* ABI version of this header (14); bumped when a signature changes or an entry point is added. */
+/* ABI version of this header (15); bumped when a signature changes or an entry point is added. */
 int odl_fp8_abi_version(void);
+
+/*
+ * Per-device set-up, for the device that is current on the calling thread: looks up the addresses of the two small
+ * objects in the library's device image (the partial maxima of odl_fp8_cast_dynamic_noalloc, the unit scale of the
+ * block-scaled GEMMs; hipGetSymbolAddress) and the device's compute-unit count.  Every entry point that needs them
+ * makes the same lookups on its first call on a device, so this call is optional -- except for callers that will
+ * make such a first call under HIP stream capture, where the lookup is not allowed: they call this once per device
+ * beforehand.  No counterpart in the reference (its backend initialises itself on import).  Idempotent, launches nothing.
+ */
+int odl_fp8_init_device(void);
 
 /* Last error message of the calling host thread ("" if none). */
 const char *odl_fp8_last_error(void);
@@ -155,7 +165,7 @@ int odl_fp8_multi_cast_delayed(const odl_fp8_mt_tensor *tensors_dev, const int32
  * Every call on a GPU uses that GPU's one array: calls that may overlap on the same GPU (different
  * streams, or different host threads without ordering between their streams) race on it and must be
  * ordered by the caller; calls on one stream are safe.  The first call on a device looks up the array's
- * address (hipGetSymbolAddress): make it once outside of graph capture.
+ * address (hipGetSymbolAddress): make it, or odl_fp8_init_device, once outside of graph capture.
  */
 #define ODL_FP8_NOALLOC_MAX_ELEMS ((int64_t)1 << 31)
 int odl_fp8_cast_dynamic_noalloc(const void *x, int src_dtype, int64_t rows, int64_t cols, int fmt, int margin,
@@ -404,15 +414,19 @@ int odl_fp8_delayed_update(float *history, int64_t H, int64_t R, int64_t ld,
  * mutable process state.  odl_fp8_gemm_variant_name returns a short description ("256x256x128 w4 s2").
  */
 int odl_fp8_gemm_num_variants(void);
-/*
- * Measurement aid (host thread-local, like odl_fp8_gemm_set_variant; NULL switches it off): launch i of the streaming
- * GEMM kernel made from this thread afterwards writes record i % capacity of records_dev, 4 x uint64 =
- * {shader-clock counter, 100 MHz counter} on entry and on exit of the kernel's first wave.  (exit - entry) of the
- * first over (exit - entry) of the second, times 100 MHz, is the average shader clock the board granted that launch.
- */
-int odl_fp8_gemm_set_clock_probe(uint64_t *records_dev, int capacity);
 const char *odl_fp8_gemm_variant_name(int variant);
 int odl_fp8_gemm_set_variant(int variant);
+/*
+ * BENCH-ONLY hook; a production build may compile it out (-DODL_FP8_NO_BENCH_HOOKS removes the entry point and the
+ * two clock reads it switches on in the streaming kernel).  Host thread-local, like odl_fp8_gemm_set_variant; NULL
+ * switches it off: launch i of the streaming GEMM kernel made from this thread afterwards writes record i % capacity
+ * of records_dev, 4 x uint64 = {shader-clock counter, 100 MHz counter} on entry and on exit of the kernel's first
+ * wave.  (exit - entry) of the first over (exit - entry) of the second, times 100 MHz, is the average shader clock
+ * the board granted that launch.  No counterpart in the reference.
+ */
+#ifndef ODL_FP8_NO_BENCH_HOOKS
+int odl_fp8_gemm_set_clock_probe(uint64_t *records_dev, int capacity);
+#endif
 
 /* ---------------------------------------------------------------------------------------------------------------
  * MXFP8: blocks of 32 consecutive elements along the contraction axis share one power-of-two scale, stored as an

@@ -166,23 +166,6 @@ def build(verbose: bool = False, keep_asm: bool = False) -> str:
     return LIB_PATH
 
 
-PROBE_LIB_PATH = os.path.join(HERE, "libodl_probe.so")
-
-
-def build_probe(verbose: bool = False) -> str:
-    """``libodl_probe.so``: the clock stamp and the register-only MFMA loop that bench.py measures with
-    (csrc/probe/probe.hip); not linked into the FP8 library."""
-    cmd = [hipcc_path(), *HIPCC_FLAGS, "-shared", os.path.join(CSRC, "probe", "probe.hip"), "-o", PROBE_LIB_PATH + ".tmp"]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    if r.returncode != 0:
-        raise RuntimeError(f"hipcc failed on probe.hip:\n{r.stdout}")
-    os.replace(PROBE_LIB_PATH + ".tmp", PROBE_LIB_PATH)
-    return PROBE_LIB_PATH
-
-
 if __name__ == "__main__":
     path = build(verbose="-v" in sys.argv, keep_asm="--asm" in sys.argv)
     print(path)
-    print(build_probe(verbose="-v" in sys.argv))

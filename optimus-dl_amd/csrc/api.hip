@@ -41,6 +41,13 @@ int device_cu_count() {
 
 }  // namespace odl
 
-extern "C" int odl_fp8_abi_version(void) { return 14; }
+extern "C" int odl_fp8_abi_version(void) { return 15; }
+
+extern "C" int odl_fp8_init_device(void) {
+    if (!odl::scratch_for_current_device("odl_fp8_init_device")) return ODL_ERR_LAUNCH;
+    if (!odl::unit_scale_for_current_device("odl_fp8_init_device")) return ODL_ERR_LAUNCH;
+    (void)odl::device_cu_count();
+    return ODL_OK;
+}
 
 extern "C" const char *odl_fp8_last_error(void) { return odl::g_err; }

@@ -20,6 +20,10 @@ typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
 int set_error(int code, const char *fmt, ...);   // defined in api.hip
 int check_launch(const char *what);              // hipGetLastError -> status
 int device_cu_count();                           // compute units of the CURRENT device (cached per device, api.hip)
+// Device addresses of the two objects in the library's device image, for the CURRENT device (looked up once per device
+// with hipGetSymbolAddress, which must not run under stream capture; odl_fp8_init_device makes both lookups):
+float *scratch_for_current_device(const char *who);            // quant.hip: partial maxima of the entry point that allocates nothing
+const float *unit_scale_for_current_device(const char *who);   // mx.hip: the 1.0f the block-scaled GEMM epilogues multiply by
 
 __device__ __forceinline__ float bits_to_float(uint32_t u) { return __builtin_bit_cast(float, u); }
 __device__ __forceinline__ uint32_t float_to_bits(float f) { return __builtin_bit_cast(uint32_t, f); }

@@ -163,6 +163,7 @@ void odl::attach_clock_probe(GemmArgs &g) {
     ++t_clock_next;
 }
 
+#ifndef ODL_FP8_NO_BENCH_HOOKS
 extern "C" int odl_fp8_gemm_set_clock_probe(uint64_t *records_dev, int capacity) {
     if (records_dev && capacity < 1) return set_error(ODL_ERR_ARG, "odl_fp8_gemm_set_clock_probe: capacity %d", capacity);
     t_clock_probe = reinterpret_cast<unsigned long long *>(records_dev);
@@ -170,6 +171,7 @@ extern "C" int odl_fp8_gemm_set_clock_probe(uint64_t *records_dev, int capacity)
     t_clock_next = 0;
     return ODL_OK;
 }
+#endif
 
 extern "C" int odl_fp8_gemm_set_variant(int variant) {
     if (variant < -1 || variant >= kNumVariants) return set_error(ODL_ERR_ARG, "odl_fp8_gemm_set_variant: %d out of range", variant);

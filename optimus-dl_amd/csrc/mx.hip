@@ -778,7 +778,7 @@ static __device__ float mx_unit_scale = 1.0f;
 
 namespace odl {
 
-static const float *unit_scale_for_current_device(const char *who) {
+const float *unit_scale_for_current_device(const char *who) {
     constexpr int kMaxDevices = 64;
     static const float *cached[kMaxDevices] = {};
     int dev = -1;

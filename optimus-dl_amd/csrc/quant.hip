@@ -1315,7 +1315,7 @@ static float *g_scratch_ptr[kMaxScratchDevices] = {};
 
 // Device address of `scratch` on the device that is current on this thread (nullptr + error text on failure).
 // Two threads that resolve the same device at once store the same pointer.
-static float *scratch_for_current_device(const char *who) {
+float *scratch_for_current_device(const char *who) {
     int dev = -1;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) { set_error(ODL_ERR_LAUNCH, "%s: hipGetDevice: %s", who, hipGetErrorString(e)); return nullptr; }

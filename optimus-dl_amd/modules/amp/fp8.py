@@ -15,13 +15,16 @@ owns the scaling policy itself:
               autocast / backward context exits                 (one pass)
   rowwise     (extension, no reference enum) one scale per row of each operand
               along its non-contracted axis
-  blockwise / mxfp8 are accepted by the parsers, as in the reference, but have
-  no kernels here: constructing a recipe with them raises NotImplementedError.
+  mxfp8       OCP microscaling: 32-element blocks along the contraction axis,
+              one E8M0 scale byte each, applied by the MFMA      (one pass)
+  blockwise   1 x 128 blocks (activations, gradients) and 128 x 128 blocks
+              (weights) with power-of-two scales, same GEMM      (one pass)
 """
 
 from __future__ import annotations
 
 import logging
+import weakref
 from collections.abc import Iterator
 from contextlib import contextmanager
 from dataclasses import dataclass
@@ -152,6 +155,8 @@ class FP8Recipe:
                 "The FP8 kernel library (libodl_fp8.so) and a visible MI355X are required for FP8 training. "
                 "Build the library with: python -m optimus_dl_amd.build"
             )
+        if torch.cuda.is_available():
+            native.init_device()      # per-device look-ups of the library, which must not happen under graph capture
         self.recipe_type = get_fp8_recipe_type_from_string(recipe_type) if isinstance(recipe_type, str) else recipe_type
         self.format = get_fp8_format_from_string(format) if isinstance(format, str) else format
         self.margin = margin
@@ -201,6 +206,8 @@ class FP8Recipe:
         # partial maxima handed over by the kernel that produced a tensor (SwiGLU, RMSNorm), so that
         # the Linear that quantises this very tensor skips its amax pass; a handful of entries
         self.producer_parts: list[tuple[tuple, torch.Tensor, torch.Tensor]] = []
+        # Fp8ParamSets attached under this recipe (delayed scaling: they re-record their weights' maxima at each refresh)
+        self._param_sets: "weakref.WeakSet" = weakref.WeakSet()
         _info_once(
             f"Created FP8 recipe with format={self.format.value}, amax_history_len={amax_history_len}, "
             f"amax_compute_algo={amax_compute_algo}"
@@ -225,6 +232,9 @@ class FP8Recipe:
             return
         algo = native.AMAX_MAX if self.amax_compute_algo == "max" else native.AMAX_MOST_RECENT
         for arena in self._store.dirty_arenas(direction):
+            if direction == "fwd":
+                for ps in self._param_sets:
+                    ps.refold(arena)
             R = arena.used
             native.delayed_update_raw(arena.history, arena.H, arena.capacity, R, arena.scale, arena.scale_inv,
                                       arena.fmt, self.margin, algo, amax_parts=arena.parts)
@@ -277,7 +287,8 @@ class FP8Recipe:
     def load_state_dict(self, model: torch.nn.Module, state: dict, strict: bool = True) -> None:
         """Restore what :meth:`state_dict` saved.  The roles of every module are reserved here, so the
         call works on a freshly built model that has not run a forward yet.  Quantised weights cached
-        under other scales are invalidated.  strict: module names that are in ``state`` and not in the
+        under other scales are invalidated (an attached ``Fp8ParamSet`` casts its weights again, so the order
+        "load the weights, attach the set, load this state" resumes on the codes of the uninterrupted run).  strict: module names that are in ``state`` and not in the
         model, or the reverse, raise ``KeyError``."""
         if not self.is_delayed:
             return
@@ -309,6 +320,16 @@ class FP8Recipe:
                     meta.first_record_epoch = -1
         for arena in touched:          # codes made under the old scales are stale
             arena.epoch += 1
+        # ... including the codes an Fp8ParamSet keeps per optimizer step (made at whatever scale was in force at
+        # its last sync, e.g. the initial scale 1 of a freshly attached set): they are dropped, and the sets attached
+        # under this recipe cast their weights again now, under the restored scales
+        for mod in mods.values():
+            cache = getattr(mod, "_wcache", None)
+            if cache is not None:
+                cache.kept = None
+                cache.key = None
+        for ps in list(self._param_sets):
+            ps.sync()
 
     # ------------------------------------------------------- producer hand-over
     @staticmethod

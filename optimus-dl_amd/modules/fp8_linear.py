@@ -229,9 +229,13 @@ class _Fp8LinearFn(torch.autograd.Function):
             ctx.wgrad_direct = (fp8_wgrad and recipe.direct_layouts
                                 and native.gemm_layouts_supported(n_out, n_in, tokens, weight.dtype))
             if pol.kind == "delayed":
-                meta = module._meta(recipe, x2d.device, "fwd", create=module.training)
+                # the histories see a forward only when it is part of training: the module in training mode AND
+                # grad mode on (the reference's backend refreshes its state on the same condition), so a validation
+                # pass under torch.no_grad() without model.eval() reads the scales and leaves the histories alone
+                record = module._records()
+                meta = module._meta(recipe, x2d.device, "fwd", create=record)
                 xq, xq_t, sx_inv = _quantise_delayed(x2d, pol.fmt_fwd, meta, ROLE_X, fp8_wgrad, recipe=recipe,
-                                                     record=module.training, margin=pol.margin)
+                                                     record=record, margin=pol.margin)
             else:
                 xq, xq_t, sx_inv = _quantise_input_shared(recipe, x2d, pol.fmt_fwd, pol.margin, fp8_wgrad)
             wq, wq_t, sw_inv = module._tensor_weight(weight, recipe, need_t=need_dgrad)
@@ -399,13 +403,17 @@ class FP8Linear(nn.Linear):
         self.fp8_meta["scaling_fwd" if direction == "fwd" else "scaling_bwd"] = meta
         return meta
 
+    def _records(self) -> bool:
+        """Whether a forward of this module feeds the delayed-scaling histories: training mode and grad mode."""
+        return self.training and torch.is_grad_enabled()
+
     def _tensor_weight(self, weight: torch.Tensor, recipe: FP8Recipe, need_t: bool):
         """Per-tensor quantised weight (and transpose), cached on the parameter version."""
         pol = recipe.recipe
         c = self._wcache
         if c.kept is not None and recipe.cache_weights and c.kept == _kept_stamp(weight, pol):
             return c.wq, c.wq_t, c.s_inv
-        record = self.training
+        record = self._records()
         meta = None
         # the codes depend on the parameter's contents, the format and how the scale is found; under delayed
         # scaling also on the scale in force, which changes with every refresh of the arena
@@ -575,6 +583,12 @@ class Fp8ParamSet:
         else:
             self._plan = native.MultiTensorPlan(sources, pol.fmt_fwd, pol.margin)
         self._index, self._metas = index, metas
+        # the rows of each arena's strip table that hold these weights' partial maxima
+        rows: dict = {}
+        for meta in metas:
+            rows.setdefault(meta.arena, []).append(meta.first + ROLE_W)
+        self._w_rows = {arena: torch.tensor(idx, dtype=torch.long, device=arena.parts.device) for arena, idx in rows.items()}
+        self._w_snap: dict = {}
 
     @torch.no_grad()
     def sync(self) -> None:
@@ -588,6 +602,9 @@ class Fp8ParamSet:
         plan.run()
         for meta in self._metas:                     # delayed: the next refresh has to fold what was just recorded
             meta.note_record(self.recipe._store)
+        # ... and so has every later refresh until the next sync: the strips are cleared by each refresh (one per
+        # microbatch), while the kept codes launch nothing that would record the weights' maxima again
+        self._w_snap = {arena: arena.parts.index_select(0, idx) for arena, idx in self._w_rows.items()}
         how = (pol.kind, pol.margin)
         for m, i in zip(self.modules, self._index):
             c = m._wcache
@@ -600,11 +617,22 @@ class Fp8ParamSet:
                 c.amax, c.key = None, None
         self.syncs += 1
 
+    def refold(self, arena) -> None:
+        """Called by the recipe before it refreshes ``arena``: the maxima recorded at the last sync count for this
+        step too (three small launches per refresh, whatever the number of weights), so the weight roles' histories
+        advance one real entry per refresh as on the per-module route, which folds its cached amax on every reuse."""
+        snap = self._w_snap.get(arena)
+        if snap is None:
+            return
+        idx = self._w_rows[arena]
+        arena.parts.index_copy_(0, idx, torch.maximum(arena.parts.index_select(0, idx), snap))
+
     @classmethod
     def attach(cls, model: nn.Module, recipe: FP8Recipe, optimizer: "torch.optim.Optimizer | None" = None) -> "Fp8ParamSet":
         """The set of every ``FP8Linear`` under ``model``, quantised once now; with an optimizer, again after each
         of its steps."""
         ps = cls([m for m in model.modules() if isinstance(m, FP8Linear)], recipe)
+        recipe._param_sets.add(ps)
         ps.sync()
         if optimizer is not None:
             ps.hook = optimizer.register_step_post_hook(lambda *_a, **_k: ps.sync())

@@ -24,7 +24,7 @@ DT_BF16, DT_F32 = 0, 1
 AMAX_MAX, AMAX_MOST_RECENT = 0, 1
 FP8_MAX = {E4M3: 448.0, E5M2: 57344.0}
 TORCH_FP8 = {E4M3: torch.float8_e4m3fn, E5M2: torch.float8_e5m2}
-ABI_VERSION = 14
+ABI_VERSION = 15
 AMAX_PARTS = 512                       # ODL_FP8_AMAX_PARTS
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
@@ -34,6 +34,7 @@ LIB_PATH = os.environ.get("ODL_FP8_LIB") or os.path.join(_HERE, "libodl_fp8.so")
 EXPORTS = (
     "odl_fp8_abi_version",
     "odl_fp8_last_error",
+    "odl_fp8_init_device",
     "odl_fp8_amax",
     "odl_fp8_scale_from_amax",
     "odl_fp8_amax_scale",
@@ -151,6 +152,30 @@ def load() -> ctypes.CDLL:
             raise NativeError(f"{LIB_PATH}: ABI {L.odl_fp8_abi_version()} != expected {ABI_VERSION}; rebuild")
         _lib = L
     return _lib
+
+
+_devices_ready: set[int] = set()
+
+
+def init_device(device: "torch.device | int | None" = None) -> None:
+    """Per-device set-up of the library (``odl_fp8_init_device``), once per device and process.  The wrappers whose
+    kernels need it (:func:`cast_dynamic_noalloc`, the block-scaled GEMMs) call it themselves; it has to happen outside
+    of HIP stream capture, so a caller that captures graphs and has not used those wrappers before calls this first
+    (``FP8Recipe`` does, when it is built)."""
+    if device is None:
+        index = torch.cuda.current_device()
+    elif isinstance(device, int):
+        index = device
+    else:
+        index = device.index if device.index is not None else torch.cuda.current_device()
+    if index in _devices_ready:
+        return
+    if torch.cuda.is_current_stream_capturing():
+        raise NativeError(f"cuda:{index} has not been set up for the FP8 library yet and the current stream is being captured: "
+                          "call optimus_dl_amd.native.init_device() once before the capture")
+    with torch.cuda.device(index):
+        _check(load().odl_fp8_init_device(), "odl_fp8_init_device")
+    _devices_ready.add(index)
 
 
 def _check(status: int, what: str) -> None:
@@ -301,6 +326,7 @@ def cast_dynamic_noalloc(x: torch.Tensor, fmt: int, margin: int, out: torch.Tens
         if t is not None and not (t.is_cuda and t.dtype == torch.uint8 and t.is_contiguous() and tuple(t.shape) == shape):
             raise NativeError(f"cast_dynamic_noalloc: {what} must be a contiguous uint8 CUDA tensor of shape {shape}")
     _f32_dev(dyn_out, 3, "cast_dynamic_noalloc dyn_out")
+    init_device(x.device)
     _check(load().odl_fp8_cast_dynamic_noalloc(x.data_ptr(), _src_dtype(x), rows, cols, fmt, margin,
                                                out.data_ptr() if out is not None else None,
                                                out_t.data_ptr() if out_t is not None else None, dyn_out.data_ptr(), _stream()),
@@ -834,10 +860,12 @@ def mx_gemm_nt(a: torch.Tensor, sa: torch.Tensor, b: torch.Tensor, sb: torch.Ten
     splits = gemm_split_count(M, N, K) if layout == MX_KSTEP else 1
     if splits > 1:
         workspace = torch.empty((splits, M, N), dtype=torch.float32, device=a.device)
+        init_device(a.device)
         _check(load().odl_fp8_mx_gemm_splitk(a.data_ptr(), sa.data_ptr(), b.data_ptr(), sb.data_ptr(), M, N, K, fmt_a, fmt_b,
                                              bias.data_ptr() if bias is not None else None, out.data_ptr(), odt, splits,
                                              workspace.data_ptr(), workspace.numel() * 4, _stream()), "odl_fp8_mx_gemm_splitk")
         return out
+    init_device(a.device)
     _check(load().odl_fp8_mx_gemm_nt(a.data_ptr(), sa.data_ptr(), b.data_ptr(), sb.data_ptr(), layout, M, N, K, fmt_a, fmt_b,
                                      bias.data_ptr() if bias is not None else None, out.data_ptr(), odt, _stream()),
            "odl_fp8_mx_gemm_nt")

@@ -253,3 +253,62 @@ def test_param_set_under_delayed_scaling_matches_the_per_module_route(N, amp):
         opt_b.step()
     finally:
         N.cast_delayed = real
+
+
+def test_param_set_records_the_weight_amax_in_every_microbatch_under_delayed_scaling(N, amp):
+    """The kept codes launch nothing for the weights, and every microbatch ends in a refresh that clears the strips of
+    partial maxima: the set folds the maxima of its last sync back in before each refresh, so the weight role's history
+    gets one real entry per refresh (as on the per-module route, which folds its cached amax on every reuse) instead
+    of one real entry and then zeros."""
+    kept = build()
+    recipe = amp.create_fp8_recipe("delayed", "hybrid", amax_history_len=4)
+    opt = torch.optim.SGD(kept.parameters(), lr=0.05)
+    ps = recipe.attach_params(kept, opt)
+    assert ps is not None
+    x = seeded_bf16((64, 256), 1.0, 470).cuda()
+    for micro in range(3):                                       # three microbatches, no optimizer step in between
+        with amp.fp8_autocast(torch.device("cuda"), recipe):
+            y, z = kept(x)
+        with amp.fp8_backward(recipe):
+            (y.float().square().mean() + z.float().square().mean()).backward()
+    for name in ("a", "b"):
+        mod = getattr(kept, name)
+        hist = mod.fp8_meta["scaling_fwd"].amax_history[:, 1]    # role 1 = the weight
+        want = mod.weight.detach().float().abs().max()
+        # the refresh rolls the history: after three refreshes three of the four rows hold the weight's amax
+        assert int((hist == want).sum()) == 3, (name, hist.tolist(), float(want))
+
+
+def test_loading_scaling_state_drops_the_codes_the_param_set_kept(N, amp):
+    """Resume order: load the weights, attach the set (which casts every weight at the initial scale 1), then load the
+    scaling state.  The codes the set made under scale 1 must not survive the load: the first step of the resumed run
+    equals the next step of the uninterrupted one bit for bit."""
+    import copy
+
+    def step(net, recipe, x):
+        for p in net.parameters():
+            p.grad = None
+        with amp.fp8_autocast(torch.device("cuda"), recipe):
+            y, z = net(x)
+            loss = y.float().square().mean() + z.float().square().mean()
+        with amp.fp8_backward(recipe):
+            loss.backward()
+        return [y.detach().clone(), z.detach().clone()] + [p.grad.detach().clone() for p in net.parameters()]
+
+    net, recipe = build(), amp.create_fp8_recipe("delayed", "hybrid", amax_history_len=4)
+    ps = recipe.attach_params(net)
+    for s in range(3):
+        step(net, recipe, seeded_bf16((64, 256), 1.0 + 0.3 * s, 480 + s).cuda())
+        ps.sync()                                                # where the optimizer step would be (weights unchanged here)
+    blob, weights = copy.deepcopy(recipe.state_dict(net)), copy.deepcopy(net.state_dict())
+
+    net2, recipe2 = build(), amp.create_fp8_recipe("delayed", "hybrid", amax_history_len=4)
+    net2.load_state_dict(weights)
+    ps2 = recipe2.attach_params(net2)                            # casts at scale 1: a weight of std 0.02 lands in the subnormals
+    recipe2.load_state_dict(net2, blob)
+    for i in range(len(ps._plan.codes)):                         # cast again under the restored scales, not left at scale 1
+        assert torch.equal(ps2._plan.codes[i], ps._plan.codes[i]) and torch.equal(ps2._plan.dyn[i], ps._plan.dyn[i])
+    x = seeded_bf16((64, 256), 2.0, 490).cuda()
+    got, want = step(net2, recipe2, x), step(net, recipe, x)
+    for i, (a, b) in enumerate(zip(got, want)):
+        assert torch.equal(a, b), f"tensor {i} of the resumed step differs"

@@ -247,3 +247,39 @@ def test_activation_checkpointing_drops_the_saved_fp8_tensors(amp):
     assert torch.equal(gx_plain, gx_ckpt)
     for a, b in zip(gw_plain, gw_ckpt):
         assert torch.equal(a, b)
+
+
+def test_no_grad_forward_in_training_mode_leaves_the_histories_alone(amp):
+    """A validation pass under torch.no_grad() WITHOUT model.eval(): the reference's backend refreshes its scaling
+    state only when grad mode is on, so such a pass reads the trained scales and records nothing."""
+    M, K, N, H = 128, 256, 128, 4
+    lin = make_linear(seeded_bf16((N, K), 0.02, 601))
+    recipe = amp.create_fp8_recipe("delayed", "hybrid", amax_history_len=H)
+    for s in range(2):
+        train_step(lin, recipe, seeded_bf16((M, K), 1.0 + s, 602 + s), seeded_bf16((M, N), 1e-3, 610 + s))
+    meta = lin.fp8_meta["scaling_fwd"]
+    hist, scale = meta.amax_history.clone(), meta.scale.clone()
+    assert lin.training
+    with torch.no_grad(), recipe.autocast():
+        y = lin(seeded_bf16((M, K), 50.0, 620).cuda())          # much larger than anything training saw
+    assert torch.equal(meta.amax_history, hist) and torch.equal(meta.scale, scale)
+    assert float(meta.pending_amax.max()) == 0.0
+    assert torch.isfinite(y.float()).all()
+
+
+def test_first_use_under_stream_capture_is_refused_until_the_device_is_set_up(monkeypatch):
+    """The per-device look-ups of the library must not run under stream capture: a wrapper that needs them raises,
+    in words, when its first use on a device would fall into a capture; after native.init_device() it goes through."""
+    from optimus_dl_amd import native as N
+
+    x = seeded_bf16((64, 128), 1.0, 630).cuda()
+    out, dyn = torch.empty((64, 128), dtype=torch.uint8, device="cuda"), torch.empty(3, device="cuda")
+    monkeypatch.setattr(N, "_devices_ready", set())
+    monkeypatch.setattr(torch.cuda, "is_current_stream_capturing", lambda: True)
+    with pytest.raises(N.NativeError, match="init_device"):
+        N.cast_dynamic_noalloc(x, N.E4M3, 0, out, None, dyn)
+    monkeypatch.undo()
+    N.init_device()
+    N.cast_dynamic_noalloc(x, N.E4M3, 0, out, None, dyn)
+    want, _, _, _, _ = N.quantize_dynamic(x, N.E4M3, 0, want_transposed=False)
+    assert torch.equal(out, want)
