@@ -337,6 +337,14 @@ int odl_fp8_cast_delayed(const void *x, int src_dtype, int64_t rows, int64_t col
  *   sa_inv   : 1 value (sa_n == 1) or M values; sb_inv: 1 or N values
  *   bias     : NULL or N fp32 values (bias_dtype must be ODL_F32), added in fp32
  *              before the single rounding to out_dtype
+ *   accumulate : 0: C is overwritten.  Non-zero: C = C + product, the old value of C joining the fp32 sum
+ *              after the bias, i.e. out = round(fl(fl(fl(acc * s) + bias) + C_old)): ONE rounding to out_dtype.
+ *              This is the accumulate flag of the backend's GEMM: the weight gradient of a microbatch added
+ *              into the gradient buffer (gradient accumulation,
+ *              optimus_dl/recipe/train/mixins/execution/iteration_mixin.py:332), and the data gradients of
+ *              Linears fed by one tensor (q/k/v, gate/up) summed without a separate pass.  Such a call runs on
+ *              the kernels whose tiles end in a separate output phase (the old values are requested one slab of
+ *              32 rows ahead), not on the streaming kernel.
  * Covers fwd (A=Xq, B=Wq), dgrad (A=dYq, B=Wq^T) and wgrad (A=dYq^T, B=Xq^T):
  * the three GEMMs of te.pytorch.Linear forward/backward.
  * K must be a multiple of 16; any M, N >= 1.
@@ -345,7 +353,7 @@ int odl_fp8_gemm_nt(const uint8_t *a, const uint8_t *b, int64_t M, int64_t N, in
                     int fmt_a, int fmt_b,
                     const float *sa_inv, int64_t sa_n, const float *sb_inv, int64_t sb_n,
                     const void *bias, int bias_dtype,
-                    void *c, int out_dtype, odl_stream_t stream);
+                    void *c, int out_dtype, int accumulate, odl_stream_t stream);
 
 /*
  * The same product for operands that need no transposed copy.  layout_a / layout_b say how an
@@ -358,7 +366,9 @@ int odl_fp8_gemm_nt(const uint8_t *a, const uint8_t *b, int64_t M, int64_t N, in
  * Results equal those of odl_fp8_gemm_nt on the transposed copies bit for bit (same order of
  * accumulation).  One scale per operand, no bias, out_dtype ODL_BF16 or ODL_F32 (weight gradients
  * of fp32 master weights); M, N, K multiples of 256, K >= 512: anything else is refused with
- * ODL_ERR_SHAPE (make the transposed copy and use odl_fp8_gemm_nt).
+ * ODL_ERR_SHAPE (make the transposed copy and use odl_fp8_gemm_nt).  There is no accumulate flag here
+ * (only the streaming kernel reads K-slow operands): C = C + product with such operands is
+ * odl_fp8_gemm_splitk with accumulate set, which takes a single run as well.
  */
 enum odl_operand_layout { ODL_K_FAST = 0, ODL_K_SLOW = 1 };
 int odl_fp8_gemm_layouts(const uint8_t *a, const uint8_t *b, int64_t M, int64_t N, int64_t K,
@@ -375,13 +385,16 @@ int odl_fp8_gemm_layouts(const uint8_t *a, const uint8_t *b, int64_t M, int64_t 
  * bit-identical where every partial sum is exact.  odl_fp8_gemm_split_count proposes `splits`
  * for a shape (1 = not worth splitting; k_slow != 0: an operand will be passed K-slow); any 2 <= splits <= 64 that leaves every run at least 512
  * long is accepted.  M, N, K multiples of 128 (256 for an operand stored K-slow), K-run >= 512.
+ * accumulate != 0: the second kernel adds the old value of C to the sum before the one rounding
+ * (C = C + product, as for odl_fp8_gemm_nt); splits == 1 is then accepted too, which is how a product
+ * with an operand stored K-slow (a weight gradient that reads dY as stored) is added into C.
  * No counterpart in the reference, whose GEMMs are cuBLASLt's choice inside te.pytorch.Linear.
  */
 int odl_fp8_gemm_split_count(int64_t M, int64_t N, int64_t K, int k_slow);
 int odl_fp8_gemm_splitk(const uint8_t *a, const uint8_t *b, int64_t M, int64_t N, int64_t K,
                         int fmt_a, int fmt_b, int layout_a, int layout_b,
                         const float *sa_inv, int64_t sa_n, const float *sb_inv, int64_t sb_n,
-                        const float *bias, void *c, int out_dtype, int splits,
+                        const float *bias, void *c, int out_dtype, int accumulate, int splits,
                         void *workspace, int64_t workspace_bytes, odl_stream_t stream);
 
 /*
@@ -461,10 +474,12 @@ int odl_fp8_mx_cast(const void *x, int src_dtype, int64_t rows, int64_t cols, in
  * M % 128 == 0, N % 128 == 0, K >= 512 and enough tiles to fill the chip the persistent streaming kernel runs (the one of
  * odl_fp8_gemm_nt, with the scale dwords riding beside the operand loads); K % 128 == 0 with 4-byte aligned scale arrays
  * otherwise runs an LDS-tiled kernel; other shapes a plain one-wave-per-tile kernel.  The first call on a device looks up a
- * constant in the library's device image (hipGetSymbolAddress): make it outside of stream capture.
+ * constant in the library's device image (hipGetSymbolAddress): make it outside of stream capture.  accumulate: as for
+ * odl_fp8_gemm_nt (C = C + product, one rounding; not on the streaming kernel).
  */
 int odl_fp8_mx_gemm_nt(const uint8_t *a, const uint8_t *sa, const uint8_t *b, const uint8_t *sb, int scales_layout, int64_t M,
-                       int64_t N, int64_t K, int fmt_a, int fmt_b, const float *bias, void *c, int out_dtype, odl_stream_t stream);
+                       int64_t N, int64_t K, int fmt_a, int fmt_b, const float *bias, void *c, int out_dtype, int accumulate,
+                       odl_stream_t stream);
 
 /*
  * odl_fp8_mx_gemm_nt with K cut into `splits` runs that are computed side by side, for outputs of few tiles and a long
@@ -474,7 +489,7 @@ int odl_fp8_mx_gemm_nt(const uint8_t *a, const uint8_t *sa, const uint8_t *b, co
  * 128; every run at least 512 long.
  */
 int odl_fp8_mx_gemm_splitk(const uint8_t *a, const uint8_t *sa, const uint8_t *b, const uint8_t *sb, int64_t M, int64_t N, int64_t K,
-                           int fmt_a, int fmt_b, const float *bias, void *c, int out_dtype, int splits, void *workspace,
+                           int fmt_a, int fmt_b, const float *bias, void *c, int out_dtype, int accumulate, int splits, void *workspace,
                            int64_t workspace_bytes, odl_stream_t stream);
 
 /*

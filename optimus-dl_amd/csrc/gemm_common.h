@@ -19,6 +19,7 @@ struct GemmArgs {
     int64_t M, N, K;
     int sa_vec, sb_vec;          // 0 = one value, 1 = one per row of A / B
     int out_dtype;               // bias, when present, is fp32
+    int accumulate = 0;          // C = C + product (one rounding) instead of C = product; not in the streaming kernel
     int tiles_m, tiles_n;
     int ta = 0, tb = 0;          // operand stored [K, M] / [K, N] (contraction index slow); streaming kernel only
     // streaming kernel only: splits > 1 cuts K into `splits` runs of `split_steps` 128-byte steps (an even number;
@@ -70,21 +71,30 @@ __device__ __forceinline__ void store_tile(const GemmArgs &g, const v16f &acc, i
         if constexpr (OUT_BF16) {
             uint16_t *c = reinterpret_cast<uint16_t *>(g.c) + m * g.N + n;
             if (INTERIOR || (n + 3 < g.N && (g.N & 3) == 0)) {
+                if (g.accumulate) {
+                    const u32x2 old = *reinterpret_cast<const u32x2 *>(c);
+                    v[0] = v[0] + bits_to_float(old.x << 16); v[1] = v[1] + bits_to_float(old.x & 0xffff0000u);
+                    v[2] = v[2] + bits_to_float(old.y << 16); v[3] = v[3] + bits_to_float(old.y & 0xffff0000u);
+                }
                 u32x2 pk = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
                 *reinterpret_cast<u32x2 *>(c) = pk;
             } else {
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
-                    if (n + e < g.N) c[e] = (uint16_t)f32_to_bf16_bits(v[e]);
+                    if (n + e < g.N) c[e] = (uint16_t)f32_to_bf16_bits(g.accumulate ? v[e] + bits_to_float((uint32_t)c[e] << 16) : v[e]);
             }
         } else {
             float *c = reinterpret_cast<float *>(g.c) + m * g.N + n;
             if (INTERIOR || (n + 3 < g.N && (g.N & 3) == 0)) {
+                if (g.accumulate) {
+                    const float4 old = *reinterpret_cast<const float4 *>(c);
+                    v[0] = v[0] + old.x; v[1] = v[1] + old.y; v[2] = v[2] + old.z; v[3] = v[3] + old.w;
+                }
                 *reinterpret_cast<float4 *>(c) = float4{v[0], v[1], v[2], v[3]};
             } else {
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
-                    if (n + e < g.N) c[e] = v[e];
+                    if (n + e < g.N) c[e] = g.accumulate ? v[e] + c[e] : v[e];
             }
         }
     }
@@ -159,6 +169,82 @@ __device__ __forceinline__ void epilogue_staged(const GemmArgs &g, v16f (&acc)[T
     }
 }
 
+// The same output path for C = C + product: the slab is staged as fp32 whatever the output type (the sum is rounded
+// once), TNS sub-tiles wide (32 * (TNS * 128 + 16) bytes of `wave_lds`), and a lane that has read back four values of
+// a row adds the four old values of C, which it requested one slab earlier (the loads of slab k + 1 are in flight
+// while slab k is scaled, staged and stored).  Ordinary stores: what is accumulated into is read again.
+template <bool OUT_BF16, int TM, int TN, int TNS>
+__device__ __forceinline__ void epilogue_staged_accumulate(const GemmArgs &g, v16f (&acc)[TM][TN], uint8_t *wave_lds,
+                                                           int64_t m_wave, int64_t n_wave, int lane) {
+    static_assert(TN % TNS == 0, "slab width must divide the wave tile");
+    constexpr int ESZ = OUT_BF16 ? 2 : 4;
+    constexpr int ROW_BYTES = TNS * 32 * 4, PITCH = ROW_BYTES + 16;
+    constexpr int LPR = ROW_BYTES / 16;            // lanes that cover one slab row with four floats each
+    constexpr int RPI = 64 / LPR, NI = 32 / RPI;   // rows per instruction, instructions per slab
+    constexpr int SLABS = TM * (TN / TNS);
+    const int lr = lane % 32, lg = lane / 32;
+    const bool vec = g.sa_vec | g.sb_vec | (g.bias != nullptr);
+    const float s_tensor = g.sa[0] * g.sb[0];
+    const float *bias = reinterpret_cast<const float *>(g.bias);
+    uint8_t *out = reinterpret_cast<uint8_t *>(g.c);
+    auto c_ptr = [&](int slab, int i) -> uint8_t * {   // where this lane's four values of instruction i of a slab live
+        const int t = slab / (TN / TNS), us = (slab % (TN / TNS)) * TNS;
+        const int r = i * RPI + lane / LPR, chunk = lane % LPR;
+        return out + ((m_wave + 32 * t + r) * g.N + n_wave + 32 * us + 4 * chunk) * ESZ;
+    };
+    auto fetch_old = [&](float (&old)[NI][4], int slab) {
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            if constexpr (OUT_BF16) {
+                const u32x2 o = *reinterpret_cast<const u32x2 *>(c_ptr(slab, i));
+                old[i][0] = bits_to_float(o.x << 16); old[i][1] = bits_to_float(o.x & 0xffff0000u);
+                old[i][2] = bits_to_float(o.y << 16); old[i][3] = bits_to_float(o.y & 0xffff0000u);
+            } else {
+                const float4 o = *reinterpret_cast<const float4 *>(c_ptr(slab, i));
+                old[i][0] = o.x; old[i][1] = o.y; old[i][2] = o.z; old[i][3] = o.w;
+            }
+        }
+    };
+    float old[2][NI][4];
+    fetch_old(old[0], 0);
+#pragma unroll
+    for (int slab = 0; slab < SLABS; ++slab) {
+        const int t = slab / (TN / TNS), us = (slab % (TN / TNS)) * TNS;
+        if (slab + 1 < SLABS) fetch_old(old[(slab + 1) & 1], slab + 1);
+        float sa = 1.0f;
+        if (vec) sa = g.sa[(m_wave + 32 * t + lr) * g.sa_vec];
+#pragma unroll
+        for (int uu = 0; uu < TNS; ++uu) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int col = 32 * uu + 8 * q + 4 * lg;    // first of this lane's 4 columns inside the slab
+                float v[4];
+                if (vec) {
+                    const int64_t n = n_wave + 32 * us + col;
+                    float sb[4] = {g.sb[0], g.sb[0], g.sb[0], g.sb[0]};
+                    if (g.sb_vec) { const float4 t4 = *reinterpret_cast<const float4 *>(g.sb + n); sb[0] = t4.x; sb[1] = t4.y; sb[2] = t4.z; sb[3] = t4.w; }
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = acc[t][us + uu][4 * q + e] * (sa * sb[e]);
+                    if (bias) { const float4 b4 = *reinterpret_cast<const float4 *>(bias + n); v[0] = v[0] + b4.x; v[1] = v[1] + b4.y; v[2] = v[2] + b4.z; v[3] = v[3] + b4.w; }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = acc[t][us + uu][4 * q + e] * s_tensor;
+                }
+                *reinterpret_cast<float4 *>(wave_lds + lr * PITCH + col * 4) = float4{v[0], v[1], v[2], v[3]};
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const int r = i * RPI + lane / LPR, chunk = lane % LPR;
+            const float4 val = *reinterpret_cast<const float4 *>(wave_lds + r * PITCH + chunk * 16);
+            const float (&o)[4] = old[slab & 1][i];
+            const float w[4] = {o[0] + val.x, o[1] + val.y, o[2] + val.z, o[3] + val.w};
+            if constexpr (OUT_BF16) *reinterpret_cast<u32x2 *>(c_ptr(slab, i)) = u32x2{pack_bf16x2(w[0], w[1]), pack_bf16x2(w[2], w[3])};
+            else *reinterpret_cast<float4 *>(c_ptr(slab, i)) = float4{w[0], w[1], w[2], w[3]};
+        }
+    }
+}
+
 // launchers implemented in gemm_tiled.hip / gemm_pipe.hip / gemm_stream.hip (fa, fb: odl_fp8_format of A and B)
 void launch_gemm_tiled(int variant, int fa, int fb, const GemmArgs &g, hipStream_t stream);
 void launch_gemm_pipe(int fa, int fb, const GemmArgs &g, int num_cus, hipStream_t stream);
@@ -168,6 +254,6 @@ void launch_gemm_stream(int fa, int fb, const GemmArgs &g, int num_cus, hipStrea
 void attach_clock_probe(GemmArgs &g);
 // gemm_fp8.hip: out = (sum of the `splits` fp32 partial results in `workspace`, in split order) * (sa x sb) (+ bias), one rounding
 void launch_splitk_reduce(const float *workspace, int splits, int64_t M, int64_t N, const float *sa, int sa_vec, const float *sb, int sb_vec,
-                          const float *bias, void *c, int out_dtype, hipStream_t stream);
+                          const float *bias, void *c, int out_dtype, int accumulate, hipStream_t stream);
 
 }  // namespace odl

@@ -46,7 +46,8 @@ __global__ __launch_bounds__(64) void gemm_nt_generic_kernel(const GemmArgs g) {
 template <bool OUT_BF16>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restrict__ parts, int splits, int64_t M, int64_t N,
                                                             const float *__restrict__ sa, int sa_vec, const float *__restrict__ sb,
-                                                            int sb_vec, const float *__restrict__ bias, void *__restrict__ out) {
+                                                            int sb_vec, const float *__restrict__ bias, void *__restrict__ out,
+                                                            int accumulate) {
     const int64_t quads = M * N / 4, slice = M * N;
     for (int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; q < quads; q += (int64_t)gridDim.x * blockDim.x) {
         const int64_t e = q * 4, m = e / N, n = e % N;
@@ -64,9 +65,19 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restr
             for (int j = 0; j < 4; ++j) v[j] = v[j] + bias[n + j];
         }
         if constexpr (OUT_BF16) {
-            *reinterpret_cast<u32x2 *>(reinterpret_cast<uint16_t *>(out) + e) = u32x2{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+            u32x2 *dst = reinterpret_cast<u32x2 *>(reinterpret_cast<uint16_t *>(out) + e);
+            if (accumulate) {                          // out = out + product: the old value joins the fp32 sum, one rounding
+                const u32x2 old = *dst;
+                v[0] = v[0] + bf16_lo(old.x); v[1] = v[1] + bf16_hi(old.x); v[2] = v[2] + bf16_lo(old.y); v[3] = v[3] + bf16_hi(old.y);
+            }
+            *dst = u32x2{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
         } else {
-            *reinterpret_cast<float4 *>(reinterpret_cast<float *>(out) + e) = float4{v[0], v[1], v[2], v[3]};
+            float4 *dst = reinterpret_cast<float4 *>(reinterpret_cast<float *>(out) + e);
+            if (accumulate) {
+                const float4 old = *dst;
+                v[0] = v[0] + old.x; v[1] = v[1] + old.y; v[2] = v[2] + old.z; v[3] = v[3] + old.w;
+            }
+            *dst = float4{v[0], v[1], v[2], v[3]};
         }
     }
 }
@@ -145,16 +156,16 @@ extern "C" const char *odl_fp8_gemm_variant_name(int variant) {
 }
 
 void odl::launch_splitk_reduce(const float *workspace, int splits, int64_t M, int64_t N, const float *sa, int sa_vec, const float *sb,
-                               int sb_vec, const float *bias, void *c, int out_dtype, hipStream_t stream) {
+                               int sb_vec, const float *bias, void *c, int out_dtype, int accumulate, hipStream_t stream) {
     const int64_t quads = M * N / 4;
     int64_t blocks = (quads + 255) / 256;
     if (blocks > 4 * (int64_t)cu_count()) blocks = 4 * (int64_t)cu_count();
     if (out_dtype == ODL_BF16)
         hipLaunchKernelGGL((splitk_reduce_kernel<true>), dim3((unsigned)blocks), dim3(256), 0, stream, workspace, splits, M, N, sa, sa_vec, sb,
-                           sb_vec, bias, c);
+                           sb_vec, bias, c, accumulate);
     else
         hipLaunchKernelGGL((splitk_reduce_kernel<false>), dim3((unsigned)blocks), dim3(256), 0, stream, workspace, splits, M, N, sa, sa_vec, sb,
-                           sb_vec, bias, c);
+                           sb_vec, bias, c, accumulate);
 }
 
 void odl::attach_clock_probe(GemmArgs &g) {
@@ -181,7 +192,7 @@ extern "C" int odl_fp8_gemm_set_variant(int variant) {
 
 extern "C" int odl_fp8_gemm_nt(const uint8_t *a, const uint8_t *b, int64_t M, int64_t N, int64_t K, int fmt_a, int fmt_b,
                                const float *sa_inv, int64_t sa_n, const float *sb_inv, int64_t sb_n, const void *bias,
-                               int bias_dtype, void *c, int out_dtype, odl_stream_t stream_) {
+                               int bias_dtype, void *c, int out_dtype, int accumulate, odl_stream_t stream_) {
     hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
     if (!a || !b || !c || !sa_inv || !sb_inv) return set_error(ODL_ERR_ARG, "odl_fp8_gemm_nt: null pointer");
     if (M < 0 || N < 0 || K < 0) return set_error(ODL_ERR_ARG, "odl_fp8_gemm_nt: negative size");
@@ -203,7 +214,9 @@ extern "C" int odl_fp8_gemm_nt(const uint8_t *a, const uint8_t *b, int64_t M, in
     const bool tiled_ok = K >= 128 && K % 128 == 0 && (double)M * (double)K < 4294967296.0 && (double)N * (double)K < 4294967296.0;
     // the pipelined and the streaming kernel address rows with 32-bit byte offsets
     const bool lim32 = (double)(M + 256) * (double)K < 2147483648.0 && (double)(N + 256) * (double)K < 2147483648.0;
-    const bool stream_ok = tiled_ok && lim32 && M % 128 == 0 && N % 128 == 0 && K >= 512;
+    // C = C + product is an epilogue of the kernels whose tiles end in a separate output phase; the streaming kernel
+    // stores a tile under the next tile's MFMAs, where nothing can wait for the old values of C
+    const bool stream_ok = tiled_ok && lim32 && M % 128 == 0 && N % 128 == 0 && K >= 512 && !accumulate;
     int variant = t_forced_variant >= 0 ? t_forced_variant : (tiled_ok ? choose_variant(M, N, stream_ok) : 0);
     if (variant != 0 && !tiled_ok) variant = 0;
     // the pipelined kernel walks K in pairs of 128-byte steps
@@ -216,6 +229,7 @@ extern "C" int odl_fp8_gemm_nt(const uint8_t *a, const uint8_t *b, int64_t M, in
     g.sa_vec = sa_n == M && M != 1;
     g.sb_vec = sb_n == N && N != 1;
     g.out_dtype = out_dtype;
+    g.accumulate = accumulate != 0;
     const int bm = variant == 0 ? 32 : kVariants[variant].bm, bn = variant == 0 ? 32 : kVariants[variant].bn;
     const int64_t tm = (M + bm - 1) / bm, tn = (N + bn - 1) / bn;
     if (tm * tn > 0x7ffffff0LL) return set_error(ODL_ERR_SHAPE, "odl_fp8_gemm_nt: too many tiles");
@@ -307,7 +321,7 @@ extern "C" int odl_fp8_gemm_split_count(int64_t M, int64_t N, int64_t K, int k_s
 
 extern "C" int odl_fp8_gemm_splitk(const uint8_t *a, const uint8_t *b, int64_t M, int64_t N, int64_t K, int fmt_a, int fmt_b,
                                    int layout_a, int layout_b, const float *sa_inv, int64_t sa_n, const float *sb_inv,
-                                   int64_t sb_n, const float *bias, void *c, int out_dtype, int splits, void *workspace,
+                                   int64_t sb_n, const float *bias, void *c, int out_dtype, int accumulate, int splits, void *workspace,
                                    int64_t workspace_bytes, odl_stream_t stream_) {
     hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
     if (!a || !b || !c || !sa_inv || !sb_inv || !workspace) return set_error(ODL_ERR_ARG, "odl_fp8_gemm_splitk: null pointer");
@@ -330,8 +344,9 @@ extern "C" int odl_fp8_gemm_splitk(const uint8_t *a, const uint8_t *b, int64_t M
     const int64_t per = ((steps + splits - 1) / (splits > 0 ? splits : 1) + 1) & ~(int64_t)1;
     // what the kernel needs to be correct: every run at least four K steps (its load pipeline is two steps deep and runs
     // in pairs).  odl_fp8_gemm_split_count proposes only runs of eight steps and more, which is where a split pays.
-    if (splits < 2 || splits > 64 || per < 4 || steps - (splits - 1) * per < 4)
-        return set_error(ODL_ERR_ARG, "odl_fp8_gemm_splitk: %d splits of K=%lld leave a run shorter than 512", splits, (long long)K);
+    // one "run" is allowed with accumulate: the way to add a product with an operand stored K-slow into C
+    if (splits < (accumulate ? 1 : 2) || splits > 64 || per < 4 || steps - (splits - 1) * per < 4)
+        return set_error(ODL_ERR_ARG, "odl_fp8_gemm_splitk: %d splits of K=%lld leave a run shorter than 512 (or fewer than 2 splits without accumulate)", splits, (long long)K);
     if (workspace_bytes < (int64_t)splits * M * N * 4)
         return set_error(ODL_ERR_ARG, "odl_fp8_gemm_splitk: workspace of %lld bytes, %lld needed", (long long)workspace_bytes,
                          (long long)splits * M * N * 4);
@@ -347,6 +362,13 @@ extern "C" int odl_fp8_gemm_splitk(const uint8_t *a, const uint8_t *b, int64_t M
     attach_clock_probe(g);
     launch_gemm_stream(fmt_a, fmt_b, g, cu_count(), stream);
     const int sa_vec = sa_n == M && M != 1, sb_vec = sb_n == N && N != 1;
-    launch_splitk_reduce((const float *)workspace, splits, M, N, sa_inv, sa_vec, sb_inv, sb_vec, bias, c, out_dtype, stream);
+    if (splits == 1) {
+        // a single run is an ordinary launch: the kernel applies the tensor scales itself, the second kernel adds C
+        const float *one = unit_scale_for_current_device("odl_fp8_gemm_splitk");
+        if (!one) return ODL_ERR_LAUNCH;
+        launch_splitk_reduce((const float *)workspace, 1, M, N, one, 0, one, 0, bias, c, out_dtype, accumulate != 0, stream);
+        return check_launch("odl_fp8_gemm_splitk");
+    }
+    launch_splitk_reduce((const float *)workspace, splits, M, N, sa_inv, sa_vec, sb_inv, sb_vec, bias, c, out_dtype, accumulate != 0, stream);
     return check_launch("odl_fp8_gemm_splitk");
 }

@@ -60,7 +60,10 @@ static_assert(staged_epilogue_bytes<true, 2>() == EPI_BYTES && staged_epilogue_b
 
 typedef __attribute__((address_space(3))) void *lds_ptr_t;
 
-template <int FA, int FB>
+// ACC: the form for C = C + product (g.accumulate).  A kernel of its own, so that the registers its epilogue needs for
+// the old values of C do not weigh on the ordinary one; its direct-to-LDS loads carry the wait states that a scalar
+// register restored from a spill needs before a vector-memory instruction reads it (this form does spill scalars).
+template <int FA, int FB, bool ACC>
 __global__ __launch_bounds__(256) void gemm_nt_pipe_kernel(const GemmArgs g) {
     __shared__ __attribute__((aligned(1024))) uint8_t sA0[REGION];
     __shared__ __attribute__((aligned(1024))) uint8_t sB0[REGION];
@@ -107,6 +110,10 @@ __global__ __launch_bounds__(256) void gemm_nt_pipe_kernel(const GemmArgs g) {
     }
     // one 1 KB direct-to-LDS load: 64 lanes x 16 bytes land at lds_addr + lane * 16
     auto dma = [&](const v4i &rsrc, uint32_t lds_addr, int vo, int so) {
+        if constexpr (ACC)
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                         ::"s"(lds_addr), "v"(vo), "s"(rsrc), "s"(so));
+        else
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                      ::"s"(lds_addr), "v"(vo), "s"(rsrc), "s"(so));
     };
@@ -265,7 +272,10 @@ __global__ __launch_bounds__(256) void gemm_nt_pipe_kernel(const GemmArgs g) {
         if (interior && (g.N % 8) == 0) {
             uint8_t *wave_lds = sEpi + wave_e * EPI_BYTES;
             const int64_t mw = cm0 + (wave_e / 2) * WM, nw = cn0 + (wave_e % 2) * WN;
-            if (g.out_dtype == ODL_BF16) epilogue_staged<true, TM, TN, 2>(g, acc, wave_lds, mw, nw, lane_e);
+            if constexpr (ACC) {
+                if (g.out_dtype == ODL_BF16) epilogue_staged_accumulate<true, TM, TN, 1>(g, acc, wave_lds, mw, nw, lane_e);
+                else epilogue_staged_accumulate<false, TM, TN, 1>(g, acc, wave_lds, mw, nw, lane_e);
+            } else if (g.out_dtype == ODL_BF16) epilogue_staged<true, TM, TN, 2>(g, acc, wave_lds, mw, nw, lane_e);
             else epilogue_staged<false, TM, TN, 1>(g, acc, wave_lds, mw, nw, lane_e);
         } else {
 #define ODL_EPILOGUE(BF)                                                                                       \
@@ -282,7 +292,8 @@ __global__ __launch_bounds__(256) void gemm_nt_pipe_kernel(const GemmArgs g) {
 
 template <int FA, int FB>
 void launch_fmt(const GemmArgs &g, int blocks_per_xcd, hipStream_t stream) {
-    hipLaunchKernelGGL((gemm_nt_pipe_kernel<FA, FB>), dim3((unsigned)(8 * blocks_per_xcd)), dim3(256), 0, stream, g);
+    if (g.accumulate) hipLaunchKernelGGL((gemm_nt_pipe_kernel<FA, FB, true>), dim3((unsigned)(8 * blocks_per_xcd)), dim3(256), 0, stream, g);
+    else hipLaunchKernelGGL((gemm_nt_pipe_kernel<FA, FB, false>), dim3((unsigned)(8 * blocks_per_xcd)), dim3(256), 0, stream, g);
 }
 
 }  // namespace

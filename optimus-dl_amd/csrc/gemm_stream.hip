@@ -630,7 +630,7 @@ bool gemm_stream_accepts(const GemmArgs &g) {
     const double esz = (g.out_dtype == ODL_F32 || g.splits > 1) ? 4.0 : 2.0;
     const bool vectors = g.splits == 1 && (g.sa_vec || g.sb_vec || g.bias != nullptr);   // only with both operands stored [rows, K]
     if (g.mx_sa && (g.ta || g.tb || g.sa_vec || g.sb_vec || !g.mx_sb)) return false;
-    return (g.out_dtype == ODL_BF16 || g.out_dtype == ODL_F32) && !(vectors && (g.ta || g.tb)) &&
+    return !g.accumulate && (g.out_dtype == ODL_BF16 || g.out_dtype == ODL_F32) && !(vectors && (g.ta || g.tb)) &&
            g.M % (g.ta ? BM : WM) == 0 && g.N % (g.tb ? BN : WN) == 0 && g.K % 128 == 0 && g.K >= 512 && (double)g.N * esz * (BM + 8) < 2147483648.0;
 }
 

@@ -196,7 +196,10 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_nt_tiled_kernel(co
         __syncthreads();
         uint8_t *wave_lds = (wave * EPI_BYTES + EPI_BYTES <= STAGE) ? lds0 + wave * EPI_BYTES
                                                                     : lds1 + (wave - STAGE / EPI_BYTES) * EPI_BYTES;
-        if (g.out_dtype == ODL_BF16) epilogue_staged<true, TM, TN, TN>(g, acc, wave_lds, m0 + wm0, n0 + wn0, lane);
+        if (g.accumulate) {
+            if (g.out_dtype == ODL_BF16) epilogue_staged_accumulate<true, TM, TN, 1>(g, acc, wave_lds, m0 + wm0, n0 + wn0, lane);
+            else epilogue_staged_accumulate<false, TM, TN, 1>(g, acc, wave_lds, m0 + wm0, n0 + wn0, lane);
+        } else if (g.out_dtype == ODL_BF16) epilogue_staged<true, TM, TN, TN>(g, acc, wave_lds, m0 + wm0, n0 + wn0, lane);
         else epilogue_staged<false, TM, TN, TN>(g, acc, wave_lds, m0 + wm0, n0 + wn0, lane);
     } else {
 #define ODL_EPILOGUE(BF)                                                                                       \

@@ -730,7 +730,10 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void mx_gemm_tiled_kernel(co
         __syncthreads();
         uint8_t *wave_lds = (wave * EPI_BYTES + EPI_BYTES <= STAGE) ? lds0 + wave * EPI_BYTES
                                                                     : lds1 + (wave - STAGE / EPI_BYTES) * EPI_BYTES;
-        if (g.out_dtype == ODL_BF16) epilogue_staged<true, TM, TN, TN>(g, acc, wave_lds, m0 + wm0, n0 + wn0, lane);
+        if (g.accumulate) {
+            if (g.out_dtype == ODL_BF16) epilogue_staged_accumulate<true, TM, TN, 1>(g, acc, wave_lds, m0 + wm0, n0 + wn0, lane);
+            else epilogue_staged_accumulate<false, TM, TN, 1>(g, acc, wave_lds, m0 + wm0, n0 + wn0, lane);
+        } else if (g.out_dtype == ODL_BF16) epilogue_staged<true, TM, TN, TN>(g, acc, wave_lds, m0 + wm0, n0 + wn0, lane);
         else epilogue_staged<false, TM, TN, TN>(g, acc, wave_lds, m0 + wm0, n0 + wn0, lane);
     } else {
 #define ODL_EPILOGUE(BF)                                                                                       \
@@ -895,7 +898,7 @@ extern "C" int odl_fp8_mx_cast(const void *x, int src_dtype, int64_t rows, int64
 }
 
 extern "C" int odl_fp8_mx_gemm_nt(const uint8_t *a, const uint8_t *sa, const uint8_t *b, const uint8_t *sb, int scales_layout, int64_t M,
-                                  int64_t N, int64_t K, int fmt_a, int fmt_b, const float *bias, void *c, int out_dtype, odl_stream_t stream_) {
+                                  int64_t N, int64_t K, int fmt_a, int fmt_b, const float *bias, void *c, int out_dtype, int accumulate, odl_stream_t stream_) {
     hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
     if (M < 0 || N < 0 || K < 0) return set_error(ODL_ERR_ARG, "odl_fp8_mx_gemm_nt: negative shape");
     if ((fmt_a != ODL_FP8_E4M3 && fmt_a != ODL_FP8_E5M2) || (fmt_b != ODL_FP8_E4M3 && fmt_b != ODL_FP8_E5M2))
@@ -916,6 +919,7 @@ extern "C" int odl_fp8_mx_gemm_nt(const uint8_t *a, const uint8_t *sa, const uin
     GemmArgs g{};
     g.a = a; g.b = b; g.c = c; g.sa = one; g.sb = one; g.bias = bias;
     g.M = M; g.N = N; g.K = K; g.sa_vec = 0; g.sb_vec = 0; g.out_dtype = out_dtype;
+    g.accumulate = accumulate != 0;
     // the tiled and the streaming kernel address rows with 32-bit offsets and read whole scale dwords (4 blocks = one
     // 128-byte K step); the streaming kernel wants the scales K-step-major and the shapes of gemm_stream_accepts, and
     // pays only when more than half the compute units get one of its 256 x 256 tiles (at exactly half, outputs of
@@ -925,7 +929,7 @@ extern "C" int odl_fp8_mx_gemm_nt(const uint8_t *a, const uint8_t *sa, const uin
     GemmArgs probe = g;
     probe.mx_sa = sa; probe.mx_sb = sb;
     const int cus = device_cu_count();
-    const bool stream_ok = ks && tiled && ((M + 255) / 256) * ((N + 255) / 256) * 2 > cus && gemm_stream_accepts(probe);
+    const bool stream_ok = !accumulate && ks && tiled && ((M + 255) / 256) * ((N + 255) / 256) * 2 > cus && gemm_stream_accepts(probe);
     const int kernel = stream_ok ? 2 : (tiled ? 1 : 0);
 #define ODL_MXG(FA_, FB_) launch_mx_gemm<FA_, FB_>(g, sa, sb, kernel, ks, cus, stream)
     if (fmt_a == ODL_FP8_E4M3 && fmt_b == ODL_FP8_E4M3) ODL_MXG(ODL_FP8_E4M3, ODL_FP8_E4M3);
@@ -967,7 +971,7 @@ extern "C" int odl_fp8_block_cast(const void *x, int src_dtype, int64_t rows, in
 // weight gradients of small layers), as odl_fp8_gemm_splitk does for per-tensor scales: every run leaves an fp32 partial
 // result in the caller's workspace, a second kernel adds them in run order, adds the bias and rounds once.
 extern "C" int odl_fp8_mx_gemm_splitk(const uint8_t *a, const uint8_t *sa, const uint8_t *b, const uint8_t *sb, int64_t M, int64_t N, int64_t K,
-                                      int fmt_a, int fmt_b, const float *bias, void *c, int out_dtype, int splits, void *workspace,
+                                      int fmt_a, int fmt_b, const float *bias, void *c, int out_dtype, int accumulate, int splits, void *workspace,
                                       int64_t workspace_bytes, odl_stream_t stream_) {
     hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
     if (!a || !sa || !b || !sb || !c || !workspace) return set_error(ODL_ERR_ARG, "odl_fp8_mx_gemm_splitk: null pointer");
@@ -1000,6 +1004,6 @@ extern "C" int odl_fp8_mx_gemm_splitk(const uint8_t *a, const uint8_t *sa, const
     if (!gemm_stream_accepts(g)) return set_error(ODL_ERR_SHAPE, "odl_fp8_mx_gemm_splitk: shape not taken by the streaming kernel");
     attach_clock_probe(g);
     launch_gemm_stream(fmt_a, fmt_b, g, device_cu_count(), stream);
-    launch_splitk_reduce((const float *)workspace, splits, M, N, one, 0, one, 0, bias, c, out_dtype, stream);
+    launch_splitk_reduce((const float *)workspace, splits, M, N, one, 0, one, 0, bias, c, out_dtype, accumulate != 0, stream);
     return check_launch("odl_fp8_mx_gemm_splitk");
 }

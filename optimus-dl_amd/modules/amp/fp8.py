@@ -206,6 +206,15 @@ class FP8Recipe:
         # partial maxima handed over by the kernel that produced a tensor (SwiGLU, RMSNorm), so that
         # the Linear that quantises this very tensor skips its amax pass; a handful of entries
         self.producer_parts: list[tuple[tuple, torch.Tensor, torch.Tensor]] = []
+        # Linears fed by one tensor (q/k/v, gate/up) run as one autograd node whose data gradients are summed by the
+        # GEMMs' accumulate flag (modules/fp8_linear.py: linear_group, SiblingGroup); False: every Linear on its own
+        self.fuse_dgrad_sum = True
+        self._sibling_groups: "weakref.WeakSet" = weakref.WeakSet()
+        # Gradient accumulation over microbatches (the reference's acc_steps > 1): with this set, a weight gradient is
+        # added straight into an existing ``weight.grad`` by the GEMM and autograd is handed None for it, instead
+        # of a separate ``grad += dw`` pass per weight and microbatch.  Off by default: tensor hooks on the weight's
+        # gradient (DDP / FSDP reducers) do not see a gradient that never passes through autograd.
+        self.fuse_wgrad_accumulation = False
         # Fp8ParamSets attached under this recipe (delayed scaling: they re-record their weights' maxima at each refresh)
         self._param_sets: "weakref.WeakSet" = weakref.WeakSet()
         _info_once(
@@ -372,6 +381,9 @@ class FP8Recipe:
             if self._depth == 0:
                 self.shared_input = None
                 self.producer_parts.clear()
+                for grp in list(self._sibling_groups):      # outputs made for siblings that were never asked for
+                    grp.clear()
+                self._sibling_groups.clear()
                 self.update_scales("fwd")
                 # gradients recorded by a backward that ran outside any backward()
                 # context are folded in here, one step late but never lost
@@ -390,6 +402,9 @@ class FP8Recipe:
             if self._depth == 0:
                 self.shared_input = None          # a forward recomputed by activation checkpointing may have left one
                 self.producer_parts.clear()
+                for grp in list(self._sibling_groups):
+                    grp.clear()
+                self._sibling_groups.clear()
                 self.update_scales("bwd")
 
     def prepare_for_backward(self, *args: Any, **kwargs: Any) -> tuple[Any, ...]:

@@ -312,15 +312,30 @@ class _Fp8LinearFn(torch.autograd.Function):
                     gq, gq_t, sg_inv, _ = _quantise_dynamic(dy2d, pol.fmt_bwd, pol.margin, g_t_needed, g_rm_needed,
                                                             parts=parts)
             if ctx.need_dgrad:
-                dx = native.gemm_nt(gq, saved["wq_t"], pol.fmt_bwd, pol.fmt_fwd, sg_inv, saved["sw_inv_t"],
-                                    out_dtype=ctx.x_dtype)
+                # a member of a group of Linears fed by one tensor adds its share into the group's gradient
+                # (the GEMM's accumulate flag) instead of leaving the sum to a separate pass
+                dx_into = getattr(ctx, "dx_into", None)
+                if dx_into is not None:
+                    dx = native.gemm_nt(gq, saved["wq_t"], pol.fmt_bwd, pol.fmt_fwd, sg_inv, saved["sw_inv_t"],
+                                        out=dx_into, accumulate=True)
+                else:
+                    dx = native.gemm_nt(gq, saved["wq_t"], pol.fmt_bwd, pol.fmt_fwd, sg_inv, saved["sw_inv_t"],
+                                        out_dtype=ctx.x_dtype)
             if fp8_wgrad:
+                # gradient accumulation over microbatches: with recipe.fuse_wgrad_accumulation the product is added
+                # straight into the existing .grad (and autograd is handed nothing to add)
+                grad_buf = module.weight.grad if recipe.fuse_wgrad_accumulation else None
+                into = grad_buf is not None and grad_buf.dtype == ctx.w_dtype and grad_buf.is_contiguous() and grad_buf.is_cuda \
+                    and tuple(grad_buf.shape) == (module.out_features, module.in_features)
                 if ctx.wgrad_direct:        # dW = dY^T . X with dY [tokens, N] as stored, X^T from the forward
                     dw = native.gemm_layouts(gq, saved["xq_t"], pol.fmt_bwd, pol.fmt_fwd, native.K_SLOW, native.K_FAST,
-                                             sg_inv, saved["sx_inv_t"], out_dtype=ctx.w_dtype)
+                                             sg_inv, saved["sx_inv_t"], out=grad_buf if into else None,
+                                             out_dtype=ctx.w_dtype, accumulate=into)
                 else:
                     dw = native.gemm_nt(gq_t, saved["xq_t"], pol.fmt_bwd, pol.fmt_fwd, sg_inv, saved["sx_inv_t"],
-                                        out_dtype=ctx.w_dtype)
+                                        out=grad_buf if into else None, out_dtype=ctx.w_dtype, accumulate=into)
+                if into:
+                    dw = None
         if ctx.need_wgrad and not recipe.wgrad:
             dw = (dy2d.t().to(saved["x_hp"].dtype) @ saved["x_hp"]).to(ctx.w_dtype)
         if ctx.has_bias and db is None:
@@ -332,8 +347,138 @@ class _Fp8LinearFn(torch.autograd.Function):
         return dx, dw, db, None, None, None
 
 
+class _MemberCtx:
+    """What ``_Fp8LinearFn.forward`` / ``backward`` expect of an autograd context, for one member of a group: the tensors
+    it saves are collected by the group's own context (so they still go through autograd's saved-tensor machinery)."""
+
+    def __init__(self, needs_input_grad: tuple):
+        self.needs_input_grad = needs_input_grad
+        self.saved_tensors: tuple = ()
+
+    def save_for_backward(self, *tensors: torch.Tensor) -> None:
+        self.saved_tensors = tensors
+
+
+class _Fp8LinearGroupFn(torch.autograd.Function):
+    """Several FP8 Linears applied to ONE input (q/k/v of an attention block, gate/up of a gated MLP) as one autograd
+    node: forward = the members' forwards (they share the quantised input anyway), backward = the members' backwards
+    with the data gradients summed by the GEMMs themselves: the first member writes dx, every further one adds its
+    product into it (``accumulate``), where separate nodes leave two extra passes over dx per block to autograd."""
+
+    @staticmethod
+    def forward(ctx, x2d: torch.Tensor, recipe: FP8Recipe, out_dtype: torch.dtype, modules: tuple, *params: torch.Tensor | None):
+        ctx.set_materialize_grads(False)         # an output that did not reach the loss arrives as None, not as zeros
+        subs, outs, saved, spans = [], [], [], []
+        for i, mod in enumerate(modules):
+            weight, bias = params[2 * i], params[2 * i + 1]
+            sub = _MemberCtx((ctx.needs_input_grad[0], ctx.needs_input_grad[4 + 2 * i], ctx.needs_input_grad[5 + 2 * i],
+                              False, False, False))
+            outs.append(_Fp8LinearFn.forward(sub, x2d, weight, bias, mod, recipe, out_dtype))
+            spans.append((len(saved), len(sub.saved_tensors)))
+            saved.extend(sub.saved_tensors)
+            sub.saved_tensors = ()
+            subs.append(sub)
+        ctx.save_for_backward(*saved)
+        ctx.subs, ctx.spans = subs, spans
+        return tuple(outs)
+
+    @staticmethod
+    def backward(ctx, *dys: torch.Tensor | None):
+        tensors = ctx.saved_tensors
+        dx = None
+        grads: list = []
+        for sub, (first, count), dy in zip(ctx.subs, ctx.spans, dys):
+            if dy is None:                       # this member's output did not reach the loss
+                grads += [None, None]
+                continue
+            sub.saved_tensors = tensors[first:first + count]
+            sub.dx_into = dx if (dx is not None and sub.need_dgrad) else None
+            dxi, dw, db, _, _, _ = _Fp8LinearFn.backward(sub, dy)
+            sub.saved_tensors = ()
+            if dxi is not None and dx is None:
+                dx = dxi
+            grads += [dw, db]
+        return (dx, None, None, None, *grads)
+
+
+@torch.compiler.disable
+def linear_group(x: torch.Tensor, modules: "tuple[FP8Linear, ...]") -> tuple[torch.Tensor, ...] | None:
+    """``tuple(m(x) for m in modules)`` as one autograd node (see ``_Fp8LinearGroupFn``), or None where the members
+    cannot run that way (no recipe, a recipe other than tensorwise / delayed, shapes the FP8 path refuses): the caller
+    then applies the modules one by one."""
+    recipe = _state.active_recipe()
+    if recipe is None or recipe.recipe.kind not in ("tensorwise", "delayed") or not recipe.fuse_dgrad_sum:
+        return None
+    if not all(m._fp8_eligible(x) for m in modules):
+        return None
+    compute_dtype = torch.get_autocast_dtype("cuda") if torch.is_autocast_enabled("cuda") else x.dtype
+    if compute_dtype not in (torch.bfloat16, torch.float32):
+        compute_dtype = torch.bfloat16
+    k = modules[0].in_features
+    x2d = x.reshape(-1, k)
+    if x2d.dtype != compute_dtype or not x2d.is_contiguous():
+        x2d = _converted_input(recipe, x2d, compute_dtype)
+    params: list = []
+    for m in modules:
+        m.fp8_calls += 1
+        m._note_grad_mode()
+        params += [m.weight, m.bias]
+    outs = _Fp8LinearGroupFn.apply(x2d, recipe, compute_dtype, tuple(modules), *params)
+    return tuple(y.reshape(*x.shape[:-1], m.out_features) for y, m in zip(outs, modules))
+
+
+class SiblingGroup:
+    """Linears of one parent module that are fed the same tensor in its forward (``wq``, ``wk``, ``wv`` of the
+    reference's attention block, attention.py:317-319; ``w1``, ``w2`` of its gated MLP, mlp.py:76-78).  The parent's
+    forward is not touched: the member that is called first computes the outputs of ALL members through
+    ``linear_group`` and keeps the others' until they are asked for with the very same tensor (same address, version,
+    shape and strides).  A member called with another tensor simply runs on its own; after that has happened the group stands
+    down for good (its members are evidently not fed one tensor: cross-attention, say), so that nothing is computed
+    for nothing twice."""
+
+    def __init__(self, modules: "list[FP8Linear]"):
+        self.modules = tuple(modules)
+        self.pending: dict = {}
+        self.key = None
+        self.x = None
+        self.misses = 0
+        self.groups_run = 0              # forwards that ran as one node for all members (for tests / logging)
+        for m in self.modules:
+            m._siblings = self
+
+    def clear(self) -> None:
+        self.pending, self.key, self.x = {}, None, None
+
+    @torch.compiler.disable          # like FP8Linear._forward_fp8: runs as written, between the compiled parts of a model
+    def forward(self, member: "FP8Linear", x: torch.Tensor) -> torch.Tensor:
+        # the same values at the same address: the same tensor object, or another handle on it (a graph compiler hands
+        # the pieces of a model it runs separately fresh handles on the same storage)
+        key = (x.data_ptr(), _state.tensor_version(x), tuple(x.shape), tuple(x.stride()), x.dtype, x.requires_grad)
+        if self.key == key and id(member) in self.pending:
+            out = self.pending.pop(id(member))
+            if not self.pending:
+                self.clear()
+            return out
+        if self.pending:                 # outputs made for siblings that were then fed something else
+            self.misses += 1
+            self.clear()
+        if self.misses or not torch.is_grad_enabled() or not x.requires_grad:
+            return member._forward_fp8(x)
+        outs = linear_group(x, self.modules)
+        if outs is None:
+            return member._forward_fp8(x)
+        recipe = _state.active_recipe()
+        recipe._sibling_groups.add(self)
+        self.groups_run += 1
+        self.key, self.x = key, x        # the entry keeps x alive: its address cannot be handed to another tensor meanwhile
+        self.pending = {id(m): y for m, y in zip(self.modules, outs) if m is not member}
+        return outs[self.modules.index(member)]
+
+
 class FP8Linear(nn.Linear):
     """Drop-in ``nn.Linear`` with an FP8 fast path (see the module docstring)."""
+
+    _siblings: "SiblingGroup | None" = None      # set on the instance by a SiblingGroup that this Linear is a member of
 
     def __init__(self, in_features: int, out_features: int, bias: bool = True, device=None, dtype=None, **kwargs: Any):
         super().__init__(in_features, out_features, bias=bias, device=device, dtype=dtype)
@@ -350,7 +495,7 @@ class FP8Linear(nn.Linear):
 
     # Quantised weights and scaling-state views are per-process run-time state: a copy or a pickle of the module
     # starts without them (they are rebuilt on first use) instead of dragging device buffers and arenas along.
-    _RUNTIME_STATE = ("_wcache", "_wcache_rowwise", "_metas", "fp8_meta", "fp8_calls")
+    _RUNTIME_STATE = ("_wcache", "_wcache_rowwise", "_metas", "fp8_meta", "fp8_calls", "_siblings", "_grad_mode")
 
     def __getstate__(self) -> dict:
         state = self.__dict__.copy()
@@ -404,8 +549,12 @@ class FP8Linear(nn.Linear):
         return meta
 
     def _records(self) -> bool:
-        """Whether a forward of this module feeds the delayed-scaling histories: training mode and grad mode."""
-        return self.training and torch.is_grad_enabled()
+        """Whether the forward in progress feeds the delayed-scaling histories: training mode and grad mode, as noted
+        by ``_note_grad_mode`` before the autograd function was entered (inside it grad mode is always off)."""
+        return self.training and self.__dict__.get("_grad_mode", True)
+
+    def _note_grad_mode(self) -> None:
+        self.__dict__["_grad_mode"] = torch.is_grad_enabled()
 
     def _tensor_weight(self, weight: torch.Tensor, recipe: FP8Recipe, need_t: bool):
         """Per-tensor quantised weight (and transpose), cached on the parameter version."""
@@ -498,6 +647,9 @@ class FP8Linear(nn.Linear):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         if _state.active_recipe() is None:
             return F.linear(x, self.weight, self.bias)
+        siblings = self._siblings
+        if siblings is not None:
+            return siblings.forward(self, x)
         return self._forward_fp8(x)
 
     # The FP8 path calls the native library through ctypes and keeps per-step state on the recipe: a graph
@@ -518,6 +670,7 @@ class FP8Linear(nn.Linear):
         if x2d.dtype != compute_dtype or not x2d.is_contiguous():
             x2d = _converted_input(recipe, x2d, compute_dtype)
         self.fp8_calls += 1
+        self._note_grad_mode()
         y = _Fp8LinearFn.apply(x2d, self.weight, self.bias, self, recipe, compute_dtype)
         return y.reshape(*x.shape[:-1], self.out_features)
 

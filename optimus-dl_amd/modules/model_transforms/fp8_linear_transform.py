@@ -34,7 +34,7 @@ from typing import Any, Callable
 import torch.nn as nn
 
 from ... import native
-from ..fp8_linear import FP8Linear
+from ..fp8_linear import FP8Linear, SiblingGroup
 from ..fused import fuse_gelu, fuse_layernorm, fuse_rmsnorm, fuse_swiglu_mlp
 from . import register_model_transform
 from .base import BaseModelTransform
@@ -105,6 +105,9 @@ class TransformerEngineTransformConfig(ModelTransformConfig):
     fuse_swiglu: bool = True           # not in the reference: SwiGLU MLPs get the fused activation
     swiglu_classes: tuple = ("SwiGLUMLP",)
     fuse_gelu: bool = True             # not in the reference: exact nn.GELU modules get the fused activation
+    # not in the reference: Linears of one parent that its forward feeds the same tensor (attention.py:317-319,
+    # mlp.py:76-78) run as one autograd node whose data gradients the GEMMs sum themselves
+    group_siblings: tuple = (("wq", "wk", "wv"), ("w1", "w2"))
 
     def __post_init__(self):
         self.linear_kwargs = dict(self.linear_kwargs or {})
@@ -134,6 +137,7 @@ class TransformerEngineTransform(BaseModelTransform):
             return model
         logger.info("Applying FP8 module replacements")
         replacements = {"Linear": 0, "RMSNorm": 0, "LayerNorm": 0, "Attention": 0}
+        self.sibling_groups = 0            # groups of Linears fed by one tensor (not module replacements: counted apart)
         self._replace_modules_recursive(model, replacements, replace_linear=self.cfg.replace_linear,
                                         replace_norm=self.cfg.replace_norm, replace_attention=self.cfg.replace_attention)
         total = sum(replacements.values())
@@ -180,6 +184,13 @@ class TransformerEngineTransform(BaseModelTransform):
         if self.cfg.fuse_gelu and self.cfg.replace_inplace and _get_module_class_name(module) == "torch.nn.modules.activation.GELU" \
                 and fuse_gelu(module):
             replacements["GELU"] = replacements.get("GELU", 0) + 1
+        if self.cfg.replace_inplace:
+            for names in tuple(self.cfg.group_siblings or ()):
+                members = [getattr(module, n, None) for n in names]
+                if all(isinstance(m, FP8Linear) for m in members) and len({id(m) for m in members}) == len(members) \
+                        and len({m.in_features for m in members}) == 1 and not any(m._siblings is not None for m in members):
+                    SiblingGroup(members)
+                    self.sibling_groups += 1
         # after the children: the three projections of an MLP are FP8 Linears by now
         if (self.cfg.fuse_swiglu and self.cfg.replace_inplace and module.__class__.__name__ in tuple(self.cfg.swiglu_classes)
                 and fuse_swiglu_mlp(module)):

@@ -131,11 +131,11 @@ def load() -> ctypes.CDLL:
         L.odl_fp8_cast.argtypes = [vp, i32, i64, i64, vp, i32, i32, vp, vp, vp]
         L.odl_fp8_cast_transpose.argtypes = [vp, i32, i64, i64, vp, i32, i32, vp, vp, vp, vp]
         L.odl_fp8_cast_delayed.argtypes = [vp, i32, i64, i64, vp, i32, vp, vp, vp, vp, vp]
-        L.odl_fp8_gemm_nt.argtypes = [vp, vp, i64, i64, i64, i32, i32, vp, i64, vp, i64, vp, i32, vp, i32, vp]
+        L.odl_fp8_gemm_nt.argtypes = [vp, vp, i64, i64, i64, i32, i32, vp, i64, vp, i64, vp, i32, vp, i32, i32, vp]
         L.odl_fp8_gemm_layouts.argtypes = [vp, vp, i64, i64, i64, i32, i32, i32, i32, vp, vp, vp, i32, vp]
         L.odl_fp8_gemm_split_count.argtypes = [i64, i64, i64, i32]
         L.odl_fp8_gemm_split_count.restype = i32
-        L.odl_fp8_gemm_splitk.argtypes = [vp, vp, i64, i64, i64, i32, i32, i32, i32, vp, i64, vp, i64, vp, vp, i32, i32, vp, i64, vp]
+        L.odl_fp8_gemm_splitk.argtypes = [vp, vp, i64, i64, i64, i32, i32, i32, i32, vp, i64, vp, i64, vp, vp, i32, i32, i32, vp, i64, vp]
         L.odl_fp8_delayed_update.argtypes = [vp, i64, i64, i64, vp, vp, vp, i32, i32, vp, vp]
         L.odl_fp8_gemm_num_variants.restype = i32
         L.odl_fp8_gemm_variant_name.argtypes = [i32]
@@ -143,9 +143,9 @@ def load() -> ctypes.CDLL:
         L.odl_fp8_gemm_set_variant.argtypes = [i32]
         L.odl_fp8_gemm_set_clock_probe.argtypes = [vp, i32]
         L.odl_fp8_mx_cast.argtypes = [vp, i32, i64, i64, i32, vp, vp, i32, vp, vp, i32, vp]
-        L.odl_fp8_mx_gemm_nt.argtypes = [vp, vp, vp, vp, i32, i64, i64, i64, i32, i32, vp, vp, i32, vp]
+        L.odl_fp8_mx_gemm_nt.argtypes = [vp, vp, vp, vp, i32, i64, i64, i64, i32, i32, vp, vp, i32, i32, vp]
         L.odl_fp8_block_cast.argtypes = [vp, i32, i64, i64, i32, i32, i32, vp, vp, vp, vp, vp]
-        L.odl_fp8_mx_gemm_splitk.argtypes = [vp, vp, vp, vp, i64, i64, i64, i32, i32, vp, vp, i32, i32, vp, i64, vp]
+        L.odl_fp8_mx_gemm_splitk.argtypes = [vp, vp, vp, vp, i64, i64, i64, i32, i32, vp, vp, i32, i32, i32, vp, i64, vp]
         for name in EXPORTS:
             getattr(L, name)  # AttributeError here = the library does not match the header
         if L.odl_fp8_abi_version() != ABI_VERSION:
@@ -721,8 +721,13 @@ def cast_delayed(x: torch.Tensor, scale: torch.Tensor, fmt: int, amax_parts: tor
 
 def gemm_nt(a: torch.Tensor, b: torch.Tensor, fmt_a: int, fmt_b: int, sa_inv: torch.Tensor, sb_inv: torch.Tensor,
             bias: torch.Tensor | None = None, out_dtype: torch.dtype = torch.bfloat16,
-            out: torch.Tensor | None = None) -> torch.Tensor:
-    """out[M,N] = (a[M,K] . b[N,K]^T) * (sa_inv x sb_inv) (+ bias); a, b uint8 FP8 codes."""
+            out: torch.Tensor | None = None, accumulate: bool = False) -> torch.Tensor:
+    """out[M,N] = (a[M,K] . b[N,K]^T) * (sa_inv x sb_inv) (+ bias); a, b uint8 FP8 codes.  A given ``out`` decides the
+    output type.  accumulate: out = out + product (needs ``out``; the old value joins the fp32 sum, one rounding)."""
+    if accumulate and out is None:
+        raise NativeError("gemm_nt(accumulate=True) needs the `out` tensor to add into")
+    if out is not None:
+        out_dtype = out.dtype
     if a.dtype != torch.uint8 or b.dtype != torch.uint8:
         raise NativeError("gemm_nt operands must be uint8 FP8 codes")
     a, b = _as_2d(a), _as_2d(b)
@@ -745,10 +750,10 @@ def gemm_nt(a: torch.Tensor, b: torch.Tensor, fmt_a: int, fmt_b: int, sa_inv: to
         raise NativeError("gemm_nt: `out` has the wrong shape / dtype / layout")
     splits = gemm_split_count(M, N, K)
     if splits > 1:
-        return _gemm_splitk(a, b, M, N, K, fmt_a, fmt_b, K_FAST, K_FAST, sa_inv, sb_inv, bias, out, splits)
+        return _gemm_splitk(a, b, M, N, K, fmt_a, fmt_b, K_FAST, K_FAST, sa_inv, sb_inv, bias, out, splits, accumulate)
     _check(load().odl_fp8_gemm_nt(a.data_ptr(), b.data_ptr(), M, N, K, fmt_a, fmt_b, sa_inv.data_ptr(), sa_inv.numel(),
                                   sb_inv.data_ptr(), sb_inv.numel(), bias.data_ptr() if bias is not None else None,
-                                  DT_F32, out.data_ptr(), odt, _stream()), "odl_fp8_gemm_nt")
+                                  DT_F32, out.data_ptr(), odt, int(accumulate), _stream()), "odl_fp8_gemm_nt")
     return out
 
 
@@ -831,7 +836,8 @@ def block_cast(x: torch.Tensor, fmt: int, margin: int = 0, two_d: bool = False, 
 
 
 def mx_gemm_nt(a: torch.Tensor, sa: torch.Tensor, b: torch.Tensor, sb: torch.Tensor, fmt_a: int, fmt_b: int,
-               bias: torch.Tensor | None = None, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+               bias: torch.Tensor | None = None, out_dtype: torch.dtype = torch.bfloat16, out: torch.Tensor | None = None,
+               accumulate: bool = False) -> torch.Tensor:
     """out[M,N] = sum over 32-blocks of 2^(sa-127) 2^(sb-127) (a_block . b_block) (+ bias); a [M,K], b [N,K] codes,
     sa, sb their E8M0 scale bytes as ``mx_cast`` returns them (both row-major [rows, K/32] or both K-step-major
     [K/128, rows, 4])."""
@@ -852,22 +858,29 @@ def mx_gemm_nt(a: torch.Tensor, sa: torch.Tensor, b: torch.Tensor, sb: torch.Ten
         raise NativeError(f"mx_gemm_nt: scale shapes {tuple(sa.shape)}, {tuple(sb.shape)} do not fit M, N, K = {M}, {N}, {K}")
     if bias is not None:
         _f32_dev(bias, N, "mx_gemm_nt bias")
+    if accumulate and out is None:
+        raise NativeError("mx_gemm_nt(accumulate=True) needs the `out` tensor to add into")
+    if out is not None:
+        out_dtype = out.dtype
+        if out.shape != (M, N) or not out.is_contiguous() or not out.is_cuda:
+            raise NativeError("mx_gemm_nt: `out` has the wrong shape / layout")
     odt = DT_BF16 if out_dtype == torch.bfloat16 else (DT_F32 if out_dtype == torch.float32 else None)
     if odt is None:
         raise NativeError(f"mx_gemm_nt: output dtype {out_dtype} is not supported (bf16 or fp32)")
-    out = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    if out is None:
+        out = torch.empty((M, N), dtype=out_dtype, device=a.device)
     # outputs of few tiles with a long contraction: K in runs side by side, like gemm_nt
     splits = gemm_split_count(M, N, K) if layout == MX_KSTEP else 1
     if splits > 1:
         workspace = torch.empty((splits, M, N), dtype=torch.float32, device=a.device)
         init_device(a.device)
         _check(load().odl_fp8_mx_gemm_splitk(a.data_ptr(), sa.data_ptr(), b.data_ptr(), sb.data_ptr(), M, N, K, fmt_a, fmt_b,
-                                             bias.data_ptr() if bias is not None else None, out.data_ptr(), odt, splits,
-                                             workspace.data_ptr(), workspace.numel() * 4, _stream()), "odl_fp8_mx_gemm_splitk")
+                                             bias.data_ptr() if bias is not None else None, out.data_ptr(), odt, int(accumulate),
+                                             splits, workspace.data_ptr(), workspace.numel() * 4, _stream()), "odl_fp8_mx_gemm_splitk")
         return out
     init_device(a.device)
     _check(load().odl_fp8_mx_gemm_nt(a.data_ptr(), sa.data_ptr(), b.data_ptr(), sb.data_ptr(), layout, M, N, K, fmt_a, fmt_b,
-                                     bias.data_ptr() if bias is not None else None, out.data_ptr(), odt, _stream()),
+                                     bias.data_ptr() if bias is not None else None, out.data_ptr(), odt, int(accumulate), _stream()),
            "odl_fp8_mx_gemm_nt")
     return out
 
@@ -886,18 +899,19 @@ def gemm_split_count(M: int, N: int, K: int, k_slow: bool = False) -> int:
     return int(load().odl_fp8_gemm_split_count(M, N, K, 1 if k_slow else 0))
 
 
-def _gemm_splitk(a, b, M, N, K, fmt_a, fmt_b, layout_a, layout_b, sa_inv, sb_inv, bias, out, splits):
+def _gemm_splitk(a, b, M, N, K, fmt_a, fmt_b, layout_a, layout_b, sa_inv, sb_inv, bias, out, splits, accumulate=False):
     workspace = torch.empty((splits, M, N), dtype=torch.float32, device=a.device)
     _check(load().odl_fp8_gemm_splitk(a.data_ptr(), b.data_ptr(), M, N, K, fmt_a, fmt_b, layout_a, layout_b, sa_inv.data_ptr(),
                                       sa_inv.numel(), sb_inv.data_ptr(), sb_inv.numel(),
-                                      bias.data_ptr() if bias is not None else None, out.data_ptr(), _src_dtype(out), splits,
-                                      workspace.data_ptr(), workspace.numel() * 4, _stream()), "odl_fp8_gemm_splitk")
+                                      bias.data_ptr() if bias is not None else None, out.data_ptr(), _src_dtype(out), int(accumulate),
+                                      splits, workspace.data_ptr(), workspace.numel() * 4, _stream()), "odl_fp8_gemm_splitk")
     return out
 
 
 def gemm_splitk(a: torch.Tensor, b: torch.Tensor, fmt_a: int, fmt_b: int, sa_inv: torch.Tensor, sb_inv: torch.Tensor,
                 splits: int, bias: torch.Tensor | None = None, out_dtype: torch.dtype = torch.bfloat16,
-                layout_a: int = K_FAST, layout_b: int = K_FAST) -> torch.Tensor:
+                layout_a: int = K_FAST, layout_b: int = K_FAST, out: torch.Tensor | None = None,
+                accumulate: bool = False) -> torch.Tensor:
     """The product of :func:`gemm_nt` / :func:`gemm_layouts` with K cut into ``splits`` runs that are computed
     side by side and added in run order (fp32).  :func:`gemm_nt` and :func:`gemm_layouts` take this route by
     themselves where :func:`gemm_split_count` says so; this entry is for choosing ``splits`` by hand."""
@@ -914,10 +928,17 @@ def gemm_splitk(a: torch.Tensor, b: torch.Tensor, fmt_a: int, fmt_b: int, sa_inv
     _f32_dev(sb_inv, sb_inv.numel(), "gemm_splitk sb_inv")
     if bias is not None:
         _f32_dev(bias, N, "gemm_splitk bias")
+    if accumulate and out is None:
+        raise NativeError("gemm_splitk(accumulate=True) needs the `out` tensor to add into")
+    if out is not None:
+        out_dtype = out.dtype
+        if out.shape != (M, N) or not out.is_contiguous():
+            raise NativeError("gemm_splitk: `out` has the wrong shape / layout")
     if out_dtype not in (torch.bfloat16, torch.float32):
         raise NativeError(f"gemm_splitk: output dtype {out_dtype} is not supported (bf16 or fp32)")
-    out = torch.empty((M, N), dtype=out_dtype, device=a.device)
-    return _gemm_splitk(a, b, M, N, K, fmt_a, fmt_b, layout_a, layout_b, sa_inv, sb_inv, bias, out, int(splits))
+    if out is None:
+        out = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    return _gemm_splitk(a, b, M, N, K, fmt_a, fmt_b, layout_a, layout_b, sa_inv, sb_inv, bias, out, int(splits), accumulate)
 
 
 def gemm_layouts_supported(M: int, N: int, K: int, out_dtype: torch.dtype = torch.bfloat16) -> bool:
@@ -930,10 +951,14 @@ def gemm_layouts_supported(M: int, N: int, K: int, out_dtype: torch.dtype = torc
 
 def gemm_layouts(a: torch.Tensor, b: torch.Tensor, fmt_a: int, fmt_b: int, layout_a: int, layout_b: int,
                  sa_inv: torch.Tensor, sb_inv: torch.Tensor, out: torch.Tensor | None = None,
-                 out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+                 out_dtype: torch.dtype = torch.bfloat16, accumulate: bool = False) -> torch.Tensor:
     """out[M,N] (bf16 or fp32) = (A . B^T) * sa_inv * sb_inv where an operand is given either as
     [rows, K] (K_FAST) or as [K, rows] (K_SLOW): no transposed copies for dgrad / wgrad.  A given
-    ``out`` decides the output type, else ``out_dtype`` does."""
+    ``out`` decides the output type, else ``out_dtype`` does.  accumulate: out = out + product (needs ``out``); the
+    product then passes through an fp32 workspace (``odl_fp8_gemm_splitk``, with one run where K is not worth cutting),
+    because the kernel that reads K-slow operands stores a tile where nothing can wait for the old values."""
+    if accumulate and out is None:
+        raise NativeError("gemm_layouts(accumulate=True) needs the `out` tensor to add into")
     if a.dtype != torch.uint8 or b.dtype != torch.uint8:
         raise NativeError("gemm_layouts operands must be uint8 FP8 codes")
     a, b = _as_2d(a), _as_2d(b)
@@ -948,8 +973,8 @@ def gemm_layouts(a: torch.Tensor, b: torch.Tensor, fmt_a: int, fmt_b: int, layou
     elif out.shape != (M, N) or out.dtype not in (torch.bfloat16, torch.float32) or not out.is_contiguous():
         raise NativeError("gemm_layouts: `out` has the wrong shape / dtype / layout")
     splits = gemm_split_count(M, N, K, layout_a == K_SLOW or layout_b == K_SLOW) if gemm_layouts_supported(M, N, K, out.dtype) else 1
-    if splits > 1:
-        return _gemm_splitk(a, b, M, N, K, fmt_a, fmt_b, layout_a, layout_b, sa_inv, sb_inv, None, out, splits)
+    if splits > 1 or accumulate:
+        return _gemm_splitk(a, b, M, N, K, fmt_a, fmt_b, layout_a, layout_b, sa_inv, sb_inv, None, out, splits, accumulate)
     _check(load().odl_fp8_gemm_layouts(a.data_ptr(), b.data_ptr(), M, N, K, fmt_a, fmt_b, layout_a, layout_b, sa_inv.data_ptr(),
                                        sb_inv.data_ptr(), out.data_ptr(), _src_dtype(out), _stream()),
            "odl_fp8_gemm_layouts")

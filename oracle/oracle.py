@@ -326,6 +326,17 @@ def t_gemm_nt(a, b, fmt_a, fmt_b, sa_inv, sb_inv, want_f32: bool = False):
     return (out.bfloat16(), out) if want_f32 else out.bfloat16()
 
 
+def t_accumulate(c_old: torch.Tensor, product_f32: torch.Tensor, bias: torch.Tensor | None = None) -> torch.Tensor:
+    """C = C + product as the GEMMs' accumulate flag defines it (include/odl_fp8.h, odl_fp8_gemm_nt): the UNROUNDED fp32
+    product (what c_gemm_nt / t_gemm_nt return with want_f32), plus the fp32 bias, plus the old C widened to fp32, each
+    addition rounded to fp32, then ONE rounding to C's type.  The backend's GEMM has the same flag (the reference
+    accumulates microbatch gradients, optimus_dl/recipe/train/mixins/execution/iteration_mixin.py:332)."""
+    v = product_f32.float()
+    if bias is not None:
+        v = v + bias.float().reshape(1, -1)
+    return (v + c_old.float()).to(c_old.dtype)
+
+
 # -------------------------------------------------- the Linear, end to end (torch)
 def linear_fwd_bwd(x, w, dy, fmt_fwd=E4M3, fmt_bwd=E5M2, rowwise=False, scales=None):
     """One FP8 Linear forward + backward on CPU with dynamic scaling.

@@ -396,7 +396,7 @@ def test_split_k_is_chosen_for_few_tiles_and_a_long_contraction(N, monkeypatch):
     a, b, sa, sb = a.cuda(), b.cuda(), sa.cuda(), sb.cuda()
     seen = []
     real = N._gemm_splitk
-    monkeypatch.setattr(N, "_gemm_splitk", lambda *args: (seen.append(args[-1]), real(*args))[1])
+    monkeypatch.setattr(N, "_gemm_splitk", lambda *args: (seen.append(args[13]), real(*args))[1])
     out = N.gemm_nt(a, b, O.E5M2, O.E4M3, sa, sb)
     assert seen == [N.gemm_split_count(768, 768, 8192)] and seen[0] > 1
     assert max_rel_err(out, O.t_gemm_nt(a.cpu(), b.cpu(), O.E5M2, O.E4M3, sa.cpu(), sb.cpu())) <= TOL
@@ -419,7 +419,7 @@ def test_split_k_entry_refuses_what_it_cannot_run(N):
 
     def call(M_=M, N_=Nn, K_=K, la=0, lb=0, splits=2, ws_bytes=ws.numel() * 4, ws_ptr=ws.data_ptr(), out_dtype=0):
         return L.odl_fp8_gemm_splitk(a.data_ptr(), b.data_ptr(), M_, N_, K_, 0, 0, la, lb, one.data_ptr(), 1, one.data_ptr(), 1,
-                                     None, out.data_ptr(), out_dtype, splits, ws_ptr, ws_bytes, s)
+                                     None, out.data_ptr(), out_dtype, 0, splits, ws_ptr, ws_bytes, s)
 
     assert call() == 0
     torch.cuda.synchronize()
@@ -462,3 +462,92 @@ def test_seeded_random_shapes_through_the_automatic_choice(N, seed):
                     out_dtype=out_dtype)
     err = max_rel_err(out, ref32.to(out_dtype))
     assert err <= (1e-3 if f32 else TOL), f"{M}x{Nn}x{K} rows={rows} cols={cols} bias={with_bias} f32={f32}: {err}"
+
+
+# ------------------------------------------------------------------ C = C + product
+def _codes(value_by_col: dict, rows: int, K: int, fmt) -> torch.Tensor:
+    x = torch.zeros((rows, K))
+    for col, v in value_by_col.items():
+        x[:, col] = v
+    q = x.to(O.TORCH_FP8[fmt]).view(torch.uint8)
+    assert torch.equal(O.t_decode(q, fmt), x), "test values must be exact in the format"
+    return q
+
+
+@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 3, 4, 5, 6, 7])
+def test_accumulate_rounds_once(N, variant):
+    """C = C + product with ONE rounding, on every kernel that can be asked for (a forced streaming variant falls back,
+    as the header says).  The product is exact (2^-8 + 2^-17); with C0 = 1 in bf16 the single rounding gives
+    1 + 2^-7 where rounding the product first would give 1 (a tie to even)."""
+    M, Nn, K = 512, 384, 512
+    a = _codes({3: 2.0 ** -4, 200: 2.0 ** -9}, M, K, O.E4M3)
+    b = _codes({3: 2.0 ** -4, 200: 2.0 ** -8}, Nn, K, O.E4M3)
+    one = torch.ones(1)
+    prod = O.t_gemm_nt(a, b, O.E4M3, O.E4M3, one, one, want_f32=True)[1]
+    assert torch.all(prod == 2.0 ** -8 + 2.0 ** -17)
+    N.gemm_set_variant(variant)
+    try:
+        c16 = torch.ones((M, Nn), dtype=torch.bfloat16, device="cuda")
+        N.gemm_nt(a.cuda(), b.cuda(), O.E4M3, O.E4M3, one.cuda(), one.cuda(), out=c16, accumulate=True)
+        assert torch.all(c16.float() == 1.0 + 2.0 ** -7), c16.float().unique()
+        assert torch.equal(c16.cpu(), O.t_accumulate(torch.ones((M, Nn), dtype=torch.bfloat16), prod))
+        c32 = torch.full((M, Nn), 2.0 ** 15, device="cuda")
+        N.gemm_nt(a.cuda(), b.cuda(), O.E4M3, O.E4M3, one.cuda(), one.cuda(), out=c32, accumulate=True)
+        assert torch.equal(c32.cpu(), O.t_accumulate(torch.full((M, Nn), 2.0 ** 15), prod))
+        assert torch.all(c32 == 2.0 ** 15 + 2.0 ** -8)
+    finally:
+        N.gemm_set_variant(-1)
+
+
+@pytest.mark.parametrize("shape", [(512, 768, 1024), (300, 200, 256), (257, 255, 384), (40, 24, 48), (1024, 512, 2048)])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+def test_accumulate_random_every_variant(N, shape, out_dtype):
+    """Random operands, scale vectors and a bias, interior and ragged tiles: out = out + product against the oracle's
+    composition (product in fp32, bias, old C, one rounding) within the GEMM tolerance, and exactly equal to what the
+    same kernel gives without the flag plus the old C where that sum needs no rounding (fp32 output, C0 = 0)."""
+    M, Nn, K = shape
+    aq, sa_inv = quantised((M, K), O.E5M2, 1e-3, 11)
+    bq, sb_inv = quantised((Nn, K), O.E4M3, 0.02, 12)
+    sa_vec = (sa_inv * torch.linspace(0.5, 2.0, M)).contiguous()
+    bias = seeded_bf16((Nn,), 1e-5, 13).float()
+    c0 = (seeded_bf16((M, Nn), 2e-5, 14).float()).to(out_dtype)
+    prod = O.t_gemm_nt(aq, bq, O.E5M2, O.E4M3, sa_vec, sb_inv, want_f32=True)[1]
+    want = O.t_accumulate(c0, prod, bias)
+    for v in [-1] + variants(N):
+        N.gemm_set_variant(v)
+        c = c0.cuda().clone()
+        N.gemm_nt(aq.cuda(), bq.cuda(), O.E5M2, O.E4M3, sa_vec.cuda(), sb_inv.cuda(), bias=bias.cuda(), out=c, accumulate=True)
+        assert max_rel_err(c, want) <= TOL, f"variant {v} {shape} {out_dtype}"
+        if out_dtype == torch.float32:
+            z = torch.zeros((M, Nn), device="cuda")
+            N.gemm_nt(aq.cuda(), bq.cuda(), O.E5M2, O.E4M3, sa_vec.cuda(), sb_inv.cuda(), bias=bias.cuda(), out=z, accumulate=True)
+            plain = N.gemm_nt(aq.cuda(), bq.cuda(), O.E5M2, O.E4M3, sa_vec.cuda(), sb_inv.cuda(), bias=bias.cuda(), out_dtype=torch.float32)
+            assert torch.equal(z, plain), f"variant {v}: adding into zeros must equal the plain product"
+    N.gemm_set_variant(-1)
+
+
+def test_accumulate_through_split_k_and_k_slow_layouts(N):
+    """The routes that pass through the fp32 workspace: a split over K (few tiles, long contraction) and an operand
+    stored K-slow (wgrad reading dY as stored), the latter also with a single run."""
+    M, Nn, K = 768, 768, 16384
+    aq, sa_inv = quantised((M, K), O.E5M2, 1e-3, 21)
+    bq, sb_inv = quantised((Nn, K), O.E4M3, 1.0, 22)
+    c0 = seeded_bf16((M, Nn), 1e-3, 23).float()
+    prod = O.t_gemm_nt(aq, bq, O.E5M2, O.E4M3, sa_inv, sb_inv, want_f32=True)[1]
+    want = O.t_accumulate(c0, prod)
+    assert N.gemm_split_count(M, Nn, K) > 1
+    c = c0.cuda().clone()
+    N.gemm_nt(aq.cuda(), bq.cuda(), O.E5M2, O.E4M3, sa_inv.cuda(), sb_inv.cuda(), out=c, accumulate=True)
+    assert max_rel_err(c, want) <= 1e-4
+    # K-slow A: the same product from a^T stored [K, M]
+    for splits in (1, 4):
+        c = c0.cuda().clone()
+        N.gemm_splitk(aq.t().contiguous().cuda(), bq.cuda(), O.E5M2, O.E4M3, sa_inv.cuda(), sb_inv.cuda(), splits,
+                      layout_a=N.K_SLOW, out=c, accumulate=True)
+        assert max_rel_err(c, want) <= 1e-4, splits
+    c = c0.cuda().clone()
+    N.gemm_layouts(aq.t().contiguous().cuda(), bq.cuda(), O.E5M2, O.E4M3, N.K_SLOW, N.K_FAST, sa_inv.cuda(), sb_inv.cuda(),
+                   out=c, accumulate=True)
+    assert max_rel_err(c, want) <= 1e-4
+    with pytest.raises(N.NativeError):
+        N.gemm_nt(aq.cuda(), bq.cuda(), O.E5M2, O.E4M3, sa_inv.cuda(), sb_inv.cuda(), accumulate=True)      # nothing to add into

@@ -491,6 +491,6 @@ def test_mx_gemm_split_over_k_matches_the_single_launch(N, shape):
     # called directly with a workspace that is too small: refused
     ws = torch.empty(16, dtype=torch.float32, device="cuda")
     out = torch.empty((M, N_), dtype=torch.float32, device="cuda")
-    rc = real(aq.data_ptr(), asc.data_ptr(), bq.data_ptr(), bsc.data_ptr(), M, N_, K, E5M2, E4M3, None, out.data_ptr(), 1, 4,
+    rc = real(aq.data_ptr(), asc.data_ptr(), bq.data_ptr(), bsc.data_ptr(), M, N_, K, E5M2, E4M3, None, out.data_ptr(), 1, 0, 4,
               ws.data_ptr(), 64, None)
     assert rc != 0

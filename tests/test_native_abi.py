@@ -162,14 +162,14 @@ def test_block_scaled_entry_points_refuse_bad_arguments_before_touching_a_device
     assert L.odl_fp8_mx_cast(p, 0, 64, 64, 0, p, p, 1, None, None, 0, None) != 0 and "multiple of 128" in err()
     assert L.odl_fp8_mx_cast(p, 0, 0, 64, 0, None, None, 0, None, None, 0, None) == 0           # nothing to do
     # GEMM: K not a multiple of 32, unknown layout, K-step-major scales with K % 128 != 0, misaligned operand
-    assert L.odl_fp8_mx_gemm_nt(p, p, p, p, 0, 64, 64, 48, 0, 0, None, p, 0, None) != 0 and "multiple of 32" in err()
-    assert L.odl_fp8_mx_gemm_nt(p, p, p, p, 5, 64, 64, 64, 0, 0, None, p, 0, None) != 0 and "scales_layout" in err()
-    assert L.odl_fp8_mx_gemm_nt(p, p, p, p, 1, 64, 64, 64, 0, 0, None, p, 0, None) != 0 and "128" in err()
-    assert L.odl_fp8_mx_gemm_nt(p + 8, p, p, p, 0, 64, 64, 64, 0, 0, None, p, 0, None) != 0 and "aligned" in err()
-    assert L.odl_fp8_mx_gemm_nt(p, p, p, p, 0, 0, 64, 64, 0, 0, None, p, 0, None) == 0           # empty output
+    assert L.odl_fp8_mx_gemm_nt(p, p, p, p, 0, 64, 64, 48, 0, 0, None, p, 0, 0, None) != 0 and "multiple of 32" in err()
+    assert L.odl_fp8_mx_gemm_nt(p, p, p, p, 5, 64, 64, 64, 0, 0, None, p, 0, 0, None) != 0 and "scales_layout" in err()
+    assert L.odl_fp8_mx_gemm_nt(p, p, p, p, 1, 64, 64, 64, 0, 0, None, p, 0, 0, None) != 0 and "128" in err()
+    assert L.odl_fp8_mx_gemm_nt(p + 8, p, p, p, 0, 64, 64, 64, 0, 0, None, p, 0, 0, None) != 0 and "aligned" in err()
+    assert L.odl_fp8_mx_gemm_nt(p, p, p, p, 0, 0, 64, 64, 0, 0, None, p, 0, 0, None) == 0           # empty output
     # split over K: too few steps per run, workspace too small
-    assert L.odl_fp8_mx_gemm_splitk(p, p, p, p, 256, 256, 1024, 0, 0, None, p, 0, 4, p, 1 << 30, None) != 0 and "shorter than 512" in err()
-    assert L.odl_fp8_mx_gemm_splitk(p, p, p, p, 256, 256, 8192, 0, 0, None, p, 0, 4, p, 64, None) != 0 and "workspace" in err()
+    assert L.odl_fp8_mx_gemm_splitk(p, p, p, p, 256, 256, 1024, 0, 0, None, p, 0, 0, 4, p, 1 << 30, None) != 0 and "shorter than 512" in err()
+    assert L.odl_fp8_mx_gemm_splitk(p, p, p, p, 256, 256, 8192, 0, 0, None, p, 0, 0, 4, p, 64, None) != 0 and "workspace" in err()
     # blockwise cast: sizes must be multiples of 128, margin in range
     assert L.odl_fp8_block_cast(p, 0, 128, 192, 0, 0, 0, p, p, None, None, None) != 0 and "multiples of 128" in err()
     assert L.odl_fp8_block_cast(p, 0, 128, 128, 0, 1000, 0, p, p, None, None, None) != 0 and "margin" in err()
