@@ -226,7 +226,10 @@ class _Fp8LinearFn(torch.autograd.Function):
             # K-slow costs the GEMM more than the copy (measured), while dy has just been written.
             tokens, n_in, n_out = x2d.shape[0], x2d.shape[1], weight.shape[0]
             fp8_wgrad = need_wgrad and recipe.wgrad
-            ctx.wgrad_direct = (fp8_wgrad and recipe.direct_layouts
+            # (not when weight gradients are added into .grad by the GEMM: the kernel that reads dy as stored cannot
+            # accumulate, and the detour through a workspace costs what the fusion saves: measured 500 us against
+            # 475 us unfused for a 14336 x 4096 fp32 gradient, where the transposed route with the flag takes 395)
+            ctx.wgrad_direct = (fp8_wgrad and recipe.direct_layouts and not recipe.fuse_wgrad_accumulation
                                 and native.gemm_layouts_supported(n_out, n_in, tokens, weight.dtype))
             if pol.kind == "delayed":
                 # the histories see a forward only when it is part of training: the module in training mode AND
