@@ -460,11 +460,22 @@ int odl_fp8_gemm_set_clock_probe(uint64_t *records_dev, int capacity);
  *                           multiple of 128).  The 4 scales a row needs for one 128-byte K step of a GEMM are one dword, and
  *                           the dwords of consecutive rows are consecutive: a GEMM tile fetches its scales for a step as
  *                           one contiguous run.  The streaming GEMM kernel takes only this layout.
+ *
+ * scale_rule: how the shared exponent of a block follows from its amax.
+ *   ODL_MX_SCALE_FLOOR  floor(log2 amax) - emax_elem: the formula of the OCP specification (section 6.3).  A block whose amax
+ *                       lies in the top eighth of its binade (mantissa above 1.75) saturates: amax itself, and anything
+ *                       beyond fp8_max * 2^shared, becomes +-fp8_max, up to 12.5 % off.
+ *   ODL_MX_SCALE_CEIL   ceil(log2(amax / fp8_max)): the smallest power of two that brings amax inside the format, i.e. the
+ *                       floor plus one where amax's mantissa exceeds 1.75; nothing saturates, and such a block loses one bit
+ *                       of resolution instead.  This is what a quantiser computes that converts amax / fp8_max to E8M0 with
+ *                       rounding up, which is how the backend behind the reference's `recipe: mxfp8` is published to work.
  */
 #define ODL_MX_SCALES_ROWMAJOR 0
 #define ODL_MX_SCALES_KSTEP 1
+#define ODL_MX_SCALE_FLOOR 0
+#define ODL_MX_SCALE_CEIL 1
 int odl_fp8_mx_cast(const void *x, int src_dtype, int64_t rows, int64_t cols, int fmt, uint8_t *out, uint8_t *scales,
-                    int scales_layout, uint8_t *out_t, uint8_t *scales_t, int scales_t_layout, odl_stream_t stream);
+                    int scales_layout, uint8_t *out_t, uint8_t *scales_t, int scales_t_layout, int scale_rule, odl_stream_t stream);
 
 /*
  * C[M, N] = sum over blocks kb of 2^(sa[m, kb] - 127) * 2^(sb[n, kb] - 127) * dot(A[m, 32 kb .. +32], B[n, 32 kb .. +32])

@@ -44,14 +44,18 @@ __device__ __forceinline__ int64_t mx_scale_at(int kstep_major, int64_t row, int
 template <int FMT> struct MxEmax { static constexpr int value = FMT == ODL_FP8_E5M2 ? 15 : 8; };
 
 // magnitude bits (fp32 layout) of a block's amax -> scale byte and the multiplier 2^-shared
+// rule 0 (ODL_MX_SCALE_FLOOR): floor(log2 amax) - emax.  rule 1 (ODL_MX_SCALE_CEIL): ceil(log2(amax / fp8_max)); fp8_max is
+// 1.75 * 2^emax in both formats, so that is one more than the floor exactly when amax's mantissa exceeds 1.75.
 template <int FMT>
-__device__ __forceinline__ void mx_scale_of(uint32_t amax_bits, uint32_t &byte, float &mul) {
+__device__ __forceinline__ void mx_scale_of(uint32_t amax_bits, int rule, uint32_t &byte, float &mul) {
     if (amax_bits >= 0x7f800000u) { byte = 0xffu; mul = 1.0f; return; }     // Inf / NaN in the block
     if (amax_bits == 0) { byte = 0u; mul = 1.0f; return; }
     // floor(log2): the exponent field, or for a subnormal (only bf16 / fp32 subnormal inputs) the position of its top bit
     int e = (int)(amax_bits >> 23) - 127;
     if ((amax_bits >> 23) == 0) e = -127 - (__builtin_clz(amax_bits) - 9);   // mantissa bit 22 is 2^-127
     int se = e - MxEmax<FMT>::value;
+    // (a subnormal amax ends at the lower clamp whatever its mantissa; its mantissa field is not normalised)
+    se += (rule != 0 && (amax_bits & 0x7fffffu) > 0x600000u && (amax_bits >> 23) != 0) ? 1 : 0;
     se = se < -127 ? -127 : se;                                            // (the upper clamp cannot be reached: e <= 127)
     byte = (uint32_t)(se + 127);
     mul = bits_to_float((uint32_t)(127 - se) << 23);                       // 2^-se, 127 - se in [8, 254]
@@ -134,7 +138,7 @@ template <int SRC, int FMT, bool WANT_ROW, bool WANT_COL>
 __global__ __launch_bounds__(kMxThreads) void mx_cast_kernel(const void *__restrict__ x, int64_t rows, int64_t cols,
                                                               uint8_t *__restrict__ out, uint8_t *__restrict__ scales,
                                                               uint8_t *__restrict__ out_t, uint8_t *__restrict__ scales_t,
-                                                              int layout, int layout_t) {
+                                                              int layout, int layout_t, int rule) {
     __shared__ __attribute__((aligned(16))) uint8_t tile[kTileC * kTileR];
     // K-step-major scale bytes leave the block as whole runs: the tile's 4 row blocks are one dword per column (256
     // contiguous bytes per tile), its 2 column blocks one 16-bit half of a dword per row.  Stored a byte at a time from
@@ -191,7 +195,7 @@ __global__ __launch_bounds__(kMxThreads) void mx_cast_kernel(const void *__restr
             m = max_quad(m);                                             // the 4 lanes tx = 4 b .. 4 b + 3 hold the block
             uint32_t byte;
             float mul;
-            mx_scale_of<FMT>(m, byte, mul);
+            mx_scale_of<FMT>(m, rule, byte, mul);
             if (col_ok && (r0 + i) < rows) {
                 uint32_t lo, hi;
                 if (__builtin_expect(m >= 0x7f800000u, 0)) {            // only a block whose amax is Inf / NaN can hold a NaN
@@ -244,7 +248,7 @@ __global__ __launch_bounds__(kMxThreads) void mx_cast_kernel(const void *__restr
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             uint32_t byte;
-            mx_scale_of<FMT>(cmax[j], byte, mul_c[j]);
+            mx_scale_of<FMT>(cmax[j], rule, byte, mul_c[j]);
             e8_c[j] = bits_to_float(byte << 23);
             // rows % 32 == 0 (host-checked): a row block is inside the matrix as a whole or not at all
             col_bytes[j / 4] |= byte << (8 * (j % 4));
@@ -800,9 +804,9 @@ const float *unit_scale_for_current_device(const char *who) {
 
 template <int SRC, int FMT>
 static void launch_mx_cast(const void *x, int64_t rows, int64_t cols, uint8_t *out, uint8_t *scales, uint8_t *out_t, uint8_t *scales_t,
-                           int layout, int layout_t, hipStream_t stream) {
+                           int layout, int layout_t, int rule, hipStream_t stream) {
     const int64_t g = ((rows + kTileR - 1) / kTileR) * ((cols + kTileC - 1) / kTileC);
-#define ODL_MX(R, C) hipLaunchKernelGGL((mx_cast_kernel<SRC, FMT, R, C>), dim3((unsigned)g), dim3(kMxThreads), 0, stream, x, rows, cols, out, scales, out_t, scales_t, layout, layout_t)
+#define ODL_MX(R, C) hipLaunchKernelGGL((mx_cast_kernel<SRC, FMT, R, C>), dim3((unsigned)g), dim3(kMxThreads), 0, stream, x, rows, cols, out, scales, out_t, scales_t, layout, layout_t, rule)
     if (out && out_t) ODL_MX(true, true);
     else if (out) ODL_MX(true, false);
     else ODL_MX(false, true);
@@ -864,9 +868,11 @@ static void launch_block_cast(const void *x, int64_t rows, int64_t cols, int mar
 using namespace odl;
 
 extern "C" int odl_fp8_mx_cast(const void *x, int src_dtype, int64_t rows, int64_t cols, int fmt, uint8_t *out, uint8_t *scales,
-                               int scales_layout, uint8_t *out_t, uint8_t *scales_t, int scales_t_layout, odl_stream_t stream_) {
+                               int scales_layout, uint8_t *out_t, uint8_t *scales_t, int scales_t_layout, int scale_rule,
+                               odl_stream_t stream_) {
     hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
     if (rows < 0 || cols < 0) return set_error(ODL_ERR_ARG, "odl_fp8_mx_cast: negative shape");
+    if (scale_rule != ODL_MX_SCALE_FLOOR && scale_rule != ODL_MX_SCALE_CEIL) return set_error(ODL_ERR_ARG, "odl_fp8_mx_cast: scale_rule %d", scale_rule);
     if (src_dtype != ODL_BF16 && src_dtype != ODL_F32) return set_error(ODL_ERR_ARG, "odl_fp8_mx_cast: src_dtype %d", src_dtype);
     if (fmt != ODL_FP8_E4M3 && fmt != ODL_FP8_E5M2) return set_error(ODL_ERR_ARG, "odl_fp8_mx_cast: fmt %d", fmt);
     if (rows * cols == 0) return ODL_OK;
@@ -888,11 +894,11 @@ extern "C" int odl_fp8_mx_cast(const void *x, int src_dtype, int64_t rows, int64
     const int64_t tiles = ((rows + kTileR - 1) / kTileR) * ((cols + kTileC - 1) / kTileC);
     if (tiles > 0x7fffffffLL) return set_error(ODL_ERR_SHAPE, "odl_fp8_mx_cast: too many tiles for one launch");
     if (src_dtype == ODL_BF16) {
-        if (fmt == ODL_FP8_E4M3) launch_mx_cast<ODL_BF16, ODL_FP8_E4M3>(x, rows, cols, out, scales, out_t, scales_t, scales_layout, scales_t_layout, stream);
-        else launch_mx_cast<ODL_BF16, ODL_FP8_E5M2>(x, rows, cols, out, scales, out_t, scales_t, scales_layout, scales_t_layout, stream);
+        if (fmt == ODL_FP8_E4M3) launch_mx_cast<ODL_BF16, ODL_FP8_E4M3>(x, rows, cols, out, scales, out_t, scales_t, scales_layout, scales_t_layout, scale_rule, stream);
+        else launch_mx_cast<ODL_BF16, ODL_FP8_E5M2>(x, rows, cols, out, scales, out_t, scales_t, scales_layout, scales_t_layout, scale_rule, stream);
     } else {
-        if (fmt == ODL_FP8_E4M3) launch_mx_cast<ODL_F32, ODL_FP8_E4M3>(x, rows, cols, out, scales, out_t, scales_t, scales_layout, scales_t_layout, stream);
-        else launch_mx_cast<ODL_F32, ODL_FP8_E5M2>(x, rows, cols, out, scales, out_t, scales_t, scales_layout, scales_t_layout, stream);
+        if (fmt == ODL_FP8_E4M3) launch_mx_cast<ODL_F32, ODL_FP8_E4M3>(x, rows, cols, out, scales, out_t, scales_t, scales_layout, scales_t_layout, scale_rule, stream);
+        else launch_mx_cast<ODL_F32, ODL_FP8_E5M2>(x, rows, cols, out, scales, out_t, scales_t, scales_layout, scales_t_layout, scale_rule, stream);
     }
     return check_launch("odl_fp8_mx_cast");
 }

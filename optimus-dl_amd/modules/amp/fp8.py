@@ -133,6 +133,7 @@ class ScalingPolicy:
     amax_history_len: int
     amax_compute_algo: str    # "max" | "most_recent"
     reduce_amax: bool         # one GPU: the cross-rank MAX all-reduce is a no-op
+    mx_scale_rule: int = 1    # mxfp8 only: native.MX_CEIL (shared exponent rounded up) or native.MX_FLOOR (OCP formula)
 
 
 class FP8Recipe:
@@ -149,6 +150,7 @@ class FP8Recipe:
         fp8_dpa: bool = False,
         fp8_mha: bool = False,
         wgrad: bool = True,
+        mx_scale_rule: str = "ceil",
     ):
         if not is_native_backend_available():
             raise ImportError(
@@ -183,9 +185,17 @@ class FP8Recipe:
             raise ValueError(f"Unsupported amax_compute_algo: {amax_compute_algo} (max, most_recent)")
         if amax_history_len < 1:
             raise ValueError("amax_history_len must be >= 1")
+        # mxfp8: how a block's shared exponent follows from its amax.  "ceil" (default): ceil(log2(amax / fp8_max)),
+        # nothing saturates -- what a quantiser gives that converts amax / fp8_max to E8M0 rounding up, as the backend
+        # behind the reference's `recipe: mxfp8` (fp8.py:301-306) is published to.  "floor": the formula of the OCP MX
+        # specification, floor(log2 amax) - emax, which lets a block amax in the top eighth of its binade saturate.
+        if mx_scale_rule not in ("ceil", "floor"):
+            raise ValueError(f"Unsupported mx_scale_rule: {mx_scale_rule} (ceil, floor)")
+        self.mx_scale_rule = mx_scale_rule
         self._recipe = ScalingPolicy(
             kind=self.recipe_type.value, fmt_fwd=fwd, fmt_bwd=bwd, margin=margin,
             amax_history_len=amax_history_len, amax_compute_algo=amax_compute_algo, reduce_amax=reduce_amax,
+            mx_scale_rule=native.MX_CEIL if mx_scale_rule == "ceil" else native.MX_FLOOR,
         )
         # the arenas that modules reserve their delayed-scaling roles in when they first run under this recipe.
         # The modules keep the views (the state is theirs): another recipe of the same shape -- the one an
@@ -424,6 +434,7 @@ def create_fp8_recipe(
     fp8_dpa: bool = False,
     fp8_mha: bool = False,
     wgrad: bool = True,
+    mx_scale_rule: str = "ceil",
 ) -> FP8Recipe | None:
     """FP8Recipe when the backend is usable, else None (callers fall back to bf16 AMP)."""
     if not is_native_backend_available():
@@ -434,7 +445,7 @@ def create_fp8_recipe(
         return None
     return FP8Recipe(recipe_type=recipe_type, format=format, margin=margin, amax_history_len=amax_history_len,
                      amax_compute_algo=amax_compute_algo, reduce_amax=reduce_amax, fp8_dpa=fp8_dpa, fp8_mha=fp8_mha,
-                     wgrad=wgrad)
+                     wgrad=wgrad, mx_scale_rule=mx_scale_rule)
 
 
 @contextmanager

@@ -123,7 +123,8 @@ def _block_cast(pol, x2d: torch.Tensor, fmt: int, want_rowmajor: bool, want_tran
     """Codes and E8M0 scale bytes of the two block-scaled recipes: 32-element blocks (mxfp8) or 128-element blocks with
     128 x 128 ones for a weight (blockwise)."""
     if pol.kind == "mxfp8":
-        return native.mx_cast(x2d, fmt, want_rowmajor=want_rowmajor, want_transposed=want_transposed)
+        return native.mx_cast(x2d, fmt, want_rowmajor=want_rowmajor, want_transposed=want_transposed,
+                              scale_rule=pol.mx_scale_rule)
     return native.block_cast(x2d, fmt, pol.margin, two_d=weight, want_rowmajor=want_rowmajor, want_transposed=want_transposed)
 
 
@@ -131,7 +132,7 @@ def _mx_input_shared(recipe: FP8Recipe, x2d: torch.Tensor, fmt: int, need_t: boo
     """Block-scaled codes and scale bytes of a Linear's input (blocks along the features; with need_t also of its
     transpose, blocks along the tokens), made once for the Linears fed by the very same tensor."""
     pol = recipe.recipe
-    key = _input_key(x2d, pol.kind, fmt, pol.margin)
+    key = _input_key(x2d, (pol.kind, pol.mx_scale_rule), fmt, pol.margin)
     hit = recipe.shared_input if recipe.share_inputs else None
     if hit is not None and hit["key"] == key and (hit["q_t"] is not None or not need_t):
         return hit["q"], hit["s_inv"], hit["q_t"], hit["s_t"]
@@ -618,7 +619,7 @@ class FP8Linear(nn.Linear):
         while the Parameter is unchanged."""
         pol = recipe.recipe
         fmt = pol.fmt_fwd
-        key = _weight_key(weight, fmt, (pol.kind, pol.margin))
+        key = _weight_key(weight, fmt, (pol.kind, pol.margin, pol.mx_scale_rule))
         hit = self._wcache_rowwise.get("mx")
         if hit is not None and hit[0] == key and recipe.cache_weights and (hit[3] is not None or not need_t):
             return hit[1:]

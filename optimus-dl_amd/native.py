@@ -142,7 +142,7 @@ def load() -> ctypes.CDLL:
         L.odl_fp8_gemm_variant_name.restype = ctypes.c_char_p
         L.odl_fp8_gemm_set_variant.argtypes = [i32]
         L.odl_fp8_gemm_set_clock_probe.argtypes = [vp, i32]
-        L.odl_fp8_mx_cast.argtypes = [vp, i32, i64, i64, i32, vp, vp, i32, vp, vp, i32, vp]
+        L.odl_fp8_mx_cast.argtypes = [vp, i32, i64, i64, i32, vp, vp, i32, vp, vp, i32, i32, vp]
         L.odl_fp8_mx_gemm_nt.argtypes = [vp, vp, vp, vp, i32, i64, i64, i64, i32, i32, vp, vp, i32, i32, vp]
         L.odl_fp8_block_cast.argtypes = [vp, i32, i64, i64, i32, i32, i32, vp, vp, vp, vp, vp]
         L.odl_fp8_mx_gemm_splitk.argtypes = [vp, vp, vp, vp, i64, i64, i64, i32, i32, vp, vp, i32, i32, i32, vp, i64, vp]
@@ -759,6 +759,7 @@ def gemm_nt(a: torch.Tensor, b: torch.Tensor, fmt_a: int, fmt_b: int, sa_inv: to
 
 MX_BLOCK = 32
 MX_ROWMAJOR, MX_KSTEP = 0, 1           # ODL_MX_SCALES_*
+MX_FLOOR, MX_CEIL = 0, 1               # ODL_MX_SCALE_*: shared exponent floor(log2 amax) - emax / ceil(log2(amax / fp8_max))
 
 
 def _mx_scales(rows: int, length: int, layout: int | None, device) -> tuple[torch.Tensor, int]:
@@ -781,11 +782,13 @@ def mx_scales_rowmajor(scales: torch.Tensor) -> torch.Tensor:
     return scales
 
 
-def mx_cast(x: torch.Tensor, fmt: int, want_rowmajor: bool = True, want_transposed: bool = False, layout: int | None = None):
+def mx_cast(x: torch.Tensor, fmt: int, want_rowmajor: bool = True, want_transposed: bool = False, layout: int | None = None,
+            scale_rule: int = MX_FLOOR):
     """MXFP8 conversion of ``x`` [rows, cols] in one launch -> (codes [rows, cols], their scales, codes_t [cols, rows],
     their scales); the pair that was not asked for is (None, None).  Scales are E8M0 bytes, one per 32 elements along
     the last axis of the codes they belong to, stored as ``_mx_scales`` describes (layout None: K-step-major where the
-    blocked axis allows it)."""
+    blocked axis allows it).  scale_rule: MX_FLOOR (the OCP formula; a block amax in the top eighth of its binade
+    saturates) or MX_CEIL (the exponent rounded up: nothing saturates)."""
     x = _as_2d(x)
     rows, cols = x.shape
     if not (want_rowmajor or want_transposed):
@@ -801,7 +804,7 @@ def mx_cast(x: torch.Tensor, fmt: int, want_rowmajor: bool = True, want_transpos
         sc_t, lay_t = _mx_scales(cols, rows, layout, dev)
     ptr = lambda t: t.data_ptr() if t is not None else None
     _check(load().odl_fp8_mx_cast(x.data_ptr(), _src_dtype(x), rows, cols, fmt, ptr(out), ptr(sc), lay, ptr(out_t), ptr(sc_t), lay_t,
-                                  _stream()), "odl_fp8_mx_cast")
+                                  int(scale_rule), _stream()), "odl_fp8_mx_cast")
     return out, sc, out_t, sc_t
 
 

@@ -257,7 +257,11 @@ ORACLE_API void oracle_gemm_nt(const uint8_t *a, const uint8_t *b, int64_t M, in
  */
 static inline int emax_elem(int fmt) { return fmt == FMT_E5M2 ? 15 : 8; }
 
-ORACLE_API void oracle_mx_quantise_bf16(const uint16_t *x, int64_t rows, int64_t cols, int fmt, uint8_t *codes, uint8_t *scales) {
+/* rule 0: the specification's floor (above).  rule 1: the exponent rounded UP, shared_exp = ceil(log2(amax / fp8_max)), the
+ * smallest power of two that brings the block's amax inside the format, so that no element saturates (the convention of
+ * quantisers that derive the scale byte from amax / fp8_max with a round-up conversion to E8M0).  fp8_max = 1.75 * 2^emax for
+ * both formats, so with amax = m * 2^e, 1 <= m < 2: ceil(log2(amax / fp8_max)) = e - emax + (m > 1.75 ? 1 : 0). */
+ORACLE_API void oracle_mx_quantise_bf16(const uint16_t *x, int64_t rows, int64_t cols, int fmt, int rule, uint8_t *codes, uint8_t *scales) {
     const int64_t nb = cols / 32;
     for (int64_t r = 0; r < rows; ++r)
         for (int64_t b = 0; b < nb; ++b) {
@@ -272,6 +276,7 @@ ORACLE_API void oracle_mx_quantise_bf16(const uint16_t *x, int64_t rows, int64_t
                 int e;                                                            /* floor(log2(amax)), subnormals included */
                 (void)frexpf(bits_f32(mag), &e);
                 int se = (e - 1) - emax_elem(fmt);
+                if (rule == 1 && frexpf(bits_f32(mag), &e) > 0.875f) se += 1;        /* frexp's mantissa is m / 2 */
                 if (se < -127) se = -127;
                 if (se > 127) se = 127;
                 sb = (uint8_t)(se + 127);

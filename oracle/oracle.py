@@ -65,7 +65,7 @@ def lib() -> ctypes.CDLL:
         L.oracle_cast_transpose_bf16.argtypes = [vp, i64, i64, vp, i32, i32, vp, vp]
         L.oracle_gemm_nt.argtypes = [vp, vp, i64, i64, i64, i32, i32, vp, i64, vp, i64, vp, vp]
         L.oracle_delayed_update.argtypes = [vp, i64, i64, vp, vp, vp, i32, i32]
-        L.oracle_mx_quantise_bf16.argtypes = [vp, i64, i64, i32, vp, vp]
+        L.oracle_mx_quantise_bf16.argtypes = [vp, i64, i64, i32, i32, vp, vp]
         L.oracle_mx_gemm_nt.argtypes = [vp, vp, vp, vp, i64, i64, i64, i32, i32, vp, vp, vp]
         L.oracle_block_quantise_bf16.argtypes = [vp, i64, i64, i64, i64, i32, i32, vp, vp]
         L.oracle_sigmoid.argtypes = [f32]
@@ -416,25 +416,32 @@ class DelayedState:
 # ------------------------------------------------------------------------ MXFP8
 MX_BLOCK = 32
 MX_EMAX = {E4M3: 8, E5M2: 15}
+MX_FLOOR, MX_CEIL = 0, 1       # shared exponent: floor(log2 amax) - emax (OCP MX v1.0) / ceil(log2(amax / fp8_max))
 
 
-def c_mx_quantise(x: torch.Tensor, fmt: int):
+def c_mx_quantise(x: torch.Tensor, fmt: int, rule: int = MX_FLOOR):
     """MXFP8 of a bf16 matrix, blocks of 32 along the last axis -> (codes uint8 [R, C], scale bytes uint8 [R, C/32])."""
     rows, cols = x.shape
     assert cols % MX_BLOCK == 0
     xb = _bf16_bits(x)
     codes, scales = np.empty((rows, cols), dtype=np.uint8), np.empty((rows, cols // MX_BLOCK), dtype=np.uint8)
-    lib().oracle_mx_quantise_bf16(_p(xb), rows, cols, fmt, _p(codes), _p(scales))
+    lib().oracle_mx_quantise_bf16(_p(xb), rows, cols, fmt, rule, _p(codes), _p(scales))
     return torch.from_numpy(codes), torch.from_numpy(scales)
 
 
-def t_mx_quantise(x: torch.Tensor, fmt: int):
-    """The same conversion with torch routines (frexp for floor(log2), exact power-of-two scaling, the CPU float8 cast)."""
+def t_mx_quantise(x: torch.Tensor, fmt: int, rule: int = MX_FLOOR):
+    """The same conversion with torch routines (frexp for floor(log2), exact power-of-two scaling, the CPU float8 cast).
+    MX_CEIL: the exponent of the smallest power of two p with amax / p <= fp8_max, found by comparing amax with
+    fp8_max * 2^k for the two candidates k (both products are exact)."""
     rows, cols = x.shape
     v = x.float().reshape(rows, cols // MX_BLOCK, MX_BLOCK)
     amax = v.abs().amax(dim=2)
     _, e = torch.frexp(amax)                                   # amax = m * 2^e with 0.5 <= m < 1: floor(log2) = e - 1
-    se = (e - 1 - MX_EMAX[fmt]).clamp(-127, 127)
+    se = e - 1 - MX_EMAX[fmt]
+    if rule == MX_CEIL:
+        fits = amax.double() <= torch.ldexp(torch.full_like(amax, FP8_MAX[fmt]).double(), se)
+        se = torch.where(fits, se, se + 1)
+    se = se.clamp(-127, 127)
     bad = ~torch.isfinite(amax)
     se = torch.where((amax == 0) | bad, torch.full_like(se, -127), se)
     scaled = torch.ldexp(v, (-se).unsqueeze(2).expand_as(v).to(torch.int32))

@@ -41,6 +41,12 @@ def _mixed(shape, seed):
     return x.bfloat16()
 
 
+def N_mod():
+    from optimus_dl_amd import native
+
+    return native
+
+
 CAST_SHAPES = [(32, 32), (128, 64), (64, 96), (160, 224), (256, 1024), (1024, 768), (96, 4096), (2016, 160)]
 
 
@@ -48,6 +54,32 @@ def _kstep(scales: torch.Tensor) -> torch.Tensor:
     """Row-major scale bytes [rows, blocks] -> the K-step-major layout [blocks / 4, rows, 4]."""
     rows, blocks = scales.shape
     return scales.reshape(rows, blocks // 4, 4).permute(1, 0, 2).contiguous()
+
+
+@pytest.mark.parametrize("shape", CAST_SHAPES)
+@pytest.mark.parametrize("fmt", [E4M3, E5M2])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_mx_cast_round_up_rule_bit_exact(N, shape, fmt, dtype):
+    """The shared exponent rounded up (ODL_MX_SCALE_CEIL): codes and scale bytes of both layouts against the C oracle and
+    its torch restatement, on data with block maxima on and around the 1.75 boundary where the two rules part."""
+    x = _mixed(shape, seed=shape[0] * 5 + shape[1] + fmt).float()
+    rows, cols = shape
+    x[0, 0], x[0, 1:32] = 1.75 * 2.0 ** 3, 0.0                      # exactly fp8_max after scaling: no bump
+    x[rows - 1, cols - 32], x[rows - 1, cols - 31:] = -1.7578125 * 2.0 ** -4, 0.0      # the next bf16 above: bump
+    x = x.bfloat16()
+    out, sc, out_t, sc_t = N.mx_cast(x.to(dtype).cuda(), fmt, want_rowmajor=True, want_transposed=True, scale_rule=N.MX_CEIL)
+    sc, sc_t = N.mx_scales_rowmajor(sc), N.mx_scales_rowmajor(sc_t)
+    wc, ws = O.c_mx_quantise(x, fmt, O.MX_CEIL)
+    assert_bytes_equal(sc, ws, f"scale bytes {shape} fmt {fmt}")
+    assert_bytes_equal(out, wc, f"codes {shape} fmt {fmt}")
+    tc, ts = O.t_mx_quantise(x, fmt, O.MX_CEIL)
+    assert_bytes_equal(sc, ts, f"scale bytes (torch restatement) {shape}")
+    assert_bytes_equal(out, tc, f"codes (torch restatement) {shape}")
+    wct, wst = O.c_mx_quantise(x.t().contiguous(), fmt, O.MX_CEIL)
+    assert_bytes_equal(sc_t, wst, f"transposed scale bytes {shape} fmt {fmt}")
+    assert_bytes_equal(out_t, wct, f"transposed codes {shape} fmt {fmt}")
+    floor_sc = N.mx_scales_rowmajor(N.mx_cast(x.to(dtype).cuda(), fmt, scale_rule=N.MX_FLOOR)[1])
+    assert int(sc[0, 0]) == int(floor_sc[0, 0]) and int(sc[rows - 1, -1]) == int(floor_sc[rows - 1, -1]) + 1
 
 
 @pytest.mark.parametrize("shape", CAST_SHAPES)
@@ -347,9 +379,10 @@ def test_mx_round_trip_error_bound_at_full_size(N):
 
 
 # ------------------------------------------------------------------------------------------------ the Linear
-def _mx_linear_reference(x, w, dy, fmt_fwd, fmt_bwd, bias=None):
-    """The three GEMMs of a Linear under MXFP8, emulated: every operand quantised along the axis its GEMM contracts."""
-    q = O.c_mx_quantise
+def _mx_linear_reference(x, w, dy, fmt_fwd, fmt_bwd, bias=None, rule=O.MX_CEIL):
+    """The three GEMMs of a Linear under MXFP8, emulated: every operand quantised along the axis its GEMM contracts, the
+    shared exponents by `rule` (the recipe's default is the round-up rule)."""
+    q = lambda t, fmt: O.c_mx_quantise(t, fmt, rule)
     y = O.t_mx_gemm_nt(*q(x, fmt_fwd), *q(w, fmt_fwd), fmt_fwd, fmt_fwd, bias=bias)
     gq, gs = q(dy, fmt_bwd)
     wtq, wts = q(w.t().contiguous(), fmt_fwd)
@@ -380,10 +413,20 @@ def test_mxfp8_linear_matches_emulation(fmt, shape):
         assert got.dtype == torch.bfloat16
         err = max_rel_err(got, ref[name])
         assert err <= 1e-2, f"{name}: {err}"
-    # and it is a Linear: near the bf16 product.  (The floor rule of the shared exponent lets a block amax in the top
-    # eighth of its binade saturate, up to 12.5 % off on that element, which the outlier channel makes visible.)
+    # and it is a Linear: near the bf16 product
     want = x.float() @ w.float().t()
-    assert max_rel_err(y, want) <= 0.2
+    assert max_rel_err(y, want) <= 0.1
+    # the same under the specification's floor rule, which lets a block amax in the top eighth of its binade saturate (up
+    # to 12.5 % off on that element, which the outlier channel makes visible)
+    floor = amp.create_fp8_recipe("mxfp8", fmt, mx_scale_rule="floor")
+    assert floor.recipe.mx_scale_rule == N_mod().MX_FLOOR and recipe.recipe.mx_scale_rule == N_mod().MX_CEIL
+    lin2 = make_linear(w)
+    y2, dx2, dw2 = run_step(lin2, floor, x, dy)
+    ref2 = _mx_linear_reference(x, w, dy, O.E4M3, fb, rule=O.MX_FLOOR)
+    for name, got in (("y", y2), ("dx", dx2), ("dw", dw2)):
+        assert max_rel_err(got, ref2[name]) <= 1e-2, name
+    assert max_rel_err(y2, want) <= 0.2
+    assert not torch.equal(y, y2)
 
 
 def test_mxfp8_linear_bias_fp32_weights_and_weight_cache():

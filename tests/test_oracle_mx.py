@@ -109,3 +109,64 @@ def test_mx_gemm_c_vs_torch_vs_float64():
     asc2[2, 1] = 255
     _, poisoned = O.c_mx_gemm_nt(ac, asc2, bc, bsc, fa, fb)
     assert torch.isnan(poisoned[2]).all() and not torch.isnan(poisoned[3]).any()
+
+
+# ------------------------------------------------------------------ the round-up rule of the shared exponent (MX_CEIL)
+@pytest.mark.parametrize("fmt", [O.E4M3, O.E5M2])
+def test_round_up_rule_hand_worked(fmt):
+    """amax = m * 2^e: the shared exponent is e - emax for m <= 1.75 (as under the floor rule) and one more for m > 1.75,
+    where the floor rule saturates.  fp8_max = 1.75 * 2^emax, so 1.75 itself still fits exactly."""
+    emax = O.MX_EMAX[fmt]
+    row = torch.zeros(1, 128, dtype=torch.bfloat16)
+    row[0, :32] = bf16([1.75] + [1.0] * 31)                       # exactly fp8_max after scaling by 2^emax: no bump
+    row[0, 32:64] = bf16([1.7578125, 1.0] + [0.0] * 30)           # the next bf16 above 1.75: one more
+    row[0, 64:96] = bf16([-1.9375, 0.5] + [0.0] * 30)
+    row[0, 96:128] = bf16([3.0] + [0.0] * 31)                     # 1.5 * 2^1
+    codes, scales = O.c_mx_quantise(row, fmt, O.MX_CEIL)
+    assert scales.tolist() == [[127 - emax, 128 - emax, 128 - emax, 128 - emax]]
+    floor_scales = O.c_mx_quantise(row, fmt, O.MX_FLOOR)[1]
+    assert floor_scales.tolist() == [[127 - emax, 127 - emax, 127 - emax, 128 - emax]]
+    back = O.t_mx_dequantise(codes, scales, fmt)
+    # nothing saturated: 1.9375 is rounded like any other value (to 2.0, the nearest code one binade up), not clamped
+    assert back[0, 0].item() == 1.75 and back[0, 64].item() == -2.0 and back[0, 65].item() == 0.5
+    assert O.t_mx_dequantise(*O.c_mx_quantise(row, fmt, O.MX_FLOOR), fmt)[0, 64].item() == -1.75         # the floor rule did
+
+
+@pytest.mark.parametrize("fmt", [O.E4M3, O.E5M2])
+def test_round_up_rule_c_vs_torch_vs_float64(fmt):
+    """C and torch restatements agree byte for byte; the scale is 2^ceil(log2(amax / fp8_max)) evaluated in float64
+    (the quotient of an 8-bit-mantissa amax and 1.75 * 2^emax, and log2 of a value that is a power of two exactly when
+    the quotient is, so ceil is safe); no element of a finite block saturates: |element| * 2^-shared <= fp8_max; and
+    the two rules differ exactly in the blocks whose amax has a mantissa above 1.75."""
+    x = seeded_bf16((96, 512), 1.0, 15)
+    x[3, 40] = 3.0e38
+    x[5, :32] = 0
+    x[7, 100] = float("inf")
+    x[9, 7] = float("nan")
+    x[11, 64:96] = (x[11, 64:96].float() * 2.0 ** -120).bfloat16()
+    x[13, 96:128] = (x[13, 96:128].float() * 2.0 ** -130).bfloat16()
+    x[15, 128] = 1.75 * 2.0 ** 5                                   # a block maximum exactly on the boundary
+    x[15, 129:160] = 0.0
+    cc, cs = O.c_mx_quantise(x, fmt, O.MX_CEIL)
+    tc, ts = O.t_mx_quantise(x, fmt, O.MX_CEIL)
+    assert_bytes_equal(cs, ts, "scale bytes, C vs torch")
+    assert_bytes_equal(cc, tc, "codes, C vs torch")
+    v = x.double().reshape(96, 16, 32)
+    amax = v.abs().amax(dim=2)
+    ok = torch.isfinite(amax) & (amax > 0)
+    q = torch.where(ok, amax, torch.ones_like(amax)) / O.FP8_MAX[fmt]
+    want = torch.where(ok, torch.ceil(torch.log2(q)).clamp(-127, 127) + 127,
+                       torch.where(amax == 0, torch.zeros_like(amax), torch.full_like(amax, 255)))
+    assert torch.equal(cs.double(), want)
+    shared = cs.double() - 127
+    fits = (v.abs() <= (O.FP8_MAX[fmt] * torch.exp2(shared)).unsqueeze(2)) | ~ok.unsqueeze(2) | (shared == -127).unsqueeze(2)
+    assert bool(fits.all()), "an element would saturate under the round-up rule"
+    fs = O.c_mx_quantise(x, fmt, O.MX_FLOOR)[1]
+    mant = amax / torch.exp2(torch.floor(torch.log2(torch.where(ok, amax, torch.ones_like(amax)))))
+    bumped = ok & (mant > 1.75) & (fs < 254) & (fs > 0)
+    assert torch.equal((cs.int() - fs.int())[ok], bumped[ok].int())
+    # error of the largest element of a block: at most half a unit of a 3-bit (E4M3) / 2-bit (E5M2) mantissa, never 12.5 %
+    back = O.t_mx_dequantise(cc, cs, fmt).double().reshape(96, 16, 32)
+    top = v.abs() == amax.unsqueeze(2)
+    rel = ((back - v).abs() / amax.unsqueeze(2).clamp_min(1e-300))[top & ok.unsqueeze(2) & (shared > -127).unsqueeze(2)]
+    assert rel.max().item() <= (2.0 ** -4 if fmt == O.E4M3 else 2.0 ** -3)
