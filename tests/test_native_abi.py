@@ -155,12 +155,13 @@ def test_block_scaled_entry_points_refuse_bad_arguments_before_touching_a_device
     err = lambda: L.odl_fp8_last_error().decode()
     p = 4096                                                     # any aligned non-null address: it is never dereferenced
     # cast: negative shape, unknown format, scale bytes without codes, blocked axis not a multiple of 32 / of 128
-    assert L.odl_fp8_mx_cast(p, 0, -1, 64, 0, p, p, 0, None, None, 0, None) != 0 and "negative" in err()
-    assert L.odl_fp8_mx_cast(p, 0, 64, 64, 7, p, p, 0, None, None, 0, None) != 0 and "fmt" in err()
-    assert L.odl_fp8_mx_cast(p, 0, 64, 64, 0, p, None, 0, None, None, 0, None) != 0 and "go together" in err()
-    assert L.odl_fp8_mx_cast(p, 0, 64, 48, 0, p, p, 0, None, None, 0, None) != 0 and "multiple of 32" in err()
-    assert L.odl_fp8_mx_cast(p, 0, 64, 64, 0, p, p, 1, None, None, 0, None) != 0 and "multiple of 128" in err()
-    assert L.odl_fp8_mx_cast(p, 0, 0, 64, 0, None, None, 0, None, None, 0, None) == 0           # nothing to do
+    assert L.odl_fp8_mx_cast(p, 0, -1, 64, 0, p, p, 0, None, None, 0, 0, None) != 0 and "negative" in err()
+    assert L.odl_fp8_mx_cast(p, 0, 64, 64, 7, p, p, 0, None, None, 0, 0, None) != 0 and "fmt" in err()
+    assert L.odl_fp8_mx_cast(p, 0, 64, 64, 0, p, None, 0, None, None, 0, 0, None) != 0 and "go together" in err()
+    assert L.odl_fp8_mx_cast(p, 0, 64, 48, 0, p, p, 0, None, None, 0, 0, None) != 0 and "multiple of 32" in err()
+    assert L.odl_fp8_mx_cast(p, 0, 64, 64, 0, p, p, 1, None, None, 0, 0, None) != 0 and "multiple of 128" in err()
+    assert L.odl_fp8_mx_cast(p, 0, 0, 64, 0, None, None, 0, None, None, 0, 0, None) == 0        # nothing to do
+    assert L.odl_fp8_mx_cast(p, 0, 64, 64, 0, p, p, 0, None, None, 0, 2, None) != 0 and "scale_rule" in err()
     # GEMM: K not a multiple of 32, unknown layout, K-step-major scales with K % 128 != 0, misaligned operand
     assert L.odl_fp8_mx_gemm_nt(p, p, p, p, 0, 64, 64, 48, 0, 0, None, p, 0, 0, None) != 0 and "multiple of 32" in err()
     assert L.odl_fp8_mx_gemm_nt(p, p, p, p, 5, 64, 64, 64, 0, 0, None, p, 0, 0, None) != 0 and "scales_layout" in err()
