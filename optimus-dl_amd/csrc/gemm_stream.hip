@@ -44,6 +44,11 @@
 //   others : nothing is younger than the loads of step kt+1            -> vmcnt(0)
 // (An L2 prefetch, one lane per 128-byte line a few steps ahead, was tried and removed: the
 // scattered loads occupy the texture path that the direct-to-LDS loads need, 14 % of the K loop.)
+//
+// Two compile-time switches exist for measuring where the energy of a launch goes (never defined in the shipped
+// build; the results are wrong on purpose): ODL_EXP_SAME_PANELS makes every tile read the operand panels of tile
+// (0, 0), so that nothing comes from beyond the L2; ODL_EXP_HALF_LDS_READS makes the second K half of a step
+// multiply the fragments of the first again, which halves the LDS-to-register traffic.
 #include "gemm_common.h"
 
 namespace odl {
@@ -175,12 +180,14 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
     auto lds_addr_of = [](const uint8_t *p) { return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) uint8_t *)p; };
     // load j of a stage: j < LOADS -> operand A, else operand B
     auto issue_one = [&](uint8_t *sa, uint8_t *sb, const v4i &da, const v4i &db, int kstep, int j) {
+
         if (j < LOADS) dma(da, lds_addr_of(sa) + (wave + j * NW) * 1024, voff_a[j], kstep * kstep_a);
         else dma(db, lds_addr_of(sb) + (wave + (j - LOADS) * NW) * 1024, voff_b[j - LOADS], kstep * kstep_b);
     };
 
     int m0 = 0, n0 = 0;
     v4i rsrc_a, rsrc_b, next_a, next_b;           // raw buffer descriptors (base, stride 0, bytes, format)
+
 
     // one 256-byte direct-to-LDS load: 64 lanes x 4 bytes land at lds_addr + lane * 4
     auto dma4 = [](const v4i &rsrc, uint32_t lds_addr, int vo, int so) {
@@ -337,8 +344,13 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             acc[i / 4][i % 4] = mma_step<FB, FA, MX, 0>(b0[i % 4], a0[i / 4], acc[i / 4][i % 4], scb[par][i % 4], sca[par][i / 4]);
+#ifdef ODL_EXP_HALF_LDS_READS         // experiment: the second K half multiplies the fragments of the first again
+            if (i < 4) a1[i] = a0[i];
+            else if (i < 8) b1[i - 4] = b0[i - 4];
+#else
             if (i < 4) a1[i] = read_a(sa_cur, i, 1);
             else if (i < 8) b1[i - 4] = read_b(sb_cur, i - 4, 1);
+#endif
             __builtin_amdgcn_sched_barrier(0);
         }
     };
@@ -553,7 +565,11 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
         bool next_padded = false;
         tile_origin(has_next ? next_pid : pid, next_m0, next_n0);
         item_steps(has_next ? next_pid : pid, next_first, next_kt, next_padded);
+#ifdef ODL_EXP_SAME_PANELS            // experiment: every tile reads the operand panels of tile (0, 0): all traffic stays in the L2
+        const v4i na = rsrc_for(g.a, 0, g.M, TA, next_first), nb = rsrc_for(g.b, 0, g.N, TB, next_first);
+#else
         const v4i na = rsrc_for(g.a, next_m0, g.M, TA, next_first), nb = rsrc_for(g.b, next_n0, g.N, TB, next_first);
+#endif
         next_a = has_next ? na : empty;
         next_b = has_next ? nb : empty;
         if constexpr (MX) {
