@@ -144,7 +144,16 @@ def timed_steps(torch, one, steps, warmup):
     synchronised on both sides); min / median / max are per step, from one HIP event between consecutive steps, so a
     single slow step (an allocator that has to grow, a first-use set-up) shows up as max >> median instead of hiding in
     the mean.  `allocator` tells whether torch's caching allocator had to go back to the driver during the timed steps."""
+    t_w = time.perf_counter()
     for _ in range(warmup):
+        one()
+    torch.cuda.synchronize()
+    # short steps: keep warming until the board has been busy for 50 ms.  After an idle spell it runs a handful of
+    # launches at a high clock, then drops well below its sustained clock and takes some 10 ms to come back; a step of
+    # 1 ms timed right after three warm-up steps sits in that transient (measured: 1.42, 1.24, 1.25 ... 1.13 ms)
+    per_step = max((time.perf_counter() - t_w) / max(warmup, 1), 1e-4)
+    extra = min(64, max(0, int(0.05 / per_step) - warmup))
+    for _ in range(extra):
         one()
     torch.cuda.synchronize()
     before = torch.cuda.memory_stats()
@@ -158,7 +167,7 @@ def timed_steps(torch, one, steps, warmup):
     wall = time.perf_counter() - t0
     after = torch.cuda.memory_stats()
     per = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(steps))
-    return {"ms_per_step": 1e3 * wall / steps, "min_ms": per[0], "median_ms": per[len(per) // 2], "max_ms": per[-1],
+    return {"ms_per_step": 1e3 * wall / steps, "warmup_steps": warmup + extra, "min_ms": per[0], "median_ms": per[len(per) // 2], "max_ms": per[-1],
             "max_over_median": per[-1] / per[len(per) // 2],
             "allocator": {"segments_allocated_during_timed_steps": after.get("num_device_alloc", 0) - before.get("num_device_alloc", 0),
                           "alloc_retries_during_timed_steps": after.get("num_alloc_retries", 0) - before.get("num_alloc_retries", 0),
@@ -362,6 +371,56 @@ def standalone_hbm(torch, native, iters=24):
     return out
 
 
+def attention_projections(torch, steps=8, warmup=3):
+    """configs[1] of BASELINE.json as it is written: ONE X [8192, 4096] feeds Wq [4096, 4096], Wk and Wv [1024, 4096]
+    (optimus_dl/modules/model/blocks/attention.py:317-319), Wo [4096, 4096] has an input of its own; forward + backward
+    of all four, weights re-quantised every step.  The transform groups q / k / v as it does in a model: X is quantised
+    once, and the three data gradients are summed by the GEMMs (the `accumulate` flag) into one dX."""
+    import torch.nn as nn
+
+    from optimus_dl_amd.modules.amp import create_fp8_recipe
+    from optimus_dl_amd.modules.model_transforms import build_model_transform
+
+    class Projections(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.wq, self.wk, self.wv = nn.Linear(4096, 4096, bias=False), nn.Linear(4096, 1024, bias=False), nn.Linear(4096, 1024, bias=False)
+            self.wo = nn.Linear(4096, 4096, bias=False)
+
+        def forward(self, x, o):
+            return self.wq(x), self.wk(x), self.wv(x), self.wo(o)
+
+    m = 8192
+    g = torch.Generator().manual_seed(0)
+    net = Projections().to("cuda", torch.bfloat16)
+    with torch.no_grad():
+        for p in net.parameters():
+            p.copy_((torch.randn(p.shape, generator=g) * 0.02).bfloat16())
+    build_model_transform({"_name": "fp8_linear"}).apply(net)
+    recipe = create_fp8_recipe("tensorwise", "hybrid")
+    x = torch.randn(m, 4096, generator=g).bfloat16().cuda().requires_grad_(True)
+    o = torch.randn(m, 4096, generator=g).bfloat16().cuda().requires_grad_(True)
+    dys = [(torch.randn(m, n, generator=g) * 1e-3).bfloat16().cuda() for n in (4096, 1024, 1024, 4096)]
+    mods = [net.wq, net.wk, net.wv, net.wo]
+
+    def one():
+        for lin in mods:
+            lin._wcache.key = None
+            lin.weight.grad = None
+        x.grad = o.grad = None
+        with recipe.autocast():
+            ys = net(x, o)
+        with recipe.backward():
+            torch.autograd.backward(ys, dys)
+
+    t = timed_steps(torch, one, steps, warmup)
+    flop = sum(6.0 * m * lin.in_features * lin.out_features for lin in mods)
+    res = {"configs[1] attention projections, tensorwise": {**t, "TFLOP/s": flop / (t["ms_per_step"] * 1e-3) / 1e12, "flop_per_step": flop}}
+    del net, x, o, dys, one
+    torch.cuda.empty_cache()
+    return res
+
+
 def other_configs(torch, steps=8, warmup=3, only=""):
     """Whole steps (forward + backward of every Linear, weights re-quantised every step) of the other
     configurations of BASELINE.json and of configuration 3 with fp32 master weights (the reference's
@@ -379,9 +438,13 @@ def other_configs(torch, steps=8, warmup=3, only=""):
         ("configs[4] delayed H=16, Llama-3-70B MLP up/down", "delayed", {"amax_history_len": 16}, [(8192, 28672), (28672, 8192)], 8192, torch.bfloat16),
     ]
     out = {}
+    if not only or only in "configs[1] attention projections, tensorwise":
+        out.update(attention_projections(torch, steps, warmup))
     for label, kind, kw, shapes, m, wdtype in cases:
         if only and only not in label:
             continue
+        if label.startswith("configs[1]"):
+            label += ", as four independent Linears (an X each)"
         recipe = create_fp8_recipe(kind, "hybrid", **kw)
         g = torch.Generator().manual_seed(0)
         mods, xs, dys = [], [], []
@@ -797,16 +860,18 @@ def main() -> int:
             gbps = ks[name]["work"] / (ks[name]["total_ms"] * 1e-3) / 1e9
             hbm[name] = {"achieved": gbps, "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": gbps / PEAK_HBM_GBPS,
                          "avg_us": ks[name]["avg_us"], "launches": ks[name]["launches"]}
-    # the same kernels by the tracked profile's kernel durations (what rocprofv3 saw inside the step on the box it ran on)
+    # for orientation, what the same kernels took inside the step in the tracked rocprofv3 run (kernel time only: no launch
+    # gap, no event).  These are CONSTANTS read from a committed file, made on another box at another time; nothing in
+    # `tracked_profile_reference` is measured by this run, and no figure of this run is derived from it.
     prof_us, prof_src = profiled_kernel_durations()
-    prof_bytes = prof_time = 0.0
-    for name in hbm:
-        if name in prof_us:
-            per_launch = ks[name]["work"] / ks[name]["launches"]
-            hbm[name]["by_profiled_kernel_time"] = {"avg_us": prof_us[name], "GB/s": per_launch / (prof_us[name] * 1e-6) / 1e9,
-                                                    "frac": per_launch / (prof_us[name] * 1e-6) / 1e9 / PEAK_HBM_GBPS}
-            prof_bytes += ks[name]["work"]
-            prof_time += prof_us[name] * 1e-6 * ks[name]["launches"]
+    tracked_reference = None
+    if prof_us:
+        tracked_reference = {"not_measured_by_this_run": True, "source": prof_src, "kernel_avg_us": {}}
+        for name in hbm:
+            if name in prof_us:
+                per_launch = ks[name]["work"] / ks[name]["launches"]
+                tracked_reference["kernel_avg_us"][name] = {"avg_us": prof_us[name],
+                                                            "frac_of_hbm_peak_at_this_run_s_bytes": per_launch / (prof_us[name] * 1e-6) / 1e9 / PEAK_HBM_GBPS}
     quant_bytes = sum(ks[n]["work"] for n in ("amax", "cast", "cast_transpose") if n in ks)
     quant_ms = sum(ks[n]["total_ms"] for n in ("amax", "cast", "cast_transpose") if n in ks)
 
@@ -834,8 +899,7 @@ def main() -> int:
         "gemm_only_tflops": gemm_tflops,
         "cast_amax_gbps": quant_bytes / (quant_ms * 1e-3) / 1e9 if quant_ms else None,
         "cast_amax_frac_of_hbm_peak": (quant_bytes / (quant_ms * 1e-3) / 1e9) / PEAK_HBM_GBPS if quant_ms else None,
-        "cast_amax_frac_of_hbm_peak_by_profiled_kernel_time": (prof_bytes / prof_time / 1e9 / PEAK_HBM_GBPS) if prof_time else None,
-        "profiled_kernel_time_source": prof_src,
+        "tracked_profile_reference": tracked_reference,
         "time_split_ms_per_step": {n: ks[n]["total_ms"] / args.steps for n in ks},
         "ms_per_step_with_kernel_events": 1e3 * wall_instrumented / args.steps,
         "roofline": {
