@@ -516,8 +516,12 @@ __device__ __forceinline__ void record_scale_inv(float s, float *__restrict__ sc
 }
 
 // ------------------------------------------------------------------------ cast
-// 16 elements per lane per step: two (bf16) or four (fp32) 16-byte loads, one
-// 16-byte store.  cols % 16 == 0 and 16-byte aligned pointers (host-checked).
+// A wave works on spans of 1024 elements: VP load instructions, each of which has the 64 lanes read 1024 contiguous
+// bytes (lane l takes the 16-byte piece h * 64 + l of the span with instruction h), one store per piece.  A lane
+// that instead read its 16 elements as neighbouring 16-byte pieces would leave every instruction a half (bf16) or a
+// quarter (fp32) of each 64-byte request, and non-temporal loads are not merged across instructions: fp32 sources ran
+// at 0.49 of the HBM peak that way (4096 x 14336, bf16 0.68).  cols % 16 == 0 and 16-byte aligned pointers
+// (host-checked), so a piece never crosses a row.
 template <int SRC, int FMT, int MODE, bool AMAX>
 __global__ __launch_bounds__(AMAX ? kFatThreads : kThreads) void cast_kernel(const void *__restrict__ x, int64_t rows, int64_t cols,
                                                          const float *__restrict__ scale, uint8_t *__restrict__ out,
@@ -525,9 +529,7 @@ __global__ __launch_bounds__(AMAX ? kFatThreads : kThreads) void cast_kernel(con
                                                          int amax_mask) {
     constexpr int kT = AMAX ? kFatThreads : kThreads;
     __shared__ uint32_t red[kT / kWave];
-    const int64_t cpr = cols / 16;                           // chunks per row
-    const int64_t nchunk = rows * cpr;
-    const int64_t stride = (int64_t)gridDim.x * kT;
+    const int64_t n = rows * cols;
     float s_t = 1.0f;
     if constexpr (MODE == ODL_SCALE_TENSOR) {
         s_t = scale[0];
@@ -535,63 +537,81 @@ __global__ __launch_bounds__(AMAX ? kFatThreads : kThreads) void cast_kernel(con
     }
     if constexpr (MODE == kScaleParts) s_t = dynamic_scale<FMT>(scale, margin, dyn_out, red, blockIdx.x == 0);
     uint32_t am = 0;
-    constexpr int VP = SRC == ODL_BF16 ? 2 : 4;              // 16-byte loads per chunk of 16 elements
-    constexpr int U = SRC == ODL_BF16 ? 2 : 1;               // chunks in flight per lane
-    auto one = [&](const int64_t i, const u32x4 (&v)[VP]) {
-        float f[16];
+    constexpr int VP = SRC == ODL_BF16 ? 2 : 4;              // 16-byte pieces per lane and span
+    constexpr int EPP = SRC == ODL_BF16 ? 8 : 4;             // elements per piece
+    constexpr int U = SRC == ODL_BF16 ? 2 : 1;               // spans in flight per wave
+    const int lane = threadIdx.x % kWave;
+    // one piece: EPP elements from element index e on
+    auto one = [&](const int64_t e, const u32x4 v) {
+        float f[8];
         if constexpr (SRC == ODL_BF16) {
-            const uint32_t w[8] = {v[0].x, v[0].y, v[0].z, v[0].w, v[1].x, v[1].y, v[1].z, v[1].w};
+            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-            for (int q = 0; q < 8; ++q) {
+            for (int q = 0; q < 4; ++q) {
                 f[2 * q] = bf16_lo(w[q]);
                 f[2 * q + 1] = bf16_hi(w[q]);
                 if constexpr (AMAX) am = max_u16x2(am, abs_bf16x2(w[q]));
             }
         } else {
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                f[4 * u] = bits_to_float(v[u].x); f[4 * u + 1] = bits_to_float(v[u].y);
-                f[4 * u + 2] = bits_to_float(v[u].z); f[4 * u + 3] = bits_to_float(v[u].w);
-                if constexpr (AMAX) am = max(am, max(max(v[u].x & 0x7fffffffu, v[u].y & 0x7fffffffu),
-                                                     max(v[u].z & 0x7fffffffu, v[u].w & 0x7fffffffu)));
-            }
+            f[0] = bits_to_float(v.x); f[1] = bits_to_float(v.y); f[2] = bits_to_float(v.z); f[3] = bits_to_float(v.w);
+            f[4] = f[5] = f[6] = f[7] = 0.0f;
+            if constexpr (AMAX) am = max(am, max(max(v.x & 0x7fffffffu, v.y & 0x7fffffffu), max(v.z & 0x7fffffffu, v.w & 0x7fffffffu)));
         }
-        float s[16];
+        float sc[8];
         if constexpr (MODE == ODL_SCALE_TENSOR || MODE == kScaleParts) {
 #pragma unroll
-            for (int j = 0; j < 16; ++j) s[j] = s_t;
+            for (int j = 0; j < 8; ++j) sc[j] = s_t;
         } else if constexpr (MODE == ODL_SCALE_ROW) {
-            const float sr = scale[i / cpr];
+            const float sr = scale[e / cols];
 #pragma unroll
-            for (int j = 0; j < 16; ++j) s[j] = sr;
+            for (int j = 0; j < 8; ++j) sc[j] = sr;
         } else {
-            const float4 *sp = reinterpret_cast<const float4 *>(scale + (i % cpr) * 16);
+            const float4 *sp = reinterpret_cast<const float4 *>(scale + e % cols);
 #pragma unroll
-            for (int u = 0; u < 4; ++u) { float4 t = sp[u]; s[4 * u] = t.x; s[4 * u + 1] = t.y; s[4 * u + 2] = t.z; s[4 * u + 3] = t.w; }
+            for (int u = 0; u < EPP / 4; ++u) { float4 t = sp[u]; sc[4 * u] = t.x; sc[4 * u + 1] = t.y; sc[4 * u + 2] = t.z; sc[4 * u + 3] = t.w; }
         }
-        u32x4 o;
-        o.x = quantise4<FMT>(f[0], f[1], f[2], f[3], s[0], s[1], s[2], s[3]);
-        o.y = quantise4<FMT>(f[4], f[5], f[6], f[7], s[4], s[5], s[6], s[7]);
-        o.z = quantise4<FMT>(f[8], f[9], f[10], f[11], s[8], s[9], s[10], s[11]);
-        o.w = quantise4<FMT>(f[12], f[13], f[14], f[15], s[12], s[13], s[14], s[15]);
-        ODL_CODE_STORE(o, reinterpret_cast<u32x4 *>(out) + i);
+        const uint32_t lo = quantise4<FMT>(f[0], f[1], f[2], f[3], sc[0], sc[1], sc[2], sc[3]);
+        if constexpr (SRC == ODL_BF16) {
+            const uint32_t hi = quantise4<FMT>(f[4], f[5], f[6], f[7], sc[4], sc[5], sc[6], sc[7]);
+            ODL_CODE_STORE((u32x2{lo, hi}), reinterpret_cast<u32x2 *>(out + e));
+        } else {
+            ODL_CODE_STORE(lo, reinterpret_cast<uint32_t *>(out + e));
+        }
     };
-    const u32x4 *px = reinterpret_cast<const u32x4 *>(x);
-    int64_t i = (int64_t)blockIdx.x * kT + threadIdx.x;
-    for (; i + (U - 1) * stride < nchunk; i += U * stride) {
+    const char *px = reinterpret_cast<const char *>(x);
+    constexpr int ESZ = SRC == ODL_BF16 ? 2 : 4;
+    const int64_t nspan = (n + 1023) / 1024;
+    const int64_t stride = (int64_t)gridDim.x * (kT / kWave);
+    int64_t sp = (int64_t)blockIdx.x * (kT / kWave) + threadIdx.x / kWave;
+    for (; sp + (U - 1) * stride < nspan; sp += U * stride) {
         u32x4 v[U][VP];
 #pragma unroll
         for (int u = 0; u < U; ++u)
 #pragma unroll
-            for (int h = 0; h < VP; ++h) v[u][h] = __builtin_nontemporal_load(px + (i + u * stride) * VP + h);
+            for (int h = 0; h < VP; ++h) {
+                const int64_t e = (sp + u * stride) * 1024 + (h * kWave + lane) * EPP;
+                v[u][h] = e < n ? __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(px + e * ESZ)) : u32x4{0, 0, 0, 0};
+            }
 #pragma unroll
-        for (int u = 0; u < U; ++u) one(i + u * stride, v[u]);
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int h = 0; h < VP; ++h) {
+                const int64_t e = (sp + u * stride) * 1024 + (h * kWave + lane) * EPP;
+                if (e < n) one(e, v[u][h]);
+            }
     }
-    for (; i < nchunk; i += stride) {
+    for (; sp < nspan; sp += stride) {
         u32x4 v[VP];
 #pragma unroll
-        for (int h = 0; h < VP; ++h) v[h] = __builtin_nontemporal_load(px + i * VP + h);
-        one(i, v);
+        for (int h = 0; h < VP; ++h) {
+            const int64_t e = sp * 1024 + (h * kWave + lane) * EPP;
+            v[h] = e < n ? __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(px + e * ESZ)) : u32x4{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int h = 0; h < VP; ++h) {
+            const int64_t e = sp * 1024 + (h * kWave + lane) * EPP;
+            if (e < n) one(e, v[h]);
+        }
     }
     if constexpr (AMAX) {
         if constexpr (SRC == ODL_BF16) am = fold_u16x2_to_f32bits(am);

@@ -210,6 +210,56 @@ def test_amax_parts_colsum(N, shape, dtype):
     assert torch.equal(colsum, again)                               # reproducible
 
 
+def colsum_in_kernel_order(x):
+    """The column sums as the kernel forms them, one fp32 addition at a time: per slab of rows, 32 row-lanes each add
+    rows ty, ty + 32, ... in order; the row-lanes are added in order; 16 groups add every 16th slab in order; the
+    groups are added in order."""
+    rows, cols = x.shape
+    cpl = 8 if x.dtype == torch.bfloat16 else 4
+    col_blocks = -(-cols // (32 * cpl))
+    slabs = 512 // col_blocks
+    rpb = -(-(-(-rows // slabs)) // 32) * 32
+    slabs = -(-rows // rpb)
+    xf = x.float()
+    slab_sums = []
+    for s in range(slabs):
+        part = xf[s * rpb:min(rows, (s + 1) * rpb)]
+        pad = (-part.shape[0]) % 32
+        if pad:
+            part = torch.cat([part, torch.zeros((pad, cols))])           # acc + 0.0 == acc
+        part = part.reshape(-1, 32, cols)
+        acc = torch.zeros((32, cols))
+        for it in range(part.shape[0]):
+            acc = acc + part[it]
+        t = acc[0]
+        for y in range(1, 32):
+            t = t + acc[y]
+        slab_sums.append(t)
+    groups = []
+    for g in range(16):
+        a = torch.zeros(cols)
+        for b in range(g, slabs, 16):
+            a = a + slab_sums[b]
+        groups.append(a)
+    t = groups[0]
+    for g in range(1, 16):
+        t = t + groups[g]
+    return t
+
+
+@pytest.mark.parametrize("shape", [(33, 256), (1000, 264), (4096, 768), (2000, 3072)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_amax_parts_colsum_adds_in_the_documented_order(N, shape, dtype):
+    """The sum is not just reproducible: it is this sequence of fp32 additions, restated here one addition at a time."""
+    x = seeded_bf16(shape, 1.0, 7 + sum(shape)).to(dtype)
+    if dtype == torch.float32:
+        x = x * 1.00390625 + 3e-4                                        # mantissas that do not fit bf16
+    want = colsum_in_kernel_order(x)
+    for _ in range(3):
+        _, colsum = N.amax_parts_colsum(x.cuda())
+        assert_f32_bits_equal(colsum, want, f"colsum order {shape} {dtype}")
+
+
 def test_amax_parts_colsum_exact_and_refusals(N):
     # integers: every partial sum is exact, so the result is too, whatever the order
     rows, cols = 515, 264
