@@ -28,7 +28,9 @@ __device__ __forceinline__ void ct_tile_of(int64_t id, int64_t tiles_r, int64_t 
 //   * the dword writes of a half-wave (8 column groups x 4 consecutive row groups) differ mod 32,
 //   * the 16-byte reads stay aligned (ds_read_b128), and 16 consecutive lanes read one whole line.
 // Offsets in bytes; `ty` is the lane's group of 4 rows (0..31), `m16` a chunk of 16 rows (0..7).
-__device__ __forceinline__ int ct_lds_rot(int col) { return 4 * (col >> 3); }
+// (the second term separates lanes whose columns 4 tx + k share col >> 3, the layout of an fp32 source; where a lane's
+// columns are 8 tx + k it is the same for all lanes of an instruction)
+__device__ __forceinline__ int ct_lds_rot(int col) { return 4 * (col >> 3) + 16 * ((col >> 2) & 1); }
 __device__ __forceinline__ int ct_lds_write_off(int col, int ty) {
     return (col >> 1) * 256 + ((((col & 1) * 32) + ty + ct_lds_rot(col)) & 63) * 4;
 }

@@ -131,9 +131,11 @@ __device__ __forceinline__ uint32_t cvt_scaled4(uint32_t p0, uint32_t p1, uint32
     }
 }
 
-// 128 x 64 tile per block of 256 lanes, lane (tx, ty) owns rows 4 ty .. 4 ty + 3 and columns 8 tx .. 8 tx + 7 as in
-// cast_transpose_kernel.  A block along the columns (32 of them) is held by 4 neighbouring lanes; a block along the rows
-// (32 of them) by the 8 lanes of a wave that share tx: both maxima are xor-shuffles inside the wave.
+// 128 x 64 tile per block of 256 lanes, lane (tx, ty) owns rows 4 ty .. 4 ty + 3 and two groups of 4 columns as in
+// cast_transpose_kernel: bf16 source, columns 8 tx .. 8 tx + 7, so a block along the columns (32 of them) is held by 4
+// neighbouring lanes; fp32 source, columns 4 tx .. + 3 and 32 + 4 tx .. + 3 (every load instruction contiguous over the
+// 8 lanes of a row), so the first groups of the 8 lanes are one block and the second groups the other.  A block along
+// the rows (32 of them) is held by the 8 lanes of a wave that share tx.  All maxima are exchanges inside the wave.
 template <int SRC, int FMT, bool WANT_ROW, bool WANT_COL>
 __global__ __launch_bounds__(kMxThreads) void mx_cast_kernel(const void *__restrict__ x, int64_t rows, int64_t cols,
                                                               uint8_t *__restrict__ out, uint8_t *__restrict__ scales,
@@ -154,8 +156,11 @@ __global__ __launch_bounds__(kMxThreads) void mx_cast_kernel(const void *__restr
     const bool staged_t = WANT_COL && layout_t == ODL_MX_SCALES_KSTEP;
     int64_t tr, tc;
     ct_tile_of(blockIdx.x, tiles_r, tiles_c, tr, tc);
-    const int64_t r0 = tr * kTileR + ty * 4, c0 = tc * kTileC + tx * 8;
-    const bool col_ok = c0 < cols;                 // cols % 8 == 0 (host-checked)
+    const int kA = SRC == ODL_BF16 ? tx * 8 : tx * 4, kB = SRC == ODL_BF16 ? tx * 8 + 4 : 32 + tx * 4;   // tile columns of the two groups
+    const int64_t r0 = tr * kTileR + ty * 4, cA = tc * kTileC + kA, cB = tc * kTileC + kB;
+    // cols % 32 == 0 where codes along the rows are wanted, % 8 otherwise (host-checked): a group of 4 is in or out as a whole
+    const bool okA = cA < cols, okB = cB < cols;
+    [[maybe_unused]] auto col_of = [&](int j) { return j < 4 ? cA + j : cB + j - 4; };      // matrix column of the lane's column j
 
     // The patch stays in registers as loaded (bf16: 4 dwords a row) and is widened row by row where it is used; magnitudes
     // of bf16 pairs are compared as packed 16-bit integers, two columns at a time.
@@ -163,11 +168,12 @@ __global__ __launch_bounds__(kMxThreads) void mx_cast_kernel(const void *__restr
     uint32_t raw[4][DW];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const bool ok = col_ok && (r0 + i) < rows;
-        const u32x4 *p = reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(x) + ((r0 + i) * cols + c0) * ESZ);
+        const bool row_ok = (r0 + i) < rows;
+        const char *row = reinterpret_cast<const char *>(x) + (r0 + i) * cols * ESZ;
 #pragma unroll
         for (int h = 0; h < DW / 4; ++h) {
-            const u32x4 v = ok ? __builtin_nontemporal_load(p + h) : u32x4{0, 0, 0, 0};
+            const bool ok = row_ok && (h == 0 ? okA : okB);
+            const u32x4 v = ok ? __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(row + (h == 0 ? cA : cB) * ESZ)) : u32x4{0, 0, 0, 0};
             raw[i][4 * h] = v.x; raw[i][4 * h + 1] = v.y; raw[i][4 * h + 2] = v.z; raw[i][4 * h + 3] = v.w;
         }
     }
@@ -184,43 +190,57 @@ __global__ __launch_bounds__(kMxThreads) void mx_cast_kernel(const void *__restr
         uint32_t row_pairs[2] = {0u, 0u};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            uint32_t m = 0;
+            // m / byte / mul: of the block that holds the lane's first group; m_b / byte_b / mul_b: of its second group's
+            uint32_t m = 0, m_b = 0;
             if constexpr (SRC == ODL_BF16) {
                 uint32_t m2 = max_u16x2(max_u16x2(abs_bf16x2(raw[i][0]), abs_bf16x2(raw[i][1])), max_u16x2(abs_bf16x2(raw[i][2]), abs_bf16x2(raw[i][3])));
-                m = fold_u16x2_to_f32bits(m2);
+                m = max_quad(fold_u16x2_to_f32bits(m2));                 // the 4 lanes tx = 4 b .. 4 b + 3 hold the block
+                m_b = m;
             } else {
 #pragma unroll
-                for (int j = 0; j < 8; ++j) m = max(m, raw[i][j] & 0x7fffffffu);
+                for (int j = 0; j < 4; ++j) { m = max(m, raw[i][j] & 0x7fffffffu); m_b = max(m_b, raw[i][4 + j] & 0x7fffffffu); }
+                m = max_with_dpp<0x141>(max_quad(m));                    // all 8 lanes of the row (row_half_mirror joins the quads)
+                m_b = max_with_dpp<0x141>(max_quad(m_b));
             }
-            m = max_quad(m);                                             // the 4 lanes tx = 4 b .. 4 b + 3 hold the block
-            uint32_t byte;
-            float mul;
+            uint32_t byte, byte_b;
+            float mul, mul_b;
             mx_scale_of<FMT>(m, rule, byte, mul);
-            if (col_ok && (r0 + i) < rows) {
+            if constexpr (SRC == ODL_BF16) { byte_b = byte; mul_b = mul; }
+            else mx_scale_of<FMT>(m_b, rule, byte_b, mul_b);
+            if ((r0 + i) < rows) {
                 uint32_t lo, hi;
-                if (__builtin_expect(m >= 0x7f800000u, 0)) {            // only a block whose amax is Inf / NaN can hold a NaN
+                if (__builtin_expect(max(m, m_b) >= 0x7f800000u, 0)) {  // only a block whose amax is Inf / NaN can hold a NaN
                     float f[8];
                     widen(i, f);
                     lo = quantise4<FMT>(f[0], f[1], f[2], f[3], mul, mul, mul, mul);
-                    hi = quantise4<FMT>(f[4], f[5], f[6], f[7], mul, mul, mul, mul);
+                    hi = quantise4<FMT>(f[4], f[5], f[6], f[7], mul_b, mul_b, mul_b, mul_b);
                 } else {                                                // the hardware divides by 2^(byte - 127) and saturates
-                    const float e8 = bits_to_float(byte << 23);
+                    const float e8 = bits_to_float(byte << 23), e8_b = bits_to_float(byte_b << 23);
                     if constexpr (SRC == ODL_BF16) {
                         lo = cvt_scaled4<SRC, FMT>(raw[i][0], raw[i][1], 0u, 0u, e8);
                         hi = cvt_scaled4<SRC, FMT>(raw[i][2], raw[i][3], 0u, 0u, e8);
                     } else {
                         lo = cvt_scaled4<SRC, FMT>(raw[i][0], raw[i][1], raw[i][2], raw[i][3], e8);
-                        hi = cvt_scaled4<SRC, FMT>(raw[i][4], raw[i][5], raw[i][6], raw[i][7], e8);
+                        hi = cvt_scaled4<SRC, FMT>(raw[i][4], raw[i][5], raw[i][6], raw[i][7], e8_b);
                     }
                 }
-                *reinterpret_cast<u32x2 *>(out + (r0 + i) * cols + c0) = u32x2{lo, hi};
+                if constexpr (SRC == ODL_BF16) {
+                    if (okA) *reinterpret_cast<u32x2 *>(out + (r0 + i) * cols + cA) = u32x2{lo, hi};
+                } else {
+                    if (okA) *reinterpret_cast<uint32_t *>(out + (r0 + i) * cols + cA) = lo;
+                    if (okB) *reinterpret_cast<uint32_t *>(out + (r0 + i) * cols + cB) = hi;
+                }
                 if (staged_r) {
-                    // both bytes of the row in one lane: row_shl:4 hands lane l the value of lane l + 4, which holds the
-                    // row's second block; the lane's four rows then go to LDS as one 8-byte write
-                    const uint32_t second = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)byte, 0x104, 0xf, 0xf, false);
+                    // both bytes of the row in one lane (bf16: row_shl:4 hands lane l the value of lane l + 4, which holds
+                    // the row's second block); the lane's four rows then go to LDS as one 8-byte write
+                    uint32_t second = byte_b;
+                    if constexpr (SRC == ODL_BF16) second = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)byte, 0x104, 0xf, 0xf, false);
                     row_pairs[i / 2] |= (byte | (second << 8)) << (16 * (i & 1));
-                } else if ((tx & 3) == 0) {
-                    scales[mx_scale_at(layout, r0 + i, c0 / kMxBlock, rows, nb)] = (uint8_t)byte;
+                } else if constexpr (SRC == ODL_BF16) {
+                    if ((tx & 3) == 0 && okA) scales[mx_scale_at(layout, r0 + i, cA / kMxBlock, rows, nb)] = (uint8_t)byte;
+                } else if (tx == 0) {
+                    if (okA) scales[mx_scale_at(layout, r0 + i, cA / kMxBlock, rows, nb)] = (uint8_t)byte;
+                    if (okB) scales[mx_scale_at(layout, r0 + i, cB / kMxBlock, rows, nb)] = (uint8_t)byte_b;
                 }
             }
         }
@@ -252,11 +272,14 @@ __global__ __launch_bounds__(kMxThreads) void mx_cast_kernel(const void *__restr
             e8_c[j] = bits_to_float(byte << 23);
             // rows % 32 == 0 (host-checked): a row block is inside the matrix as a whole or not at all
             col_bytes[j / 4] |= byte << (8 * (j % 4));
-            if (!staged_t && (ty & 7) == 0 && col_ok && r0 < rows)
-                scales_t[mx_scale_at(layout_t, c0 + j, r0 / kMxBlock, cols, nbt)] = (uint8_t)byte;
+            if (!staged_t && (ty & 7) == 0 && (j < 4 ? okA : okB) && r0 < rows)
+                scales_t[mx_scale_at(layout_t, col_of(j), r0 / kMxBlock, cols, nbt)] = (uint8_t)byte;
         }
-        // staged: the wave's row block is one plane of 64 bytes, a lane's 8 columns one 8-byte write
-        if (staged_t && (ty & 7) == 0) *reinterpret_cast<u32x2 *>(&stage_t[(ty / 8) * kTileC + tx * 8]) = u32x2{col_bytes[0], col_bytes[1]};
+        // staged: the wave's row block is one plane of 64 bytes, a lane's two groups of 4 columns a 4-byte write each
+        if (staged_t && (ty & 7) == 0) {
+            *reinterpret_cast<uint32_t *>(&stage_t[(ty / 8) * kTileC + kA]) = col_bytes[0];
+            *reinterpret_cast<uint32_t *>(&stage_t[(ty / 8) * kTileC + kB]) = col_bytes[1];
+        }
         uint32_t worst = 0;                                              // Inf / NaN in any of the lane's 8 column blocks?
 #pragma unroll
         for (int j = 0; j < 8; ++j) worst = max(worst, cmax[j]);
@@ -291,8 +314,8 @@ __global__ __launch_bounds__(kMxThreads) void mx_cast_kernel(const void *__restr
         }
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
-            *reinterpret_cast<uint32_t *>(&tile[ct_lds_write_off(tx * 8 + k, ty)]) = tl[k];
-            *reinterpret_cast<uint32_t *>(&tile[ct_lds_write_off(tx * 8 + 4 + k, ty)]) = th[k];
+            *reinterpret_cast<uint32_t *>(&tile[ct_lds_write_off(kA + k, ty)]) = tl[k];
+            *reinterpret_cast<uint32_t *>(&tile[ct_lds_write_off(kB + k, ty)]) = th[k];
         }
         __syncthreads();
 #pragma unroll

@@ -647,9 +647,12 @@ __global__ __launch_bounds__(kThreads) void cast_generic_kernel(const void *__re
 }
 
 // -------------------------------------------------------------- cast+transpose
-// Tile = 128 rows x 64 cols of x per block of 256 lanes.  A lane owns a 4 x 8
-// patch: four 16-byte (bf16) loads, one per row.  The row-major codes leave as
-// 8-byte stores (a wave covers whole 64-byte row segments); the transposed codes
+// Tile = 128 rows x 64 cols of x per block of 256 lanes.  A lane owns 4 rows x 8 columns: bf16 source, columns
+// 8 tx .. 8 tx + 7 (one 16-byte load a row); fp32 source, columns 4 tx .. 4 tx + 3 and 32 + 4 tx .. 32 + 4 tx + 3 (two
+// loads a row, each of which has the 8 lanes of a row read 128 contiguous bytes: non-temporal loads are not merged
+// across instructions, and with a lane's 32 bytes side by side every instruction used half of each 64-byte request;
+// 4096 x 14336 fp32 ran at 0.55 of the HBM peak that way).  The row-major codes leave as
+// 8-byte (fp32 source: two 4-byte) stores (a wave covers whole 64-byte row segments); the transposed codes
 // go through a 4x4 byte transpose in registers (v_perm_b32) and an LDS tile
 // [64 cols][128 rows] so that they leave as 16-byte stores along the row axis:
 // both outputs are written in full 64/128-byte segments.  (Tile helpers: ct_tile.h.)
@@ -657,6 +660,35 @@ __global__ __launch_bounds__(kThreads) void cast_generic_kernel(const void *__re
 // One 128 x 64 tile (tr, tc) of x: convert, write the row-major codes, transpose through `tile` (LDS), write the
 // transposed codes.  `st` is the per-tensor scale (modes TENSOR and parts), `scale` the vector of the ROW / COL modes.
 // Ends after the transposed stores: a caller that reuses `tile` puts a barrier in between.
+// first tile column of the lane's group g (0 / 1) of 4 columns
+template <int SRC>
+__device__ __forceinline__ int ct_group_col(int tx, int g) { return SRC == ODL_BF16 ? tx * 8 + 4 * g : tx * 4 + 32 * g; }
+
+// the lane's 8 elements of row r: columns cA .. cA + 3 and cB .. cB + 3 (bf16: cB = cA + 4, one load)
+template <int SRC>
+__device__ __forceinline__ void ct_load_row(const void *__restrict__ x, int64_t r, int64_t rows, int64_t cols, int64_t cA, int64_t cB,
+                                            bool okA, bool okB, u32x4 (&raw)[SRC == ODL_BF16 ? 1 : 2]) {
+    constexpr int ESZ = SRC == ODL_BF16 ? 2 : 4;
+    const bool row_ok = r < rows;
+    const char *row = reinterpret_cast<const char *>(x) + r * cols * ESZ;
+    raw[0] = (okA && row_ok) ? __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(row + cA * ESZ)) : u32x4{0, 0, 0, 0};
+    if constexpr (SRC != ODL_BF16)
+        raw[1] = (okB && row_ok) ? __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(row + cB * ESZ)) : u32x4{0, 0, 0, 0};
+}
+
+// the lane's 8 row-major codes of row r
+template <int SRC>
+__device__ __forceinline__ void ct_store_row(uint8_t *__restrict__ out, int64_t r, int64_t rows, int64_t cols, int64_t cA, int64_t cB,
+                                             bool okA, bool okB, uint32_t lo, uint32_t hi) {
+    if (r >= rows) return;
+    if constexpr (SRC == ODL_BF16) {
+        if (okA) ODL_CODE_STORE((u32x2{lo, hi}), reinterpret_cast<u32x2 *>(out + r * cols + cA));
+    } else {
+        if (okA) ODL_CODE_STORE(lo, reinterpret_cast<uint32_t *>(out + r * cols + cA));
+        if (okB) ODL_CODE_STORE(hi, reinterpret_cast<uint32_t *>(out + r * cols + cB));
+    }
+}
+
 template <int SRC, int FMT, int MODE, bool AMAX, bool WRITE_ROWMAJOR>
 __device__ __forceinline__ void ct_one_tile(const void *__restrict__ x, int64_t rows, int64_t cols, const float *__restrict__ scale,
                                             float st, uint8_t *__restrict__ out, uint8_t *__restrict__ out_t, int64_t tr,
@@ -664,8 +696,10 @@ __device__ __forceinline__ void ct_one_tile(const void *__restrict__ x, int64_t 
     constexpr int ESZ = SRC == ODL_BF16 ? 2 : 4;
     const int tx = threadIdx.x % 8;                 // 8 lanes across 64 columns
     const int ty = threadIdx.x / 8;                 // 32 lane-rows, 4 rows each
-    const int64_t r0 = tr * kTileR + ty * 4, c0 = tc * kTileC + tx * 8;
-    const bool col_ok = c0 < cols;                  // cols % 8 == 0 (host-checked), so the whole 8-wide patch is in or out
+    // tile columns of the lane's two groups of 4 (codes lo / hi below)
+    const int kA = ct_group_col<SRC>(tx, 0), kB = ct_group_col<SRC>(tx, 1);
+    const int64_t r0 = tr * kTileR + ty * 4, cA = tc * kTileC + kA, cB = tc * kTileC + kB;
+    const bool okA = cA < cols, okB = cB < cols;    // cols % 8 == 0 (host-checked), so a group of 4 is in or out as a whole
 
     float s_col[8];
 #pragma unroll
@@ -674,9 +708,12 @@ __device__ __forceinline__ void ct_one_tile(const void *__restrict__ x, int64_t 
 #pragma unroll
         for (int j = 0; j < 8; ++j) s_col[j] = st;
     } else if constexpr (MODE == ODL_SCALE_COL) {
-        if (col_ok) {
-            float4 t0 = *reinterpret_cast<const float4 *>(scale + c0), t1 = *reinterpret_cast<const float4 *>(scale + c0 + 4);
+        if (okA) {
+            const float4 t0 = *reinterpret_cast<const float4 *>(scale + cA);
             s_col[0] = t0.x; s_col[1] = t0.y; s_col[2] = t0.z; s_col[3] = t0.w;
+        }
+        if (okB) {
+            const float4 t1 = *reinterpret_cast<const float4 *>(scale + cB);
             s_col[4] = t1.x; s_col[5] = t1.y; s_col[6] = t1.z; s_col[7] = t1.w;
         }
     }
@@ -684,12 +721,7 @@ __device__ __forceinline__ void ct_one_tile(const void *__restrict__ x, int64_t 
     // ---- load the 4 x 8 patch (rows beyond the matrix read as zero)
     u32x4 raw[4][ESZ / 2];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const bool ok = col_ok && (r0 + i) < rows;
-        const u32x4 *p = reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(x) + ((r0 + i) * cols + c0) * ESZ);
-#pragma unroll
-        for (int h = 0; h < ESZ / 2; ++h) raw[i][h] = ok ? __builtin_nontemporal_load(p + h) : u32x4{0, 0, 0, 0};
-    }
+    for (int i = 0; i < 4; ++i) ct_load_row<SRC>(x, r0 + i, rows, cols, cA, cB, okA, okB, raw[i]);
 
     uint32_t lo[4], hi[4];                          // codes of columns 0..3 / 4..7 for each of the 4 rows
 #pragma unroll
@@ -722,10 +754,7 @@ __device__ __forceinline__ void ct_one_tile(const void *__restrict__ x, int64_t 
         }
         lo[i] = quantise4<FMT>(f[0], f[1], f[2], f[3], s[0], s[1], s[2], s[3]);
         hi[i] = quantise4<FMT>(f[4], f[5], f[6], f[7], s[4], s[5], s[6], s[7]);
-        if constexpr (WRITE_ROWMAJOR) {
-            if (col_ok && (r0 + i) < rows)
-                ODL_CODE_STORE((u32x2{lo[i], hi[i]}), reinterpret_cast<u32x2 *>(out + (r0 + i) * cols + c0));
-        }
+        if constexpr (WRITE_ROWMAJOR) ct_store_row<SRC>(out, r0 + i, rows, cols, cA, cB, okA, okB, lo[i], hi[i]);
     }
 
     // ---- transpose in registers, stage through LDS
@@ -734,8 +763,8 @@ __device__ __forceinline__ void ct_one_tile(const void *__restrict__ x, int64_t 
     transpose4x4(hi, th);
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
-        *reinterpret_cast<uint32_t *>(&tile[ct_lds_write_off(tx * 8 + k, ty)]) = tl[k];
-        *reinterpret_cast<uint32_t *>(&tile[ct_lds_write_off(tx * 8 + 4 + k, ty)]) = th[k];
+        *reinterpret_cast<uint32_t *>(&tile[ct_lds_write_off(kA + k, ty)]) = tl[k];
+        *reinterpret_cast<uint32_t *>(&tile[ct_lds_write_off(kB + k, ty)]) = th[k];
     }
     __syncthreads();
     // 64 tile-columns x 8 chunks of 16 rows = 512 chunks, two per lane
@@ -818,20 +847,16 @@ __global__ __launch_bounds__(kThreads) void cast_rowcol_kernel(const void *__res
         if (tr == 0 && c < cols) { s_col_out[c] = sc; s_col_inv[c] = __fdiv_rn(1.0f, sc); }
     }
     __syncthreads();
-    const int64_t r0 = tr * kTileR + ty * 4, c0 = tc * kTileC + tx * 8;
-    const bool col_ok = c0 < cols;                  // cols % 8 == 0 (host-checked)
+    const int kA = ct_group_col<SRC>(tx, 0), kB = ct_group_col<SRC>(tx, 1);     // the lane's columns, as in ct_one_tile
+    const int64_t r0 = tr * kTileR + ty * 4, cA = tc * kTileC + kA, cB = tc * kTileC + kB;
+    const bool okA = cA < cols, okB = cB < cols;    // cols % 8 == 0 (host-checked)
     float sc_col[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) sc_col[j] = s_col[tx * 8 + j];
+    for (int j = 0; j < 4; ++j) { sc_col[j] = s_col[kA + j]; sc_col[4 + j] = s_col[kB + j]; }
 
     u32x4 raw[4][ESZ / 2];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const bool ok = col_ok && (r0 + i) < rows;
-        const u32x4 *p = reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(x) + ((r0 + i) * cols + c0) * ESZ);
-#pragma unroll
-        for (int h = 0; h < ESZ / 2; ++h) raw[i][h] = ok ? __builtin_nontemporal_load(p + h) : u32x4{0, 0, 0, 0};
-    }
+    for (int i = 0; i < 4; ++i) ct_load_row<SRC>(x, r0 + i, rows, cols, cA, cB, okA, okB, raw[i]);
     uint32_t lo[4], hi[4];                          // column-scaled codes of columns 0..3 / 4..7 for each of the 4 rows
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -848,7 +873,7 @@ __global__ __launch_bounds__(kThreads) void cast_rowcol_kernel(const void *__res
         const float sr = s_row[ty * 4 + i];
         const uint32_t rlo = quantise4<FMT>(f[0], f[1], f[2], f[3], sr, sr, sr, sr);
         const uint32_t rhi = quantise4<FMT>(f[4], f[5], f[6], f[7], sr, sr, sr, sr);
-        if (col_ok && (r0 + i) < rows) ODL_CODE_STORE((u32x2{rlo, rhi}), reinterpret_cast<u32x2 *>(out + (r0 + i) * cols + c0));
+        ct_store_row<SRC>(out, r0 + i, rows, cols, cA, cB, okA, okB, rlo, rhi);
         lo[i] = quantise4<FMT>(f[0], f[1], f[2], f[3], sc_col[0], sc_col[1], sc_col[2], sc_col[3]);
         hi[i] = quantise4<FMT>(f[4], f[5], f[6], f[7], sc_col[4], sc_col[5], sc_col[6], sc_col[7]);
     }
@@ -858,8 +883,8 @@ __global__ __launch_bounds__(kThreads) void cast_rowcol_kernel(const void *__res
     transpose4x4(hi, th);
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
-        *reinterpret_cast<uint32_t *>(&tile[ct_lds_write_off(tx * 8 + k, ty)]) = tl[k];
-        *reinterpret_cast<uint32_t *>(&tile[ct_lds_write_off(tx * 8 + 4 + k, ty)]) = th[k];
+        *reinterpret_cast<uint32_t *>(&tile[ct_lds_write_off(kA + k, ty)]) = tl[k];
+        *reinterpret_cast<uint32_t *>(&tile[ct_lds_write_off(kB + k, ty)]) = th[k];
     }
     __syncthreads();
 #pragma unroll
