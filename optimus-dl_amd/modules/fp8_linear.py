@@ -231,7 +231,8 @@ class _Fp8LinearFn(torch.autograd.Function):
             # accumulate, and the detour through a workspace costs what the fusion saves: measured 500 us against
             # 475 us unfused for a 14336 x 4096 fp32 gradient, where the transposed route with the flag takes 395)
             ctx.wgrad_direct = (fp8_wgrad and recipe.direct_layouts and not recipe.fuse_wgrad_accumulation
-                                and native.gemm_layouts_supported(n_out, n_in, tokens, weight.dtype))
+                                and native.gemm_layouts_supported(n_out, n_in, tokens, weight.dtype)
+                                and native.wgrad_direct_pays(n_out, n_in, tokens))
             if pol.kind == "delayed":
                 # the histories see a forward only when it is part of training: the module in training mode AND
                 # grad mode on (the reference's backend refreshes its state on the same condition), so a validation

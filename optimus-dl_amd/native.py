@@ -952,6 +952,19 @@ def gemm_layouts_supported(M: int, N: int, K: int, out_dtype: torch.dtype = torc
             and (M + 256) * K < 2**31 and (N + 256) * K < 2**31 and N * out_dtype.itemsize * 264 < 2**31)
 
 
+def wgrad_direct_pays(n_out: int, n_in: int, tokens: int) -> bool:
+    """Whether the weight gradient [n_out, n_in] = dY^T . X is better computed from the row-major codes of dY
+    (:func:`gemm_layouts`, K-slow operand, no transposed copy of dY) than from a transposed copy with :func:`gemm_nt`.
+    The kernel that reads K-slow operands works on whole 256 x 256 tiles: it pays where those fill the chip, and for
+    small gradients, where both routes are a handful of short launches and the copy is one more.  In between it either
+    leaves compute units idle or splits the contraction and adds a reduction pass, and 128 x 128 tiles over the
+    transposed copy are faster.  Measured at 8192 tokens, cast of dY included, direct / transposed in us:
+    1024 x 4096 61.7 / 52.2, 2048 x 4096 90.3 / 81.2, 1024 x 3072 53.3 / 48.7, 3072 x 1024 68.2 / 64.6;
+    4096 x 4096 129.9 / 136.3, 2048 x 1024 54.2 / 56.2, 2304 x 768 53.8 / 58.7, 1024 x 1024 38.1 / 41.9."""
+    tiles = (n_out // 256) * (n_in // 256)
+    return tiles >= 192 or n_out * n_in < 2_200_000
+
+
 def gemm_layouts(a: torch.Tensor, b: torch.Tensor, fmt_a: int, fmt_b: int, layout_a: int, layout_b: int,
                  sa_inv: torch.Tensor, sb_inv: torch.Tensor, out: torch.Tensor | None = None,
                  out_dtype: torch.dtype = torch.bfloat16, accumulate: bool = False) -> torch.Tensor:

@@ -553,6 +553,28 @@ def test_wgrad_reads_dy_as_stored_and_matches_the_transposed_copy_route(amp, mon
         assert max_rel_err(results[True][2], ref["dw"]) <= TOL
 
 
+def test_mid_sized_weight_gradients_take_the_transposed_copy(amp, monkeypatch):
+    """A gradient whose 256 x 256 tiles neither fill the chip nor are few enough not to matter is computed from a
+    transposed copy of dy (native.wgrad_direct_pays); the two routes give the same bits."""
+    from optimus_dl_amd import native
+
+    assert native.wgrad_direct_pays(14336, 4096, 8192) and native.wgrad_direct_pays(4096, 4096, 8192)
+    assert native.wgrad_direct_pays(768, 768, 8192) and native.wgrad_direct_pays(2304, 768, 8192)
+    assert not native.wgrad_direct_pays(1024, 4096, 8192) and not native.wgrad_direct_pays(2048, 4096, 8192)
+    M, K, N = 512, 4096, 1024
+    x, w, dy = seeded_bf16((M, K), 1.0, 60), seeded_bf16((N, K), 0.02, 61), seeded_bf16((M, N), 1e-3, 62)
+    results = {}
+    for force_direct in (False, True):
+        if force_direct:
+            monkeypatch.setattr(native, "wgrad_direct_pays", lambda *a: True)
+        calls = _count_calls(monkeypatch, native, "gemm_layouts")
+        recipe = amp.create_fp8_recipe("tensorwise", "hybrid")
+        results[force_direct] = run_step(make_linear(w), recipe, x, dy)
+        assert (len(calls) == 1) == force_direct
+    for got, want in zip(results[False], results[True]):
+        assert torch.equal(got, want)
+
+
 @pytest.mark.parametrize("seed", range(24))
 def test_seeded_random_linears_match_the_oracle(amp, seed):
     """Layer sizes on the grids the kernels distinguish, tokens likewise, bf16 or fp32 master weights, with and
