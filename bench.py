@@ -166,9 +166,11 @@ def timed_steps(torch, one, steps, warmup):
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     after = torch.cuda.memory_stats()
-    per = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(steps))
+    in_order = [marks[i].elapsed_time(marks[i + 1]) for i in range(steps)]
+    per = sorted(in_order)
     return {"ms_per_step": 1e3 * wall / steps, "warmup_steps": warmup + extra, "min_ms": per[0], "median_ms": per[len(per) // 2], "max_ms": per[-1],
-            "max_over_median": per[-1] / per[len(per) // 2],
+            "max_over_median": per[-1] / per[len(per) // 2], "slowest_step": in_order.index(per[-1]),
+            "per_step_ms": [round(t, 3) for t in in_order],
             "allocator": {"segments_allocated_during_timed_steps": after.get("num_device_alloc", 0) - before.get("num_device_alloc", 0),
                           "alloc_retries_during_timed_steps": after.get("num_alloc_retries", 0) - before.get("num_alloc_retries", 0),
                           "reserved_mib_before": before.get("reserved_bytes.all.current", 0) >> 20,

@@ -81,18 +81,25 @@ __device__ __forceinline__ uint32_t amax_chunks(const void *__restrict__ x, int6
             }
         }
     }
-    for (; i < n16; i += stride) {
-        u32x4 v = p[i];
-        if constexpr (SRC == ODL_BF16) {
-            m0 = max_u16x2(m0, abs_bf16x2(v.x));
-            m1 = max_u16x2(m1, abs_bf16x2(v.y));
-            m2 = max_u16x2(m2, abs_bf16x2(v.z));
-            m3 = max_u16x2(m3, abs_bf16x2(v.w));
-        } else {
-            m0 = max(m0, v.x & 0x7fffffffu);
-            m1 = max(m1, v.y & 0x7fffffffu);
-            m2 = max(m2, v.z & 0x7fffffffu);
-            m3 = max(m3, v.w & 0x7fffffffu);
+    // the rest (fewer than UNROLL chunks for this lane) as one more batch of loads with the missing ones left out:
+    // taken one at a time they were up to UNROLL - 1 memory latencies in a row at the end of every block
+    if (i < n16) {
+        u32x4 v[UNROLL - 1];
+#pragma unroll
+        for (int u = 0; u < UNROLL - 1; ++u) v[u] = (i + u * stride < n16) ? p[i + u * stride] : u32x4{0, 0, 0, 0};
+#pragma unroll
+        for (int u = 0; u < UNROLL - 1; ++u) {
+            if constexpr (SRC == ODL_BF16) {
+                m0 = max_u16x2(m0, abs_bf16x2(v[u].x));
+                m1 = max_u16x2(m1, abs_bf16x2(v[u].y));
+                m2 = max_u16x2(m2, abs_bf16x2(v[u].z));
+                m3 = max_u16x2(m3, abs_bf16x2(v[u].w));
+            } else {
+                m0 = max(m0, v[u].x & 0x7fffffffu);
+                m1 = max(m1, v[u].y & 0x7fffffffu);
+                m2 = max(m2, v[u].z & 0x7fffffffu);
+                m3 = max(m3, v[u].w & 0x7fffffffu);
+            }
         }
     }
     if constexpr (SRC == ODL_BF16) return fold_u16x2_to_f32bits(max_u16x2(max_u16x2(m0, m1), max_u16x2(m2, m3)));
