@@ -362,7 +362,7 @@ __device__ __forceinline__ void block_scale_of(uint32_t amax_bits, int margin, u
 // 64-column tile of ct_tile.h (a 256-byte line per pair of columns, rotated by 16 bytes per 8 columns), the second half
 // rotated by 16 bytes more.  The dword writes of a half-wave (8 column groups of 16 x 4 row groups) then differ mod 32,
 // and the 16-byte reads stay aligned with 16 consecutive lanes reading one whole line.
-__device__ __forceinline__ int block_col_slot(int col) { return col + 4 * (col >> 6); }
+__device__ __forceinline__ int block_col_slot(int col) { return col + 4 * (col >> 5); }
 
 __device__ __forceinline__ int block_lds_off(int col, int dw) {
     const int half = col >> 6, c = col & 63;
@@ -383,11 +383,12 @@ __global__ __launch_bounds__(256, SRC == ODL_BF16 ? 8 : 4) void block_cast_kerne
                                                          uint8_t *__restrict__ out, uint32_t *__restrict__ scales,
                                                          uint8_t *__restrict__ out_t, uint32_t *__restrict__ scales_t) {
     __shared__ __attribute__((aligned(16))) uint8_t tile[WANT_COL ? 128 * 128 : 16];
-    // red and col_e8 hold one value per column at block_col_slot(column): columns 64..127 sit four dwords further on, so
-    // that the eight lanes (tx = 0..7) that touch columns 16 tx + j in one instruction land in eight different groups of
-    // banks (columns c and c + 64 would otherwise share theirs)
-    __shared__ __attribute__((aligned(16))) uint32_t red[4][128 + 4];   // per wave: column maxima (1-D), or slot 0: the wave's maximum (2-D)
-    __shared__ __attribute__((aligned(16))) float col_e8[128 + 4];      // per column: its E8M0 byte where a float keeps its exponent
+    // red and col_e8 hold one value per column at block_col_slot(column): every 32 columns sit four dwords further on.
+    // The 8-byte write of the column maxima is served 16 lanes at a time over 32 banks (measured: with the 8 lanes tx
+    // on dwords 8 tx + j, lanes tx and tx + 4 met, 4 conflict cycles per wave); with the pitch the 16 lanes (8 tx, two
+    // neighbouring column pairs each) cover 32 consecutive dwords.  The 16-byte reads of col_e8 stay on 32 different banks.
+    __shared__ __attribute__((aligned(16))) uint32_t red[4][144];       // per wave: column maxima (1-D), or slot 0: the wave's maximum (2-D)
+    __shared__ __attribute__((aligned(16))) float col_e8[144];          // per column: its E8M0 byte where a float keeps its exponent
     __shared__ int odd_tile;                                       // 1-D blocks: some column of the tile holds Inf / NaN
     __shared__ uint32_t row_dw[128];                               // 1-D blocks, both outputs: the scale dwords of the tile's rows
     saturate_fp8_conversions();
@@ -456,6 +457,7 @@ __global__ __launch_bounds__(256, SRC == ODL_BF16 ? 8 : 4) void block_cast_kerne
     }
 
     if constexpr (WANT_ROW) {
+        [[maybe_unused]] uint32_t keep_row = 0;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             float e8 = e8_all;
@@ -467,11 +469,10 @@ __global__ __launch_bounds__(256, SRC == ODL_BF16 ? 8 : 4) void block_cast_kerne
                 float mul;
                 block_scale_of<FMT>(m, margin, dword, mul);
                 e8 = e8_of(dword);
-                // with the transposed output to follow, the tile's 128 row dwords leave as one 512-byte run after the next barrier
-                if (tx == 0) {
-                    if constexpr (WANT_COL) row_dw[ty * 4 + i] = dword;
-                    else scales[tc * rows + r0 + i] = dword;
-                }
+                // with the transposed output to follow, the tile's 128 row dwords leave as one 512-byte run after the next
+                // barrier: lane tx = i of the 8 that hold the row keeps it, and the lanes tx < 4 store one dword each
+                if constexpr (WANT_COL) { if (tx == i) keep_row = dword; }
+                else if (tx == 0) scales[tc * rows + r0 + i] = dword;
             }
             uint32_t q[4];
             if (__builtin_expect(m >= 0x7f800000u, 0)) {
@@ -498,29 +499,32 @@ __global__ __launch_bounds__(256, SRC == ODL_BF16 ? 8 : 4) void block_cast_kerne
                 for (int g = 0; g < 4; ++g) *reinterpret_cast<uint32_t *>(o + group_col(g)) = q[g];
             }
         }
+        if constexpr (!TWO_D && WANT_COL) { if (tx < 4) row_dw[ty * 4 + tx] = keep_row; }
     }
 
     if constexpr (WANT_COL) {
         bool plain = m_all < 0x7f800000u;                                // no Inf / NaN anywhere in the tile
         if constexpr (!TWO_D) {
-            // column maxima: over the lane's 4 rows, over the 8 lanes of the wave with this tx (32 rows), over the 4 waves
-            [[maybe_unused]] uint32_t m_even = 0;
+            // column maxima: over the lane's 4 rows, over the 8 lanes of the wave with this tx (32 rows), over the 4 waves.
+            // After the exchange all 8 lanes with this tx hold the maxima of the lane's 8 column pairs; lane p = ty & 7 of
+            // them keeps pair p, so the wave stores its 128 maxima with ONE 8-byte write per lane that covers the row of
+            // `red` exactly (eight writes of 8 lanes each were counted as one conflict cycle apiece)
+            const int p = ty & 7;
+            uint32_t keep_lo = 0, keep_hi = 0;
 #pragma unroll
             for (int d = 0; d < DW; ++d) {
                 uint32_t m;
-                // after the exchange all 8 lanes with this tx hold the maximum: each of them stores one eighth of the 16
-                // columns (an 8-byte store), instead of one lane storing all of them through the same few banks
                 if constexpr (SRC == ODL_BF16) {
                     m = max_u16x2(max_u16x2(abs_bf16x2(raw[0][d]), abs_bf16x2(raw[1][d])), max_u16x2(abs_bf16x2(raw[2][d]), abs_bf16x2(raw[3][d])));
                     m = max_stride8_u16x2(m);
-                    if ((ty & 7) == d) *reinterpret_cast<u32x2 *>(&red[wave][block_col_slot(group_col(d / 2) + 2 * (d & 1))]) = u32x2{m << 16, m & 0xffff0000u};
+                    if (p == d) { keep_lo = m << 16; keep_hi = m & 0xffff0000u; }
                 } else {
                     m = max(max(raw[0][d] & 0x7fffffffu, raw[1][d] & 0x7fffffffu), max(raw[2][d] & 0x7fffffffu, raw[3][d] & 0x7fffffffu));
                     m = max_stride8(m);
-                    if ((d & 1) && (ty & 7) == d / 2) *reinterpret_cast<u32x2 *>(&red[wave][block_col_slot(group_col(d / 4) + (d & 3) - 1)]) = u32x2{m_even, m};
-                    m_even = m;
+                    if (p == d / 2) { if (d & 1) keep_hi = m; else keep_lo = m; }
                 }
             }
+            *reinterpret_cast<u32x2 *>(&red[wave][block_col_slot(group_col(p / 2) + 2 * (p & 1))]) = u32x2{keep_lo, keep_hi};
             if (threadIdx.x == 0) odd_tile = 0;
             __syncthreads();
             if (threadIdx.x < 128) {
