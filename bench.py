@@ -337,7 +337,15 @@ def standalone_hbm(torch, native, iters=24):
                 "cast": (lambda x: native.cast(x, scale, native.E4M3, native.SCALE_TENSOR), 3 * E),
                 "cast_transpose": (lambda x: native.cast_transpose(x, scale, native.E4M3, native.SCALE_TENSOR), 4 * E),
                 "amax_then_cast_transpose": (lambda x: native.quantize_dynamic(x, native.E4M3, 0), 6 * E),
+                # the block-scaled casts: codes in both layouts plus their scale bytes, no amax pass
+                "mx_cast_both_layouts": (lambda x: native.mx_cast(x, native.E4M3, True, True), 4 * E + 2 * (E // 32)),
+                "block_cast_1d_both_layouts": (lambda x: native.block_cast(x, native.E4M3, 0, False, True, True), 4 * E + 8 * (E // 128)),
             }
+            if cols == D_MODEL and rows == M_TOKENS:   # fp32 sources (master weights, an fp32 residual stream)
+                xs32c = [x.float() for x in xs]
+                c32 = {id(x): y for x, y in zip(xs, xs32c)}
+                kernels["cast_fp32_in"] = (lambda x: native.cast(c32[id(x)], scale, native.E4M3, native.SCALE_TENSOR), 5 * E)
+                kernels["cast_transpose_fp32_in"] = (lambda x: native.cast_transpose(c32[id(x)], scale, native.E4M3, native.SCALE_TENSOR), 6 * E)
         if cols == D_FF:                   # the SwiGLU producers run on the [tokens, d_ff] activations
             nxt = {id(x): (xs[(i + 1) % nbuf], xs[(i + 2) % nbuf]) for i, x in enumerate(xs)}
             kernels["swiglu_fwd_amax"] = (lambda x: native.swiglu_amax_parts(x, nxt[id(x)][0]), 6 * E)
@@ -763,6 +771,9 @@ def main() -> int:
     ap.add_argument("--other-configs-only", default="",
                     help="run only the whole steps of the other configurations whose label contains this text (e.g. mxfp8, rowwise, "
                          "delayed) and print them (for profiling)")
+    ap.add_argument("--no-dgrad-sum-fusion", action="store_true",
+                    help="leave the data-gradient sums of Linears fed by one tensor (q/k/v, gate/up) to autograd instead of the "
+                         "GEMMs' accumulate flag (FP8Recipe.fuse_dgrad_sum = False), for A/B traces")
     ap.add_argument("--clock-probe-only", action="store_true",
                     help="run only the clock probe (GEMM back to back on Gaussian / zero operands, register-only MFMA loop) and print it")
     ap.add_argument("--power-probe-only", action="store_true",
@@ -791,6 +802,16 @@ def main() -> int:
     if args.clock_probe_only:
         print(json.dumps({"clock_probe": clock_probe(torch, native)}))
         return 0
+    if args.no_dgrad_sum_fusion:
+        from optimus_dl_amd.modules.amp import fp8 as _fp8
+
+        _recipe_init = _fp8.FP8Recipe.__init__
+
+        def _init_without_fusion(self, *a, **k):
+            _recipe_init(self, *a, **k)
+            self.fuse_dgrad_sum = False
+
+        _fp8.FP8Recipe.__init__ = _init_without_fusion
     if args.other_configs_only:
         print(json.dumps({"other_configs_fwd_bwd": other_configs(torch, steps=args.steps, only=args.other_configs_only)}))
         return 0
