@@ -480,10 +480,39 @@ class SiblingGroup:
         return outs[self.modules.index(member)]
 
 
+def keep_layers_in_bf16(model: nn.Module, at_start: int = 1, at_end: int = 1) -> list[str]:
+    """``first_last_layers_bf16`` with ``num_layers_at_start_in_bf16`` / ``num_layers_at_end_in_bf16``
+    (optimus_dl/modules/optim/config.py:44-49,62-66: "retain first and last N layers in BF16"; the reference declares
+    the keys and never reads them).  The layers are the entries of the model's block list: the ``nn.ModuleList`` with
+    the most entries among those whose every entry holds an FP8 Linear (``transformer.h`` of the reference's GPT-2 /
+    Llama / Qwen3 trees).  The FP8 Linears inside its first ``at_start`` and last ``at_end`` entries get
+    ``fp8_enabled = False`` and run in the autocast dtype; everything else (embedding, head, the other blocks) is left as
+    it is.  Returns the qualified names of the Linears switched off (empty when no such list exists)."""
+    best_name, best = "", None
+    for name, mod in model.named_modules():
+        if isinstance(mod, nn.ModuleList) and len(mod) > 0 and (best is None or len(mod) > len(best)):
+            if all(any(isinstance(m, FP8Linear) for m in entry.modules()) for entry in mod):
+                best_name, best = name, mod
+    if best is None:
+        return []
+    n = len(best)
+    picked = sorted(set(range(min(max(at_start, 0), n))) | set(range(max(n - max(at_end, 0), 0), n)))
+    names = []
+    for i in picked:
+        for sub, m in best[i].named_modules():
+            if isinstance(m, FP8Linear):
+                m.fp8_enabled = False
+                names.append(".".join(x for x in (best_name, str(i), sub) if x))
+    return names
+
+
 class FP8Linear(nn.Linear):
     """Drop-in ``nn.Linear`` with an FP8 fast path (see the module docstring)."""
 
     _siblings: "SiblingGroup | None" = None      # set on the instance by a SiblingGroup that this Linear is a member of
+    # False: this Linear stays in the autocast dtype under an FP8 recipe too (``first_last_layers_bf16`` of the
+    # reference's config, optimus_dl/modules/optim/config.py:62-66; set by ``keep_layers_in_bf16``)
+    fp8_enabled: bool = True
 
     def __init__(self, in_features: int, out_features: int, bias: bool = True, device=None, dtype=None, **kwargs: Any):
         super().__init__(in_features, out_features, bias=bias, device=device, dtype=dtype)
@@ -630,7 +659,7 @@ class FP8Linear(nn.Linear):
 
     # ------------------------------------------------------------------ forward
     def _fp8_eligible(self, x: torch.Tensor) -> bool:
-        if not x.is_cuda or not self.weight.is_cuda:
+        if not self.fp8_enabled or not x.is_cuda or not self.weight.is_cuda:
             return False
         if self.weight.dtype not in (torch.bfloat16, torch.float32):
             _warn_once(f"FP8Linear: weight dtype {self.weight.dtype} is not bf16/fp32; running as a plain Linear")
@@ -650,7 +679,7 @@ class FP8Linear(nn.Linear):
         return True
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        if _state.active_recipe() is None:
+        if _state.active_recipe() is None or not self.fp8_enabled:
             return F.linear(x, self.weight, self.bias)
         siblings = self._siblings
         if siblings is not None:
@@ -789,7 +818,7 @@ class Fp8ParamSet:
     def attach(cls, model: nn.Module, recipe: FP8Recipe, optimizer: "torch.optim.Optimizer | None" = None) -> "Fp8ParamSet":
         """The set of every ``FP8Linear`` under ``model``, quantised once now; with an optimizer, again after each
         of its steps."""
-        ps = cls([m for m in model.modules() if isinstance(m, FP8Linear)], recipe)
+        ps = cls([m for m in model.modules() if isinstance(m, FP8Linear) and m.fp8_enabled], recipe)
         recipe._param_sets.add(ps)
         ps.sync()
         if optimizer is not None:

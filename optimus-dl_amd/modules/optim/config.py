@@ -4,7 +4,8 @@ configs/train/optimization/amp/fp8_{hybrid,e4m3}.yaml fill in).
 
 Keys the reference declares but never reads (param, wgrad, first_last_layers_bf16,
 num_layers_at_*_in_bf16, tp_only_amax_red) are accepted; ``wgrad=False`` is
-honoured here (weight gradients in bf16), the others are carried through.
+honoured here (weight gradients in bf16), ``param`` and ``first_last_layers_bf16`` act through
+``TrainingContext.attach_fp8_params`` / ``apply_fp8_layer_policy``, ``tp_only_amax_red`` is carried through.
 """
 
 from __future__ import annotations

@@ -102,6 +102,19 @@ class TrainingContext:
             return None
         return self._fp8_recipe.attach_params(model, optimizer)
 
+    def apply_fp8_layer_policy(self, model: torch.nn.Module) -> list[str]:
+        """``amp.fp8.first_last_layers_bf16: true``: the FP8 Linears of the model's first
+        ``num_layers_at_start_in_bf16`` and last ``num_layers_at_end_in_bf16`` blocks run in the autocast dtype
+        (optimus_dl/modules/optim/config.py:44-49,62-66; the reference declares the keys and never reads them).  Call
+        once, after the model transform and before ``attach_fp8_params``.  Returns the names of the Linears kept out of
+        FP8 (empty when the key is off or FP8 is not in use)."""
+        fp8 = self.optimization_config.amp.fp8
+        if self._fp8_recipe is None or not fp8.first_last_layers_bf16:
+            return []
+        from ..modules.fp8_linear import keep_layers_in_bf16
+
+        return keep_layers_in_bf16(model, fp8.num_layers_at_start_in_bf16, fp8.num_layers_at_end_in_bf16)
+
     def _create_fp8_autocast(self, device: torch.device, fp8_recipe: FP8Recipe | None) -> Any:
         if fp8_recipe is not None:
             return lambda: fp8_autocast(device=device, fp8_recipe=fp8_recipe)   # a fresh context per microbatch

@@ -224,6 +224,42 @@ def test_e5m2_delayed_is_refused_and_every_recipe_type_constructs(amp):
     assert rec.recipe_type == amp.Fp8RecipeType.DELAYED and rec.format == amp.Fp8Format.HYBRID and rec.recipe is not None
 
 
+def test_first_and_last_blocks_stay_in_bf16_when_the_config_says_so(amp):
+    """amp.fp8.first_last_layers_bf16 with one layer at each end (optimus_dl/modules/optim/config.py:62-66): the Linears
+    of blocks 0 and 3 of a 4-block model never take the FP8 path, those of blocks 1 and 2 and the head do, and a
+    training step still runs through the reference-shaped glue."""
+    from optimus_dl_amd.modules.fp8_linear import FP8Linear
+    from optimus_dl_amd.modules.model import Llama, LlamaConfig
+    from optimus_dl_amd.modules.model_transforms import build_model_transform
+    from optimus_dl_amd.modules.optim.config import AmpConfig, Fp8Config, OptimizationConfig
+    from optimus_dl_amd.recipe import TrainingContext, execute_backward_pass, execute_forward_pass
+
+    torch.manual_seed(0)
+    model = Llama(LlamaConfig(vocab_size=512, n_layer=4, n_head=4, n_kv_head=2, n_embd=128, intermediate_size=256)).cuda()
+    model = build_model_transform({"_name": "transformer_engine"}).apply(model, device=torch.device("cuda"))
+    cfg = OptimizationConfig(amp=AmpConfig(enabled=True, dtype="torch.float8_e4m3fn", fp8=Fp8Config(
+        enabled=True, recipe="tensorwise", first_last_layers_bf16=True, num_layers_at_start_in_bf16=1, num_layers_at_end_in_bf16=1)))
+    tc = TrainingContext(cfg)
+    ctx = tc.setup_training_context(torch.device("cuda"))
+    names = tc.apply_fp8_layer_policy(model)
+    assert len(names) == 2 * 7 and all(n.startswith(("transformer.h.0.", "transformer.h.3.")) for n in names)
+
+    def crit(m, batch):
+        logits = m(batch["input_ids"])["logits"].float()
+        return torch.nn.functional.cross_entropy(logits.view(-1, logits.shape[-1]), batch["labels"].view(-1))
+
+    ids = torch.randint(0, 512, (8, 33), generator=torch.Generator().manual_seed(1))
+    batch = {"input_ids": ids[:, :-1].cuda(), "labels": ids[:, 1:].cuda()}
+    loss = execute_forward_pass(model, batch, crit, ctx["amp_ctx"])
+    execute_backward_pass(loss, ctx["scaler"], ctx["fp8_backward_ctx"])
+    assert torch.isfinite(loss)
+    for i, blk in enumerate(model.transformer.h):
+        calls = [m.fp8_calls for m in blk.modules() if isinstance(m, FP8Linear)]
+        assert all(c == 0 for c in calls) if i in (0, 3) else all(c == 1 for c in calls), (i, calls)
+        assert all(m.weight.grad is not None for m in blk.modules() if isinstance(m, FP8Linear))
+    assert model.lm_head.fp8_calls == 1
+
+
 def test_wgrad_false_keeps_weight_gradient_in_bf16(amp):
     M, K, N = 128, 256, 128
     x, w, dy = seeded_bf16((M, K), 1.0, 0), seeded_bf16((N, K), 0.02, 1), seeded_bf16((M, N), 1e-3, 2)

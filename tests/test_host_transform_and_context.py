@@ -238,6 +238,36 @@ def test_forward_backward_helpers_accept_instance_or_factory():
     assert len(calls) == 2 and lin.weight.grad is not None
 
 
+def test_first_and_last_blocks_can_stay_out_of_fp8(monkeypatch):
+    """first_last_layers_bf16 / num_layers_at_{start,end}_in_bf16 (optimus_dl/modules/optim/config.py:62-66): the block
+    list is found by structure, the Linears of the chosen blocks are marked and nothing else is touched."""
+    from optimus_dl_amd.modules.fp8_linear import keep_layers_in_bf16
+
+    monkeypatch.setattr(T, "_HAVE_TE", True)
+    m = Llama(LlamaConfig(vocab_size=256, n_layer=5, n_head=4, n_kv_head=2, n_embd=64, intermediate_size=128))
+    build_model_transform({"_name": "transformer_engine"}).apply(m)
+    names = keep_layers_in_bf16(m, at_start=1, at_end=2)
+    assert len(names) == 3 * 7 and "transformer.h.0.attn.wq" in names and "transformer.h.4.mlp.c_proj" in names
+    off = {i for i in range(5) if not m.transformer.h[i].attn.wq.fp8_enabled}
+    assert off == {0, 3, 4}
+    for i in range(5):
+        flags = {mod.fp8_enabled for mod in m.transformer.h[i].modules() if isinstance(mod, FP8Linear)}
+        assert flags == {i not in off}
+    assert m.lm_head.fp8_enabled                                          # the head is not a block
+    assert keep_layers_in_bf16(nn.Sequential(nn.Linear(4, 4)), 1, 1) == []  # no block list: nothing to do
+    # more layers asked for than there are: all of them, each once
+    m2 = GPT2(GPT2Config(vocab_size=256, n_layer=2, n_head=4, n_embd=64, block_size=32))
+    build_model_transform({"_name": "transformer_engine"}).apply(m2)
+    assert len(keep_layers_in_bf16(m2, at_start=3, at_end=3)) == 2 * 6
+    # the training context reads the keys; without an FP8 recipe (this machine has no GPU) it does nothing
+    ctx = TrainingContext(opt("torch.bfloat16", fp8_enabled=False, first_last_layers_bf16=True))
+    ctx.setup_training_context(torch.device("cpu"))
+    assert ctx.apply_fp8_layer_policy(m) == []
+    # a Linear that is switched off is a plain Linear even inside an FP8 context
+    out = m(torch.randint(0, 256, (2, 16)))["logits"]
+    assert out.shape == (2, 16, 256)
+
+
 # ------------------------------------------------- fused producers: transform and hand-over (host side)
 def _llama_tree():
     from optimus_dl_amd.modules.model import Llama, LlamaConfig
