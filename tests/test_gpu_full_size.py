@@ -513,3 +513,114 @@ def test_block_scaled_gemm_at_baseline_shapes(N, M, Nn, K, recipe):
     # one more on every scale byte of A: every output doubled (exact in bf16 away from overflow)
     doubled = N.mx_gemm_nt(aq, asc + 1, bq, bsc, O.E5M2, O.E4M3)
     assert torch.equal(doubled.float(), out.float() * 2)
+
+
+def test_fp32_source_quantisation_at_a_weight_shape(N):
+    """fp32 master weights are the reference's usual AMP set-up: every cast also takes an fp32 source.  W of the up
+    projection (4096 x 14336 as stored for the down projection's input side) with genuine fp32 mantissas: per-tensor
+    codes in both layouts, MXFP8 codes and scale bytes, 128 x 128 block codes, against the oracle on samples and through
+    the identities that hold at any size."""
+    rows_n, cols_n = 4096, 14336
+    g = torch.Generator(device="cuda").manual_seed(91)
+    x = torch.randn((rows_n, cols_n), generator=g, device="cuda", dtype=torch.float32) * 0.02 + 3e-5
+    assert not torch.equal(x.bfloat16().float(), x)                       # not representable in bf16: the fp32 path is what runs
+    q, q_t, scale, scale_inv, amax = quantise(N, x, O.E4M3)
+    assert_f32_bits_equal(amax, x.abs().max().reshape(1), "amax vs torch")
+    assert_f32_bits_equal(scale, torch.tensor([O.c_scale(float(amax), O.E4M3, 0, 1.0)]), "scale")
+    assert torch.equal(q_t, q.t().contiguous())
+    assert torch.equal(N.cast(x, scale, O.E4M3), q)
+    rows = torch.tensor([0, 5, 127, 128, rows_n // 2 + 1, rows_n - 1]).cuda()
+    assert_bytes_equal(q[rows], O.t_cast(x[rows].cpu(), scale.cpu(), O.E4M3), "codes of sampled rows")
+    # the partial maxima + cast route gives the same codes as amax -> scale -> cast
+    q2, q2_t, _, scale2, _ = N.quantize_dynamic(x, O.E4M3)
+    assert torch.equal(q2, q) and torch.equal(q2_t, q_t)
+    assert_f32_bits_equal(scale2, scale, "scale of the dynamic route")
+    # MXFP8, both shared-exponent rules: sampled rows (blocks along the columns) and sampled columns (blocks along the rows)
+    for rule in (N.MX_FLOOR, N.MX_CEIL):
+        mq, ms, mq_t, ms_t = N.mx_cast(x, O.E4M3, True, True, scale_rule=rule)
+        wc, ws = O.t_mx_quantise(x[rows].cpu(), O.E4M3, rule)        # (the C oracle takes bf16; its torch twin any float)
+        assert_bytes_equal(mq[rows], wc, f"mx codes of sampled rows, rule {rule}")
+        assert_bytes_equal(N.mx_scales_rowmajor(ms)[rows], ws, f"mx scale bytes of sampled rows, rule {rule}")
+        cols = torch.tensor([0, 3, 31, 32, 4097, cols_n - 1]).cuda()
+        wct, wst = O.t_mx_quantise(x[:, cols].t().contiguous().cpu(), O.E4M3, rule)
+        assert_bytes_equal(mq_t[cols], wct, f"mx codes of sampled columns, rule {rule}")
+        assert_bytes_equal(N.mx_scales_rowmajor(ms_t)[cols], wst, f"mx scale bytes of sampled columns, rule {rule}")
+    # 128 x 128 blocks (weights of the blockwise recipe): one set of scales serves both layouts
+    bq, bs, bq_t, bs_t = N.block_cast(x, O.E4M3, 0, True, True, True)
+    assert torch.equal(bq_t, bq.t().contiguous())
+    strip = slice(rows_n - 128, rows_n)
+    wc, ws = O.t_block_quantise(x[strip].cpu(), 128, 128, O.E4M3, 0)
+    assert_bytes_equal(bq[strip], wc, "block codes of the last row of tiles")
+    # 1 x 128 blocks (activations): a sampled strip of rows, and of columns for the transposed codes
+    aq, as_, aq_t, as_t = N.block_cast(x, O.E4M3, 0, False, True, True)
+    wc, ws = O.t_block_quantise(x[rows].cpu(), 1, 128, O.E4M3, 0)
+    assert_bytes_equal(aq[rows], wc, "1 x 128 block codes of sampled rows")
+    wct, wst = O.t_block_quantise(x[:, cols].t().contiguous().cpu(), 1, 128, O.E4M3, 0)
+    assert_bytes_equal(aq_t[cols], wct, "128 x 1 block codes of sampled columns")
+
+
+def test_config_2_grouped_projections_sum_their_data_gradients_in_the_gemms(N):
+    """configs[1] as BASELINE writes it: ONE X for Wq, Wk, Wv.  The transform ties the three into a group: the outputs
+    and weight gradients are the bits of the separate modules, and dX, summed by the accumulating GEMMs with one rounding,
+    stays within the roundings that autograd's bf16 sum of three rounded products makes."""
+    import torch.nn as nn
+
+    from optimus_dl_amd import native
+    from optimus_dl_amd.modules import amp
+    from optimus_dl_amd.modules.model_transforms import build_model_transform
+
+    class Projections(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.wq, self.wk, self.wv = nn.Linear(4096, 4096, bias=False), nn.Linear(4096, 1024, bias=False), nn.Linear(4096, 1024, bias=False)
+
+        def forward(self, x):
+            return self.wq(x), self.wk(x), self.wv(x)
+
+    M = 8192
+    net = Projections().to("cuda", torch.bfloat16)
+    with torch.no_grad():
+        for i, p in enumerate(net.parameters()):
+            p.copy_(draw(tuple(p.shape), 0.02, 100 + i))
+    t = build_model_transform({"_name": "fp8_linear"})
+    t.apply(net)
+    assert t.sibling_groups == 1
+    dys = [draw((M, n), 1e-3, 110 + i) for i, n in enumerate((4096, 1024, 1024))]
+    results = {}
+    for fused in (True, False):
+        recipe = amp.create_fp8_recipe("tensorwise", "hybrid")
+        recipe.fuse_dgrad_sum = fused
+        x = draw((M, 4096), 1.0, 120).requires_grad_(True)
+        for p in net.parameters():
+            p.grad = None
+        calls = []
+        real = native.gemm_nt
+        native.gemm_nt = lambda *a, **k: (calls.append(bool(k.get("accumulate"))), real(*a, **k))[1]
+        try:
+            with recipe.autocast():
+                ys = net(x)
+            with recipe.backward():
+                torch.autograd.backward(ys, dys)
+        finally:
+            native.gemm_nt = real
+        assert sum(calls) == (2 if fused else 0), calls
+        results[fused] = ([y.detach() for y in ys], x.grad, [p.grad for p in net.parameters()])
+    for a, b in zip(results[True][0], results[False][0]):
+        assert torch.equal(a, b)
+    for a, b in zip(results[True][2], results[False][2]):
+        assert torch.equal(a, b)
+    dx_f, dx_s = results[True][1].float(), results[False][1].float()
+    assert torch.isfinite(dx_f).all()
+    # the separate route rounds each product and each of the two sums to bf16 (up to 4 half-units of the largest term)
+    bound = 4 * 2.0 ** -9 * dx_s.abs().max()
+    assert float((dx_f - dx_s).abs().max()) <= float(bound)
+    # and against the oracle on a sample: dX = sum of Q(dY_i) . Q(W_i^T)^T with the codes the kernels made
+    ri = torch.randperm(M, generator=torch.Generator().manual_seed(5))[:32].sort().values.cuda()
+    ci = torch.randperm(4096, generator=torch.Generator().manual_seed(6))[:256].sort().values.cuda()
+    ref = torch.zeros((32, 256))
+    for dy, lin in zip(dys, (net.wq, net.wk, net.wv)):
+        gq, _, _, _, sgi = native.quantize_dynamic(dy, O.E5M2, want_transposed=False)
+        _, wq_t, _, _, swi = native.quantize_dynamic(lin.weight.detach(), O.E4M3)
+        ref += O.t_gemm_nt(gq[ri].cpu(), wq_t[ci].cpu(), O.E5M2, O.E4M3, sgi.cpu(), swi.cpu(), want_f32=True)[1]
+    got = results[True][1][ri][:, ci].float().cpu()
+    assert max_rel_err(got, ref) <= TOL
