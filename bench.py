@@ -139,6 +139,15 @@ class KernelTimer:
         return out
 
 
+def weights_changed(module):
+    """What an optimizer step does to the module's weight as far as the FP8 path can tell: the Parameter's version
+    counter moves, so every cached quantisation of it (per module, per group of siblings, per parameter set) is out of
+    date and the next forward quantises the weight again.  No kernel is launched for it."""
+    import torch
+
+    torch.autograd.graph.increment_version(module.weight)
+
+
 def timed_steps(torch, one, steps, warmup):
     """`warmup` untimed calls of `one`, then `steps` timed ones.  ms_per_step is wall time over all of them (host clock,
     synchronised on both sides); min / median / max are per step, from one HIP event between consecutive steps, so a
@@ -415,7 +424,7 @@ def attention_projections(torch, steps=8, warmup=3):
 
     def one():
         for lin in mods:
-            lin._wcache.key = None
+            weights_changed(lin)
             lin.weight.grad = None
         x.grad = o.grad = None
         with recipe.autocast():
@@ -468,8 +477,7 @@ def other_configs(torch, steps=8, warmup=3, only=""):
 
         def one():
             for lin, x, dy in zip(mods, xs, dys):
-                lin._wcache.key = None
-                lin._wcache_rowwise.clear()
+                weights_changed(lin)
                 lin.weight.grad = None
                 x.grad = None
                 with recipe.autocast():
@@ -503,7 +511,7 @@ def mlp_block(torch, native, recipe, steps=10, warmup=3):
 
         def one():
             for lin in (mlp.w1, mlp.w2, mlp.c_proj):
-                lin._wcache.key = None
+                weights_changed(lin)
                 lin.weight.grad = None
             x.grad = None
             with recipe.autocast():
@@ -546,7 +554,7 @@ def llama_block(torch, steps=12, warmup=4):
             x.grad = None
             for m in blk.modules():
                 if hasattr(m, "_wcache"):
-                    m._wcache.key = None
+                    weights_changed(m)
             if cfg:
                 with A.fp8_autocast(torch.device("cuda"), recipe):
                     y = blk(x)
@@ -609,8 +617,7 @@ def whole_models(torch, which=("gpt2_124m", "qwen3_0.6b"), steps=5, warmup=3, la
                 else:
                     for m in model.modules():
                         if hasattr(m, "_wcache"):
-                            m._wcache.key = None
-                            m._wcache_rowwise.clear()
+                            weights_changed(m)
                 if cfg:
                     with A.fp8_autocast(torch.device("cuda"), recipe):
                         loss = F.cross_entropy(model(ids)["logits"].view(-1, V).float(), tgt)
@@ -837,7 +844,7 @@ def main() -> int:
     def one_step():
         for name, _, _ in LAYERS:
             lin, d = layers[name], data[name]
-            lin._wcache.key = None            # weights change every optimizer step: re-quantise them every step
+            weights_changed(lin)              # weights change every optimizer step: re-quantise them every step
             lin.weight.grad = None
             d["x"].grad = None
             with recipe.autocast():
