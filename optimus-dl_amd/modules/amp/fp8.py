@@ -225,6 +225,10 @@ class FP8Recipe:
         # of a separate ``grad += dw`` pass per weight and microbatch.  Off by default: tensor hooks on the weight's
         # gradient (DDP / FSDP reducers) do not see a gradient that never passes through autograd.
         self.fuse_wgrad_accumulation = False
+        # Members of such a group whose weight gradients are each a GEMM of few tiles over a transposed copy of dy (k and v
+        # of a grouped-query attention block) get them from ONE GEMM over their transposed codes side by side; the
+        # gradients are then row ranges of one matrix.  False: a GEMM per member
+        self.fuse_sibling_wgrad = True
         # Fp8ParamSets attached under this recipe (delayed scaling: they re-record their weights' maxima at each refresh)
         self._param_sets: "weakref.WeakSet" = weakref.WeakSet()
         _info_once(

@@ -292,17 +292,29 @@ def amax_parts_colsum(x: torch.Tensor):
     return parts, colsum
 
 
+def _codes_out(t: torch.Tensor, shape: tuple, device, what: str) -> torch.Tensor:
+    if t.dtype != torch.uint8 or tuple(t.shape) != tuple(shape) or not t.is_contiguous() or t.device != device:
+        raise NativeError(f"{what}: a contiguous uint8 tensor {tuple(shape)} on {device} expected, got {t.dtype} {tuple(t.shape)} on {t.device}")
+    return t
+
+
 def cast_dynamic(x: torch.Tensor, parts: torch.Tensor, fmt: int, margin: int = 0, want_rowmajor: bool = True,
-                 want_transposed: bool = True):
-    """Cast with the per-tensor scale derived inside the kernel from the partial maxima.
+                 want_transposed: bool = True, out_t: torch.Tensor | None = None):
+    """Cast with the per-tensor scale derived inside the kernel from the partial maxima.  out_t: where the transposed
+    codes go (a [cols, rows] uint8 tensor of the caller's, e.g. a run of rows of a larger buffer that holds the codes of
+    several tensors); implies want_transposed.
     -> (q or None, q_t or None, amax, scale, scale_inv); the last three are fp32[1]."""
+    want_transposed = want_transposed or out_t is not None
     if not (want_rowmajor or want_transposed):
         raise NativeError("cast_dynamic: nothing to produce")
     x = _as_2d(x)
     rows, cols = x.shape
     _f32_dev(parts, AMAX_PARTS, "cast_dynamic parts")
     q = torch.empty((rows, cols), dtype=torch.uint8, device=x.device) if want_rowmajor else None
-    q_t = torch.empty((cols, rows), dtype=torch.uint8, device=x.device) if want_transposed else None
+    if out_t is not None:
+        q_t = _codes_out(out_t, (cols, rows), x.device, "cast_dynamic out_t")
+    else:
+        q_t = torch.empty((cols, rows), dtype=torch.uint8, device=x.device) if want_transposed else None
     dyn = torch.empty(3, dtype=torch.float32, device=x.device)
     _check(load().odl_fp8_cast_dynamic(x.data_ptr(), _src_dtype(x), rows, cols, parts.data_ptr(), fmt, margin,
                                        q.data_ptr() if q is not None else None, q_t.data_ptr() if q_t is not None else None,
@@ -424,11 +436,11 @@ class MultiTensorPlan:
 
 
 def quantize_dynamic(x: torch.Tensor, fmt: int, margin: int = 0, want_rowmajor: bool = True, want_transposed: bool = True,
-                     parts: torch.Tensor | None = None):
+                     parts: torch.Tensor | None = None, out_t: torch.Tensor | None = None):
     """Current scaling of one tensor in two launches: partial maxima, then a cast that derives the
     scale itself.  parts: the partial maxima, when the kernel that produced x already delivered
     them (one launch then).  -> (q or None, q_t or None, amax, scale, scale_inv)."""
-    return cast_dynamic(x, amax_parts(x) if parts is None else parts, fmt, margin, want_rowmajor, want_transposed)
+    return cast_dynamic(x, amax_parts(x) if parts is None else parts, fmt, margin, want_rowmajor, want_transposed, out_t=out_t)
 
 
 def _bf16_dense(t: torch.Tensor, what: str) -> torch.Tensor:
@@ -695,7 +707,7 @@ def cast_transpose(x: torch.Tensor, scale: torch.Tensor, fmt: int, mode: int = S
 
 
 def cast_delayed(x: torch.Tensor, scale: torch.Tensor, fmt: int, amax_parts: torch.Tensor | None = None,
-                 want_rowmajor: bool = True, want_transposed: bool = False):
+                 want_rowmajor: bool = True, want_transposed: bool = False, out_t: torch.Tensor | None = None):
     """The cast of the delayed-scaling recipe, one launch: codes with the per-tensor ``scale`` in force
     (row-major, transposed, or both), this step's partial maxima folded into ``amax_parts``
     (AMAX_PARTS floats of a role, accumulated, cleared by the next ``delayed_update``; None: nothing is
@@ -706,10 +718,14 @@ def cast_delayed(x: torch.Tensor, scale: torch.Tensor, fmt: int, amax_parts: tor
     _f32_dev(scale, 1, "cast_delayed scale")
     if amax_parts is not None:
         _f32_dev(amax_parts, AMAX_PARTS, "cast_delayed amax_parts")
+    want_transposed = want_transposed or out_t is not None       # out_t: the caller's [cols, rows] buffer, as in cast_dynamic
     if not (want_rowmajor or want_transposed):
         raise NativeError("cast_delayed: neither layout asked for")
     out = torch.empty((rows, cols), dtype=torch.uint8, device=x.device) if want_rowmajor else None
-    out_t = torch.empty((cols, rows), dtype=torch.uint8, device=x.device) if want_transposed else None
+    if out_t is not None:
+        _codes_out(out_t, (cols, rows), x.device, "cast_delayed out_t")
+    else:
+        out_t = torch.empty((cols, rows), dtype=torch.uint8, device=x.device) if want_transposed else None
     scale_inv = torch.empty(1, dtype=torch.float32, device=x.device)
     _check(load().odl_fp8_cast_delayed(x.data_ptr(), _src_dtype(x), rows, cols, scale.data_ptr(), fmt,
                                        out.data_ptr() if out is not None else None,

@@ -116,7 +116,7 @@ def test_sibling_group_launches_no_separate_adds(amp, monkeypatch):
     with recipe.backward():
         (q.float().sum() + v.float().sum()).backward()             # k is not used: its Linear has no backward at all
     assert calls.count(True) == 1 and net.wk.weight.grad is not None
-    assert len(calls) == 3 + 2 * 2                                  # 3 forwards, dgrad + wgrad for q and v (128 tokens: no K-slow wgrad)
+    assert len(calls) == 3 + 2 + 1                                  # 3 forwards, a dgrad each for q and v, ONE wgrad for both (128 tokens: no K-slow wgrad)
 
 
 def test_sibling_group_stands_down_when_members_get_different_inputs(amp):
