@@ -123,13 +123,8 @@ static void launch_gemm_generic(int fa, int fb, const GemmArgs &g, hipStream_t s
 
 static int cu_count() { return device_cu_count(); }
 
-static int choose_variant(int64_t M, int64_t N, int64_t K, bool stream_ok, bool accumulate) {
+static int choose_variant(int64_t M, int64_t N, bool stream_ok) {
     const int cus = cu_count();
-    // C = C + product over a short contraction is mostly output phase (the old values read, the new ones written): two
-    // 128 x 128 blocks per compute unit overlap one's output phase with the other's MFMAs, which one 256 x 256 block
-    // cannot (measured: 8192 x 4096 x 1024 50.0 against 56.9 us, 16384 x 768 x 768 21.8 against 23.3; from K = 2048 on
-    // the pipelined 256 x 256 kernel is ahead again: 16384 x 768 x 3072 43.9 against 47.7)
-    if (accumulate && K <= 1024) return 4;
     // an output of at most cus / 2 tiles of 256 x 256 leaves half the chip idle with the big tiles: the 128 x 128
     // kernel (two blocks per compute unit) spreads it four times wider (measured 15-20 % faster than either
     // 256-wide kernel at 8192 x 1024, 8192 x 768 and 2048 x 4096 outputs, K = 768 .. 4096)
@@ -222,7 +217,7 @@ extern "C" int odl_fp8_gemm_nt(const uint8_t *a, const uint8_t *b, int64_t M, in
     // C = C + product is an epilogue of the kernels whose tiles end in a separate output phase; the streaming kernel
     // stores a tile under the next tile's MFMAs, where nothing can wait for the old values of C
     const bool stream_ok = tiled_ok && lim32 && M % 128 == 0 && N % 128 == 0 && K >= 512 && !accumulate;
-    int variant = t_forced_variant >= 0 ? t_forced_variant : (tiled_ok ? choose_variant(M, N, K, stream_ok, accumulate != 0) : 0);
+    int variant = t_forced_variant >= 0 ? t_forced_variant : (tiled_ok ? choose_variant(M, N, stream_ok) : 0);
     if (variant != 0 && !tiled_ok) variant = 0;
     // the pipelined kernel walks K in pairs of 128-byte steps
     const bool pipe_ok = tiled_ok && K % 256 == 0 && lim32;
