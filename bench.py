@@ -122,10 +122,10 @@ class KernelTimer:
         wrap("amax", lambda x, *r, **kw: float(x.numel() * esz(x)))                                       # bytes
         wrap("amax_scale", lambda x, *r, **kw: float(x.numel() * esz(x)), record_as="amax")       # amax + scale, one launch
         wrap("amax_parts", lambda x, *r, **kw: float(x.numel() * esz(x)), record_as="amax")
-        wrap("cast_dynamic", lambda x, parts, fmt, margin=0, want_rowmajor=True, want_transposed=True:
-             float(x.numel() * (esz(x) + int(want_rowmajor) + int(want_transposed))),
-             record_as=lambda x, parts, fmt, margin=0, want_rowmajor=True, want_transposed=True:
-             "cast_transpose" if want_transposed else "cast")
+        wrap("cast_dynamic", lambda x, parts, fmt, margin=0, want_rowmajor=True, want_transposed=True, out_t=None:
+             float(x.numel() * (esz(x) + int(want_rowmajor) + int(want_transposed or out_t is not None))),
+             record_as=lambda x, parts, fmt, margin=0, want_rowmajor=True, want_transposed=True, out_t=None:
+             "cast_transpose" if (want_transposed or out_t is not None) else "cast")
         wrap("cast", lambda x, *r, **kw: float(x.numel() * (esz(x) + 1)))
         wrap("cast_transpose",
              lambda x, *r, **kw: float(x.numel() * (esz(x) + (2 if kw.get("want_rowmajor", True) else 1))))
