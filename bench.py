@@ -781,6 +781,9 @@ def main() -> int:
     ap.add_argument("--no-dgrad-sum-fusion", action="store_true",
                     help="leave the data-gradient sums of Linears fed by one tensor (q/k/v, gate/up) to autograd instead of the "
                          "GEMMs' accumulate flag (FP8Recipe.fuse_dgrad_sum = False), for A/B traces")
+    ap.add_argument("--dgrad-sum-by-accumulate", action="store_true",
+                    help="sum those data gradients with the GEMMs' accumulate flag only, not by one GEMM over all members' "
+                         "operands (FP8Recipe.fuse_dgrad_gemm = False), for A/B traces")
     ap.add_argument("--clock-probe-only", action="store_true",
                     help="run only the clock probe (GEMM back to back on Gaussian / zero operands, register-only MFMA loop) and print it")
     ap.add_argument("--power-probe-only", action="store_true",
@@ -809,14 +812,15 @@ def main() -> int:
     if args.clock_probe_only:
         print(json.dumps({"clock_probe": clock_probe(torch, native)}))
         return 0
-    if args.no_dgrad_sum_fusion:
+    if args.no_dgrad_sum_fusion or args.dgrad_sum_by_accumulate:
         from optimus_dl_amd.modules.amp import fp8 as _fp8
 
         _recipe_init = _fp8.FP8Recipe.__init__
 
         def _init_without_fusion(self, *a, **k):
             _recipe_init(self, *a, **k)
-            self.fuse_dgrad_sum = False
+            self.fuse_dgrad_sum = not args.no_dgrad_sum_fusion
+            self.fuse_dgrad_gemm = not args.dgrad_sum_by_accumulate
 
         _fp8.FP8Recipe.__init__ = _init_without_fusion
     if args.other_configs_only:

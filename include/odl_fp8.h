@@ -356,6 +356,28 @@ int odl_fp8_gemm_nt(const uint8_t *a, const uint8_t *b, int64_t M, int64_t N, in
                     void *c, int out_dtype, int accumulate, odl_stream_t stream);
 
 /*
+ * A sum of such products in one call:
+ *   C[M, N] = sum over s < pairs of (A_s[M, K[s]] . B_s[N, K[s]]^T) * (sa_inv[s][0] * sb_inv[s][0])
+ * a, b, sa_inv, sb_inv: HOST arrays of `pairs` device pointers, K a host array of `pairs` lengths (all read
+ * during the call); one scale per operand, no bias, out_dtype ODL_BF16 or ODL_F32, C is overwritten.  This is
+ * the data gradient of Linears that are fed one tensor, dX = sum_s dY_s . W_s (q / k / v of the reference's
+ * attention block, optimus_dl/modules/model/blocks/attention.py:317-319; gate / up of its gated MLP,
+ * optimus_dl/modules/model/blocks/mlp.py:76-78): te.pytorch.Linear computes one dgrad per Linear and autograd
+ * adds them up; here the streaming kernel runs the contraction through all pairs on one set of accumulators,
+ * multiplying them by (scale product of pair s) / (scale product of pair s + 1) where it passes from one pair
+ * to the next, and applies the last pair's scale product in its epilogue:
+ *   C = round(((acc_0 r_0 + acc_1) r_1 + ... + acc_last) s_last), every step in fp32, ONE rounding to out_dtype.
+ * That route is taken for 2 .. 4 pairs with M % 128 == 0, N % 128 == 0, every K[s] % 256 == 0 and >= 512 and
+ * every operand under 2 GiB.  Anything else (up to 64 pairs, K[s] % 16 == 0) runs as one odl_fp8_gemm_nt per
+ * pair, the second and later ones with accumulate set: one rounding to out_dtype per pair.  The two routes
+ * agree within those roundings and bit for bit where every partial sum and every scale ratio is exact
+ * (powers of two).
+ */
+int odl_fp8_gemm_nt_sum(int pairs, const uint8_t *const *a, const uint8_t *const *b, const int64_t *K,
+                        int64_t M, int64_t N, int fmt_a, int fmt_b, const float *const *sa_inv,
+                        const float *const *sb_inv, void *c, int out_dtype, odl_stream_t stream);
+
+/*
  * The same product for operands that need no transposed copy.  layout_a / layout_b say how an
  * operand is stored: ODL_K_FAST = [rows, K] row-major (what odl_fp8_gemm_nt takes), ODL_K_SLOW =
  * [K, rows] row-major.  With per-tensor scaling the three GEMMs of te.pytorch.Linear then read the

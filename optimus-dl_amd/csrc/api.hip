@@ -41,7 +41,7 @@ int device_cu_count() {
 
 }  // namespace odl
 
-extern "C" int odl_fp8_abi_version(void) { return 15; }
+extern "C" int odl_fp8_abi_version(void) { return 16; }
 
 extern "C" int odl_fp8_init_device(void) {
     if (!odl::scratch_for_current_device("odl_fp8_init_device")) return ODL_ERR_LAUNCH;

@@ -33,6 +33,16 @@ struct GemmArgs {
     const uint8_t *mx_sa = nullptr, *mx_sb = nullptr;
 };
 
+// A contraction that runs over several operand pairs (streaming kernel only):
+// C = sum_s (A_s . B_s^T) * (sa_s * sb_s), A_s [M, k[s]] and B_s [N, k[s]] with the contraction index fast, one scale per
+// operand.  Passed beside GemmArgs, whose a, b, sa, sb and K are then not read.
+struct GemmPairs {
+    int count = 0;
+    int k[4] = {0, 0, 0, 0};
+    const uint8_t *a[4] = {nullptr, nullptr, nullptr, nullptr}, *b[4] = {nullptr, nullptr, nullptr, nullptr};
+    const float *sa[4] = {nullptr, nullptr, nullptr, nullptr}, *sb[4] = {nullptr, nullptr, nullptr, nullptr};
+};
+
 __device__ __forceinline__ int swz(int row) { return (row ^ (row >> 3)) & 7; }
 
 // D[i][j] += sum_k first[i][k] * second[j][k]; lane l supplies row l%32 and 32 K-bytes
@@ -250,6 +260,8 @@ void launch_gemm_tiled(int variant, int fa, int fb, const GemmArgs &g, hipStream
 void launch_gemm_pipe(int fa, int fb, const GemmArgs &g, int num_cus, hipStream_t stream);
 bool gemm_stream_accepts(const GemmArgs &g);
 void launch_gemm_stream(int fa, int fb, const GemmArgs &g, int num_cus, hipStream_t stream);
+bool gemm_stream_accepts_pairs(const GemmArgs &g, const GemmPairs &pairs);
+void launch_gemm_stream_pairs(int fa, int fb, const GemmArgs &g, const GemmPairs &pairs, int num_cus, hipStream_t stream);
 // gemm_fp8.hip: hands the calling thread's clock-probe record (odl_fp8_gemm_set_clock_probe), if any, to a streaming launch
 void attach_clock_probe(GemmArgs &g);
 // gemm_fp8.hip: out = (sum of the `splits` fp32 partial results in `workspace`, in split order) * (sa x sb) (+ bias), one rounding

@@ -247,6 +247,55 @@ extern "C" int odl_fp8_gemm_nt(const uint8_t *a, const uint8_t *b, int64_t M, in
     return check_launch("odl_fp8_gemm_nt");
 }
 
+extern "C" int odl_fp8_gemm_nt_sum(int pairs, const uint8_t *const *a, const uint8_t *const *b, const int64_t *K, int64_t M, int64_t N,
+                                   int fmt_a, int fmt_b, const float *const *sa_inv, const float *const *sb_inv, void *c,
+                                   int out_dtype, odl_stream_t stream_) {
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    if (pairs < 1 || pairs > 64) return set_error(ODL_ERR_ARG, "odl_fp8_gemm_nt_sum: %d operand pairs (1 .. 64)", pairs);
+    if (!a || !b || !K || !sa_inv || !sb_inv || !c) return set_error(ODL_ERR_ARG, "odl_fp8_gemm_nt_sum: null pointer");
+    if (M < 0 || N < 0) return set_error(ODL_ERR_ARG, "odl_fp8_gemm_nt_sum: negative size");
+    if ((fmt_a != ODL_FP8_E4M3 && fmt_a != ODL_FP8_E5M2) || (fmt_b != ODL_FP8_E4M3 && fmt_b != ODL_FP8_E5M2))
+        return set_error(ODL_ERR_ARG, "odl_fp8_gemm_nt_sum: formats %d, %d", fmt_a, fmt_b);
+    if (out_dtype != ODL_BF16 && out_dtype != ODL_F32) return set_error(ODL_ERR_ARG, "odl_fp8_gemm_nt_sum: out_dtype %d", out_dtype);
+    for (int s = 0; s < pairs; ++s) {
+        if (!a[s] || !b[s] || !sa_inv[s] || !sb_inv[s]) return set_error(ODL_ERR_ARG, "odl_fp8_gemm_nt_sum: null pointer in pair %d", s);
+        if (K[s] <= 0 || K[s] % 16 != 0)
+            return set_error(ODL_ERR_SHAPE, "odl_fp8_gemm_nt_sum: K[%d]=%lld must be a positive multiple of 16", s, (long long)K[s]);
+        if ((reinterpret_cast<uintptr_t>(a[s]) & 15) || (reinterpret_cast<uintptr_t>(b[s]) & 15))
+            return set_error(ODL_ERR_SHAPE, "odl_fp8_gemm_nt_sum: operands must be 16-byte aligned (pair %d)", s);
+    }
+    if (reinterpret_cast<uintptr_t>(c) & 15) return set_error(ODL_ERR_SHAPE, "odl_fp8_gemm_nt_sum: output must be 16-byte aligned");
+    if (M == 0 || N == 0) return ODL_OK;
+
+    // one launch of the streaming kernel when every pair suits it ...
+    if (pairs <= 4 && (t_forced_variant < 0 || t_forced_variant == kStreamVariant)) {
+        GemmArgs g;
+        GemmPairs gp;
+        g.a = a[0]; g.b = b[0]; g.c = c; g.sa = sa_inv[0]; g.sb = sb_inv[0]; g.bias = nullptr;
+        g.M = M; g.N = N; g.K = K[0];
+        g.sa_vec = 0; g.sb_vec = 0;
+        g.out_dtype = out_dtype;
+        g.tiles_m = (int)((M + 255) / 256); g.tiles_n = (int)((N + 255) / 256);
+        gp.count = pairs;
+        bool fits = true;
+        for (int s = 0; s < pairs; ++s) {
+            fits = fits && K[s] < 2147483648LL;
+            gp.k[s] = (int)K[s]; gp.a[s] = a[s]; gp.b[s] = b[s]; gp.sa[s] = sa_inv[s]; gp.sb[s] = sb_inv[s];
+        }
+        if (fits && (pairs > 1 || t_forced_variant == kStreamVariant) && gemm_stream_accepts_pairs(g, gp)) {
+            launch_gemm_stream_pairs(fmt_a, fmt_b, g, gp, cu_count(), stream);
+            return check_launch("odl_fp8_gemm_nt_sum");
+        }
+    }
+    // ... otherwise a GEMM per pair, the second and later ones adding into C (one rounding to the output type per pair)
+    for (int s = 0; s < pairs; ++s) {
+        const int rc = odl_fp8_gemm_nt(a[s], b[s], M, N, K[s], fmt_a, fmt_b, sa_inv[s], 1, sb_inv[s], 1, nullptr, ODL_F32, c, out_dtype,
+                                       s > 0, stream_);
+        if (rc != ODL_OK) return rc;
+    }
+    return ODL_OK;
+}
+
 extern "C" int odl_fp8_gemm_layouts(const uint8_t *a, const uint8_t *b, int64_t M, int64_t N, int64_t K, int fmt_a, int fmt_b,
                                     int layout_a, int layout_b, const float *sa_inv, const float *sb_inv, void *c,
                                     int out_dtype, odl_stream_t stream_) {

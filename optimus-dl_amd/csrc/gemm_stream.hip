@@ -51,6 +51,8 @@
 // multiply the fragments of the first again, which halves the LDS-to-register traffic.
 #include "gemm_common.h"
 
+#include <type_traits>
+
 namespace odl {
 
 namespace {
@@ -88,9 +90,16 @@ __device__ __forceinline__ v16f mma_step(const v8i &b, const v8i &a, const v16f 
     else return mfma_32x32x64<FB, FA>(b, a, c);
 }
 
-template <int FA, int FB, bool TA, bool TB, bool F32, int EPI, bool MX = false>
-__global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
+// SEG: the contraction runs over gp.count operand pairs with a scale product each (the data gradients of Linears that are
+// fed one tensor: dX = sum_s dY_s . W_s).  A block stays on its tile through all pairs; the load pipeline crosses from one
+// pair to the next exactly as it crosses from one tile to the next (other descriptors, other row pitch), and where a tile
+// ends with a fold, a pair ends with the accumulators multiplied by (scale product of this pair) / (that of the next)
+// under the first MFMAs of the next pair.  After the last pair the fold applies the last pair's scale product, so
+// C = ((acc_0 r_0 + acc_1) r_1 + ...) s_last in fp32 with one rounding to the output type.
+template <int FA, int FB, bool TA, bool TB, bool F32, int EPI, bool MX, bool SEG>
+__device__ __forceinline__ void gemm_nt_stream_body(const GemmArgs &g, const GemmPairs &gp) {
     static_assert(!MX || (!TA && !TB && EPI != 1), "block scales: both operands stored [rows, K], no scale vectors");
+    static_assert(!SEG || (!TA && !TB && EPI == 0 && !MX), "operand pairs: both stored [rows, K], one scale each");
     constexpr int ESZ = F32 ? 4 : 2;
     constexpr int VEC_BYTES = 3 * 128 * 4;     // per wave: 128 row scales, 128 column scales, 128 bias values
     __shared__ __attribute__((aligned(1024))) uint8_t sA0[REGION];
@@ -100,6 +109,7 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
     __shared__ __attribute__((aligned(16))) uint8_t sEpi[NW * SLAB];
     __shared__ __attribute__((aligned(16))) uint8_t sVec[EPI > 0 ? NW * VEC_BYTES : 16];
     __shared__ __attribute__((aligned(16))) uint32_t sScale[MX ? 2 * 512 : 4];     // [stage][A rows 0..255 | B rows 0..255], permuted
+    __shared__ float sRatio[4];
 
     const int lane = threadIdx.x % 64;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
@@ -150,9 +160,9 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
         tn0 = __builtin_amdgcn_readfirstlane(((p % in_group) / group_rows) * BN);
     };
     // descriptor of an operand for the tile rows from row0 on and the K steps from first_step on
-    auto rsrc_for = [&](const uint8_t *base, int row0, int64_t rows, bool transposed, int first_step) -> v4i {
+    auto rsrc_for = [&](const uint8_t *base, int row0, int64_t rows, bool transposed, int first_step, int nk) -> v4i {
         // an operand is smaller than 2 GiB (checked by the caller): 32-bit products, which stay scalar
-        const int k0 = first_step * 128, nrows = (int)rows, nk = (int)g.K;
+        const int k0 = first_step * 128, nrows = (int)rows;
         if (transposed) {                          // [K, rows] storage: the tile starts at column row0 of K-row k0
             const uint64_t addr = reinterpret_cast<uint64_t>(base) + (uint32_t)(k0 * nrows + row0);
             return v4i{(int)(uint32_t)addr, (int)(uint32_t)(addr >> 32), (nk - k0) * nrows - row0, 0x00020000};
@@ -165,12 +175,20 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
 #pragma unroll
     for (int j = 0; j < LOADS; ++j) {
         const int row = (wave + j * NW) * 8 + lane / 8;                   // K fast: 8 rows of 128 bytes per load
-        const int nt = row * (int)g.K + (((lane % 8) ^ swz(row)) << 4);
+        const int nt = row * (SEG ? gp.k[0] : (int)g.K) + (((lane % 8) ^ swz(row)) << 4);
         const int kb = (wave + j * NW) * 4 + lane / 16;                   // K slow: 4 K-rows of 256 bytes per load
         const int chunk = ((lane % 16) ^ ((kb & 7) << 1)) << 4;
         voff_a[j] = TA ? kb * (int)g.M + chunk : nt;
         voff_b[j] = TB ? kb * (int)g.N + chunk : nt;
     }
+    // SEG: the same offsets for operands of another row length (both stored [rows, K])
+    auto set_voffs = [&](int nk) {
+#pragma unroll
+        for (int j = 0; j < LOADS; ++j) {
+            const int row = (wave + j * NW) * 8 + lane / 8;
+            voff_a[j] = voff_b[j] = row * nk + (((lane % 8) ^ swz(row)) << 4);
+        }
+    };
     const int kstep_a = TA ? 128 * (int)g.M : 128, kstep_b = TB ? 128 * (int)g.N : 128;   // bytes between K steps
     // one 1 KB direct-to-LDS load: 64 lanes x 16 bytes land at lds_addr + lane * 16
     auto dma = [&](const v4i &rsrc, uint32_t lds_addr, int vo, int so) {
@@ -305,8 +323,16 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
     // ---- output side of the folded epilogue
     const int n2 = (int)g.N * ESZ;                // bytes per output row
     const int c_soff0 = (wm0 * (int)g.N + wn0) * ESZ;
+    auto uniform = [](float v) { return bits_to_float((uint32_t)__builtin_amdgcn_readfirstlane((int)float_to_bits(v))); };
+    // SEG: between pair s and s + 1 the accumulators take sRatio[s] = (scale product of s) / (that of s + 1); kept in
+    // LDS (read once per pair) rather than in scalar registers, of which the K loop leaves none to spare
+    if constexpr (SEG) {
+        const int s = (int)threadIdx.x;
+        if (s + 1 < gp.count) sRatio[s] = (gp.sa[s][0] * gp.sb[s][0]) / (gp.sa[s + 1][0] * gp.sb[s + 1][0]);
+        // (first read after the K loop of the first pair, many barriers from here)
+    }
     const float s_tensor = g.splits > 1 ? 1.0f :       // partial results leave unscaled
-        bits_to_float((uint32_t)__builtin_amdgcn_readfirstlane((int)float_to_bits(g.sa[0] * g.sb[0])));
+        SEG ? uniform(gp.sa[gp.count - 1][0] * gp.sb[gp.count - 1][0]) : uniform(g.sa[0] * g.sb[0]);
     // M and N are multiples of 128 = the wave tile: in the last tile row / column of a matrix that is not a
     // multiple of 256 a wave is either wholly inside or wholly outside.  One that is outside computes on the
     // zeros that the bounded operand loads deliver and stores through the empty descriptor (nothing is written).
@@ -359,6 +385,24 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             acc[i / 4][i % 4] = mma_step<FB, FA, MX, 0>(b0[i % 4], a0[i / 4], zero16, scb[0][i % 4], sca[0][i / 4]);
+            if (i < 4) a1[i] = read_a(sa_cur, i, 1);
+            else if (i < 8) b1[i - 4] = read_b(sb_cur, i - 4, 1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    // SEG, phase A of step 0 of a later operand pair of the same tile: the accumulators carry on, multiplied by the
+    // ratio of the two pairs' scale products (sub-tile i while MFMA i - 1 runs)
+    auto phase_a_rescale = [&](const uint8_t *sa_cur, const uint8_t *sb_cur, const int pair) {
+        const float ratio = sRatio[pair];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            // (the statement makes this read of the accumulators another one than the fold's, for the compiler: it would
+            // otherwise read them out once, ahead of the branch between the two, into registers that do not exist)
+            asm volatile("" : "+a"(acc[i / 4][i % 4]));
+            v16f carried;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) carried[e] = acc[i / 4][i % 4][e] * ratio;
+            acc[i / 4][i % 4] = mma_step<FB, FA, MX, 0>(b0[i % 4], a0[i / 4], carried, scb[0][i % 4], sca[0][i / 4]);
             if (i < 4) a1[i] = read_a(sa_cur, i, 1);
             else if (i < 8) b1[i - 4] = read_b(sb_cur, i - 4, 1);
             __builtin_amdgcn_sched_barrier(0);
@@ -529,11 +573,16 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
 
     // ---- first tile: steps 0 and 1 requested and awaited, then phase A of step 0
     tile_origin(pid, m0, n0);
-    {
+    int seg = 0;                                  // SEG: the operand pair the block is on
+    if constexpr (SEG) {
+        KT = gp.k[0] / 128;                    // an even number of steps, at least 4 (checked by the caller)
+        rsrc_a = rsrc_for(gp.a[0], m0, g.M, false, 0, gp.k[0]);
+        rsrc_b = rsrc_for(gp.b[0], n0, g.N, false, 0, gp.k[0]);
+    } else {
         int first_step = 0;
         item_steps(pid, first_step, KT, padded);
-        rsrc_a = rsrc_for(g.a, m0, g.M, TA, first_step);
-        rsrc_b = rsrc_for(g.b, n0, g.N, TB, first_step);
+        rsrc_a = rsrc_for(g.a, m0, g.M, TA, first_step, (int)g.K);
+        rsrc_b = rsrc_for(g.b, n0, g.N, TB, first_step, (int)g.K);
         if constexpr (MX) scale_origin(m0, n0, first_step, sc_off_a, sc_off_b, sc_in_a, sc_in_b);
     }
     next_a = empty;
@@ -557,18 +606,26 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
     for (int u = 0; u < TN; ++u) b0[u] = read_b(sB0, u, 0);
     phase_a_first(sA0, sB0);
 
-    while (true) {
-        // the block's next tile, if any (scalar work only; no branches around vector code)
-        const int next_pid = pid + stride;
+    // One trip: the rest of the current item (a tile; SEG: one operand pair of a tile) and phase A of the next.
+    // ENDS: the item ends its tile (always, without SEG).  -> whether the block has another item.
+    auto trip = [&](auto ends_tile) -> bool {
+        constexpr bool tile_ends = decltype(ends_tile)::value;
+        // the block's next tile, if any (scalar work only; no branches around vector code).  SEG: the next operand pair
+        // of this tile, or the first pair of the next tile
+        const int next_seg = tile_ends ? 0 : seg + 1;
+        const int next_pid = tile_ends ? pid + stride : pid;
         const bool has_next = next_pid < pid_end;
         int next_m0 = 0, next_n0 = 0, next_first = 0, next_kt = 0;
         bool next_padded = false;
         tile_origin(has_next ? next_pid : pid, next_m0, next_n0);
-        item_steps(has_next ? next_pid : pid, next_first, next_kt, next_padded);
+        const int next_nk = SEG ? gp.k[next_seg] : (int)g.K;
+        if constexpr (SEG) next_kt = next_nk / 128;
+        else item_steps(has_next ? next_pid : pid, next_first, next_kt, next_padded);
+        const uint8_t *const base_a = SEG ? gp.a[next_seg] : g.a, *const base_b = SEG ? gp.b[next_seg] : g.b;
 #ifdef ODL_EXP_SAME_PANELS            // experiment: every tile reads the operand panels of tile (0, 0): all traffic stays in the L2
-        const v4i na = rsrc_for(g.a, 0, g.M, TA, next_first), nb = rsrc_for(g.b, 0, g.N, TB, next_first);
+        const v4i na = rsrc_for(base_a, 0, g.M, TA, next_first, next_nk), nb = rsrc_for(base_b, 0, g.N, TB, next_first, next_nk);
 #else
-        const v4i na = rsrc_for(g.a, next_m0, g.M, TA, next_first), nb = rsrc_for(g.b, next_n0, g.N, TB, next_first);
+        const v4i na = rsrc_for(base_a, next_m0, g.M, TA, next_first, next_nk), nb = rsrc_for(base_b, next_n0, g.N, TB, next_first, next_nk);
 #endif
         next_a = has_next ? na : empty;
         next_b = has_next ? nb : empty;
@@ -581,13 +638,17 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
         // ---- rest of step 0 (its phase A ran at the end of the previous trip), then steps 1 .. KT-1.
         // The first trip's step 0 and every drained tile's step 0 carry 32 stores (dropped ones
         // count too), the first tile's none: vmcnt(32) is then simply satisfied earlier.
-        sync(true);
+        // SEG: a later pair of a tile follows a rescale, which stores nothing: every load must have landed
+        if (SEG && seg > 0) sync(false);
+        else sync(true);
         phase_b(sA0, sB0, sA1, sB1, 0, 0);
         step(sA1, sB1, sA0, sB0, 1, 1);
         for (int kt = 2; kt < KT - 2; kt += 2) {
             step(sA0, sB0, sA1, sB1, kt, 0);
             step(sA1, sB1, sA0, sB0, kt + 1, 1);
         }
+        // the two steps that follow request the next item's first two: its row pitch from here on
+        if constexpr (SEG) set_voffs(next_nk);
         step(sA0, sB0, sA1, sB1, KT - 2, 0);
         if constexpr (EPI > 0) request_vectors(m0, n0);
         step(sA1, sB1, sA0, sB0, KT - 1, 1);
@@ -607,13 +668,38 @@ __global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
         sc_off_b = sc_next_b;
         sc_in_a = sc_nin_a;
         sc_in_b = sc_nin_b;
-        phase_a_fold(sA0, sB0, rsrc_c);
-        if (!has_next) break;
+        const int pair = seg;
+        seg = next_seg;
+        if constexpr (tile_ends) phase_a_fold(sA0, sB0, rsrc_c);
+        else phase_a_rescale(sA0, sB0, pair);
+        return has_next;
+    };
+    if constexpr (SEG) {
+        // two copies of the trip, one ending in the rescale and one in the fold, instead of a branch between the two at
+        // the end of one: with the branch the compiler does not keep the accumulators where they are (it spills them)
+        while (true) {
+            while (seg + 1 < gp.count) trip(std::false_type{});
+            if (!trip(std::true_type{})) break;
+        }
+    } else {
+        while (trip(std::true_type{})) {
+        }
     }
     if (stamps) {
         g.clock_out[2] = clock64();
         g.clock_out[3] = wall_clock64();
     }
+}
+
+template <int FA, int FB, bool TA, bool TB, bool F32, int EPI, bool MX = false>
+__global__ __launch_bounds__(256) void gemm_nt_stream_kernel(const GemmArgs g) {
+    gemm_nt_stream_body<FA, FB, TA, TB, F32, EPI, MX, false>(g, GemmPairs{});
+}
+
+// the same kernel over several operand pairs (see SEG above)
+template <int FA, int FB, bool F32>
+__global__ __launch_bounds__(256) void gemm_nt_stream_pairs_kernel(const GemmArgs g, const GemmPairs gp) {
+    gemm_nt_stream_body<FA, FB, false, false, F32, 0, false, true>(g, gp);
 }
 
 template <int FA, int FB, bool F32>
@@ -650,6 +736,21 @@ bool gemm_stream_accepts(const GemmArgs &g) {
            g.M % (g.ta ? BM : WM) == 0 && g.N % (g.tb ? BN : WN) == 0 && g.K % 128 == 0 && g.K >= 512 && (double)g.N * esz * (BM + 8) < 2147483648.0;
 }
 
+// Operand pairs: each a whole even number of K steps, four at least (the load pipeline is two steps deep and crosses
+// from one pair to the next in its last two), every operand addressed with 32-bit byte offsets.
+bool gemm_stream_accepts_pairs(const GemmArgs &g, const GemmPairs &gp) {
+    const double esz = g.out_dtype == ODL_F32 ? 4.0 : 2.0;
+    if (gp.count < 1 || gp.count > 4 || g.accumulate || g.ta || g.tb || g.sa_vec || g.sb_vec || g.bias || g.mx_sa || g.mx_sb || g.splits > 1)
+        return false;
+    for (int s = 0; s < gp.count; ++s) {
+        const int k = gp.k[s];
+        if (!gp.a[s] || !gp.b[s] || !gp.sa[s] || !gp.sb[s] || k < 512 || k % 256 != 0) return false;
+        if ((double)(g.M + 256) * k >= 2147483648.0 || (double)(g.N + 256) * k >= 2147483648.0) return false;
+    }
+    return (g.out_dtype == ODL_BF16 || g.out_dtype == ODL_F32) && g.M > 0 && g.N > 0 && g.M % WM == 0 && g.N % WN == 0 &&
+           (double)g.N * esz * (BM + 8) < 2147483648.0;
+}
+
 // One block per CU at most (the kernel needs ~150 KB of LDS), 8 | grid so that the
 // round-robin placement gives every XCD the same number of blocks.
 void launch_gemm_stream(int fa, int fb, const GemmArgs &args, int num_cus, hipStream_t stream) {
@@ -667,6 +768,31 @@ void launch_gemm_stream(int fa, int fb, const GemmArgs &args, int num_cus, hipSt
     else if (fa == ODL_FP8_E5M2 && fb == ODL_FP8_E4M3) launch_fmt<ODL_FP8_E5M2, ODL_FP8_E4M3>(g, bpx, stream);
     else if (fa == ODL_FP8_E4M3 && fb == ODL_FP8_E5M2) launch_fmt<ODL_FP8_E4M3, ODL_FP8_E5M2>(g, bpx, stream);
     else launch_fmt<ODL_FP8_E5M2, ODL_FP8_E5M2>(g, bpx, stream);
+}
+
+namespace {
+
+template <int FA, int FB>
+void launch_pairs_fmt(const GemmArgs &g, const GemmPairs &gp, int blocks_per_xcd, hipStream_t stream) {
+    const dim3 grid((unsigned)(8 * blocks_per_xcd)), block(256);
+    if (g.out_dtype == ODL_F32) hipLaunchKernelGGL((gemm_nt_stream_pairs_kernel<FA, FB, true>), grid, block, 0, stream, g, gp);
+    else hipLaunchKernelGGL((gemm_nt_stream_pairs_kernel<FA, FB, false>), grid, block, 0, stream, g, gp);
+}
+
+}  // namespace
+
+void launch_gemm_stream_pairs(int fa, int fb, const GemmArgs &args, const GemmPairs &gp, int num_cus, hipStream_t stream) {
+    GemmArgs g = args;
+    g.splits = 1;
+    g.split_steps = 0;
+    const int per_xcd = (g.tiles_m * g.tiles_n + 7) / 8;
+    int bpx = num_cus / 8;
+    if (bpx < 1) bpx = 1;
+    if (bpx > per_xcd) bpx = per_xcd;
+    if (fa == ODL_FP8_E4M3 && fb == ODL_FP8_E4M3) launch_pairs_fmt<ODL_FP8_E4M3, ODL_FP8_E4M3>(g, gp, bpx, stream);
+    else if (fa == ODL_FP8_E5M2 && fb == ODL_FP8_E4M3) launch_pairs_fmt<ODL_FP8_E5M2, ODL_FP8_E4M3>(g, gp, bpx, stream);
+    else if (fa == ODL_FP8_E4M3 && fb == ODL_FP8_E5M2) launch_pairs_fmt<ODL_FP8_E4M3, ODL_FP8_E5M2>(g, gp, bpx, stream);
+    else launch_pairs_fmt<ODL_FP8_E5M2, ODL_FP8_E5M2>(g, gp, bpx, stream);
 }
 
 }  // namespace odl

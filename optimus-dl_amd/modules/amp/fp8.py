@@ -219,6 +219,9 @@ class FP8Recipe:
         # Linears fed by one tensor (q/k/v, gate/up) run as one autograd node whose data gradients are summed by the
         # GEMMs' accumulate flag (modules/fp8_linear.py: linear_group, SiblingGroup); False: every Linear on its own
         self.fuse_dgrad_sum = True
+        # ... and by ONE GEMM that runs its contraction through all members' operands where the shapes allow
+        # (native.gemm_nt_sum: no read-modify-write of dx per further member); False: always the accumulate flag
+        self.fuse_dgrad_gemm = True
         self._sibling_groups: "weakref.WeakSet" = weakref.WeakSet()
         # Gradient accumulation over microbatches (the reference's acc_steps > 1): with this set, a weight gradient is
         # added straight into an existing ``weight.grad`` by the GEMM and autograd is handed None for it, instead

@@ -322,10 +322,14 @@ class _Fp8LinearFn(torch.autograd.Function):
                     gq, gq_t, sg_inv, _ = _quantise_dynamic(dy2d, pol.fmt_bwd, pol.margin, g_t_needed, g_rm_needed,
                                                             parts=parts, out_t=gq_t_out)
             if ctx.need_dgrad:
-                # a member of a group of Linears fed by one tensor adds its share into the group's gradient
-                # (the GEMM's accumulate flag) instead of leaving the sum to a separate pass
+                # a member of a group of Linears fed by one tensor leaves its operands to the group's one GEMM over
+                # all members, or adds its share into the group's gradient (the GEMM's accumulate flag), instead of
+                # leaving the sum to a separate pass
+                dx_pairs = getattr(ctx, "dx_pairs", None)
                 dx_into = getattr(ctx, "dx_into", None)
-                if dx_into is not None:
+                if dx_pairs is not None:
+                    dx_pairs.append((gq, saved["wq_t"], sg_inv, saved["sw_inv_t"]))
+                elif dx_into is not None:
                     dx = native.gemm_nt(gq, saved["wq_t"], pol.fmt_bwd, pol.fmt_fwd, sg_inv, saved["sw_inv_t"],
                                         out=dx_into, accumulate=True)
                 else:
@@ -425,6 +429,25 @@ class _Fp8LinearGroupFn(torch.autograd.Function):
         return picked, torch.empty((rows, tokens), dtype=torch.uint8, device=xq_t.device), xq_t, sx_inv_t
 
     @staticmethod
+    def _dgrad_in_one_gemm(ctx, dys) -> "list | None":
+        """An empty list for the members to put their dgrad operands in (codes of dy, codes of W^T, the two inverse
+        scales) where ONE GEMM computes dx = sum over members of dy_s . W_s (``native.gemm_nt_sum``), else None: the
+        members then add into dx one by one.  One launch where per-tensor scales and the shapes allow: the k and v
+        shares of a grouped-query block (contractions of 1024) are, added into a cold 64 MB dx, bound by reading and
+        writing it (63 us each at 8192 tokens against 40 for the bare product); carried through one set of
+        accumulators they cost what their share of the contraction costs."""
+        recipe = ctx.subs[0].recipe
+        if not getattr(recipe, "fuse_dgrad_gemm", True) or recipe.recipe.kind not in ("tensorwise", "delayed"):
+            return None
+        live = [sub for sub, dy in zip(ctx.subs, dys) if dy is not None and sub.need_dgrad]
+        if len(live) < 2 or any(dy is not None and not sub.need_dgrad for sub, dy in zip(ctx.subs, dys)):
+            return None
+        tokens = next(dy for dy in dys if dy is not None).shape[0]
+        if not native.dgrad_sum_in_one_launch(tokens, live[0].module.in_features, [sub.module.out_features for sub in live]):
+            return None
+        return []
+
+    @staticmethod
     def backward(ctx, *dys: torch.Tensor | None):
         tensors = ctx.saved_tensors
         dx = None
@@ -436,17 +459,25 @@ class _Fp8LinearGroupFn(torch.autograd.Function):
                 n = ctx.subs[i].module.out_features
                 ctx.subs[i].wgrad_joint = {"codes_t": joint[1][at:at + n], "rows": (at, at + n)}
                 at += n
+        dx_pairs = _Fp8LinearGroupFn._dgrad_in_one_gemm(ctx, dys)
         for sub, (first, count), dy in zip(ctx.subs, ctx.spans, dys):
             if dy is None:                       # this member's output did not reach the loss
                 grads += [None, None]
                 continue
             sub.saved_tensors = tensors[first:first + count]
+            sub.dx_pairs = dx_pairs
             sub.dx_into = dx if (dx is not None and sub.need_dgrad) else None
             dxi, dw, db, _, _, _ = _Fp8LinearFn.backward(sub, dy)
             sub.saved_tensors = ()
+            sub.dx_pairs = None
             if dxi is not None and dx is None:
                 dx = dxi
             grads += [dw, db]
+        if dx_pairs:
+            pol = ctx.subs[0].recipe.recipe
+            gqs, wq_ts, sg_invs, sw_invs = zip(*dx_pairs)
+            dx = native.gemm_nt_sum(list(gqs), list(wq_ts), pol.fmt_bwd, pol.fmt_fwd, list(sg_invs), list(sw_invs),
+                                    out_dtype=ctx.subs[0].x_dtype)
         if joint is not None:
             picked, codes_t, xq_t, sx_inv_t = joint
             pol = ctx.subs[0].recipe.recipe

@@ -24,7 +24,7 @@ DT_BF16, DT_F32 = 0, 1
 AMAX_MAX, AMAX_MOST_RECENT = 0, 1
 FP8_MAX = {E4M3: 448.0, E5M2: 57344.0}
 TORCH_FP8 = {E4M3: torch.float8_e4m3fn, E5M2: torch.float8_e5m2}
-ABI_VERSION = 15
+ABI_VERSION = 16
 AMAX_PARTS = 512                       # ODL_FP8_AMAX_PARTS
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
@@ -61,6 +61,7 @@ EXPORTS = (
     "odl_fp8_cast_transpose",
     "odl_fp8_cast_delayed",
     "odl_fp8_gemm_nt",
+    "odl_fp8_gemm_nt_sum",
     "odl_fp8_gemm_layouts",
     "odl_fp8_gemm_split_count",
     "odl_fp8_gemm_splitk",
@@ -132,6 +133,7 @@ def load() -> ctypes.CDLL:
         L.odl_fp8_cast_transpose.argtypes = [vp, i32, i64, i64, vp, i32, i32, vp, vp, vp, vp]
         L.odl_fp8_cast_delayed.argtypes = [vp, i32, i64, i64, vp, i32, vp, vp, vp, vp, vp]
         L.odl_fp8_gemm_nt.argtypes = [vp, vp, i64, i64, i64, i32, i32, vp, i64, vp, i64, vp, i32, vp, i32, i32, vp]
+        L.odl_fp8_gemm_nt_sum.argtypes = [i32, vp, vp, vp, i64, i64, i32, i32, vp, vp, vp, i32, vp]
         L.odl_fp8_gemm_layouts.argtypes = [vp, vp, i64, i64, i64, i32, i32, i32, i32, vp, vp, vp, i32, vp]
         L.odl_fp8_gemm_split_count.argtypes = [i64, i64, i64, i32]
         L.odl_fp8_gemm_split_count.restype = i32
@@ -773,6 +775,40 @@ def gemm_nt(a: torch.Tensor, b: torch.Tensor, fmt_a: int, fmt_b: int, sa_inv: to
     return out
 
 
+def gemm_nt_sum(a: "list[torch.Tensor]", b: "list[torch.Tensor]", fmt_a: int, fmt_b: int, sa_inv: "list[torch.Tensor]",
+                sb_inv: "list[torch.Tensor]", out_dtype: torch.dtype = torch.bfloat16, out: torch.Tensor | None = None) -> torch.Tensor:
+    """out[M,N] = sum_s (a[s][M,K_s] . b[s][N,K_s]^T) * (sa_inv[s] * sb_inv[s]); uint8 FP8 codes, one scale per operand.
+    One launch where the shapes suit the streaming kernel (2 .. 4 pairs, M and N multiples of 128, every K_s a multiple
+    of 256 and at least 512), otherwise one GEMM per pair, the later ones adding into ``out``."""
+    n = len(a)
+    if n < 1 or len(b) != n or len(sa_inv) != n or len(sb_inv) != n:
+        raise NativeError(f"gemm_nt_sum: {len(a)} / {len(b)} operands, {len(sa_inv)} / {len(sb_inv)} scales")
+    if out is not None:
+        out_dtype = out.dtype
+    odt = DT_BF16 if out_dtype == torch.bfloat16 else (DT_F32 if out_dtype == torch.float32 else None)
+    if odt is None:
+        raise NativeError(f"gemm_nt_sum: output dtype {out_dtype} is not supported (bf16 or fp32)")
+    a, b = [_as_2d(t) for t in a], [_as_2d(t) for t in b]
+    M, N = a[0].shape[0], b[0].shape[0]
+    for s in range(n):
+        if a[s].dtype != torch.uint8 or b[s].dtype != torch.uint8:
+            raise NativeError("gemm_nt_sum operands must be uint8 FP8 codes")
+        if a[s].shape[0] != M or b[s].shape[0] != N or a[s].shape[1] != b[s].shape[1]:
+            raise NativeError(f"gemm_nt_sum: pair {s} is {tuple(a[s].shape)} x {tuple(b[s].shape)}, expected [{M}, K] x [{N}, K]")
+        _f32_dev(sa_inv[s], 1, "gemm_nt_sum sa_inv")
+        _f32_dev(sb_inv[s], 1, "gemm_nt_sum sb_inv")
+    if out is None:
+        out = torch.empty((M, N), dtype=out_dtype, device=a[0].device)
+    elif out.shape != (M, N) or not out.is_contiguous():
+        raise NativeError("gemm_nt_sum: `out` has the wrong shape / layout")
+    ptrs = ctypes.c_void_p * n
+    ks = (ctypes.c_int64 * n)(*[t.shape[1] for t in a])
+    _check(load().odl_fp8_gemm_nt_sum(n, ptrs(*[t.data_ptr() for t in a]), ptrs(*[t.data_ptr() for t in b]), ks, M, N, fmt_a, fmt_b,
+                                      ptrs(*[t.data_ptr() for t in sa_inv]), ptrs(*[t.data_ptr() for t in sb_inv]), out.data_ptr(),
+                                      odt, _stream()), "odl_fp8_gemm_nt_sum")
+    return out
+
+
 MX_BLOCK = 32
 MX_ROWMAJOR, MX_KSTEP = 0, 1           # ODL_MX_SCALES_*
 MX_FLOOR, MX_CEIL = 0, 1               # ODL_MX_SCALE_*: shared exponent floor(log2 amax) - emax / ceil(log2(amax / fp8_max))
@@ -979,6 +1015,17 @@ def wgrad_direct_pays(n_out: int, n_in: int, tokens: int) -> bool:
     4096 x 4096 129.9 / 136.3, 2048 x 1024 54.2 / 56.2, 2304 x 768 53.8 / 58.7, 1024 x 1024 38.1 / 41.9."""
     tiles = (n_out // 256) * (n_in // 256)
     return tiles >= 192 or n_out * n_in < 2_200_000
+
+
+def dgrad_sum_in_one_launch(tokens: int, n_in: int, n_outs: "list[int]") -> bool:
+    """Whether the data gradient of Linears fed by one tensor, dX [tokens, n_in] = sum_s dY_s [tokens, n_outs[s]] . W_s, runs
+    as ONE launch of :func:`gemm_nt_sum` (the streaming kernel carrying its accumulators from one pair to the next): the
+    shapes that kernel takes, and an output of more 256 x 256 tiles than half the 256 compute units (smaller ones are better
+    served by the per-pair GEMMs that add into dX: those pick 128 x 128 tiles or split the contraction)."""
+    if not 2 <= len(n_outs) <= 4 or tokens % 128 or n_in % 128 or any(k % 256 or k < 512 for k in n_outs):
+        return False
+    tiles = ((tokens + 255) // 256) * ((n_in + 255) // 256)
+    return tiles > 128 and all((tokens + 256) * k < 2**31 and (n_in + 256) * k < 2**31 for k in n_outs)
 
 
 def gemm_layouts(a: torch.Tensor, b: torch.Tensor, fmt_a: int, fmt_b: int, layout_a: int, layout_b: int,

@@ -337,6 +337,18 @@ def t_accumulate(c_old: torch.Tensor, product_f32: torch.Tensor, bias: torch.Ten
     return (v + c_old.float()).to(c_old.dtype)
 
 
+def t_gemm_nt_sum(pairs, fmt_a, fmt_b, want_f32: bool = False):
+    """sum_s (a_s . b_s^T) * (sa_s * sb_s) over pairs (a_s, b_s, sa_inv_s, sb_inv_s): the data gradient of Linears that are
+    fed one tensor (the reference's wq / wk / wv, optimus_dl/modules/model/blocks/attention.py:317-319, and w1 / w2,
+    optimus_dl/modules/model/blocks/mlp.py:76-78, whose per-Linear data gradients autograd adds up).  Every scaled
+    product in fp32 (t_gemm_nt), added in pair order in fp32, ONE rounding to bf16."""
+    total = None
+    for a, b, sa_inv, sb_inv in pairs:
+        part = t_gemm_nt(a, b, fmt_a, fmt_b, sa_inv, sb_inv, want_f32=True)[1]
+        total = part if total is None else total + part
+    return (total.bfloat16(), total) if want_f32 else total.bfloat16()
+
+
 # -------------------------------------------------- the Linear, end to end (torch)
 def linear_fwd_bwd(x, w, dy, fmt_fwd=E4M3, fmt_bwd=E5M2, rowwise=False, scales=None):
     """One FP8 Linear forward + backward on CPU with dynamic scaling.

@@ -173,3 +173,64 @@ def test_fused_wgrad_accumulation_over_microbatches(amp, wdtype):
         # four roundings to bf16 of running sums on either route: a few units of the largest intermediate value apart
         assert (ga.float() - gb.float()).abs().max().item() <= 2.0 ** -6 * ga.float().abs().max().item()
     assert torch.equal(lin_a.bias.grad, lin_b.bias.grad)
+
+
+class WideAttn(nn.Module):
+    """The same three projections at a size whose data gradient fills the chip with 256 x 256 tiles."""
+
+    def __init__(self, d=2304, q=1024, kv=512):
+        super().__init__()
+        self.wq, self.wk, self.wv = nn.Linear(d, q, bias=False), nn.Linear(d, kv, bias=False), nn.Linear(d, kv, bias=False)
+
+    def forward(self, x):
+        return self.wq(x), self.wk(x), self.wv(x)
+
+
+def build_wide(group=True):
+    from optimus_dl_amd.modules.model_transforms import build_model_transform
+
+    torch.manual_seed(1)
+    net = WideAttn().to("cuda", torch.bfloat16)
+    build_model_transform({"_name": "fp8_linear"} if group else {"_name": "fp8_linear", "group_siblings": ()}).apply(net)
+    return net
+
+
+@pytest.mark.parametrize("kind", ["tensorwise", "delayed"])
+def test_sibling_group_data_gradient_from_one_gemm(amp, kind, monkeypatch):
+    """4096 tokens x 2304 features (144 tiles): the group's data gradient comes from ONE launch over the three members'
+    operands (no GEMM with the accumulate flag, no dgrad of a member's own), outputs and weight gradients are the bits of
+    the separate Linears, and the data gradient lies as close to the fp32 sum of the three products as the sum that the
+    accumulate flag forms (``fuse_dgrad_gemm = False``) and as the one autograd forms, or closer."""
+    from optimus_dl_amd import native as N
+
+    kw = {"amax_history_len": 4} if kind == "delayed" else {}
+    grouped, stepwise, plain = build_wide(), build_wide(), build_wide(False)
+    r1, r2, r3 = (amp.create_fp8_recipe(kind, "hybrid", **kw) for _ in range(3))
+    r2.fuse_dgrad_gemm = False
+    sums, accs = [], []
+    real_sum, real_nt = N.gemm_nt_sum, N.gemm_nt
+    monkeypatch.setattr(N, "gemm_nt_sum", lambda *a, **k: (sums.append(len(a[0])), real_sum(*a, **k))[1])
+    monkeypatch.setattr(N, "gemm_nt", lambda *a, **k: (accs.append(bool(k.get("accumulate", False))), real_nt(*a, **k))[1])
+    x = seeded_bf16((4096, 2304), 1.0, 900).cuda()
+    dys = [seeded_bf16((4096, n), 1e-3 * (4.0 ** i), 910 + i).cuda() for i, n in enumerate((1024, 512, 512))]
+    got = run(grouped, r1, x, dys)
+    assert sums == [3] and accs.count(True) == 0
+    sums.clear(); accs.clear()
+    mid = run(stepwise, r2, x, dys)
+    assert sums == [] and accs.count(True) == 2
+    want = run(plain, r3, x, dys)
+    for a, b in zip(got[0] + got[2], want[0] + want[2]):
+        assert torch.equal(a, b)
+    if kind == "tensorwise":
+        probe, rp = build_wide(False), amp.create_fp8_recipe(kind, "hybrid")
+        parts = []
+        for i in range(3):
+            sel = [dys[j] if j == i else torch.zeros_like(dys[j]) for j in range(3)]
+            parts.append(run(probe, rp, x, sel)[1].float())
+        exact = parts[0] + parts[1] + parts[2]                      # (each part rounded to bf16 once: 2^-9 relative)
+        err = lambda t: (t.float() - exact).abs().max().item()
+        assert err(got[1]) <= err(mid[1]) * 1.05 + 1e-12 and err(got[1]) <= err(want[1]) * 1.05 + 1e-12
+        bound = (parts[0].abs() + parts[1].abs() + parts[2].abs()) * 2.0 ** -6 + 1e-12
+        assert bool(((got[1].float() - exact).abs() <= bound).all())
+    else:
+        assert (got[1].float() - want[1].float()).abs().max().item() <= 3 * 2.0 ** -8 * want[1].float().abs().max().item()

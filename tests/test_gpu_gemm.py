@@ -551,3 +551,106 @@ def test_accumulate_through_split_k_and_k_slow_layouts(N):
     assert max_rel_err(c, want) <= 1e-4
     with pytest.raises(N.NativeError):
         N.gemm_nt(aq.cuda(), bq.cuda(), O.E5M2, O.E4M3, sa_inv.cuda(), sb_inv.cuda(), accumulate=True)      # nothing to add into
+
+
+# ---------------------------------------------------------------- sums of products in one launch (odl_fp8_gemm_nt_sum)
+def _pow2_pairs(M, Nn, ks, seed):
+    g = torch.Generator().manual_seed(seed)
+    vals = torch.tensor([0.0, 1.0, -1.0, 2.0, -2.0, 0.5, -0.5, 4.0])
+    a = [vals[torch.randint(0, 8, (M, k), generator=g)].to(torch.float8_e5m2).view(torch.uint8) for k in ks]
+    b = [vals[torch.randint(0, 8, (Nn, k), generator=g)].to(torch.float8_e4m3fn).view(torch.uint8) for k in ks]
+    return a, b
+
+
+@pytest.mark.parametrize("ks", [(512, 512), (1024, 512, 768), (512, 2048, 512, 1024)])
+@pytest.mark.parametrize("variant", [-1, 2, 5])
+def test_sum_of_products_power_of_two_is_bit_exact(N, ks, variant):
+    """Power-of-two values and scales: every partial sum and every ratio of scale products is exact, so the one-launch
+    route (accumulators carried from pair to pair, multiplied by the ratio in between) and the oracle must agree bit for
+    bit, in fp32 and in bf16; so must the per-pair route (forced variants 2 and 5: a GEMM per pair adding into C) in
+    fp32, and in bf16 with the oracle's composition of its one rounding per pair.
+    M and N end in half a tile (384 = 256 + 128, 640 = 2 x 256 + 128).  A pair skipped or read twice, a ratio applied the
+    wrong way round or to the wrong pair, or the wrong row pitch after a pair of another length all show."""
+    M, Nn = 384, 640
+    a, b = _pow2_pairs(M, Nn, ks, 31)
+    scales = [(torch.tensor([2.0 ** (3 - 2 * i)]), torch.tensor([2.0 ** (i - 6)])) for i in range(len(ks))]
+    ref16, ref32 = O.t_gemm_nt_sum([(x, y, p, q) for x, y, (p, q) in zip(a, b, scales)], O.E5M2, O.E4M3, want_f32=True)
+    if variant >= 0:
+        # a GEMM per pair rounds to the output type after every pair (the accumulate flag's definition)
+        for i, (x, y, (p, q)) in enumerate(zip(a, b, scales)):
+            part = O.t_gemm_nt(x, y, O.E5M2, O.E4M3, p, q, want_f32=True)[1]
+            ref16 = part.bfloat16() if i == 0 else O.t_accumulate(ref16, part)
+    dev = lambda ts: [t.cuda() for t in ts]
+    N.gemm_set_variant(variant)
+    try:
+        for out_dtype, ref in ((torch.float32, ref32), (torch.bfloat16, ref16)):
+            out = N.gemm_nt_sum(dev(a), dev(b), O.E5M2, O.E4M3, dev([p for p, _ in scales]), dev([q for _, q in scales]),
+                                out_dtype=out_dtype)
+            assert torch.equal(out.cpu(), ref), f"{out_dtype}: max diff {(out.cpu().float() - ref.float()).abs().max()}"
+    finally:
+        N.gemm_set_variant(-1)
+
+
+@pytest.mark.parametrize("shape", [(512, 768, (1024, 512)), (1024, 1280, (512, 1536, 768)), (256, 256, (512, 512, 512, 512))])
+def test_sum_of_products_random_operands_and_far_apart_scales(N, shape):
+    """Quantised Gaussian operands whose scale products lie up to 2^20 apart between pairs: against the oracle within the
+    GEMM tolerance in bf16 and within fp32 rounding of a few thousand additions in fp32; the per-pair route (a rounding
+    to the output type per pair) agrees with the one-launch route within the GEMM tolerance too."""
+    M, Nn, ks = shape
+    pairs, dev_args = [], ([], [], [], [])
+    for i, k in enumerate(ks):
+        aq, sa_inv = quantised((M, k), O.E5M2, 1e-3 * 32.0 ** i, 40 + i)
+        bq, sb_inv = quantised((Nn, k), O.E4M3, 0.02 * 32.0 ** i, 50 + i)
+        pairs.append((aq, bq, sa_inv, sb_inv))
+        for lst, t in zip(dev_args, (aq, bq, sa_inv, sb_inv)):
+            lst.append(t.cuda())
+    ref16, ref32 = O.t_gemm_nt_sum(pairs, O.E5M2, O.E4M3, want_f32=True)
+    out32 = N.gemm_nt_sum(dev_args[0], dev_args[1], O.E5M2, O.E4M3, dev_args[2], dev_args[3], out_dtype=torch.float32)
+    assert max_rel_err(out32, ref32) <= 2e-5
+    out16 = N.gemm_nt_sum(dev_args[0], dev_args[1], O.E5M2, O.E4M3, dev_args[2], dev_args[3])
+    assert max_rel_err(out16, ref16) <= TOL
+    assert torch.equal(out16, out32.bfloat16())                     # one rounding of the same fp32 values
+    N.gemm_set_variant(5)
+    try:
+        seq = N.gemm_nt_sum(dev_args[0], dev_args[1], O.E5M2, O.E4M3, dev_args[2], dev_args[3])
+    finally:
+        N.gemm_set_variant(-1)
+    assert max_rel_err(seq, ref16) <= TOL
+
+
+def test_sum_of_products_more_tiles_than_compute_units(N):
+    """288 tiles: blocks walk on to a second tile, whose first pair follows a fold and not a rescale, with the loads of
+    that pair requested while the last pair of the tile before was still being multiplied."""
+    M, Nn, ks = 4096, 4608, (512, 1024)
+    a, b = _pow2_pairs(M, Nn, ks, 61)
+    scales = [(torch.tensor([0.5]), torch.tensor([0.25])), (torch.tensor([4.0]), torch.tensor([2.0 ** -7]))]
+    ref = O.t_gemm_nt_sum([(x, y, p, q) for x, y, (p, q) in zip(a, b, scales)], O.E5M2, O.E4M3)
+    out = N.gemm_nt_sum([t.cuda() for t in a], [t.cuda() for t in b], O.E5M2, O.E4M3, [p.cuda() for p, _ in scales],
+                        [q.cuda() for _, q in scales])
+    assert torch.equal(out.cpu(), ref)
+
+
+def test_sum_of_products_shapes_outside_the_one_launch_route_and_errors(N):
+    """A contraction that is no multiple of 256, an output that is no multiple of 128 and a single pair all go the
+    per-pair way and still match the oracle; mismatched operands are refused before anything is launched."""
+    for M, Nn, ks in ((512, 384, (384, 512)), (200, 136, (512, 1024)), (256, 256, (64,)), (256, 384, (512, 512, 512, 512, 512))):
+        pairs, dev_args = [], ([], [], [], [])
+        for i, k in enumerate(ks):
+            aq, sa_inv = quantised((M, k), O.E5M2, 1e-3, 70 + i)
+            bq, sb_inv = quantised((Nn, k), O.E4M3, 0.02, 80 + i)
+            pairs.append((aq, bq, sa_inv, sb_inv))
+            for lst, t in zip(dev_args, (aq, bq, sa_inv, sb_inv)):
+                lst.append(t.cuda())
+        ref = O.t_gemm_nt_sum(pairs, O.E5M2, O.E4M3)
+        out = N.gemm_nt_sum(dev_args[0], dev_args[1], O.E5M2, O.E4M3, dev_args[2], dev_args[3])
+        assert max_rel_err(out, ref) <= TOL, (M, Nn, ks)
+    one = torch.ones(1, device="cuda")
+    a = torch.zeros((256, 512), dtype=torch.uint8, device="cuda")
+    with pytest.raises(N.NativeError):
+        N.gemm_nt_sum([a, a], [a, a[:, :256].contiguous()], O.E5M2, O.E4M3, [one, one], [one, one])       # K differs inside a pair
+    with pytest.raises(N.NativeError):
+        N.gemm_nt_sum([a, a[:128]], [a, a], O.E5M2, O.E4M3, [one, one], [one, one])                        # M differs between pairs
+    with pytest.raises(N.NativeError):
+        N.gemm_nt_sum([a, a], [a, a], O.E5M2, O.E4M3, [one], [one, one])                                   # a scale missing
+    with pytest.raises(N.NativeError):
+        N.gemm_nt_sum([a] * 65, [a] * 65, O.E5M2, O.E4M3, [one] * 65, [one] * 65)                          # more pairs than the call takes

@@ -224,3 +224,23 @@ def test_python_delayed_state_equals_c_oracle():
             st.update()
             O.c_delayed_update(hist, scale, inv, fmts, margin=2, algo=algo)
             assert np.array_equal(st.history, hist) and np.array_equal(st.scale, scale) and np.array_equal(st.scale_inv, inv)
+
+
+def test_sum_of_products_equals_one_product_over_joined_operands():
+    """With one scale pair for all, the sum over operand pairs is the product of the operands joined along the
+    contraction; on power-of-two values every partial sum is exact, so the two must agree bit for bit.  A pair dropped,
+    counted twice or scaled by another pair's scales breaks it."""
+    g = torch.Generator().manual_seed(3)
+    vals = torch.tensor([0.0, 1.0, -1.0, 2.0, -2.0, 0.5, -0.5, 4.0])
+    ks = (64, 32, 96)
+    a = [vals[torch.randint(0, 8, (24, k), generator=g)].to(torch.float8_e5m2).view(torch.uint8) for k in ks]
+    b = [vals[torch.randint(0, 8, (40, k), generator=g)].to(torch.float8_e4m3fn).view(torch.uint8) for k in ks]
+    sa, sb = torch.tensor([0.5]), torch.tensor([0.125])
+    joined = O.t_gemm_nt(torch.cat(a, 1), torch.cat(b, 1), O.E5M2, O.E4M3, sa, sb, want_f32=True)[1]
+    got16, got32 = O.t_gemm_nt_sum([(x, y, sa, sb) for x, y in zip(a, b)], O.E5M2, O.E4M3, want_f32=True)
+    assert torch.equal(got32, joined) and torch.equal(got16, joined.bfloat16())
+    # a scale of its own per pair: linear in each
+    scales = [(torch.tensor([2.0 ** -i]), torch.tensor([2.0 ** i * 0.25])) for i in range(3)]
+    want = sum(O.t_gemm_nt(x, y, O.E5M2, O.E4M3, p, q, want_f32=True)[1] for x, y, (p, q) in zip(a, b, scales))
+    got = O.t_gemm_nt_sum([(x, y, p, q) for x, y, (p, q) in zip(a, b, scales)], O.E5M2, O.E4M3, want_f32=True)[1]
+    assert torch.equal(got, want) and torch.equal(got, joined * 0.25 / 0.0625)
