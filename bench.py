@@ -390,11 +390,11 @@ def standalone_hbm(torch, native, iters=24):
     return out
 
 
-def attention_projections(torch, steps=8, warmup=3):
-    """configs[1] of BASELINE.json as it is written: ONE X [8192, 4096] feeds Wq [4096, 4096], Wk and Wv [1024, 4096]
-    (optimus_dl/modules/model/blocks/attention.py:317-319), Wo [4096, 4096] has an input of its own; forward + backward
-    of all four, weights re-quantised every step.  The transform groups q / k / v as it does in a model: X is quantised
-    once, and the three data gradients are summed by the GEMMs (the `accumulate` flag) into one dX."""
+def sibling_linears(torch, label, grouped, alone, m, steps=8, warmup=3):
+    """Linears fed ONE X (``grouped``: name -> (in, out), names the transform ties into a sibling group) and Linears with
+    an input of their own (``alone``), forward + backward of all, weights re-quantised every step.  The transform groups
+    the former as it does in a model: X is quantised once, and their data gradients come out as one dX (one GEMM over
+    all members' operands, or GEMMs that add into it)."""
     import torch.nn as nn
 
     from optimus_dl_amd.modules.amp import create_fp8_recipe
@@ -403,13 +403,12 @@ def attention_projections(torch, steps=8, warmup=3):
     class Projections(nn.Module):
         def __init__(self):
             super().__init__()
-            self.wq, self.wk, self.wv = nn.Linear(4096, 4096, bias=False), nn.Linear(4096, 1024, bias=False), nn.Linear(4096, 1024, bias=False)
-            self.wo = nn.Linear(4096, 4096, bias=False)
+            for name, (k, n) in {**grouped, **alone}.items():
+                setattr(self, name, nn.Linear(k, n, bias=False))
 
-        def forward(self, x, o):
-            return self.wq(x), self.wk(x), self.wv(x), self.wo(o)
+        def forward(self, x, others):
+            return [getattr(self, name)(x) for name in grouped] + [getattr(self, name)(o) for name, o in zip(alone, others)]
 
-    m = 8192
     g = torch.Generator().manual_seed(0)
     net = Projections().to("cuda", torch.bfloat16)
     with torch.no_grad():
@@ -417,27 +416,45 @@ def attention_projections(torch, steps=8, warmup=3):
             p.copy_((torch.randn(p.shape, generator=g) * 0.02).bfloat16())
     build_model_transform({"_name": "fp8_linear"}).apply(net)
     recipe = create_fp8_recipe("tensorwise", "hybrid")
-    x = torch.randn(m, 4096, generator=g).bfloat16().cuda().requires_grad_(True)
-    o = torch.randn(m, 4096, generator=g).bfloat16().cuda().requires_grad_(True)
-    dys = [(torch.randn(m, n, generator=g) * 1e-3).bfloat16().cuda() for n in (4096, 1024, 1024, 4096)]
-    mods = [net.wq, net.wk, net.wv, net.wo]
+    k_in = next(iter(grouped.values()))[0]
+    x = torch.randn(m, k_in, generator=g).bfloat16().cuda().requires_grad_(True)
+    others = [torch.randn(m, k, generator=g).bfloat16().cuda().requires_grad_(True) for k, _ in alone.values()]
+    mods = [getattr(net, name) for name in (*grouped, *alone)]
+    dys = [(torch.randn(m, lin.out_features, generator=g) * 1e-3).bfloat16().cuda() for lin in mods]
 
     def one():
         for lin in mods:
             weights_changed(lin)
             lin.weight.grad = None
-        x.grad = o.grad = None
+        x.grad = None
+        for o in others:
+            o.grad = None
         with recipe.autocast():
-            ys = net(x, o)
+            ys = net(x, others)
         with recipe.backward():
             torch.autograd.backward(ys, dys)
 
     t = timed_steps(torch, one, steps, warmup)
     flop = sum(6.0 * m * lin.in_features * lin.out_features for lin in mods)
-    res = {"configs[1] attention projections, tensorwise": {**t, "TFLOP/s": flop / (t["ms_per_step"] * 1e-3) / 1e12, "flop_per_step": flop}}
-    del net, x, o, dys, one
+    res = {label: {**t, "TFLOP/s": flop / (t["ms_per_step"] * 1e-3) / 1e12, "flop_per_step": flop}}
+    del net, x, others, dys, one
     torch.cuda.empty_cache()
     return res
+
+
+def attention_projections(torch, steps=8, warmup=3):
+    """configs[1] of BASELINE.json as it is written: ONE X [8192, 4096] feeds Wq [4096, 4096], Wk and Wv [1024, 4096]
+    (optimus_dl/modules/model/blocks/attention.py:317-319), Wo [4096, 4096] has an input of its own."""
+    return sibling_linears(torch, "configs[1] attention projections, tensorwise",
+                           {"wq": (4096, 4096), "wk": (4096, 1024), "wv": (4096, 1024)}, {"wo": (4096, 4096)}, 8192, steps, warmup)
+
+
+def mlp_one_input(torch, steps=8, warmup=3):
+    """configs[2] with W_gate and W_up fed the ONE X that BASELINE.json names (optimus_dl/modules/model/blocks/mlp.py:76-78
+    feeds w1 and w2 the same tensor); W_down has an input of its own, as in the headline.  Same GEMM work as the
+    headline step, which gives every Linear an X of its own: one quantisation of X less, and one dX instead of two."""
+    return sibling_linears(torch, "configs[2] with gate and up fed one X (a sibling group)",
+                           {"w1": (D_MODEL, D_FF), "w2": (D_MODEL, D_FF)}, {"c_proj": (D_FF, D_MODEL)}, M_TOKENS, steps, warmup)
 
 
 def other_configs(torch, steps=8, warmup=3, only=""):
@@ -459,6 +476,8 @@ def other_configs(torch, steps=8, warmup=3, only=""):
     out = {}
     if not only or only in "configs[1] attention projections, tensorwise":
         out.update(attention_projections(torch, steps, warmup))
+    if not only or only in "configs[2] with gate and up fed one X (a sibling group)":
+        out.update(mlp_one_input(torch, steps, warmup))
     for label, kind, kw, shapes, m, wdtype in cases:
         if only and only not in label:
             continue

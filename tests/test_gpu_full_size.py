@@ -632,3 +632,30 @@ def test_config_2_grouped_projections_sum_their_data_gradients_in_the_gemms(N):
     # the one launch rounds the fp32 sum once: closer to it than a rounding per member
     err = {route: float((results[route][1][ri][:, ci].float().cpu() - ref).abs().max()) for route in ("one gemm", "accumulate")}
     assert err["one gemm"] <= err["accumulate"] * 1.05 + 1e-12, err
+
+
+def test_gate_and_up_data_gradient_in_one_launch_at_config_3_size(N):
+    """dX [8192, 4096] = dY_gate . W_gate + dY_up . W_up with contractions of 14336 each (configs[2] with gate and up fed
+    one X): the one-launch route against a GEMM per pair adding into fp32 on the GPU (whole matrix) and against the
+    oracle on sampled rows and columns; bf16 output = one rounding of the same fp32 values."""
+    M, K, F = 8192, 4096, 14336
+    gq, sg = [], []
+    wq, sw = [], []
+    for i in range(2):
+        q, _, _, _, s_inv = N.quantize_dynamic(draw((M, F), 1e-3 * (3.0 ** i), 300 + i), O.E5M2, want_transposed=False)
+        gq.append(q); sg.append(s_inv)
+        _, q_t, _, _, s_inv = N.quantize_dynamic(draw((F, K), 0.02 / (2.0 ** i), 310 + i), O.E4M3)
+        wq.append(q_t); sw.append(s_inv)
+    one = N.gemm_nt_sum(gq, wq, O.E5M2, O.E4M3, sg, sw, out_dtype=torch.float32)
+    N.gemm_set_variant(5)
+    try:
+        seq = N.gemm_nt_sum(gq, wq, O.E5M2, O.E4M3, sg, sw, out_dtype=torch.float32)
+    finally:
+        N.gemm_set_variant(-1)
+    assert max_rel_err(one, seq) <= 2e-5
+    assert torch.equal(N.gemm_nt_sum(gq, wq, O.E5M2, O.E4M3, sg, sw), one.bfloat16())
+    ri = torch.randperm(M, generator=torch.Generator().manual_seed(7))[:48].sort().values.cuda()
+    ci = torch.randperm(K, generator=torch.Generator().manual_seed(8))[:192].sort().values.cuda()
+    ref = O.t_gemm_nt_sum([(gq[i][ri].cpu(), wq[i][ci].cpu(), sg[i].cpu(), sw[i].cpu()) for i in range(2)], O.E5M2, O.E4M3,
+                          want_f32=True)[1]
+    assert max_rel_err(one[ri][:, ci].cpu(), ref) <= 2e-5

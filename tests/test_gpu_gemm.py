@@ -654,3 +654,41 @@ def test_sum_of_products_shapes_outside_the_one_launch_route_and_errors(N):
         N.gemm_nt_sum([a, a], [a, a], O.E5M2, O.E4M3, [one], [one, one])                                   # a scale missing
     with pytest.raises(N.NativeError):
         N.gemm_nt_sum([a] * 65, [a] * 65, O.E5M2, O.E4M3, [one] * 65, [one] * 65)                          # more pairs than the call takes
+
+
+def test_sum_of_products_shape_sweep_against_the_per_pair_route(N):
+    """Seeded sweep over pair counts, contraction lengths (equal and unequal, 512 .. 2304) and output shapes (whole and
+    half tiles at either edge, one tile, more tiles than fit one round of a small grid): the one-launch route against a
+    GEMM per pair adding into an fp32 C, which shares no code with it beyond the MFMA.  fp32 outputs, so the only
+    differences are the order of fp32 additions and the ratio multiplications."""
+    g = torch.Generator().manual_seed(77)
+    lengths = [512, 768, 1024, 1280, 1536, 2304]
+    shapes = [(128, 128), (256, 256), (384, 128), (128, 640), (640, 896), (1152, 256), (2176, 1408)]
+    for case in range(21):
+        M, Nn = shapes[case % len(shapes)]
+        pairs = 2 + case % 3
+        ks = [lengths[int(torch.randint(0, len(lengths), (1,), generator=g))] for _ in range(pairs)]
+        a = [torch.randint(0, 256, (M, k), generator=g, dtype=torch.uint8) for k in ks]
+        b = [torch.randint(0, 256, (Nn, k), generator=g, dtype=torch.uint8) for k in ks]
+        for t in a:                                   # no NaN / Inf codes (e5m2: exponent 31; e4m3: 0x7f / 0xff)
+            t[(t & 0x7C) == 0x7C] = 0x3C
+        for t in b:
+            t[(t & 0x7F) == 0x7F] = 0x38
+        sa = [torch.rand(1, generator=g) * 2.0 ** float(torch.randint(-12, 4, (1,), generator=g)) + 2.0 ** -20 for _ in ks]
+        sb = [torch.rand(1, generator=g) * 2.0 ** float(torch.randint(-12, 4, (1,), generator=g)) + 2.0 ** -20 for _ in ks]
+        dev = lambda ts: [t.cuda() for t in ts]
+        one = N.gemm_nt_sum(dev(a), dev(b), O.E5M2, O.E4M3, dev(sa), dev(sb), out_dtype=torch.float32)
+        N.gemm_set_variant(2)
+        try:
+            seq = N.gemm_nt_sum(dev(a), dev(b), O.E5M2, O.E4M3, dev(sa), dev(sb), out_dtype=torch.float32)
+        finally:
+            N.gemm_set_variant(-1)
+        assert torch.isfinite(one).all(), (case, M, Nn, ks)
+        assert max_rel_err(one, seq) <= 2e-5, (case, M, Nn, ks, max_rel_err(one, seq))
+        if case % 7 == 0:
+            # uniformly drawn codes span the formats' whole range (products 2^-25 .. 2^24.6 side by side) and the sums cancel
+            # heavily: the matrix instruction's adder keeps fewer bits below the largest product of its 64 than an fp32
+            # sum does (both routes above share that), so against the oracle the bound is 1e-4 of the largest output,
+            # still a hundredth of the GEMM tolerance and far below what a wrong pair, ratio or pitch would give
+            ref = O.t_gemm_nt_sum(list(zip(a, b, sa, sb)), O.E5M2, O.E4M3, want_f32=True)[1]
+            assert max_rel_err(one, ref) <= 1e-4, (case, M, Nn, ks)
