@@ -152,7 +152,9 @@ def timed_steps(torch, one, steps, warmup):
     """`warmup` untimed calls of `one`, then `steps` timed ones.  ms_per_step is wall time over all of them (host clock,
     synchronised on both sides); min / median / max are per step, from one HIP event between consecutive steps, so a
     single slow step (an allocator that has to grow, a first-use set-up) shows up as max >> median instead of hiding in
-    the mean.  `allocator` tells whether torch's caching allocator had to go back to the driver during the timed steps."""
+    the mean.  host_issue_ms_per_step is the time the host took to queue the launches of the timed steps (close to
+    ms_per_step: the host, not the GPU, sets the pace).  `allocator` tells whether torch's caching allocator had to go back
+    to the driver during the timed steps."""
     t_w = time.perf_counter()
     for _ in range(warmup):
         one()
@@ -172,12 +174,13 @@ def timed_steps(torch, one, steps, warmup):
     for i in range(steps):
         one()
         marks[i + 1].record()
+    issued = time.perf_counter() - t0          # the host has queued every launch; the GPU is still working
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     after = torch.cuda.memory_stats()
     in_order = [marks[i].elapsed_time(marks[i + 1]) for i in range(steps)]
     per = sorted(in_order)
-    return {"ms_per_step": 1e3 * wall / steps, "warmup_steps": warmup + extra, "min_ms": per[0], "median_ms": per[len(per) // 2], "max_ms": per[-1],
+    return {"ms_per_step": 1e3 * wall / steps, "host_issue_ms_per_step": 1e3 * issued / steps, "warmup_steps": warmup + extra, "min_ms": per[0], "median_ms": per[len(per) // 2], "max_ms": per[-1],
             "max_over_median": per[-1] / per[len(per) // 2], "slowest_step": in_order.index(per[-1]),
             "per_step_ms": [round(t, 3) for t in in_order],
             "allocator": {"segments_allocated_during_timed_steps": after.get("num_device_alloc", 0) - before.get("num_device_alloc", 0),

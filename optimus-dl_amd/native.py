@@ -186,7 +186,14 @@ def _check(status: int, what: str) -> None:
         raise NativeError(f"{what} refused (status {status}): {msg}")
 
 
+# the handle of the current stream without building a torch.cuda.Stream object around it: that constructor and the
+# device look-ups on its way cost 10 us a call, 0.4 ms over the 40 launches of a small step
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream() -> int:
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 
