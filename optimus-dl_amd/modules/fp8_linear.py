@@ -378,8 +378,9 @@ class _MemberCtx:
 class _Fp8LinearGroupFn(torch.autograd.Function):
     """Several FP8 Linears applied to ONE input (q/k/v of an attention block, gate/up of a gated MLP) as one autograd
     node: forward = the members' forwards (they share the quantised input anyway), backward = the members' backwards
-    with the data gradients summed by the GEMMs themselves: the first member writes dx, every further one adds its
-    product into it (``accumulate``), where separate nodes leave two extra passes over dx per block to autograd."""
+    with the data gradients summed by the GEMMs themselves: ONE GEMM whose contraction runs through all members'
+    operands where the shapes allow (``native.gemm_nt_sum``), else the first member writes dx and every further one adds
+    its product into it (``accumulate``); separate nodes leave two extra passes over dx per block to autograd."""
 
     @staticmethod
     def forward(ctx, x2d: torch.Tensor, recipe: FP8Recipe, out_dtype: torch.dtype, modules: tuple, *params: torch.Tensor | None):
