@@ -234,3 +234,44 @@ def test_sibling_group_data_gradient_from_one_gemm(amp, kind, monkeypatch):
         assert bool(((got[1].float() - exact).abs() <= bound).all())
     else:
         assert (got[1].float() - want[1].float()).abs().max().item() <= 3 * 2.0 ** -8 * want[1].float().abs().max().item()
+
+
+def test_one_gemm_data_gradient_replays_from_a_graph(amp):
+    """The call that sums the members' products takes host arrays of device pointers and hands them to the kernel by value:
+    captured in a graph it must replay on new data like everything else (three replays, eager work and synchronisations
+    in between, each against eager on the same buffers)."""
+    net, recipe = build_wide(), amp.create_fp8_recipe("tensorwise", "hybrid")
+    x_static = torch.zeros((4096, 2304), dtype=torch.bfloat16, device="cuda", requires_grad=True)
+    dy_static = [torch.zeros((4096, n), dtype=torch.bfloat16, device="cuda") for n in (1024, 512, 512)]
+    params = [net.wq.weight, net.wk.weight, net.wv.weight]
+
+    def fwd_bwd():
+        for lin in (net.wq, net.wk, net.wv):
+            lin._wcache.key = None
+        with recipe.autocast():
+            ys = net(x_static)
+        with recipe.backward():
+            grads = torch.autograd.grad(ys, (x_static, *params), dy_static)
+        return (*ys, *grads)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            fwd_bwd()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs_g = fwd_bwd()
+    for rep in range(3):
+        with torch.no_grad():
+            x_static.copy_(seeded_bf16((4096, 2304), 1.0 + rep, 950 + rep).cuda())
+            for i, d in enumerate(dy_static):
+                d.copy_(seeded_bf16(tuple(d.shape), 1e-3 * (rep + 1) * 3.0 ** i, 960 + 3 * rep + i).cuda())
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in outs_g]
+        want = fwd_bwd()
+        torch.cuda.synchronize()
+        for i, (a, b) in enumerate(zip(got, want)):
+            assert torch.equal(a, b), f"replay {rep}: output {i} differs from eager"
