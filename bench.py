@@ -797,6 +797,8 @@ def main() -> int:
                     help="run only the whole-model step of gpt2_124m or qwen3_0.6b with the default transform and print it (for profiling)")
     ap.add_argument("--recipe", default="tensorwise",
                     help="with --whole-models-only: the scaling recipe (tensorwise, delayed, rowwise, mxfp8, blockwise)")
+    ap.add_argument("--llama-block-only", action="store_true",
+                    help="run only the Llama-3-8B decoder block (bf16 autocast, FP8 Linears, FP8 Linears + fused producers) and print it (for profiling)")
     ap.add_argument("--other-configs-only", default="",
                     help="run only the whole steps of the other configurations whose label contains this text (e.g. mxfp8, rowwise, "
                          "delayed) and print them (for profiling)")
@@ -845,6 +847,9 @@ def main() -> int:
             self.fuse_dgrad_gemm = not args.dgrad_sum_by_accumulate
 
         _fp8.FP8Recipe.__init__ = _init_without_fusion
+    if args.llama_block_only:
+        print(json.dumps({"llama3_8b_block_fwd_bwd": llama_block(torch, steps=args.steps)}))
+        return 0
     if args.other_configs_only:
         print(json.dumps({"other_configs_fwd_bwd": other_configs(torch, steps=args.steps, only=args.other_configs_only)}))
         return 0
