@@ -146,6 +146,27 @@ def _mx_input_shared(recipe: FP8Recipe, x2d: torch.Tensor, fmt: int, need_t: boo
     return q, sc, q_t, sc_t
 
 
+def _rowwise_input_shared(recipe: FP8Recipe, x2d: torch.Tensor, fmt: int, margin: int, need_t: bool):
+    """Rowwise codes of a Linear's input: per-row scales for the forward GEMM and, with need_t, the transposed codes with
+    per-column scales for wgrad, made once for the Linears fed by the very same tensor (two passes over x for q / k / v
+    together instead of two each).  -> (xq, sx_inv, xq_t or None, sx_inv_t or None)."""
+    key = _input_key(x2d, "rowwise", fmt, margin)
+    hit = recipe.shared_input if recipe.share_inputs else None
+    if hit is not None and hit["key"] == key and (hit["q_t"] is not None or not need_t):
+        return hit["q"], hit["s_inv"], hit["q_t"], hit["s_t"]
+    if need_t:
+        q, s_inv, q_t, s_t, _, _ = native.quantize_rowcol(x2d, fmt, margin)
+    else:
+        (q, s_inv), q_t, s_t = _quantise_axis(x2d, fmt, margin, R, False), None, None
+    if recipe.share_inputs:
+        entry = {"key": key, "x": x2d, "q": q, "q_t": q_t, "s_inv": s_inv, "s_t": s_t}
+        prev = recipe.shared_input
+        if prev is not None and prev.get("x") is x2d:
+            entry["src_key"], entry["src"] = prev.get("src_key"), prev.get("src")
+        recipe.shared_input = entry
+    return q, s_inv, q_t, s_t
+
+
 def _converted_input(recipe: FP8Recipe, x2d: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
     """x2d in the compute dtype, contiguous.  Linears fed by the same tensor get the same
     converted tensor back (one conversion, and one quantisation downstream); autograd sees an
@@ -212,11 +233,12 @@ class _Fp8LinearFn(torch.autograd.Function):
             if need_dgrad:
                 saved["wq_t"], saved["ws_t"] = wq_t, ws_t
         elif pol.kind == "rowwise":
-            if need_wgrad and recipe.wgrad:
-                # both operands of x in two passes over it: rows for this GEMM, columns (transposed) for wgrad
-                xq, sx_inv, saved["xq_t"], saved["sx_inv_t"], _, _ = native.quantize_rowcol(x2d, pol.fmt_fwd, pol.margin)
-            else:
-                xq, sx_inv = _quantise_axis(x2d, pol.fmt_fwd, pol.margin, R, False)
+            # both operands of x in two passes over it: rows for this GEMM, columns (transposed) for wgrad; shared by the
+            # Linears fed the very same tensor
+            fp8_wgrad = need_wgrad and recipe.wgrad
+            xq, sx_inv, xq_t, sx_inv_t = _rowwise_input_shared(recipe, x2d, pol.fmt_fwd, pol.margin, fp8_wgrad)
+            if fp8_wgrad:
+                saved["xq_t"], saved["sx_inv_t"] = xq_t, sx_inv_t
             if not recipe.cache_weights:
                 module._wcache_rowwise.clear()          # the backward of this call still finds what is made now
             wq, sw_inv = module._rowwise_weight(weight, pol, "row", both=need_dgrad)

@@ -371,6 +371,50 @@ def test_linears_fed_by_the_same_tensor_quantise_it_once(amp, monkeypatch, in_dt
             assert torch.equal(a, b)
 
 
+def test_rowwise_linears_fed_by_the_same_tensor_quantise_it_once(amp, monkeypatch):
+    """The rowwise recipe quantises an input in two passes (row scales for the forward, column scales and the transposed
+    codes for wgrad): Linears fed the very same tensor share them; same bits as quantising per Linear; Linears with frozen
+    weights (no wgrad) take the row pass only and share that."""
+    from optimus_dl_amd import native
+
+    M, K, N = 256, 512, 384
+    x = seeded_bf16((M, K), 1.0, 44)
+    wg, wu = seeded_bf16((N, K), 0.02, 45), seeded_bf16((N, K), 0.02, 46)
+    dy = seeded_bf16((M, N), 1e-3, 47).cuda()
+
+    def count_of(fn):
+        calls = []
+        orig = getattr(native, fn)
+        monkeypatch.setattr(native, fn, lambda *a, **k: (calls.append(tuple(a[0].shape)), orig(*a, **k))[1])
+        return calls
+
+    def run(share):
+        recipe = amp.create_fp8_recipe("rowwise", "hybrid")
+        recipe.share_inputs = share
+        gate, up = make_linear(wg), make_linear(wu)
+        xd = x.cuda().requires_grad_(True)
+        with recipe.autocast():
+            h = gate(xd) * up(xd)
+        with recipe.backward():
+            h.backward(dy)
+        assert recipe.shared_input is None
+        gate.weight.requires_grad_(False)
+        up.weight.requires_grad_(False)
+        with recipe.autocast():
+            e = gate(xd) + up(xd)
+        return h.detach(), xd.grad.detach(), gate.weight.grad.detach(), up.weight.grad.detach(), e.detach()
+
+    both, rows_only = count_of("quantize_rowcol"), count_of("amax")
+    shared = run(True)
+    n_shared = (len([c for c in both if c == (M, K)]), len([c for c in rows_only if c == (M, K)]))
+    both.clear(); rows_only.clear()
+    separate = run(False)
+    n_separate = (len([c for c in both if c == (M, K)]), len([c for c in rows_only if c == (M, K)]))
+    assert n_shared == (1, 1) and n_separate == (2, 2), (n_shared, n_separate)
+    for a, b in zip(shared, separate):
+        assert torch.equal(a, b)
+
+
 def test_shared_input_is_not_reused_after_an_in_place_change_or_for_another_tensor(amp, monkeypatch):
     from optimus_dl_amd import native
 
