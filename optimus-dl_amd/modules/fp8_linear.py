@@ -316,7 +316,11 @@ class _Fp8LinearFn(torch.autograd.Function):
                 gq_t, sg_inv_t = _quantise_axis(dy2d, pol.fmt_bwd, pol.margin, C, True)
             if ctx.need_dgrad:
                 wq_t, sw_inv_t = module._rowwise_weight(saved["weight"], pol, "col")
-                dx = native.gemm_nt(gq, wq_t, pol.fmt_bwd, pol.fmt_fwd, sg_inv, sw_inv_t, out_dtype=ctx.x_dtype)
+                dx_into = getattr(ctx, "dx_into", None)      # a later member of a sibling group adds into the group's dx
+                if dx_into is not None:
+                    dx = native.gemm_nt(gq, wq_t, pol.fmt_bwd, pol.fmt_fwd, sg_inv, sw_inv_t, out=dx_into, accumulate=True)
+                else:
+                    dx = native.gemm_nt(gq, wq_t, pol.fmt_bwd, pol.fmt_fwd, sg_inv, sw_inv_t, out_dtype=ctx.x_dtype)
             if fp8_wgrad:
                 dw = native.gemm_nt(gq_t, saved["xq_t"], pol.fmt_bwd, pol.fmt_fwd, sg_inv_t, saved["sx_inv_t"],
                                     out_dtype=ctx.w_dtype)
@@ -516,10 +520,10 @@ class _Fp8LinearGroupFn(torch.autograd.Function):
 @torch.compiler.disable
 def linear_group(x: torch.Tensor, modules: "tuple[FP8Linear, ...]") -> tuple[torch.Tensor, ...] | None:
     """``tuple(m(x) for m in modules)`` as one autograd node (see ``_Fp8LinearGroupFn``), or None where the members
-    cannot run that way (no recipe, a recipe other than tensorwise / delayed, shapes the FP8 path refuses): the caller
+    cannot run that way (no recipe, a block-scaled recipe, shapes the FP8 path refuses): the caller
     then applies the modules one by one."""
     recipe = _state.active_recipe()
-    if recipe is None or recipe.recipe.kind not in ("tensorwise", "delayed") or not recipe.fuse_dgrad_sum:
+    if recipe is None or recipe.recipe.kind not in ("tensorwise", "delayed", "rowwise") or not recipe.fuse_dgrad_sum:
         return None
     if not all(m._fp8_eligible(x) for m in modules):
         return None

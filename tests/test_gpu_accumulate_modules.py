@@ -50,7 +50,7 @@ def run(net, recipe, x, dys):
     return [o.detach() for o in outs], xd.grad, [p.grad for p in net.parameters()]
 
 
-@pytest.mark.parametrize("kind", ["tensorwise", "delayed"])
+@pytest.mark.parametrize("kind", ["tensorwise", "delayed", "rowwise"])
 @pytest.mark.parametrize("bias", [False, True])
 def test_sibling_group_equals_separate_linears(amp, kind, bias):
     """Outputs and weight gradients are the same bits (same kernels on the same operands); the data gradient is the sum
